@@ -1,0 +1,200 @@
+"""Test-side loaders and helpers for the two CPU checkers.
+
+* ``oracle``  -- this repository's C restatement of the ggml-cpu algorithms
+  (``oracle/liboracle.so``, built from ``oracle/oracle.c``).
+* ``ref``     -- the reference's own ggml + ggml-cpu, compiled from the reference
+  checkout into ``oracle/_ref/<isa>/`` and driven through ``oracle/ref_harness.cpp``.
+  It exists only where it was prebuilt; tests that need it skip otherwise.
+
+Tensors cross both C boundaries as a small descriptor (type, ne[4], nb[4] in bytes,
+data pointer) in ggml's convention: ``ne[0]`` is the fastest dimension, so a numpy
+array of shape ``(n3, n2, n1, n0)`` maps to ``ne = [n0, n1, n2, n3]``.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+
+F32, F16, Q8_0, I32 = 0, 1, 8, 26
+QK8_0 = 32
+Q8_BLOCK_BYTES = 34
+
+
+class Tensor(C.Structure):
+    _fields_ = [
+        ("type", C.c_int32),
+        ("_pad", C.c_int32),
+        ("ne", C.c_int64 * 4),
+        ("nb", C.c_uint64 * 4),
+        ("data", C.c_void_p),
+    ]
+
+
+_NP_TYPES = {np.dtype(np.float32): F32, np.dtype(np.float16): F16, np.dtype(np.int32): I32}
+
+
+def desc(a, ttype=None):
+    """Descriptor of a numpy array (any strides, at most 4 dims, last dim dense)."""
+    assert a.ndim <= 4
+    if ttype is None:
+        ttype = _NP_TYPES[a.dtype]
+    shape = (1,) * (4 - a.ndim) + tuple(a.shape)
+    strides = list(a.strides)
+    # leading broadcast dims get the stride ggml would give a dense tensor
+    while len(strides) < 4:
+        strides.insert(0, strides[0] * shape[4 - len(strides)] if strides else a.itemsize)
+    t = Tensor()
+    t.type = ttype
+    for i in range(4):
+        t.ne[i] = shape[3 - i]
+        t.nb[i] = strides[3 - i]
+    assert t.nb[0] == a.itemsize, "fastest dimension must be dense"
+    t.data = a.ctypes.data
+    t._keep = a
+    return t
+
+
+def desc_q8(raw, ne0):
+    """Descriptor of a Q8_0 tensor held as uint8 rows: shape (..., rows, ne0/32*34)."""
+    assert raw.dtype == np.uint8 and raw.flags.c_contiguous
+    assert raw.shape[-1] == ne0 // QK8_0 * Q8_BLOCK_BYTES
+    shape = (1,) * (4 - raw.ndim) + tuple(raw.shape)
+    t = Tensor()
+    t.type = Q8_0
+    t.ne[0] = ne0
+    t.ne[1], t.ne[2], t.ne[3] = shape[2], shape[1], shape[0]
+    rowb = shape[3]
+    t.nb[0] = Q8_BLOCK_BYTES
+    t.nb[1] = rowb
+    t.nb[2] = rowb * shape[2]
+    t.nb[3] = rowb * shape[2] * shape[1]
+    t.data = raw.ctypes.data
+    t._keep = raw
+    return t
+
+
+def ptr(a, ctype):
+    return None if a is None else a.ctypes.data_as(C.POINTER(ctype))
+
+
+# ----------------------------------------------------------------------------- oracle
+_oracle = None
+
+
+def load_oracle():
+    global _oracle
+    if _oracle is not None:
+        return _oracle
+    path = os.path.join(ORACLE_DIR, "liboracle.so")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", ORACLE_DIR, "oracle"], stdout=subprocess.DEVNULL)
+    lib = C.CDLL(path)
+    TP = C.POINTER(Tensor)
+    f32p, i32p, u16p = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint16)
+    lib.orc_fp32_to_fp16.restype = C.c_uint16
+    lib.orc_fp32_to_fp16.argtypes = [C.c_float]
+    lib.orc_fp16_to_fp32.restype = C.c_float
+    lib.orc_fp16_to_fp32.argtypes = [C.c_uint16]
+    lib.orc_fp32_to_fp16_row.argtypes = [f32p, u16p, C.c_int64]
+    lib.orc_fp16_to_fp32_row.argtypes = [u16p, f32p, C.c_int64]
+    for name in ("orc_quantize_row_q8_0_ref", "orc_quantize_row_q8_0_x86"):
+        getattr(lib, name).argtypes = [f32p, C.c_void_p, C.c_int64]
+    lib.orc_dequantize_row_q8_0.argtypes = [C.c_void_p, f32p, C.c_int64]
+    for name in ("orc_vec_dot_q8_0_q8_0", "orc_vec_dot_q8_0_q8_0_avx2"):
+        getattr(lib, name).restype = C.c_float
+        getattr(lib, name).argtypes = [C.c_int64, C.c_void_p, C.c_void_p]
+    lib.orc_mul_mat.argtypes = [TP, TP, TP, C.c_int]
+    lib.orc_mul_mat_f64.argtypes = [TP, TP, TP]
+    lib.orc_rms_norm.argtypes = [TP, TP, C.c_float]
+    lib.orc_rope.argtypes = [TP, i32p, f32p, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6
+    lib.orc_soft_max.argtypes = [TP, TP, f32p, TP, C.c_float, C.c_float]
+    lib.orc_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]
+    lib.orc_flash_attn_ext_f64.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float]
+    i64p, u64p = C.POINTER(C.c_int64), C.POINTER(C.c_uint64)
+    lib.orc_kv_read_view.argtypes = [C.c_int] * 5 + [i64p, u64p, u64p]
+    lib.orc_kv_write_view.argtypes = [C.c_int] * 6 + [i64p, u64p, u64p]
+    lib.orc_causal_mask.argtypes = [i32p, C.c_int, C.c_int, u16p]
+    lib.orc_cfg_pair_constants.argtypes = [C.c_int, i32p, u16p]
+    lib.orc_t_span.argtypes = [C.c_int, C.c_float, f32p]
+    _oracle = lib
+    return lib
+
+
+# -------------------------------------------------------------------------- reference
+_ref = None
+_ref_tried = False
+
+
+def cpu_isa():
+    try:
+        flags = open("/proc/cpuinfo").read()
+    except OSError:
+        return "avx2"
+    need = ("avx512f", "avx512bw", "avx512dq", "avx512vl", "avx512cd", "avx512_vnni")
+    return "avx512" if all(f in flags for f in need) else "avx2"
+
+
+def ref_dir():
+    return os.path.join(ORACLE_DIR, "_ref", cpu_isa())
+
+
+def load_ref():
+    """The reference's ggml-cpu behind oracle/ref_harness.cpp, or None when not prebuilt."""
+    global _ref, _ref_tried
+    if _ref_tried:
+        return _ref
+    _ref_tried = True
+    path = os.path.join(ref_dir(), "libref_harness.so")
+    if not os.path.exists(path):
+        return None
+    C.CDLL(os.path.join(ref_dir(), "libggml-ref.so"), mode=C.RTLD_GLOBAL)
+    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    TP = C.POINTER(Tensor)
+    f32p, i32p, u16p, f64p = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint16), C.POINTER(C.c_double)
+    lib.rh_load_plugin.argtypes = [C.c_char_p]
+    lib.rh_device_name.restype = C.c_char_p
+    lib.rh_device_name.argtypes = [C.c_int]
+    lib.rh_use_device.argtypes = [C.c_char_p, C.c_int, C.c_int]
+    lib.rh_fp32_to_fp16_row.argtypes = [f32p, u16p, C.c_int64]
+    lib.rh_fp16_to_fp32_row.argtypes = [u16p, f32p, C.c_int64]
+    lib.rh_quantize_q8_0.restype = C.c_size_t
+    lib.rh_quantize_q8_0.argtypes = [f32p, C.c_void_p, C.c_int64, C.c_int64]
+    lib.rh_dequantize_q8_0.argtypes = [C.c_void_p, f32p, C.c_int64]
+    lib.rh_quantize_q8_0_cpu.argtypes = [f32p, C.c_void_p, C.c_int64]
+    lib.rh_vec_dot_q8_0_q8_0.restype = C.c_float
+    lib.rh_vec_dot_q8_0_q8_0.argtypes = [C.c_int64, C.c_void_p, C.c_void_p]
+    lib.rh_mul_mat.argtypes = [TP, TP, TP, C.c_int, f64p]
+    lib.rh_rms_norm.argtypes = [TP, TP, C.c_float, C.c_int, f64p]
+    lib.rh_rope.argtypes = [TP, i32p, f32p, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [C.c_int, f64p]
+    lib.rh_soft_max.argtypes = [TP, TP, f32p, TP, C.c_float, C.c_float, C.c_int, f64p]
+    lib.rh_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, C.c_int, f64p]
+    assert lib.rh_use_device(b"CPU", min(8, os.cpu_count() or 1), 0) == 0
+    _ref = lib
+    return lib
+
+
+# ------------------------------------------------------------------- seeded test data
+def rng(*key):
+    """A generator seeded by a readable key, e.g. rng("cfg1", "q")."""
+    import zlib
+    return np.random.default_rng(zlib.crc32("/".join(str(k) for k in key).encode()))
+
+
+def quantize_q8_0(w):
+    """Q8_0 rows (uint8, 34 bytes per 32 weights) with the oracle's weight quantizer."""
+    lib = load_oracle()
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    k = w.shape[-1]
+    out = np.empty(w.shape[:-1] + (k // QK8_0 * Q8_BLOCK_BYTES,), dtype=np.uint8)
+    lib.orc_quantize_row_q8_0_ref(ptr(w, C.c_float), out.ctypes.data, w.size)
+    return out
+
+
+def nmse(a, b):
+    a = np.asarray(a, dtype=np.float64).ravel()
+    b = np.asarray(b, dtype=np.float64).ravel()
+    return float(((a - b) ** 2).sum() / max((a ** 2).sum(), 1e-300))
