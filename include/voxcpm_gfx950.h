@@ -1,0 +1,148 @@
+/*
+ * voxcpm_gfx950.h -- C ABI of the MI355X (gfx950) kernels behind VoxCPM.cpp's attention
+ * hot path.  One shared library, libvoxcpm_gfx950.so; plain pointers and sizes only.
+ *
+ * Each vx_<op> entry point computes exactly one ggml operator with ggml's semantics, so a
+ * ggml backend's graph_compute can forward a node to it unchanged: the ggml backend plugin
+ * in this repository (libggml-gfx950.so) is that caller, and the entry points below are
+ * what its dispatch switch binds -- the counterpart, for this path, of the per-op
+ * functions ggml-cpu reaches from ggml_compute_forward()
+ * (third_party/ggml/src/ggml-cpu/ggml-cpu.c:1680-2089 in the reference).
+ *
+ * Tensors are described as ggml describes them: ne[0] is the fastest dimension, nb[] are
+ * byte strides, `data` is a DEVICE pointer.  Types use ggml's numbering.  Every op
+ * validates shapes, types and strides on the host before launching anything and returns a
+ * vx_status; nothing here falls back to the CPU.
+ *
+ * Streams: `stream` is a hipStream_t passed as void* (NULL = the null stream).  All work
+ * is enqueued asynchronously on it.  Ops that need scratch memory take it from a
+ * per-stream workspace the library grows on demand with hipMalloc.
+ */
+#ifndef VOXCPM_GFX950_H
+#define VOXCPM_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VX_API __attribute__((visibility("default")))
+
+/* enum ggml_type values (third_party/ggml/include/ggml.h:389-431) */
+enum vx_type { VX_TYPE_F32 = 0, VX_TYPE_F16 = 1, VX_TYPE_Q8_0 = 8, VX_TYPE_I32 = 26 };
+
+typedef enum vx_status {
+    VX_OK = 0,
+    VX_ERR_NO_DEVICE = 1,   /* no gfx950 device / HIP runtime unusable */
+    VX_ERR_UNSUPPORTED = 2, /* shape / type / stride combination this build does not claim */
+    VX_ERR_INVALID = 3,     /* arguments violate the operator's contract */
+    VX_ERR_HIP = 4,         /* a HIP call failed; see vx_last_error() */
+    VX_ERR_ALLOC = 5
+} vx_status;
+
+/* struct ggml_tensor's {type, ne, nb, data} (third_party/ggml/include/ggml.h:655-691) */
+typedef struct vx_tensor {
+    int32_t  type;
+    int32_t  _pad;
+    int64_t  ne[4];
+    uint64_t nb[4];
+    void *   data;
+} vx_tensor;
+
+typedef void * vx_stream;
+
+/* ---- runtime --------------------------------------------------------------------------
+ * Replaces what ggml_backend_reg/device/buffer entries need from a device runtime
+ * (third_party/ggml/src/ggml-backend-impl.h:17-58, 140-182): count devices, describe
+ * them, allocate, copy, fill, synchronise. */
+VX_API int          vx_device_count(void);                 /* gfx950 devices visible; 0 if none */
+VX_API vx_status    vx_init(int device);                   /* make `device` current for this thread */
+VX_API const char * vx_last_error(void);                   /* thread-local message of the last failure */
+VX_API vx_status    vx_device_info(int device, char * name, size_t name_len,
+                                   size_t * free_bytes, size_t * total_bytes, int * compute_units);
+VX_API vx_status    vx_malloc(void ** ptr, size_t bytes);
+VX_API vx_status    vx_free(void * ptr);
+VX_API vx_status    vx_malloc_host(void ** ptr, size_t bytes);   /* pinned host memory */
+VX_API vx_status    vx_free_host(void * ptr);
+VX_API vx_status    vx_memcpy_h2d(void * dst, const void * src, size_t bytes, vx_stream stream);
+VX_API vx_status    vx_memcpy_d2h(void * dst, const void * src, size_t bytes, vx_stream stream);
+VX_API vx_status    vx_memcpy_d2d(void * dst, const void * src, size_t bytes, vx_stream stream);
+VX_API vx_status    vx_memset(void * dst, int value, size_t bytes, vx_stream stream);
+VX_API vx_status    vx_stream_create(vx_stream * stream);
+VX_API vx_status    vx_stream_destroy(vx_stream stream);
+VX_API vx_status    vx_stream_synchronize(vx_stream stream);
+
+/* ---- GGML_OP_RMS_NORM -------------------------------------------------------------------
+ * replaces ggml_compute_forward_rms_norm (ggml/src/ggml-cpu/ops.cpp:3710-3777).
+ * src, dst F32, same shape, ne[0] dense; rows may be strided; dst may alias src. */
+VX_API vx_status vx_rms_norm(const vx_tensor * src, const vx_tensor * dst, float eps, vx_stream stream);
+
+/* ---- GGML_OP_ROPE ------------------------------------------------------------------------
+ * replaces ggml_compute_forward_rope (ggml/src/ggml-cpu/ops.cpp:5589-5882) for F32 tensors,
+ * mode 0 (NORMAL) and 2 (NEOX); argument meaning as ggml_rope_ext
+ * (ggml/include/ggml.h:1767-1781).  pos: device int32[ne2]; freq_factors: device
+ * float[>= n_dims/2] or NULL; dst may alias src. */
+VX_API vx_status vx_rope(const vx_tensor * src, const int32_t * pos, const float * freq_factors,
+                         const vx_tensor * dst, int n_dims, int mode, int n_ctx_orig,
+                         float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                         float beta_fast, float beta_slow, vx_stream stream);
+
+/* ---- GGML_OP_SOFT_MAX ----------------------------------------------------------------------
+ * replaces ggml_compute_forward_soft_max (ggml/src/ggml-cpu/ops.cpp:5225-5353):
+ * dst = softmax(scale*src + slope(head)*mask) with optional sinks.  src F32; mask F16|F32
+ * [ne0, >=ne1, ne2 | 1.., ne3 | 1..] or NULL; sinks device float[ne2] or NULL; dst F32
+ * contiguous, may alias src. */
+VX_API vx_status vx_soft_max(const vx_tensor * src, const vx_tensor * mask, const float * sinks,
+                             const vx_tensor * dst, float scale, float max_bias, vx_stream stream);
+
+/* ---- GGML_OP_FLASH_ATTN_EXT ----------------------------------------------------------------
+ * replaces ggml_compute_forward_flash_attn_ext (ggml/src/ggml-cpu/ops.cpp:8109-8853).
+ * q [D, n_q, Hq, ne3] F32; k [D, n_kv, Hkv, ne3'] F16|F32; v like k; mask [n_kv, >=n_q,
+ * ne32, ne33] F16 or NULL; sinks device float[Hq] or NULL; dst [D, Hq, n_q, ne3] F32
+ * contiguous.  D (= DK = DV) in {64, 128}.  Row strides are free (permuted views and
+ * KV-cache views are fine); the innermost dimension must be dense. */
+VX_API vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                   const vx_tensor * mask, const float * sinks, const vx_tensor * dst,
+                                   float scale, float max_bias, float logit_softcap,
+                                   vx_stream stream);
+
+/* ---- GGML_OP_MUL_MAT -----------------------------------------------------------------------
+ * replaces ggml_compute_forward_mul_mat (ggml/src/ggml-cpu/ggml-cpu.c:1139-1421):
+ * dst[ne01, ne11, ne12, ne13] = src0[ne00, ne01, ne02, ne03]^T x src1[ne00, ne11, ne12, ne13],
+ * src0 broadcast over dims 2,3.  src0 Q8_0 | F16 | F32 (rows dense), src1 F32, dst F32
+ * contiguous.
+ * act_mode selects how src1 enters the product for Q8_0 weights:
+ *   VX_ACT_FLOAT -- weights dequantised in registers (q*d exactly), activations as f16/f32
+ *   VX_ACT_Q8    -- activations quantised to Q8_0 blocks first, integer block dots scaled
+ *                   by d_w*d_x: the arithmetic ggml-cpu performs
+ *                   (ggml/src/ggml-cpu/arch/x86/quants.c:290-386, 1012-1078). */
+enum vx_act_mode { VX_ACT_FLOAT = 0, VX_ACT_Q8 = 1 };
+VX_API vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst,
+                            int act_mode, vx_stream stream);
+
+/* ---- supports queries ------------------------------------------------------------------------
+ * what ggml_backend_device_i::supports_op asks (ggml/src/ggml-backend-impl.h:163-164):
+ * 1 if the matching vx_<op> call would be accepted, 0 otherwise.  No device needed. */
+VX_API int vx_supports_rms_norm(const vx_tensor * src, const vx_tensor * dst);
+VX_API int vx_supports_rope(const vx_tensor * src, const vx_tensor * dst, int n_dims, int mode);
+VX_API int vx_supports_soft_max(const vx_tensor * src, const vx_tensor * mask, const vx_tensor * dst);
+VX_API int vx_supports_flash_attn_ext(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                      const vx_tensor * mask, const vx_tensor * dst);
+VX_API int vx_supports_mul_mat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
+
+/* ---- KV-cache helpers ----------------------------------------------------------------------
+ * MiniCPMKVCache's views (src/minicpm.cpp:200-236) as descriptors over one device cache
+ * tensor [head_dim, max_length, n_kv_heads] of element size `es`. */
+VX_API vx_status vx_kv_read_view(const vx_tensor * cache, int seq_len, vx_tensor * view);
+VX_API vx_status vx_kv_write_view(const vx_tensor * cache, int start, int n_tokens, vx_tensor * view);
+/* ggml_cpy(cur, write view): rows of `src` F32 [D, Hkv, n_tokens] (any strides) stored into
+ * `view` (F16 or F32), converting to the cache type with round-to-nearest-even -- what
+ * ggml-cpu's CPY does for f32 -> f16 (ggml/src/ggml-cpu/ops.cpp:47-268, 526-565). */
+VX_API vx_status vx_kv_store(const vx_tensor * src, const vx_tensor * view, vx_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

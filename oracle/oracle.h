@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-/* same numbering as enum ggml_type (ggml/include/ggml.h:383-425) */
+/* same numbering as enum ggml_type (ggml/include/ggml.h:389-431) */
 enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q8_0 = 8, ORC_I32 = 26 };
 
 typedef struct orc_tensor {

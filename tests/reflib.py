@@ -198,3 +198,124 @@ def nmse(a, b):
     a = np.asarray(a, dtype=np.float64).ravel()
     b = np.asarray(b, dtype=np.float64).ravel()
     return float(((a - b) ** 2).sum() / max((a ** 2).sum(), 1e-300))
+
+
+# --------------------------------------------------------- numpy-level op wrappers
+ORC_FA_AUTO, ORC_FA_VEC, ORC_FA_TILED, ORC_FA_SPLIT_KV = 0, 1, 2, 3
+
+
+def _as4(a):
+    return a.reshape((1,) * (4 - a.ndim) + a.shape)
+
+
+def fa_out_shape(q, v):
+    q4, v4 = _as4(q), _as4(v)
+    return (q4.shape[0], q4.shape[2], q4.shape[1], v4.shape[3])
+
+
+def oracle_fa(q, k, v, mask=None, scale=0.125, max_bias=0.0, softcap=0.0, sinks=None, path=ORC_FA_VEC, nth=1,
+              f64=False):
+    """q (ne3,Hq,n_q,D) f32, k/v (ne3',Hkv,n_kv,D) f16|f32, mask (..,>=n_q,n_kv) f16 -> (ne3,n_q,Hq,D)."""
+    lib = load_oracle()
+    out = np.zeros(fa_out_shape(q, v), np.float32)
+    md = desc(mask) if mask is not None else None
+    sp = ptr(sinks, C.c_float)
+    if f64:
+        rc = lib.orc_flash_attn_ext_f64(desc(q), desc(k), desc(v), md, sp, desc(out), scale, max_bias, softcap)
+    else:
+        rc = lib.orc_flash_attn_ext(desc(q), desc(k), desc(v), md, sp, desc(out), scale, max_bias, softcap, path, nth)
+    assert rc == 0, f"oracle flash_attn_ext rc={rc}"
+    return out
+
+
+def ref_fa(q, k, v, mask=None, scale=0.125, max_bias=0.0, softcap=0.0, sinks=None, reps=0):
+    lib = load_ref()
+    out = np.zeros(fa_out_shape(q, v), np.float32)
+    sec = (C.c_double * 2)()
+    rc = lib.rh_flash_attn_ext(desc(q), desc(k), desc(v), desc(mask) if mask is not None else None,
+                               ptr(sinks, C.c_float), desc(out), scale, max_bias, softcap, reps, sec)
+    assert rc == 0, f"reference flash_attn_ext rc={rc}"
+    return (out, (sec[0], sec[1])) if reps else out
+
+
+def oracle_rms_norm(x, eps):
+    out = np.zeros(x.shape, np.float32)
+    assert load_oracle().orc_rms_norm(desc(x), desc(out), eps) == 0
+    return out
+
+
+def ref_rms_norm(x, eps):
+    out = np.zeros(x.shape, np.float32)
+    assert load_ref().rh_rms_norm(desc(x), desc(out), eps, 0, None) == 0
+    return out
+
+
+def oracle_rope(x, pos, ff, n_dims, mode, n_ctx_orig=32768, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0,
+                attn_factor=1.0, beta_fast=32.0, beta_slow=1.0):
+    out = np.zeros(x.shape, np.float32)
+    rc = load_oracle().orc_rope(desc(x), ptr(pos, C.c_int32), ptr(ff, C.c_float), desc(out), n_dims, mode,
+                                n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow)
+    assert rc == 0, rc
+    return out
+
+
+def ref_rope(x, pos, ff, n_dims, mode, n_ctx_orig=32768, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0,
+             attn_factor=1.0, beta_fast=32.0, beta_slow=1.0):
+    out = np.zeros(x.shape, np.float32)
+    rc = load_ref().rh_rope(desc(x), ptr(pos, C.c_int32), ptr(ff, C.c_float), desc(out), n_dims, mode, n_ctx_orig,
+                            freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, 0, None)
+    assert rc == 0, rc
+    return out
+
+
+def oracle_soft_max(x, mask, scale, max_bias, sinks=None):
+    out = np.zeros(x.shape, np.float32)
+    rc = load_oracle().orc_soft_max(desc(x), desc(mask) if mask is not None else None, ptr(sinks, C.c_float),
+                                    desc(out), scale, max_bias)
+    assert rc == 0, rc
+    return out
+
+
+def ref_soft_max(x, mask, scale, max_bias, sinks=None):
+    out = np.zeros(x.shape, np.float32)
+    rc = load_ref().rh_soft_max(desc(x), desc(mask) if mask is not None else None, ptr(sinks, C.c_float),
+                                desc(out), scale, max_bias, 0, None)
+    assert rc == 0, rc
+    return out
+
+
+def _w_desc(w, k):
+    return desc_q8(w, k) if w.dtype == np.uint8 else desc(w)
+
+
+def mm_out(w, x, k):
+    wd = _w_desc(w, k)
+    return np.zeros(tuple(x.shape[:-1]) + (wd.ne[1],), np.float32)
+
+
+def oracle_mul_mat(w, x, k=None, act_mode=0, f64=False):
+    """w: f16/f32 (.., rows, K) or Q8_0 bytes with k=K; x (.., tokens, K) f32 -> (.., tokens, rows)."""
+    k = x.shape[-1] if k is None else k
+    out = mm_out(w, x, k)
+    lib = load_oracle()
+    rc = lib.orc_mul_mat_f64(_w_desc(w, k), desc(x), desc(out)) if f64 else \
+        lib.orc_mul_mat(_w_desc(w, k), desc(x), desc(out), act_mode)
+    assert rc == 0, rc
+    return out
+
+
+def ref_mul_mat(w, x, k=None, reps=0):
+    k = x.shape[-1] if k is None else k
+    out = mm_out(w, x, k)
+    sec = (C.c_double * 2)()
+    rc = load_ref().rh_mul_mat(_w_desc(w, k), desc(x), desc(out), reps, sec)
+    assert rc == 0, rc
+    return (out, (sec[0], sec[1])) if reps else out
+
+
+def causal_mask(n_q, n_kv, n_past=0):
+    """create_causal_mask of the reference for query positions n_past..n_past+n_q-1."""
+    pos = np.arange(n_past, n_past + n_q, dtype=np.int32)
+    m = np.empty((n_q, n_kv), np.uint16)
+    load_oracle().orc_causal_mask(ptr(pos, C.c_int32), n_q, n_kv, ptr(m, C.c_uint16))
+    return m.view(np.float16)

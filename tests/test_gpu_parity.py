@@ -1,0 +1,402 @@
+"""GPU parity: every claimed ggml op, called through the C ABI of libvoxcpm_gfx950.so on
+cuda:0, against the CPU oracle (oracle/liboracle.so) on the same seeded inputs -- and, where
+the reference's own ggml-cpu was prebuilt (oracle/_ref), against that as well.
+
+Tolerances.  Attention: 2e-3 max-abs against the fp32-accumulating ggml-cpu arithmetic
+(K/V handed to the oracle as F32 tensors holding the f16 cache values), the bar the task
+states.  MUL_MAT: VX_ACT_Q8 reproduces ggml-cpu's integer block dots, so it is held to
+1e-5 relative; VX_ACT_FLOAT (weights dequantised exactly, activations as f16) is held to
+ggml's own backend-test bar, NMSE <= 5e-4 against ggml-cpu, and to 1e-5 NMSE against the
+fp64 dequantise-then-multiply reference.  RMS_NORM / ROPE / SOFT_MAX: 1e-5 max-abs or better.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import reflib
+from reflib import nmse, rng
+
+pytestmark = pytest.mark.gpu
+
+FA_TOL = 2e-3
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def sync_np(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+# ------------------------------------------------------------------------------ RMS_NORM
+@pytest.mark.parametrize("shape", [(1, 1024), (2, 1024), (512, 1024), (3, 5, 64), (7, 1025), (2, 3, 4, 4096), (5, 10000)])
+@pytest.mark.parametrize("eps", [1e-5, 0.0, 0.1])
+def test_rms_norm(gpu, shape, eps):
+    say(f"rms_norm shape={shape} eps={eps}")
+    x = rng("rms", shape).standard_normal(shape).astype(np.float32)
+    want = reflib.oracle_rms_norm(x, eps)
+    got = sync_np(gpu.rms_norm(dev(x), eps))
+    assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+    # scale invariance: rms_norm(c*x) == rms_norm(x) when eps is negligible
+    if eps == 0.0:
+        got2 = sync_np(gpu.rms_norm(dev(x * np.float32(8.0)), eps))
+        assert np.abs(got2 - got).max() <= 1e-6
+
+
+def test_rms_norm_strided_and_inplace(gpu):
+    import torch
+    say("rms_norm strided view + in place")
+    base = rng("rms", "strided").standard_normal((6, 2048)).astype(np.float32)
+    xv = base[:, :1024]  # row stride 2048 floats
+    want = reflib.oracle_rms_norm(np.ascontiguousarray(xv), 1e-5)
+    t = dev(base)
+    view = t[:, :1024]
+    got = sync_np(gpu.rms_norm(view, 1e-5, out=torch.empty((6, 1024), device="cuda")))
+    assert np.abs(got - want).max() <= 1e-6
+    gpu.rms_norm(view, 1e-5, out=view)  # in place on the strided view
+    after = sync_np(t)
+    assert np.abs(after[:, :1024] - want).max() <= 1e-6
+    assert np.array_equal(after[:, 1024:], base[:, 1024:])  # neighbours untouched
+
+
+# ---------------------------------------------------------------------------------- ROPE
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("case", ["decode", "prefill", "long", "partial", "yarn"])
+def test_rope(gpu, mode, case):
+    say(f"rope mode={mode} case={case}")
+    if case == "decode":
+        shape, pos = (2, 1, 16, 64), np.array([4095], np.int32)
+    elif case == "prefill":
+        shape, pos = (1, 256, 16, 64), np.arange(256, dtype=np.int32)
+    elif case == "long":
+        shape, pos = (1, 64, 2, 64), np.arange(8192 - 64, 8192, dtype=np.int32)
+    elif case == "partial":
+        shape, pos = (1, 9, 3, 80), np.arange(9, dtype=np.int32) * 37
+    else:
+        shape, pos = (1, 33, 4, 128), np.arange(33, dtype=np.int32) * 301
+    x = rng("rope", case, mode).standard_normal(shape).astype(np.float32)
+    n_dims = 64 if case in ("decode", "prefill", "long", "partial") else 128
+    ff = (1.0 + rng("rope", "ff").random(n_dims // 2)).astype(np.float32) if case != "partial" else None
+    kw = dict(n_ctx_orig=32768, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
+              beta_fast=32.0, beta_slow=1.0)
+    if case == "yarn":
+        kw.update(freq_scale=0.25, ext_factor=1.0, attn_factor=1.3, n_ctx_orig=4096)
+    want = reflib.oracle_rope(x, pos, ff, n_dims, mode, **kw)
+    got = sync_np(gpu.rope_ext(dev(x), dev(pos), None if ff is None else dev(ff), n_dims, mode, kw["n_ctx_orig"],
+                               kw["freq_base"], kw["freq_scale"], kw["ext_factor"], kw["attn_factor"],
+                               kw["beta_fast"], kw["beta_slow"]))
+    err = np.abs(got - want).max()
+    say(f"   max-abs {err:.3e}")
+    # only sinf/cosf differ from the host libm (the angle chain is replayed exactly)
+    assert err <= 2e-5
+    # each rotated pair keeps its norm (times attn_factor)
+    if case == "prefill":
+        h = n_dims // 2
+        pairs_in = x[..., :h] ** 2 + x[..., h:] ** 2 if mode == 2 else x[..., 0::2] ** 2 + x[..., 1::2] ** 2
+        pairs_out = got[..., :h] ** 2 + got[..., h:] ** 2 if mode == 2 else got[..., 0::2] ** 2 + got[..., 1::2] ** 2
+        assert np.allclose(pairs_in, pairs_out, rtol=1e-4, atol=1e-5)
+
+
+def test_rope_inplace_pos0(gpu):
+    say("rope in place, position 0 is the identity")
+    x = rng("rope", "id").standard_normal((1, 3, 16, 64)).astype(np.float32)
+    t = dev(x)
+    gpu.rope_ext(t, dev(np.zeros(3, np.int32)), None, 64, 2, 32768, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, out=t)
+    assert np.array_equal(sync_np(t), x)
+
+
+# ------------------------------------------------------------------------------ SOFT_MAX
+@pytest.mark.parametrize("ncols", [7, 64, 1000, 8192, 20000])
+@pytest.mark.parametrize("mask_type", [None, np.float16, np.float32])
+def test_soft_max(gpu, ncols, mask_type):
+    say(f"soft_max ncols={ncols} mask={mask_type}")
+    x = rng("sm", ncols).standard_normal((2, 4, 5, ncols)).astype(np.float32)
+    mask = None if mask_type is None else rng("sm", "m", ncols).standard_normal((1, 1, 5, ncols)).astype(mask_type)
+    max_bias = 8.0 if mask is not None else 0.0
+    sinks = rng("sm", "sinks").standard_normal(4).astype(np.float32) if ncols == 64 else None
+    want = reflib.oracle_soft_max(x, mask, 0.3, max_bias, sinks)
+    got = sync_np(gpu.soft_max_ext(dev(x), None if mask is None else dev(mask), 0.3, max_bias,
+                                   None if sinks is None else dev(sinks)))
+    assert np.abs(got - want).max() <= 1e-6
+    if sinks is None:
+        assert np.allclose(got.sum(-1), 1.0, atol=1e-5)
+
+
+# ------------------------------------------------------------------------ FLASH_ATTN_EXT
+def fa_case(gpu, q, k, v, mask=None, scale=0.125, max_bias=0.0, softcap=0.0, sinks=None, tol=FA_TOL, name=""):
+    """q, k, v, mask: numpy arrays (possibly strided views).  Returns the max-abs error."""
+    import torch
+    kf = np.ascontiguousarray(k).astype(np.float32)
+    vf = np.ascontiguousarray(v).astype(np.float32)
+    want = reflib.oracle_fa(np.ascontiguousarray(q), kf, vf, mask, scale, max_bias, softcap, sinks,
+                            path=reflib.ORC_FA_VEC)
+
+    def same_view(a):  # device tensor with the same shape and strides as the numpy view
+        base = a
+        while base.base is not None and isinstance(base.base, np.ndarray):
+            base = base.base
+        tb = torch.from_numpy(base).cuda()
+        off = (a.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // a.itemsize
+        return torch.as_strided(tb.view(-1), a.shape, [s // a.itemsize for s in a.strides], off)
+
+    got = sync_np(gpu.flash_attn_ext(same_view(q), same_view(k), same_view(v), None if mask is None else dev(mask),
+                                     scale, max_bias, softcap, None if sinks is None else dev(sinks)))
+    err = float(np.abs(got - want).max())
+    say(f"   {name} max-abs vs oracle(fp32 acc) {err:.3e}")
+    assert np.isfinite(got).all()
+    assert err <= tol, (name, err)
+    return got, want
+
+
+def qkv(tag, B, Hq, Hkv, n_q, n_kv, D=64, kv_dtype=np.float16):
+    q = rng(tag, "q").standard_normal((B, Hq, n_q, D)).astype(np.float32)
+    k = rng(tag, "k").standard_normal((B, Hkv, n_kv, D)).astype(kv_dtype)
+    v = rng(tag, "v").standard_normal((B, Hkv, n_kv, D)).astype(kv_dtype)
+    return q, k, v
+
+
+def test_fa_cfg1_prefill_causal(gpu):
+    say("flash_attn cfg1: T=KV=256, 16/2 heads, D=64, f16 KV, causal mask")
+    q, k, v = qkv("cfg1", 1, 16, 2, 256, 256)
+    got, want = fa_case(gpu, q, k, v, reflib.causal_mask(256, 256), name="cfg1")
+    if reflib.load_ref() is not None:
+        r = reflib.ref_fa(q, k, v, reflib.causal_mask(256, 256))  # ggml-cpu tiled path (fp32)
+        e = float(np.abs(got - r).max())
+        say(f"   vs ggml-cpu (reference build) {e:.3e}")
+        assert e <= FA_TOL
+
+
+@pytest.mark.parametrize("L", [128, 512, 2048, 4096])
+def test_fa_cfg2_decode(gpu, L):
+    say(f"flash_attn cfg2 decode: B=2, 16/2 heads, D=64, f16 KV, L={L}")
+    q, k, v = qkv(("cfg2", L), 2, 16, 2, 1, L)
+    got, want = fa_case(gpu, q, k, v, None, name=f"decode L={L}")
+    f64 = reflib.oracle_fa(q, k, v, f64=True)
+    say(f"   vs fp64 brute force {np.abs(got - f64).max():.3e}")
+    if reflib.load_ref() is not None:
+        r16 = reflib.ref_fa(q, k, v)  # ggml-cpu with F16-typed K/V: accumulates in f16
+        say(f"   raw diff vs ggml-cpu F16-typed path {np.abs(got - r16).max():.3e} "
+            f"(that path itself is {np.abs(r16 - f64).max():.3e} from fp64)")
+        r32 = reflib.ref_fa(q, k.astype(np.float32), v.astype(np.float32))
+        assert np.abs(got - r32).max() <= FA_TOL
+
+
+def test_fa_cfg3_locdit_cfg_pair(gpu):
+    say("flash_attn cfg3 LocDiT: 8 requests x CFG pair of 7 tokens, 16/2 heads, block-diagonal mask")
+    import ctypes as C
+    L = 7
+    pos = np.zeros(2 * L, np.int32)
+    m = np.zeros((2 * L, 2 * L), np.uint16)
+    reflib.load_oracle().orc_cfg_pair_constants(L, reflib.ptr(pos, C.c_int32), reflib.ptr(m, C.c_uint16))
+    mask = m.view(np.float16)
+    q, k, v = qkv("cfg3", 8, 16, 2, 2 * L, 2 * L, kv_dtype=np.float32)  # LocDiT K/V are F32 activations
+    got, _ = fa_case(gpu, q, k, v, mask, name="locdit pair")
+    # the pair equals two independent 7-token attentions
+    for br in range(2):
+        sl = slice(br * L, (br + 1) * L)
+        solo = reflib.oracle_fa(np.ascontiguousarray(q[:, :, sl]), np.ascontiguousarray(k[:, :, sl]),
+                                np.ascontiguousarray(v[:, :, sl]), None)
+        assert np.abs(got[:, sl] - solo).max() <= FA_TOL
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(5, 5), (1, 1), (3, 113), (16, 512), (35, 1024), (75, 113), (2, 33)])
+@pytest.mark.parametrize("masked", [False, True])
+def test_fa_ragged(gpu, n_q, n_kv, masked):
+    say(f"flash_attn ragged n_q={n_q} n_kv={n_kv} mask={masked}")
+    q, k, v = qkv(("rag", n_q, n_kv), 3, 8, 2, n_q, n_kv)
+    mask = None
+    if masked:
+        mm = rng("rag", "m", n_q, n_kv).standard_normal((1, 1, n_q, n_kv)).astype(np.float32)
+        mm[rng("rag", "d", n_q, n_kv).random(mm.shape) < 0.3] = -np.inf
+        mask = mm.astype(np.float16)
+    fa_case(gpu, q, k, v, mask, name="ragged")
+
+
+def test_fa_special_cases(gpu):
+    say("flash_attn special cases: n_kv=1 -> out = v; equal keys -> mean(V); fully masked row -> 0")
+    q, k, v = qkv("sp1", 1, 16, 2, 4, 1)
+    got, _ = fa_case(gpu, q, k, v, None, name="n_kv=1")
+    for h in range(16):
+        assert np.abs(got[0, :, h] - v[0, h // 8, 0].astype(np.float32)).max() <= 1e-6
+    q, k, v = qkv("sp2", 1, 16, 2, 3, 200)
+    k[:] = k[:, :, :1]
+    got, _ = fa_case(gpu, q, k, v, None, name="equal keys")
+    mean_v = v.astype(np.float32).mean(axis=2)  # (1, Hkv, D)
+    for h in range(16):
+        assert np.abs(got[0, :, h] - mean_v[0, h // 8]).max() <= 1e-4
+    q, k, v = qkv("sp3", 2, 16, 2, 6, 70)
+    mask = np.zeros((1, 1, 6, 70), np.float16)
+    mask[0, 0, 2, :] = -np.inf
+    mask[0, 0, 4, 10:] = -np.inf
+    got, _ = fa_case(gpu, q, k, v, mask, name="masked rows")
+    assert np.array_equal(got[:, 2], np.zeros_like(got[:, 2]))
+    # permuting the keys leaves the result unchanged
+    perm = rng("sp4").permutation(70)
+    got2, _ = fa_case(gpu, q, np.ascontiguousarray(k[:, :, perm]), np.ascontiguousarray(v[:, :, perm]),
+                      np.ascontiguousarray(mask[..., perm]), name="permuted keys")
+    assert np.abs(got - got2).max() <= 1e-5
+
+
+def test_fa_graph_views(gpu):
+    say("flash_attn on the strided views attention_forward builds: q/k/v permuted [D,T,H], KV-cache read view")
+    T, Hq, Hkv, D, maxlen = 40, 16, 2, 64, 96
+    qb = rng("views", "q").standard_normal((1, T, Hq, D)).astype(np.float32)    # [D, Hq, T] as produced by MUL_MAT
+    q = qb.transpose(0, 2, 1, 3)                                                 # ggml_permute(q, 0, 2, 1, 3)
+    cache_k = rng("views", "k").standard_normal((1, Hkv, maxlen, D)).astype(np.float16)
+    cache_v = rng("views", "v").standard_normal((1, Hkv, maxlen, D)).astype(np.float16)
+    k, v = cache_k[:, :, :T], cache_v[:, :, :T]                                  # get_k/get_v(seq_len = T)
+    fa_case(gpu, q, k, v, reflib.causal_mask(T, T), name="views")
+
+
+@pytest.mark.parametrize("kv_dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("D", [64, 128])
+def test_fa_dtypes_and_head_sizes(gpu, kv_dtype, D):
+    say(f"flash_attn D={D} kv={kv_dtype.__name__}")
+    q, k, v = qkv(("dt", D, kv_dtype.__name__), 2, 8, 2, 9, 300, D=D, kv_dtype=kv_dtype)
+    fa_case(gpu, q, k, v, reflib.causal_mask(9, 300, n_past=291), scale=1.0 / np.sqrt(D), name="dtype")
+
+
+def test_fa_sinks_softcap_alibi(gpu):
+    say("flash_attn with sinks, logit soft cap and ALiBi slopes")
+    q, k, v = qkv("ext", 2, 12, 4, 4, 150)
+    mask = rng("ext", "m").standard_normal((1, 1, 4, 150)).astype(np.float16)
+    sinks = rng("ext", "s").standard_normal(12).astype(np.float32)
+    fa_case(gpu, q, k, v, mask, max_bias=8.0, name="alibi")
+    fa_case(gpu, q, k, v, mask, softcap=10.0, name="softcap")
+    fa_case(gpu, q, k, v, mask, sinks=sinks, name="sinks")
+    q, k, v = qkv("ext2", 1, 12, 4, 1, 2000)
+    fa_case(gpu, q, k, v, None, sinks=sinks, name="sinks + split")
+
+
+def test_fa_cfg5_shape_properties(gpu):
+    """BASELINE config 5 decode shape (batch 16, L = 8192): too big for the scalar oracle in
+    seconds, so check a sample of (batch, head) slices against it plus convexity everywhere."""
+    import torch
+    say("flash_attn cfg5 decode shape: B=16, L=8192, 16/2 heads")
+    B, L = 16, 8192
+    q, k, v = qkv("cfg5", B, 16, 2, 1, L)
+    got = sync_np(gpu.flash_attn_ext(dev(q), dev(k), dev(v), None, 0.125))
+    assert np.isfinite(got).all()
+    vmin = v.astype(np.float32).min(axis=2)  # (B, Hkv, D)
+    vmax = v.astype(np.float32).max(axis=2)
+    for h in range(16):
+        assert (got[:, 0, h] >= vmin[:, h // 8] - 1e-5).all() and (got[:, 0, h] <= vmax[:, h // 8] + 1e-5).all()
+    for b in (0, 7, 15):
+        want = reflib.oracle_fa(q[b:b + 1], k[b:b + 1].astype(np.float32), v[b:b + 1].astype(np.float32))
+        err = np.abs(got[b:b + 1] - want).max()
+        say(f"   batch {b}: max-abs {err:.3e}")
+        assert err <= FA_TOL
+
+
+# ------------------------------------------------------------------------------- MUL_MAT
+def mm_inputs(tag, M, K, N, batch=()):
+    w = (rng(tag, "w").standard_normal(batch + (M, K)) * 0.02).astype(np.float32)
+    x = rng(tag, "x").standard_normal(batch + (N, K)).astype(np.float32)
+    return w, x
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 1), (1024, 1024, 2), (128, 1024, 2), (4096, 1024, 2), (1024, 4096, 2),
+                                   (1024, 1024, 5), (1024, 1024, 16), (1024, 1024, 17), (1000, 1024, 33),
+                                   (3072, 1024, 112), (1024, 1024, 512), (70, 96, 130)])
+def test_mul_mat_q8_0(gpu, M, K, N):
+    say(f"mul_mat Q8_0 M={M} K={K} N={N}")
+    w, x = mm_inputs(("q8", M, K, N), M, K, N)
+    wq = reflib.quantize_q8_0(w)
+    cpu = reflib.oracle_mul_mat(wq, x, K, act_mode=0)          # ggml-cpu arithmetic (int8 x int8)
+    f64 = reflib.oracle_mul_mat(wq, x, K, f64=True)            # dequantise, multiply in fp64
+    got_q8 = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_Q8, w_ne0=K))
+    got_fl = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_FLOAT, w_ne0=K))
+    scale = np.abs(cpu).max()
+    e_q8 = np.abs(got_q8 - cpu).max() / scale
+    say(f"   ACT_Q8 vs ggml-cpu arithmetic: rel max {e_q8:.3e};  ACT_FLOAT: nmse vs cpu {nmse(cpu, got_fl):.3e}, "
+        f"vs fp64 dequant {nmse(f64, got_fl):.3e}")
+    assert e_q8 <= 1e-5
+    assert nmse(cpu, got_fl) <= 5e-4
+    assert nmse(f64, got_fl) <= 1e-5
+
+
+@pytest.mark.parametrize("wtype", [np.float16, np.float32])
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300)])
+def test_mul_mat_float_weights(gpu, wtype, M, K, N):
+    say(f"mul_mat {wtype.__name__} weights M={M} K={K} N={N}")
+    w, x = mm_inputs(("fw", M, K, N), M, K, N)
+    w = w.astype(wtype)
+    cpu = reflib.oracle_mul_mat(w, x, act_mode=0)
+    f64 = reflib.oracle_mul_mat(w, x, f64=True)
+    got = sync_np(gpu.mul_mat(dev(w), dev(x)))
+    say(f"   nmse vs ggml-cpu arithmetic {nmse(cpu, got):.3e}, vs fp64 {nmse(f64, got):.3e}")
+    assert nmse(cpu, got) <= 1e-6
+    assert nmse(f64, got) <= 1e-6
+
+
+def test_mul_mat_broadcast_and_views(gpu):
+    say("mul_mat batch broadcast (ne12 = 4 over ne02 = 2) and a QKV row-slice view")
+    w, _ = mm_inputs("bc", 96, 128, 1, batch=(1, 2))
+    x = rng("bc", "x").standard_normal((1, 4, 9, 128)).astype(np.float32)
+    wq = reflib.quantize_q8_0(w)
+    cpu = reflib.oracle_mul_mat(wq, x, 128, act_mode=0)
+    got = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_Q8, w_ne0=128))
+    assert np.abs(got - cpu).max() <= 1e-5 * np.abs(cpu).max()
+
+
+def test_q8_0_dequant_is_exact(gpu):
+    """x = unit vectors: the ACT_FLOAT product then *is* the dequantised weight, which must equal
+    ggml's dequantize_row_q8_0 bit for bit."""
+    import ctypes as C
+    say("Q8_0 dequantisation exact: W x I == dequantize_row_q8_0(W)")
+    K, M = 256, 80
+    w = (rng("deq", "w").standard_normal((M, K)) * 0.05).astype(np.float32)
+    wq = reflib.quantize_q8_0(w)
+    deq = np.zeros((M, K), np.float32)
+    reflib.load_oracle().orc_dequantize_row_q8_0(wq.ctypes.data, reflib.ptr(deq, C.c_float), M * K)
+    eye = np.eye(K, dtype=np.float32)
+    got = sync_np(gpu.mul_mat(dev(wq), dev(eye), gpu.ACT_FLOAT, w_ne0=K))  # (K tokens, M rows)
+    assert np.array_equal(got.T, deq)
+
+
+# ------------------------------------------------------------------------------ KV cache
+@pytest.mark.parametrize("cache_dtype", [np.float16, np.float32])
+def test_kv_cache_views_and_store(gpu, cache_dtype):
+    import ctypes as C
+    import torch
+    say(f"kv cache views + store, cache {cache_dtype.__name__}")
+    D, maxlen, Hkv = 64, 48, 2
+    es = np.dtype(cache_dtype).itemsize
+    orc = reflib.load_oracle()
+    cache = torch.zeros((Hkv, maxlen, D), dtype=torch.float16 if es == 2 else torch.float32, device="cuda")
+    cd = gpu.desc(cache)
+    host = np.zeros((Hkv, maxlen, D), cache_dtype)
+    start = 0
+    for n_tok in (5, 1, 1, 7):
+        cur = rng("kv", start).standard_normal((n_tok, Hkv, D)).astype(np.float32)  # [D, Hkv, n_tokens]
+        wv = gpu.VxTensor()
+        gpu.check(gpu.lib().vx_kv_write_view(cd, start, n_tok, wv), "kv_write_view")
+        ne, nb, off = (C.c_int64 * 3)(), (C.c_uint64 * 3)(), C.c_uint64()
+        orc.orc_kv_write_view(D, maxlen, Hkv, es, start, n_tok, ne, nb, C.byref(off))
+        assert [wv.ne[i] for i in range(3)] == list(ne) and [wv.nb[i] for i in range(3)] == list(nb)
+        assert wv.data - cache.data_ptr() == off.value
+        gpu.check(gpu.lib().vx_kv_store(gpu.desc(dev(cur)), wv, torch.cuda.current_stream().cuda_stream), "kv_store")
+        host[:, start:start + n_tok] = cur.transpose(1, 0, 2).astype(cache_dtype)
+        start += n_tok
+        rv = gpu.VxTensor()
+        gpu.check(gpu.lib().vx_kv_read_view(cd, start, rv), "kv_read_view")
+        orc.orc_kv_read_view(D, maxlen, Hkv, es, start, ne, nb, C.byref(off))
+        assert [rv.ne[i] for i in range(3)] == list(ne) and [rv.nb[i] for i in range(3)] == list(nb) and off.value == 0
+    got = sync_np(cache)
+    assert np.array_equal(got.view(np.uint16 if es == 2 else np.uint32), host.view(np.uint16 if es == 2 else np.uint32))
+    # attention over the read view equals attention over the dense copy
+    q = rng("kv", "q").standard_normal((1, 16, 1, D)).astype(np.float32)
+    other = torch.from_numpy(host.copy()).cuda()
+    out = gpu.flash_attn_ext(dev(q), cache[None, :, :start], other[None, :, :start], None, 0.125)
+    want = reflib.oracle_fa(q, host[None, :, :start].astype(np.float32), host[None, :, :start].astype(np.float32))
+    assert np.abs(sync_np(out) - want).max() <= FA_TOL

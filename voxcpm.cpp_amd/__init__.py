@@ -1,0 +1,192 @@
+"""Python-side plumbing over libvoxcpm_gfx950.so (the C ABI in include/voxcpm_gfx950.h).
+
+The product is the shared library and the ggml backend plugin beside it; this package
+only loads the library with ctypes and wraps torch tensors (used purely as device memory
+and streams) into the library's tensor descriptors, for the parity tests and bench.py.
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libvoxcpm_gfx950.so")
+PLUGIN_PATH = os.path.join(LIB_DIR, "libggml-gfx950.so")
+
+F32, F16, Q8_0, I32 = 0, 1, 8, 26
+ACT_FLOAT, ACT_Q8 = 0, 1
+QK8_0, Q8_BLOCK_BYTES = 32, 34
+
+
+class VxError(RuntimeError):
+    pass
+
+
+class VxTensor(C.Structure):
+    _fields_ = [
+        ("type", C.c_int32),
+        ("_pad", C.c_int32),
+        ("ne", C.c_int64 * 4),
+        ("nb", C.c_uint64 * 4),
+        ("data", C.c_void_p),
+    ]
+
+
+EXPORTS = [
+    "vx_device_count", "vx_init", "vx_last_error", "vx_device_info", "vx_malloc", "vx_free",
+    "vx_malloc_host", "vx_free_host", "vx_memcpy_h2d", "vx_memcpy_d2h", "vx_memcpy_d2d", "vx_memset",
+    "vx_stream_create", "vx_stream_destroy", "vx_stream_synchronize",
+    "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_mul_mat",
+    "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
+    "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
+]
+
+_lib = None
+
+
+def lib():
+    """The loaded C library; raises VxError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise VxError(f"{LIB_PATH} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                      "(or make -C voxcpm.cpp_amd/csrc) first")
+    l = C.CDLL(LIB_PATH)
+    TP = C.POINTER(VxTensor)
+    vp, f32p, i32p = C.c_void_p, C.c_void_p, C.c_void_p  # device pointers travel as integers
+    l.vx_last_error.restype = C.c_char_p
+    l.vx_init.argtypes = [C.c_int]
+    l.vx_device_info.argtypes = [C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
+    l.vx_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    l.vx_free.argtypes = [vp]
+    l.vx_malloc_host.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    l.vx_free_host.argtypes = [vp]
+    for n in ("vx_memcpy_h2d", "vx_memcpy_d2h", "vx_memcpy_d2d"):
+        getattr(l, n).argtypes = [vp, vp, C.c_size_t, vp]
+    l.vx_memset.argtypes = [vp, C.c_int, C.c_size_t, vp]
+    l.vx_stream_create.argtypes = [C.POINTER(C.c_void_p)]
+    l.vx_stream_destroy.argtypes = [vp]
+    l.vx_stream_synchronize.argtypes = [vp]
+    l.vx_rms_norm.argtypes = [TP, TP, C.c_float, vp]
+    l.vx_rope.argtypes = [TP, i32p, f32p, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [vp]
+    l.vx_soft_max.argtypes = [TP, TP, f32p, TP, C.c_float, C.c_float, vp]
+    l.vx_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, vp]
+    l.vx_mul_mat.argtypes = [TP, TP, TP, C.c_int, vp]
+    l.vx_supports_rms_norm.argtypes = [TP, TP]
+    l.vx_supports_rope.argtypes = [TP, TP, C.c_int, C.c_int]
+    l.vx_supports_soft_max.argtypes = [TP, TP, TP]
+    l.vx_supports_flash_attn_ext.argtypes = [TP, TP, TP, TP, TP]
+    l.vx_supports_mul_mat.argtypes = [TP, TP, TP]
+    l.vx_kv_read_view.argtypes = [TP, C.c_int, TP]
+    l.vx_kv_write_view.argtypes = [TP, C.c_int, C.c_int, TP]
+    l.vx_kv_store.argtypes = [TP, TP, vp]
+    _lib = l
+    return l
+
+
+def check(status, what=""):
+    if status != 0:
+        raise VxError(f"{what} failed with status {status}: {lib().vx_last_error().decode()}")
+
+
+def make_desc(ttype, ne, nb, data):
+    t = VxTensor()
+    t.type = ttype
+    for i in range(4):
+        t.ne[i] = ne[i]
+        t.nb[i] = nb[i]
+    t.data = data
+    return t
+
+
+_TORCH_TYPES = None
+
+
+def desc(t):
+    """Descriptor of a torch tensor (<= 4 dims, any strides, last dim dense): numpy/torch
+    shape (n3, n2, n1, n0) becomes ggml ne = [n0, n1, n2, n3]."""
+    import torch
+    global _TORCH_TYPES
+    if _TORCH_TYPES is None:
+        _TORCH_TYPES = {torch.float32: F32, torch.float16: F16, torch.int32: I32}
+    if t is None:
+        return None
+    assert t.dim() <= 4
+    es = t.element_size()
+    shape = [1] * (4 - t.dim()) + list(t.shape)
+    strides = [s * es for s in t.stride()]
+    while len(strides) < 4:
+        strides.insert(0, (strides[0] * shape[4 - len(strides)]) if strides else es)
+    d = make_desc(_TORCH_TYPES[t.dtype], shape[::-1], strides[::-1], t.data_ptr())
+    d._keep = t
+    return d
+
+
+def desc_q8(raw, ne0):
+    """Descriptor of Q8_0 rows held in a contiguous uint8 torch tensor (..., rows, ne0/32*34)."""
+    assert raw.is_contiguous() and raw.shape[-1] == ne0 // QK8_0 * Q8_BLOCK_BYTES
+    shape = [1] * (4 - raw.dim()) + list(raw.shape)
+    rowb = shape[3]
+    d = make_desc(Q8_0, [ne0, shape[2], shape[1], shape[0]],
+                  [Q8_BLOCK_BYTES, rowb, rowb * shape[2], rowb * shape[2] * shape[1]], raw.data_ptr())
+    d._keep = raw
+    return d
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+# ---- one function per ggml operator, same argument meaning as the ggml_* graph builders ----
+def rms_norm(x, eps, out=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    check(lib().vx_rms_norm(desc(x), desc(out), eps, _stream()), "vx_rms_norm")
+    return out
+
+
+def rope_ext(x, pos, freq_factors, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor,
+             attn_factor, beta_fast, beta_slow, out=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    check(lib().vx_rope(desc(x), _p(pos), _p(freq_factors), desc(out), n_dims, mode, n_ctx_orig, freq_base,
+                        freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, _stream()), "vx_rope")
+    return out
+
+
+def soft_max_ext(x, mask, scale, max_bias, sinks=None, out=None):
+    import torch
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device) if out is None else out
+    check(lib().vx_soft_max(desc(x), desc(mask), _p(sinks), desc(out), scale, max_bias, _stream()), "vx_soft_max")
+    return out
+
+
+def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, logit_softcap=0.0, sinks=None, out=None):
+    """q (ne3, Hq, n_q, D) f32; k, v (ne3', Hkv, n_kv, D) f16|f32 (any row strides); mask
+    (ne33, ne32, >=n_q, n_kv) f16 or None.  Returns (ne3, n_q, Hq, D) f32, ggml's permuted result."""
+    import torch
+    if out is None:
+        out = torch.empty((q.shape[-4] if q.dim() == 4 else 1, q.shape[-2], q.shape[-3], v.shape[-1]),
+                          dtype=torch.float32, device=q.device)
+    check(lib().vx_flash_attn_ext(desc(q), desc(k), desc(v), desc(mask), _p(sinks), desc(out), scale, max_bias,
+                                  logit_softcap, _stream()), "vx_flash_attn_ext")
+    return out
+
+
+def mul_mat(w, x, act_mode=ACT_FLOAT, w_ne0=None, out=None):
+    """w: weights (ne03, ne02, rows, K) f16|f32, or Q8_0 bytes (.., rows, K/32*34) uint8 with
+    w_ne0=K; x (ne13, ne12, tokens, K) f32.  Returns (ne13, ne12, tokens, rows) f32."""
+    import torch
+    wd = desc_q8(w, w_ne0) if w.dtype == torch.uint8 else desc(w)
+    xd = desc(x)
+    if out is None:
+        shape = list(x.shape[:-1]) + [wd.ne[1]]
+        out = torch.empty(shape, dtype=torch.float32, device=x.device)
+    check(lib().vx_mul_mat(wd, xd, desc(out), act_mode, _stream()), "vx_mul_mat")
+    return out

@@ -1,0 +1,277 @@
+// mul_mat.hip -- GGML_OP_MUL_MAT on gfx950 for Q8_0 / F16 / F32 weights and F32 activations.
+//
+// dst[token][row] = sum_k x[token][k] * W[row][k], computed on the matrix cores as
+// D[m = token][n = weight row] with v_mfma_f32_16x16x32_f16.  K = 32 of that instruction is
+// exactly one Q8_0 block, so for quantised weights every MFMA yields the block's partial
+// dot product with the weights still *integers* (int8 -> f16 is exact), and the block scale
+// d is applied in fp32 afterwards: acc += d * partial.  The effective weight is q*d exactly,
+// the value ggml's dequantize_row_q8_0 produces (ggml/src/ggml-quants.c:401-415).
+//
+// Operands (lane = 16*j + c):
+//   B = W^T   lane c = weight row, k-slots 8j..8j+7 of the block: 8 bytes of a Q8_0 block
+//             (2-byte aligned) turned into f16 with one xor, two byte permutes and two
+//             packed subtracts per dword (bias trick: 0x6400|u is 1024+u in f16).
+//   A = x     lane c = token; converted to f16 once per work-group and parked in LDS in
+//             operand order, swizzled so both the staging writes and the operand reads
+//             are bank-conflict free.
+// With VX_ACT_Q8 the staging step quantises each 32-wide activation block the way
+// ggml-cpu's x86 build does (id = 127/max, round half to even, d rounded to f16;
+// ggml/src/ggml-cpu/arch/x86/quants.c:290-386): the MFMA then produces ggml-cpu's exact
+// integer block dot and the scale is d_w * d_x.
+//
+// Tiling: a work-group is 4 waves.  GEMM shape (many tokens): 64 rows x 16*TT tokens, each
+// wave 16 rows.  GEMV shape (<= 16 tokens): 16 rows, the 4 waves split K and reduce through
+// LDS, so a 1024-row projection still spreads over 64 work-groups.
+//
+// Algorithmic HBM bytes: weights once (34 bytes per 32 weights) + activations + output.
+#include "vx_common.hpp"
+
+namespace {
+
+struct mm_args {
+    const char * w; const char * x; char * dst;
+    int64_t K, M, N;
+    uint64_t nb01, nb02, nb03, nb11, nb12, nb13, nb1, nb2, nb3;
+    int ne12, r2, r3;
+    int x_aligned; // src1 rows allow 16-byte vector loads
+};
+
+constexpr int WT_Q8 = 0, WT_F16 = 1, WT_F32 = 2;
+constexpr int KC_BLOCKS = 4; // 32-wide k blocks staged per round
+
+__device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// 8 int8 (two dwords) -> 8 f16, exactly
+__device__ __forceinline__ half8_t q8_to_half8(uint32_t lo, uint32_t hi) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t bias = 0x64646464u;
+    lo ^= 0x80808080u;
+    hi ^= 0x80808080u;
+    u32x4 r;
+    r[0] = __builtin_amdgcn_perm(bias, lo, 0x04010400u);
+    r[1] = __builtin_amdgcn_perm(bias, lo, 0x04030402u);
+    r[2] = __builtin_amdgcn_perm(bias, hi, 0x04010400u);
+    r[3] = __builtin_amdgcn_perm(bias, hi, 0x04030402u);
+    half8_t h = __builtin_bit_cast(half8_t, r);
+    const _Float16 off = (_Float16) 1152.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] -= off;
+    return h;
+}
+
+__device__ __forceinline__ int lds_slot(int kbl, int tt, int TT, int j, int c) {
+    return ((kbl * TT + tt) * 4 + j) * 16 + ((c + 4 * kbl + j) & 15);
+}
+
+template <int WT, int TT, bool ACT_Q8, bool KSPLIT>
+__global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
+    __shared__ half8_t xs[KC_BLOCKS * TT * 64];
+    __shared__ float   xd[ACT_Q8 ? KC_BLOCKS * TT * 16 : 1];
+    __shared__ float4_t red[KSPLIT ? 3 * TT * 64 : 1];
+
+    const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
+    const int j = lane >> 4, c = lane & 15;
+
+    const int     batch = blockIdx.z;
+    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+
+    const int64_t tok0 = (int64_t) blockIdx.y * 16 * TT;
+    const int64_t row0 = KSPLIT ? (int64_t) blockIdx.x * 16 : (int64_t) blockIdx.x * 64 + wid * 16;
+    const int64_t row  = min(row0 + c, a.M - 1);
+    const char *  wrow = wb + (uint64_t) row * a.nb01;
+
+    float4_t acc[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[tt] = float4_t{0, 0, 0, 0};
+
+    const int64_t nkb = (a.K + 31) / 32;
+    for (int64_t kb0 = 0; kb0 < nkb; kb0 += KC_BLOCKS) {
+        // ---- stage 16*TT tokens x 128 k of activations as f16 operands
+#pragma unroll
+        for (int it = 0; it < TT; ++it) {
+            const int unit = tid + 256 * it;
+            const int t = unit >> 4, u = unit & 15; // token within tile, 8-wide k unit
+            const int kbl = u >> 2, uj = u & 3;
+            const int64_t tok = tok0 + t;
+            const int64_t k   = (kb0 + kbl) * 32 + uj * 8;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+            if (tok < a.N && k < a.K) {
+                const float * xp = (const float *) (xb + (uint64_t) tok * a.nb11) + k;
+                if (a.x_aligned && k + 8 <= a.K) {
+                    const float4_t v0 = ((const float4_t *) xp)[0], v1 = ((const float4_t *) xp)[1];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) if (k + i < a.K) v[i] = xp[i];
+                }
+            }
+            half8_t h;
+            if constexpr (ACT_Q8) {
+                float amax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                const float d  = amax / 127.f;
+                const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
+                if (uj == 0) xd[(kbl * TT + (t >> 4)) * 16 + (t & 15)] = (float) (_Float16) d;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
+            }
+            xs[lds_slot(kbl, t >> 4, TT, uj, t & 15)] = h;
+        }
+        __syncthreads();
+
+        // ---- multiply
+#pragma unroll
+        for (int kbl = 0; kbl < KC_BLOCKS; ++kbl) {
+            if (KSPLIT && kbl != wid) continue;
+            const int64_t kb = kb0 + kbl;
+            if (kb >= nkb) break;
+            half8_t bop;
+            float   dw = 1.0f;
+            if constexpr (WT == WT_Q8) {
+                const char * bp = wrow + (uint64_t) kb * VX_Q8_BLOCK;
+                dw = (float) *(const _Float16 *) bp;
+                uint32_t q2[2];
+                __builtin_memcpy(q2, bp + 2 + 8 * j, 8);
+                bop = q8_to_half8(q2[0], q2[1]);
+            } else if constexpr (WT == WT_F16) {
+                const int64_t k = kb * 32 + 8 * j;
+                if (k + 8 <= a.K) {
+                    __builtin_memcpy(&bop, wrow + (uint64_t) k * 2, 16);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) bop[i] = k + i < a.K ? ((const _Float16 *) wrow)[k + i] : (_Float16) 0.0f;
+                }
+            } else {
+                const int64_t k = kb * 32 + 8 * j;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) bop[i] = k + i < a.K ? (_Float16) ((const float *) wrow)[k + i] : (_Float16) 0.0f;
+            }
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                const half8_t aop = xs[lds_slot(kbl, tt, TT, j, c)];
+                if constexpr (WT == WT_Q8) {
+                    const float4_t blk = mfma16(aop, bop, float4_t{0, 0, 0, 0});
+                    if constexpr (ACT_Q8) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[tt][r] += blk[r] * (dw * xd[(kbl * TT + tt) * 16 + 4 * j + r]);
+                    } else {
+                        acc[tt] += blk * dw;
+                    }
+                } else {
+                    acc[tt] = mfma16(aop, bop, acc[tt]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    if constexpr (KSPLIT) {
+        if (wid > 0) {
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) red[((wid - 1) * TT + tt) * 64 + lane] = acc[tt];
+        }
+        __syncthreads();
+        if (wid > 0) return;
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int ww = 0; ww < 3; ++ww) acc[tt] += red[(ww * TT + tt) * 64 + lane];
+    }
+
+    // lane (j,c), register r: token tok0 + 16*tt + 4j + r, row row0 + c
+    if (row0 + c < a.M) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t tok = tok0 + 16 * tt + 4 * j + r;
+                if (tok < a.N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) (row0 + c) * 4) = acc[tt][r];
+            }
+    }
+}
+
+template <int WT, bool ACT_Q8>
+void launch(const mm_args & a, int nbatch, hipStream_t st) {
+    if (a.N <= 16) {
+        const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
+        mm_kernel<WT, 1, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
+    } else if (a.N <= 32) {
+        const dim3 grid((unsigned) ((a.M + 63) / 64), 1, (unsigned) nbatch);
+        mm_kernel<WT, 2, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+    } else {
+        const dim3 grid((unsigned) ((a.M + 63) / 64), (unsigned) ((a.N + 63) / 64), (unsigned) nbatch);
+        mm_kernel<WT, 4, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+    }
+}
+
+} // namespace
+
+extern "C" int vx_supports_mul_mat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst) {
+    if (!src0 || !src1 || !dst) return 0;
+    if (src0->type != VX_TYPE_Q8_0 && src0->type != VX_TYPE_F16 && src0->type != VX_TYPE_F32) return 0;
+    if (src1->type != VX_TYPE_F32 || dst->type != VX_TYPE_F32) return 0;
+    if (!vx_positive(src0) || !vx_positive(src1)) return 0;
+    if (src0->ne[0] != src1->ne[0]) return 0;
+    if (src0->type == VX_TYPE_Q8_0 && src0->ne[0] % VX_QK8_0) return 0;
+    if (src1->ne[2] % src0->ne[2] || src1->ne[3] % src0->ne[3]) return 0;
+    if (dst->ne[0] != src0->ne[1] || dst->ne[1] != src1->ne[1] || dst->ne[2] != src1->ne[2] || dst->ne[3] != src1->ne[3]) return 0;
+    if (src0->nb[0] != vx_type_size(src0->type) || src1->nb[0] != 4 || dst->nb[0] != 4) return 0;
+    // weight rows must not overlap or interleave (transposed views stay on the CPU)
+    if (src0->nb[1] < vx_row_size(src0->type, src0->ne[0])) return 0;
+    if (src0->type == VX_TYPE_F16 && (src0->nb[1] % 2 || src0->nb[2] % 2 || src0->nb[3] % 2)) return 0;
+    if (src0->type == VX_TYPE_F32 && (src0->nb[1] % 4 || src0->nb[2] % 4 || src0->nb[3] % 4)) return 0;
+    if (src1->nb[1] % 4 || src1->nb[2] % 4 || src1->nb[3] % 4) return 0;
+    if (dst->nb[1] % 4 || dst->nb[2] % 4 || dst->nb[3] % 4 || dst->nb[1] < (uint64_t) dst->ne[0] * 4) return 0;
+    if (src1->ne[2] * src1->ne[3] > 65535) return 0;
+    if ((src1->ne[1] + 63) / 64 > 65535) return 0;
+    return 1;
+}
+
+extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int act_mode,
+                                vx_stream stream) {
+    if (!src0 || !src1 || !dst || !src0->data || !src1->data || !dst->data)
+        return vx_fail(VX_ERR_INVALID, "mul_mat: null tensor");
+    if (!vx_supports_mul_mat(src0, src1, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: needs src0 Q8_0/F16/F32 with dense rows, src1 F32, dst F32, matching shapes");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat: bad act_mode");
+    if (src0->type == VX_TYPE_F16 && (uintptr_t) src0->data % 2) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: F16 weights must be 2-byte aligned");
+    if (src0->type == VX_TYPE_F32 && (uintptr_t) src0->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: F32 weights must be 4-byte aligned");
+    if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: F32 tensors must be 4-byte aligned");
+
+    mm_args a;
+    a.w = (const char *) src0->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
+    a.K = src0->ne[0]; a.M = src0->ne[1]; a.N = src1->ne[1];
+    a.nb01 = src0->nb[1]; a.nb02 = src0->nb[2]; a.nb03 = src0->nb[3];
+    a.nb11 = src1->nb[1]; a.nb12 = src1->nb[2]; a.nb13 = src1->nb[3];
+    a.nb1 = dst->nb[1]; a.nb2 = dst->nb[2]; a.nb3 = dst->nb[3];
+    a.ne12 = (int) src1->ne[2];
+    a.r2 = (int) (src1->ne[2] / src0->ne[2]); a.r3 = (int) (src1->ne[3] / src0->ne[3]);
+    a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
+    const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
+    hipStream_t st = (hipStream_t) stream;
+
+    switch (src0->type) {
+        case VX_TYPE_Q8_0:
+            if (act_mode == VX_ACT_Q8) launch<WT_Q8, true>(a, nbatch, st);
+            else                       launch<WT_Q8, false>(a, nbatch, st);
+            break;
+        case VX_TYPE_F16: launch<WT_F16, false>(a, nbatch, st); break;
+        default:          launch<WT_F32, false>(a, nbatch, st); break;
+    }
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}

@@ -1,0 +1,115 @@
+// vx_common.hpp -- shared host/device helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/voxcpm_gfx950.h"
+
+#define VX_WAVE 64
+#define VX_QK8_0 32
+#define VX_Q8_BLOCK 34 /* bytes: f16 d + 32 int8 */
+
+// ---- error plumbing -------------------------------------------------------------------
+void       vx_set_error(const char * fmt, ...) __attribute__((format(printf, 1, 2)));
+vx_status  vx_fail(vx_status st, const char * fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define VX_HIP(call)                                                                         \
+    do {                                                                                     \
+        hipError_t e_ = (call);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return vx_fail(VX_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                           __FILE__, __LINE__);                                              \
+    } while (0)
+
+#define VX_LAUNCH_CHECK()                                                                    \
+    do {                                                                                     \
+        hipError_t e_ = hipGetLastError();                                                   \
+        if (e_ != hipSuccess)                                                                \
+            return vx_fail(VX_ERR_HIP, "kernel launch failed: %s (%s:%d)",                   \
+                           hipGetErrorString(e_), __FILE__, __LINE__);                       \
+    } while (0)
+
+// per-stream scratch memory, grown on demand (never shrinks); valid until the next call
+// that asks for more on the same stream
+vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr);
+
+// ---- host-side tensor predicates ---------------------------------------------------------
+static inline size_t vx_type_size(int type) {
+    switch (type) {
+        case VX_TYPE_F32: return 4;
+        case VX_TYPE_F16: return 2;
+        case VX_TYPE_I32: return 4;
+        case VX_TYPE_Q8_0: return VX_Q8_BLOCK;
+        default: return 0;
+    }
+}
+static inline int64_t vx_blck(int type) { return type == VX_TYPE_Q8_0 ? VX_QK8_0 : 1; }
+static inline size_t  vx_row_size(int type, int64_t ne0) { return vx_type_size(type) * (size_t)(ne0 / vx_blck(type)); }
+static inline int64_t vx_nelements(const vx_tensor * t) { return t->ne[0] * t->ne[1] * t->ne[2] * t->ne[3]; }
+static inline int64_t vx_nrows(const vx_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
+static inline bool vx_same_shape(const vx_tensor * a, const vx_tensor * b) {
+    return a->ne[0] == b->ne[0] && a->ne[1] == b->ne[1] && a->ne[2] == b->ne[2] && a->ne[3] == b->ne[3];
+}
+static inline bool vx_is_contiguous(const vx_tensor * t) {
+    size_t nb = vx_type_size(t->type);
+    if (t->nb[0] != nb) return false;
+    nb = vx_row_size(t->type, t->ne[0]);
+    for (int i = 1; i < 4; ++i) {
+        if (t->ne[i] != 1 && t->nb[i] != nb) return false;
+        nb *= (size_t) t->ne[i];
+    }
+    return true;
+}
+static inline bool vx_positive(const vx_tensor * t) {
+    return t->ne[0] > 0 && t->ne[1] > 0 && t->ne[2] > 0 && t->ne[3] > 0;
+}
+
+// ---- device helpers ------------------------------------------------------------------------
+#ifdef __HIPCC__
+
+// 4-d strides passed to kernels by value
+struct vx_dims {
+    int64_t  ne[4];
+    uint64_t nb[4];
+};
+static inline vx_dims vx_dims_of(const vx_tensor * t) {
+    vx_dims d;
+    for (int i = 0; i < 4; ++i) { d.ne[i] = t->ne[i]; d.nb[i] = t->nb[i]; }
+    return d;
+}
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float    float4_t __attribute__((ext_vector_type(4)));
+typedef float    float16_t __attribute__((ext_vector_type(16)));
+typedef int      int4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float vx_wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double vx_wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float vx_wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ALiBi slope of head h (ggml/src/ggml-cpu/ops.cpp:8177-8200); m0, m1 computed on the host
+__device__ __forceinline__ float vx_alibi_slope(float max_bias, uint32_t h, uint32_t n_head_log2, float m0, float m1) {
+    if (!(max_bias > 0.0f)) return 1.0f;
+    return h < n_head_log2 ? powf(m0, (float)(h + 1)) : powf(m1, (float)(2 * (h - n_head_log2) + 1));
+}
+
+#endif // __HIPCC__
