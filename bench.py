@@ -1,0 +1,298 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Prints ONE JSON line.  The default workload is BASELINE config 2: backbone-shaped decode
+attention -- 24 layers x GQA attention (16 Q / 2 KV heads, head_dim 64), batch 2, one new
+token per step, f16 KV cache of length 4096.  A step is one pass over the 24 layers (24
+calls of vx_flash_attn_ext, each on its own layer's resident cache); `value` is the
+algorithmic KV bytes of a step divided by its wall time, inputs already in HBM.
+
+The same line carries, under "others", shorter measurements of the other BASELINE shapes
+(other KV lengths, the batch-16 / 8192-key decode, prefill attention, LocDiT attention,
+the Q8_0 projections), a `roofline` object for the dominant kernel of the headline
+workload and a `cpu_baseline` object: the reference's own ggml-cpu (oracle/_ref) timed on
+this machine's host cores on one layer of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA, published
+
+HQ, HKV, D, LAYERS = 16, 2, 64, 24
+
+
+def kv_bytes(batch, length, es=2):
+    """algorithmic HBM bytes of one decode attention launch: every K and V element once"""
+    return 2 * batch * HKV * length * D * es
+
+
+class Timer:
+    """HIP events on torch's current stream (the stream every vx_* call is enqueued on)."""
+
+    def __init__(self):
+        import torch
+        self.torch = torch
+        self.e0 = torch.cuda.Event(enable_timing=True)
+        self.e1 = torch.cuda.Event(enable_timing=True)
+
+    def run(self, fn, iters, warmup=3):
+        for _ in range(warmup):
+            fn()
+        self.torch.cuda.synchronize()
+        self.e0.record()
+        for _ in range(iters):
+            fn()
+        self.e1.record()
+        self.torch.cuda.synchronize()
+        return self.e0.elapsed_time(self.e1) * 1e-3 / iters  # seconds per call
+
+
+def graphed(fn, stream):
+    """Capture fn's launches (all on `stream`) into a HIP graph; returns the replay callable.
+    fn runs eagerly first so that the library's per-stream scratch exists before capture."""
+    import torch
+    with torch.cuda.stream(stream):
+        fn()
+        fn()
+    stream.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        fn()
+    return g.replay
+
+
+def decode_attn_setup(pkg, batch, length, layers):
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(1234 + length)
+    caches = []
+    for _ in range(layers):
+        k = torch.randn((batch, HKV, length, D), generator=g, device="cuda", dtype=torch.float32).half()
+        v = torch.randn((batch, HKV, length, D), generator=g, device="cuda", dtype=torch.float32).half()
+        caches.append((k, v))
+    q = torch.randn((batch, HQ, 1, D), generator=g, device="cuda", dtype=torch.float32)
+    out = torch.empty((batch, 1, HQ, D), device="cuda", dtype=torch.float32)
+    lib = pkg.lib()
+    qd, od = pkg.desc(q), pkg.desc(out)
+    descs = [(pkg.desc(k), pkg.desc(v)) for k, v in caches]
+
+    def step():
+        for kd, vd in descs:
+            rc = lib.vx_flash_attn_ext(qd, kd, vd, None, None, od, 0.125, 0.0, 0.0, torch.cuda.current_stream().cuda_stream)
+            if rc:
+                pkg.check(rc, "vx_flash_attn_ext")
+
+    def one_layer():
+        kd, vd = descs[0]
+        rc = lib.vx_flash_attn_ext(qd, kd, vd, None, None, od, 0.125, 0.0, 0.0, torch.cuda.current_stream().cuda_stream)
+        if rc:
+            pkg.check(rc, "vx_flash_attn_ext")
+
+    return step, one_layer, (q, caches, out)
+
+
+def prefill_attn_setup(pkg, batch, T):
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import reflib
+    g = torch.Generator(device="cuda").manual_seed(99 + T)
+    q = torch.randn((batch, HQ, T, D), generator=g, device="cuda", dtype=torch.float32)
+    k = torch.randn((batch, HKV, T, D), generator=g, device="cuda", dtype=torch.float32).half()
+    v = torch.randn((batch, HKV, T, D), generator=g, device="cuda", dtype=torch.float32).half()
+    mask = torch.from_numpy(reflib.causal_mask(T, T)).cuda()
+    out = torch.empty((batch, T, HQ, D), device="cuda", dtype=torch.float32)
+    lib = pkg.lib()
+    qd, kd, vd, md, od = pkg.desc(q), pkg.desc(k), pkg.desc(v), pkg.desc(mask), pkg.desc(out)
+
+    def call():
+        rc = lib.vx_flash_attn_ext(qd, kd, vd, md, None, od, 0.125, 0.0, 0.0, torch.cuda.current_stream().cuda_stream)
+        if rc:
+            pkg.check(rc, "vx_flash_attn_ext")
+
+    flops = 4.0 * HQ * D * T * (T + 1) / 2 * batch  # causal-exact
+    return call, flops, (q, k, v, mask, out)
+
+
+def locdit_attn_setup(pkg, requests=8, branch=7, layers=4, timesteps=10):
+    import torch
+    import reflib
+    L = 2 * branch
+    pos = np.zeros(L, np.int32)
+    m = np.zeros((L, L), np.uint16)
+    reflib.load_oracle().orc_cfg_pair_constants(branch, reflib.ptr(pos, C.c_int32), reflib.ptr(m, C.c_uint16))
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn((requests, HQ, L, D), generator=g, device="cuda")
+    k = torch.randn((requests, HKV, L, D), generator=g, device="cuda")
+    v = torch.randn((requests, HKV, L, D), generator=g, device="cuda")
+    mask = torch.from_numpy(m.view(np.float16)).cuda()
+    out = torch.empty((requests, L, HQ, D), device="cuda")
+    lib = pkg.lib()
+    qd, kd, vd, md, od = pkg.desc(q), pkg.desc(k), pkg.desc(v), pkg.desc(mask), pkg.desc(out)
+    n_calls = layers * (timesteps - 1)  # the first Euler step is skipped under cfg-zero-star
+
+    def solve():
+        for _ in range(n_calls):
+            rc = lib.vx_flash_attn_ext(qd, kd, vd, md, None, od, 0.125, 0.0, 0.0, torch.cuda.current_stream().cuda_stream)
+            if rc:
+                pkg.check(rc, "vx_flash_attn_ext")
+
+    return solve, n_calls, (q, k, v, mask, out)
+
+
+def q8_proj_setup(pkg, M, K, N):
+    import torch
+    import reflib
+    w = (reflib.rng("bench", "w", M, K).standard_normal((M, K)) * 0.02).astype(np.float32)
+    wq = torch.from_numpy(reflib.quantize_q8_0(w)).cuda()
+    x = torch.randn((N, K), device="cuda")
+    out = torch.empty((N, M), device="cuda")
+    lib = pkg.lib()
+    wd, xd, od = pkg.desc_q8(wq, K), pkg.desc(x), pkg.desc(out)
+
+    def call():
+        rc = lib.vx_mul_mat(wd, xd, od, pkg.ACT_FLOAT, torch.cuda.current_stream().cuda_stream)
+        if rc:
+            pkg.check(rc, "vx_mul_mat")
+
+    return call, (wq, x, out)
+
+
+def cpu_baseline(batch, length, threads):
+    """ggml-cpu (the reference build in oracle/_ref) on one layer of the decode workload."""
+    import reflib
+    ref = reflib.load_ref()
+    q = reflib.rng("cpu", "q").standard_normal((batch, HQ, 1, D)).astype(np.float32)
+    k = reflib.rng("cpu", "k").standard_normal((batch, HKV, length, D)).astype(np.float16)
+    v = reflib.rng("cpu", "v").standard_normal((batch, HKV, length, D)).astype(np.float16)
+    if ref is not None:
+        assert ref.rh_use_device(b"CPU", threads, 0) == 0
+        # size the sample to roughly 10 s of CPU work
+        _, (mean1, _) = reflib.ref_fa(q, k, v, reps=20)
+        reps = int(max(50, min(20000, 10.0 / max(mean1, 1e-6))))
+        _, (mean, best) = reflib.ref_fa(q, k, v, reps=reps)
+        return {"value": kv_bytes(batch, length) / mean / 1e9, "unit": "GB/s", "cores": threads, "kind": "reference",
+                "sample": f"{reps} repeats of one layer's ggml_flash_attn_ext on ggml-cpu (batch {batch}, KV {length}, "
+                          f"f16 K/V), mean {mean * 1e6:.1f} us, best {best * 1e6:.1f} us"}
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        reflib.oracle_fa(q, k.astype(np.float32), v.astype(np.float32))
+    mean = (time.perf_counter() - t0) / reps
+    return {"value": kv_bytes(batch, length) / mean / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} repeats of one layer on the scalar C oracle (oracle/_ref not prebuilt)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--length", type=int, default=4096, help="KV length of the headline decode workload")
+    ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the ggml-cpu baseline")
+    ap.add_argument("--eager", action="store_true", help="launch every call from Python instead of replaying a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path has no cross-GPU step); run with --gpus 1")
+
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    pkg.check(pkg.lib().vx_init(0), "vx_init")
+    timer = Timer()
+
+    # ---- headline: config 2, L = args.length -------------------------------------------
+    B, L = 2, args.length
+    side = torch.cuda.Stream()
+    step_eager, one_layer, keep = decode_attn_setup(pkg, B, L, LAYERS)
+    eager_sec = timer.run(step_eager, iters=20)
+    # the 24 launches of a step replayed as one HIP graph: what a C++ host looping over graph
+    # nodes achieves, without the Python call overhead of this script
+    step = graphed(step_eager, side) if not args.eager else step_eager
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    sec_per_step = (time.perf_counter() - t0) / args.steps
+    step_bytes = LAYERS * kv_bytes(B, L)
+    value = step_bytes / sec_per_step / 1e9
+
+    # dominant kernel: one vx_flash_attn_ext call (split-KV kernel + combine), HIP events
+    launch_sec = timer.run(step, iters=200, warmup=10) / LAYERS
+    achieved = kv_bytes(B, L) / launch_sec / 1e9
+    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64,f16> (+ combine)", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "launch_us": launch_sec * 1e6, "bytes_per_launch": kv_bytes(B, L),
+                "note": "average over the 24 launches of a graph-replayed step (HIP events on the launch stream)"}
+    del keep
+
+    others = {}
+    if not args.no_others:
+        for L2 in (128, 512, 2048, 4096):
+            st, one, keep = decode_attn_setup(pkg, 2, L2, LAYERS)
+            s = timer.run(graphed(st, side), iters=50)
+            others[f"cfg2_decode_attn_L{L2}"] = {"us_per_layer": s / LAYERS * 1e6,
+                                                  "GB/s": LAYERS * kv_bytes(2, L2) / s / 1e9}
+            del keep
+        st, one, keep = decode_attn_setup(pkg, 16, 8192, 4)
+        s = timer.run(graphed(st, side), iters=100, warmup=10) / 4
+        others["cfg5_decode_attn_B16_L8192"] = {"us_per_layer": s * 1e6, "GB/s": kv_bytes(16, 8192) / s / 1e9,
+                                                "hbm_frac": kv_bytes(16, 8192) / s / 1e9 / HBM_PEAK_GBS}
+        del keep
+        for name, b, T, it in (("cfg1_prefill_attn_T256", 1, 256, 200), ("cfg5_prefill_attn_T4096_B1", 1, 4096, 5)):
+            call, flops, keep = prefill_attn_setup(pkg, b, T)
+            s = timer.run(call, iters=it, warmup=2)
+            others[name] = {"us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
+                            "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}
+            del keep
+        solve, n_calls, keep = locdit_attn_setup(pkg)
+        s = timer.run(graphed(solve, side), iters=20)
+        others["cfg3_locdit_attn_16seq_x7"] = {"us_per_cfm_solve": s * 1e6, "launches_per_solve": n_calls,
+                                               "us_per_attention": s / n_calls * 1e6}
+        del keep
+        for name, M, K, N in (("q8_0_proj_1024x1024_n2", 1024, 1024, 2), ("q8_0_ffn_up_4096x1024_n2", 4096, 1024, 2),
+                              ("q8_0_proj_1024x1024_n1024", 1024, 1024, 1024)):
+            call, keep = q8_proj_setup(pkg, M, K, N)
+            s = timer.run(call, iters=200, warmup=5)
+            wbytes = M * K // 32 * 34
+            others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12}
+            del keep
+
+    cpu = None
+    if not args.no_cpu:
+        threads = min(16, os.cpu_count() or 1)
+        cpu = cpu_baseline(B, L, threads)
+
+    line = {
+        "metric": "decode attention HBM GB/s (backbone-shaped decode, 24 layers, batch 2)",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 K/V, f32 accumulate", "data": "synthetic (seeded N(0,1))",
+        "config": {"workload": f"BASELINE config 2: 24 layers x GQA decode attention, 16/2 heads, head_dim 64, "
+                               f"batch 2, f16 KV length {L}", "decode_attn_steps_per_s": 1.0 / sec_per_step,
+                   "launch": "eager from Python" if args.eager else "one HIP graph replay per step",
+                   "eager_python_ms_per_step": eager_sec * 1e3},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,12 +1,17 @@
-// fattn.hip -- GGML_OP_FLASH_ATTN_EXT on gfx950: the column-packed wave kernel (decode,
-// LocDiT-sized sequences, and the general fallback) plus the split-KV combine.
+// fattn.hip -- GGML_OP_FLASH_ATTN_EXT on gfx950: the column-packed kernel used for decode,
+// LocDiT-sized sequences and as the general path.
 //
 // Work decomposition.  For one batch element b and one KV head g, every (query row iq1,
 // query head of the GQA group) pair is a *column*: col = iq1 * gqa + head_in_group.  A
 // wavefront owns 16 consecutive columns -- in decode that is the 8 query heads sharing the
 // KV head (x2 rows when n_q = 2), in LocDiT 2 rows x 8 heads -- and one contiguous range
-// of keys (a split).  Everything a wave needs stays in its registers: there is no LDS and
-// no barrier, so waves retire independently and occupancy alone hides HBM latency.
+// of keys.  Its K/V stream never touches LDS: operands are loaded from global memory
+// straight into MFMA layout, one 32-key tile in flight ahead of the one being consumed.
+// When there are too few columns to fill the chip the keys are cut further (flash-decoding):
+// several waves take adjacent key ranges of the same columns and write (max, sum, O)
+// partials that a second, small kernel merges.  (Merging inside the first kernel, by the
+// last wave to arrive, needs device-scope release/acquire fences; on this multi-die part
+// those write back and invalidate L2 and cost several times what the second launch does.)
 //
 // MFMA formulation (v_mfma_f32_16x16x32_f16, lane = 16*j + c):
 //   S^T = K * Q^T      A = K rows as they lie in memory (lane c = key, 8 consecutive d per
@@ -19,8 +24,8 @@
 //                      d per lane while memory has 8 *d* of one key; the transpose is done
 //                      by the matrix core itself: V (as it lies in memory) times a 0/1
 //                      selection matrix lands V^T in accumulator layout, exactly, and a
-//                      convert makes it the A operand.  Matrix throughput is ~6x what HBM
-//                      can feed in this regime, so spending it on the transpose is free.
+//                      convert makes it the A operand.  Matrix throughput is several times
+//                      what HBM can feed in this regime, so the transpose costs nothing.
 // Precision: Q, P (and K, V when they are F32) are split into f16 hi + lo parts and both
 // parts multiplied, so the products carry ~22 bits; accumulation and softmax are fp32.
 //
@@ -30,6 +35,7 @@
 #include "vx_common.hpp"
 
 #include <cmath>
+#include <cstdlib>
 
 namespace {
 
@@ -37,8 +43,8 @@ struct fa_args {
     const char * q; const char * k; const char * v; const char * mask;
     const float * sinks;
     float * dst;
-    float * part_o;  // [gcol][split][D]
-    float * part_ml; // [gcol][split][2]
+    float * part_o;   // [tile][split][16 columns][D]   split partials, un-normalised
+    float * part_ml;  // [tile][split][16 columns][2]   running max, running sum
     uint64_t nbq1, nbq2, nbq3, nbk1, nbk2, nbk3, nbv1, nbv2, nbv3, nbm1, nbm2, nbm3;
     int n_q, n_kv, Hq, Hkv, gqa, ne3, rk3, nem2, nem3;
     int n_col_tiles, n_splits, chunk;
@@ -48,6 +54,15 @@ struct fa_args {
 
 __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// two floats -> packed halves, round toward zero: one instruction.  Used where the value is
+// exactly representable (transposed f16 data) or where a lo part picks up the remainder.
+__device__ __forceinline__ void pk2(half8_t & dst, int i, float a, float b) {
+    typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
+    const fp16x2 v = __builtin_amdgcn_cvt_pkrtz(a, b);
+    dst[i]     = (_Float16) v[0];
+    dst[i + 1] = (_Float16) v[1];
 }
 
 // 8 consecutive elements -> f16 hi (+ lo) operand
@@ -71,7 +86,29 @@ template <> struct kv_load<true> {
     }
 };
 
-template <int D, bool KV_F32>
+// the K and V rows one wave consumes per iteration: 32 keys, as MFMA operands
+template <int NP, bool KV_F32> struct kv_tile {
+    half8_t khi[2][NP], klo[2][NP], vhi[2][NP], vlo[2][NP];
+};
+
+// sinks (ops.cpp:8306-8322), normalisation and the permuted store of ggml's result for 4
+// consecutive d of one column
+__device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float M, float L, int b, int g, int col,
+                                          int D, int d0) {
+    const int iq1 = col / a.gqa, head = g * a.gqa + col % a.gqa;
+    if (a.sinks) {
+        const float sk = a.sinks[head] * 1.44269504088896341f; // M is in the log2 domain
+        float ms = 1.0f, vs = 1.0f;
+        if (sk > M) { ms = __builtin_amdgcn_exp2f(M - sk); } else { vs = __builtin_amdgcn_exp2f(sk - M); }
+        acc *= ms;
+        L = L * ms + vs;
+    }
+    const float inv = L == 0.0f ? 0.0f : 1.0f / L;
+    *(float4_t *) (a.dst + (((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D + d0) = acc * inv;
+}
+
+// One wave (= one block) = 16 columns x one key range.
+template <int D, bool KV_F32, bool HAS_MASK>
 __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     constexpr int NP  = D / 32;          // MFMAs along the head dimension
     constexpr int SEG = D / 4;           // elements of a row owned by lane-group j
@@ -85,6 +122,7 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     const int sp = w % a.n_splits;    w /= a.n_splits;
     const int g  = w % a.Hkv;
     const int b  = w / a.Hkv;
+    const int tile = (b * a.Hkv + g) * a.n_col_tiles + ct;
 
     const int  ncols  = a.n_q * a.gqa;
     const int  col    = ct * 16 + c;
@@ -92,14 +130,39 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     const int  iq1    = col_ok ? col / a.gqa : 0;
     const int  head   = g * a.gqa + (col_ok ? col % a.gqa : 0);
 
+    const char * kbase = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3 + (uint64_t) (SEG * j) * ES;
+    const char * vbase = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3 + (uint64_t) (SEG * j) * ES;
+
+    const int kv0 = sp * a.chunk;
+    const int kv1 = min(a.n_kv, kv0 + a.chunk);
+
+    // rows this lane loads (MFMA row c of each 16-key half); clamped, masked out later
+    auto load_tile = [&](int kb, kv_tile<NP, KV_F32> & t) {
+        const int key0 = min(kb + c, a.n_kv - 1), key1 = min(kb + 16 + c, a.n_kv - 1);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            kv_load<KV_F32>::run(kbase + (uint64_t) key0 * a.nbk1 + p * 8 * ES, t.khi[0][p], t.klo[0][p]);
+            kv_load<KV_F32>::run(kbase + (uint64_t) key1 * a.nbk1 + p * 8 * ES, t.khi[1][p], t.klo[1][p]);
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            kv_load<KV_F32>::run(vbase + (uint64_t) key0 * a.nbv1 + p * 8 * ES, t.vhi[0][p], t.vlo[0][p]);
+            kv_load<KV_F32>::run(vbase + (uint64_t) key1 * a.nbv1 + p * 8 * ES, t.vhi[1][p], t.vlo[1][p]);
+        }
+    };
+
+    // two tiles alternate in registers: while one is consumed the other is in flight
+    kv_tile<NP, KV_F32> t0, t1;
+    load_tile(kv0, t0);
+
     // ---- Q^T operand: column c, elements d = SEG*j + 8p + i, split into hi + lo
     half8_t qhi[NP], qlo[NP];
     {
         const float * qp = (const float *) (a.q + (uint64_t) iq1 * a.nbq1 + (uint64_t) head * a.nbq2 + (uint64_t) b * a.nbq3) + SEG * j;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            float4_t x0 = {0, 0, 0, 0}, x1 = {0, 0, 0, 0};
-            if (col_ok) { x0 = ((const float4_t *) (qp + 8 * p))[0]; x1 = ((const float4_t *) (qp + 8 * p))[1]; }
+            float4_t x0 = ((const float4_t *) (qp + 8 * p))[0], x1 = ((const float4_t *) (qp + 8 * p))[1];
+            if (!col_ok) { x0 = float4_t{0, 0, 0, 0}; x1 = float4_t{0, 0, 0, 0}; }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 qhi[p][i]     = (_Float16) x0[i];
@@ -118,14 +181,12 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) sel[u][i] = (j == 2 * u + (c >> 3) && i == (c & 7)) ? (_Float16) 1.0f : (_Float16) 0.0f;
 
-    const float slope = vx_alibi_slope(a.max_bias, (uint32_t) head, a.n_head_log2, a.m0, a.m1);
-    const char * mrow = a.mask ? a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (head % a.nem2) * a.nbm2 + (uint64_t) (b % a.nem3) * a.nbm3 : nullptr;
-
-    const char * kbase = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3 + (uint64_t) (SEG * j) * ES;
-    const char * vbase = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3 + (uint64_t) (SEG * j) * ES;
-
-    const int kv0 = sp * a.chunk;
-    const int kv1 = min(a.n_kv, kv0 + a.chunk);
+    float slope = 1.0f;
+    const __half * mrow = nullptr;
+    if constexpr (HAS_MASK) {
+        slope = vx_alibi_slope(a.max_bias, (uint32_t) head, a.n_head_log2, a.m0, a.m1) * 1.44269504088896341f;
+        mrow  = (const __half *) (a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (head % a.nem2) * a.nbm2 + (uint64_t) (b % a.nem3) * a.nbm3);
+    }
 
     float4_t o[NP][2];
 #pragma unroll
@@ -133,21 +194,19 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     float m = -INFINITY; // running max of column c (identical in the 4 lanes of a column)
     float l = 0.0f;      // this lane's share of the running sum
 
-    for (int kb = kv0; kb < kv1; kb += 32) {
-        // rows this lane loads (as MFMA row c of each 16-key half); clamped, masked out below
-        const int key0 = min(kb + c, a.n_kv - 1), key1 = min(kb + 16 + c, a.n_kv - 1);
-
-        half8_t khi[2][NP], klo[2][NP], vhi[2][NP], vlo[2][NP];
+    auto consume = [&](const kv_tile<NP, KV_F32> & t, int kb) {
+        // additive mask of this lane's 8 keys (kb + 16h + 4j + r); loads are clamped, the
+        // out-of-range keys are switched off below
+        float mv[2][4];
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            kv_load<KV_F32>::run(kbase + (uint64_t) key0 * a.nbk1 + p * 8 * ES, khi[0][p], klo[0][p]);
-            kv_load<KV_F32>::run(kbase + (uint64_t) key1 * a.nbk1 + p * 8 * ES, khi[1][p], klo[1][p]);
-        }
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            kv_load<KV_F32>::run(vbase + (uint64_t) key0 * a.nbv1 + p * 8 * ES, vhi[0][p], vlo[0][p]);
-            kv_load<KV_F32>::run(vbase + (uint64_t) key1 * a.nbv1 + p * 8 * ES, vhi[1][p], vlo[1][p]);
-        }
+            for (int r = 0; r < 4; ++r) {
+                const int key = kb + 16 * h + 4 * j + r;
+                float x = 0.0f;
+                if constexpr (HAS_MASK) x = slope * __half2float(mrow[min(key, a.n_kv - 1)]); // slope carries log2(e)
+                mv[h][r] = key < kv1 ? x : -INFINITY;
+            }
 
         // ---- S^T for the two 16-key halves
         float4_t s[2];
@@ -156,156 +215,159 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
             float4_t acc = {0, 0, 0, 0};
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
-                acc = mfma16(khi[h][p], qlo[p], acc);
-                if constexpr (KV_F32) acc = mfma16(klo[h][p], qhi[p], acc);
-                acc = mfma16(khi[h][p], qhi[p], acc);
+                acc = mfma16(t.khi[h][p], qlo[p], acc);
+                if constexpr (KV_F32) acc = mfma16(t.klo[h][p], qhi[p], acc);
+                acc = mfma16(t.khi[h][p], qhi[p], acc);
             }
             s[h] = acc;
         }
 
-        // ---- scale, soft cap, mask; keys of lane (j,c): kb + 16h + 4j + r
+        // ---- scale, soft cap, mask
         float cmax = -INFINITY;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key = kb + 16 * h + 4 * j + r;
+                // a.scale carries log2(e) (the soft cap path applies it after tanh)
                 float x = s[h][r] * a.scale;
                 if (a.softcap != 0.0f) x = a.softcap * tanhf(x);
-                if (key < kv1) {
-                    if (mrow) x += slope * __half2float(((const __half *) mrow)[key]);
-                } else {
-                    x = -INFINITY;
-                }
+                x += mv[h][r];
                 s[h][r] = x;
                 cmax = fmaxf(cmax, x);
             }
         cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
         cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
 
-        const float m_new = fmaxf(m, cmax);
-        if (__builtin_amdgcn_ballot_w64(m_new != -INFINITY) == 0) continue; // every column fully masked so far
-
-        const float alpha = (m_new == -INFINITY) ? 1.0f : __expf(m - m_new); // m = -inf -> 0
+        // a column whose keys are all masked so far keeps m = -inf; shifting by 0 instead
+        // keeps exp(-inf - shift) = 0 without a branch
+        const float m_new  = fmaxf(m, cmax);
+        const float shift  = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha  = __builtin_amdgcn_exp2f(m - shift); // m = -inf -> 0
         float psum = 0.0f;
         half8_t phi, plo;
+        float pvv[8];
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float pv = (m_new == -INFINITY) ? 0.0f : __expf(s[h][r] - m_new);
-                psum += pv;
-                const _Float16 ph = (_Float16) pv;
-                phi[4 * h + r] = ph;
-                plo[4 * h + r] = (_Float16) (pv - (float) ph);
+                pvv[4 * h + r] = __builtin_amdgcn_exp2f(s[h][r] - shift);
+                psum += pvv[4 * h + r];
             }
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) pk2(phi, i, pvv[i], pvv[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) pk2(plo, i, pvv[i] - (float) phi[i], pvv[i + 1] - (float) phi[i + 1]);
         l = l * alpha + psum;
         m = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) { // the maxima rarely move late in a row
 #pragma unroll
-        for (int p = 0; p < NP; ++p) { o[p][0] *= alpha; o[p][1] *= alpha; }
+            for (int p = 0; p < NP; ++p) { o[p][0] *= alpha; o[p][1] *= alpha; }
+        }
 
         // ---- O^T += V^T P^T, V^T produced by the matrix core
 #pragma unroll
         for (int p = 0; p < NP; ++p)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                float4_t t0 = mfma16(vhi[0][p], sel[u], float4_t{0, 0, 0, 0});
-                float4_t t1 = mfma16(vhi[1][p], sel[u], float4_t{0, 0, 0, 0});
-                if constexpr (KV_F32) { t0 = mfma16(vlo[0][p], sel[u], t0); t1 = mfma16(vlo[1][p], sel[u], t1); }
+                float4_t t0 = mfma16(t.vhi[0][p], sel[u], float4_t{0, 0, 0, 0});
+                float4_t t1 = mfma16(t.vhi[1][p], sel[u], float4_t{0, 0, 0, 0});
+                if constexpr (KV_F32) { t0 = mfma16(t.vlo[0][p], sel[u], t0); t1 = mfma16(t.vlo[1][p], sel[u], t1); }
                 half8_t vt;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) { vt[r] = (_Float16) t0[r]; vt[4 + r] = (_Float16) t1[r]; }
+                for (int r = 0; r < 4; r += 2) { pk2(vt, r, t0[r], t0[r + 1]); pk2(vt, 4 + r, t1[r], t1[r + 1]); }
                 o[p][u] = mfma16(vt, plo, o[p][u]);
                 o[p][u] = mfma16(vt, phi, o[p][u]);
                 if constexpr (KV_F32) {
                     half8_t vl;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        vl[r]     = (_Float16) (t0[r] - (float) vt[r]);
-                        vl[4 + r] = (_Float16) (t1[r] - (float) vt[4 + r]);
+                    for (int r = 0; r < 4; r += 2) {
+                        pk2(vl, r, t0[r] - (float) vt[r], t0[r + 1] - (float) vt[r + 1]);
+                        pk2(vl, 4 + r, t1[r] - (float) vt[4 + r], t1[r + 1] - (float) vt[4 + r + 1]);
                     }
                     o[p][u] = mfma16(vl, phi, o[p][u]);
                 }
             }
+    };
+
+    // The prefetches are unconditional (the tile index is clamped to the wave's last tile, a
+    // cache hit) so that the wait before each use counts a fixed number of younger loads; a
+    // conditional prefetch forces the compiler to wait for everything and exposes the whole
+    // memory latency in every iteration.
+    const int klast = kv0 + ((kv1 - kv0 - 1) / 32) * 32;
+    for (int kb = kv0; kb < kv1; kb += 64) {
+        load_tile(min(kb + 32, klast), t1);
+        consume(t0, kb);
+        if (kb + 32 >= kv1) break;
+        load_tile(min(kb + 64, klast), t0);
+        consume(t1, kb + 32);
     }
 
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
+    if (!col_ok) return;
 
     // lane (j,c), tile (p,u), register r holds d = SEG*(2u + j/2) + 8p + 4*(j%2) + r of column c
     if (a.n_splits == 1) {
-        if (a.sinks) { // ops.cpp:8306-8322
-            const float sk = a.sinks[head];
-            float ms = 1.0f, vs = 1.0f;
-            if (sk > m) { ms = __expf(m - sk); } else { vs = __expf(sk - m); }
-#pragma unroll
-            for (int p = 0; p < NP; ++p) { o[p][0] *= ms; o[p][1] *= ms; }
-            l = l * ms + vs;
-        }
-        const float inv = l == 0.0f ? 0.0f : 1.0f / l;
-        if (col_ok) {
-            float * out = a.dst + (((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D;
-#pragma unroll
-            for (int p = 0; p < NP; ++p)
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int d0 = SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1);
-                    *(float4_t *) (out + d0) = o[p][u] * inv;
-                }
-        }
-    } else if (col_ok) {
-        const uint64_t gcol = ((uint64_t) b * a.Hkv + g) * ncols + col;
-        float * po = a.part_o + (gcol * a.n_splits + sp) * D;
 #pragma unroll
         for (int p = 0; p < NP; ++p)
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int d0 = SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1);
-                *(float4_t *) (po + d0) = o[p][u];
-            }
-        if (j == 0) {
-            float * pml = a.part_ml + (gcol * a.n_splits + sp) * 2;
-            pml[0] = m;
-            pml[1] = l;
-        }
+            for (int u = 0; u < 2; ++u)
+                fa_finish(a, o[p][u], m, l, b, g, col, D, SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1));
+    } else {
+        const uint64_t pbase = ((uint64_t) tile * a.n_splits + sp) * 16 + c;
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                *(float4_t *) (a.part_o + pbase * D + SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1)) = o[p][u];
+        if (j == 0) { a.part_ml[pbase * 2] = m; a.part_ml[pbase * 2 + 1] = l; }
     }
 }
 
-// merges the split partials of one column: the arithmetic of
-// ggml_flash_attn_ext_reduce_partials (ggml/src/ggml-cpu/ops.cpp:8637-8705) with the global
-// maximum taken first.  One block of D threads per column.
-template <int D>
-__global__ __launch_bounds__(D) void fattn_combine_kernel(const fa_args a) {
-    const int      ncols = a.n_q * a.gqa;
-    const uint64_t gcol  = blockIdx.x;
-    const int      col   = (int) (gcol % ncols);
-    const int      bg    = (int) (gcol / ncols);
-    const int      g = bg % a.Hkv, b = bg / a.Hkv;
-    const int      iq1 = col / a.gqa, head = g * a.gqa + col % a.gqa;
-    const int      d = threadIdx.x;
+// Merges the split partials: the arithmetic of ggml_flash_attn_ext_reduce_partials
+// (ggml/src/ggml-cpu/ops.cpp:8637-8705) with the global maximum taken first.  A block takes
+// 4 of a tile's 16 columns; thread = (column, 4 consecutive d, one of SG split groups), the
+// groups' sums meet in LDS.
+constexpr int FA_MERGE_MAX_SPLITS = 256;
+template <int D, int SG>
+__global__ __launch_bounds__(4 * (D / 4) * SG) void fattn_merge_kernel(const fa_args a) {
+    constexpr int DU = D / 4;
+    __shared__ float    sh_m[FA_MERGE_MAX_SPLITS][4], sh_l[FA_MERGE_MAX_SPLITS][4];
+    __shared__ float4_t sh_acc[SG][4 * DU];
+    const int tile = blockIdx.x >> 2, cq = blockIdx.x & 3;
+    const int ct = tile % a.n_col_tiles;
+    const int bg = tile / a.n_col_tiles;
+    const int g = bg % a.Hkv, b = bg / a.Hkv;
+    const int ncols = a.n_q * a.gqa;
+    const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + cq * 4; // + split*16 + column
 
-    const float * pml = a.part_ml + gcol * a.n_splits * 2;
-    const float * po  = a.part_o + gcol * a.n_splits * D;
+    for (int i = threadIdx.x; i < 4 * a.n_splits; i += blockDim.x) {
+        const int s2 = i >> 2, cc = i & 3;
+        const float2 ml = *(const float2 *) (a.part_ml + (tbase + (uint64_t) s2 * 16 + cc) * 2);
+        sh_m[s2][cc] = ml.x;
+        sh_l[s2][cc] = ml.y;
+    }
+    __syncthreads();
+
+    const int sg = threadIdx.x / (4 * DU), e = threadIdx.x % (4 * DU);
+    const int cc = e / DU, d0 = 4 * (e % DU);
     float M = -INFINITY;
-    for (int s = 0; s < a.n_splits; ++s) M = fmaxf(M, pml[2 * s]);
-    float acc = 0.0f, L = 0.0f;
-    if (M != -INFINITY) {
-        for (int s = 0; s < a.n_splits; ++s) {
-            const float ms = pml[2 * s];
-            if (ms == -INFINITY) continue;
-            const float wgt = __expf(ms - M);
-            acc += wgt * po[(uint64_t) s * D + d];
-            L += wgt * pml[2 * s + 1];
-        }
-    }
-    if (a.sinks) {
-        const float sk = a.sinks[head];
-        float ms = 1.0f, vs = 1.0f;
-        if (sk > M) { ms = __expf(M - sk); } else { vs = __expf(sk - M); }
-        acc *= ms;
-        L = L * ms + vs;
-    }
-    a.dst[(((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D + d] = L == 0.0f ? 0.0f : acc / L;
+    for (int s2 = 0; s2 < a.n_splits; ++s2) M = fmaxf(M, sh_m[s2][cc]);
+    const float shift = (M == -INFINITY) ? 0.0f : M;
+
+    float4_t acc = {0, 0, 0, 0};
+    const float4_t * po = (const float4_t *) (a.part_o + (tbase + cc) * D + d0); // + split * 4*D float4
+#pragma unroll 8
+    for (int s2 = sg; s2 < a.n_splits; s2 += SG) acc += po[(uint64_t) s2 * 4 * D] * __builtin_amdgcn_exp2f(sh_m[s2][cc] - shift);
+    sh_acc[sg][e] = acc;
+    __syncthreads();
+    if (sg != 0) return;
+#pragma unroll
+    for (int gg = 1; gg < SG; ++gg) acc += sh_acc[gg][e];
+    float L = 0.0f;
+    for (int s2 = 0; s2 < a.n_splits; ++s2) L += sh_l[s2][cc] * __builtin_amdgcn_exp2f(sh_m[s2][cc] - shift);
+    const int col = ct * 16 + cq * 4 + cc;
+    if (col < ncols) fa_finish(a, acc, M, L, b, g, col, D, d0);
 }
 
 int g_num_cus = 0;
@@ -322,6 +384,12 @@ int num_cus() {
 
 bool aligned16(const vx_tensor * t) {
     return ((uintptr_t) t->data % 16 == 0) && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+}
+
+template <int D, bool KV_F32>
+void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
+    if (a.mask) fattn_cols16_kernel<D, KV_F32, true><<<dim3((unsigned) nblocks), dim3(64), 0, st>>>(a);
+    else        fattn_cols16_kernel<D, KV_F32, false><<<dim3((unsigned) nblocks), dim3(64), 0, st>>>(a);
 }
 
 } // namespace
@@ -378,34 +446,43 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     a.gqa = a.Hq / a.Hkv; a.ne3 = (int) q->ne[3]; a.rk3 = (int) (q->ne[3] / k->ne[3]);
     a.nem2 = mask ? (int) mask->ne[2] : 1; a.nem3 = mask ? (int) mask->ne[3] : 1;
     a.scale = scale; a.softcap = logit_softcap; a.max_bias = max_bias;
-    if (logit_softcap != 0.0f) a.scale /= logit_softcap; // ops.cpp:8173-8175
+    // the kernels work in the log2 domain: p = 2^(x*log2(e) - m)
+    const float LOG2E = 1.44269504088896341f;
+    if (logit_softcap != 0.0f) { a.scale /= logit_softcap; a.softcap *= LOG2E; } // ops.cpp:8173-8175
+    else                       { a.scale *= LOG2E; }
     a.n_head_log2 = 1u << (uint32_t) floor(log2((double) a.Hq));
     a.m0 = powf(2.0f, -(max_bias) / a.n_head_log2);
     a.m1 = powf(2.0f, -(max_bias / 2.0f) / a.n_head_log2);
 
     const int ncols = a.n_q * a.gqa;
     a.n_col_tiles   = (ncols + 15) / 16;
-    const int64_t base_waves = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
+    const int64_t tiles = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
 
-    // split the keys so that the launch has about 8 waves per CU, at least 64 keys each
-    const int64_t target = (int64_t) 8 * num_cus();
-    int64_t want = (target + base_waves - 1) / base_waves;
-    const int64_t max_splits = (a.n_kv + 63) / 64;
-    if (want > max_splits) want = max_splits;
-    if (want < 1) want = 1;
-    int chunk = (int) ((a.n_kv + want - 1) / want);
-    chunk     = (chunk + 31) / 32 * 32;
-    a.chunk    = chunk;
-    a.n_splits = (a.n_kv + chunk - 1) / chunk;
+    // Work split.  Enough 16-column tiles to fill the chip: one wave per tile over all keys.
+    // Otherwise cut the keys (flash-decoding) aiming at ~8 waves per CU, at least `min_chunk`
+    // keys per wave, and merge the partials with a second small kernel.
+    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 128; }();
+    a.n_splits = 1;
+    a.chunk    = (a.n_kv + 31) / 32 * 32;
+    if (tiles < (int64_t) 4 * num_cus()) {
+        int64_t want = ((int64_t) 8 * num_cus() + tiles - 1) / tiles;
+        const int64_t max_splits = (a.n_kv + min_chunk - 1) / min_chunk;
+        if (want > max_splits) want = max_splits;
+        if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;
+        if (want < 1) want = 1;
+        int chunk  = (int) ((a.n_kv + want - 1) / want);
+        chunk      = (chunk + 31) / 32 * 32;
+        a.chunk    = chunk;
+        a.n_splits = (a.n_kv + chunk - 1) / chunk;
+    }
 
-    const int64_t nblocks = base_waves * a.n_splits;
+    const int64_t nblocks = tiles * a.n_splits;
     if (nblocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext: launch too large");
     const int D = (int) q->ne[0];
-    const int64_t gcols = (int64_t) a.ne3 * a.Hkv * ncols;
 
     if (a.n_splits > 1) {
-        const size_t o_bytes = (size_t) gcols * a.n_splits * D * sizeof(float);
-        const size_t ml_bytes = (size_t) gcols * a.n_splits * 2 * sizeof(float);
+        const size_t o_bytes  = (size_t) nblocks * 16 * D * sizeof(float);
+        const size_t ml_bytes = (size_t) nblocks * 16 * 2 * sizeof(float);
         void * ws = nullptr;
         vx_status rc = vx_workspace(st, o_bytes + ml_bytes, &ws);
         if (rc != VX_OK) return rc;
@@ -414,18 +491,13 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     }
 
     const bool f32 = k->type == VX_TYPE_F32;
-    const dim3 grid((unsigned) nblocks), block(64);
-    if (D == 64) {
-        if (f32) fattn_cols16_kernel<64, true><<<grid, block, 0, st>>>(a);
-        else     fattn_cols16_kernel<64, false><<<grid, block, 0, st>>>(a);
-    } else {
-        if (f32) fattn_cols16_kernel<128, true><<<grid, block, 0, st>>>(a);
-        else     fattn_cols16_kernel<128, false><<<grid, block, 0, st>>>(a);
-    }
+    if (D == 64) { if (f32) launch_cols16<64, true>(a, (int) nblocks, st); else launch_cols16<64, false>(a, (int) nblocks, st); }
+    else         { if (f32) launch_cols16<128, true>(a, (int) nblocks, st); else launch_cols16<128, false>(a, (int) nblocks, st); }
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
-        if (D == 64) fattn_combine_kernel<64><<<dim3((unsigned) gcols), dim3(64), 0, st>>>(a);
-        else         fattn_combine_kernel<128><<<dim3((unsigned) gcols), dim3(128), 0, st>>>(a);
+        const dim3 grid((unsigned) (tiles * 4));
+        if (D == 64) fattn_merge_kernel<64, 4><<<grid, dim3(256), 0, st>>>(a);
+        else         fattn_merge_kernel<128, 2><<<grid, dim3(256), 0, st>>>(a);
         VX_LAUNCH_CHECK();
     }
     return VX_OK;

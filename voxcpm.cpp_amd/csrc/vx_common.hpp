@@ -37,6 +37,9 @@ vx_status  vx_fail(vx_status st, const char * fmt, ...) __attribute__((format(pr
 // per-stream scratch memory, grown on demand (never shrinks); valid until the next call
 // that asks for more on the same stream
 vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr);
+// per-stream array of `count` ints that is all zero whenever no kernel of this library is
+// running on the stream: kernels that use it as arrival counters put every entry back to zero
+vx_status vx_counters(hipStream_t stream, size_t count, void ** ptr);
 
 // ---- host-side tensor predicates ---------------------------------------------------------
 static inline size_t vx_type_size(int type) {

@@ -14,7 +14,8 @@ struct workspace {
     size_t bytes = 0;
 };
 std::mutex                                    g_ws_mutex;
-std::unordered_map<unsigned long long, workspace> g_ws; // key: device << 48 ^ stream handle
+std::unordered_map<unsigned long long, workspace> g_ws;  // key: device << 56 ^ stream handle
+std::unordered_map<unsigned long long, workspace> g_cnt; // zero-initialised counters, same key
 
 } // namespace
 
@@ -55,6 +56,33 @@ vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr) {
             return vx_fail(VX_ERR_ALLOC, "workspace hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
         }
         ws.bytes = want;
+    }
+    *ptr = ws.ptr;
+    return VX_OK;
+}
+
+vx_status vx_counters(hipStream_t stream, size_t count, void ** ptr) {
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    const unsigned long long key = ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
+    const size_t bytes = count * sizeof(int);
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    workspace & ws = g_cnt[key];
+    if (ws.bytes < bytes) {
+        if (ws.ptr) {
+            VX_HIP(hipStreamSynchronize(stream));
+            VX_HIP(hipFree(ws.ptr));
+            ws.ptr   = nullptr;
+            ws.bytes = 0;
+        }
+        size_t want = bytes < 4096 ? 4096 : 2 * bytes;
+        hipError_t e = hipMalloc(&ws.ptr, want);
+        if (e != hipSuccess) {
+            ws.ptr = nullptr;
+            return vx_fail(VX_ERR_ALLOC, "counter hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+        }
+        ws.bytes = want;
+        VX_HIP(hipMemsetAsync(ws.ptr, 0, want, stream));
     }
     *ptr = ws.ptr;
     return VX_OK;
