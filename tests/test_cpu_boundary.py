@@ -1,0 +1,135 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+header declares, refuses work without a device instead of falling back, the supports_*
+truth table, and the ggml plugin's behaviour on a GPU-less host."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import reflib
+
+ROOT = reflib.ROOT
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "voxcpm_gfx950.h")).read()
+    return sorted(set(re.findall(r"VX_API\s+[\w\s\*]+?\b(vx_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(pkg):
+    lib = pkg.lib()
+    names = declared_symbols()
+    assert len(names) >= 25
+    assert set(names) == set(pkg.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def have_gpu(pkg):
+    return pkg.lib().vx_device_count() > 0
+
+
+def test_no_device_is_an_error_not_a_fallback(pkg):
+    lib = pkg.lib()
+    if have_gpu(pkg):
+        pytest.skip("a GPU is present")
+    assert lib.vx_device_count() == 0
+    assert lib.vx_init(0) == 1  # VX_ERR_NO_DEVICE
+    assert b"gfx950" in lib.vx_last_error()
+
+
+def D(pkg, ttype, ne, nb, data=0x1000):
+    return pkg.make_desc(ttype, ne, nb, data)
+
+
+def f32(pkg, ne):
+    nb = [4, 4 * ne[0], 4 * ne[0] * ne[1], 4 * ne[0] * ne[1] * ne[2]]
+    return D(pkg, pkg.F32, ne, nb)
+
+
+def f16(pkg, ne):
+    nb = [2, 2 * ne[0], 2 * ne[0] * ne[1], 2 * ne[0] * ne[1] * ne[2]]
+    return D(pkg, pkg.F16, ne, nb)
+
+
+def q8(pkg, ne):
+    rb = ne[0] // 32 * 34
+    return D(pkg, pkg.Q8_0, ne, [34, rb, rb * ne[1], rb * ne[1] * ne[2]])
+
+
+def test_supports_truth_table(pkg):
+    lib = pkg.lib()
+    # RMS_NORM: F32 only, equal shapes
+    assert lib.vx_supports_rms_norm(f32(pkg, [1024, 7, 1, 1]), f32(pkg, [1024, 7, 1, 1])) == 1
+    assert lib.vx_supports_rms_norm(f16(pkg, [1024, 7, 1, 1]), f16(pkg, [1024, 7, 1, 1])) == 0
+    assert lib.vx_supports_rms_norm(f32(pkg, [1024, 7, 1, 1]), f32(pkg, [1024, 8, 1, 1])) == 0
+    # ROPE: modes 0 (NORMAL) and 2 (NEOX) only
+    x = f32(pkg, [64, 16, 5, 1])
+    assert lib.vx_supports_rope(x, x, 64, 2) == 1 and lib.vx_supports_rope(x, x, 64, 0) == 1
+    assert lib.vx_supports_rope(x, x, 64, 8) == 0 and lib.vx_supports_rope(x, x, 64, 24) == 0
+    assert lib.vx_supports_rope(x, x, 66, 2) == 0 and lib.vx_supports_rope(x, x, 63, 2) == 0
+    # FLASH_ATTN_EXT: D in {64,128}, K/V same type F16|F32, mask F16, GQA divisibility
+    q, dst = f32(pkg, [64, 1, 16, 2]), f32(pkg, [64, 16, 1, 2])
+    k = f16(pkg, [64, 4096, 2, 2])
+    assert lib.vx_supports_flash_attn_ext(q, k, k, None, dst) == 1
+    assert lib.vx_supports_flash_attn_ext(q, k, f32(pkg, [64, 4096, 2, 2]), None, dst) == 0
+    assert lib.vx_supports_flash_attn_ext(q, f16(pkg, [64, 4096, 3, 2]), f16(pkg, [64, 4096, 3, 2]), None, dst) == 0
+    q80, d80 = f32(pkg, [80, 1, 16, 2]), f32(pkg, [80, 16, 1, 2])
+    assert lib.vx_supports_flash_attn_ext(q80, f16(pkg, [80, 64, 2, 2]), f16(pkg, [80, 64, 2, 2]), None, d80) == 0
+    assert lib.vx_supports_flash_attn_ext(q, k, k, f16(pkg, [4096, 1, 1, 1]), dst) == 1
+    assert lib.vx_supports_flash_attn_ext(q, k, k, f32(pkg, [4096, 1, 1, 1]), dst) == 0
+    # MUL_MAT: Q8_0 / F16 / F32 weights x F32 activations
+    x2, o2 = f32(pkg, [1024, 2, 1, 1]), f32(pkg, [4096, 2, 1, 1])
+    assert lib.vx_supports_mul_mat(q8(pkg, [1024, 4096, 1, 1]), x2, o2) == 1
+    assert lib.vx_supports_mul_mat(f16(pkg, [1024, 4096, 1, 1]), x2, o2) == 1
+    assert lib.vx_supports_mul_mat(q8(pkg, [1024, 4096, 1, 1]), f16(pkg, [1024, 2, 1, 1]), o2) == 0
+    assert lib.vx_supports_mul_mat(q8(pkg, [1024, 4096, 1, 1]), f32(pkg, [512, 2, 1, 1]), o2) == 0
+    transposed = D(pkg, pkg.F32, [1024, 4096, 1, 1], [4 * 4096, 4, 4 * 1024 * 4096, 4 * 1024 * 4096])
+    assert lib.vx_supports_mul_mat(transposed, x2, o2) == 0
+
+
+def test_ops_validate_before_touching_the_device(pkg):
+    """Contract violations are reported by status + message; nothing is launched."""
+    lib = pkg.lib()
+    x = f32(pkg, [64, 16, 5, 1])
+    assert lib.vx_rms_norm(x, x, -1.0, None) == 3                       # VX_ERR_INVALID: eps < 0
+    assert lib.vx_rms_norm(f16(pkg, [64, 1, 1, 1]), f16(pkg, [64, 1, 1, 1]), 1e-5, None) == 2  # UNSUPPORTED
+    assert b"F32" in lib.vx_last_error()
+    assert lib.vx_flash_attn_ext(None, None, None, None, None, None, 1.0, 0.0, 0.0, None) == 3
+    q, dst = f32(pkg, [64, 1, 16, 2]), f32(pkg, [64, 16, 1, 2])
+    k = f16(pkg, [64, 4096, 2, 2])
+    assert lib.vx_flash_attn_ext(q, k, k, None, None, dst, 0.125, 8.0, 0.0, None) == 3  # max_bias needs a mask
+    assert lib.vx_mul_mat(q8(pkg, [1024, 8, 1, 1]), f32(pkg, [1024, 2, 1, 1]), f32(pkg, [8, 2, 1, 1]), 7, None) == 3
+
+
+def test_kv_views_match_reference_layout(pkg):
+    """MiniCPMKVCache view shapes (reference tests/test_minicpm.cpp:775-809: cache (2 layers,
+    2 kv heads, max_length 16, head_dim 8); get_k(seq 4) -> [8,4,2]; get_k_slot(3) -> [8,2,1];
+    get_v_batch(5, 2) -> [8,2,2]) and the oracle's stride/offset formulas."""
+    lib, orc = pkg.lib(), reflib.load_oracle()
+    cache = pkg.make_desc(pkg.F32, [8, 16, 2, 1], [4, 32, 512, 1024], 0x10000)
+    v = pkg.VxTensor()
+    assert lib.vx_kv_read_view(cache, 4, v) == 0 and list(v.ne)[:3] == [8, 4, 2]
+    assert lib.vx_kv_read_view(cache, 7, v) == 0 and list(v.ne)[:3] == [8, 7, 2]
+    assert lib.vx_kv_write_view(cache, 3, 1, v) == 0 and list(v.ne)[:3] == [8, 2, 1]
+    assert lib.vx_kv_write_view(cache, 5, 2, v) == 0 and list(v.ne)[:3] == [8, 2, 2]
+    ne, nb, off = (C.c_int64 * 3)(), (C.c_uint64 * 3)(), C.c_uint64()
+    orc.orc_kv_write_view(8, 16, 2, 4, 5, 2, ne, nb, C.byref(off))
+    assert list(v.nb)[:3] == list(nb) and v.data - 0x10000 == off.value == 5 * 32
+    assert lib.vx_kv_read_view(cache, 17, v) == 3 and lib.vx_kv_write_view(cache, 15, 2, v) == 3
+
+
+def test_plugin_on_a_gpuless_host(pkg, ref):
+    """ggml's loader must reject the plugin cleanly (score 0) when no gfx950 device exists,
+    leaving ggml-cpu as the only device."""
+    if have_gpu(pkg):
+        pytest.skip("a GPU is present")
+    if not os.path.exists(pkg.PLUGIN_PATH):
+        pytest.skip("plugin not built")
+    plug = C.CDLL(pkg.PLUGIN_PATH)
+    assert plug.ggml_backend_score() == 0
+    assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) != 0
+    names = [ref.rh_device_name(i).decode() for i in range(ref.rh_device_count())]
+    assert names == ["CPU"]

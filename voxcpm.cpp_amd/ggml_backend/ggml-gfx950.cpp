@@ -1,0 +1,484 @@
+// ggml-gfx950.cpp -- a ggml backend for AMD MI355X (gfx950) that claims the operators of
+// VoxCPM.cpp's attention hot path and nothing else:
+//
+//     GGML_OP_FLASH_ATTN_EXT, GGML_OP_ROPE, GGML_OP_SOFT_MAX, GGML_OP_RMS_NORM,
+//     GGML_OP_MUL_MAT (Q8_0 / F16 / F32 weights, F32 activations)
+//
+// plus the view ops every backend accepts.  Everything else is answered with
+// supports_op() == false, so ggml's scheduler keeps it on ggml-cpu.  The file is host-only
+// C++: it implements ggml's five backend vtables (ggml/src/ggml-backend-impl.h:17-204 of
+// the reference checkout) and forwards every claimed node, unchanged, to the C ABI of
+// libvoxcpm_gfx950.so (include/voxcpm_gfx950.h), where the hand-written HIP kernels live.
+//
+// It is built against the reference's ggml headers and loaded like any dynamically loaded
+// ggml backend: ggml_backend_load("libggml-gfx950.so") or GGML_BACKEND_PATH
+// (ggml/src/ggml-backend-reg.cpp:194-238, 561-565).  ggml's own symbols are resolved from
+// the host process.  With no gfx950 device visible, ggml_backend_score() returns 0 and the
+// registry reports zero devices; nothing aborts.
+#include "ggml-backend-impl.h"
+#include "ggml-backend.h"
+#include "ggml-impl.h"
+#include "ggml.h"
+
+#include "voxcpm_gfx950.h"
+
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace {
+
+constexpr size_t GFX950_ALIGNMENT = 256;
+
+// ------------------------------------------------------------------ tensor descriptors
+vx_tensor to_vx(const ggml_tensor * t) {
+    vx_tensor v;
+    v.type = (int32_t) t->type;
+    v._pad = 0;
+    for (int i = 0; i < 4; ++i) {
+        v.ne[i] = t->ne[i];
+        v.nb[i] = t->nb[i];
+    }
+    v.data = t->data;
+    return v;
+}
+
+bool type_known(ggml_type t) {
+    return t == GGML_TYPE_F32 || t == GGML_TYPE_F16 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_I32;
+}
+
+int mul_mat_act_mode() {
+    static const int mode = [] {
+        const char * e = getenv("GGML_GFX950_MUL_MAT_ACT");
+        return (e && strcmp(e, "q8") == 0) ? VX_ACT_Q8 : VX_ACT_FLOAT;
+    }();
+    return mode;
+}
+
+// --------------------------------------------------------------------- per-device state
+struct device_ctx {
+    int         index;
+    std::string name;
+    std::string description;
+};
+
+struct backend_ctx {
+    int       device;
+    vx_stream stream;
+};
+
+struct buffer_ctx {
+    int    device;
+    void * base;
+};
+
+ggml_backend_buffer_type_t device_buffer_type(ggml_backend_dev_t dev);
+
+// ------------------------------------------------------------------------------ buffers
+void buffer_free(ggml_backend_buffer_t buffer) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    vx_init(ctx->device);
+    vx_free(ctx->base);
+    delete ctx;
+}
+
+void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) buffer->context)->base; }
+
+void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    vx_init(ctx->device);
+    if (vx_memset((char *) tensor->data + offset, value, size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
+        GGML_ABORT("ggml-gfx950: memset_tensor failed: %s", vx_last_error());
+}
+
+void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    vx_init(ctx->device);
+    if (vx_memcpy_h2d((char *) tensor->data + offset, data, size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
+        GGML_ABORT("ggml-gfx950: set_tensor failed: %s", vx_last_error());
+}
+
+void buffer_get_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    vx_init(ctx->device);
+    if (vx_memcpy_d2h(data, (const char *) tensor->data + offset, size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
+        GGML_ABORT("ggml-gfx950: get_tensor failed: %s", vx_last_error());
+}
+
+bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, ggml_tensor * dst) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
+    vx_init(ctx->device);
+    vx_status rc;
+    if (ggml_backend_buffer_is_host(src->buffer)) {
+        rc = vx_memcpy_h2d(dst->data, src->data, ggml_nbytes(src), nullptr);
+    } else if (src->buffer->buft == buffer->buft) {
+        rc = vx_memcpy_d2d(dst->data, src->data, ggml_nbytes(src), nullptr);
+    } else {
+        return false;
+    }
+    if (rc == VX_OK) rc = vx_stream_synchronize(nullptr);
+    if (rc != VX_OK) GGML_ABORT("ggml-gfx950: cpy_tensor failed: %s", vx_last_error());
+    return true;
+}
+
+void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    vx_init(ctx->device);
+    if (vx_memset(ctx->base, value, buffer->size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
+        GGML_ABORT("ggml-gfx950: clear failed: %s", vx_last_error());
+}
+
+const ggml_backend_buffer_i buffer_iface = {
+    /* .free_buffer   = */ buffer_free,
+    /* .get_base      = */ buffer_get_base,
+    /* .init_tensor   = */ nullptr,
+    /* .memset_tensor = */ buffer_memset_tensor,
+    /* .set_tensor    = */ buffer_set_tensor,
+    /* .get_tensor    = */ buffer_get_tensor,
+    /* .cpy_tensor    = */ buffer_cpy_tensor,
+    /* .clear         = */ buffer_clear,
+    /* .reset         = */ nullptr,
+};
+
+// -------------------------------------------------------------------- device buffer type
+const char * buft_get_name(ggml_backend_buffer_type_t buft) {
+    return ((device_ctx *) buft->device->context)->name.c_str();
+}
+
+ggml_backend_buffer_t buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    device_ctx * dctx = (device_ctx *) buft->device->context;
+    if (vx_init(dctx->index) != VX_OK) {
+        GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
+        return nullptr;
+    }
+    void * base = nullptr;
+    if (vx_malloc(&base, size) != VX_OK) {
+        GGML_LOG_ERROR("ggml-gfx950: allocating %zu bytes on %s failed: %s\n", size, dctx->name.c_str(), vx_last_error());
+        return nullptr;
+    }
+    return ggml_backend_buffer_init(buft, buffer_iface, new buffer_ctx{ dctx->index, base }, size);
+}
+
+size_t buft_get_alignment(ggml_backend_buffer_type_t) { return GFX950_ALIGNMENT; }
+
+bool buft_is_host(ggml_backend_buffer_type_t) { return false; }
+
+// ---------------------------------------------------------------- pinned host buffer type
+// System memory allocated with hipHostMalloc: when ggml's scheduler puts its CPU-side compute
+// buffers here (as VoxCPM.cpp does for CUDA, src/backend.cpp:275-281), split copies are DMA
+// from pinned memory.  Tensor access is ggml's own CPU buffer code.
+void host_buffer_free(ggml_backend_buffer_t buffer) { vx_free_host(buffer->context); }
+
+const char * host_buft_get_name(ggml_backend_buffer_type_t) { return "GFX950_Host"; }
+
+ggml_backend_buffer_t host_buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    void * ptr = nullptr;
+    if (vx_malloc_host(&ptr, size) != VX_OK) {
+        GGML_LOG_WARN("ggml-gfx950: pinned allocation of %zu bytes failed (%s), using pageable memory\n", size, vx_last_error());
+        return ggml_backend_buft_alloc_buffer(ggml_backend_cpu_buffer_type(), size);
+    }
+    ggml_backend_buffer_t buffer = ggml_backend_cpu_buffer_from_ptr(ptr, size);
+    buffer->buft              = buft;
+    buffer->iface.free_buffer = host_buffer_free;
+    return buffer;
+}
+
+size_t host_buft_get_alignment(ggml_backend_buffer_type_t) { return GFX950_ALIGNMENT; }
+bool   host_buft_is_host(ggml_backend_buffer_type_t) { return true; }
+
+// ----------------------------------------------------------------------------- supports_op
+bool supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
+    for (int i = 0; i < GGML_MAX_SRC; ++i)
+        if (op->src[i] && !type_known(op->src[i]->type)) return false;
+
+    switch (op->op) {
+        case GGML_OP_NONE:
+        case GGML_OP_RESHAPE:
+        case GGML_OP_VIEW:
+        case GGML_OP_PERMUTE:
+        case GGML_OP_TRANSPOSE:
+            return true;
+        case GGML_OP_RMS_NORM: {
+            const vx_tensor s = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_rms_norm(&s, &d) != 0;
+        }
+        case GGML_OP_ROPE: {
+            const int n_dims = ((const int32_t *) op->op_params)[1];
+            const int mode   = ((const int32_t *) op->op_params)[2];
+            if (op->src[1] == nullptr || op->src[1]->type != GGML_TYPE_I32) return false;
+            if (op->src[2] && (op->src[2]->type != GGML_TYPE_F32 || op->src[2]->ne[0] < n_dims / 2)) return false;
+            const vx_tensor s = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_rope(&s, &d, n_dims, mode) != 0;
+        }
+        case GGML_OP_SOFT_MAX: {
+            const vx_tensor s = to_vx(op->src[0]), d = to_vx(op);
+            vx_tensor m;
+            if (op->src[1]) m = to_vx(op->src[1]);
+            if (op->src[2] && (op->src[2]->type != GGML_TYPE_F32 || op->src[2]->ne[0] != op->src[0]->ne[2])) return false;
+            return vx_supports_soft_max(&s, op->src[1] ? &m : nullptr, &d) != 0;
+        }
+        case GGML_OP_FLASH_ATTN_EXT: {
+            const vx_tensor q = to_vx(op->src[0]), k = to_vx(op->src[1]), v = to_vx(op->src[2]), d = to_vx(op);
+            vx_tensor m;
+            if (op->src[3]) m = to_vx(op->src[3]);
+            if (op->src[4] && (op->src[4]->type != GGML_TYPE_F32 || op->src[4]->ne[0] != op->src[0]->ne[2])) return false;
+            return vx_supports_flash_attn_ext(&q, &k, &v, op->src[3] ? &m : nullptr, &d) != 0;
+        }
+        case GGML_OP_MUL_MAT: {
+            const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
+            return vx_supports_mul_mat(&a, &b, &d) != 0;
+        }
+        default:
+            return false;
+    }
+}
+
+// --------------------------------------------------------------------------- graph_compute
+vx_status compute_node(backend_ctx * ctx, ggml_tensor * node) {
+    switch (node->op) {
+        case GGML_OP_RMS_NORM: {
+            float eps;
+            memcpy(&eps, node->op_params, sizeof(float));
+            const vx_tensor s = to_vx(node->src[0]), d = to_vx(node);
+            return vx_rms_norm(&s, &d, eps, ctx->stream);
+        }
+        case GGML_OP_ROPE: {
+            const int32_t * p = (const int32_t *) node->op_params; // ggml.c:4112-4123
+            float f[6];
+            memcpy(f, p + 5, sizeof(f));
+            const vx_tensor s = to_vx(node->src[0]), d = to_vx(node);
+            return vx_rope(&s, (const int32_t *) node->src[1]->data, node->src[2] ? (const float *) node->src[2]->data : nullptr,
+                           &d, p[1], p[2], p[4], f[0], f[1], f[2], f[3], f[4], f[5], ctx->stream);
+        }
+        case GGML_OP_SOFT_MAX: {
+            float scale, max_bias;
+            memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+            const vx_tensor s = to_vx(node->src[0]), d = to_vx(node);
+            vx_tensor m;
+            if (node->src[1]) m = to_vx(node->src[1]);
+            return vx_soft_max(&s, node->src[1] ? &m : nullptr, node->src[2] ? (const float *) node->src[2]->data : nullptr,
+                               &d, scale, max_bias, ctx->stream);
+        }
+        case GGML_OP_FLASH_ATTN_EXT: {
+            float scale, max_bias, softcap; // ggml.c:5312-5313
+            memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+            memcpy(&softcap, (const float *) node->op_params + 2, sizeof(float));
+            const vx_tensor q = to_vx(node->src[0]), k = to_vx(node->src[1]), v = to_vx(node->src[2]), d = to_vx(node);
+            vx_tensor m;
+            if (node->src[3]) m = to_vx(node->src[3]);
+            return vx_flash_attn_ext(&q, &k, &v, node->src[3] ? &m : nullptr,
+                                     node->src[4] ? (const float *) node->src[4]->data : nullptr, &d, scale, max_bias,
+                                     softcap, ctx->stream);
+        }
+        case GGML_OP_MUL_MAT: {
+            const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]), d = to_vx(node);
+            return vx_mul_mat(&a, &b, &d, mul_mat_act_mode(), ctx->stream);
+        }
+        default:
+            return VX_ERR_UNSUPPORTED;
+    }
+}
+
+const char * backend_get_name(ggml_backend_t backend) {
+    return ((device_ctx *) backend->device->context)->name.c_str();
+}
+
+void backend_free(ggml_backend_t backend) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    vx_init(ctx->device);
+    vx_stream_synchronize(ctx->stream);
+    vx_stream_destroy(ctx->stream);
+    delete ctx;
+    delete backend;
+}
+
+void backend_synchronize(ggml_backend_t backend) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    vx_init(ctx->device);
+    if (vx_stream_synchronize(ctx->stream) != VX_OK) GGML_ABORT("ggml-gfx950: synchronize failed: %s", vx_last_error());
+}
+
+void backend_set_tensor_async(ggml_backend_t backend, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    vx_init(ctx->device);
+    if (vx_memcpy_h2d((char *) tensor->data + offset, data, size, ctx->stream) != VX_OK)
+        GGML_ABORT("ggml-gfx950: set_tensor_async failed: %s", vx_last_error());
+}
+
+void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    vx_init(ctx->device);
+    if (vx_memcpy_d2h(data, (const char *) tensor->data + offset, size, ctx->stream) != VX_OK)
+        GGML_ABORT("ggml-gfx950: get_tensor_async failed: %s", vx_last_error());
+}
+
+ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    if (vx_init(ctx->device) != VX_OK) {
+        GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
+        return GGML_STATUS_FAILED;
+    }
+    for (int i = 0; i < cgraph->n_nodes; ++i) {
+        ggml_tensor * node = cgraph->nodes[i];
+        // the same two skips ggml-cpu applies (ggml/src/ggml-cpu/ggml-cpu.c:2956-2966)
+        if (ggml_op_is_empty(node->op) || ggml_is_empty(node)) continue;
+        if ((node->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+        const vx_status rc = compute_node(ctx, node);
+        if (rc != VX_OK) {
+            GGML_LOG_ERROR("ggml-gfx950: node %d (%s, op %s) failed with status %d: %s\n", i, node->name,
+                           ggml_op_name(node->op), (int) rc, rc == VX_ERR_UNSUPPORTED && !*vx_last_error() ? "operator not claimed by this backend" : vx_last_error());
+            return GGML_STATUS_FAILED;
+        }
+    }
+    return GGML_STATUS_SUCCESS;
+}
+
+const ggml_backend_i backend_iface = {
+    /* .get_name           = */ backend_get_name,
+    /* .free               = */ backend_free,
+    /* .set_tensor_async   = */ backend_set_tensor_async,
+    /* .get_tensor_async   = */ backend_get_tensor_async,
+    /* .cpy_tensor_async   = */ nullptr,
+    /* .synchronize        = */ backend_synchronize,
+    /* .graph_plan_create  = */ nullptr,
+    /* .graph_plan_free    = */ nullptr,
+    /* .graph_plan_update  = */ nullptr,
+    /* .graph_plan_compute = */ nullptr,
+    /* .graph_compute      = */ backend_graph_compute,
+    /* .event_record       = */ nullptr,
+    /* .event_wait         = */ nullptr,
+    /* .graph_optimize     = */ nullptr,
+};
+
+ggml_guid_t backend_guid() {
+    static ggml_guid guid = { 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x2d, 0x76, 0x6f, 0x78, 0x63, 0x70, 0x6d, 0x2d, 0x30, 0x31 };
+    return &guid;
+}
+
+// ---------------------------------------------------------------------------------- device
+const char * dev_get_name(ggml_backend_dev_t dev) { return ((device_ctx *) dev->context)->name.c_str(); }
+const char * dev_get_description(ggml_backend_dev_t dev) { return ((device_ctx *) dev->context)->description.c_str(); }
+
+void dev_get_memory(ggml_backend_dev_t dev, size_t * free, size_t * total) {
+    *free = *total = 0;
+    vx_device_info(((device_ctx *) dev->context)->index, nullptr, 0, free, total, nullptr);
+}
+
+enum ggml_backend_dev_type dev_get_type(ggml_backend_dev_t) { return GGML_BACKEND_DEVICE_TYPE_GPU; }
+
+void dev_get_props(ggml_backend_dev_t dev, ggml_backend_dev_props * props) {
+    props->name        = dev_get_name(dev);
+    props->description = dev_get_description(dev);
+    props->type        = dev_get_type(dev);
+    props->device_id   = nullptr;
+    dev_get_memory(dev, &props->memory_free, &props->memory_total);
+    props->caps = { /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
+}
+
+ggml_backend_t dev_init_backend(ggml_backend_dev_t dev, const char *) {
+    device_ctx * dctx = (device_ctx *) dev->context;
+    if (vx_init(dctx->index) != VX_OK) {
+        GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
+        return nullptr;
+    }
+    vx_stream stream = nullptr;
+    if (vx_stream_create(&stream) != VX_OK) {
+        GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
+        return nullptr;
+    }
+    return new ggml_backend{ backend_guid(), backend_iface, dev, new backend_ctx{ dctx->index, stream } };
+}
+
+ggml_backend_buffer_type_t dev_get_host_buffer_type(ggml_backend_dev_t dev) {
+    static ggml_backend_buffer_type host_buft = {
+        /* .iface   = */ { host_buft_get_name, host_buft_alloc_buffer, host_buft_get_alignment, nullptr, nullptr, host_buft_is_host },
+        /* .device  = */ nullptr,
+        /* .context = */ nullptr,
+    };
+    host_buft.device = dev;
+    return &host_buft;
+}
+
+bool dev_supports_buft(ggml_backend_dev_t dev, ggml_backend_buffer_type_t buft) { return buft == device_buffer_type(dev); }
+
+const ggml_backend_device_i device_iface = {
+    /* .get_name             = */ dev_get_name,
+    /* .get_description      = */ dev_get_description,
+    /* .get_memory           = */ dev_get_memory,
+    /* .get_type             = */ dev_get_type,
+    /* .get_props            = */ dev_get_props,
+    /* .init_backend         = */ dev_init_backend,
+    /* .get_buffer_type      = */ device_buffer_type,
+    /* .get_host_buffer_type = */ dev_get_host_buffer_type,
+    /* .buffer_from_host_ptr = */ nullptr,
+    /* .supports_op          = */ supports_op,
+    /* .supports_buft        = */ dev_supports_buft,
+    /* .offload_op           = */ nullptr,
+    /* .event_new            = */ nullptr,
+    /* .event_free           = */ nullptr,
+    /* .event_synchronize    = */ nullptr,
+};
+
+// --------------------------------------------------------------------------------- registry
+struct reg_ctx {
+    std::vector<ggml_backend_device *>      devices;
+    std::vector<ggml_backend_buffer_type *> bufts;
+};
+
+reg_ctx * registry_state(ggml_backend_reg_t reg) {
+    static reg_ctx ctx;
+    static std::once_flag once;
+    std::call_once(once, [reg] {
+        const int n = vx_device_count();
+        for (int i = 0; i < n; ++i) {
+            char desc[256] = "";
+            vx_device_info(i, desc, sizeof(desc), nullptr, nullptr, nullptr);
+            device_ctx * dctx = new device_ctx{ i, "GFX950_" + std::to_string(i), desc };
+            ggml_backend_device * dev = new ggml_backend_device{ device_iface, reg, dctx };
+            ctx.devices.push_back(dev);
+            ctx.bufts.push_back(new ggml_backend_buffer_type{
+                { buft_get_name, buft_alloc_buffer, buft_get_alignment, nullptr, nullptr, buft_is_host }, dev, nullptr });
+        }
+    });
+    return &ctx;
+}
+
+ggml_backend_buffer_type_t device_buffer_type(ggml_backend_dev_t dev) {
+    return registry_state(dev->reg)->bufts[((device_ctx *) dev->context)->index];
+}
+
+const char * reg_get_name(ggml_backend_reg_t) { return "GFX950"; }
+size_t       reg_get_device_count(ggml_backend_reg_t reg) { return registry_state(reg)->devices.size(); }
+
+ggml_backend_dev_t reg_get_device(ggml_backend_reg_t reg, size_t index) {
+    reg_ctx * ctx = registry_state(reg);
+    GGML_ASSERT(index < ctx->devices.size());
+    return ctx->devices[index];
+}
+
+void * reg_get_proc_address(ggml_backend_reg_t, const char *) { return nullptr; }
+
+} // namespace
+
+extern "C" {
+
+GGML_BACKEND_API ggml_backend_reg_t ggml_backend_gfx950_reg(void) {
+    static ggml_backend_reg reg = {
+        /* .api_version = */ GGML_BACKEND_API_VERSION,
+        /* .iface       = */ { reg_get_name, reg_get_device_count, reg_get_device, reg_get_proc_address },
+        /* .context     = */ nullptr,
+    };
+    return &reg;
+}
+
+// entry points ggml's loader looks up (ggml/src/ggml-backend-impl.h:215-251)
+GGML_BACKEND_API ggml_backend_reg_t ggml_backend_init(void) { return ggml_backend_gfx950_reg(); }
+GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_count() > 0 ? 100 : 0; }
+
+} // extern "C"
