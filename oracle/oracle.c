@@ -327,7 +327,8 @@ int orc_rope(const orc_tensor * src, const int32_t * pos, const float * freq_fac
             float mscale = attn_factor;
             if (ext_factor != 0.0f) {
                 const float ramp_mix = yarn_ramp(corr_dims[0], corr_dims[1], (int)i0) * ext_factor;
-                th = theta_interp * (1 - ramp_mix) + theta_extrap * ramp_mix;
+                /* the reference's x86 build contracts this sum into one fused multiply-add */
+                th = fmaf(theta_interp, (1 - ramp_mix), theta_extrap * ramp_mix);
                 mscale *= 1.0f + 0.1f * logf(1.0f / freq_scale);
             }
             cache[i0 + 0] = cosf(th) * mscale;

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(256) void rope_kernel(const char * __restrict__ src
         // rope_yarn_ramp takes i0/2 as an int and clamps in fp32 (ops.cpp:5589-5592)
         const float yv       = ((float) ip - p.corr_lo) / fmaxf(0.001f, p.corr_hi - p.corr_lo);
         const float ramp_mix = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * p.ext_factor;
-        th                   = theta_interp * (1.0f - ramp_mix) + theta_extrap * ramp_mix;
+        // ggml-cpu's x86 build contracts this sum into one fused multiply-add
+        th                   = fmaf(theta_interp, 1.0f - ramp_mix, theta_extrap * ramp_mix);
         mscale *= 1.0f + 0.1f * logf(1.0f / p.freq_scale);
     }
     const float c  = cosf(th) * mscale;
