@@ -249,8 +249,8 @@ def main():
             others[f"cfg2_decode_attn_L{L2}"] = {"us_per_layer": s / LAYERS * 1e6,
                                                   "GB/s": LAYERS * kv_bytes(2, L2) / s / 1e9}
             del keep
-        st, one, keep = decode_attn_setup(pkg, 16, 8192, 4)
-        s = timer.run(graphed(st, side), iters=100, warmup=10) / 4
+        st, one, keep = decode_attn_setup(pkg, 16, 8192, LAYERS)  # 1.5 GiB of KV: no cache reuse
+        s = timer.run(graphed(st, side), iters=20, warmup=3) / LAYERS
         others["cfg5_decode_attn_B16_L8192"] = {"us_per_layer": s * 1e6, "GB/s": kv_bytes(16, 8192) / s / 1e9,
                                                 "hbm_frac": kv_bytes(16, 8192) / s / 1e9 / HBM_PEAK_GBS}
         del keep

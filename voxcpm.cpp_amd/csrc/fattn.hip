@@ -108,8 +108,8 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
 }
 
 // One wave (= one block) = 16 columns x one key range.
-template <int D, bool KV_F32, bool HAS_MASK>
-__global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
+template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fattn_cols16_kernel(const fa_args a) {
     constexpr int NP  = D / 32;          // MFMAs along the head dimension
     constexpr int SEG = D / 4;           // elements of a row owned by lane-group j
     constexpr int ES  = KV_F32 ? 4 : 2;  // bytes per K/V element
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     const __half * mrow = nullptr;
     if constexpr (HAS_MASK) {
         slope = vx_alibi_slope(a.max_bias, (uint32_t) head, a.n_head_log2, a.m0, a.m1) * 1.44269504088896341f;
-        mrow  = (const __half *) (a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (head % a.nem2) * a.nbm2 + (uint64_t) (b % a.nem3) * a.nbm3);
+        if (a.mask) mrow = (const __half *) (a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (head % a.nem2) * a.nbm2 + (uint64_t) (b % a.nem3) * a.nbm3);
     }
 
     float4_t o[NP][2];
@@ -195,18 +195,21 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
     float l = 0.0f;      // this lane's share of the running sum
 
     auto consume = [&](const kv_tile<NP, KV_F32> & t, int kb) {
-        // additive mask of this lane's 8 keys (kb + 16h + 4j + r); loads are clamped, the
-        // out-of-range keys are switched off below
+        // additive mask of this lane's 8 keys (kb + 16h + 4j + r); loads are clamped, keys
+        // past the end of the range (only in a wave's last tile) are switched off
+        const bool tail = kb + 32 > kv1; // wave-uniform
         float mv[2][4];
+        if (HAS_MASK || tail) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = kb + 16 * h + 4 * j + r;
-                float x = 0.0f;
-                if constexpr (HAS_MASK) x = slope * __half2float(mrow[min(key, a.n_kv - 1)]); // slope carries log2(e)
-                mv[h][r] = key < kv1 ? x : -INFINITY;
-            }
+                for (int r = 0; r < 4; ++r) {
+                    const int key = kb + 16 * h + 4 * j + r;
+                    float x = 0.0f;
+                    if constexpr (HAS_MASK) { if (mrow) x = slope * __half2float(mrow[min(key, a.n_kv - 1)]); } // slope carries log2(e)
+                    mv[h][r] = key < kv1 ? x : -INFINITY;
+                }
+        }
 
         // ---- S^T for the two 16-key halves
         float4_t s[2];
@@ -230,8 +233,8 @@ __global__ __launch_bounds__(64) void fattn_cols16_kernel(const fa_args a) {
             for (int r = 0; r < 4; ++r) {
                 // a.scale carries log2(e) (the soft cap path applies it after tanh)
                 float x = s[h][r] * a.scale;
-                if (a.softcap != 0.0f) x = a.softcap * tanhf(x);
-                x += mv[h][r];
+                if constexpr (SOFTCAP) x = a.softcap * tanhf(x);
+                if (HAS_MASK || tail) x += mv[h][r];
                 s[h][r] = x;
                 cmax = fmaxf(cmax, x);
             }
@@ -388,8 +391,14 @@ bool aligned16(const vx_tensor * t) {
 
 template <int D, bool KV_F32>
 void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
-    if (a.mask) fattn_cols16_kernel<D, KV_F32, true><<<dim3((unsigned) nblocks), dim3(64), 0, st>>>(a);
-    else        fattn_cols16_kernel<D, KV_F32, false><<<dim3((unsigned) nblocks), dim3(64), 0, st>>>(a);
+    const dim3 grid((unsigned) nblocks), block(64);
+    if (a.softcap != 0.0f) { // rare: always take the masked variant
+        fattn_cols16_kernel<D, KV_F32, true, true><<<grid, block, 0, st>>>(a);
+    } else if (a.mask) {
+        fattn_cols16_kernel<D, KV_F32, true, false><<<grid, block, 0, st>>>(a);
+    } else {
+        fattn_cols16_kernel<D, KV_F32, false, false><<<grid, block, 0, st>>>(a);
+    }
 }
 
 } // namespace
@@ -459,13 +468,13 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     const int64_t tiles = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
 
     // Work split.  Enough 16-column tiles to fill the chip: one wave per tile over all keys.
-    // Otherwise cut the keys (flash-decoding) aiming at ~8 waves per CU, at least `min_chunk`
+    // Otherwise cut the keys (flash-decoding) aiming at ~4 waves per CU, at least `min_chunk`
     // keys per wave, and merge the partials with a second small kernel.
-    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 128; }();
+    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 64; }();
     a.n_splits = 1;
     a.chunk    = (a.n_kv + 31) / 32 * 32;
     if (tiles < (int64_t) 4 * num_cus()) {
-        int64_t want = ((int64_t) 8 * num_cus() + tiles - 1) / tiles;
+        int64_t want = ((int64_t) 4 * num_cus() + tiles - 1) / tiles;
         const int64_t max_splits = (a.n_kv + min_chunk - 1) / min_chunk;
         if (want > max_splits) want = max_splits;
         if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;
