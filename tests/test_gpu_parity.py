@@ -298,6 +298,42 @@ def test_fa_cfg5_shape_properties(gpu):
         assert err <= FA_TOL
 
 
+@pytest.mark.parametrize("case", ["causal", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
+def test_fa_prefill_kernel(gpu, case):
+    """Shapes large enough to take the LDS-tiled prefill kernel (>= 256 columns per KV head,
+    >= 64 work-groups)."""
+    say(f"flash_attn prefill kernel: {case}")
+    B, Hq, Hkv, T, KV = 4, 16, 2, 512, 512
+    mask, sinks, max_bias, kvt = None, None, 0.0, np.float16
+    if case == "causal":
+        mask = reflib.causal_mask(T, KV)
+    elif case == "past":
+        T, KV = 300, 700
+        mask = reflib.causal_mask(T, KV, n_past=KV - T)
+    elif case == "f32kv":
+        kvt = np.float32
+        mask = reflib.causal_mask(T, KV)
+    elif case == "random_mask":
+        T, KV = 256, 333
+        mm = rng("pf", "m").standard_normal((1, 1, T, KV)).astype(np.float32)
+        mm[rng("pf", "d").random(mm.shape) < 0.4] = -np.inf
+        mm[:, :, 17, :] = -np.inf
+        mask = mm.astype(np.float16)
+    elif case == "mha":
+        B, Hq, Hkv, T, KV = 2, 4, 4, 2048, 128
+        mask = None
+    elif case == "sinks_alibi":
+        T, KV = 256, 256
+        mask = rng("pf", "am").standard_normal((1, 1, T, KV)).astype(np.float16)
+        sinks = rng("pf", "s").standard_normal(Hq).astype(np.float32)
+        max_bias = 8.0
+    elif case == "ragged":
+        B, T, KV = 5, 250, 999
+        mask = reflib.causal_mask(T, KV, n_past=KV - T)
+    q, k, v = qkv(("pf", case), B, Hq, Hkv, T, KV, kv_dtype=kvt)
+    fa_case(gpu, q, k, v, mask, max_bias=max_bias, sinks=sinks, name=f"prefill {case}")
+
+
 # ------------------------------------------------------------------------------- MUL_MAT
 def mm_inputs(tag, M, K, N, batch=()):
     w = (rng(tag, "w").standard_normal(batch + (M, K)) * 0.02).astype(np.float32)

@@ -441,6 +441,13 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext: max_bias > 0 requires a mask");
 
     hipStream_t st = (hipStream_t) stream;
+    {   // many query rows: the LDS-tiled kernel
+        static const bool no_prefill = getenv("VX_FA_NO_PREFILL") != nullptr;
+        if (!no_prefill) {
+            const vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, dst, scale, max_bias, logit_softcap, st);
+            if (rc != VX_ERR_UNSUPPORTED) return rc;
+        }
+    }
     fa_args a;
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
     a.mask = mask ? (const char *) mask->data : nullptr;
