@@ -203,11 +203,24 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the ggml-cpu baseline")
     ap.add_argument("--eager", action="store_true", help="launch every call from Python instead of replaying a HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
+                         "launch that hardware byte counters are scaled by) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no cross-GPU step); run with --gpus 1")
 
     import torch
+    if args.calibrate_copy:
+        n = 64 << 20  # float32 elements: 256 MiB read + 256 MiB written per launch
+        x = torch.ones(n, device="cuda", dtype=torch.float32)
+        y = torch.empty_like(x)
+        for _ in range(5):
+            torch.mul(x, 2.0, out=y)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy": {"kernel": "torch elementwise mul (vectorized_elementwise_kernel)",
+                                             "bytes_read": 4 * n, "bytes_written": 4 * n, "launches": 5}}))
+        return
     import __graft_entry__ as entry
     pkg = entry.load_package()
     pkg.check(pkg.lib().vx_init(0), "vx_init")

@@ -328,49 +328,80 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 }
 
 // Merges the split partials: the arithmetic of ggml_flash_attn_ext_reduce_partials
-// (ggml/src/ggml-cpu/ops.cpp:8637-8705) with the global maximum taken first.  A block takes
-// 4 of a tile's 16 columns; thread = (column, 4 consecutive d, one of SG split groups), the
-// groups' sums meet in LDS.
+// (ggml/src/ggml-cpu/ops.cpp:8637-8705) with the global maximum taken first.  One wave per
+// output column.  Lane = (split phase q, 4 consecutive d): the D/4 lanes of a phase read one
+// split's row as one coalesced line, the 64/(D/4) phases take interleaved splits.  The (max,
+// sum) pairs are read one split per lane; every load of the first 64 splits is issued before
+// anything waits, so the kernel costs one trip to memory, a few cross-lane steps and a store.
 constexpr int FA_MERGE_MAX_SPLITS = 256;
-template <int D, int SG>
-__global__ __launch_bounds__(4 * (D / 4) * SG) void fattn_merge_kernel(const fa_args a) {
-    constexpr int DU = D / 4;
-    __shared__ float    sh_m[FA_MERGE_MAX_SPLITS][4], sh_l[FA_MERGE_MAX_SPLITS][4];
-    __shared__ float4_t sh_acc[SG][4 * DU];
-    const int tile = blockIdx.x >> 2, cq = blockIdx.x & 3;
+template <int D>
+__global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
+    constexpr int DU = D / 4;       // lanes per row
+    constexpr int PH = 64 / DU;     // split phases
+    constexpr int NB = 16;          // rows a lane has in flight
+    const int tile = blockIdx.x >> 4, c = blockIdx.x & 15;
     const int ct = tile % a.n_col_tiles;
     const int bg = tile / a.n_col_tiles;
     const int g = bg % a.Hkv, b = bg / a.Hkv;
-    const int ncols = a.n_q * a.gqa;
-    const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + cq * 4; // + split*16 + column
+    const int col = ct * 16 + c;
+    if (col >= a.n_q * a.gqa) return;
+    const int lane = threadIdx.x, q = lane / DU, d0 = 4 * (lane % DU);
+    const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + c; // + split * 16
+    const int nsl = (a.n_splits + 63) >> 6;                         // (max, sum) pairs per lane
 
-    for (int i = threadIdx.x; i < 4 * a.n_splits; i += blockDim.x) {
-        const int s2 = i >> 2, cc = i & 3;
-        const float2 ml = *(const float2 *) (a.part_ml + (tbase + (uint64_t) s2 * 16 + cc) * 2);
-        sh_m[s2][cc] = ml.x;
-        sh_l[s2][cc] = ml.y;
+    float m[FA_MERGE_MAX_SPLITS / 64], l[FA_MERGE_MAX_SPLITS / 64];
+#pragma unroll
+    for (int i = 0; i < FA_MERGE_MAX_SPLITS / 64; ++i) {
+        m[i] = -INFINITY; l[i] = 0.0f;
+        const int s2 = lane + 64 * i;
+        if (i < nsl && s2 < a.n_splits) {
+            const float2 ml = *(const float2 *) (a.part_ml + (tbase + (uint64_t) s2 * 16) * 2);
+            m[i] = ml.x; l[i] = ml.y;
+        }
     }
-    __syncthreads();
+    const float4_t * po = (const float4_t *) (a.part_o + tbase * D + d0); // + split * 4*D float4
+    float4_t rows[NB];
+    auto load_rows = [&](int j0) {
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj) {
+            const int s2 = q + PH * (j0 + jj);
+            rows[jj] = s2 < a.n_splits ? po[(uint64_t) s2 * 4 * D] : float4_t{0, 0, 0, 0};
+        }
+    };
+    load_rows(0);
 
-    const int sg = threadIdx.x / (4 * DU), e = threadIdx.x % (4 * DU);
-    const int cc = e / DU, d0 = 4 * (e % DU);
-    float M = -INFINITY;
-    for (int s2 = 0; s2 < a.n_splits; ++s2) M = fmaxf(M, sh_m[s2][cc]);
+    float M = m[0];
+#pragma unroll
+    for (int i = 1; i < FA_MERGE_MAX_SPLITS / 64; ++i) M = fmaxf(M, m[i]);
+    M = vx_wave_max(M);
     const float shift = (M == -INFINITY) ? 0.0f : M;
+    float L = 0.0f;
+#pragma unroll
+    for (int i = 0; i < FA_MERGE_MAX_SPLITS / 64; ++i) {
+        m[i] = __builtin_amdgcn_exp2f(m[i] - shift); // from here on: the split's weight
+        L += l[i] * m[i];
+    }
+    L = vx_wave_sum(L);
 
     float4_t acc = {0, 0, 0, 0};
-    const float4_t * po = (const float4_t *) (a.part_o + (tbase + cc) * D + d0); // + split * 4*D float4
-#pragma unroll 8
-    for (int s2 = sg; s2 < a.n_splits; s2 += SG) acc += po[(uint64_t) s2 * 4 * D] * __builtin_amdgcn_exp2f(sh_m[s2][cc] - shift);
-    sh_acc[sg][e] = acc;
-    __syncthreads();
-    if (sg != 0) return;
+    const int per = (a.n_splits + PH - 1) / PH; // rows per lane
+    for (int j0 = 0; j0 < per; j0 += NB) {
+        if (j0) load_rows(j0);
+        const int i = (PH * j0) >> 6;           // the NB * PH splits of a batch lie in one 64-group
+        float wsel = m[0];
 #pragma unroll
-    for (int gg = 1; gg < SG; ++gg) acc += sh_acc[gg][e];
-    float L = 0.0f;
-    for (int s2 = 0; s2 < a.n_splits; ++s2) L += sh_l[s2][cc] * __builtin_amdgcn_exp2f(sh_m[s2][cc] - shift);
-    const int col = ct * 16 + cq * 4 + cc;
-    if (col < ncols) fa_finish(a, acc, M, L, b, g, col, D, d0);
+        for (int k = 1; k < FA_MERGE_MAX_SPLITS / 64; ++k) wsel = (i == k) ? m[k] : wsel;
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj) {
+            const int s2 = q + PH * (j0 + jj);
+            acc += rows[jj] * __shfl(wsel, s2 & 63, 64);
+        }
+    }
+#pragma unroll
+    for (int off = DU; off < 64; off <<= 1)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], off, 64);
+    if (q == 0) fa_finish(a, acc, M, L, b, g, col, D, d0);
 }
 
 int g_num_cus = 0;
@@ -511,9 +542,9 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     else         { if (f32) launch_cols16<128, true>(a, (int) nblocks, st); else launch_cols16<128, false>(a, (int) nblocks, st); }
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
-        const dim3 grid((unsigned) (tiles * 4));
-        if (D == 64) fattn_merge_kernel<64, 4><<<grid, dim3(256), 0, st>>>(a);
-        else         fattn_merge_kernel<128, 2><<<grid, dim3(256), 0, st>>>(a);
+        const dim3 grid((unsigned) (tiles * 16));
+        if (D == 64) fattn_merge_kernel<64><<<grid, dim3(64), 0, st>>>(a);
+        else         fattn_merge_kernel<128><<<grid, dim3(64), 0, st>>>(a);
         VX_LAUNCH_CHECK();
     }
     return VX_OK;
