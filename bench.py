@@ -33,6 +33,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA, published
 
 HQ, HKV, D, LAYERS = 16, 2, 64, 24
 
+# (batch, KV length) -> HBM bytes per vx_flash_attn_ext call, measured with hardware counters
+# (see --calibrate-copy); algorithmic bytes of the same call: kv_bytes(2, 4096) = 4194304
+MEASURED_TRAFFIC_BYTES = {(2, 4096): 5654 * 1024}
+
 
 def kv_bytes(batch, length, es=2):
     """algorithmic HBM bytes of one decode attention launch: every K and V element once"""
@@ -248,8 +252,11 @@ def main():
     # dominant kernel: one vx_flash_attn_ext call (split-KV kernel + combine), HIP events
     launch_sec = timer.run(step, iters=200, warmup=10) / LAYERS
     achieved = kv_bytes(B, L) / launch_sec / 1e9
-    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64,f16> (+ combine)", "achieved": achieved,
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+    # HBM bytes per call from rocprofv3 FETCH_SIZE / WRITE_SIZE (split kernel + merge kernel, scaled
+    # by the same counters on a 256 MiB copy: x2.000 and x1.000), taken at the default length only
+    traffic = MEASURED_TRAFFIC_BYTES.get((B, L))
+    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64,f16> + fattn_merge_kernel<64>", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "launch_us": launch_sec * 1e6, "bytes_per_launch": kv_bytes(B, L),
                 "note": "average over the 24 launches of a graph-replayed step (HIP events on the launch stream)"}
     del keep

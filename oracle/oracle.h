@@ -7,7 +7,7 @@
  * Every function follows one piece of the reference (paths relative to the
  * reference checkout; ggml/ = third_party/ggml/) and says which.  How each one is
  * pinned (against the reference's own ggml-cpu built into oracle/_ref, closed forms,
- * brute force, invariants) is listed beside it; tests/test_oracle_*.py run the pins.
+ * brute force, invariants) is listed beside it; tests/test_oracle.py runs the pins.
  *
  * Tensors use ggml's conventions: ne[0] is the fastest dimension, nb[] are strides in
  * bytes, a Q8_0 row is ne[0]/32 blocks of {f16 d; int8 qs[32]} (34 bytes).

@@ -298,6 +298,44 @@ def test_fa_cfg5_shape_properties(gpu):
         assert err <= FA_TOL
 
 
+def test_fa_full_size_invariants(gpu):
+    """Properties that hold at any size, checked at BASELINE config 5's shapes where the scalar
+    oracle is too slow: permuting the keys (K and V rows together) leaves decode attention
+    unchanged; the output is linear in V; prefill attention without a mask equals the
+    wave kernel's result on a sample of rows (two independent kernels, same arithmetic)."""
+    import torch
+    say("flash_attn full-size invariants: B=16, L=8192 decode; T=4096 prefill")
+    B, L = 16, 8192
+    q, k, v = qkv("cfg5inv", B, 16, 2, 1, L)
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    base = gpu.flash_attn_ext(qd, kd, vd, None, 0.125).clone()
+    perm = torch.from_numpy(rng("cfg5inv", "perm").permutation(L)).cuda()
+    got = gpu.flash_attn_ext(qd, kd[:, :, perm].contiguous(), vd[:, :, perm].contiguous(), None, 0.125)
+    e_perm = float((got - base).abs().max())
+    v2 = dev(rng("cfg5inv", "v2").standard_normal(v.shape).astype(np.float16))
+    o2 = gpu.flash_attn_ext(qd, kd, v2, None, 0.125).clone()
+    vsum = (vd.float() + 2.0 * v2.float())  # F32 V: the sum is not f16-representable
+    o12 = gpu.flash_attn_ext(qd, kd.float(), vsum, None, 0.125)
+    e_lin = float((o12 - (base + 2.0 * o2)).abs().max())
+    say(f"   key permutation: max-abs {e_perm:.3e};  linearity in V: max-abs {e_lin:.3e}")
+    assert e_perm <= 2e-5
+    assert e_lin <= 2e-5
+
+    T = 4096
+    q, k, v = qkv("cfg5pre", 1, 16, 2, T, T)
+    mask = dev(reflib.causal_mask(T, T))
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    full = gpu.flash_attn_ext(qd, kd, vd, mask, 0.125).clone()          # LDS-tiled kernel
+    rows = [0, 1, 63, 64, 2047, 4095]
+    for r in rows:                                                         # wave kernel: one row, keys 0..r
+        one = gpu.flash_attn_ext(qd[:, :, r:r + 1].contiguous(), kd[:, :, :r + 1].contiguous(),
+                                 vd[:, :, :r + 1].contiguous(), None, 0.125)
+        err = float((one[0, 0] - full[0, r]).abs().max())
+        say(f"   prefill row {r}: max-abs vs single-row decode {err:.3e}")
+        assert err <= FA_TOL
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("case", ["causal", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
 def test_fa_prefill_kernel(gpu, case):
     """Shapes large enough to take the LDS-tiled prefill kernel (>= 256 columns per KV head,

@@ -187,7 +187,21 @@ vx_status vx_stream_create(vx_stream * stream) {
     return VX_OK;
 }
 vx_status vx_stream_destroy(vx_stream stream) {
-    if (stream) VX_HIP(hipStreamDestroy((hipStream_t) stream));
+    if (!stream) return VX_OK;
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    VX_HIP(hipStreamSynchronize((hipStream_t) stream));
+    {   // the stream's scratch blocks go with it
+        const unsigned long long key = ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        for (auto * map : {&g_ws, &g_cnt}) {
+            auto it = map->find(key);
+            if (it == map->end()) continue;
+            if (it->second.ptr) (void) hipFree(it->second.ptr);
+            map->erase(it);
+        }
+    }
+    VX_HIP(hipStreamDestroy((hipStream_t) stream));
     return VX_OK;
 }
 vx_status vx_stream_synchronize(vx_stream stream) {
