@@ -142,6 +142,47 @@ VX_API vx_status vx_kv_write_view(const vx_tensor * cache, int start, int n_toke
  * ggml-cpu's CPY does for f32 -> f16 (ggml/src/ggml-cpu/ops.cpp:47-268, 526-565). */
 VX_API vx_status vx_kv_store(const vx_tensor * src, const vx_tensor * view, vx_stream stream);
 
+/* ---- glue operators of the decoder layer -----------------------------------------------------
+ * The operators src/minicpm.cpp:572-775 puts between the projections and attention, so that a
+ * whole layer can stay on the device.  F32 unless stated; any strides (16-byte accesses when
+ * rows are dense and aligned); `op` arguments use ggml's enum values. */
+enum { VX_BIN_ADD = 0, VX_BIN_SUB = 1, VX_BIN_MUL = 2, VX_BIN_DIV = 3 };
+/* enum ggml_unary_op (third_party/ggml/include/ggml.h:578-603), the ones implemented */
+enum { VX_UNARY_ABS = 0, VX_UNARY_SGN = 1, VX_UNARY_NEG = 2, VX_UNARY_STEP = 3, VX_UNARY_TANH = 4,
+       VX_UNARY_RELU = 6, VX_UNARY_SIGMOID = 7, VX_UNARY_SILU = 10, VX_UNARY_EXP = 13 };
+/* enum ggml_glu_op (ggml.h:605-614) */
+enum { VX_GLU_REGLU = 0, VX_GLU_SWIGLU = 2 };
+
+/* GGML_OP_ADD / SUB / MUL / DIV: replaces apply_binary_op (ggml/src/ggml-cpu/binary-ops.cpp:50-112);
+ * dst has src0's shape, src1 is repeated over it (ggml_can_repeat). */
+VX_API vx_status vx_binary(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_ADD1: dst = src0 + src1[0] (ggml/src/ggml-cpu/ops.cpp:772-830) */
+VX_API vx_status vx_add1(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_SCALE: dst = src * scale (+ bias, fused) (ops.cpp:4374-4424) */
+VX_API vx_status vx_scale(const vx_tensor * src, const vx_tensor * dst, float scale, float bias, vx_stream stream);
+/* GGML_OP_UNARY (ops.cpp:9617-9719; SILU = x / (1 + expf(-x)), vec.h:1061-1063) */
+VX_API vx_status vx_unary(int op, const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_GLU: dst = act(a) * b; src1 == NULL means a, b are the halves of src0's rows
+ * (swapped exchanges them) (ops.cpp:3127-3185, 9721-9760) */
+VX_API vx_status vx_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int swapped, vx_stream stream);
+/* GGML_OP_CPY / CONT / DUP between F32 and F16 tensors holding the same number of elements:
+ * element i of src (row-major over src's shape) lands in element i of dst
+ * (ggml_compute_forward_dup, ops.cpp:526-565); F32 -> F16 rounds to nearest even. */
+VX_API vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_CONCAT along `dim`, F32 / F16 / I32 (ops.cpp:1891-2095) */
+VX_API vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim, vx_stream stream);
+/* GGML_OP_SUM: every element summed in double, rounded once (ops.cpp:1275-1300) */
+VX_API vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+
+VX_API int vx_supports_binary(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
+VX_API int vx_supports_add1(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
+VX_API int vx_supports_unary_like(const vx_tensor * src, const vx_tensor * dst); /* SCALE */
+VX_API int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * dst);
+VX_API int vx_supports_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
+VX_API int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst);
+VX_API int vx_supports_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim);
+VX_API int vx_supports_sum(const vx_tensor * src, const vx_tensor * dst);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,7 +16,9 @@ from reflib import nmse, rng
 
 pytestmark = pytest.mark.gpu
 
-OPS = ["RMS_NORM", "ROPE", "SOFT_MAX", "FLASH_ATTN_EXT", "MUL_MAT"]
+OPS = ["RMS_NORM", "ROPE", "SOFT_MAX", "FLASH_ATTN_EXT", "MUL_MAT",
+       # the glue of a decoder layer
+       "ADD", "SUB", "MUL", "DIV", "ADD1", "SCALE", "CPY", "CONT", "DUP", "CONCAT", "SUM", "SILU", "SWIGLU"]
 
 
 def plugin_path(pkg):

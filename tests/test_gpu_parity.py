@@ -474,3 +474,95 @@ def test_kv_cache_views_and_store(gpu, cache_dtype):
     out = gpu.flash_attn_ext(dev(q), cache[None, :, :start], other[None, :, :start], None, 0.125)
     want = reflib.oracle_fa(q, host[None, :, :start].astype(np.float32), host[None, :, :start].astype(np.float32))
     assert np.abs(sync_np(out) - want).max() <= FA_TOL
+
+
+# ------------------------------------------------------------------- glue ops of a decoder layer
+def test_glue_binary_broadcast_and_views(gpu):
+    """ADD/SUB/MUL/DIV are single IEEE operations: bit-exact against numpy, with ggml's
+    broadcast (norm weight over tokens, bias column) and with strided operands."""
+    import torch
+    say("glue: binary ops")
+    a = rng("glue", "a").standard_normal((2, 3, 5, 1024)).astype(np.float32)
+    cases = {"same": a * 0.5 + 1, "row": rng("glue", "w").standard_normal((1024,)).astype(np.float32),
+             "col": rng("glue", "c").standard_normal((2, 1, 5, 1)).astype(np.float32),
+             "odd": rng("glue", "o").standard_normal((3, 1, 1024)).astype(np.float32)}
+    fns = {gpu.BIN_ADD: np.add, gpu.BIN_SUB: np.subtract, gpu.BIN_MUL: np.multiply, gpu.BIN_DIV: np.divide}
+    for name, b in cases.items():
+        b4 = b.reshape((1,) * (4 - b.ndim) + b.shape)
+        for op, fn in fns.items():
+            got = sync_np(gpu.binary(op, dev(a), dev(b4)))
+            assert np.array_equal(got, fn(a, b4)), (name, op)
+    # odd row length (scalar path) and a permuted src0 / transposed src1
+    x = rng("glue", "x").standard_normal((4, 7, 33)).astype(np.float32)
+    y = rng("glue", "y").standard_normal((4, 33, 7)).astype(np.float32)
+    got = sync_np(gpu.binary(gpu.BIN_ADD, dev(x), dev(y).transpose(1, 2)))
+    assert np.array_equal(got, x + y.transpose(0, 2, 1))
+
+
+def test_glue_scale_add1_unary_glu(gpu):
+    import torch
+    say("glue: scale / add1 / unary / glu")
+    x = (rng("glue2", "x").standard_normal((3, 130, 1024)) * 3).astype(np.float32)
+    got = sync_np(gpu.scale(dev(x), 0.37))
+    assert np.array_equal(got, x * np.float32(0.37))
+    got = sync_np(gpu.scale(dev(x), 0.37, 1.5))
+    want = (x.astype(np.float64) * np.float64(np.float32(0.37)) + 1.5).astype(np.float32)  # fused multiply-add
+    assert np.abs(got - want).max() <= 1e-6 and (got != want).mean() < 1e-3
+    s = np.array([0.25], np.float32)
+    assert np.array_equal(sync_np(gpu.add1(dev(x), dev(s))), x + s[0])
+    x64 = x.astype(np.float64)
+    silu = x64 / (1 + np.exp(-x64))
+    got = sync_np(gpu.unary(gpu.UNARY_SILU, dev(x)))
+    assert np.abs(got - silu).max() <= 2e-6
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_RELU, dev(x))), np.maximum(x, 0))
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_NEG, dev(x))), -x)
+    up = rng("glue2", "up").standard_normal(x.shape).astype(np.float32)
+    got = sync_np(gpu.glu(gpu.GLU_SWIGLU, dev(x), dev(up)))
+    assert np.abs(got - silu * up).max() <= 1e-5
+    # one-tensor form: halves of the row, and swapped
+    gu = np.concatenate([x, up], axis=-1)
+    assert np.array_equal(sync_np(gpu.glu(gpu.GLU_SWIGLU, dev(gu))), got)
+    ug = np.concatenate([up, x], axis=-1)
+    assert np.array_equal(sync_np(gpu.glu(gpu.GLU_SWIGLU, dev(ug), swapped=True)), got)
+    # views of a fused gate|up projection, as mlp_forward builds them
+    t = dev(gu)
+    assert np.array_equal(sync_np(gpu.glu(gpu.GLU_SWIGLU, t[..., :1024], t[..., 1024:])), got)
+
+
+@pytest.mark.parametrize("cache_dtype", [np.float16, np.float32])
+def test_glue_cpy_cont_concat_sum(gpu, cache_dtype):
+    """The KV append of attention_forward: CPY of the rotated keys into the cache's write view,
+    CONT + SUM of that view, CONCAT of the past view with the current keys."""
+    import torch
+    say(f"glue: cpy / cont / concat / sum, cache {np.dtype(cache_dtype).name}")
+    D, Hkv, maxlen, n_past, T = 64, 2, 96, 37, 5
+    tt = torch.float16 if cache_dtype == np.float16 else torch.float32
+    cache0 = rng("glue3", "cache").standard_normal((Hkv, maxlen, D)).astype(cache_dtype)
+    kcur = rng("glue3", "k").standard_normal((T, Hkv, D)).astype(np.float32)
+    cache = dev(cache0)
+    wview = cache[:, n_past:n_past + T].transpose(0, 1)          # (T, Hkv, D): ggml [D, Hkv, T]
+    gpu.cpy(dev(kcur), wview)
+    want = cache0.copy()
+    want[:, n_past:n_past + T] = kcur.transpose(1, 0, 2).astype(cache_dtype)
+    assert np.array_equal(sync_np(cache), want)
+    cont = torch.empty((T, Hkv, D), dtype=tt, device="cuda")
+    gpu.cpy(wview, cont)
+    assert np.array_equal(sync_np(cont), want[:, n_past:n_past + T].transpose(1, 0, 2))
+    if cache_dtype == np.float32:
+        got = float(sync_np(gpu.sum_all(wview))[0])
+        assert got == np.float32(kcur.astype(np.float64).sum())
+    # reshaping copy: same element count, different shapes (element i -> element i)
+    flat = torch.empty((T * Hkv * D // 8, 8), dtype=torch.float32, device="cuda")
+    gpu.cpy(wview, flat)
+    assert np.array_equal(sync_np(flat).reshape(-1), want[:, n_past:n_past + T].transpose(1, 0, 2).astype(np.float32).reshape(-1))
+    # concat(past view [D, n_past, Hkv], permuted current keys [D, T, Hkv]) along ggml dim 1
+    past = cache[:, :n_past]
+    cur = dev(kcur.astype(cache_dtype)).transpose(0, 1)          # (Hkv, T, D), strided
+    got = sync_np(gpu.concat(past, cur, 1))
+    assert np.array_equal(got, np.concatenate([want[:, :n_past], kcur.transpose(1, 0, 2).astype(cache_dtype)], axis=1))
+    # other dims, odd sizes (element path)
+    a = rng("glue3", "a").standard_normal((2, 3, 5, 7)).astype(cache_dtype)
+    for gd in range(4):
+        shp = list(a.shape); shp[3 - gd] += 2
+        b = rng("glue3", "b", gd).standard_normal([2 if i == 3 - gd else n for i, n in enumerate(a.shape)]).astype(cache_dtype)
+        assert np.array_equal(sync_np(gpu.concat(dev(a), dev(b), gd)), np.concatenate([a, b], axis=3 - gd))

@@ -39,7 +39,14 @@ EXPORTS = [
     "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_mul_mat",
     "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
     "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
+    "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum",
+    "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
+    "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
 ]
+
+BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV = 0, 1, 2, 3
+UNARY_ABS, UNARY_SGN, UNARY_NEG, UNARY_STEP, UNARY_TANH, UNARY_RELU, UNARY_SIGMOID, UNARY_SILU, UNARY_EXP = 0, 1, 2, 3, 4, 6, 7, 10, 13
+GLU_REGLU, GLU_SWIGLU = 0, 2
 
 _lib = None
 
@@ -81,6 +88,22 @@ def lib():
     l.vx_kv_read_view.argtypes = [TP, C.c_int, TP]
     l.vx_kv_write_view.argtypes = [TP, C.c_int, C.c_int, TP]
     l.vx_kv_store.argtypes = [TP, TP, vp]
+    l.vx_binary.argtypes = [C.c_int, TP, TP, TP, vp]
+    l.vx_add1.argtypes = [TP, TP, TP, vp]
+    l.vx_scale.argtypes = [TP, TP, C.c_float, C.c_float, vp]
+    l.vx_unary.argtypes = [C.c_int, TP, TP, vp]
+    l.vx_glu.argtypes = [C.c_int, TP, TP, TP, C.c_int, vp]
+    l.vx_cpy.argtypes = [TP, TP, vp]
+    l.vx_concat.argtypes = [TP, TP, TP, C.c_int, vp]
+    l.vx_sum.argtypes = [TP, TP, vp]
+    l.vx_supports_binary.argtypes = [C.c_int, TP, TP, TP]
+    l.vx_supports_add1.argtypes = [TP, TP, TP]
+    l.vx_supports_unary_like.argtypes = [TP, TP]
+    l.vx_supports_unary.argtypes = [C.c_int, TP, TP]
+    l.vx_supports_glu.argtypes = [C.c_int, TP, TP, TP]
+    l.vx_supports_cpy.argtypes = [TP, TP]
+    l.vx_supports_concat.argtypes = [TP, TP, TP, C.c_int]
+    l.vx_supports_sum.argtypes = [TP, TP]
     _lib = l
     return l
 
@@ -189,4 +212,66 @@ def mul_mat(w, x, act_mode=ACT_FLOAT, w_ne0=None, out=None):
         shape = list(x.shape[:-1]) + [wd.ne[1]]
         out = torch.empty(shape, dtype=torch.float32, device=x.device)
     check(lib().vx_mul_mat(wd, xd, desc(out), act_mode, _stream()), "vx_mul_mat")
+    return out
+
+
+# ---- glue operators (torch dim d corresponds to ggml dim ndim-1-d) ----
+def binary(op, a, b, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(lib().vx_binary(op, desc(a), desc(b), desc(out), _stream()), "vx_binary")
+    return out
+
+
+def add1(a, b, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(lib().vx_add1(desc(a), desc(b), desc(out), _stream()), "vx_add1")
+    return out
+
+
+def scale(a, s, bias=0.0, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(lib().vx_scale(desc(a), desc(out), s, bias, _stream()), "vx_scale")
+    return out
+
+
+def unary(op, a, out=None):
+    import torch
+    out = torch.empty_like(a) if out is None else out
+    check(lib().vx_unary(op, desc(a), desc(out), _stream()), "vx_unary")
+    return out
+
+
+def glu(op, a, b=None, swapped=False, out=None):
+    import torch
+    if out is None:
+        shape = list(a.shape)
+        if b is None:
+            shape[-1] //= 2
+        out = torch.empty(shape, dtype=torch.float32, device=a.device)
+    check(lib().vx_glu(op, desc(a), desc(b), desc(out), int(swapped), _stream()), "vx_glu")
+    return out
+
+
+def cpy(src, dst):
+    check(lib().vx_cpy(desc(src), desc(dst), _stream()), "vx_cpy")
+    return dst
+
+
+def concat(a, b, ggml_dim, out=None):
+    import torch
+    if out is None:
+        shape = list(a.shape)
+        shape[a.dim() - 1 - ggml_dim] += b.shape[b.dim() - 1 - ggml_dim]
+        out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    check(lib().vx_concat(desc(a), desc(b), desc(out), ggml_dim, _stream()), "vx_concat")
+    return out
+
+
+def sum_all(a, out=None):
+    import torch
+    out = torch.empty((1,), dtype=torch.float32, device=a.device) if out is None else out
+    check(lib().vx_sum(desc(a), desc(out), _stream()), "vx_sum")
     return out

@@ -511,7 +511,9 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 64; }();
     a.n_splits = 1;
     a.chunk    = (a.n_kv + 31) / 32 * 32;
-    if (tiles < (int64_t) 4 * num_cus()) {
+    // Up to 256 keys one wave finishes (0.5 us per 32-key step) before a split plus the merge
+    // launch would.
+    if (tiles < (int64_t) 4 * num_cus() && a.n_kv > 256) {
         int64_t want = ((int64_t) 4 * num_cus() + tiles - 1) / tiles;
         const int64_t max_splits = (a.n_kv + min_chunk - 1) / min_chunk;
         if (want > max_splits) want = max_splits;

@@ -1,0 +1,420 @@
+// glue.hip -- the small operators between the projections and attention in the MiniCPM / LocDiT
+// graphs (src/minicpm.cpp:572-775): residual ADD, norm-weight MUL, SCALE, ADD1, the KV append
+// CPY / CONT, CONCAT of past and current keys, SUM (the reference's write-ordering trick),
+// SILU and SWIGLU.  All of them move each byte once: they exist so that a whole decoder layer
+// stays on the device and no scheduler split (with its blocking copy) falls between two
+// claimed operators.
+//
+// One indexing scheme serves all of them: a thread owns VEC consecutive elements of one dst row;
+// rows are flattened over (i1, i2, i3).  VEC = 4 (16-byte accesses) when every operand is dense
+// and 16-byte aligned along dim 0, VEC = 1 otherwise (any strides, ggml's broadcast rules).
+#include "vx_common.hpp"
+
+#include <cmath>
+
+namespace {
+
+enum ew_op : int {
+    EW_ADD, EW_SUB, EW_MUL, EW_DIV,   // dst = src0 (op) src1, src1 broadcast (ggml_can_repeat)
+    EW_ADD1,                          // dst = src0 + src1[0]
+    EW_SCALE,                         // dst = src0 * p0 (+ p1)
+    EW_UNARY,                         // dst = f(src0), f = aux
+    EW_GLU,                           // dst = act(a) * b, act = aux
+};
+
+struct ew_args {
+    const char * s0; const char * s1; char * d;
+    int64_t  ne[4];     // dst shape
+    int64_t  ne1[4];    // src1 shape (broadcast)
+    uint64_t nb0[4], nb1[4], nbd[4];
+    float p0, p1;
+    int aux;
+    int64_t nchunk;     // blocks per row
+};
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ float unary_f(int op, float x) {
+    switch (op) {
+        case VX_UNARY_ABS:     return fabsf(x);
+        case VX_UNARY_SGN:     return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f);
+        case VX_UNARY_NEG:     return -x;
+        case VX_UNARY_STEP:    return x > 0.0f ? 1.0f : 0.0f;
+        case VX_UNARY_TANH:    return tanhf(x);
+        case VX_UNARY_RELU:    return x > 0.0f ? x : 0.0f;
+        case VX_UNARY_SIGMOID: return 1.0f / (1.0f + expf(-x));
+        case VX_UNARY_SILU:    return silu_f(x);
+        case VX_UNARY_EXP:     return expf(x);
+        default:               return x;
+    }
+}
+
+template <int OP>
+__device__ __forceinline__ float ew_apply(const ew_args & a, float x, float y) {
+    if constexpr (OP == EW_ADD)   return x + y;
+    if constexpr (OP == EW_SUB)   return x - y;
+    if constexpr (OP == EW_MUL)   return x * y;
+    if constexpr (OP == EW_DIV)   return x / y;
+    if constexpr (OP == EW_ADD1)  return x + y;
+    if constexpr (OP == EW_SCALE) return a.p1 == 0.0f ? x * a.p0 : fmaf(x, a.p0, a.p1); // vec_scale / vec_mad1
+    if constexpr (OP == EW_UNARY) return unary_f(a.aux, x);
+    if constexpr (OP == EW_GLU)   return (a.aux == VX_GLU_REGLU ? (x > 0.0f ? x : 0.0f) : silu_f(x)) * y;
+    return x;
+}
+
+template <int OP> constexpr bool ew_has_src1() { return OP == EW_ADD || OP == EW_SUB || OP == EW_MUL || OP == EW_DIV || OP == EW_GLU; }
+
+template <int OP, int VEC>
+__global__ __launch_bounds__(256) void ew_kernel(const ew_args a) {
+    const int64_t row   = blockIdx.x / a.nchunk;
+    const int64_t chunk = blockIdx.x % a.nchunk;
+    const int64_t i0    = (chunk * 256 + threadIdx.x) * VEC;
+    if (i0 >= a.ne[0]) return;
+    const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
+    const char * p0 = a.s0 + i1 * a.nb0[1] + i2 * a.nb0[2] + i3 * a.nb0[3];
+    char *       pd = a.d + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+    const char * p1 = nullptr;
+    float yb = 0.0f;
+    if constexpr (ew_has_src1<OP>()) p1 = a.s1 + (i1 % a.ne1[1]) * a.nb1[1] + (i2 % a.ne1[2]) * a.nb1[2] + (i3 % a.ne1[3]) * a.nb1[3];
+    if constexpr (OP == EW_ADD1) yb = *(const float *) a.s1;
+
+    if constexpr (VEC == 4) {
+        const float4_t x = *(const float4_t *) (p0 + i0 * 4);
+        float4_t y = {yb, yb, yb, yb};
+        if constexpr (ew_has_src1<OP>()) y = *(const float4_t *) (p1 + i0 * 4);
+        float4_t r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = ew_apply<OP>(a, x[k], y[k]);
+        *(float4_t *) (pd + i0 * 4) = r;
+    } else {
+        const float x = *(const float *) (p0 + i0 * a.nb0[0]);
+        float y = yb;
+        if constexpr (ew_has_src1<OP>()) y = *(const float *) (p1 + (i0 % a.ne1[0]) * a.nb1[0]);
+        *(float *) (pd + i0 * a.nbd[0]) = ew_apply<OP>(a, x, y);
+    }
+}
+
+bool al16(const void * p, const uint64_t * nb) {
+    return (uintptr_t) p % 16 == 0 && nb[1] % 16 == 0 && nb[2] % 16 == 0 && nb[3] % 16 == 0;
+}
+
+template <int OP>
+vx_status ew_launch(ew_args & a, hipStream_t st) {
+    const int64_t rows = a.ne[1] * a.ne[2] * a.ne[3];
+    if (a.ne[0] <= 0 || rows <= 0) return VX_OK;
+    bool vec = a.ne[0] % 4 == 0 && a.nb0[0] == 4 && a.nbd[0] == 4 && al16(a.s0, a.nb0) && al16(a.d, a.nbd);
+    if (ew_has_src1<OP>()) vec = vec && a.ne1[0] == a.ne[0] && a.nb1[0] == 4 && al16(a.s1, a.nb1);
+    const int V = vec ? 4 : 1;
+    a.nchunk    = (a.ne[0] + 256 * V - 1) / (256 * V);
+    const int64_t blocks = rows * a.nchunk;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "elementwise op: launch too large");
+    if (vec) ew_kernel<OP, 4><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    else     ew_kernel<OP, 1><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+void ew_fill(ew_args & a, const vx_tensor * s0, const vx_tensor * s1, const vx_tensor * d) {
+    a.s0 = (const char *) s0->data; a.s1 = s1 ? (const char *) s1->data : nullptr; a.d = (char *) d->data;
+    for (int i = 0; i < 4; ++i) {
+        a.ne[i] = d->ne[i]; a.nb0[i] = s0->nb[i]; a.nbd[i] = d->nb[i];
+        a.ne1[i] = s1 ? s1->ne[i] : 1; a.nb1[i] = s1 ? s1->nb[i] : 0;
+    }
+    a.p0 = a.p1 = 0.0f; a.aux = 0; a.nchunk = 1;
+}
+
+bool f32(const vx_tensor * t) { return t && t->type == VX_TYPE_F32; }
+bool can_repeat(const vx_tensor * small, const vx_tensor * big) {
+    for (int i = 0; i < 4; ++i) if (small->ne[i] <= 0 || big->ne[i] % small->ne[i]) return false;
+    return true;
+}
+bool fl_type(int t) { return t == VX_TYPE_F32 || t == VX_TYPE_F16; }
+bool nb_multiple(const vx_tensor * t, uint64_t m) {
+    return t->nb[0] % m == 0 && t->nb[1] % m == 0 && t->nb[2] % m == 0 && t->nb[3] % m == 0;
+}
+
+// ---- CPY / CONT / DUP -----------------------------------------------------------------------
+// Element i of src (row-major order of src's shape) goes to element i of dst (row-major order of
+// dst's shape): ggml_compute_forward_dup's rule; the shapes only have to hold the same count.
+struct cpy_args {
+    const char * s; char * d;
+    int64_t  nes[4], ned[4];
+    uint64_t nbs[4], nbd[4];
+    int64_t  n;
+};
+
+template <typename TS, typename TD, int VEC>
+__global__ __launch_bounds__(256) void cpy_kernel(const cpy_args a) {
+    const int64_t e = ((int64_t) blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (e >= a.n) return;
+    int64_t r = e;
+    const int64_t s0 = r % a.nes[0]; r /= a.nes[0];
+    const int64_t s1 = r % a.nes[1]; r /= a.nes[1];
+    const int64_t s2 = r % a.nes[2]; const int64_t s3 = r / a.nes[2];
+    const char * ps = a.s + s0 * a.nbs[0] + s1 * a.nbs[1] + s2 * a.nbs[2] + s3 * a.nbs[3];
+    r = e;
+    const int64_t d0 = r % a.ned[0]; r /= a.ned[0];
+    const int64_t d1 = r % a.ned[1]; r /= a.ned[1];
+    const int64_t d2 = r % a.ned[2]; const int64_t d3 = r / a.ned[2];
+    char * pd = a.d + d0 * a.nbd[0] + d1 * a.nbd[1] + d2 * a.nbd[2] + d3 * a.nbd[3];
+    if constexpr (VEC == 1) {
+        *(TD *) pd = (TD) (float) *(const TS *) ps;
+    } else { // 4 consecutive elements of a dense run on both sides
+        typedef TS vs_t __attribute__((ext_vector_type(4)));
+        typedef TD vd_t __attribute__((ext_vector_type(4)));
+        const vs_t x = *(const vs_t *) ps;
+        vd_t y;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) y[k] = (TD) (float) x[k];
+        *(vd_t *) pd = y;
+    }
+}
+
+template <typename TS, typename TD>
+vx_status cpy_launch(const cpy_args & a, bool vec, hipStream_t st) {
+    const int V = vec ? 4 : 1;
+    const int64_t blocks = (a.n / V + 255) / 256;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "cpy: launch too large");
+    if (vec) cpy_kernel<TS, TD, 4><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    else     cpy_kernel<TS, TD, 1><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// ---- CONCAT -----------------------------------------------------------------------------------
+struct cat_args {
+    const char * s0; const char * s1; char * d;
+    int64_t  ne[4], ne0[4];   // dst shape, src0 shape
+    uint64_t nb0[4], nb1[4], nbd[4];
+    int dim;
+    int64_t n;                 // dst units (elements, or 16-byte groups when VEC)
+};
+
+// UNIT = bytes moved per thread (element size, or 16 for a dense run along dim 0)
+template <int UNIT, int ES>
+__global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
+    const int64_t u = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (u >= a.n) return;
+    constexpr int EPU = UNIT / ES; // elements per unit
+    const int64_t units0 = a.ne[0] / EPU;
+    int64_t r = u;
+    int64_t i[4];
+    i[0] = (r % units0) * EPU; r /= units0;
+    i[1] = r % a.ne[1]; r /= a.ne[1];
+    i[2] = r % a.ne[2]; i[3] = r / a.ne[2];
+    char * pd = a.d + i[0] * a.nbd[0] + i[1] * a.nbd[1] + i[2] * a.nbd[2] + i[3] * a.nbd[3];
+    const char * ps;
+    if (i[a.dim] < a.ne0[a.dim]) {
+        ps = a.s0 + i[0] * a.nb0[0] + i[1] * a.nb0[1] + i[2] * a.nb0[2] + i[3] * a.nb0[3];
+    } else {
+        i[a.dim] -= a.ne0[a.dim];
+        ps = a.s1 + i[0] * a.nb1[0] + i[1] * a.nb1[1] + i[2] * a.nb1[2] + i[3] * a.nb1[3];
+    }
+    if constexpr (UNIT == 16)     *(int4_t *) pd = *(const int4_t *) ps;
+    else if constexpr (UNIT == 4) *(int32_t *) pd = *(const int32_t *) ps;
+    else                          *(int16_t *) pd = *(const int16_t *) ps;
+}
+
+// ---- SUM ---------------------------------------------------------------------------------------
+// ggml sums every element in double and rounds once (ops.cpp:1275-1300): one block, fp64 lanes.
+__global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst) {
+    __shared__ double part[16];
+    const int64_t n = s.ne[0] * s.ne[1] * s.ne[2] * s.ne[3];
+    double acc = 0.0;
+    for (int64_t e = threadIdx.x; e < n; e += 1024) {
+        int64_t r = e;
+        const int64_t i0 = r % s.ne[0]; r /= s.ne[0];
+        const int64_t i1 = r % s.ne[1]; r /= s.ne[1];
+        const int64_t i2 = r % s.ne[2]; const int64_t i3 = r / s.ne[2];
+        acc += (double) *(const float *) (src + i0 * s.nb[0] + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3]);
+    }
+    acc = vx_wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int w = 0; w < 16; ++w) t += part[w];
+        *dst = (float) t;
+    }
+}
+
+} // namespace
+
+// ================================================================================== C ABI
+
+extern "C" int vx_supports_binary(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst) {
+    if (op < VX_BIN_ADD || op > VX_BIN_DIV) return 0;
+    if (!f32(src0) || !f32(src1) || !f32(dst)) return 0;
+    if (!vx_positive(src0) || !vx_same_shape(src0, dst) || !can_repeat(src1, src0)) return 0;
+    return nb_multiple(src0, 4) && nb_multiple(src1, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_binary(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_binary(op, src0, src1, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "binary op %d: F32 operands, src1 repeatable over src0", op);
+    if (!src0->data || !src1->data || !dst->data) return vx_fail(VX_ERR_INVALID, "binary op: null data");
+    ew_args a; ew_fill(a, src0, src1, dst);
+    switch (op) {
+        case VX_BIN_ADD: return ew_launch<EW_ADD>(a, (hipStream_t) stream);
+        case VX_BIN_SUB: return ew_launch<EW_SUB>(a, (hipStream_t) stream);
+        case VX_BIN_MUL: return ew_launch<EW_MUL>(a, (hipStream_t) stream);
+        default:         return ew_launch<EW_DIV>(a, (hipStream_t) stream);
+    }
+}
+
+extern "C" int vx_supports_add1(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst) {
+    if (!f32(src0) || !f32(src1) || !f32(dst)) return 0;
+    if (!vx_positive(src0) || !vx_same_shape(src0, dst) || vx_nelements(src1) != 1) return 0;
+    return nb_multiple(src0, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_add1(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_add1(src0, src1, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "add1: F32 tensor plus F32 scalar");
+    if (!src0->data || !src1->data || !dst->data) return vx_fail(VX_ERR_INVALID, "add1: null data");
+    ew_args a; ew_fill(a, src0, nullptr, dst);
+    a.s1 = (const char *) src1->data;
+    return ew_launch<EW_ADD1>(a, (hipStream_t) stream);
+}
+
+extern "C" int vx_supports_unary_like(const vx_tensor * src, const vx_tensor * dst) {
+    if (!f32(src) || !f32(dst)) return 0;
+    if (!vx_positive(src) || !vx_same_shape(src, dst)) return 0;
+    return nb_multiple(src, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_scale(const vx_tensor * src, const vx_tensor * dst, float scale, float bias, vx_stream stream) {
+    if (!vx_supports_unary_like(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "scale: F32 tensors of one shape");
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "scale: null data");
+    ew_args a; ew_fill(a, src, nullptr, dst);
+    a.p0 = scale; a.p1 = bias;
+    return ew_launch<EW_SCALE>(a, (hipStream_t) stream);
+}
+
+extern "C" int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * dst) {
+    switch (op) {
+        case VX_UNARY_ABS: case VX_UNARY_SGN: case VX_UNARY_NEG: case VX_UNARY_STEP: case VX_UNARY_TANH:
+        case VX_UNARY_RELU: case VX_UNARY_SIGMOID: case VX_UNARY_SILU: case VX_UNARY_EXP: break;
+        default: return 0;
+    }
+    return vx_supports_unary_like(src, dst);
+}
+
+extern "C" vx_status vx_unary(int op, const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_unary(op, src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "unary op %d: F32 tensors of one shape", op);
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "unary: null data");
+    ew_args a; ew_fill(a, src, nullptr, dst);
+    a.aux = op;
+    return ew_launch<EW_UNARY>(a, (hipStream_t) stream);
+}
+
+extern "C" int vx_supports_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst) {
+    if (op != VX_GLU_SWIGLU && op != VX_GLU_REGLU) return 0;
+    if (!f32(src0) || !f32(dst) || (src1 && !f32(src1))) return 0;
+    if (!vx_positive(src0) || src0->nb[0] != 4 || dst->nb[0] != 4) return 0;
+    if (src1) {
+        if (!vx_same_shape(src0, src1) || !vx_same_shape(src0, dst) || src1->nb[0] != 4) return 0;
+        if (!nb_multiple(src1, 4)) return 0;
+    } else {
+        if (src0->ne[0] % 2 || dst->ne[0] != src0->ne[0] / 2) return 0;
+        for (int i = 1; i < 4; ++i) if (dst->ne[i] != src0->ne[i]) return 0;
+    }
+    return nb_multiple(src0, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int swapped,
+                            vx_stream stream) {
+    if (!vx_supports_glu(op, src0, src1, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "glu op %d: F32 SWIGLU / REGLU with dense rows", op);
+    if (!src0->data || !dst->data || (src1 && !src1->data)) return vx_fail(VX_ERR_INVALID, "glu: null data");
+    // one tensor: the row's halves are the two operands (ops.cpp:3165-3168); `swapped` only
+    // applies there.  x feeds the activation, y the gate.
+    vx_tensor x = *src0, y = src1 ? *src1 : *src0;
+    if (!src1) {
+        const int64_t nc = src0->ne[0] / 2;
+        x.ne[0] = y.ne[0] = nc;
+        x.data = (char *) src0->data + (swapped ? nc * 4 : 0);
+        y.data = (char *) src0->data + (swapped ? 0 : nc * 4);
+    }
+    ew_args a; ew_fill(a, &x, &y, dst);
+    a.aux = op;
+    return ew_launch<EW_GLU>(a, (hipStream_t) stream);
+}
+
+extern "C" int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst) {
+    if (!src || !dst || !fl_type(src->type) || !fl_type(dst->type)) return 0;
+    if (!vx_positive(src) || !vx_positive(dst) || vx_nelements(src) != vx_nelements(dst)) return 0;
+    return nb_multiple(src, vx_type_size(src->type)) && nb_multiple(dst, vx_type_size(dst->type));
+}
+
+extern "C" vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_cpy(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "cpy: F32/F16 tensors holding the same number of elements");
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "cpy: null data");
+    cpy_args a;
+    a.s = (const char *) src->data; a.d = (char *) dst->data; a.n = vx_nelements(src);
+    for (int i = 0; i < 4; ++i) { a.nes[i] = src->ne[i]; a.ned[i] = dst->ne[i]; a.nbs[i] = src->nb[i]; a.nbd[i] = dst->nb[i]; }
+    const size_t ss = vx_type_size(src->type), ds = vx_type_size(dst->type);
+    const bool vec = src->ne[0] % 4 == 0 && dst->ne[0] % 4 == 0 && src->nb[0] == ss && dst->nb[0] == ds &&
+                     (uintptr_t) src->data % (4 * ss) == 0 && (uintptr_t) dst->data % (4 * ds) == 0 &&
+                     src->nb[1] % (4 * ss) == 0 && src->nb[2] % (4 * ss) == 0 && src->nb[3] % (4 * ss) == 0 &&
+                     dst->nb[1] % (4 * ds) == 0 && dst->nb[2] % (4 * ds) == 0 && dst->nb[3] % (4 * ds) == 0;
+    hipStream_t st = (hipStream_t) stream;
+    if (src->type == VX_TYPE_F32) {
+        return dst->type == VX_TYPE_F32 ? cpy_launch<float, float>(a, vec, st) : cpy_launch<float, _Float16>(a, vec, st);
+    }
+    return dst->type == VX_TYPE_F32 ? cpy_launch<_Float16, float>(a, vec, st) : cpy_launch<_Float16, _Float16>(a, vec, st);
+}
+
+extern "C" int vx_supports_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim) {
+    if (!src0 || !src1 || !dst || dim < 0 || dim > 3) return 0;
+    if (src0->type != src1->type || src0->type != dst->type) return 0;
+    if (src0->type != VX_TYPE_F32 && src0->type != VX_TYPE_F16 && src0->type != VX_TYPE_I32) return 0;
+    if (!vx_positive(src0) || !vx_positive(src1)) return 0;
+    for (int i = 0; i < 4; ++i) {
+        if (i == dim) { if (dst->ne[i] != src0->ne[i] + src1->ne[i]) return 0; }
+        else if (src0->ne[i] != src1->ne[i] || dst->ne[i] != src0->ne[i]) return 0;
+    }
+    const uint64_t es = vx_type_size(src0->type);
+    return nb_multiple(src0, es) && nb_multiple(src1, es) && nb_multiple(dst, es);
+}
+
+extern "C" vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim, vx_stream stream) {
+    if (!vx_supports_concat(src0, src1, dst, dim)) return vx_fail(VX_ERR_UNSUPPORTED, "concat: F32/F16/I32 tensors equal outside dim %d", dim);
+    if (!src0->data || !src1->data || !dst->data) return vx_fail(VX_ERR_INVALID, "concat: null data");
+    cat_args a;
+    a.s0 = (const char *) src0->data; a.s1 = (const char *) src1->data; a.d = (char *) dst->data; a.dim = dim;
+    for (int i = 0; i < 4; ++i) {
+        a.ne[i] = dst->ne[i]; a.ne0[i] = src0->ne[i];
+        a.nb0[i] = src0->nb[i]; a.nb1[i] = src1->nb[i]; a.nbd[i] = dst->nb[i];
+    }
+    const int es = (int) vx_type_size(src0->type);
+    const int epu = 16 / es;
+    auto dense16 = [&](const vx_tensor * t) {
+        return t->nb[0] == (uint64_t) es && (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+    };
+    const bool vec = dim != 0 && dst->ne[0] % epu == 0 && dense16(src0) && dense16(src1) && dense16(dst);
+    const int64_t n_el = vx_nelements(dst);
+    a.n = vec ? n_el / epu : n_el;
+    const int64_t blocks = (a.n + 255) / 256;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "concat: launch too large");
+    const dim3 grid((unsigned) blocks), block(256);
+    hipStream_t st = (hipStream_t) stream;
+    if (vec)          { if (es == 4) concat_kernel<16, 4><<<grid, block, 0, st>>>(a); else concat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
+    else if (es == 4) concat_kernel<4, 4><<<grid, block, 0, st>>>(a);
+    else              concat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+extern "C" int vx_supports_sum(const vx_tensor * src, const vx_tensor * dst) {
+    if (!f32(src) || !f32(dst)) return 0;
+    if (!vx_positive(src) || vx_nelements(dst) != 1) return 0;
+    // rows must be dense: ggml-cpu asserts nb[0] == sizeof(float) (ops.cpp:1286) and reads rows as
+    // contiguous regardless.  One block walks the tensor: meant for the small tensors the graphs sum.
+    return src->nb[0] == 4 && vx_nelements(src) <= (int64_t) 1 << 24 && nb_multiple(src, 4);
+}
+
+extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_sum(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "sum: F32 tensor of at most 2^24 elements to an F32 scalar");
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "sum: null data");
+    sum_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}

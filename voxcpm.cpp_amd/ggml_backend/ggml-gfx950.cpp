@@ -4,7 +4,9 @@
 //     GGML_OP_FLASH_ATTN_EXT, GGML_OP_ROPE, GGML_OP_SOFT_MAX, GGML_OP_RMS_NORM,
 //     GGML_OP_MUL_MAT (Q8_0 / F16 / F32 weights, F32 activations)
 //
-// plus the view ops every backend accepts.  Everything else is answered with
+// plus the glue between them in a decoder layer (ADD, SUB, MUL, DIV, ADD1, SCALE, CPY, CONT,
+// DUP, CONCAT, SUM, UNARY silu & co, GLU swiglu), so that a MiniCPM layer needs no scheduler
+// split, and the view ops every backend accepts.  Everything else is answered with
 // supports_op() == false, so ggml's scheduler keeps it on ggml-cpu.  The file is host-only
 // C++: it implements ggml's five backend vtables (ggml/src/ggml-backend-impl.h:17-204 of
 // the reference checkout) and forwards every claimed node, unchanged, to the C ABI of
@@ -48,6 +50,15 @@ vx_tensor to_vx(const ggml_tensor * t) {
 
 bool type_known(ggml_type t) {
     return t == GGML_TYPE_F32 || t == GGML_TYPE_F16 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_I32;
+}
+
+int binary_code(ggml_op op) {
+    switch (op) {
+        case GGML_OP_ADD: return VX_BIN_ADD;
+        case GGML_OP_SUB: return VX_BIN_SUB;
+        case GGML_OP_MUL: return VX_BIN_MUL;
+        default:          return VX_BIN_DIV;
+    }
 }
 
 int mul_mat_act_mode() {
@@ -232,6 +243,45 @@ bool supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
             return vx_supports_mul_mat(&a, &b, &d) != 0;
         }
+        case GGML_OP_ADD:
+        case GGML_OP_SUB:
+        case GGML_OP_MUL:
+        case GGML_OP_DIV: {
+            const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
+            return vx_supports_binary(binary_code(op->op), &a, &b, &d) != 0;
+        }
+        case GGML_OP_ADD1: {
+            const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
+            return vx_supports_add1(&a, &b, &d) != 0;
+        }
+        case GGML_OP_SCALE: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_unary_like(&a, &d) != 0;
+        }
+        case GGML_OP_UNARY: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_unary((int) ggml_get_unary_op(op), &a, &d) != 0;
+        }
+        case GGML_OP_GLU: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            vx_tensor b;
+            if (op->src[1]) b = to_vx(op->src[1]);
+            return vx_supports_glu((int) ggml_get_glu_op(op), &a, op->src[1] ? &b : nullptr, &d) != 0;
+        }
+        case GGML_OP_DUP:
+        case GGML_OP_CPY:
+        case GGML_OP_CONT: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_cpy(&a, &d) != 0;
+        }
+        case GGML_OP_CONCAT: {
+            const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
+            return vx_supports_concat(&a, &b, &d, ((const int32_t *) op->op_params)[0]) != 0;
+        }
+        case GGML_OP_SUM: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_sum(&a, &d) != 0;
+        }
         default:
             return false;
     }
@@ -240,6 +290,49 @@ bool supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
 // --------------------------------------------------------------------------- graph_compute
 vx_status compute_node(backend_ctx * ctx, ggml_tensor * node) {
     switch (node->op) {
+        case GGML_OP_ADD:
+        case GGML_OP_SUB:
+        case GGML_OP_MUL:
+        case GGML_OP_DIV: {
+            const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]), d = to_vx(node);
+            return vx_binary(binary_code(node->op), &a, &b, &d, ctx->stream);
+        }
+        case GGML_OP_ADD1: {
+            const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]), d = to_vx(node);
+            return vx_add1(&a, &b, &d, ctx->stream);
+        }
+        case GGML_OP_SCALE: {
+            float sc, bias; // ggml.c: scale, bias
+            memcpy(&sc, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&bias, (const float *) node->op_params + 1, sizeof(float));
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_scale(&a, &d, sc, bias, ctx->stream);
+        }
+        case GGML_OP_UNARY: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_unary((int) ggml_get_unary_op(node), &a, &d, ctx->stream);
+        }
+        case GGML_OP_GLU: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            vx_tensor b;
+            if (node->src[1]) b = to_vx(node->src[1]);
+            return vx_glu((int) ggml_get_glu_op(node), &a, node->src[1] ? &b : nullptr, &d,
+                          ((const int32_t *) node->op_params)[1], ctx->stream);
+        }
+        case GGML_OP_DUP:
+        case GGML_OP_CPY:
+        case GGML_OP_CONT: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_cpy(&a, &d, ctx->stream);
+        }
+        case GGML_OP_CONCAT: {
+            const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]), d = to_vx(node);
+            return vx_concat(&a, &b, &d, ((const int32_t *) node->op_params)[0], ctx->stream);
+        }
+        case GGML_OP_SUM: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_sum(&a, &d, ctx->stream);
+        }
         case GGML_OP_RMS_NORM: {
             float eps;
             memcpy(&eps, node->op_params, sizeof(float));
