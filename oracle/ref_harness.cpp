@@ -15,6 +15,7 @@
 #include <ggml-cpu.h>
 
 #include <chrono>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -212,6 +213,211 @@ int rh_flash_attn_ext(const rh_tensor * q, const rh_tensor * k, const rh_tensor 
     ggml_tensor * out = ggml_flash_attn_ext(g.ctx, tq, tk, tv, tm, scale, max_bias, logit_softcap);
     if (sinks) ggml_flash_attn_ext_add_sinks(out, g.input(&ts));
     return g.run(out, dst, reps, seconds);
+}
+
+} // extern "C"
+
+// ---- MiniCPM backbone --------------------------------------------------------------------
+// The decoder stack as the reference builds it (src/minicpm.cpp:572-846: rms_norm*weight,
+// separate Q/K/V projections, NEOX rope with frequency factors, KV append through ggml_cpy into
+// the cache's write view plus the sum*0 ordering trick, concat(past view, current), flash
+// attention, output projection, muP residual scale, SwiGLU MLP), on whichever backend
+// rh_use_device selected.  Independent sequences ride in ne[3] (batch); batch 1 is the
+// reference's graph node for node.  Weights are Q8_0; norms, rope factors F32.
+namespace {
+
+struct bb_layer {
+    ggml_tensor * w[7];       // q k v o gate up down
+    ggml_tensor * ln[2];      // input_layernorm, post_layernorm
+    ggml_tensor * kc, * vc;   // [D, max_len, Hkv, B]
+};
+
+struct backbone {
+    int n_layer, hidden, n_heads, n_kv, head_dim, ffn, max_len, batch;
+    float eps, residual_scale;
+    bool  use_mup, fused_glu;
+    ggml_context *        wctx = nullptr;
+    ggml_backend_buffer_t wbuf = nullptr;
+    std::vector<bb_layer> layers;
+    ggml_tensor *         final_norm = nullptr;
+    ggml_tensor *         rope_factors = nullptr;
+};
+
+backbone * g_bb = nullptr;
+
+ggml_tensor * bb_norm(ggml_context * c, const backbone & m, ggml_tensor * x, ggml_tensor * w) {
+    return ggml_mul(c, ggml_rms_norm(c, x, m.eps), w);
+}
+
+ggml_tensor * bb_rope(ggml_context * c, const backbone & m, ggml_tensor * x, ggml_tensor * pos) {
+    return ggml_rope_ext(c, x, pos, m.rope_factors, m.head_dim, GGML_ROPE_TYPE_NEOX, 32768, 10000.0f, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f);
+}
+
+ggml_tensor * bb_layer_forward(ggml_context * c, const backbone & m, const bb_layer & L, ggml_tensor * x, ggml_tensor * pos,
+                               ggml_tensor * mask, int T, int n_past, bool write_kv, std::vector<ggml_tensor *> & roots) {
+    const int D = m.head_dim, B = m.batch;
+    ggml_tensor * cur = bb_norm(c, m, x, L.ln[0]);
+    ggml_tensor * q = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[0], cur), D, m.n_heads, T, B);
+    ggml_tensor * k = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[1], cur), D, m.n_kv, T, B);
+    ggml_tensor * v = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[2], cur), D, m.n_kv, T, B);
+    q = bb_rope(c, m, q, pos);
+    k = bb_rope(c, m, k, pos);
+
+    ggml_tensor * kv_sync = nullptr;
+    if (write_kv) {
+        auto write_view = [&](ggml_tensor * cache) {
+            return ggml_view_4d(c, cache, D, m.n_kv, T, B, cache->nb[2], cache->nb[1], cache->nb[3], (size_t) n_past * cache->nb[1]);
+        };
+        ggml_tensor * kw = ggml_cpy(c, k, write_view(L.kc));
+        ggml_tensor * vw = ggml_cpy(c, v, write_view(L.vc));
+        if (L.kc->type == GGML_TYPE_F32) {
+            kv_sync = ggml_add(c, ggml_sum(c, ggml_cont(c, kw)), ggml_sum(c, ggml_cont(c, vw)));
+            kv_sync = ggml_scale(c, kv_sync, 0.0f);
+        } else { // the ordering chain is typed for the F32 cache; an F16 cache appends as extra graph roots
+            roots.push_back(kw);
+            roots.push_back(vw);
+        }
+    }
+    ggml_tensor * k_all = ggml_permute(c, k, 0, 2, 1, 3);
+    ggml_tensor * v_all = ggml_permute(c, v, 0, 2, 1, 3);
+    if (n_past > 0) {
+        auto past_view = [&](ggml_tensor * cache) {
+            return ggml_view_4d(c, cache, D, n_past, m.n_kv, B, cache->nb[1], cache->nb[2], cache->nb[3], 0);
+        };
+        if (L.kc->type != GGML_TYPE_F32) { // an F16 cache: concat needs one type
+            k_all = ggml_cast(c, k_all, L.kc->type);
+            v_all = ggml_cast(c, v_all, L.vc->type);
+        }
+        k_all = ggml_concat(c, past_view(L.kc), k_all, 1);
+        v_all = ggml_concat(c, past_view(L.vc), v_all, 1);
+    }
+    q = ggml_permute(c, q, 0, 2, 1, 3);
+    ggml_tensor * attn = ggml_flash_attn_ext(c, q, k_all, v_all, mask, 1.0f / sqrtf((float) D), 0.0f, 0.0f);
+    if (kv_sync) attn = ggml_add1(c, attn, kv_sync);
+    attn = ggml_reshape_2d(c, attn, (int64_t) m.n_heads * D, (int64_t) T * B);
+    ggml_tensor * attn_out = ggml_mul_mat(c, L.w[3], attn);
+    if (m.use_mup) attn_out = ggml_scale(c, attn_out, m.residual_scale);
+    ggml_tensor * h = ggml_add(c, x, attn_out);
+
+    cur = bb_norm(c, m, h, L.ln[1]);
+    ggml_tensor * gate = ggml_mul_mat(c, L.w[4], cur);
+    ggml_tensor * up   = ggml_mul_mat(c, L.w[5], cur);
+    ggml_tensor * act  = m.fused_glu ? ggml_swiglu_split(c, gate, up) : ggml_mul(c, ggml_silu(c, gate), up);
+    ggml_tensor * down = ggml_mul_mat(c, L.w[6], act);
+    if (m.use_mup) down = ggml_scale(c, down, m.residual_scale);
+    return ggml_add(c, h, down);
+}
+
+} // namespace
+
+extern "C" {
+
+void rh_bb_free(void) {
+    if (!g_bb) return;
+    if (g_bb->wbuf) ggml_backend_buffer_free(g_bb->wbuf);
+    if (g_bb->wctx) ggml_free(g_bb->wctx);
+    delete g_bb;
+    g_bb = nullptr;
+}
+
+// kv_type: GGML_TYPE_F32 (0, the reference's cache, src/minicpm.cpp:182-183) or GGML_TYPE_F16 (1)
+int rh_bb_create(int n_layer, int hidden, int n_heads, int n_kv, int head_dim, int ffn, int max_len, int batch,
+                 float eps, int use_mup, float scale_depth, int kv_type) {
+    if (!g_backend) return 100;
+    rh_bb_free();
+    backbone * m = new backbone;
+    m->n_layer = n_layer; m->hidden = hidden; m->n_heads = n_heads; m->n_kv = n_kv; m->head_dim = head_dim;
+    m->ffn = ffn; m->max_len = max_len; m->batch = batch; m->eps = eps; m->use_mup = use_mup != 0;
+    m->residual_scale = use_mup ? scale_depth / sqrtf((float) (n_layer > 0 ? n_layer : 1)) : 1.0f;
+    ggml_init_params ip = { ggml_tensor_overhead() * ((size_t) n_layer * 11 + 4), nullptr, true };
+    m->wctx = ggml_init(ip);
+    const int64_t qd = (int64_t) n_heads * head_dim, kd = (int64_t) n_kv * head_dim;
+    const int64_t shapes[7][2] = { { hidden, qd }, { hidden, kd }, { hidden, kd }, { qd, hidden }, { hidden, ffn }, { hidden, ffn }, { ffn, hidden } };
+    m->layers.resize((size_t) n_layer);
+    for (auto & L : m->layers) {
+        for (int i = 0; i < 7; ++i) L.w[i] = ggml_new_tensor_2d(m->wctx, GGML_TYPE_Q8_0, shapes[i][0], shapes[i][1]);
+        for (int i = 0; i < 2; ++i) L.ln[i] = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, hidden);
+        L.kc = ggml_new_tensor_4d(m->wctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
+        L.vc = ggml_new_tensor_4d(m->wctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
+    }
+    m->final_norm   = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, hidden);
+    m->rope_factors = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, head_dim / 2);
+    m->wbuf = ggml_backend_alloc_ctx_tensors(m->wctx, g_backend);
+    if (!m->wbuf) { g_bb = m; rh_bb_free(); return 101; }
+    ggml_backend_buffer_clear(m->wbuf, 0);
+    // mlp_forward fuses SwiGLU when the weights are not in host memory (src/minicpm.cpp:729-745)
+    m->fused_glu = !ggml_backend_buffer_is_host(m->wbuf);
+    g_bb = m;
+    return 0;
+}
+
+// which: 0..6 = q k v o gate up down (Q8_0 rows), 7 = input_layernorm, 8 = post_layernorm;
+// layer -1: which 0 = final norm, 1 = rope frequency factors
+int rh_bb_set(int layer, int which, const void * data, size_t nbytes) {
+    if (!g_bb) return 100;
+    ggml_tensor * t = nullptr;
+    if (layer < 0) t = which == 0 ? g_bb->final_norm : g_bb->rope_factors;
+    else if (layer < g_bb->n_layer) t = which < 7 ? g_bb->layers[(size_t) layer].w[which] : g_bb->layers[(size_t) layer].ln[which - 7];
+    if (!t || ggml_nbytes(t) != nbytes) return 101;
+    ggml_backend_tensor_set(t, data, 0, nbytes);
+    return 0;
+}
+
+// x: [hidden, n_tokens, batch] F32 (dense); mask: F16 [n_past + n_tokens, n_tokens] or NULL;
+// out: [hidden, n_tokens, batch] after the final norm.  Graph and compute buffer are rebuilt on
+// every call, as the reference does per step (src/voxcpm.cpp:489-495); only the graph_compute
+// calls are timed.
+int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_past, int write_kv, float * out,
+                  int reps, double * seconds) {
+    if (!g_bb || !g_backend) return 100;
+    const backbone & m = *g_bb;
+    const int T = n_tokens, B = m.batch;
+    if (n_past + T > m.max_len) return 104;
+    const size_t n_nodes = (size_t) m.n_layer * 64 + 64;
+    ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
+    ggml_context * c = ggml_init(ip);
+    ggml_tensor * inp = ggml_new_tensor_2d(c, GGML_TYPE_F32, m.hidden, (int64_t) T * B);
+    ggml_tensor * pos = ggml_new_tensor_1d(c, GGML_TYPE_I32, T);
+    ggml_tensor * msk = mask ? ggml_new_tensor_2d(c, GGML_TYPE_F16, n_past + T, T) : nullptr;
+    ggml_set_input(inp); ggml_set_input(pos);
+    if (msk) ggml_set_input(msk);
+    ggml_tensor * h = inp;
+    std::vector<ggml_tensor *> roots;
+    for (const auto & L : m.layers) h = bb_layer_forward(c, m, L, h, pos, msk, T, n_past, write_kv != 0, roots);
+    h = bb_norm(c, m, h, m.final_norm);
+    ggml_set_output(h);
+    ggml_cgraph * gf = ggml_new_graph_custom(c, n_nodes, false);
+    ggml_build_forward_expand(gf, h);
+    for (ggml_tensor * r : roots) ggml_build_forward_expand(gf, r);
+    ggml_gallocr_t ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend));
+    int rc = 0;
+    if (!ggml_gallocr_alloc_graph(ga, gf)) rc = 101;
+    if (!rc) {
+        ggml_backend_tensor_set(inp, x, 0, ggml_nbytes(inp));
+        std::vector<int32_t> p((size_t) T);
+        for (int i = 0; i < T; ++i) p[(size_t) i] = n_past + i;
+        ggml_backend_tensor_set(pos, p.data(), 0, ggml_nbytes(pos));
+        if (msk) ggml_backend_tensor_set(msk, mask, 0, ggml_nbytes(msk));
+        if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
+    }
+    if (!rc && reps > 0 && seconds) {
+        double best = 1e30, total = 0;
+        for (int r = 0; r < reps && !rc; ++r) {
+            auto t0 = std::chrono::steady_clock::now();
+            if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
+            auto t1 = std::chrono::steady_clock::now();
+            const double dt = std::chrono::duration<double>(t1 - t0).count();
+            total += dt;
+            if (dt < best) best = dt;
+        }
+        seconds[0] = total / reps;
+        seconds[1] = best;
+    }
+    if (!rc && out) ggml_backend_tensor_get(h, out, 0, ggml_nbytes(h));
+    if (seconds) seconds[2] = (double) ggml_graph_n_nodes(gf);
+    ggml_gallocr_free(ga);
+    ggml_free(c);
+    return rc;
 }
 
 } // extern "C"

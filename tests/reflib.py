@@ -172,6 +172,9 @@ def load_ref():
     lib.rh_rope.argtypes = [TP, i32p, f32p, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [C.c_int, f64p]
     lib.rh_soft_max.argtypes = [TP, TP, f32p, TP, C.c_float, C.c_float, C.c_int, f64p]
     lib.rh_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, C.c_int, f64p]
+    lib.rh_bb_create.argtypes = [C.c_int] * 8 + [C.c_float, C.c_int, C.c_float, C.c_int]
+    lib.rh_bb_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    lib.rh_bb_forward.argtypes = [f32p, u16p, C.c_int, C.c_int, C.c_int, f32p, C.c_int, f64p]
     assert lib.rh_use_device(b"CPU", min(8, os.cpu_count() or 1), 0) == 0
     _ref = lib
     return lib
@@ -319,3 +322,53 @@ def causal_mask(n_q, n_kv, n_past=0):
     m = np.empty((n_q, n_kv), np.uint16)
     load_oracle().orc_causal_mask(ptr(pos, C.c_int32), n_q, n_kv, ptr(m, C.c_uint16))
     return m.view(np.float16)
+
+
+# ------------------------------------------------------------------- MiniCPM backbone
+BB_WEIGHTS = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+
+
+def backbone_params(tag, n_layer, hidden=1024, n_heads=16, n_kv=2, head_dim=64, ffn=4096):
+    """Seeded weights of BASELINE config 4: N(0, 0.02) quantised to Q8_0 with the reference's
+    weight quantizer, norm weights near 1, rope frequency factors in [1, 2)."""
+    qd, kd = n_heads * head_dim, n_kv * head_dim
+    shapes = {"q_proj": (qd, hidden), "k_proj": (kd, hidden), "v_proj": (kd, hidden), "o_proj": (hidden, qd),
+              "gate_proj": (ffn, hidden), "up_proj": (ffn, hidden), "down_proj": (hidden, ffn)}
+    layers = []
+    for li in range(n_layer):
+        lw = {n: quantize_q8_0((rng(tag, li, n).standard_normal(shapes[n]) * 0.02).astype(np.float32)) for n in BB_WEIGHTS}
+        for n in ("input_layernorm", "post_layernorm"):
+            lw[n] = (1.0 + 0.1 * rng(tag, li, n).standard_normal(hidden)).astype(np.float32)
+        layers.append(lw)
+    final = (1.0 + 0.1 * rng(tag, "final").standard_normal(hidden)).astype(np.float32)
+    factors = (1.0 + rng(tag, "rope").random(head_dim // 2)).astype(np.float32)
+    return {"layers": layers, "final_norm": final, "rope_factors": factors, "shapes": shapes,
+            "dims": dict(n_layer=n_layer, hidden=hidden, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, ffn=ffn)}
+
+
+def ref_backbone_create(params, max_len, batch, use_mup=False, kv_f16=False, eps=1e-5):
+    """Builds the decoder stack on the harness's current device (rh_use_device) and uploads params."""
+    lib = load_ref()
+    d = params["dims"]
+    rc = lib.rh_bb_create(d["n_layer"], d["hidden"], d["n_heads"], d["n_kv"], d["head_dim"], d["ffn"], max_len, batch,
+                          eps, int(use_mup), 1.4, 1 if kv_f16 else 0)
+    assert rc == 0, rc
+    for li, lw in enumerate(params["layers"]):
+        for wi, n in enumerate(BB_WEIGHTS + ("input_layernorm", "post_layernorm")):
+            a = np.ascontiguousarray(lw[n])
+            assert lib.rh_bb_set(li, wi, a.ctypes.data, a.nbytes) == 0, (li, n)
+    assert lib.rh_bb_set(-1, 0, params["final_norm"].ctypes.data, params["final_norm"].nbytes) == 0
+    assert lib.rh_bb_set(-1, 1, params["rope_factors"].ctypes.data, params["rope_factors"].nbytes) == 0
+
+
+def ref_backbone_forward(x, n_past, mask=None, write_kv=True, reps=0):
+    """x: (batch, n_tokens, hidden) f32.  Returns (out, seconds[mean, best], n_nodes)."""
+    lib = load_ref()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    sec = np.zeros(3, np.float64)
+    m = None if mask is None else np.ascontiguousarray(mask).view(np.uint16)
+    rc = lib.rh_bb_forward(ptr(x, C.c_float), None if m is None else ptr(m, C.c_uint16), x.shape[1], n_past, int(write_kv),
+                           ptr(out, C.c_float), reps, ptr(sec, C.c_double))
+    assert rc == 0, rc
+    return out, sec[:2].copy(), int(sec[2])

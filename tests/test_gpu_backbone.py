@@ -1,0 +1,74 @@
+"""The whole decoder stack (BASELINE config 4's shape, fewer layers) three ways on the same seeded
+Q8_0 weights: the reference-structured ggml graph on ggml-cpu (oracle/_ref), the same graph run
+entirely on the gfx950 backend plugin through ggml's own graph_compute, and the host-side
+mirror in voxcpm.cpp_amd/backbone.py issuing vx_* calls through the C ABI.  Prefill, then decode
+steps that read the KV cache the earlier calls appended."""
+import numpy as np
+import pytest
+
+import reflib
+from reflib import nmse, rng
+
+pytestmark = pytest.mark.gpu
+
+N_LAYER, MAX_LEN, BATCH, T0, STEPS = 3, 64, 2, 9, 3
+
+
+def run_reference(params, xs, device, kv_f16, use_mup):
+    ref = reflib.load_ref()
+    assert ref.rh_use_device(device, 8, 0) == 0
+    reflib.ref_backbone_create(params, MAX_LEN, BATCH, use_mup=use_mup, kv_f16=kv_f16)
+    outs, n_past = [], 0
+    for x in xs:
+        T = x.shape[1]
+        mask = reflib.causal_mask(T, T) if T > 1 else None
+        o, _, n_nodes = reflib.ref_backbone_forward(x, n_past, mask)
+        outs.append(o)
+        n_past += T
+    ref.rh_bb_free()
+    assert ref.rh_use_device(b"CPU", 8, 0) == 0
+    return outs, n_nodes
+
+
+@pytest.mark.parametrize("kv_f16,use_mup", [(False, True), (True, False)])
+def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
+    import torch
+    from voxcpm_cpp_amd import backbone as bb
+    print(f"backbone: {N_LAYER} layers, batch {BATCH}, prefill {T0} + {STEPS} decode steps, kv_f16={kv_f16} mup={use_mup}", flush=True)
+    params = reflib.backbone_params("bb", N_LAYER)
+    xs = [rng("bb", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)]
+    xs += [rng("bb", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(STEPS)]
+
+    cpu, n_nodes = run_reference(params, xs, b"CPU", kv_f16, use_mup)
+    print(f"   ggml-cpu graph: {n_nodes} nodes per decode step", flush=True)
+
+    # the same ggml graph, every node on the plugin (direct ggml_backend_graph_compute, no scheduler)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug, _ = run_reference(params, xs, b"GFX950_0", kv_f16, use_mup)
+    for i, (a, b) in enumerate(zip(cpu, plug)):
+        e = nmse(a, b)
+        print(f"   plugin vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+        assert e <= 1e-4
+
+    # the C-ABI mirror, Q8 activations (ggml-cpu's arithmetic) and float activations.  Even with
+    # ggml-cpu's integer dots an activation one ulp away can round to the neighbouring int8, so the
+    # stack agrees to ~1e-5 NMSE, not bit for bit; float activations sit at ggml's own 5e-4 / op bar.
+    for act, bar in ((gpu.ACT_Q8, 5e-5), (gpu.ACT_FLOAT, 1e-4)):
+        m = bb.MiniCPMBackbone(n_layer=N_LAYER, max_length=MAX_LEN, batch=BATCH, use_mup=use_mup, kv_f16=kv_f16, act_mode=act)
+        for li, lw in enumerate(params["layers"]):
+            for n in reflib.BB_WEIGHTS:
+                m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+            for n in ("input_layernorm", "post_layernorm"):
+                m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+        m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+        m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+        n_past = 0
+        for i, x in enumerate(xs):
+            T = x.shape[1]
+            mask = torch.from_numpy(reflib.causal_mask(T, T)).cuda() if T > 1 else None
+            got = m.forward(torch.from_numpy(x).cuda(), n_past, mask)
+            torch.cuda.synchronize()
+            e = nmse(cpu[i], got.cpu().numpy())
+            print(f"   C ABI mirror (act_mode {act}) vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+            assert e <= bar
+            n_past += T

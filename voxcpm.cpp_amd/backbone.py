@@ -1,0 +1,185 @@
+"""Host-side mirror of the reference's MiniCPM decoder stack over the C ABI.
+
+`MiniCPMBackbone.forward` issues, operator for operator, what `MiniCPMModel::layer_forward`,
+`attention_forward` and `mlp_forward` put into a ggml graph (src/minicpm.cpp:572-846 of the
+reference): rms_norm * weight, separate Q/K/V projections, NEOX rope with frequency factors,
+the KV append (ggml_cpy into the cache's write view, followed by the cont/sum/scale-by-zero
+chain the reference uses to order the write), concat(past view, current keys), flash
+attention, add1, the output projection, the muP residual scale and the SwiGLU MLP.  Every
+operator is one vx_* call on device tensors; nothing is computed on the host.
+
+Independent sequences (the CFG pair, concurrent streams) ride in the batch dimension, which is
+ggml's ne[3]; with batch 1 the call sequence is the reference's graph node for node.
+
+A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and intermediates
+are built once, so a plan can be replayed from a captured HIP graph.
+"""
+import math
+
+from . import (ACT_FLOAT, BIN_ADD, BIN_MUL, F16, F32, GLU_SWIGLU, _p, _stream, check, desc, desc_q8, lib)
+
+WEIGHT_NAMES = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+
+
+class MiniCPMBackbone:
+    def __init__(self, n_layer=24, hidden=1024, n_heads=16, n_kv_heads=2, head_dim=64, ffn=4096, max_length=1024,
+                 batch=1, eps=1e-5, use_mup=False, scale_depth=1.4, kv_f16=False, act_mode=ACT_FLOAT,
+                 rope_base=10000.0, rope_original_max=32768):
+        import torch
+        self.torch = torch
+        self.n_layer, self.hidden, self.n_heads, self.n_kv, self.D = n_layer, hidden, n_heads, n_kv_heads, head_dim
+        self.ffn, self.max_length, self.batch, self.eps = ffn, max_length, batch, eps
+        self.use_mup = use_mup
+        self.residual_scale = scale_depth / math.sqrt(max(1, n_layer)) if use_mup else 1.0
+        self.act_mode = act_mode
+        self.rope_base, self.rope_original_max = rope_base, rope_original_max
+        self.kv_dtype = torch.float16 if kv_f16 else torch.float32
+        dev = "cuda"
+        # KV cache, src/minicpm.cpp:178-187: per layer K and V [head_dim, max_length, n_kv_heads] (x batch)
+        self.k_cache = [torch.zeros((batch, n_kv_heads, max_length, head_dim), dtype=self.kv_dtype, device=dev) for _ in range(n_layer)]
+        self.v_cache = [torch.zeros((batch, n_kv_heads, max_length, head_dim), dtype=self.kv_dtype, device=dev) for _ in range(n_layer)]
+        self.weights = [dict() for _ in range(n_layer)]   # name -> (uint8 Q8_0 rows, K)
+        self.norms = [dict() for _ in range(n_layer)]     # "input_layernorm" / "post_layernorm" -> f32 [hidden]
+        self.final_norm = None
+        self.rope_factors = None                          # f32 [head_dim / 2] or None
+
+    # ---- loading --------------------------------------------------------------------------
+    def set_weight(self, layer, name, q8_rows, K):
+        """q8_rows: uint8 tensor (rows, K/32*34) of Q8_0 blocks, on the device."""
+        self.weights[layer][name] = (q8_rows, K)
+
+    def set_norm(self, layer, name, w):
+        if layer < 0:
+            self.final_norm = w
+        else:
+            self.norms[layer][name] = w
+
+    def clear_cache(self):
+        for t in self.k_cache + self.v_cache:
+            t.zero_()
+
+    # ---- one (n_tokens, n_past) call list -----------------------------------------------------
+    def plan(self, x, n_tokens, n_past, mask=None, write_kv=True):
+        """x: (batch, n_tokens, hidden) f32 device tensor, read at replay time.  Returns
+        (run, out): run() enqueues the whole stack on torch's current stream; out is the
+        (batch, n_tokens, hidden) result tensor it fills."""
+        torch, L = self.torch, lib()
+        B, T, H, Hkv, D = self.batch, n_tokens, self.n_heads, self.n_kv, self.D
+        assert x.shape == (B, T, self.hidden) and x.dtype == torch.float32 and x.is_contiguous()
+        assert n_past + T <= self.max_length
+        dev = x.device
+        f32 = torch.float32
+        N = B * T
+
+        def new(*shape, dtype=f32):
+            return torch.empty(shape, dtype=dtype, device=dev)
+
+        pos = torch.arange(n_past, n_past + T, dtype=torch.int32, device=dev)
+        seq_len = n_past + T
+        attn_factor = 1.0
+        if seq_len > self.rope_original_max > 1:  # apply_rope, src/minicpm.cpp:590-594
+            attn_factor = math.sqrt(1.0 + math.log(seq_len / self.rope_original_max) / math.log(self.rope_original_max))
+        keep = [pos, x, mask]
+        calls = []
+
+        def call(fn, *args):
+            calls.append((fn, args))
+
+        # buffers reused by every layer (the stack is sequential)
+        normed, q, k, v = new(N, self.hidden), new(N, H * D), new(N, Hkv * D), new(N, Hkv * D)
+        kcont, vcont = new(B, T, Hkv, D, dtype=self.kv_dtype), new(B, T, Hkv, D, dtype=self.kv_dtype)
+        sk, sv = new(1, dtype=self.kv_dtype), new(1, dtype=self.kv_dtype)
+        sync = new(1, dtype=self.kv_dtype)
+        kall = new(B, Hkv, seq_len, D, dtype=self.kv_dtype) if n_past > 0 else None
+        vall = new(B, Hkv, seq_len, D, dtype=self.kv_dtype) if n_past > 0 else None
+        kcast = new(B, Hkv, T, D, dtype=self.kv_dtype) if (n_past > 0 and self.kv_dtype != f32) else None
+        vcast = new(B, Hkv, T, D, dtype=self.kv_dtype) if (n_past > 0 and self.kv_dtype != f32) else None
+        attn, attn_o = new(B, T, H, D), new(N, self.hidden)
+        gate, up, act, down = new(N, self.ffn), new(N, self.ffn), new(N, self.ffn), new(N, self.hidden)
+        hs = [new(N, self.hidden) for _ in range(2)]   # residual stream ping-pong
+        h_mid = new(N, self.hidden)
+        out = new(B, T, self.hidden)
+        keep += [normed, q, k, v, kcont, vcont, sk, sv, sync, kall, vall, kcast, vcast, attn, attn_o, gate, up, act, down, h_mid, out] + hs
+        # The cont/sum/scale-by-zero chain only exists to order the cache write inside a ggml graph
+        # and is typed for the reference's F32 cache (ggml's SCALE and ADD1 are F32 operators); with an
+        # F16 cache the append is the bare ggml_cpy, ordered by the stream.
+        chain = write_kv and self.kv_dtype == f32
+        scale = 1.0 / math.sqrt(D)
+        ff = _p(self.rope_factors)
+        cur_x = x.view(N, self.hidden)
+        for li in range(self.n_layer):
+            w, nrm = self.weights[li], self.norms[li]
+            kc, vc = self.k_cache[li], self.v_cache[li]
+            wd = {n: desc_q8(*w[n]) for n in WEIGHT_NAMES}
+            # -- attention_forward
+            call(L.vx_rms_norm, desc(cur_x), desc(normed), self.eps)
+            call(L.vx_binary, BIN_MUL, desc(normed), desc(nrm["input_layernorm"]), desc(normed))
+            call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
+            call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
+            call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
+            q4, k4, v4 = q.view(B, T, H, D), k.view(B, T, Hkv, D), v.view(B, T, Hkv, D)
+            for t4 in (q4, k4):
+                call(L.vx_rope, desc(t4), _p(pos), ff, desc(t4), D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0,
+                     attn_factor, 32.0, 1.0)
+            if write_kv:
+                kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236
+                vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
+                call(L.vx_cpy, desc(k4), desc(kw))
+                call(L.vx_cpy, desc(v4), desc(vw))
+                keep += [kw, vw]
+            if chain:
+                call(L.vx_cpy, desc(kw), desc(kcont))
+                call(L.vx_sum, desc(kcont), desc(sk))
+                call(L.vx_cpy, desc(vw), desc(vcont))
+                call(L.vx_sum, desc(vcont), desc(sv))
+                call(L.vx_binary, BIN_ADD, desc(sk), desc(sv), desc(sync))
+                call(L.vx_scale, desc(sync), desc(sync), 0.0, 0.0)
+            k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)
+            if n_past > 0:
+                if kcast is not None:
+                    call(L.vx_cpy, desc(k_all), desc(kcast))
+                    call(L.vx_cpy, desc(v_all), desc(vcast))
+                    k_all, v_all = kcast, vcast
+                call(L.vx_concat, desc(kc[:, :, :n_past]), desc(k_all), desc(kall), 1)
+                call(L.vx_concat, desc(vc[:, :, :n_past]), desc(v_all), desc(vall), 1)
+                k_all, v_all = kall, vall
+            call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
+                 scale, 0.0, 0.0)
+            if chain:
+                call(L.vx_add1, desc(attn), desc(sync), desc(attn))
+            call(L.vx_mul_mat, wd["o_proj"], desc(attn.view(N, H * D)), desc(attn_o), self.act_mode)
+            if self.use_mup:
+                call(L.vx_scale, desc(attn_o), desc(attn_o), self.residual_scale, 0.0)
+            call(L.vx_binary, BIN_ADD, desc(cur_x), desc(attn_o), desc(h_mid))
+            # -- mlp_forward
+            call(L.vx_rms_norm, desc(h_mid), desc(normed), self.eps)
+            call(L.vx_binary, BIN_MUL, desc(normed), desc(nrm["post_layernorm"]), desc(normed))
+            call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
+            call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
+            call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)
+            call(L.vx_mul_mat, wd["down_proj"], desc(act), desc(down), self.act_mode)
+            if self.use_mup:
+                call(L.vx_scale, desc(down), desc(down), self.residual_scale, 0.0)
+            nxt = hs[li % 2]
+            call(L.vx_binary, BIN_ADD, desc(h_mid), desc(down), desc(nxt))
+            cur_x = nxt
+        o2 = out.view(N, self.hidden)
+        call(L.vx_rms_norm, desc(cur_x), desc(o2), self.eps)
+        call(L.vx_binary, BIN_MUL, desc(o2), desc(self.final_norm), desc(o2))
+
+        def run():
+            st = _stream()
+            for fn, args in calls:
+                rc = fn(*args, st)
+                if rc:
+                    check(rc, fn.__name__)
+
+        run._keep = keep
+        run.n_calls = len(calls)
+        return run, out
+
+    def forward(self, x, n_past=0, mask=None, write_kv=True):
+        """MiniCPMModel::forward / forward_step: x (batch, n_tokens, hidden) -> same shape."""
+        run, out = self.plan(x.contiguous(), x.shape[1], n_past, mask, write_kv)
+        run()
+        return out
