@@ -198,6 +198,76 @@ def cpu_baseline(batch, length, threads):
             "sample": f"{reps} repeats of one layer on the scalar C oracle (oracle/_ref not prebuilt)"}
 
 
+def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256):
+    """BASELINE config 4: the whole decoder stack with Q8_0 weights (hidden 1024, 16/2 heads, FFN 4096),
+    batch 2, prefill 512 tokens then 256 decode steps.  The GPU side is the host-side mirror of the
+    reference's layer_forward over the C ABI (voxcpm.cpp_amd/backbone.py, F32 KV cache as in the
+    reference); a decode step is replayed from a captured HIP graph.  Four KV lengths spread over the
+    256-step range are captured and each replayed steps/4 times, so the timed work is that of the
+    512 -> 768 decode.  ggml-cpu runs the reference-structured graph of the same stack beside it."""
+    import torch
+    import reflib
+    bbmod = __import__("voxcpm_cpp_amd.backbone", fromlist=["MiniCPMBackbone"])
+    params = reflib.backbone_params("bench-bb", 1)   # one layer's seeded weights, placed in `layers` separate buffers
+    lw = params["layers"][0]
+    max_len = prefill + steps
+    m = bbmod.MiniCPMBackbone(n_layer=layers, max_length=max_len, batch=batch, use_mup=True, kv_f16=False)
+    for li in range(layers):
+        for n in reflib.BB_WEIGHTS:
+            m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+        for n in ("input_layernorm", "post_layernorm"):
+            m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+    m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+    m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+    weight_bytes = layers * sum(lw[n].nbytes for n in reflib.BB_WEIGHTS)
+
+    xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
+    mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
+    run_p, _ = m.plan(xp, prefill, 0, mask)
+    t_prefill = timer.run(run_p, iters=3, warmup=1)
+
+    x1 = torch.randn((batch, 1, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    points = [prefill + (2 * i + 1) * steps // 8 for i in range(4)]
+    replays, n_calls = [], 0
+    for n_past in points:
+        run_d, _ = m.plan(x1, 1, n_past)
+        n_calls = run_d.n_calls
+        replays.append((graphed(run_d, side), run_d))
+    per = steps // 4
+    for rp, _ in replays:
+        rp()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for rp, _ in replays:
+        for _ in range(per):
+            rp()
+    torch.cuda.synchronize()
+    t_step = (time.perf_counter() - t0) / (per * 4)
+    kvb = layers * 2 * batch * HKV * (prefill + steps // 2) * D * 4
+    res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
+           "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
+           "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": batch * prefill / t_prefill,
+           "kv_cache": "f32 (the reference's cache type)", "launch": "captured HIP graph per step, KV lengths " + str(points)}
+    del replays, m
+    ref = reflib.load_ref() if with_cpu else None
+    if ref is not None:
+        assert ref.rh_use_device(b"CPU", threads, 0) == 0
+        params["dims"]["n_layer"] = layers
+        params["layers"] = [lw] * layers
+        reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=False)
+        xph = xp.cpu().numpy()
+        tp0 = time.perf_counter()
+        reflib.ref_backbone_forward(xph, 0, reflib.causal_mask(prefill, prefill))
+        cpu_prefill = time.perf_counter() - tp0
+        _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), prefill + steps // 2, None, reps=40)
+        ref.rh_bb_free()
+        res["ggml_cpu"] = {"decode_steps_per_s": 1.0 / mean, "ms_per_step": mean * 1e3, "best_ms": best * 1e3, "threads": threads,
+                           "graph_nodes": n_nodes, "prefill_ms": cpu_prefill * 1e3,
+                           "sample": f"40 repeats of the decode step at KV length {prefill + steps // 2}, one prefill"}
+        res["speedup_vs_ggml_cpu"] = mean / t_step
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -293,9 +363,12 @@ def main():
             others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12}
             del keep
 
+    threads = min(16, os.cpu_count() or 1)
+    if not args.no_others:
+        others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu)
+
     cpu = None
     if not args.no_cpu:
-        threads = min(16, os.cpu_count() or 1)
         cpu = cpu_baseline(B, L, threads)
 
     line = {

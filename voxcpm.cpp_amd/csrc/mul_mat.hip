@@ -20,8 +20,8 @@
 // integer block dot and the scale is d_w * d_x.
 //
 // Tiling: a work-group is 4 waves.  GEMM shape (many tokens): 64 rows x 16*TT tokens, each
-// wave 16 rows.  GEMV shape (<= 16 tokens): 16 rows, the 4 waves split K and reduce through
-// LDS, so a 1024-row projection still spreads over 64 work-groups.
+// wave 16 rows.  GEMV shape (<= 16 tokens): its own streaming kernel (gemv_kernel below); the
+// staged K-split variant of the GEMM kernel remains for F32 weights and ragged K.
 //
 // Algorithmic HBM bytes: weights once (34 bytes per 32 weights) + activations + output.
 #include "vx_common.hpp"
@@ -204,8 +204,177 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
     }
 }
 
+
+// ---- GEMV shape: at most 16 tokens (decode) ---------------------------------------------------
+// Pure weight streaming, so the kernel is built around memory-level parallelism: a work-group owns
+// 16 weight rows, its NW waves take interleaved 32-wide k blocks of those rows, and every wave
+// issues the loads of all its blocks (GV_UNROLL at a time, normally all of them) before anything
+// else happens.  While they fly the work-group converts the few activation rows to f16 (or
+// quantises them, VX_ACT_Q8) into LDS, [token][k].  Then one MFMA per block -- tokens that do not
+// exist are zero lanes of the A operand -- and a fixed-order reduction of the waves' partial sums
+// through LDS.  With K = 1024 and 4 waves, or K = 4096 and 16 waves, the whole matrix is requested
+// in one round trip to HBM.
+constexpr int GV_UNROLL = 8;
+
+template <int WT, bool ACT_Q8, int NW>
+__global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
+    extern __shared__ __attribute__((aligned(16))) char gv_smem[];
+    const int64_t nkb = a.K / 32;
+    _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][K]
+    float *    xd  = (float *) (gv_smem + (size_t) a.N * a.K * 2);           // [N][K/32] (ACT_Q8)
+    float4_t * red = (float4_t *) (gv_smem + (size_t) a.N * a.K * 2 + (ACT_Q8 ? (size_t) a.N * nkb * 4 : 0));
+
+    const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
+    const int j = lane >> 4, c = lane & 15;
+    const int     batch = blockIdx.z;
+    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    const int64_t row0 = (int64_t) blockIdx.x * 16;
+    const char *  wrow = wb + (uint64_t) min(row0 + c, a.M - 1) * a.nb01;
+    const int     N = (int) a.N;
+
+    // ---- this wave's weight blocks: kb = wid + NW * i
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    u32x2    wq[GV_UNROLL];
+    half8_t  wh[GV_UNROLL];
+    _Float16 wdv[GV_UNROLL];
+    auto load_blocks = [&](int64_t i0) {
+#pragma unroll
+        for (int u = 0; u < GV_UNROLL; ++u) {
+            const int64_t kb = min((int64_t) wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, result unused
+            if constexpr (WT == WT_Q8) {
+                const char * bp = wrow + (uint64_t) kb * VX_Q8_BLOCK;
+                wdv[u] = *(const _Float16 *) bp;
+                __builtin_memcpy(&wq[u], bp + 2 + 8 * j, 8);
+            } else {
+                __builtin_memcpy(&wh[u], wrow + (uint64_t) (kb * 32 + 8 * j) * 2, 16);
+            }
+        }
+    };
+    // ---- activations -> LDS.  A thread's first unit (8 consecutive k of one token; usually its only
+    // one) is requested before the weights: loads return in order, so its conversion then waits for
+    // an L2 hit only, not for the weight stream behind it.
+    const int upr = (int) (a.K / 8), units = N * upr;
+    auto fetch = [&](int unit, float4_t & v0, float4_t & v1) {
+        const int t = unit / upr, u = unit % upr;
+        const float * xp = (const float *) (xb + (uint64_t) t * a.nb11) + 8 * u;
+        if (a.x_aligned) {
+            v0 = ((const float4_t *) xp)[0]; v1 = ((const float4_t *) xp)[1];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v0[i] = xp[i]; v1[i] = xp[4 + i]; }
+        }
+    };
+    auto stage = [&](int unit, const float4_t & v0, const float4_t & v1) {
+        const int t = unit / upr, u = unit % upr;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
+        half8_t h;
+        if constexpr (ACT_Q8) { // 4 consecutive units = one 32-wide block (K/8 is a multiple of 4)
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+            amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+            const float d  = amax / 127.f;
+            const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
+            if ((u & 3) == 0) xd[t * nkb + (u >> 2)] = (float) (_Float16) d;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
+        }
+        *(half8_t *) (xs + (size_t) t * a.K + 8 * u) = h;
+    };
+    float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0};
+    if (tid < units) fetch(tid, f0, f1);
+    load_blocks(0);
+    if (tid < units) stage(tid, f0, f1);
+    for (int unit = tid + 64 * NW; unit < units; unit += 64 * NW) {
+        fetch(unit, f0, f1);
+        stage(unit, f0, f1);
+    }
+    __syncthreads();
+
+    float4_t acc = {0, 0, 0, 0};
+    const int64_t per = (nkb + NW - 1) / NW; // blocks per wave
+    for (int64_t i0 = 0; i0 < per; i0 += GV_UNROLL) {
+        if (i0) load_blocks(i0);
+#pragma unroll
+        for (int u = 0; u < GV_UNROLL; ++u) {
+            const int64_t kb = (int64_t) wid + NW * (i0 + u);
+            if (kb >= nkb) break; // wave-uniform
+            half8_t aop = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (c < N) aop = *(const half8_t *) (xs + (size_t) c * a.K + kb * 32 + 8 * j);
+            if constexpr (WT == WT_Q8) {
+                const half8_t  bop = q8_to_half8(wq[u][0], wq[u][1]);
+                const float4_t blk = mfma16(aop, bop, float4_t{0, 0, 0, 0});
+                const float    dw  = (float) wdv[u];
+                if constexpr (ACT_Q8) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[r] += blk[r] * (dw * (4 * j + r < N ? xd[(4 * j + r) * nkb + kb] : 0.0f));
+                } else {
+                    acc += blk * dw;
+                }
+            } else {
+                acc = mfma16(aop, wh[u], acc);
+            }
+        }
+    }
+
+    if constexpr (NW > 1) {
+        if (wid > 0) red[(wid - 1) * 64 + lane] = acc;
+        __syncthreads();
+        if (wid > 0) return;
+#pragma unroll
+        for (int ww = 0; ww < NW - 1; ++ww) acc += red[ww * 64 + lane];
+    }
+    // lane (j,c), register r: token 4j + r, row row0 + c
+    if (row0 + c < a.M) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int tok = 4 * j + r;
+            if (tok < N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) (row0 + c) * 4) = acc[r];
+        }
+    }
+}
+
+size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
+    return (size_t) a.N * a.K * 2 + (act_q8 ? (size_t) a.N * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16;
+}
+
+// waves per work-group: about GV_UNROLL blocks per wave, so every load is issued up front
+int gemv_waves(const mm_args & a) {
+    const int64_t nkb = a.K / 32;
+    int nw = 1;
+    while (nw < 16 && nkb > (int64_t) nw * GV_UNROLL) nw *= 2;
+    return nw;
+}
+
+template <int WT, bool ACT_Q8>
+bool launch_gemv(const mm_args & a, int nbatch, hipStream_t st) {
+    if (a.N > 16 || a.K % 32 || a.K < 32) return false;
+    const int nw = gemv_waves(a);
+    const size_t smem = gemv_smem(a, ACT_Q8, nw);
+    if (smem > 64 * 1024) return false;
+    const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
+    switch (nw) {
+        case 1:  gemv_kernel<WT, ACT_Q8, 1><<<grid, dim3(64), smem, st>>>(a); break;
+        case 2:  gemv_kernel<WT, ACT_Q8, 2><<<grid, dim3(128), smem, st>>>(a); break;
+        case 4:  gemv_kernel<WT, ACT_Q8, 4><<<grid, dim3(256), smem, st>>>(a); break;
+        case 8:  gemv_kernel<WT, ACT_Q8, 8><<<grid, dim3(512), smem, st>>>(a); break;
+        default: gemv_kernel<WT, ACT_Q8, 16><<<grid, dim3(1024), smem, st>>>(a); break;
+    }
+    return true;
+}
+
 template <int WT, bool ACT_Q8>
 void launch(const mm_args & a, int nbatch, hipStream_t st) {
+    if constexpr (WT != WT_F32) { if (launch_gemv<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
         mm_kernel<WT, 1, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
