@@ -34,6 +34,8 @@ struct mm_args {
     uint64_t nb01, nb02, nb03, nb11, nb12, nb13, nb1, nb2, nb3;
     int ne12, r2, r3;
     int x_aligned; // src1 rows allow 16-byte vector loads
+    int w_aligned; // Q8_0 rows start on dword boundaries
+    int rows_wg;   // GEMV: weight rows per work-group (16, 8 or 4)
 };
 
 constexpr int WT_Q8 = 0, WT_F16 = 1, WT_F32 = 2;
@@ -59,6 +61,33 @@ __device__ __forceinline__ half8_t q8_to_half8(uint32_t lo, uint32_t hi) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) h[i] -= off;
     return h;
+}
+
+// The 8 quants lane-group j needs from Q8_0 block kb of a row: bytes 34*kb + 2 + 8j .. +8, which are
+// only 2-byte aligned.  Vector loads that are not dword-aligned are served lane by lane and run
+// several times slower, so when the row itself is dword-aligned (al4) the lane fetches the three
+// aligned dwords that cover its bytes (never outside the block) and shifts them into place;
+// whether a shift is needed depends only on the parity of kb.
+struct q8_raw { uint32_t w0, w1, w2; };
+__device__ __forceinline__ q8_raw q8_load(const char * wrow, int64_t kb, int j, bool al4) {
+    q8_raw r;
+    if (al4) {
+        const char * p = (const char *) __builtin_assume_aligned(wrow + kb * VX_Q8_BLOCK + 8 * j - ((kb & 1) ? 2 : 0), 4);
+        uint32_t v[3];
+        __builtin_memcpy(v, p, 12);
+        r.w0 = v[0]; r.w1 = v[1]; r.w2 = v[2];
+    } else {
+        uint32_t v[2];
+        __builtin_memcpy(v, wrow + kb * VX_Q8_BLOCK + 2 + 8 * j, 8);
+        r.w0 = 0; r.w1 = v[0]; r.w2 = v[1];
+    }
+    return r;
+}
+__device__ __forceinline__ half8_t q8_unpack(const q8_raw & r, int64_t kb, bool al4) {
+    const bool shifted = al4 && !(kb & 1); // even blocks start on a dword: the quants sit 2 bytes in
+    const uint32_t lo = shifted ? __builtin_amdgcn_alignbit(r.w1, r.w0, 16) : r.w1;
+    const uint32_t hi = shifted ? __builtin_amdgcn_alignbit(r.w2, r.w1, 16) : r.w2;
+    return q8_to_half8(lo, hi);
 }
 
 __device__ __forceinline__ int lds_slot(int kbl, int tt, int TT, int j, int c) {
@@ -144,9 +173,7 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
             if constexpr (WT == WT_Q8) {
                 const char * bp = wrow + (uint64_t) kb * VX_Q8_BLOCK;
                 dw = (float) *(const _Float16 *) bp;
-                uint32_t q2[2];
-                __builtin_memcpy(q2, bp + 2 + 8 * j, 8);
-                bop = q8_to_half8(q2[0], q2[1]);
+                bop = q8_unpack(q8_load(wrow, kb, j, false), kb, false);
             } else if constexpr (WT == WT_F16) {
                 const int64_t k = kb * 32 + 8 * j;
                 if (k + 8 <= a.K) {
@@ -216,7 +243,7 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
 // in one round trip to HBM.
 constexpr int GV_UNROLL = 8;
 
-template <int WT, bool ACT_Q8, int NW>
+template <int WT, bool ACT_Q8, int NW, bool AL4>
 __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
     const int64_t nkb = a.K / 32;
@@ -231,23 +258,30 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
-    const int64_t row0 = (int64_t) blockIdx.x * 16;
+    // R = a.rows_wg of the 16 MFMA columns carry weight rows; fewer rows per work-group put a short
+    // matrix on more CUs (a CU sustains only so many outstanding lines, so 64 work-groups cannot
+    // pull what 256 can).  Lanes c >= R load nothing; their columns are never stored.
+    const int     R = a.rows_wg;
+    const int64_t row0 = (int64_t) blockIdx.x * R;
+    const bool    row_ok = c < R && row0 + c < a.M;
     const char *  wrow = wb + (uint64_t) min(row0 + c, a.M - 1) * a.nb01;
     const int     N = (int) a.N;
 
     // ---- this wave's weight blocks: kb = wid + NW * i
-    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-    u32x2    wq[GV_UNROLL];
+    constexpr bool al4 = AL4;
+    q8_raw   wq[GV_UNROLL];
     half8_t  wh[GV_UNROLL];
     _Float16 wdv[GV_UNROLL];
     auto load_blocks = [&](int64_t i0) {
 #pragma unroll
         for (int u = 0; u < GV_UNROLL; ++u) {
             const int64_t kb = min((int64_t) wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, result unused
-            if constexpr (WT == WT_Q8) {
+            if (!row_ok) {
+                wq[u] = q8_raw{0, 0, 0}; wdv[u] = (_Float16) 0.0f; wh[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            } else if constexpr (WT == WT_Q8) {
                 const char * bp = wrow + (uint64_t) kb * VX_Q8_BLOCK;
                 wdv[u] = *(const _Float16 *) bp;
-                __builtin_memcpy(&wq[u], bp + 2 + 8 * j, 8);
+                wq[u]  = q8_load(wrow, kb, j, al4);
             } else {
                 __builtin_memcpy(&wh[u], wrow + (uint64_t) (kb * 32 + 8 * j) * 2, 16);
             }
@@ -311,7 +345,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             half8_t aop = {0, 0, 0, 0, 0, 0, 0, 0};
             if (c < N) aop = *(const half8_t *) (xs + (size_t) c * a.K + kb * 32 + 8 * j);
             if constexpr (WT == WT_Q8) {
-                const half8_t  bop = q8_to_half8(wq[u][0], wq[u][1]);
+                const half8_t  bop = q8_unpack(wq[u], kb, al4);
                 const float4_t blk = mfma16(aop, bop, float4_t{0, 0, 0, 0});
                 const float    dw  = (float) wdv[u];
                 if constexpr (ACT_Q8) {
@@ -334,7 +368,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         for (int ww = 0; ww < NW - 1; ++ww) acc += red[ww * 64 + lane];
     }
     // lane (j,c), register r: token 4j + r, row row0 + c
-    if (row0 + c < a.M) {
+    if (row_ok) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int tok = 4 * j + r;
@@ -356,19 +390,29 @@ int gemv_waves(const mm_args & a) {
 }
 
 template <int WT, bool ACT_Q8>
-bool launch_gemv(const mm_args & a, int nbatch, hipStream_t st) {
+bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
+    mm_args a = a0;
     if (a.N > 16 || a.K % 32 || a.K < 32) return false;
+    a.rows_wg = 16;
+    while (a.rows_wg > 4 && (a.M + a.rows_wg - 1) / a.rows_wg * nbatch < 128) a.rows_wg /= 2;
     const int nw = gemv_waves(a);
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
     if (smem > 64 * 1024) return false;
-    const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
+    const dim3 grid((unsigned) ((a.M + a.rows_wg - 1) / a.rows_wg), 1, (unsigned) nbatch);
+    const dim3 block((unsigned) (64 * nw));
+#define VX_GEMV(NW_)                                                                                       \
+    do {                                                                                                   \
+        if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true><<<grid, block, smem, st>>>(a);  \
+        else                            gemv_kernel<WT, ACT_Q8, NW_, false><<<grid, block, smem, st>>>(a); \
+    } while (0)
     switch (nw) {
-        case 1:  gemv_kernel<WT, ACT_Q8, 1><<<grid, dim3(64), smem, st>>>(a); break;
-        case 2:  gemv_kernel<WT, ACT_Q8, 2><<<grid, dim3(128), smem, st>>>(a); break;
-        case 4:  gemv_kernel<WT, ACT_Q8, 4><<<grid, dim3(256), smem, st>>>(a); break;
-        case 8:  gemv_kernel<WT, ACT_Q8, 8><<<grid, dim3(512), smem, st>>>(a); break;
-        default: gemv_kernel<WT, ACT_Q8, 16><<<grid, dim3(1024), smem, st>>>(a); break;
+        case 1:  VX_GEMV(1); break;
+        case 2:  VX_GEMV(2); break;
+        case 4:  VX_GEMV(4); break;
+        case 8:  VX_GEMV(8); break;
+        default: VX_GEMV(16); break;
     }
+#undef VX_GEMV
     return true;
 }
 
@@ -429,6 +473,8 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
     a.nb1 = dst->nb[1]; a.nb2 = dst->nb[2]; a.nb3 = dst->nb[3];
     a.ne12 = (int) src1->ne[2];
     a.r2 = (int) (src1->ne[2] / src0->ne[2]); a.r3 = (int) (src1->ne[3] / src0->ne[3]);
+    a.rows_wg   = 16;
+    a.w_aligned = ((uintptr_t) src0->data % 4 == 0) && src0->nb[1] % 4 == 0 && src0->nb[2] % 4 == 0 && src0->nb[3] % 4 == 0;
     a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
