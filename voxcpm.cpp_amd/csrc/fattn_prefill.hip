@@ -62,6 +62,18 @@ __device__ __forceinline__ void pk2(half8_t & dst, int i, float a, float b) {
     dst[i + 1] = (_Float16) v[1];
 }
 
+// "does any of these 8 scores exceed a positive bound" on the bit patterns: as signed integers,
+// floats above a positive bound (and NaNs) compare above its pattern, everything negative below.
+// Integer max needs none of the canonicalising self-max instructions fmaxf() gets in front of
+// operands that come out of the matrix core.
+__device__ __forceinline__ int imax8(const float4_t & x, const float4_t & y) {
+    const int4_t a = __builtin_bit_cast(int4_t, x), b = __builtin_bit_cast(int4_t, y);
+    return max(max(max(a[0], a[1]), max(a[2], a[3])), max(max(b[0], b[1]), max(b[2], b[3])));
+}
+__device__ __forceinline__ float fmax8(const float4_t & x, const float4_t & y) {
+    return fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(y[0], y[1]), fmaxf(y[2], y[3])));
+}
+
 // classifies mask tiles: one wave per (key tile, row block, mask batch)
 __global__ __launch_bounds__(64) void pf_mask_flags_kernel(const char * mask, uint64_t nbm1, uint64_t nbm2, uint64_t nbm3,
                                                            int nem2, int n_q, int n_kv, int RB, int n_rb, int n_tiles,
@@ -202,7 +214,26 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
         const char * kg = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3;
         const char * vg = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3;
         half8_t kreg[2], vreg[2];
+        // a thread's byte offsets inside a full tile never change: the tile's base is scalar arithmetic
+        // and the loads take (scalar base, 32-bit lane offset); only a ragged last tile clamps per lane
+        uint32_t koff[2], voff[2];
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            koff[hh] = (uint32_t) ((hh * 32 + ld_key) * a.nbk1 + ld_chunk * 16);
+            voff[hh] = (uint32_t) ((hh * 32 + ld_key) * a.nbv1 + ld_chunk * 16);
+        }
+        const bool off32_ok = !KV_F32 && (uint64_t) PF_KT * a.nbk1 < (1ull << 31) && (uint64_t) PF_KT * a.nbv1 < (1ull << 31);
         auto load_global = [&](int tile) {
+            if (off32_ok && (tile + 1) * PF_KT <= a.n_kv) { // wave-uniform
+                const char * kt = kg + (uint64_t) tile * PF_KT * a.nbk1;
+                const char * vt = vg + (uint64_t) tile * PF_KT * a.nbv1;
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    kreg[hh] = *(const half8_t *) (kt + koff[hh]);
+                    vreg[hh] = *(const half8_t *) (vt + voff[hh]);
+                }
+                return;
+            }
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 const int key = min(tile * PF_KT + hh * 32 + ld_key, a.n_kv - 1);
@@ -228,9 +259,12 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                 *(half8_t *) &k_lds[buf][kl][ld_chunk * 8] = kreg[hh];
                 // V^T, keys stored in P^T operand order: key 32hh + 16h + 4jj + r -> 32hh + 8jj + 4h + r
                 const int k32 = ld_key, h = k32 >> 4, jj = (k32 >> 2) & 3, r = k32 & 3;
-                const int pos = hh * 32 + 8 * jj + 4 * h + r;
+                const int grp8 = hh * 4 + jj, sub = 4 * h + r;
+                // d = 8 * ld_chunk + i sits in physical row 8 * i + ld_chunk, key group xor-ed with i: the 8
+                // chunks a wave writes at once land in 8 consecutive rows (distinct banks), and the 16 rows
+                // an operand read touches spread over all banks as well
 #pragma unroll
-                for (int i = 0; i < 8; ++i) vt_lds[buf][ld_chunk * 8 + i][pos] = vreg[hh][i];
+                for (int i = 0; i < 8; ++i) vt_lds[buf][8 * i + ld_chunk][((grp8 ^ i) << 3) + sub] = vreg[hh][i];
             }
         };
 
@@ -240,9 +274,9 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 
         for (int it = 0; it < n_active; ++it) {
             const int buf = it & 1;
-            const int tile = tile_list[it];
+            const int tile = __builtin_amdgcn_readfirstlane(tile_list[it]);
             const bool mixed = tile_flag[it] == 2;
-            load_global(tile_list[min(it + 1, n_active - 1)]); // unconditional: keeps the wait counts exact
+            load_global(__builtin_amdgcn_readfirstlane(tile_list[min(it + 1, n_active - 1)])); // unconditional: keeps the wait counts exact
 
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
@@ -254,14 +288,13 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                     for (int p = 0; p < NP; ++p) ak[h][p] = *(const half8_t *) &k_lds[buf][hh * 32 + h * 16 + c][SEG * j + 8 * p];
                 half8_t av[4];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) av[t] = *(const half8_t *) &vt_lds[buf][16 * t + c][hh * 32 + 8 * j];
+                for (int t = 0; t < 4; ++t) av[t] = *(const half8_t *) &vt_lds[buf][(c & 7) * 8 + 2 * t + (c >> 3)][((hh * 4 + j) ^ (c & 7)) << 3];
 
 #pragma unroll
                 for (int cg = 0; cg < PF_CT; cg += PF_GRP) {
                     // scores of PF_GRP column tiles, then ONE wave-uniform decision for the group, so
                     // the common path is straight-line code the scheduler can interleave
                     float4_t s[PF_GRP][2];
-                    float    cmax[PF_GRP];
 #pragma unroll
                     for (int u = 0; u < PF_GRP; ++u) {
 #pragma unroll
@@ -272,18 +305,13 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                             s[u][h] = acc; // = score * log2(e) - m_ref
                         }
                     }
-                    float gmax = -INFINITY;
+                    int gmax = 0;
 #pragma unroll
-                    for (int u = 0; u < PF_GRP; ++u) {
-                        cmax[u] = fmaxf(fmaxf(fmaxf(s[u][0][0], s[u][0][1]), fmaxf(s[u][0][2], s[u][0][3])),
-                                        fmaxf(fmaxf(s[u][1][0], s[u][1][1]), fmaxf(s[u][1][2], s[u][1][3])));
-                        gmax = fmaxf(gmax, cmax[u]);
-                    }
-                    if (mixed || !all_seen || __builtin_amdgcn_ballot_w64(gmax > PF_LAZY) != 0) {
+                    for (int u = 0; u < PF_GRP; ++u) gmax = max(gmax, imax8(s[u][0], s[u][1]));
+                    if (mixed || !all_seen || __builtin_amdgcn_ballot_w64(gmax > __builtin_bit_cast(int, PF_LAZY)) != 0) {
 #pragma unroll
                         for (int u = 0; u < PF_GRP; ++u) {
                             const int ct = cg + u;
-                            float cm = cmax[u];
                             if (mixed) { // element-wise mask / bounds (diagonal and tail tiles only)
                                 const int col  = wave * 64 + ct * 16 + c;
                                 const bool ok  = col < ncols_blk;
@@ -300,9 +328,8 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                                         if (mrow) x = slope * __half2float(mrow[min(key, a.n_kv - 1)]);
                                         s[u][h][r] += key < a.n_kv ? x : -INFINITY;
                                     }
-                                cm = fmaxf(fmaxf(fmaxf(s[u][0][0], s[u][0][1]), fmaxf(s[u][0][2], s[u][0][3])),
-                                           fmaxf(fmaxf(s[u][1][0], s[u][1][1]), fmaxf(s[u][1][2], s[u][1][3])));
                             }
+                            float cm = fmax8(s[u][0], s[u][1]);
                             cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
                             cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
                             // move the reference: up to the new maximum, or (first visible key of the
