@@ -216,21 +216,18 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
         half8_t kreg[2], vreg[2];
         // a thread's byte offsets inside a full tile never change: the tile's base is scalar arithmetic
         // and the loads take (scalar base, 32-bit lane offset); only a ragged last tile clamps per lane
-        uint32_t koff[2], voff[2];
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-            koff[hh] = (uint32_t) ((hh * 32 + ld_key) * a.nbk1 + ld_chunk * 16);
-            voff[hh] = (uint32_t) ((hh * 32 + ld_key) * a.nbv1 + ld_chunk * 16);
-        }
-        const bool off32_ok = !KV_F32 && (uint64_t) PF_KT * a.nbk1 < (1ull << 31) && (uint64_t) PF_KT * a.nbv1 < (1ull << 31);
+        // (K and V share the offsets when their row strides agree, which every cache layout does)
+        const uint32_t koff = (uint32_t) (ld_key * a.nbk1 + ld_chunk * 16);
+        const bool off32_ok = !KV_F32 && a.nbk1 == a.nbv1 && (uint64_t) PF_KT * a.nbk1 < (1ull << 31);
+        const uint32_t half_off = (uint32_t) (32 * a.nbk1); // scalar
         auto load_global = [&](int tile) {
             if (off32_ok && (tile + 1) * PF_KT <= a.n_kv) { // wave-uniform
                 const char * kt = kg + (uint64_t) tile * PF_KT * a.nbk1;
                 const char * vt = vg + (uint64_t) tile * PF_KT * a.nbv1;
 #pragma unroll
                 for (int hh = 0; hh < 2; ++hh) {
-                    kreg[hh] = *(const half8_t *) (kt + koff[hh]);
-                    vreg[hh] = *(const half8_t *) (vt + voff[hh]);
+                    kreg[hh] = *(const half8_t *) (kt + hh * half_off + koff);
+                    vreg[hh] = *(const half8_t *) (vt + hh * half_off + koff);
                 }
                 return;
             }
