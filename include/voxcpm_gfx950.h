@@ -174,6 +174,20 @@ VX_API vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, const
 /* GGML_OP_SUM: every element summed in double, rounded once (ops.cpp:1275-1300) */
 VX_API vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
 
+/* ---- adjacent node pairs as one launch ----------------------------------------------------------
+ * What a backend's graph_compute may substitute for two consecutive nodes whose intermediate has no
+ * other reader; every rounding happens where the two separate nodes would round, so results are
+ * bit-identical to running them one after the other.  No counterpart in ggml-cpu (it runs the nodes
+ * separately: ops.cpp:3710-3777 + binary-ops.cpp:50-112, ops.cpp:4374-4424). */
+/* RMS_NORM(src) -> MUL(., weight): weight one F32 row of src's ne[0] (MiniCPMModel::rms_norm, src/minicpm.cpp:572-580) */
+VX_API vx_status vx_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst, float eps, vx_stream stream);
+/* SCALE(x, scale) -> ADD(a, .): dst = a + x * scale (the muP residual, src/minicpm.cpp:765-775) */
+VX_API vx_status vx_scale_add(const vx_tensor * a, const vx_tensor * x, const vx_tensor * dst, float scale, vx_stream stream);
+/* ADD(a, b) -> SCALE(., scale, bias): dst = (a + b) * scale + bias (the kv_sync tail, src/minicpm.cpp:685-689) */
+VX_API vx_status vx_add_scale(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst, float scale, float bias, vx_stream stream);
+VX_API int vx_supports_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst);
+VX_API int vx_supports_fused_pair(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst);
+
 VX_API int vx_supports_binary(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_add1(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_unary_like(const vx_tensor * src, const vx_tensor * dst); /* SCALE */

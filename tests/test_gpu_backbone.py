@@ -53,8 +53,10 @@ def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
     # the C-ABI mirror, Q8 activations (ggml-cpu's arithmetic) and float activations.  Even with
     # ggml-cpu's integer dots an activation one ulp away can round to the neighbouring int8, so the
     # stack agrees to ~1e-5 NMSE, not bit for bit; float activations sit at ggml's own 5e-4 / op bar.
-    for act, bar in ((gpu.ACT_Q8, 5e-5), (gpu.ACT_FLOAT, 1e-4)):
-        m = bb.MiniCPMBackbone(n_layer=N_LAYER, max_length=MAX_LEN, batch=BATCH, use_mup=use_mup, kv_f16=kv_f16, act_mode=act)
+    unfused = {}
+    for act, bar, fuse in ((gpu.ACT_Q8, 5e-5, True), (gpu.ACT_FLOAT, 1e-4, False), (gpu.ACT_FLOAT, 1e-4, True)):
+        m = bb.MiniCPMBackbone(n_layer=N_LAYER, max_length=MAX_LEN, batch=BATCH, use_mup=use_mup, kv_f16=kv_f16, act_mode=act,
+                               fuse_pairs=fuse)
         for li, lw in enumerate(params["layers"]):
             for n in reflib.BB_WEIGHTS:
                 m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
@@ -69,6 +71,10 @@ def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
             got = m.forward(torch.from_numpy(x).cuda(), n_past, mask)
             torch.cuda.synchronize()
             e = nmse(cpu[i], got.cpu().numpy())
-            print(f"   C ABI mirror (act_mode {act}) vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+            print(f"   C ABI mirror (act_mode {act}, fused pairs {fuse}) vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
             assert e <= bar
+            if act == gpu.ACT_FLOAT and not fuse:
+                unfused[i] = got.cpu().numpy()
+            elif act == gpu.ACT_FLOAT:   # the one-launch pairs round where the separate nodes do
+                assert np.array_equal(unfused[i], got.cpu().numpy()), f"fused pairs changed the result of call {i}"
             n_past += T

@@ -13,6 +13,10 @@ ggml's ne[3]; with batch 1 the call sequence is the reference's graph node for n
 
 A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and intermediates
 are built once, so a plan can be replayed from a captured HIP graph.
+
+With `fuse_pairs=True` the four adjacent-node pairs the ggml backend plugin runs as one launch
+(rms_norm+mul, scale+add, cont+sum, add+scale) are issued as the plugin issues them; the results
+are bit-identical to the unfused sequence.
 """
 import math
 
@@ -24,7 +28,7 @@ WEIGHT_NAMES = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", 
 class MiniCPMBackbone:
     def __init__(self, n_layer=24, hidden=1024, n_heads=16, n_kv_heads=2, head_dim=64, ffn=4096, max_length=1024,
                  batch=1, eps=1e-5, use_mup=False, scale_depth=1.4, kv_f16=False, act_mode=ACT_FLOAT,
-                 rope_base=10000.0, rope_original_max=32768):
+                 rope_base=10000.0, rope_original_max=32768, fuse_pairs=True):
         import torch
         self.torch = torch
         self.n_layer, self.hidden, self.n_heads, self.n_kv, self.D = n_layer, hidden, n_heads, n_kv_heads, head_dim
@@ -32,6 +36,7 @@ class MiniCPMBackbone:
         self.use_mup = use_mup
         self.residual_scale = scale_depth / math.sqrt(max(1, n_layer)) if use_mup else 1.0
         self.act_mode = act_mode
+        self.fuse_pairs = fuse_pairs
         self.rope_base, self.rope_original_max = rope_base, rope_original_max
         self.kv_dtype = torch.float16 if kv_f16 else torch.float32
         dev = "cuda"
@@ -85,6 +90,23 @@ class MiniCPMBackbone:
         def call(fn, *args):
             calls.append((fn, args))
 
+        fuse = self.fuse_pairs
+
+        def norm(xin, w, dst):          # MiniCPMModel::rms_norm
+            if fuse:
+                call(L.vx_rms_norm_mul, desc(xin), desc(w), desc(dst), self.eps)
+            else:
+                call(L.vx_rms_norm, desc(xin), desc(dst), self.eps)
+                call(L.vx_binary, BIN_MUL, desc(dst), desc(w), desc(dst))
+
+        def residual(res, branch, dst):  # optional muP scale, then the residual add
+            if self.use_mup and fuse:
+                call(L.vx_scale_add, desc(res), desc(branch), desc(dst), self.residual_scale)
+                return
+            if self.use_mup:
+                call(L.vx_scale, desc(branch), desc(branch), self.residual_scale, 0.0)
+            call(L.vx_binary, BIN_ADD, desc(res), desc(branch), desc(dst))
+
         # buffers reused by every layer (the stack is sequential)
         normed, q, k, v = new(N, self.hidden), new(N, H * D), new(N, Hkv * D), new(N, Hkv * D)
         kcont, vcont = new(B, T, Hkv, D, dtype=self.kv_dtype), new(B, T, Hkv, D, dtype=self.kv_dtype)
@@ -112,8 +134,7 @@ class MiniCPMBackbone:
             kc, vc = self.k_cache[li], self.v_cache[li]
             wd = {n: desc_q8(*w[n]) for n in WEIGHT_NAMES}
             # -- attention_forward
-            call(L.vx_rms_norm, desc(cur_x), desc(normed), self.eps)
-            call(L.vx_binary, BIN_MUL, desc(normed), desc(nrm["input_layernorm"]), desc(normed))
+            norm(cur_x, nrm["input_layernorm"], normed)
             call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
             call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
             call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
@@ -127,7 +148,11 @@ class MiniCPMBackbone:
                 call(L.vx_cpy, desc(k4), desc(kw))
                 call(L.vx_cpy, desc(v4), desc(vw))
                 keep += [kw, vw]
-            if chain:
+            if chain and fuse:
+                call(L.vx_sum, desc(kw), desc(sk))       # cont + sum
+                call(L.vx_sum, desc(vw), desc(sv))
+                call(L.vx_add_scale, desc(sk), desc(sv), desc(sync), 0.0, 0.0)
+            elif chain:
                 call(L.vx_cpy, desc(kw), desc(kcont))
                 call(L.vx_sum, desc(kcont), desc(sk))
                 call(L.vx_cpy, desc(vw), desc(vcont))
@@ -148,24 +173,18 @@ class MiniCPMBackbone:
             if chain:
                 call(L.vx_add1, desc(attn), desc(sync), desc(attn))
             call(L.vx_mul_mat, wd["o_proj"], desc(attn.view(N, H * D)), desc(attn_o), self.act_mode)
-            if self.use_mup:
-                call(L.vx_scale, desc(attn_o), desc(attn_o), self.residual_scale, 0.0)
-            call(L.vx_binary, BIN_ADD, desc(cur_x), desc(attn_o), desc(h_mid))
+            residual(cur_x, attn_o, h_mid)
             # -- mlp_forward
-            call(L.vx_rms_norm, desc(h_mid), desc(normed), self.eps)
-            call(L.vx_binary, BIN_MUL, desc(normed), desc(nrm["post_layernorm"]), desc(normed))
+            norm(h_mid, nrm["post_layernorm"], normed)
             call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
             call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
             call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)
             call(L.vx_mul_mat, wd["down_proj"], desc(act), desc(down), self.act_mode)
-            if self.use_mup:
-                call(L.vx_scale, desc(down), desc(down), self.residual_scale, 0.0)
             nxt = hs[li % 2]
-            call(L.vx_binary, BIN_ADD, desc(h_mid), desc(down), desc(nxt))
+            residual(h_mid, down, nxt)
             cur_x = nxt
         o2 = out.view(N, self.hidden)
-        call(L.vx_rms_norm, desc(cur_x), desc(o2), self.eps)
-        call(L.vx_binary, BIN_MUL, desc(o2), desc(self.final_norm), desc(o2))
+        norm(cur_x, self.final_norm, o2)
 
         def run():
             st = _stream()

@@ -20,6 +20,8 @@ enum ew_op : int {
     EW_SCALE,                         // dst = src0 * p0 (+ p1)
     EW_UNARY,                         // dst = f(src0), f = aux
     EW_GLU,                           // dst = act(a) * b, act = aux
+    EW_SCALE_ADD,                     // dst = src0 + src1 * p0   (SCALE feeding ADD)
+    EW_ADD_SCALE,                     // dst = (src0 + src1) * p0 (+ p1)   (ADD feeding SCALE)
 };
 
 struct ew_args {
@@ -49,6 +51,14 @@ __device__ __forceinline__ float unary_f(int op, float x) {
     }
 }
 
+// a + x * s with the product rounded first, as a SCALE node followed by an ADD node rounds it
+// (the compiler would otherwise contract the pair into one fused multiply-add)
+__device__ __forceinline__ float mul_then_add(float x, float s, float a) {
+#pragma clang fp contract(off)
+    const float t = x * s;
+    return a + t;
+}
+
 template <int OP>
 __device__ __forceinline__ float ew_apply(const ew_args & a, float x, float y) {
     if constexpr (OP == EW_ADD)   return x + y;
@@ -59,10 +69,15 @@ __device__ __forceinline__ float ew_apply(const ew_args & a, float x, float y) {
     if constexpr (OP == EW_SCALE) return a.p1 == 0.0f ? x * a.p0 : fmaf(x, a.p0, a.p1); // vec_scale / vec_mad1
     if constexpr (OP == EW_UNARY) return unary_f(a.aux, x);
     if constexpr (OP == EW_GLU)   return (a.aux == VX_GLU_REGLU ? (x > 0.0f ? x : 0.0f) : silu_f(x)) * y;
+    // the fused pairs round exactly where the two separate nodes would (no contraction)
+    if constexpr (OP == EW_SCALE_ADD) return mul_then_add(y, a.p0, x);
+    if constexpr (OP == EW_ADD_SCALE) { const float t = x + y; return a.p1 == 0.0f ? t * a.p0 : fmaf(t, a.p0, a.p1); }
     return x;
 }
 
-template <int OP> constexpr bool ew_has_src1() { return OP == EW_ADD || OP == EW_SUB || OP == EW_MUL || OP == EW_DIV || OP == EW_GLU; }
+template <int OP> constexpr bool ew_has_src1() {
+    return OP == EW_ADD || OP == EW_SUB || OP == EW_MUL || OP == EW_DIV || OP == EW_GLU || OP == EW_SCALE_ADD || OP == EW_ADD_SCALE;
+}
 
 template <int OP, int VEC>
 __global__ __launch_bounds__(256) void ew_kernel(const ew_args a) {
@@ -287,6 +302,30 @@ extern "C" vx_status vx_scale(const vx_tensor * src, const vx_tensor * dst, floa
     ew_args a; ew_fill(a, src, nullptr, dst);
     a.p0 = scale; a.p1 = bias;
     return ew_launch<EW_SCALE>(a, (hipStream_t) stream);
+}
+
+// SCALE(x) feeding ADD(a, .) and ADD(a, b) feeding SCALE, as one launch each; a, b/x, dst of one shape
+extern "C" int vx_supports_fused_pair(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst) {
+    if (!f32(a) || !f32(b) || !f32(dst)) return 0;
+    if (!vx_positive(a) || !vx_same_shape(a, dst) || !vx_same_shape(a, b)) return 0;
+    return nb_multiple(a, 4) && nb_multiple(b, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_scale_add(const vx_tensor * a, const vx_tensor * x, const vx_tensor * dst, float scale, vx_stream stream) {
+    if (!vx_supports_fused_pair(a, x, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "scale_add: F32 tensors of one shape");
+    if (!a->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "scale_add: null data");
+    ew_args e; ew_fill(e, a, x, dst);
+    e.p0 = scale;
+    return ew_launch<EW_SCALE_ADD>(e, (hipStream_t) stream);
+}
+
+extern "C" vx_status vx_add_scale(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst, float scale, float bias,
+                                  vx_stream stream) {
+    if (!vx_supports_fused_pair(a, b, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "add_scale: F32 tensors of one shape");
+    if (!a->data || !b->data || !dst->data) return vx_fail(VX_ERR_INVALID, "add_scale: null data");
+    ew_args e; ew_fill(e, a, b, dst);
+    e.p0 = scale; e.p1 = bias;
+    return ew_launch<EW_ADD_SCALE>(e, (hipStream_t) stream);
 }
 
 extern "C" int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * dst) {

@@ -15,7 +15,8 @@ constexpr int RN_MAX_VEC = 8; // float4 chunks cached per thread before falling 
 
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict__ src, char * __restrict__ dst,
-                                                         vx_dims s, vx_dims d, float eps, int rows_per_block) {
+                                                         vx_dims s, vx_dims d, float eps, int rows_per_block,
+                                                         const float * __restrict__ w) {
     constexpr int WAVES = BLOCK / VX_WAVE;
     __shared__ double red[WAVES];
 
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict
     const float * x  = (const float *) (src + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3]);
     float *       y  = (float *) (dst + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]);
 
-    const bool vec_ok = (ne00 % 4 == 0) && (((uintptr_t) x | (uintptr_t) y) % 16 == 0);
+    const bool vec_ok = (ne00 % 4 == 0) && (((uintptr_t) x | (uintptr_t) y | (uintptr_t) w) % 16 == 0);
     const int64_t nvec = vec_ok ? ne00 / 4 : 0;
 
     float4 cache[RN_MAX_VEC];
@@ -85,16 +86,22 @@ __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict
             if (iv < nvec) {
                 float4 v = cache[c];
                 v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+                if (w) { const float4 g = ((const float4 *) w)[iv]; v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w; }
                 ((float4 *) y)[iv] = v;
             }
         }
         for (int64_t iv = lane_id + (int64_t) RN_MAX_VEC * nlanes; iv < nvec; iv += nlanes) {
             float4 v = ((const float4 *) x)[iv];
             v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+            if (w) { const float4 g = ((const float4 *) w)[iv]; v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w; }
             ((float4 *) y)[iv] = v;
         }
     } else {
-        for (int64_t i = lane_id; i < ne00; i += nlanes) y[i] = x[i] * scale;
+        for (int64_t i = lane_id; i < ne00; i += nlanes) {
+            float v = x[i] * scale; // rounded here, as the separate RMS_NORM node would store it
+            if (w) v *= w[i];
+            y[i] = v;
+        }
     }
 }
 
@@ -109,21 +116,39 @@ extern "C" int vx_supports_rms_norm(const vx_tensor * src, const vx_tensor * dst
     return 1;
 }
 
-extern "C" vx_status vx_rms_norm(const vx_tensor * src, const vx_tensor * dst, float eps, vx_stream stream) {
-    if (!src || !dst || !src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "rms_norm: null tensor");
-    if (!vx_supports_rms_norm(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "rms_norm: needs F32 tensors of equal shape with dense rows");
-    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "rms_norm: eps must be >= 0");
+static vx_status rms_norm_launch(const vx_tensor * src, const vx_tensor * dst, float eps, const float * w, vx_stream stream) {
     const int64_t nrows = vx_nrows(src);
     const vx_dims s = vx_dims_of(src), d = vx_dims_of(dst);
     hipStream_t   st = (hipStream_t) stream;
     if (src->ne[0] <= 1024) {
         const int rpb = 4; // one wave per row
         rms_norm_kernel<256><<<dim3((unsigned) ((nrows + rpb - 1) / rpb)), dim3(256), 0, st>>>(
-            (const char *) src->data, (char *) dst->data, s, d, eps, rpb);
+            (const char *) src->data, (char *) dst->data, s, d, eps, rpb, w);
     } else {
         rms_norm_kernel<256><<<dim3((unsigned) nrows), dim3(256), 0, st>>>(
-            (const char *) src->data, (char *) dst->data, s, d, eps, 1);
+            (const char *) src->data, (char *) dst->data, s, d, eps, 1, w);
     }
     VX_LAUNCH_CHECK();
     return VX_OK;
+}
+
+extern "C" vx_status vx_rms_norm(const vx_tensor * src, const vx_tensor * dst, float eps, vx_stream stream) {
+    if (!src || !dst || !src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "rms_norm: null tensor");
+    if (!vx_supports_rms_norm(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "rms_norm: needs F32 tensors of equal shape with dense rows");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "rms_norm: eps must be >= 0");
+    return rms_norm_launch(src, dst, eps, nullptr, stream);
+}
+
+extern "C" int vx_supports_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst) {
+    if (!vx_supports_rms_norm(src, dst) || !weight || weight->type != VX_TYPE_F32) return 0;
+    return weight->ne[0] == src->ne[0] && weight->ne[1] == 1 && weight->ne[2] == 1 && weight->ne[3] == 1 && weight->nb[0] == 4;
+}
+
+extern "C" vx_status vx_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst, float eps,
+                                     vx_stream stream) {
+    if (!src || !dst || !weight || !src->data || !dst->data || !weight->data) return vx_fail(VX_ERR_INVALID, "rms_norm_mul: null tensor");
+    if (!vx_supports_rms_norm_mul(src, weight, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "rms_norm_mul: needs F32 tensors of equal shape with dense rows and one weight row");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "rms_norm_mul: eps must be >= 0");
+    return rms_norm_launch(src, dst, eps, (const float *) weight->data, stream);
 }

@@ -29,6 +29,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 namespace {
@@ -411,18 +412,81 @@ void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor
         GGML_ABORT("ggml-gfx950: get_tensor_async failed: %s", vx_last_error());
 }
 
+// Two consecutive nodes as one launch, when the first one's value has no other reader (checked by
+// the caller).  Returns false when the pair is not one of the known shapes; *rc is the launch status.
+bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_status * rc) {
+    const vx_tensor d = to_vx(next);
+    if (node->op == GGML_OP_RMS_NORM && next->op == GGML_OP_MUL && next->src[0] == node) {
+        // MiniCPMModel::rms_norm: ggml_mul(ggml_rms_norm(x), weight)
+        const vx_tensor s = to_vx(node->src[0]), w = to_vx(next->src[1]);
+        if (!vx_supports_rms_norm_mul(&s, &w, &d)) return false;
+        float eps;
+        memcpy(&eps, node->op_params, sizeof(float));
+        *rc = vx_rms_norm_mul(&s, &w, &d, eps, ctx->stream);
+        return true;
+    }
+    if (node->op == GGML_OP_SCALE && next->op == GGML_OP_ADD && next->src[1] == node && next->src[0] != node) {
+        float sc, bias;
+        memcpy(&sc, (const float *) node->op_params + 0, sizeof(float));
+        memcpy(&bias, (const float *) node->op_params + 1, sizeof(float));
+        const vx_tensor a = to_vx(next->src[0]), x = to_vx(node->src[0]);
+        if (bias != 0.0f || !vx_supports_fused_pair(&a, &x, &d)) return false;
+        *rc = vx_scale_add(&a, &x, &d, sc, ctx->stream);
+        return true;
+    }
+    if (node->op == GGML_OP_ADD && next->op == GGML_OP_SCALE && next->src[0] == node) {
+        float sc, bias;
+        memcpy(&sc, (const float *) next->op_params + 0, sizeof(float));
+        memcpy(&bias, (const float *) next->op_params + 1, sizeof(float));
+        const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]);
+        if (!vx_supports_fused_pair(&a, &b, &d)) return false;
+        *rc = vx_add_scale(&a, &b, &d, sc, bias, ctx->stream);
+        return true;
+    }
+    if (node->op == GGML_OP_CONT && next->op == GGML_OP_SUM && next->src[0] == node) {
+        // the sum does not care where the elements lie: read them where they are
+        const vx_tensor s = to_vx(node->src[0]);
+        if (node->src[0]->type != GGML_TYPE_F32 || !vx_supports_sum(&s, &d)) return false;
+        *rc = vx_sum(&s, &d, ctx->stream);
+        return true;
+    }
+    return false;
+}
+
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     if (vx_init(ctx->device) != VX_OK) {
         GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
         return GGML_STATUS_FAILED;
     }
+    // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
+    // nodes is only run as one launch when nothing else looks at the value between them
+    static const bool fusion = getenv("GGML_GFX950_NO_FUSION") == nullptr;
+    std::unordered_map<const ggml_tensor *, int> readers;
+    if (fusion && cgraph->n_nodes > 1) {
+        readers.reserve((size_t) cgraph->n_nodes * 2);
+        for (int i = 0; i < cgraph->n_nodes; ++i) {
+            const ggml_tensor * n = cgraph->nodes[i];
+            for (int k = 0; k < GGML_MAX_SRC; ++k)
+                if (n->src[k]) readers[n->src[k]]++;
+            if (n->view_src) readers[n->view_src]++;
+        }
+    }
     for (int i = 0; i < cgraph->n_nodes; ++i) {
         ggml_tensor * node = cgraph->nodes[i];
         // the same two skips ggml-cpu applies (ggml/src/ggml-cpu/ggml-cpu.c:2956-2966)
         if (ggml_op_is_empty(node->op) || ggml_is_empty(node)) continue;
         if ((node->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
-        const vx_status rc = compute_node(ctx, node);
+        vx_status rc = VX_ERR_UNSUPPORTED;
+        bool fused = false;
+        if (fusion && i + 1 < cgraph->n_nodes) {
+            ggml_tensor * next = cgraph->nodes[i + 1];
+            const bool private_value = (node->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (next->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 &&
+                                       readers[node] == 1;
+            if (private_value) fused = compute_pair(ctx, node, next, &rc);
+        }
+        if (fused) ++i;
+        else rc = compute_node(ctx, node);
         if (rc != VX_OK) {
             GGML_LOG_ERROR("ggml-gfx950: node %d (%s, op %s) failed with status %d: %s\n", i, node->name,
                            ggml_op_name(node->op), (int) rc, rc == VX_ERR_UNSUPPORTED && !*vx_last_error() ? "operator not claimed by this backend" : vx_last_error());
