@@ -280,6 +280,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
+    ap.add_argument("--profile", choices=["prefill", "backbone"], default=None,
+                    help="run only this secondary workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no cross-GPU step); run with --gpus 1")
@@ -299,6 +301,16 @@ def main():
     pkg = entry.load_package()
     pkg.check(pkg.lib().vx_init(0), "vx_init")
     timer = Timer()
+
+    if args.profile == "prefill":   # config 5 prefill attention, 16 streams x 4096 tokens
+        call, flops, keep = prefill_attn_setup(pkg, 16, 4096)
+        s = timer.run(call, iters=5, warmup=2)
+        print(json.dumps({"profile": "cfg5_prefill_attn_T4096_B16", "us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
+                          "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}))
+        return
+    if args.profile == "backbone":  # config 4 decode steps, eager launches so that every kernel is traced
+        print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16)}))
+        return
 
     # ---- headline: config 2, L = args.length -------------------------------------------
     B, L = 2, args.length
@@ -344,7 +356,8 @@ def main():
         others["cfg5_decode_attn_B16_L8192"] = {"us_per_layer": s * 1e6, "GB/s": kv_bytes(16, 8192) / s / 1e9,
                                                 "hbm_frac": kv_bytes(16, 8192) / s / 1e9 / HBM_PEAK_GBS}
         del keep
-        for name, b, T, it in (("cfg1_prefill_attn_T256", 1, 256, 200), ("cfg5_prefill_attn_T4096_B1", 1, 4096, 5)):
+        for name, b, T, it in (("cfg1_prefill_attn_T256", 1, 256, 200), ("cfg5_prefill_attn_T4096_B1", 1, 4096, 5),
+                                  ("cfg5_prefill_attn_T4096_B16", 16, 4096, 3)):
             call, flops, keep = prefill_attn_setup(pkg, b, T)
             s = timer.run(call, iters=it, warmup=2)
             others[name] = {"us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,

@@ -231,17 +231,26 @@ __global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
 }
 
 // ---- SUM ---------------------------------------------------------------------------------------
-// ggml sums every element in double and rounds once (ops.cpp:1275-1300): one block, fp64 lanes.
+// ggml sums every element in double and rounds once (ops.cpp:1275-1300): one block, fp64 lanes, a
+// fixed reduction order.  Rows are dense (checked by the caller); 16-byte loads when VEC.
+template <bool VEC>
 __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst) {
     __shared__ double part[16];
-    const int64_t n = s.ne[0] * s.ne[1] * s.ne[2] * s.ne[3];
+    constexpr int W = VEC ? 4 : 1;
+    const uint32_t per_row = (uint32_t) (s.ne[0] / W);
+    const uint32_t n = per_row * (uint32_t) (s.ne[1] * s.ne[2] * s.ne[3]); // < 2^24, checked by the caller
+    const uint32_t ne1 = (uint32_t) s.ne[1], ne2 = (uint32_t) s.ne[2];
     double acc = 0.0;
-    for (int64_t e = threadIdx.x; e < n; e += 1024) {
-        int64_t r = e;
-        const int64_t i0 = r % s.ne[0]; r /= s.ne[0];
-        const int64_t i1 = r % s.ne[1]; r /= s.ne[1];
-        const int64_t i2 = r % s.ne[2]; const int64_t i3 = r / s.ne[2];
-        acc += (double) *(const float *) (src + i0 * s.nb[0] + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3]);
+    for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+        const uint32_t row = e / per_row, iv = e - row * per_row;
+        const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
+        const char * p = src + (uint64_t) iv * (4 * W) + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3];
+        if constexpr (VEC) {
+            const float4_t v = *(const float4_t *) p;
+            acc += (double) v[0]; acc += (double) v[1]; acc += (double) v[2]; acc += (double) v[3];
+        } else {
+            acc += (double) *(const float *) p;
+        }
     }
     acc = vx_wave_sum(acc);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
@@ -453,7 +462,9 @@ extern "C" int vx_supports_sum(const vx_tensor * src, const vx_tensor * dst) {
 extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
     if (!vx_supports_sum(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "sum: F32 tensor of at most 2^24 elements to an F32 scalar");
     if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "sum: null data");
-    sum_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
+    const bool vec = src->ne[0] % 4 == 0 && al16(src->data, src->nb);
+    if (vec) sum_kernel<true><<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
+    else     sum_kernel<false><<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
