@@ -369,9 +369,10 @@ def main():
                                                "us_per_attention": s / n_calls * 1e6}
         del keep
         for name, M, K, N in (("q8_0_proj_1024x1024_n2", 1024, 1024, 2), ("q8_0_ffn_up_4096x1024_n2", 4096, 1024, 2),
-                              ("q8_0_proj_1024x1024_n1024", 1024, 1024, 1024)):
+                              ("q8_0_proj_1024x1024_n1024", 1024, 1024, 1024), ("q8_0_ffn_up_4096x1024_n1024", 4096, 1024, 1024),
+                              ("q8_0_proj_1024x1024_n16384", 1024, 1024, 16384)):
             call, keep = q8_proj_setup(pkg, M, K, N)
-            s = timer.run(call, iters=200, warmup=5)
+            s = timer.run(call, iters=200 if N <= 1024 else 20, warmup=5)
             wbytes = M * K // 32 * 34
             others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12}
             del keep

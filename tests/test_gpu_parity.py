@@ -381,7 +381,9 @@ def mm_inputs(tag, M, K, N, batch=()):
 
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 1), (1024, 1024, 2), (128, 1024, 2), (4096, 1024, 2), (1024, 4096, 2),
                                    (1024, 1024, 5), (1024, 1024, 16), (1024, 1024, 17), (1000, 1024, 33),
-                                   (3072, 1024, 112), (1024, 1024, 512), (70, 96, 130)])
+                                   (3072, 1024, 112), (1024, 1024, 512), (70, 96, 130),
+                                   # the 128 x 128 pipelined GEMM: full tiles, and ragged rows / tokens / odd block count
+                                   (4096, 1024, 1024), (2000, 1056, 1700)])
 def test_mul_mat_q8_0(gpu, M, K, N):
     say(f"mul_mat Q8_0 M={M} K={K} N={N}")
     w, x = mm_inputs(("q8", M, K, N), M, K, N)
@@ -400,7 +402,7 @@ def test_mul_mat_q8_0(gpu, M, K, N):
 
 
 @pytest.mark.parametrize("wtype", [np.float16, np.float32])
-@pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300)])
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300), (2048, 256, 1600)])
 def test_mul_mat_float_weights(gpu, wtype, M, K, N):
     say(f"mul_mat {wtype.__name__} weights M={M} K={K} N={N}")
     w, x = mm_inputs(("fw", M, K, N), M, K, N)

@@ -513,8 +513,9 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     a.chunk    = (a.n_kv + 31) / 32 * 32;
     // Up to 256 keys one wave finishes (0.5 us per 32-key step) before a split plus the merge
     // launch would.
-    if (tiles < (int64_t) 4 * num_cus() && a.n_kv > 256) {
-        int64_t want = ((int64_t) 4 * num_cus() + tiles - 1) / tiles;
+    static const int waves_per_cu = [] { const char * e = getenv("VX_FA_WAVES_PER_CU"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 32 ? v : 4; }();
+    if (tiles < (int64_t) waves_per_cu * num_cus() && a.n_kv > 256) {
+        int64_t want = ((int64_t) waves_per_cu * num_cus() + tiles - 1) / tiles;
         const int64_t max_splits = (a.n_kv + min_chunk - 1) / min_chunk;
         if (want > max_splits) want = max_splits;
         if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;

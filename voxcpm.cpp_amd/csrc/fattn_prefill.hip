@@ -74,20 +74,34 @@ __device__ __forceinline__ float fmax8(const float4_t & x, const float4_t & y) {
     return fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(y[0], y[1]), fmaxf(y[2], y[3])));
 }
 
-// classifies mask tiles: one wave per (key tile, row block, mask batch)
+// classifies mask tiles: one wave per (key tile, row block, mask batch).  A lane reads 8 keys
+// (16 bytes) of a row, so the wave covers 8 rows of the 64-key tile per step.
 __global__ __launch_bounds__(64) void pf_mask_flags_kernel(const char * mask, uint64_t nbm1, uint64_t nbm2, uint64_t nbm3,
                                                            int nem2, int n_q, int n_kv, int RB, int n_rb, int n_tiles,
-                                                           uint8_t * flags) {
+                                                           int vec_ok, uint8_t * flags) {
     const int tile = blockIdx.x, rb = blockIdx.y, mb = blockIdx.z;
-    const int key  = tile * PF_KT + threadIdx.x;
     const char * mp = mask + (uint64_t) (mb % nem2) * nbm2 + (uint64_t) (mb / nem2) * nbm3;
+    const int r0 = rb * RB, r1 = min(n_q, (rb + 1) * RB);
     bool any_visible = false, any_nonzero = false;
-    if (key < n_kv) {
-        const int r1 = min(n_q, (rb + 1) * RB);
-        for (int r = rb * RB; r < r1; ++r) {
-            const uint16_t bits = ((const uint16_t *) (mp + (uint64_t) r * nbm1))[key];
-            any_visible |= bits != 0xFC00u;
-            any_nonzero |= (bits & 0x7FFFu) != 0;
+    if (vec_ok && (tile + 1) * PF_KT <= n_kv) {
+        const int sub = threadIdx.x >> 3, part = threadIdx.x & 7; // row within the step, 8-key group
+        for (int r = r0 + sub; r < r1; r += 8) {
+            const int4_t v = *(const int4_t *) (mp + (uint64_t) r * nbm1 + ((uint64_t) tile * PF_KT + part * 8) * 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = (uint32_t) v[i];
+                any_visible |= (w & 0xFFFFu) != 0xFC00u || (w >> 16) != 0xFC00u;
+                any_nonzero |= (w & 0x7FFF7FFFu) != 0;
+            }
+        }
+    } else {
+        const int key = tile * PF_KT + threadIdx.x;
+        if (key < n_kv) {
+            for (int r = r0; r < r1; ++r) {
+                const uint16_t bits = ((const uint16_t *) (mp + (uint64_t) r * nbm1))[key];
+                any_visible |= bits != 0xFC00u;
+                any_nonzero |= (bits & 0x7FFFu) != 0;
+            }
         }
     }
     const bool vis = __builtin_amdgcn_ballot_w64(any_visible) != 0;
@@ -441,7 +455,8 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
         vx_status rc = vx_workspace(st, (size_t) nmb * n_rb * n_tiles, &ws);
         if (rc != VX_OK) return rc;
         pf_mask_flags_kernel<<<dim3((unsigned) n_tiles, (unsigned) n_rb, (unsigned) nmb), dim3(64), 0, st>>>(
-            a.mask, a.nbm1, a.nbm2, a.nbm3, a.nem2, n_q, n_kv, RB, n_rb, n_tiles, (uint8_t *) ws);
+            a.mask, a.nbm1, a.nbm2, a.nbm3, a.nem2, n_q, n_kv, RB, n_rb, n_tiles,
+            (int) ((uintptr_t) a.mask % 16 == 0 && a.nbm1 % 16 == 0 && a.nbm2 % 16 == 0 && a.nbm3 % 16 == 0), (uint8_t *) ws);
         VX_LAUNCH_CHECK();
         a.flags = (const uint8_t *) ws;
     }

@@ -416,8 +416,223 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     return true;
 }
 
+
+// ---- GEMM shape: many tokens (prefill) --------------------------------------------------------------
+// A work-group of 4 waves (2 x 2) owns 128 weight rows x 128 tokens, each wave 64 x 64 as 4 x 4 MFMA
+// tiles, so an operand fetched from LDS (activations) or dequantised in registers (weights) feeds four
+// MFMAs.  K is walked in rounds of GM_KC blocks.  Both streams are software-pipelined: the raw Q8_0
+// bytes of round r+1 are requested right after round r's have been turned into operands, and the
+// activations of round r+1 are requested before round r's MFMAs and converted into the other LDS
+// buffer after them -- one barrier per round, no load waits in front of the matrix work.
+constexpr int GM_KC = 2;
+
+template <int WT, bool ACT_Q8, bool AL4>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm128_kernel(const mm_args a) {
+    constexpr int TT = 8; // 16-token tiles per work-group
+    __shared__ half8_t xs[2][GM_KC * TT * 64];
+    __shared__ float   xd[2][ACT_Q8 ? GM_KC * TT * 16 : 1];
+
+    const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
+    const int j = lane >> 4, c = lane & 15;
+    const int wr = wid >> 1, wt = wid & 1;
+
+    const int     batch = blockIdx.z;
+    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+
+    // Tile order.  Work-groups are dealt to the 8 XCDs round-robin and each XCD has its own L2, so the
+    // token tiles are partitioned over the XCDs (tile ty goes to XCD ty % 8) and inside an XCD the row
+    // tiles of one token tile run side by side: its activations are fetched into that L2 once, and the
+    // weights stream through it once per couple of token tiles instead of once per work-group.
+    const int64_t gx = (a.M + 127) / 128, gy = (a.N + 127) / 128;
+    const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int64_t ty = (slot / gx) * 8 + xcd;
+    if (ty >= gy) return; // padding of the last group of 8 token tiles (whole work-group)
+    const int64_t tok0 = ty * 128;
+    const int64_t row0 = (slot % gx) * 128 + wr * 64;
+    // addresses are (uniform base + uniform round offset) + a 32-bit lane offset that never changes, so the
+    // loads take a scalar base and no per-load vector address arithmetic (the launcher checks the ranges)
+    uint32_t woff[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) woff[rt] = (uint32_t) (min(row0 + 16 * rt + c, a.M - 1) * a.nb01);
+    constexpr bool al4 = AL4;
+    const int64_t nkb = a.K / 32, nround = (nkb + GM_KC - 1) / GM_KC;
+    constexpr int WBLK = WT == WT_Q8 ? VX_Q8_BLOCK : 64; // bytes of one 32-wide block of a row
+
+    // ---- weight stream: raw bytes of one round
+    q8_raw   wq[GM_KC][4];
+    _Float16 wdv[GM_KC][4];
+    half8_t  wh[GM_KC][4];
+    auto load_weights = [&](int64_t round) {
+#pragma unroll
+        for (int kbl = 0; kbl < GM_KC; ++kbl) {
+            const int64_t kb = min(round * GM_KC + kbl, nkb - 1); // clamped: a valid address, result unused
+            const char * wk = wb + (uint64_t) kb * WBLK;          // uniform
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                if constexpr (WT == WT_Q8) {
+                    wdv[kbl][rt] = *(const _Float16 *) (wk + woff[rt]);
+                    if constexpr (AL4) {
+                        const bool odd = (kb & 1) != 0; // uniform
+                        const char * p = (const char *) __builtin_assume_aligned(wk + (odd ? -2 : 0) + (woff[rt] + 8u * (uint32_t) j), 4);
+                        uint32_t v[3];
+                        __builtin_memcpy(v, p, 12);
+                        wq[kbl][rt] = q8_raw{v[0], v[1], v[2]};
+                    } else {
+                        wq[kbl][rt] = q8_load(wk + woff[rt], 0, j, false);
+                    }
+                } else {
+                    __builtin_memcpy(&wh[kbl][rt], wk + (woff[rt] + 16u * (uint32_t) j), 16);
+                }
+            }
+        }
+    };
+    // ---- activation stream: a thread moves 4 units (8 consecutive k of one token) per round
+    float4_t xr[4][2];
+    uint32_t xoff[4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int unit = tid + 256 * it;
+        xoff[it] = (uint32_t) ((uint64_t) (unit >> 3) * a.nb11 + (uint64_t) (unit & 7) * 32);
+    }
+    const char * xtile = xb + (uint64_t) tok0 * a.nb11; // uniform
+    auto load_acts = [&](int64_t round) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int unit = tid + 256 * it;
+            const int t = unit >> 3, u = unit & 7;
+            const int64_t tok = tok0 + t, k = (round * GM_KC) * 32 + u * 8;
+            xr[it][0] = float4_t{0, 0, 0, 0}; xr[it][1] = float4_t{0, 0, 0, 0};
+            if (tok < a.N && k < a.K) {
+                const float * xp = (const float *) (xtile + (uint64_t) round * (GM_KC * 32 * 4) + xoff[it]);
+                if (a.x_aligned) { xr[it][0] = ((const float4_t *) xp)[0]; xr[it][1] = ((const float4_t *) xp)[1]; }
+                else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { xr[it][0][i] = xp[i]; xr[it][1][i] = xp[4 + i]; }
+                }
+            }
+        }
+    };
+    auto store_acts = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int unit = tid + 256 * it;
+            const int t = unit >> 3, u = unit & 7, kbl = u >> 2, uj = u & 3;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[i] = xr[it][0][i]; v[4 + i] = xr[it][1][i]; }
+            half8_t h;
+            if constexpr (ACT_Q8) {
+                float amax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                const float d  = amax / 127.f;
+                const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
+                if (uj == 0) xd[buf][(kbl * TT + (t >> 4)) * 16 + (t & 15)] = (float) (_Float16) d;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
+            }
+            xs[buf][lds_slot(kbl, t >> 4, TT, uj, t & 15)] = h;
+        }
+    };
+
+    float4_t acc[4][4]; // [row tile][token tile]
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) acc[rt][tt] = float4_t{0, 0, 0, 0};
+
+    load_weights(0);
+    load_acts(0);
+    store_acts(0);
+    __syncthreads();
+
+    for (int64_t round = 0; round < nround; ++round) {
+        const int buf = (int) (round & 1);
+        // this round's weights become operands; their registers take the next round's bytes
+        half8_t bop[GM_KC][4];
+        float   dw[GM_KC][4];
+#pragma unroll
+        for (int kbl = 0; kbl < GM_KC; ++kbl)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                if constexpr (WT == WT_Q8) {
+                    bop[kbl][rt] = q8_unpack(wq[kbl][rt], min(round * GM_KC + kbl, nkb - 1), al4);
+                    dw[kbl][rt]  = (float) wdv[kbl][rt];
+                } else {
+                    bop[kbl][rt] = wh[kbl][rt];
+                    dw[kbl][rt]  = 1.0f;
+                }
+            }
+        const bool more = round + 1 < nround; // uniform
+        if (more) { load_weights(round + 1); load_acts(round + 1); }
+
+#pragma unroll
+        for (int kbl = 0; kbl < GM_KC; ++kbl) {
+            if (round * GM_KC + kbl >= nkb) break; // uniform: K holds an odd number of blocks
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                const half8_t aop = xs[buf][lds_slot(kbl, wt * 4 + tt, TT, j, c)];
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) {
+                    if constexpr (WT == WT_Q8) {
+                        const float4_t blk = mfma16(aop, bop[kbl][rt], float4_t{0, 0, 0, 0});
+                        if constexpr (ACT_Q8) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) acc[rt][tt][r] += blk[r] * (dw[kbl][rt] * xd[buf][(kbl * TT + wt * 4 + tt) * 16 + 4 * j + r]);
+                        } else {
+                            acc[rt][tt] += blk * dw[kbl][rt];
+                        }
+                    } else {
+                        acc[rt][tt] = mfma16(aop, bop[kbl][rt], acc[rt][tt]);
+                    }
+                }
+            }
+        }
+        if (more) store_acts(buf ^ 1);
+        __syncthreads();
+    }
+
+    // lane (j,c), tile (rt, tt), register r: token tok0 + 64 wt + 16 tt + 4j + r, row row0 + 16 rt + c
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const int64_t row = row0 + 16 * rt + c;
+        if (row >= a.M) continue;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t tok = tok0 + 64 * wt + 16 * tt + 4 * j + r;
+                if (tok < a.N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4) = acc[rt][tt][r];
+            }
+    }
+}
+
+template <int WT, bool ACT_Q8>
+bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
+    if (WT == WT_F32 || a.K % 32 || a.K < 32 || a.N < 128) return false;
+    const int64_t gx = (a.M + 127) / 128, gy = (a.N + 127) / 128;
+    if (gx * gy * nbatch < 192) return false; // small problems spread wider on the 64 x 64 tiles
+    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
+    if (blocks > 0x7fffffff) return false;
+    // 32-bit lane offsets inside the kernel: rows of the weight matrix and the 128 tokens of a tile
+    if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 128 * a.nb11 + 256 >= (1ull << 32)) return false;
+    const dim3 grid((unsigned) blocks, 1, (unsigned) nbatch);
+    if (WT == WT_Q8 && a.w_aligned) gemm128_kernel<WT, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
+    else                            gemm128_kernel<WT, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+    return true;
+}
+
 template <int WT, bool ACT_Q8>
 void launch(const mm_args & a, int nbatch, hipStream_t st) {
+    if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if constexpr (WT != WT_F32) { if (launch_gemv<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
