@@ -90,6 +90,48 @@ def test_supports_truth_table(pkg):
     assert lib.vx_supports_mul_mat(transposed, x2, o2) == 0
 
 
+def test_supports_truth_table_glue(pkg):
+    """The glue operators of a decoder layer and the fused pairs: what supports_op will answer."""
+    lib = pkg.lib()
+    a = f32(pkg, [1024, 5, 3, 2])
+    assert lib.vx_supports_binary(pkg.BIN_ADD, a, a, a) == 1
+    assert lib.vx_supports_binary(pkg.BIN_MUL, a, f32(pkg, [1024, 1, 1, 1]), a) == 1      # norm weight over tokens
+    assert lib.vx_supports_binary(pkg.BIN_MUL, a, f32(pkg, [1, 5, 1, 2]), a) == 1          # bias column
+    assert lib.vx_supports_binary(pkg.BIN_ADD, a, f32(pkg, [1000, 5, 3, 2]), a) == 0       # not repeatable
+    assert lib.vx_supports_binary(pkg.BIN_ADD, a, a, f32(pkg, [1024, 5, 3, 1])) == 0
+    assert lib.vx_supports_binary(pkg.BIN_ADD, f16(pkg, [8, 1, 1, 1]), f16(pkg, [8, 1, 1, 1]), f16(pkg, [8, 1, 1, 1])) == 0
+    assert lib.vx_supports_binary(7, a, a, a) == 0
+    one = f32(pkg, [1, 1, 1, 1])
+    assert lib.vx_supports_add1(a, one, a) == 1 and lib.vx_supports_add1(a, f32(pkg, [2, 1, 1, 1]), a) == 0
+    assert lib.vx_supports_unary(pkg.UNARY_SILU, a, a) == 1
+    assert lib.vx_supports_unary(8, a, a) == 0                                               # GELU: not claimed
+    gu = f32(pkg, [8192, 2, 1, 1])
+    half = f32(pkg, [4096, 2, 1, 1])
+    assert lib.vx_supports_glu(pkg.GLU_SWIGLU, half, half, half) == 1
+    assert lib.vx_supports_glu(pkg.GLU_SWIGLU, gu, None, half) == 1
+    assert lib.vx_supports_glu(pkg.GLU_SWIGLU, gu, None, gu) == 0
+    assert lib.vx_supports_glu(1, half, half, half) == 0                                     # GEGLU: not claimed
+    # CPY: F32/F16 both ways, equal element counts, any shapes
+    assert lib.vx_supports_cpy(f32(pkg, [64, 2, 5, 2]), f16(pkg, [64, 2, 5, 2])) == 1
+    assert lib.vx_supports_cpy(f32(pkg, [64, 2, 5, 2]), f32(pkg, [128, 10, 1, 1])) == 1
+    assert lib.vx_supports_cpy(f32(pkg, [64, 2, 5, 2]), f32(pkg, [64, 2, 5, 1])) == 0
+    assert lib.vx_supports_cpy(q8(pkg, [64, 2, 1, 1]), f32(pkg, [64, 2, 1, 1])) == 0
+    # CONCAT: same type, equal outside the dim
+    past, cur, both = f32(pkg, [64, 37, 2, 2]), f32(pkg, [64, 1, 2, 2]), f32(pkg, [64, 38, 2, 2])
+    assert lib.vx_supports_concat(past, cur, both, 1) == 1
+    assert lib.vx_supports_concat(past, cur, both, 0) == 0
+    assert lib.vx_supports_concat(past, f16(pkg, [64, 1, 2, 2]), both, 1) == 0
+    # SUM: dense F32 rows to a scalar
+    assert lib.vx_supports_sum(a, one) == 1 and lib.vx_supports_sum(a, f32(pkg, [2, 1, 1, 1])) == 0
+    permuted = D(pkg, pkg.F32, [5, 1024, 1, 1], [4096, 4, 20480, 20480])
+    assert lib.vx_supports_sum(permuted, one) == 0
+    # fused pairs
+    w = f32(pkg, [1024, 1, 1, 1])
+    assert lib.vx_supports_rms_norm_mul(a, w, a) == 1
+    assert lib.vx_supports_rms_norm_mul(a, f32(pkg, [1024, 5, 1, 1]), a) == 0
+    assert lib.vx_supports_fused_pair(a, a, a) == 1 and lib.vx_supports_fused_pair(a, w, a) == 0
+
+
 def test_ops_validate_before_touching_the_device(pkg):
     """Contract violations are reported by status + message; nothing is launched."""
     lib = pkg.lib()
