@@ -386,16 +386,28 @@ def main():
         cpu = cpu_baseline(B, L, threads)
 
     line = {
-        "metric": "decode attention HBM GB/s (backbone-shaped decode, 24 layers, batch 2)",
+        # BASELINE.json's metric, verbatim; `value` is its decode component on config 2 (see config.value_is),
+        # the prefill TFLOP/s and backbone steps/s components are repeated under "components"
+        "metric": "attn TFLOP/s (prefill) & HBM GB/s (decode) vs roofline; backbone decode steps/s",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 K/V, f32 accumulate", "data": "synthetic (seeded N(0,1))",
         "config": {"workload": f"BASELINE config 2: 24 layers x GQA decode attention, 16/2 heads, head_dim 64, "
-                               f"batch 2, f16 KV length {L}", "decode_attn_steps_per_s": 1.0 / sec_per_step,
+                               f"batch 2, f16 KV length {L}",
+                   "value_is": "decode attention HBM GB/s: algorithmic K/V bytes of the 24 calls of a step / wall time of the step",
+                   "decode_attn_steps_per_s": 1.0 / sec_per_step,
                    "launch": "eager from Python" if args.eager else "one HIP graph replay per step",
                    "eager_python_ms_per_step": eager_sec * 1e3},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "components": {
+            "decode_attn_GB/s_cfg2": value,
+            "decode_attn_hbm_frac_cfg5_B16_L8192": others.get("cfg5_decode_attn_B16_L8192", {}).get("hbm_frac"),
+            "prefill_attn_TFLOP/s_cfg5_T4096_B16": others.get("cfg5_prefill_attn_T4096_B16", {}).get("TFLOP/s_causal_exact"),
+            "prefill_attn_mfma_frac_cfg5_T4096_B16": others.get("cfg5_prefill_attn_T4096_B16", {}).get("mfma_frac"),
+            "backbone_decode_steps_per_s_cfg4": others.get("cfg4_backbone_24layers_b2", {}).get("decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_ggml_cpu": others.get("cfg4_backbone_24layers_b2", {}).get("ggml_cpu", {}).get("decode_steps_per_s"),
+        },
         "others": others,
     }
     print(json.dumps(line))
