@@ -185,6 +185,17 @@ VX_API vx_status vx_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight
 VX_API vx_status vx_scale_add(const vx_tensor * a, const vx_tensor * x, const vx_tensor * dst, float scale, vx_stream stream);
 /* ADD(a, b) -> SCALE(., scale, bias): dst = (a + b) * scale + bias (the kv_sync tail, src/minicpm.cpp:685-689) */
 VX_API vx_status vx_add_scale(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst, float scale, float bias, vx_stream stream);
+/* FLASH_ATTN_EXT(...) -> ADD1(., addend): the scalar the reference adds after attention to order its cache
+ * write (src/minicpm.cpp:711-713); addend is a device F32 scalar, added after the normalisation */
+VX_API vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                        const vx_tensor * mask, const float * sinks, const float * addend,
+                                        const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
+                                        vx_stream stream);
+/* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for at most 16 tokens
+ * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
+VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
+                                   int act_mode, vx_stream stream);
+VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst);
 VX_API int vx_supports_fused_pair(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst);
 

@@ -15,7 +15,7 @@ A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and i
 are built once, so a plan can be replayed from a captured HIP graph.
 
 With `fuse_pairs=True` the four adjacent-node pairs the ggml backend plugin runs as one launch
-(rms_norm+mul, scale+add, cont+sum, add+scale) are issued as the plugin issues them; the results
+(rms_norm+mul, scale+add, cont+sum, add+scale, flash_attn_ext+add1, and the gate/up/SwiGLU triple at decode size) are issued as the plugin issues them; the results
 are bit-identical to the unfused sequence.
 """
 import math
@@ -168,17 +168,24 @@ class MiniCPMBackbone:
                 call(L.vx_concat, desc(kc[:, :, :n_past]), desc(k_all), desc(kall), 1)
                 call(L.vx_concat, desc(vc[:, :, :n_past]), desc(v_all), desc(vall), 1)
                 k_all, v_all = kall, vall
-            call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
-                 scale, 0.0, 0.0)
-            if chain:
-                call(L.vx_add1, desc(attn), desc(sync), desc(attn))
+            if chain and fuse:       # attention + add1 as one launch
+                call(L.vx_flash_attn_ext_add1, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, _p(sync),
+                     desc(attn), scale, 0.0, 0.0)
+            else:
+                call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
+                     scale, 0.0, 0.0)
+                if chain:
+                    call(L.vx_add1, desc(attn), desc(sync), desc(attn))
             call(L.vx_mul_mat, wd["o_proj"], desc(attn.view(N, H * D)), desc(attn_o), self.act_mode)
             residual(cur_x, attn_o, h_mid)
             # -- mlp_forward
             norm(h_mid, nrm["post_layernorm"], normed)
-            call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
-            call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
-            call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)
+            if fuse and N <= 16:     # gate, up and SwiGLU as one launch
+                call(L.vx_mul_mat_swiglu, wd["gate_proj"], wd["up_proj"], desc(normed), desc(act), self.act_mode)
+            else:
+                call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
+                call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
+                call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)
             call(L.vx_mul_mat, wd["down_proj"], desc(act), desc(down), self.act_mode)
             nxt = hs[li % 2]
             residual(h_mid, down, nxt)

@@ -42,6 +42,7 @@ namespace {
 struct fa_args {
     const char * q; const char * k; const char * v; const char * mask;
     const float * sinks;
+    const float * add1; // optional scalar added to every output element (a fused GGML_OP_ADD1)
     float * dst;
     float * part_o;   // [tile][split][16 columns][D]   split partials, un-normalised
     float * part_ml;  // [tile][split][16 columns][2]   running max, running sum
@@ -104,7 +105,9 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
         L = L * ms + vs;
     }
     const float inv = L == 0.0f ? 0.0f : 1.0f / L;
-    *(float4_t *) (a.dst + (((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D + d0) = acc * inv;
+    float4_t r = acc * inv;
+    if (a.add1) r += *a.add1; // rounded after the normalisation, as the separate ADD1 node would
+    *(float4_t *) (a.dst + (((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D + d0) = r;
 }
 
 // One wave (= one block) = 16 columns x one key range.
@@ -463,6 +466,13 @@ extern "C" int vx_supports_flash_attn_ext(const vx_tensor * q, const vx_tensor *
 extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
                                        const vx_tensor * mask, const float * sinks, const vx_tensor * dst,
                                        float scale, float max_bias, float logit_softcap, vx_stream stream) {
+    return vx_flash_attn_ext_add1(q, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, stream);
+}
+
+extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                            const vx_tensor * mask, const float * sinks, const float * addend,
+                                            const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
+                                            vx_stream stream) {
     if (!q || !k || !v || !dst || !q->data || !k->data || !v->data || !dst->data || (mask && !mask->data))
         return vx_fail(VX_ERR_INVALID, "flash_attn_ext: null tensor");
     if (!vx_supports_flash_attn_ext(q, k, v, mask, dst))
@@ -475,7 +485,7 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     {   // many query rows: the LDS-tiled kernel
         static const bool no_prefill = getenv("VX_FA_NO_PREFILL") != nullptr;
         if (!no_prefill) {
-            const vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, dst, scale, max_bias, logit_softcap, st);
+            const vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, addend, dst, scale, max_bias, logit_softcap, st);
             if (rc != VX_ERR_UNSUPPORTED) return rc;
         }
     }
@@ -483,6 +493,7 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
     a.mask = mask ? (const char *) mask->data : nullptr;
     a.sinks = sinks;
+    a.add1 = addend;
     a.dst = (float *) dst->data;
     a.part_o = nullptr; a.part_ml = nullptr;
     a.nbq1 = q->nb[1]; a.nbq2 = q->nb[2]; a.nbq3 = q->nb[3];

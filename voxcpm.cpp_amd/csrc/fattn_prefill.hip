@@ -41,6 +41,7 @@ constexpr float PF_LAZY = 8.0f; // log2 units a score may exceed its reference b
 struct pf_args {
     const char * q; const char * k; const char * v; const char * mask;
     const float * sinks;
+    const float * add1; // optional scalar added to every output element (a fused GGML_OP_ADD1)
     float * dst;
     const uint8_t * flags; // [nem3][nem2][n_rb][n_tiles]: 0 skip, 1 no mask, 2 apply mask
     uint64_t nbq1, nbq2, nbq3, nbk1, nbk2, nbk3, nbv1, nbv2, nbv3, nbm1, nbm2, nbm3;
@@ -404,7 +405,11 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
         if (ok) {
             float * out = a.dst + (((uint64_t) b * a.n_q + row) * a.Hq + hd) * D;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) *(float4_t *) (out + 16 * t + 4 * j) = o[ct][t] * inv;
+            for (int t = 0; t < 4; ++t) {
+                float4_t r = o[ct][t] * inv;
+                if (a.add1) r += *a.add1;
+                *(float4_t *) (out + 16 * t + 4 * j) = r;
+            }
         }
     }
 }
@@ -414,8 +419,8 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 // Called by vx_flash_attn_ext when the shape suits this kernel; returns VX_ERR_UNSUPPORTED
 // (without touching the error string) when the caller should use the general kernel.
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
-                           const float * sinks, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
-                           hipStream_t st) {
+                           const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
+                           float logit_softcap, hipStream_t st) {
     if (q->ne[0] != 64 || logit_softcap != 0.0f) return VX_ERR_UNSUPPORTED;
     // F32 K/V would be rounded to f16 here (error up to ~1e-3); the general kernel keeps hi + lo parts
     if (k->type != VX_TYPE_F16) return VX_ERR_UNSUPPORTED;
@@ -431,6 +436,7 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
     a.mask = mask ? (const char *) mask->data : nullptr;
     a.sinks = sinks;
+    a.add1 = addend;
     a.dst = (float *) dst->data;
     a.flags = nullptr;
     a.nbq1 = q->nb[1]; a.nbq2 = q->nb[2]; a.nbq3 = q->nb[3];

@@ -36,6 +36,7 @@ struct mm_args {
     int x_aligned; // src1 rows allow 16-byte vector loads
     int w_aligned; // Q8_0 rows start on dword boundaries
     int rows_wg;   // GEMV: weight rows per work-group (16, 8 or 4)
+    const char * w2; // GEMV, fused gate/up + SwiGLU: the second weight matrix (same shape and strides), else null
 };
 
 constexpr int WT_Q8 = 0, WT_F16 = 1, WT_F32 = 2;
@@ -261,10 +262,15 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // R = a.rows_wg of the 16 MFMA columns carry weight rows; fewer rows per work-group put a short
     // matrix on more CUs (a CU sustains only so many outstanding lines, so 64 work-groups cannot
     // pull what 256 can).  Lanes c >= R load nothing; their columns are never stored.
-    const int     R = a.rows_wg;
-    const int64_t row0 = (int64_t) blockIdx.x * R;
-    const bool    row_ok = c < R && row0 + c < a.M;
-    const char *  wrow = wb + (uint64_t) min(row0 + c, a.M - 1) * a.nb01;
+    // With a second matrix (SwiGLU: dst = silu(W x) * (W2 x)) the MFMA columns are split: the first half of
+    // them carries rows of W, the second half the same rows of W2, and the epilogue pairs them up.
+    const bool    dual = a.w2 != nullptr;                 // uniform
+    const int     R  = a.rows_wg, Rr = dual ? R / 2 : R;   // MFMA columns in use, output rows per work-group
+    const int     cr = dual ? c % Rr : c;
+    const int64_t row0 = (int64_t) blockIdx.x * Rr;
+    const bool    row_ok = c < R && row0 + cr < a.M;
+    const char *  wsel = (dual && c >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
+    const char *  wrow = wsel + (uint64_t) min(row0 + cr, a.M - 1) * a.nb01;
     const int     N = (int) a.N;
 
     // ---- this wave's weight blocks: kb = wid + NW * i
@@ -368,7 +374,14 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         for (int ww = 0; ww < NW - 1; ++ww) acc += red[ww * 64 + lane];
     }
     // lane (j,c), register r: token 4j + r, row row0 + c
-    if (row_ok) {
+    if (dual) { // lane c < Rr holds W's row, lane c + Rr the same row of W2: dst = silu(gate) * up
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float up = __shfl(acc[r], lane + Rr, 64);
+            acc[r] = (acc[r] / (1.0f + expf(-acc[r]))) * up;
+        }
+    }
+    if (row_ok && c < Rr) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int tok = 4 * j + r;
@@ -394,11 +407,13 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     mm_args a = a0;
     if (a.N > 16 || a.K % 32 || a.K < 32) return false;
     a.rows_wg = 16;
-    while (a.rows_wg > 4 && (a.M + a.rows_wg - 1) / a.rows_wg * nbatch < 128) a.rows_wg /= 2;
+    const int split = a.w2 ? 2 : 1; // with two matrices a work-group's MFMA columns hold half as many output rows
+    while (a.rows_wg > 4 && (a.M * split + a.rows_wg - 1) / a.rows_wg * nbatch < 128) a.rows_wg /= 2;
     const int nw = gemv_waves(a);
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
     if (smem > 64 * 1024) return false;
-    const dim3 grid((unsigned) ((a.M + a.rows_wg - 1) / a.rows_wg), 1, (unsigned) nbatch);
+    const int rows_out = a.rows_wg / split;
+    const dim3 grid((unsigned) ((a.M + rows_out - 1) / rows_out), 1, (unsigned) nbatch);
     const dim3 block((unsigned) (64 * nw));
 #define VX_GEMV(NW_)                                                                                       \
     do {                                                                                                   \
@@ -689,6 +704,7 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
     a.ne12 = (int) src1->ne[2];
     a.r2 = (int) (src1->ne[2] / src0->ne[2]); a.r3 = (int) (src1->ne[3] / src0->ne[3]);
     a.rows_wg   = 16;
+    a.w2        = nullptr;
     a.w_aligned = ((uintptr_t) src0->data % 4 == 0) && src0->nb[1] % 4 == 0 && src0->nb[2] % 4 == 0 && src0->nb[3] % 4 == 0;
     a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
@@ -702,6 +718,49 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
         case VX_TYPE_F16: launch<WT_F16, false>(a, nbatch, st); break;
         default:          launch<WT_F32, false>(a, nbatch, st); break;
     }
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// MUL_MAT(gate) , MUL_MAT(up) , GLU(SWIGLU split) as one launch for decode-sized token counts
+// (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747).  Both products are formed exactly as vx_mul_mat
+// forms them (same block order, same reduction order), so the result equals the three separate nodes'.
+extern "C" int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst) {
+    if (!vx_supports_mul_mat(gate, src1, dst) || !up) return 0;
+    if (gate->type != VX_TYPE_Q8_0 && gate->type != VX_TYPE_F16) return 0;
+    if (up->type != gate->type) return 0;
+    for (int i = 0; i < 4; ++i) if (up->ne[i] != gate->ne[i] || up->nb[i] != gate->nb[i]) return 0;
+    if (src1->ne[1] > 16 || gate->ne[0] % 32 || gate->ne[0] < 32) return 0;
+    return (size_t) src1->ne[1] * gate->ne[0] * 2 + (size_t) src1->ne[1] * (gate->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+}
+
+extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
+                                       int act_mode, vx_stream stream) {
+    if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
+        return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
+    if (!vx_supports_mul_mat_swiglu(gate, up, src1, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, at most 16 tokens");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
+    if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
+    mm_args a;
+    a.w = (const char *) gate->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
+    a.K = gate->ne[0]; a.M = gate->ne[1]; a.N = src1->ne[1];
+    a.nb01 = gate->nb[1]; a.nb02 = gate->nb[2]; a.nb03 = gate->nb[3];
+    a.nb11 = src1->nb[1]; a.nb12 = src1->nb[2]; a.nb13 = src1->nb[3];
+    a.nb1 = dst->nb[1]; a.nb2 = dst->nb[2]; a.nb3 = dst->nb[3];
+    a.ne12 = (int) src1->ne[2];
+    a.r2 = (int) (src1->ne[2] / gate->ne[2]); a.r3 = (int) (src1->ne[3] / gate->ne[3]);
+    a.rows_wg   = 16;
+    a.w2        = (const char *) up->data;
+    a.w_aligned = (((uintptr_t) gate->data | (uintptr_t) up->data) % 4 == 0) && gate->nb[1] % 4 == 0 && gate->nb[2] % 4 == 0 && gate->nb[3] % 4 == 0;
+    a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
+    const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
+    hipStream_t st = (hipStream_t) stream;
+    bool ok;
+    if (gate->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
+    else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: shape outside the streaming kernel");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

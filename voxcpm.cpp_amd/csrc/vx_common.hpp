@@ -43,8 +43,8 @@ vx_status vx_counters(hipStream_t stream, size_t count, void ** ptr);
 
 // LDS-tiled prefill kernel (fattn_prefill.hip); VX_ERR_UNSUPPORTED means "use the general kernel"
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
-                           const float * sinks, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
-                           hipStream_t stream);
+                           const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
+                           float logit_softcap, hipStream_t stream);
 
 // ---- host-side tensor predicates ---------------------------------------------------------
 static inline size_t vx_type_size(int type) {

@@ -443,6 +443,22 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
         *rc = vx_add_scale(&a, &b, &d, sc, bias, ctx->stream);
         return true;
     }
+    if (node->op == GGML_OP_FLASH_ATTN_EXT && next->op == GGML_OP_ADD1 && next->src[0] == node && next->src[1] != node &&
+        next->src[1]->type == GGML_TYPE_F32 && ggml_nelements(next->src[1]) == 1) {
+        // attention_forward's ggml_add1(attn, kv_sync): the scalar is added in the attention kernel's epilogue
+        const vx_tensor q = to_vx(node->src[0]), k = to_vx(node->src[1]), v = to_vx(node->src[2]);
+        vx_tensor m;
+        if (node->src[3]) m = to_vx(node->src[3]);
+        if (node->src[4] && (node->src[4]->type != GGML_TYPE_F32 || node->src[4]->ne[0] != node->src[0]->ne[2])) return false;
+        if (!vx_supports_flash_attn_ext(&q, &k, &v, node->src[3] ? &m : nullptr, &d)) return false;
+        float scale, max_bias, softcap;
+        memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+        memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+        memcpy(&softcap, (const float *) node->op_params + 2, sizeof(float));
+        *rc = vx_flash_attn_ext_add1(&q, &k, &v, node->src[3] ? &m : nullptr, node->src[4] ? (const float *) node->src[4]->data : nullptr,
+                                     (const float *) next->src[1]->data, &d, scale, max_bias, softcap, ctx->stream);
+        return true;
+    }
     if (node->op == GGML_OP_CONT && next->op == GGML_OP_SUM && next->src[0] == node) {
         // the sum does not care where the elements lie: read them where they are
         const vx_tensor s = to_vx(node->src[0]);
@@ -483,7 +499,21 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
             ggml_tensor * next = cgraph->nodes[i + 1];
             const bool private_value = (node->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (next->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 &&
                                        readers[node] == 1;
-            if (private_value) fused = compute_pair(ctx, node, next, &rc);
+            // mlp_forward's MUL_MAT(gate), MUL_MAT(up), SWIGLU(gate, up) at decode size: one launch
+            if (private_value && i + 2 < cgraph->n_nodes && node->op == GGML_OP_MUL_MAT && next->op == GGML_OP_MUL_MAT) {
+                ggml_tensor * glu = cgraph->nodes[i + 2];
+                if (glu->op == GGML_OP_GLU && (glu->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 && glu->src[0] == node && glu->src[1] == next &&
+                    ggml_get_glu_op(glu) == GGML_GLU_OP_SWIGLU && ((const int32_t *) glu->op_params)[1] == 0 &&
+                    next->src[1] == node->src[1] && (next->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && readers[next] == 1) {
+                    const vx_tensor g = to_vx(node->src[0]), u = to_vx(next->src[0]), x = to_vx(node->src[1]), d = to_vx(glu);
+                    if (vx_supports_mul_mat_swiglu(&g, &u, &x, &d)) {
+                        rc = vx_mul_mat_swiglu(&g, &u, &x, &d, mul_mat_act_mode(), ctx->stream);
+                        fused = true;
+                        ++i; // one more node than a pair
+                    }
+                }
+            }
+            if (!fused && private_value) fused = compute_pair(ctx, node, next, &rc);
         }
         if (fused) ++i;
         else rc = compute_node(ctx, node);
