@@ -18,6 +18,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -415,6 +416,12 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     }
     if (!rc && out) ggml_backend_tensor_get(h, out, 0, ggml_nbytes(h));
     if (seconds) seconds[2] = (double) ggml_graph_n_nodes(gf);
+    if (getenv("RH_DUMP_GRAPH")) { // node order of the graph, for inspection
+        for (int i = 0; i < ggml_graph_n_nodes(gf); ++i) {
+            ggml_tensor * n = ggml_graph_node(gf, i);
+            fprintf(stderr, "%3d %s\n", i, ggml_op_desc(n));
+        }
+    }
     ggml_gallocr_free(ga);
     ggml_free(c);
     return rc;

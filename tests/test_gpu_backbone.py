@@ -45,6 +45,9 @@ def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
     # the same ggml graph, every node on the plugin (direct ggml_backend_graph_compute, no scheduler)
     assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
     plug, _ = run_reference(params, xs, b"GFX950_0", kv_f16, use_mup)
+    import ctypes
+    plugin_launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()  # of the last decode step
+    print(f"   plugin: {plugin_launches} operator launches for the {n_nodes}-node decode graph", flush=True)
     for i, (a, b) in enumerate(zip(cpu, plug)):
         e = nmse(a, b)
         print(f"   plugin vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
@@ -68,7 +71,10 @@ def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
         for i, x in enumerate(xs):
             T = x.shape[1]
             mask = torch.from_numpy(reflib.causal_mask(T, T)).cuda() if T > 1 else None
-            got = m.forward(torch.from_numpy(x).cuda(), n_past, mask)
+            run, got = m.plan(torch.from_numpy(x).cuda(), T, n_past, mask)
+            run()
+            if fuse and i == len(xs) - 1:  # the mirror issues exactly what the plugin issues for the reference's graph
+                assert run.n_calls == plugin_launches, (run.n_calls, plugin_launches)
             torch.cuda.synchronize()
             e = nmse(cpu[i], got.cpu().numpy())
             print(f"   C ABI mirror (act_mode {act}, fused pairs {fuse}) vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)

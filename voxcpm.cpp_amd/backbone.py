@@ -14,8 +14,9 @@ ggml's ne[3]; with batch 1 the call sequence is the reference's graph node for n
 A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and intermediates
 are built once, so a plan can be replayed from a captured HIP graph.
 
-With `fuse_pairs=True` the four adjacent-node pairs the ggml backend plugin runs as one launch
-(rms_norm+mul, scale+add, cont+sum, add+scale, flash_attn_ext+add1, and the gate/up/SwiGLU triple at decode size) are issued as the plugin issues them; the results
+With `fuse_pairs=True` the adjacent nodes the ggml backend plugin runs as one launch (rms_norm+mul,
+scale+add, cont+sum, add+scale, and the gate/up/SwiGLU triple at decode size) are issued as the plugin
+issues them, so a plan has as many launches as the plugin needs for the reference's graph; the results
 are bit-identical to the unfused sequence.
 """
 import math
@@ -142,23 +143,8 @@ class MiniCPMBackbone:
             for t4 in (q4, k4):
                 call(L.vx_rope, desc(t4), _p(pos), ff, desc(t4), D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0,
                      attn_factor, 32.0, 1.0)
-            if write_kv:
-                kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236
-                vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
-                call(L.vx_cpy, desc(k4), desc(kw))
-                call(L.vx_cpy, desc(v4), desc(vw))
-                keep += [kw, vw]
-            if chain and fuse:
-                call(L.vx_sum, desc(kw), desc(sk))       # cont + sum
-                call(L.vx_sum, desc(vw), desc(sv))
-                call(L.vx_add_scale, desc(sk), desc(sv), desc(sync), 0.0, 0.0)
-            elif chain:
-                call(L.vx_cpy, desc(kw), desc(kcont))
-                call(L.vx_sum, desc(kcont), desc(sk))
-                call(L.vx_cpy, desc(vw), desc(vcont))
-                call(L.vx_sum, desc(vcont), desc(sv))
-                call(L.vx_binary, BIN_ADD, desc(sk), desc(sv), desc(sync))
-                call(L.vx_scale, desc(sync), desc(sync), 0.0, 0.0)
+            # from here on in the order ggml_build_forward_expand gives the reference's graph: concat, attention,
+            # then the cache append with its ordering chain, then add1 (only adjacent nodes are run as one launch)
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)
             if n_past > 0:
                 if kcast is not None:
@@ -168,14 +154,26 @@ class MiniCPMBackbone:
                 call(L.vx_concat, desc(kc[:, :, :n_past]), desc(k_all), desc(kall), 1)
                 call(L.vx_concat, desc(vc[:, :, :n_past]), desc(v_all), desc(vall), 1)
                 k_all, v_all = kall, vall
-            if chain and fuse:       # attention + add1 as one launch
-                call(L.vx_flash_attn_ext_add1, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, _p(sync),
-                     desc(attn), scale, 0.0, 0.0)
-            else:
-                call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
-                     scale, 0.0, 0.0)
-                if chain:
-                    call(L.vx_add1, desc(attn), desc(sync), desc(attn))
+            call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
+                 scale, 0.0, 0.0)
+            if write_kv:
+                kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236
+                vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
+                keep += [kw, vw]
+                for src4, wv, cont, ssum in ((k4, kw, kcont, sk), (v4, vw, vcont, sv)):
+                    call(L.vx_cpy, desc(src4), desc(wv))
+                    if chain and fuse:
+                        call(L.vx_sum, desc(wv), desc(ssum))       # cont + sum
+                    elif chain:
+                        call(L.vx_cpy, desc(wv), desc(cont))
+                        call(L.vx_sum, desc(cont), desc(ssum))
+            if chain and fuse:
+                call(L.vx_add_scale, desc(sk), desc(sv), desc(sync), 0.0, 0.0)
+            elif chain:
+                call(L.vx_binary, BIN_ADD, desc(sk), desc(sv), desc(sync))
+                call(L.vx_scale, desc(sync), desc(sync), 0.0, 0.0)
+            if chain:
+                call(L.vx_add1, desc(attn), desc(sync), desc(attn))
             call(L.vx_mul_mat, wd["o_proj"], desc(attn.view(N, H * D)), desc(attn_o), self.act_mode)
             residual(cur_x, attn_o, h_mid)
             # -- mlp_forward

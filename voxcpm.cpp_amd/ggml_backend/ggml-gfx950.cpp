@@ -469,8 +469,11 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
     return false;
 }
 
+int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
+
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
+    int launches = 0;
     if (vx_init(ctx->device) != VX_OK) {
         GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
         return GGML_STATUS_FAILED;
@@ -517,12 +520,14 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         }
         if (fused) ++i;
         else rc = compute_node(ctx, node);
+        ++launches;
         if (rc != VX_OK) {
             GGML_LOG_ERROR("ggml-gfx950: node %d (%s, op %s) failed with status %d: %s\n", i, node->name,
                            ggml_op_name(node->op), (int) rc, rc == VX_ERR_UNSUPPORTED && !*vx_last_error() ? "operator not claimed by this backend" : vx_last_error());
             return GGML_STATUS_FAILED;
         }
     }
+    g_last_launches = launches;
     return GGML_STATUS_SUCCESS;
 }
 
@@ -669,3 +674,7 @@ GGML_BACKEND_API ggml_backend_reg_t ggml_backend_init(void) { return ggml_backen
 GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_count() > 0 ? 100 : 0; }
 
 } // extern "C"
+
+// Diagnostic: how many operator calls the most recent graph_compute of this process issued (an attention
+// call counts once although it may launch a split and a merge kernel).
+extern "C" __attribute__((visibility("default"))) int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
