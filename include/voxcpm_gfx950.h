@@ -196,6 +196,22 @@ VX_API vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
                                    int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst);
+/* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for at most 16 tokens,
+ * the residual updates of MiniCPMModel::layer_forward (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32
+ * of dst's shape */
+VX_API vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,
+                                      const vx_tensor * dst, float scale, int act_mode, vx_stream stream);
+VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,
+                                         const vx_tensor * dst);
+/* The reference's KV append with its write-ordering scalar (attention_forward, src/minicpm.cpp:682-713), nine graph
+ * nodes as one launch:  CPY(k, k_slot) CONT SUM , CPY(v, v_slot) CONT SUM , ADD , SCALE(scale, bias) , ADD1(x, .)
+ *   k_slot <- k ; v_slot <- v ; dst = x + ((sum(k_slot) + sum(v_slot)) * scale + bias)
+ * All F32; a cache write of at most 16384 elements (decode-sized), x of at most 65536; k_slot / v_slot with
+ * dense rows.  The sums are formed in vx_sum's order, so dst equals what the separate nodes give. */
+VX_API vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                                  const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream);
+VX_API int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                                     const vx_tensor * x, const vx_tensor * dst);
 VX_API int vx_supports_rms_norm_mul(const vx_tensor * src, const vx_tensor * weight, const vx_tensor * dst);
 VX_API int vx_supports_fused_pair(const vx_tensor * a, const vx_tensor * b, const vx_tensor * dst);
 

@@ -1,0 +1,232 @@
+"""GPU: every entry point that runs several adjacent graph nodes as one launch must give,
+bit for bit, what the same nodes give when each is its own launch (the separate launches are
+held to the CPU oracle and ggml-cpu in test_gpu_parity.py / test_gpu_ggml_backend.py).
+Covered here: RMS_NORM+MUL, SCALE+ADD, ADD+SCALE, FLASH_ATTN_EXT+ADD1, MUL_MAT+MUL_MAT+SWIGLU,
+MUL_MAT(+SCALE)+ADD, and the nine-node cache write with its ordering scalar.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import reflib
+from reflib import rng
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def q8_dev(w):
+    return dev(reflib.quantize_q8_0(w)), w.shape[1]
+
+
+def ok(pkg, rc, what):
+    pkg.check(rc, what)
+
+
+def same_bits(a, b):
+    import torch
+    return torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+@pytest.mark.parametrize("shape", [(2, 1024), (18, 1024), (3, 5, 4096), (7, 1025)])
+def test_rms_norm_mul(pkg, gpu, shape):
+    import torch
+    say(f"fused rms_norm+mul {shape}")
+    L, d = pkg.lib(), pkg.desc
+    x = dev(rng("f-rms", shape).standard_normal(shape).astype(np.float32))
+    w = dev((1 + 0.1 * rng("f-rms-w", shape).standard_normal(shape[-1])).astype(np.float32))
+    a, b = torch.empty_like(x), torch.empty_like(x)
+    ok(pkg, L.vx_rms_norm(d(x), d(a), 1e-5, None), "rms_norm")
+    ok(pkg, L.vx_binary(pkg.BIN_MUL, d(a), d(w), d(a), None), "mul")
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(w), d(b), 1e-5, None), "rms_norm_mul")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    # in place, as ggml-alloc may lay it out
+    xc = x.clone()
+    ok(pkg, L.vx_rms_norm_mul(d(xc), d(w), d(xc), 1e-5, None), "rms_norm_mul in place")
+    torch.cuda.synchronize()
+    assert torch.equal(a, xc)
+
+
+@pytest.mark.parametrize("shape", [(2, 1024), (2, 3, 1030), (1, 1)])
+def test_scale_add_and_add_scale(pkg, gpu, shape):
+    import torch
+    say(f"fused scale+add / add+scale {shape}")
+    L, d = pkg.lib(), pkg.desc
+    x = dev(rng("f-sa", shape).standard_normal(shape).astype(np.float32))
+    y = dev(rng("f-sa-y", shape).standard_normal(shape).astype(np.float32))
+    t, o1, o2 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    for s in (0.2857738, 0.0, -3.0):
+        ok(pkg, L.vx_scale(d(y), d(t), s, 0.0, None), "scale")
+        ok(pkg, L.vx_binary(pkg.BIN_ADD, d(x), d(t), d(o1), None), "add")
+        ok(pkg, L.vx_scale_add(d(x), d(y), d(o2), s, None), "scale_add")
+        torch.cuda.synchronize()
+        assert torch.equal(o1, o2)
+        for bias in (0.0, 0.75):
+            ok(pkg, L.vx_binary(pkg.BIN_ADD, d(x), d(y), d(t), None), "add")
+            ok(pkg, L.vx_scale(d(t), d(o1), s, bias, None), "scale")
+            ok(pkg, L.vx_add_scale(d(x), d(y), d(o2), s, bias, None), "add_scale")
+            torch.cuda.synchronize()
+            assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("T,n_kv,kv_f16", [(1, 640, False), (1, 4096, True), (512, 512, True), (7, 300, False)])
+def test_flash_attn_add1(pkg, gpu, T, n_kv, kv_f16):
+    import torch
+    say(f"fused flash_attn+add1 T={T} n_kv={n_kv} f16={kv_f16}")
+    L, d = pkg.lib(), pkg.desc
+    B, H, Hkv, D = 2, 16, 2, 64
+    g = rng("f-fa", T, n_kv)
+    q = dev(g.standard_normal((B, H, T, D)).astype(np.float32))
+    kt = np.float16 if kv_f16 else np.float32
+    k = dev(g.standard_normal((B, Hkv, n_kv, D)).astype(kt))
+    v = dev(g.standard_normal((B, Hkv, n_kv, D)).astype(kt))
+    mask = dev(reflib.causal_mask(T, n_kv, n_kv - T)) if T > 1 else None
+    addend = dev(np.array([0.375], dtype=np.float32))
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    ok(pkg, L.vx_flash_attn_ext(d(q), d(k), d(v), d(mask), None, d(a), 0.125, 0.0, 0.0, None), "fa")
+    ok(pkg, L.vx_add1(d(a), d(addend), d(a), None), "add1")
+    ok(pkg, L.vx_flash_attn_ext_add1(d(q), d(k), d(v), d(mask), None, addend.data_ptr(), d(b), 0.125, 0.0, 0.0, None), "fa_add1")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("M,K,N,nb", [(4096, 1024, 1, 2), (4096, 1024, 2, 1), (1000, 512, 16, 1), (24, 4096, 3, 2)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+def test_mul_mat_swiglu(pkg, gpu, M, K, N, nb, act):
+    import torch
+    say(f"fused gate/up/swiglu M={M} K={K} N={N} batch={nb} act={act}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-swiglu", M, K, N)
+    wg, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    wu, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    x = dev(g.standard_normal((nb, 1, N, K)).astype(np.float32))
+    gate = torch.empty((nb, 1, N, M), dtype=torch.float32, device="cuda")
+    up, a, b = torch.empty_like(gate), torch.empty_like(gate), torch.empty_like(gate)
+    ok(pkg, L.vx_mul_mat(pkg.desc_q8(wg, K), d(x), d(gate), mode, None), "gate")
+    ok(pkg, L.vx_mul_mat(pkg.desc_q8(wu, K), d(x), d(up), mode, None), "up")
+    ok(pkg, L.vx_glu(pkg.GLU_SWIGLU, d(gate), d(up), d(a), 0, None), "glu")
+    ok(pkg, L.vx_mul_mat_swiglu(pkg.desc_q8(wg, K), pkg.desc_q8(wu, K), d(x), d(b), mode, None), "mul_mat_swiglu")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
+    import torch
+    say(f"fused mul_mat+scale+add M={M} K={K} N={N} batch={nb} act={act}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-mmsa", M, K, N)
+    w, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    x = dev(g.standard_normal((nb, 1, N, K)).astype(np.float32))
+    res_wide = dev(g.standard_normal((nb, 1, N, M + 8)).astype(np.float32))
+    res = res_wide[..., :M]                      # a residual with its own row stride
+    prod = torch.empty((nb, 1, N, M), dtype=torch.float32, device="cuda")
+    a, b = torch.empty_like(prod), torch.empty_like(prod)
+    for s in (0.2857738, 1.0):
+        ok(pkg, L.vx_mul_mat(pkg.desc_q8(w, K), d(x), d(prod), mode, None), "mul_mat")
+        ok(pkg, L.vx_scale(d(prod), d(prod), s, 0.0, None), "scale")
+        ok(pkg, L.vx_binary(pkg.BIN_ADD, d(res), d(prod), d(a), None), "add")
+        ok(pkg, L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(x), d(res), d(b), s, mode, None), "mul_mat_scale_add")
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
+    # in place on the residual, the layout ggml-alloc gives the reference's graph
+    r2 = res.contiguous()
+    ok(pkg, L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(x), d(r2), d(r2), 1.0, mode, None), "mul_mat_scale_add in place")
+    torch.cuda.synchronize()
+    assert torch.equal(a, r2)
+    # token counts beyond the streaming kernel are refused, not computed some other way
+    xl = dev(np.zeros((1, 1, 17, K), dtype=np.float32))
+    rl = torch.zeros((1, 1, 17, M), dtype=torch.float32, device="cuda")
+    assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl)) == 0
+    assert L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl), 1.0, mode, None) != 0
+
+
+@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2)])
+@pytest.mark.parametrize("poison", [None, "nan", "inf"])
+def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):
+    import torch
+    say(f"fused cache write + ordering scalar B={B} T={T} Hkv={Hkv} D={D} poison={poison}")
+    L, d = pkg.lib(), pkg.desc
+    g = rng("f-kvs", B, T, Hkv, D)
+    max_len, n_past = 40, 17
+    k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    if poison == "nan":
+        k[0, 0, 0, 1] = float("nan")
+    if poison == "inf":
+        v[-1, -1, -1, -1] = float("inf")
+    attn = dev(g.standard_normal((B, T, H, D)).astype(np.float32))
+    caches = [torch.zeros((B, Hkv, max_len, D), dtype=torch.float32, device="cuda") for _ in range(4)]
+    kc1, vc1, kc2, vc2 = caches
+
+    def slot(c):  # the reference's write view [D, Hkv, T, B] of a cache [D, max_len, Hkv, B]
+        return c[:, :, n_past:n_past + T].transpose(1, 2)
+
+    for scale, bias in ((0.0, 0.0), (0.5, 0.0), (0.25, 1.5)):
+        # separate nodes: CPY, CONT, SUM (twice), ADD, SCALE, ADD1
+        cont = torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda")
+        sk, sv, sync = (torch.empty(1, dtype=torch.float32, device="cuda") for _ in range(3))
+        a = torch.empty_like(attn)
+        for src, c, s in ((k, kc1, sk), (v, vc1, sv)):
+            ok(pkg, L.vx_cpy(d(src), d(slot(c)), None), "cpy")
+            ok(pkg, L.vx_cpy(d(slot(c)), d(cont), None), "cont")
+            ok(pkg, L.vx_sum(d(cont), d(s), None), "sum")
+        ok(pkg, L.vx_binary(pkg.BIN_ADD, d(sk), d(sv), d(sync), None), "add")
+        ok(pkg, L.vx_scale(d(sync), d(sync), scale, bias, None), "scale")
+        ok(pkg, L.vx_add1(d(attn), d(sync), d(a), None), "add1")
+        # one launch
+        b = torch.empty_like(attn)
+        assert L.vx_supports_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(attn), d(b)) == 1
+        ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(attn), d(b), scale, bias, None), "kv_store_sync")
+        torch.cuda.synchronize()
+        assert same_bits(kc1, kc2) and same_bits(vc1, vc2)
+        assert torch.equal(torch.isnan(a), torch.isnan(b))
+        assert torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
+        if poison is None:
+            assert torch.equal(kc2[:, :, n_past:n_past + T], k.transpose(1, 2))
+        else:
+            assert not bool(torch.isfinite(b).any())   # a NaN or infinity in the cache write poisons the output, as in the reference
+    # in place on x, and a permuted source (ggml hands k over as a permuted view)
+    kp = k.transpose(1, 2).contiguous().transpose(1, 2)
+    x2 = attn.clone()
+    ok(pkg, L.vx_kv_store_sync(d(kp), d(slot(kc2)), d(v), d(slot(vc2)), d(x2), d(x2), 0.25, 1.5, None), "kv_store_sync in place")
+    torch.cuda.synchronize()
+    assert torch.equal(b.nan_to_num(123.0), x2.nan_to_num(123.0)) and same_bits(kc1, kc2)
+
+
+def test_kv_store_sync_limits(pkg, gpu):
+    import torch
+    say("fused cache write: sizes beyond one block are refused")
+    L, d = pkg.lib(), pkg.desc
+    k = torch.zeros((2, 512, 2, 64), dtype=torch.float32, device="cuda")
+    c = torch.zeros((2, 2, 600, 64), dtype=torch.float32, device="cuda")
+    x = torch.zeros((2, 512, 16, 64), dtype=torch.float32, device="cuda")
+    s = c[:, :, :512].transpose(1, 2)
+    assert L.vx_supports_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x)) == 0
+    assert L.vx_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x), 0.0, 0.0, None) != 0
+
+
+@pytest.mark.parametrize("shape", [(2, 512, 2, 64), (3, 70000), (1, 20000)])
+def test_sum_large_matches_fp64(pkg, gpu, shape):
+    import torch
+    say(f"sum over {shape}: several blocks, fp64 partials")
+    x = rng("f-sum", shape).standard_normal(shape).astype(np.float32)
+    got = gpu.sum_all(dev(x))
+    torch.cuda.synchronize()
+    want = np.float32(x.astype(np.float64).sum())
+    assert abs(float(got.cpu().numpy().reshape(-1)[0]) - float(want)) <= 2e-6 * max(1.0, abs(float(want)))

@@ -15,9 +15,10 @@ A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and i
 are built once, so a plan can be replayed from a captured HIP graph.
 
 With `fuse_pairs=True` the adjacent nodes the ggml backend plugin runs as one launch (rms_norm+mul,
-scale+add, cont+sum, add+scale, and the gate/up/SwiGLU triple at decode size) are issued as the plugin
-issues them, so a plan has as many launches as the plugin needs for the reference's graph; the results
-are bit-identical to the unfused sequence.
+scale+add, cont+sum, add+scale, and at decode size the gate/up/SwiGLU triple, projection+scale+add and
+the nine-node cache write with its ordering scalar) are issued as the plugin issues them, so a plan
+has as many launches as the plugin needs for the reference's graph; the results are bit-identical
+to the unfused sequence.
 """
 import math
 
@@ -100,6 +101,14 @@ class MiniCPMBackbone:
                 call(L.vx_rms_norm, desc(xin), desc(dst), self.eps)
                 call(L.vx_binary, BIN_MUL, desc(dst), desc(w), desc(dst))
 
+        def project_residual(wdesc, xin, branch, res, dst):  # projection, optional muP scale, residual add
+            sc = self.residual_scale if self.use_mup else 1.0
+            if fuse and L.vx_supports_mul_mat_scale_add(wdesc, desc(xin), desc(res), desc(dst)):
+                call(L.vx_mul_mat_scale_add, wdesc, desc(xin), desc(res), desc(dst), sc, self.act_mode)
+                return
+            call(L.vx_mul_mat, wdesc, desc(xin), desc(branch), self.act_mode)
+            residual(res, branch, dst)
+
         def residual(res, branch, dst):  # optional muP scale, then the residual add
             if self.use_mup and fuse:
                 call(L.vx_scale_add, desc(res), desc(branch), desc(dst), self.residual_scale)
@@ -156,10 +165,15 @@ class MiniCPMBackbone:
                 k_all, v_all = kall, vall
             call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
                  scale, 0.0, 0.0)
+            grouped = False
             if write_kv:
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236
                 vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
                 keep += [kw, vw]
+                grouped = bool(chain and fuse and L.vx_supports_kv_store_sync(desc(k4), desc(kw), desc(v4), desc(vw), desc(attn), desc(attn)))
+            if grouped:      # both cache writes, their sums, add, scale and add1 as one launch
+                call(L.vx_kv_store_sync, desc(k4), desc(kw), desc(v4), desc(vw), desc(attn), desc(attn), 0.0, 0.0)
+            elif write_kv:
                 for src4, wv, cont, ssum in ((k4, kw, kcont, sk), (v4, vw, vcont, sv)):
                     call(L.vx_cpy, desc(src4), desc(wv))
                     if chain and fuse:
@@ -167,15 +181,16 @@ class MiniCPMBackbone:
                     elif chain:
                         call(L.vx_cpy, desc(wv), desc(cont))
                         call(L.vx_sum, desc(cont), desc(ssum))
-            if chain and fuse:
+            if grouped:
+                pass
+            elif chain and fuse:
                 call(L.vx_add_scale, desc(sk), desc(sv), desc(sync), 0.0, 0.0)
             elif chain:
                 call(L.vx_binary, BIN_ADD, desc(sk), desc(sv), desc(sync))
                 call(L.vx_scale, desc(sync), desc(sync), 0.0, 0.0)
-            if chain:
+            if chain and not grouped:
                 call(L.vx_add1, desc(attn), desc(sync), desc(attn))
-            call(L.vx_mul_mat, wd["o_proj"], desc(attn.view(N, H * D)), desc(attn_o), self.act_mode)
-            residual(cur_x, attn_o, h_mid)
+            project_residual(wd["o_proj"], attn.view(N, H * D), attn_o, cur_x, h_mid)
             # -- mlp_forward
             norm(h_mid, nrm["post_layernorm"], normed)
             if fuse and N <= 16:     # gate, up and SwiGLU as one launch
@@ -184,9 +199,8 @@ class MiniCPMBackbone:
                 call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
                 call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
                 call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)
-            call(L.vx_mul_mat, wd["down_proj"], desc(act), desc(down), self.act_mode)
             nxt = hs[li % 2]
-            residual(h_mid, down, nxt)
+            project_residual(wd["down_proj"], act, down, h_mid, nxt)
             cur_x = nxt
         o2 = out.view(N, self.hidden)
         norm(cur_x, self.final_norm, o2)

@@ -231,17 +231,32 @@ __global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
 }
 
 // ---- SUM ---------------------------------------------------------------------------------------
-// ggml sums every element in double and rounds once (ops.cpp:1275-1300): one block, fp64 lanes, a
-// fixed reduction order.  Rows are dense (checked by the caller); 16-byte loads when VEC.
+// ggml sums every element in double and rounds once (ops.cpp:1275-1300): fp64 lanes, a fixed reduction
+// order.  Rows are dense (checked by the caller); 16-byte loads when VEC.  Small tensors (the ones
+// the decode graphs sum) take one block; large ones take SUM_BLOCKS blocks that leave fp64 partials for
+// a second, one-wave launch.
+constexpr int SUM_BLOCKS = 128;
+
+// the block's 1024 lane totals -> one double, the same value in every thread
+__device__ __forceinline__ double block_total(double acc, double * part /* 16 doubles of LDS */) {
+    acc = vx_wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    double t = 0.0;
+    for (int w = 0; w < 16; ++w) t += part[w];
+    __syncthreads(); // part may be written again
+    return t;
+}
+
 template <bool VEC>
-__global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst) {
+__global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst, double * partials) {
     __shared__ double part[16];
     constexpr int W = VEC ? 4 : 1;
     const uint32_t per_row = (uint32_t) (s.ne[0] / W);
     const uint32_t n = per_row * (uint32_t) (s.ne[1] * s.ne[2] * s.ne[3]); // < 2^24, checked by the caller
     const uint32_t ne1 = (uint32_t) s.ne[1], ne2 = (uint32_t) s.ne[2];
     double acc = 0.0;
-    for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+    for (uint32_t e = blockIdx.x * 1024 + threadIdx.x; e < n; e += gridDim.x * 1024) {
         const uint32_t row = e / per_row, iv = e - row * per_row;
         const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
         const char * p = src + (uint64_t) iv * (4 * W) + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3];
@@ -252,13 +267,106 @@ __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, 
             acc += (double) *(const float *) p;
         }
     }
-    acc = vx_wave_sum(acc);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
-    __syncthreads();
+    const double t = block_total(acc, part);
+    if (threadIdx.x == 0) {
+        if (partials) partials[blockIdx.x] = t;
+        else          *dst = (float) t;
+    }
+}
+
+__global__ __launch_bounds__(64) void sum_partials_kernel(const double * partials, int n, float * dst) {
     if (threadIdx.x == 0) {
         double t = 0.0;
-        for (int w = 0; w < 16; ++w) t += part[w];
+        for (int i = 0; i < n; ++i) t += partials[i];
         *dst = (float) t;
+    }
+}
+
+// ---- KV append + the reference's write-ordering scalar, one block ---------------------------------
+// attention_forward (src/minicpm.cpp:682-713) copies the new keys and values into their cache slots,
+// sums both copies, scales the total (by zero) and adds it to the attention output, so that the
+// writes are ancestors of the graph's result:
+//     CPY(k, k_slot) CONT SUM , CPY(v, v_slot) CONT SUM , ADD , SCALE , ADD1(x, .)
+// Here the block stores both slots, forms the two sums in sum_kernel's order (so the scalar is the
+// one the separate nodes produce, NaN and infinity included) and writes dst = x + scalar.
+constexpr int KVS_PRE = 4; // x elements per thread requested before anything else
+
+struct kvs_side {
+    const char * s; char * d;
+    int64_t  nes[4], ned[4];
+    uint64_t nbs[4], nbd[4];
+    int vec; // slot rows allow 16-byte accesses: the test vx_sum applies to its operand
+};
+
+struct kvs_args {
+    kvs_side k, v;
+    const char * x; char * d;
+    int64_t  ne[4];
+    uint64_t nbx[4], nbd[4];
+    float scale, bias;
+};
+
+template <bool VEC>
+__device__ __forceinline__ double store_and_sum(const kvs_side & a) {
+    constexpr int W = VEC ? 4 : 1;
+    const uint32_t ne0 = (uint32_t) a.ned[0], per_row = ne0 / W;
+    const uint32_t n = per_row * (uint32_t) (a.ned[1] * a.ned[2] * a.ned[3]);
+    const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
+    const uint32_t s0n = (uint32_t) a.nes[0], s1n = (uint32_t) a.nes[1], s2n = (uint32_t) a.nes[2];
+    double acc = 0.0;
+    for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+        const uint32_t row = e / per_row, iv = e - row * per_row;
+        const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
+        char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+        float v[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) { // element number row * ne0 + iv * W + k of the source, in its own shape
+            uint32_t r = row * ne0 + iv * W + k;
+            const uint32_t j0 = r % s0n; r /= s0n;
+            const uint32_t j1 = r % s1n; r /= s1n;
+            const uint32_t j2 = r % s2n, j3 = r / s2n;
+            v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
+        }
+        if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
+        else               *(float *) pd = v[0];
+#pragma unroll
+        for (int k = 0; k < W; ++k) acc += (double) v[k];
+    }
+    return acc;
+}
+
+__global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
+    __shared__ double part[16];
+    const uint32_t n0 = (uint32_t) a.ne[0], n1 = (uint32_t) a.ne[1], n2 = (uint32_t) a.ne[2];
+    const uint32_t nx = n0 * n1 * (uint32_t) (n2 * a.ne[3]);
+    auto offsets = [&](uint32_t e, uint64_t & ox, uint64_t & od) {
+        uint32_t r = e;
+        const uint32_t i0 = r % n0; r /= n0;
+        const uint32_t i1 = r % n1; r /= n1;
+        const uint32_t i2 = r % n2, i3 = r / n2;
+        ox = i0 * a.nbx[0] + i1 * a.nbx[1] + i2 * a.nbx[2] + i3 * a.nbx[3];
+        od = i0 * a.nbd[0] + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+    };
+    float    xv[KVS_PRE];
+    uint64_t xo[KVS_PRE];
+#pragma unroll
+    for (int p = 0; p < KVS_PRE; ++p) {
+        const uint32_t e = threadIdx.x + 1024 * p;
+        xv[p] = 0.0f; xo[p] = 0;
+        if (e < nx) { uint64_t ox; offsets(e, ox, xo[p]); xv[p] = *(const float *) (a.x + ox); }
+    }
+    const double ak = a.k.vec ? store_and_sum<true>(a.k) : store_and_sum<false>(a.k);
+    const float  sk = (float) block_total(ak, part);
+    const double av = a.v.vec ? store_and_sum<true>(a.v) : store_and_sum<false>(a.v);
+    const float  sv = (float) block_total(av, part);
+    const float  t  = sk + sv;                                                  // the ADD node
+    const float  y  = a.bias == 0.0f ? t * a.scale : fmaf(t, a.scale, a.bias);  // the SCALE node
+#pragma unroll
+    for (int p = 0; p < KVS_PRE; ++p)
+        if (threadIdx.x + 1024 * p < nx) *(float *) (a.d + xo[p]) = xv[p] + y;  // the ADD1 node
+    for (uint32_t e = threadIdx.x + 1024 * KVS_PRE; e < nx; e += 1024) {
+        uint64_t ox, od; offsets(e, ox, od);
+        *(float *) (a.d + od) = *(const float *) (a.x + ox) + y;
     }
 }
 
@@ -463,8 +571,54 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
     if (!vx_supports_sum(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "sum: F32 tensor of at most 2^24 elements to an F32 scalar");
     if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "sum: null data");
     const bool vec = src->ne[0] % 4 == 0 && al16(src->data, src->nb);
-    if (vec) sum_kernel<true><<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
-    else     sum_kernel<false><<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data);
+    hipStream_t st = (hipStream_t) stream;
+    const int64_t units = vx_nelements(src) / (vec ? 4 : 1);
+    double * partials = nullptr;
+    int blocks = 1;
+    if (units > 16 * 1024) { // more than 16 units per thread of one block: spread the walk
+        void * ws = nullptr;
+        const vx_status rc = vx_workspace(st, SUM_BLOCKS * sizeof(double), &ws);
+        if (rc != VX_OK) return rc;
+        partials = (double *) ws; blocks = SUM_BLOCKS;
+    }
+    if (vec) sum_kernel<true><<<dim3(blocks), dim3(1024), 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    else     sum_kernel<false><<<dim3(blocks), dim3(1024), 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    if (partials) sum_partials_kernel<<<dim3(1), dim3(64), 0, st>>>(partials, blocks, (float *) dst->data);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+static bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot) {
+    if (!f32(src) || !f32(slot) || !vx_positive(src)) return false;
+    if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > 16384) return false;
+    return slot->nb[0] == 4 && nb_multiple(slot, 4) && nb_multiple(src, 4);
+}
+
+extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                                         const vx_tensor * x, const vx_tensor * dst) {
+    if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;
+    if (!kvs_side_ok(k, k_slot) || !kvs_side_ok(v, v_slot)) return 0;
+    if (!f32(x) || !f32(dst) || !vx_positive(x) || !vx_same_shape(x, dst) || vx_nelements(x) > 65536) return 0;
+    return nb_multiple(x, 4) && nb_multiple(dst, 4);
+}
+
+extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                                      const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream) {
+    if (!vx_supports_kv_store_sync(k, k_slot, v, v_slot, x, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors, at most 16384 elements per cache write and 65536 in x");
+    if (!k->data || !k_slot->data || !v->data || !v_slot->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "kv_store_sync: null data");
+    kvs_args a;
+    auto side = [](kvs_side & o, const vx_tensor * src, const vx_tensor * slot) {
+        o.s = (const char *) src->data; o.d = (char *) slot->data;
+        for (int i = 0; i < 4; ++i) { o.nes[i] = src->ne[i]; o.ned[i] = slot->ne[i]; o.nbs[i] = src->nb[i]; o.nbd[i] = slot->nb[i]; }
+        o.vec = slot->ne[0] % 4 == 0 && al16(slot->data, slot->nb);
+    };
+    side(a.k, k, k_slot);
+    side(a.v, v, v_slot);
+    a.x = (const char *) x->data; a.d = (char *) dst->data;
+    for (int i = 0; i < 4; ++i) { a.ne[i] = x->ne[i]; a.nbx[i] = x->nb[i]; a.nbd[i] = dst->nb[i]; }
+    a.scale = scale; a.bias = bias;
+    kv_store_sync_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -37,7 +37,17 @@ struct mm_args {
     int w_aligned; // Q8_0 rows start on dword boundaries
     int rows_wg;   // GEMV: weight rows per work-group (16, 8 or 4)
     const char * w2; // GEMV, fused gate/up + SwiGLU: the second weight matrix (same shape and strides), else null
+    const char * res; // GEMV, fused residual update: dst = res + res_scale * (W x); null for a plain product
+    uint64_t rnb1, rnb2, rnb3;
+    float res_scale;
 };
+
+// a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
+__device__ __forceinline__ float scaled_residual(float x, float s, float a) {
+#pragma clang fp contract(off)
+    const float t = x * s;
+    return a + t;
+}
 
 constexpr int WT_Q8 = 0, WT_F16 = 1, WT_F32 = 2;
 constexpr int KC_BLOCKS = 4; // 32-wide k blocks staged per round
@@ -332,6 +342,14 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     };
     float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0};
     if (tid < units) fetch(tid, f0, f1);
+    // the residual values the storing wave will need, requested ahead of the weight stream as well
+    float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (a.res && wid == 0 && row_ok && c < Rr) {
+        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) (row0 + c) * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
+    }
     load_blocks(0);
     if (tid < units) stage(tid, f0, f1);
     for (int unit = tid + 64 * NW; unit < units; unit += 64 * NW) {
@@ -380,6 +398,10 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             const float up = __shfl(acc[r], lane + Rr, 64);
             acc[r] = (acc[r] / (1.0f + expf(-acc[r]))) * up;
         }
+    }
+    if (a.res) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = scaled_residual(acc[r], a.res_scale, resv[r]);
     }
     if (row_ok && c < Rr) {
 #pragma unroll
@@ -695,7 +717,7 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
     if (src0->type == VX_TYPE_F32 && (uintptr_t) src0->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: F32 weights must be 4-byte aligned");
     if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat: F32 tensors must be 4-byte aligned");
 
-    mm_args a;
+    mm_args a = {};
     a.w = (const char *) src0->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
     a.K = src0->ne[0]; a.M = src0->ne[1]; a.N = src1->ne[1];
     a.nb01 = src0->nb[1]; a.nb02 = src0->nb[2]; a.nb03 = src0->nb[3];
@@ -743,7 +765,7 @@ extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor *
     if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
     if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
         return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
-    mm_args a;
+    mm_args a = {};
     a.w = (const char *) gate->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
     a.K = gate->ne[0]; a.M = gate->ne[1]; a.N = src1->ne[1];
     a.nb01 = gate->nb[1]; a.nb02 = gate->nb[2]; a.nb03 = gate->nb[3];
@@ -761,6 +783,51 @@ extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor *
     if (gate->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
     else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
     if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: shape outside the streaming kernel");
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// MUL_MAT , SCALE , ADD as one launch for decode-sized token counts: dst = residual + scale * (W x)
+// (MiniCPMModel::layer_forward's residual updates, src/minicpm.cpp:749-786).  The product is formed
+// exactly as vx_mul_mat forms it and then rounded, scaled and added as the two separate nodes would.
+extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst) {
+    if (!vx_supports_mul_mat(src0, src1, dst) || !residual) return 0;
+    if (src0->type != VX_TYPE_Q8_0 && src0->type != VX_TYPE_F16) return 0;
+    if (residual->type != VX_TYPE_F32 || !vx_same_shape(residual, dst) || residual->nb[0] != 4) return 0;
+    if (residual->nb[1] % 4 || residual->nb[2] % 4 || residual->nb[3] % 4) return 0;
+    if (src1->ne[1] > 16 || src0->ne[0] % 32 || src0->ne[0] < 32) return 0;
+    return (size_t) src1->ne[1] * src0->ne[0] * 2 + (size_t) src1->ne[1] * (src0->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+}
+
+extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst,
+                                          float scale, int act_mode, vx_stream stream) {
+    if (!src0 || !src1 || !residual || !dst || !src0->data || !src1->data || !residual->data || !dst->data)
+        return vx_fail(VX_ERR_INVALID, "mul_mat_scale_add: null tensor");
+    if (!vx_supports_mul_mat_scale_add(src0, src1, residual, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: Q8_0/F16 weights, at most 16 tokens, F32 residual of dst's shape");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_scale_add: bad act_mode");
+    if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (uintptr_t) residual->data % 4 || (src0->type == VX_TYPE_F16 && (uintptr_t) src0->data % 2))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: misaligned tensor data");
+    mm_args a = {};
+    a.w = (const char *) src0->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
+    a.K = src0->ne[0]; a.M = src0->ne[1]; a.N = src1->ne[1];
+    a.nb01 = src0->nb[1]; a.nb02 = src0->nb[2]; a.nb03 = src0->nb[3];
+    a.nb11 = src1->nb[1]; a.nb12 = src1->nb[2]; a.nb13 = src1->nb[3];
+    a.nb1 = dst->nb[1]; a.nb2 = dst->nb[2]; a.nb3 = dst->nb[3];
+    a.ne12 = (int) src1->ne[2];
+    a.r2 = (int) (src1->ne[2] / src0->ne[2]); a.r3 = (int) (src1->ne[3] / src0->ne[3]);
+    a.rows_wg   = 16;
+    a.res       = (const char *) residual->data;
+    a.rnb1 = residual->nb[1]; a.rnb2 = residual->nb[2]; a.rnb3 = residual->nb[3];
+    a.res_scale = scale;
+    a.w_aligned = ((uintptr_t) src0->data % 4 == 0) && src0->nb[1] % 4 == 0 && src0->nb[2] % 4 == 0 && src0->nb[3] % 4 == 0;
+    a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
+    const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
+    hipStream_t st = (hipStream_t) stream;
+    bool ok;
+    if (src0->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
+    else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: shape outside the streaming kernel");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

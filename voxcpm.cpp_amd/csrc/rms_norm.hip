@@ -39,6 +39,7 @@ __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict
     const int64_t nvec = vec_ok ? ne00 / 4 : 0;
 
     float4 cache[RN_MAX_VEC];
+    float4 gain[RN_MAX_VEC]; // the weight row is requested together with x, not after the reduction
     double sum = 0.0;
     if (vec_ok) {
 #pragma unroll
@@ -46,6 +47,7 @@ __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict
             const int64_t iv = lane_id + (int64_t) c * nlanes;
             if (iv < nvec) {
                 const float4 v = ((const float4 *) x)[iv];
+                if (w) gain[c] = ((const float4 *) w)[iv];
                 cache[c]       = v;
                 sum += (double) (v.x * v.x);
                 sum += (double) (v.y * v.y);
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(BLOCK) void rms_norm_kernel(const char * __restrict
             if (iv < nvec) {
                 float4 v = cache[c];
                 v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
-                if (w) { const float4 g = ((const float4 *) w)[iv]; v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w; }
+                if (w) { const float4 g = gain[c]; v.x *= g.x; v.y *= g.y; v.z *= g.z; v.w *= g.w; }
                 ((float4 *) y)[iv] = v;
             }
         }

@@ -52,10 +52,15 @@ __global__ __launch_bounds__(256) void rope_kernel(const char * __restrict__ src
         return;
     }
 
+    // every load is requested before the angle arithmetic, so one memory round trip covers them all
+    const int ia = p.mode == 0 ? 2 * ip : ip;
+    const int ib = p.mode == 0 ? 2 * ip + 1 : ip + npairs;
+    const float x0 = x[ia], x1 = x[ib];
+    const float ff = freq_factors ? freq_factors[ip] : 1.0f;
+
     float theta = (float) pos[i2];
     for (int k = 0; k < ip; ++k) theta *= p.theta_scale;
 
-    const float ff           = freq_factors ? freq_factors[ip] : 1.0f;
     const float theta_extrap = theta / ff;
     const float theta_interp = p.freq_scale * theta_extrap;
     float       th           = theta_interp;
@@ -71,9 +76,6 @@ __global__ __launch_bounds__(256) void rope_kernel(const char * __restrict__ src
     const float c  = cosf(th) * mscale;
     const float sn = sinf(th) * mscale;
 
-    const int ia = p.mode == 0 ? 2 * ip : ip;
-    const int ib = p.mode == 0 ? 2 * ip + 1 : ip + npairs;
-    const float x0 = x[ia], x1 = x[ib];
     y[ia] = x0 * c - x1 * sn;
     y[ib] = x0 * sn + x1 * c;
 }

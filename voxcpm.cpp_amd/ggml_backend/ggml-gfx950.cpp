@@ -412,6 +412,26 @@ void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor
         GGML_ABORT("ggml-gfx950: get_tensor_async failed: %s", vx_last_error());
 }
 
+// ggml-alloc hands a node's output the memory of tensors that died before it.  Run as separate
+// launches that is harmless; one launch that covers several nodes writes the last node's output while
+// it may still be reading an operand of the first, so every group checks where its output lies.
+bool overlaps(const ggml_tensor * a, const ggml_tensor * b) {
+    if (!a || !b || !a->data || !b->data) return false;
+    const char * a0 = (const char *) a->data;
+    const char * b0 = (const char *) b->data;
+    return a0 < b0 + ggml_nbytes(b) && b0 < a0 + ggml_nbytes(a);
+}
+// operand that work-groups other than the one writing an output element read: must not touch dst
+bool apart(const ggml_tensor * dst, const ggml_tensor * in) { return !overlaps(dst, in); }
+// operand whose element i is read only by the thread that writes element i of dst: may also BE dst
+bool apart_or_same(const ggml_tensor * dst, const ggml_tensor * in) {
+    if (!overlaps(dst, in)) return true;
+    if (dst->data != in->data) return false;
+    for (int i = 0; i < GGML_MAX_DIMS; ++i)
+        if (dst->ne[i] != in->ne[i] || dst->nb[i] != in->nb[i]) return false;
+    return true;
+}
+
 // Two consecutive nodes as one launch, when the first one's value has no other reader (checked by
 // the caller).  Returns false when the pair is not one of the known shapes; *rc is the launch status.
 bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_status * rc) {
@@ -419,7 +439,7 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
     if (node->op == GGML_OP_RMS_NORM && next->op == GGML_OP_MUL && next->src[0] == node) {
         // MiniCPMModel::rms_norm: ggml_mul(ggml_rms_norm(x), weight)
         const vx_tensor s = to_vx(node->src[0]), w = to_vx(next->src[1]);
-        if (!vx_supports_rms_norm_mul(&s, &w, &d)) return false;
+        if (!vx_supports_rms_norm_mul(&s, &w, &d) || !apart_or_same(next, node->src[0]) || !apart(next, next->src[1])) return false;
         float eps;
         memcpy(&eps, node->op_params, sizeof(float));
         *rc = vx_rms_norm_mul(&s, &w, &d, eps, ctx->stream);
@@ -430,7 +450,7 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
         memcpy(&sc, (const float *) node->op_params + 0, sizeof(float));
         memcpy(&bias, (const float *) node->op_params + 1, sizeof(float));
         const vx_tensor a = to_vx(next->src[0]), x = to_vx(node->src[0]);
-        if (bias != 0.0f || !vx_supports_fused_pair(&a, &x, &d)) return false;
+        if (bias != 0.0f || !vx_supports_fused_pair(&a, &x, &d) || !apart_or_same(next, next->src[0]) || !apart_or_same(next, node->src[0])) return false;
         *rc = vx_scale_add(&a, &x, &d, sc, ctx->stream);
         return true;
     }
@@ -439,7 +459,7 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
         memcpy(&sc, (const float *) next->op_params + 0, sizeof(float));
         memcpy(&bias, (const float *) next->op_params + 1, sizeof(float));
         const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]);
-        if (!vx_supports_fused_pair(&a, &b, &d)) return false;
+        if (!vx_supports_fused_pair(&a, &b, &d) || !apart_or_same(next, node->src[0]) || !apart_or_same(next, node->src[1])) return false;
         *rc = vx_add_scale(&a, &b, &d, sc, bias, ctx->stream);
         return true;
     }
@@ -451,6 +471,8 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
         if (node->src[3]) m = to_vx(node->src[3]);
         if (node->src[4] && (node->src[4]->type != GGML_TYPE_F32 || node->src[4]->ne[0] != node->src[0]->ne[2])) return false;
         if (!vx_supports_flash_attn_ext(&q, &k, &v, node->src[3] ? &m : nullptr, &d)) return false;
+        for (int k_ = 0; k_ < 5; ++k_) if (!apart(next, node->src[k_])) return false;
+        if (!apart(next, next->src[1])) return false;
         float scale, max_bias, softcap;
         memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
         memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
@@ -462,11 +484,90 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
     if (node->op == GGML_OP_CONT && next->op == GGML_OP_SUM && next->src[0] == node) {
         // the sum does not care where the elements lie: read them where they are
         const vx_tensor s = to_vx(node->src[0]);
-        if (node->src[0]->type != GGML_TYPE_F32 || !vx_supports_sum(&s, &d)) return false;
+        if (node->src[0]->type != GGML_TYPE_F32 || !vx_supports_sum(&s, &d) || !apart(next, node->src[0])) return false;
         *rc = vx_sum(&s, &d, ctx->stream);
         return true;
     }
     return false;
+}
+
+typedef std::unordered_map<const ggml_tensor *, int> reader_map;
+
+// a node whose value only the group's next member looks at, so it need not be stored
+bool private_to_group(const reader_map & readers, const ggml_tensor * t) {
+    const auto it = readers.find(t);
+    return (t->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (t->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 && it != readers.end() && it->second == 1;
+}
+
+// index of the next node that does work (views and empty tensors are skipped), or n_nodes
+int next_real(const ggml_cgraph * g, int i) {
+    int k = i + 1;
+    while (k < g->n_nodes && (ggml_op_is_empty(g->nodes[k]->op) || ggml_is_empty(g->nodes[k]))) ++k;
+    return k;
+}
+
+// attention_forward's cache write and ordering scalar (src/minicpm.cpp:682-713) at decode size:
+//   CPY(k, slot) CONT SUM , CPY(v, slot) CONT SUM , ADD , SCALE , ADD1(attn, .)     -> one launch.
+// Returns the index of the group's last node, or -1.
+int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
+    ggml_tensor * n[9];
+    int idx = i;
+    for (int k = 0; k < 9; ++k) {
+        if (idx >= g->n_nodes) return -1;
+        n[k] = g->nodes[idx];
+        if ((n[k]->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return -1;
+        if (k < 8) idx = next_real(g, idx);
+    }
+    static const ggml_op want[9] = { GGML_OP_CPY, GGML_OP_CONT, GGML_OP_SUM, GGML_OP_CPY, GGML_OP_CONT, GGML_OP_SUM, GGML_OP_ADD, GGML_OP_SCALE, GGML_OP_ADD1 };
+    for (int k = 0; k < 9; ++k) if (n[k]->op != want[k]) return -1;
+    if (n[1]->src[0] != n[0] || n[2]->src[0] != n[1] || n[4]->src[0] != n[3] || n[5]->src[0] != n[4]) return -1;
+    if (!((n[6]->src[0] == n[2] && n[6]->src[1] == n[5]) || (n[6]->src[0] == n[5] && n[6]->src[1] == n[2]))) return -1;
+    if (n[7]->src[0] != n[6] || n[8]->src[1] != n[7]) return -1;
+    ggml_tensor * x = n[8]->src[0];
+    for (int k = 0; k < 8; ++k) if (x == n[k] || !private_to_group(readers, n[k])) return -1;
+    // the copies must be plain F32 -> F32 writes into the cache (the CPY node is a view of its destination)
+    for (int c = 0; c < 4; c += 3) {
+        if (n[c]->src[0]->type != GGML_TYPE_F32 || n[c]->type != GGML_TYPE_F32 || n[c]->src[1] == nullptr || n[c]->data != n[c]->src[1]->data) return -1;
+        if (n[c + 1]->type != GGML_TYPE_F32) return -1;
+    }
+    ggml_tensor * dst = n[8];
+    if (!apart(dst, n[0]->src[0]) || !apart(dst, n[3]->src[0]) || !apart(dst, n[0]) || !apart(dst, n[3]) || !apart_or_same(dst, x)) return -1;
+    if (!apart(n[0], x) || !apart(n[3], x) || !apart(n[0], n[3]->src[0]) || !apart(n[3], n[0]->src[0]) || !apart(n[0], n[3])) return -1;
+    const vx_tensor k = to_vx(n[0]->src[0]), ks = to_vx(n[0]), v = to_vx(n[3]->src[0]), vs = to_vx(n[3]), xx = to_vx(x), d = to_vx(dst);
+    if (!vx_supports_kv_store_sync(&k, &ks, &v, &vs, &xx, &d)) return -1;
+    float sc, bias;
+    memcpy(&sc, (const float *) n[7]->op_params + 0, sizeof(float));
+    memcpy(&bias, (const float *) n[7]->op_params + 1, sizeof(float));
+    *rc = vx_kv_store_sync(&k, &ks, &v, &vs, &xx, &d, sc, bias, ctx->stream);
+    return idx;
+}
+
+// layer_forward's residual updates (src/minicpm.cpp:762-777) at decode size:
+//   MUL_MAT(w, x) [SCALE] ADD(residual, .)   -> one launch.  Returns the index of the ADD, or -1.
+int compute_mul_mat_residual_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
+    ggml_tensor * mm = g->nodes[i];
+    if (mm->op != GGML_OP_MUL_MAT || !private_to_group(readers, mm) || i + 1 >= g->n_nodes) return -1;
+    ggml_tensor * val = mm;
+    float sc = 1.0f;
+    int ia = i + 1;
+    if (g->nodes[ia]->op == GGML_OP_SCALE) {
+        ggml_tensor * scn = g->nodes[ia];
+        float bias;
+        memcpy(&sc, (const float *) scn->op_params + 0, sizeof(float));
+        memcpy(&bias, (const float *) scn->op_params + 1, sizeof(float));
+        if (scn->src[0] != mm || bias != 0.0f || !private_to_group(readers, scn)) return -1;
+        val = scn;
+        if (++ia >= g->n_nodes) return -1;
+    }
+    ggml_tensor * add = g->nodes[ia];
+    if (add->op != GGML_OP_ADD || (add->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return -1;
+    ggml_tensor * residual = add->src[0] == val ? add->src[1] : add->src[0];
+    if ((add->src[0] != val && add->src[1] != val) || residual == val || residual == mm) return -1;
+    if (!apart(add, mm->src[0]) || !apart(add, mm->src[1]) || !apart_or_same(add, residual)) return -1;
+    const vx_tensor w = to_vx(mm->src[0]), x = to_vx(mm->src[1]), r = to_vx(residual), d = to_vx(add);
+    if (!vx_supports_mul_mat_scale_add(&w, &x, &r, &d)) return -1;
+    *rc = vx_mul_mat_scale_add(&w, &x, &r, &d, sc, mul_mat_act_mode(), ctx->stream);
+    return ia;
 }
 
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
@@ -481,7 +582,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
     // nodes is only run as one launch when nothing else looks at the value between them
     static const bool fusion = getenv("GGML_GFX950_NO_FUSION") == nullptr;
-    std::unordered_map<const ggml_tensor *, int> readers;
+    reader_map readers;
     if (fusion && cgraph->n_nodes > 1) {
         readers.reserve((size_t) cgraph->n_nodes * 2);
         for (int i = 0; i < cgraph->n_nodes; ++i) {
@@ -499,6 +600,15 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         vx_status rc = VX_ERR_UNSUPPORTED;
         bool fused = false;
         if (fusion && i + 1 < cgraph->n_nodes) {
+            int last = -1;
+            if (node->op == GGML_OP_CPY) last = compute_kv_store_group(ctx, cgraph, i, readers, &rc);
+            else if (node->op == GGML_OP_MUL_MAT) last = compute_mul_mat_residual_group(ctx, cgraph, i, readers, &rc);
+            if (last >= 0) {
+                fused = true;
+                i = last - 1; // the common increment below steps onto the group's last node
+            }
+        }
+        if (!fused && fusion && i + 1 < cgraph->n_nodes) {
             ggml_tensor * next = cgraph->nodes[i + 1];
             const bool private_value = (node->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (next->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 &&
                                        readers[node] == 1;
@@ -509,7 +619,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
                     ggml_get_glu_op(glu) == GGML_GLU_OP_SWIGLU && ((const int32_t *) glu->op_params)[1] == 0 &&
                     next->src[1] == node->src[1] && (next->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && readers[next] == 1) {
                     const vx_tensor g = to_vx(node->src[0]), u = to_vx(next->src[0]), x = to_vx(node->src[1]), d = to_vx(glu);
-                    if (vx_supports_mul_mat_swiglu(&g, &u, &x, &d)) {
+                    if (vx_supports_mul_mat_swiglu(&g, &u, &x, &d) && apart(glu, node->src[1])) {
                         rc = vx_mul_mat_swiglu(&g, &u, &x, &d, mul_mat_act_mode(), ctx->stream);
                         fused = true;
                         ++i; // one more node than a pair
