@@ -191,6 +191,19 @@ VX_API vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k
                                         const vx_tensor * mask, const float * sinks, const float * addend,
                                         const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
                                         vx_stream stream);
+/* CONCAT(k_past, k_cur, dim 1) , CONCAT(v_past, v_cur, dim 1) -> FLASH_ATTN_EXT: the reference appends the step's
+ * keys and values to the cached ones before attention (attention_forward, src/minicpm.cpp:694-706).  Here the
+ * kernel reads keys 0 .. ne1(k_past)-1 from k_past / v_past and the rest from k_cur / v_cur, so the
+ * concatenated tensors are never written.  Both segments of one type, head_dim, head and batch counts; mask
+ * over all keys.  Query counts the LDS-tiled prefill kernel would take are not supported (use CONCAT).
+ * Result identical to vx_concat x2 + vx_flash_attn_ext. */
+VX_API vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                       const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                       const float * sinks, const vx_tensor * dst, float scale, float max_bias,
+                                       float logit_softcap, vx_stream stream);
+VX_API int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                          const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                          const vx_tensor * dst);
 /* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for at most 16 tokens
  * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,

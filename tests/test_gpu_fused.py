@@ -230,3 +230,54 @@ def test_sum_large_matches_fp64(pkg, gpu, shape):
     torch.cuda.synchronize()
     want = np.float32(x.astype(np.float64).sum())
     assert abs(float(got.cpu().numpy().reshape(-1)[0]) - float(want)) <= 2e-6 * max(1.0, abs(float(want)))
+
+
+@pytest.mark.parametrize("T,n_past,kv_f16,D", [(1, 639, False, 64), (1, 4095, True, 64), (1, 100, True, 128), (2, 31, False, 64),
+                                                (5, 1000, False, 128), (1, 1, True, 64), (40, 24, True, 64)])
+def test_flash_attn_two_segments(pkg, gpu, T, n_past, kv_f16, D):
+    import torch
+    say(f"attention over cached + current keys T={T} n_past={n_past} f16={kv_f16} D={D}")
+    L, d = pkg.lib(), pkg.desc
+    B, H, Hkv = 2, 16, 2
+    g = rng("f-kv2", T, n_past, D)
+    kt = torch.float16 if kv_f16 else torch.float32
+    q = dev(g.standard_normal((B, H, T, D)).astype(np.float32))
+    cache_k = dev(g.standard_normal((B, Hkv, n_past + 7, D)).astype(np.float32)).to(kt)
+    cache_v = dev(g.standard_normal((B, Hkv, n_past + 7, D)).astype(np.float32)).to(kt)
+    kp, vp = cache_k[:, :, :n_past], cache_v[:, :, :n_past]          # views of a longer cache
+    # the step's keys as the projection leaves them, [B, T, Hkv, D], seen through ggml_permute(0, 2, 1, 3)
+    kc = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32)).to(kt).transpose(1, 2)
+    vc = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32)).to(kt).transpose(1, 2)
+    n_kv = n_past + T
+    mask = dev(reflib.causal_mask(T, n_kv, n_past)) if T > 1 else None
+    kall = torch.empty((B, Hkv, n_kv, D), dtype=kt, device="cuda")
+    vall = torch.empty_like(kall)
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    ok(pkg, L.vx_concat(d(kp), d(kc), d(kall), 1, None), "concat k")
+    ok(pkg, L.vx_concat(d(vp), d(vc), d(vall), 1, None), "concat v")
+    sc = 1.0 / np.sqrt(D)
+    ok(pkg, L.vx_flash_attn_ext(d(q), d(kall), d(vall), d(mask), None, d(a), sc, 0.0, 0.0, None), "fa")
+    assert L.vx_supports_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(vp), d(vc), d(mask), d(b)) == 1
+    ok(pkg, L.vx_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(vp), d(vc), d(mask), None, d(b), sc, 0.0, 0.0, None), "fa_kv2")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_flash_attn_two_segments_declines_prefill_shapes(pkg, gpu):
+    import torch
+    say("two-segment attention leaves prefill-sized f16 shapes to concat + the tiled kernel")
+    L, d = pkg.lib(), pkg.desc
+    B, H, Hkv, D, T, n_past = 2, 16, 2, 64, 512, 512
+    q = torch.zeros((B, H, T, D), dtype=torch.float32, device="cuda")
+    kp = torch.zeros((B, Hkv, n_past, D), dtype=torch.float16, device="cuda")
+    kc = torch.zeros((B, Hkv, T, D), dtype=torch.float16, device="cuda")
+    mask = dev(reflib.causal_mask(T, n_past + T, n_past))
+    o = torch.zeros((B, T, H, D), dtype=torch.float32, device="cuda")
+    assert L.vx_supports_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(kp), d(kc), d(mask), d(o)) == 0
+    assert L.vx_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(kp), d(kc), d(mask), None, d(o), 0.125, 0.0, 0.0, None) != 0
+    # mismatched segment types are refused as well
+    kc32 = kc[:, :, :1].float()
+    q1 = q[:, :, :1].contiguous()
+    o1 = torch.zeros((B, 1, H, D), dtype=torch.float32, device="cuda")
+    assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp), d(kc32), d(kp), d(kc32), None, d(o1)) == 0

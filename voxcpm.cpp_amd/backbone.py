@@ -15,8 +15,9 @@ A `plan` is the prepared call list for one (n_tokens, n_past): descriptors and i
 are built once, so a plan can be replayed from a captured HIP graph.
 
 With `fuse_pairs=True` the adjacent nodes the ggml backend plugin runs as one launch (rms_norm+mul,
-scale+add, cont+sum, add+scale, and at decode size the gate/up/SwiGLU triple, projection+scale+add and
-the nine-node cache write with its ordering scalar) are issued as the plugin issues them, so a plan
+scale+add, cont+sum, add+scale, and at decode size the gate/up/SwiGLU triple, projection+scale+add, the
+nine-node cache write with its ordering scalar, and attention over cached + current keys without the
+two concats) are issued as the plugin issues them, so a plan
 has as many launches as the plugin needs for the reference's graph; the results are bit-identical
 to the unfused sequence.
 """
@@ -160,11 +161,24 @@ class MiniCPMBackbone:
                     call(L.vx_cpy, desc(k_all), desc(kcast))
                     call(L.vx_cpy, desc(v_all), desc(vcast))
                     k_all, v_all = kcast, vcast
-                call(L.vx_concat, desc(kc[:, :, :n_past]), desc(k_all), desc(kall), 1)
-                call(L.vx_concat, desc(vc[:, :, :n_past]), desc(v_all), desc(vall), 1)
-                k_all, v_all = kall, vall
-            call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
-                 scale, 0.0, 0.0)
+                kp, vp = kc[:, :, :n_past], vc[:, :, :n_past]
+                qd = desc(q4.transpose(1, 2))
+                # The plugin lets attention read the cached and the current keys where they lie (no concat) when the
+                # current keys are still alive at the attention node.  In the reference's graph they are when the
+                # cache write, their other reader, comes later: F32 cache with write_kv.  The F16 cast of the
+                # current keys dies at the concat and ggml-alloc hands its memory on, so there the concats stay.
+                alive = write_kv and kcast is None
+                if fuse and alive and L.vx_supports_flash_attn_ext_kv2(qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), desc(attn)):
+                    call(L.vx_flash_attn_ext_kv2, qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), None, desc(attn),
+                         scale, 0.0, 0.0)
+                    k_all = None
+                else:
+                    call(L.vx_concat, desc(kp), desc(k_all), desc(kall), 1)
+                    call(L.vx_concat, desc(vp), desc(v_all), desc(vall), 1)
+                    k_all, v_all = kall, vall
+            if k_all is not None:
+                call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
+                     scale, 0.0, 0.0)
             grouped = False
             if write_kv:
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236

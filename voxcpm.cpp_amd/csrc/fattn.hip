@@ -47,6 +47,11 @@ struct fa_args {
     float * part_o;   // [tile][split][16 columns][D]   split partials, un-normalised
     float * part_ml;  // [tile][split][16 columns][2]   running max, running sum
     uint64_t nbq1, nbq2, nbq3, nbk1, nbk2, nbk3, nbv1, nbv2, nbv3, nbm1, nbm2, nbm3;
+    // keys n_kv1 .. n_kv-1 may lie in a second pair of tensors (the current step's K and V, which the
+    // reference appends to the cached ones with GGML_OP_CONCAT before attention); null = one segment
+    const char * k2; const char * v2;
+    uint64_t nbk1b, nbk2b, nbk3b, nbv1b, nbv2b, nbv3b;
+    int n_kv1;
     int n_q, n_kv, Hq, Hkv, gqa, ne3, rk3, nem2, nem3;
     int n_col_tiles, n_splits, chunk;
     float scale, softcap, max_bias, m0, m1;
@@ -111,7 +116,7 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
 }
 
 // One wave (= one block) = 16 columns x one key range.
-template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP>
+template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP, bool TWO_SEG>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fattn_cols16_kernel(const fa_args a) {
     constexpr int NP  = D / 32;          // MFMAs along the head dimension
     constexpr int SEG = D / 4;           // elements of a row owned by lane-group j
@@ -136,21 +141,36 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     const char * kbase = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3 + (uint64_t) (SEG * j) * ES;
     const char * vbase = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3 + (uint64_t) (SEG * j) * ES;
 
+    const char * kbase2 = kbase;
+    const char * vbase2 = vbase;
+    if constexpr (TWO_SEG) {
+        kbase2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) (b / a.rk3) * a.nbk3b + (uint64_t) (SEG * j) * ES;
+        vbase2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) (b / a.rk3) * a.nbv3b + (uint64_t) (SEG * j) * ES;
+    }
+
     const int kv0 = sp * a.chunk;
     const int kv1 = min(a.n_kv, kv0 + a.chunk);
 
     // rows this lane loads (MFMA row c of each 16-key half); clamped, masked out later
     auto load_tile = [&](int kb, kv_tile<NP, KV_F32> & t) {
         const int key0 = min(kb + c, a.n_kv - 1), key1 = min(kb + 16 + c, a.n_kv - 1);
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            kv_load<KV_F32>::run(kbase + (uint64_t) key0 * a.nbk1 + p * 8 * ES, t.khi[0][p], t.klo[0][p]);
-            kv_load<KV_F32>::run(kbase + (uint64_t) key1 * a.nbk1 + p * 8 * ES, t.khi[1][p], t.klo[1][p]);
+        const char * k0p = kbase + (uint64_t) key0 * a.nbk1;
+        const char * k1p = kbase + (uint64_t) key1 * a.nbk1;
+        const char * v0p = vbase + (uint64_t) key0 * a.nbv1;
+        const char * v1p = vbase + (uint64_t) key1 * a.nbv1;
+        if constexpr (TWO_SEG) {
+            if (key0 >= a.n_kv1) { k0p = kbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbk1b; v0p = vbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbv1b; }
+            if (key1 >= a.n_kv1) { k1p = kbase2 + (uint64_t) (key1 - a.n_kv1) * a.nbk1b; v1p = vbase2 + (uint64_t) (key1 - a.n_kv1) * a.nbv1b; }
         }
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            kv_load<KV_F32>::run(vbase + (uint64_t) key0 * a.nbv1 + p * 8 * ES, t.vhi[0][p], t.vlo[0][p]);
-            kv_load<KV_F32>::run(vbase + (uint64_t) key1 * a.nbv1 + p * 8 * ES, t.vhi[1][p], t.vlo[1][p]);
+            kv_load<KV_F32>::run(k0p + p * 8 * ES, t.khi[0][p], t.klo[0][p]);
+            kv_load<KV_F32>::run(k1p + p * 8 * ES, t.khi[1][p], t.klo[1][p]);
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            kv_load<KV_F32>::run(v0p + p * 8 * ES, t.vhi[0][p], t.vlo[0][p]);
+            kv_load<KV_F32>::run(v1p + p * 8 * ES, t.vhi[1][p], t.vlo[1][p]);
         }
     };
 
@@ -426,12 +446,18 @@ bool aligned16(const vx_tensor * t) {
 template <int D, bool KV_F32>
 void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
     const dim3 grid((unsigned) nblocks), block(64);
+    if (a.k2) {
+        if (a.softcap != 0.0f) fattn_cols16_kernel<D, KV_F32, true, true, true><<<grid, block, 0, st>>>(a);
+        else if (a.mask)       fattn_cols16_kernel<D, KV_F32, true, false, true><<<grid, block, 0, st>>>(a);
+        else                   fattn_cols16_kernel<D, KV_F32, false, false, true><<<grid, block, 0, st>>>(a);
+        return;
+    }
     if (a.softcap != 0.0f) { // rare: always take the masked variant
-        fattn_cols16_kernel<D, KV_F32, true, true><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, true, true, false><<<grid, block, 0, st>>>(a);
     } else if (a.mask) {
-        fattn_cols16_kernel<D, KV_F32, true, false><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, true, false, false><<<grid, block, 0, st>>>(a);
     } else {
-        fattn_cols16_kernel<D, KV_F32, false, false><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, false, false, false><<<grid, block, 0, st>>>(a);
     }
 }
 
@@ -469,6 +495,13 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
     return vx_flash_attn_ext_add1(q, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, stream);
 }
 
+// K/V as one tensor each (k2 == v2 == null) or as two key segments: k, v hold keys 0 .. n_kv1-1 and
+// k2, v2 the rest; kall / vall describe the whole (for the one-segment case they are k and v).
+static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * k2, const vx_tensor * v2,
+                        const vx_tensor * kall, const vx_tensor * vall, const vx_tensor * mask, const float * sinks,
+                        const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
+                        hipStream_t st);
+
 extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
                                             const vx_tensor * mask, const float * sinks, const float * addend,
                                             const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
@@ -489,7 +522,60 @@ extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor
             if (rc != VX_ERR_UNSUPPORTED) return rc;
         }
     }
+    return fa_run(q, k, v, nullptr, nullptr, k, v, mask, sinks, addend, dst, scale, max_bias, logit_softcap, st);
+}
+
+// CONCAT(k_past, k_cur) , CONCAT(v_past, v_cur) , FLASH_ATTN_EXT as one launch that reads both segments
+// where they lie.  The whole of K (V) has the first segment's shape with ne[1] = the two key counts added.
+static bool kv2_whole(const vx_tensor * a, const vx_tensor * b, vx_tensor * whole) {
+    if (!a || !b || a->type != b->type || !vx_positive(a) || !vx_positive(b)) return false;
+    if (a->ne[0] != b->ne[0] || a->ne[2] != b->ne[2] || a->ne[3] != b->ne[3]) return false;
+    if (b->nb[0] != vx_type_size(b->type)) return false;
+    for (int i = 1; i < 4; ++i) if (b->nb[i] % 16) return false;
+    *whole = *a;
+    whole->ne[1] = a->ne[1] + b->ne[1];
+    return true;
+}
+
+extern "C" int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                              const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                              const vx_tensor * dst) {
+    vx_tensor kall, vall;
+    if (!q || !kv2_whole(k_past, k_cur, &kall) || !kv2_whole(v_past, v_cur, &vall)) return 0;
+    if (k_past->ne[1] != v_past->ne[1]) return 0;
+    if (!vx_supports_flash_attn_ext(q, &kall, &vall, mask, dst)) return 0;
+    // a shape the LDS-tiled kernel would take as one tensor stays with it (same results either way)
+    return vx_fattn_prefill_accepts(q, &kall, 0.0f) ? 0 : 1;
+}
+
+extern "C" vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                           const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                           const float * sinks, const vx_tensor * dst, float scale, float max_bias,
+                                           float logit_softcap, vx_stream stream) {
+    if (!q || !k_past || !k_cur || !v_past || !v_cur || !dst || !q->data || !k_past->data || !k_cur->data || !v_past->data ||
+        !v_cur->data || !dst->data || (mask && !mask->data))
+        return vx_fail(VX_ERR_INVALID, "flash_attn_ext_kv2: null tensor");
+    if (!vx_supports_flash_attn_ext_kv2(q, k_past, k_cur, v_past, v_cur, mask, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_kv2: two K/V segments of one type and head layout, otherwise as flash_attn_ext; decode-sized query counts");
+    if (!aligned16(q) || !aligned16(k_past) || !aligned16(v_past) || !aligned16(k_cur) || !aligned16(v_cur) || (uintptr_t) dst->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_kv2: tensor data must be 16-byte aligned");
+    if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_kv2: max_bias > 0 requires a mask");
+    vx_tensor kall, vall;
+    kv2_whole(k_past, k_cur, &kall);
+    kv2_whole(v_past, v_cur, &vall);
+    return fa_run(q, k_past, v_past, k_cur, v_cur, &kall, &vall, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream);
+}
+
+static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * k2, const vx_tensor * v2,
+                        const vx_tensor * kall, const vx_tensor * vall, const vx_tensor * mask, const float * sinks,
+                        const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
+                        hipStream_t st) {
+    (void) vall;
     fa_args a;
+    a.k2 = k2 ? (const char *) k2->data : nullptr; a.v2 = v2 ? (const char *) v2->data : nullptr;
+    a.nbk1b = k2 ? k2->nb[1] : 0; a.nbk2b = k2 ? k2->nb[2] : 0; a.nbk3b = k2 ? k2->nb[3] : 0;
+    a.nbv1b = v2 ? v2->nb[1] : 0; a.nbv2b = v2 ? v2->nb[2] : 0; a.nbv3b = v2 ? v2->nb[3] : 0;
+    a.n_kv1 = (int) k->ne[1];
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
     a.mask = mask ? (const char *) mask->data : nullptr;
     a.sinks = sinks;
@@ -500,7 +586,7 @@ extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor
     a.nbk1 = k->nb[1]; a.nbk2 = k->nb[2]; a.nbk3 = k->nb[3];
     a.nbv1 = v->nb[1]; a.nbv2 = v->nb[2]; a.nbv3 = v->nb[3];
     a.nbm1 = mask ? mask->nb[1] : 0; a.nbm2 = mask ? mask->nb[2] : 0; a.nbm3 = mask ? mask->nb[3] : 0;
-    a.n_q = (int) q->ne[1]; a.n_kv = (int) k->ne[1]; a.Hq = (int) q->ne[2]; a.Hkv = (int) k->ne[2];
+    a.n_q = (int) q->ne[1]; a.n_kv = (int) kall->ne[1]; a.Hq = (int) q->ne[2]; a.Hkv = (int) k->ne[2];
     a.gqa = a.Hq / a.Hkv; a.ne3 = (int) q->ne[3]; a.rk3 = (int) (q->ne[3] / k->ne[3]);
     a.nem2 = mask ? (int) mask->ne[2] : 1; a.nem3 = mask ? (int) mask->ne[3] : 1;
     a.scale = scale; a.softcap = logit_softcap; a.max_bias = max_bias;

@@ -418,19 +418,27 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 
 // Called by vx_flash_attn_ext when the shape suits this kernel; returns VX_ERR_UNSUPPORTED
 // (without touching the error string) when the caller should use the general kernel.
-vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
-                           const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
-                           float logit_softcap, hipStream_t st) {
-    if (q->ne[0] != 64 || logit_softcap != 0.0f) return VX_ERR_UNSUPPORTED;
+bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float logit_softcap) {
+    if (q->ne[0] != 64 || logit_softcap != 0.0f) return false;
     // F32 K/V would be rounded to f16 here (error up to ~1e-3); the general kernel keeps hi + lo parts
-    if (k->type != VX_TYPE_F16) return VX_ERR_UNSUPPORTED;
+    if (k->type != VX_TYPE_F16) return false;
     const int Hq = (int) q->ne[2], Hkv = (int) k->ne[2], gqa = Hq / Hkv;
-    if (gqa > PF_COLS || (PF_COLS % gqa) != 0) return VX_ERR_UNSUPPORTED;
+    if (gqa > PF_COLS || (PF_COLS % gqa) != 0) return false;
     const int n_q = (int) q->ne[1], n_kv = (int) k->ne[1];
     const int RB = PF_COLS / gqa, n_rb = (n_q + RB - 1) / RB, n_tiles = (n_kv + PF_KT - 1) / PF_KT;
     const int n_groups = (int) q->ne[3] * Hkv;
-    if (n_q * gqa < PF_COLS || n_tiles > PF_MAX_TILES) return VX_ERR_UNSUPPORTED;
-    if ((int64_t) n_rb * n_groups < 64) return VX_ERR_UNSUPPORTED; // too few work-groups: the wave kernel spreads wider
+    if (n_q * gqa < PF_COLS || n_tiles > PF_MAX_TILES) return false;
+    return (int64_t) n_rb * n_groups >= 64; // too few work-groups: the wave kernel spreads wider
+}
+
+vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                           const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
+                           float logit_softcap, hipStream_t st) {
+    if (!vx_fattn_prefill_accepts(q, k, logit_softcap)) return VX_ERR_UNSUPPORTED;
+    const int Hq = (int) q->ne[2], Hkv = (int) k->ne[2], gqa = Hq / Hkv;
+    const int n_q = (int) q->ne[1], n_kv = (int) k->ne[1];
+    const int RB = PF_COLS / gqa, n_rb = (n_q + RB - 1) / RB, n_tiles = (n_kv + PF_KT - 1) / PF_KT;
+    const int n_groups = (int) q->ne[3] * Hkv;
 
     pf_args a;
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;

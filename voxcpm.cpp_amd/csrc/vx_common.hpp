@@ -46,6 +46,9 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
                            const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
                            float logit_softcap, hipStream_t stream);
 
+// whether vx_fattn_prefill would take this shape (k describes all keys)
+bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float logit_softcap);
+
 // ---- host-side tensor predicates ---------------------------------------------------------
 static inline size_t vx_type_size(int type) {
     switch (type) {

@@ -570,6 +570,61 @@ int compute_mul_mat_residual_group(backend_ctx * ctx, const ggml_cgraph * g, int
     return ia;
 }
 
+// attention_forward appends the step's keys and values to the cached ones with two CONCATs and hands
+// the results to FLASH_ATTN_EXT (src/minicpm.cpp:694-706).  When nothing else reads the concatenated
+// tensors, the attention kernel reads both segments where they lie and the CONCATs are never run.
+// The CONCATs' operands must then still be intact when the attention node is reached: no node in
+// between (nor the attention's own output) may have been given their memory.
+struct kv2_group { const ggml_tensor * kcat; const ggml_tensor * vcat; };
+
+void find_kv2_groups(const ggml_cgraph * g, const reader_map & readers, std::unordered_map<const ggml_tensor *, kv2_group> & by_fa,
+                     std::unordered_map<const ggml_tensor *, const ggml_tensor *> & absorbed) {
+    for (int i = 0; i < g->n_nodes; ++i) {
+        const ggml_tensor * f = g->nodes[i];
+        if (f->op != GGML_OP_FLASH_ATTN_EXT || (f->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+        const ggml_tensor * cat[2] = { f->src[1], f->src[2] };
+        int at[2] = { -1, -1 };
+        bool ok = true;
+        for (int c = 0; c < 2 && ok; ++c) {
+            ok = cat[c] && cat[c]->op == GGML_OP_CONCAT && ((const int32_t *) cat[c]->op_params)[0] == 1 && private_to_group(readers, cat[c]) &&
+                 absorbed.find(cat[c]) == absorbed.end();
+            for (int k = i - 1; ok && k >= 0 && k >= i - 32; --k)
+                if (g->nodes[k] == cat[c]) { at[c] = k; break; }
+            ok = ok && at[c] >= 0;
+        }
+        if (!ok || cat[0] == cat[1]) continue;
+        if (f->src[4] && (f->src[4]->type != GGML_TYPE_F32 || f->src[4]->ne[0] != f->src[0]->ne[2])) continue;
+        const vx_tensor q = to_vx(f->src[0]), kp = to_vx(cat[0]->src[0]), kc = to_vx(cat[0]->src[1]), vp = to_vx(cat[1]->src[0]),
+                        vc = to_vx(cat[1]->src[1]), d = to_vx(f);
+        vx_tensor m;
+        if (f->src[3]) m = to_vx(f->src[3]);
+        if (!vx_supports_flash_attn_ext_kv2(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, &d)) continue;
+        for (int c = 0; c < 2 && ok; ++c)
+            for (int k = at[c] + 1; k <= i && ok; ++k) {
+                const ggml_tensor * n = g->nodes[k];
+                if (n == cat[0] || n == cat[1] || ggml_op_is_empty(n->op) || ggml_is_empty(n) || (n->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+                ok = apart(n, cat[c]->src[0]) && apart(n, cat[c]->src[1]);
+            }
+        if (!ok) continue;
+        by_fa[f] = kv2_group{ cat[0], cat[1] };
+        absorbed[cat[0]] = f;
+        absorbed[cat[1]] = f;
+    }
+}
+
+vx_status compute_kv2_attention(backend_ctx * ctx, const ggml_tensor * f, const kv2_group & grp) {
+    float scale, max_bias, softcap;
+    memcpy(&scale, (const float *) f->op_params + 0, sizeof(float));
+    memcpy(&max_bias, (const float *) f->op_params + 1, sizeof(float));
+    memcpy(&softcap, (const float *) f->op_params + 2, sizeof(float));
+    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcat->src[1]), vp = to_vx(grp.vcat->src[0]),
+                    vc = to_vx(grp.vcat->src[1]), d = to_vx(f);
+    vx_tensor m;
+    if (f->src[3]) m = to_vx(f->src[3]);
+    return vx_flash_attn_ext_kv2(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
+                                 &d, scale, max_bias, softcap, ctx->stream);
+}
+
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
 
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
@@ -592,13 +647,29 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
             if (n->view_src) readers[n->view_src]++;
         }
     }
+    std::unordered_map<const ggml_tensor *, kv2_group> kv2_by_fa;
+    std::unordered_map<const ggml_tensor *, const ggml_tensor *> kv2_absorbed;
+    if (fusion && cgraph->n_nodes > 2) find_kv2_groups(cgraph, readers, kv2_by_fa, kv2_absorbed);
     for (int i = 0; i < cgraph->n_nodes; ++i) {
         ggml_tensor * node = cgraph->nodes[i];
         // the same two skips ggml-cpu applies (ggml/src/ggml-cpu/ggml-cpu.c:2956-2966)
         if (ggml_op_is_empty(node->op) || ggml_is_empty(node)) continue;
         if ((node->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+        if (kv2_absorbed.count(node)) continue; // a CONCAT the attention node reads through
         vx_status rc = VX_ERR_UNSUPPORTED;
         bool fused = false;
+        if (node->op == GGML_OP_FLASH_ATTN_EXT) {
+            const auto it = kv2_by_fa.find(node);
+            if (it != kv2_by_fa.end()) {
+                rc = compute_kv2_attention(ctx, node, it->second);
+                ++launches;
+                if (rc != VX_OK) {
+                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, two-segment attention) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    return GGML_STATUS_FAILED;
+                }
+                continue;
+            }
+        }
         if (fusion && i + 1 < cgraph->n_nodes) {
             int last = -1;
             if (node->op == GGML_OP_CPY) last = compute_kv_store_group(ctx, cgraph, i, readers, &rc);
