@@ -204,6 +204,19 @@ VX_API vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_
 VX_API int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
                                           const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
                                           const vx_tensor * dst);
+/* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
+ * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for at most 16
+ * tokens.  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE
+ * outputs [head_dim, heads, tokens, batch] and v_dst the third product, shaped like x with rows for K, all contiguous.  mode must be NEOX (2) with n_dims ==
+ * head_dim; the remaining arguments are vx_rope's.  Results equal vx_mul_mat x3 + vx_rope x2 bit for bit. */
+VX_API vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
+                                  const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst,
+                                  const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig,
+                                  float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast,
+                                  float beta_slow, int act_mode, vx_stream stream);
+VX_API int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
+                                     const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims,
+                                     int mode);
 /* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for at most 16 tokens
  * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,

@@ -281,3 +281,51 @@ def test_flash_attn_two_segments_declines_prefill_shapes(pkg, gpu):
     q1 = q[:, :, :1].contiguous()
     o1 = torch.zeros((B, 1, H, D), dtype=torch.float32, device="cuda")
     assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp), d(kc32), d(kp), d(kc32), None, d(o1)) == 0
+
+
+@pytest.mark.parametrize("T,B,H,Hkv,D,K", [(1, 2, 16, 2, 64, 1024), (1, 1, 16, 2, 64, 1024), (3, 2, 8, 8, 128, 512), (16, 1, 4, 1, 32, 256)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+@pytest.mark.parametrize("yarn", [False, True])
+def test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn):
+    import torch
+    say(f"fused q/k/v projections + rope T={T} B={B} H={H}/{Hkv} D={D} K={K} act={act} yarn={yarn}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-qkv", T, B, H, D, K)
+    wq, _ = q8_dev((0.05 * g.standard_normal((H * D, K))).astype(np.float32))
+    wk, _ = q8_dev((0.05 * g.standard_normal((Hkv * D, K))).astype(np.float32))
+    wv, _ = q8_dev((0.05 * g.standard_normal((Hkv * D, K))).astype(np.float32))
+    x = dev(g.standard_normal((B, 1, T, K)).astype(np.float32))
+    pos = torch.arange(700, 700 + T, dtype=torch.int32, device="cuda")
+    ff = dev((1.0 + g.random(D // 2)).astype(np.float32))
+    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.1, 32.0, 1.0) if not yarn else (D, 2, 512, 10000.0, 0.5, 1.0, 1.0, 32.0, 1.0)
+
+    def outs():
+        return (torch.empty((B, T, H, D), dtype=torch.float32, device="cuda"),
+                torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda"),
+                torch.empty((B, 1, T, Hkv * D), dtype=torch.float32, device="cuda"))
+
+    q1, k1, v1 = outs()
+    for w, o, M in ((wq, q1, H * D), (wk, k1, Hkv * D), (wv, v1, Hkv * D)):
+        ok(pkg, L.vx_mul_mat(pkg.desc_q8(w, K), d(x), d(o.view(B, 1, T, M)), mode, None), "mul_mat")
+    for o in (q1, k1):
+        ok(pkg, L.vx_rope(d(o), pos.data_ptr(), ff.data_ptr(), d(o), *rope_args, None), "rope")
+    q2, k2, v2 = outs()
+    assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D, 2) == 1
+    ok(pkg, L.vx_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), pos.data_ptr(), ff.data_ptr(),
+                               d(q2), d(k2), d(v2), *rope_args, mode, None), "qkv_proj_rope")
+    torch.cuda.synchronize()
+    assert torch.equal(v1, v2)
+    assert torch.equal(k1, k2)
+    assert torch.equal(q1, q2)
+    if B * T <= 16:   # the same with every sequence's tokens flattened into one token dimension, as a 2-D activation tensor
+        q3, k3, v3 = outs()
+        xf, vf = x.view(B * T, K), v3.view(B * T, Hkv * D)
+        assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(xf), d(q3), d(k3), d(vf), D, 2) == 1
+        ok(pkg, L.vx_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(xf), pos.data_ptr(), ff.data_ptr(),
+                                   d(q3), d(k3), d(vf), *rope_args, mode, None), "qkv_proj_rope flattened")
+        torch.cuda.synchronize()
+        assert torch.equal(q1, q3) and torch.equal(k1, k3) and torch.equal(v1, v3)
+    # NORMAL-mode rotation and partial rotation are left to the separate operators
+    assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D, 0) == 0
+    assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D // 2, 2) == 0

@@ -16,8 +16,8 @@ are built once, so a plan can be replayed from a captured HIP graph.
 
 With `fuse_pairs=True` the adjacent nodes the ggml backend plugin runs as one launch (rms_norm+mul,
 scale+add, cont+sum, add+scale, and at decode size the gate/up/SwiGLU triple, projection+scale+add, the
-nine-node cache write with its ordering scalar, and attention over cached + current keys without the
-two concats) are issued as the plugin issues them, so a plan
+nine-node cache write with its ordering scalar, the q/k/v projections with both rotations, and attention
+over cached + current keys without the two concats) are issued as the plugin issues them, so a plan
 has as many launches as the plugin needs for the reference's graph; the results are bit-identical
 to the unfused sequence.
 """
@@ -146,13 +146,21 @@ class MiniCPMBackbone:
             wd = {n: desc_q8(*w[n]) for n in WEIGHT_NAMES}
             # -- attention_forward
             norm(cur_x, nrm["input_layernorm"], normed)
-            call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
-            call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
-            call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
             q4, k4, v4 = q.view(B, T, H, D), k.view(B, T, Hkv, D), v.view(B, T, Hkv, D)
-            for t4 in (q4, k4):
-                call(L.vx_rope, desc(t4), _p(pos), ff, desc(t4), D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0,
-                     attn_factor, 32.0, 1.0)
+            rope_args = (D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0, attn_factor, 32.0, 1.0)
+            # (with an F16 cache the reference's graph casts the rotated keys between the K and V projections; the plugin
+            # only groups the projections when no other node runs between them)
+            plain_order = n_past == 0 or self.kv_dtype == f32
+            if fuse and plain_order and L.vx_supports_qkv_proj_rope(wd["q_proj"], wd["k_proj"], wd["v_proj"], desc(normed), desc(q4), desc(k4), desc(v), D, 2):
+                # the three projections and both rotations as one launch (decode-sized token counts)
+                call(L.vx_qkv_proj_rope, wd["q_proj"], wd["k_proj"], wd["v_proj"], desc(normed), _p(pos), ff, desc(q4), desc(k4), desc(v),
+                     *rope_args, self.act_mode)
+            else:
+                call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
+                call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
+                call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
+                for t4 in (q4, k4):
+                    call(L.vx_rope, desc(t4), _p(pos), ff, desc(t4), *rope_args)
             # from here on in the order ggml_build_forward_expand gives the reference's graph: concat, attention,
             # then the cache append with its ordering chain, then add1 (only adjacent nodes are run as one launch)
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)

@@ -25,8 +25,18 @@
 //
 // Algorithmic HBM bytes: weights once (34 bytes per 32 weights) + activations + output.
 #include "vx_common.hpp"
+#include "rope_common.hpp"
 
 namespace {
+
+constexpr int GV_MAX_SEG = 3;
+struct gv_seg {
+    const char * w; char * dst;
+    int64_t  M;
+    uint64_t nb01, nb1, nb2, nb3; // weight row stride; dst strides of token, ne2, ne3
+    int wg0;                      // first work-group of this matrix
+    int rope;                     // rotate (row d, row d + head_dim/2) pairs of every head before storing
+};
 
 struct mm_args {
     const char * w; const char * x; char * dst;
@@ -40,6 +50,14 @@ struct mm_args {
     const char * res; // GEMV, fused residual update: dst = res + res_scale * (W x); null for a plain product
     uint64_t rnb1, rnb2, rnb3;
     float res_scale;
+    // GEMV over several weight matrices that share the activations (the Q, K and V projections), each
+    // with its own destination and optionally the NEOX rotation of GGML_OP_ROPE applied before the store
+    gv_seg seg[GV_MAX_SEG];
+    int nseg;
+    const int32_t * pos; const float * ff;
+    rope_params rp;
+    int head_dim;
+    int rope_T; // tokens per sequence: token n of the flattened (token, batch) order sits at position pos[n % rope_T]
 };
 
 // a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
@@ -254,7 +272,7 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
 // in one round trip to HBM.
 constexpr int GV_UNROLL = 8;
 
-template <int WT, bool ACT_Q8, int NW, bool AL4>
+template <int WT, bool ACT_Q8, int NW, bool AL4, bool SEG>
 __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
     const int64_t nkb = a.K / 32;
@@ -266,9 +284,23 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const int j = lane >> 4, c = lane & 15;
     const int     batch = blockIdx.z;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
-    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    int64_t       M = a.M;
+    uint64_t      nb01 = a.nb01, nb1 = a.nb1;
+    int           wl = blockIdx.x; // work-group index within its matrix
+    bool          rope = false;
+    if constexpr (SEG) {
+        int sg = 0;
+        if (a.nseg > 1 && wl >= a.seg[1].wg0) sg = 1;
+        if (a.nseg > 2 && wl >= a.seg[2].wg0) sg = 2;
+        const gv_seg & S = a.seg[sg];
+        wb = S.w; db = S.dst + (uint64_t) i12 * S.nb2 + (uint64_t) i13 * S.nb3;
+        M = S.M; nb01 = S.nb01; nb1 = S.nb1;
+        wl -= S.wg0;
+        rope = S.rope != 0;
+    }
     // R = a.rows_wg of the 16 MFMA columns carry weight rows; fewer rows per work-group put a short
     // matrix on more CUs (a CU sustains only so many outstanding lines, so 64 work-groups cannot
     // pull what 256 can).  Lanes c >= R load nothing; their columns are never stored.
@@ -277,10 +309,19 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const bool    dual = a.w2 != nullptr;                 // uniform
     const int     R  = a.rows_wg, Rr = dual ? R / 2 : R;   // MFMA columns in use, output rows per work-group
     const int     cr = dual ? c % Rr : c;
-    const int64_t row0 = (int64_t) blockIdx.x * Rr;
-    const bool    row_ok = c < R && row0 + cr < a.M;
+    // the weight row of MFMA column c.  Plain: consecutive rows.  With the rotation the R columns hold R/2
+    // pairs (d, d + head_dim/2) of one head, first elements in columns 0 .. R/2-1, partners in the rest.
+    int64_t       row = (int64_t) wl * Rr + cr;
+    const int     h2 = R >> 1, half_dim = a.head_dim >> 1;
+    int           pair = 0; // index of the pair within its head: the rotation's frequency index
+    if (SEG && rope) {
+        const int64_t f = (int64_t) wl * h2 + (c & (h2 - 1));
+        pair = (int) (f % half_dim);
+        row  = (f / half_dim) * a.head_dim + pair + (c >= h2 ? half_dim : 0);
+    }
+    const bool    row_ok = c < R && row < M;
     const char *  wsel = (dual && c >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
-    const char *  wrow = wsel + (uint64_t) min(row0 + cr, a.M - 1) * a.nb01;
+    const char *  wrow = wsel + (uint64_t) min(row, M - 1) * nb01;
     const int     N = (int) a.N;
 
     // ---- this wave's weight blocks: kb = wid + NW * i
@@ -345,12 +386,20 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
-        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) (row0 + c) * 4;
+        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) row * 4;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
     }
     load_blocks(0);
+    // the rotation's cos / sin for this lane's (token, pair) values: computed while the weights fly
+    float rc[4] = {1.0f, 1.0f, 1.0f, 1.0f}, rs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (SEG && rope && wid == 0 && row_ok) {
+        const float ffv = a.ff ? a.ff[pair] : 1.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * N + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
+    }
     if (tid < units) stage(tid, f0, f1);
     for (int unit = tid + 64 * NW; unit < units; unit += 64 * NW) {
         fetch(unit, f0, f1);
@@ -403,11 +452,21 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] = scaled_residual(acc[r], a.res_scale, resv[r]);
     }
+    if (SEG && rope) { // column c < R/2 holds x0 of its pair, column c + R/2 the partner x1
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float other = __shfl_xor(acc[r], h2, 64);
+            const bool  first = c < h2;
+            float y0, y1;
+            rope_rotate(first ? acc[r] : other, first ? other : acc[r], rc[r], rs[r], y0, y1);
+            acc[r] = first ? y0 : y1;
+        }
+    }
     if (row_ok && c < Rr) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int tok = 4 * j + r;
-            if (tok < N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) (row0 + c) * 4) = acc[r];
+            if (tok < N) *(float *) (db + (uint64_t) tok * nb1 + (uint64_t) row * 4) = acc[r];
         }
     }
 }
@@ -430,17 +489,32 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     if (a.N > 16 || a.K % 32 || a.K < 32) return false;
     a.rows_wg = 16;
     const int split = a.w2 ? 2 : 1; // with two matrices a work-group's MFMA columns hold half as many output rows
-    while (a.rows_wg > 4 && (a.M * split + a.rows_wg - 1) / a.rows_wg * nbatch < 128) a.rows_wg /= 2;
+    auto groups = [&](int rows_wg) { // work-groups per batch entry
+        if (a.nseg == 0) return (a.M * split + rows_wg - 1) / rows_wg;
+        int64_t n = 0;
+        for (int i = 0; i < a.nseg; ++i) n += (a.seg[i].M + rows_wg - 1) / rows_wg;
+        return n;
+    };
+    while (a.rows_wg > 4 && groups(a.rows_wg) * nbatch < 128) a.rows_wg /= 2;
     const int nw = gemv_waves(a);
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
     if (smem > 64 * 1024) return false;
-    const int rows_out = a.rows_wg / split;
-    const dim3 grid((unsigned) ((a.M + rows_out - 1) / rows_out), 1, (unsigned) nbatch);
+    int64_t nwg = groups(a.rows_wg);
+    if (a.nseg > 0) {
+        int wg0 = 0;
+        for (int i = 0; i < a.nseg; ++i) { a.seg[i].wg0 = wg0; wg0 += (int) ((a.seg[i].M + a.rows_wg - 1) / a.rows_wg); }
+    }
+    const dim3 grid((unsigned) nwg, 1, (unsigned) nbatch);
     const dim3 block((unsigned) (64 * nw));
-#define VX_GEMV(NW_)                                                                                       \
-    do {                                                                                                   \
-        if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true><<<grid, block, smem, st>>>(a);  \
-        else                            gemv_kernel<WT, ACT_Q8, NW_, false><<<grid, block, smem, st>>>(a); \
+#define VX_GEMV(NW_)                                                                                                   \
+    do {                                                                                                               \
+        if (a.nseg > 0) {                                                                                              \
+            if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true, true><<<grid, block, smem, st>>>(a);    \
+            else                            gemv_kernel<WT, ACT_Q8, NW_, false, true><<<grid, block, smem, st>>>(a);   \
+        } else {                                                                                                       \
+            if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true, false><<<grid, block, smem, st>>>(a);   \
+            else                            gemv_kernel<WT, ACT_Q8, NW_, false, false><<<grid, block, smem, st>>>(a);  \
+        }                                                                                                              \
     } while (0)
     switch (nw) {
         case 1:  VX_GEMV(1); break;
@@ -828,6 +902,89 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     if (src0->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
     else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
     if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: shape outside the streaming kernel");
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// The Q, K and V projections of one attention block with the NEOX rotation of Q and K, one launch:
+//   MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x)
+// (MiniCPMModel::attention_forward, src/minicpm.cpp:640-680).  q_dst and k_dst are the ROPE nodes'
+// outputs [head_dim, heads, tokens, batch], v_dst is the third MUL_MAT's [rows, tokens, 1, batch]
+// (or, like x, with the batch flattened into the token dimension).
+// Every product is formed as vx_mul_mat forms it and rotated with vx_rope's arithmetic.
+static bool qkv_rope_dst_ok(const vx_tensor * w, const vx_tensor * x, const vx_tensor * dst, int head_dim) {
+    if (!dst || dst->type != VX_TYPE_F32 || !vx_is_contiguous(dst)) return false;
+    if (dst->ne[0] != head_dim || dst->ne[0] * dst->ne[1] != w->ne[1]) return false;
+    // x is [K, tokens, 1, batch] or, with every sequence's tokens flattened into dim 1, [K, tokens * batch, 1, 1]
+    if (x->ne[3] == 1) return dst->ne[2] * dst->ne[3] == x->ne[1];
+    return dst->ne[2] == x->ne[1] && dst->ne[3] == x->ne[3];
+}
+
+extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
+                                         const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode) {
+    if (!wq || !wk || !wv || !x || !q_dst || !k_dst || !v_dst) return 0;
+    if (wq->type != VX_TYPE_Q8_0 && wq->type != VX_TYPE_F16) return 0;
+    const vx_tensor * ws[3] = { wq, wk, wv };
+    for (const vx_tensor * w : ws) {
+        if (w->type != wq->type || w->ne[0] != wq->ne[0] || w->ne[2] != 1 || w->ne[3] != 1 || !vx_positive(w)) return 0;
+        if (w->nb[0] != vx_type_size(w->type) || w->nb[1] < vx_row_size(w->type, w->ne[0])) return 0;
+        if (w->type == VX_TYPE_F16 && w->nb[1] % 2) return 0;
+    }
+    if (x->type != VX_TYPE_F32 || !vx_positive(x) || x->ne[0] != wq->ne[0] || x->ne[2] != 1 || x->nb[0] != 4) return 0;
+    if (x->nb[1] % 4 || x->nb[3] % 4 || x->ne[3] > 65535) return 0;
+    if (x->ne[1] > 16 || wq->ne[0] % 32 || wq->ne[0] < 32) return 0;
+    if (mode != 2 || n_dims <= 0 || n_dims % 16) return 0; // NEOX over the whole head; pairs split evenly over work-groups
+    if (!qkv_rope_dst_ok(wq, x, q_dst, n_dims) || !qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return 0;
+    if (v_dst->type != VX_TYPE_F32 || !vx_is_contiguous(v_dst)) return 0;
+    if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
+    return (size_t) x->ne[1] * wq->ne[0] * 2 + (size_t) x->ne[1] * (wq->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+}
+
+extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
+                                      const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst, const vx_tensor * k_dst,
+                                      const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                                      float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
+                                      vx_stream stream) {
+    if (!vx_supports_qkv_proj_rope(wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode))
+        return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: three Q8_0/F16 matrices over one activation tensor of at most 16 tokens, NEOX rotation over the whole head, contiguous outputs");
+    if (!pos || !wq->data || !wk->data || !wv->data || !x->data || !q_dst->data || !k_dst->data || !v_dst->data)
+        return vx_fail(VX_ERR_INVALID, "qkv_proj_rope: null data");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "qkv_proj_rope: bad act_mode");
+    const vx_tensor * ws[3] = { wq, wk, wv };
+    const vx_tensor * ds[3] = { q_dst, k_dst, v_dst };
+    if ((uintptr_t) x->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: misaligned activations");
+    mm_args a = {};
+    a.x = (const char *) x->data;
+    a.K = wq->ne[0]; a.N = x->ne[1];
+    a.M = 0;
+    a.nb11 = x->nb[1]; a.nb12 = x->nb[2]; a.nb13 = x->nb[3];
+    a.ne12 = 1; a.r2 = 1; a.r3 = 1;
+    a.rows_wg = 16;
+    a.w_aligned = 1;
+    a.nseg = 3;
+    for (int i = 0; i < 3; ++i) {
+        if ((uintptr_t) ds[i]->data % 4 || (ws[i]->type == VX_TYPE_F16 && (uintptr_t) ws[i]->data % 2))
+            return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: misaligned tensor data");
+        gv_seg & s = a.seg[i];
+        s.w = (const char *) ws[i]->data; s.dst = (char *) ds[i]->data;
+        s.M = ws[i]->ne[1]; s.nb01 = ws[i]->nb[1];
+        s.nb1 = (uint64_t) s.M * 4; s.nb2 = 0; s.nb3 = (uint64_t) s.M * 4 * x->ne[1]; // the contiguous [rows, tokens, 1, batch] view of dst
+        s.rope = i < 2;
+        a.w_aligned = a.w_aligned && ((uintptr_t) ws[i]->data % 4 == 0) && ws[i]->nb[1] % 4 == 0;
+        a.M += s.M;
+    }
+    a.w = a.seg[0].w; a.dst = a.seg[0].dst;
+    a.x_aligned = ((uintptr_t) x->data % 16 == 0) && x->nb[1] % 16 == 0 && x->nb[3] % 16 == 0;
+    a.pos = pos; a.ff = freq_factors;
+    a.rp = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    a.head_dim = n_dims;
+    a.rope_T   = (int) q_dst->ne[2];
+    const int nbatch = (int) x->ne[3];
+    hipStream_t st = (hipStream_t) stream;
+    bool ok;
+    if (wq->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
+    else                          ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: shape outside the streaming kernel");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

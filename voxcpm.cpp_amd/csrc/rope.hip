@@ -9,24 +9,12 @@
 //
 // One thread per (pair, row); a row is one (head, token, batch) vector.  HBM-bound at
 // 8 bytes per element; in decode it is a handful of rows and purely launch latency.
-#include "vx_common.hpp"
-
-#include <cmath>
+#include "rope_common.hpp"
 
 // the angle arithmetic must round like the host code it mirrors: no fused multiply-adds
 #pragma clang fp contract(off)
 
 namespace {
-
-struct rope_params {
-    int   n_dims;
-    int   mode; // 0 NORMAL, 2 NEOX
-    float theta_scale;
-    float freq_scale;
-    float ext_factor;
-    float attn_factor;
-    float corr_lo, corr_hi;
-};
 
 __global__ __launch_bounds__(256) void rope_kernel(const char * __restrict__ src, char * __restrict__ dst, vx_dims s,
                                                    vx_dims d, const int32_t * __restrict__ pos,
@@ -58,30 +46,12 @@ __global__ __launch_bounds__(256) void rope_kernel(const char * __restrict__ src
     const float x0 = x[ia], x1 = x[ib];
     const float ff = freq_factors ? freq_factors[ip] : 1.0f;
 
-    float theta = (float) pos[i2];
-    for (int k = 0; k < ip; ++k) theta *= p.theta_scale;
-
-    const float theta_extrap = theta / ff;
-    const float theta_interp = p.freq_scale * theta_extrap;
-    float       th           = theta_interp;
-    float       mscale       = p.attn_factor;
-    if (p.ext_factor != 0.0f) {
-        // rope_yarn_ramp takes i0/2 as an int and clamps in fp32 (ops.cpp:5589-5592)
-        const float yv       = ((float) ip - p.corr_lo) / fmaxf(0.001f, p.corr_hi - p.corr_lo);
-        const float ramp_mix = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * p.ext_factor;
-        // ggml-cpu's x86 build contracts this sum into one fused multiply-add
-        th                   = fmaf(theta_interp, 1.0f - ramp_mix, theta_extrap * ramp_mix);
-        mscale *= 1.0f + 0.1f * logf(1.0f / p.freq_scale);
-    }
-    const float c  = cosf(th) * mscale;
-    const float sn = sinf(th) * mscale;
-
-    y[ia] = x0 * c - x1 * sn;
-    y[ib] = x0 * sn + x1 * c;
-}
-
-float yarn_corr_dim(int n_dims, int n_ctx_orig, float n_rot, float base) {
-    return n_dims * logf(n_ctx_orig / (n_rot * 2 * (float) M_PI)) / (2 * logf(base));
+    float c, sn;
+    rope_cos_sin(p, (float) pos[i2], ip, ff, c, sn);
+    float y0, y1;
+    rope_rotate(x0, x1, c, sn, y0, y1);
+    y[ia] = y0;
+    y[ib] = y1;
 }
 
 } // namespace
@@ -104,19 +74,7 @@ extern "C" vx_status vx_rope(const vx_tensor * src, const int32_t * pos, const f
     if (!src || !dst || !src->data || !dst->data || !pos) return vx_fail(VX_ERR_INVALID, "rope: null argument");
     if (!vx_supports_rope(src, dst, n_dims, mode))
         return vx_fail(VX_ERR_UNSUPPORTED, "rope: needs F32 tensors of equal shape, dense rows, mode 0 or 2, even n_dims <= ne0");
-    rope_params p;
-    p.n_dims      = n_dims;
-    p.mode        = mode;
-    p.theta_scale = powf(freq_base, -2.0f / n_dims); // host libm, as ggml-cpu (ops.cpp:5775)
-    p.freq_scale  = freq_scale;
-    p.ext_factor  = ext_factor;
-    p.attn_factor = attn_factor;
-    {   // ggml_rope_yarn_corr_dims (ggml/src/ggml.c:4280-4294)
-        const float start = floorf(yarn_corr_dim(n_dims, n_ctx_orig, beta_fast, freq_base));
-        const float end   = ceilf(yarn_corr_dim(n_dims, n_ctx_orig, beta_slow, freq_base));
-        p.corr_lo = fmaxf(0.0f, start);
-        p.corr_hi = fminf((float) (n_dims - 1), end);
-    }
+    const rope_params p = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
     const int64_t total = vx_nrows(src) * (src->ne[0] / 2);
     const unsigned grid = (unsigned) ((total + 255) / 256);
     rope_kernel<<<dim3(grid), dim3(256), 0, (hipStream_t) stream>>>((const char *) src->data, (char *) dst->data,

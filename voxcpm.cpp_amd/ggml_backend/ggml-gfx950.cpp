@@ -30,6 +30,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 namespace {
@@ -625,6 +626,76 @@ vx_status compute_kv2_attention(backend_ctx * ctx, const ggml_tensor * f, const 
                                  &d, scale, max_bias, softcap, ctx->stream);
 }
 
+// attention_forward's three projections and the rotation of Q and K (src/minicpm.cpp:669-680) at decode size:
+//   MUL_MAT(wq, x) RESHAPE ROPE  [views]  MUL_MAT(wk, x) RESHAPE ROPE  [views, absorbed CONCAT]  MUL_MAT(wv, x)
+// -> one launch at the first node; the other four are marked done.  K's and V's outputs are written earlier
+// than their nodes' turn, which is safe because every node in between that does work belongs to the group.
+typedef std::unordered_map<const ggml_tensor *, const ggml_tensor *> absorbed_map;
+
+const ggml_tensor * rope_of_projection(const ggml_cgraph * g, int & idx, const ggml_tensor * mm, const reader_map & readers,
+                                       const absorbed_map & absorbed) {
+    // the next node that does work must be a ROPE over (a reshape of) mm, and nothing else may read mm
+    int k = idx + 1;
+    while (k < g->n_nodes && (ggml_op_is_empty(g->nodes[k]->op) || ggml_is_empty(g->nodes[k]) || absorbed.count(g->nodes[k]))) ++k;
+    if (k >= g->n_nodes) return nullptr;
+    const ggml_tensor * r = g->nodes[k];
+    if (r->op != GGML_OP_ROPE || (r->flags & GGML_TENSOR_FLAG_COMPUTE) == 0 || (mm->flags & GGML_TENSOR_FLAG_OUTPUT) != 0) return nullptr;
+    const ggml_tensor * in = r->src[0];
+    const auto rd = [&](const ggml_tensor * t) { const auto it = readers.find(t); return it == readers.end() ? 0 : it->second; };
+    if (in == mm) {
+        if (rd(mm) != 1) return nullptr;
+    } else {
+        if (in->op != GGML_OP_RESHAPE || in->src[0] != mm || in->view_src != mm || (in->flags & GGML_TENSOR_FLAG_OUTPUT) != 0) return nullptr;
+        if (rd(mm) != 2 || rd(in) != 1) return nullptr; // mm: the reshape's operand and view source; the reshape: the rope
+    }
+    idx = k;
+    return r;
+}
+
+bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, const absorbed_map & absorbed,
+                       std::unordered_set<const ggml_tensor *> & done, vx_status * rc) {
+    const ggml_tensor * mq = g->nodes[i];
+    int idx = i;
+    const ggml_tensor * rq = rope_of_projection(g, idx, mq, readers, absorbed);
+    if (!rq) return false;
+    auto next_work = [&](int k) {
+        ++k;
+        while (k < g->n_nodes && (ggml_op_is_empty(g->nodes[k]->op) || ggml_is_empty(g->nodes[k]) || absorbed.count(g->nodes[k]))) ++k;
+        return k;
+    };
+    idx = next_work(idx);
+    if (idx >= g->n_nodes) return false;
+    const ggml_tensor * mk = g->nodes[idx];
+    if (mk->op != GGML_OP_MUL_MAT || mk->src[1] != mq->src[1] || (mk->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return false;
+    const ggml_tensor * rk = rope_of_projection(g, idx, mk, readers, absorbed);
+    if (!rk) return false;
+    idx = next_work(idx);
+    if (idx >= g->n_nodes) return false;
+    const ggml_tensor * mv = g->nodes[idx];
+    if (mv->op != GGML_OP_MUL_MAT || mv->src[1] != mq->src[1] || (mv->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return false;
+    // one rotation for both: same positions, factors and parameters
+    if (rq->src[1] != rk->src[1] || rq->src[2] != rk->src[2] || memcmp(rq->op_params, rk->op_params, 11 * sizeof(int32_t)) != 0) return false;
+    if (!rq->src[1] || rq->src[1]->type != GGML_TYPE_I32 || rq->src[1]->ne[0] != rq->ne[2]) return false;
+    if (rq->src[2] && (rq->src[2]->type != GGML_TYPE_F32 || rq->src[2]->ne[0] < rq->ne[0] / 2)) return false;
+    const int32_t * ip = (const int32_t *) rq->op_params;
+    const int n_dims = ip[1], mode = ip[2], n_ctx_orig = ip[4];
+    float fp[6];
+    memcpy(fp, ip + 5, sizeof(fp));
+    const ggml_tensor * x = mq->src[1];
+    const ggml_tensor * outs[3] = { rq, rk, mv };
+    for (int a = 0; a < 3; ++a) {
+        if (!apart(outs[a], x)) return false;
+        for (int b = a + 1; b < 3; ++b) if (!apart(outs[a], outs[b])) return false;
+    }
+    const vx_tensor wq = to_vx(mq->src[0]), wk = to_vx(mk->src[0]), wv = to_vx(mv->src[0]), xx = to_vx(x), dq = to_vx(rq), dk = to_vx(rk),
+                    dv = to_vx(mv);
+    if (!vx_supports_qkv_proj_rope(&wq, &wk, &wv, &xx, &dq, &dk, &dv, n_dims, mode)) return false;
+    *rc = vx_qkv_proj_rope(&wq, &wk, &wv, &xx, (const int32_t *) rq->src[1]->data, rq->src[2] ? (const float *) rq->src[2]->data : nullptr,
+                           &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3], fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
+    done.insert(rq); done.insert(mk); done.insert(rk); done.insert(mv);
+    return true;
+}
+
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
 
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
@@ -649,6 +720,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     }
     std::unordered_map<const ggml_tensor *, kv2_group> kv2_by_fa;
     std::unordered_map<const ggml_tensor *, const ggml_tensor *> kv2_absorbed;
+    std::unordered_set<const ggml_tensor *> done;
     if (fusion && cgraph->n_nodes > 2) find_kv2_groups(cgraph, readers, kv2_by_fa, kv2_absorbed);
     for (int i = 0; i < cgraph->n_nodes; ++i) {
         ggml_tensor * node = cgraph->nodes[i];
@@ -656,8 +728,17 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         if (ggml_op_is_empty(node->op) || ggml_is_empty(node)) continue;
         if ((node->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
         if (kv2_absorbed.count(node)) continue; // a CONCAT the attention node reads through
+        if (done.count(node)) continue;         // computed ahead of its turn by a group
         vx_status rc = VX_ERR_UNSUPPORTED;
         bool fused = false;
+        if (fusion && node->op == GGML_OP_MUL_MAT && compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc)) {
+            ++launches;
+            if (rc != VX_OK) {
+                GGML_LOG_ERROR("ggml-gfx950: node %d (%s, q/k/v projections + rope) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                return GGML_STATUS_FAILED;
+            }
+            continue;
+        }
         if (node->op == GGML_OP_FLASH_ATTN_EXT) {
             const auto it = kv2_by_fa.find(node);
             if (it != kv2_by_fa.end()) {
