@@ -217,6 +217,24 @@ VX_API vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, co
 VX_API int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
                                      const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims,
                                      int mode);
+/* RMS_NORM(x) , MUL(., norm_w) in front of vx_qkv_proj_rope / vx_mul_mat_swiglu: MiniCPMModel::rms_norm
+ * (src/minicpm.cpp:572-580) as layer_forward applies it before attention and before the MLP (:761, :770), joined to
+ * the projections' launch.  x is the un-normalised hidden state, rows of at most 1024 floats, 16-byte aligned;
+ * norm_w one F32 row.  The normalised tensor is not stored.  Results equal vx_rms_norm_mul followed by the
+ * projection call, bit for bit. */
+VX_API vx_status vx_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * wq,
+                                       const vx_tensor * wk, const vx_tensor * wv, const int32_t * pos,
+                                       const float * freq_factors, const vx_tensor * q_dst, const vx_tensor * k_dst,
+                                       const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base,
+                                       float freq_scale, float ext_factor, float attn_factor, float beta_fast,
+                                       float beta_slow, int act_mode, vx_stream stream);
+VX_API int vx_supports_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * wq,
+                                          const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * q_dst,
+                                          const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode);
+VX_API vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate,
+                                        const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream);
+VX_API int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate,
+                                           const vx_tensor * up, const vx_tensor * dst);
 /* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for at most 16 tokens
  * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,

@@ -329,3 +329,72 @@ def test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn):
     # NORMAL-mode rotation and partial rotation are left to the separate operators
     assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D, 0) == 0
     assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D // 2, 2) == 0
+
+
+@pytest.mark.parametrize("T,B,K,M", [(1, 2, 1024, 4096), (2, 1, 1024, 4096), (16, 1, 512, 1000), (3, 2, 256, 64)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+def test_norm_mul_mat_swiglu(pkg, gpu, T, B, K, M, act):
+    import torch
+    say(f"fused rms_norm+mul in front of gate/up/swiglu T={T} B={B} K={K} M={M} act={act}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-nswiglu", T, B, K, M)
+    wg, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    wu, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    x = dev((3.0 * g.standard_normal((B, 1, T, K))).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    normed = torch.empty_like(x)
+    a = torch.empty((B, 1, T, M), dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    ok(pkg, L.vx_mul_mat_swiglu(pkg.desc_q8(wg, K), pkg.desc_q8(wu, K), d(normed), d(a), mode, None), "mul_mat_swiglu")
+    assert L.vx_supports_norm_mul_mat_swiglu(d(x), d(nw), pkg.desc_q8(wg, K), pkg.desc_q8(wu, K), d(b)) == 1
+    ok(pkg, L.vx_norm_mul_mat_swiglu(d(x), d(nw), 1e-5, pkg.desc_q8(wg, K), pkg.desc_q8(wu, K), d(b), mode, None), "norm_mul_mat_swiglu")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_norm_prologue_limits(pkg, gpu):
+    import torch
+    say("norm prologue: rows beyond 1024 floats stay with the separate RMS_NORM")
+    L, d = pkg.lib(), pkg.desc
+    K, M = 2048, 64
+    w, _ = q8_dev(np.zeros((M, K), dtype=np.float32))
+    x = torch.zeros((1, 1, 1, K), dtype=torch.float32, device="cuda")
+    nw = torch.ones(K, dtype=torch.float32, device="cuda")
+    o = torch.zeros((1, 1, 1, M), dtype=torch.float32, device="cuda")
+    assert L.vx_supports_norm_mul_mat_swiglu(d(x), d(nw), pkg.desc_q8(w, K), pkg.desc_q8(w, K), d(o)) == 0
+    assert L.vx_norm_mul_mat_swiglu(d(x), d(nw), 1e-5, pkg.desc_q8(w, K), pkg.desc_q8(w, K), d(o), pkg.ACT_FLOAT, None) != 0
+
+
+@pytest.mark.parametrize("T,B,H,Hkv,D,K", [(1, 2, 16, 2, 64, 1024), (4, 2, 8, 2, 64, 512), (1, 1, 4, 4, 128, 1024)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+def test_norm_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act):
+    import torch
+    say(f"fused rms_norm+mul in front of q/k/v projections + rope T={T} B={B} H={H}/{Hkv} D={D} K={K} act={act}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-nqkv", T, B, H, D, K)
+    ws = [q8_dev((0.05 * g.standard_normal((n * D, K))).astype(np.float32))[0] for n in (H, Hkv, Hkv)]
+    wd = [pkg.desc_q8(w, K) for w in ws]
+    x = dev((2.0 * g.standard_normal((B * T, K))).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    pos = torch.arange(300, 300 + T, dtype=torch.int32, device="cuda")
+    ff = dev((1.0 + g.random(D // 2)).astype(np.float32))
+    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+
+    def outs():
+        return (torch.empty((B, T, H, D), dtype=torch.float32, device="cuda"),
+                torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda"),
+                torch.empty((B * T, Hkv * D), dtype=torch.float32, device="cuda"))
+
+    q1, k1, v1 = outs()
+    normed = torch.empty_like(x)
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    ok(pkg, L.vx_qkv_proj_rope(*wd, d(normed), pos.data_ptr(), ff.data_ptr(), d(q1), d(k1), d(v1), *rope_args, mode, None), "qkv_proj_rope")
+    q2, k2, v2 = outs()
+    assert L.vx_supports_norm_qkv_proj_rope(d(x), d(nw), *wd, d(q2), d(k2), d(v2), D, 2) == 1
+    ok(pkg, L.vx_norm_qkv_proj_rope(d(x), d(nw), 1e-5, *wd, pos.data_ptr(), ff.data_ptr(), d(q2), d(k2), d(v2), *rope_args, mode, None),
+       "norm_qkv_proj_rope")
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)

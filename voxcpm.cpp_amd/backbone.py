@@ -16,8 +16,8 @@ are built once, so a plan can be replayed from a captured HIP graph.
 
 With `fuse_pairs=True` the adjacent nodes the ggml backend plugin runs as one launch (rms_norm+mul,
 scale+add, cont+sum, add+scale, and at decode size the gate/up/SwiGLU triple, projection+scale+add, the
-nine-node cache write with its ordering scalar, the q/k/v projections with both rotations, and attention
-over cached + current keys without the two concats) are issued as the plugin issues them, so a plan
+nine-node cache write with its ordering scalar, the q/k/v projections with both rotations, rms_norm joined
+to the projections behind it, and attention over cached + current keys without the two concats) are issued as the plugin issues them, so a plan
 has as many launches as the plugin needs for the reference's graph; the results are bit-identical
 to the unfused sequence.
 """
@@ -145,17 +145,22 @@ class MiniCPMBackbone:
             kc, vc = self.k_cache[li], self.v_cache[li]
             wd = {n: desc_q8(*w[n]) for n in WEIGHT_NAMES}
             # -- attention_forward
-            norm(cur_x, nrm["input_layernorm"], normed)
             q4, k4, v4 = q.view(B, T, H, D), k.view(B, T, Hkv, D), v.view(B, T, Hkv, D)
             rope_args = (D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0, attn_factor, 32.0, 1.0)
             # (with an F16 cache the reference's graph casts the rotated keys between the K and V projections; the plugin
             # only groups the projections when no other node runs between them)
             plain_order = n_past == 0 or self.kv_dtype == f32
-            if fuse and plain_order and L.vx_supports_qkv_proj_rope(wd["q_proj"], wd["k_proj"], wd["v_proj"], desc(normed), desc(q4), desc(k4), desc(v), D, 2):
-                # the three projections and both rotations as one launch (decode-sized token counts)
-                call(L.vx_qkv_proj_rope, wd["q_proj"], wd["k_proj"], wd["v_proj"], desc(normed), _p(pos), ff, desc(q4), desc(k4), desc(v),
+            wqkv = (wd["q_proj"], wd["k_proj"], wd["v_proj"])
+            nw_in = nrm["input_layernorm"]
+            if fuse and plain_order and L.vx_supports_norm_qkv_proj_rope(desc(cur_x), desc(nw_in), *wqkv, desc(q4), desc(k4), desc(v), D, 2):
+                # rms_norm, the three projections and both rotations as one launch (decode-sized token counts)
+                call(L.vx_norm_qkv_proj_rope, desc(cur_x), desc(nw_in), self.eps, *wqkv, _p(pos), ff, desc(q4), desc(k4), desc(v),
                      *rope_args, self.act_mode)
+            elif fuse and plain_order and L.vx_supports_qkv_proj_rope(*wqkv, desc(normed), desc(q4), desc(k4), desc(v), D, 2):
+                norm(cur_x, nw_in, normed)
+                call(L.vx_qkv_proj_rope, *wqkv, desc(normed), _p(pos), ff, desc(q4), desc(k4), desc(v), *rope_args, self.act_mode)
             else:
+                norm(cur_x, nw_in, normed)
                 call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
                 call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
                 call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
@@ -214,10 +219,15 @@ class MiniCPMBackbone:
                 call(L.vx_add1, desc(attn), desc(sync), desc(attn))
             project_residual(wd["o_proj"], attn.view(N, H * D), attn_o, cur_x, h_mid)
             # -- mlp_forward
-            norm(h_mid, nrm["post_layernorm"], normed)
-            if fuse and N <= 16:     # gate, up and SwiGLU as one launch
+            nw_post = nrm["post_layernorm"]
+            if fuse and L.vx_supports_norm_mul_mat_swiglu(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], desc(act)):
+                # rms_norm, gate, up and SwiGLU as one launch
+                call(L.vx_norm_mul_mat_swiglu, desc(h_mid), desc(nw_post), self.eps, wd["gate_proj"], wd["up_proj"], desc(act), self.act_mode)
+            elif fuse and N <= 16:     # gate, up and SwiGLU as one launch
+                norm(h_mid, nw_post, normed)
                 call(L.vx_mul_mat_swiglu, wd["gate_proj"], wd["up_proj"], desc(normed), desc(act), self.act_mode)
             else:
+                norm(h_mid, nw_post, normed)
                 call(L.vx_mul_mat, wd["gate_proj"], desc(normed), desc(gate), self.act_mode)
                 call(L.vx_mul_mat, wd["up_proj"], desc(normed), desc(up), self.act_mode)
                 call(L.vx_glu, GLU_SWIGLU, desc(gate), desc(up), desc(act), 0)

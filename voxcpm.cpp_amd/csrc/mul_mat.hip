@@ -58,6 +58,10 @@ struct mm_args {
     rope_params rp;
     int head_dim;
     int rope_T; // tokens per sequence: token n of the flattened (token, batch) order sits at position pos[n % rope_T]
+    // GEMV with RMS_NORM and the norm-weight MUL applied to the activations as they are staged
+    // (x is then the un-normalised tensor): x[t][k] / rms(x[t]) * norm_w[k], rounded after each product
+    const float * norm_w;
+    float norm_eps;
 };
 
 // a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
@@ -279,6 +283,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][K]
     float *    xd  = (float *) (gv_smem + (size_t) a.N * a.K * 2);           // [N][K/32] (ACT_Q8)
     float4_t * red = (float4_t *) (gv_smem + (size_t) a.N * a.K * 2 + (ACT_Q8 ? (size_t) a.N * nkb * 4 : 0));
+    float *    nsc = (float *) (red + (NW > 1 ? NW - 1 : 0) * 64); // [16] per-token 1 / rms (fused RMS_NORM)
 
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
@@ -358,11 +363,19 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             for (int i = 0; i < 4; ++i) { v0[i] = xp[i]; v1[i] = xp[4 + i]; }
         }
     };
-    auto stage = [&](int unit, const float4_t & v0, const float4_t & v1) {
+    auto stage = [&](int unit, const float4_t & v0, const float4_t & v1, const float4_t & g0, const float4_t & g1) {
         const int t = unit / upr, u = unit % upr;
         float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
+        if (a.norm_w) { // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
+            const float sc = nsc[t];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i]     *= sc; v[i]     *= g0[i];
+                v[4 + i] *= sc; v[4 + i] *= g1[i];
+            }
+        }
         half8_t h;
         if constexpr (ACT_Q8) { // 4 consecutive units = one 32-wide block (K/8 is a multiple of 4)
             float amax = 0.0f;
@@ -381,8 +394,13 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         }
         *(half8_t *) (xs + (size_t) t * a.K + 8 * u) = h;
     };
-    float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0};
+    float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0}, g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
     if (tid < units) fetch(tid, f0, f1);
+    auto fetch_gain = [&](int unit, float4_t & a0, float4_t & a1) { // the norm weights of a unit's 8 columns (16-byte aligned)
+        const float4_t * gp = (const float4_t *) (a.norm_w + 8 * (unit % upr));
+        a0 = gp[0]; a1 = gp[1];
+    };
+    if (a.norm_w && tid < units) fetch_gain(tid, g0, g1);
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
@@ -400,10 +418,18 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         for (int r = 0; r < 4; ++r)
             if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * N + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
     }
-    if (tid < units) stage(tid, f0, f1);
+    if (a.norm_w) { // one wave per token, as the RMS_NORM kernel has it
+        for (int t = wid; t < N; t += NW) {
+            const float sc = vx_rms_scale_wave((const float *) (xb + (uint64_t) t * a.nb11), a.K, lane, a.norm_eps);
+            if (lane == 0) nsc[t] = sc;
+        }
+        __syncthreads();
+    }
+    if (tid < units) stage(tid, f0, f1, g0, g1);
     for (int unit = tid + 64 * NW; unit < units; unit += 64 * NW) {
         fetch(unit, f0, f1);
-        stage(unit, f0, f1);
+        if (a.norm_w) fetch_gain(unit, g0, g1);
+        stage(unit, f0, f1, g0, g1);
     }
     __syncthreads();
 
@@ -472,7 +498,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
 }
 
 size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
-    return (size_t) a.N * a.K * 2 + (act_q8 ? (size_t) a.N * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16;
+    return (size_t) a.N * a.K * 2 + (act_q8 ? (size_t) a.N * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float);
 }
 
 // waves per work-group: about GV_UNROLL blocks per wave, so every load is issued up front
@@ -827,11 +853,44 @@ extern "C" int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tenso
     if (up->type != gate->type) return 0;
     for (int i = 0; i < 4; ++i) if (up->ne[i] != gate->ne[i] || up->nb[i] != gate->nb[i]) return 0;
     if (src1->ne[1] > 16 || gate->ne[0] % 32 || gate->ne[0] < 32) return 0;
-    return (size_t) src1->ne[1] * gate->ne[0] * 2 + (size_t) src1->ne[1] * (gate->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+    return (size_t) src1->ne[1] * gate->ne[0] * 2 + (size_t) src1->ne[1] * (gate->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
 }
+
+// whether the activations of a streaming-kernel launch can be normalised on the fly: rows of at most 1024
+// floats (the RMS_NORM kernel's wave-per-row regime), everything 16-byte aligned, one F32 weight row
+static bool norm_prologue_ok(const vx_tensor * x, const vx_tensor * norm_w) {
+    if (!norm_w || norm_w->type != VX_TYPE_F32 || norm_w->nb[0] != 4) return false;
+    if (norm_w->ne[0] != x->ne[0] || norm_w->ne[1] != 1 || norm_w->ne[2] != 1 || norm_w->ne[3] != 1) return false;
+    if (x->ne[0] > 1024 || x->ne[0] % 8) return false;
+    return x->nb[1] % 16 == 0 && x->nb[2] % 16 == 0 && x->nb[3] % 16 == 0;
+}
+
+static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * norm_w, float eps,
+                            const vx_tensor * dst, int act_mode, vx_stream stream);
 
 extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
                                        int act_mode, vx_stream stream) {
+    return swiglu_run(gate, up, src1, nullptr, 0.0f, dst, act_mode, stream);
+}
+
+// RMS_NORM , MUL(norm weight) , MUL_MAT(gate) , MUL_MAT(up) , GLU(SWIGLU): mlp_forward behind its rms_norm
+// (src/minicpm.cpp:572-580, 718-747) as one launch; x is the un-normalised hidden state.
+extern "C" int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up,
+                                               const vx_tensor * dst) {
+    return vx_supports_mul_mat_swiglu(gate, up, x, dst) && norm_prologue_ok(x, norm_w);
+}
+
+extern "C" vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate,
+                                            const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream) {
+    if (!x || !norm_w || !gate || !up || !dst || !norm_w->data) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: null tensor");
+    if (!vx_supports_norm_mul_mat_swiglu(x, norm_w, gate, up, dst) || (uintptr_t) x->data % 16 || (uintptr_t) norm_w->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "norm_mul_mat_swiglu: as mul_mat_swiglu, with 16-byte aligned rows of at most 1024 floats and one F32 norm weight row");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: eps must be >= 0");
+    return swiglu_run(gate, up, x, norm_w, eps, dst, act_mode, stream);
+}
+
+static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * norm_w, float eps,
+                            const vx_tensor * dst, int act_mode, vx_stream stream) {
     if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
         return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
     if (!vx_supports_mul_mat_swiglu(gate, up, src1, dst))
@@ -849,6 +908,8 @@ extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor *
     a.r2 = (int) (src1->ne[2] / gate->ne[2]); a.r3 = (int) (src1->ne[3] / gate->ne[3]);
     a.rows_wg   = 16;
     a.w2        = (const char *) up->data;
+    a.norm_w    = norm_w ? (const float *) norm_w->data : nullptr;
+    a.norm_eps  = eps;
     a.w_aligned = (((uintptr_t) gate->data | (uintptr_t) up->data) % 4 == 0) && gate->nb[1] % 4 == 0 && gate->nb[2] % 4 == 0 && gate->nb[3] % 4 == 0;
     a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
@@ -870,7 +931,7 @@ extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_te
     if (residual->type != VX_TYPE_F32 || !vx_same_shape(residual, dst) || residual->nb[0] != 4) return 0;
     if (residual->nb[1] % 4 || residual->nb[2] % 4 || residual->nb[3] % 4) return 0;
     if (src1->ne[1] > 16 || src0->ne[0] % 32 || src0->ne[0] < 32) return 0;
-    return (size_t) src1->ne[1] * src0->ne[0] * 2 + (size_t) src1->ne[1] * (src0->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+    return (size_t) src1->ne[1] * src0->ne[0] * 2 + (size_t) src1->ne[1] * (src0->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
 }
 
 extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst,
@@ -937,14 +998,51 @@ extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor *
     if (!qkv_rope_dst_ok(wq, x, q_dst, n_dims) || !qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return 0;
     if (v_dst->type != VX_TYPE_F32 || !vx_is_contiguous(v_dst)) return 0;
     if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
-    return (size_t) x->ne[1] * wq->ne[0] * 2 + (size_t) x->ne[1] * (wq->ne[0] / 32) * 4 + 15 * 64 * 16 <= 64 * 1024;
+    return (size_t) x->ne[1] * wq->ne[0] * 2 + (size_t) x->ne[1] * (wq->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
 }
+
+static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,
+                         const vx_tensor * x, const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst,
+                         const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base,
+                         float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
+                         vx_stream stream);
 
 extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
                                       const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst, const vx_tensor * k_dst,
                                       const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                                       float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
                                       vx_stream stream) {
+    return qkv_run(nullptr, 0.0f, wq, wk, wv, x, pos, freq_factors, q_dst, k_dst, v_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale,
+                   ext_factor, attn_factor, beta_fast, beta_slow, act_mode, stream);
+}
+
+// RMS_NORM , MUL(norm weight) in front of the three projections: layer_forward's input rms_norm
+// (src/minicpm.cpp:572-580, 761) joins the launch; x is the un-normalised hidden state.
+extern "C" int vx_supports_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * wq, const vx_tensor * wk,
+                                              const vx_tensor * wv, const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst,
+                                              int n_dims, int mode) {
+    return vx_supports_qkv_proj_rope(wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode) && norm_prologue_ok(x, norm_w);
+}
+
+extern "C" vx_status vx_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * wq,
+                                           const vx_tensor * wk, const vx_tensor * wv, const int32_t * pos, const float * freq_factors,
+                                           const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode,
+                                           int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                                           float beta_fast, float beta_slow, int act_mode, vx_stream stream) {
+    if (!x || !norm_w || !norm_w->data) return vx_fail(VX_ERR_INVALID, "norm_qkv_proj_rope: null tensor");
+    if (!vx_supports_norm_qkv_proj_rope(x, norm_w, wq, wk, wv, q_dst, k_dst, v_dst, n_dims, mode) || (uintptr_t) x->data % 16 ||
+        (uintptr_t) norm_w->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: as qkv_proj_rope, with 16-byte aligned rows of at most 1024 floats and one F32 norm weight row");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "norm_qkv_proj_rope: eps must be >= 0");
+    return qkv_run(norm_w, eps, wq, wk, wv, x, pos, freq_factors, q_dst, k_dst, v_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale,
+                   ext_factor, attn_factor, beta_fast, beta_slow, act_mode, stream);
+}
+
+static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,
+                         const vx_tensor * x, const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst,
+                         const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base,
+                         float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
+                         vx_stream stream) {
     if (!vx_supports_qkv_proj_rope(wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode))
         return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: three Q8_0/F16 matrices over one activation tensor of at most 16 tokens, NEOX rotation over the whole head, contiguous outputs");
     if (!pos || !wq->data || !wk->data || !wv->data || !x->data || !q_dst->data || !k_dst->data || !v_dst->data)
@@ -979,6 +1077,8 @@ extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk
     a.rp = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
     a.head_dim = n_dims;
     a.rope_T   = (int) q_dst->ne[2];
+    a.norm_w   = norm_w ? (const float *) norm_w->data : nullptr;
+    a.norm_eps = eps;
     const int nbatch = (int) x->ne[3];
     hipStream_t st = (hipStream_t) stream;
     bool ok;

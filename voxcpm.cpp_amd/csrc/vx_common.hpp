@@ -111,6 +111,27 @@ __device__ __forceinline__ double vx_wave_sum(double v) {
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
+// 1 / rms of one dense, 16-byte aligned row of ne00 <= 2048 floats, by one wave, exactly as the RMS_NORM
+// kernel's wave-per-row path forms it: fp32 squares, fp64 lane sums in float4 order, xor butterfly, one
+// rounding of the mean to fp32.  The same value in every lane.
+__device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00, int lane, float eps) {
+    const int64_t nvec = ne00 / 4;
+    double sum = 0.0;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int64_t iv = lane + (int64_t) c * 64;
+        if (iv < nvec) {
+            const float4 v = ((const float4 *) x)[iv];
+            sum += (double) (v.x * v.x);
+            sum += (double) (v.y * v.y);
+            sum += (double) (v.z * v.z);
+            sum += (double) (v.w * v.w);
+        }
+    }
+    sum = vx_wave_sum(sum);
+    const float mean = (float) (sum / (double) ne00);
+    return 1.0f / sqrtf(mean + eps);
+}
 __device__ __forceinline__ float vx_wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));

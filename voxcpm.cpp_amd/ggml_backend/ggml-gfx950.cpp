@@ -652,8 +652,13 @@ const ggml_tensor * rope_of_projection(const ggml_cgraph * g, int & idx, const g
     return r;
 }
 
+// norm / scale: the RMS_NORM and norm-weight MUL nodes right in front of the group when the normalised tensor has no
+// reader outside it (then i is the RMS_NORM's index and the group starts two nodes later), else null.
 bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, const absorbed_map & absorbed,
-                       std::unordered_set<const ggml_tensor *> & done, vx_status * rc) {
+                       std::unordered_set<const ggml_tensor *> & done, vx_status * rc, const ggml_tensor * norm = nullptr,
+                       const ggml_tensor * scale = nullptr) {
+    if (norm) i += 2;
+    if (i >= g->n_nodes || g->nodes[i]->op != GGML_OP_MUL_MAT) return false;
     const ggml_tensor * mq = g->nodes[i];
     int idx = i;
     const ggml_tensor * rq = rope_of_projection(g, idx, mq, readers, absorbed);
@@ -681,7 +686,8 @@ bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const re
     const int n_dims = ip[1], mode = ip[2], n_ctx_orig = ip[4];
     float fp[6];
     memcpy(fp, ip + 5, sizeof(fp));
-    const ggml_tensor * x = mq->src[1];
+    if (norm && mq->src[1] != scale) return false;
+    const ggml_tensor * x = norm ? norm->src[0] : mq->src[1];
     const ggml_tensor * outs[3] = { rq, rk, mv };
     for (int a = 0; a < 3; ++a) {
         if (!apart(outs[a], x)) return false;
@@ -689,9 +695,21 @@ bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const re
     }
     const vx_tensor wq = to_vx(mq->src[0]), wk = to_vx(mk->src[0]), wv = to_vx(mv->src[0]), xx = to_vx(x), dq = to_vx(rq), dk = to_vx(rk),
                     dv = to_vx(mv);
-    if (!vx_supports_qkv_proj_rope(&wq, &wk, &wv, &xx, &dq, &dk, &dv, n_dims, mode)) return false;
-    *rc = vx_qkv_proj_rope(&wq, &wk, &wv, &xx, (const int32_t *) rq->src[1]->data, rq->src[2] ? (const float *) rq->src[2]->data : nullptr,
-                           &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3], fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
+    const int32_t * posd = (const int32_t *) rq->src[1]->data;
+    const float *   ffd  = rq->src[2] ? (const float *) rq->src[2]->data : nullptr;
+    if (norm) {
+        const vx_tensor nw = to_vx(scale->src[1]);
+        float eps;
+        memcpy(&eps, norm->op_params, sizeof(float));
+        if (!vx_supports_norm_qkv_proj_rope(&xx, &nw, &wq, &wk, &wv, &dq, &dk, &dv, n_dims, mode) || (uintptr_t) xx.data % 16 || (uintptr_t) nw.data % 16) return false;
+        *rc = vx_norm_qkv_proj_rope(&xx, &nw, eps, &wq, &wk, &wv, posd, ffd, &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3],
+                                    fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
+        done.insert(scale); done.insert(mq);
+    } else {
+        if (!vx_supports_qkv_proj_rope(&wq, &wk, &wv, &xx, &dq, &dk, &dv, n_dims, mode)) return false;
+        *rc = vx_qkv_proj_rope(&wq, &wk, &wv, &xx, posd, ffd, &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3], fp[4], fp[5],
+                               mul_mat_act_mode(), ctx->stream);
+    }
     done.insert(rq); done.insert(mk); done.insert(rk); done.insert(mv);
     return true;
 }
@@ -731,6 +749,44 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         if (done.count(node)) continue;         // computed ahead of its turn by a group
         vx_status rc = VX_ERR_UNSUPPORTED;
         bool fused = false;
+        if (fusion && node->op == GGML_OP_RMS_NORM && i + 2 < cgraph->n_nodes) {
+            // MiniCPMModel::rms_norm (RMS_NORM, MUL by the norm weight) whose value only the projections behind it read:
+            // the normalisation joins their launch and the normalised tensor is never stored
+            ggml_tensor * mul = cgraph->nodes[i + 1];
+            const auto rd = [&](const ggml_tensor * t) { const auto it = readers.find(t); return it == readers.end() ? 0 : it->second; };
+            const bool norm_pair = mul->op == GGML_OP_MUL && mul->src[0] == node && mul->src[1] != node && rd(node) == 1 &&
+                                   (node->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (mul->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 &&
+                                   (mul->flags & GGML_TENSOR_FLAG_COMPUTE) != 0;
+            bool grouped = false;
+            if (norm_pair && rd(mul) == 3) {
+                grouped = compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc, node, mul);
+            } else if (norm_pair && rd(mul) == 2 && i + 4 < cgraph->n_nodes) {
+                ggml_tensor * gate = cgraph->nodes[i + 2];
+                ggml_tensor * up   = cgraph->nodes[i + 3];
+                ggml_tensor * glu  = cgraph->nodes[i + 4];
+                if (gate->op == GGML_OP_MUL_MAT && up->op == GGML_OP_MUL_MAT && glu->op == GGML_OP_GLU && gate->src[1] == mul && up->src[1] == mul &&
+                    glu->src[0] == gate && glu->src[1] == up && ggml_get_glu_op(glu) == GGML_GLU_OP_SWIGLU && ((const int32_t *) glu->op_params)[1] == 0 &&
+                    private_to_group(readers, gate) && private_to_group(readers, up) && (glu->flags & GGML_TENSOR_FLAG_COMPUTE) != 0) {
+                    const vx_tensor x = to_vx(node->src[0]), nw = to_vx(mul->src[1]), gw = to_vx(gate->src[0]), uw = to_vx(up->src[0]), d = to_vx(glu);
+                    float eps;
+                    memcpy(&eps, node->op_params, sizeof(float));
+                    if (vx_supports_norm_mul_mat_swiglu(&x, &nw, &gw, &uw, &d) && (uintptr_t) x.data % 16 == 0 && (uintptr_t) nw.data % 16 == 0 &&
+                        apart(glu, node->src[0])) {
+                        rc = vx_norm_mul_mat_swiglu(&x, &nw, eps, &gw, &uw, &d, mul_mat_act_mode(), ctx->stream);
+                        done.insert(mul); done.insert(gate); done.insert(up); done.insert(glu);
+                        grouped = true;
+                    }
+                }
+            }
+            if (grouped) {
+                ++launches;
+                if (rc != VX_OK) {
+                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, rms_norm + projections) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    return GGML_STATUS_FAILED;
+                }
+                continue;
+            }
+        }
         if (fusion && node->op == GGML_OP_MUL_MAT && compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc)) {
             ++launches;
             if (rc != VX_OK) {
