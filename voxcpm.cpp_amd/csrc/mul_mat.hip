@@ -401,6 +401,9 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         a0 = gp[0]; a1 = gp[1];
     };
     if (a.norm_w && tid < units) fetch_gain(tid, g0, g1);
+    // the row this wave normalises first (token wid), also requested ahead of the weights
+    vx_rms_row nrow;
+    if (a.norm_w && wid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) wid * a.nb11), a.K, lane);
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
@@ -420,7 +423,8 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     }
     if (a.norm_w) { // one wave per token, as the RMS_NORM kernel has it
         for (int t = wid; t < N; t += NW) {
-            const float sc = vx_rms_scale_wave((const float *) (xb + (uint64_t) t * a.nb11), a.K, lane, a.norm_eps);
+            if (t != wid) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
+            const float sc = vx_rms_row_scale(nrow, a.K, lane, a.norm_eps);
             if (lane == 0) nsc[t] = sc;
         }
         __syncthreads();

@@ -114,14 +114,24 @@ __device__ __forceinline__ double vx_wave_sum(double v) {
 // 1 / rms of one dense, 16-byte aligned row of ne00 <= 2048 floats, by one wave, exactly as the RMS_NORM
 // kernel's wave-per-row path forms it: fp32 squares, fp64 lane sums in float4 order, xor butterfly, one
 // rounding of the mean to fp32.  The same value in every lane.
-__device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00, int lane, float eps) {
+// The load and the arithmetic are separate so that a caller can request the row ahead of other traffic.
+struct vx_rms_row { float4 v[8]; };
+__device__ __forceinline__ void vx_rms_row_load(vx_rms_row & r, const float * x, int64_t ne00, int lane) {
+    const int64_t nvec = ne00 / 4;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int64_t iv = lane + (int64_t) c * 64;
+        r.v[c] = iv < nvec ? ((const float4 *) x)[iv] : float4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+}
+__device__ __forceinline__ float vx_rms_row_scale(const vx_rms_row & r, int64_t ne00, int lane, float eps) {
     const int64_t nvec = ne00 / 4;
     double sum = 0.0;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
         const int64_t iv = lane + (int64_t) c * 64;
         if (iv < nvec) {
-            const float4 v = ((const float4 *) x)[iv];
+            const float4 v = r.v[c];
             sum += (double) (v.x * v.x);
             sum += (double) (v.y * v.y);
             sum += (double) (v.z * v.z);
@@ -131,6 +141,11 @@ __device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00
     sum = vx_wave_sum(sum);
     const float mean = (float) (sum / (double) ne00);
     return 1.0f / sqrtf(mean + eps);
+}
+__device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00, int lane, float eps) {
+    vx_rms_row r;
+    vx_rms_row_load(r, x, ne00, lane);
+    return vx_rms_row_scale(r, ne00, lane, eps);
 }
 __device__ __forceinline__ float vx_wave_max(float v) {
 #pragma unroll
