@@ -204,6 +204,22 @@ VX_API vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_
 VX_API int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
                                           const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
                                           const vx_tensor * dst);
+/* The decode attention block of attention_forward (src/minicpm.cpp:682-713) as one call: vx_flash_attn_ext_kv2
+ * followed by vx_kv_store_sync on its result, with the cache write and the ordering scalar folded into the kernel
+ * that merges the key-range partials.  k_src / v_src are the CPY sources (the values of k_cur / v_cur in the shape
+ * the reference copies them), k_slot / v_slot the cache views written; sync_scale / sync_bias the SCALE node's
+ * parameters.  Needs more than 256 keys in all (the split path).  Result and cache contents equal the two
+ * separate calls'. */
+VX_API vx_status vx_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                             const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                             const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                             const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst,
+                                             float scale, float max_bias, float logit_softcap, float sync_scale,
+                                             float sync_bias, vx_stream stream);
+VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                                const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                                const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                                const vx_tensor * v_slot, const vx_tensor * dst);
 /* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
  * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for at most 16
  * tokens.  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE

@@ -11,13 +11,13 @@ from reflib import nmse, rng
 
 pytestmark = pytest.mark.gpu
 
-N_LAYER, MAX_LEN, BATCH, T0, STEPS = 3, 64, 2, 9, 3
+N_LAYER, BATCH, STEPS = 3, 2, 3
 
 
-def run_reference(params, xs, device, kv_f16, use_mup):
+def run_reference(params, xs, device, kv_f16, use_mup, max_len):
     ref = reflib.load_ref()
     assert ref.rh_use_device(device, 8, 0) == 0
-    reflib.ref_backbone_create(params, MAX_LEN, BATCH, use_mup=use_mup, kv_f16=kv_f16)
+    reflib.ref_backbone_create(params, max_len, BATCH, use_mup=use_mup, kv_f16=kv_f16)
     outs, n_past = [], 0
     for x in xs:
         T = x.shape[1]
@@ -30,21 +30,24 @@ def run_reference(params, xs, device, kv_f16, use_mup):
     return outs, n_nodes
 
 
-@pytest.mark.parametrize("kv_f16,use_mup", [(False, True), (True, False)])
-def test_backbone_three_ways(gpu, ref, kv_f16, use_mup):
+# prefill 9: decode attention over a dozen keys (one wave per tile); prefill 300: more than 256 keys, the
+# split + merge path with the cache write folded into the merge, as at the benchmark's KV lengths
+@pytest.mark.parametrize("kv_f16,use_mup,T0", [(False, True, 9), (True, False, 9), (False, True, 300)])
+def test_backbone_three_ways(gpu, ref, kv_f16, use_mup, T0):
     import torch
     from voxcpm_cpp_amd import backbone as bb
+    MAX_LEN = T0 + 55
     print(f"backbone: {N_LAYER} layers, batch {BATCH}, prefill {T0} + {STEPS} decode steps, kv_f16={kv_f16} mup={use_mup}", flush=True)
     params = reflib.backbone_params("bb", N_LAYER)
     xs = [rng("bb", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)]
     xs += [rng("bb", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(STEPS)]
 
-    cpu, n_nodes = run_reference(params, xs, b"CPU", kv_f16, use_mup)
+    cpu, n_nodes = run_reference(params, xs, b"CPU", kv_f16, use_mup, MAX_LEN)
     print(f"   ggml-cpu graph: {n_nodes} nodes per decode step", flush=True)
 
     # the same ggml graph, every node on the plugin (direct ggml_backend_graph_compute, no scheduler)
     assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
-    plug, _ = run_reference(params, xs, b"GFX950_0", kv_f16, use_mup)
+    plug, _ = run_reference(params, xs, b"GFX950_0", kv_f16, use_mup, MAX_LEN)
     import ctypes
     plugin_launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()  # of the last decode step
     print(f"   plugin: {plugin_launches} operator launches for the {n_nodes}-node decode graph", flush=True)

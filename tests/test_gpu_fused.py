@@ -398,3 +398,45 @@ def test_norm_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act):
        "norm_qkv_proj_rope")
     torch.cuda.synchronize()
     assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@pytest.mark.parametrize("T,n_past,B,Hkv,D", [(1, 639, 2, 2, 64), (1, 300, 1, 2, 64), (2, 1000, 2, 4, 128), (3, 4000, 2, 2, 64)])
+@pytest.mark.parametrize("poison", [None, "nan"])
+def test_flash_attn_two_segments_with_cache_write(pkg, gpu, T, n_past, B, Hkv, D, poison):
+    import torch
+    say(f"attention over cached + current keys with the cache write folded in T={T} n_past={n_past} B={B} Hkv={Hkv} D={D} {poison}")
+    L, d = pkg.lib(), pkg.desc
+    H = 8 * Hkv
+    g = rng("f-kv2s", T, n_past, B, D)
+    q = dev(g.standard_normal((B, H, T, D)).astype(np.float32))
+    caches = [dev(g.standard_normal((B, Hkv, n_past + T + 5, D)).astype(np.float32)) for _ in range(2)]
+    caches += [c.clone() for c in caches]
+    kc1, vc1, kc2, vc2 = caches
+    k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))   # as the projection + rope leave them
+    v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    if poison:
+        v[0, 0, 0, 3] = float("nan")
+    kcur, vcur = k.transpose(1, 2), v.transpose(1, 2)
+    mask = dev(reflib.causal_mask(T, n_past + T, n_past)) if T > 1 else None
+    sc = 1.0 / np.sqrt(D)
+
+    def slot(c):
+        return c[:, :, n_past:n_past + T].transpose(1, 2)
+
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    for sync_scale, sync_bias in ((0.0, 0.0), (0.125, 0.5)):
+        ok(pkg, L.vx_flash_attn_ext_kv2(d(q), d(kc1[:, :, :n_past]), d(kcur), d(vc1[:, :, :n_past]), d(vcur), d(mask), None, d(a), sc, 0.0, 0.0, None), "kv2")
+        ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc1)), d(v), d(slot(vc1)), d(a), d(a), sync_scale, sync_bias, None), "kv_store_sync")
+        assert L.vx_supports_flash_attn_ext_kv2_store(d(q), d(kc2[:, :, :n_past]), d(kcur), d(vc2[:, :, :n_past]), d(vcur), d(mask),
+                                                      d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b)) == 1
+        ok(pkg, L.vx_flash_attn_ext_kv2_store(d(q), d(kc2[:, :, :n_past]), d(kcur), d(vc2[:, :, :n_past]), d(vcur), d(mask), None,
+                                              d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b), sc, 0.0, 0.0, sync_scale, sync_bias, None), "kv2_store")
+        torch.cuda.synchronize()
+        assert same_bits(kc1, kc2) and same_bits(vc1, vc2)
+        assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(7.0), b.nan_to_num(7.0))
+        if poison:
+            assert bool(torch.isnan(b).all())
+    # too few keys for the split path: refused, the separate calls remain
+    assert L.vx_supports_flash_attn_ext_kv2_store(d(q), d(kc2[:, :, :100]), d(kcur), d(vc2[:, :, :100]), d(vcur), None,
+                                                  d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b)) == 0

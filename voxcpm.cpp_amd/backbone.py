@@ -169,6 +169,7 @@ class MiniCPMBackbone:
             # from here on in the order ggml_build_forward_expand gives the reference's graph: concat, attention,
             # then the cache append with its ordering chain, then add1 (only adjacent nodes are run as one launch)
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)
+            stored = False
             if n_past > 0:
                 if kcast is not None:
                     call(L.vx_cpy, desc(k_all), desc(kcast))
@@ -181,7 +182,17 @@ class MiniCPMBackbone:
                 # cache write, their other reader, comes later: F32 cache with write_kv.  The F16 cast of the
                 # current keys dies at the concat and ggml-alloc hands its memory on, so there the concats stay.
                 alive = write_kv and kcast is None
-                if fuse and alive and L.vx_supports_flash_attn_ext_kv2(qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), desc(attn)):
+                kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # the cache's write views, ggml [D, Hkv, T, B]
+                vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
+                if fuse and alive and L.vx_supports_flash_attn_ext_kv2_store(qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask),
+                                                                             desc(k4), desc(kw), desc(v4), desc(vw), desc(attn)):
+                    # attention, the cache write and its ordering scalar as one call (two kernels)
+                    keep += [kw, vw]
+                    call(L.vx_flash_attn_ext_kv2_store, qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), None,
+                         desc(k4), desc(kw), desc(v4), desc(vw), desc(attn), scale, 0.0, 0.0, 0.0, 0.0)
+                    k_all = None
+                    stored = True
+                elif fuse and alive and L.vx_supports_flash_attn_ext_kv2(qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), desc(attn)):
                     call(L.vx_flash_attn_ext_kv2, qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask), None, desc(attn),
                          scale, 0.0, 0.0)
                     k_all = None
@@ -192,13 +203,15 @@ class MiniCPMBackbone:
             if k_all is not None:
                 call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
                      scale, 0.0, 0.0)
-            grouped = False
-            if write_kv:
+            grouped = stored
+            if write_kv and not stored:
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236
                 vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
                 keep += [kw, vw]
                 grouped = bool(chain and fuse and L.vx_supports_kv_store_sync(desc(k4), desc(kw), desc(v4), desc(vw), desc(attn), desc(attn)))
-            if grouped:      # both cache writes, their sums, add, scale and add1 as one launch
+            if stored:
+                pass
+            elif grouped:      # both cache writes, their sums, add, scale and add1 as one launch
                 call(L.vx_kv_store_sync, desc(k4), desc(kw), desc(v4), desc(vw), desc(attn), desc(attn), 0.0, 0.0)
             elif write_kv:
                 for src4, wv, cont, ssum in ((k4, kw, kcont, sk), (v4, vw, vcont, sv)):

@@ -33,6 +33,7 @@
 // (one tile per KV head) that is n_kv * D * 2 * sizeof(kv) per (b, g), the figure the
 // benchmark divides by.
 #include "vx_common.hpp"
+#include "kvs_common.hpp"
 
 #include <cmath>
 #include <cstdlib>
@@ -49,6 +50,11 @@ struct fa_args {
     uint64_t nbq1, nbq2, nbq3, nbk1, nbk2, nbk3, nbv1, nbv2, nbv3, nbm1, nbm2, nbm3;
     // keys n_kv1 .. n_kv-1 may lie in a second pair of tensors (the current step's K and V, which the
     // reference appends to the cached ones with GGML_OP_CONCAT before attention); null = one segment
+    // the reference's cache write with its ordering scalar folded into the merge kernel (has_kvs):
+    // block 0 stores both slots, every block forms the two sums and adds the scalar to its column
+    kvs_side kvs_k, kvs_v;
+    float kvs_scale, kvs_bias;
+    int has_kvs;
     const char * k2; const char * v2;
     uint64_t nbk1b, nbk2b, nbk3b, nbv1b, nbv2b, nbv3b;
     int n_kv1;
@@ -100,7 +106,8 @@ template <int NP, bool KV_F32> struct kv_tile {
 // sinks (ops.cpp:8306-8322), normalisation and the permuted store of ggml's result for 4
 // consecutive d of one column
 __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float M, float L, int b, int g, int col,
-                                          int D, int d0) {
+                                          int D, int d0, bool has_addend, float addend) {
+#pragma clang fp contract(off) // the normalised value is rounded before the addend joins it, as two nodes would
     const int iq1 = col / a.gqa, head = g * a.gqa + col % a.gqa;
     if (a.sinks) {
         const float sk = a.sinks[head] * 1.44269504088896341f; // M is in the log2 domain
@@ -111,7 +118,7 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
     }
     const float inv = L == 0.0f ? 0.0f : 1.0f / L;
     float4_t r = acc * inv;
-    if (a.add1) r += *a.add1; // rounded after the normalisation, as the separate ADD1 node would
+    if (has_addend) r += addend; // rounded after the normalisation, as the separate ADD1 node would
     *(float4_t *) (a.dst + (((uint64_t) b * a.n_q + iq1) * a.Hq + head) * D + d0) = r;
 }
 
@@ -338,7 +345,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         for (int p = 0; p < NP; ++p)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
-                fa_finish(a, o[p][u], m, l, b, g, col, D, SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1));
+                fa_finish(a, o[p][u], m, l, b, g, col, D, SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1), a.add1 != nullptr, a.add1 ? *a.add1 : 0.0f);
     } else {
         const uint64_t pbase = ((uint64_t) tile * a.n_splits + sp) * 16 + c;
 #pragma unroll
@@ -369,6 +376,8 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     const int col = ct * 16 + c;
     if (col >= a.n_q * a.gqa) return;
     const int lane = threadIdx.x, q = lane / DU, d0 = 4 * (lane % DU);
+    bool  has_addend = a.add1 != nullptr;
+    float addend     = has_addend ? *a.add1 : 0.0f;
     const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + c; // + split * 16
     const int nsl = (a.n_splits + 63) >> 6;                         // (max, sum) pairs per lane
 
@@ -393,6 +402,13 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     };
     load_rows(0);
 
+    if (a.has_kvs) { // the sources are a few hundred floats: every block re-forms the sums, the first one stores
+        const bool   store = blockIdx.x == 0;
+        const double tk = a.kvs_k.vec ? kvs_wave_total<true>(a.kvs_k, lane, store) : kvs_wave_total<false>(a.kvs_k, lane, store);
+        const double tv = a.kvs_v.vec ? kvs_wave_total<true>(a.kvs_v, lane, store) : kvs_wave_total<false>(a.kvs_v, lane, store);
+        addend     = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
+        has_addend = true;
+    }
     float M = m[0];
 #pragma unroll
     for (int i = 1; i < FA_MERGE_MAX_SPLITS / 64; ++i) M = fmaxf(M, m[i]);
@@ -424,7 +440,7 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     for (int off = DU; off < 64; off <<= 1)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], off, 64);
-    if (q == 0) fa_finish(a, acc, M, L, b, g, col, D, d0);
+    if (q == 0) fa_finish(a, acc, M, L, b, g, col, D, d0, has_addend, addend);
 }
 
 int g_num_cus = 0;
@@ -441,6 +457,34 @@ int num_cus() {
 
 bool aligned16(const vx_tensor * t) {
     return ((uintptr_t) t->data % 16 == 0) && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+}
+
+// Work split.  Enough 16-column tiles to fill the chip: one wave per tile over all keys.
+// Otherwise cut the keys (flash-decoding) aiming at ~4 waves per CU, at least `min_chunk`
+// keys per wave, and merge the partials with a second small kernel.
+void fa_split_plan(int64_t tiles, int n_kv, int * n_splits, int * chunk_out) {
+    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 64; }();
+    *n_splits  = 1;
+    *chunk_out = (n_kv + 31) / 32 * 32;
+    // Up to 256 keys one wave finishes (0.5 us per 32-key step) before a split plus the merge
+    // launch would.
+    static const int waves_per_cu = [] { const char * e = getenv("VX_FA_WAVES_PER_CU"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 32 ? v : 4; }();
+    if (tiles < (int64_t) waves_per_cu * num_cus() && n_kv > 256) {
+        int64_t want = ((int64_t) waves_per_cu * num_cus() + tiles - 1) / tiles;
+        const int64_t max_splits = (n_kv + min_chunk - 1) / min_chunk;
+        if (want > max_splits) want = max_splits;
+        if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;
+        if (want < 1) want = 1;
+        int chunk  = (int) ((n_kv + want - 1) / want);
+        chunk      = (chunk + 31) / 32 * 32;
+        *chunk_out = chunk;
+        *n_splits  = (n_kv + chunk - 1) / chunk;
+    }
+}
+
+int64_t fa_tiles(const vx_tensor * q, const vx_tensor * k) {
+    const int64_t gqa = q->ne[2] / k->ne[2];
+    return q->ne[3] * k->ne[2] * ((q->ne[1] * gqa + 15) / 16);
 }
 
 template <int D, bool KV_F32>
@@ -500,7 +544,9 @@ extern "C" vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k,
 static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * k2, const vx_tensor * v2,
                         const vx_tensor * kall, const vx_tensor * vall, const vx_tensor * mask, const float * sinks,
                         const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
-                        hipStream_t st);
+                        hipStream_t st, const vx_tensor * ks_src = nullptr, const vx_tensor * ks_slot = nullptr,
+                        const vx_tensor * vs_src = nullptr, const vx_tensor * vs_slot = nullptr, float kvs_scale = 0.0f,
+                        float kvs_bias = 0.0f);
 
 extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
                                             const vx_tensor * mask, const float * sinks, const float * addend,
@@ -566,12 +612,53 @@ extern "C" vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor 
     return fa_run(q, k_past, v_past, k_cur, v_cur, &kall, &vall, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream);
 }
 
+// The reference's decode attention block in two kernels: attention over cached + current keys, with the cache
+// write and its ordering scalar (CPY CONT SUM x2, ADD, SCALE, ADD1; src/minicpm.cpp:682-713) folded into the
+// kernel that merges the key-range partials.  k_src / v_src are the CPY sources (the same values as k_cur /
+// v_cur, in the shape the reference copies them), k_slot / v_slot the cache views they are written to.
+extern "C" int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                                    const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                                    const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                                    const vx_tensor * v_slot, const vx_tensor * dst) {
+    if (!vx_supports_flash_attn_ext_kv2(q, k_past, k_cur, v_past, v_cur, mask, dst)) return 0;
+    if (!kvs_side_ok(k_src, k_slot) || !kvs_side_ok(v_src, v_slot)) return 0;
+    vx_tensor kall;
+    kv2_whole(k_past, k_cur, &kall);
+    int n_splits, chunk;
+    fa_split_plan(fa_tiles(q, &kall), (int) kall.ne[1], &n_splits, &chunk);
+    return n_splits > 1; // the write rides on the merge kernel
+}
+
+extern "C" vx_status vx_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
+                                                 const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
+                                                 const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                                 const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst, float scale,
+                                                 float max_bias, float logit_softcap, float sync_scale, float sync_bias,
+                                                 vx_stream stream) {
+    if (!q || !k_past || !k_cur || !v_past || !v_cur || !k_src || !k_slot || !v_src || !v_slot || !dst || !q->data || !k_past->data ||
+        !k_cur->data || !v_past->data || !v_cur->data || !k_src->data || !k_slot->data || !v_src->data || !v_slot->data || !dst->data ||
+        (mask && !mask->data))
+        return vx_fail(VX_ERR_INVALID, "flash_attn_ext_kv2_store: null tensor");
+    if (!vx_supports_flash_attn_ext_kv2_store(q, k_past, k_cur, v_past, v_cur, mask, k_src, k_slot, v_src, v_slot, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_kv2_store: as flash_attn_ext_kv2 with more than 256 keys, F32 cache writes of at most 16384 elements");
+    if (!aligned16(q) || !aligned16(k_past) || !aligned16(v_past) || !aligned16(k_cur) || !aligned16(v_cur) || (uintptr_t) dst->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_kv2_store: tensor data must be 16-byte aligned");
+    if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_kv2_store: max_bias > 0 requires a mask");
+    vx_tensor kall, vall;
+    kv2_whole(k_past, k_cur, &kall);
+    kv2_whole(v_past, v_cur, &vall);
+    return fa_run(q, k_past, v_past, k_cur, v_cur, &kall, &vall, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream,
+                  k_src, k_slot, v_src, v_slot, sync_scale, sync_bias);
+}
+
 static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * k2, const vx_tensor * v2,
                         const vx_tensor * kall, const vx_tensor * vall, const vx_tensor * mask, const float * sinks,
                         const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
-                        hipStream_t st) {
+                        hipStream_t st, const vx_tensor * ks_src, const vx_tensor * ks_slot, const vx_tensor * vs_src,
+                        const vx_tensor * vs_slot, float kvs_scale, float kvs_bias) {
     (void) vall;
     fa_args a;
+    a.has_kvs = 0;
     a.k2 = k2 ? (const char *) k2->data : nullptr; a.v2 = v2 ? (const char *) v2->data : nullptr;
     a.nbk1b = k2 ? k2->nb[1] : 0; a.nbk2b = k2 ? k2->nb[2] : 0; a.nbk3b = k2 ? k2->nb[3] : 0;
     a.nbv1b = v2 ? v2->nb[1] : 0; a.nbv2b = v2 ? v2->nb[2] : 0; a.nbv3b = v2 ? v2->nb[3] : 0;
@@ -602,25 +689,13 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     a.n_col_tiles   = (ncols + 15) / 16;
     const int64_t tiles = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
 
-    // Work split.  Enough 16-column tiles to fill the chip: one wave per tile over all keys.
-    // Otherwise cut the keys (flash-decoding) aiming at ~4 waves per CU, at least `min_chunk`
-    // keys per wave, and merge the partials with a second small kernel.
-    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 64; }();
-    a.n_splits = 1;
-    a.chunk    = (a.n_kv + 31) / 32 * 32;
-    // Up to 256 keys one wave finishes (0.5 us per 32-key step) before a split plus the merge
-    // launch would.
-    static const int waves_per_cu = [] { const char * e = getenv("VX_FA_WAVES_PER_CU"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 32 ? v : 4; }();
-    if (tiles < (int64_t) waves_per_cu * num_cus() && a.n_kv > 256) {
-        int64_t want = ((int64_t) waves_per_cu * num_cus() + tiles - 1) / tiles;
-        const int64_t max_splits = (a.n_kv + min_chunk - 1) / min_chunk;
-        if (want > max_splits) want = max_splits;
-        if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;
-        if (want < 1) want = 1;
-        int chunk  = (int) ((a.n_kv + want - 1) / want);
-        chunk      = (chunk + 31) / 32 * 32;
-        a.chunk    = chunk;
-        a.n_splits = (a.n_kv + chunk - 1) / chunk;
+    fa_split_plan(tiles, a.n_kv, &a.n_splits, &a.chunk);
+    if (ks_src) {
+        if (a.n_splits == 1) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_kv2_store: needs a key count that is split across waves");
+        kvs_side_fill(a.kvs_k, ks_src, ks_slot);
+        kvs_side_fill(a.kvs_v, vs_src, vs_slot);
+        a.kvs_scale = kvs_scale; a.kvs_bias = kvs_bias;
+        a.has_kvs = 1;
     }
 
     const int64_t nblocks = tiles * a.n_splits;

@@ -9,6 +9,7 @@
 // rows are flattened over (i1, i2, i3).  VEC = 4 (16-byte accesses) when every operand is dense
 // and 16-byte aligned along dim 0, VEC = 1 otherwise (any strides, ggml's broadcast rules).
 #include "vx_common.hpp"
+#include "kvs_common.hpp"
 
 #include <cmath>
 
@@ -291,13 +292,6 @@ __global__ __launch_bounds__(64) void sum_partials_kernel(const double * partial
 // one the separate nodes produce, NaN and infinity included) and writes dst = x + scalar.
 constexpr int KVS_PRE = 4; // x elements per thread requested before anything else
 
-struct kvs_side {
-    const char * s; char * d;
-    int64_t  nes[4], ned[4];
-    uint64_t nbs[4], nbd[4];
-    int vec; // slot rows allow 16-byte accesses: the test vx_sum applies to its operand
-};
-
 struct kvs_args {
     kvs_side k, v;
     const char * x; char * d;
@@ -308,30 +302,9 @@ struct kvs_args {
 
 template <bool VEC>
 __device__ __forceinline__ double store_and_sum(const kvs_side & a) {
-    constexpr int W = VEC ? 4 : 1;
-    const uint32_t ne0 = (uint32_t) a.ned[0], per_row = ne0 / W;
-    const uint32_t n = per_row * (uint32_t) (a.ned[1] * a.ned[2] * a.ned[3]);
-    const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
-    const uint32_t s0n = (uint32_t) a.nes[0], s1n = (uint32_t) a.nes[1], s2n = (uint32_t) a.nes[2];
+    const uint32_t n = kvs_units(a, VEC);
     double acc = 0.0;
-    for (uint32_t e = threadIdx.x; e < n; e += 1024) {
-        const uint32_t row = e / per_row, iv = e - row * per_row;
-        const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
-        char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
-        float v[W];
-#pragma unroll
-        for (int k = 0; k < W; ++k) { // element number row * ne0 + iv * W + k of the source, in its own shape
-            uint32_t r = row * ne0 + iv * W + k;
-            const uint32_t j0 = r % s0n; r /= s0n;
-            const uint32_t j1 = r % s1n; r /= s1n;
-            const uint32_t j2 = r % s2n, j3 = r / s2n;
-            v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
-        }
-        if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
-        else               *(float *) pd = v[0];
-#pragma unroll
-        for (int k = 0; k < W; ++k) acc += (double) v[k];
-    }
+    for (uint32_t e = threadIdx.x; e < n; e += 1024) kvs_unit<VEC>(a, e, true, acc);
     return acc;
 }
 
@@ -359,8 +332,7 @@ __global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
     const float  sk = (float) block_total(ak, part);
     const double av = a.v.vec ? store_and_sum<true>(a.v) : store_and_sum<false>(a.v);
     const float  sv = (float) block_total(av, part);
-    const float  t  = sk + sv;                                                  // the ADD node
-    const float  y  = a.bias == 0.0f ? t * a.scale : fmaf(t, a.scale, a.bias);  // the SCALE node
+    const float  y  = kvs_scalar(sk, sv, a.scale, a.bias);
 #pragma unroll
     for (int p = 0; p < KVS_PRE; ++p)
         if (threadIdx.x + 1024 * p < nx) *(float *) (a.d + xo[p]) = xv[p] + y;  // the ADD1 node
@@ -588,12 +560,6 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
     return VX_OK;
 }
 
-static bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot) {
-    if (!f32(src) || !f32(slot) || !vx_positive(src)) return false;
-    if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > 16384) return false;
-    return slot->nb[0] == 4 && nb_multiple(slot, 4) && nb_multiple(src, 4);
-}
-
 extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                          const vx_tensor * x, const vx_tensor * dst) {
     if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;
@@ -608,13 +574,8 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
         return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors, at most 16384 elements per cache write and 65536 in x");
     if (!k->data || !k_slot->data || !v->data || !v_slot->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "kv_store_sync: null data");
     kvs_args a;
-    auto side = [](kvs_side & o, const vx_tensor * src, const vx_tensor * slot) {
-        o.s = (const char *) src->data; o.d = (char *) slot->data;
-        for (int i = 0; i < 4; ++i) { o.nes[i] = src->ne[i]; o.ned[i] = slot->ne[i]; o.nbs[i] = src->nb[i]; o.nbd[i] = slot->nb[i]; }
-        o.vec = slot->ne[0] % 4 == 0 && al16(slot->data, slot->nb);
-    };
-    side(a.k, k, k_slot);
-    side(a.v, v, v_slot);
+    kvs_side_fill(a.k, k, k_slot);
+    kvs_side_fill(a.v, v, v_slot);
     a.x = (const char *) x->data; a.d = (char *) dst->data;
     for (int i = 0; i < 4; ++i) { a.ne[i] = x->ne[i]; a.nbx[i] = x->nb[i]; a.nbd[i] = dst->nb[i]; }
     a.scale = scale; a.bias = bias;

@@ -1,0 +1,84 @@
+// kvs_common.hpp -- the cache write of attention_forward with its ordering sums, shared by the one-block
+// kernel that runs the whole nine-node group and by the attention merge kernel that folds the group in.
+#pragma once
+#include "vx_common.hpp"
+
+// one cache write: source tensor (F32, any strides) -> slot view of the cache (F32, dense rows); element i
+// of the source in its own row-major order goes to element i of the slot in the slot's
+struct kvs_side {
+    const char * s; char * d;
+    int64_t  nes[4], ned[4];
+    uint64_t nbs[4], nbd[4];
+    int vec; // slot rows allow 16-byte accesses: the test vx_sum applies to its operand
+};
+
+// host side: what one cache write may look like, and its kernel argument
+static inline bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot) {
+    if (!src || !slot || src->type != VX_TYPE_F32 || slot->type != VX_TYPE_F32 || !vx_positive(src)) return false;
+    if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > 16384) return false;
+    for (int i = 0; i < 4; ++i) if (src->nb[i] % 4 || slot->nb[i] % 4) return false;
+    return slot->nb[0] == 4;
+}
+static inline void kvs_side_fill(kvs_side & o, const vx_tensor * src, const vx_tensor * slot) {
+    o.s = (const char *) src->data; o.d = (char *) slot->data;
+    for (int i = 0; i < 4; ++i) { o.nes[i] = src->ne[i]; o.ned[i] = slot->ne[i]; o.nbs[i] = src->nb[i]; o.nbd[i] = slot->nb[i]; }
+    o.vec = slot->ne[0] % 4 == 0 && (uintptr_t) slot->data % 16 == 0 && slot->nb[1] % 16 == 0 && slot->nb[2] % 16 == 0 && slot->nb[3] % 16 == 0;
+}
+
+#ifdef __HIPCC__
+// Unit e of the slot (4 consecutive elements when VEC, else one): fetch from the source, optionally store,
+// add to acc in element order -- the inner step of GGML_OP_SUM's walk over the written slot.
+template <bool VEC>
+__device__ __forceinline__ void kvs_unit(const kvs_side & a, uint32_t e, bool store, double & acc) {
+    constexpr int W = VEC ? 4 : 1;
+    const uint32_t ne0 = (uint32_t) a.ned[0], per_row = ne0 / W;
+    const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
+    const uint32_t s0n = (uint32_t) a.nes[0], s1n = (uint32_t) a.nes[1], s2n = (uint32_t) a.nes[2];
+    const uint32_t row = e / per_row, iv = e - row * per_row;
+    const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
+    char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+    float v[W];
+#pragma unroll
+    for (int k = 0; k < W; ++k) { // element number row * ne0 + iv * W + k of the source, in its own shape
+        uint32_t r = row * ne0 + iv * W + k;
+        const uint32_t j0 = r % s0n; r /= s0n;
+        const uint32_t j1 = r % s1n; r /= s1n;
+        const uint32_t j2 = r % s2n, j3 = r / s2n;
+        v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
+    }
+    if (store) {
+        if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
+        else               *(float *) pd = v[0];
+    }
+#pragma unroll
+    for (int k = 0; k < W; ++k) acc += (double) v[k];
+}
+
+__device__ __forceinline__ uint32_t kvs_units(const kvs_side & a, bool vec) {
+    return (uint32_t) (a.ned[0] / (vec ? 4 : 1)) * (uint32_t) (a.ned[1] * a.ned[2] * a.ned[3]);
+}
+
+// The sum a 1024-thread block forms (thread t walks units t, t + 1024, ...; each wave reduces by xor
+// butterfly; the 16 wave totals are added in order), formed by ONE wave that plays the 16 waves in turn:
+// the same additions in the same order, so the same double.
+template <bool VEC>
+__device__ __forceinline__ double kvs_wave_total(const kvs_side & a, int lane, bool store) {
+    const uint32_t n = kvs_units(a, VEC);
+    double total = 0.0;
+    int w = 0;
+    for (; w < 16; ++w) {
+        if ((uint32_t) w * 64 >= n) break; // the remaining waves of the block would hold no unit
+        double acc = 0.0;
+        for (uint32_t e = (uint32_t) w * 64 + lane; e < n; e += 1024) kvs_unit<VEC>(a, e, store, acc);
+        total += vx_wave_sum(acc);
+    }
+    if (w < 16) total += 0.0; // their zeros, added once (it only matters for the sign of a zero total)
+    return total;
+}
+
+// the scalar the reference adds to the attention output: (sum(k_slot) + sum(v_slot)) * scale + bias
+__device__ __forceinline__ float kvs_scalar(float sk, float sv, float scale, float bias) {
+    const float t = sk + sv;                                       // the ADD node
+    return bias == 0.0f ? t * scale : fmaf(t, scale, bias);        // the SCALE node
+}
+#endif

@@ -24,6 +24,7 @@
 
 #include "voxcpm_gfx950.h"
 
+#include <cstddef>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -424,6 +425,30 @@ bool overlaps(const ggml_tensor * a, const ggml_tensor * b) {
 }
 // operand that work-groups other than the one writing an output element read: must not touch dst
 bool apart(const ggml_tensor * dst, const ggml_tensor * in) { return !overlaps(dst, in); }
+// Two views that interleave in memory without sharing an element, like the cached keys [0, n_past) and the slot
+// being written [n_past, n_past + n_tokens) of one KV cache tensor: every row of the small view is located in
+// the regular lattice of the big one (rows of ne0 elements every nb1 bytes, ne1 of them every nb2, ...).
+bool apart_rows(const ggml_tensor * small, const ggml_tensor * big) {
+    if (!overlaps(small, big)) return true;
+    const size_t es = ggml_type_size(big->type);
+    if (ggml_is_quantized(big->type) || ggml_is_quantized(small->type) || small->nb[0] != ggml_type_size(small->type) || big->nb[0] != es) return false;
+    const int64_t big_row = (int64_t) (es * big->ne[0]), len = (int64_t) (small->nb[0] * small->ne[0]);
+    if ((int64_t) big->nb[1] < big_row || big->nb[2] < big->nb[1] * (size_t) big->ne[1] || big->nb[3] < big->nb[2] * (size_t) big->ne[2]) return false;
+    if (small->ne[1] * small->ne[2] * small->ne[3] > 65536) return false;
+    for (int64_t i3 = 0; i3 < small->ne[3]; ++i3)
+        for (int64_t i2 = 0; i2 < small->ne[2]; ++i2)
+            for (int64_t i1 = 0; i1 < small->ne[1]; ++i1) {
+                const int64_t o = ((const char *) small->data + i1 * small->nb[1] + i2 * small->nb[2] + i3 * small->nb[3]) - (const char *) big->data;
+                if (o + len <= 0) continue;
+                if (o < 0) return false;
+                const int64_t j3 = o / (int64_t) big->nb[3], r3 = o % (int64_t) big->nb[3];
+                const int64_t j2 = r3 / (int64_t) big->nb[2], r2 = r3 % (int64_t) big->nb[2];
+                const int64_t j1 = r2 / (int64_t) big->nb[1], rem = r2 % (int64_t) big->nb[1];
+                if (rem + len > (int64_t) big->nb[1]) return false; // reaches into the next row: not worth deciding
+                if (j3 < big->ne[3] && j2 < big->ne[2] && j1 < big->ne[1] && rem < big_row) return false;
+            }
+    return true;
+}
 // operand whose element i is read only by the thread that writes element i of dst: may also BE dst
 bool apart_or_same(const ggml_tensor * dst, const ggml_tensor * in) {
     if (!overlaps(dst, in)) return true;
@@ -510,8 +535,8 @@ int next_real(const ggml_cgraph * g, int i) {
 // attention_forward's cache write and ordering scalar (src/minicpm.cpp:682-713) at decode size:
 //   CPY(k, slot) CONT SUM , CPY(v, slot) CONT SUM , ADD , SCALE , ADD1(attn, .)     -> one launch.
 // Returns the index of the group's last node, or -1.
-int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
-    ggml_tensor * n[9];
+// the nine nodes from index i on, checked for shape and privacy; returns the index of the last one or -1
+int match_kv_store_group(const ggml_cgraph * g, int i, const reader_map & readers, ggml_tensor * n[9]) {
     int idx = i;
     for (int k = 0; k < 9; ++k) {
         if (idx >= g->n_nodes) return -1;
@@ -534,6 +559,15 @@ int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, cons
     ggml_tensor * dst = n[8];
     if (!apart(dst, n[0]->src[0]) || !apart(dst, n[3]->src[0]) || !apart(dst, n[0]) || !apart(dst, n[3]) || !apart_or_same(dst, x)) return -1;
     if (!apart(n[0], x) || !apart(n[3], x) || !apart(n[0], n[3]->src[0]) || !apart(n[3], n[0]->src[0]) || !apart(n[0], n[3])) return -1;
+    return idx;
+}
+
+int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
+    ggml_tensor * n[9];
+    const int idx = match_kv_store_group(g, i, readers, n);
+    if (idx < 0) return -1;
+    ggml_tensor * x = n[8]->src[0];
+    ggml_tensor * dst = n[8];
     const vx_tensor k = to_vx(n[0]->src[0]), ks = to_vx(n[0]), v = to_vx(n[3]->src[0]), vs = to_vx(n[3]), xx = to_vx(x), d = to_vx(dst);
     if (!vx_supports_kv_store_sync(&k, &ks, &v, &vs, &xx, &d)) return -1;
     float sc, bias;
@@ -611,6 +645,37 @@ void find_kv2_groups(const ggml_cgraph * g, const reader_map & readers, std::uno
         absorbed[cat[0]] = f;
         absorbed[cat[1]] = f;
     }
+}
+
+// FLASH_ATTN_EXT over absorbed CONCATs directly followed by the cache-write group on its result (the decode
+// step of attention_forward): one call, the write rides on the kernel that merges the key-range partials.
+// Returns the index of the group's last node, or -1.
+int compute_kv2_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i, const kv2_group & grp, const reader_map & readers, vx_status * rc) {
+    const ggml_tensor * f = g->nodes[i];
+    const int j = next_real(g, i);
+    if (j >= g->n_nodes || g->nodes[j]->op != GGML_OP_CPY || !private_to_group(readers, f)) return -1;
+    ggml_tensor * n[9];
+    const int last = match_kv_store_group(g, j, readers, n);
+    if (last < 0 || n[8]->src[0] != f) return -1;
+    const ggml_tensor * dst = n[8];
+    const ggml_tensor * reads[] = { f->src[0], f->src[3], f->src[4], grp.kcat->src[0], grp.kcat->src[1], grp.vcat->src[0], grp.vcat->src[1] };
+    for (const ggml_tensor * r : reads)
+        if (r && (!apart(dst, r) || !apart_rows(n[0], r) || !apart_rows(n[3], r))) return -1;
+    float scale, max_bias, softcap, sc, bias;
+    memcpy(&scale, (const float *) f->op_params + 0, sizeof(float));
+    memcpy(&max_bias, (const float *) f->op_params + 1, sizeof(float));
+    memcpy(&softcap, (const float *) f->op_params + 2, sizeof(float));
+    memcpy(&sc, (const float *) n[7]->op_params + 0, sizeof(float));
+    memcpy(&bias, (const float *) n[7]->op_params + 1, sizeof(float));
+    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcat->src[1]), vp = to_vx(grp.vcat->src[0]),
+                    vc = to_vx(grp.vcat->src[1]), ksrc = to_vx(n[0]->src[0]), ks = to_vx(n[0]), vsrc = to_vx(n[3]->src[0]), vs = to_vx(n[3]),
+                    d = to_vx(dst);
+    vx_tensor m;
+    if (f->src[3]) m = to_vx(f->src[3]);
+    if (!vx_supports_flash_attn_ext_kv2_store(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, &ksrc, &ks, &vsrc, &vs, &d)) return -1;
+    *rc = vx_flash_attn_ext_kv2_store(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
+                                      &ksrc, &ks, &vsrc, &vs, &d, scale, max_bias, softcap, sc, bias, ctx->stream);
+    return last;
 }
 
 vx_status compute_kv2_attention(backend_ctx * ctx, const ggml_tensor * f, const kv2_group & grp) {
@@ -798,7 +863,9 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         if (node->op == GGML_OP_FLASH_ATTN_EXT) {
             const auto it = kv2_by_fa.find(node);
             if (it != kv2_by_fa.end()) {
-                rc = compute_kv2_attention(ctx, node, it->second);
+                const int last = compute_kv2_attention_store(ctx, cgraph, i, it->second, readers, &rc);
+                if (last >= 0) i = last;
+                else rc = compute_kv2_attention(ctx, node, it->second);
                 ++launches;
                 if (rc != VX_OK) {
                     GGML_LOG_ERROR("ggml-gfx950: node %d (%s, two-segment attention) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
