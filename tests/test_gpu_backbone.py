@@ -87,3 +87,68 @@ def test_backbone_three_ways(gpu, ref, kv_f16, use_mup, T0):
             elif act == gpu.ACT_FLOAT:   # the one-launch pairs round where the separate nodes do
                 assert np.array_equal(unfused[i], got.cpu().numpy()), f"fused pairs changed the result of call {i}"
             n_past += T
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+@pytest.mark.parametrize("T0", [9, 300])
+def test_plugin_groups_fall_back_when_memory_is_reused(gpu, ref, kv_f16, T0):
+    """Graph shapes in which ggml-alloc hands the memory of a group's operand to a later node: decode steps that do
+    not write the cache (the step's keys die at the CONCAT), repeated steps at one position, and the same with
+    grouping switched off.  The plugin must give ggml-cpu's result in all of them, and the grouped and the
+    node-by-node runs must agree bit for bit."""
+    import ctypes
+    import os
+    import subprocess
+    import sys
+    max_len = T0 + 20
+    params = reflib.backbone_params("bb", N_LAYER)
+    xp = rng("bbf", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)
+    xs = [rng("bbf", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(3)]
+
+    def run(device):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=kv_f16)
+        outs = [reflib.ref_backbone_forward(xp, 0, reflib.causal_mask(T0, T0))[0]]
+        outs.append(reflib.ref_backbone_forward(xs[0], T0, None, write_kv=False)[0])     # peek: cache untouched
+        outs.append(reflib.ref_backbone_forward(xs[1], T0, None, write_kv=False)[0])
+        outs.append(reflib.ref_backbone_forward(xs[0], T0, None, write_kv=True)[0])      # now append
+        outs.append(reflib.ref_backbone_forward(xs[2], T0 + 1, None, write_kv=False)[0])
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs
+
+    cpu = run(b"CPU")
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug = run(b"GFX950_0")
+    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    print(f"backbone without cache write: kv_f16={kv_f16} T0={T0}, {launches} launches for the last step", flush=True)
+    for i, (a, b) in enumerate(zip(cpu, plug)):
+        e = nmse(a, b)
+        print(f"   plugin vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+        assert e <= 1e-4
+    assert np.array_equal(plug[1], plug[3]), "the appended step must repeat the peeked one"
+    # the same calls with every node as its own launch, in a fresh process (the switch is read once)
+    code = (
+        "import sys, numpy as np; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "import reflib, __graft_entry__ as e\n"
+        "from reflib import rng\n"
+        "pkg = e.load_package(); ref = reflib.load_ref()\n"
+        "assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) == 0 and ref.rh_use_device(b'GFX950_0', 8, 0) == 0\n"
+        "params = reflib.backbone_params('bb', %d)\n"
+        "reflib.ref_backbone_create(params, %d, %d, use_mup=True, kv_f16=%r)\n"
+        "xp = rng('bbf', 'x', 0).standard_normal((%d, %d, 1024)).astype(np.float32)\n"
+        "xs = [rng('bbf', 'x', i + 1).standard_normal((%d, 1, 1024)).astype(np.float32) for i in range(3)]\n"
+        "o = [reflib.ref_backbone_forward(xp, 0, reflib.causal_mask(%d, %d))[0]]\n"
+        "o.append(reflib.ref_backbone_forward(xs[0], %d, None, write_kv=False)[0])\n"
+        "o.append(reflib.ref_backbone_forward(xs[1], %d, None, write_kv=False)[0])\n"
+        "o.append(reflib.ref_backbone_forward(xs[0], %d, None, write_kv=True)[0])\n"
+        "o.append(reflib.ref_backbone_forward(xs[2], %d, None, write_kv=False)[0])\n"
+        "np.save(sys.argv[1], np.stack([a.reshape(-1)[:2048] for a in o[1:]]))\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)), N_LAYER, max_len, BATCH,
+         kv_f16, BATCH, T0, BATCH, T0, T0, T0, T0, T0, T0 + 1)
+    out_path = f"/tmp/bb_nofusion_{int(kv_f16)}_{T0}.npy"
+    env = dict(os.environ, GGML_GFX950_NO_FUSION="1")
+    subprocess.run([sys.executable, "-c", code, out_path], check=True, env=env, timeout=200)
+    plain = np.load(out_path)
+    grouped = np.stack([a.reshape(-1)[:2048] for a in plug[1:]])
+    assert np.array_equal(plain, grouped), "grouped launches changed a result"
