@@ -221,8 +221,8 @@ VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_te
                                                 const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
                                                 const vx_tensor * v_slot, const vx_tensor * dst);
 /* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
- * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for at most 16
- * tokens.  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE
+ * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for few tokens
+ * (as above).  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE
  * outputs [head_dim, heads, tokens, batch] and v_dst the third product, shaped like x with rows for K, all contiguous.  mode must be NEOX (2) with n_dims ==
  * head_dim; the remaining arguments are vx_rope's.  Results equal vx_mul_mat x3 + vx_rope x2 bit for bit. */
 VX_API vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
@@ -251,12 +251,12 @@ VX_API vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * n
                                         const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream);
 VX_API int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate,
                                            const vx_tensor * up, const vx_tensor * dst);
-/* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for at most 16 tokens
+/* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for few tokens (16, or more while tokens x rows <= 256 Ki)
  * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
                                    int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst);
-/* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for at most 16 tokens,
+/* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for few tokens (as above),
  * the residual updates of MiniCPMModel::layer_forward (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32
  * of dst's shape */
 VX_API vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,

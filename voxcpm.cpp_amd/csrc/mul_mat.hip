@@ -27,6 +27,8 @@
 #include "vx_common.hpp"
 #include "rope_common.hpp"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int GV_MAX_SEG = 3;
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
 }
 
 
-// ---- GEMV shape: at most 16 tokens (decode) ---------------------------------------------------
+// ---- GEMV shape: few tokens (decode, LocDiT) --------------------------------------------------
 // Pure weight streaming, so the kernel is built around memory-level parallelism: a work-group owns
 // 16 weight rows, its NW waves take interleaved 32-wide k blocks of those rows, and every wave
 // issues the loads of all its blocks (GV_UNROLL at a time, normally all of them) before anything
@@ -281,15 +283,19 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
     const int64_t nkb = a.K / 32;
     _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][K]
-    float *    xd  = (float *) (gv_smem + (size_t) a.N * a.K * 2);           // [N][K/32] (ACT_Q8)
-    float4_t * red = (float4_t *) (gv_smem + (size_t) a.N * a.K * 2 + (ACT_Q8 ? (size_t) a.N * nkb * 4 : 0));
+    const int NL = (int) (a.N < 16 ? a.N : 16);                              // tokens a work-group stages
+    float *    xd  = (float *) (gv_smem + (size_t) NL * a.K * 2);            // [NL][K/32] (ACT_Q8)
+    float4_t * red = (float4_t *) (gv_smem + (size_t) NL * a.K * 2 + (ACT_Q8 ? (size_t) NL * nkb * 4 : 0));
     float *    nsc = (float *) (red + (NW > 1 ? NW - 1 : 0) * 64); // [16] per-token 1 / rms (fused RMS_NORM)
 
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
     const int     batch = blockIdx.z;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
-    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    // more than 16 tokens: blockIdx.y picks a chunk of 16; the chunks' work-groups stream the same weight
+    // rows, which the first one pulls into L2
+    const int     tok0 = 16 * (int) blockIdx.y;
+    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) tok0 * a.nb11;
     const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
     int64_t       M = a.M;
@@ -327,7 +333,8 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const bool    row_ok = c < R && row < M;
     const char *  wsel = (dual && c >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
     const char *  wrow = wsel + (uint64_t) min(row, M - 1) * nb01;
-    const int     N = (int) a.N;
+    const int     N = min(16, (int) a.N - tok0); // tokens of this chunk
+    db += (uint64_t) tok0 * nb1;
 
     // ---- this wave's weight blocks: kb = wid + NW * i
     constexpr bool al4 = AL4;
@@ -407,7 +414,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
-        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) row * 4;
+        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) tok0 * a.rnb1 + (uint64_t) row * 4;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
@@ -419,7 +426,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         const float ffv = a.ff ? a.ff[pair] : 1.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-            if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * N + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
+            if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * (int) a.N + tok0 + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
     }
     if (a.norm_w) { // one wave per token, as the RMS_NORM kernel has it
         for (int t = wid; t < N; t += NW) {
@@ -501,8 +508,22 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     }
 }
 
+constexpr size_t GV_MAX_LDS = 160 * 1024; // what a gfx950 CU has
+
+// Shapes the streaming kernel takes: up to 16 tokens always; more (in chunks of 16, the chunks re-reading
+// the weight rows from L2) while tokens x rows stays small -- measured against the tiled kernels: 1024 rows win up
+// to 256 tokens, 4096 rows up to 64.  VX_GEMV_MAX_TOKENS=16 restores the 16-token limit.
+bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
+    static const int64_t max_tokens = [] { const char * e = getenv("VX_GEMV_MAX_TOKENS"); const int n = e ? atoi(e) : 0; return n >= 16 ? (int64_t) n : (int64_t) 1 << 30; }();
+    if (K % 32 || K < 32 || N < 1) return false;
+    if (N > 16 && (N > max_tokens || N * rows > 256 * 1024)) return false;
+    const size_t nl = (size_t) (N < 16 ? N : 16);
+    return nl * K * 2 + nl * (K / 32) * 4 + 15 * 64 * 16 + 16 * sizeof(float) <= GV_MAX_LDS;
+}
+
 size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
-    return (size_t) a.N * a.K * 2 + (act_q8 ? (size_t) a.N * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float);
+    const size_t nl = (size_t) (a.N < 16 ? a.N : 16);
+    return nl * a.K * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float);
 }
 
 // waves per work-group: about GV_UNROLL blocks per wave, so every load is issued up front
@@ -516,7 +537,11 @@ int gemv_waves(const mm_args & a) {
 template <int WT, bool ACT_Q8>
 bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     mm_args a = a0;
-    if (a.N > 16 || a.K % 32 || a.K < 32) return false;
+    {
+        int64_t rows = a.w2 ? 2 * a.M : a.M;
+        if (a.nseg > 0) { rows = 0; for (int i = 0; i < a.nseg; ++i) rows += a.seg[i].M; }
+        if (!gemv_shape_ok(a.N, rows, a.K)) return false;
+    }
     a.rows_wg = 16;
     const int split = a.w2 ? 2 : 1; // with two matrices a work-group's MFMA columns hold half as many output rows
     auto groups = [&](int rows_wg) { // work-groups per batch entry
@@ -525,25 +550,39 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
         for (int i = 0; i < a.nseg; ++i) n += (a.seg[i].M + rows_wg - 1) / rows_wg;
         return n;
     };
-    while (a.rows_wg > 4 && groups(a.rows_wg) * nbatch < 128) a.rows_wg /= 2;
+    const int64_t nchunk = (a.N + 15) / 16;
+    while (a.rows_wg > 4 && groups(a.rows_wg) * nbatch * nchunk < 128) a.rows_wg /= 2;
     const int nw = gemv_waves(a);
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
-    if (smem > 64 * 1024) return false;
+    if (smem > GV_MAX_LDS) return false;
     int64_t nwg = groups(a.rows_wg);
     if (a.nseg > 0) {
         int wg0 = 0;
         for (int i = 0; i < a.nseg; ++i) { a.seg[i].wg0 = wg0; wg0 += (int) ((a.seg[i].M + a.rows_wg - 1) / a.rows_wg); }
     }
-    const dim3 grid((unsigned) nwg, 1, (unsigned) nbatch);
+    const dim3 grid((unsigned) nwg, (unsigned) nchunk, (unsigned) nbatch);
     const dim3 block((unsigned) (64 * nw));
+    // above 64 KiB of LDS a kernel has to be told once that it may be given that much
+#define VX_GEMV_GO(...)                                                                                                \
+    do {                                                                                                               \
+        if (smem > 64 * 1024) {                                                                                        \
+            static bool raised = false;                                                                                \
+            if (!raised) {                                                                                             \
+                if (hipFuncSetAttribute((const void *) __VA_ARGS__, hipFuncAttributeMaxDynamicSharedMemorySize,        \
+                                        (int) GV_MAX_LDS) != hipSuccess) { (void) hipGetLastError(); return false; }   \
+                raised = true;                                                                                         \
+            }                                                                                                          \
+        }                                                                                                              \
+        __VA_ARGS__<<<grid, block, smem, st>>>(a);                                                                     \
+    } while (0)
 #define VX_GEMV(NW_)                                                                                                   \
     do {                                                                                                               \
         if (a.nseg > 0) {                                                                                              \
-            if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true, true><<<grid, block, smem, st>>>(a);    \
-            else                            gemv_kernel<WT, ACT_Q8, NW_, false, true><<<grid, block, smem, st>>>(a);   \
+            if (WT == WT_Q8 && a.w_aligned) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, true>);                      \
+            else                            VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, false, true>);                     \
         } else {                                                                                                       \
-            if (WT == WT_Q8 && a.w_aligned) gemv_kernel<WT, ACT_Q8, NW_, true, false><<<grid, block, smem, st>>>(a);   \
-            else                            gemv_kernel<WT, ACT_Q8, NW_, false, false><<<grid, block, smem, st>>>(a);  \
+            if (WT == WT_Q8 && a.w_aligned) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, false>);                     \
+            else                            VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, false, false>);                    \
         }                                                                                                              \
     } while (0)
     switch (nw) {
@@ -554,6 +593,7 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
         default: VX_GEMV(16); break;
     }
 #undef VX_GEMV
+#undef VX_GEMV_GO
     return true;
 }
 
@@ -773,8 +813,8 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
 
 template <int WT, bool ACT_Q8>
 void launch(const mm_args & a, int nbatch, hipStream_t st) {
-    if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if constexpr (WT != WT_F32) { if (launch_gemv<WT, ACT_Q8>(a, nbatch, st)) return; }
+    if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
         mm_kernel<WT, 1, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
@@ -856,8 +896,7 @@ extern "C" int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tenso
     if (gate->type != VX_TYPE_Q8_0 && gate->type != VX_TYPE_F16) return 0;
     if (up->type != gate->type) return 0;
     for (int i = 0; i < 4; ++i) if (up->ne[i] != gate->ne[i] || up->nb[i] != gate->nb[i]) return 0;
-    if (src1->ne[1] > 16 || gate->ne[0] % 32 || gate->ne[0] < 32) return 0;
-    return (size_t) src1->ne[1] * gate->ne[0] * 2 + (size_t) src1->ne[1] * (gate->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
+    return gemv_shape_ok(src1->ne[1], 2 * gate->ne[1], gate->ne[0]);
 }
 
 // whether the activations of a streaming-kernel launch can be normalised on the fly: rows of at most 1024
@@ -898,7 +937,7 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
     if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
         return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
     if (!vx_supports_mul_mat_swiglu(gate, up, src1, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, at most 16 tokens");
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, a token count the streaming kernel takes");
     if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
     if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
         return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
@@ -934,8 +973,7 @@ extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_te
     if (src0->type != VX_TYPE_Q8_0 && src0->type != VX_TYPE_F16) return 0;
     if (residual->type != VX_TYPE_F32 || !vx_same_shape(residual, dst) || residual->nb[0] != 4) return 0;
     if (residual->nb[1] % 4 || residual->nb[2] % 4 || residual->nb[3] % 4) return 0;
-    if (src1->ne[1] > 16 || src0->ne[0] % 32 || src0->ne[0] < 32) return 0;
-    return (size_t) src1->ne[1] * src0->ne[0] * 2 + (size_t) src1->ne[1] * (src0->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
+    return gemv_shape_ok(src1->ne[1], src0->ne[1], src0->ne[0]);
 }
 
 extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst,
@@ -943,7 +981,7 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     if (!src0 || !src1 || !residual || !dst || !src0->data || !src1->data || !residual->data || !dst->data)
         return vx_fail(VX_ERR_INVALID, "mul_mat_scale_add: null tensor");
     if (!vx_supports_mul_mat_scale_add(src0, src1, residual, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: Q8_0/F16 weights, at most 16 tokens, F32 residual of dst's shape");
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: Q8_0/F16 weights, a token count the streaming kernel takes, F32 residual of dst's shape");
     if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_scale_add: bad act_mode");
     if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (uintptr_t) residual->data % 4 || (src0->type == VX_TYPE_F16 && (uintptr_t) src0->data % 2))
         return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: misaligned tensor data");
@@ -997,12 +1035,12 @@ extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor *
     }
     if (x->type != VX_TYPE_F32 || !vx_positive(x) || x->ne[0] != wq->ne[0] || x->ne[2] != 1 || x->nb[0] != 4) return 0;
     if (x->nb[1] % 4 || x->nb[3] % 4 || x->ne[3] > 65535) return 0;
-    if (x->ne[1] > 16 || wq->ne[0] % 32 || wq->ne[0] < 32) return 0;
+    if (wq->ne[0] % 32 || wq->ne[0] < 32) return 0;
     if (mode != 2 || n_dims <= 0 || n_dims % 16) return 0; // NEOX over the whole head; pairs split evenly over work-groups
     if (!qkv_rope_dst_ok(wq, x, q_dst, n_dims) || !qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return 0;
     if (v_dst->type != VX_TYPE_F32 || !vx_is_contiguous(v_dst)) return 0;
     if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
-    return (size_t) x->ne[1] * wq->ne[0] * 2 + (size_t) x->ne[1] * (wq->ne[0] / 32) * 4 + 15 * 64 * 16 + 64 <= 64 * 1024;
+    return gemv_shape_ok(x->ne[1], wq->ne[1] + wk->ne[1] + wv->ne[1], wq->ne[0]);
 }
 
 static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,
@@ -1048,7 +1086,7 @@ static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * 
                          float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
                          vx_stream stream) {
     if (!vx_supports_qkv_proj_rope(wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode))
-        return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: three Q8_0/F16 matrices over one activation tensor of at most 16 tokens, NEOX rotation over the whole head, contiguous outputs");
+        return vx_fail(VX_ERR_UNSUPPORTED, "qkv_proj_rope: three Q8_0/F16 matrices over one activation tensor, a token count the streaming kernel takes, NEOX rotation over the whole head, contiguous outputs");
     if (!pos || !wq->data || !wk->data || !wv->data || !x->data || !q_dst->data || !k_dst->data || !v_dst->data)
         return vx_fail(VX_ERR_INVALID, "qkv_proj_rope: null data");
     if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "qkv_proj_rope: bad act_mode");
