@@ -268,6 +268,54 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     return res
 
 
+def locdit_stack_bench(pkg, timer, side, threads, with_cpu, requests=8, branch=7, layers=4, timesteps=10):
+    """BASELINE config 3 as a whole decoder pass: LocDiT runs the MiniCPM layer stack non-causally over the CFG
+    pair laid out as one 2 x 7-token sequence with a block-diagonal mask (src/locdit.cpp:400-464), no cache write;
+    8 concurrent requests ride in the batch dimension.  One CFM solve is (timesteps - 1) such passes."""
+    import torch
+    import reflib
+    bbmod = __import__("voxcpm_cpp_amd.backbone", fromlist=["MiniCPMBackbone"])
+    T = 2 * branch
+    pos = np.zeros(T, np.int32)
+    mk = np.zeros((T, T), np.uint16)
+    reflib.load_oracle().orc_cfg_pair_constants(branch, reflib.ptr(pos, C.c_int32), reflib.ptr(mk, C.c_uint16))
+    params = reflib.backbone_params("bench-locdit", 1)
+    lw = params["layers"][0]
+    m = bbmod.MiniCPMBackbone(n_layer=layers, max_length=T, batch=requests, use_mup=False, kv_f16=False)
+    for li in range(layers):
+        for n in reflib.BB_WEIGHTS:
+            m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+        for n in ("input_layernorm", "post_layernorm"):
+            m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+    m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+    m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+    x = torch.randn((requests, T, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    mask = torch.from_numpy(mk.view(np.float16)).cuda()
+    run, _ = m.plan(x, T, 0, mask, write_kv=False)
+    s = timer.run(graphed(run, side), iters=50, warmup=5)
+    res = {"us_per_decoder_pass": s * 1e6, "us_per_cfm_solve": s * (timesteps - 1) * 1e6, "launches_per_pass": run.n_calls,
+           "shape": f"{layers} layers, {requests} requests x {T} tokens (CFG pair), non-causal, Q8_0 weights"}
+    # one request alone (the reference's own call shape: 14 tokens, every projection on the streaming kernel)
+    m1 = bbmod.MiniCPMBackbone(n_layer=layers, max_length=T, batch=1, use_mup=False, kv_f16=False)
+    m1.weights, m1.norms, m1.final_norm, m1.rope_factors = m.weights, m.norms, m.final_norm, m.rope_factors
+    run1, _ = m1.plan(x[:1].contiguous(), T, 0, mask, write_kv=False)
+    s1 = timer.run(graphed(run1, side), iters=50, warmup=5)
+    res["one_request"] = {"us_per_decoder_pass": s1 * 1e6, "launches_per_pass": run1.n_calls}
+    del m, m1
+    ref = reflib.load_ref() if with_cpu else None
+    if ref is not None:
+        assert ref.rh_use_device(b"CPU", threads, 0) == 0
+        params["dims"]["n_layer"] = layers
+        params["layers"] = [lw] * layers
+        reflib.ref_backbone_create(params, T, requests, use_mup=False, kv_f16=False)
+        _, (mean, best), _ = reflib.ref_backbone_forward(x.cpu().numpy(), 0, mk.view(np.float16), write_kv=False, reps=40)
+        ref.rh_bb_free()
+        res["ggml_cpu_us_per_decoder_pass"] = mean * 1e6
+        res["ggml_cpu_threads"] = threads
+        res["speedup_vs_ggml_cpu"] = mean / s
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -380,6 +428,7 @@ def main():
     threads = min(16, os.cpu_count() or 1)
     if not args.no_others:
         others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu)
+        others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, not args.no_cpu)
 
     cpu = None
     if not args.no_cpu:
