@@ -132,6 +132,68 @@ def test_supports_truth_table_glue(pkg):
     assert lib.vx_supports_fused_pair(a, a, a) == 1 and lib.vx_supports_fused_pair(a, w, a) == 0
 
 
+def test_supports_truth_table_node_groups(pkg):
+    """The one-launch groups of a decoder layer: which shapes the plugin may hand to them."""
+    lib = pkg.lib()
+    K, H, Hkv, Dh = 1024, 16, 2, 64
+    wq, wk, wo = q8(pkg, [K, H * Dh, 1, 1]), q8(pkg, [K, Hkv * Dh, 1, 1]), q8(pkg, [K, K, 1, 1])
+    wdown = q8(pkg, [4096, K, 1, 1])
+
+    def acts(n, k=K):
+        return f32(pkg, [k, n, 1, 1])
+
+    # projection + scale + residual: the streaming kernel's token counts (16, or tokens x rows <= 256 Ki)
+    for n, want in ((1, 1), (16, 1), (17, 1), (256, 1), (257, 0)):
+        assert lib.vx_supports_mul_mat_scale_add(wo, acts(n), acts(n), acts(n)) == want, n
+    assert lib.vx_supports_mul_mat_scale_add(wdown, acts(14, 4096), acts(14), acts(14)) == 1      # 16 x 4096 halves of LDS
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), acts(3), acts(2)) == 0                  # residual of another shape
+    assert lib.vx_supports_mul_mat_scale_add(f32(pkg, [K, K, 1, 1]), acts(2), acts(2), acts(2)) == 0   # F32 weights
+    # gate / up / SwiGLU: both matrices count as rows
+    wg = q8(pkg, [K, 4096, 1, 1])
+    ffn = lambda n: f32(pkg, [4096, n, 1, 1])
+    for n, want in ((2, 1), (16, 1), (32, 1), (33, 0)):
+        assert lib.vx_supports_mul_mat_swiglu(wg, wg, acts(n), ffn(n)) == want, n
+    assert lib.vx_supports_mul_mat_swiglu(wg, q8(pkg, [K, 2048, 1, 1]), acts(2), ffn(2)) == 0
+    # q/k/v + rope: NEOX over the whole head only; batch in dim 3 or flattened into the token dimension
+    q_dst, k_dst = f32(pkg, [Dh, H, 1, 2]), f32(pkg, [Dh, Hkv, 1, 2])
+    xb, vb = f32(pkg, [K, 1, 1, 2]), f32(pkg, [Hkv * Dh, 1, 1, 2])
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, wk, xb, q_dst, k_dst, vb, Dh, 2) == 1
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, wk, acts(2), q_dst, k_dst, f32(pkg, [Hkv * Dh, 2, 1, 1]), Dh, 2) == 1
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, wk, xb, q_dst, k_dst, vb, Dh, 0) == 0            # NORMAL pairing
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, wk, xb, q_dst, k_dst, vb, Dh // 2, 2) == 0       # partial rotation
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, wk, acts(3), q_dst, k_dst, vb, Dh, 2) == 0       # token counts disagree
+    assert lib.vx_supports_qkv_proj_rope(wq, wk, f32(pkg, [K, Hkv * Dh, 1, 1]), xb, q_dst, k_dst, vb, Dh, 2) == 0
+    # rms_norm in front: rows of at most 1024 floats, one weight row
+    nw = f32(pkg, [K, 1, 1, 1])
+    assert lib.vx_supports_norm_qkv_proj_rope(xb, nw, wq, wk, wk, q_dst, k_dst, vb, Dh, 2) == 1
+    assert lib.vx_supports_norm_qkv_proj_rope(xb, f32(pkg, [K, 2, 1, 1]), wq, wk, wk, q_dst, k_dst, vb, Dh, 2) == 0
+    assert lib.vx_supports_norm_mul_mat_swiglu(acts(2), nw, wg, wg, ffn(2)) == 1
+    w2k = q8(pkg, [2048, 64, 1, 1])
+    assert lib.vx_supports_norm_mul_mat_swiglu(acts(1, 2048), f32(pkg, [2048, 1, 1, 1]), w2k, w2k, f32(pkg, [64, 1, 1, 1])) == 0
+    # cache write + ordering scalar: F32, decode-sized
+    k_src, slot = f32(pkg, [Dh, Hkv, 1, 2]), D(pkg, pkg.F32, [Dh, Hkv, 1, 2], [4, 4 * Dh * 768, 4 * Dh, 4 * Dh * 768 * Hkv])
+    attn = f32(pkg, [Dh, H, 1, 2])
+    assert lib.vx_supports_kv_store_sync(k_src, slot, k_src, slot, attn, attn) == 1
+    assert lib.vx_supports_kv_store_sync(k_src, f16(pkg, [Dh, Hkv, 1, 2]), k_src, slot, attn, attn) == 0      # F16 cache
+    big = f32(pkg, [Dh, Hkv, 512, 2])
+    assert lib.vx_supports_kv_store_sync(big, big, big, big, attn, attn) == 0                                     # prefill-sized
+    # attention over cached + current keys
+    q = f32(pkg, [Dh, 1, H, 2])
+    past = D(pkg, pkg.F32, [Dh, 640, Hkv, 2], [4, 4 * Dh, 4 * Dh * 768, 4 * Dh * 768 * Hkv])
+    cur = D(pkg, pkg.F32, [Dh, 1, Hkv, 2], [4, 4 * Dh * Hkv, 4 * Dh, 4 * Dh * Hkv])
+    assert lib.vx_supports_flash_attn_ext_kv2(q, past, cur, past, cur, None, attn) == 1
+    assert lib.vx_supports_flash_attn_ext_kv2(q, past, f16(pkg, [Dh, 1, Hkv, 2]), past, cur, None, attn) == 0   # segment types differ
+    assert lib.vx_supports_flash_attn_ext_kv2(q, past, f32(pkg, [Dh, 1, 4, 2]), past, cur, None, attn) == 0      # head counts differ
+    assert lib.vx_supports_flash_attn_ext_kv2_store(q, past, cur, past, cur, None, k_src, slot, k_src, slot, attn) == 1
+    short = D(pkg, pkg.F32, [Dh, 100, Hkv, 2], [4, 4 * Dh, 4 * Dh * 768, 4 * Dh * 768 * Hkv])
+    assert lib.vx_supports_flash_attn_ext_kv2(q, short, cur, short, cur, None, attn) == 1
+    assert lib.vx_supports_flash_attn_ext_kv2_store(q, short, cur, short, cur, None, k_src, slot, k_src, slot, attn) == 0  # no merge kernel to ride on
+    # null operands are refused, not dereferenced
+    assert lib.vx_supports_flash_attn_ext_kv2(q, past, None, past, cur, None, attn) == 0
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), None, acts(2)) == 0
+    assert lib.vx_supports_kv_store_sync(k_src, slot, None, slot, attn, attn) == 0
+
+
 def test_ops_validate_before_touching_the_device(pkg):
     """Contract violations are reported by status + message; nothing is launched."""
     lib = pkg.lib()
