@@ -223,7 +223,9 @@ VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_te
 /* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
  * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for few tokens
  * (as above).  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE
- * outputs [head_dim, heads, tokens, batch] and v_dst the third product, shaped like x with rows for K, all contiguous.  mode must be NEOX (2) with n_dims ==
+ * outputs [head_dim, heads, tokens, batch], contiguous; v_dst the third product, shaped like x with rows for K (dense
+ * rows, any row stride: it may be the v rows of one wider q/k/v product, the reference's fused qkv_proj layout, with
+ * wq / wk / wv row ranges of that one matrix).  mode must be NEOX (2) with n_dims ==
  * head_dim; the remaining arguments are vx_rope's.  Results equal vx_mul_mat x3 + vx_rope x2 bit for bit. */
 VX_API vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
                                   const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst,

@@ -231,6 +231,7 @@ struct bb_layer {
     ggml_tensor * w[7];       // q k v o gate up down
     ggml_tensor * ln[2];      // input_layernorm, post_layernorm
     ggml_tensor * kc, * vc;   // [D, max_len, Hkv, B]
+    ggml_tensor * qkv = nullptr, * gate_up = nullptr; // row-fused copies (rh_bb_fuse_weights), as the reference makes for LocDiT
 };
 
 struct backbone {
@@ -239,6 +240,8 @@ struct backbone {
     bool  use_mup, fused_glu;
     ggml_context *        wctx = nullptr;
     ggml_backend_buffer_t wbuf = nullptr;
+    ggml_context *        fctx = nullptr;
+    ggml_backend_buffer_t fbuf = nullptr;
     std::vector<bb_layer> layers;
     ggml_tensor *         final_norm = nullptr;
     ggml_tensor *         rope_factors = nullptr;
@@ -258,9 +261,18 @@ ggml_tensor * bb_layer_forward(ggml_context * c, const backbone & m, const bb_la
                                ggml_tensor * mask, int T, int n_past, bool write_kv, std::vector<ggml_tensor *> & roots) {
     const int D = m.head_dim, B = m.batch;
     ggml_tensor * cur = bb_norm(c, m, x, L.ln[0]);
-    ggml_tensor * q = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[0], cur), D, m.n_heads, T, B);
-    ggml_tensor * k = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[1], cur), D, m.n_kv, T, B);
-    ggml_tensor * v = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[2], cur), D, m.n_kv, T, B);
+    ggml_tensor * q, * k, * v;
+    if (L.qkv) { // one product, three strided views of it (src/minicpm.cpp:644-668)
+        ggml_tensor * qkv = ggml_mul_mat(c, L.qkv, cur);
+        const size_t  es = qkv->nb[0], qrows = (size_t) m.n_heads * D, krows = (size_t) m.n_kv * D;
+        q = ggml_view_4d(c, qkv, D, m.n_heads, T, B, D * es, qkv->nb[1], (size_t) T * qkv->nb[1], 0);
+        k = ggml_view_4d(c, qkv, D, m.n_kv, T, B, D * es, qkv->nb[1], (size_t) T * qkv->nb[1], qrows * es);
+        v = ggml_view_4d(c, qkv, D, m.n_kv, T, B, D * es, qkv->nb[1], (size_t) T * qkv->nb[1], (qrows + krows) * es);
+    } else {
+        q = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[0], cur), D, m.n_heads, T, B);
+        k = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[1], cur), D, m.n_kv, T, B);
+        v = ggml_reshape_4d(c, ggml_mul_mat(c, L.w[2], cur), D, m.n_kv, T, B);
+    }
     q = bb_rope(c, m, q, pos);
     k = bb_rope(c, m, k, pos);
 
@@ -301,9 +313,18 @@ ggml_tensor * bb_layer_forward(ggml_context * c, const backbone & m, const bb_la
     ggml_tensor * h = ggml_add(c, x, attn_out);
 
     cur = bb_norm(c, m, h, L.ln[1]);
-    ggml_tensor * gate = ggml_mul_mat(c, L.w[4], cur);
-    ggml_tensor * up   = ggml_mul_mat(c, L.w[5], cur);
-    ggml_tensor * act  = m.fused_glu ? ggml_swiglu_split(c, gate, up) : ggml_mul(c, ggml_silu(c, gate), up);
+    ggml_tensor * gate, * up;
+    bool glu = m.fused_glu;
+    if (L.gate_up) { // one product, two views of it, always the fused GLU (src/minicpm.cpp:724-731)
+        ggml_tensor * gu = ggml_mul_mat(c, L.gate_up, cur);
+        gate = ggml_view_2d(c, gu, m.ffn, gu->ne[1], gu->nb[1], 0);
+        up   = ggml_view_2d(c, gu, m.ffn, gu->ne[1], gu->nb[1], (size_t) m.ffn * gu->nb[0]);
+        glu  = true;
+    } else {
+        gate = ggml_mul_mat(c, L.w[4], cur);
+        up   = ggml_mul_mat(c, L.w[5], cur);
+    }
+    ggml_tensor * act  = glu ? ggml_swiglu_split(c, gate, up) : ggml_mul(c, ggml_silu(c, gate), up);
     ggml_tensor * down = ggml_mul_mat(c, L.w[6], act);
     if (m.use_mup) down = ggml_scale(c, down, m.residual_scale);
     return ggml_add(c, h, down);
@@ -315,6 +336,8 @@ extern "C" {
 
 void rh_bb_free(void) {
     if (!g_bb) return;
+    if (g_bb->fbuf) ggml_backend_buffer_free(g_bb->fbuf);
+    if (g_bb->fctx) ggml_free(g_bb->fctx);
     if (g_bb->wbuf) ggml_backend_buffer_free(g_bb->wbuf);
     if (g_bb->wctx) ggml_free(g_bb->wctx);
     delete g_bb;
@@ -349,6 +372,35 @@ int rh_bb_create(int n_layer, int hidden, int n_heads, int n_kv, int head_dim, i
     // mlp_forward fuses SwiGLU when the weights are not in host memory (src/minicpm.cpp:729-745)
     m->fused_glu = !ggml_backend_buffer_is_host(m->wbuf);
     g_bb = m;
+    return 0;
+}
+
+// Row-fused weight copies, as MiniCPMModel::load_from_store makes them for the LocDiT decoder on a GPU backend
+// (src/minicpm.cpp:427-492): qkv_proj = rows of q, k, v; gate_up_proj = rows of gate, up.  Call after rh_bb_set.
+int rh_bb_fuse_weights(void) {
+    if (!g_bb || !g_backend || g_bb->fctx) return 100;
+    backbone & m = *g_bb;
+    ggml_init_params ip = { ggml_tensor_overhead() * ((size_t) m.n_layer * 2 + 2), nullptr, true };
+    m.fctx = ggml_init(ip);
+    for (auto & L : m.layers) {
+        L.qkv     = ggml_new_tensor_2d(m.fctx, L.w[0]->type, L.w[0]->ne[0], L.w[0]->ne[1] + L.w[1]->ne[1] + L.w[2]->ne[1]);
+        L.gate_up = ggml_new_tensor_2d(m.fctx, L.w[4]->type, L.w[4]->ne[0], L.w[4]->ne[1] + L.w[5]->ne[1]);
+    }
+    m.fbuf = ggml_backend_alloc_ctx_tensors(m.fctx, g_backend);
+    if (!m.fbuf) return 101;
+    std::vector<uint8_t> scratch;
+    auto copy_rows = [&](ggml_tensor * src, ggml_tensor * dst, int64_t row0) {
+        scratch.resize(ggml_nbytes(src));
+        ggml_backend_tensor_get(src, scratch.data(), 0, scratch.size());
+        ggml_backend_tensor_set(dst, scratch.data(), (size_t) row0 * dst->nb[1], scratch.size());
+    };
+    for (auto & L : m.layers) {
+        copy_rows(L.w[0], L.qkv, 0);
+        copy_rows(L.w[1], L.qkv, L.w[0]->ne[1]);
+        copy_rows(L.w[2], L.qkv, L.w[0]->ne[1] + L.w[1]->ne[1]);
+        copy_rows(L.w[4], L.gate_up, 0);
+        copy_rows(L.w[5], L.gate_up, L.w[4]->ne[1]);
+    }
     return 0;
 }
 

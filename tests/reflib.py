@@ -346,8 +346,10 @@ def backbone_params(tag, n_layer, hidden=1024, n_heads=16, n_kv=2, head_dim=64, 
             "dims": dict(n_layer=n_layer, hidden=hidden, n_heads=n_heads, n_kv=n_kv, head_dim=head_dim, ffn=ffn)}
 
 
-def ref_backbone_create(params, max_len, batch, use_mup=False, kv_f16=False, eps=1e-5):
-    """Builds the decoder stack on the harness's current device (rh_use_device) and uploads params."""
+def ref_backbone_create(params, max_len, batch, use_mup=False, kv_f16=False, eps=1e-5, fused_weights=False):
+    """Builds the decoder stack on the harness's current device (rh_use_device) and uploads params.
+    fused_weights: the graph variant the reference uses for the LocDiT decoder on a GPU backend, one product
+    over row-fused q/k/v (and gate/up) weights with strided views of it."""
     lib = load_ref()
     d = params["dims"]
     rc = lib.rh_bb_create(d["n_layer"], d["hidden"], d["n_heads"], d["n_kv"], d["head_dim"], d["ffn"], max_len, batch,
@@ -359,6 +361,8 @@ def ref_backbone_create(params, max_len, batch, use_mup=False, kv_f16=False, eps
             assert lib.rh_bb_set(li, wi, a.ctypes.data, a.nbytes) == 0, (li, n)
     assert lib.rh_bb_set(-1, 0, params["final_norm"].ctypes.data, params["final_norm"].nbytes) == 0
     assert lib.rh_bb_set(-1, 1, params["rope_factors"].ctypes.data, params["rope_factors"].nbytes) == 0
+    if fused_weights:
+        assert lib.rh_bb_fuse_weights() == 0
 
 
 def ref_backbone_forward(x, n_past, mask=None, write_kv=True, reps=0):

@@ -152,3 +152,56 @@ def test_plugin_groups_fall_back_when_memory_is_reused(gpu, ref, kv_f16, T0):
     plain = np.load(out_path)
     grouped = np.stack([a.reshape(-1)[:2048] for a in plug[1:]])
     assert np.array_equal(plain, grouped), "grouped launches changed a result"
+
+
+@pytest.mark.parametrize("T0,causal", [(9, True), (300, True), (14, False)])
+def test_plugin_on_row_fused_weight_graphs(gpu, ref, T0, causal):
+    """The graph variant the reference builds for the LocDiT decoder on a GPU backend (one MUL_MAT over row-fused
+    q/k/v weights with strided views, one over gate/up): plugin against ggml-cpu, the launch count of the grouped
+    decode layer, and grouped against node-by-node results.  causal=False is the LocDiT call shape: the CFG pair as
+    one 14-token sequence, block-diagonal mask, no cache write."""
+    import ctypes
+    params = reflib.backbone_params("bb", N_LAYER)
+    max_len = T0 + 20
+    xp = rng("bbw", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)
+    xs = [rng("bbw", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(2)]
+    if causal:
+        mask0 = reflib.causal_mask(T0, T0)
+    else:
+        pos = np.zeros(T0, np.int32)
+        mk = np.zeros((T0, T0), np.uint16)
+        reflib.load_oracle().orc_cfg_pair_constants(T0 // 2, reflib.ptr(pos, ctypes.c_int32), reflib.ptr(mk, ctypes.c_uint16))
+        mask0 = mk.view(np.float16)
+
+    def run(device, fused_weights):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=False, fused_weights=fused_weights)
+        outs = [reflib.ref_backbone_forward(xp, 0, mask0, write_kv=causal)[0]]
+        if causal:
+            outs.append(reflib.ref_backbone_forward(xs[0], T0, None)[0])
+            outs.append(reflib.ref_backbone_forward(xs[1], T0 + 1, None)[0])
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs
+
+    cpu = run(b"CPU", True)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug = run(b"GFX950_0", True)
+    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    print(f"row-fused weights, T0={T0} causal={causal}: {launches} launches for the last graph", flush=True)
+    for i, (a, b) in enumerate(zip(cpu, plug)):
+        e = nmse(a, b)
+        print(f"   plugin vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+        assert e <= 1e-4
+    # five launches per layer and the final norm, the same groups as with separate weight tensors; up to 256 keys the
+    # attention takes one kernel and the cache write is a launch of its own
+    per_layer = 6 if causal and T0 + 2 <= 256 else 5
+    assert launches == N_LAYER * per_layer + 1, launches
+    # the separate-weights graph: the same rows through the same streaming kernel while the token count is small
+    # (identical results); a long prefill tiles the wider fused matrices differently
+    plain = run(b"GFX950_0", False)
+    for a, b in zip(plug, plain):
+        if BATCH * T0 <= 32:
+            assert np.array_equal(a, b)
+        else:
+            assert nmse(a, b) <= 1e-6

@@ -1038,7 +1038,9 @@ extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor *
     if (wq->ne[0] % 32 || wq->ne[0] < 32) return 0;
     if (mode != 2 || n_dims <= 0 || n_dims % 16) return 0; // NEOX over the whole head; pairs split evenly over work-groups
     if (!qkv_rope_dst_ok(wq, x, q_dst, n_dims) || !qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return 0;
-    if (v_dst->type != VX_TYPE_F32 || !vx_is_contiguous(v_dst)) return 0;
+    // v_dst may be a row range of a wider tensor (the v rows of one fused q/k/v product): dense rows, any row stride
+    if (v_dst->type != VX_TYPE_F32 || v_dst->nb[0] != 4 || v_dst->nb[1] % 4 || v_dst->nb[3] % 4) return 0;
+    if (v_dst->nb[1] < (uint64_t) v_dst->ne[0] * 4 || (v_dst->ne[3] > 1 && v_dst->nb[3] < v_dst->nb[1] * (uint64_t) v_dst->ne[1])) return 0;
     if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
     return gemv_shape_ok(x->ne[1], wq->ne[1] + wk->ne[1] + wv->ne[1], wq->ne[0]);
 }
@@ -1109,6 +1111,7 @@ static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * 
         s.w = (const char *) ws[i]->data; s.dst = (char *) ds[i]->data;
         s.M = ws[i]->ne[1]; s.nb01 = ws[i]->nb[1];
         s.nb1 = (uint64_t) s.M * 4; s.nb2 = 0; s.nb3 = (uint64_t) s.M * 4 * x->ne[1]; // the contiguous [rows, tokens, 1, batch] view of dst
+        if (i == 2) { s.nb1 = v_dst->nb[1]; s.nb3 = v_dst->nb[3]; }
         s.rope = i < 2;
         a.w_aligned = a.w_aligned && ((uintptr_t) ws[i]->data % 4 == 0) && ws[i]->nb[1] % 4 == 0;
         a.M += s.M;

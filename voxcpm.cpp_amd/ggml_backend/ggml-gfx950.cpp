@@ -779,6 +779,140 @@ bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const re
     return true;
 }
 
+// The reference's row-fused weights (MiniCPMModel::load_from_store makes them for the LocDiT decoder on a GPU backend,
+// src/minicpm.cpp:427-492): one MUL_MAT over qkv_proj, strided views of it as q, k, v, ROPE on the q and k views
+// (src/minicpm.cpp:644-680)
+//   [RMS_NORM MUL] MUL_MAT(qkv_proj, x) VIEW ROPE [views] VIEW ROPE        -> one launch: the multi-matrix kernel walks
+// three row ranges of the one matrix, writes the rotated q and k to the ROPE nodes' outputs and v where it lies in the
+// product.  A row range of a matrix as a descriptor of its own:
+vx_tensor row_range(const ggml_tensor * w, int64_t row0, int64_t rows) {
+    vx_tensor t = to_vx(w);
+    t.data  = (char *) w->data + (size_t) row0 * w->nb[1];
+    t.ne[1] = rows;
+    return t;
+}
+
+// view of the product mm covering rows [row0, row0 + rows) of every token, as [head_dim, heads, tokens, batch]
+bool is_row_view(const ggml_tensor * v, const ggml_tensor * mm, int64_t * row0, int64_t * rows) {
+    if (!v || v->op != GGML_OP_VIEW || v->view_src != mm || v->type != GGML_TYPE_F32 || mm->type != GGML_TYPE_F32) return false;
+    const ptrdiff_t off = (const char *) v->data - (const char *) mm->data;
+    if (off < 0 || off % 4 || (size_t) off >= mm->nb[1]) return false;
+    *row0 = off / 4;
+    *rows = v->ne[0] * v->ne[1];
+    if (*row0 + *rows > mm->ne[0]) return false;
+    if (v->nb[0] != 4 || v->nb[1] != (size_t) v->ne[0] * 4 || v->nb[2] != mm->nb[1]) return false;
+    if (v->ne[3] > 1 && v->nb[3] != (size_t) v->ne[2] * mm->nb[1]) return false;
+    return v->ne[2] * v->ne[3] == mm->ne[1] * mm->ne[2] * mm->ne[3] && mm->ne[2] == 1;
+}
+
+bool compute_fused_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, const absorbed_map & absorbed,
+                             std::unordered_set<const ggml_tensor *> & done, vx_status * rc, const ggml_tensor * norm = nullptr,
+                             const ggml_tensor * scale = nullptr) {
+    if (norm) i += 2;
+    if (i >= g->n_nodes || g->nodes[i]->op != GGML_OP_MUL_MAT) return false;
+    const ggml_tensor * mm = g->nodes[i];
+    if ((mm->flags & GGML_TENSOR_FLAG_OUTPUT) != 0 || (norm && mm->src[1] != scale)) return false;
+    const auto rd = [&](const ggml_tensor * t) { const auto it = readers.find(t); return it == readers.end() ? 0 : it->second; };
+    // the next two nodes that do work: ROPE over row views of mm
+    const ggml_tensor * rope[2] = { nullptr, nullptr };
+    int k = i;
+    for (int n = 0; n < 2; ++n) {
+        ++k;
+        while (k < g->n_nodes && (ggml_op_is_empty(g->nodes[k]->op) || ggml_is_empty(g->nodes[k]) || absorbed.count(g->nodes[k]))) ++k;
+        if (k >= g->n_nodes || g->nodes[k]->op != GGML_OP_ROPE || (g->nodes[k]->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return false;
+        rope[n] = g->nodes[k];
+    }
+    const ggml_tensor * rq = rope[0], * rk = rope[1];
+    int64_t q0, qn, k0, kn;
+    if (!is_row_view(rq->src[0], mm, &q0, &qn) || !is_row_view(rk->src[0], mm, &k0, &kn)) return false;
+    if (rd(rq->src[0]) != 1 || rd(rk->src[0]) != 1) return false;          // the un-rotated q and k rows are never stored
+    const int64_t M = mm->ne[0], vn = M - qn - kn;
+    if (q0 != 0 || k0 != qn || vn <= 0) return false;
+    // everything else that looks at the product must look at the v rows only (views of views share view_src)
+    for (int n = 0; n < g->n_nodes; ++n) {
+        const ggml_tensor * t = g->nodes[n];
+        if (t == rq->src[0] || t == rk->src[0]) continue;
+        bool reads = t->view_src == mm;
+        for (int s2 = 0; s2 < GGML_MAX_SRC && !reads; ++s2) reads = t->src[s2] == mm && !ggml_op_is_empty(t->op);
+        if (!reads) continue;
+        if (t->view_src != mm || !ggml_op_is_empty(t->op)) return false;
+        const ptrdiff_t off = (const char *) t->data - (const char *) mm->data;
+        if (off < 0 || (int64_t) ((size_t) off % mm->nb[1]) < (qn + kn) * 4) return false;
+    }
+    if (rq->src[1] != rk->src[1] || rq->src[2] != rk->src[2] || memcmp(rq->op_params, rk->op_params, 11 * sizeof(int32_t)) != 0) return false;
+    if (!rq->src[1] || rq->src[1]->type != GGML_TYPE_I32 || rq->src[1]->ne[0] != rq->ne[2]) return false;
+    if (rq->src[2] && (rq->src[2]->type != GGML_TYPE_F32 || rq->src[2]->ne[0] < rq->ne[0] / 2)) return false;
+    const int32_t * ip = (const int32_t *) rq->op_params;
+    const int n_dims = ip[1], mode = ip[2], n_ctx_orig = ip[4];
+    float fp[6];
+    memcpy(fp, ip + 5, sizeof(fp));
+    const ggml_tensor * x = norm ? norm->src[0] : mm->src[1];
+    if (!apart(rq, x) || !apart(rk, x) || !apart(mm, x) || !apart(rq, rk) || !apart(rq, mm) || !apart(rk, mm)) return false;
+    const ggml_tensor * W = mm->src[0];
+    const vx_tensor wq = row_range(W, 0, qn), wk = row_range(W, qn, kn), wv = row_range(W, qn + kn, vn), xx = to_vx(x), dq = to_vx(rq), dk = to_vx(rk);
+    vx_tensor dv = to_vx(mm);                       // the v rows of the product, where they lie
+    dv.data  = (char *) mm->data + (size_t) (qn + kn) * 4;
+    dv.ne[0] = vn;
+    const int32_t * posd = (const int32_t *) rq->src[1]->data;
+    const float *   ffd  = rq->src[2] ? (const float *) rq->src[2]->data : nullptr;
+    if (norm) {
+        const vx_tensor nw = to_vx(scale->src[1]);
+        float eps;
+        memcpy(&eps, norm->op_params, sizeof(float));
+        if (!vx_supports_norm_qkv_proj_rope(&xx, &nw, &wq, &wk, &wv, &dq, &dk, &dv, n_dims, mode) || (uintptr_t) xx.data % 16 || (uintptr_t) nw.data % 16) return false;
+        *rc = vx_norm_qkv_proj_rope(&xx, &nw, eps, &wq, &wk, &wv, posd, ffd, &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3],
+                                    fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
+        done.insert(scale); done.insert(mm);
+    } else {
+        if (!vx_supports_qkv_proj_rope(&wq, &wk, &wv, &xx, &dq, &dk, &dv, n_dims, mode)) return false;
+        *rc = vx_qkv_proj_rope(&wq, &wk, &wv, &xx, posd, ffd, &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3], fp[4], fp[5],
+                               mul_mat_act_mode(), ctx->stream);
+    }
+    done.insert(rq); done.insert(rk);
+    return true;
+}
+
+//   [RMS_NORM MUL] MUL_MAT(gate_up_proj, x) VIEW VIEW GLU(SWIGLU split)   (src/minicpm.cpp:724-745)  -> one launch:
+// the gate rows and the up rows of the one matrix share the MFMA columns of the SwiGLU kernel.
+bool compute_fused_gate_up_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers,
+                                 std::unordered_set<const ggml_tensor *> & done, vx_status * rc, const ggml_tensor * norm = nullptr,
+                                 const ggml_tensor * scale = nullptr) {
+    if (norm) i += 2;
+    if (i >= g->n_nodes || g->nodes[i]->op != GGML_OP_MUL_MAT) return false;
+    const ggml_tensor * mm = g->nodes[i];
+    if ((mm->flags & GGML_TENSOR_FLAG_OUTPUT) != 0 || (norm && mm->src[1] != scale) || mm->ne[2] != 1 || mm->ne[3] != 1) return false;
+    const auto rd = [&](const ggml_tensor * t) { const auto it = readers.find(t); return it == readers.end() ? 0 : it->second; };
+    const int kg = next_real(g, i);
+    if (kg >= g->n_nodes) return false;
+    const ggml_tensor * glu = g->nodes[kg];
+    if (glu->op != GGML_OP_GLU || (glu->flags & GGML_TENSOR_FLAG_COMPUTE) == 0 || ggml_get_glu_op(glu) != GGML_GLU_OP_SWIGLU ||
+        ((const int32_t *) glu->op_params)[1] != 0 || !glu->src[1]) return false;
+    const ggml_tensor * vg = glu->src[0], * vu = glu->src[1];
+    const int64_t ffn = mm->ne[0] / 2;
+    for (const ggml_tensor * v : { vg, vu }) {
+        if (v->op != GGML_OP_VIEW || v->view_src != mm || rd(v) != 1 || v->ne[0] != ffn || v->ne[1] != mm->ne[1] || v->ne[2] != 1 || v->ne[3] != 1 ||
+            v->nb[0] != 4 || v->nb[1] != mm->nb[1]) return false;
+    }
+    if (mm->ne[0] != 2 * ffn || rd(mm) != 4 || vg->data != mm->data || (const char *) vu->data != (const char *) mm->data + (size_t) ffn * 4) return false;
+    const ggml_tensor * x = norm ? norm->src[0] : mm->src[1];
+    if (!apart(glu, x)) return false;
+    const ggml_tensor * W = mm->src[0];
+    const vx_tensor gw = row_range(W, 0, ffn), uw = row_range(W, ffn, ffn), xx = to_vx(x), d = to_vx(glu);
+    if (norm) {
+        const vx_tensor nw = to_vx(scale->src[1]);
+        float eps;
+        memcpy(&eps, norm->op_params, sizeof(float));
+        if (!vx_supports_norm_mul_mat_swiglu(&xx, &nw, &gw, &uw, &d) || (uintptr_t) xx.data % 16 || (uintptr_t) nw.data % 16) return false;
+        *rc = vx_norm_mul_mat_swiglu(&xx, &nw, eps, &gw, &uw, &d, mul_mat_act_mode(), ctx->stream);
+        done.insert(scale); done.insert(mm);
+    } else {
+        if (!vx_supports_mul_mat_swiglu(&gw, &uw, &xx, &d)) return false;
+        *rc = vx_mul_mat_swiglu(&gw, &uw, &xx, &d, mul_mat_act_mode(), ctx->stream);
+    }
+    done.insert(glu);
+    return true;
+}
+
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
 
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
@@ -825,6 +959,9 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
             bool grouped = false;
             if (norm_pair && rd(mul) == 3) {
                 grouped = compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc, node, mul);
+            } else if (norm_pair && rd(mul) == 1) { // one product over row-fused weights behind the norm
+                grouped = compute_fused_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc, node, mul) ||
+                          compute_fused_gate_up_group(ctx, cgraph, i, readers, done, &rc, node, mul);
             } else if (norm_pair && rd(mul) == 2 && i + 4 < cgraph->n_nodes) {
                 ggml_tensor * gate = cgraph->nodes[i + 2];
                 ggml_tensor * up   = cgraph->nodes[i + 3];
@@ -852,7 +989,10 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
                 continue;
             }
         }
-        if (fusion && node->op == GGML_OP_MUL_MAT && compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc)) {
+        if (fusion && node->op == GGML_OP_MUL_MAT &&
+            (compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc) ||
+             compute_fused_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc) ||
+             compute_fused_gate_up_group(ctx, cgraph, i, readers, done, &rc))) {
             ++launches;
             if (rc != VX_OK) {
                 GGML_LOG_ERROR("ggml-gfx950: node %d (%s, q/k/v projections + rope) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
