@@ -248,6 +248,11 @@ struct backbone {
 };
 
 backbone * g_bb = nullptr;
+// Test switches (rh_bb_options): run the stack through ggml_backend_sched over {device, CPU} instead of a direct
+// graph_compute, and add per layer a small term computed by an operator no accelerator plugin here claims (GELU of
+// the normalised hidden state), so that the scheduler cuts the graph and a value in the middle of the device's part
+// is also read from the CPU's part.
+bool g_bb_sched = false, g_bb_probe = false;
 
 ggml_tensor * bb_norm(ggml_context * c, const backbone & m, ggml_tensor * x, ggml_tensor * w) {
     return ggml_mul(c, ggml_rms_norm(c, x, m.eps), w);
@@ -327,7 +332,9 @@ ggml_tensor * bb_layer_forward(ggml_context * c, const backbone & m, const bb_la
     ggml_tensor * act  = glu ? ggml_swiglu_split(c, gate, up) : ggml_mul(c, ggml_silu(c, gate), up);
     ggml_tensor * down = ggml_mul_mat(c, L.w[6], act);
     if (m.use_mup) down = ggml_scale(c, down, m.residual_scale);
-    return ggml_add(c, h, down);
+    ggml_tensor * res = ggml_add(c, h, down);
+    if (g_bb_probe) res = ggml_add(c, res, ggml_scale(c, ggml_gelu(c, cur), 1e-2f)); // cur: the post-attention normalised state
+    return res;
 }
 
 } // namespace
@@ -373,6 +380,11 @@ int rh_bb_create(int n_layer, int hidden, int n_heads, int n_kv, int head_dim, i
     m->fused_glu = !ggml_backend_buffer_is_host(m->wbuf);
     g_bb = m;
     return 0;
+}
+
+void rh_bb_options(int use_sched, int probe) {
+    g_bb_sched = use_sched != 0;
+    g_bb_probe = probe != 0;
 }
 
 // Row-fused weight copies, as MiniCPMModel::load_from_store makes them for the LocDiT decoder on a GPU backend
@@ -442,6 +454,30 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     ggml_cgraph * gf = ggml_new_graph_custom(c, n_nodes, false);
     ggml_build_forward_expand(gf, h);
     for (ggml_tensor * r : roots) ggml_build_forward_expand(gf, r);
+    if (g_bb_sched) { // the scheduler path VoxCPM takes with VOXCPM_ENABLE_SCHEDULER (src/backend.cpp:263-283)
+        ggml_backend_t cpu = ggml_backend_init_by_type(GGML_BACKEND_DEVICE_TYPE_CPU, nullptr);
+        if (!cpu) { ggml_free(c); return 105; }
+        ggml_backend_cpu_set_n_threads(cpu, 8);
+        ggml_backend_t backs[2] = { g_backend, cpu };
+        const bool same = ggml_backend_dev_type(ggml_backend_get_device(g_backend)) == GGML_BACKEND_DEVICE_TYPE_CPU;
+        ggml_backend_sched_t sched = ggml_backend_sched_new(same ? backs + 1 : backs, nullptr, same ? 1 : 2, n_nodes, false, true);
+        int rcs = 0;
+        if (!sched || !ggml_backend_sched_alloc_graph(sched, gf)) rcs = 101;
+        if (!rcs) {
+            ggml_backend_tensor_set(inp, x, 0, ggml_nbytes(inp));
+            std::vector<int32_t> p((size_t) T);
+            for (int i = 0; i < T; ++i) p[(size_t) i] = n_past + i;
+            ggml_backend_tensor_set(pos, p.data(), 0, ggml_nbytes(pos));
+            if (msk) ggml_backend_tensor_set(msk, mask, 0, ggml_nbytes(msk));
+            if (ggml_backend_sched_graph_compute(sched, gf) != GGML_STATUS_SUCCESS) rcs = 102;
+        }
+        if (!rcs && out) ggml_backend_tensor_get(h, out, 0, ggml_nbytes(h));
+        if (seconds) { seconds[0] = seconds[1] = 0.0; seconds[2] = sched ? (double) ggml_backend_sched_get_n_splits(sched) : 0.0; }
+        if (sched) ggml_backend_sched_free(sched);
+        ggml_backend_free(cpu);
+        ggml_free(c);
+        return rcs;
+    }
     ggml_gallocr_t ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend));
     int rc = 0;
     if (!ggml_gallocr_alloc_graph(ga, gf)) rc = 101;

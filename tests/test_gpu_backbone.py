@@ -205,3 +205,42 @@ def test_plugin_on_row_fused_weight_graphs(gpu, ref, T0, causal):
             assert np.array_equal(a, b)
         else:
             assert nmse(a, b) <= 1e-6
+
+
+@pytest.mark.parametrize("T0", [9, 300])
+def test_plugin_under_the_scheduler_with_a_cross_split_reader(gpu, ref, T0):
+    """ggml_backend_sched over {plugin, CPU} on a graph that holds, per layer, an operator the plugin does not claim
+    (GELU) reading the normalised hidden state in the middle of a group: the scheduler cuts the graph there, and the
+    value that a group would keep to itself has to be stored for the CPU's part.  Checked against ggml-cpu running
+    the same graph."""
+    params = reflib.backbone_params("bb", N_LAYER)
+    max_len = T0 + 20
+    xp = rng("bbs", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)
+    xs = [rng("bbs", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(2)]
+
+    def run(device, sched):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        ref.rh_bb_options(int(sched), 1)
+        try:
+            reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=False)
+            outs, splits = [], 0
+            o, _, splits = reflib.ref_backbone_forward(xp, 0, reflib.causal_mask(T0, T0))
+            outs.append(o)
+            for i, x in enumerate(xs):
+                o, _, splits = reflib.ref_backbone_forward(x, T0 + i, None)
+                outs.append(o)
+            ref.rh_bb_free()
+        finally:
+            ref.rh_bb_options(0, 0)
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs, splits
+
+    cpu, _ = run(b"CPU", False)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug, splits = run(b"GFX950_0", True)
+    print(f"scheduler with probe, T0={T0}: {splits} splits in the decode graph", flush=True)
+    assert splits > N_LAYER          # the graph really was cut around every GELU
+    for i, (a, b) in enumerate(zip(cpu, plug)):
+        e = nmse(a, b)
+        print(f"   plugin + scheduler vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+        assert e <= 1e-4

@@ -928,11 +928,25 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     reader_map readers;
     if (fusion && cgraph->n_nodes > 1) {
         readers.reserve((size_t) cgraph->n_nodes * 2);
+        reader_map as_operand; // uses as src[] only, the quantity ggml's own use counts hold
+        as_operand.reserve((size_t) cgraph->n_nodes * 2);
         for (int i = 0; i < cgraph->n_nodes; ++i) {
             const ggml_tensor * n = cgraph->nodes[i];
             for (int k = 0; k < GGML_MAX_SRC; ++k)
-                if (n->src[k]) readers[n->src[k]]++;
+                if (n->src[k]) { readers[n->src[k]]++; as_operand[n->src[k]]++; }
             if (n->view_src) readers[n->view_src]++;
+        }
+        // Under ggml_backend_sched this graph is a window of a larger one (ggml_graph_view shares the whole
+        // graph's hash set and use counts): a node that is also read from another split must be stored like
+        // an output.  Such nodes get a reader count no group accepts.
+        if (cgraph->use_counts && cgraph->visited_hash_set.keys && cgraph->visited_hash_set.size > 0) {
+            for (int i = 0; i < cgraph->n_nodes; ++i) {
+                const ggml_tensor * n = cgraph->nodes[i];
+                const size_t pos = ggml_hash_find(&cgraph->visited_hash_set, n);
+                if (pos == GGML_HASHSET_FULL || !ggml_bitset_get(cgraph->visited_hash_set.used, pos)) continue;
+                const auto it = as_operand.find(n);
+                if (cgraph->use_counts[pos] > (it == as_operand.end() ? 0 : it->second)) readers[n] += 1 << 20;
+            }
         }
     }
     std::unordered_map<const ggml_tensor *, kv2_group> kv2_by_fa;
