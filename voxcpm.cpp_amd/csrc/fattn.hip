@@ -365,7 +365,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 // anything waits, so the kernel costs one trip to memory, a few cross-lane steps and a store.
 constexpr int FA_MERGE_MAX_SPLITS = 256;
 template <int D>
-__global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
+__global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
     constexpr int DU = D / 4;       // lanes per row
     constexpr int PH = 64 / DU;     // split phases
     constexpr int NB = 16;          // rows a lane has in flight
@@ -374,7 +374,22 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     const int bg = tile / a.n_col_tiles;
     const int g = bg % a.Hkv, b = bg / a.Hkv;
     const int col = ct * 16 + c;
-    if (col >= a.n_q * a.gqa) return;
+    if (col >= a.n_q * a.gqa) return; // whole block
+    // With the cache write folded in the block has a second wave: it stores the slots (block 0), forms the two sums
+    // (a chain of fp64 cross-lane steps) and hands over the scalar, while the first wave merges.
+    __shared__ float kvs_addend;
+    if (threadIdx.x >= 64) {
+        const int  lane1 = threadIdx.x - 64;
+        const bool store = blockIdx.x == 0;
+        double tk, tv;
+        if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
+        else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
+        else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
+        else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
+        if (lane1 == 0) kvs_addend = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
+        __syncthreads();
+        return;
+    }
     const int lane = threadIdx.x, q = lane / DU, d0 = 4 * (lane % DU);
     bool  has_addend = a.add1 != nullptr;
     float addend     = has_addend ? *a.add1 : 0.0f;
@@ -402,13 +417,6 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     };
     load_rows(0);
 
-    if (a.has_kvs) { // the sources are a few hundred floats: every block re-forms the sums, the first one stores
-        const bool   store = blockIdx.x == 0;
-        const double tk = a.kvs_k.vec ? kvs_wave_total<true>(a.kvs_k, lane, store) : kvs_wave_total<false>(a.kvs_k, lane, store);
-        const double tv = a.kvs_v.vec ? kvs_wave_total<true>(a.kvs_v, lane, store) : kvs_wave_total<false>(a.kvs_v, lane, store);
-        addend     = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
-        has_addend = true;
-    }
     float M = m[0];
 #pragma unroll
     for (int i = 1; i < FA_MERGE_MAX_SPLITS / 64; ++i) M = fmaxf(M, m[i]);
@@ -440,6 +448,11 @@ __global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     for (int off = DU; off < 64; off <<= 1)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], off, 64);
+    if (a.has_kvs) { // uniform: the block was launched with its second wave
+        __syncthreads();
+        addend     = kvs_addend;
+        has_addend = true;
+    }
     if (q == 0) fa_finish(a, acc, M, L, b, g, col, D, d0, has_addend, addend);
 }
 
@@ -718,8 +731,9 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
         const dim3 grid((unsigned) (tiles * 16));
-        if (D == 64) fattn_merge_kernel<64><<<grid, dim3(64), 0, st>>>(a);
-        else         fattn_merge_kernel<128><<<grid, dim3(64), 0, st>>>(a);
+        const dim3 mblock(a.has_kvs ? 128 : 64); // the second wave carries the folded cache write
+        if (D == 64) fattn_merge_kernel<64><<<grid, mblock, 0, st>>>(a);
+        else         fattn_merge_kernel<128><<<grid, mblock, 0, st>>>(a);
         VX_LAUNCH_CHECK();
     }
     return VX_OK;

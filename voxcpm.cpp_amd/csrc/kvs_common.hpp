@@ -10,6 +10,7 @@ struct kvs_side {
     int64_t  nes[4], ned[4];
     uint64_t nbs[4], nbd[4];
     int vec; // slot rows allow 16-byte accesses: the test vx_sum applies to its operand
+    int src_dense; // the source is contiguous in its own order (element i at byte 4 i) and 16-byte aligned
 };
 
 // host side: what one cache write may look like, and its kernel argument
@@ -23,6 +24,7 @@ static inline void kvs_side_fill(kvs_side & o, const vx_tensor * src, const vx_t
     o.s = (const char *) src->data; o.d = (char *) slot->data;
     for (int i = 0; i < 4; ++i) { o.nes[i] = src->ne[i]; o.ned[i] = slot->ne[i]; o.nbs[i] = src->nb[i]; o.nbd[i] = slot->nb[i]; }
     o.vec = slot->ne[0] % 4 == 0 && (uintptr_t) slot->data % 16 == 0 && slot->nb[1] % 16 == 0 && slot->nb[2] % 16 == 0 && slot->nb[3] % 16 == 0;
+    o.src_dense = vx_is_contiguous(src) && (uintptr_t) src->data % 16 == 0;
 }
 
 #ifdef __HIPCC__
@@ -32,21 +34,27 @@ template <bool VEC>
 __device__ __forceinline__ void kvs_unit(const kvs_side & a, uint32_t e, bool store, double & acc) {
     constexpr int W = VEC ? 4 : 1;
     const uint32_t ne0 = (uint32_t) a.ned[0], per_row = ne0 / W;
-    const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
-    const uint32_t s0n = (uint32_t) a.nes[0], s1n = (uint32_t) a.nes[1], s2n = (uint32_t) a.nes[2];
-    const uint32_t row = e / per_row, iv = e - row * per_row;
-    const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
-    char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
     float v[W];
+    if (a.src_dense) { // no index arithmetic: unit e holds elements e W .. e W + W - 1 of the source
+        const float * ps = (const float *) a.s + (size_t) e * W;
+        if constexpr (VEC) { const float4_t t = *(const float4_t *) ps; v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3]; }
+        else               { v[0] = *ps; }
+    } else {
+        const uint32_t s0n = (uint32_t) a.nes[0], s1n = (uint32_t) a.nes[1], s2n = (uint32_t) a.nes[2];
 #pragma unroll
-    for (int k = 0; k < W; ++k) { // element number row * ne0 + iv * W + k of the source, in its own shape
-        uint32_t r = row * ne0 + iv * W + k;
-        const uint32_t j0 = r % s0n; r /= s0n;
-        const uint32_t j1 = r % s1n; r /= s1n;
-        const uint32_t j2 = r % s2n, j3 = r / s2n;
-        v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
+        for (int k = 0; k < W; ++k) { // element number e W + k of the source, in its own shape
+            uint32_t r = e * W + k;
+            const uint32_t j0 = r % s0n; r /= s0n;
+            const uint32_t j1 = r % s1n; r /= s1n;
+            const uint32_t j2 = r % s2n, j3 = r / s2n;
+            v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
+        }
     }
     if (store) {
+        const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
+        const uint32_t row = e / per_row, iv = e - row * per_row;
+        const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
+        char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
         if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
         else               *(float *) pd = v[0];
     }
@@ -74,6 +82,25 @@ __device__ __forceinline__ double kvs_wave_total(const kvs_side & a, int lane, b
     }
     if (w < 16) total += 0.0; // their zeros, added once (it only matters for the sign of a zero total)
     return total;
+}
+
+// both cache writes of a step at once: the two sides' loads are in flight together
+template <bool VK, bool VV>
+__device__ __forceinline__ void kvs_wave_totals(const kvs_side & k, const kvs_side & v, int lane, bool store, double & tk, double & tv) {
+    const uint32_t nk = kvs_units(k, VK), nv = kvs_units(v, VV);
+    tk = 0.0; tv = 0.0;
+    int wk = 0, wv = 0;
+    for (int w = 0; w < 16; ++w) {
+        const bool dk = (uint32_t) w * 64 < nk, dv = (uint32_t) w * 64 < nv; // uniform
+        if (!dk && !dv) break;
+        double ak = 0.0, av = 0.0;
+        if (dk) for (uint32_t e = (uint32_t) w * 64 + lane; e < nk; e += 1024) kvs_unit<VK>(k, e, store, ak);
+        if (dv) for (uint32_t e = (uint32_t) w * 64 + lane; e < nv; e += 1024) kvs_unit<VV>(v, e, store, av);
+        if (dk) { tk += vx_wave_sum(ak); ++wk; }
+        if (dv) { tv += vx_wave_sum(av); ++wv; }
+    }
+    if (wk < 16) tk += 0.0; // the zeros of the block's idle waves, added once (sign of a zero total)
+    if (wv < 16) tv += 0.0;
 }
 
 // the scalar the reference adds to the attention output: (sum(k_slot) + sum(v_slot)) * scale + bias
