@@ -198,7 +198,7 @@ def cpu_baseline(batch, length, threads):
             "sample": f"{reps} repeats of one layer on the scalar C oracle (oracle/_ref not prebuilt)"}
 
 
-def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256):
+def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256, do_prefill=True, cpu_reps=40):
     """BASELINE config 4: the whole decoder stack with Q8_0 weights (hidden 1024, 16/2 heads, FFN 4096),
     batch 2, prefill 512 tokens then 256 decode steps.  The GPU side is the host-side mirror of the
     reference's layer_forward over the C ABI (voxcpm.cpp_amd/backbone.py, F32 KV cache as in the
@@ -221,10 +221,17 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
     weight_bytes = layers * sum(lw[n].nbytes for n in reflib.BB_WEIGHTS)
 
-    xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
-    mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
-    run_p, _ = m.plan(xp, prefill, 0, mask)
-    t_prefill = timer.run(run_p, iters=3, warmup=1)
+    t_prefill = None
+    xp = None
+    if do_prefill:
+        xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
+        mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
+        run_p, _ = m.plan(xp, prefill, 0, mask)
+        t_prefill = timer.run(run_p, iters=3, warmup=1)
+    else:   # long caches: decode over seeded cache contents instead of a real prefill
+        gk = torch.Generator(device="cuda").manual_seed(11)
+        for t in m.k_cache + m.v_cache:
+            t.normal_(generator=gk)
 
     x1 = torch.randn((batch, 1, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
     points = [prefill + (2 * i + 1) * steps // 8 for i in range(4)]
@@ -246,7 +253,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     kvb = layers * 2 * batch * HKV * (prefill + steps // 2) * D * 4
     res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
            "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
-           "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": batch * prefill / t_prefill,
+           "prefill_ms": t_prefill * 1e3 if t_prefill else None, "prefill_tokens_per_s": batch * prefill / t_prefill if t_prefill else None,
            "kv_cache": "f32 (the reference's cache type)", "launch": "captured HIP graph per step, KV lengths " + str(points)}
     del replays, m
     ref = reflib.load_ref() if with_cpu else None
@@ -255,15 +262,17 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         params["dims"]["n_layer"] = layers
         params["layers"] = [lw] * layers
         reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=False)
-        xph = xp.cpu().numpy()
-        tp0 = time.perf_counter()
-        reflib.ref_backbone_forward(xph, 0, reflib.causal_mask(prefill, prefill))
-        cpu_prefill = time.perf_counter() - tp0
-        _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), prefill + steps // 2, None, reps=40)
+        cpu_prefill = None
+        if do_prefill:
+            xph = xp.cpu().numpy()
+            tp0 = time.perf_counter()
+            reflib.ref_backbone_forward(xph, 0, reflib.causal_mask(prefill, prefill))
+            cpu_prefill = time.perf_counter() - tp0
+        _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), prefill + steps // 2, None, reps=cpu_reps)
         ref.rh_bb_free()
         res["ggml_cpu"] = {"decode_steps_per_s": 1.0 / mean, "ms_per_step": mean * 1e3, "best_ms": best * 1e3, "threads": threads,
-                           "graph_nodes": n_nodes, "prefill_ms": cpu_prefill * 1e3,
-                           "sample": f"40 repeats of the decode step at KV length {prefill + steps // 2}, one prefill"}
+                           "graph_nodes": n_nodes, "prefill_ms": cpu_prefill * 1e3 if cpu_prefill else None,
+                           "sample": f"{cpu_reps} repeats of the decode step at KV length {prefill + steps // 2}" + (", one prefill" if do_prefill else ", cache contents as left by allocation")}
         res["speedup_vs_ggml_cpu"] = mean / t_step
     return res
 
@@ -429,6 +438,10 @@ def main():
     if not args.no_others:
         others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu)
         others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, not args.no_cpu)
+        # BASELINE config 5 as a whole stack: 8 streams x CFG pair (batch 16) decoding from KV length 4096 towards 8192
+        # (F32 cache as in the reference; the decode steps run over seeded cache contents)
+        others["cfg5_backbone_24layers_b16_L4096"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu, batch=16, prefill=4096,
+                                                                    steps=256, do_prefill=False, cpu_reps=3)
 
     cpu = None
     if not args.no_cpu:
@@ -459,7 +472,7 @@ def main():
         },
         "others": others,
     }
-    print(json.dumps(line))
+    print(json.dumps(line, allow_nan=False))
 
 
 if __name__ == "__main__":
