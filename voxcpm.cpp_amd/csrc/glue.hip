@@ -256,8 +256,12 @@ __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, 
     const uint32_t per_row = (uint32_t) (s.ne[0] / W);
     const uint32_t n = per_row * (uint32_t) (s.ne[1] * s.ne[2] * s.ne[3]); // < 2^24, checked by the caller
     const uint32_t ne1 = (uint32_t) s.ne[1], ne2 = (uint32_t) s.ne[2];
+    const bool one_wave = n <= VX_SUM_ONE_WAVE_UNITS && gridDim.x == 1; // uniform
+    if (one_wave && threadIdx.x >= 64) return;
+    const uint32_t first = one_wave ? threadIdx.x : blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t step  = one_wave ? 64 : gridDim.x * blockDim.x;
     double acc = 0.0;
-    for (uint32_t e = blockIdx.x * 1024 + threadIdx.x; e < n; e += gridDim.x * 1024) {
+    for (uint32_t e = first; e < n; e += step) {
         const uint32_t row = e / per_row, iv = e - row * per_row;
         const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
         const char * p = src + (uint64_t) iv * (4 * W) + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3];
@@ -267,6 +271,11 @@ __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, 
         } else {
             acc += (double) *(const float *) p;
         }
+    }
+    if (one_wave) {
+        acc = vx_wave_sum(acc);
+        if (threadIdx.x == 0) *dst = (float) acc;
+        return;
     }
     const double t = block_total(acc, part);
     if (threadIdx.x == 0) {
@@ -300,12 +309,23 @@ struct kvs_args {
     float scale, bias;
 };
 
+// stores the slot and returns the sum of what was stored, the same value in every thread of the block
 template <bool VEC>
-__device__ __forceinline__ double store_and_sum(const kvs_side & a) {
+__device__ __forceinline__ float store_and_sum(const kvs_side & a, double * part) {
     const uint32_t n = kvs_units(a, VEC);
+    if (n <= VX_SUM_ONE_WAVE_UNITS) { // the one-wave order of small sums
+        if (threadIdx.x < 64) {
+            const double t = kvs_wave_total<VEC>(a, threadIdx.x, true);
+            if (threadIdx.x == 0) part[0] = t;
+        }
+        __syncthreads();
+        const float r = (float) part[0];
+        __syncthreads();
+        return r;
+    }
     double acc = 0.0;
     for (uint32_t e = threadIdx.x; e < n; e += 1024) kvs_unit<VEC>(a, e, true, acc);
-    return acc;
+    return (float) block_total(acc, part);
 }
 
 __global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
@@ -328,10 +348,8 @@ __global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
         xv[p] = 0.0f; xo[p] = 0;
         if (e < nx) { uint64_t ox; offsets(e, ox, xo[p]); xv[p] = *(const float *) (a.x + ox); }
     }
-    const double ak = a.k.vec ? store_and_sum<true>(a.k) : store_and_sum<false>(a.k);
-    const float  sk = (float) block_total(ak, part);
-    const double av = a.v.vec ? store_and_sum<true>(a.v) : store_and_sum<false>(a.v);
-    const float  sv = (float) block_total(av, part);
+    const float sk = a.k.vec ? store_and_sum<true>(a.k, part) : store_and_sum<false>(a.k, part);
+    const float sv = a.v.vec ? store_and_sum<true>(a.v, part) : store_and_sum<false>(a.v, part);
     const float  y  = kvs_scalar(sk, sv, a.scale, a.bias);
 #pragma unroll
     for (int p = 0; p < KVS_PRE; ++p)
@@ -553,8 +571,9 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
         if (rc != VX_OK) return rc;
         partials = (double *) ws; blocks = SUM_BLOCKS;
     }
-    if (vec) sum_kernel<true><<<dim3(blocks), dim3(1024), 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
-    else     sum_kernel<false><<<dim3(blocks), dim3(1024), 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    const dim3 block(units <= VX_SUM_ONE_WAVE_UNITS ? 64 : 1024); // small sums are one wave's work
+    if (vec) sum_kernel<true><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    else     sum_kernel<false><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
     if (partials) sum_partials_kernel<<<dim3(1), dim3(64), 0, st>>>(partials, blocks, (float *) dst->data);
     VX_LAUNCH_CHECK();
     return VX_OK;

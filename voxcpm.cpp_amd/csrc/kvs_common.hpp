@@ -66,12 +66,17 @@ __device__ __forceinline__ uint32_t kvs_units(const kvs_side & a, bool vec) {
     return (uint32_t) (a.ned[0] / (vec ? 4 : 1)) * (uint32_t) (a.ned[1] * a.ned[2] * a.ned[3]);
 }
 
-// The sum a 1024-thread block forms (thread t walks units t, t + 1024, ...; each wave reduces by xor
-// butterfly; the 16 wave totals are added in order), formed by ONE wave that plays the 16 waves in turn:
-// the same additions in the same order, so the same double.
+// The sum of a cache write as GGML_OP_SUM's kernels form it, by one wave.  Small writes: the one-wave order itself.
+// Larger ones: a 1024-thread block's order (thread t walks units t, t + 1024, ...; each wave reduces by xor
+// butterfly; the 16 wave totals are added in order), replayed wave by wave: the same additions in the same order.
 template <bool VEC>
 __device__ __forceinline__ double kvs_wave_total(const kvs_side & a, int lane, bool store) {
     const uint32_t n = kvs_units(a, VEC);
+    if (n <= VX_SUM_ONE_WAVE_UNITS) {
+        double acc = 0.0;
+        for (uint32_t e = lane; e < n; e += 64) kvs_unit<VEC>(a, e, store, acc);
+        return vx_wave_sum(acc);
+    }
     double total = 0.0;
     int w = 0;
     for (; w < 16; ++w) {
@@ -88,6 +93,22 @@ __device__ __forceinline__ double kvs_wave_total(const kvs_side & a, int lane, b
 template <bool VK, bool VV>
 __device__ __forceinline__ void kvs_wave_totals(const kvs_side & k, const kvs_side & v, int lane, bool store, double & tk, double & tv) {
     const uint32_t nk = kvs_units(k, VK), nv = kvs_units(v, VV);
+    if (nk <= VX_SUM_ONE_WAVE_UNITS && nv <= VX_SUM_ONE_WAVE_UNITS) { // both in the one-wave order, loads side by side
+        double ak = 0.0, av = 0.0;
+        const uint32_t nmax = nk > nv ? nk : nv;
+        for (uint32_t e = lane; e < nmax; e += 64) {
+            if (e < nk) kvs_unit<VK>(k, e, store, ak);
+            if (e < nv) kvs_unit<VV>(v, e, store, av);
+        }
+        tk = vx_wave_sum(ak);
+        tv = vx_wave_sum(av);
+        return;
+    }
+    if (nk <= VX_SUM_ONE_WAVE_UNITS || nv <= VX_SUM_ONE_WAVE_UNITS) { // mixed sizes: each side in its own order
+        tk = kvs_wave_total<VK>(k, lane, store);
+        tv = kvs_wave_total<VV>(v, lane, store);
+        return;
+    }
     tk = 0.0; tv = 0.0;
     int wk = 0, wv = 0;
     for (int w = 0; w < 16; ++w) {

@@ -80,6 +80,11 @@ static inline bool vx_positive(const vx_tensor * t) {
     return t->ne[0] > 0 && t->ne[1] > 0 && t->ne[2] > 0 && t->ne[3] > 0;
 }
 
+// GGML_OP_SUM over at most this many units (a unit = 4 consecutive elements of a dense, 16-byte aligned row, else
+// one element) is formed by ONE wave: lane l adds units l, l + 64, ... in fp64, then one xor butterfly.  Every
+// kernel that forms such a sum (the SUM kernel, the cache-write group, the attention merge) uses this order.
+#define VX_SUM_ONE_WAVE_UNITS 1024
+
 // ---- device helpers ------------------------------------------------------------------------
 #ifdef __HIPCC__
 
