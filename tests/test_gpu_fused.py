@@ -441,3 +441,50 @@ def test_flash_attn_two_segments_with_cache_write(pkg, gpu, T, n_past, B, Hkv, D
     # too few keys for the split path: refused, the separate calls remain
     assert L.vx_supports_flash_attn_ext_kv2_store(d(q), d(kc2[:, :, :100]), d(kcur), d(vc2[:, :, :100]), d(vcur), None,
                                                   d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b)) == 0
+
+
+@pytest.mark.parametrize("N", [2, 14, 40])
+def test_groups_with_f16_weights(pkg, gpu, N):
+    import torch
+    say(f"node groups over F16 weight matrices, {N} tokens")
+    L, d = pkg.lib(), pkg.desc
+    H, Hkv, D, K, F = 4, 2, 64, 512, 768
+    g = rng("f-f16", N)
+    mk = lambda m: dev((0.05 * g.standard_normal((m, K))).astype(np.float16))
+    wq, wk, wv, wg, wu = mk(H * D), mk(Hkv * D), mk(Hkv * D), mk(F), mk(F)
+    wo = dev((0.05 * g.standard_normal((K, H * D))).astype(np.float16))
+    x = dev(g.standard_normal((N, K)).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    pos = torch.arange(5, 5 + N, dtype=torch.int32, device="cuda")
+    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+    mode = pkg.ACT_FLOAT
+    # rms_norm + q/k/v + rope
+    normed = torch.empty_like(x)
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    q1 = torch.empty((1, N, H, D), dtype=torch.float32, device="cuda")
+    k1 = torch.empty((1, N, Hkv, D), dtype=torch.float32, device="cuda")
+    v1 = torch.empty((N, Hkv * D), dtype=torch.float32, device="cuda")
+    for w, o, M in ((wq, q1, H * D), (wk, k1, Hkv * D), (wv, v1, Hkv * D)):
+        ok(pkg, L.vx_mul_mat(d(w), d(normed), d(o.view(N, M)), mode, None), "mul_mat")
+    for o in (q1, k1):
+        ok(pkg, L.vx_rope(d(o), pos.data_ptr(), None, d(o), *rope_args, None), "rope")
+    q2, k2, v2 = torch.empty_like(q1), torch.empty_like(k1), torch.empty_like(v1)
+    assert L.vx_supports_norm_qkv_proj_rope(d(x), d(nw), d(wq), d(wk), d(wv), d(q2), d(k2), d(v2), D, 2) == 1
+    ok(pkg, L.vx_norm_qkv_proj_rope(d(x), d(nw), 1e-5, d(wq), d(wk), d(wv), pos.data_ptr(), None, d(q2), d(k2), d(v2), *rope_args, mode, None), "norm_qkv")
+    # rms_norm + gate/up + SwiGLU
+    ga, up, a1, a2 = (torch.empty((N, F), dtype=torch.float32, device="cuda") for _ in range(4))
+    ok(pkg, L.vx_mul_mat(d(wg), d(normed), d(ga), mode, None), "gate")
+    ok(pkg, L.vx_mul_mat(d(wu), d(normed), d(up), mode, None), "up")
+    ok(pkg, L.vx_glu(pkg.GLU_SWIGLU, d(ga), d(up), d(a1), 0, None), "glu")
+    ok(pkg, L.vx_norm_mul_mat_swiglu(d(x), d(nw), 1e-5, d(wg), d(wu), d(a2), mode, None), "norm_swiglu")
+    # projection + scale + residual
+    attn = q1.view(N, H * D)
+    prod, r1, r2 = (torch.empty((N, K), dtype=torch.float32, device="cuda") for _ in range(3))
+    ok(pkg, L.vx_mul_mat(d(wo), d(attn), d(prod), mode, None), "o")
+    ok(pkg, L.vx_scale(d(prod), d(prod), 0.3, 0.0, None), "scale")
+    ok(pkg, L.vx_binary(pkg.BIN_ADD, d(x), d(prod), d(r1), None), "add")
+    ok(pkg, L.vx_mul_mat_scale_add(d(wo), d(attn), d(x), d(r2), 0.3, mode, None), "mul_mat_scale_add")
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert torch.equal(a1, a2)
+    assert torch.equal(r1, r2)
