@@ -383,7 +383,9 @@ def mm_inputs(tag, M, K, N, batch=()):
                                    (1024, 1024, 5), (1024, 1024, 16), (1024, 1024, 17), (1000, 1024, 33),
                                    (3072, 1024, 112), (1024, 1024, 512), (70, 96, 130),
                                    # the 128 x 128 pipelined GEMM: full tiles, and ragged rows / tokens / odd block count
-                                   (4096, 1024, 1024), (2000, 1056, 1700)])
+                                   (4096, 1024, 1024), (2000, 1056, 1700),
+                                   # a long K on a small grid: K cut across work-groups, partials added by a second kernel
+                                   (1024, 4096, 600), (1000, 2176, 300)])
 def test_mul_mat_q8_0(gpu, M, K, N):
     say(f"mul_mat Q8_0 M={M} K={K} N={N}")
     w, x = mm_inputs(("q8", M, K, N), M, K, N)

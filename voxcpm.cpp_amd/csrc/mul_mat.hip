@@ -60,6 +60,10 @@ struct mm_args {
     rope_params rp;
     int head_dim;
     int rope_T; // tokens per sequence: token n of the flattened (token, batch) order sits at position pos[n % rope_T]
+    // tiled kernel, long K on a small grid: the K range is cut across ksplit work-groups that leave fp32 partials
+    // [batch][split][token][row] for a second kernel to add in split order (ksplit <= 1: off)
+    int ksplit;
+    float * partial;
     // GEMV with RMS_NORM and the norm-weight MUL applied to the activations as they are staged
     // (x is then the un-normalised tensor): x[t][k] / rms(x[t]) * norm_w[k], rounded after each product
     const float * norm_w;
@@ -138,11 +142,17 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
 
-    const int     batch = blockIdx.z;
+    const int     nsplit = (!KSPLIT && a.ksplit > 1) ? a.ksplit : 1; // uniform
+    const int     batch = (int) blockIdx.z / nsplit, split = (int) blockIdx.z % nsplit;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
     const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    uint64_t      dnb1 = a.nb1;
+    if (nsplit > 1) { // this work-group's share goes to its slab of the partial buffer, dense [token][row]
+        db   = (char *) (a.partial + ((uint64_t) batch * nsplit + split) * (uint64_t) a.N * a.M);
+        dnb1 = (uint64_t) a.M * 4;
+    }
 
     const int64_t tok0 = (int64_t) blockIdx.y * 16 * TT;
     const int64_t row0 = KSPLIT ? (int64_t) blockIdx.x * 16 : (int64_t) blockIdx.x * 64 + wid * 16;
@@ -153,8 +163,11 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) acc[tt] = float4_t{0, 0, 0, 0};
 
-    const int64_t nkb = (a.K + 31) / 32;
-    for (int64_t kb0 = 0; kb0 < nkb; kb0 += KC_BLOCKS) {
+    const int64_t nkb_all = (a.K + 31) / 32;
+    const int64_t per_split = ((nkb_all + nsplit - 1) / nsplit + KC_BLOCKS - 1) / KC_BLOCKS * KC_BLOCKS;
+    const int64_t kb_first = (int64_t) split * per_split;
+    const int64_t nkb = min(nkb_all, kb_first + per_split);
+    for (int64_t kb0 = kb_first; kb0 < nkb; kb0 += KC_BLOCKS) {
         // ---- stage 16*TT tokens x 128 k of activations as f16 operands
 #pragma unroll
         for (int it = 0; it < TT; ++it) {
@@ -261,9 +274,23 @@ __global__ __launch_bounds__(256) void mm_kernel(const mm_args a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t tok = tok0 + 16 * tt + 4 * j + r;
-                if (tok < a.N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) (row0 + c) * 4) = acc[tt][r];
+                if (tok < a.N) *(float *) (db + (uint64_t) tok * dnb1 + (uint64_t) (row0 + c) * 4) = acc[tt][r];
             }
     }
+}
+
+// adds the K-split partials in split order: one thread per 4 consecutive rows of one token
+__global__ __launch_bounds__(256) void mm_splitk_reduce_kernel(const mm_args a) {
+    const int64_t m4 = a.M / 4;
+    const int64_t u = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (u >= a.N * m4) return;
+    const int64_t tok = u / m4, r4 = (u % m4) * 4;
+    const int     batch = blockIdx.z;
+    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const float * p = a.partial + (uint64_t) batch * a.ksplit * (uint64_t) a.N * a.M + (uint64_t) tok * a.M + r4;
+    float4_t acc = *(const float4_t *) p;
+    for (int s = 1; s < a.ksplit; ++s) acc += *(const float4_t *) (p + (uint64_t) s * a.N * a.M);
+    *(float4_t *) (a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3 + (uint64_t) tok * a.nb1 + (uint64_t) r4 * 4) = acc;
 }
 
 
@@ -822,7 +849,28 @@ void launch(const mm_args & a, int nbatch, hipStream_t st) {
         const dim3 grid((unsigned) ((a.M + 63) / 64), 1, (unsigned) nbatch);
         mm_kernel<WT, 2, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
     } else {
-        const dim3 grid((unsigned) ((a.M + 63) / 64), (unsigned) ((a.N + 63) / 64), (unsigned) nbatch);
+        // A long K on a grid that leaves most CUs with one work-group is a chain of ~3 us rounds: cut K so that every
+        // split walks about 1024 of it, and add the partials in a second launch.
+        const int64_t gx = (a.M + 63) / 64, gy = (a.N + 63) / 64;
+        int ks = 1;
+        if (a.K >= 2048 && a.K % 128 == 0 && a.M % 4 == 0 && gx * gy * nbatch <= 512 && (uintptr_t) a.dst % 16 == 0 && a.nb1 % 16 == 0 &&
+            a.nb2 % 16 == 0 && a.nb3 % 16 == 0) {
+            ks = (int) (a.K / 1024);
+            if (ks > 8) ks = 8;
+        }
+        if (ks > 1 && (int64_t) nbatch * ks <= 65535) {
+            void * ws = nullptr;
+            if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) == VX_OK) {
+                mm_args b = a;
+                b.ksplit = ks; b.partial = (float *) ws;
+                mm_kernel<WT, 4, ACT_Q8, false><<<dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st>>>(b);
+                const int64_t units = a.N * (a.M / 4);
+                mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+                return;
+            }
+            (void) hipGetLastError();
+        }
+        const dim3 grid((unsigned) gx, (unsigned) gy, (unsigned) nbatch);
         mm_kernel<WT, 4, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
     }
 }
