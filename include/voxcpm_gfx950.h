@@ -149,7 +149,11 @@ VX_API vx_status vx_kv_store(const vx_tensor * src, const vx_tensor * view, vx_s
 enum { VX_BIN_ADD = 0, VX_BIN_SUB = 1, VX_BIN_MUL = 2, VX_BIN_DIV = 3 };
 /* enum ggml_unary_op (third_party/ggml/include/ggml.h:578-603), the ones implemented */
 enum { VX_UNARY_ABS = 0, VX_UNARY_SGN = 1, VX_UNARY_NEG = 2, VX_UNARY_STEP = 3, VX_UNARY_TANH = 4,
-       VX_UNARY_RELU = 6, VX_UNARY_SIGMOID = 7, VX_UNARY_SILU = 10, VX_UNARY_EXP = 13 };
+       VX_UNARY_RELU = 6, VX_UNARY_SIGMOID = 7, VX_UNARY_SILU = 10, VX_UNARY_EXP = 13,
+       VX_UNARY_FLOOR = 18, VX_UNARY_CEIL = 19, VX_UNARY_ROUND = 20, VX_UNARY_TRUNC = 21,
+       /* ggml's stand-alone elementwise ops (GGML_OP_SQR / SQRT / LOG / SIN / COS,
+        * ggml/src/ggml-cpu/unary-ops.cpp:52-70), served by the same call; codes of this library */
+       VX_UNARY_SQR = 100, VX_UNARY_SQRT = 101, VX_UNARY_LOG = 102, VX_UNARY_SIN = 103, VX_UNARY_COS = 104 };
 /* enum ggml_glu_op (ggml.h:605-614) */
 enum { VX_GLU_REGLU = 0, VX_GLU_SWIGLU = 2 };
 
@@ -167,12 +171,25 @@ VX_API vx_status vx_unary(int op, const vx_tensor * src, const vx_tensor * dst, 
 VX_API vx_status vx_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int swapped, vx_stream stream);
 /* GGML_OP_CPY / CONT / DUP between F32 and F16 tensors holding the same number of elements:
  * element i of src (row-major over src's shape) lands in element i of dst
- * (ggml_compute_forward_dup, ops.cpp:526-565); F32 -> F16 rounds to nearest even. */
+ * (ggml_compute_forward_dup, ops.cpp:526-565); F32 -> F16 rounds to nearest even.  Also I32 -> F32
+ * (ggml_cast of position ids, src/minicpm.cpp:606), F32 -> I32 (C truncation) and I32 -> I32. */
 VX_API vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
 /* GGML_OP_CONCAT along `dim`, F32 / F16 / I32 (ops.cpp:1891-2095) */
 VX_API vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim, vx_stream stream);
 /* GGML_OP_SUM: every element summed in double, rounded once (ops.cpp:1275-1300) */
 VX_API vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_ARANGE: dst[i] = start + step * i over a contiguous F32 tensor, the product rounded before the sum
+ * (ggml_compute_forward_arange_f32, ops.cpp:7881-7902); the element count is dst's (ggml fixes it at graph build) */
+VX_API vx_status vx_arange(const vx_tensor * dst, float start, float step, vx_stream stream);
+/* GGML_OP_REPEAT: src tiled over dst, every dst dim a whole multiple of src's; F32 / F16 / I32, any strides
+ * (ggml_compute_forward_repeat, ops.cpp:1689-1810).  The reference builds its attention masks from ARANGE +
+ * REPEAT (src/minicpm.cpp:602-620, src/locdit.cpp:283-305). */
+VX_API vx_status vx_repeat(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_GET_ROWS: dst[:, i, j, k] = row rows[i, j, k] of table matrix (j, k), as F32; table F32 / F16 / Q8_0
+ * (dequantised exactly as dequantize_row_q8_0, ggml/src/ggml-quants.c:401-415) or I32 (dst I32); rows I32
+ * (ggml_compute_forward_get_rows, ops.cpp:4653-4870; the token embedding, src/components.cpp:223).  An index
+ * outside the table makes ggml-cpu abort; here it is clamped into the table. */
+VX_API vx_status vx_get_rows(const vx_tensor * table, const vx_tensor * rows, const vx_tensor * dst, vx_stream stream);
 
 /* ---- adjacent node pairs as one launch ----------------------------------------------------------
  * What a backend's graph_compute may substitute for two consecutive nodes whose intermediate has no
@@ -283,6 +300,9 @@ VX_API int vx_supports_unary_like(const vx_tensor * src, const vx_tensor * dst);
 VX_API int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * dst);
 VX_API int vx_supports_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst);
+VX_API int vx_supports_arange(const vx_tensor * dst);
+VX_API int vx_supports_repeat(const vx_tensor * src, const vx_tensor * dst);
+VX_API int vx_supports_get_rows(const vx_tensor * table, const vx_tensor * rows, const vx_tensor * dst);
 VX_API int vx_supports_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim);
 VX_API int vx_supports_sum(const vx_tensor * src, const vx_tensor * dst);
 

@@ -252,7 +252,7 @@ backbone * g_bb = nullptr;
 // graph_compute, and add per layer a small term computed by an operator no accelerator plugin here claims (GELU of
 // the normalised hidden state), so that the scheduler cuts the graph and a value in the middle of the device's part
 // is also read from the CPU's part.
-bool g_bb_sched = false, g_bb_probe = false;
+bool g_bb_sched = false, g_bb_probe = false, g_bb_whole = false;
 
 ggml_tensor * bb_norm(ggml_context * c, const backbone & m, ggml_tensor * x, ggml_tensor * w) {
     return ggml_mul(c, ggml_rms_norm(c, x, m.eps), w);
@@ -387,6 +387,12 @@ void rh_bb_options(int use_sched, int probe) {
     g_bb_probe = probe != 0;
 }
 
+// When on, the graph also holds what the reference puts around the decoder stack: the causal mask is built from
+// the position ids by the node chain of MiniCPMModel::create_causal_mask (src/minicpm.cpp:602-620: ARANGE, CAST,
+// REPEAT x2, SUB, ADD1, STEP, SCALE, CAST + CONT) instead of being handed in, and the input rows go through a
+// GET_ROWS (the embedding lookup of src/components.cpp:223, here over the input matrix with identity ids).
+void rh_bb_whole_graph(int on) { g_bb_whole = on != 0; }
+
 // Row-fused weight copies, as MiniCPMModel::load_from_store makes them for the LocDiT decoder on a GPU backend
 // (src/minicpm.cpp:427-492): qkv_proj = rows of q, k, v; gate_up_proj = rows of gate, up.  Call after rh_bb_set.
 int rh_bb_fuse_weights(void) {
@@ -443,10 +449,27 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     ggml_context * c = ggml_init(ip);
     ggml_tensor * inp = ggml_new_tensor_2d(c, GGML_TYPE_F32, m.hidden, (int64_t) T * B);
     ggml_tensor * pos = ggml_new_tensor_1d(c, GGML_TYPE_I32, T);
+    const bool whole = g_bb_whole && !g_bb_sched;
     ggml_tensor * msk = mask ? ggml_new_tensor_2d(c, GGML_TYPE_F16, n_past + T, T) : nullptr;
+    ggml_tensor * ids = whole ? ggml_new_tensor_1d(c, GGML_TYPE_I32, (int64_t) T * B) : nullptr;
     ggml_set_input(inp); ggml_set_input(pos);
     if (msk) ggml_set_input(msk);
     ggml_tensor * h = inp;
+    if (whole) {
+        ggml_set_input(ids);
+        h = ggml_get_rows(c, inp, ids);
+        if (mask) { // the mask values handed in are not used: the graph derives them from pos
+            const int total = n_past + T;
+            ggml_tensor * keys = ggml_reshape_2d(c, ggml_arange(c, 0.0f, (float) total, 1.0f), total, 1);
+            ggml_tensor * qpos = ggml_reshape_2d(c, ggml_cast(c, pos, GGML_TYPE_F32), 1, T);
+            ggml_tensor * target = ggml_new_tensor_2d(c, GGML_TYPE_F32, total, T);
+            ggml_tensor * mk = ggml_sub(c, ggml_repeat(c, keys, target), ggml_repeat(c, qpos, target));
+            mk = ggml_add1(c, mk, ggml_arange(c, -0.5f, 0.5f, 1.0f));
+            mk = ggml_scale(c, ggml_step(c, mk), -1.0e9f);
+            msk = ggml_cont(c, ggml_cast(c, mk, GGML_TYPE_F16));
+        }
+    }
+    const bool mask_is_input = msk && !(whole && mask);
     std::vector<ggml_tensor *> roots;
     for (const auto & L : m.layers) h = bb_layer_forward(c, m, L, h, pos, msk, T, n_past, write_kv != 0, roots);
     h = bb_norm(c, m, h, m.final_norm);
@@ -486,7 +509,12 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
         std::vector<int32_t> p((size_t) T);
         for (int i = 0; i < T; ++i) p[(size_t) i] = n_past + i;
         ggml_backend_tensor_set(pos, p.data(), 0, ggml_nbytes(pos));
-        if (msk) ggml_backend_tensor_set(msk, mask, 0, ggml_nbytes(msk));
+        if (mask_is_input) ggml_backend_tensor_set(msk, mask, 0, ggml_nbytes(msk));
+        if (ids) {
+            std::vector<int32_t> id((size_t) T * B);
+            for (size_t i = 0; i < id.size(); ++i) id[i] = (int32_t) i;
+            ggml_backend_tensor_set(ids, id.data(), 0, ggml_nbytes(ids));
+        }
         if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
     }
     if (!rc && reps > 0 && seconds) {

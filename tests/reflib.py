@@ -176,6 +176,8 @@ def load_ref():
     lib.rh_bb_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_options.argtypes = [C.c_int, C.c_int]
     lib.rh_bb_options.restype = None
+    lib.rh_bb_whole_graph.argtypes = [C.c_int]
+    lib.rh_bb_whole_graph.restype = None
     lib.rh_bb_fuse_weights.argtypes = []
     lib.rh_bb_forward.argtypes = [f32p, u16p, C.c_int, C.c_int, C.c_int, f32p, C.c_int, f64p]
     assert lib.rh_use_device(b"CPU", min(8, os.cpu_count() or 1), 0) == 0

@@ -125,6 +125,32 @@ def test_supports_truth_table_glue(pkg):
     assert lib.vx_supports_sum(a, one) == 1 and lib.vx_supports_sum(a, f32(pkg, [2, 1, 1, 1])) == 0
     permuted = D(pkg, pkg.F32, [5, 1024, 1, 1], [4096, 4, 20480, 20480])
     assert lib.vx_supports_sum(permuted, one) == 0
+    # the ops around the stacks: masks (ARANGE, REPEAT, I32 -> F32 cast), embeddings (GET_ROWS), rounding, sin / cos
+    def i32(ne):
+        return D(pkg, pkg.I32, ne, [4, 4 * ne[0], 4 * ne[0] * ne[1], 4 * ne[0] * ne[1] * ne[2]])
+    assert lib.vx_supports_cpy(i32([5, 1, 1, 1]), f32(pkg, [5, 1, 1, 1])) == 1
+    assert lib.vx_supports_cpy(f32(pkg, [5, 1, 1, 1]), i32([5, 1, 1, 1])) == 1
+    assert lib.vx_supports_cpy(i32([5, 1, 1, 1]), i32([1, 5, 1, 1])) == 1
+    assert lib.vx_supports_cpy(i32([5, 1, 1, 1]), f16(pkg, [5, 1, 1, 1])) == 0              # ggml-cpu has no such copy either
+    assert lib.vx_supports_arange(f32(pkg, [4096, 1, 1, 1])) == 1
+    assert lib.vx_supports_arange(f16(pkg, [8, 1, 1, 1])) == 0
+    assert lib.vx_supports_arange(D(pkg, pkg.F32, [8, 1, 1, 1], [8, 64, 64, 64])) == 0      # ggml-cpu asserts dense elements
+    assert lib.vx_supports_repeat(f32(pkg, [4096, 1, 1, 1]), f32(pkg, [4096, 512, 1, 1])) == 1  # key positions over queries
+    assert lib.vx_supports_repeat(f32(pkg, [1, 512, 1, 1]), f32(pkg, [4096, 512, 1, 1])) == 1   # query positions over keys
+    assert lib.vx_supports_repeat(f32(pkg, [3, 1, 1, 1]), f32(pkg, [4096, 1, 1, 1])) == 0       # not a whole multiple
+    assert lib.vx_supports_repeat(f32(pkg, [8, 1, 1, 1]), f16(pkg, [16, 1, 1, 1])) == 0
+    vocab = 73448
+    for table in (f32(pkg, [1024, vocab, 1, 1]), f16(pkg, [1024, vocab, 1, 1]), q8(pkg, [1024, vocab, 1, 1])):
+        assert lib.vx_supports_get_rows(table, i32([7, 1, 1, 1]), f32(pkg, [1024, 7, 1, 1])) == 1
+        assert lib.vx_supports_get_rows(table, i32([7, 1, 1, 1]), f32(pkg, [1024, 8, 1, 1])) == 0
+        assert lib.vx_supports_get_rows(table, f32(pkg, [7, 1, 1, 1]), f32(pkg, [1024, 7, 1, 1])) == 0   # indices must be I32
+        assert lib.vx_supports_get_rows(table, i32([7, 2, 1, 1]), f32(pkg, [1024, 7, 2, 1])) == 0        # one table matrix per index column
+    assert lib.vx_supports_get_rows(i32([16, 9, 1, 1]), i32([3, 1, 1, 1]), i32([16, 3, 1, 1])) == 1
+    assert lib.vx_supports_get_rows(i32([16, 9, 1, 1]), i32([3, 1, 1, 1]), f32(pkg, [16, 3, 1, 1])) == 0
+    for op in (pkg.UNARY_FLOOR, pkg.UNARY_CEIL, pkg.UNARY_ROUND, pkg.UNARY_TRUNC, pkg.UNARY_SQR, pkg.UNARY_SQRT,
+               pkg.UNARY_LOG, pkg.UNARY_SIN, pkg.UNARY_COS):
+        assert lib.vx_supports_unary(op, a, a) == 1, op
+    assert lib.vx_supports_unary(105, a, a) == 0 and lib.vx_supports_unary(17, a, a) == 0
     # fused pairs
     w = f32(pkg, [1024, 1, 1, 1])
     assert lib.vx_supports_rms_norm_mul(a, w, a) == 1

@@ -244,3 +244,38 @@ def test_plugin_under_the_scheduler_with_a_cross_split_reader(gpu, ref, T0):
         e = nmse(a, b)
         print(f"   plugin + scheduler vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
         assert e <= 1e-4
+
+
+@pytest.mark.parametrize("T0", [9, 300])
+def test_plugin_runs_the_whole_forward_graph_without_a_scheduler(gpu, ref, T0):
+    """VoxCPM's default is a direct graph_compute on one backend (src/backend.cpp:569), which only works when every node
+    of the graph is claimed.  Here the graph also holds the reference's mask-building chain (ARANGE, CAST, REPEAT,
+    SUB, ADD1, STEP, SCALE, CAST, CONT: src/minicpm.cpp:602-620) and an embedding GET_ROWS: the plugin must run it
+    as it stands, and give bit for bit what it gives when the finished mask is handed in."""
+    params = reflib.backbone_params("bb", N_LAYER)
+    max_len = T0 + 20
+    xp = rng("bbg", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)
+    xs = rng("bbg", "x", 1).standard_normal((BATCH, 1, 1024)).astype(np.float32)
+    mask0 = reflib.causal_mask(T0, T0)
+
+    def run(device, whole):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        ref.rh_bb_whole_graph(int(whole))
+        try:
+            reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=False)
+            outs = [reflib.ref_backbone_forward(xp, 0, mask0)[0], reflib.ref_backbone_forward(xs, T0, None)[0]]
+        finally:
+            ref.rh_bb_whole_graph(0)
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs
+
+    cpu = run(b"CPU", True)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    whole = run(b"GFX950_0", True)
+    handed = run(b"GFX950_0", False)
+    for i, (a, b, c) in enumerate(zip(cpu, whole, handed)):
+        e = nmse(a, b)
+        print(f"   whole graph on the plugin vs ggml-cpu, call {i}: nmse {e:.3e}", flush=True)
+        assert e <= 1e-4
+        assert np.array_equal(b, c), i

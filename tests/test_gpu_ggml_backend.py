@@ -18,7 +18,10 @@ pytestmark = pytest.mark.gpu
 
 OPS = ["RMS_NORM", "ROPE", "SOFT_MAX", "FLASH_ATTN_EXT", "MUL_MAT",
        # the glue of a decoder layer
-       "ADD", "SUB", "MUL", "DIV", "ADD1", "SCALE", "CPY", "CONT", "DUP", "CONCAT", "SUM", "SILU", "SWIGLU"]
+       "ADD", "SUB", "MUL", "DIV", "ADD1", "SCALE", "CPY", "CONT", "DUP", "CONCAT", "SUM", "SILU", "SWIGLU",
+       # the ops around the stacks: masks, token embeddings, the timestep embedding, FSQ's rounding
+       "ARANGE", "REPEAT", "GET_ROWS", "SIN", "COS", "SQR", "SQRT", "LOG", "ROUND", "FLOOR", "CEIL", "TRUNC",
+       "STEP", "ABS", "EXP", "TANH"]
 
 
 def plugin_path(pkg):

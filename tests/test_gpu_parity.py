@@ -570,3 +570,129 @@ def test_glue_cpy_cont_concat_sum(gpu, cache_dtype):
         shp = list(a.shape); shp[3 - gd] += 2
         b = rng("glue3", "b", gd).standard_normal([2 if i == 3 - gd else n for i, n in enumerate(a.shape)]).astype(cache_dtype)
         assert np.array_equal(sync_np(gpu.concat(dev(a), dev(b), gd)), np.concatenate([a, b], axis=3 - gd))
+
+
+# ------------------------------------------- the ops around the decoder stacks (masks, embeddings)
+def test_glue_arange_repeat_and_the_mask_chains(gpu):
+    """ARANGE / REPEAT are exact; chained with SUB, ADD1, STEP / ABS, SCALE and the F32 -> F16 cast
+    they build the reference's causal mask (src/minicpm.cpp:602-620) and CFG-pair mask
+    (src/locdit.cpp:283-305), compared here with the masks written down directly."""
+    import torch
+    say("glue: arange / repeat / mask chains")
+    for start, stop, step in ((0.0, 10.0, 1.0), (-0.5, 0.5, 1.0), (0.3, 77.1, 0.7), (5.0, -3.0, -0.25)):
+        got = sync_np(gpu.arange(start, stop, step))
+        f = np.float32
+        n = int(np.ceil((f(stop) - f(start)) / f(step)))
+        want = (f(start) + (f(step) * np.arange(n, dtype=np.float32)).astype(np.float32)).astype(np.float32)
+        assert got.shape == (n,) and np.array_equal(got, want), (start, stop, step)
+    for dt in (np.float32, np.float16, np.int32):
+        a = (rng("rep", str(dt)).standard_normal((2, 1, 3, 8)) * 100).astype(dt)
+        for reps in ((1, 1, 1, 1), (1, 4, 1, 2), (3, 2, 2, 1), (2, 1, 1, 5)):
+            shape = tuple(n * r for n, r in zip(a.shape, reps))
+            assert np.array_equal(sync_np(gpu.repeat(dev(a), shape)), np.tile(a, reps)), (dt, reps)
+        b = a[..., :5]                                            # odd rows, strided source
+        assert np.array_equal(sync_np(gpu.repeat(dev(a)[..., :5], (2, 2, 3, 10))), np.tile(b, (1, 2, 1, 2)))
+    # causal mask for 5 queries at positions 3..7 over 8 keys
+    total, pos = 8, np.arange(3, 8, dtype=np.int32)
+    keys = gpu.arange(0.0, float(total), 1.0).reshape(1, total)
+    qpos = torch.empty((len(pos), 1), dtype=torch.float32, device="cuda")
+    gpu.cpy(dev(pos).reshape(len(pos), 1), qpos)                  # ggml_cast I32 -> F32
+    grid_k, grid_q = gpu.repeat(keys, (len(pos), total)), gpu.repeat(qpos, (len(pos), total))
+    m = gpu.binary(gpu.BIN_SUB, grid_k, grid_q)
+    m = gpu.add1(m, gpu.arange(-0.5, 0.5, 1.0))
+    m = gpu.scale(gpu.unary(gpu.UNARY_STEP, m), -1e9)
+    m16 = torch.empty(m.shape, dtype=torch.float16, device="cuda")
+    gpu.cpy(m, m16)
+    want = np.where(np.arange(total)[None, :] > pos[:, None], -np.inf, -0.0).astype(np.float16)
+    assert np.array_equal(sync_np(m16).view(np.uint16), want.view(np.uint16))
+    # CFG-pair mask: two branches of 7 tokens see only themselves
+    L = 7
+    ids = gpu.unary(gpu.UNARY_STEP, gpu.add1(gpu.arange(0.0, 2.0 * L, 1.0), gpu.arange(0.5 - L, 1.5 - L, 1.0)))
+    kg, qg = gpu.repeat(ids.reshape(1, 2 * L), (2 * L, 2 * L)), gpu.repeat(ids.reshape(2 * L, 1), (2 * L, 2 * L))
+    m = gpu.scale(gpu.unary(gpu.UNARY_ABS, gpu.binary(gpu.BIN_SUB, kg, qg)), -1e9)
+    m16 = torch.empty(m.shape, dtype=torch.float16, device="cuda")
+    gpu.cpy(m, m16)
+    br = np.arange(2 * L) >= L
+    want = np.where(br[None, :] != br[:, None], -np.inf, 0.0).astype(np.float16)
+    assert np.array_equal(sync_np(m16), want)
+
+
+def test_glue_get_rows(gpu):
+    """GET_ROWS gathers exactly: F32 / I32 rows as bits, F16 widened, Q8_0 as quant * scale (one rounding,
+    the oracle's dequantisation); batched tables and a strided index view as ggml's tests use them."""
+    import torch
+    say("glue: get_rows")
+    n_vocab, nc = 517, 96
+    idx = rng("gr", "idx").integers(0, n_vocab, size=(33,)).astype(np.int32)
+    tab = rng("gr", "t").standard_normal((n_vocab, nc)).astype(np.float32)
+    assert np.array_equal(sync_np(gpu.get_rows(dev(tab), dev(idx))), tab[idx])
+    t16 = tab.astype(np.float16)
+    assert np.array_equal(sync_np(gpu.get_rows(dev(t16), dev(idx))), t16[idx].astype(np.float32))
+    ti = (tab * 1e8).astype(np.int32)
+    got = sync_np(gpu.get_rows(dev(ti), dev(idx)))
+    assert got.dtype == np.int32 and np.array_equal(got, ti[idx])
+    raw = reflib.quantize_q8_0(tab)                               # (n_vocab, nc / 32 * 34) bytes
+    blocks = raw.reshape(n_vocab, nc // 32, 34)
+    d = blocks[:, :, :2].copy().view(np.float16).astype(np.float32)            # (n_vocab, nb, 1)
+    q = blocks[:, :, 2:].view(np.int8).astype(np.float32)
+    deq = (q * d).reshape(n_vocab, nc)
+    got = sync_np(gpu.get_rows(dev(raw), dev(idx), ne0=nc))
+    assert np.array_equal(got, deq[idx])
+    # batched: table (2, 3, rows, nc), indices (2, 3, n): matrix (j, k) serves index column (j, k)
+    tb = rng("gr", "tb").standard_normal((2, 3, 11, 40)).astype(np.float32)
+    ib = rng("gr", "ib").integers(0, 11, size=(2, 3, 6)).astype(np.int32)
+    want = np.take_along_axis(tb, ib[..., None].astype(np.int64), axis=2)
+    assert np.array_equal(sync_np(gpu.get_rows(dev(tb), dev(ib))), want)
+    # strided indices (every other entry) and a strided destination
+    wide = torch.zeros((17, 2 * nc), dtype=torch.float32, device="cuda")
+    gpu.get_rows(dev(tab), dev(idx)[::2], out=wide[:, :nc])
+    assert np.array_equal(sync_np(wide)[:, :nc], tab[idx[::2]]) and not sync_np(wide)[:, nc:].any()
+    # an index outside the table stays inside it (ggml-cpu aborts there)
+    bad = np.array([-5, n_vocab + 3], np.int32)
+    assert np.array_equal(sync_np(gpu.get_rows(dev(tab), dev(bad))), tab[[0, n_vocab - 1]])
+
+
+def test_glue_rounding_unaries_and_integer_copies(gpu):
+    """FLOOR / CEIL / ROUND / TRUNC / SQR / SQRT are single correctly rounded operations: bit-exact against
+    numpy (ROUND rounds halves away from zero as roundf does); SIN / COS / LOG within 2 ulp-sized steps of
+    the fp64 value (ggml-cpu calls libm's sinf / cosf / logf); I32 <-> F32 copies are C casts."""
+    import torch
+    say("glue: rounding unaries, sin / cos / log, integer copies")
+    x = (rng("un", "x").standard_normal((3, 7, 130)) * 37).astype(np.float32)
+    x[0, 0, :8] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.0, -0.0]
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_FLOOR, dev(x))), np.floor(x))
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_CEIL, dev(x))), np.ceil(x))
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_TRUNC, dev(x))), np.trunc(x))
+    away = (np.sign(x) * np.floor(np.abs(x.astype(np.float64)) + 0.5)).astype(np.float32)
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_ROUND, dev(x))), away)
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_SQR, dev(x))), x * x)
+    assert np.array_equal(sync_np(gpu.unary(gpu.UNARY_SQRT, dev(np.abs(x)))), np.sqrt(np.abs(x)))
+    x64 = x.astype(np.float64)
+    for op, fn in ((gpu.UNARY_SIN, np.sin), (gpu.UNARY_COS, np.cos)):
+        got = sync_np(gpu.unary(op, dev(x)))
+        assert np.abs(got - fn(x64)).max() <= 2.5e-7
+    xl = np.abs(x) + np.float32(1e-3)
+    got = sync_np(gpu.unary(gpu.UNARY_LOG, dev(xl)))
+    assert np.abs(got - np.log(xl.astype(np.float64))).max() <= 1e-6
+    # the LocDiT timestep embedding's tail (src/locdit.cpp:198-212): sin / cos of t * exp(-k * i)
+    i = gpu.arange(0.0, 128.0, 1.0)
+    emb = gpu.scale(gpu.unary(gpu.UNARY_EXP, gpu.scale(i, -float(np.log(10000.0) / 127))), 1000.0 * 0.37)
+    s = sync_np(gpu.unary(gpu.UNARY_SIN, emb))
+    e64 = np.exp(np.arange(128) * -(np.log(10000.0) / 127)) * 370.0
+    assert np.abs(s - np.sin(e64)).max() <= 5e-4                  # the argument (up to 370) carries its own fp32 roundings
+    # integer copies
+    ints = np.array([[0, 1, -1, 2**24 + 1, -(2**24) - 3, 2**31 - 1, -(2**31), 123456789]], np.int32)
+    f = torch.empty(ints.shape, dtype=torch.float32, device="cuda")
+    gpu.cpy(dev(ints), f)
+    assert np.array_equal(sync_np(f), ints.astype(np.float32))
+    ii = torch.empty(ints.shape, dtype=torch.int32, device="cuda")
+    gpu.cpy(dev(ints), ii)
+    assert np.array_equal(sync_np(ii), ints)                      # bits, not through float
+    vals = np.array([[0.0, 0.9, -0.9, 7.5, -7.5, 16777217.0, -2.0e9, 1.9e9]], np.float32)
+    gpu.cpy(dev(vals), ii)
+    assert np.array_equal(sync_np(ii), vals.astype(np.int32))
+    # transposing I32 -> F32 copy (strided source)
+    grid = np.arange(35, dtype=np.int32).reshape(5, 7)
+    ft = torch.empty((7, 5), dtype=torch.float32, device="cuda")
+    gpu.cpy(dev(grid).t(), ft)
+    assert np.array_equal(sync_np(ft), grid.T.astype(np.float32))

@@ -42,11 +42,14 @@ EXPORTS = [
     "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum",
     "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
+    "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
     "vx_rms_norm_mul", "vx_scale_add", "vx_add_scale", "vx_flash_attn_ext_add1", "vx_mul_mat_swiglu", "vx_supports_mul_mat_swiglu", "vx_mul_mat_scale_add", "vx_supports_mul_mat_scale_add", "vx_kv_store_sync", "vx_supports_kv_store_sync", "vx_flash_attn_ext_kv2", "vx_supports_flash_attn_ext_kv2", "vx_flash_attn_ext_kv2_store", "vx_supports_flash_attn_ext_kv2_store", "vx_qkv_proj_rope", "vx_supports_qkv_proj_rope", "vx_norm_qkv_proj_rope", "vx_supports_norm_qkv_proj_rope", "vx_norm_mul_mat_swiglu", "vx_supports_norm_mul_mat_swiglu", "vx_supports_rms_norm_mul", "vx_supports_fused_pair",
 ]
 
 BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV = 0, 1, 2, 3
 UNARY_ABS, UNARY_SGN, UNARY_NEG, UNARY_STEP, UNARY_TANH, UNARY_RELU, UNARY_SIGMOID, UNARY_SILU, UNARY_EXP = 0, 1, 2, 3, 4, 6, 7, 10, 13
+UNARY_FLOOR, UNARY_CEIL, UNARY_ROUND, UNARY_TRUNC = 18, 19, 20, 21
+UNARY_SQR, UNARY_SQRT, UNARY_LOG, UNARY_SIN, UNARY_COS = 100, 101, 102, 103, 104   # ggml's stand-alone ops
 GLU_REGLU, GLU_SWIGLU = 0, 2
 
 _lib = None
@@ -105,6 +108,12 @@ def lib():
     l.vx_supports_cpy.argtypes = [TP, TP]
     l.vx_supports_concat.argtypes = [TP, TP, TP, C.c_int]
     l.vx_supports_sum.argtypes = [TP, TP]
+    l.vx_arange.argtypes = [TP, C.c_float, C.c_float, vp]
+    l.vx_repeat.argtypes = [TP, TP, vp]
+    l.vx_get_rows.argtypes = [TP, TP, TP, vp]
+    l.vx_supports_arange.argtypes = [TP]
+    l.vx_supports_repeat.argtypes = [TP, TP]
+    l.vx_supports_get_rows.argtypes = [TP, TP, TP]
     l.vx_rms_norm_mul.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_scale_add.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_add_scale.argtypes = [TP, TP, TP, C.c_float, C.c_float, vp]
@@ -290,6 +299,38 @@ def concat(a, b, ggml_dim, out=None):
         shape[a.dim() - 1 - ggml_dim] += b.shape[b.dim() - 1 - ggml_dim]
         out = torch.empty(shape, dtype=a.dtype, device=a.device)
     check(lib().vx_concat(desc(a), desc(b), desc(out), ggml_dim, _stream()), "vx_concat")
+    return out
+
+
+def arange(start, stop, step, device="cuda"):
+    """ggml_arange: ceil((stop - start) / step) values start + step * i."""
+    import math
+    import numpy as np
+    import torch
+    n = int(math.ceil((np.float32(stop) - np.float32(start)) / np.float32(step)))
+    out = torch.empty((n,), dtype=torch.float32, device=device)
+    check(lib().vx_arange(desc(out), start, step, _stream()), "vx_arange")
+    return out
+
+
+def repeat(a, shape, out=None):
+    """ggml_repeat: `a` tiled to `shape` (torch order), each dim a whole multiple of a's."""
+    import torch
+    out = torch.empty(shape, dtype=a.dtype, device=a.device) if out is None else out
+    check(lib().vx_repeat(desc(a), desc(out), _stream()), "vx_repeat")
+    return out
+
+
+def get_rows(table, rows, ne0=None, out=None):
+    """ggml_get_rows: `table` a float / int32 torch tensor, or Q8_0 rows as uint8 with the row length `ne0`;
+    `rows` int32 indices; result (..., rows, ne0) F32 (I32 for an I32 table)."""
+    import torch
+    td = desc_q8(table, ne0) if ne0 is not None else desc(table)
+    nc = ne0 if ne0 is not None else table.shape[-1]
+    if out is None:
+        shape = list(rows.shape) + [nc]
+        out = torch.empty(shape, dtype=torch.int32 if table.dtype == torch.int32 else torch.float32, device=rows.device)
+    check(lib().vx_get_rows(td, desc(rows), desc(out), _stream()), "vx_get_rows")
     return out
 
 

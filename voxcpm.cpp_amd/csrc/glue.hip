@@ -12,6 +12,7 @@
 #include "kvs_common.hpp"
 
 #include <cmath>
+#include <type_traits>
 
 namespace {
 
@@ -48,6 +49,15 @@ __device__ __forceinline__ float unary_f(int op, float x) {
         case VX_UNARY_SIGMOID: return 1.0f / (1.0f + expf(-x));
         case VX_UNARY_SILU:    return silu_f(x);
         case VX_UNARY_EXP:     return expf(x);
+        case VX_UNARY_FLOOR:   return floorf(x);
+        case VX_UNARY_CEIL:    return ceilf(x);
+        case VX_UNARY_ROUND:   return roundf(x); // halves away from zero, as libm's
+        case VX_UNARY_TRUNC:   return truncf(x);
+        case VX_UNARY_SQR:     return x * x;
+        case VX_UNARY_SQRT:    return sqrtf(x);
+        case VX_UNARY_LOG:     return logf(x);
+        case VX_UNARY_SIN:     return sinf(x);
+        case VX_UNARY_COS:     return cosf(x);
         default:               return x;
     }
 }
@@ -159,6 +169,14 @@ struct cpy_args {
     int64_t  n;
 };
 
+// same type: the bits (integers above 2^24 and NaN payloads survive); otherwise through float, as
+// ggml_compute_forward_dup_flt converts (ggml/src/ggml-cpu/common.h:34-40: I32 <-> F32 are C casts)
+template <typename TS, typename TD>
+__device__ __forceinline__ TD cpy_convert(TS x) {
+    if constexpr (std::is_same<TS, TD>::value) return x;
+    else                                       return (TD) (float) x;
+}
+
 template <typename TS, typename TD, int VEC>
 __global__ __launch_bounds__(256) void cpy_kernel(const cpy_args a) {
     const int64_t e = ((int64_t) blockIdx.x * 256 + threadIdx.x) * VEC;
@@ -174,14 +192,14 @@ __global__ __launch_bounds__(256) void cpy_kernel(const cpy_args a) {
     const int64_t d2 = r % a.ned[2]; const int64_t d3 = r / a.ned[2];
     char * pd = a.d + d0 * a.nbd[0] + d1 * a.nbd[1] + d2 * a.nbd[2] + d3 * a.nbd[3];
     if constexpr (VEC == 1) {
-        *(TD *) pd = (TD) (float) *(const TS *) ps;
+        *(TD *) pd = cpy_convert<TS, TD>(*(const TS *) ps);
     } else { // 4 consecutive elements of a dense run on both sides
         typedef TS vs_t __attribute__((ext_vector_type(4)));
         typedef TD vd_t __attribute__((ext_vector_type(4)));
         const vs_t x = *(const vs_t *) ps;
         vd_t y;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) y[k] = (TD) (float) x[k];
+        for (int k = 0; k < 4; ++k) y[k] = cpy_convert<TS, TD>(x[k]);
         *(vd_t *) pd = y;
     }
 }
@@ -229,6 +247,75 @@ __global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
     if constexpr (UNIT == 16)     *(int4_t *) pd = *(const int4_t *) ps;
     else if constexpr (UNIT == 4) *(int32_t *) pd = *(const int32_t *) ps;
     else                          *(int16_t *) pd = *(const int16_t *) ps;
+}
+
+// ---- ARANGE / REPEAT / GET_ROWS -----------------------------------------------------------------
+// The ops the reference's graphs use around the decoder stacks: the causal and CFG-pair masks are
+// built from ARANGE + REPEAT (src/minicpm.cpp:602-620, src/locdit.cpp:283-305), token embeddings are
+// a GET_ROWS (src/components.cpp:223).  With them a whole forward graph stays on the device.
+__global__ __launch_bounds__(256) void arange_kernel(float * d, int64_t n, float start, float step) {
+#pragma clang fp contract(off)
+    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float t = step * (float) i; // product rounded, then the sum: ops.cpp:7899
+    d[i] = start + t;
+}
+
+struct rep_args {
+    const char * s; char * d;
+    int64_t  ne[4], nes[4];   // dst shape, src shape
+    uint64_t nbs[4], nbd[4];
+    int64_t  n;               // dst units
+};
+
+// UNIT bytes per thread: the element, or 16 when src rows are whole 16-byte groups
+template <int UNIT, int ES>
+__global__ __launch_bounds__(256) void repeat_kernel(const rep_args a) {
+    const int64_t u = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (u >= a.n) return;
+    constexpr int EPU = UNIT / ES;
+    const int64_t units0 = a.ne[0] / EPU;
+    int64_t r = u;
+    const int64_t i0 = (r % units0) * EPU; r /= units0;
+    const int64_t i1 = r % a.ne[1]; r /= a.ne[1];
+    const int64_t i2 = r % a.ne[2]; const int64_t i3 = r / a.ne[2];
+    char *       pd = a.d + i0 * a.nbd[0] + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+    const char * ps = a.s + (i0 % a.nes[0]) * a.nbs[0] + (i1 % a.nes[1]) * a.nbs[1] + (i2 % a.nes[2]) * a.nbs[2] + (i3 % a.nes[3]) * a.nbs[3];
+    if constexpr (UNIT == 16)     *(int4_t *) pd = *(const int4_t *) ps;
+    else if constexpr (UNIT == 4) *(int32_t *) pd = *(const int32_t *) ps;
+    else                          *(int16_t *) pd = *(const int16_t *) ps;
+}
+
+struct rows_args {
+    const char * table; const char * idx; char * d;
+    int64_t  nc, n_rows_table;       // row length, rows per table matrix
+    int64_t  ne10, ne11, ne12;       // index tensor shape
+    uint64_t nb01, nb02, nb03, nb10, nb11, nb12, nb1, nb2, nb3;
+    int64_t  nchunk;
+};
+
+// one block per (index, 256 * VEC columns).  WT: 0 = 4-byte elements copied as bits (F32, I32),
+// 1 = F16 widened, 2 = Q8_0 dequantised as dequantize_row_q8_0 does (quant * f16 scale, one rounding)
+template <int WT>
+__global__ __launch_bounds__(256) void get_rows_kernel(const rows_args a) {
+    const int64_t r = blockIdx.x / a.nchunk, chunk = blockIdx.x % a.nchunk;
+    const int64_t i10 = r % a.ne10, i11 = (r / a.ne10) % a.ne11, i12 = r / (a.ne10 * a.ne11);
+    int64_t row = *(const int32_t *) (a.idx + i10 * a.nb10 + i11 * a.nb11 + i12 * a.nb12);
+    // ggml-cpu aborts on an index outside the table (ops.cpp:4689); a kernel cannot, so it stays in bounds
+    row = row < 0 ? 0 : (row >= a.n_rows_table ? a.n_rows_table - 1 : row);
+    const char * src = a.table + row * a.nb01 + i11 * a.nb02 + i12 * a.nb03;
+    char *       dst = a.d + i10 * a.nb1 + i11 * a.nb2 + i12 * a.nb3;
+    const int64_t c = chunk * 256 + threadIdx.x;
+    if (c >= a.nc) return;
+    if constexpr (WT == 0) {
+        *(int32_t *) (dst + c * 4) = *(const int32_t *) (src + c * 4);
+    } else if constexpr (WT == 1) {
+        *(float *) (dst + c * 4) = (float) *(const _Float16 *) (src + c * 2);
+    } else {
+        const char * blk = src + (c >> 5) * 34;
+        const float  d   = (float) *(const _Float16 *) blk;
+        *(float *) (dst + c * 4) = (float) *(const int8_t *) (blk + 2 + (c & 31)) * d;
+    }
 }
 
 // ---- SUM ---------------------------------------------------------------------------------------
@@ -438,7 +525,9 @@ extern "C" vx_status vx_add_scale(const vx_tensor * a, const vx_tensor * b, cons
 extern "C" int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * dst) {
     switch (op) {
         case VX_UNARY_ABS: case VX_UNARY_SGN: case VX_UNARY_NEG: case VX_UNARY_STEP: case VX_UNARY_TANH:
-        case VX_UNARY_RELU: case VX_UNARY_SIGMOID: case VX_UNARY_SILU: case VX_UNARY_EXP: break;
+        case VX_UNARY_RELU: case VX_UNARY_SIGMOID: case VX_UNARY_SILU: case VX_UNARY_EXP:
+        case VX_UNARY_FLOOR: case VX_UNARY_CEIL: case VX_UNARY_ROUND: case VX_UNARY_TRUNC:
+        case VX_UNARY_SQR: case VX_UNARY_SQRT: case VX_UNARY_LOG: case VX_UNARY_SIN: case VX_UNARY_COS: break;
         default: return 0;
     }
     return vx_supports_unary_like(src, dst);
@@ -485,13 +574,17 @@ extern "C" vx_status vx_glu(int op, const vx_tensor * src0, const vx_tensor * sr
 }
 
 extern "C" int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst) {
-    if (!src || !dst || !fl_type(src->type) || !fl_type(dst->type)) return 0;
+    if (!src || !dst) return 0;
+    // F32 / F16 in any combination; I32 to and from F32 (ggml_cast of position ids) and I32 to I32
+    const bool ints = (src->type == VX_TYPE_I32 && (dst->type == VX_TYPE_F32 || dst->type == VX_TYPE_I32)) ||
+                      (src->type == VX_TYPE_F32 && dst->type == VX_TYPE_I32);
+    if (!ints && (!fl_type(src->type) || !fl_type(dst->type))) return 0;
     if (!vx_positive(src) || !vx_positive(dst) || vx_nelements(src) != vx_nelements(dst)) return 0;
     return nb_multiple(src, vx_type_size(src->type)) && nb_multiple(dst, vx_type_size(dst->type));
 }
 
 extern "C" vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
-    if (!vx_supports_cpy(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "cpy: F32/F16 tensors holding the same number of elements");
+    if (!vx_supports_cpy(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "cpy: F32/F16 (or I32 <-> F32) tensors holding the same number of elements");
     if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "cpy: null data");
     cpy_args a;
     a.s = (const char *) src->data; a.d = (char *) dst->data; a.n = vx_nelements(src);
@@ -502,6 +595,10 @@ extern "C" vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_str
                      src->nb[1] % (4 * ss) == 0 && src->nb[2] % (4 * ss) == 0 && src->nb[3] % (4 * ss) == 0 &&
                      dst->nb[1] % (4 * ds) == 0 && dst->nb[2] % (4 * ds) == 0 && dst->nb[3] % (4 * ds) == 0;
     hipStream_t st = (hipStream_t) stream;
+    if (src->type == VX_TYPE_I32) {
+        return dst->type == VX_TYPE_I32 ? cpy_launch<int32_t, int32_t>(a, vec, st) : cpy_launch<int32_t, float>(a, vec, st);
+    }
+    if (dst->type == VX_TYPE_I32) return cpy_launch<float, int32_t>(a, vec, st);
     if (src->type == VX_TYPE_F32) {
         return dst->type == VX_TYPE_F32 ? cpy_launch<float, float>(a, vec, st) : cpy_launch<float, _Float16>(a, vec, st);
     }
@@ -545,6 +642,89 @@ extern "C" vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, c
     if (vec)          { if (es == 4) concat_kernel<16, 4><<<grid, block, 0, st>>>(a); else concat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
     else if (es == 4) concat_kernel<4, 4><<<grid, block, 0, st>>>(a);
     else              concat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+extern "C" int vx_supports_arange(const vx_tensor * dst) {
+    return f32(dst) && vx_positive(dst) && vx_is_contiguous(dst);
+}
+
+extern "C" vx_status vx_arange(const vx_tensor * dst, float start, float step, vx_stream stream) {
+    if (!vx_supports_arange(dst)) return vx_fail(VX_ERR_UNSUPPORTED, "arange: a contiguous F32 tensor");
+    if (!dst->data) return vx_fail(VX_ERR_INVALID, "arange: null data");
+    const int64_t n = vx_nelements(dst), blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "arange: launch too large");
+    arange_kernel<<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>((float *) dst->data, n, start, step);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+extern "C" int vx_supports_repeat(const vx_tensor * src, const vx_tensor * dst) {
+    if (!src || !dst || src->type != dst->type) return 0;
+    if (src->type != VX_TYPE_F32 && src->type != VX_TYPE_F16 && src->type != VX_TYPE_I32) return 0;
+    if (!vx_positive(src) || !vx_positive(dst) || !can_repeat(src, dst)) return 0;
+    const uint64_t es = vx_type_size(src->type);
+    return nb_multiple(src, es) && nb_multiple(dst, es);
+}
+
+extern "C" vx_status vx_repeat(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_repeat(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "repeat: F32/F16/I32, dst a whole multiple of src in every dim");
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "repeat: null data");
+    rep_args a;
+    a.s = (const char *) src->data; a.d = (char *) dst->data;
+    for (int i = 0; i < 4; ++i) { a.ne[i] = dst->ne[i]; a.nes[i] = src->ne[i]; a.nbs[i] = src->nb[i]; a.nbd[i] = dst->nb[i]; }
+    const int es = (int) vx_type_size(src->type), epu = 16 / es;
+    auto dense16 = [&](const vx_tensor * t) {
+        return t->nb[0] == (uint64_t) es && (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+    };
+    const bool vec = src->ne[0] % epu == 0 && dense16(src) && dense16(dst);
+    const int64_t n_el = vx_nelements(dst);
+    a.n = vec ? n_el / epu : n_el;
+    const int64_t blocks = (a.n + 255) / 256;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "repeat: launch too large");
+    const dim3 grid((unsigned) blocks), block(256);
+    hipStream_t st = (hipStream_t) stream;
+    if (vec)          { if (es == 4) repeat_kernel<16, 4><<<grid, block, 0, st>>>(a); else repeat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
+    else if (es == 4) repeat_kernel<4, 4><<<grid, block, 0, st>>>(a);
+    else              repeat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+extern "C" int vx_supports_get_rows(const vx_tensor * table, const vx_tensor * rows, const vx_tensor * dst) {
+    if (!table || !rows || !dst || rows->type != VX_TYPE_I32) return 0;
+    const int tt = table->type;
+    if (tt != VX_TYPE_F32 && tt != VX_TYPE_F16 && tt != VX_TYPE_Q8_0 && tt != VX_TYPE_I32) return 0;
+    if (dst->type != (tt == VX_TYPE_I32 ? VX_TYPE_I32 : VX_TYPE_F32)) return 0;
+    if (!vx_positive(table) || !vx_positive(rows) || !vx_positive(dst)) return 0;
+    if (tt == VX_TYPE_Q8_0 && table->ne[0] % 32) return 0;
+    // ggml_get_rows (ggml.c): dst = [ne00, ne10, ne11, ne12]; table matrices are picked by (i11, i12)
+    if (rows->ne[3] != 1 || table->ne[2] != rows->ne[1] || table->ne[3] != rows->ne[2]) return 0;
+    if (dst->ne[0] != table->ne[0] || dst->ne[1] != rows->ne[0] || dst->ne[2] != rows->ne[1] || dst->ne[3] != rows->ne[2]) return 0;
+    if (table->nb[0] != vx_type_size(tt) || dst->nb[0] != 4) return 0;
+    const uint64_t ts = tt == VX_TYPE_F16 || tt == VX_TYPE_Q8_0 ? 2 : 4;
+    return nb_multiple(rows, 4) && nb_multiple(dst, 4) && table->nb[1] % ts == 0 && table->nb[2] % ts == 0 && table->nb[3] % ts == 0;
+}
+
+extern "C" vx_status vx_get_rows(const vx_tensor * table, const vx_tensor * rows, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_get_rows(table, rows, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "get_rows: F32/F16/Q8_0/I32 table with dense rows, I32 indices");
+    if (!table->data || !rows->data || !dst->data) return vx_fail(VX_ERR_INVALID, "get_rows: null data");
+    rows_args a;
+    a.table = (const char *) table->data; a.idx = (const char *) rows->data; a.d = (char *) dst->data;
+    a.nc = table->ne[0]; a.n_rows_table = table->ne[1];
+    a.ne10 = rows->ne[0]; a.ne11 = rows->ne[1]; a.ne12 = rows->ne[2];
+    a.nb01 = table->nb[1]; a.nb02 = table->nb[2]; a.nb03 = table->nb[3];
+    a.nb10 = rows->nb[0]; a.nb11 = rows->nb[1]; a.nb12 = rows->nb[2];
+    a.nb1 = dst->nb[1]; a.nb2 = dst->nb[2]; a.nb3 = dst->nb[3];
+    a.nchunk = (a.nc + 255) / 256;
+    const int64_t blocks = vx_nelements(rows) * a.nchunk;
+    if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "get_rows: launch too large");
+    const dim3 grid((unsigned) blocks), block(256);
+    hipStream_t st = (hipStream_t) stream;
+    if (table->type == VX_TYPE_F16)       get_rows_kernel<1><<<grid, block, 0, st>>>(a);
+    else if (table->type == VX_TYPE_Q8_0) get_rows_kernel<2><<<grid, block, 0, st>>>(a);
+    else                                  get_rows_kernel<0><<<grid, block, 0, st>>>(a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -64,6 +64,18 @@ int binary_code(ggml_op op) {
     }
 }
 
+// ggml's stand-alone elementwise ops that the library serves through vx_unary; -1 for any other op
+int standalone_unary_code(ggml_op op) {
+    switch (op) {
+        case GGML_OP_SQR:  return VX_UNARY_SQR;
+        case GGML_OP_SQRT: return VX_UNARY_SQRT;
+        case GGML_OP_LOG:  return VX_UNARY_LOG;
+        case GGML_OP_SIN:  return VX_UNARY_SIN;
+        case GGML_OP_COS:  return VX_UNARY_COS;
+        default:           return -1;
+    }
+}
+
 int mul_mat_act_mode() {
     static const int mode = [] {
         const char * e = getenv("GGML_GFX950_MUL_MAT_ACT");
@@ -285,6 +297,26 @@ bool supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
             return vx_supports_sum(&a, &d) != 0;
         }
+        case GGML_OP_SQR:
+        case GGML_OP_SQRT:
+        case GGML_OP_LOG:
+        case GGML_OP_SIN:
+        case GGML_OP_COS: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_unary(standalone_unary_code(op->op), &a, &d) != 0;
+        }
+        case GGML_OP_ARANGE: {
+            const vx_tensor d = to_vx(op);
+            return vx_supports_arange(&d) != 0;
+        }
+        case GGML_OP_REPEAT: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_repeat(&a, &d) != 0;
+        }
+        case GGML_OP_GET_ROWS: {
+            const vx_tensor a = to_vx(op->src[0]), b = to_vx(op->src[1]), d = to_vx(op);
+            return vx_supports_get_rows(&a, &b, &d) != 0;
+        }
         default:
             return false;
     }
@@ -335,6 +367,29 @@ vx_status compute_node(backend_ctx * ctx, ggml_tensor * node) {
         case GGML_OP_SUM: {
             const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
             return vx_sum(&a, &d, ctx->stream);
+        }
+        case GGML_OP_SQR:
+        case GGML_OP_SQRT:
+        case GGML_OP_LOG:
+        case GGML_OP_SIN:
+        case GGML_OP_COS: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_unary(standalone_unary_code(node->op), &a, &d, ctx->stream);
+        }
+        case GGML_OP_ARANGE: {
+            float start, step; // ggml.c: start, stop, step
+            memcpy(&start, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&step, (const float *) node->op_params + 2, sizeof(float));
+            const vx_tensor d = to_vx(node);
+            return vx_arange(&d, start, step, ctx->stream);
+        }
+        case GGML_OP_REPEAT: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_repeat(&a, &d, ctx->stream);
+        }
+        case GGML_OP_GET_ROWS: {
+            const vx_tensor a = to_vx(node->src[0]), b = to_vx(node->src[1]), d = to_vx(node);
+            return vx_get_rows(&a, &b, &d, ctx->stream);
         }
         case GGML_OP_RMS_NORM: {
             float eps;
