@@ -301,6 +301,30 @@ VX_API int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * ds
 VX_API int vx_supports_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst);
 VX_API int vx_supports_arange(const vx_tensor * dst);
+
+/* ---- a run of tiny nodes as one launch -------------------------------------------------------------
+ * Around the decoder stacks the reference's graphs hold chains of operators over a few hundred values: bias adds,
+ * the CONCATs that assemble LocDiT's CFG-pair sequence (src/locdit.cpp:401-464), the guidance arithmetic and the Euler
+ * update of UnifiedCFM (src/unified_cfm.cpp:30-149).  vx_small_graph runs up to 16 such nodes, in the order given, in ONE
+ * launch (one work-group, a barrier between nodes); every node writes its own dst as its separate call would, with the
+ * same arithmetic and the same summation order, so the results are those of the separate calls.  Each tensor of a node
+ * holds at most 16384 elements.  No counterpart in ggml-cpu, which runs the nodes one by one. */
+enum { VX_NODE_ADD = 0, VX_NODE_SUB = 1, VX_NODE_MUL = 2, VX_NODE_DIV = 3,  /* vx_binary                        */
+       VX_NODE_ADD1 = 4,                                                    /* vx_add1                          */
+       VX_NODE_SCALE = 5,                                                   /* vx_scale: p0 = scale, p1 = bias  */
+       VX_NODE_UNARY = 6,                                                   /* vx_unary: aux = VX_UNARY_*       */
+       VX_NODE_CPY = 7,                                                     /* vx_cpy (CPY / CONT / DUP)        */
+       VX_NODE_CONCAT = 8,                                                  /* vx_concat: aux = dim             */
+       VX_NODE_REPEAT = 9,                                                  /* vx_repeat                        */
+       VX_NODE_SUM = 10,                                                    /* vx_sum                           */
+       VX_NODE_ARANGE = 11 };                                               /* vx_arange: p0 = start, p1 = step */
+typedef struct vx_small_node {
+    int32_t op, aux;
+    float   p0, p1;
+    const vx_tensor * src0, * src1, * dst;   /* src1 NULL where the operator has one operand, src0 NULL for ARANGE */
+} vx_small_node;
+VX_API vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx_stream stream);
+VX_API int vx_supports_small_node(const vx_small_node * node);
 VX_API int vx_supports_repeat(const vx_tensor * src, const vx_tensor * dst);
 VX_API int vx_supports_get_rows(const vx_tensor * table, const vx_tensor * rows, const vx_tensor * dst);
 VX_API int vx_supports_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim);

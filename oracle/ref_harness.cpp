@@ -543,4 +543,158 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     return rc;
 }
 
+// ---- a whole CFM solve as one graph ---------------------------------------------------------------------------
+// The graph UnifiedCFM::forward builds (src/unified_cfm.cpp:88-184) around the LocDiT estimator's CFG-pair pass
+// (src/locdit.cpp:248-258, 401-464): per Euler step the noisy patches are projected to the hidden size, the
+// conditioned and unconditioned branches ride as ONE sequence of 2 * (1 + prefix + patch) tokens through the
+// decoder stack (block-diagonal mask, positions i mod branch length, no cache write), both branches are projected
+// back, combined by classifier-free guidance (zero-star scale: SUM, MUL, DIV, REPEAT, ARANGE for eps) and x takes
+// the step.  The decoder is the stack made by rh_bb_create (batch 1; call rh_bb_fuse_weights for the row-fused
+// variant the reference uses on GPU backends); the estimator's own projections are Q8_0 like every matrix the
+// reference's quantizer writes for a Q8_0 model file (src/quantize.cpp:411-428), their biases F32.
+namespace {
+struct cfm_extra {
+    ggml_context *        ctx = nullptr;
+    ggml_backend_buffer_t buf = nullptr;
+    ggml_tensor * w[3] = { nullptr, nullptr, nullptr }; // in_proj, cond_proj [feat, hidden]; out_proj [hidden, feat]
+    ggml_tensor * b[3] = { nullptr, nullptr, nullptr };
+    int feat = 0;
+};
+cfm_extra * g_cfm = nullptr;
+} // namespace
+
+void rh_cfm_free(void) {
+    if (!g_cfm) return;
+    if (g_cfm->buf) ggml_backend_buffer_free(g_cfm->buf);
+    if (g_cfm->ctx) ggml_free(g_cfm->ctx);
+    delete g_cfm;
+    g_cfm = nullptr;
+}
+
+// weights as Q8_0 rows: in_w, cond_w [hidden][feat]; out_w [feat][hidden] (rows of ne0 = the input size); F32 biases
+// hidden / hidden / feat
+int rh_cfm_create(int feat, const void * in_w, const float * in_b, const void * cond_w, const float * cond_b,
+                  const void * out_w, const float * out_b) {
+    if (!g_bb || !g_backend || g_bb->batch != 1) return 100;
+    rh_cfm_free();
+    cfm_extra * e = new cfm_extra;
+    e->feat = feat;
+    ggml_init_params ip = { ggml_tensor_overhead() * 8, nullptr, true };
+    e->ctx = ggml_init(ip);
+    const int64_t H = g_bb->hidden;
+    e->w[0] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, feat, H); e->b[0] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, H);
+    e->w[1] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, feat, H); e->b[1] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, H);
+    e->w[2] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, H, feat); e->b[2] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, feat);
+    e->buf = ggml_backend_alloc_ctx_tensors(e->ctx, g_backend);
+    g_cfm = e;
+    if (!e->buf) { rh_cfm_free(); return 101; }
+    const void *  ws[3] = { in_w, cond_w, out_w };
+    const float * bs[3] = { in_b, cond_b, out_b };
+    for (int i = 0; i < 3; ++i) {
+        ggml_backend_tensor_set(e->w[i], ws[i], 0, ggml_nbytes(e->w[i]));
+        ggml_backend_tensor_set(e->b[i], bs[i], 0, ggml_nbytes(e->b[i]));
+    }
+    return 0;
+}
+
+// z [feat, patch], mu [hidden], cond [feat, prefix], time_table [hidden, n_steps] (the combined time embedding of every
+// step, as LocDiTModel::precompute_cfg_time_table hands it over), t_span n_steps + 1 values, pair_pos / pair_mask the
+// CFG-pair constants for a branch of 1 + prefix + patch tokens.  out [feat, patch].  seconds: mean, best, node count.
+int rh_cfm_solve(const float * z, const float * mu, const float * cond, const float * time_table, const float * t_span,
+                 int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
+                 int zero_star, float * out, int reps, double * seconds) {
+    if (!g_bb || !g_cfm || !g_backend || n_steps < 1 || prefix < 1) return 100;
+    const backbone & m = *g_bb;
+    const cfm_extra & e = *g_cfm;
+    const int H = m.hidden, F = e.feat, L = 1 + prefix + patch, T = 2 * L;
+    if (T > m.max_len) return 104;
+    const size_t n_nodes = (size_t) n_steps * ((size_t) m.n_layer * 64 + 96) + 64;
+    ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
+    ggml_context * c = ggml_init(ip);
+    ggml_tensor * zin  = ggml_new_tensor_2d(c, GGML_TYPE_F32, F, patch);
+    ggml_tensor * muin = ggml_new_tensor_1d(c, GGML_TYPE_F32, H);
+    ggml_tensor * cin  = ggml_new_tensor_2d(c, GGML_TYPE_F32, F, prefix);
+    ggml_tensor * tab  = ggml_new_tensor_1d(c, GGML_TYPE_F32, (int64_t) H * n_steps);
+    ggml_tensor * pos  = ggml_new_tensor_1d(c, GGML_TYPE_I32, T);
+    ggml_tensor * msk  = ggml_new_tensor_2d(c, GGML_TYPE_F16, T, T);
+    for (ggml_tensor * t : { zin, muin, cin, tab, pos, msk }) ggml_set_input(t);
+
+    std::vector<ggml_tensor *> roots;
+    ggml_tensor * x = zin;
+    ggml_tensor * cond_proj = ggml_add(c, ggml_mul_mat(c, e.w[1], cin), e.b[1]);
+    float t = t_span[0], dt = t_span[0] - t_span[1];
+    const int zero_init_steps = n_steps > 1 ? std::max(1, (int) ((float) (n_steps + 1) * 0.04f)) : 0;
+    for (int step = 1; step <= n_steps; ++step) {
+        ggml_tensor * dphi;
+        if (zero_star && step <= zero_init_steps) {
+            dphi = ggml_scale(c, x, 0.0f);
+        } else {
+            ggml_tensor * x_proj   = ggml_add(c, ggml_mul_mat(c, e.w[0], x), e.b[0]);
+            ggml_tensor * combined = ggml_view_1d(c, tab, H, (size_t) (step - 1) * H * sizeof(float));
+            ggml_tensor * comb_c   = ggml_reshape_2d(c, ggml_add(c, ggml_reshape_1d(c, combined, H), muin), H, 1);
+            ggml_tensor * comb_u   = ggml_reshape_2d(c, combined, H, 1);
+            ggml_tensor * seq_c    = ggml_concat(c, ggml_concat(c, comb_c, cond_proj, 1), x_proj, 1);
+            ggml_tensor * seq_u    = ggml_concat(c, ggml_concat(c, comb_u, cond_proj, 1), x_proj, 1);
+            ggml_tensor * h        = ggml_concat(c, seq_c, seq_u, 1);
+            for (const auto & Lr : m.layers) h = bb_layer_forward(c, m, Lr, h, pos, msk, T, 0, false, roots);
+            h = bb_norm(c, m, h, m.final_norm);
+            ggml_tensor * hc = ggml_view_2d(c, h, H, patch, h->nb[1], (size_t) (prefix + 1) * h->nb[1]);
+            ggml_tensor * hu = ggml_view_2d(c, h, H, patch, h->nb[1], (size_t) (L + prefix + 1) * h->nb[1]);
+            ggml_tensor * vc = ggml_add(c, ggml_mul_mat(c, e.w[2], hc), e.b[2]);
+            ggml_tensor * vu = ggml_add(c, ggml_mul_mat(c, e.w[2], hu), e.b[2]);
+            if (zero_star) {
+                ggml_tensor * dot = ggml_sum(c, ggml_mul(c, vc, vu));
+                ggml_tensor * nrm = ggml_sum(c, ggml_mul(c, vu, vu));
+                ggml_tensor * st  = ggml_div(c, dot, ggml_add(c, nrm, ggml_arange(c, 1.0e-8f, 1.0e-8f + 1.0f, 1.0f)));
+                ggml_tensor * us  = ggml_mul(c, vu, ggml_repeat(c, st, vu));
+                dphi = ggml_add(c, us, ggml_scale(c, ggml_sub(c, vc, us), cfg_value));
+            } else {
+                dphi = ggml_add(c, vu, ggml_scale(c, ggml_sub(c, vc, vu), cfg_value));
+            }
+        }
+        x = ggml_sub(c, x, ggml_scale(c, dphi, dt));
+        t -= dt;
+        if (step < n_steps) dt = t - t_span[step + 1];
+    }
+    ggml_set_output(x);
+    ggml_cgraph * gf = ggml_new_graph_custom(c, n_nodes, false);
+    ggml_build_forward_expand(gf, x);
+
+    ggml_gallocr_t ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend));
+    int rc = 0;
+    if (!ggml_gallocr_alloc_graph(ga, gf)) rc = 101;
+    auto upload = [&] { // inputs may share memory with later nodes of the graph: written before every run
+        ggml_backend_tensor_set(zin, z, 0, ggml_nbytes(zin));
+        ggml_backend_tensor_set(muin, mu, 0, ggml_nbytes(muin));
+        ggml_backend_tensor_set(cin, cond, 0, ggml_nbytes(cin));
+        ggml_backend_tensor_set(tab, time_table, 0, ggml_nbytes(tab));
+        ggml_backend_tensor_set(pos, pair_pos, 0, ggml_nbytes(pos));
+        ggml_backend_tensor_set(msk, pair_mask, 0, ggml_nbytes(msk));
+    };
+    if (!rc) {
+        upload();
+        if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
+    }
+    if (!rc && out) ggml_backend_tensor_get(x, out, 0, ggml_nbytes(x));
+    if (!rc && reps > 0 && seconds) {
+        double best = 1e30, total = 0;
+        for (int r = 0; r < reps && !rc; ++r) {
+            upload();
+            auto t0 = std::chrono::steady_clock::now();
+            if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
+            auto t1 = std::chrono::steady_clock::now();
+            const double d = std::chrono::duration<double>(t1 - t0).count();
+            total += d;
+            if (d < best) best = d;
+        }
+        seconds[0] = total / reps;
+        seconds[1] = best;
+    }
+    if (seconds) seconds[2] = (double) ggml_graph_n_nodes(gf);
+    ggml_gallocr_free(ga);
+    ggml_free(c);
+    return rc;
+}
+
+
 } // extern "C"

@@ -178,6 +178,12 @@ def load_ref():
     lib.rh_bb_options.restype = None
     lib.rh_bb_whole_graph.argtypes = [C.c_int]
     lib.rh_bb_whole_graph.restype = None
+    f32p_, i32p_, u16p_ = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint16)
+    lib.rh_cfm_create.argtypes = [C.c_int, C.c_void_p, f32p_, C.c_void_p, f32p_, C.c_void_p, f32p_]
+    lib.rh_cfm_solve.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int,
+                                 f32p_, C.c_int, C.POINTER(C.c_double)]
+    lib.rh_cfm_free.argtypes = []
+    lib.rh_cfm_free.restype = None
     lib.rh_bb_fuse_weights.argtypes = []
     lib.rh_bb_forward.argtypes = [f32p, u16p, C.c_int, C.c_int, C.c_int, f32p, C.c_int, f64p]
     assert lib.rh_use_device(b"CPU", min(8, os.cpu_count() or 1), 0) == 0
@@ -379,5 +385,49 @@ def ref_backbone_forward(x, n_past, mask=None, write_kv=True, reps=0):
     m = None if mask is None else np.ascontiguousarray(mask).view(np.uint16)
     rc = lib.rh_bb_forward(ptr(x, C.c_float), None if m is None else ptr(m, C.c_uint16), x.shape[1], n_past, int(write_kv),
                            ptr(out, C.c_float), reps, ptr(sec, C.c_double))
+    assert rc == 0, rc
+    return out, sec[:2].copy(), int(sec[2])
+
+
+def cfm_params(tag, feat=64, hidden=1024):
+    """Seeded weights of the LocDiT estimator's own projections (in_proj, cond_proj: feat -> hidden; out_proj:
+    hidden -> feat; quantised to Q8_0 on upload), scaled so that activations stay O(1)."""
+    g = lambda *k: rng(tag, *k)
+    return {"feat": feat, "hidden": hidden,
+            "in_w": (g("in_w").standard_normal((hidden, feat)) / np.sqrt(feat)).astype(np.float32),
+            "in_b": (0.1 * g("in_b").standard_normal(hidden)).astype(np.float32),
+            "cond_w": (g("cond_w").standard_normal((hidden, feat)) / np.sqrt(feat)).astype(np.float32),
+            "cond_b": (0.1 * g("cond_b").standard_normal(hidden)).astype(np.float32),
+            "out_w": (g("out_w").standard_normal((feat, hidden)) / np.sqrt(hidden)).astype(np.float32),
+            "out_b": (0.1 * g("out_b").standard_normal(feat)).astype(np.float32)}
+
+
+def ref_cfm_create(p):
+    """The estimator's projections beside the decoder stack made by ref_backbone_create (batch 1)."""
+    lib = load_ref()
+    f = lambda a: ptr(np.ascontiguousarray(a), C.c_float)
+    q = {n: quantize_q8_0(p[n]) for n in ("in_w", "cond_w", "out_w")}   # Q8_0, as the reference's quantizer stores them
+    rc = lib.rh_cfm_create(p["feat"], q["in_w"].ctypes.data, f(p["in_b"]), q["cond_w"].ctypes.data, f(p["cond_b"]),
+                           q["out_w"].ctypes.data, f(p["out_b"]))
+    assert rc == 0, rc
+
+
+def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_star=True, reps=0):
+    """One UnifiedCFM solve as a single graph on the harness's device.  z (patch, feat), mu (hidden,), cond (prefix, feat),
+    table (n_steps, hidden).  Returns (x (patch, feat), seconds[mean, best], n_nodes)."""
+    lib, orc = load_ref(), load_oracle()
+    z, mu, cond, table = (np.ascontiguousarray(a, dtype=np.float32) for a in (z, mu, cond, table))
+    patch, prefix = z.shape[0], cond.shape[0]
+    L = 1 + prefix + patch
+    t_span = np.zeros(n_steps + 1, np.float32)
+    orc.orc_t_span(n_steps, sway, ptr(t_span, C.c_float))
+    pos = np.zeros(2 * L, np.int32)
+    mk = np.zeros((2 * L, 2 * L), np.uint16)
+    orc.orc_cfg_pair_constants(L, ptr(pos, C.c_int32), ptr(mk, C.c_uint16))
+    out = np.empty_like(z)
+    sec = np.zeros(3, np.float64)
+    rc = lib.rh_cfm_solve(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), ptr(table, C.c_float), ptr(t_span, C.c_float),
+                          n_steps, patch, prefix, ptr(pos, C.c_int32), ptr(mk, C.c_uint16), cfg_value, int(zero_star),
+                          ptr(out, C.c_float), reps, ptr(sec, C.c_double))
     assert rc == 0, rc
     return out, sec[:2].copy(), int(sec[2])

@@ -488,3 +488,133 @@ def test_groups_with_f16_weights(pkg, gpu, N):
     assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
     assert torch.equal(a1, a2)
     assert torch.equal(r1, r2)
+
+
+# ------------------------------------------------------------------------- runs of tiny nodes
+def _run_both(gpu, program, tensors):
+    """program: list of (op, dst, src0, src1, aux, p0, p1) over names in `tensors` (name -> numpy array, the initial
+    contents).  Runs it node by node through the separate entry points and as ONE vx_small_graph launch, each on its
+    own copy of the tensors; returns both sets of device tensors."""
+    import torch
+    sets = []
+    for mode in ("separate", "one launch"):
+        T = {k: dev(v) for k, v in tensors.items()}
+        g = lambda n: None if n is None else (T[n[0]][n[1]] if isinstance(n, tuple) else T[n])   # (name, index) = a view
+        if mode == "separate":
+            for op, dst, s0, s1, aux, p0, p1 in program:
+                d, a, b = g(dst), g(s0), g(s1)
+                if op <= gpu.NODE_DIV: gpu.binary(op, a, b, out=d)
+                elif op == gpu.NODE_ADD1: gpu.add1(a, b, out=d)
+                elif op == gpu.NODE_SCALE: gpu.scale(a, p0, p1, out=d)
+                elif op == gpu.NODE_UNARY: gpu.unary(aux, a, out=d)
+                elif op == gpu.NODE_CPY: gpu.cpy(a, d)
+                elif op == gpu.NODE_CONCAT: gpu.concat(a, b, aux, out=d)
+                elif op == gpu.NODE_REPEAT: gpu.repeat(a, None, out=d)
+                elif op == gpu.NODE_SUM: gpu.sum_all(a, out=d)
+                else: gpu.check(gpu.lib().vx_arange(gpu.desc(d), p0, p1, None), "arange")
+        else:
+            nodes = [gpu.small_node(op, g(dst), g(s0), g(s1), aux, p0, p1) for op, dst, s0, s1, aux, p0, p1 in program]
+            for i in range(0, len(nodes), 16):
+                gpu.small_graph(nodes[i:i + 16])
+        torch.cuda.synchronize()
+        sets.append(T)
+    return sets
+
+
+def _assert_same(sets, what):
+    import torch
+    a, b = sets
+    for k in a:
+        x, y = a[k].contiguous(), b[k].contiguous()
+        assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (what, k)
+
+
+def test_small_graph_cfg_guidance_and_euler_update(gpu):
+    """The node chain UnifiedCFM puts behind the estimator (src/unified_cfm.cpp:30-86, 146): zero-star scale from two
+    SUMs, ARANGE for eps, DIV, REPEAT, the guidance combination and the Euler update of x -- 16 nodes, one launch, every
+    intermediate and the result bit-identical to the separate launches; NaN / infinity in the velocities included."""
+    say("small graph: CFG guidance + Euler update")
+    N = gpu
+    for poison in (None, np.nan, np.inf):
+        t = {"vc": rng("sg", "vc").standard_normal((2, 64)).astype(np.float32), "vu": rng("sg", "vu").standard_normal((2, 64)).astype(np.float32),
+             "x": rng("sg", "x").standard_normal((2, 64)).astype(np.float32), "bias": rng("sg", "b").standard_normal((64,)).astype(np.float32)}
+        if poison is not None:
+            t["vu"][1, 7] = poison
+        for name in ("pc", "pu", "uu", "us", "rep", "diff", "cs", "dphi", "step", "xn", "vcb", "vub"):
+            t[name] = np.zeros((2, 64), np.float32)
+        for name in ("dot", "nrm", "eps", "den", "st"):
+            t[name] = np.zeros((1,), np.float32)
+        prog = [(N.NODE_ADD, "vcb", "vc", "bias", 0, 0, 0), (N.NODE_ADD, "vub", "vu", "bias", 0, 0, 0),
+                (N.NODE_MUL, "pc", "vcb", "vub", 0, 0, 0), (N.NODE_SUM, "dot", "pc", None, 0, 0, 0),
+                (N.NODE_MUL, "uu", "vub", "vub", 0, 0, 0), (N.NODE_SUM, "nrm", "uu", None, 0, 0, 0),
+                (N.NODE_ARANGE, "eps", None, None, 0, 1e-8, 1.0), (N.NODE_ADD, "den", "nrm", "eps", 0, 0, 0),
+                (N.NODE_DIV, "st", "dot", "den", 0, 0, 0), (N.NODE_REPEAT, "rep", "st", None, 0, 0, 0),
+                (N.NODE_MUL, "us", "vub", "rep", 0, 0, 0), (N.NODE_SUB, "diff", "vcb", "us", 0, 0, 0),
+                (N.NODE_SCALE, "cs", "diff", None, 0, 2.0, 0.0), (N.NODE_ADD, "dphi", "us", "cs", 0, 0, 0),
+                (N.NODE_SCALE, "step", "dphi", None, 0, 0.0937, 0.0), (N.NODE_SUB, "xn", "x", "step", 0, 0, 0)]
+        sets = _run_both(gpu, prog, t)
+        _assert_same(sets, f"guidance poison={poison}")
+        if poison is None:
+            import torch
+            xn = sets[1]["xn"].cpu().numpy().astype(np.float64)
+            vc, vu = (t["vc"] + t["bias"]).astype(np.float64), (t["vu"] + t["bias"]).astype(np.float64)
+            st = (vc * vu).sum() / ((vu * vu).sum() + 1e-8)
+            want = t["x"] - 0.0937 * (st * vu + 2.0 * (vc - st * vu))
+            assert np.abs(xn - want).max() <= 1e-5
+
+
+def test_small_graph_sequence_assembly_copies_and_sums(gpu):
+    """CONCATs that assemble LocDiT's 14-token CFG-pair sequence (src/locdit.cpp:441-452), casts, strided and in-place
+    operands, and SUMs in each of vx_sum's single-block orders (one wave in 16-byte units, one wave element-wise on an
+    odd row length, the 1024-thread block beyond 1024 units)."""
+    import torch
+    say("small graph: concat / cpy / repeat / sum orders")
+    N = gpu
+    H = 1024
+    t = {"tok_c": rng("sg2", "tc").standard_normal((1, H)).astype(np.float32), "tok_u": rng("sg2", "tu").standard_normal((1, H)).astype(np.float32),
+         "cond": rng("sg2", "c").standard_normal((4, H)).astype(np.float32), "xp": rng("sg2", "x").standard_normal((2, H)).astype(np.float32),
+         "a5": np.zeros((5, H), np.float32), "b5": np.zeros((5, H), np.float32), "a7": np.zeros((7, H), np.float32), "b7": np.zeros((7, H), np.float32),
+         "pair": np.zeros((14, H), np.float32), "pair16": np.zeros((14, H), np.float16), "back": np.zeros((14, H), np.float32),
+         "ids": np.arange(14, dtype=np.int32), "idf": np.zeros((14,), np.float32), "idi": np.zeros((14,), np.int32),
+         "odd": rng("sg2", "odd").standard_normal((3, 333)).astype(np.float32), "s_vec": np.zeros((1,), np.float32),
+         "s_odd": np.zeros((1,), np.float32), "s_blk": np.zeros((1,), np.float32), "s_view": np.zeros((1,), np.float32),
+         "tile": np.zeros((3, 2, 4, 8), np.float32), "seed": rng("sg2", "seed").standard_normal((1, 2, 1, 8)).astype(np.float32),
+         "cat0": np.zeros((2, 2056), np.float32), "wide": rng("sg2", "w").standard_normal((2, 1028)).astype(np.float32)}
+    prog = [(N.NODE_CONCAT, "a5", "tok_c", "cond", 1, 0, 0), (N.NODE_CONCAT, "a7", "a5", "xp", 1, 0, 0),
+            (N.NODE_CONCAT, "b5", "tok_u", "cond", 1, 0, 0), (N.NODE_CONCAT, "b7", "b5", "xp", 1, 0, 0),
+            (N.NODE_CONCAT, "pair", "a7", "b7", 1, 0, 0),
+            (N.NODE_CPY, "pair16", "pair", None, 0, 0, 0), (N.NODE_CPY, "back", "pair16", None, 0, 0, 0),
+            (N.NODE_CPY, "idf", "ids", None, 0, 0, 0), (N.NODE_CPY, "idi", "idf", None, 0, 0, 0),
+            (N.NODE_SUM, "s_vec", "xp", None, 0, 0, 0),          # 512 units of 16 bytes: one wave
+            (N.NODE_SUM, "s_odd", "odd", None, 0, 0, 0),         # 999 single elements: one wave, element order
+            (N.NODE_SUM, "s_blk", "pair", None, 0, 0, 0),        # 3584 units: the 1024-thread block
+            (N.NODE_SUM, "s_view", ("pair", slice(3, 7)), None, 0, 0, 0),   # rows 3..6 of the sequence: a view
+            (N.NODE_REPEAT, "tile", "seed", None, 0, 0, 0),
+            (N.NODE_CONCAT, "cat0", "wide", "wide", 0, 0, 0),    # along dim 0, rows of 1028
+            (N.NODE_UNARY, "xp", "xp", None, N.UNARY_SILU, 0, 0),           # in place
+            (N.NODE_ADD1, "cond", "cond", "s_vec", 0, 0, 0),     # in place, scalar from an earlier node of the run
+            (N.NODE_SCALE, "back", "back", None, 0, 0.5, 1.25)]
+    sets = _run_both(gpu, prog, t)
+    _assert_same(sets, "assembly")
+    got = sets[1]
+    pair = np.concatenate([t["tok_c"], t["cond"], t["xp"], t["tok_u"], t["cond"], t["xp"]], axis=0)
+    assert np.array_equal(got["pair"].cpu().numpy(), pair)
+    assert float(got["s_blk"].cpu()[0]) == np.float32(pair.astype(np.float64).sum())
+    assert np.array_equal(got["idi"].cpu().numpy(), np.arange(14, dtype=np.int32))
+    assert np.array_equal(got["tile"].cpu().numpy(), np.tile(t["seed"], (3, 1, 4, 1)))
+
+
+def test_small_graph_limits(gpu, pkg):
+    """What a run may hold: at most 16 nodes, tensors of at most 16384 elements, only the tiny operators."""
+    import torch
+    L = pkg.lib()
+    small = torch.zeros((4, 1024), dtype=torch.float32, device="cuda")
+    big = torch.zeros((17, 1024), dtype=torch.float32, device="cuda")
+    nd = gpu.small_node(gpu.NODE_ADD, small, small, small)
+    assert L.vx_supports_small_node(nd) == 1
+    assert L.vx_supports_small_node(gpu.small_node(gpu.NODE_ADD, big, big, big)) == 0
+    assert L.vx_supports_small_node(gpu.small_node(12, small, small, small)) == 0
+    assert L.vx_supports_small_node(gpu.small_node(gpu.NODE_UNARY, small, small, aux=8)) == 0       # GELU
+    arr = (pkg.VxSmallNode * 17)(*([nd] * 17))
+    assert L.vx_small_graph(arr, 17, None) == 2   # VX_ERR_UNSUPPORTED
+    assert L.vx_small_graph(arr, 0, None) == 2   # VX_ERR_UNSUPPORTED

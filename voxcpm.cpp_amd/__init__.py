@@ -32,6 +32,18 @@ class VxTensor(C.Structure):
     ]
 
 
+class VxSmallNode(C.Structure):
+    _fields_ = [
+        ("op", C.c_int32),
+        ("aux", C.c_int32),
+        ("p0", C.c_float),
+        ("p1", C.c_float),
+        ("src0", C.POINTER(VxTensor)),
+        ("src1", C.POINTER(VxTensor)),
+        ("dst", C.POINTER(VxTensor)),
+    ]
+
+
 EXPORTS = [
     "vx_device_count", "vx_init", "vx_last_error", "vx_device_info", "vx_malloc", "vx_free",
     "vx_malloc_host", "vx_free_host", "vx_memcpy_h2d", "vx_memcpy_d2h", "vx_memcpy_d2d", "vx_memset",
@@ -43,6 +55,7 @@ EXPORTS = [
     "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
     "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
+    "vx_small_graph", "vx_supports_small_node",
     "vx_rms_norm_mul", "vx_scale_add", "vx_add_scale", "vx_flash_attn_ext_add1", "vx_mul_mat_swiglu", "vx_supports_mul_mat_swiglu", "vx_mul_mat_scale_add", "vx_supports_mul_mat_scale_add", "vx_kv_store_sync", "vx_supports_kv_store_sync", "vx_flash_attn_ext_kv2", "vx_supports_flash_attn_ext_kv2", "vx_flash_attn_ext_kv2_store", "vx_supports_flash_attn_ext_kv2_store", "vx_qkv_proj_rope", "vx_supports_qkv_proj_rope", "vx_norm_qkv_proj_rope", "vx_supports_norm_qkv_proj_rope", "vx_norm_mul_mat_swiglu", "vx_supports_norm_mul_mat_swiglu", "vx_supports_rms_norm_mul", "vx_supports_fused_pair",
 ]
 
@@ -51,6 +64,8 @@ UNARY_ABS, UNARY_SGN, UNARY_NEG, UNARY_STEP, UNARY_TANH, UNARY_RELU, UNARY_SIGMO
 UNARY_FLOOR, UNARY_CEIL, UNARY_ROUND, UNARY_TRUNC = 18, 19, 20, 21
 UNARY_SQR, UNARY_SQRT, UNARY_LOG, UNARY_SIN, UNARY_COS = 100, 101, 102, 103, 104   # ggml's stand-alone ops
 GLU_REGLU, GLU_SWIGLU = 0, 2
+(NODE_ADD, NODE_SUB, NODE_MUL, NODE_DIV, NODE_ADD1, NODE_SCALE, NODE_UNARY, NODE_CPY, NODE_CONCAT, NODE_REPEAT, NODE_SUM,
+ NODE_ARANGE) = range(12)
 
 _lib = None
 
@@ -114,6 +129,8 @@ def lib():
     l.vx_supports_arange.argtypes = [TP]
     l.vx_supports_repeat.argtypes = [TP, TP]
     l.vx_supports_get_rows.argtypes = [TP, TP, TP]
+    l.vx_small_graph.argtypes = [C.POINTER(VxSmallNode), C.c_int, vp]
+    l.vx_supports_small_node.argtypes = [C.POINTER(VxSmallNode)]
     l.vx_rms_norm_mul.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_scale_add.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_add_scale.argtypes = [TP, TP, TP, C.c_float, C.c_float, vp]
@@ -332,6 +349,27 @@ def get_rows(table, rows, ne0=None, out=None):
         out = torch.empty(shape, dtype=torch.int32 if table.dtype == torch.int32 else torch.float32, device=rows.device)
     check(lib().vx_get_rows(td, desc(rows), desc(out), _stream()), "vx_get_rows")
     return out
+
+
+def small_node(op, dst, src0=None, src1=None, aux=0, p0=0.0, p1=0.0):
+    """One node of a small graph: tensors as descriptors (VxTensor) or torch tensors."""
+    nd = VxSmallNode()
+    nd.op, nd.aux, nd.p0, nd.p1 = op, aux, p0, p1
+    keep = []
+    for name, t in (("src0", src0), ("src1", src1), ("dst", dst)):
+        if t is None:
+            continue
+        d = t if isinstance(t, VxTensor) else desc(t)
+        keep.append(d)
+        setattr(nd, name, C.pointer(d))
+    nd._keep = keep
+    return nd
+
+
+def small_graph(nodes):
+    """Runs up to 16 tiny nodes (small_node) in the order given as one launch."""
+    arr = (VxSmallNode * len(nodes))(*nodes)
+    check(lib().vx_small_graph(arr, len(nodes), _stream()), "vx_small_graph")
 
 
 def sum_all(a, out=None):

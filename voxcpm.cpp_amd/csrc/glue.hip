@@ -70,19 +70,20 @@ __device__ __forceinline__ float mul_then_add(float x, float s, float a) {
     return a + t;
 }
 
+// p0, p1, aux: the node's parameters (scale and bias, the unary / GLU code)
 template <int OP>
-__device__ __forceinline__ float ew_apply(const ew_args & a, float x, float y) {
+__device__ __forceinline__ float ew_apply(float p0, float p1, int aux, float x, float y) {
     if constexpr (OP == EW_ADD)   return x + y;
     if constexpr (OP == EW_SUB)   return x - y;
     if constexpr (OP == EW_MUL)   return x * y;
     if constexpr (OP == EW_DIV)   return x / y;
     if constexpr (OP == EW_ADD1)  return x + y;
-    if constexpr (OP == EW_SCALE) return a.p1 == 0.0f ? x * a.p0 : fmaf(x, a.p0, a.p1); // vec_scale / vec_mad1
-    if constexpr (OP == EW_UNARY) return unary_f(a.aux, x);
-    if constexpr (OP == EW_GLU)   return (a.aux == VX_GLU_REGLU ? (x > 0.0f ? x : 0.0f) : silu_f(x)) * y;
+    if constexpr (OP == EW_SCALE) return p1 == 0.0f ? x * p0 : fmaf(x, p0, p1); // vec_scale / vec_mad1
+    if constexpr (OP == EW_UNARY) return unary_f(aux, x);
+    if constexpr (OP == EW_GLU)   return (aux == VX_GLU_REGLU ? (x > 0.0f ? x : 0.0f) : silu_f(x)) * y;
     // the fused pairs round exactly where the two separate nodes would (no contraction)
-    if constexpr (OP == EW_SCALE_ADD) return mul_then_add(y, a.p0, x);
-    if constexpr (OP == EW_ADD_SCALE) { const float t = x + y; return a.p1 == 0.0f ? t * a.p0 : fmaf(t, a.p0, a.p1); }
+    if constexpr (OP == EW_SCALE_ADD) return mul_then_add(y, p0, x);
+    if constexpr (OP == EW_ADD_SCALE) { const float t = x + y; return p1 == 0.0f ? t * p0 : fmaf(t, p0, p1); }
     return x;
 }
 
@@ -110,13 +111,13 @@ __global__ __launch_bounds__(256) void ew_kernel(const ew_args a) {
         if constexpr (ew_has_src1<OP>()) y = *(const float4_t *) (p1 + i0 * 4);
         float4_t r;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) r[k] = ew_apply<OP>(a, x[k], y[k]);
+        for (int k = 0; k < 4; ++k) r[k] = ew_apply<OP>(a.p0, a.p1, a.aux, x[k], y[k]);
         *(float4_t *) (pd + i0 * 4) = r;
     } else {
         const float x = *(const float *) (p0 + i0 * a.nb0[0]);
         float y = yb;
         if constexpr (ew_has_src1<OP>()) y = *(const float *) (p1 + (i0 % a.ne1[0]) * a.nb1[0]);
-        *(float *) (pd + i0 * a.nbd[0]) = ew_apply<OP>(a, x, y);
+        *(float *) (pd + i0 * a.nbd[0]) = ew_apply<OP>(a.p0, a.p1, a.aux, x, y);
     }
 }
 
@@ -253,12 +254,16 @@ __global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
 // The ops the reference's graphs use around the decoder stacks: the causal and CFG-pair masks are
 // built from ARANGE + REPEAT (src/minicpm.cpp:602-620, src/locdit.cpp:283-305), token embeddings are
 // a GET_ROWS (src/components.cpp:223).  With them a whole forward graph stays on the device.
-__global__ __launch_bounds__(256) void arange_kernel(float * d, int64_t n, float start, float step) {
+__device__ __forceinline__ float arange_value(float start, float step, int64_t i) {
 #pragma clang fp contract(off)
+    const float t = step * (float) i; // product rounded, then the sum: ops.cpp:7899
+    return start + t;
+}
+
+__global__ __launch_bounds__(256) void arange_kernel(float * d, int64_t n, float start, float step) {
     const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    const float t = step * (float) i; // product rounded, then the sum: ops.cpp:7899
-    d[i] = start + t;
+    d[i] = arange_value(start, step, i);
 }
 
 struct rep_args {
@@ -336,17 +341,12 @@ __device__ __forceinline__ double block_total(double acc, double * part /* 16 do
     return t;
 }
 
+// one lane's share of a sum: units first, first + step, ... (< n) added in that order in fp64
 template <bool VEC>
-__global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst, double * partials) {
-    __shared__ double part[16];
+__device__ __forceinline__ double sum_lane(const char * src, const vx_dims & s, uint32_t first, uint32_t step, uint32_t n) {
     constexpr int W = VEC ? 4 : 1;
     const uint32_t per_row = (uint32_t) (s.ne[0] / W);
-    const uint32_t n = per_row * (uint32_t) (s.ne[1] * s.ne[2] * s.ne[3]); // < 2^24, checked by the caller
     const uint32_t ne1 = (uint32_t) s.ne[1], ne2 = (uint32_t) s.ne[2];
-    const bool one_wave = n <= VX_SUM_ONE_WAVE_UNITS && gridDim.x == 1; // uniform
-    if (one_wave && threadIdx.x >= 64) return;
-    const uint32_t first = one_wave ? threadIdx.x : blockIdx.x * blockDim.x + threadIdx.x;
-    const uint32_t step  = one_wave ? 64 : gridDim.x * blockDim.x;
     double acc = 0.0;
     for (uint32_t e = first; e < n; e += step) {
         const uint32_t row = e / per_row, iv = e - row * per_row;
@@ -359,6 +359,18 @@ __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, 
             acc += (double) *(const float *) p;
         }
     }
+    return acc;
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, float * dst, double * partials) {
+    __shared__ double part[16];
+    const uint32_t n = (uint32_t) (s.ne[0] / (VEC ? 4 : 1)) * (uint32_t) (s.ne[1] * s.ne[2] * s.ne[3]); // < 2^24, checked by the caller
+    const bool one_wave = n <= VX_SUM_ONE_WAVE_UNITS && gridDim.x == 1; // uniform
+    if (one_wave && threadIdx.x >= 64) return;
+    const uint32_t first = one_wave ? threadIdx.x : blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t step  = one_wave ? 64 : gridDim.x * blockDim.x;
+    double acc = sum_lane<VEC>(src, s, first, step, n);
     if (one_wave) {
         acc = vx_wave_sum(acc);
         if (threadIdx.x == 0) *dst = (float) acc;
@@ -376,6 +388,265 @@ __global__ __launch_bounds__(64) void sum_partials_kernel(const double * partial
         double t = 0.0;
         for (int i = 0; i < n; ++i) t += partials[i];
         *dst = (float) t;
+    }
+}
+
+// ---- a run of tiny nodes as one launch --------------------------------------------------------------
+// Around the decoder stacks the reference's graphs hold chains of operators on a few hundred values (bias
+// adds, the CONCATs that assemble LocDiT's 14-token sequence, the guidance arithmetic and the Euler update of
+// UnifiedCFM, src/unified_cfm.cpp:30-149): a dependent launch each, microseconds for nothing.  One work-group
+// of 1024 threads runs such a run node after node.  Every node writes its result to its own memory as its
+// separate kernel would, with that kernel's arithmetic (the same device functions, sums in the same order), and
+// also into a slot of LDS while there is room: a later node of the run whose operand is exactly that tensor reads
+// the slot, so the common chain costs an LDS round trip per node instead of a trip through L2.  An operand that
+// merely overlaps something written earlier in the run (a view of it) is read from memory after a full barrier.
+constexpr int SG_MAX_NODES = 16;
+constexpr int SG_MAX_ELEMS = 16384;
+constexpr int SG_LDS_ELEMS = 12288; // 48 KiB of 4-byte slots (an F16 value sits in the low half of its slot)
+
+enum sg_kind : int { SG_EW2 = 0, SG_ADD1, SG_SCALE, SG_UNARY, SG_CPY, SG_CONCAT, SG_REPEAT, SG_SUM, SG_ARANGE };
+
+struct sg_tensor {
+    char *  p;
+    int32_t ne[4];
+    int64_t nb[4];
+    int32_t type;
+    int32_t lds;         // first LDS slot of this tensor's row-major image, or -1
+};
+struct sg_node {
+    int32_t kind, aux;   // aux: binary / unary code, CONCAT dim, SUM's 16-byte-unit flag
+    float   p0, p1;
+    int32_t wait_memory; // an operand (or the destination) overlaps memory written earlier in the run without being that tensor
+    int32_t flat;        // 1: element e of the destination takes element e (or the only element) of every operand, all of
+                         // them dense or imaged in LDS -- no index arithmetic; 2: a CONCAT of such tensors along their outermost dim
+    int32_t one0, one1;  // with flat: operand 0 / 1 is a single element
+    sg_tensor s0, s1, d;
+};
+struct sg_args {
+    int32_t n, pad;
+    sg_node node[SG_MAX_NODES];
+};
+
+__device__ __forceinline__ void sg_index(const sg_tensor & t, uint32_t e, uint32_t (&i)[4]) {
+    i[0] = e % (uint32_t) t.ne[0]; e /= (uint32_t) t.ne[0];
+    i[1] = e % (uint32_t) t.ne[1]; e /= (uint32_t) t.ne[1];
+    i[2] = e % (uint32_t) t.ne[2]; i[3] = e / (uint32_t) t.ne[2];
+}
+__device__ __forceinline__ uint32_t sg_count(const sg_tensor & t) { return (uint32_t) (t.ne[0] * t.ne[1] * t.ne[2] * t.ne[3]); }
+
+// the bits of element i of t (i taken modulo t's shape when REP: ggml's repeat rule), from its LDS image or from memory
+template <bool REP>
+__device__ __forceinline__ uint32_t sg_get(const sg_tensor & t, const uint32_t (&i)[4], const uint32_t * lds) {
+    uint32_t j[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) j[q] = REP ? i[q] % (uint32_t) t.ne[q] : i[q];
+    if (t.lds >= 0) return lds[(uint32_t) t.lds + ((j[3] * (uint32_t) t.ne[2] + j[2]) * (uint32_t) t.ne[1] + j[1]) * (uint32_t) t.ne[0] + j[0]];
+    const char * p = t.p + j[0] * t.nb[0] + j[1] * t.nb[1] + j[2] * t.nb[2] + j[3] * t.nb[3];
+    return t.type == VX_TYPE_F16 ? (uint32_t) *(const uint16_t *) p : *(const uint32_t *) p;
+}
+// element e (row-major) = index i of the destination: to memory, and to the LDS image when it has one
+__device__ __forceinline__ void sg_put(const sg_tensor & t, uint32_t e, const uint32_t (&i)[4], uint32_t bits, uint32_t * lds) {
+    char * p = t.p + i[0] * t.nb[0] + i[1] * t.nb[1] + i[2] * t.nb[2] + i[3] * t.nb[3];
+    if (t.type == VX_TYPE_F16) *(uint16_t *) p = (uint16_t) bits;
+    else                       *(uint32_t *) p = bits;
+    if (t.lds >= 0) lds[(uint32_t) t.lds + e] = bits;
+}
+// the same for the flat case: element e in row-major order of a dense tensor (or its LDS image)
+__device__ __forceinline__ uint32_t sg_get_flat(const sg_tensor & t, uint32_t e, const uint32_t * lds) {
+    if (t.lds >= 0) return lds[(uint32_t) t.lds + e];
+    return t.type == VX_TYPE_F16 ? (uint32_t) ((const uint16_t *) t.p)[e] : ((const uint32_t *) t.p)[e];
+}
+__device__ __forceinline__ void sg_put_flat(const sg_tensor & t, uint32_t e, uint32_t bits, uint32_t * lds) {
+    if (t.type == VX_TYPE_F16) ((uint16_t *) t.p)[e] = (uint16_t) bits;
+    else                       ((uint32_t *) t.p)[e] = bits;
+    if (t.lds >= 0) lds[(uint32_t) t.lds + e] = bits;
+}
+__device__ __forceinline__ float    sg_f(uint32_t b) { return __builtin_bit_cast(float, b); }
+__device__ __forceinline__ uint32_t sg_b(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+template <typename TS, typename TD>
+__device__ __forceinline__ uint32_t sg_convert(uint32_t bits) {
+    TS x;
+    if constexpr (sizeof(TS) == 2) x = __builtin_bit_cast(TS, (uint16_t) bits); else x = __builtin_bit_cast(TS, bits);
+    const TD y = cpy_convert<TS, TD>(x);
+    if constexpr (sizeof(TD) == 2) return (uint32_t) __builtin_bit_cast(uint16_t, y); else return __builtin_bit_cast(uint32_t, y);
+}
+
+// one lane's share of a sum over an LDS image: the units of sum_lane (4 consecutive elements, or 1), same order
+template <bool VEC>
+__device__ __forceinline__ double sum_lane_lds(const uint32_t * img, uint32_t first, uint32_t step, uint32_t n) {
+    constexpr int W = VEC ? 4 : 1;
+    double acc = 0.0;
+    for (uint32_t e = first; e < n; e += step)
+#pragma unroll
+        for (int q = 0; q < W; ++q) acc += (double) sg_f(img[e * W + q]);
+    return acc;
+}
+
+__global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
+    __shared__ double   part[16];
+    __shared__ uint32_t lds[SG_LDS_ELEMS];
+    // The node table is fetched ONCE, by all threads together, into LDS: kernel arguments live in host-visible memory, and
+    // reading a node's fields where they are first needed costs a trip there per cache line and node.
+    __shared__ __attribute__((aligned(16))) uint32_t table[(sizeof(sg_args) + 3) / 4];
+    static_assert(sizeof(sg_args) <= 4 * 1024, "one dword per thread");
+    if (threadIdx.x < (sizeof(sg_args) + 3) / 4) table[threadIdx.x] = ((const uint32_t *) &a0)[threadIdx.x];
+    __syncthreads();
+    const sg_args & a = *(const sg_args *) table;
+    for (int k = 0; k < a.n; ++k) { // uniform: every thread walks every node and meets every barrier
+        const sg_node & nd = a.node[k];
+        if (k > 0) {
+            if (nd.wait_memory) {
+                __syncthreads(); // earlier nodes' stores to memory are complete and visible to the work-group
+            } else {             // only the LDS images carry values between the nodes: no wait for stores in flight
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            }
+        }
+        const uint32_t n = sg_count(nd.d);
+        if (nd.flat == 1) { // dense operands of the destination's shape (or single elements): no index arithmetic
+            for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                uint32_t r;
+                if (nd.kind == SG_ARANGE) {
+                    r = sg_b(arange_value(nd.p0, nd.p1, (int64_t) e));
+                } else {
+                    const uint32_t xb = sg_get_flat(nd.s0, nd.one0 ? 0 : e, lds);
+                    const float x = sg_f(xb);
+                    switch (nd.kind) {
+                        case SG_EW2: {
+                            const float y = sg_f(sg_get_flat(nd.s1, nd.one1 ? 0 : e, lds));
+                            switch (nd.aux) {
+                                case VX_BIN_ADD: r = sg_b(ew_apply<EW_ADD>(0, 0, 0, x, y)); break;
+                                case VX_BIN_SUB: r = sg_b(ew_apply<EW_SUB>(0, 0, 0, x, y)); break;
+                                case VX_BIN_MUL: r = sg_b(ew_apply<EW_MUL>(0, 0, 0, x, y)); break;
+                                default:         r = sg_b(ew_apply<EW_DIV>(0, 0, 0, x, y)); break;
+                            }
+                        } break;
+                        case SG_ADD1:  r = sg_b(ew_apply<EW_ADD1>(0, 0, 0, x, sg_f(sg_get_flat(nd.s1, 0, lds)))); break;
+                        case SG_SCALE: r = sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, x, 0.0f)); break;
+                        case SG_UNARY: r = sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, x, 0.0f)); break;
+                        default: // SG_CPY between dense tensors (element e to element e), SG_REPEAT of one value
+                            if (nd.s0.type == VX_TYPE_I32)      r = nd.d.type == VX_TYPE_I32 ? xb : sg_convert<int32_t, float>(xb);
+                            else if (nd.d.type == VX_TYPE_I32)  r = sg_convert<float, int32_t>(xb);
+                            else if (nd.s0.type == VX_TYPE_F32) r = nd.d.type == VX_TYPE_F32 ? xb : sg_convert<float, _Float16>(xb);
+                            else                                r = nd.d.type == VX_TYPE_F32 ? sg_convert<_Float16, float>(xb) : xb;
+                            break;
+                    }
+                }
+                sg_put_flat(nd.d, e, r, lds);
+            }
+            continue;
+        }
+        if (nd.flat == 2) { // CONCAT along the outermost dim: the first operand's elements, then the second's
+            const uint32_t n0 = sg_count(nd.s0);
+            for (uint32_t e = threadIdx.x; e < n; e += 1024)
+                sg_put_flat(nd.d, e, e < n0 ? sg_get_flat(nd.s0, e, lds) : sg_get_flat(nd.s1, e - n0, lds), lds);
+            continue;
+        }
+        switch (nd.kind) {
+            case SG_EW2:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    const float x = sg_f(sg_get<false>(nd.s0, i, lds)), y = sg_f(sg_get<true>(nd.s1, i, lds));
+                    float r;
+                    switch (nd.aux) {
+                        case VX_BIN_ADD: r = ew_apply<EW_ADD>(0, 0, 0, x, y); break;
+                        case VX_BIN_SUB: r = ew_apply<EW_SUB>(0, 0, 0, x, y); break;
+                        case VX_BIN_MUL: r = ew_apply<EW_MUL>(0, 0, 0, x, y); break;
+                        default:         r = ew_apply<EW_DIV>(0, 0, 0, x, y); break;
+                    }
+                    sg_put(nd.d, e, i, sg_b(r), lds);
+                }
+                break;
+            case SG_ADD1: {
+                const uint32_t zero[4] = { 0, 0, 0, 0 };
+                const float y = sg_f(sg_get<false>(nd.s1, zero, lds));
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_ADD1>(0, 0, 0, sg_f(sg_get<false>(nd.s0, i, lds)), y)), lds);
+                }
+            } break;
+            case SG_SCALE:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, sg_f(sg_get<false>(nd.s0, i, lds)), 0.0f)), lds);
+                }
+                break;
+            case SG_UNARY:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, sg_f(sg_get<false>(nd.s0, i, lds)), 0.0f)), lds);
+                }
+                break;
+            case SG_CPY: // element e of the source shape -> element e of the destination shape
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t is[4], id[4];
+                    sg_index(nd.s0, e, is);
+                    sg_index(nd.d, e, id);
+                    const uint32_t x = sg_get<false>(nd.s0, is, lds);
+                    uint32_t y;
+                    if (nd.s0.type == VX_TYPE_I32)      y = nd.d.type == VX_TYPE_I32 ? x : sg_convert<int32_t, float>(x);
+                    else if (nd.d.type == VX_TYPE_I32)  y = sg_convert<float, int32_t>(x);
+                    else if (nd.s0.type == VX_TYPE_F32) y = nd.d.type == VX_TYPE_F32 ? x : sg_convert<float, _Float16>(x);
+                    else                                y = nd.d.type == VX_TYPE_F32 ? sg_convert<_Float16, float>(x) : x;
+                    sg_put(nd.d, e, id, y, lds);
+                }
+                break;
+            case SG_CONCAT:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4], j[4];
+                    sg_index(nd.d, e, i);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) j[q] = i[q];
+                    uint32_t off = 0;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) if (q == nd.aux) off = (uint32_t) nd.s0.ne[q];
+                    bool second = false;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) if (q == nd.aux && i[q] >= off) { j[q] = i[q] - off; second = true; }
+                    sg_put(nd.d, e, i, second ? sg_get<false>(nd.s1, j, lds) : sg_get<false>(nd.s0, j, lds), lds);
+                }
+                break;
+            case SG_REPEAT:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    sg_put(nd.d, e, i, sg_get<true>(nd.s0, i, lds), lds);
+                }
+                break;
+            case SG_SUM: { // vx_sum's two single-block orders: one wave up to VX_SUM_ONE_WAVE_UNITS units, the block beyond
+                vx_dims s;
+                for (int q = 0; q < 4; ++q) { s.ne[q] = nd.s0.ne[q]; s.nb[q] = (uint64_t) nd.s0.nb[q]; }
+                const uint32_t units = sg_count(nd.s0) / (nd.aux ? 4 : 1);
+                const bool one_wave = units <= VX_SUM_ONE_WAVE_UNITS;
+                const uint32_t step = one_wave ? 64 : 1024;
+                double acc = 0.0;
+                if (!one_wave || threadIdx.x < 64) {
+                    if (nd.s0.lds >= 0) acc = nd.aux ? sum_lane_lds<true>(lds + nd.s0.lds, threadIdx.x, step, units) : sum_lane_lds<false>(lds + nd.s0.lds, threadIdx.x, step, units);
+                    else                acc = nd.aux ? sum_lane<true>(nd.s0.p, s, threadIdx.x, step, units) : sum_lane<false>(nd.s0.p, s, threadIdx.x, step, units);
+                }
+                double t;
+                if (one_wave) t = threadIdx.x < 64 ? vx_wave_sum(acc) : 0.0;
+                else          t = block_total(acc, part);
+                if (threadIdx.x == 0) {
+                    const uint32_t zero[4] = { 0, 0, 0, 0 };
+                    sg_put(nd.d, 0, zero, sg_b((float) t), lds);
+                }
+            } break;
+            case SG_ARANGE:
+                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                    uint32_t i[4];
+                    sg_index(nd.d, e, i);
+                    sg_put(nd.d, e, i, sg_b(arange_value(nd.p0, nd.p1, (int64_t) e)), lds);
+                }
+                break;
+            default: break;
+        }
     }
 }
 
@@ -725,6 +996,145 @@ extern "C" vx_status vx_get_rows(const vx_tensor * table, const vx_tensor * rows
     if (table->type == VX_TYPE_F16)       get_rows_kernel<1><<<grid, block, 0, st>>>(a);
     else if (table->type == VX_TYPE_Q8_0) get_rows_kernel<2><<<grid, block, 0, st>>>(a);
     else                                  get_rows_kernel<0><<<grid, block, 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// ---- vx_small_graph -------------------------------------------------------------------------------
+static bool sg_fits(const vx_tensor * t) {
+    if (!t || !vx_positive(t) || vx_nelements(t) > SG_MAX_ELEMS) return false;
+    for (int i = 0; i < 4; ++i) if (t->nb[i] > ((uint64_t) 1 << 40)) return false;
+    return true;
+}
+
+extern "C" int vx_supports_small_node(const vx_small_node * nd) {
+    if (!nd || !nd->dst || !sg_fits(nd->dst)) return 0;
+    const vx_tensor * a = nd->src0, * b = nd->src1, * d = nd->dst;
+    switch (nd->op) {
+        case VX_NODE_ADD: case VX_NODE_SUB: case VX_NODE_MUL: case VX_NODE_DIV:
+            return sg_fits(a) && sg_fits(b) && vx_supports_binary(nd->op - VX_NODE_ADD, a, b, d);
+        case VX_NODE_ADD1:   return sg_fits(a) && b && vx_supports_add1(a, b, d);
+        case VX_NODE_SCALE:  return sg_fits(a) && vx_supports_unary_like(a, d);
+        case VX_NODE_UNARY:  return sg_fits(a) && vx_supports_unary(nd->aux, a, d);
+        case VX_NODE_CPY:    return sg_fits(a) && vx_supports_cpy(a, d);
+        case VX_NODE_CONCAT: return sg_fits(a) && sg_fits(b) && vx_supports_concat(a, b, d, nd->aux);
+        case VX_NODE_REPEAT: return sg_fits(a) && vx_supports_repeat(a, d);
+        case VX_NODE_SUM:    return sg_fits(a) && vx_supports_sum(a, d);
+        case VX_NODE_ARANGE: return vx_supports_arange(d);
+        default:             return 0;
+    }
+}
+
+static sg_tensor sg_desc(const vx_tensor * t) {
+    sg_tensor r = {};
+    r.lds = -1;
+    if (!t) return r;
+    r.p = (char *) t->data; r.type = t->type;
+    for (int i = 0; i < 4; ++i) { r.ne[i] = (int32_t) t->ne[i]; r.nb[i] = (int64_t) t->nb[i]; }
+    return r;
+}
+
+namespace {
+// what the host remembers of the run so far: which tensors have an LDS image, and which bytes were written
+struct sg_span { uintptr_t lo, hi; };
+sg_span sg_span_of(const vx_tensor * t) {
+    uintptr_t hi = (uintptr_t) t->data + vx_type_size(t->type);
+    for (int i = 0; i < 4; ++i) hi += (uintptr_t) (t->ne[i] - 1) * t->nb[i];
+    return { (uintptr_t) t->data, hi };
+}
+bool sg_same(const vx_tensor * a, const vx_tensor * b) {
+    if (a->data != b->data || a->type != b->type) return false;
+    for (int i = 0; i < 4; ++i) if (a->ne[i] != b->ne[i] || a->nb[i] != b->nb[i]) return false;
+    return true;
+}
+struct sg_image { vx_tensor t; int32_t off; bool valid; };
+} // namespace
+
+extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx_stream stream) {
+    if (!nodes || n_nodes < 1 || n_nodes > SG_MAX_NODES) return vx_fail(VX_ERR_UNSUPPORTED, "small graph: 1 to %d nodes", SG_MAX_NODES);
+    sg_args a = {};
+    a.n = n_nodes;
+    sg_image images[SG_MAX_NODES];
+    sg_span  written[SG_MAX_NODES];
+    vx_tensor written_t[SG_MAX_NODES];
+    int n_images = 0, n_written = 0;
+    int32_t lds_used = 0;
+    for (int k = 0; k < n_nodes; ++k) {
+        const vx_small_node & nd = nodes[k];
+        if (!vx_supports_small_node(&nd)) return vx_fail(VX_ERR_UNSUPPORTED, "small graph: node %d (op %d) is not a small elementwise / copy / sum node", k, nd.op);
+        if (!nd.dst->data || (nd.src0 && !nd.src0->data) || (nd.src1 && !nd.src1->data)) return vx_fail(VX_ERR_INVALID, "small graph: null data in node %d", k);
+        sg_node & g = a.node[k];
+        g.s0 = sg_desc(nd.op == VX_NODE_ARANGE ? nullptr : nd.src0); g.s1 = sg_desc(nd.src1); g.d = sg_desc(nd.dst);
+        g.p0 = nd.p0; g.p1 = nd.p1; g.aux = nd.aux;
+        switch (nd.op) {
+            case VX_NODE_ADD: case VX_NODE_SUB: case VX_NODE_MUL: case VX_NODE_DIV: g.kind = SG_EW2; g.aux = nd.op - VX_NODE_ADD; break;
+            case VX_NODE_ADD1:   g.kind = SG_ADD1; break;
+            case VX_NODE_SCALE:  g.kind = SG_SCALE; break;
+            case VX_NODE_UNARY:  g.kind = SG_UNARY; break;
+            case VX_NODE_CPY:    g.kind = SG_CPY; break;
+            case VX_NODE_CONCAT: g.kind = SG_CONCAT; break;
+            case VX_NODE_REPEAT: g.kind = SG_REPEAT; break;
+            case VX_NODE_SUM:    g.kind = SG_SUM; g.aux = nd.src0->ne[0] % 4 == 0 && al16(nd.src0->data, nd.src0->nb); break; // vx_sum's unit rule
+            default:             g.kind = SG_ARANGE; break;
+        }
+        // operands: the LDS image of exactly this tensor, else memory -- after a full barrier if the run wrote there
+        const vx_tensor * ops[2] = { nd.op == VX_NODE_ARANGE ? nullptr : nd.src0, nd.src1 };
+        sg_tensor * gops[2] = { &g.s0, &g.s1 };
+        for (int o = 0; o < 2; ++o) {
+            if (!ops[o]) continue;
+            for (int m = 0; m < n_images; ++m)
+                if (images[m].valid && sg_same(&images[m].t, ops[o])) gops[o]->lds = images[m].off;
+            if (gops[o]->lds >= 0) continue;
+            const sg_span sp = sg_span_of(ops[o]);
+            for (int m = 0; m < n_written; ++m) if (sp.lo < written[m].hi && written[m].lo < sp.hi) g.wait_memory = 1;
+        }
+        // destination: keeps its image when it is rewritten as the same tensor; any other overlap retires the image
+        // and orders the stores through memory
+        const sg_span dsp = sg_span_of(nd.dst);
+        int mine = -1;
+        for (int m = 0; m < n_images; ++m) {
+            if (!images[m].valid) continue;
+            if (sg_same(&images[m].t, nd.dst)) { mine = m; continue; }
+            const sg_span sp = sg_span_of(&images[m].t);
+            if (dsp.lo < sp.hi && sp.lo < dsp.hi) images[m].valid = false;
+        }
+        for (int m = 0; m < n_written; ++m)
+            if (dsp.lo < written[m].hi && written[m].lo < dsp.hi && !sg_same(&written_t[m], nd.dst)) g.wait_memory = 1;
+        const int32_t cnt = (int32_t) vx_nelements(nd.dst);
+        if (mine >= 0) {
+            g.d.lds = images[mine].off;
+        } else if (lds_used + cnt <= SG_LDS_ELEMS) {
+            images[n_images] = { *nd.dst, lds_used, true };
+            g.d.lds = lds_used;
+            lds_used += cnt;
+            ++n_images;
+        }
+        written[n_written] = dsp; written_t[n_written] = *nd.dst; ++n_written;
+        // the flat forms: dense row-major tensors (or LDS images) indexed by the destination's element number
+        if (vx_is_contiguous(nd.dst)) {
+            auto flat_operand = [&](const vx_tensor * t, const sg_tensor & gt, int32_t * one) {
+                *one = 0;
+                if (vx_nelements(t) == 1) { *one = 1; return true; }
+                return vx_same_shape(t, nd.dst) && (gt.lds >= 0 || vx_is_contiguous(t));
+            };
+            const bool f0 = ops[0] ? flat_operand(ops[0], g.s0, &g.one0) : true;
+            const bool f1 = ops[1] ? flat_operand(ops[1], g.s1, &g.one1) : true;
+            switch (g.kind) {
+                case SG_EW2: case SG_SCALE: case SG_UNARY: if (f0 && f1) g.flat = 1; break;
+                case SG_ADD1:   if (f0) g.flat = 1; break;
+                case SG_REPEAT: if (g.one0) g.flat = 1; break; // one value over the whole destination
+                case SG_ARANGE: g.flat = 1; break;
+                case SG_CPY:    if (g.s0.lds >= 0 || vx_is_contiguous(ops[0])) g.flat = 1; break; // element e -> element e whatever the shapes
+                case SG_CONCAT: {
+                    bool outer = true;
+                    for (int q = nd.aux + 1; q < 4; ++q) outer = outer && nd.dst->ne[q] == 1;
+                    if (outer && (g.s0.lds >= 0 || vx_is_contiguous(ops[0])) && (g.s1.lds >= 0 || vx_is_contiguous(ops[1]))) g.flat = 2;
+                } break;
+                default: break;
+            }
+        }
+    }
+    small_graph_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -1019,7 +1019,9 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
 extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst) {
     if (!vx_supports_mul_mat(src0, src1, dst) || !residual) return 0;
     if (src0->type != VX_TYPE_Q8_0 && src0->type != VX_TYPE_F16) return 0;
-    if (residual->type != VX_TYPE_F32 || !vx_same_shape(residual, dst) || residual->nb[0] != 4) return 0;
+    if (residual->type != VX_TYPE_F32 || residual->ne[0] != dst->ne[0] || residual->nb[0] != 4) return 0;
+    // dst's shape, or one row / one matrix repeated over it (a bias: ggml_add repeats src1)
+    for (int i = 1; i < 4; ++i) if (residual->ne[i] != dst->ne[i] && residual->ne[i] != 1) return 0;
     if (residual->nb[1] % 4 || residual->nb[2] % 4 || residual->nb[3] % 4) return 0;
     return gemv_shape_ok(src1->ne[1], src0->ne[1], src0->ne[0]);
 }
@@ -1043,7 +1045,10 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     a.r2 = (int) (src1->ne[2] / src0->ne[2]); a.r3 = (int) (src1->ne[3] / src0->ne[3]);
     a.rows_wg   = 16;
     a.res       = (const char *) residual->data;
-    a.rnb1 = residual->nb[1]; a.rnb2 = residual->nb[2]; a.rnb3 = residual->nb[3];
+    // a repeated dim of the residual (a bias row) is walked with stride 0
+    a.rnb1 = residual->ne[1] == dst->ne[1] ? residual->nb[1] : 0;
+    a.rnb2 = residual->ne[2] == dst->ne[2] ? residual->nb[2] : 0;
+    a.rnb3 = residual->ne[3] == dst->ne[3] ? residual->nb[3] : 0;
     a.res_scale = scale;
     a.w_aligned = ((uintptr_t) src0->data % 4 == 0) && src0->nb[1] % 4 == 0 && src0->nb[2] % 4 == 0 && src0->nb[3] % 4 == 0;
     a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;

@@ -632,6 +632,76 @@ int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, cons
     return idx;
 }
 
+// A graph node as a node of vx_small_graph (tiny elementwise / copy / concat / repeat / sum / arange work); t holds the
+// descriptors the node points to.  False for every other operator and for tensors above the small-graph size.
+bool small_node_of(const ggml_tensor * n, vx_small_node * out, vx_tensor (&t)[3]) {
+    *out = vx_small_node{};
+    t[2] = to_vx(n);
+    out->dst = &t[2];
+    if (n->src[0]) { t[0] = to_vx(n->src[0]); out->src0 = &t[0]; }
+    bool two = false;
+    switch (n->op) {
+        case GGML_OP_ADD: case GGML_OP_SUB: case GGML_OP_MUL: case GGML_OP_DIV:
+            out->op = VX_NODE_ADD + binary_code(n->op); two = true; break;
+        case GGML_OP_ADD1:   out->op = VX_NODE_ADD1; two = true; break;
+        case GGML_OP_SCALE:
+            out->op = VX_NODE_SCALE;
+            memcpy(&out->p0, (const float *) n->op_params + 0, sizeof(float));
+            memcpy(&out->p1, (const float *) n->op_params + 1, sizeof(float));
+            break;
+        case GGML_OP_UNARY:  out->op = VX_NODE_UNARY; out->aux = (int) ggml_get_unary_op(n); break;
+        case GGML_OP_SQR: case GGML_OP_SQRT: case GGML_OP_LOG: case GGML_OP_SIN: case GGML_OP_COS:
+            out->op = VX_NODE_UNARY; out->aux = standalone_unary_code(n->op); break;
+        case GGML_OP_DUP: case GGML_OP_CPY: case GGML_OP_CONT: out->op = VX_NODE_CPY; break;
+        case GGML_OP_CONCAT: out->op = VX_NODE_CONCAT; out->aux = ((const int32_t *) n->op_params)[0]; two = true; break;
+        case GGML_OP_REPEAT: out->op = VX_NODE_REPEAT; break;
+        case GGML_OP_SUM:    out->op = VX_NODE_SUM; break;
+        case GGML_OP_ARANGE:
+            out->op = VX_NODE_ARANGE;
+            memcpy(&out->p0, (const float *) n->op_params + 0, sizeof(float));
+            memcpy(&out->p1, (const float *) n->op_params + 2, sizeof(float));
+            out->src0 = nullptr;
+            break;
+        default: return false;
+    }
+    if (n->op != GGML_OP_ARANGE && !n->src[0]) return false;
+    if (two) {
+        if (!n->src[1]) return false;
+        t[1] = to_vx(n->src[1]);
+        out->src1 = &t[1];
+    }
+    return vx_supports_small_node(out) != 0;
+}
+
+// The run of tiny nodes that starts at node i (at most 16, view nodes in between skipped) as ONE launch: the bias adds,
+// sequence-assembling CONCATs, guidance arithmetic and Euler update around the LocDiT estimator (src/locdit.cpp:401-464,
+// src/unified_cfm.cpp:30-149).  Every node still writes its own tensor, in graph order, so no reader analysis is needed.
+// The run stops in front of anything another group claims.  Returns the index of the run's last node, or -1 when fewer
+// than two nodes qualify.
+int compute_small_run(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers,
+                      const std::unordered_map<const ggml_tensor *, const ggml_tensor *> & absorbed,
+                      const std::unordered_set<const ggml_tensor *> & done, vx_status * rc) {
+    constexpr int MAX_RUN = 16;
+    vx_small_node nodes[MAX_RUN];
+    vx_tensor     ts[MAX_RUN][3];
+    int count = 0, last = -1;
+    for (int j = i; j < g->n_nodes && count < MAX_RUN; ++j) {
+        const ggml_tensor * n = g->nodes[j];
+        if (ggml_op_is_empty(n->op) || ggml_is_empty(n)) continue;
+        if ((n->flags & GGML_TENSOR_FLAG_COMPUTE) == 0 || absorbed.count(n) || done.count(n)) break;
+        if (n->op == GGML_OP_CPY) { // the cache-write group has its own launch
+            ggml_tensor * tmp[9];
+            if (match_kv_store_group(g, j, readers, tmp) >= 0) break;
+        }
+        if (!small_node_of(n, &nodes[count], ts[count])) break;
+        ++count;
+        last = j;
+    }
+    if (count < 2) return -1;
+    *rc = vx_small_graph(nodes, count, ctx->stream);
+    return last;
+}
+
 // layer_forward's residual updates (src/minicpm.cpp:762-777) at decode size:
 //   MUL_MAT(w, x) [SCALE] ADD(residual, .)   -> one launch.  Returns the index of the ADD, or -1.
 int compute_mul_mat_residual_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
@@ -1087,6 +1157,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
             int last = -1;
             if (node->op == GGML_OP_CPY) last = compute_kv_store_group(ctx, cgraph, i, readers, &rc);
             else if (node->op == GGML_OP_MUL_MAT) last = compute_mul_mat_residual_group(ctx, cgraph, i, readers, &rc);
+            if (last < 0) last = compute_small_run(ctx, cgraph, i, readers, kv2_absorbed, done, &rc);
             if (last >= 0) {
                 fused = true;
                 i = last - 1; // the common increment below steps onto the group's last node
