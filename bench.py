@@ -325,6 +325,57 @@ def locdit_stack_bench(pkg, timer, side, threads, with_cpu, requests=8, branch=7
     return res
 
 
+def cfm_solve_bench(pkg, timer, side, threads, with_cpu, layers=4, patch=2, prefix=4, timesteps=10):
+    """BASELINE config 3 as one whole UnifiedCFM solve of one request (src/unified_cfm.cpp:88-149): per Euler step the
+    input projection, the assembly of the 14-token CFG-pair sequence, the 4-layer decoder pass, the output projections
+    and the zero-star guidance arithmetic with the update of x -- every launch of the solve, replayed from one HIP graph.
+    ggml-cpu runs the same solve as the one graph the reference builds."""
+    import torch
+    import reflib
+    bbmod = __import__("voxcpm_cpp_amd.backbone", fromlist=["MiniCPMBackbone"])
+    cfmmod = __import__("voxcpm_cpp_amd.cfm", fromlist=["LocDiTCfmSolver"])
+    params = reflib.backbone_params("bench-locdit", 1)
+    lw = params["layers"][0]
+    cp = reflib.cfm_params("bench-cfm")
+    T = 2 * (1 + prefix + patch)
+    dec = bbmod.MiniCPMBackbone(n_layer=layers, max_length=T, batch=1, use_mup=False, kv_f16=False)
+    for li in range(layers):
+        for n in reflib.BB_WEIGHTS:
+            dec.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+        for n in ("input_layernorm", "post_layernorm"):
+            dec.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+    dec.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+    dec.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+    q8 = lambda w, b: (torch.from_numpy(reflib.quantize_q8_0(w)).cuda(), w.shape[1], torch.from_numpy(b).cuda())
+    solver = cfmmod.LocDiTCfmSolver(dec, 64, q8(cp["in_w"], cp["in_b"]), q8(cp["cond_w"], cp["cond_b"]), q8(cp["out_w"], cp["out_b"]))
+    rs = np.random.default_rng(11)
+    z, mu = rs.standard_normal((patch, 64)).astype(np.float32), rs.standard_normal(1024).astype(np.float32)
+    cond, table = rs.standard_normal((prefix, 64)).astype(np.float32), rs.standard_normal((timesteps, 1024)).astype(np.float32)
+    t_span = np.zeros(timesteps + 1, np.float32)
+    reflib.load_oracle().orc_t_span(timesteps, 1.0, reflib.ptr(t_span, C.c_float))
+    run, _ = solver.plan(*(torch.from_numpy(a).cuda() for a in (z, mu, cond, table)), t_span, cfg_value=2.0)
+    s = timer.run(graphed(run, side), iters=30, warmup=3)
+    res = {"us_per_cfm_solve": s * 1e6, "launches_per_solve": run.n_calls, "launches_per_step": run.n_calls / (timesteps - 1),
+           "shape": f"one request: {timesteps} Euler steps ({timesteps - 1} estimator passes under zero-star), {layers} layers, "
+                    f"CFG pair as one {T}-token sequence, Q8_0 weights"}
+    del solver, dec
+    ref = reflib.load_ref() if with_cpu else None
+    if ref is not None:
+        assert ref.rh_use_device(b"CPU", threads, 0) == 0
+        params["dims"]["n_layer"] = layers
+        params["layers"] = [lw] * layers
+        reflib.ref_backbone_create(params, T, 1, use_mup=False, kv_f16=False, fused_weights=True)
+        reflib.ref_cfm_create(cp)
+        _, (mean, best), n_nodes = reflib.ref_cfm_solve(z, mu, cond, table, n_steps=timesteps, reps=10)
+        ref.rh_cfm_free()
+        ref.rh_bb_free()
+        res["ggml_cpu_us_per_cfm_solve"] = mean * 1e6
+        res["ggml_cpu_threads"] = threads
+        res["ggml_graph_nodes"] = n_nodes
+        res["speedup_vs_ggml_cpu"] = mean / s
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -438,6 +489,7 @@ def main():
     if not args.no_others:
         others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu)
         others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, not args.no_cpu)
+        others["cfg3_cfm_solve_one_request"] = cfm_solve_bench(pkg, timer, side, threads, not args.no_cpu)
         # BASELINE config 5 as a whole stack: 8 streams x CFG pair (batch 16) decoding from KV length 4096 towards 8192
         # (F32 cache as in the reference; the decode steps run over seeded cache contents)
         others["cfg5_backbone_24layers_b16_L4096"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu, batch=16, prefill=4096,

@@ -151,6 +151,17 @@ def test_supports_truth_table_glue(pkg):
                pkg.UNARY_LOG, pkg.UNARY_SIN, pkg.UNARY_COS):
         assert lib.vx_supports_unary(op, a, a) == 1, op
     assert lib.vx_supports_unary(105, a, a) == 0 and lib.vx_supports_unary(17, a, a) == 0
+    # nodes of a one-launch run: the tiny operators, tensors of at most 16384 elements
+    v, sc1 = f32(pkg, [64, 2, 1, 1]), f32(pkg, [1, 1, 1, 1])
+    seq = f32(pkg, [1024, 14, 1, 1])
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_MUL, v, v, v)) == 1
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_SUM, sc1, v)) == 1
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_REPEAT, v, sc1)) == 1
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_ARANGE, sc1)) == 1
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_CONCAT, seq, f32(pkg, [1024, 7, 1, 1]), f32(pkg, [1024, 7, 1, 1]), aux=1)) == 1
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_ADD, a, a, a)) == 0            # 30720 elements: its own launch
+    assert lib.vx_supports_small_node(pkg.small_node(pkg.NODE_UNARY, v, v, aux=8)) == 0      # GELU is not claimed at all
+    assert lib.vx_supports_small_node(pkg.small_node(12, v, v, v)) == 0
     # fused pairs
     w = f32(pkg, [1024, 1, 1, 1])
     assert lib.vx_supports_rms_norm_mul(a, w, a) == 1
@@ -173,6 +184,8 @@ def test_supports_truth_table_node_groups(pkg):
         assert lib.vx_supports_mul_mat_scale_add(wo, acts(n), acts(n), acts(n)) == want, n
     assert lib.vx_supports_mul_mat_scale_add(wdown, acts(14, 4096), acts(14), acts(14)) == 1      # 16 x 4096 halves of LDS
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), acts(3), acts(2)) == 0                  # residual of another shape
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(1), acts(14)) == 1                # a bias row, repeated over the tokens
+    assert lib.vx_supports_mul_mat_scale_add(q8(pkg, [64, K, 1, 1]), acts(2, 64), acts(1), acts(2)) == 1   # LocDiT's in_proj + bias
     assert lib.vx_supports_mul_mat_scale_add(f32(pkg, [K, K, 1, 1]), acts(2), acts(2), acts(2)) == 0   # F32 weights
     # gate / up / SwiGLU: both matrices count as rows
     wg = q8(pkg, [K, 4096, 1, 1])

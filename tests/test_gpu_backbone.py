@@ -347,3 +347,24 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
     assert p.returncode == 0, p.stderr[-2000:]
     bits = [l for l in p.stdout.splitlines() if l.startswith("BITS ")][0][5:]
     assert bytes.fromhex(bits) == plug.tobytes()
+    # the C-ABI mirror of the solve (voxcpm.cpp_amd/cfm.py): the plugin's launches issued by hand, the same bits
+    import torch
+    from voxcpm_cpp_amd import backbone as bb, cfm
+    dec = bb.MiniCPMBackbone(n_layer=4, max_length=32, batch=1, use_mup=True, kv_f16=False)
+    for li, lw in enumerate(params["layers"]):
+        for n in reflib.BB_WEIGHTS:
+            dec.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+        for n in ("input_layernorm", "post_layernorm"):
+            dec.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+    dec.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+    dec.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+    q8 = lambda w, b: (torch.from_numpy(reflib.quantize_q8_0(w)).cuda(), w.shape[1], torch.from_numpy(b).cuda())
+    solver = cfm.LocDiTCfmSolver(dec, 64, q8(cp["in_w"], cp["in_b"]), q8(cp["cond_w"], cp["cond_b"]), q8(cp["out_w"], cp["out_b"]))
+    t_span = np.zeros(11, np.float32)
+    reflib.load_oracle().orc_t_span(10, 1.0, reflib.ptr(t_span, ctypes.c_float))
+    run, x = solver.plan(*(torch.from_numpy(a).cuda() for a in (z, mu, cond, table)), t_span, cfg_value=2.0)
+    run()
+    torch.cuda.synchronize()
+    print(f"   C ABI mirror: {run.n_calls} calls per solve", flush=True)
+    assert launches - 2 <= run.n_calls <= launches, (run.n_calls, launches)   # ggml's node order splits one run of tiny nodes in two
+    assert x.cpu().numpy().tobytes() == plug.tobytes()

@@ -67,10 +67,11 @@ class MiniCPMBackbone:
             t.zero_()
 
     # ---- one (n_tokens, n_past) call list -----------------------------------------------------
-    def plan(self, x, n_tokens, n_past, mask=None, write_kv=True):
+    def plan(self, x, n_tokens, n_past, mask=None, write_kv=True, positions=None):
         """x: (batch, n_tokens, hidden) f32 device tensor, read at replay time.  Returns
         (run, out): run() enqueues the whole stack on torch's current stream; out is the
-        (batch, n_tokens, hidden) result tensor it fills."""
+        (batch, n_tokens, hidden) result tensor it fills.  positions: int32 device tensor of n_tokens rope
+        positions (default n_past .. n_past + n_tokens - 1; LocDiT's CFG pair passes i mod branch length)."""
         torch, L = self.torch, lib()
         B, T, H, Hkv, D = self.batch, n_tokens, self.n_heads, self.n_kv, self.D
         assert x.shape == (B, T, self.hidden) and x.dtype == torch.float32 and x.is_contiguous()
@@ -82,7 +83,8 @@ class MiniCPMBackbone:
         def new(*shape, dtype=f32):
             return torch.empty(shape, dtype=dtype, device=dev)
 
-        pos = torch.arange(n_past, n_past + T, dtype=torch.int32, device=dev)
+        pos = torch.arange(n_past, n_past + T, dtype=torch.int32, device=dev) if positions is None else positions
+        assert pos.dtype == torch.int32 and pos.numel() == T
         seq_len = n_past + T
         attn_factor = 1.0
         if seq_len > self.rope_original_max > 1:  # apply_rope, src/minicpm.cpp:590-594
