@@ -301,6 +301,12 @@ VX_API int vx_supports_unary(int op, const vx_tensor * src, const vx_tensor * ds
 VX_API int vx_supports_glu(int op, const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst);
 VX_API int vx_supports_cpy(const vx_tensor * src, const vx_tensor * dst);
 VX_API int vx_supports_arange(const vx_tensor * dst);
+/* The order in which vx_mul_mat and the groups built on it sum the K blocks of a product with few tokens, as an opaque
+ * number: products with equal K, equal token count of the call and equal number are summed identically.  The number depends
+ * on the row count M, so a backend that replaces one product over a row-fused matrix (the reference's qkv_proj /
+ * gate_up_proj, src/minicpm.cpp:427-492) by products over its row ranges compares the two before it promises the same bits.
+ * No counterpart in the reference. */
+VX_API int vx_mul_mat_sum_order(int64_t K, int64_t tokens, int64_t M);
 
 /* ---- a run of tiny nodes as one launch -------------------------------------------------------------
  * Around the decoder stacks the reference's graphs hold chains of operators over a few hundred values: bias adds,

@@ -55,7 +55,7 @@ EXPORTS = [
     "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
     "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
-    "vx_small_graph", "vx_supports_small_node",
+    "vx_small_graph", "vx_supports_small_node", "vx_mul_mat_sum_order",
     "vx_rms_norm_mul", "vx_scale_add", "vx_add_scale", "vx_flash_attn_ext_add1", "vx_mul_mat_swiglu", "vx_supports_mul_mat_swiglu", "vx_mul_mat_scale_add", "vx_supports_mul_mat_scale_add", "vx_kv_store_sync", "vx_supports_kv_store_sync", "vx_flash_attn_ext_kv2", "vx_supports_flash_attn_ext_kv2", "vx_flash_attn_ext_kv2_store", "vx_supports_flash_attn_ext_kv2_store", "vx_qkv_proj_rope", "vx_supports_qkv_proj_rope", "vx_norm_qkv_proj_rope", "vx_supports_norm_qkv_proj_rope", "vx_norm_mul_mat_swiglu", "vx_supports_norm_mul_mat_swiglu", "vx_supports_rms_norm_mul", "vx_supports_fused_pair",
 ]
 
@@ -131,6 +131,7 @@ def lib():
     l.vx_supports_get_rows.argtypes = [TP, TP, TP]
     l.vx_small_graph.argtypes = [C.POINTER(VxSmallNode), C.c_int, vp]
     l.vx_supports_small_node.argtypes = [C.POINTER(VxSmallNode)]
+    l.vx_mul_mat_sum_order.argtypes = [C.c_int64, C.c_int64, C.c_int64]
     l.vx_rms_norm_mul.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_scale_add.argtypes = [TP, TP, TP, C.c_float, vp]
     l.vx_add_scale.argtypes = [TP, TP, TP, C.c_float, C.c_float, vp]

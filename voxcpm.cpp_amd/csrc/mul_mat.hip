@@ -314,6 +314,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     float *    xd  = (float *) (gv_smem + (size_t) NL * a.K * 2);            // [NL][K/32] (ACT_Q8)
     float4_t * red = (float4_t *) (gv_smem + (size_t) NL * a.K * 2 + (ACT_Q8 ? (size_t) NL * nkb * 4 : 0));
     float *    nsc = (float *) (red + (NW > 1 ? NW - 1 : 0) * 64); // [16] per-token 1 / rms (fused RMS_NORM)
+    float2 *   rcs = (float2 *) (nsc + 16);                          // [4][64] cos / sin exchanged between waves (SEG)
 
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
@@ -438,6 +439,8 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // the row this wave normalises first (token wid), also requested ahead of the weights
     vx_rms_row nrow;
     if (a.norm_w && wid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) wid * a.nb11), a.K, lane);
+    vx_rms_row nrow2; // the wave's second token (more tokens than waves), requested up front as well
+    if (a.norm_w && wid + NW < N) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (wid + NW) * a.nb11), a.K, lane);
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
@@ -449,17 +452,33 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     load_blocks(0);
     // the rotation's cos / sin for this lane's (token, pair) values: computed while the weights fly
     float rc[4] = {1.0f, 1.0f, 1.0f, 1.0f}, rs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (SEG && rope && wid == 0 && row_ok) {
+    // an angle costs a chain of multiplications and two accurate trigonometric evaluations: with four waves or more, wave r
+    // computes token slot r of every lane and the storing wave collects the four through LDS
+    constexpr bool ROPE_SPREAD = SEG && NW >= 4;
+    if (SEG && rope && row_ok && (ROPE_SPREAD ? wid < 4 : wid == 0)) {
         const float ffv = a.ff ? a.ff[pair] : 1.0f;
+        if constexpr (ROPE_SPREAD) {
+            float cv = 1.0f, sv = 0.0f;
+            if (4 * j + wid < N) rope_cos_sin(a.rp, (float) a.pos[(batch * (int) a.N + tok0 + 4 * j + wid) % a.rope_T], pair, ffv, cv, sv);
+            rcs[wid * 64 + lane] = float2{cv, sv};
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * (int) a.N + tok0 + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
+            for (int r = 0; r < 4; ++r)
+                if (4 * j + r < N) rope_cos_sin(a.rp, (float) a.pos[(batch * (int) a.N + tok0 + 4 * j + r) % a.rope_T], pair, ffv, rc[r], rs[r]);
+        }
     }
-    if (a.norm_w) { // one wave per token, as the RMS_NORM kernel has it
-        for (int t = wid; t < N; t += NW) {
+    if (a.norm_w) { // one wave per token, as the RMS_NORM kernel has it; a wave with several tokens takes two at a time
+        for (int t = wid; t < N; t += 2 * NW) {
             if (t != wid) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
-            const float sc = vx_rms_row_scale(nrow, a.K, lane, a.norm_eps);
-            if (lane == 0) nsc[t] = sc;
+            if (t + NW < N) {
+                if (t != wid) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (t + NW) * a.nb11), a.K, lane);
+                float s1, s2;
+                vx_rms_row_scale2(nrow, nrow2, a.K, lane, a.norm_eps, s1, s2);
+                if (lane == 0) { nsc[t] = s1; nsc[t + NW] = s2; }
+            } else {
+                const float sc = vx_rms_row_scale(nrow, a.K, lane, a.norm_eps);
+                if (lane == 0) nsc[t] = sc;
+            }
         }
         __syncthreads();
     }
@@ -470,6 +489,12 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         stage(unit, f0, f1, g0, g1);
     }
     __syncthreads();
+    if constexpr (ROPE_SPREAD) {
+        if (rope && row_ok && wid == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { const float2 v = rcs[r * 64 + lane]; rc[r] = v.x; rs[r] = v.y; }
+        }
+    }
 
     float4_t acc = {0, 0, 0, 0};
     const int64_t per = (nkb + NW - 1) / NW; // blocks per wave
@@ -535,7 +560,8 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     }
 }
 
-constexpr size_t GV_MAX_LDS = 160 * 1024; // what a gfx950 CU has
+constexpr size_t GV_MAX_LDS  = 160 * 1024;    // what a gfx950 CU has
+constexpr size_t GV_ROPE_LDS = 4 * 64 * 8;     // cos / sin of four token slots per lane, exchanged between waves
 
 // Shapes the streaming kernel takes: up to 16 tokens always; more (in chunks of 16, the chunks re-reading
 // the weight rows from L2) while tokens x rows stays small -- measured against the tiled kernels: 1024 rows win up
@@ -545,19 +571,37 @@ bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
     if (K % 32 || K < 32 || N < 1) return false;
     if (N > 16 && (N > max_tokens || N * rows > 256 * 1024)) return false;
     const size_t nl = (size_t) (N < 16 ? N : 16);
-    return nl * K * 2 + nl * (K / 32) * 4 + 15 * 64 * 16 + 16 * sizeof(float) <= GV_MAX_LDS;
+    return nl * K * 2 + nl * (K / 32) * 4 + 15 * 64 * 16 + 16 * sizeof(float) + GV_ROPE_LDS <= GV_MAX_LDS;
 }
 
 size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
     const size_t nl = (size_t) (a.N < 16 ? a.N : 16);
-    return nl * a.K * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float);
+    return nl * a.K * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
+           (a.nseg > 0 ? GV_ROPE_LDS : 0);
 }
 
-// waves per work-group: about GV_UNROLL blocks per wave, so every load is issued up front
-int gemv_waves(const mm_args & a) {
-    const int64_t nkb = a.K / 32;
+// waves per work-group for a matrix of M rows: about GV_UNROLL blocks per wave, so every load is issued up front.  More
+// than a handful of tokens: the activations' work (staging, a fused RMS_NORM's wave-per-token sums in fp64, the rotation's
+// angles) outweighs the K walk and a matrix of few rows spreads it over 16 waves (norm + q/k/v + rope at 14 tokens: 12.8 ->
+// 9.8 us); a tall matrix already fills the CUs with work-groups and is slower with more waves (4096 x 2 rows: 9.3 -> 13.5 us
+// with 8).  The count -- and with it the order in which a product's K blocks are summed -- depends on K, on all tokens of the
+// call and on M, never on what is fused to the product.
+int gemv_waves_for(int64_t K, int64_t tokens, int64_t M) {
+    const int64_t nkb = K / 32;
     int nw = 1;
     while (nw < 16 && nkb > (int64_t) nw * GV_UNROLL) nw *= 2;
+    static const int many = [] { const char * e = getenv("VX_GEMV_MANY_TOKENS"); return e ? atoi(e) : 5; }();
+    if (tokens >= many && tokens <= 16 && nkb >= 16 && M <= 2048) nw = 16; // one chunk of tokens; several chunks multiply the waves instead
+    return nw;
+}
+
+// A launch over several matrices (the q / k / v segments, the gate / up pair) has one wave count: every matrix must get the
+// count it would get in a launch of its own.  -1 when they disagree: such a shape is left to the separate launches.
+int gemv_waves(const mm_args & a, int nbatch) {
+    const int64_t tokens = a.N * nbatch;
+    if (a.nseg == 0) return gemv_waves_for(a.K, tokens, a.M);
+    const int nw = gemv_waves_for(a.K, tokens, a.seg[0].M);
+    for (int i = 1; i < a.nseg; ++i) if (gemv_waves_for(a.K, tokens, a.seg[i].M) != nw) return -1;
     return nw;
 }
 
@@ -579,7 +623,8 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     };
     const int64_t nchunk = (a.N + 15) / 16;
     while (a.rows_wg > 4 && groups(a.rows_wg) * nbatch * nchunk < 128) a.rows_wg /= 2;
-    const int nw = gemv_waves(a);
+    const int nw = gemv_waves(a, nbatch);
+    if (nw < 0) return false;
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
     if (smem > GV_MAX_LDS) return false;
     int64_t nwg = groups(a.rows_wg);
@@ -1095,7 +1140,21 @@ extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor *
     if (v_dst->type != VX_TYPE_F32 || v_dst->nb[0] != 4 || v_dst->nb[1] % 4 || v_dst->nb[3] % 4) return 0;
     if (v_dst->nb[1] < (uint64_t) v_dst->ne[0] * 4 || (v_dst->ne[3] > 1 && v_dst->nb[3] < v_dst->nb[1] * (uint64_t) v_dst->ne[1])) return 0;
     if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
+    {
+        const int64_t tokens = x->ne[1] * x->ne[2] * x->ne[3];
+        const int nw = gemv_waves_for(wq->ne[0], tokens, wq->ne[1]);
+        if (gemv_waves_for(wq->ne[0], tokens, wk->ne[1]) != nw || gemv_waves_for(wq->ne[0], tokens, wv->ne[1]) != nw) return 0;
+    }
     return gemv_shape_ok(x->ne[1], wq->ne[1] + wk->ne[1] + wv->ne[1], wq->ne[0]);
+}
+
+// The order in which vx_mul_mat (and every group built on it) sums the K blocks of a product, as an opaque number: two
+// products with equal K, token count of the call and number are summed identically.  It depends on the row count, so a backend
+// that runs a product over a row range of a matrix in place of the product over the whole matrix (the reference's row-fused
+// qkv_proj / gate_up_proj) compares the two before promising identical bits.
+extern "C" int vx_mul_mat_sum_order(int64_t K, int64_t tokens, int64_t M) {
+    if (K < 32 || K % 32 || tokens < 1 || M < 1) return 0;
+    return gemv_waves_for(K, tokens, M);
 }
 
 static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,

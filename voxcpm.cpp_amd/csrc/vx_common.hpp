@@ -129,7 +129,7 @@ __device__ __forceinline__ void vx_rms_row_load(vx_rms_row & r, const float * x,
         r.v[c] = iv < nvec ? ((const float4 *) x)[iv] : float4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 }
-__device__ __forceinline__ float vx_rms_row_scale(const vx_rms_row & r, int64_t ne00, int lane, float eps) {
+__device__ __forceinline__ double vx_rms_row_lane_sum(const vx_rms_row & r, int64_t ne00, int lane) {
     const int64_t nvec = ne00 / 4;
     double sum = 0.0;
 #pragma unroll
@@ -143,9 +143,27 @@ __device__ __forceinline__ float vx_rms_row_scale(const vx_rms_row & r, int64_t 
             sum += (double) (v.w * v.w);
         }
     }
-    sum = vx_wave_sum(sum);
+    return sum;
+}
+__device__ __forceinline__ float vx_rms_finish(double sum, int64_t ne00, float eps) {
     const float mean = (float) (sum / (double) ne00);
     return 1.0f / sqrtf(mean + eps);
+}
+__device__ __forceinline__ float vx_rms_row_scale(const vx_rms_row & r, int64_t ne00, int lane, float eps) {
+    return vx_rms_finish(vx_wave_sum(vx_rms_row_lane_sum(r, ne00, lane)), ne00, eps);
+}
+// two rows by one wave: the same arithmetic per row, the two cross-lane chains issued side by side
+__device__ __forceinline__ void vx_rms_row_scale2(const vx_rms_row & r1, const vx_rms_row & r2, int64_t ne00, int lane, float eps,
+                                                  float & s1, float & s2) {
+    double a = vx_rms_row_lane_sum(r1, ne00, lane), b = vx_rms_row_lane_sum(r2, ne00, lane);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const double ta = __shfl_xor(a, off, 64), tb = __shfl_xor(b, off, 64);
+        a += ta;
+        b += tb;
+    }
+    s1 = vx_rms_finish(a, ne00, eps);
+    s2 = vx_rms_finish(b, ne00, eps);
 }
 __device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00, int lane, float eps) {
     vx_rms_row r;

@@ -974,6 +974,12 @@ bool compute_fused_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, co
     const ggml_tensor * x = norm ? norm->src[0] : mm->src[1];
     if (!apart(rq, x) || !apart(rk, x) || !apart(mm, x) || !apart(rq, rk) || !apart(rq, mm) || !apart(rk, mm)) return false;
     const ggml_tensor * W = mm->src[0];
+    {   // the row ranges must be summed as the one product over all rows would be
+        const int64_t tokens = x->ne[1] * x->ne[2] * x->ne[3];
+        const int order = vx_mul_mat_sum_order(W->ne[0], tokens, M);
+        if (order <= 0 || vx_mul_mat_sum_order(W->ne[0], tokens, qn) != order || vx_mul_mat_sum_order(W->ne[0], tokens, kn) != order ||
+            vx_mul_mat_sum_order(W->ne[0], tokens, vn) != order) return false;
+    }
     const vx_tensor wq = row_range(W, 0, qn), wk = row_range(W, qn, kn), wv = row_range(W, qn + kn, vn), xx = to_vx(x), dq = to_vx(rq), dk = to_vx(rk);
     vx_tensor dv = to_vx(mm);                       // the v rows of the product, where they lie
     dv.data  = (char *) mm->data + (size_t) (qn + kn) * 4;
@@ -1022,6 +1028,11 @@ bool compute_fused_gate_up_group(backend_ctx * ctx, const ggml_cgraph * g, int i
     const ggml_tensor * x = norm ? norm->src[0] : mm->src[1];
     if (!apart(glu, x)) return false;
     const ggml_tensor * W = mm->src[0];
+    {   // the two halves must be summed as the one product over all rows would be
+        const int64_t tokens = x->ne[1] * x->ne[2] * x->ne[3];
+        const int order = vx_mul_mat_sum_order(W->ne[0], tokens, 2 * ffn);
+        if (order <= 0 || vx_mul_mat_sum_order(W->ne[0], tokens, ffn) != order) return false;
+    }
     const vx_tensor gw = row_range(W, 0, ffn), uw = row_range(W, ffn, ffn), xx = to_vx(x), d = to_vx(glu);
     if (norm) {
         const vx_tensor nw = to_vx(scale->src[1]);
