@@ -388,7 +388,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
-    ap.add_argument("--profile", choices=["prefill", "backbone"], default=None,
+    ap.add_argument("--profile", choices=["prefill", "backbone", "cfm"], default=None,
                     help="run only this secondary workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -415,6 +415,9 @@ def main():
         s = timer.run(call, iters=5, warmup=2)
         print(json.dumps({"profile": "cfg5_prefill_attn_T4096_B16", "us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
                           "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}))
+        return
+    if args.profile == "cfm":       # config 3: whole CFM solves of one request, replayed from a HIP graph
+        print(json.dumps({"profile": "cfg3_cfm_solve_one_request", **cfm_solve_bench(pkg, timer, torch.cuda.Stream(), 1, False)}))
         return
     if args.profile == "backbone":  # config 4 decode steps, eager launches so that every kernel is traced
         print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16)}))
