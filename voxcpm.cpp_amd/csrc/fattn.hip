@@ -360,9 +360,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 // Merges the split partials: the arithmetic of ggml_flash_attn_ext_reduce_partials
 // (ggml/src/ggml-cpu/ops.cpp:8637-8705) with the global maximum taken first.  One wave per
 // output column.  Lane = (split phase q, 4 consecutive d): the D/4 lanes of a phase read one
-// split's row as one coalesced line, the 64/(D/4) phases take interleaved splits.  The (max,
-// sum) pairs are read one split per lane; every load of the first 64 splits is issued before
-// anything waits, so the kernel costs one trip to memory, a few cross-lane steps and a store.
+// split's row as one coalesced line, the 64/(D/4) phases take interleaved splits.  A lane reads
+// the (max, sum) pairs of its own splits too; every load of the first 16 splits per phase is
+// issued before anything waits, so the kernel costs one trip to memory, a few cross-lane steps
+// between the phases and a store.
 constexpr int FA_MERGE_MAX_SPLITS = 256;
 template <int D>
 __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
@@ -394,60 +395,56 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
     bool  has_addend = a.add1 != nullptr;
     float addend     = has_addend ? *a.add1 : 0.0f;
     const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + c; // + split * 16
-    const int nsl = (a.n_splits + 63) >> 6;                         // (max, sum) pairs per lane
-
-    float m[FA_MERGE_MAX_SPLITS / 64], l[FA_MERGE_MAX_SPLITS / 64];
-#pragma unroll
-    for (int i = 0; i < FA_MERGE_MAX_SPLITS / 64; ++i) {
-        m[i] = -INFINITY; l[i] = 0.0f;
-        const int s2 = lane + 64 * i;
-        if (i < nsl && s2 < a.n_splits) {
-            const float2 ml = *(const float2 *) (a.part_ml + (tbase + (uint64_t) s2 * 16) * 2);
-            m[i] = ml.x; l[i] = ml.y;
-        }
-    }
-    const float4_t * po = (const float4_t *) (a.part_o + tbase * D + d0); // + split * 4*D float4
+    // A lane works on the splits of its phase only: q, q + PH, q + 2 PH, ...  It reads their (max, sum) pairs and rows itself
+    // and forms their weights itself, so the only cross-lane traffic is between the PH phases (log2 PH steps for the maximum,
+    // the sum and the accumulator) -- no broadcast of weights from other lanes.
+    const int per = (a.n_splits + PH - 1) / PH; // splits per lane
+    const float2 *   pml = (const float2 *) (a.part_ml + tbase * 2);           // + split * 16 pairs
+    const float4_t * po  = (const float4_t *) (a.part_o + tbase * D + d0);     // + split * 4 * D float4
+    float    mv[NB], lv[NB];
     float4_t rows[NB];
-    auto load_rows = [&](int j0) {
+    auto load_batch = [&](int j0) { // every load of a batch is issued before anything waits
 #pragma unroll
         for (int jj = 0; jj < NB; ++jj) {
-            const int s2 = q + PH * (j0 + jj);
-            rows[jj] = s2 < a.n_splits ? po[(uint64_t) s2 * 4 * D] : float4_t{0, 0, 0, 0};
+            const int  s2 = q + PH * (j0 + jj);
+            const bool ok = j0 + jj < per && s2 < a.n_splits;
+            const float2 ml = ok ? pml[(uint64_t) s2 * 16] : float2{-INFINITY, 0.0f};
+            mv[jj] = ml.x; lv[jj] = ml.y;
+            rows[jj] = ok ? po[(uint64_t) s2 * 4 * D] : float4_t{0, 0, 0, 0};
         }
     };
-    load_rows(0);
-
-    float M = m[0];
+    load_batch(0);
+    float M = -INFINITY;
 #pragma unroll
-    for (int i = 1; i < FA_MERGE_MAX_SPLITS / 64; ++i) M = fmaxf(M, m[i]);
-    M = vx_wave_max(M);
-    const float shift = (M == -INFINITY) ? 0.0f : M;
-    float L = 0.0f;
-#pragma unroll
-    for (int i = 0; i < FA_MERGE_MAX_SPLITS / 64; ++i) {
-        m[i] = __builtin_amdgcn_exp2f(m[i] - shift); // from here on: the split's weight
-        L += l[i] * m[i];
-    }
-    L = vx_wave_sum(L);
-
-    float4_t acc = {0, 0, 0, 0};
-    const int per = (a.n_splits + PH - 1) / PH; // rows per lane
-    for (int j0 = 0; j0 < per; j0 += NB) {
-        if (j0) load_rows(j0);
-        const int i = (PH * j0) >> 6;           // the NB * PH splits of a batch lie in one 64-group
-        float wsel = m[0];
-#pragma unroll
-        for (int k = 1; k < FA_MERGE_MAX_SPLITS / 64; ++k) wsel = (i == k) ? m[k] : wsel;
+    for (int jj = 0; jj < NB; ++jj) M = fmaxf(M, mv[jj]);
+    for (int j0 = NB; j0 < per; j0 += NB) { // more than NB splits per lane: their maxima in a pass of their own
 #pragma unroll
         for (int jj = 0; jj < NB; ++jj) {
             const int s2 = q + PH * (j0 + jj);
-            acc += rows[jj] * __shfl(wsel, s2 & 63, 64);
+            if (j0 + jj < per && s2 < a.n_splits) M = fmaxf(M, pml[(uint64_t) s2 * 16].x);
         }
     }
 #pragma unroll
-    for (int off = DU; off < 64; off <<= 1)
+    for (int off = DU; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+    const float shift = (M == -INFINITY) ? 0.0f : M;
+
+    float    L   = 0.0f;
+    float4_t acc = {0, 0, 0, 0};
+    for (int j0 = 0; j0 < per; j0 += NB) {
+        if (j0) load_batch(j0);
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj) {
+            const float wgt = __builtin_amdgcn_exp2f(mv[jj] - shift); // the split's weight (0 for a slot past the end: max = -inf)
+            L   += lv[jj] * wgt;
+            acc += rows[jj] * wgt;
+        }
+    }
+#pragma unroll
+    for (int off = DU; off < 64; off <<= 1) {
+        L += __shfl_xor(L, off, 64);
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], off, 64);
+    }
     if (a.has_kvs) { // uniform: the block was launched with its second wave
         __syncthreads();
         addend     = kvs_addend;
