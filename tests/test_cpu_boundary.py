@@ -187,6 +187,15 @@ def test_supports_truth_table_node_groups(pkg):
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(1), acts(14)) == 1                # a bias row, repeated over the tokens
     assert lib.vx_supports_mul_mat_scale_add(q8(pkg, [64, K, 1, 1]), acts(2, 64), acts(1), acts(2)) == 1   # LocDiT's in_proj + bias
     assert lib.vx_supports_mul_mat_scale_add(f32(pkg, [K, K, 1, 1]), acts(2), acts(2), acts(2)) == 0   # F32 weights
+    # the order in which a product's K blocks are summed depends on its shape alone; what the plugin compares before it
+    # replaces one product over a row-fused matrix by products over its row ranges
+    order = lib.vx_mul_mat_sum_order
+    assert order(K, 2, 1280) == order(K, 2, 1024) == order(K, 2, 128) > 0          # decode: q, k, v ranges of qkv_proj
+    assert order(K, 14, 1280) == order(K, 14, 1024) == order(K, 14, 128)           # LocDiT's 14-token pair
+    assert order(K, 14, 8192) == order(K, 14, 4096)                                # gate_up_proj and its halves
+    assert order(K, 14, 1024) != order(K, 14, 4096)                                # few rows spread the token work over more waves
+    assert order(K, 14, 1024) != order(K, 2, 1024) and order(K, 112, 1024) == order(K, 2, 1024)
+    assert order(K, 0, 1024) == 0 and order(33, 2, 1024) == 0
     # gate / up / SwiGLU: both matrices count as rows
     wg = q8(pkg, [K, 4096, 1, 1])
     ffn = lambda n: f32(pkg, [4096, n, 1, 1])
