@@ -558,6 +558,10 @@ struct cfm_extra {
     ggml_backend_buffer_t buf = nullptr;
     ggml_tensor * w[3] = { nullptr, nullptr, nullptr }; // in_proj, cond_proj [feat, hidden]; out_proj [hidden, feat]
     ggml_tensor * b[3] = { nullptr, nullptr, nullptr };
+    // time_mlp and delta_time_mlp: linear1, linear2 (Q8_0 [hidden, hidden]) and their biases (rh_cfm_set_time_mlp)
+    ggml_tensor * tw[4] = { nullptr, nullptr, nullptr, nullptr };
+    ggml_tensor * tb[4] = { nullptr, nullptr, nullptr, nullptr };
+    bool has_time_mlp = false;
     int feat = 0;
 };
 cfm_extra * g_cfm = nullptr;
@@ -579,9 +583,13 @@ int rh_cfm_create(int feat, const void * in_w, const float * in_b, const void * 
     rh_cfm_free();
     cfm_extra * e = new cfm_extra;
     e->feat = feat;
-    ggml_init_params ip = { ggml_tensor_overhead() * 8, nullptr, true };
+    ggml_init_params ip = { ggml_tensor_overhead() * 16, nullptr, true };
     e->ctx = ggml_init(ip);
     const int64_t H = g_bb->hidden;
+    for (int i = 0; i < 4; ++i) {
+        e->tw[i] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, H, H);
+        e->tb[i] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, H);
+    }
     e->w[0] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, feat, H); e->b[0] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, H);
     e->w[1] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, feat, H); e->b[1] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, H);
     e->w[2] = ggml_new_tensor_2d(e->ctx, GGML_TYPE_Q8_0, H, feat); e->b[2] = ggml_new_tensor_1d(e->ctx, GGML_TYPE_F32, feat);
@@ -597,6 +605,19 @@ int rh_cfm_create(int feat, const void * in_w, const float * in_b, const void * 
     return 0;
 }
 
+// The weights of LocDiT's two timestep MLPs (src/locdit.cpp:213-246): which 0, 1 = time_mlp linear1, linear2; 2, 3 =
+// delta_time_mlp linear1, linear2; Q8_0 rows [hidden][hidden] and F32 bias.  With them set, rh_cfm_solve called without a
+// time table computes the combined time embedding of every step in the graph, as UnifiedCFM::forward does when it was not
+// handed a precomputed table: ARANGE(t), the sinusoidal embedding (ARANGE, SCALE, EXP, SCALE, REPEAT, MUL, SIN, COS, CONCAT),
+// two MUL_MAT + ADD + SILU layers, plus the delta-time embedding of zero.
+int rh_cfm_set_time_mlp(int which, const void * w, const float * b) {
+    if (!g_cfm || which < 0 || which > 3) return 100;
+    ggml_backend_tensor_set(g_cfm->tw[which], w, 0, ggml_nbytes(g_cfm->tw[which]));
+    ggml_backend_tensor_set(g_cfm->tb[which], b, 0, ggml_nbytes(g_cfm->tb[which]));
+    if (which == 3) g_cfm->has_time_mlp = true;
+    return 0;
+}
+
 // z [feat, patch], mu [hidden], cond [feat, prefix], time_table [hidden, n_steps] (the combined time embedding of every
 // step, as LocDiTModel::precompute_cfg_time_table hands it over), t_span n_steps + 1 values, pair_pos / pair_mask the
 // CFG-pair constants for a branch of 1 + prefix + patch tokens.  out [feat, patch].  seconds: mean, best, node count.
@@ -604,11 +625,12 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
                  int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
                  int zero_star, float * out, int reps, double * seconds) {
     if (!g_bb || !g_cfm || !g_backend || n_steps < 1 || prefix < 1) return 100;
+    if (!time_table && !g_cfm->has_time_mlp) return 103;
     const backbone & m = *g_bb;
     const cfm_extra & e = *g_cfm;
     const int H = m.hidden, F = e.feat, L = 1 + prefix + patch, T = 2 * L;
     if (T > m.max_len) return 104;
-    const size_t n_nodes = (size_t) n_steps * ((size_t) m.n_layer * 64 + 96) + 64;
+    const size_t n_nodes = (size_t) n_steps * ((size_t) m.n_layer * 64 + 160) + 128;
     ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
     ggml_context * c = ggml_init(ip);
     ggml_tensor * zin  = ggml_new_tensor_2d(c, GGML_TYPE_F32, F, patch);
@@ -622,6 +644,17 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
     std::vector<ggml_tensor *> roots;
     ggml_tensor * x = zin;
     ggml_tensor * cond_proj = ggml_add(c, ggml_mul_mat(c, e.w[1], cin), e.b[1]);
+    // LocDiTModel::sinusoidal_embedding + timestep_mlp (src/locdit.cpp:186-232)
+    auto time_embedding = [&](ggml_tensor * scalar, int mlp) {
+        const int   half = H / 2;
+        const float ev   = logf(10000.0f) / (float) (half - 1);
+        ggml_tensor * emb = ggml_scale(c, ggml_exp(c, ggml_scale(c, ggml_arange(c, 0.0f, (float) half, 1.0f), -ev)), 1000.0f);
+        emb = ggml_mul(c, emb, ggml_repeat(c, ggml_reshape_1d(c, scalar, 1), emb));
+        ggml_tensor * sc = ggml_concat(c, ggml_sin(c, emb), ggml_cos(c, emb), 0);
+        ggml_tensor * h1 = ggml_silu(c, ggml_add(c, ggml_mul_mat(c, e.tw[2 * mlp], sc), e.tb[2 * mlp]));
+        return ggml_add(c, ggml_mul_mat(c, e.tw[2 * mlp + 1], h1), e.tb[2 * mlp + 1]);
+    };
+    ggml_tensor * delta_zero = time_table ? nullptr : time_embedding(ggml_arange(c, 0.0f, 1.0f, 1.0f), 1);
     float t = t_span[0], dt = t_span[0] - t_span[1];
     const int zero_init_steps = n_steps > 1 ? std::max(1, (int) ((float) (n_steps + 1) * 0.04f)) : 0;
     for (int step = 1; step <= n_steps; ++step) {
@@ -630,7 +663,8 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
             dphi = ggml_scale(c, x, 0.0f);
         } else {
             ggml_tensor * x_proj   = ggml_add(c, ggml_mul_mat(c, e.w[0], x), e.b[0]);
-            ggml_tensor * combined = ggml_view_1d(c, tab, H, (size_t) (step - 1) * H * sizeof(float));
+            ggml_tensor * combined = time_table ? ggml_view_1d(c, tab, H, (size_t) (step - 1) * H * sizeof(float))
+                                                : ggml_add(c, time_embedding(ggml_arange(c, t, t + 1.0f, 1.0f), 0), delta_zero);
             ggml_tensor * comb_c   = ggml_reshape_2d(c, ggml_add(c, ggml_reshape_1d(c, combined, H), muin), H, 1);
             ggml_tensor * comb_u   = ggml_reshape_2d(c, combined, H, 1);
             ggml_tensor * seq_c    = ggml_concat(c, ggml_concat(c, comb_c, cond_proj, 1), x_proj, 1);
@@ -667,7 +701,7 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
         ggml_backend_tensor_set(zin, z, 0, ggml_nbytes(zin));
         ggml_backend_tensor_set(muin, mu, 0, ggml_nbytes(muin));
         ggml_backend_tensor_set(cin, cond, 0, ggml_nbytes(cin));
-        ggml_backend_tensor_set(tab, time_table, 0, ggml_nbytes(tab));
+        if (time_table) ggml_backend_tensor_set(tab, time_table, 0, ggml_nbytes(tab));
         ggml_backend_tensor_set(pos, pair_pos, 0, ggml_nbytes(pos));
         ggml_backend_tensor_set(msk, pair_mask, 0, ggml_nbytes(msk));
     };

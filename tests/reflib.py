@@ -182,6 +182,7 @@ def load_ref():
     lib.rh_cfm_create.argtypes = [C.c_int, C.c_void_p, f32p_, C.c_void_p, f32p_, C.c_void_p, f32p_]
     lib.rh_cfm_solve.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int,
                                  f32p_, C.c_int, C.POINTER(C.c_double)]
+    lib.rh_cfm_set_time_mlp.argtypes = [C.c_int, C.c_void_p, f32p_]
     lib.rh_cfm_free.argtypes = []
     lib.rh_cfm_free.restype = None
     lib.rh_bb_fuse_weights.argtypes = []
@@ -399,7 +400,10 @@ def cfm_params(tag, feat=64, hidden=1024):
             "cond_w": (g("cond_w").standard_normal((hidden, feat)) / np.sqrt(feat)).astype(np.float32),
             "cond_b": (0.1 * g("cond_b").standard_normal(hidden)).astype(np.float32),
             "out_w": (g("out_w").standard_normal((feat, hidden)) / np.sqrt(hidden)).astype(np.float32),
-            "out_b": (0.1 * g("out_b").standard_normal(feat)).astype(np.float32)}
+            "out_b": (0.1 * g("out_b").standard_normal(feat)).astype(np.float32),
+            # time_mlp linear1 / linear2, delta_time_mlp linear1 / linear2 (src/locdit.cpp:213-246)
+            "time_w": [(g("time_w", i).standard_normal((hidden, hidden)) / np.sqrt(hidden)).astype(np.float32) for i in range(4)],
+            "time_b": [(0.1 * g("time_b", i).standard_normal(hidden)).astype(np.float32) for i in range(4)]}
 
 
 def ref_cfm_create(p):
@@ -410,13 +414,17 @@ def ref_cfm_create(p):
     rc = lib.rh_cfm_create(p["feat"], q["in_w"].ctypes.data, f(p["in_b"]), q["cond_w"].ctypes.data, f(p["cond_b"]),
                            q["out_w"].ctypes.data, f(p["out_b"]))
     assert rc == 0, rc
+    for i in range(4):
+        wq = quantize_q8_0(p["time_w"][i])
+        assert lib.rh_cfm_set_time_mlp(i, wq.ctypes.data, f(p["time_b"][i])) == 0
 
 
 def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_star=True, reps=0):
     """One UnifiedCFM solve as a single graph on the harness's device.  z (patch, feat), mu (hidden,), cond (prefix, feat),
     table (n_steps, hidden).  Returns (x (patch, feat), seconds[mean, best], n_nodes)."""
     lib, orc = load_ref(), load_oracle()
-    z, mu, cond, table = (np.ascontiguousarray(a, dtype=np.float32) for a in (z, mu, cond, table))
+    z, mu, cond = (np.ascontiguousarray(a, dtype=np.float32) for a in (z, mu, cond))
+    table = None if table is None else np.ascontiguousarray(table, dtype=np.float32)   # None: the time embeddings are built in the graph
     patch, prefix = z.shape[0], cond.shape[0]
     L = 1 + prefix + patch
     t_span = np.zeros(n_steps + 1, np.float32)
@@ -426,7 +434,7 @@ def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_
     orc.orc_cfg_pair_constants(L, ptr(pos, C.c_int32), ptr(mk, C.c_uint16))
     out = np.empty_like(z)
     sec = np.zeros(3, np.float64)
-    rc = lib.rh_cfm_solve(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), ptr(table, C.c_float), ptr(t_span, C.c_float),
+    rc = lib.rh_cfm_solve(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), None if table is None else ptr(table, C.c_float), ptr(t_span, C.c_float),
                           n_steps, patch, prefix, ptr(pos, C.c_int32), ptr(mk, C.c_uint16), cfg_value, int(zero_star),
                           ptr(out, C.c_float), reps, ptr(sec, C.c_double))
     assert rc == 0, rc

@@ -284,12 +284,16 @@ def test_plugin_runs_the_whole_forward_graph_without_a_scheduler(gpu, ref, T0):
         assert np.array_equal(b, c), i
 
 
-def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
+@pytest.mark.parametrize("time_table", [True, False])
+def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref, time_table):
     """BASELINE config 3 as the reference builds it (src/unified_cfm.cpp:88-184 around src/locdit.cpp:401-464): ten
     Euler steps of the LocDiT estimator in ONE graph -- input projection, the CFG pair as one 14-token non-causal
     sequence through 4 decoder layers with row-fused weights, output projection of both branches, the zero-star
     guidance scale (MUL, SUM, ARANGE, DIV, REPEAT) and the update of x.  Direct graph_compute on the plugin against
-    ggml-cpu, grouped launches against node-by-node ones (same bits), and the launch count of a solve."""
+    ggml-cpu, grouped launches against node-by-node ones (same bits), and the launch count of a solve.
+    time_table=False: the combined time embedding of every step is computed in the graph too, as UnifiedCFM::forward does
+    without a precomputed table (sinusoidal embedding -- ARANGE, SCALE, EXP, REPEAT, MUL, SIN, COS, CONCAT -- and the two
+    timestep MLPs, src/locdit.cpp:186-246)."""
     import ctypes
     import subprocess
     import sys
@@ -298,7 +302,7 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
     z = rng("cfm", "z").standard_normal((2, 64)).astype(np.float32)
     mu = rng("cfm", "mu").standard_normal(1024).astype(np.float32)
     cond = rng("cfm", "cond").standard_normal((4, 64)).astype(np.float32)
-    table = rng("cfm", "table").standard_normal((10, 1024)).astype(np.float32)
+    table = rng("cfm", "table").standard_normal((10, 1024)).astype(np.float32) if time_table else None
 
     def run(device, reps=0):
         assert ref.rh_use_device(device, 8, 0) == 0
@@ -321,8 +325,9 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
           f"ggml-cpu (8 threads) {cpu_s[1] * 1e3:.2f} ms, plugin {plug_s[1] * 1e3:.3f} ms per solve", flush=True)
     assert e <= 1e-3
     # nine estimator passes (step 1 is zero under zero-star): 4 layers x 5 launches + the final norm for the decoder,
-    # at most 26 for the projections, the five CONCATs, the guidance arithmetic and the update of x
-    assert launches <= 9 * (4 * 5 + 1 + 26) + 5, (launches, n_nodes)
+    # at most 26 for the projections, the five CONCATs, the guidance arithmetic and the update of x (and at most 12 more
+    # per step for a time embedding built in the graph)
+    assert launches <= 9 * (4 * 5 + 1 + 26 + (0 if time_table else 12)) + 5 + (0 if time_table else 12), (launches, n_nodes)
     # node by node in a fresh process: the groups must not change a bit
     code = (
         "import sys, numpy as np\n"
@@ -336,7 +341,7 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
         "z = rng('cfm', 'z').standard_normal((2, 64)).astype(np.float32)\n"
         "mu = rng('cfm', 'mu').standard_normal(1024).astype(np.float32)\n"
         "cond = rng('cfm', 'cond').standard_normal((4, 64)).astype(np.float32)\n"
-        "table = rng('cfm', 'table').standard_normal((10, 1024)).astype(np.float32)\n"
+        f"table = rng('cfm', 'table').standard_normal((10, 1024)).astype(np.float32) if {time_table} else None\n"
         "reflib.ref_backbone_create(params, 32, 1, use_mup=True, kv_f16=False, fused_weights=True)\n"
         "reflib.ref_cfm_create(cp)\n"
         "out = reflib.ref_cfm_solve(z, mu, cond, table)[0]\n"
@@ -347,6 +352,8 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref):
     assert p.returncode == 0, p.stderr[-2000:]
     bits = [l for l in p.stdout.splitlines() if l.startswith("BITS ")][0][5:]
     assert bytes.fromhex(bits) == plug.tobytes()
+    if not time_table:
+        return
     # the C-ABI mirror of the solve (voxcpm.cpp_amd/cfm.py): the plugin's launches issued by hand, the same bits
     import torch
     from voxcpm_cpp_amd import backbone as bb, cfm
