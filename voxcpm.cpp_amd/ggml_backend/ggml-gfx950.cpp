@@ -572,7 +572,44 @@ bool compute_pair(backend_ctx * ctx, ggml_tensor * node, ggml_tensor * next, vx_
     return false;
 }
 
-typedef std::unordered_map<const ggml_tensor *, int> reader_map;
+// tensor -> count, for the graph analysis that runs in front of the first launch of every graph_compute: a flat
+// open-addressing table (a node-based map costs more than 100 us on a 1200-node graph, all of it latency of the call)
+class reader_map {
+  public:
+    struct slot { const ggml_tensor * first; int second; };
+    void reserve(size_t n) {
+        size_t cap = 64;
+        while (cap < 2 * n) cap <<= 1;
+        if (cap <= slots_.size()) return;
+        std::vector<slot> old;
+        old.swap(slots_);
+        slots_.assign(cap, slot{ nullptr, 0 });
+        used_ = 0;
+        for (const slot & o : old) if (o.first) (*this)[o.first] = o.second;
+    }
+    int & operator[](const ggml_tensor * key) {
+        if (2 * (used_ + 1) > slots_.size()) reserve(slots_.empty() ? 32 : slots_.size());
+        slot * s = probe(key);
+        if (!s->first) { s->first = key; ++used_; }
+        return s->second;
+    }
+    const slot * find(const ggml_tensor * key) const {
+        if (slots_.empty()) return nullptr;
+        const slot * s = const_cast<reader_map *>(this)->probe(key);
+        return s->first ? s : nullptr;
+    }
+    const slot * end() const { return nullptr; }
+
+  private:
+    slot * probe(const ggml_tensor * key) {
+        const size_t mask = slots_.size() - 1;
+        size_t i = (size_t) ((((uintptr_t) key >> 4) * 0x9E3779B97F4A7C15ull) >> 32) & mask;
+        while (slots_[i].first && slots_[i].first != key) i = (i + 1) & mask;
+        return &slots_[i];
+    }
+    std::vector<slot> slots_;
+    size_t            used_ = 0;
+};
 
 // a node whose value only the group's next member looks at, so it need not be stored
 bool private_to_group(const reader_map & readers, const ggml_tensor * t) {
@@ -1064,18 +1101,22 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     reader_map readers;
     if (fusion && cgraph->n_nodes > 1) {
         readers.reserve((size_t) cgraph->n_nodes * 2);
+        // Under ggml_backend_sched this graph is a window of a larger one (ggml_graph_view: no leafs of its own, the
+        // whole graph's hash set and use counts): a node that is also read from another split must be stored like
+        // an output.  Such nodes get a reader count no group accepts.  A whole graph needs none of this.
+        const bool window = cgraph->leafs == nullptr && cgraph->use_counts && cgraph->visited_hash_set.keys && cgraph->visited_hash_set.size > 0;
         reader_map as_operand; // uses as src[] only, the quantity ggml's own use counts hold
-        as_operand.reserve((size_t) cgraph->n_nodes * 2);
+        if (window) as_operand.reserve((size_t) cgraph->n_nodes * 2);
         for (int i = 0; i < cgraph->n_nodes; ++i) {
             const ggml_tensor * n = cgraph->nodes[i];
             for (int k = 0; k < GGML_MAX_SRC; ++k)
-                if (n->src[k]) { readers[n->src[k]]++; as_operand[n->src[k]]++; }
+                if (n->src[k]) {
+                    readers[n->src[k]]++;
+                    if (window) as_operand[n->src[k]]++;
+                }
             if (n->view_src) readers[n->view_src]++;
         }
-        // Under ggml_backend_sched this graph is a window of a larger one (ggml_graph_view shares the whole
-        // graph's hash set and use counts): a node that is also read from another split must be stored like
-        // an output.  Such nodes get a reader count no group accepts.
-        if (cgraph->use_counts && cgraph->visited_hash_set.keys && cgraph->visited_hash_set.size > 0) {
+        if (window) {
             for (int i = 0; i < cgraph->n_nodes; ++i) {
                 const ggml_tensor * n = cgraph->nodes[i];
                 const size_t pos = ggml_hash_find(&cgraph->visited_hash_set, n);
