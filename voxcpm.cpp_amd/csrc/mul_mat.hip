@@ -883,9 +883,253 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
     return true;
 }
 
+// ---- GEMM shape, both operands through LDS -----------------------------------------------------------
+// Same 128 x 128 tile and 2 x 2 waves as above.  Fetching the weights straight into the MFMA layout makes every
+// 16-lane group of a load touch 16 different rows, i.e. 16 cache lines for 12 useful bytes each, and the
+// per-CU cache that serves one line per cycle becomes the limit of the whole kernel.  Here a thread fetches
+// (row, block, 8-quant group) units in row-major order, so that 16 lanes cover two 68-byte runs, turns its
+// quants into f16 once for the work-group, and parks them in LDS in the operand layout; activations are
+// fetched 256 contiguous bytes per 16 lanes.  One barrier per round of GL_KC blocks, the global loads of
+// round r+1 in flight during round r's MFMAs.
+constexpr int    GL_KC   = 2;
+// LDS of a work-group that owns 32 RT rows x 32 CT tokens: both operands double-buffered, and the block scales
+constexpr size_t gl_lds(int RT, int CT) { return 2 * GL_KC * (2 * RT + 2 * CT) * 64 * sizeof(half8_t) + 2 * GL_KC * 32 * RT * sizeof(float); }
+
+// FOLD: the block scale is multiplied into the f16 weights as they are parked (q * d rounded to f16, relative
+// error 2^-12 on average -- the size of the activations' own rounding) and the MFMAs accumulate across blocks;
+// otherwise the weights stay the exact integers and each 32-wide partial product is scaled in fp32.
+// A wave owns RT x CT MFMA tiles (16 rows x 16 tokens each), the work-group 2 x 2 waves.
+template <int WT, bool FOLD, int RT, int CT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_lds_kernel(const mm_args a) {
+    static_assert(GL_KC == 2, "the parity of a block inside a round is its index in the round");
+    constexpr int  TR = 2 * RT, TC = 2 * CT; // 16-wide tiles per work-group: rows, tokens
+    constexpr int  ROWS = 16 * TR, TOKS = 16 * TC;
+    constexpr bool POST = WT == WT_Q8 && !FOLD; // scale after the MFMA
+    extern __shared__ __align__(16) char gl_smem[];
+    constexpr int XOPS = GL_KC * TC * 64, WOPS = GL_KC * TR * 64;
+    half8_t * xs = (half8_t *) gl_smem;                       // [2][XOPS] activations
+    half8_t * ws = xs + 2 * XOPS;                             // [2][WOPS] weights
+    float *   wd = (float *) (ws + 2 * WOPS);                 // [2][GL_KC * ROWS] block scales
+
+    const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
+    const int j = lane >> 4, c = lane & 15;
+    const int wr = wid >> 1, wt = wid & 1;
+
+    const int     batch = blockIdx.z;
+    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+    char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+
+    // token tiles partitioned over the XCDs, row tiles of one token tile side by side (see gemm128_kernel)
+    const int64_t gx = (a.M + ROWS - 1) / ROWS, gy = (a.N + TOKS - 1) / TOKS;
+    const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int64_t ty = (slot / gx) * 8 + xcd;
+    if (ty >= gy) return;
+    const int64_t tok0 = ty * TOKS;
+    const int64_t rowg = (slot % gx) * ROWS;
+    const int64_t nround = a.K / (32 * GL_KC); // the launcher takes whole rounds only
+
+    // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
+    // products are computed and dropped), so no load carries a predicate.  Addresses are a uniform base
+    // plus a 32-bit lane offset that never changes (the launcher checks the ranges).
+    // ---- weight stream: unit = (row, block of the round, group of 8 k), RT per thread and round
+    constexpr int WUNIT = WT == WT_Q8 ? 3 : 4; // dwords fetched per unit
+    uint32_t wraw[RT][WUNIT];
+    uint32_t woff[RT];
+#pragma unroll
+    for (int it = 0; it < RT; ++it) {
+        const int unit = tid + 256 * it;
+        const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
+        const uint64_t rowoff = (uint64_t) min(rowg + row, a.M - 1) * a.nb01;
+        if constexpr (WT == WT_Q8) woff[it] = (uint32_t) (rowoff + kbl * VX_Q8_BLOCK + 8 * uj - (kbl ? 2 : 0));
+        else                       woff[it] = (uint32_t) (rowoff + kbl * 64 + 16 * uj);
+    }
+    constexpr int WROUND = GL_KC * (WT == WT_Q8 ? VX_Q8_BLOCK : 64); // bytes of a row walked per round
+    auto load_weights = [&](int64_t round) {
+        const char * wk = wb + (uint64_t) round * WROUND; // uniform
+#pragma unroll
+        for (int it = 0; it < RT; ++it) {
+            const char * p = (const char *) __builtin_assume_aligned(wk + woff[it], WT == WT_Q8 ? 4 : 16);
+            __builtin_memcpy(wraw[it], p, 4 * WUNIT);
+        }
+    };
+    // where a unit goes in LDS: the same place every round
+    uint32_t wslot[RT];
+#pragma unroll
+    for (int it = 0; it < RT; ++it) {
+        const int unit = tid + 256 * it;
+        wslot[it] = (uint32_t) lds_slot((unit >> 2) & 1, unit >> 7, TR, unit & 3, (unit >> 3) & 15);
+    }
+    auto store_weights = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < RT; ++it) {
+            const int unit = tid + 256 * it;
+            const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
+            half8_t h;
+            if constexpr (WT == WT_Q8) {
+                // an even block starts on a dword with its scale in front; the fetch of an odd block starts 2 bytes early
+                h = q8_unpack(q8_raw{wraw[it][0], wraw[it][1], wraw[it][2]}, kbl, true);
+                const uint32_t bits = kbl ? wraw[it][0] >> 16 : wraw[it][0] & 0xffffu; // the scale, in the unit with uj == 0
+                if constexpr (FOLD) {
+                    // the four units of a block sit in four neighbouring lanes: take the scale from the first
+                    const uint32_t b0 = (uint32_t) __builtin_amdgcn_update_dpp(0, (int) bits, 0x00 /* quad_perm 0,0,0,0 */, 0xf, 0xf, true);
+                    const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t) b0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) h[i] *= d;
+                } else {
+                    if (uj == 0) wd[(buf * GL_KC + kbl) * ROWS + row] = (float) __builtin_bit_cast(_Float16, (uint16_t) bits);
+                }
+            } else {
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                h = __builtin_bit_cast(half8_t, u32x4{wraw[it][0], wraw[it][1], wraw[it][2], wraw[it][3]});
+            }
+            ws[buf * WOPS + wslot[it]] = h;
+        }
+    };
+    // ---- activation stream: unit = (token, 16-byte piece of its 256 bytes of the round), 2 CT per thread and round
+    float4_t xr[2 * CT];
+    const int xchunk = tid & 15;
+    uint32_t xoff[2 * CT];
+#pragma unroll
+    for (int i = 0; i < 2 * CT; ++i) {
+        const int64_t tok = min(tok0 + (tid >> 4) + 16 * i, a.N - 1);
+        xoff[i] = (uint32_t) ((uint64_t) (tok - tok0) * a.nb11 + (uint64_t) xchunk * 16);
+    }
+    const char * xtile = xb + (uint64_t) tok0 * a.nb11;
+    auto load_acts = [&](int64_t round) {
+        const char * base = xtile + (uint64_t) round * (GL_KC * 128); // uniform
+#pragma unroll
+        for (int i = 0; i < 2 * CT; ++i) xr[i] = *(const float4_t *) (base + xoff[i]);
+    };
+    // byte offset of token (tid >> 4)'s piece in LDS; token + 16 i is the next 16-token tile, 64 slots on
+    const uint32_t xslot = (uint32_t) lds_slot(xchunk >> 3, 0, TC, (xchunk & 7) >> 1, tid >> 4) * 16 + 8 * (xchunk & 1);
+    auto store_acts = [&](int buf) {
+        typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int i = 0; i < 2 * CT; ++i) {
+            half4_t h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = (_Float16) xr[i][e];
+            *(half4_t *) ((char *) (xs + buf * XOPS + 64 * i) + xslot) = h;
+        }
+    };
+
+    float4_t acc[RT][CT]; // [row tile][token tile]
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < CT; ++tt) acc[rt][tt] = float4_t{0, 0, 0, 0};
+
+    // operand slots of this lane for the two blocks of a round (tile 0; a tile is 64 slots)
+    const int ra0 = lds_slot(0, 0, TC, j, c), ra1 = lds_slot(1, 0, TC, j, c);
+    const int rb0 = lds_slot(0, 0, TR, j, c), rb1 = lds_slot(1, 0, TR, j, c);
+    auto multiply_block = [&](int buf, int kbl) {
+        const int ra = buf * XOPS + (kbl ? ra1 : ra0), rb = buf * WOPS + (kbl ? rb1 : rb0);
+        half8_t bop[RT];
+        float   dw[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            bop[rt] = ws[rb + 64 * (wr * RT + rt)];
+            dw[rt]  = POST ? wd[(buf * GL_KC + kbl) * ROWS + wr * (16 * RT) + 16 * rt + c] : 1.0f;
+        }
+#pragma unroll
+        for (int tt = 0; tt < CT; ++tt) {
+            const half8_t aop = xs[ra + 64 * (wt * CT + tt)];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                if constexpr (POST) {
+                    const float4_t blk = mfma16(aop, bop[rt], float4_t{0, 0, 0, 0});
+                    acc[rt][tt] += blk * dw[rt];
+                } else {
+                    acc[rt][tt] = mfma16(aop, bop[rt], acc[rt][tt]);
+                }
+            }
+            if constexpr (POST) __builtin_amdgcn_sched_barrier(0); // keeps the live partial products to one token tile's
+        }
+    };
+
+    load_weights(0);
+    load_acts(0);
+    store_weights(0);
+    store_acts(0);
+    __syncthreads();
+
+    for (int64_t round = 0; round < nround; ++round) {
+        const int buf = (int) (round & 1);
+        const bool more = round + 1 < nround; // uniform
+        if (more) { load_weights(round + 1); load_acts(round + 1); }
+        if constexpr (POST) {
+#pragma unroll 1 // unrolled, the two blocks' operand fetches are hoisted together and the kernel spills
+            for (int kbl = 0; kbl < GL_KC; ++kbl) multiply_block(buf, kbl);
+        } else {
+            multiply_block(buf, 0);
+            multiply_block(buf, 1);
+        }
+        if (more) { store_weights(buf ^ 1); store_acts(buf ^ 1); }
+        __syncthreads();
+    }
+
+    // lane (j,c), tile (rt, tt), register r: token tok0 + 16 (CT wt + tt) + 4j + r, row rowg + 16 (RT wr + rt) + c
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int64_t row = rowg + 16 * (RT * wr + rt) + c;
+        if (row >= a.M) continue;
+#pragma unroll
+        for (int tt = 0; tt < CT; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t tok = tok0 + 16 * (CT * wt + tt) + 4 * j + r;
+                if (tok < a.N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4) = acc[rt][tt][r];
+            }
+    }
+}
+
+template <int WT, bool FOLD, int RT, int CT>
+bool launch_gemm_lds_tile(const mm_args & a, int64_t blocks, int nbatch, hipStream_t st) {
+    constexpr size_t lds = gl_lds(RT, CT);
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        if (hipFuncSetAttribute((const void *) gemm_lds_kernel<WT, FOLD, RT, CT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
+            (void) hipGetLastError();
+            return false;
+        }
+        raised = true;
+    }
+    gemm_lds_kernel<WT, FOLD, RT, CT><<<dim3((unsigned) blocks, 1, (unsigned) nbatch), dim3(256), lds, st>>>(a);
+    return true;
+}
+
+// VX_GEMM_LDS: 0 = off (the register-operand kernels), 1 = block scale applied in fp32 after each MFMA (exact q * d),
+// 2 (default) = scale folded into the f16 weights.
+int gemm_lds_mode() { const char * e = getenv("VX_GEMM_LDS"); return e ? atoi(e) : 2; }
+
+template <int WT>
+bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
+    const int mode = gemm_lds_mode();
+    if (mode == 0 || WT == WT_F32 || a.K % (32 * GL_KC) || a.N < 64 || !a.x_aligned) return false;
+    if (WT == WT_Q8 && !a.w_aligned) return false;
+    if (WT == WT_F16 && (((uintptr_t) a.w | a.nb01 | a.nb02 | a.nb03) % 16 != 0)) return false;
+    // 32-bit lane offsets: rows of the weight matrix, the 128 tokens of a tile
+    if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 128 * a.nb11 + 256 >= (1ull << 32)) return false;
+    const bool fold = WT == WT_Q8 && mode != 1;
+    // 128 x 128 tiles once they fill most of the chip, else 64 x 64
+    const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
+    const int64_t rows = big ? 128 : 64, toks = big ? 128 : 64;
+    const int64_t gx = (a.M + rows - 1) / rows, gy = (a.N + toks - 1) / toks;
+    if (!big && gx * gy * nbatch < 64) return false;
+    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
+    if (blocks > 0x7fffffff) return false;
+    if constexpr (WT == WT_Q8) {
+        if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 4>(a, blocks, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2>(a, blocks, nbatch, st);
+    }
+    return big ? launch_gemm_lds_tile<WT, false, 4, 4>(a, blocks, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2>(a, blocks, nbatch, st);
+}
+
 template <int WT, bool ACT_Q8>
 void launch(const mm_args & a, int nbatch, hipStream_t st) {
     if constexpr (WT != WT_F32) { if (launch_gemv<WT, ACT_Q8>(a, nbatch, st)) return; }
+    if constexpr (WT != WT_F32 && !ACT_Q8) { if (launch_gemm_lds<WT>(a, nbatch, st)) return; }
     if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
