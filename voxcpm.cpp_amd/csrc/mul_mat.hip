@@ -28,6 +28,7 @@
 #include "rope_common.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 
@@ -892,17 +893,20 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
 // fetched 256 contiguous bytes per 16 lanes.  One barrier per round of GL_KC blocks, the global loads of
 // round r+1 in flight during round r's MFMAs.
 constexpr int    GL_KC   = 2;
-// LDS of a work-group that owns 32 RT rows x 32 CT tokens: both operands double-buffered, and the block scales
-constexpr size_t gl_lds(int RT, int CT) { return 2 * GL_KC * (2 * RT + 2 * CT) * 64 * sizeof(half8_t) + 2 * GL_KC * 32 * RT * sizeof(float); }
+// LDS of a work-group that owns 16 TR rows x 16 TC tokens: both operands double-buffered, and the block scales
+constexpr size_t gl_lds(int TR, int TC) { return 2 * GL_KC * (TR + TC) * 64 * sizeof(half8_t) + 2 * GL_KC * 16 * TR * sizeof(float); }
 
 // FOLD: the block scale is multiplied into the f16 weights as they are parked (q * d rounded to f16, relative
 // error 2^-12 on average -- the size of the activations' own rounding) and the MFMAs accumulate across blocks;
 // otherwise the weights stay the exact integers and each 32-wide partial product is scaled in fp32.
-// A wave owns RT x CT MFMA tiles (16 rows x 16 tokens each), the work-group 2 x 2 waves.
-template <int WT, bool FOLD, int RT, int CT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_lds_kernel(const mm_args a) {
+// A wave owns RT x CT MFMA tiles (16 rows x 16 tokens each), the work-group WR x WC waves.
+template <int WT, bool FOLD, int RT, int CT, int WR, int WC>
+__global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT * CT >= 16 ? 2 : 4))) void gemm_lds_kernel(const mm_args a) {
     static_assert(GL_KC == 2, "the parity of a block inside a round is its index in the round");
-    constexpr int  TR = 2 * RT, TC = 2 * CT; // 16-wide tiles per work-group: rows, tokens
+    constexpr int  TR = WR * RT, TC = WC * CT; // 16-wide tiles per work-group: rows, tokens
+    constexpr int  NT = 64 * WR * WC;          // threads
+    constexpr int  WU = 16 * TR * 8 / NT, XU = 16 * TC * 16 / NT; // weight / activation units per thread and round
+    static_assert(WU * NT == 16 * TR * 8 && XU * NT == 16 * TC * 16 && NT % 256 == 0, "units divide evenly over the threads");
     constexpr int  ROWS = 16 * TR, TOKS = 16 * TC;
     constexpr bool POST = WT == WT_Q8 && !FOLD; // scale after the MFMA
     extern __shared__ __align__(16) char gl_smem[];
@@ -913,7 +917,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
-    const int wr = wid >> 1, wt = wid & 1;
+    const int wr = wid / WC, wt = wid % WC;
 
     const int     batch = blockIdx.z;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
@@ -933,44 +937,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
     // products are computed and dropped), so no load carries a predicate.  Addresses are a uniform base
     // plus a 32-bit lane offset that never changes (the launcher checks the ranges).
-    // ---- weight stream: unit = (row, block of the round, group of 8 k), RT per thread and round
+    // ---- weight stream: unit = (row, block of the round, group of 8 k), WU per thread and round
     constexpr int WUNIT = WT == WT_Q8 ? 3 : 4; // dwords fetched per unit
-    uint32_t wraw[RT][WUNIT];
-    uint32_t woff[RT];
+    uint32_t wraw[2][WU][WUNIT]; // two register sets: the rounds after next and next
+    uint32_t woff[WU];
 #pragma unroll
-    for (int it = 0; it < RT; ++it) {
-        const int unit = tid + 256 * it;
+    for (int it = 0; it < WU; ++it) {
+        const int unit = tid + NT * it;
         const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
         const uint64_t rowoff = (uint64_t) min(rowg + row, a.M - 1) * a.nb01;
         if constexpr (WT == WT_Q8) woff[it] = (uint32_t) (rowoff + kbl * VX_Q8_BLOCK + 8 * uj - (kbl ? 2 : 0));
         else                       woff[it] = (uint32_t) (rowoff + kbl * 64 + 16 * uj);
     }
     constexpr int WROUND = GL_KC * (WT == WT_Q8 ? VX_Q8_BLOCK : 64); // bytes of a row walked per round
-    auto load_weights = [&](int64_t round) {
+    auto load_weights = [&](int64_t round, auto SET) {
+        constexpr int S = decltype(SET)::value;
         const char * wk = wb + (uint64_t) round * WROUND; // uniform
 #pragma unroll
-        for (int it = 0; it < RT; ++it) {
+        for (int it = 0; it < WU; ++it) {
             const char * p = (const char *) __builtin_assume_aligned(wk + woff[it], WT == WT_Q8 ? 4 : 16);
-            __builtin_memcpy(wraw[it], p, 4 * WUNIT);
+            __builtin_memcpy(wraw[S][it], p, 4 * WUNIT);
         }
     };
     // where a unit goes in LDS: the same place every round
-    uint32_t wslot[RT];
+    uint32_t wslot[WU];
 #pragma unroll
-    for (int it = 0; it < RT; ++it) {
-        const int unit = tid + 256 * it;
+    for (int it = 0; it < WU; ++it) {
+        const int unit = tid + NT * it;
         wslot[it] = (uint32_t) lds_slot((unit >> 2) & 1, unit >> 7, TR, unit & 3, (unit >> 3) & 15);
     }
-    auto store_weights = [&](int buf) {
+    auto store_weights = [&](int buf, auto SET) {
+        constexpr int S = decltype(SET)::value;
 #pragma unroll
-        for (int it = 0; it < RT; ++it) {
-            const int unit = tid + 256 * it;
+        for (int it = 0; it < WU; ++it) {
+            const int unit = tid + NT * it;
             const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
             half8_t h;
             if constexpr (WT == WT_Q8) {
                 // an even block starts on a dword with its scale in front; the fetch of an odd block starts 2 bytes early
-                h = q8_unpack(q8_raw{wraw[it][0], wraw[it][1], wraw[it][2]}, kbl, true);
-                const uint32_t bits = kbl ? wraw[it][0] >> 16 : wraw[it][0] & 0xffffu; // the scale, in the unit with uj == 0
+                h = q8_unpack(q8_raw{wraw[S][it][0], wraw[S][it][1], wraw[S][it][2]}, kbl, true);
+                const uint32_t bits = kbl ? wraw[S][it][0] >> 16 : wraw[S][it][0] & 0xffffu; // the scale, in the unit with uj == 0
                 if constexpr (FOLD) {
                     // the four units of a block sit in four neighbouring lanes: take the scale from the first
                     const uint32_t b0 = (uint32_t) __builtin_amdgcn_update_dpp(0, (int) bits, 0x00 /* quad_perm 0,0,0,0 */, 0xf, 0xf, true);
@@ -982,36 +988,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                 }
             } else {
                 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                h = __builtin_bit_cast(half8_t, u32x4{wraw[it][0], wraw[it][1], wraw[it][2], wraw[it][3]});
+                h = __builtin_bit_cast(half8_t, u32x4{wraw[S][it][0], wraw[S][it][1], wraw[S][it][2], wraw[S][it][3]});
             }
             ws[buf * WOPS + wslot[it]] = h;
         }
     };
-    // ---- activation stream: unit = (token, 16-byte piece of its 256 bytes of the round), 2 CT per thread and round
-    float4_t xr[2 * CT];
+    // ---- activation stream: unit = (token, 16-byte piece of its 256 bytes of the round), XU per thread and round
+    float4_t xr[2][XU];
     const int xchunk = tid & 15;
-    uint32_t xoff[2 * CT];
+    uint32_t xoff[XU];
 #pragma unroll
-    for (int i = 0; i < 2 * CT; ++i) {
-        const int64_t tok = min(tok0 + (tid >> 4) + 16 * i, a.N - 1);
+    for (int i = 0; i < XU; ++i) {
+        const int64_t tok = min(tok0 + (tid >> 4) + (NT / 16) * i, a.N - 1);
         xoff[i] = (uint32_t) ((uint64_t) (tok - tok0) * a.nb11 + (uint64_t) xchunk * 16);
     }
     const char * xtile = xb + (uint64_t) tok0 * a.nb11;
-    auto load_acts = [&](int64_t round) {
+    auto load_acts = [&](int64_t round, auto SET) {
+        constexpr int S = decltype(SET)::value;
         const char * base = xtile + (uint64_t) round * (GL_KC * 128); // uniform
 #pragma unroll
-        for (int i = 0; i < 2 * CT; ++i) xr[i] = *(const float4_t *) (base + xoff[i]);
+        for (int i = 0; i < XU; ++i) xr[S][i] = *(const float4_t *) (base + xoff[i]);
     };
-    // byte offset of token (tid >> 4)'s piece in LDS; token + 16 i is the next 16-token tile, 64 slots on
-    const uint32_t xslot = (uint32_t) lds_slot(xchunk >> 3, 0, TC, (xchunk & 7) >> 1, tid >> 4) * 16 + 8 * (xchunk & 1);
-    auto store_acts = [&](int buf) {
+    // byte offset of token (tid >> 4)'s piece in LDS; unit i is NT / 16 tokens = NT / 256 tiles of 64 slots further on
+    const uint32_t xslot = (uint32_t) lds_slot(xchunk >> 3, tid >> 8, TC, (xchunk & 7) >> 1, (tid >> 4) & 15) * 16 + 8 * (xchunk & 1);
+    auto store_acts = [&](int buf, auto SET) {
+        constexpr int S = decltype(SET)::value;
         typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int i = 0; i < 2 * CT; ++i) {
+        for (int i = 0; i < XU; ++i) {
             half4_t h;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = (_Float16) xr[i][e];
-            *(half4_t *) ((char *) (xs + buf * XOPS + 64 * i) + xslot) = h;
+            for (int e = 0; e < 4; ++e) h[e] = (_Float16) xr[S][i][e];
+            *(half4_t *) ((char *) (xs + buf * XOPS + 64 * (NT / 256) * i) + xslot) = h;
         }
     };
 
@@ -1049,16 +1057,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
     };
 
-    load_weights(0);
-    load_acts(0);
-    store_weights(0);
-    store_acts(0);
+    // Round r's operands are in LDS buffer r & 1 while round r+1 waits in register set (r+1) & 1 and round
+    // r+2 is being fetched into set r & 1: a fetch has a whole round (MFMAs, conversion, barrier) and the next
+    // round's MFMAs to arrive before it is converted.
+    using set0 = std::integral_constant<int, 0>;
+    using set1 = std::integral_constant<int, 1>;
+    load_weights(0, set0{});
+    load_acts(0, set0{});
+    if (nround > 1) { load_weights(1, set1{}); load_acts(1, set1{}); }
+    store_weights(0, set0{});
+    store_acts(0, set0{});
     __syncthreads();
 
-    for (int64_t round = 0; round < nround; ++round) {
-        const int buf = (int) (round & 1);
-        const bool more = round + 1 < nround; // uniform
-        if (more) { load_weights(round + 1); load_acts(round + 1); }
+    auto one_round = [&](int64_t round, auto SET) { // SET = round & 1
+        using other = std::integral_constant<int, 1 - decltype(SET)::value>;
+        const int buf = decltype(SET)::value;
+        if (round + 2 < nround) { load_weights(round + 2, SET); load_acts(round + 2, SET); }
         if constexpr (POST) {
 #pragma unroll 1 // unrolled, the two blocks' operand fetches are hoisted together and the kernel spills
             for (int kbl = 0; kbl < GL_KC; ++kbl) multiply_block(buf, kbl);
@@ -1066,11 +1080,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
             multiply_block(buf, 0);
             multiply_block(buf, 1);
         }
-        if (more) { store_weights(buf ^ 1); store_acts(buf ^ 1); }
+        if (round + 1 < nround) { store_weights(buf ^ 1, other{}); store_acts(buf ^ 1, other{}); }
         __syncthreads();
+    };
+    for (int64_t round = 0; round < nround; round += 2) {
+        one_round(round, set0{});
+        if (round + 1 < nround) one_round(round + 1, set1{});
     }
 
     // lane (j,c), tile (rt, tt), register r: token tok0 + 16 (CT wt + tt) + 4j + r, row rowg + 16 (RT wr + rt) + c
+    if (tok0 + TOKS <= a.N && rowg + ROWS <= a.M) { // uniform: a tile inside the matrix stores without tests,
+        // at a uniform base plus one 32-bit lane offset (the launcher checks the range)
+        char * tb = db + (uint64_t) tok0 * a.nb1 + (uint64_t) rowg * 4;
+        const uint32_t loff = (uint32_t) ((uint64_t) (16 * CT * wt + 4 * j) * a.nb1 + (uint64_t) (16 * RT * wr + c) * 4);
+#pragma unroll
+        for (int tt = 0; tt < CT; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                char * tr = tb + (uint64_t) (16 * tt + r) * a.nb1; // uniform
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) *(float *) (tr + 64 * rt + loff) = acc[rt][tt][r];
+            }
+        return;
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int64_t row = rowg + 16 * (RT * wr + rt) + c;
@@ -1085,18 +1117,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
 }
 
-template <int WT, bool FOLD, int RT, int CT>
-bool launch_gemm_lds_tile(const mm_args & a, int64_t blocks, int nbatch, hipStream_t st) {
-    constexpr size_t lds = gl_lds(RT, CT);
+template <int WT, bool FOLD, int RT, int CT, int WR, int WC>
+bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
+    constexpr size_t lds = gl_lds(RT * WR, CT * WC);
+    const int64_t gx = (a.M + 16 * RT * WR - 1) / (16 * RT * WR), gy = (a.N + 16 * CT * WC - 1) / (16 * CT * WC);
+    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
+    if (blocks > 0x7fffffff) return false;
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
-        if (hipFuncSetAttribute((const void *) gemm_lds_kernel<WT, FOLD, RT, CT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
+        if (hipFuncSetAttribute((const void *) gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
             (void) hipGetLastError();
             return false;
         }
         raised = true;
     }
-    gemm_lds_kernel<WT, FOLD, RT, CT><<<dim3((unsigned) blocks, 1, (unsigned) nbatch), dim3(256), lds, st>>>(a);
+    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC><<<dim3((unsigned) blocks, 1, (unsigned) nbatch), dim3(64 * WR * WC), lds, st>>>(a);
     return true;
 }
 
@@ -1110,20 +1145,29 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     if (mode == 0 || WT == WT_F32 || a.K % (32 * GL_KC) || a.N < 64 || !a.x_aligned) return false;
     if (WT == WT_Q8 && !a.w_aligned) return false;
     if (WT == WT_F16 && (((uintptr_t) a.w | a.nb01 | a.nb02 | a.nb03) % 16 != 0)) return false;
-    // 32-bit lane offsets: rows of the weight matrix, the 128 tokens of a tile
-    if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 128 * a.nb11 + 256 >= (1ull << 32)) return false;
+    // 32-bit lane offsets: rows of the weight matrix, the (up to 256) tokens of a tile
+    if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 256 * a.nb11 + 256 >= (1ull << 32) ||
+        (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32)) return false;
     const bool fold = WT == WT_Q8 && mode != 1;
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
-    const int64_t rows = big ? 128 : 64, toks = big ? 128 : 64;
-    const int64_t gx = (a.M + rows - 1) / rows, gy = (a.N + toks - 1) / toks;
-    if (!big && gx * gy * nbatch < 64) return false;
-    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
-    if (blocks > 0x7fffffff) return false;
-    if constexpr (WT == WT_Q8) {
-        if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 4>(a, blocks, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2>(a, blocks, nbatch, st);
-    }
-    return big ? launch_gemm_lds_tile<WT, false, 4, 4>(a, blocks, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2>(a, blocks, nbatch, st);
+    if (!big && ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch < 64) return false;
+    static const int shape = [] { const char * e = getenv("VX_GEMM_SHAPE"); return e ? atoi(e) : 0; }();
+#define VX_GL(FOLD_)                                                                                                   \
+    do {                                                                                                               \
+        if (!big && shape == 5) return launch_gemm_lds_tile<WT, FOLD_, 2, 1, 2, 2>(a, nbatch, st);                     \
+        if (!big && shape == 6) return launch_gemm_lds_tile<WT, FOLD_, 1, 2, 2, 2>(a, nbatch, st);                     \
+        if (!big && shape == 7) return launch_gemm_lds_tile<WT, FOLD_, 1, 1, 2, 2>(a, nbatch, st);                     \
+        if (!big) return launch_gemm_lds_tile<WT, FOLD_, 2, 2, 2, 2>(a, nbatch, st);                                   \
+        if (shape == 1) return launch_gemm_lds_tile<WT, FOLD_, 4, 2, 2, 4>(a, nbatch, st);                             \
+        if (shape == 2) return launch_gemm_lds_tile<WT, FOLD_, 2, 4, 4, 2>(a, nbatch, st);                             \
+        if (shape == 3) return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 4, 2>(a, nbatch, st);                             \
+        if (shape == 4) return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 2, 4>(a, nbatch, st);                             \
+        return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 2, 2>(a, nbatch, st);                                             \
+    } while (0)
+    if constexpr (WT == WT_Q8) { if (fold) VX_GL(true); }
+    VX_GL(false);
+#undef VX_GL
 }
 
 template <int WT, bool ACT_Q8>
