@@ -114,7 +114,9 @@ VX_API vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k, con
  * src0 broadcast over dims 2,3.  src0 Q8_0 | F16 | F32 (rows dense), src1 F32, dst F32
  * contiguous.
  * act_mode selects how src1 enters the product for Q8_0 weights:
- *   VX_ACT_FLOAT -- weights dequantised in registers (q*d exactly), activations as f16/f32
+ *   VX_ACT_FLOAT -- weights dequantised on the fly (q*d exactly; with the environment variable
+ *                   VX_GEMM_LDS=2 the tiled kernel for >= 64 tokens rounds q*d once to f16 instead),
+ *                   activations as f16/f32
  *   VX_ACT_Q8    -- activations quantised to Q8_0 blocks first, integer block dots scaled
  *                   by d_w*d_x: the arithmetic ggml-cpu performs
  *                   (ggml/src/ggml-cpu/arch/x86/quants.c:290-386, 1012-1078). */

@@ -445,8 +445,8 @@ def test_q8_0_dequant_is_exact(gpu):
 @pytest.mark.parametrize("M", [512, 2048])
 def test_q8_0_dequant_on_the_tiled_gemm(gpu, M, monkeypatch):
     """The same unit-vector probe at shapes that run on the LDS-tiled GEMM (64 x 64 and 128 x 128 tiles).  With
-    VX_GEMM_LDS=1 the block scale is applied in fp32 and the product is the dequantised weight bit for bit; by
-    default the scale is folded into the f16 operand, i.e. the weight is q * d rounded once to f16."""
+    the default (VX_GEMM_LDS=1) the block scale is applied in fp32 and the product is the dequantised weight bit for
+    bit; with VX_GEMM_LDS=2 the scale is folded into the f16 operand, i.e. the weight is q * d rounded once to f16."""
     import ctypes as C
     K = 1536
     say(f"Q8_0 dequantisation on the tiled GEMM, M={M}: exact scale mode, folded scale mode")
@@ -456,6 +456,9 @@ def test_q8_0_dequant_on_the_tiled_gemm(gpu, M, monkeypatch):
     deq = np.zeros((M, K), np.float32)
     reflib.load_oracle().orc_dequantize_row_q8_0(wq.ctypes.data, reflib.ptr(deq, C.c_float), M * K)
     eye = np.eye(K, dtype=np.float32)
+    monkeypatch.delenv("VX_GEMM_LDS", raising=False)
+    got = sync_np(gpu.mul_mat(dev(wq), dev(eye), gpu.ACT_FLOAT, w_ne0=K))
+    assert np.array_equal(got.T, deq)
     monkeypatch.setenv("VX_GEMM_LDS", "1")
     got = sync_np(gpu.mul_mat(dev(wq), dev(eye), gpu.ACT_FLOAT, w_ne0=K))
     assert np.array_equal(got.T, deq)

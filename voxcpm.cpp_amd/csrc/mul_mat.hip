@@ -906,7 +906,7 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     constexpr int  TR = WR * RT, TC = WC * CT; // 16-wide tiles per work-group: rows, tokens
     constexpr int  NT = 64 * WR * WC;          // threads
     constexpr int  WU = 16 * TR * 8 / NT, XU = 16 * TC * 16 / NT; // weight / activation units per thread and round
-    static_assert(WU * NT == 16 * TR * 8 && XU * NT == 16 * TC * 16 && NT % 256 == 0, "units divide evenly over the threads");
+    static_assert(WU * NT == 16 * TR * 8 && XU * NT == 16 * TC * 16 && NT % 256 == 0 && WU % 2 == 0, "units divide evenly over the threads");
     constexpr int  ROWS = 16 * TR, TOKS = 16 * TC;
     constexpr bool POST = WT == WT_Q8 && !FOLD; // scale after the MFMA
     extern __shared__ __align__(16) char gl_smem[];
@@ -935,43 +935,48 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     const int64_t nround = a.K / (32 * GL_KC); // the launcher takes whole rounds only
 
     // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
-    // products are computed and dropped), so no load carries a predicate.  Addresses are a uniform base
-    // plus a 32-bit lane offset that never changes (the launcher checks the ranges).
-    // ---- weight stream: unit = (row, block of the round, group of 8 k), WU per thread and round
+    // products are computed and dropped), so no load carries a predicate.  They are buffer loads: a uniform
+    // base in a resource descriptor, a 32-bit lane offset that never changes and a scalar offset per round
+    // (the launcher checks the ranges), so a load costs no address arithmetic.
+    const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void *) wb, 0, -1, 0x00020000);
+    // ---- weight stream: unit = (row, block of the round, group of 8 k), WU per thread and round.  Unit `it` of a
+    // thread belongs to block it & 1, so a block's parity -- where its quants sit in the dwords -- is known at compile time.
     constexpr int WUNIT = WT == WT_Q8 ? 3 : 4; // dwords fetched per unit
     uint32_t wraw[2][WU][WUNIT]; // two register sets: the rounds after next and next
-    uint32_t woff[WU];
+    uint32_t woff[WU / 2];       // block 0 of the pair; block 1 is 32 bytes on (Q8_0: 34 - 2) or 64 (F16)
+    uint32_t wslot[WU];          // where a unit goes in LDS: the same place every round
 #pragma unroll
     for (int it = 0; it < WU; ++it) {
-        const int unit = tid + NT * it;
-        const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
+        const int idx = tid + NT * (it >> 1), kbl = it & 1;
+        const int row = idx >> 2, uj = idx & 3;
         const uint64_t rowoff = (uint64_t) min(rowg + row, a.M - 1) * a.nb01;
-        if constexpr (WT == WT_Q8) woff[it] = (uint32_t) (rowoff + kbl * VX_Q8_BLOCK + 8 * uj - (kbl ? 2 : 0));
-        else                       woff[it] = (uint32_t) (rowoff + kbl * 64 + 16 * uj);
+        if (kbl == 0) woff[it >> 1] = (uint32_t) (rowoff + (WT == WT_Q8 ? 8 : 16) * uj);
+        wslot[it] = (uint32_t) lds_slot(kbl, row >> 4, TR, uj, row & 15);
     }
     constexpr int WROUND = GL_KC * (WT == WT_Q8 ? VX_Q8_BLOCK : 64); // bytes of a row walked per round
     auto load_weights = [&](int64_t round, auto SET) {
         constexpr int S = decltype(SET)::value;
-        const char * wk = wb + (uint64_t) round * WROUND; // uniform
+        const int so = (int) (round * WROUND); // uniform
 #pragma unroll
         for (int it = 0; it < WU; ++it) {
-            const char * p = (const char *) __builtin_assume_aligned(wk + woff[it], WT == WT_Q8 ? 4 : 16);
-            __builtin_memcpy(wraw[S][it], p, 4 * WUNIT);
+            const uint32_t vo = woff[it >> 1] + (it & 1) * (WT == WT_Q8 ? 32 : 64);
+            if constexpr (WT == WT_Q8) {
+                typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+                const u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(wres, (int) vo, so, 0);
+                wraw[S][it][0] = v[0]; wraw[S][it][1] = v[1]; wraw[S][it][2] = v[2];
+            } else {
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(wres, (int) vo, so, 0);
+                wraw[S][it][0] = v[0]; wraw[S][it][1] = v[1]; wraw[S][it][2] = v[2]; wraw[S][it][3] = v[3];
+            }
         }
     };
-    // where a unit goes in LDS: the same place every round
-    uint32_t wslot[WU];
-#pragma unroll
-    for (int it = 0; it < WU; ++it) {
-        const int unit = tid + NT * it;
-        wslot[it] = (uint32_t) lds_slot((unit >> 2) & 1, unit >> 7, TR, unit & 3, (unit >> 3) & 15);
-    }
     auto store_weights = [&](int buf, auto SET) {
         constexpr int S = decltype(SET)::value;
 #pragma unroll
         for (int it = 0; it < WU; ++it) {
-            const int unit = tid + NT * it;
-            const int row = unit >> 3, kbl = (unit >> 2) & 1, uj = unit & 3;
+            const int idx = tid + NT * (it >> 1), kbl = it & 1;
+            const int row = idx >> 2, uj = idx & 3;
             half8_t h;
             if constexpr (WT == WT_Q8) {
                 // an even block starts on a dword with its scale in front; the fetch of an odd block starts 2 bytes early
@@ -1002,12 +1007,15 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
         const int64_t tok = min(tok0 + (tid >> 4) + (NT / 16) * i, a.N - 1);
         xoff[i] = (uint32_t) ((uint64_t) (tok - tok0) * a.nb11 + (uint64_t) xchunk * 16);
     }
-    const char * xtile = xb + (uint64_t) tok0 * a.nb11;
+    const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void *) (xb + (uint64_t) tok0 * a.nb11), 0, -1, 0x00020000);
     auto load_acts = [&](int64_t round, auto SET) {
         constexpr int S = decltype(SET)::value;
-        const char * base = xtile + (uint64_t) round * (GL_KC * 128); // uniform
+        const int so = (int) (round * (GL_KC * 128)); // uniform
 #pragma unroll
-        for (int i = 0; i < XU; ++i) xr[S][i] = *(const float4_t *) (base + xoff[i]);
+        for (int i = 0; i < XU; ++i) {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            xr[S][i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(xres, (int) xoff[i], so, 0));
+        }
     };
     // byte offset of token (tid >> 4)'s piece in LDS; unit i is NT / 16 tokens = NT / 256 tiles of 64 slots further on
     const uint32_t xslot = (uint32_t) lds_slot(xchunk >> 3, tid >> 8, TC, (xchunk & 7) >> 1, (tid >> 4) & 15) * 16 + 8 * (xchunk & 1);
@@ -1135,9 +1143,10 @@ bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
     return true;
 }
 
-// VX_GEMM_LDS: 0 = off (the register-operand kernels), 1 = block scale applied in fp32 after each MFMA (exact q * d),
-// 2 (default) = scale folded into the f16 weights.
-int gemm_lds_mode() { const char * e = getenv("VX_GEMM_LDS"); return e ? atoi(e) : 2; }
+// VX_GEMM_LDS: 0 = off (the register-operand kernels), 1 (default) = block scale applied in fp32 after each MFMA, so
+// that a weight enters the sum as exactly q * d; 2 = scale folded into the f16 weights (q * d rounded once to f16,
+// 10-22 % faster).  Read on every call: a product of this size takes tens of microseconds.
+int gemm_lds_mode() { const char * e = getenv("VX_GEMM_LDS"); return e ? atoi(e) : 1; }
 
 template <int WT>
 bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
@@ -1147,27 +1156,17 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     if (WT == WT_F16 && (((uintptr_t) a.w | a.nb01 | a.nb02 | a.nb03) % 16 != 0)) return false;
     // 32-bit lane offsets: rows of the weight matrix, the (up to 256) tokens of a tile
     if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 256 * a.nb11 + 256 >= (1ull << 32) ||
-        (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32)) return false;
-    const bool fold = WT == WT_Q8 && mode != 1;
+        (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32) || a.K >= (1ll << 28)) return false;
+    const bool fold = WT == WT_Q8 && mode == 2;
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     if (!big && ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch < 64) return false;
-    static const int shape = [] { const char * e = getenv("VX_GEMM_SHAPE"); return e ? atoi(e) : 0; }();
-#define VX_GL(FOLD_)                                                                                                   \
-    do {                                                                                                               \
-        if (!big && shape == 5) return launch_gemm_lds_tile<WT, FOLD_, 2, 1, 2, 2>(a, nbatch, st);                     \
-        if (!big && shape == 6) return launch_gemm_lds_tile<WT, FOLD_, 1, 2, 2, 2>(a, nbatch, st);                     \
-        if (!big && shape == 7) return launch_gemm_lds_tile<WT, FOLD_, 1, 1, 2, 2>(a, nbatch, st);                     \
-        if (!big) return launch_gemm_lds_tile<WT, FOLD_, 2, 2, 2, 2>(a, nbatch, st);                                   \
-        if (shape == 1) return launch_gemm_lds_tile<WT, FOLD_, 4, 2, 2, 4>(a, nbatch, st);                             \
-        if (shape == 2) return launch_gemm_lds_tile<WT, FOLD_, 2, 4, 4, 2>(a, nbatch, st);                             \
-        if (shape == 3) return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 4, 2>(a, nbatch, st);                             \
-        if (shape == 4) return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 2, 4>(a, nbatch, st);                             \
-        return launch_gemm_lds_tile<WT, FOLD_, 4, 4, 2, 2>(a, nbatch, st);                                             \
-    } while (0)
-    if constexpr (WT == WT_Q8) { if (fold) VX_GL(true); }
-    VX_GL(false);
-#undef VX_GL
+    // 128 x 128: 8 waves of 64 rows x 32 tokens (4 waves per SIMD with two work-groups per CU measured 5-10 % above
+    // 4 waves of 64 x 64); 64 x 64: 4 waves of 32 x 32
+    if constexpr (WT == WT_Q8) {
+        if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2>(a, nbatch, st);
+    }
+    return big ? launch_gemm_lds_tile<WT, false, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(a, nbatch, st);
 }
 
 template <int WT, bool ACT_Q8>
