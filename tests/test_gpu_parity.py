@@ -336,6 +336,20 @@ def test_fa_full_size_invariants(gpu):
     torch.cuda.synchronize()
 
 
+def test_fa_prefill_kernel_on_request_for_f32_kv(gpu, monkeypatch):
+    """F32 K/V take the hi/lo wave kernel by default (error ~1e-6); with VX_FA_F32_PREFILL=1 they are rounded to
+    f16 into the LDS-tiled kernel, which must then hold the same 2e-3 bar as an f16 cache does."""
+    say("flash_attn prefill kernel, F32 K/V: default route, then the f16-staging route on request")
+    B, Hq, Hkv, T = 2, 16, 2, 1024
+    q, k, v = qkv(("pf32", T), B, Hq, Hkv, T, T, kv_dtype=np.float32)
+    mask = reflib.causal_mask(T, T)
+    monkeypatch.delenv("VX_FA_F32_PREFILL", raising=False)
+    fa_case(gpu, q, k, v, mask, tol=2e-5, name="F32 K/V, default")
+    monkeypatch.setenv("VX_FA_F32_PREFILL", "1")
+    got, want = fa_case(gpu, q, k, v, mask, name="F32 K/V, f16 staging")
+    assert np.abs(got - want).max() > 2e-5       # it did take the other kernel
+
+
 @pytest.mark.parametrize("case", ["causal", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
 def test_fa_prefill_kernel(gpu, case):
     """Shapes large enough to take the LDS-tiled prefill kernel (>= 256 columns per KV head,
