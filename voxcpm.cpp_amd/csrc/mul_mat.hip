@@ -348,20 +348,40 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // them carries rows of W, the second half the same rows of W2, and the epilogue pairs them up.
     const bool    dual = a.w2 != nullptr;                 // uniform
     const int     R  = a.rows_wg, Rr = dual ? R / 2 : R;   // MFMA columns in use, output rows per work-group
-    const int     cr = dual ? c % Rr : c;
-    // the weight row of MFMA column c.  Plain: consecutive rows.  With the rotation the R columns hold R/2
+    // the weight row of MFMA column cc.  Plain: consecutive rows.  With the rotation the R columns hold R/2
     // pairs (d, d + head_dim/2) of one head, first elements in columns 0 .. R/2-1, partners in the rest.
-    int64_t       row = (int64_t) wl * Rr + cr;
     const int     h2 = R >> 1, half_dim = a.head_dim >> 1;
-    int           pair = 0; // index of the pair within its head: the rotation's frequency index
-    if (SEG && rope) {
-        const int64_t f = (int64_t) wl * h2 + (c & (h2 - 1));
-        pair = (int) (f % half_dim);
-        row  = (f / half_dim) * a.head_dim + pair + (c >= h2 ? half_dim : 0);
-    }
-    const bool    row_ok = c < R && row < M;
-    const char *  wsel = (dual && c >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
-    const char *  wrow = wsel + (uint64_t) min(row, M - 1) * nb01;
+    auto column = [&](int cc, int64_t & row_, int & pair_, bool & ok_, const char *& wrow_) {
+        const int cr = dual ? cc % Rr : cc;
+        row_  = (int64_t) wl * Rr + cr;
+        pair_ = 0; // index of the pair within its head: the rotation's frequency index
+        if (SEG && rope) {
+            const int64_t f = (int64_t) wl * h2 + (cc & (h2 - 1));
+            pair_ = (int) (f % half_dim);
+            row_  = (f / half_dim) * a.head_dim + pair_ + (cc >= h2 ? half_dim : 0);
+        }
+        ok_ = cc < R && row_ < M;
+        const char * wsel = (dual && cc >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
+        wrow_ = wsel + (uint64_t) min(row_, M - 1) * nb01;
+    };
+    int64_t       row;
+    int           pair;
+    bool          row_ok;
+    const char *  wrow;
+    column(c, row, pair, row_ok, wrow);
+    // Fetching in MFMA layout -- lane (j,c) = chunk j of row c -- makes every 16-lane group of a load touch 16 rows,
+    // 16 cache lines for 12 useful bytes each, and the CU's vector cache serves one line per cycle.  With dword-aligned
+    // Q8_0 rows the fetch is therefore done in row-major lane order (lane l = chunk l & 3 of column l >> 2: four rows
+    // per 16 lanes) and the dwords are handed to their MFMA lanes by a cross-lane permute once they have arrived;
+    // the block scale rides in the first dword of chunk 0, so it needs no load of its own.
+    constexpr bool PERM = WT == WT_Q8 && AL4;
+    int64_t       row_ld;
+    int           pair_ld;
+    bool          ld_ok = row_ok;
+    const char *  wrow_ld = wrow;
+    if constexpr (PERM) column(lane >> 2, row_ld, pair_ld, ld_ok, wrow_ld);
+    const int     j_ld = PERM ? (lane & 3) : j;
+    const int     perm_src = (4 * c + j) * 4, perm_src0 = (4 * c) * 4; // byte addresses of the source lanes
     const int     N = min(16, (int) a.N - tok0); // tokens of this chunk
     db += (uint64_t) tok0 * nb1;
 
@@ -374,12 +394,11 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
 #pragma unroll
         for (int u = 0; u < GV_UNROLL; ++u) {
             const int64_t kb = min((int64_t) wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, result unused
-            if (!row_ok) {
+            if (!ld_ok) {
                 wq[u] = q8_raw{0, 0, 0}; wdv[u] = (_Float16) 0.0f; wh[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
             } else if constexpr (WT == WT_Q8) {
-                const char * bp = wrow + (uint64_t) kb * VX_Q8_BLOCK;
-                wdv[u] = *(const _Float16 *) bp;
-                wq[u]  = q8_load(wrow, kb, j, al4);
+                if constexpr (!PERM) wdv[u] = *(const _Float16 *) (wrow_ld + (uint64_t) kb * VX_Q8_BLOCK);
+                wq[u] = q8_load(wrow_ld, kb, j_ld, al4);
             } else {
                 __builtin_memcpy(&wh[u], wrow + (uint64_t) (kb * 32 + 8 * j) * 2, 16);
             }
@@ -508,9 +527,20 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             half8_t aop = {0, 0, 0, 0, 0, 0, 0, 0};
             if (c < N) aop = *(const half8_t *) (xs + (size_t) c * a.K + kb * 32 + 8 * j);
             if constexpr (WT == WT_Q8) {
-                const half8_t  bop = q8_unpack(wq[u], kb, al4);
+                q8_raw raw = wq[u];
+                float  dw;
+                if constexpr (PERM) {
+                    const uint32_t first = (uint32_t) __builtin_amdgcn_ds_bpermute(perm_src0, (int) raw.w0); // chunk 0 of this lane's row
+                    raw.w0 = (uint32_t) __builtin_amdgcn_ds_bpermute(perm_src, (int) raw.w0);
+                    raw.w1 = (uint32_t) __builtin_amdgcn_ds_bpermute(perm_src, (int) raw.w1);
+                    raw.w2 = (uint32_t) __builtin_amdgcn_ds_bpermute(perm_src, (int) raw.w2);
+                    // an even block starts on a dword with its scale in front; the fetch of an odd block starts 2 bytes early
+                    dw = (float) __builtin_bit_cast(_Float16, (uint16_t) ((kb & 1) ? first >> 16 : first & 0xffffu));
+                } else {
+                    dw = (float) wdv[u];
+                }
+                const half8_t  bop = q8_unpack(raw, kb, al4);
                 const float4_t blk = mfma16(aop, bop, float4_t{0, 0, 0, 0});
-                const float    dw  = (float) wdv[u];
                 if constexpr (ACT_Q8) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc[r] += blk[r] * (dw * (4 * j + r < N ? xd[(4 * j + r) * nkb + kb] : 0.0f));
@@ -1013,7 +1043,6 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
         const int so = (int) (round * (GL_KC * 128)); // uniform
 #pragma unroll
         for (int i = 0; i < XU; ++i) {
-            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
             xr[S][i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(xres, (int) xoff[i], so, 0));
         }
     };
