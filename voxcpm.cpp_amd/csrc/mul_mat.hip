@@ -915,13 +915,12 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
 }
 
 // ---- GEMM shape, both operands through LDS -----------------------------------------------------------
-// Same 128 x 128 tile and 2 x 2 waves as above.  Fetching the weights straight into the MFMA layout makes every
-// 16-lane group of a load touch 16 different rows, i.e. 16 cache lines for 12 useful bytes each, and the
-// per-CU cache that serves one line per cycle becomes the limit of the whole kernel.  Here a thread fetches
-// (row, block, 8-quant group) units in row-major order, so that 16 lanes cover two 68-byte runs, turns its
-// quants into f16 once for the work-group, and parks them in LDS in the operand layout; activations are
-// fetched 256 contiguous bytes per 16 lanes.  One barrier per round of GL_KC blocks, the global loads of
-// round r+1 in flight during round r's MFMAs.
+// Fetching the weights straight into the MFMA layout, as the kernels above do, makes every 16-lane group of a
+// load touch 16 different rows, i.e. 16 cache lines for 12 useful bytes each, and the per-CU vector cache, which
+// serves about one line per cycle, becomes the limit of the whole kernel.  Here a thread fetches (row, block,
+// 8-quant group) units in row-major lane order, so that 16 lanes cover four 32-byte runs, turns its quants into
+// f16 once for the work-group, and parks them in LDS in the operand layout; activations are fetched 256
+// contiguous bytes per 16 lanes.  One barrier per round of GL_KC blocks; the global loads run two rounds ahead.
 constexpr int    GL_KC   = 2;
 // LDS of a work-group that owns 16 TR rows x 16 TC tokens: both operands double-buffered, and the block scales
 constexpr size_t gl_lds(int TR, int TC) { return 2 * GL_KC * (TR + TC) * 64 * sizeof(half8_t) + 2 * GL_KC * 16 * TR * sizeof(float); }
