@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void mm_splitk_reduce_kernel(const mm_args a) 
 // in one round trip to HBM.
 constexpr int GV_UNROLL = 8;
 
-template <int WT, bool ACT_Q8, int NW, bool AL4, bool SEG>
+template <int WT, bool ACT_Q8, int NW, bool AL4, bool SEG, int UNR = GV_UNROLL>
 __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
     const int64_t nkb = a.K / 32;
@@ -387,12 +387,12 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
 
     // ---- this wave's weight blocks: kb = wid + NW * i
     constexpr bool al4 = AL4;
-    q8_raw   wq[GV_UNROLL];
-    half8_t  wh[GV_UNROLL];
-    _Float16 wdv[GV_UNROLL];
+    q8_raw   wq[UNR];
+    half8_t  wh[UNR];
+    _Float16 wdv[UNR];
     auto load_blocks = [&](int64_t i0) {
 #pragma unroll
-        for (int u = 0; u < GV_UNROLL; ++u) {
+        for (int u = 0; u < UNR; ++u) {
             const int64_t kb = min((int64_t) wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, result unused
             if (!ld_ok) {
                 wq[u] = q8_raw{0, 0, 0}; wdv[u] = (_Float16) 0.0f; wh[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
@@ -518,10 +518,10 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
 
     float4_t acc = {0, 0, 0, 0};
     const int64_t per = (nkb + NW - 1) / NW; // blocks per wave
-    for (int64_t i0 = 0; i0 < per; i0 += GV_UNROLL) {
+    for (int64_t i0 = 0; i0 < per; i0 += UNR) {
         if (i0) load_blocks(i0);
 #pragma unroll
-        for (int u = 0; u < GV_UNROLL; ++u) {
+        for (int u = 0; u < UNR; ++u) {
             const int64_t kb = (int64_t) wid + NW * (i0 + u);
             if (kb >= nkb) break; // wave-uniform
             half8_t aop = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -611,7 +611,9 @@ size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
            (a.nseg > 0 ? GV_ROPE_LDS : 0);
 }
 
-// waves per work-group for a matrix of M rows: about GV_UNROLL blocks per wave, so every load is issued up front.  More
+// waves per work-group for a matrix of M rows: about 4 blocks per wave for one chunk of tokens (K = 1024: 8 waves; measured
+// against 8 blocks per wave: decode step 1.03 -> 0.96 ms), 8 when chunks of 16 tokens multiply the work-groups; either way
+// every load is issued up front.  More
 // than a handful of tokens: the activations' work (staging, a fused RMS_NORM's wave-per-token sums in fp64, the rotation's
 // angles) outweighs the K walk and a matrix of few rows spreads it over 16 waves (norm + q/k/v + rope at 14 tokens: 12.8 ->
 // 9.8 us); a tall matrix already fills the CUs with work-groups and is slower with more waves (4096 x 2 rows: 9.3 -> 13.5 us
@@ -620,7 +622,8 @@ size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
 int gemv_waves_for(int64_t K, int64_t tokens, int64_t M) {
     const int64_t nkb = K / 32;
     int nw = 1;
-    while (nw < 16 && nkb > (int64_t) nw * GV_UNROLL) nw *= 2;
+    const int bpw = tokens <= 16 ? 4 : GV_UNROLL; // blocks per wave aimed at
+    while (nw < 16 && nkb > (int64_t) nw * bpw) nw *= 2;
     static const int many = [] { const char * e = getenv("VX_GEMV_MANY_TOKENS"); return e ? atoi(e) : 5; }();
     if (tokens >= many && tokens <= 16 && nkb >= 16 && M <= 2048) nw = 16; // one chunk of tokens; several chunks multiply the waves instead
     return nw;
@@ -681,13 +684,17 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
 #define VX_GEMV(NW_)                                                                                                   \
     do {                                                                                                               \
         if (a.nseg > 0) {                                                                                              \
-            if (WT == WT_Q8 && a.w_aligned) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, true>);                      \
+            if (WT == WT_Q8 && a.w_aligned && few) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, true, 4>);            \
+            else if (WT == WT_Q8 && a.w_aligned)   VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, true>);               \
             else                            VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, false, true>);                     \
         } else {                                                                                                       \
-            if (WT == WT_Q8 && a.w_aligned) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, false>);                     \
+            if (WT == WT_Q8 && a.w_aligned && few) VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, false, 4>);           \
+            else if (WT == WT_Q8 && a.w_aligned)   VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, true, false>);              \
             else                            VX_GEMV_GO(gemv_kernel<WT, ACT_Q8, NW_, false, false>);                    \
         }                                                                                                              \
     } while (0)
+    // a wave with at most four blocks requests four: the loads past a wave's last block are clamped re-reads of it
+    const bool few = (a.K / 32 + nw - 1) / nw <= 4;
     switch (nw) {
         case 1:  VX_GEMV(1); break;
         case 2:  VX_GEMV(2); break;
