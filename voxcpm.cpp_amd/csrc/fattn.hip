@@ -471,9 +471,12 @@ bool aligned16(const vx_tensor * t) {
 
 // Work split.  Enough 16-column tiles to fill the chip: one wave per tile over all keys.
 // Otherwise cut the keys (flash-decoding) aiming at ~4 waves per CU, at least `min_chunk`
-// keys per wave, and merge the partials with a second small kernel.
+// keys per wave and at most `cap` ranges, and merge the partials with a second small kernel.
+// One 32-key step per wave is the fastest cut of a short cache (640 keys: 20 ranges, decode step
+// 0.96 -> 0.92 ms against 64-key ranges); beyond 64 ranges the merge costs more than the cut saves
+// (4096 keys in 128 ranges: 14.6 us against 8.2 us in 64).
 void fa_split_plan(int64_t tiles, int n_kv, int * n_splits, int * chunk_out) {
-    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 64; }();
+    static const int min_chunk = [] { const char * e = getenv("VX_FA_MIN_CHUNK"); const int v = e ? atoi(e) : 0; return v >= 32 ? v / 32 * 32 : 32; }();
     *n_splits  = 1;
     *chunk_out = (n_kv + 31) / 32 * 32;
     // Up to 256 keys one wave finishes (0.5 us per 32-key step) before a split plus the merge
@@ -483,7 +486,8 @@ void fa_split_plan(int64_t tiles, int n_kv, int * n_splits, int * chunk_out) {
         int64_t want = ((int64_t) waves_per_cu * num_cus() + tiles - 1) / tiles;
         const int64_t max_splits = (n_kv + min_chunk - 1) / min_chunk;
         if (want > max_splits) want = max_splits;
-        if (want > FA_MERGE_MAX_SPLITS) want = FA_MERGE_MAX_SPLITS;
+        static const int cap = [] { const char * e = getenv("VX_FA_MAX_SPLITS"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= FA_MERGE_MAX_SPLITS ? v : 64; }();
+        if (want > cap) want = cap;
         if (want < 1) want = 1;
         int chunk  = (int) ((n_kv + want - 1) / want);
         chunk      = (chunk + 31) / 32 * 32;
