@@ -398,6 +398,8 @@ def mm_inputs(tag, M, K, N, batch=()):
                                    (3072, 1024, 112), (1024, 1024, 512), (70, 96, 130),
                                    # the 128 x 128 pipelined GEMM: full tiles, and ragged rows / tokens / odd block count
                                    (4096, 1024, 1024), (2000, 1056, 1700),
+                                   # operands through LDS: ragged rows and tokens on 128 x 128 and 64 x 64 tiles, few rows
+                                   (2000, 1024, 1700), (1000, 1024, 333), (64, 1024, 4100), (130, 2048, 9000),
                                    # a long K on a small grid: K cut across work-groups, partials added by a second kernel
                                    (1024, 4096, 600), (1000, 2176, 300)])
 def test_mul_mat_q8_0(gpu, M, K, N):
@@ -418,7 +420,8 @@ def test_mul_mat_q8_0(gpu, M, K, N):
 
 
 @pytest.mark.parametrize("wtype", [np.float16, np.float32])
-@pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300), (2048, 256, 1600)])
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300), (2048, 256, 1600),
+                                   (1000, 256, 3000), (200, 192, 700)])
 def test_mul_mat_float_weights(gpu, wtype, M, K, N):
     say(f"mul_mat {wtype.__name__} weights M={M} K={K} N={N}")
     w, x = mm_inputs(("fw", M, K, N), M, K, N)
