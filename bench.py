@@ -388,7 +388,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
-    ap.add_argument("--profile", choices=["prefill", "backbone", "cfm"], default=None,
+    ap.add_argument("--profile", choices=["prefill", "backbone", "cfm", "gemm"], default=None,
                     help="run only this secondary workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -415,6 +415,13 @@ def main():
         s = timer.run(call, iters=5, warmup=2)
         print(json.dumps({"profile": "cfg5_prefill_attn_T4096_B16", "us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
                           "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}))
+        return
+    if args.profile == "gemm":      # the prefill-sized Q8_0 projection, 4096 rows x 1024 x 16384 tokens
+        M, K, N = 4096, 1024, 16384
+        call, keep = q8_proj_setup(pkg, M, K, N)
+        s = timer.run(call, iters=5, warmup=2)
+        print(json.dumps({"profile": "q8_0_mul_mat_4096x1024x16384", "us": s * 1e6, "TFLOP/s": 2.0 * M * K * N / s / 1e12,
+                          "mfma_frac": 2.0 * M * K * N / s / 1e12 / MFMA_F16_PEAK_TFLOPS, "VX_GEMM_LDS": os.environ.get("VX_GEMM_LDS", "1")}))
         return
     if args.profile == "cfm":       # config 3: whole CFM solves of one request, replayed from a HIP graph
         print(json.dumps({"profile": "cfg3_cfm_solve_one_request", **cfm_solve_bench(pkg, timer, torch.cuda.Stream(), 1, False)}))
