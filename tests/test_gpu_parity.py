@@ -442,6 +442,13 @@ def test_mul_mat_broadcast_and_views(gpu):
     cpu = reflib.oracle_mul_mat(wq, x, 128, act_mode=0)
     got = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_Q8, w_ne0=128))
     assert np.abs(got - cpu).max() <= 1e-5 * np.abs(cpu).max()
+    # the same broadcast with enough tokens for the LDS-tiled kernel (one grid plane per batch entry)
+    w, _ = mm_inputs("bc2", 192, 128, 1, batch=(1, 2))
+    x = rng("bc2", "x").standard_normal((1, 4, 400, 128)).astype(np.float32)
+    wq = reflib.quantize_q8_0(w)
+    f64 = reflib.oracle_mul_mat(wq, x, 128, f64=True)
+    got = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_FLOAT, w_ne0=128))
+    assert got.shape == f64.shape and nmse(f64, got) <= 1e-6
 
 
 def test_q8_0_dequant_is_exact(gpu):
