@@ -127,8 +127,22 @@ bool al16(const void * p, const uint64_t * nb) {
 
 template <int OP>
 vx_status ew_launch(ew_args & a, hipStream_t st) {
+    if (a.ne[0] <= 0 || a.ne[1] * a.ne[2] * a.ne[3] <= 0) return VX_OK;
+    // A block walks one row.  Short rows that follow each other in memory in every operand (attention-shaped tensors:
+    // 64 elements per row, 16384 rows at a 2 x 512-token prefill) are joined into long ones first, so that a block's
+    // 256 threads all have an element.
+    while (a.ne[0] < 1024 && a.ne[1] > 1 && a.nb0[0] == 4 && a.nbd[0] == 4 && a.nb0[1] == (uint64_t) a.ne[0] * 4 && a.nbd[1] == (uint64_t) a.ne[0] * 4 &&
+           (!ew_has_src1<OP>() || (a.ne1[0] == a.ne[0] && a.ne1[1] == a.ne[1] && a.nb1[0] == 4 && a.nb1[1] == (uint64_t) a.ne[0] * 4))) {
+        a.ne[0] *= a.ne[1];
+        a.ne1[0] = ew_has_src1<OP>() ? a.ne[0] : a.ne1[0];
+        for (int i = 1; i < 3; ++i) {
+            a.ne[i] = a.ne[i + 1]; a.ne1[i] = a.ne1[i + 1];
+            a.nb0[i] = a.nb0[i + 1]; a.nb1[i] = a.nb1[i + 1]; a.nbd[i] = a.nbd[i + 1];
+        }
+        a.ne[3] = 1; a.ne1[3] = 1;
+        a.nb0[3] = a.nb0[2] * (uint64_t) a.ne[2]; a.nb1[3] = a.nb1[2] * (uint64_t) a.ne1[2]; a.nbd[3] = a.nbd[2] * (uint64_t) a.ne[2];
+    }
     const int64_t rows = a.ne[1] * a.ne[2] * a.ne[3];
-    if (a.ne[0] <= 0 || rows <= 0) return VX_OK;
     bool vec = a.ne[0] % 4 == 0 && a.nb0[0] == 4 && a.nbd[0] == 4 && al16(a.s0, a.nb0) && al16(a.d, a.nbd);
     if (ew_has_src1<OP>()) vec = vec && a.ne1[0] == a.ne[0] && a.nb1[0] == 4 && al16(a.s1, a.nb1);
     const int V = vec ? 4 : 1;
