@@ -397,10 +397,14 @@ __global__ __launch_bounds__(1024) void sum_kernel(const char * src, vx_dims s, 
     }
 }
 
-__global__ __launch_bounds__(64) void sum_partials_kernel(const double * partials, int n, float * dst) {
+// adds the blocks' partials in block order; they are fetched by as many lanes at once (one trip to memory, not n)
+__global__ __launch_bounds__(SUM_BLOCKS) void sum_partials_kernel(const double * partials, int n, float * dst) {
+    __shared__ double part[SUM_BLOCKS];
+    if ((int) threadIdx.x < n) part[threadIdx.x] = partials[threadIdx.x];
+    __syncthreads();
     if (threadIdx.x == 0) {
         double t = 0.0;
-        for (int i = 0; i < n; ++i) t += partials[i];
+        for (int i = 0; i < n; ++i) t += part[i];
         *dst = (float) t;
     }
 }
@@ -1178,7 +1182,7 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
     const dim3 block(units <= VX_SUM_ONE_WAVE_UNITS ? 64 : 1024); // small sums are one wave's work
     if (vec) sum_kernel<true><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
     else     sum_kernel<false><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
-    if (partials) sum_partials_kernel<<<dim3(1), dim3(64), 0, st>>>(partials, blocks, (float *) dst->data);
+    if (partials) sum_partials_kernel<<<dim3(1), dim3(SUM_BLOCKS), 0, st>>>(partials, blocks, (float *) dst->data);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
