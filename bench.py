@@ -222,12 +222,18 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     weight_bytes = layers * sum(lw[n].nbytes for n in reflib.BB_WEIGHTS)
 
     t_prefill = None
+    t_prefill_f16 = None
     xp = None
     if do_prefill:
         xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
         mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
         run_p, _ = m.plan(xp, prefill, 0, mask)
         t_prefill = timer.run(run_p, iters=3, warmup=1)
+        # the same prefill with the F32 cache rounded to f16 on its way into the LDS-tiled attention kernel (opt-in, read per call)
+        os.environ["VX_FA_F32_PREFILL"] = "1"
+        t_prefill_f16 = timer.run(run_p, iters=3, warmup=1)
+        del os.environ["VX_FA_F32_PREFILL"]
+        timer.run(run_p, iters=1, warmup=0)  # leave the cache as the default route writes it
     else:   # long caches: decode over seeded cache contents instead of a real prefill
         gk = torch.Generator(device="cuda").manual_seed(11)
         for t in m.k_cache + m.v_cache:
@@ -254,6 +260,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
            "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
            "prefill_ms": t_prefill * 1e3 if t_prefill else None, "prefill_tokens_per_s": batch * prefill / t_prefill if t_prefill else None,
+           "prefill_ms_VX_FA_F32_PREFILL": t_prefill_f16 * 1e3 if t_prefill else None,
            "kv_cache": "f32 (the reference's cache type)", "launch": "captured HIP graph per step, KV lengths " + str(points)}
     del replays, m
     ref = reflib.load_ref() if with_cpu else None
