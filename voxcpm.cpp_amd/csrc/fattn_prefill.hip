@@ -110,7 +110,9 @@ __global__ __launch_bounds__(64) void pf_mask_flags_kernel(const char * mask, ui
     if (threadIdx.x == 0) flags[((uint64_t) mb * n_rb + rb) * n_tiles + tile] = !vis ? 0 : (nz ? 2 : 1);
 }
 
-template <bool KV_F32>
+// CT: 16-column tiles per wave.  PF_CT for large problems; half of it (work-groups of half as many columns, twice as many
+// of them) when the grid would leave most of the chip idle.
+template <bool KV_F32, int CT = PF_CT>
 __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2))) void pf_kernel(const pf_args a) {
     constexpr int D = 64, NP = 2, SEG = 16;
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][PF_KT][PF_ROW];
@@ -176,10 +178,10 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 
     // ---- this wave's columns
     const int ncols_blk = min(a.n_q - row0, a.RB) * a.gqa; // valid columns of the block
-    half8_t qhi[PF_CT][NP];
+    half8_t qhi[CT][NP];
 #pragma unroll
-    for (int ct = 0; ct < PF_CT; ++ct) {
-        const int  col = wave * 64 + ct * 16 + c;
+    for (int ct = 0; ct < CT; ++ct) {
+        const int  col = wave * (16 * CT) + ct * 16 + c;
         const bool ok  = col < ncols_blk;
         const int  row = row0 + (ok ? col / a.gqa : 0);
         const int  hd  = g * a.gqa + (ok ? col % a.gqa : 0);
@@ -211,10 +213,10 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
     // score of the wave runs more than PF_LAZY above its reference (or the tile carries mask
     // values, or a column has not seen a key yet) does the slow block run: it moves m_ref up
     // and rescales O.  Values up to 2^PF_LAZY sit comfortably in f16 and fp32.
-    float4_t o[PF_CT][4], ol[PF_CT], negm[PF_CT];
-    bool     seen[PF_CT];
+    float4_t o[CT][4], ol[CT], negm[CT];
+    bool     seen[CT];
 #pragma unroll
-    for (int ct = 0; ct < PF_CT; ++ct) {
+    for (int ct = 0; ct < CT; ++ct) {
         negm[ct] = float4_t{0, 0, 0, 0};
         seen[ct] = false;
         ol[ct] = float4_t{0, 0, 0, 0};
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                 for (int t = 0; t < 4; ++t) av[t] = *(const half8_t *) &vt_lds[buf][(c & 7) * 8 + 2 * t + (c >> 3)][((hh * 4 + j) ^ (c & 7)) << 3];
 
 #pragma unroll
-                for (int cg = 0; cg < PF_CT; cg += PF_GRP) {
+                for (int cg = 0; cg < CT; cg += PF_GRP) {
                     // scores of PF_GRP column tiles, then ONE wave-uniform decision for the group, so
                     // the common path is straight-line code the scheduler can interleave
                     float4_t s[PF_GRP][2];
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                         for (int u = 0; u < PF_GRP; ++u) {
                             const int ct = cg + u;
                             if (mixed) { // element-wise mask / bounds (diagonal and tail tiles only)
-                                const int col  = wave * 64 + ct * 16 + c;
+                                const int col  = wave * (16 * CT) + ct * 16 + c;
                                 const bool ok  = col < ncols_blk;
                                 const int row  = row0 + (ok ? col / a.gqa : 0);
                                 const int hd   = g * a.gqa + (ok ? col % a.gqa : 0);
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
             if (!all_seen) {
                 bool every = true;
 #pragma unroll
-                for (int ct = 0; ct < PF_CT; ++ct) every = every && seen[ct];
+                for (int ct = 0; ct < CT; ++ct) every = every && seen[ct];
                 all_seen = __builtin_amdgcn_ballot_w64(!every) == 0;
             }
             store_lds(buf ^ 1);
@@ -387,8 +389,8 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 
     // ---- finish: lane (j,c), d-tile t, register r holds d = 16t + 4j + r of column c
 #pragma unroll
-    for (int ct = 0; ct < PF_CT; ++ct) {
-        const int  col = wave * 64 + ct * 16 + c;
+    for (int ct = 0; ct < CT; ++ct) {
+        const int  col = wave * (16 * CT) + ct * 16 + c;
         const bool ok  = col < ncols_blk;
         const int  row = row0 + (ok ? col / a.gqa : 0);
         const int  hd  = g * a.gqa + (ok ? col % a.gqa : 0);
@@ -430,7 +432,7 @@ bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float lo
         return false;
     }
     const int Hq = (int) q->ne[2], Hkv = (int) k->ne[2], gqa = Hq / Hkv;
-    if (gqa > PF_COLS || (PF_COLS % gqa) != 0) return false;
+    if (gqa > PF_COLS / 2 || ((PF_COLS / 2) % gqa) != 0) return false;
     const int n_q = (int) q->ne[1], n_kv = (int) k->ne[1];
     const int RB = PF_COLS / gqa, n_rb = (n_q + RB - 1) / RB, n_tiles = (n_kv + PF_KT - 1) / PF_KT;
     const int n_groups = (int) q->ne[3] * Hkv;
@@ -444,8 +446,11 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     if (!vx_fattn_prefill_accepts(q, k, logit_softcap)) return VX_ERR_UNSUPPORTED;
     const int Hq = (int) q->ne[2], Hkv = (int) k->ne[2], gqa = Hq / Hkv;
     const int n_q = (int) q->ne[1], n_kv = (int) k->ne[1];
-    const int RB = PF_COLS / gqa, n_rb = (n_q + RB - 1) / RB, n_tiles = (n_kv + PF_KT - 1) / PF_KT;
     const int n_groups = (int) q->ne[3] * Hkv;
+    // work-groups of 256 columns; of 128 while 256 would put fewer than two work-groups on every CU
+    const bool half_cols = (int64_t) ((n_q + PF_COLS / gqa - 1) / (PF_COLS / gqa)) * n_groups < 512;
+    const int cols = half_cols ? PF_COLS / 2 : PF_COLS;
+    const int RB = cols / gqa, n_rb = (n_q + RB - 1) / RB, n_tiles = (n_kv + PF_KT - 1) / PF_KT;
 
     pf_args a;
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
@@ -482,8 +487,13 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
         a.flags = (const uint8_t *) ws;
     }
     const dim3 grid((unsigned) (n_rb * n_groups)), block(64 * PF_WAVES);
-    if (a.kv_f32) pf_kernel<true><<<grid, block, 0, st>>>(a);
-    else          pf_kernel<false><<<grid, block, 0, st>>>(a);
+    if (half_cols) {
+        if (a.kv_f32) pf_kernel<true, PF_CT / 2><<<grid, block, 0, st>>>(a);
+        else          pf_kernel<false, PF_CT / 2><<<grid, block, 0, st>>>(a);
+    } else {
+        if (a.kv_f32) pf_kernel<true><<<grid, block, 0, st>>>(a);
+        else          pf_kernel<false><<<grid, block, 0, st>>>(a);
+    }
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
