@@ -353,7 +353,7 @@ def test_fa_prefill_kernel_on_request_for_f32_kv(gpu, monkeypatch):
 @pytest.mark.parametrize("case", ["causal", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
 def test_fa_prefill_kernel(gpu, case):
     """Shapes large enough to take the LDS-tiled prefill kernel (>= 256 columns per KV head,
-    >= 64 work-groups)."""
+    >= 32 work-groups of 256 columns)."""
     say(f"flash_attn prefill kernel: {case}")
     B, Hq, Hkv, T, KV = 4, 16, 2, 512, 512
     mask, sinks, max_bias, kvt = None, None, 0.0, np.float16
