@@ -350,14 +350,17 @@ def test_fa_prefill_kernel_on_request_for_f32_kv(gpu, monkeypatch):
     assert np.abs(got - want).max() > 2e-5       # it did take the other kernel
 
 
-@pytest.mark.parametrize("case", ["causal", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
+@pytest.mark.parametrize("case", ["causal", "wide", "past", "nomask", "f32kv", "random_mask", "mha", "sinks_alibi", "ragged"])
 def test_fa_prefill_kernel(gpu, case):
     """Shapes large enough to take the LDS-tiled prefill kernel (>= 256 columns per KV head,
     >= 32 work-groups of 256 columns)."""
     say(f"flash_attn prefill kernel: {case}")
     B, Hq, Hkv, T, KV = 4, 16, 2, 512, 512
     mask, sinks, max_bias, kvt = None, None, 0.0, np.float16
-    if case == "causal":
+    if case == "causal":          # 128 work-groups: the half-width (128-column) form
+        mask = reflib.causal_mask(T, KV)
+    elif case == "wide":          # 512 work-groups of 256 columns: the full-width form
+        B = 16
         mask = reflib.causal_mask(T, KV)
     elif case == "past":
         T, KV = 300, 700
