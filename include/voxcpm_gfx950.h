@@ -16,7 +16,7 @@
  *
  * Streams: `stream` is a hipStream_t passed as void* (NULL = the null stream).  All work
  * is enqueued asynchronously on it.  Ops that need scratch memory take it from a
- * per-stream workspace the library grows on demand with hipMalloc.
+ * per-stream workspace the library grows on demand with hipMalloc (see vx_workspace_reserve).
  */
 #ifndef VOXCPM_GFX950_H
 #define VOXCPM_GFX950_H
@@ -73,6 +73,15 @@ VX_API vx_status    vx_memset(void * dst, int value, size_t bytes, vx_stream str
 VX_API vx_status    vx_stream_create(vx_stream * stream);
 VX_API vx_status    vx_stream_destroy(vx_stream stream);
 VX_API vx_status    vx_stream_synchronize(vx_stream stream);
+/* The per-stream workspace (split-KV partials, split-K partials, block sums, mask classification).  It grows on
+ * demand; a block that was handed out keeps its address and stays allocated until vx_stream_destroy, also after a
+ * larger block has replaced it, so launches already queued and HIP graphs already captured from the stream stay
+ * valid.  A call that would have to grow the workspace while the stream is being captured returns
+ * VX_ERR_UNSUPPORTED: reserve the largest size first.  No counterpart in the reference (ggml-cpu takes its scratch
+ * from the compute plan's work buffer, ggml/src/ggml-cpu/ggml-cpu.c:2700-2935). */
+VX_API vx_status    vx_workspace_reserve(vx_stream stream, size_t bytes);
+/* current block, its size and the number of superseded blocks still held for this stream (any out pointer may be NULL) */
+VX_API vx_status    vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int * retired_blocks);
 
 /* ---- GGML_OP_RMS_NORM -------------------------------------------------------------------
  * replaces ggml_compute_forward_rms_norm (ggml/src/ggml-cpu/ops.cpp:3710-3777).

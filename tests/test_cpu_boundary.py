@@ -288,3 +288,14 @@ def test_plugin_on_a_gpuless_host(pkg, ref):
     assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) != 0
     names = [ref.rh_device_name(i).decode() for i in range(ref.rh_device_count())]
     assert names == ["CPU"]
+
+
+def test_workspace_growth_policy(tmp_path):
+    """The per-stream workspace never frees or moves a block it has handed out (a captured HIP graph keeps the
+    address), refuses to grow during a capture, and releases everything with the stream: the policy header,
+    compiled for the host with a counting allocator."""
+    import subprocess
+    exe = str(tmp_path / "ws_policy_check")
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-o", exe, os.path.join(ROOT, "tests", "ws_policy_check.cpp")])
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", out.stdout + out.stderr

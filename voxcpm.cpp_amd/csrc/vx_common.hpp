@@ -34,12 +34,10 @@ vx_status  vx_fail(vx_status st, const char * fmt, ...) __attribute__((format(pr
                            hipGetErrorString(e_), __FILE__, __LINE__);                       \
     } while (0)
 
-// per-stream scratch memory, grown on demand (never shrinks); valid until the next call
-// that asks for more on the same stream
+// per-stream scratch memory, grown on demand.  A block stays allocated at its address until the stream is
+// destroyed, also after a larger one has replaced it (ws_policy.hpp), so launches already queued and graphs
+// already captured keep valid arguments; growth during a stream capture is refused.
 vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr);
-// per-stream array of `count` ints that is all zero whenever no kernel of this library is
-// running on the stream: kernels that use it as arrival counters put every entry back to zero
-vx_status vx_counters(hipStream_t stream, size_t count, void ** ptr);
 
 // LDS-tiled prefill kernel (fattn_prefill.hip); VX_ERR_UNSUPPORTED means "use the general kernel"
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,

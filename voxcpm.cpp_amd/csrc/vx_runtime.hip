@@ -1,5 +1,6 @@
 // vx_runtime.hip -- device discovery, memory, streams and the per-stream workspace.
 #include "vx_common.hpp"
+#include "ws_policy.hpp"
 
 #include <cstring>
 #include <mutex>
@@ -9,13 +10,12 @@ namespace {
 
 thread_local char g_err[512] = "";
 
-struct workspace {
-    void * ptr   = nullptr;
-    size_t bytes = 0;
-};
-std::mutex                                    g_ws_mutex;
-std::unordered_map<unsigned long long, workspace> g_ws;  // key: device << 56 ^ stream handle
-std::unordered_map<unsigned long long, workspace> g_cnt; // zero-initialised counters, same key
+std::mutex                                      g_ws_mutex;
+std::unordered_map<unsigned long long, vx_ws_state> g_ws; // key: device << 56 ^ stream handle
+
+unsigned long long ws_key(int dev, hipStream_t stream) {
+    return ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
+}
 
 } // namespace
 
@@ -37,54 +37,25 @@ vx_status vx_fail(vx_status st, const char * fmt, ...) {
 vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr) {
     int dev = 0;
     VX_HIP(hipGetDevice(&dev));
-    const unsigned long long key = ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    workspace & ws = g_ws[key];
-    if (ws.bytes < bytes) {
-        if (ws.ptr) {
-            // work already queued on this stream may still read the old block
-            VX_HIP(hipStreamSynchronize(stream));
-            VX_HIP(hipFree(ws.ptr));
-            ws.ptr   = nullptr;
-            ws.bytes = 0;
-        }
-        size_t want = bytes < (size_t) (1u << 20) ? (size_t) (1u << 20) : bytes + bytes / 4;
-        want        = (want + 255) & ~(size_t) 255;
-        hipError_t e = hipMalloc(&ws.ptr, want);
-        if (e != hipSuccess) {
-            ws.ptr = nullptr;
-            return vx_fail(VX_ERR_ALLOC, "workspace hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
-        }
-        ws.bytes = want;
+    vx_ws_state & ws = g_ws[ws_key(dev, stream)];
+    bool capturing = false;
+    if (bytes > ws.cur.bytes) { // only a growing request needs to know
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cs) != hipSuccess) (void) hipGetLastError();
+        capturing = cs != hipStreamCaptureStatusNone;
     }
-    *ptr = ws.ptr;
-    return VX_OK;
-}
-
-vx_status vx_counters(hipStream_t stream, size_t count, void ** ptr) {
-    int dev = 0;
-    VX_HIP(hipGetDevice(&dev));
-    const unsigned long long key = ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
-    const size_t bytes = count * sizeof(int);
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    workspace & ws = g_cnt[key];
-    if (ws.bytes < bytes) {
-        if (ws.ptr) {
-            VX_HIP(hipStreamSynchronize(stream));
-            VX_HIP(hipFree(ws.ptr));
-            ws.ptr   = nullptr;
-            ws.bytes = 0;
-        }
-        size_t want = bytes < 4096 ? 4096 : 2 * bytes;
-        hipError_t e = hipMalloc(&ws.ptr, want);
-        if (e != hipSuccess) {
-            ws.ptr = nullptr;
-            return vx_fail(VX_ERR_ALLOC, "counter hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
-        }
-        ws.bytes = want;
-        VX_HIP(hipMemsetAsync(ws.ptr, 0, want, stream));
-    }
-    *ptr = ws.ptr;
+    hipError_t err = hipSuccess;
+    const vx_ws_result r = vx_ws_request(ws, bytes, capturing, [&](size_t want) -> void * {
+        void * p = nullptr;
+        err      = hipMalloc(&p, want);
+        return err == hipSuccess ? p : nullptr;
+    }, ptr);
+    if (r == VX_WS_CAPTURING)
+        return vx_fail(VX_ERR_UNSUPPORTED, "the stream is being captured and the call needs %zu bytes of workspace but %zu are reserved: "
+                       "call vx_workspace_reserve(stream, bytes) before the capture begins", bytes, ws.cur.bytes);
+    if (r == VX_WS_ALLOC_FAILED)
+        return vx_fail(VX_ERR_ALLOC, "workspace hipMalloc for %zu bytes failed: %s", bytes, hipGetErrorString(err));
     return VX_OK;
 }
 
@@ -191,17 +162,29 @@ vx_status vx_stream_destroy(vx_stream stream) {
     int dev = 0;
     VX_HIP(hipGetDevice(&dev));
     VX_HIP(hipStreamSynchronize((hipStream_t) stream));
-    {   // the stream's scratch blocks go with it
-        const unsigned long long key = ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
+    {   // the stream's scratch blocks, live and retired, go with it
         std::lock_guard<std::mutex> lock(g_ws_mutex);
-        for (auto * map : {&g_ws, &g_cnt}) {
-            auto it = map->find(key);
-            if (it == map->end()) continue;
-            if (it->second.ptr) (void) hipFree(it->second.ptr);
-            map->erase(it);
+        auto it = g_ws.find(ws_key(dev, (hipStream_t) stream));
+        if (it != g_ws.end()) {
+            vx_ws_release_all(it->second, [](void * p) { (void) hipFree(p); });
+            g_ws.erase(it);
         }
     }
     VX_HIP(hipStreamDestroy((hipStream_t) stream));
+    return VX_OK;
+}
+vx_status vx_workspace_reserve(vx_stream stream, size_t bytes) {
+    void * p = nullptr;
+    return vx_workspace((hipStream_t) stream, bytes, &p);
+}
+vx_status vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int * retired_blocks) {
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws.find(ws_key(dev, (hipStream_t) stream));
+    if (ptr) *ptr = it == g_ws.end() ? nullptr : it->second.cur.ptr;
+    if (bytes) *bytes = it == g_ws.end() ? 0 : it->second.cur.bytes;
+    if (retired_blocks) *retired_blocks = it == g_ws.end() ? 0 : (int) it->second.retired.size();
     return VX_OK;
 }
 vx_status vx_stream_synchronize(vx_stream stream) {
