@@ -117,6 +117,22 @@ VX_API vx_status vx_flash_attn_ext(const vx_tensor * q, const vx_tensor * k, con
                                    float scale, float max_bias, float logit_softcap,
                                    vx_stream stream);
 
+/* vx_flash_attn_ext for callers that must not allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same results as
+ * vx_flash_attn_ext wherever that call takes the key-range (split-KV) kernels, i.e. decode and LocDiT-sized query
+ * counts; long prefills run on the same kernels too (within the operator's 2e-3 tolerance of the LDS-tiled kernel
+ * vx_flash_attn_ext would choose, and slower).  The partial results of the key ranges go to a fixed array of
+ * VX_FLASH_ATTN_EXT_STATIC_SCRATCH_BYTES that is part of the loaded library on each GPU (held until the process ends)
+ * instead of the per-stream workspace; the call performs no hipMalloc / hipFree.  A shape whose partials would not fit
+ * is refused with VX_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (different streams, different threads) race; issue them on one stream or order them yourself.  Nothing in the
+ * array needs clearing between calls (every partial that is read has been written by the same call). */
+#define VX_FLASH_ATTN_EXT_STATIC_SCRATCH_BYTES ((size_t) 16 << 20)
+VX_API vx_status vx_flash_attn_ext_static(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                          const vx_tensor * mask, const float * sinks, const vx_tensor * dst,
+                                          float scale, float max_bias, float logit_softcap,
+                                          vx_stream stream);
+
 /* ---- GGML_OP_MUL_MAT -----------------------------------------------------------------------
  * replaces ggml_compute_forward_mul_mat (ggml/src/ggml-cpu/ggml-cpu.c:1139-1421):
  * dst[ne01, ne11, ne12, ne13] = src0[ne00, ne01, ne02, ne03]^T x src1[ne00, ne11, ne12, ne13],

@@ -48,7 +48,7 @@ EXPORTS = [
     "vx_device_count", "vx_init", "vx_last_error", "vx_device_info", "vx_malloc", "vx_free",
     "vx_malloc_host", "vx_free_host", "vx_memcpy_h2d", "vx_memcpy_d2h", "vx_memcpy_d2d", "vx_memset",
     "vx_stream_create", "vx_stream_destroy", "vx_stream_synchronize", "vx_workspace_reserve", "vx_workspace_info",
-    "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_mul_mat",
+    "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_flash_attn_ext_static", "vx_mul_mat",
     "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
     "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
     "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum",
@@ -100,6 +100,7 @@ def lib():
     l.vx_rope.argtypes = [TP, i32p, f32p, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [vp]
     l.vx_soft_max.argtypes = [TP, TP, f32p, TP, C.c_float, C.c_float, vp]
     l.vx_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, vp]
+    l.vx_flash_attn_ext_static.argtypes = l.vx_flash_attn_ext.argtypes
     l.vx_mul_mat.argtypes = [TP, TP, TP, C.c_int, vp]
     l.vx_supports_rms_norm.argtypes = [TP, TP]
     l.vx_supports_rope.argtypes = [TP, TP, C.c_int, C.c_int]
@@ -251,6 +252,18 @@ def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, logit_softcap=0.0, sinks=
                           dtype=torch.float32, device=q.device)
     check(lib().vx_flash_attn_ext(desc(q), desc(k), desc(v), desc(mask), _p(sinks), desc(out), scale, max_bias,
                                   logit_softcap, _stream()), "vx_flash_attn_ext")
+    return out
+
+
+def flash_attn_ext_static(q, k, v, mask, scale, max_bias=0.0, logit_softcap=0.0, sinks=None, out=None):
+    """flash_attn_ext through the entry point that allocates nothing; `out` must be given by callers that
+    may not allocate either."""
+    import torch
+    if out is None:
+        out = torch.empty((q.shape[-4] if q.dim() == 4 else 1, q.shape[-2], q.shape[-3], v.shape[-1]),
+                          dtype=torch.float32, device=q.device)
+    check(lib().vx_flash_attn_ext_static(desc(q), desc(k), desc(v), desc(mask), _p(sinks), desc(out), scale, max_bias,
+                                         logit_softcap, _stream()), "vx_flash_attn_ext_static")
     return out
 
 

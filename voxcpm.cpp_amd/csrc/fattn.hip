@@ -37,6 +37,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 
 namespace {
 
@@ -560,7 +561,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
                         const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
                         hipStream_t st, const vx_tensor * ks_src = nullptr, const vx_tensor * ks_slot = nullptr,
                         const vx_tensor * vs_src = nullptr, const vx_tensor * vs_slot = nullptr, float kvs_scale = 0.0f,
-                        float kvs_bias = 0.0f);
+                        float kvs_bias = 0.0f, void * fixed_ws = nullptr, size_t fixed_ws_bytes = 0);
 
 extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
                                             const vx_tensor * mask, const float * sinks, const float * addend,
@@ -665,11 +666,62 @@ extern "C" vx_status vx_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_t
                   k_src, k_slot, v_src, v_slot, sync_scale, sync_bias);
 }
 
+// ---- the entry point that allocates nothing ------------------------------------------------------------
+// The key-range partials of vx_flash_attn_ext_static live in a fixed array in device memory that is part of the
+// loaded code object: every GPU the library runs on holds its own copy, at its own address, until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress -- the address kernels must be
+// given is looked up once per device and kept.
+constexpr size_t FA_STATIC_SCRATCH_BYTES = VX_FLASH_ATTN_EXT_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_SCRATCH_BYTES];
+
+constexpr int FA_MAX_DEVICES = 64;
+static void *     g_scratch_ptr[FA_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// the address of `scratch` on the current device, looked up on the first request
+static vx_status fa_static_scratch(void ** ptr) {
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= FA_MAX_DEVICES) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_static: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void * p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return vx_fail(VX_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return VX_OK;
+}
+
+vx_status vx_fattn_static_setup(void) {
+    void * p = nullptr;
+    return fa_static_scratch(&p);
+}
+
+extern "C" vx_status vx_flash_attn_ext_static(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v,
+                                              const vx_tensor * mask, const float * sinks, const vx_tensor * dst,
+                                              float scale, float max_bias, float logit_softcap, vx_stream stream) {
+    if (!q || !k || !v || !dst || !q->data || !k->data || !v->data || !dst->data || (mask && !mask->data))
+        return vx_fail(VX_ERR_INVALID, "flash_attn_ext_static: null tensor");
+    if (!vx_supports_flash_attn_ext(q, k, v, mask, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_static: needs q F32, k/v both F16 or both F32, D in {64,128}, dense rows, 16-byte aligned strides, contiguous dst, F16 mask");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (uintptr_t) dst->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_static: tensor data must be 16-byte aligned");
+    if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_static: max_bias > 0 requires a mask");
+    void * ws = nullptr;
+    const vx_status rc = fa_static_scratch(&ws);
+    if (rc != VX_OK) return rc;
+    return fa_run(q, k, v, nullptr, nullptr, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream,
+                  nullptr, nullptr, nullptr, nullptr, 0.0f, 0.0f, ws, FA_STATIC_SCRATCH_BYTES);
+}
+
 static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * k2, const vx_tensor * v2,
                         const vx_tensor * kall, const vx_tensor * vall, const vx_tensor * mask, const float * sinks,
                         const float * addend, const vx_tensor * dst, float scale, float max_bias, float logit_softcap,
                         hipStream_t st, const vx_tensor * ks_src, const vx_tensor * ks_slot, const vx_tensor * vs_src,
-                        const vx_tensor * vs_slot, float kvs_scale, float kvs_bias) {
+                        const vx_tensor * vs_slot, float kvs_scale, float kvs_bias, void * fixed_ws, size_t fixed_ws_bytes) {
     (void) vall;
     fa_args a;
     a.has_kvs = 0;
@@ -719,9 +771,15 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     if (a.n_splits > 1) {
         const size_t o_bytes  = (size_t) nblocks * 16 * D * sizeof(float);
         const size_t ml_bytes = (size_t) nblocks * 16 * 2 * sizeof(float);
-        void * ws = nullptr;
-        vx_status rc = vx_workspace(st, o_bytes + ml_bytes, &ws);
-        if (rc != VX_OK) return rc;
+        void * ws = fixed_ws;
+        if (fixed_ws) { // the caller's fixed block: nothing is allocated, larger shapes are refused
+            if (o_bytes + ml_bytes > fixed_ws_bytes)
+                return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_static: the key-range partials of this shape need %zu bytes, the fixed scratch holds %zu "
+                               "(use vx_flash_attn_ext, which allocates)", o_bytes + ml_bytes, fixed_ws_bytes);
+        } else {
+            vx_status rc = vx_workspace(st, o_bytes + ml_bytes, &ws);
+            if (rc != VX_OK) return rc;
+        }
         a.part_o  = (float *) ws;
         a.part_ml = (float *) ((char *) ws + o_bytes);
     }

@@ -39,6 +39,10 @@ vx_status  vx_fail(vx_status st, const char * fmt, ...) __attribute__((format(pr
 // already captured keep valid arguments; growth during a stream capture is refused.
 vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr);
 
+// vx_flash_attn_ext_static's fixed scratch array (fattn.hip): the per-device address lookup that vx_init performs
+// so that the first call of the entry point does no set-up work
+vx_status vx_fattn_static_setup(void);
+
 // LDS-tiled prefill kernel (fattn_prefill.hip); VX_ERR_UNSUPPORTED means "use the general kernel"
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                            const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,

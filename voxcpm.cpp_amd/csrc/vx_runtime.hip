@@ -84,7 +84,7 @@ vx_status vx_init(int device) {
     if (n <= 0) return vx_fail(VX_ERR_NO_DEVICE, "no gfx950 device visible to HIP");
     if (device < 0 || device >= n) return vx_fail(VX_ERR_INVALID, "device %d out of range (0..%d)", device, n - 1);
     VX_HIP(hipSetDevice(device));
-    return VX_OK;
+    return vx_fattn_static_setup(); // the fixed scratch array's address on this device
 }
 
 vx_status vx_device_info(int device, char * name, size_t name_len, size_t * free_bytes, size_t * total_bytes,
