@@ -434,6 +434,23 @@ int rh_bb_set(int layer, int which, const void * data, size_t nbytes) {
     return 0;
 }
 
+// Fills (or reads back) one layer's K (which = 0) or V (which = 1) cache, the whole tensor [head_dim, max_len, n_kv, batch]
+// in the cache's own type: lets a test start a decode step from a long seeded past without running the prefill.
+int rh_bb_cache_set(int layer, int which, const void * data, size_t nbytes) {
+    if (!g_bb || layer < 0 || layer >= g_bb->n_layer) return 100;
+    ggml_tensor * t = which == 0 ? g_bb->layers[(size_t) layer].kc : g_bb->layers[(size_t) layer].vc;
+    if (ggml_nbytes(t) != nbytes) return 101;
+    ggml_backend_tensor_set(t, data, 0, nbytes);
+    return 0;
+}
+int rh_bb_cache_get(int layer, int which, void * data, size_t nbytes) {
+    if (!g_bb || layer < 0 || layer >= g_bb->n_layer) return 100;
+    ggml_tensor * t = which == 0 ? g_bb->layers[(size_t) layer].kc : g_bb->layers[(size_t) layer].vc;
+    if (ggml_nbytes(t) != nbytes) return 101;
+    ggml_backend_tensor_get(t, data, 0, nbytes);
+    return 0;
+}
+
 // x: [hidden, n_tokens, batch] F32 (dense); mask: F16 [n_past + n_tokens, n_tokens] or NULL;
 // out: [hidden, n_tokens, batch] after the final norm.  Graph and compute buffer are rebuilt on
 // every call, as the reference does per step (src/voxcpm.cpp:489-495); only the graph_compute

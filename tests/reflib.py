@@ -174,6 +174,8 @@ def load_ref():
     lib.rh_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, C.c_int, f64p]
     lib.rh_bb_create.argtypes = [C.c_int] * 8 + [C.c_float, C.c_int, C.c_float, C.c_int]
     lib.rh_bb_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    lib.rh_bb_cache_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    lib.rh_bb_cache_get.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_options.argtypes = [C.c_int, C.c_int]
     lib.rh_bb_options.restype = None
     lib.rh_bb_whole_graph.argtypes = [C.c_int]

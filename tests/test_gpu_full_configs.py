@@ -1,0 +1,208 @@
+"""BASELINE configurations 4 and 5 at their full sizes, against the reference's ggml-cpu (oracle/_ref).
+
+cfg 4: the 24-layer backbone, batch 2, a 512-token prefill and then all 256 decode steps; every call runs on ggml-cpu,
+       on the plugin (the reference-structured graph through ggml's graph_compute) and on the C-ABI mirror, each backend
+       reading the cache it wrote itself; outputs are compared at the prefill and at KV lengths 512, 640 and 767.
+cfg 5: 8 streams x CFG pair (batch 16), an f16 KV cache already holding 4096+ seeded tokens, one decode step through the
+       stack; and the 16 x 4096-token prefill attention against the oracle on sampled rows.
+
+Bars.  ggml-cpu quantises the activations of every product to int8 blocks (a step of amax/127 per block).  VX_ACT_FLOAT
+rounds them to f16 instead, so the two stacks differ by ggml-cpu's own quantisation noise, which the residual stream
+carries along without amplifying it: measured 2.0e-5 .. 2.5e-5 NMSE at 24 layers, the same as at 3.  VX_ACT_Q8 repeats
+ggml-cpu's integer arithmetic product by product (1e-5 relative, tests/test_gpu_parity.py), but a stack of quantisers is
+not continuous: a difference d in front of a quantiser of step s comes out with mean square d*s (a rounding flips with
+probability d/s and then moves the value by s), so differences of one ulp in a summation order grow layer by layer to
+the step itself and the stacks decorrelate to the same noise level, 2.1e-5 .. 2.4e-5 measured.  The bar is 1e-4 for both
+modes (ggml's own per-operator bar in test-backend-ops is 5e-4).  The mirror runs the plugin's launches on buffers of its
+own (other addresses, a tiled product may be cut differently): 1e-6 against the plugin with float activations; with
+quantised activations the argument above applies and the bar is the one against ggml-cpu."""
+import ctypes
+import sys
+
+import numpy as np
+import pytest
+
+import reflib
+from reflib import nmse, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def load_mirror(gpu, params, n_layer, max_len, batch, use_mup, kv_f16, act):
+    import torch
+    from voxcpm_cpp_amd import backbone as bb
+    m = bb.MiniCPMBackbone(n_layer=n_layer, max_length=max_len, batch=batch, use_mup=use_mup, kv_f16=kv_f16, act_mode=act)
+    for li, lw in enumerate(params["layers"]):
+        for n in reflib.BB_WEIGHTS:
+            m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+        for n in ("input_layernorm", "post_layernorm"):
+            m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+    m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+    m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+    return m
+
+
+@pytest.mark.parametrize("act", ["float", "q8"])
+def test_backbone_cfg4_full(gpu, ref, act):
+    """24 layers, batch 2, prefill 512, 256 decode steps (src/minicpm.cpp:749-846 is the loop this follows)."""
+    import torch
+    N_LAYER, BATCH, T0, STEPS = 24, 2, 512, 256
+    MAX_LEN = T0 + STEPS
+    check_at = {0: "prefill", 1: "KV 512", 129: "KV 640", 256: "KV 767"}   # call index -> label
+    act_mode = gpu.ACT_Q8 if act == "q8" else gpu.ACT_FLOAT
+    bar = 1e-4
+    mirror_bar = 1e-4 if act == "q8" else 1e-6
+    say(f"cfg 4 at full size: {N_LAYER} layers, batch {BATCH}, prefill {T0} + {STEPS} decode steps, activations {act}")
+    params = reflib.backbone_params("bb4", N_LAYER)
+    xs = [rng("bb4", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)]
+    xs += [rng("bb4", "x", i + 1).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(STEPS)]
+    mask0 = reflib.causal_mask(T0, T0)
+
+    def run(device, threads):
+        assert ref.rh_use_device(device, threads, 0) == 0
+        reflib.ref_backbone_create(params, MAX_LEN, BATCH, use_mup=True, kv_f16=False)
+        outs, n_past = {}, 0
+        for i, x in enumerate(xs):
+            o, _, _ = reflib.ref_backbone_forward(x, n_past, mask0 if i == 0 else None)
+            if i in check_at:
+                outs[i] = o
+            n_past += x.shape[1]
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs
+
+    say("   ggml-cpu ...")
+    cpu = run(b"CPU", 16)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+    before = plugin.ggml_backend_gfx950_set_mul_mat_act(act_mode)
+    try:
+        say("   plugin ...")
+        plug = run(b"GFX950_0", 8)
+    finally:
+        plugin.ggml_backend_gfx950_set_mul_mat_act(before)
+    launches = plugin.ggml_backend_gfx950_last_launches()
+    say(f"   plugin: {launches} launches for the last decode step")
+    assert launches == N_LAYER * 5 + 1
+    for i, label in check_at.items():
+        e = nmse(cpu[i], plug[i])
+        say(f"   plugin vs ggml-cpu at {label}: nmse {e:.3e}")
+        assert np.isfinite(plug[i]).all() and e <= bar, (label, e)
+
+    say("   C-ABI mirror ...")
+    m = load_mirror(gpu, params, N_LAYER, MAX_LEN, BATCH, True, False, act_mode)
+    n_past = 0
+    for i, x in enumerate(xs):
+        T = x.shape[1]
+        run_, got = m.plan(torch.from_numpy(x).cuda(), T, n_past, torch.from_numpy(mask0).cuda() if i == 0 else None)
+        run_()
+        if i in check_at:
+            torch.cuda.synchronize()
+            g = got.cpu().numpy()
+            e = nmse(cpu[i], g)
+            say(f"   mirror vs ggml-cpu at {check_at[i]}: nmse {e:.3e}")
+            assert e <= bar, (check_at[i], e)
+            # the mirror issues the plugin's launches on its own buffers: the same kernels on the same values
+            same = np.array_equal(g, plug[i])
+            say(f"      mirror == plugin bit for bit: {same}")
+            assert nmse(plug[i], g) <= mirror_bar, check_at[i]
+        n_past += T
+
+
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_backbone_cfg5_stack_step(gpu, ref, kv_f16):
+    """Batch 16 (8 streams x CFG pair), a KV cache that already holds 4100 seeded tokens (f16 as BASELINE config 5 names
+    it, and F32 as the reference allocates it), one decode step that appends token 4100, then a second step that reads it
+    back: 4 layers, plugin and mirror against ggml-cpu."""
+    import torch
+    N_LAYER, BATCH, PAST, MAX_LEN = 4, 16, 4100, 4160
+    say(f"cfg 5 stack: {N_LAYER} layers, batch {BATCH}, {'f16' if kv_f16 else 'F32'} KV cache holding {PAST} tokens, two decode steps")
+    params = reflib.backbone_params("bb5", N_LAYER)
+    xs = [rng("bb5", "x", i).standard_normal((BATCH, 1, 1024)).astype(np.float32) for i in range(2)]
+    dt = np.float16 if kv_f16 else np.float32
+    caches = {}
+    for li in range(N_LAYER):
+        for w in (0, 1):
+            c = np.zeros((BATCH, 2, MAX_LEN, 64), dt)
+            c[:, :, :PAST] = rng("bb5", "cache", li, w).standard_normal((BATCH, 2, PAST, 64)).astype(dt)
+            caches[(li, w)] = c
+
+    def run(device, threads):
+        assert ref.rh_use_device(device, threads, 0) == 0
+        reflib.ref_backbone_create(params, MAX_LEN, BATCH, use_mup=True, kv_f16=kv_f16)
+        for (li, w), c in caches.items():
+            assert ref.rh_bb_cache_set(li, w, c.ctypes.data, c.nbytes) == 0
+        outs = [reflib.ref_backbone_forward(x, PAST + i, None)[0] for i, x in enumerate(xs)]
+        slot = np.empty_like(caches[(0, 0)])
+        assert ref.rh_bb_cache_get(N_LAYER - 1, 0, slot.ctypes.data, slot.nbytes) == 0
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return outs, slot
+
+    cpu, cpu_cache = run(b"CPU", 16)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug, plug_cache = run(b"GFX950_0", 8)
+    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    say(f"   plugin: {launches} launches for the decode step")
+    for i in range(2):
+        e = nmse(cpu[i], plug[i])
+        say(f"   plugin vs ggml-cpu, step {i}: nmse {e:.3e}")
+        assert np.isfinite(plug[i]).all() and e <= 2e-4
+    # the cache: the seeded past untouched, the two appended tokens close to ggml-cpu's
+    assert np.array_equal(plug_cache[:, :, :PAST], caches[(N_LAYER - 1, 0)][:, :, :PAST])
+    new_cpu, new_plug = cpu_cache[:, :, PAST:PAST + 2].astype(np.float32), plug_cache[:, :, PAST:PAST + 2].astype(np.float32)
+    assert np.abs(new_plug).max() > 0 and nmse(new_cpu, new_plug) <= 2e-4
+    assert not plug_cache[:, :, PAST + 2:].any()
+
+    m = load_mirror(gpu, params, N_LAYER, MAX_LEN, BATCH, True, kv_f16, gpu.ACT_FLOAT)
+    for li in range(N_LAYER):
+        m.k_cache[li].copy_(torch.from_numpy(caches[(li, 0)]).cuda())
+        m.v_cache[li].copy_(torch.from_numpy(caches[(li, 1)]).cuda())
+    for i, x in enumerate(xs):
+        run_, got = m.plan(torch.from_numpy(x).cuda(), 1, PAST + i, None)
+        run_()
+        torch.cuda.synchronize()
+        g = got.cpu().numpy()
+        e = nmse(cpu[i], g)
+        say(f"   mirror vs ggml-cpu, step {i}: nmse {e:.3e} ({run_.n_calls} calls)")
+        assert e <= 2e-4
+        say(f"      mirror == plugin bit for bit: {np.array_equal(g, plug[i])}")
+        assert nmse(plug[i], g) <= 1e-6
+
+
+def test_fa_cfg5_prefill_b16_t4096(gpu):
+    """The 16 x 4096-token causal prefill attention of config 5 (f16 K/V) on the LDS-tiled kernel: every output finite
+    and inside the convex hull of its stream's V, and sampled (stream, row) pairs against the oracle -- row r of a causal
+    prefill is a decode attention over keys 0..r."""
+    import torch
+    B, Hq, Hkv, T, D = 16, 16, 2, 4096, 64
+    say(f"cfg 5 prefill attention: B={B}, T={T}, {Hq}/{Hkv} heads, f16 K/V, causal")
+    q = torch.from_numpy(rng("cfg5pf", "q").standard_normal((B, Hq, T, D)).astype(np.float32)).cuda()
+    k = rng("cfg5pf", "k").standard_normal((B, Hkv, T, D)).astype(np.float16)
+    v = rng("cfg5pf", "v").standard_normal((B, Hkv, T, D)).astype(np.float16)
+    mask = torch.from_numpy(reflib.causal_mask(T, T)).cuda()
+    out = gpu.flash_attn_ext(q, torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), mask, 0.125)   # (B, T, Hq, D)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    vf = torch.from_numpy(v.astype(np.float32)).cuda()
+    vmin = torch.cummin(vf, dim=2).values   # (B, Hkv, T, D): hull of keys 0..r
+    vmax = torch.cummax(vf, dim=2).values
+    for h in range(Hq):
+        o = out[:, :, h]                     # (B, T, D)
+        assert bool((o >= vmin[:, h // 8] - 2e-3).all()) and bool((o <= vmax[:, h // 8] + 2e-3).all()), h
+    gen = rng("cfg5pf", "rows")
+    pairs = [(0, 0), (0, 1), (15, T - 1), (7, 63), (7, 64), (3, 2047), (3, 2048)] + \
+            [(int(gen.integers(B)), int(gen.integers(T))) for _ in range(25)]
+    worst = 0.0
+    qh = q.cpu().numpy()
+    for b, r in pairs:
+        want = reflib.oracle_fa(qh[b:b + 1, :, r:r + 1], k[b:b + 1, :, :r + 1].astype(np.float32), v[b:b + 1, :, :r + 1].astype(np.float32))
+        err = float(np.abs(out[b, r].cpu().numpy() - want[0, 0]).max())
+        worst = max(worst, err)
+        assert err <= 2e-3, (b, r, err)
+    say(f"   {len(pairs)} sampled rows against the oracle: worst max-abs {worst:.3e}")

@@ -76,12 +76,14 @@ int standalone_unary_code(ggml_op op) {
     }
 }
 
+// how activations enter a Q8_0 product: the environment's choice at load time, or a later ggml_backend_gfx950_set_mul_mat_act
+int g_mul_mat_act = -1;
 int mul_mat_act_mode() {
-    static const int mode = [] {
+    if (g_mul_mat_act < 0) {
         const char * e = getenv("GGML_GFX950_MUL_MAT_ACT");
-        return (e && strcmp(e, "q8") == 0) ? VX_ACT_Q8 : VX_ACT_FLOAT;
-    }();
-    return mode;
+        g_mul_mat_act = (e && strcmp(e, "q8") == 0) ? VX_ACT_Q8 : VX_ACT_FLOAT;
+    }
+    return g_mul_mat_act;
 }
 
 // --------------------------------------------------------------------- per-device state
@@ -1395,3 +1397,10 @@ GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_
 // Diagnostic: how many operator calls the most recent graph_compute of this process issued (an attention
 // call counts once although it may launch a split and a merge kernel).
 extern "C" __attribute__((visibility("default"))) int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
+// Selects VX_ACT_FLOAT (0) or VX_ACT_Q8 (1) for the Q8_0 products of later graph_compute calls; returns the previous
+// mode.  The environment variable GGML_GFX950_MUL_MAT_ACT=q8 sets the initial one.
+extern "C" __attribute__((visibility("default"))) int ggml_backend_gfx950_set_mul_mat_act(int mode) {
+    const int before = mul_mat_act_mode();
+    if (mode == VX_ACT_FLOAT || mode == VX_ACT_Q8) g_mul_mat_act = mode;
+    return before;
+}
