@@ -238,8 +238,10 @@ VX_API vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor * k
 /* CONCAT(k_past, k_cur, dim 1) , CONCAT(v_past, v_cur, dim 1) -> FLASH_ATTN_EXT: the reference appends the step's
  * keys and values to the cached ones before attention (attention_forward, src/minicpm.cpp:694-706).  Here the
  * kernel reads keys 0 .. ne1(k_past)-1 from k_past / v_past and the rest from k_cur / v_cur, so the
- * concatenated tensors are never written.  Both segments of one type, head_dim, head and batch counts; mask
- * over all keys.  Query counts the LDS-tiled prefill kernel would take are not supported (use CONCAT).
+ * concatenated tensors are never written.  Both segments of one type -- or k_past / v_past F16 (an F16 cache) and
+ * k_cur / v_cur F32 (the step's keys as the projections left them; head_dim 64): the kernel then rounds them to f16,
+ * to nearest even, as it loads them, which is what a CPY node to an F16 tensor in front of the CONCAT stores --, same
+ * head_dim, head and batch counts; mask over all keys.  Query counts the LDS-tiled prefill kernel would take are not supported (use CONCAT).
  * Result identical to vx_concat x2 + vx_flash_attn_ext. */
 VX_API vx_status vx_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
                                        const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
@@ -252,8 +254,9 @@ VX_API int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tensor *
  * followed by vx_kv_store_sync on its result, with the cache write and the ordering scalar folded into the kernel
  * that merges the key-range partials.  k_src / v_src are the CPY sources (the values of k_cur / v_cur in the shape
  * the reference copies them), k_slot / v_slot the cache views written; sync_scale / sync_bias the SCALE node's
- * parameters.  Needs more than 256 keys in all (the split path).  Result and cache contents equal the two
- * separate calls'. */
+ * parameters.  Needs more than 256 keys in all (the split path).  The slots may be F32 or F16; an F16 slot receives
+ * the values rounded to nearest even and the ordering sums are taken over the rounded values (the slot read back as
+ * F32).  Result and cache contents equal the two separate calls'. */
 VX_API vx_status vx_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_tensor * k_past, const vx_tensor * k_cur,
                                              const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
                                              const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
@@ -312,8 +315,10 @@ VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor
 /* The reference's KV append with its write-ordering scalar (attention_forward, src/minicpm.cpp:682-713), nine graph
  * nodes as one launch:  CPY(k, k_slot) CONT SUM , CPY(v, v_slot) CONT SUM , ADD , SCALE(scale, bias) , ADD1(x, .)
  *   k_slot <- k ; v_slot <- v ; dst = x + ((sum(k_slot) + sum(v_slot)) * scale + bias)
- * All F32; a cache write of at most 16384 elements (decode-sized), x of at most 65536; k_slot / v_slot with
- * dense rows.  The sums are formed in vx_sum's order, so dst equals what the separate nodes give. */
+ * k, v, x F32; a cache write of at most 16384 elements (decode-sized), x of at most 65536; k_slot / v_slot with
+ * dense rows, F32 or F16.  With F16 slots the node sequence is CPY(k, k_slot) CPY(k_slot -> F32) SUM ...: the values are
+ * rounded to nearest even on the way in and the sums see the rounded values.  The sums are formed in vx_sum's order,
+ * so dst equals what the separate nodes give. */
 VX_API vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                   const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream);
 VX_API int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,

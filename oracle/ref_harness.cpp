@@ -290,11 +290,11 @@ ggml_tensor * bb_layer_forward(ggml_context * c, const backbone & m, const bb_la
         ggml_tensor * vw = ggml_cpy(c, v, write_view(L.vc));
         if (L.kc->type == GGML_TYPE_F32) {
             kv_sync = ggml_add(c, ggml_sum(c, ggml_cont(c, kw)), ggml_sum(c, ggml_cont(c, vw)));
-            kv_sync = ggml_scale(c, kv_sync, 0.0f);
-        } else { // the ordering chain is typed for the F32 cache; an F16 cache appends as extra graph roots
-            roots.push_back(kw);
-            roots.push_back(vw);
+        } else { // an F16 cache: SCALE and ADD1 are F32 operators in ggml, so the written slots are read back as F32 for the sums
+            kv_sync = ggml_add(c, ggml_sum(c, ggml_cast(c, kw, GGML_TYPE_F32)), ggml_sum(c, ggml_cast(c, vw, GGML_TYPE_F32)));
         }
+        kv_sync = ggml_scale(c, kv_sync, 0.0f);
+        (void) roots;
     }
     ggml_tensor * k_all = ggml_permute(c, k, 0, 2, 1, 3);
     ggml_tensor * v_all = ggml_permute(c, v, 0, 2, 1, 3);

@@ -225,7 +225,11 @@ def test_supports_truth_table_node_groups(pkg):
     k_src, slot = f32(pkg, [Dh, Hkv, 1, 2]), D(pkg, pkg.F32, [Dh, Hkv, 1, 2], [4, 4 * Dh * 768, 4 * Dh, 4 * Dh * 768 * Hkv])
     attn = f32(pkg, [Dh, H, 1, 2])
     assert lib.vx_supports_kv_store_sync(k_src, slot, k_src, slot, attn, attn) == 1
-    assert lib.vx_supports_kv_store_sync(k_src, f16(pkg, [Dh, Hkv, 1, 2]), k_src, slot, attn, attn) == 0      # F16 cache
+    slot16 = D(pkg, pkg.F16, [Dh, Hkv, 1, 2], [2, 2 * Dh * 768, 2 * Dh, 2 * Dh * 768 * Hkv])
+    assert lib.vx_supports_kv_store_sync(k_src, slot16, k_src, slot16, attn, attn) == 1                         # F16 cache: rounded on the way
+    assert lib.vx_supports_kv_store_sync(k_src, D(pkg, pkg.F16, [Dh, Hkv, 1, 2], [2, 2 * Dh * 768, 2 * Dh, 2 * Dh * 768 * Hkv], 0x1002),
+                                         k_src, slot, attn, attn) == 0                                            # slot not 8-byte aligned
+    assert lib.vx_supports_kv_store_sync(f16(pkg, [Dh, Hkv, 1, 2]), slot16, k_src, slot, attn, attn) == 0       # F16 source
     big = f32(pkg, [Dh, Hkv, 512, 2])
     assert lib.vx_supports_kv_store_sync(big, big, big, big, attn, attn) == 0                                     # prefill-sized
     # attention over cached + current keys

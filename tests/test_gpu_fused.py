@@ -277,11 +277,112 @@ def test_flash_attn_two_segments_declines_prefill_shapes(pkg, gpu):
     o = torch.zeros((B, T, H, D), dtype=torch.float32, device="cuda")
     assert L.vx_supports_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(kp), d(kc), d(mask), d(o)) == 0
     assert L.vx_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(kp), d(kc), d(mask), None, d(o), 0.125, 0.0, 0.0, None) != 0
-    # mismatched segment types are refused as well
+    # an F32 cache with F16 current keys, and K / V segments of different kinds, are refused as well
     kc32 = kc[:, :, :1].float()
     q1 = q[:, :, :1].contiguous()
     o1 = torch.zeros((B, 1, H, D), dtype=torch.float32, device="cuda")
-    assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp), d(kc32), d(kp), d(kc32), None, d(o1)) == 0
+    assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp.float()), d(kc[:, :, :1]), d(kp.float()), d(kc[:, :, :1]), None, d(o1)) == 0
+    assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp), d(kc32), d(kp), d(kc[:, :, :1]), None, d(o1)) == 0
+    assert L.vx_supports_flash_attn_ext_kv2(d(q1), d(kp), d(kc32), d(kp), d(kc32), None, d(o1)) == 1   # F16 cache + the step's F32 keys
+
+
+@pytest.mark.parametrize("T,n_past,B", [(1, 639, 2), (1, 4095, 2), (1, 8191, 16), (1, 1, 2), (1, 31, 2), (1, 32, 2), (1, 33, 1), (2, 62, 2),
+                                        (5, 1000, 2), (40, 24, 2), (14, 300, 3)])
+def test_flash_attn_two_segments_f16_cache_f32_step(pkg, gpu, T, n_past, B):
+    """An F16 cache and the step's keys and values still in F32 (as the projections and the rotation left them): the
+    kernel rounds them to f16 as it loads them, so the result must equal CPY(F32 -> F16) x2, CONCAT x2, FLASH_ATTN_EXT
+    bit for bit."""
+    import torch
+    say(f"attention over an f16 cache + F32 current keys T={T} n_past={n_past} B={B}")
+    L, d = pkg.lib(), pkg.desc
+    H, Hkv, D = 16, 2, 64
+    g = rng("f-kv2m", T, n_past, B)
+    q = dev(g.standard_normal((B, H, T, D)).astype(np.float32))
+    cache_k = dev(g.standard_normal((B, Hkv, n_past + 3, D)).astype(np.float16))
+    cache_v = dev(g.standard_normal((B, Hkv, n_past + 3, D)).astype(np.float16))
+    kp, vp = cache_k[:, :, :n_past], cache_v[:, :, :n_past]
+    k32 = g.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    v32 = g.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    k32[0, 0, 0, :6] = [65504.0, 70000.0, 1e-8, 6.1e-5, -3.0e-8, 1.00048828125]   # f16 max, overflow, underflow, subnormals, a tie
+    kc, vc = dev(k32).transpose(1, 2), dev(v32).transpose(1, 2)          # ggml_permute(0, 2, 1, 3) of [D, Hkv, T, B]
+    n_kv = n_past + T
+    mask = dev(reflib.causal_mask(T, n_kv, n_past)) if T > 1 else None
+    k16 = torch.empty((B, Hkv, T, D), dtype=torch.float16, device="cuda")
+    v16 = torch.empty_like(k16)
+    kall = torch.empty((B, Hkv, n_kv, D), dtype=torch.float16, device="cuda")
+    vall = torch.empty_like(kall)
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    b = torch.full_like(a, 3.0)
+    ok(pkg, L.vx_cpy(d(kc), d(k16), None), "cast k")
+    ok(pkg, L.vx_cpy(d(vc), d(v16), None), "cast v")
+    ok(pkg, L.vx_concat(d(kp), d(k16), d(kall), 1, None), "concat k")
+    ok(pkg, L.vx_concat(d(vp), d(v16), d(vall), 1, None), "concat v")
+    ok(pkg, L.vx_flash_attn_ext(d(q), d(kall), d(vall), d(mask), None, d(a), 0.125, 0.0, 0.0, None), "fa")
+    assert L.vx_supports_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(vp), d(vc), d(mask), d(b)) == 1
+    ok(pkg, L.vx_flash_attn_ext_kv2(d(q), d(kp), d(kc), d(vp), d(vc), d(mask), None, d(b), 0.125, 0.0, 0.0, None), "fa_kv2 mixed")
+    torch.cuda.synchronize()
+    assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(5.0), b.nan_to_num(5.0))
+
+
+@pytest.mark.parametrize("T,n_past,B", [(1, 639, 2), (1, 300, 1), (1, 4100, 16), (3, 4000, 2), (1, 100, 2)])
+@pytest.mark.parametrize("poison", [None, "nan"])
+def test_f16_cache_write_with_ordering_scalar(pkg, gpu, T, n_past, B, poison):
+    """The cache write of attention_forward into an F16 cache: CPY(k -> f16 slot), CPY(slot -> F32), SUM (twice), ADD,
+    SCALE, ADD1 as separate nodes against vx_kv_store_sync, and -- with more than 256 keys -- against
+    vx_flash_attn_ext_kv2_store, which also reads the F32 keys of the step in place."""
+    import torch
+    say(f"f16 cache write with the ordering scalar T={T} n_past={n_past} B={B} {poison}")
+    L, d = pkg.lib(), pkg.desc
+    H, Hkv, D = 16, 2, 64
+    g = rng("f-kvs16", T, n_past, B)
+    q = dev(g.standard_normal((B, H, T, D)).astype(np.float32))
+    caches = [dev(g.standard_normal((B, Hkv, n_past + T + 5, D)).astype(np.float16)) for _ in range(2)]
+    caches += [c.clone() for c in caches] + [c.clone() for c in caches]
+    kc1, vc1, kc2, vc2, kc3, vc3 = caches
+    k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    if poison:
+        v[0, 0, 0, 3] = float("nan")
+    kcur, vcur = k.transpose(1, 2), v.transpose(1, 2)
+    mask = dev(reflib.causal_mask(T, n_past + T, n_past)) if T > 1 else None
+
+    def slot(c):
+        return c[:, :, n_past:n_past + T].transpose(1, 2)
+
+    for sync_scale, sync_bias in ((0.0, 0.0), (0.125, 0.5)):
+        # node by node
+        a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+        ok(pkg, L.vx_flash_attn_ext_kv2(d(q), d(kc1[:, :, :n_past]), d(kcur), d(vc1[:, :, :n_past]), d(vcur), d(mask), None, d(a), 0.125, 0.0, 0.0, None), "kv2")
+        cont = torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda")
+        sk, sv, sync = (torch.empty(1, dtype=torch.float32, device="cuda") for _ in range(3))
+        a1 = torch.empty_like(a)
+        for src, c, s_ in ((k, kc1, sk), (v, vc1, sv)):
+            ok(pkg, L.vx_cpy(d(src), d(slot(c)), None), "cpy")
+            ok(pkg, L.vx_cpy(d(slot(c)), d(cont), None), "cast back")
+            ok(pkg, L.vx_sum(d(cont), d(s_), None), "sum")
+        ok(pkg, L.vx_binary(pkg.BIN_ADD, d(sk), d(sv), d(sync), None), "add")
+        ok(pkg, L.vx_scale(d(sync), d(sync), sync_scale, sync_bias, None), "scale")
+        ok(pkg, L.vx_add1(d(a), d(sync), d(a1), None), "add1")
+        # the write group as one launch
+        b = torch.empty_like(a)
+        assert L.vx_supports_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(a), d(b)) == 1
+        ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(a), d(b), sync_scale, sync_bias, None), "kv_store_sync f16")
+        torch.cuda.synchronize()
+        assert same_bits(kc1, kc2) and same_bits(vc1, vc2)
+        assert torch.equal(torch.isnan(a1), torch.isnan(b)) and torch.equal(a1.nan_to_num(7.0), b.nan_to_num(7.0))
+        # attention + write as one call
+        c_ = torch.empty_like(a)
+        want = 1 if n_past + T > 256 else 0
+        assert L.vx_supports_flash_attn_ext_kv2_store(d(q), d(kc3[:, :, :n_past]), d(kcur), d(vc3[:, :, :n_past]), d(vcur), d(mask),
+                                                      d(k), d(slot(kc3)), d(v), d(slot(vc3)), d(c_)) == want
+        if want:
+            ok(pkg, L.vx_flash_attn_ext_kv2_store(d(q), d(kc3[:, :, :n_past]), d(kcur), d(vc3[:, :, :n_past]), d(vcur), d(mask), None,
+                                                  d(k), d(slot(kc3)), d(v), d(slot(vc3)), d(c_), 0.125, 0.0, 0.0, sync_scale, sync_bias, None), "kv2_store f16")
+            torch.cuda.synchronize()
+            assert same_bits(kc1, kc3) and same_bits(vc1, vc3)
+            assert torch.equal(torch.isnan(a1), torch.isnan(c_)) and torch.equal(a1.nan_to_num(7.0), c_.nan_to_num(7.0))
+    if not poison:
+        assert torch.equal(kc2[:, :, n_past:n_past + T], k.transpose(1, 2).to(torch.float16))
 
 
 @pytest.mark.parametrize("T,B,H,Hkv,D,K", [(1, 2, 16, 2, 64, 1024), (1, 1, 16, 2, 64, 1024), (3, 2, 8, 8, 128, 512), (16, 1, 4, 1, 32, 256), (14, 8, 16, 2, 64, 1024), (21, 1, 16, 2, 64, 1024)])

@@ -122,9 +122,9 @@ class MiniCPMBackbone:
 
         # buffers reused by every layer (the stack is sequential)
         normed, q, k, v = new(N, self.hidden), new(N, H * D), new(N, Hkv * D), new(N, Hkv * D)
-        kcont, vcont = new(B, T, Hkv, D, dtype=self.kv_dtype), new(B, T, Hkv, D, dtype=self.kv_dtype)
-        sk, sv = new(1, dtype=self.kv_dtype), new(1, dtype=self.kv_dtype)
-        sync = new(1, dtype=self.kv_dtype)
+        kcont, vcont = new(B, T, Hkv, D), new(B, T, Hkv, D)   # the written slot as dense F32 (CONT, or the cast back from F16)
+        sk, sv = new(1), new(1)
+        sync = new(1)
         kall = new(B, Hkv, seq_len, D, dtype=self.kv_dtype) if n_past > 0 else None
         vall = new(B, Hkv, seq_len, D, dtype=self.kv_dtype) if n_past > 0 else None
         kcast = new(B, Hkv, T, D, dtype=self.kv_dtype) if (n_past > 0 and self.kv_dtype != f32) else None
@@ -135,10 +135,11 @@ class MiniCPMBackbone:
         h_mid = new(N, self.hidden)
         out = new(B, T, self.hidden)
         keep += [normed, q, k, v, kcont, vcont, sk, sv, sync, kall, vall, kcast, vcast, attn, attn_o, gate, up, act, down, h_mid, out] + hs
-        # The cont/sum/scale-by-zero chain only exists to order the cache write inside a ggml graph
-        # and is typed for the reference's F32 cache (ggml's SCALE and ADD1 are F32 operators); with an
-        # F16 cache the append is the bare ggml_cpy, ordered by the stream.
-        chain = write_kv and self.kv_dtype == f32
+        # The cont/sum/scale-by-zero chain only exists to order the cache write inside a ggml graph.  It is typed
+        # F32 (ggml's SCALE and ADD1 are F32 operators): with an F16 cache the written slot is read back through a
+        # cast to F32 where the F32 cache has its CONT.
+        chain = write_kv
+        f16_cache = self.kv_dtype != f32
         scale = 1.0 / math.sqrt(D)
         ff = _p(self.rope_factors)
         cur_x = x.view(N, self.hidden)
@@ -149,9 +150,10 @@ class MiniCPMBackbone:
             # -- attention_forward
             q4, k4, v4 = q.view(B, T, H, D), k.view(B, T, Hkv, D), v.view(B, T, Hkv, D)
             rope_args = (D, 2, self.rope_original_max, self.rope_base, 1.0, 0.0, attn_factor, 32.0, 1.0)
-            # (with an F16 cache the reference's graph casts the rotated keys between the K and V projections; the plugin
-            # only groups the projections when no other node runs between them)
-            plain_order = n_past == 0 or self.kv_dtype == f32
+            # (with an F16 cache the graph casts the rotated keys between the K and V projections; the plugin only groups
+            # the projections when no other node runs between them, i.e. when attention reads the F32 keys in place and
+            # the casts are never run -- which needs the keys alive at the attention node: a step that writes the cache)
+            plain_order = n_past == 0 or not f16_cache or write_kv
             wqkv = (wd["q_proj"], wd["k_proj"], wd["v_proj"])
             nw_in = nrm["input_layernorm"]
             if fuse and plain_order and L.vx_supports_norm_qkv_proj_rope(desc(cur_x), desc(nw_in), *wqkv, desc(q4), desc(k4), desc(v), D, 2):
@@ -173,17 +175,17 @@ class MiniCPMBackbone:
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)
             stored = False
             if n_past > 0:
-                if kcast is not None:
+                kp, vp = kc[:, :, :n_past], vc[:, :, :n_past]
+                qd = desc(q4.transpose(1, 2))
+                # The plugin lets attention read the cached and the current keys where they lie (no concat, and with an
+                # F16 cache no cast: the kernel rounds the F32 keys as it loads them) when the current keys are still
+                # alive at the attention node.  In the reference's graph they are when the cache write, their other
+                # reader, comes later: a step that writes the cache.
+                alive = write_kv
+                if not (fuse and alive) and kcast is not None:
                     call(L.vx_cpy, desc(k_all), desc(kcast))
                     call(L.vx_cpy, desc(v_all), desc(vcast))
                     k_all, v_all = kcast, vcast
-                kp, vp = kc[:, :, :n_past], vc[:, :, :n_past]
-                qd = desc(q4.transpose(1, 2))
-                # The plugin lets attention read the cached and the current keys where they lie (no concat) when the
-                # current keys are still alive at the attention node.  In the reference's graph they are when the
-                # cache write, their other reader, comes later: F32 cache with write_kv.  The F16 cast of the
-                # current keys dies at the concat and ggml-alloc hands its memory on, so there the concats stay.
-                alive = write_kv and kcast is None
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # the cache's write views, ggml [D, Hkv, T, B]
                 vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
                 if fuse and alive and L.vx_supports_flash_attn_ext_kv2_store(qd, desc(kp), desc(k_all), desc(vp), desc(v_all), desc(mask),
@@ -199,6 +201,10 @@ class MiniCPMBackbone:
                          scale, 0.0, 0.0)
                     k_all = None
                 else:
+                    if k_all.dtype != kp.dtype:   # (a shape the two-segment kernel leaves to the tiled one)
+                        call(L.vx_cpy, desc(k_all), desc(kcast))
+                        call(L.vx_cpy, desc(v_all), desc(vcast))
+                        k_all, v_all = kcast, vcast
                     call(L.vx_concat, desc(kp), desc(k_all), desc(kall), 1)
                     call(L.vx_concat, desc(vp), desc(v_all), desc(vall), 1)
                     k_all, v_all = kall, vall
@@ -218,7 +224,7 @@ class MiniCPMBackbone:
             elif write_kv:
                 for src4, wv, cont, ssum in ((k4, kw, kcont, sk), (v4, vw, vcont, sv)):
                     call(L.vx_cpy, desc(src4), desc(wv))
-                    if chain and fuse:
+                    if chain and fuse and not f16_cache:
                         call(L.vx_sum, desc(wv), desc(ssum))       # cont + sum
                     elif chain:
                         call(L.vx_cpy, desc(wv), desc(cont))

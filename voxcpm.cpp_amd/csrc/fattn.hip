@@ -59,6 +59,7 @@ struct fa_args {
     const char * k2; const char * v2;
     uint64_t nbk1b, nbk2b, nbk3b, nbv1b, nbv2b, nbv3b;
     int n_kv1;
+    int seg2_f32; // the second segment holds F32 values while the first is an F16 cache (rounded to f16 as they are loaded)
     int n_q, n_kv, Hq, Hkv, gqa, ne3, rk3, nem2, nem3;
     int n_col_tiles, n_splits, chunk;
     float scale, softcap, max_bias, m0, m1;
@@ -124,7 +125,11 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
 }
 
 // One wave (= one block) = 16 columns x one key range.
-template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP, bool TWO_SEG>
+// TWO_SEG: 0 = K and V are one tensor each; 1 = keys from n_kv1 on lie in a second pair of tensors of the same type;
+// 2 = the first pair is an F16 cache and the second pair F32 (the step's own keys and values, as the projections
+// left them): they are rounded to f16, to nearest even, while they are loaded -- exactly what a CPY node to an F16
+// tensor in front of a CONCAT would have stored.
+template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP, int TWO_SEG>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fattn_cols16_kernel(const fa_args a) {
     constexpr int NP  = D / 32;          // MFMAs along the head dimension
     constexpr int SEG = D / 4;           // elements of a row owned by lane-group j
@@ -151,22 +156,29 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 
     const char * kbase2 = kbase;
     const char * vbase2 = vbase;
-    if constexpr (TWO_SEG) {
-        kbase2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) (b / a.rk3) * a.nbk3b + (uint64_t) (SEG * j) * ES;
-        vbase2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) (b / a.rk3) * a.nbv3b + (uint64_t) (SEG * j) * ES;
+    if constexpr (TWO_SEG != 0) {
+        constexpr int ES2 = TWO_SEG == 2 ? 4 : ES;
+        kbase2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) (b / a.rk3) * a.nbk3b + (uint64_t) (SEG * j) * ES2;
+        vbase2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) (b / a.rk3) * a.nbv3b + (uint64_t) (SEG * j) * ES2;
     }
 
     const int kv0 = sp * a.chunk;
     const int kv1 = min(a.n_kv, kv0 + a.chunk);
+    // Mixed types: 32-key tiles that lie wholly in the cache (tile starts below `pure`) stream through the pipelined
+    // loop; the tile that straddles the boundary and any tile behind it -- one tile in all at decode -- are loaded
+    // lane by lane from whichever tensor holds the key.  Key ranges start at multiples of 32, so tiles do too.
+    const int pure   = TWO_SEG == 2 ? a.n_kv1 / 32 * 32 : 0;
+    const int kv1p   = TWO_SEG == 2 ? min(kv1, pure) : kv1;  // end of the pipelined tiles
+    const int kclamp = TWO_SEG == 2 ? a.n_kv1 - 1 : a.n_kv - 1;
 
     // rows this lane loads (MFMA row c of each 16-key half); clamped, masked out later
     auto load_tile = [&](int kb, kv_tile<NP, KV_F32> & t) {
-        const int key0 = min(kb + c, a.n_kv - 1), key1 = min(kb + 16 + c, a.n_kv - 1);
+        const int key0 = min(kb + c, kclamp), key1 = min(kb + 16 + c, kclamp);
         const char * k0p = kbase + (uint64_t) key0 * a.nbk1;
         const char * k1p = kbase + (uint64_t) key1 * a.nbk1;
         const char * v0p = vbase + (uint64_t) key0 * a.nbv1;
         const char * v1p = vbase + (uint64_t) key1 * a.nbv1;
-        if constexpr (TWO_SEG) {
+        if constexpr (TWO_SEG == 1) {
             if (key0 >= a.n_kv1) { k0p = kbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbk1b; v0p = vbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbv1b; }
             if (key1 >= a.n_kv1) { k1p = kbase2 + (uint64_t) (key1 - a.n_kv1) * a.nbk1b; v1p = vbase2 + (uint64_t) (key1 - a.n_kv1) * a.nbv1b; }
         }
@@ -182,9 +194,45 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         }
     };
 
+    // a tile at or behind the type boundary: each lane reads its two keys from the tensor that holds them
+    auto load_mixed = [&](int kb, kv_tile<NP, KV_F32> & t) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int key = min(kb + 16 * h + c, a.n_kv - 1);
+            if (key < a.n_kv1) {
+                const char * kp = kbase + (uint64_t) key * a.nbk1;
+                const char * vp = vbase + (uint64_t) key * a.nbv1;
+#pragma unroll
+                for (int p = 0; p < NP; ++p) {
+                    kv_load<KV_F32>::run(kp + p * 8 * ES, t.khi[h][p], t.klo[h][p]);
+                    kv_load<KV_F32>::run(vp + p * 8 * ES, t.vhi[h][p], t.vlo[h][p]);
+                }
+            } else {
+                const char * kp = kbase2 + (uint64_t) (key - a.n_kv1) * a.nbk1b;
+                const char * vp = vbase2 + (uint64_t) (key - a.n_kv1) * a.nbv1b;
+#pragma unroll
+                for (int p = 0; p < NP; ++p) {
+                    const float4_t ka = ((const float4_t *) (kp + p * 32))[0], kb4 = ((const float4_t *) (kp + p * 32))[1];
+                    const float4_t va = ((const float4_t *) (vp + p * 32))[0], vb4 = ((const float4_t *) (vp + p * 32))[1];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        t.khi[h][p][i] = (_Float16) ka[i]; t.khi[h][p][4 + i] = (_Float16) kb4[i];
+                        t.vhi[h][p][i] = (_Float16) va[i]; t.vhi[h][p][4 + i] = (_Float16) vb4[i];
+                    }
+                }
+            }
+        }
+    };
+
     // two tiles alternate in registers: while one is consumed the other is in flight
-    kv_tile<NP, KV_F32> t0, t1;
-    load_tile(kv0, t0);
+    kv_tile<NP, KV_F32> t0, t1, t2;
+    const int kmix = max(kv0, pure); // first tile of the lane-by-lane part (TWO_SEG == 2)
+    if constexpr (TWO_SEG == 2) {
+        if (kmix < kv1) load_mixed(kmix, t2);  // requested first, consumed last
+        if (kv0 < kv1p) load_tile(kv0, t0);
+    } else {
+        load_tile(kv0, t0);
+    }
 
     // ---- Q^T operand: column c, elements d = SEG*j + 8p + i, split into hi + lo
     half8_t qhi[NP], qlo[NP];
@@ -327,13 +375,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     // cache hit) so that the wait before each use counts a fixed number of younger loads; a
     // conditional prefetch forces the compiler to wait for everything and exposes the whole
     // memory latency in every iteration.
-    const int klast = kv0 + ((kv1 - kv0 - 1) / 32) * 32;
-    for (int kb = kv0; kb < kv1; kb += 64) {
+    const int klast = kv0 + ((kv1p - kv0 - 1) / 32) * 32;
+    for (int kb = kv0; kb < kv1p; kb += 64) {
         load_tile(min(kb + 32, klast), t1);
         consume(t0, kb);
-        if (kb + 32 >= kv1) break;
+        if (kb + 32 >= kv1p) break;
         load_tile(min(kb + 64, klast), t0);
         consume(t1, kb + 32);
+    }
+    if constexpr (TWO_SEG == 2) {
+        for (int kb = kmix; kb < kv1; kb += 32) {
+            if (kb != kmix) load_mixed(kb, t2);
+            consume(t2, kb);
+        }
     }
 
     l += __shfl_xor(l, 16, 64);
@@ -505,18 +559,26 @@ int64_t fa_tiles(const vx_tensor * q, const vx_tensor * k) {
 template <int D, bool KV_F32>
 void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
     const dim3 grid((unsigned) nblocks), block(64);
+    if constexpr (D == 64 && !KV_F32) {
+        if (a.k2 && a.seg2_f32) { // an F16 cache and the step's F32 keys
+            if (a.softcap != 0.0f) fattn_cols16_kernel<D, false, true, true, 2><<<grid, block, 0, st>>>(a);
+            else if (a.mask)       fattn_cols16_kernel<D, false, true, false, 2><<<grid, block, 0, st>>>(a);
+            else                   fattn_cols16_kernel<D, false, false, false, 2><<<grid, block, 0, st>>>(a);
+            return;
+        }
+    }
     if (a.k2) {
-        if (a.softcap != 0.0f) fattn_cols16_kernel<D, KV_F32, true, true, true><<<grid, block, 0, st>>>(a);
-        else if (a.mask)       fattn_cols16_kernel<D, KV_F32, true, false, true><<<grid, block, 0, st>>>(a);
-        else                   fattn_cols16_kernel<D, KV_F32, false, false, true><<<grid, block, 0, st>>>(a);
+        if (a.softcap != 0.0f) fattn_cols16_kernel<D, KV_F32, true, true, 1><<<grid, block, 0, st>>>(a);
+        else if (a.mask)       fattn_cols16_kernel<D, KV_F32, true, false, 1><<<grid, block, 0, st>>>(a);
+        else                   fattn_cols16_kernel<D, KV_F32, false, false, 1><<<grid, block, 0, st>>>(a);
         return;
     }
     if (a.softcap != 0.0f) { // rare: always take the masked variant
-        fattn_cols16_kernel<D, KV_F32, true, true, false><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, true, true, 0><<<grid, block, 0, st>>>(a);
     } else if (a.mask) {
-        fattn_cols16_kernel<D, KV_F32, true, false, false><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, true, false, 0><<<grid, block, 0, st>>>(a);
     } else {
-        fattn_cols16_kernel<D, KV_F32, false, false, false><<<grid, block, 0, st>>>(a);
+        fattn_cols16_kernel<D, KV_F32, false, false, 0><<<grid, block, 0, st>>>(a);
     }
 }
 
@@ -588,8 +650,10 @@ extern "C" vx_status vx_flash_attn_ext_add1(const vx_tensor * q, const vx_tensor
 
 // CONCAT(k_past, k_cur) , CONCAT(v_past, v_cur) , FLASH_ATTN_EXT as one launch that reads both segments
 // where they lie.  The whole of K (V) has the first segment's shape with ne[1] = the two key counts added.
+// The second segment may be F32 behind an F16 first one (head_dim 64): the step's keys as the projections left them.
 static bool kv2_whole(const vx_tensor * a, const vx_tensor * b, vx_tensor * whole) {
-    if (!a || !b || a->type != b->type || !vx_positive(a) || !vx_positive(b)) return false;
+    if (!a || !b || !vx_positive(a) || !vx_positive(b)) return false;
+    if (a->type != b->type && !(a->type == VX_TYPE_F16 && b->type == VX_TYPE_F32 && a->ne[0] == 64)) return false;
     if (a->ne[0] != b->ne[0] || a->ne[2] != b->ne[2] || a->ne[3] != b->ne[3]) return false;
     if (b->nb[0] != vx_type_size(b->type)) return false;
     for (int i = 1; i < 4; ++i) if (b->nb[i] % 16) return false;
@@ -603,7 +667,7 @@ extern "C" int vx_supports_flash_attn_ext_kv2(const vx_tensor * q, const vx_tens
                                               const vx_tensor * dst) {
     vx_tensor kall, vall;
     if (!q || !kv2_whole(k_past, k_cur, &kall) || !kv2_whole(v_past, v_cur, &vall)) return 0;
-    if (k_past->ne[1] != v_past->ne[1]) return 0;
+    if (k_past->ne[1] != v_past->ne[1] || k_cur->type != v_cur->type) return 0;
     if (!vx_supports_flash_attn_ext(q, &kall, &vall, mask, dst)) return 0;
     // a shape the LDS-tiled kernel would take as one tensor stays with it (same results either way)
     return vx_fattn_prefill_accepts(q, &kall, 0.0f) ? 0 : 1;
@@ -729,6 +793,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     a.nbk1b = k2 ? k2->nb[1] : 0; a.nbk2b = k2 ? k2->nb[2] : 0; a.nbk3b = k2 ? k2->nb[3] : 0;
     a.nbv1b = v2 ? v2->nb[1] : 0; a.nbv2b = v2 ? v2->nb[2] : 0; a.nbv3b = v2 ? v2->nb[3] : 0;
     a.n_kv1 = (int) k->ne[1];
+    a.seg2_f32 = k2 && k2->type == VX_TYPE_F32 && k->type == VX_TYPE_F16;
     a.q = (const char *) q->data; a.k = (const char *) k->data; a.v = (const char *) v->data;
     a.mask = mask ? (const char *) mask->data : nullptr;
     a.sinks = sinks;

@@ -3,27 +3,40 @@
 #pragma once
 #include "vx_common.hpp"
 
-// one cache write: source tensor (F32, any strides) -> slot view of the cache (F32, dense rows); element i
-// of the source in its own row-major order goes to element i of the slot in the slot's
+// one cache write: source tensor (F32, any strides) -> slot view of the cache (F32 or F16, dense rows); element i
+// of the source in its own row-major order goes to element i of the slot in the slot's.  With an F16 cache the value
+// is rounded to nearest even on the way (what GGML_OP_CPY does) and the ordering sum adds the ROUNDED values in fp64:
+// the sum of the slot read back as F32, i.e. of the node sequence CPY(k, slot) , CPY(slot -> F32) , SUM.
 struct kvs_side {
     const char * s; char * d;
     int64_t  nes[4], ned[4];
     uint64_t nbs[4], nbd[4];
-    int vec; // slot rows allow 16-byte accesses: the test vx_sum applies to its operand
+    int vec; // units of 4 elements: the test vx_sum applies to the tensor it sums (the slot view, or its dense F32 copy)
     int src_dense; // the source is contiguous in its own order (element i at byte 4 i) and 16-byte aligned
+    int dst_f16;
 };
 
 // host side: what one cache write may look like, and its kernel argument
 static inline bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot) {
-    if (!src || !slot || src->type != VX_TYPE_F32 || slot->type != VX_TYPE_F32 || !vx_positive(src)) return false;
+    if (!src || !slot || src->type != VX_TYPE_F32 || (slot->type != VX_TYPE_F32 && slot->type != VX_TYPE_F16) || !vx_positive(src)) return false;
     if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > 16384) return false;
-    for (int i = 0; i < 4; ++i) if (src->nb[i] % 4 || slot->nb[i] % 4) return false;
+    for (int i = 0; i < 4; ++i) if (src->nb[i] % 4) return false;
+    if (slot->type == VX_TYPE_F16) {
+        // the sum is taken over a dense F32 copy of the slot (vx_sum's 4-element units need ne0 % 4 == 0 only); the
+        // stores are 8 bytes wide
+        if (slot->nb[0] != 2 || slot->ne[0] % 4 || (uintptr_t) slot->data % 8) return false;
+        for (int i = 1; i < 4; ++i) if (slot->nb[i] % 8) return false;
+        return true;
+    }
+    for (int i = 0; i < 4; ++i) if (slot->nb[i] % 4) return false;
     return slot->nb[0] == 4;
 }
 static inline void kvs_side_fill(kvs_side & o, const vx_tensor * src, const vx_tensor * slot) {
     o.s = (const char *) src->data; o.d = (char *) slot->data;
     for (int i = 0; i < 4; ++i) { o.nes[i] = src->ne[i]; o.ned[i] = slot->ne[i]; o.nbs[i] = src->nb[i]; o.nbd[i] = slot->nb[i]; }
+    o.dst_f16 = slot->type == VX_TYPE_F16;
     o.vec = slot->ne[0] % 4 == 0 && (uintptr_t) slot->data % 16 == 0 && slot->nb[1] % 16 == 0 && slot->nb[2] % 16 == 0 && slot->nb[3] % 16 == 0;
+    if (o.dst_f16) o.vec = 1; // kvs_side_ok has checked what the 8-byte stores need
     o.src_dense = vx_is_contiguous(src) && (uintptr_t) src->data % 16 == 0;
 }
 
@@ -50,13 +63,24 @@ __device__ __forceinline__ void kvs_unit(const kvs_side & a, uint32_t e, bool st
             v[k] = *(const float *) (a.s + j0 * a.nbs[0] + j1 * a.nbs[1] + j2 * a.nbs[2] + j3 * a.nbs[3]);
         }
     }
+    _Float16 h[W];
+    if (a.dst_f16) { // uniform: the slot holds halves; the sum below sees what a reader of the slot would
+#pragma unroll
+        for (int k = 0; k < W; ++k) { h[k] = (_Float16) v[k]; v[k] = (float) h[k]; }
+    }
     if (store) {
         const uint32_t ne1 = (uint32_t) a.ned[1], ne2 = (uint32_t) a.ned[2];
         const uint32_t row = e / per_row, iv = e - row * per_row;
         const uint32_t i1 = row % ne1, r2 = row / ne1, i2 = r2 % ne2, i3 = r2 / ne2;
-        char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
-        if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
-        else               *(float *) pd = v[0];
+        if (a.dst_f16) {
+            char * pd = a.d + (uint64_t) iv * (2 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+            if constexpr (VEC) *(half4_t *) pd = half4_t{h[0], h[1], h[2], h[3]};
+            else               *(_Float16 *) pd = h[0];
+        } else {
+            char * pd = a.d + (uint64_t) iv * (4 * W) + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+            if constexpr (VEC) *(float4_t *) pd = float4_t{v[0], v[1], v[2], v[3]};
+            else               *(float *) pd = v[0];
+        }
     }
 #pragma unroll
     for (int k = 0; k < W; ++k) acc += (double) v[k];

@@ -619,6 +619,13 @@ bool private_to_group(const reader_map & readers, const ggml_tensor * t) {
     return (t->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (t->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 && it != readers.end() && it->second == 1;
 }
 
+// the same for the result of ggml_cast, a CPY node that names itself as its second operand (one reader more)
+bool private_cast_node(const reader_map & readers, const ggml_tensor * t) {
+    const auto it = readers.find(t);
+    return t->op == GGML_OP_CPY && t->src[1] == t && (t->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && (t->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 &&
+           it != readers.end() && it->second == 2;
+}
+
 // index of the next node that does work (views and empty tensors are skipped), or n_nodes
 int next_real(const ggml_cgraph * g, int i) {
     int k = i + 1;
@@ -638,17 +645,28 @@ int match_kv_store_group(const ggml_cgraph * g, int i, const reader_map & reader
         if ((n[k]->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return -1;
         if (k < 8) idx = next_real(g, idx);
     }
+    // (with an F16 cache the sums are typed F32 through a cast of the written slot, CPY to a new F32 tensor, where the F32
+    // cache has its CONT)
     static const ggml_op want[9] = { GGML_OP_CPY, GGML_OP_CONT, GGML_OP_SUM, GGML_OP_CPY, GGML_OP_CONT, GGML_OP_SUM, GGML_OP_ADD, GGML_OP_SCALE, GGML_OP_ADD1 };
-    for (int k = 0; k < 9; ++k) if (n[k]->op != want[k]) return -1;
+    for (int k = 0; k < 9; ++k) {
+        const bool cast_back = (k == 1 || k == 4) && n[k]->op == GGML_OP_CPY && n[k - 1]->type == GGML_TYPE_F16 && n[k]->src[1] == n[k] &&
+                               ggml_is_contiguous(n[k]);
+        if (n[k]->op != want[k] && !cast_back) return -1;
+    }
     if (n[1]->src[0] != n[0] || n[2]->src[0] != n[1] || n[4]->src[0] != n[3] || n[5]->src[0] != n[4]) return -1;
     if (!((n[6]->src[0] == n[2] && n[6]->src[1] == n[5]) || (n[6]->src[0] == n[5] && n[6]->src[1] == n[2]))) return -1;
     if (n[7]->src[0] != n[6] || n[8]->src[1] != n[7]) return -1;
     ggml_tensor * x = n[8]->src[0];
-    for (int k = 0; k < 8; ++k) if (x == n[k] || !private_to_group(readers, n[k])) return -1;
-    // the copies must be plain F32 -> F32 writes into the cache (the CPY node is a view of its destination)
+    for (int k = 0; k < 8; ++k) {
+        const bool cast_back = (k == 1 || k == 4) && n[k]->op == GGML_OP_CPY;
+        if (x == n[k] || !(cast_back ? private_cast_node(readers, n[k]) : private_to_group(readers, n[k]))) return -1;
+    }
+    // the copies must be plain F32 -> F32 / F16 writes into the cache (the CPY node is a view of its destination)
     for (int c = 0; c < 4; c += 3) {
-        if (n[c]->src[0]->type != GGML_TYPE_F32 || n[c]->type != GGML_TYPE_F32 || n[c]->src[1] == nullptr || n[c]->data != n[c]->src[1]->data) return -1;
+        if (n[c]->src[0]->type != GGML_TYPE_F32 || (n[c]->type != GGML_TYPE_F32 && n[c]->type != GGML_TYPE_F16) || n[c]->src[1] == nullptr ||
+            n[c]->data != n[c]->src[1]->data) return -1;
         if (n[c + 1]->type != GGML_TYPE_F32) return -1;
+        if ((n[c]->type == GGML_TYPE_F16) != (n[c + 1]->op == GGML_OP_CPY)) return -1;
     }
     ggml_tensor * dst = n[8];
     if (!apart(dst, n[0]->src[0]) || !apart(dst, n[3]->src[0]) || !apart(dst, n[0]) || !apart(dst, n[3]) || !apart_or_same(dst, x)) return -1;
@@ -774,7 +792,19 @@ int compute_mul_mat_residual_group(backend_ctx * ctx, const ggml_cgraph * g, int
 // tensors, the attention kernel reads both segments where they lie and the CONCATs are never run.
 // The CONCATs' operands must then still be intact when the attention node is reached: no node in
 // between (nor the attention's own output) may have been given their memory.
-struct kv2_group { const ggml_tensor * kcat; const ggml_tensor * vcat; };
+// With an F16 cache the step's keys reach the CONCAT through a cast (CPY to a new F16 tensor).  When only the CONCAT
+// reads the cast, the attention kernel reads the F32 source instead and rounds while it loads, and the cast is never run.
+struct kv2_group {
+    const ggml_tensor * kcat; const ggml_tensor * vcat;
+    const ggml_tensor * kcur; const ggml_tensor * vcur; // the second segments as the kernel reads them
+};
+
+// the F32 source behind a private F32 -> F16 cast node, or null
+const ggml_tensor * private_cast_source(const reader_map & readers, const ggml_tensor * t) {
+    if (t->op != GGML_OP_CPY || t->src[1] != t || t->type != GGML_TYPE_F16 || !t->src[0] || t->src[0]->type != GGML_TYPE_F32) return nullptr;
+    if (!private_cast_node(readers, t) || !ggml_are_same_shape(t, t->src[0])) return nullptr;
+    return t->src[0];
+}
 
 void find_kv2_groups(const ggml_cgraph * g, const reader_map & readers, std::unordered_map<const ggml_tensor *, kv2_group> & by_fa,
                      std::unordered_map<const ggml_tensor *, const ggml_tensor *> & absorbed) {
@@ -782,32 +812,45 @@ void find_kv2_groups(const ggml_cgraph * g, const reader_map & readers, std::uno
         const ggml_tensor * f = g->nodes[i];
         if (f->op != GGML_OP_FLASH_ATTN_EXT || (f->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
         const ggml_tensor * cat[2] = { f->src[1], f->src[2] };
+        const ggml_tensor * cur[2] = { nullptr, nullptr };  // the second segment: the CONCAT's operand, or the source of its cast
+        const ggml_tensor * cast[2] = { nullptr, nullptr };
         int at[2] = { -1, -1 };
         bool ok = true;
         for (int c = 0; c < 2 && ok; ++c) {
             ok = cat[c] && cat[c]->op == GGML_OP_CONCAT && ((const int32_t *) cat[c]->op_params)[0] == 1 && private_to_group(readers, cat[c]) &&
                  absorbed.find(cat[c]) == absorbed.end();
+            if (!ok) break;
+            cur[c] = cat[c]->src[1];
+            const ggml_tensor * target = cat[c];
+            if (const ggml_tensor * src = private_cast_source(readers, cur[c])) {
+                if (absorbed.find(cur[c]) != absorbed.end()) { ok = false; break; }
+                cast[c] = cur[c];
+                cur[c]  = src;
+                target  = cast[c];   // the F32 source must stay intact from the cast's position on
+            }
             for (int k = i - 1; ok && k >= 0 && k >= i - 32; --k)
-                if (g->nodes[k] == cat[c]) { at[c] = k; break; }
+                if (g->nodes[k] == target) { at[c] = k; break; }
             ok = ok && at[c] >= 0;
         }
-        if (!ok || cat[0] == cat[1]) continue;
+        if (!ok || cat[0] == cat[1] || (cast[0] == nullptr) != (cast[1] == nullptr)) continue;
         if (f->src[4] && (f->src[4]->type != GGML_TYPE_F32 || f->src[4]->ne[0] != f->src[0]->ne[2])) continue;
-        const vx_tensor q = to_vx(f->src[0]), kp = to_vx(cat[0]->src[0]), kc = to_vx(cat[0]->src[1]), vp = to_vx(cat[1]->src[0]),
-                        vc = to_vx(cat[1]->src[1]), d = to_vx(f);
+        const vx_tensor q = to_vx(f->src[0]), kp = to_vx(cat[0]->src[0]), kc = to_vx(cur[0]), vp = to_vx(cat[1]->src[0]),
+                        vc = to_vx(cur[1]), d = to_vx(f);
         vx_tensor m;
         if (f->src[3]) m = to_vx(f->src[3]);
         if (!vx_supports_flash_attn_ext_kv2(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, &d)) continue;
         for (int c = 0; c < 2 && ok; ++c)
             for (int k = at[c] + 1; k <= i && ok; ++k) {
                 const ggml_tensor * n = g->nodes[k];
-                if (n == cat[0] || n == cat[1] || ggml_op_is_empty(n->op) || ggml_is_empty(n) || (n->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
-                ok = apart(n, cat[c]->src[0]) && apart(n, cat[c]->src[1]);
+                if (n == cat[0] || n == cat[1] || n == cast[0] || n == cast[1] || ggml_op_is_empty(n->op) || ggml_is_empty(n) ||
+                    (n->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+                ok = apart(n, cat[c]->src[0]) && apart(n, cur[c]);
             }
         if (!ok) continue;
-        by_fa[f] = kv2_group{ cat[0], cat[1] };
+        by_fa[f] = kv2_group{ cat[0], cat[1], cur[0], cur[1] };
         absorbed[cat[0]] = f;
         absorbed[cat[1]] = f;
+        if (cast[0]) { absorbed[cast[0]] = f; absorbed[cast[1]] = f; }
     }
 }
 
@@ -822,7 +865,7 @@ int compute_kv2_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i,
     const int last = match_kv_store_group(g, j, readers, n);
     if (last < 0 || n[8]->src[0] != f) return -1;
     const ggml_tensor * dst = n[8];
-    const ggml_tensor * reads[] = { f->src[0], f->src[3], f->src[4], grp.kcat->src[0], grp.kcat->src[1], grp.vcat->src[0], grp.vcat->src[1] };
+    const ggml_tensor * reads[] = { f->src[0], f->src[3], f->src[4], grp.kcat->src[0], grp.kcur, grp.vcat->src[0], grp.vcur };
     for (const ggml_tensor * r : reads)
         if (r && (!apart(dst, r) || !apart_rows(n[0], r) || !apart_rows(n[3], r))) return -1;
     float scale, max_bias, softcap, sc, bias;
@@ -831,8 +874,8 @@ int compute_kv2_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i,
     memcpy(&softcap, (const float *) f->op_params + 2, sizeof(float));
     memcpy(&sc, (const float *) n[7]->op_params + 0, sizeof(float));
     memcpy(&bias, (const float *) n[7]->op_params + 1, sizeof(float));
-    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcat->src[1]), vp = to_vx(grp.vcat->src[0]),
-                    vc = to_vx(grp.vcat->src[1]), ksrc = to_vx(n[0]->src[0]), ks = to_vx(n[0]), vsrc = to_vx(n[3]->src[0]), vs = to_vx(n[3]),
+    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcur), vp = to_vx(grp.vcat->src[0]),
+                    vc = to_vx(grp.vcur), ksrc = to_vx(n[0]->src[0]), ks = to_vx(n[0]), vsrc = to_vx(n[3]->src[0]), vs = to_vx(n[3]),
                     d = to_vx(dst);
     vx_tensor m;
     if (f->src[3]) m = to_vx(f->src[3]);
@@ -847,8 +890,8 @@ vx_status compute_kv2_attention(backend_ctx * ctx, const ggml_tensor * f, const 
     memcpy(&scale, (const float *) f->op_params + 0, sizeof(float));
     memcpy(&max_bias, (const float *) f->op_params + 1, sizeof(float));
     memcpy(&softcap, (const float *) f->op_params + 2, sizeof(float));
-    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcat->src[1]), vp = to_vx(grp.vcat->src[0]),
-                    vc = to_vx(grp.vcat->src[1]), d = to_vx(f);
+    const vx_tensor q = to_vx(f->src[0]), kp = to_vx(grp.kcat->src[0]), kc = to_vx(grp.kcur), vp = to_vx(grp.vcat->src[0]),
+                    vc = to_vx(grp.vcur), d = to_vx(f);
     vx_tensor m;
     if (f->src[3]) m = to_vx(f->src[3]);
     return vx_flash_attn_ext_kv2(&q, &kp, &kc, &vp, &vc, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
