@@ -1,19 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Prints ONE JSON line.  The default workload is BASELINE config 2: backbone-shaped decode
-attention -- 24 layers x GQA attention (16 Q / 2 KV heads, head_dim 64), batch 2, one new
-token per step, f16 KV cache of length 4096.  A step is one pass over the 24 layers (24
-calls of vx_flash_attn_ext, each on its own layer's resident cache); `value` is the
-algorithmic KV bytes of a step divided by its wall time, inputs already in HBM.
+Prints ONE JSON line.  The headline workload is BASELINE config 5's decode attention, the largest
+single-GPU configuration: 8 synthesis streams x CFG pair (batch 16), 16 Q / 2 KV heads, head_dim 64,
+one new token per step over an f16 KV cache of 8192 keys, 24 layers.  A step is one pass over the 24
+layers (24 calls of vx_flash_attn_ext, each on its own layer's resident cache: 1.5 GiB of K/V per
+step, so nothing is served from a cache); `value` is the algorithmic K/V bytes of a step divided by
+its wall time, inputs already in HBM.
 
-The same line carries, under "others", shorter measurements of the other BASELINE shapes
-(other KV lengths, the batch-16 / 8192-key decode, prefill attention, LocDiT attention,
-the Q8_0 projections), a `roofline` object for the dominant kernel of the headline
-workload and a `cpu_baseline` object: the reference's own ggml-cpu (oracle/_ref) timed on
-this machine's host cores on one layer of the same workload.
+The same line carries a `roofline` object for that call (published peak, the peak a plain streaming
+read reaches on this box, measured HBM traffic when a counter profile of the current kernels is on
+file), a `cpu_baseline` object (the reference's own ggml-cpu, oracle/_ref, timed on this machine's
+host cores on one layer of the same workload, at the box's core share and at 8 threads), and under
+"others" the other BASELINE shapes: config 2's decode lengths, prefill attention, LocDiT attention
+and the CFM solve, the Q8_0 projections, and the config 4 / 5 decoder stacks with F32 and f16 caches.
 """
 import argparse
 import ctypes as C
@@ -33,9 +35,20 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # dense f16/bf16 MFMA, published
 
 HQ, HKV, D, LAYERS = 16, 2, 64, 24
 
-# (batch, KV length) -> HBM bytes per vx_flash_attn_ext call, measured with hardware counters
-# (see --calibrate-copy); algorithmic bytes of the same call: kv_bytes(2, 4096) = 4194304
-MEASURED_TRAFFIC_BYTES = {(2, 4096): 5654 * 1024}
+
+def measured_traffic(batch, length):
+    """HBM bytes per vx_flash_attn_ext call from the counter profile on file for this shape (rocprofv3 FETCH_SIZE /
+    WRITE_SIZE scaled by a plain copy; profiles/decode_attn_*_hbm_counters.txt carries a line
+    `traffic_bytes_per_call: N` and the commit it was taken at), or None."""
+    path = os.path.join(ROOT, "profiles", f"decode_attn_B{batch}_L{length}_hbm_counters.txt")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    import re
+    m = re.search(r"^traffic_bytes_per_call:\s*(\d+)", text, re.M)
+    c = re.search(r"^commit:\s*(\S+)", text, re.M)
+    return (int(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
 def kv_bytes(batch, length, es=2):
@@ -173,45 +186,62 @@ def q8_proj_setup(pkg, M, K, N):
     return call, (wq, x, out)
 
 
-def cpu_baseline(batch, length, threads):
-    """ggml-cpu (the reference build in oracle/_ref) on one layer of the decode workload."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def stats(times):
+    """mean / median / p90 / best of a list of seconds, as the reference's benchmark reports them
+    (benchmark/voxcpm_benchmark.cpp:623-669)."""
+    t = np.sort(np.asarray(times, np.float64))
+    return {"mean": float(t.mean()), "median": float(np.median(t)), "p90": float(t[min(len(t) - 1, int(np.ceil(0.9 * len(t))) - 1)]),
+            "best": float(t[0]), "repeats": int(len(t))}
+
+
+def cpu_baseline(batch, length, core_share):
+    """ggml-cpu (the reference build in oracle/_ref) on one layer of the headline decode workload: at every core
+    of this box's share and at 8 threads (the reference's own benchmark setting, README.md:504), a few seconds each."""
     import reflib
     ref = reflib.load_ref()
     q = reflib.rng("cpu", "q").standard_normal((batch, HQ, 1, D)).astype(np.float32)
     k = reflib.rng("cpu", "k").standard_normal((batch, HKV, length, D)).astype(np.float16)
     v = reflib.rng("cpu", "v").standard_normal((batch, HKV, length, D)).astype(np.float16)
-    if ref is not None:
+    nbytes = kv_bytes(batch, length)
+    if ref is None:
+        t0 = time.perf_counter()
+        reflib.oracle_fa(q[:1], k[:1].astype(np.float32), v[:1].astype(np.float32))
+        sec = (time.perf_counter() - t0) * batch
+        return {"value": nbytes / sec / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "one stream of one layer on the scalar C oracle, scaled to the batch (oracle/_ref not prebuilt)"}
+    runs = {}
+    for threads in sorted({core_share, min(8, core_share)}, reverse=True):
         assert ref.rh_use_device(b"CPU", threads, 0) == 0
-        # size the sample to roughly 10 s of CPU work
-        _, (mean1, _) = reflib.ref_fa(q, k, v, reps=20)
-        reps = int(max(50, min(20000, 10.0 / max(mean1, 1e-6))))
-        _, (mean, best) = reflib.ref_fa(q, k, v, reps=reps)
-        return {"value": kv_bytes(batch, length) / mean / 1e9, "unit": "GB/s", "cores": threads, "kind": "reference",
-                "sample": f"{reps} repeats of one layer's ggml_flash_attn_ext on ggml-cpu (batch {batch}, KV {length}, "
-                          f"f16 K/V), mean {mean * 1e6:.1f} us, best {best * 1e6:.1f} us"}
-    t0 = time.perf_counter()
-    reps = 3
-    for _ in range(reps):
-        reflib.oracle_fa(q, k.astype(np.float32), v.astype(np.float32))
-    mean = (time.perf_counter() - t0) / reps
-    return {"value": kv_bytes(batch, length) / mean / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} repeats of one layer on the scalar C oracle (oracle/_ref not prebuilt)"}
+        _, (mean1, _) = reflib.ref_fa(q, k, v, reps=3)
+        reps = int(max(5, min(2000, 6.0 / max(mean1, 1e-6))))   # about 6 s of CPU work per setting
+        reflib.ref_fa(q, k, v, reps=reps)
+        st = stats(reflib.ref_last_times())
+        runs[threads] = {"GB/s": nbytes / st["mean"] / 1e9, "us": {n: st[n] * 1e6 for n in ("mean", "median", "p90", "best")}, "repeats": st["repeats"]}
+    assert ref.rh_use_device(b"CPU", min(8, core_share), 0) == 0
+    top = runs[core_share]
+    return {"value": top["GB/s"], "unit": "GB/s", "cores": core_share, "kind": "reference", "cpu": cpu_model(),
+            "host_logical_cpus": os.cpu_count(),
+            "sample": f"{top['repeats']} repeats of one layer's ggml_flash_attn_ext on ggml-cpu (batch {batch}, KV {length}, f16 K/V, "
+                      f"{nbytes >> 20} MiB of K/V): mean {top['us']['mean']:.0f} us, median {top['us']['median']:.0f}, p90 {top['us']['p90']:.0f}; "
+                      f"{core_share} threads = this box's core share for one GPU",
+            "by_threads": {str(t): r for t, r in runs.items()}}
 
 
-def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256, do_prefill=True, cpu_reps=40):
-    """BASELINE config 4: the whole decoder stack with Q8_0 weights (hidden 1024, 16/2 heads, FFN 4096),
-    batch 2, prefill 512 tokens then 256 decode steps.  The GPU side is the host-side mirror of the
-    reference's layer_forward over the C ABI (voxcpm.cpp_amd/backbone.py, F32 KV cache as in the
-    reference); a decode step is replayed from a captured HIP graph.  Four KV lengths spread over the
-    256-step range are captured and each replayed steps/4 times, so the timed work is that of the
-    512 -> 768 decode.  ggml-cpu runs the reference-structured graph of the same stack beside it."""
+def load_stack(pkg, layers, max_len, batch, kv_f16, lw, params, use_mup=True):
     import torch
     import reflib
     bbmod = __import__("voxcpm_cpp_amd.backbone", fromlist=["MiniCPMBackbone"])
-    params = reflib.backbone_params("bench-bb", 1)   # one layer's seeded weights, placed in `layers` separate buffers
-    lw = params["layers"][0]
-    max_len = prefill + steps
-    m = bbmod.MiniCPMBackbone(n_layer=layers, max_length=max_len, batch=batch, use_mup=True, kv_f16=False)
+    m = bbmod.MiniCPMBackbone(n_layer=layers, max_length=max_len, batch=batch, use_mup=use_mup, kv_f16=kv_f16)
     for li in range(layers):
         for n in reflib.BB_WEIGHTS:
             m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
@@ -219,25 +249,46 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
             m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
     m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
     m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
-    weight_bytes = layers * sum(lw[n].nbytes for n in reflib.BB_WEIGHTS)
+    return m
 
-    t_prefill = None
+
+def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256, kv_f16=False,
+                   cpu_reps=40, cpu_prefill=True, plugin_reps=40, f32_prefill_switch=True):
+    """A whole decoder stack with Q8_0 weights (hidden 1024, 16/2 heads, FFN 4096): BASELINE config 4 (batch 2,
+    prefill 512 tokens then 256 decode steps) or config 5 (batch 16, prefill 4096, decode to 8192).  The GPU side is
+    the host-side mirror of the reference's layer_forward over the C ABI (voxcpm.cpp_amd/backbone.py), a decode step
+    replayed from a captured HIP graph: four KV lengths spread over the decode range are captured and each replayed
+    steps/4 times, so the timed work is that of the whole decode.  Beside it: the same step through the product
+    boundary -- the reference-structured graph handed to the plugin's graph_compute by ggml, eager, rebuilt per call
+    as the reference does -- and ggml-cpu on that graph."""
+    import torch
+    import reflib
+    params = reflib.backbone_params("bench-bb", 1)   # one layer's seeded weights, placed in `layers` separate buffers
+    lw = params["layers"][0]
+    max_len = prefill + steps
+    m = load_stack(pkg, layers, max_len, batch, kv_f16, lw, params)
+    weight_bytes = layers * sum(lw[n].nbytes for n in reflib.BB_WEIGHTS)
+    es = 2 if kv_f16 else 4
+
+    gk = torch.Generator(device="cuda").manual_seed(11)
+    for t in m.k_cache + m.v_cache:      # seeded cache contents; the prefill overwrites its part
+        if kv_f16:
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gk).half())
+        else:
+            t.normal_(generator=gk)
+    xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
+    mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
+    run_p, _ = m.plan(xp, prefill, 0, mask)
+    big = batch * prefill > 4096
+    t_prefill = timer.run(run_p, iters=1 if big else 3, warmup=1)
     t_prefill_f16 = None
-    xp = None
-    if do_prefill:
-        xp = torch.randn((batch, prefill, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
-        mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
-        run_p, _ = m.plan(xp, prefill, 0, mask)
-        t_prefill = timer.run(run_p, iters=3, warmup=1)
+    if not kv_f16 and f32_prefill_switch:
         # the same prefill with the F32 cache rounded to f16 on its way into the LDS-tiled attention kernel (opt-in, read per call)
         os.environ["VX_FA_F32_PREFILL"] = "1"
-        t_prefill_f16 = timer.run(run_p, iters=3, warmup=1)
+        t_prefill_f16 = timer.run(run_p, iters=1 if big else 3, warmup=1)
         del os.environ["VX_FA_F32_PREFILL"]
         timer.run(run_p, iters=1, warmup=0)  # leave the cache as the default route writes it
-    else:   # long caches: decode over seeded cache contents instead of a real prefill
-        gk = torch.Generator(device="cuda").manual_seed(11)
-        for t in m.k_cache + m.v_cache:
-            t.normal_(generator=gk)
+    del run_p, mask
 
     x1 = torch.randn((batch, 1, 1024), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
     points = [prefill + (2 * i + 1) * steps // 8 for i in range(4)]
@@ -246,7 +297,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         run_d, _ = m.plan(x1, 1, n_past)
         n_calls = run_d.n_calls
         replays.append((graphed(run_d, side), run_d))
-    per = steps // 4
+    per = max(1, min(64, steps // 4))
     for rp, _ in replays:
         rp()
     torch.cuda.synchronize()
@@ -256,30 +307,47 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
             rp()
     torch.cuda.synchronize()
     t_step = (time.perf_counter() - t0) / (per * 4)
-    kvb = layers * 2 * batch * HKV * (prefill + steps // 2) * D * 4
+    kvb = layers * 2 * batch * HKV * (prefill + steps // 2) * D * es
     res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
            "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
-           "prefill_ms": t_prefill * 1e3 if t_prefill else None, "prefill_tokens_per_s": batch * prefill / t_prefill if t_prefill else None,
-           "prefill_ms_VX_FA_F32_PREFILL": t_prefill_f16 * 1e3 if t_prefill else None,
-           "kv_cache": "f32 (the reference's cache type)", "launch": "captured HIP graph per step, KV lengths " + str(points)}
-    del replays, m
-    ref = reflib.load_ref() if with_cpu else None
-    if ref is not None:
+           "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": batch * prefill / t_prefill,
+           "prefill_ms_VX_FA_F32_PREFILL": t_prefill_f16 * 1e3 if t_prefill_f16 else None,
+           "kv_cache": "f16" if kv_f16 else "f32 (the reference's cache type)",
+           "launch": f"captured HIP graph per step, KV lengths {points} ({per} replays each)"}
+    del replays, m, xp
+    torch.cuda.empty_cache()
+    ref = reflib.load_ref()
+    mid = prefill + steps // 2
+    params["dims"]["n_layer"] = layers
+    params["layers"] = [lw] * layers
+    if ref is not None and plugin_reps > 0:
+        # through the product boundary: ggml hands the reference-structured graph to the plugin's graph_compute
+        assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) == 0
+        assert ref.rh_use_device(b"GFX950_0", 1, 0) == 0
+        reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=kv_f16)
+        _, _, n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps)
+        st = stats(reflib.ref_last_times())
+        ref.rh_bb_free()
+        launches = C.CDLL(pkg.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+        res["plugin_graph_compute"] = {"decode_steps_per_s": 1.0 / st["mean"], "ms_per_step": {n: st[n] * 1e3 for n in ("mean", "median", "p90", "best")},
+                                       "graph_nodes": n_nodes, "launches": launches, "kv_length": mid,
+                                       "how": "ggml_backend_graph_compute on libggml-gfx950.so, eager, synchronised per call"}
         assert ref.rh_use_device(b"CPU", threads, 0) == 0
-        params["dims"]["n_layer"] = layers
-        params["layers"] = [lw] * layers
-        reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=False)
-        cpu_prefill = None
-        if do_prefill:
-            xph = xp.cpu().numpy()
+    if ref is not None and with_cpu:
+        assert ref.rh_use_device(b"CPU", threads, 0) == 0
+        reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=kv_f16)
+        cpu_pf = None
+        if cpu_prefill:
+            xph = np.random.default_rng(7).standard_normal((batch, prefill, 1024)).astype(np.float32)
             tp0 = time.perf_counter()
             reflib.ref_backbone_forward(xph, 0, reflib.causal_mask(prefill, prefill))
-            cpu_prefill = time.perf_counter() - tp0
-        _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), prefill + steps // 2, None, reps=cpu_reps)
+            cpu_pf = time.perf_counter() - tp0
+        _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=cpu_reps)
+        st = stats(reflib.ref_last_times())
         ref.rh_bb_free()
-        res["ggml_cpu"] = {"decode_steps_per_s": 1.0 / mean, "ms_per_step": mean * 1e3, "best_ms": best * 1e3, "threads": threads,
-                           "graph_nodes": n_nodes, "prefill_ms": cpu_prefill * 1e3 if cpu_prefill else None,
-                           "sample": f"{cpu_reps} repeats of the decode step at KV length {prefill + steps // 2}" + (", one prefill" if do_prefill else ", cache contents as left by allocation")}
+        res["ggml_cpu"] = {"decode_steps_per_s": 1.0 / mean, "ms_per_step": mean * 1e3, "median_ms": st["median"] * 1e3, "p90_ms": st["p90"] * 1e3,
+                           "best_ms": best * 1e3, "threads": threads, "graph_nodes": n_nodes, "prefill_ms": cpu_pf * 1e3 if cpu_pf else None,
+                           "sample": f"{cpu_reps} repeats of the decode step at KV length {mid}" + (", one prefill" if cpu_prefill else ", cache contents as left by allocation, no prefill (it would take minutes)")}
         res["speedup_vs_ggml_cpu"] = mean / t_step
     return res
 
@@ -383,20 +451,55 @@ def cfm_solve_bench(pkg, timer, side, threads, with_cpu, layers=4, patch=2, pref
     return res
 
 
+def load_peaks():
+    lib = C.CDLL(os.path.join(ROOT, "voxcpm.cpp_amd", "lib", "libvx_peaks.so"))
+    lib.vxp_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
+    lib.vxp_mfma_f16.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.vxp_mfma_f16_flop.argtypes = [C.c_int, C.c_int]
+    lib.vxp_mfma_f16_flop.restype = C.c_double
+    return lib
+
+
+def peaks_bench(timer):
+    """What this box delivers on the two simplest kernels: a streaming read (1 GiB at once; and 64 MiB per launch over 24
+    distinct buffers, the size and reuse pattern of the headline attention call) and a loop of independent f16 MFMAs."""
+    import torch
+    lib = load_peaks()
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    sink = torch.zeros(1 << 20, dtype=torch.int32, device="cuda")
+    big = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    big.fill_(1)
+    s_big = timer.run(lambda: lib.vxp_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), 0, st()), iters=20, warmup=3)
+    chunk = 64 << 20
+    parts = [big[i * chunk:(i + 1) * chunk] for i in range(16)] + [torch.ones(chunk, dtype=torch.uint8, device="cuda") for _ in range(8)]
+
+    def sweep():
+        for p_ in parts:
+            lib.vxp_stream_read(p_.data_ptr(), chunk, sink.data_ptr(), 0, st())
+
+    s_chunk = timer.run(sweep, iters=10, warmup=2) / len(parts)
+    fsink = torch.zeros(4096 * 256, dtype=torch.float32, device="cuda")
+    blocks, iters = 2048, 4096
+    s_mfma = timer.run(lambda: lib.vxp_mfma_f16(blocks, iters, fsink.data_ptr(), st()), iters=5, warmup=2)
+    return {"hbm_stream_read_1GiB_GB/s": big.numel() / s_big / 1e9,
+            "hbm_stream_read_64MiB_per_launch_GB/s": chunk / s_chunk / 1e9, "hbm_stream_read_64MiB_us": s_chunk * 1e6,
+            "mfma_f16_TFLOP/s": lib.vxp_mfma_f16_flop(blocks, iters) / s_mfma / 1e12,
+            "how": "libvx_peaks.so: 16-byte nontemporal loads, 8 in flight per lane, 8 blocks per CU; 8 independent v_mfma_f32_32x32x16_f16 per wave in a loop"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--length", type=int, default=4096, help="KV length of the headline decode workload")
     ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the ggml-cpu baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the ggml-cpu baselines")
     ap.add_argument("--eager", action="store_true", help="launch every call from Python instead of replaying a HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
-    ap.add_argument("--profile", choices=["prefill", "backbone", "cfm", "gemm"], default=None,
-                    help="run only this secondary workload a few times (for rocprofv3) and print its figures")
+    ap.add_argument("--profile", choices=["decode5", "decode2", "prefill", "prefill1", "backbone", "backbone16", "cfm", "gemm", "peaks"], default=None,
+                    help="run only this workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no cross-GPU step); run with --gpus 1")
@@ -417,10 +520,21 @@ def main():
     pkg.check(pkg.lib().vx_init(0), "vx_init")
     timer = Timer()
 
-    if args.profile == "prefill":   # config 5 prefill attention, 16 streams x 4096 tokens
-        call, flops, keep = prefill_attn_setup(pkg, 16, 4096)
+    if args.profile in ("decode5", "decode2"):   # the decode attention call alone, eager, every layer's own cache
+        b, L = (16, 8192) if args.profile == "decode5" else (2, 4096)
+        st, one, keep = decode_attn_setup(pkg, b, L, LAYERS)
+        s = timer.run(st, iters=5, warmup=2) / LAYERS
+        print(json.dumps({"profile": f"decode_attn_B{b}_L{L}", "us_per_call": s * 1e6, "GB/s": kv_bytes(b, L) / s / 1e9,
+                          "calls": 7 * LAYERS, "bytes_per_call": kv_bytes(b, L)}))
+        return
+    if args.profile == "peaks":
+        print(json.dumps({"profile": "peaks", **peaks_bench(timer)}))
+        return
+    if args.profile in ("prefill", "prefill1"):   # config 5 prefill attention, 16 streams (or one) x 4096 tokens
+        nb = 16 if args.profile == "prefill" else 1
+        call, flops, keep = prefill_attn_setup(pkg, nb, 4096)
         s = timer.run(call, iters=5, warmup=2)
-        print(json.dumps({"profile": "cfg5_prefill_attn_T4096_B16", "us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
+        print(json.dumps({"profile": f"cfg5_prefill_attn_T4096_B{nb}", "us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
                           "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}))
         return
     if args.profile == "gemm":      # the prefill-sized Q8_0 projection, 4096 rows x 1024 x 16384 tokens
@@ -433,15 +547,19 @@ def main():
     if args.profile == "cfm":       # config 3: whole CFM solves of one request, replayed from a HIP graph
         print(json.dumps({"profile": "cfg3_cfm_solve_one_request", **cfm_solve_bench(pkg, timer, torch.cuda.Stream(), 1, False)}))
         return
-    if args.profile == "backbone":  # config 4 decode steps, eager launches so that every kernel is traced
-        print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16)}))
+    if args.profile == "backbone":  # config 4 decode steps (f16 cache)
+        print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16, kv_f16=True, plugin_reps=5)}))
+        return
+    if args.profile == "backbone16":  # config 5 decode steps (f16 cache)
+        print(json.dumps({"profile": "cfg5_backbone_24layers_b16", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, batch=16, prefill=4096,
+                                                                                     steps=4096, kv_f16=True, plugin_reps=3)}))
         return
 
-    # ---- headline: config 2, L = args.length -------------------------------------------
-    B, L = 2, args.length
+    # ---- headline: config 5 decode attention, batch 16, 8192 keys, 24 layers ------------------------
+    B, L = 16, 8192
     side = torch.cuda.Stream()
     step_eager, one_layer, keep = decode_attn_setup(pkg, B, L, LAYERS)
-    eager_sec = timer.run(step_eager, iters=20)
+    eager_sec = timer.run(step_eager, iters=10)
     # the 24 launches of a step replayed as one HIP graph: what a C++ host looping over graph
     # nodes achieves, without the Python call overhead of this script
     step = graphed(step_eager, side) if not args.eager else step_eager
@@ -456,75 +574,88 @@ def main():
     step_bytes = LAYERS * kv_bytes(B, L)
     value = step_bytes / sec_per_step / 1e9
 
-    # dominant kernel: one vx_flash_attn_ext call (split-KV kernel + combine), HIP events
-    launch_sec = timer.run(step, iters=200, warmup=10) / LAYERS
+    # dominant kernel: one vx_flash_attn_ext call (split-KV kernel + the merge of its partials), HIP events on the launch stream
+    launch_sec = timer.run(step, iters=100, warmup=10) / LAYERS
     achieved = kv_bytes(B, L) / launch_sec / 1e9
-    # HBM bytes per call from rocprofv3 FETCH_SIZE / WRITE_SIZE (split kernel + merge kernel, scaled
-    # by the same counters on a 256 MiB copy: x2.000 and x1.000), taken at the default length only
-    traffic = MEASURED_TRAFFIC_BYTES.get((B, L))
-    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64,f16> + fattn_merge_kernel<64>", "achieved": achieved,
+    traffic, traffic_commit = measured_traffic(B, L)
+    peaks = peaks_bench(timer)
+    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64, f16 K/V> + fattn_merge_kernel<64>", "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "traffic_source": (f"profiles/decode_attn_B{B}_L{L}_hbm_counters.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain copy, taken at commit {traffic_commit})"
+                                   if traffic else None),
+                "achievable_peak": peaks["hbm_stream_read_64MiB_per_launch_GB/s"],
+                "frac_of_achievable": achieved / peaks["hbm_stream_read_64MiB_per_launch_GB/s"],
+                "achievable_peak_is": "a plain streaming read of 64 MiB per launch over 24 distinct buffers, measured in this run (libvx_peaks.so); "
+                                      f"1 GiB in one launch: {peaks['hbm_stream_read_1GiB_GB/s']:.0f} GB/s",
                 "launch_us": launch_sec * 1e6, "bytes_per_launch": kv_bytes(B, L),
-                "note": "average over the 24 launches of a graph-replayed step (HIP events on the launch stream)"}
-    del keep
+                "note": "average over the 24 calls of a graph-replayed step, each two kernels (HIP events on the launch stream)"}
+    del keep, step, step_eager, one_layer
+    torch.cuda.empty_cache()
 
-    others = {}
+    others = {"peaks_measured_on_this_box": peaks}
     if not args.no_others:
         for L2 in (128, 512, 2048, 4096):
             st, one, keep = decode_attn_setup(pkg, 2, L2, LAYERS)
             s = timer.run(graphed(st, side), iters=50)
-            others[f"cfg2_decode_attn_L{L2}"] = {"us_per_layer": s / LAYERS * 1e6,
-                                                  "GB/s": LAYERS * kv_bytes(2, L2) / s / 1e9}
-            del keep
-        st, one, keep = decode_attn_setup(pkg, 16, 8192, LAYERS)  # 1.5 GiB of KV: no cache reuse
-        s = timer.run(graphed(st, side), iters=20, warmup=3) / LAYERS
-        others["cfg5_decode_attn_B16_L8192"] = {"us_per_layer": s * 1e6, "GB/s": kv_bytes(16, 8192) / s / 1e9,
-                                                "hbm_frac": kv_bytes(16, 8192) / s / 1e9 / HBM_PEAK_GBS}
-        del keep
+            others[f"cfg2_decode_attn_B2_L{L2}"] = {"us_per_layer": s / LAYERS * 1e6, "GB/s": LAYERS * kv_bytes(2, L2) / s / 1e9,
+                                                     "hbm_frac": LAYERS * kv_bytes(2, L2) / s / 1e9 / HBM_PEAK_GBS}
+            del keep, st, one
         for name, b, T, it in (("cfg1_prefill_attn_T256", 1, 256, 200), ("cfg5_prefill_attn_T4096_B1", 1, 4096, 5),
                                   ("cfg5_prefill_attn_T4096_B16", 16, 4096, 3)):
             call, flops, keep = prefill_attn_setup(pkg, b, T)
             s = timer.run(call, iters=it, warmup=2)
             others[name] = {"us": s * 1e6, "TFLOP/s_causal_exact": flops / s / 1e12,
-                            "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS}
-            del keep
+                            "mfma_frac": flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                            "frac_of_measured_mfma_loop": flops / s / 1e12 / peaks["mfma_f16_TFLOP/s"]}
+            del keep, call
         solve, n_calls, keep = locdit_attn_setup(pkg)
         s = timer.run(graphed(solve, side), iters=20)
         others["cfg3_locdit_attn_16seq_x7"] = {"us_per_cfm_solve": s * 1e6, "launches_per_solve": n_calls,
                                                "us_per_attention": s / n_calls * 1e6}
-        del keep
+        del keep, solve
         for name, M, K, N in (("q8_0_proj_1024x1024_n2", 1024, 1024, 2), ("q8_0_ffn_up_4096x1024_n2", 4096, 1024, 2),
                               ("q8_0_proj_1024x1024_n1024", 1024, 1024, 1024), ("q8_0_ffn_up_4096x1024_n1024", 4096, 1024, 1024),
-                              ("q8_0_proj_1024x1024_n16384", 1024, 1024, 16384)):
+                              ("q8_0_proj_1024x1024_n16384", 1024, 1024, 16384), ("q8_0_ffn_up_4096x1024_n16384", 4096, 1024, 16384)):
             call, keep = q8_proj_setup(pkg, M, K, N)
             s = timer.run(call, iters=200 if N <= 1024 else 20, warmup=5)
             wbytes = M * K // 32 * 34
             others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12}
-            del keep
+            del keep, call
+        torch.cuda.empty_cache()
 
-    threads = min(16, os.cpu_count() or 1)
+    threads = min(16, os.cpu_count() or 1)   # a one-GPU box's share of the host
     if not args.no_others:
-        others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu)
-        others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, not args.no_cpu)
-        others["cfg3_cfm_solve_one_request"] = cfm_solve_bench(pkg, timer, side, threads, not args.no_cpu)
-        # BASELINE config 5 as a whole stack: 8 streams x CFG pair (batch 16) decoding from KV length 4096 towards 8192
-        # (F32 cache as in the reference; the decode steps run over seeded cache contents)
-        others["cfg5_backbone_24layers_b16_L4096"] = backbone_bench(pkg, timer, side, threads, not args.no_cpu, batch=16, prefill=4096,
-                                                                    steps=256, do_prefill=False, cpu_reps=3)
+        cpu_on = not args.no_cpu
+        # BASELINE config 4 with the reference's F32 cache and with the f16 cache BASELINE's configs name
+        others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, cpu_on)
+        others["cfg4_backbone_24layers_b2_f16kv"] = backbone_bench(pkg, timer, side, threads, False, kv_f16=True)
+        others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, cpu_on)
+        others["cfg3_cfm_solve_one_request"] = cfm_solve_bench(pkg, timer, side, threads, cpu_on)
+        # BASELINE config 5 as a whole stack: 8 streams x CFG pair (batch 16), prefill 4096 tokens, decode from 4096 to 8192
+        others["cfg5_backbone_24layers_b16_f16kv"] = backbone_bench(pkg, timer, side, threads, cpu_on, batch=16, prefill=4096, steps=4096,
+                                                                    kv_f16=True, cpu_reps=3, cpu_prefill=False, plugin_reps=10)
+        others["cfg5_backbone_24layers_b16"] = backbone_bench(pkg, timer, side, threads, False, batch=16, prefill=4096, steps=4096,
+                                                              kv_f16=False, plugin_reps=0, f32_prefill_switch=False)
 
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(B, L, threads)
 
+    def pick(name, *path):
+        v = others.get(name, {})
+        for k_ in path:
+            v = v.get(k_, {}) if isinstance(v, dict) else {}
+        return v if not isinstance(v, dict) else None
+
     line = {
-        # BASELINE.json's metric, verbatim; `value` is its decode component on config 2 (see config.value_is),
+        # BASELINE.json's metric, verbatim; `value` is its decode component on config 5 (see config.value_is),
         # the prefill TFLOP/s and backbone steps/s components are repeated under "components"
         "metric": "attn TFLOP/s (prefill) & HBM GB/s (decode) vs roofline; backbone decode steps/s",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec_per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 K/V, f32 accumulate", "data": "synthetic (seeded N(0,1))",
-        "config": {"workload": f"BASELINE config 2: 24 layers x GQA decode attention, 16/2 heads, head_dim 64, "
-                               f"batch 2, f16 KV length {L}",
+        "config": {"workload": f"BASELINE config 5 decode: 24 layers x GQA decode attention, 16/2 heads, head_dim 64, "
+                               f"8 streams x CFG pair (batch {B}), f16 KV length {L}",
                    "value_is": "decode attention HBM GB/s: algorithmic K/V bytes of the 24 calls of a step / wall time of the step",
                    "decode_attn_steps_per_s": 1.0 / sec_per_step,
                    "launch": "eager from Python" if args.eager else "one HIP graph replay per step",
@@ -532,12 +663,17 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "components": {
-            "decode_attn_GB/s_cfg2": value,
-            "decode_attn_hbm_frac_cfg5_B16_L8192": others.get("cfg5_decode_attn_B16_L8192", {}).get("hbm_frac"),
-            "prefill_attn_TFLOP/s_cfg5_T4096_B16": others.get("cfg5_prefill_attn_T4096_B16", {}).get("TFLOP/s_causal_exact"),
-            "prefill_attn_mfma_frac_cfg5_T4096_B16": others.get("cfg5_prefill_attn_T4096_B16", {}).get("mfma_frac"),
-            "backbone_decode_steps_per_s_cfg4": others.get("cfg4_backbone_24layers_b2", {}).get("decode_steps_per_s"),
-            "backbone_decode_steps_per_s_cfg4_ggml_cpu": others.get("cfg4_backbone_24layers_b2", {}).get("ggml_cpu", {}).get("decode_steps_per_s"),
+            "decode_attn_GB/s_cfg5_B16_L8192": value,
+            "decode_attn_hbm_frac_cfg5_B16_L8192": value / HBM_PEAK_GBS,
+            "decode_attn_GB/s_cfg2_B2_L4096": pick("cfg2_decode_attn_B2_L4096", "GB/s"),
+            "prefill_attn_TFLOP/s_cfg5_T4096_B16": pick("cfg5_prefill_attn_T4096_B16", "TFLOP/s_causal_exact"),
+            "prefill_attn_mfma_frac_cfg5_T4096_B16": pick("cfg5_prefill_attn_T4096_B16", "mfma_frac"),
+            "prefill_attn_mfma_frac_cfg5_T4096_B1": pick("cfg5_prefill_attn_T4096_B1", "mfma_frac"),
+            "backbone_decode_steps_per_s_cfg4": pick("cfg4_backbone_24layers_b2", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_f16kv": pick("cfg4_backbone_24layers_b2_f16kv", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_through_plugin": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_ggml_cpu": pick("cfg4_backbone_24layers_b2", "ggml_cpu", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg5_f16kv": pick("cfg5_backbone_24layers_b16_f16kv", "decode_steps_per_s"),
         },
         "others": others,
     }

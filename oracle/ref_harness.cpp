@@ -40,6 +40,7 @@ namespace {
 
 ggml_backend_t g_backend = nullptr;
 std::string    g_backend_name;
+std::vector<double> g_last_times; // seconds of every timed repeat of the most recent timed run (rh_last_times)
 
 size_t row_bytes(ggml_type type, int64_t ne0) { return ggml_row_size(type, ne0); }
 
@@ -84,11 +85,13 @@ struct op_graph {
         if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) return 102;
         if (reps > 0 && seconds) {
             double best = 1e30, total = 0;
+            g_last_times.clear();
             for (int r = 0; r < reps; ++r) {
                 auto t0 = std::chrono::steady_clock::now();
                 if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) return 102;
                 auto t1 = std::chrono::steady_clock::now();
                 const double dt = std::chrono::duration<double>(t1 - t0).count();
+                g_last_times.push_back(dt);
                 total += dt;
                 if (dt < best) best = dt;
             }
@@ -132,6 +135,13 @@ int rh_use_device(const char * name, int n_threads, int use_ref) {
         ggml_backend_cpu_set_use_ref(g_backend, use_ref != 0);
     }
     return 0;
+}
+
+// the seconds of each timed repeat of the most recent run that was given reps > 0; returns how many there are
+int rh_last_times(double * out, int max) {
+    const int n = (int) g_last_times.size();
+    for (int i = 0; i < n && i < max; ++i) out[i] = g_last_times[(size_t) i];
+    return n;
 }
 
 void rh_release(void) {
@@ -536,11 +546,13 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     }
     if (!rc && reps > 0 && seconds) {
         double best = 1e30, total = 0;
+        g_last_times.clear();
         for (int r = 0; r < reps && !rc; ++r) {
             auto t0 = std::chrono::steady_clock::now();
             if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
             auto t1 = std::chrono::steady_clock::now();
             const double dt = std::chrono::duration<double>(t1 - t0).count();
+            g_last_times.push_back(dt);
             total += dt;
             if (dt < best) best = dt;
         }
@@ -729,12 +741,14 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
     if (!rc && out) ggml_backend_tensor_get(x, out, 0, ggml_nbytes(x));
     if (!rc && reps > 0 && seconds) {
         double best = 1e30, total = 0;
+        g_last_times.clear();
         for (int r = 0; r < reps && !rc; ++r) {
             upload();
             auto t0 = std::chrono::steady_clock::now();
             if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
             auto t1 = std::chrono::steady_clock::now();
             const double d = std::chrono::duration<double>(t1 - t0).count();
+            g_last_times.push_back(d);
             total += d;
             if (d < best) best = d;
         }

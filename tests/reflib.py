@@ -174,6 +174,7 @@ def load_ref():
     lib.rh_flash_attn_ext.argtypes = [TP, TP, TP, TP, f32p, TP, C.c_float, C.c_float, C.c_float, C.c_int, f64p]
     lib.rh_bb_create.argtypes = [C.c_int] * 8 + [C.c_float, C.c_int, C.c_float, C.c_int]
     lib.rh_bb_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    lib.rh_last_times.argtypes = [f64p, C.c_int]
     lib.rh_bb_cache_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_cache_get.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_options.argtypes = [C.c_int, C.c_int]
@@ -195,6 +196,14 @@ def load_ref():
 
 
 # ------------------------------------------------------------------- seeded test data
+def ref_last_times():
+    """Seconds of every timed repeat of the harness's most recent timed run (numpy array)."""
+    lib = load_ref()
+    buf = np.zeros(1 << 16, np.float64)
+    n = lib.rh_last_times(ptr(buf, C.c_double), buf.size)
+    return buf[:min(n, buf.size)].copy()
+
+
 def rng(*key):
     """A generator seeded by a readable key, e.g. rng("cfg1", "q")."""
     import zlib
