@@ -253,7 +253,7 @@ def load_stack(pkg, layers, max_len, batch, kv_f16, lw, params, use_mup=True):
 
 
 def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, prefill=512, steps=256, kv_f16=False,
-                   cpu_reps=40, cpu_prefill=True, plugin_reps=40, f32_prefill_switch=True):
+                   cpu_reps=40, cpu_prefill=True, plugin_reps=40, f32_prefill_switch=False):
     """A whole decoder stack with Q8_0 weights (hidden 1024, 16/2 heads, FFN 4096): BASELINE config 4 (batch 2,
     prefill 512 tokens then 256 decode steps) or config 5 (batch 16, prefill 4096, decode to 8192).  The GPU side is
     the host-side mirror of the reference's layer_forward over the C ABI (voxcpm.cpp_amd/backbone.py), a decode step
@@ -282,9 +282,9 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     big = batch * prefill > 4096
     t_prefill = timer.run(run_p, iters=1 if big else 3, warmup=1)
     t_prefill_f16 = None
-    if not kv_f16 and f32_prefill_switch:
-        # the same prefill with the F32 cache rounded to f16 on its way into the LDS-tiled attention kernel (opt-in, read per call)
-        os.environ["VX_FA_F32_PREFILL"] = "1"
+    if f32_prefill_switch:
+        # the same prefill with its F32 keys and values on the hi/lo wave kernel instead of the LDS-tiled one (read per call)
+        os.environ["VX_FA_F32_PREFILL"] = "0"
         t_prefill_f16 = timer.run(run_p, iters=1 if big else 3, warmup=1)
         del os.environ["VX_FA_F32_PREFILL"]
         timer.run(run_p, iters=1, warmup=0)  # leave the cache as the default route writes it
@@ -311,7 +311,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
            "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
            "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": batch * prefill / t_prefill,
-           "prefill_ms_VX_FA_F32_PREFILL": t_prefill_f16 * 1e3 if t_prefill_f16 else None,
+           "prefill_ms_VX_FA_F32_PREFILL=0": t_prefill_f16 * 1e3 if t_prefill_f16 else None,
            "kv_cache": "f16" if kv_f16 else "f32 (the reference's cache type)",
            "launch": f"captured HIP graph per step, KV lengths {points} ({per} replays each)"}
     del replays, m, xp
@@ -627,7 +627,7 @@ def main():
     if not args.no_others:
         cpu_on = not args.no_cpu
         # BASELINE config 4 with the reference's F32 cache and with the f16 cache BASELINE's configs name
-        others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, cpu_on)
+        others["cfg4_backbone_24layers_b2"] = backbone_bench(pkg, timer, side, threads, cpu_on, f32_prefill_switch=True)
         others["cfg4_backbone_24layers_b2_f16kv"] = backbone_bench(pkg, timer, side, threads, False, kv_f16=True)
         others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, cpu_on)
         others["cfg3_cfm_solve_one_request"] = cfm_solve_bench(pkg, timer, side, threads, cpu_on)
@@ -635,7 +635,7 @@ def main():
         others["cfg5_backbone_24layers_b16_f16kv"] = backbone_bench(pkg, timer, side, threads, cpu_on, batch=16, prefill=4096, steps=4096,
                                                                     kv_f16=True, cpu_reps=3, cpu_prefill=False, plugin_reps=10)
         others["cfg5_backbone_24layers_b16"] = backbone_bench(pkg, timer, side, threads, False, batch=16, prefill=4096, steps=4096,
-                                                              kv_f16=False, plugin_reps=0, f32_prefill_switch=False)
+                                                              kv_f16=False, plugin_reps=0)
 
     cpu = None
     if not args.no_cpu:

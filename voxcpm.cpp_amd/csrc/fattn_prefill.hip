@@ -117,6 +117,9 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
     constexpr int D = 64, NP = 2, SEG = 16;
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][PF_KT][PF_ROW];
     __shared__ __attribute__((aligned(16))) _Float16 vt_lds[2][D][PF_ROW];
+    // F32 values keep their low halves (v - f16(v), itself rounded to f16) in a second image, so that P V carries V to
+    // about 22 bits: without it an output dominated by one key is off by half an f16 ulp of that value
+    __shared__ __attribute__((aligned(16))) _Float16 vtl_lds[KV_F32 ? 2 : 1][KV_F32 ? D : 1][KV_F32 ? PF_ROW : 8];
     __shared__ uint16_t tile_list[PF_MAX_TILES];
     __shared__ uint8_t  tile_flag[PF_MAX_TILES];
     __shared__ int      n_active_s;
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
         const int ld_key = tid >> 3, ld_chunk = tid & 7;
         const char * kg = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3;
         const char * vg = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3;
-        half8_t kreg[2], vreg[2];
+        half8_t kreg[2], vreg[2], vlreg[2];
         // a thread's byte offsets inside a full tile never change: the tile's base is scalar arithmetic
         // and the loads take (scalar base, 32-bit lane offset); only a ragged last tile clamps per lane
         // (K and V share the offsets when their row strides agree, which every cache layout does)
@@ -259,6 +262,8 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                     for (int i = 0; i < 4; ++i) {
                         kreg[hh][i] = (_Float16) k0[i]; kreg[hh][4 + i] = (_Float16) k1[i];
                         vreg[hh][i] = (_Float16) v0[i]; vreg[hh][4 + i] = (_Float16) v1[i];
+                        vlreg[hh][i]     = (_Float16) (v0[i] - (float) vreg[hh][i]);
+                        vlreg[hh][4 + i] = (_Float16) (v1[i] - (float) vreg[hh][4 + i]);
                     }
                 } else {
                     kreg[hh] = *(const half8_t *) (kg + (uint64_t) key * a.nbk1 + ld_chunk * 16);
@@ -279,6 +284,10 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                 // an operand read touches spread over all banks as well
 #pragma unroll
                 for (int i = 0; i < 8; ++i) vt_lds[buf][8 * i + ld_chunk][((grp8 ^ i) << 3) + sub] = vreg[hh][i];
+                if constexpr (KV_F32) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) vtl_lds[buf][8 * i + ld_chunk][((grp8 ^ i) << 3) + sub] = vlreg[hh][i];
+                }
             }
         };
 
@@ -303,6 +312,11 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                 half8_t av[4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) av[t] = *(const half8_t *) &vt_lds[buf][(c & 7) * 8 + 2 * t + (c >> 3)][((hh * 4 + j) ^ (c & 7)) << 3];
+                half8_t avl[4];
+                if constexpr (KV_F32) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) avl[t] = *(const half8_t *) &vtl_lds[buf][(c & 7) * 8 + 2 * t + (c >> 3)][((hh * 4 + j) ^ (c & 7)) << 3];
+                }
 
 #pragma unroll
                 for (int cg = 0; cg < CT; cg += PF_GRP) {
@@ -371,6 +385,10 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
                                 pk2(pb, 4 * h + r, __builtin_amdgcn_exp2f(s[u][h][r]), __builtin_amdgcn_exp2f(s[u][h][r + 1]));
 #pragma unroll
                         for (int t = 0; t < 4; ++t) o[ct][t] = mfma16(av[t], pb, o[ct][t]);
+                        if constexpr (KV_F32) {
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) o[ct][t] = mfma16(avl[t], pb, o[ct][t]);
+                        }
                         ol[ct] = mfma16(ones, pb, ol[ct]);
                     }
                 }
@@ -422,12 +440,14 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
 // (without touching the error string) when the caller should use the general kernel.
 bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float logit_softcap) {
     if (q->ne[0] != 64 || logit_softcap != 0.0f) return false;
-    // F32 K/V are rounded to f16 as they are staged here (relative 2^-11 per element: an output can be off by
-    // half an f16 ulp of a V value, 1.6e-3 measured on unit-scale data), where the general kernel keeps hi + lo
-    // parts (1e-6).  So F32 K/V come here only on request: VX_FA_F32_PREFILL=1, read on every call.
+    // F32 K/V (the reference's own cache type, and what a prefill sees: the keys straight from the projections) are
+    // staged as f16 here -- K rounded like Q is, V as a high and a low half, so the result carries the same error as with
+    // an f16 cache (the rounding of P, about 1.3e-3 on unit-scale data against the 2e-3 bar).  The general kernel keeps
+    // hi + lo parts of everything (1e-6) and is 10 - 20 times slower on such shapes; VX_FA_F32_PREFILL=0 sends F32 K/V
+    // there (read on every call).
     if (k->type == VX_TYPE_F32) {
         const char * e = getenv("VX_FA_F32_PREFILL");
-        if (!e || atoi(e) == 0) return false;
+        if (e && atoi(e) == 0) return false;
     } else if (k->type != VX_TYPE_F16) {
         return false;
     }
