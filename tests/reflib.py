@@ -450,3 +450,79 @@ def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_
                           ptr(out, C.c_float), reps, ptr(sec, C.c_double))
     assert rc == 0, rc
     return out, sec[:2].copy(), int(sec[2])
+
+
+# ------------------------------------------------- the reference's own module layer (oracle/vox_harness.cpp)
+_vox = None
+
+
+def load_vox():
+    """libvox_harness.so: VoxCPMBackend / VoxCPMWeightStore / MiniCPMModel compiled from the reference's sources,
+    or None when oracle/_ref was not prebuilt."""
+    global _vox
+    if _vox is not None:
+        return _vox
+    path = os.path.join(ref_dir(), "libvox_harness.so")
+    if not os.path.exists(path):
+        return None
+    C.CDLL(os.path.join(ref_dir(), "libggml-ref.so"), mode=C.RTLD_GLOBAL)   # a plugin resolves ggml's symbols from the process
+    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    lib.vh_last_error.restype = C.c_char_p
+    lib.vh_backend_name.restype = C.c_char_p
+    lib.vh_weight_bytes.restype = C.c_size_t
+    lib.vh_gguf_begin.argtypes = [C.c_char_p, C.c_size_t]
+    lib.vh_gguf_u32.argtypes = [C.c_char_p, C.c_uint32]
+    lib.vh_gguf_f32.argtypes = [C.c_char_p, C.c_float]
+    lib.vh_gguf_str.argtypes = [C.c_char_p, C.c_char_p]
+    lib.vh_gguf_f32_array.argtypes = [C.c_char_p, C.c_void_p, C.c_int]
+    lib.vh_gguf_tensor.argtypes = [C.c_char_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_size_t]
+    lib.vh_load_plugin.argtypes = [C.c_char_p]
+    lib.vh_open.argtypes = [C.c_int, C.c_int]
+    lib.vh_minicpm_load.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
+    lib.vh_minicpm_run.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_double)]
+    lib.vh_cache_get.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    _vox = lib
+    return lib
+
+
+GGML_TYPE_F32, GGML_TYPE_Q8_0 = 0, 8
+GGUF_LAYER_NAMES = {"q_proj": "attn_q", "k_proj": "attn_k", "v_proj": "attn_v", "o_proj": "attn_output",
+                    "gate_proj": "ffn_gate", "up_proj": "ffn_up", "down_proj": "ffn_down",
+                    "input_layernorm": "attn_norm", "post_layernorm": "ffn_norm"}
+
+
+def write_minicpm_gguf(path, params, prefix, max_len, use_mup=True):
+    """A synthetic model file for MiniCPMModel::load_from_store (src/minicpm.cpp:296-360, 522-570): the decoder stack of
+    backbone_params() under `prefix` ("residual_lm" or "locdit"), written with the reference's gguf API."""
+    lib = load_vox()
+    d = params["dims"]
+    total = sum(a.nbytes for lw in params["layers"] for a in lw.values()) + (64 << 20)
+    ok = lambda rc: (_ for _ in ()).throw(AssertionError(lib.vh_last_error())) if rc else None
+    ok(lib.vh_gguf_begin(path.encode(), total))
+    for key, v in (("llama.embedding_length", d["hidden"]), ("llama.feed_forward_length", d["ffn"]),
+                   ("llama.attention.head_count", d["n_heads"]), ("llama.attention.head_count_kv", d["n_kv"]),
+                   ("llama.context_length", max_len), ("voxcpm_lm_config_use_mup", int(use_mup)),
+                   ("voxcpm_lm_config_rope_scaling_original_max_position_embeddings", 32768),
+                   ("voxcpm_residual_lm_num_layers", d["n_layer"]),
+                   ("voxcpm_dit_config_hidden_dim", d["hidden"]), ("voxcpm_dit_config_ffn_dim", d["ffn"]),
+                   ("voxcpm_dit_config_num_heads", d["n_heads"]), ("voxcpm_dit_config_num_layers", d["n_layer"])):
+        ok(lib.vh_gguf_u32(key.encode(), v))
+    for key, v in (("llama.attention.layer_norm_rms_epsilon", 1e-5), ("llama.rope.freq_base", 10000.0),
+                   ("voxcpm_lm_config_scale_depth", 1.4)):
+        ok(lib.vh_gguf_f32(key.encode(), v))
+    ff = np.ascontiguousarray(params["rope_factors"], np.float32)
+    for key in ("voxcpm_lm_config_rope_scaling_short_factor", "voxcpm_lm_config_rope_scaling_long_factor"):
+        ok(lib.vh_gguf_f32_array(key.encode(), ff.ctypes.data, ff.size))
+    pre = prefix + "." if prefix else ""
+    fn = np.ascontiguousarray(params["final_norm"], np.float32)
+    ok(lib.vh_gguf_tensor((pre + "output_norm.weight").encode(), GGML_TYPE_F32, fn.size, 0, fn.ctypes.data, fn.nbytes))
+    for li, lw in enumerate(params["layers"]):
+        for n, gname in GGUF_LAYER_NAMES.items():
+            a = np.ascontiguousarray(lw[n])
+            name = f"{pre}blk.{li}.{gname}.weight".encode()
+            if n in params["shapes"]:
+                rows, k = params["shapes"][n]
+                ok(lib.vh_gguf_tensor(name, GGML_TYPE_Q8_0, k, rows, a.ctypes.data, a.nbytes))
+            else:
+                ok(lib.vh_gguf_tensor(name, GGML_TYPE_F32, a.size, 0, a.ctypes.data, a.nbytes))
+    ok(lib.vh_gguf_end())

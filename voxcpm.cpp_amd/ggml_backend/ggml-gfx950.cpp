@@ -1407,7 +1407,16 @@ ggml_backend_buffer_type_t device_buffer_type(ggml_backend_dev_t dev) {
     return registry_state(dev->reg)->bufts[((device_ctx *) dev->context)->index];
 }
 
-const char * reg_get_name(ggml_backend_reg_t) { return "GFX950"; }
+// The registry name.  VoxCPM.cpp chooses its GPU device by this name -- it looks for "cuda" or "vulkan" in it
+// (src/backend.cpp:75-105 of the reference) -- so an unpatched VoxCPM build finds this backend when the environment
+// names an alias, e.g. GGML_GFX950_REG_NAME=CUDA-gfx950 with `--backend cuda`; device names stay GFX950_<i>.
+const char * reg_get_name(ggml_backend_reg_t) {
+    static const std::string name = [] {
+        const char * e = getenv("GGML_GFX950_REG_NAME");
+        return std::string(e && *e ? e : "GFX950");
+    }();
+    return name.c_str();
+}
 size_t       reg_get_device_count(ggml_backend_reg_t reg) { return registry_state(reg)->devices.size(); }
 
 ggml_backend_dev_t reg_get_device(ggml_backend_reg_t reg, size_t index) {
