@@ -180,6 +180,93 @@ int vh_minicpm_run(const float * x, int n_tokens, int position, float * out, int
     return 0;
 }
 
+// ---- weight placement -----------------------------------------------------------------------------------------------
+// A model file loaded the way VoxCPMWeightStore::load_from_file does (gguf_init_from_file with no_alloc, one pass over
+// the tensor data, src/weight-store.cpp:58-122), except that the tensors are allocated by the backend's own placement
+// helper (reached through ggml_backend_reg_get_proc_address): the transformer stacks' weights in device memory, the
+// AudioVAE's in pinned host memory.  Then a graph that uses one weight of each kind -- a Q8_0 projection of the stack
+// and the AudioVAE's fc_mu projection + bias + GELU -- runs under ggml_backend_sched over {device, CPU}.
+// use_placement = 0: everything in one buffer of `device` (what the reference does).
+// flags[0] = splits of the scheduled graph, [1] = stack weight in host memory, [2] = audio_vae weight in host memory,
+// [3] = device buffer bytes, [4] = host buffer bytes
+int vh_placed_run(const char * gguf_path, const char * device, int use_placement, const char * w_stack, const char * w_vae,
+                  const char * b_vae, const float * x, int n_tokens, float * out, int64_t * flags) {
+    ggml_context * wctx = nullptr;
+    gguf_init_params gp = { true, &wctx };
+    gguf_context * gg = gguf_init_from_file(gguf_path, gp);
+    if (!gg || !wctx) return fail("gguf_init_from_file failed");
+    ggml_backend_dev_t dev = ggml_backend_dev_by_name(device);
+    if (!dev) return fail("no such device");
+    ggml_backend_t backend = ggml_backend_dev_init(dev, nullptr);
+    ggml_backend_t cpu     = ggml_backend_init_by_type(GGML_BACKEND_DEVICE_TYPE_CPU, nullptr);
+    if (!backend || !cpu) return fail("backend init failed");
+    ggml_backend_cpu_set_n_threads(cpu, 8);
+    ggml_backend_buffer_t dbuf = nullptr, hbuf = nullptr;
+    int rc = 0;
+    if (use_placement) {
+        typedef bool (*alloc_fn)(ggml_context *, ggml_backend_t, ggml_backend_buffer_t *, ggml_backend_buffer_t *);
+        alloc_fn fn = (alloc_fn) ggml_backend_reg_get_proc_address(ggml_backend_dev_backend_reg(dev), "ggml_backend_gfx950_alloc_weights");
+        if (!fn) rc = fail("the backend exports no placement helper");
+        else if (!fn(wctx, backend, &dbuf, &hbuf)) rc = fail("placement failed");
+    } else {
+        dbuf = ggml_backend_alloc_ctx_tensors(wctx, backend);
+        if (!dbuf) rc = fail("allocation failed");
+        else ggml_backend_buffer_set_usage(dbuf, GGML_BACKEND_BUFFER_USAGE_WEIGHTS);
+    }
+    if (!rc) { // one pass over the file
+        FILE * f = fopen(gguf_path, "rb");
+        std::vector<char> tmp;
+        const size_t base = gguf_get_data_offset(gg);
+        for (int64_t i = 0; f && i < gguf_get_n_tensors(gg); ++i) {
+            ggml_tensor * t = ggml_get_tensor(wctx, gguf_get_tensor_name(gg, i));
+            tmp.resize(ggml_nbytes(t));
+            if (fseek(f, (long) (base + gguf_get_tensor_offset(gg, i)), SEEK_SET) != 0 || fread(tmp.data(), 1, tmp.size(), f) != tmp.size()) { rc = fail("short read"); break; }
+            ggml_backend_tensor_set(t, tmp.data(), 0, tmp.size());
+        }
+        if (f) fclose(f); else rc = fail("cannot open the model file");
+    }
+    ggml_tensor * ws = rc ? nullptr : ggml_get_tensor(wctx, w_stack);
+    ggml_tensor * wv = rc ? nullptr : ggml_get_tensor(wctx, w_vae);
+    ggml_tensor * bv = rc ? nullptr : ggml_get_tensor(wctx, b_vae);
+    if (!rc && (!ws || !wv || !bv)) rc = fail("tensor not found");
+    if (!rc) {
+        ggml_init_params ip = { ggml_tensor_overhead() * 32 + ggml_graph_overhead(), nullptr, true };
+        ggml_context * c = ggml_init(ip);
+        ggml_tensor * inp = ggml_new_tensor_2d(c, GGML_TYPE_F32, ws->ne[0], n_tokens);
+        ggml_set_input(inp);
+        ggml_tensor * y = ggml_mul_mat(c, ws, inp);                          // the stack's projection: device weight
+        ggml_tensor * z = ggml_gelu(c, ggml_add(c, ggml_mul_mat(c, wv, y), bv)); // the AudioVAE side: host weights, GELU is not claimed
+        ggml_set_output(z);
+        ggml_cgraph * gf = ggml_new_graph(c);
+        ggml_build_forward_expand(gf, z);
+        ggml_backend_t backs[2] = { backend, cpu };
+        const bool same = ggml_backend_dev_type(dev) == GGML_BACKEND_DEVICE_TYPE_CPU;
+        ggml_backend_sched_t sched = ggml_backend_sched_new(same ? backs + 1 : backs, nullptr, same ? 1 : 2, 64, false, true);
+        if (!sched || !ggml_backend_sched_alloc_graph(sched, gf)) rc = fail("scheduler allocation failed");
+        if (!rc) {
+            ggml_backend_tensor_set(inp, x, 0, ggml_nbytes(inp));
+            if (ggml_backend_sched_graph_compute(sched, gf) != GGML_STATUS_SUCCESS) rc = fail("scheduled compute failed");
+        }
+        if (!rc) {
+            ggml_backend_tensor_get(z, out, 0, ggml_nbytes(z));
+            flags[0] = ggml_backend_sched_get_n_splits(sched);
+            flags[1] = ggml_backend_buffer_is_host(ws->buffer) ? 1 : 0;
+            flags[2] = ggml_backend_buffer_is_host(wv->buffer) ? 1 : 0;
+            flags[3] = dbuf ? (int64_t) ggml_backend_buffer_get_size(dbuf) : 0;
+            flags[4] = hbuf ? (int64_t) ggml_backend_buffer_get_size(hbuf) : 0;
+        }
+        if (sched) ggml_backend_sched_free(sched);
+        ggml_free(c);
+    }
+    if (dbuf) ggml_backend_buffer_free(dbuf);
+    if (hbuf) ggml_backend_buffer_free(hbuf);
+    ggml_backend_free(cpu);
+    ggml_backend_free(backend);
+    gguf_free(gg);
+    ggml_free(wctx);
+    return rc;
+}
+
 // one layer's K (which = 0) or V (1) cache as the reference allocated it: [head_dim, max_length, n_kv_heads] F32
 int vh_cache_get(int layer, int which, float * out, size_t nbytes) {
     if (!g_cache || !g_backend) return 1;

@@ -481,6 +481,8 @@ def load_vox():
     lib.vh_minicpm_load.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
     lib.vh_minicpm_run.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_double)]
     lib.vh_cache_get.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
+    lib.vh_placed_run.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_char_p, C.c_char_p, C.c_char_p, C.c_void_p, C.c_int, C.c_void_p,
+                                  C.POINTER(C.c_int64)]
     _vox = lib
     return lib
 
@@ -491,7 +493,7 @@ GGUF_LAYER_NAMES = {"q_proj": "attn_q", "k_proj": "attn_k", "v_proj": "attn_v", 
                     "input_layernorm": "attn_norm", "post_layernorm": "ffn_norm"}
 
 
-def write_minicpm_gguf(path, params, prefix, max_len, use_mup=True):
+def write_minicpm_gguf(path, params, prefix, max_len, use_mup=True, extra=()):
     """A synthetic model file for MiniCPMModel::load_from_store (src/minicpm.cpp:296-360, 522-570): the decoder stack of
     backbone_params() under `prefix` ("residual_lm" or "locdit"), written with the reference's gguf API."""
     lib = load_vox()
@@ -525,4 +527,7 @@ def write_minicpm_gguf(path, params, prefix, max_len, use_mup=True):
                 ok(lib.vh_gguf_tensor(name, GGML_TYPE_Q8_0, k, rows, a.ctypes.data, a.nbytes))
             else:
                 ok(lib.vh_gguf_tensor(name, GGML_TYPE_F32, a.size, 0, a.ctypes.data, a.nbytes))
+    for name, a in extra:   # further F32 tensors (name, array of 1 or 2 dims)
+        a = np.ascontiguousarray(a, np.float32)
+        ok(lib.vh_gguf_tensor(name.encode(), GGML_TYPE_F32, a.shape[-1], a.shape[0] if a.ndim == 2 else 0, a.ctypes.data, a.nbytes))
     ok(lib.vh_gguf_end())

@@ -303,3 +303,36 @@ def test_workspace_growth_policy(tmp_path):
     subprocess.check_call(["g++", "-std=c++17", "-O1", "-o", exe, os.path.join(ROOT, "tests", "ws_policy_check.cpp")])
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.strip() == "ok", out.stdout + out.stderr
+
+
+def test_weight_placement_policy(pkg):
+    """Which tensors of a VoxCPM model file the plugin's placement helper sends to device memory and which to pinned
+    host memory, by the reference's GGUF tensor names (src/minicpm.cpp:522-570, src/locdit.cpp, src/audio-vae.cpp:164-303):
+    what the claimed operators consume goes to the device, the AudioVAE's weights stay with ggml-cpu."""
+    import ctypes
+    if not os.path.exists(pkg.PLUGIN_PATH):
+        pytest.skip("the ggml plugin was not built")
+    # the plugin resolves ggml's symbols from the process, as every dynamically loaded ggml backend does
+    ref_dir = reflib.ref_dir()
+    if not os.path.exists(os.path.join(ref_dir, "libggml-ref.so")):
+        pytest.skip("oracle/_ref was not prebuilt")
+    ctypes.CDLL(os.path.join(ref_dir, "libggml-ref.so"), mode=ctypes.RTLD_GLOBAL)
+    plugin = ctypes.CDLL(pkg.PLUGIN_PATH)
+    on_device = lambda n: plugin.ggml_backend_gfx950_weight_on_device(n.encode())
+    for name in ("token_embd.weight", "output_norm.weight", "blk.0.attn_q.weight", "blk.23.ffn_down.weight", "blk.3.attn_norm.weight",
+                 "residual_lm.blk.5.attn_k.weight", "residual_lm.output_norm.weight", "locenc.in_proj.weight", "locenc.blk.0.ffn_up.weight",
+                 "locdit.in_proj.weight", "locdit.cond_proj.bias", "locdit.time_mlp.linear_1.weight", "locdit.blk.3.attn_v.weight",
+                 "fsq.in_proj.weight", "stop.stop_proj.weight", "stop.stop_head.weight"):
+        assert on_device(name) == 1, name
+    for name in ("audio_vae.encoder.block.0.weight", "audio_vae.encoder.fc_mu.weight", "audio_vae.encoder.fc_mu.bias",
+                 "audio_vae.decoder.model.0.weight", "audio_vae.decoder.model.1.block.0.block.1.alpha", "audio_vae.decoder.model.7.bias"):
+        assert on_device(name) == 0, name
+    # every helper is also handed out by name, the way ggml exposes backend-specific functions
+    reg = plugin.ggml_backend_gfx950_reg
+    reg.restype = ctypes.c_void_p
+    ggml = ctypes.CDLL(os.path.join(ref_dir, "libggml-ref.so"))
+    ggml.ggml_backend_reg_get_proc_address.restype = ctypes.c_void_p
+    ggml.ggml_backend_reg_get_proc_address.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+    for fn in ("ggml_backend_gfx950_weight_on_device", "ggml_backend_gfx950_alloc_weights", "ggml_backend_gfx950_last_launches"):
+        assert ggml.ggml_backend_reg_get_proc_address(reg(), fn.encode())
+    assert not ggml.ggml_backend_reg_get_proc_address(reg(), b"no_such_function")

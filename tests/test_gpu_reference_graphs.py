@@ -114,3 +114,44 @@ def test_plugin_on_graphs_built_by_the_reference(gpu, ref, tmp_path):
         assert nmse(cpu[i], o[0]) <= 1e-10
         pos += x.shape[0]
     ref.rh_bb_free()
+
+
+def test_weight_placement_under_the_scheduler(gpu, ref, tmp_path):
+    """A model file with the stack's weights and AudioVAE weights, allocated by the plugin's placement helper (stack ->
+    device buffer, audio_vae.* -> pinned host buffer) instead of the reference's one-buffer rule, and a graph with one
+    weight of each kind under ggml_backend_sched over {plugin, CPU}: the projection of the stack runs on the plugin, the
+    AudioVAE side (host weights, an operator the plugin does not claim) on ggml-cpu, and the result equals ggml-cpu's."""
+    import ctypes
+    vox = reflib.load_vox()
+    if vox is None:
+        pytest.skip("oracle/_ref/libvox_harness.so was not prebuilt")
+    params = reflib.backbone_params("place", 1)
+    g = rng("place", "vae")
+    extra = [("audio_vae.encoder.fc_mu.weight", (g.standard_normal((64, 1024)) / 32).astype(np.float32)),
+             ("audio_vae.encoder.fc_mu.bias", (0.1 * g.standard_normal(64)).astype(np.float32)),
+             ("audio_vae.decoder.model.0.weight", g.standard_normal((7, 64)).astype(np.float32))]
+    gguf = str(tmp_path / "placed.gguf")
+    reflib.write_minicpm_gguf(gguf, params, "residual_lm", 4096, extra=extra)
+    T = 9
+    x = rng("place", "x").standard_normal((T, 1024)).astype(np.float32)
+    names = (b"residual_lm.blk.0.attn_q.weight", b"audio_vae.encoder.fc_mu.weight", b"audio_vae.encoder.fc_mu.bias")
+
+    def run(device, placement):
+        out = np.zeros((T, 64), np.float32)
+        flags = (ctypes.c_int64 * 5)()
+        rc = vox.vh_placed_run(gguf.encode(), device, placement, *names, x.ctypes.data, T, out.ctypes.data, flags)
+        assert rc == 0, vox.vh_last_error()
+        return out, list(flags)
+
+    cpu, cf = run(b"CPU", 0)
+    assert vox.vh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    placed, pf = run(b"GFX950_0", 1)
+    one_buf, of = run(b"GFX950_0", 0)
+    print(f"placement: splits {pf[0]}, stack weight on host {pf[1]}, audio_vae weight on host {pf[2]}, device buffer {pf[3] >> 20} MiB, "
+          f"host buffer {pf[4]} bytes; one-buffer rule: splits {of[0]}, device buffer {of[3] >> 20} MiB", flush=True)
+    assert pf[1] == 0 and pf[2] == 1 and pf[3] > 15 << 20 and 0 < pf[4] < 1 << 20
+    assert of[1] == 0 and of[2] == 0 and of[4] == 0          # the reference's rule: everything on the device
+    assert pf[0] == 2                                          # the plugin's part, then ggml-cpu's
+    e = nmse(cpu, placed)
+    print(f"   placed weights vs ggml-cpu: nmse {e:.3e};  one buffer vs ggml-cpu: nmse {nmse(cpu, one_buf):.3e}", flush=True)
+    assert e <= 1e-4 and nmse(cpu, one_buf) <= 1e-4

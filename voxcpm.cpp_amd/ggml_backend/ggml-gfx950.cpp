@@ -22,6 +22,8 @@
 #include "ggml-impl.h"
 #include "ggml.h"
 
+#include "ggml-alloc.h"
+#include "ggml-gfx950.h"
 #include "voxcpm_gfx950.h"
 
 #include <cstddef>
@@ -1425,7 +1427,14 @@ ggml_backend_dev_t reg_get_device(ggml_backend_reg_t reg, size_t index) {
     return ctx->devices[index];
 }
 
-void * reg_get_proc_address(ggml_backend_reg_t, const char *) { return nullptr; }
+void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
+    if (!name) return nullptr;
+    if (strcmp(name, "ggml_backend_gfx950_weight_on_device") == 0) return (void *) ggml_backend_gfx950_weight_on_device;
+    if (strcmp(name, "ggml_backend_gfx950_alloc_weights") == 0) return (void *) ggml_backend_gfx950_alloc_weights;
+    if (strcmp(name, "ggml_backend_gfx950_last_launches") == 0) return (void *) ggml_backend_gfx950_last_launches;
+    if (strcmp(name, "ggml_backend_gfx950_set_mul_mat_act") == 0) return (void *) ggml_backend_gfx950_set_mul_mat_act;
+    return nullptr;
+}
 
 } // namespace
 
@@ -1448,10 +1457,61 @@ GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_
 
 // Diagnostic: how many operator calls the most recent graph_compute of this process issued (an attention
 // call counts once although it may launch a split and a merge kernel).
-extern "C" __attribute__((visibility("default"))) int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
+extern "C" int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
+
+// ---- weight placement (declared and explained in ggml-gfx950.h) ------------------------------------------------------
+extern "C" int ggml_backend_gfx950_weight_on_device(const char * tensor_name) {
+    if (!tensor_name) return 1;
+    return strncmp(tensor_name, "audio_vae.", 10) == 0 ? 0 : 1;
+}
+
+extern "C" bool ggml_backend_gfx950_alloc_weights(struct ggml_context * ctx, ggml_backend_t backend, ggml_backend_buffer_t * device_buffer,
+                                                  ggml_backend_buffer_t * host_buffer) {
+    if (device_buffer) *device_buffer = nullptr;
+    if (host_buffer) *host_buffer = nullptr;
+    if (!ctx || !backend || !device_buffer || !host_buffer) return false;
+    ggml_backend_dev_t dev = ggml_backend_get_device(backend);
+    if (!dev) return false;
+    ggml_backend_buffer_type_t host_buft = ggml_backend_dev_host_buffer_type(dev);
+    ggml_backend_buffer_type_t dev_buft  = ggml_backend_dev_buffer_type(dev);
+    if (!host_buft || !dev_buft) return false;
+    // the host share first: its tensors are placed one after the other in one pinned block
+    const size_t align = ggml_backend_buft_get_alignment(host_buft);
+    size_t host_bytes = 0, n_host = 0, n_dev = 0;
+    for (ggml_tensor * t = ggml_get_first_tensor(ctx); t; t = ggml_get_next_tensor(ctx, t)) {
+        if (t->data || t->view_src) continue;
+        if (ggml_backend_gfx950_weight_on_device(t->name)) { ++n_dev; continue; }
+        host_bytes += GGML_PAD(ggml_backend_buft_get_alloc_size(host_buft, t), align);
+        ++n_host;
+    }
+    if (n_host) {
+        *host_buffer = ggml_backend_buft_alloc_buffer(host_buft, host_bytes);
+        if (!*host_buffer) return false;
+        ggml_backend_buffer_set_usage(*host_buffer, GGML_BACKEND_BUFFER_USAGE_WEIGHTS);
+        ggml_tallocr talloc = ggml_tallocr_new(*host_buffer);
+        for (ggml_tensor * t = ggml_get_first_tensor(ctx); t; t = ggml_get_next_tensor(ctx, t)) {
+            if (t->data || t->view_src || ggml_backend_gfx950_weight_on_device(t->name)) continue;
+            if (ggml_tallocr_alloc(&talloc, t) != GGML_STATUS_SUCCESS) {
+                ggml_backend_buffer_free(*host_buffer);
+                *host_buffer = nullptr;
+                return false;
+            }
+        }
+    }
+    if (n_dev) { // ggml allocates whatever is still unallocated (views included) in one buffer of the device type
+        *device_buffer = ggml_backend_alloc_ctx_tensors_from_buft(ctx, dev_buft);
+        if (!*device_buffer) {
+            if (*host_buffer) ggml_backend_buffer_free(*host_buffer);
+            *host_buffer = nullptr;
+            return false;
+        }
+        ggml_backend_buffer_set_usage(*device_buffer, GGML_BACKEND_BUFFER_USAGE_WEIGHTS);
+    }
+    return true;
+}
 // Selects VX_ACT_FLOAT (0) or VX_ACT_Q8 (1) for the Q8_0 products of later graph_compute calls; returns the previous
 // mode.  The environment variable GGML_GFX950_MUL_MAT_ACT=q8 sets the initial one.
-extern "C" __attribute__((visibility("default"))) int ggml_backend_gfx950_set_mul_mat_act(int mode) {
+extern "C" int ggml_backend_gfx950_set_mul_mat_act(int mode) {
     const int before = mul_mat_act_mode();
     if (mode == VX_ACT_FLOAT || mode == VX_ACT_Q8) g_mul_mat_act = mode;
     return before;
