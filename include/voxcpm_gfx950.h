@@ -83,6 +83,18 @@ VX_API vx_status    vx_workspace_reserve(vx_stream stream, size_t bytes);
 /* current block, its size and the number of superseded blocks still held for this stream (any out pointer may be NULL) */
 VX_API vx_status    vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int * retired_blocks);
 
+/* Recording the launches of a stream and replaying them as one unit (a HIP graph).  The reference builds and launches
+ * its step graph anew on every call (src/voxcpm.cpp:485-495); a backend that recognises a graph it has already run can
+ * replay the recorded launches instead of issuing them one by one.  Between begin and end every vx_* call on `stream`
+ * is recorded, not executed; a call that would have to grow the workspace fails (see vx_workspace_reserve) and the
+ * caller should end the recording, discard it and run eagerly.  The pointers and shapes of the recorded calls are
+ * baked in: replay only while they are all still valid.  No counterpart in ggml-cpu. */
+typedef void * vx_graph;
+VX_API vx_status    vx_graph_begin(vx_stream stream);
+VX_API vx_status    vx_graph_end(vx_stream stream, vx_graph * graph);   /* *graph = NULL when nothing usable was recorded */
+VX_API vx_status    vx_graph_launch(vx_graph graph, vx_stream stream);
+VX_API vx_status    vx_graph_destroy(vx_graph graph);
+
 /* ---- GGML_OP_RMS_NORM -------------------------------------------------------------------
  * replaces ggml_compute_forward_rms_norm (ggml/src/ggml-cpu/ops.cpp:3710-3777).
  * src, dst F32, same shape, ne[0] dense; rows may be strided; dst may alias src. */

@@ -175,6 +175,8 @@ def load_ref():
     lib.rh_bb_create.argtypes = [C.c_int] * 8 + [C.c_float, C.c_int, C.c_float, C.c_int]
     lib.rh_bb_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_last_times.argtypes = [f64p, C.c_int]
+    lib.rh_out_after_reps.argtypes = [C.c_int]
+    lib.rh_out_after_reps.restype = None
     lib.rh_bb_cache_set.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_cache_get.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     lib.rh_bb_options.argtypes = [C.c_int, C.c_int]

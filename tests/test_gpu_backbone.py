@@ -372,3 +372,50 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref, time_table):
     print(f"   C ABI mirror: {run.n_calls} calls per solve", flush=True)
     assert launches - 2 <= run.n_calls <= launches, (run.n_calls, launches)   # ggml's node order splits one run of tiny nodes in two
     assert x.cpu().numpy().tobytes() == plug.tobytes()
+
+
+def test_plugin_replays_a_recurring_graph(gpu, ref):
+    """A graph the plugin has run twice is recorded on its third run and replayed from then on (a CFM solve has the same
+    shapes and addresses on every call; the reference rebuilds and relaunches it each time, src/voxcpm.cpp:485-495).
+    The replays must give what node-by-node launches give, with the host writing fresh inputs between them, with other
+    graphs run in between, and a graph of another shape must never be mistaken for a recorded one."""
+    import ctypes
+    params = reflib.backbone_params("locdit", 4)
+    cp = reflib.cfm_params("cfm")
+    mu = rng("cfmr", "mu").standard_normal(1024).astype(np.float32)
+    cond = rng("cfmr", "cond").standard_normal((4, 64)).astype(np.float32)
+    table = rng("cfmr", "table").standard_normal((10, 1024)).astype(np.float32)
+    zs = [rng("cfmr", "z", i).standard_normal((2, 64)).astype(np.float32) for i in range(3)]
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+
+    def solve_all(device, replay, reps):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        before = plugin.ggml_backend_gfx950_set_graph_replay(int(replay))
+        ref.rh_out_after_reps(1)
+        try:
+            reflib.ref_backbone_create(params, 32, 1, use_mup=True, kv_f16=False, fused_weights=True)
+            reflib.ref_cfm_create(cp)
+            outs = []
+            for z in zs:
+                outs.append(reflib.ref_cfm_solve(z, mu, cond, table, reps=reps)[0])            # the last repeat's result
+                outs.append(reflib.ref_cfm_solve(z[:1], mu, cond[:2], table, reps=0)[0])       # another shape in between
+            return outs
+        finally:
+            ref.rh_out_after_reps(0)
+            plugin.ggml_backend_gfx950_set_graph_replay(before)
+            ref.rh_cfm_free()
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plain = solve_all(b"GFX950_0", False, 4)
+    n0 = plugin.ggml_backend_gfx950_replays()
+    replayed = solve_all(b"GFX950_0", True, 4)
+    n1 = plugin.ggml_backend_gfx950_replays()
+    print(f"recurring CFM solve graph: {n1 - n0} of {len(zs) * 6} graph_compute calls were replays", flush=True)
+    assert n1 - n0 >= len(zs) * 2          # runs 3, 4, 5 of every five identical computes at the least
+    for i, (a, b) in enumerate(zip(plain, replayed)):
+        assert np.array_equal(a, b), f"solve {i}: a replay differs from node-by-node launches"
+    cpu = solve_all(b"CPU", False, 0)
+    for i, (a, b) in enumerate(zip(cpu, replayed)):
+        assert nmse(a, b) <= 1e-3, i

@@ -187,6 +187,39 @@ vx_status vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int *
     if (retired_blocks) *retired_blocks = it == g_ws.end() ? 0 : (int) it->second.retired.size();
     return VX_OK;
 }
+vx_status vx_graph_begin(vx_stream stream) {
+    VX_HIP(hipStreamBeginCapture((hipStream_t) stream, hipStreamCaptureModeThreadLocal));
+    return VX_OK;
+}
+vx_status vx_graph_end(vx_stream stream, vx_graph * graph) {
+    if (!graph) return vx_fail(VX_ERR_INVALID, "vx_graph_end: null out pointer");
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture((hipStream_t) stream, &g);
+    if (e != hipSuccess || !g) { // an invalidated recording: the stream is usable again, nothing to replay
+        (void) hipGetLastError();
+        if (g) (void) hipGraphDestroy(g);
+        return VX_OK;
+    }
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e2 = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void) hipGraphDestroy(g);
+    if (e2 != hipSuccess || !exec) {
+        (void) hipGetLastError();
+        return VX_OK;
+    }
+    *graph = (vx_graph) exec;
+    return VX_OK;
+}
+vx_status vx_graph_launch(vx_graph graph, vx_stream stream) {
+    if (!graph) return vx_fail(VX_ERR_INVALID, "vx_graph_launch: null graph");
+    VX_HIP(hipGraphLaunch((hipGraphExec_t) graph, (hipStream_t) stream));
+    return VX_OK;
+}
+vx_status vx_graph_destroy(vx_graph graph) {
+    if (graph) VX_HIP(hipGraphExecDestroy((hipGraphExec_t) graph));
+    return VX_OK;
+}
 vx_status vx_stream_synchronize(vx_stream stream) {
     VX_HIP(hipStreamSynchronize((hipStream_t) stream));
     return VX_OK;

@@ -95,9 +95,28 @@ struct device_ctx {
     std::string description;
 };
 
+// A graph this backend has run before, recognised by a fingerprint of everything a launch depends on (operators,
+// parameters, shapes, strides and addresses of every node and operand): from its third identical run on, the recorded
+// launches are replayed as one HIP graph instead of being analysed and issued again.
+struct seen_graph {
+    uint64_t cheap = 0;      // a quick signature; only graphs that agree on it are fingerprinted in full
+    uint64_t fingerprint = 0;
+    int      runs = 0;       // identical runs so far
+    int      launches = 0;
+    bool     no_replay = false; // recording failed once: keep launching it node by node
+    vx_graph recorded = nullptr;
+    uint64_t last_use = 0;
+};
+
 struct backend_ctx {
     int       device;
     vx_stream stream;
+    std::vector<seen_graph> seen;   // a handful of entries, least recently used one replaced
+    uint64_t  clock = 0;
+    // what graph_optimize worked out for a graph object, for the graph_compute that follows on the same object
+    const ggml_cgraph * opt_graph = nullptr;
+    uint64_t  opt_cheap = 0, opt_fingerprint = 0;
+    int       replays = 0;          // diagnostic: graph_compute calls served by a replay
 };
 
 struct buffer_ctx {
@@ -448,6 +467,7 @@ void backend_free(ggml_backend_t backend) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     vx_init(ctx->device);
     vx_stream_synchronize(ctx->stream);
+    for (seen_graph & g : ctx->seen) if (g.recorded) vx_graph_destroy(g.recorded);
     vx_stream_destroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -1134,14 +1154,140 @@ bool compute_fused_gate_up_group(backend_ctx * ctx, const ggml_cgraph * g, int i
 }
 
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
+int g_replays = 0;       // graph_compute calls of this process that were served by replaying recorded launches
+int g_replay_on = -1;    // recognise recurring graphs and replay them (GGML_GFX950_GRAPH_REPLAY, ggml_backend_gfx950_set_graph_replay)
+
+// ---- recognising a graph ---------------------------------------------------------------------------------------------
+inline uint64_t mix64(uint64_t h, uint64_t v) {
+    h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
+    return h * 0xff51afd7ed558ccdull;
+}
+// cheap: node count, and per node the operator, the output address and the two outer extents (what changes from one
+// decode step to the next: the key count) -- a few hundred nanoseconds per thousand nodes
+uint64_t graph_cheap_signature(const ggml_cgraph * g) {
+    uint64_t h = (uint64_t) g->n_nodes;
+    for (int i = 0; i < g->n_nodes; ++i) {
+        const ggml_tensor * n = g->nodes[i];
+        h = mix64(h, (uint64_t) (uintptr_t) n->data ^ ((uint64_t) n->op << 56) ^ ((uint64_t) n->ne[1] << 20) ^ ((uint64_t) n->ne[2] << 40));
+    }
+    return h | 1;
+}
+void fingerprint_tensor(uint64_t & h, const ggml_tensor * t) {
+    h = mix64(h, (uint64_t) (uintptr_t) t->data);
+    h = mix64(h, ((uint64_t) t->type << 32) ^ (uint64_t) t->op ^ ((uint64_t) t->flags << 48));
+    for (int d = 0; d < GGML_MAX_DIMS; ++d) h = mix64(h, (uint64_t) t->ne[d] ^ ((uint64_t) t->nb[d] << 24));
+}
+// full: everything a launch is derived from
+uint64_t graph_fingerprint(const ggml_cgraph * g) {
+    uint64_t h = 0x243F6A8885A308D3ull ^ (uint64_t) g->n_nodes;
+    for (int i = 0; i < g->n_nodes; ++i) {
+        const ggml_tensor * n = g->nodes[i];
+        fingerprint_tensor(h, n);
+        const uint64_t * op = (const uint64_t *) n->op_params;
+        for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(uint64_t); ++k) h = mix64(h, op[k]);
+        for (int k = 0; k < GGML_MAX_SRC; ++k) {
+            if (!n->src[k]) { h = mix64(h, 0x55); continue; }
+            fingerprint_tensor(h, n->src[k]);
+        }
+        h = mix64(h, (uint64_t) (uintptr_t) (n->view_src ? n->view_src->data : nullptr) ^ (uint64_t) n->view_offs);
+    }
+    return h | 1;
+}
+
+ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out);
+
+// graph_optimize (ggml/src/ggml-backend-impl.h:118-119): ggml_backend_sched calls it once per split when it lays a graph
+// out.  Nothing is reordered; the graph's signatures are worked out here, once, so that the graph_compute calls on the
+// same graph object need not hash it again.
+void backend_graph_optimize(ggml_backend_t backend, ggml_cgraph * cgraph) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    ctx->opt_graph = nullptr;
+    if (!cgraph || cgraph->n_nodes < 8) return;
+    ctx->opt_cheap       = graph_cheap_signature(cgraph);
+    ctx->opt_fingerprint = graph_fingerprint(cgraph);
+    ctx->opt_graph       = cgraph;
+}
 
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
-    int launches = 0;
     if (vx_init(ctx->device) != VX_OK) {
         GGML_LOG_ERROR("ggml-gfx950: %s\n", vx_last_error());
         return GGML_STATUS_FAILED;
     }
+    // GGML_GFX950_GRAPH_REPLAY=0 switches the recognition off; test-backend-ops style one-node graphs never qualify
+    if (g_replay_on < 0) { const char * e = getenv("GGML_GFX950_GRAPH_REPLAY"); g_replay_on = !(e && atoi(e) == 0); }
+    int launches = 0;
+    if (!g_replay_on || cgraph->n_nodes < 8) {
+        const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+        g_last_launches = launches;
+        return st;
+    }
+    const uint64_t cheap = graph_cheap_signature(cgraph);
+    const bool from_opt = ctx->opt_graph == cgraph && ctx->opt_cheap == cheap;
+    seen_graph * entry = nullptr;
+    for (seen_graph & g : ctx->seen) if (g.cheap == cheap) { entry = &g; break; }
+    ++ctx->clock;
+    if (!entry) { // first sight: remember the cheap signature only (a decode step's graph never comes back)
+        constexpr size_t MAX_SEEN = 8;
+        if (ctx->seen.size() < MAX_SEEN) { ctx->seen.emplace_back(); entry = &ctx->seen.back(); }
+        else {
+            entry = &ctx->seen[0];
+            for (seen_graph & g : ctx->seen) if (g.last_use < entry->last_use) entry = &g;
+            if (entry->recorded) vx_graph_destroy(entry->recorded);
+            *entry = seen_graph{};
+        }
+        entry->cheap = cheap;
+        entry->runs = 1;
+        entry->last_use = ctx->clock;
+        const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+        entry->launches = launches;
+        g_last_launches = launches;
+        return st;
+    }
+    entry->last_use = ctx->clock;
+    const uint64_t fp = from_opt ? ctx->opt_fingerprint : graph_fingerprint(cgraph);
+    if (entry->fingerprint != fp) { // second sight (or a different graph with the same quick signature): start counting
+        if (entry->recorded) vx_graph_destroy(entry->recorded);
+        entry->recorded = nullptr;
+        entry->fingerprint = fp;
+        entry->runs = 1;
+        entry->no_replay = false;
+    }
+    ++entry->runs;
+    if (entry->recorded) {
+        if (vx_graph_launch(entry->recorded, ctx->stream) == VX_OK) {
+            ++g_replays;
+            g_last_launches = entry->launches;
+            return GGML_STATUS_SUCCESS;
+        }
+        vx_graph_destroy(entry->recorded);
+        entry->recorded = nullptr;
+        entry->no_replay = true;
+    }
+    if (entry->runs >= 3 && !entry->no_replay) { // the same graph for the third time: record its launches, then replay them
+        if (vx_graph_begin(ctx->stream) == VX_OK) {
+            const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+            vx_graph rec = nullptr;
+            vx_graph_end(ctx->stream, &rec);
+            if (st == GGML_STATUS_SUCCESS && rec && vx_graph_launch(rec, ctx->stream) == VX_OK) {
+                entry->recorded = rec;
+                entry->launches = launches;
+                ++g_replays;
+                g_last_launches = launches;
+                return GGML_STATUS_SUCCESS;
+            }
+            if (rec) vx_graph_destroy(rec);
+        }
+        entry->no_replay = true; // e.g. a launch that must allocate: this graph stays with node-by-node launches
+    }
+    const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+    entry->launches = launches;
+    g_last_launches = launches;
+    return st;
+}
+
+ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out) {
+    int launches = 0;
     // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
     // nodes is only run as one launch when nothing else looks at the value between them
     static const bool fusion = getenv("GGML_GFX950_NO_FUSION") == nullptr;
@@ -1291,7 +1437,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
             return GGML_STATUS_FAILED;
         }
     }
-    g_last_launches = launches;
+    *launches_out = launches;
     return GGML_STATUS_SUCCESS;
 }
 
@@ -1309,7 +1455,7 @@ const ggml_backend_i backend_iface = {
     /* .graph_compute      = */ backend_graph_compute,
     /* .event_record       = */ nullptr,
     /* .event_wait         = */ nullptr,
-    /* .graph_optimize     = */ nullptr,
+    /* .graph_optimize     = */ backend_graph_optimize,
 };
 
 ggml_guid_t backend_guid() {
@@ -1432,6 +1578,8 @@ void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
     if (strcmp(name, "ggml_backend_gfx950_weight_on_device") == 0) return (void *) ggml_backend_gfx950_weight_on_device;
     if (strcmp(name, "ggml_backend_gfx950_alloc_weights") == 0) return (void *) ggml_backend_gfx950_alloc_weights;
     if (strcmp(name, "ggml_backend_gfx950_last_launches") == 0) return (void *) ggml_backend_gfx950_last_launches;
+    if (strcmp(name, "ggml_backend_gfx950_replays") == 0) return (void *) ggml_backend_gfx950_replays;
+    if (strcmp(name, "ggml_backend_gfx950_set_graph_replay") == 0) return (void *) ggml_backend_gfx950_set_graph_replay;
     if (strcmp(name, "ggml_backend_gfx950_set_mul_mat_act") == 0) return (void *) ggml_backend_gfx950_set_mul_mat_act;
     return nullptr;
 }
@@ -1458,6 +1606,15 @@ GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_
 // Diagnostic: how many operator calls the most recent graph_compute of this process issued (an attention
 // call counts once although it may launch a split and a merge kernel).
 extern "C" int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
+// how many graph_compute calls of this process were served by replaying a recorded graph
+extern "C" int ggml_backend_gfx950_replays(void) { return g_replays; }
+// switches the recognition of recurring graphs on (1) or off (0); returns the previous setting
+extern "C" int ggml_backend_gfx950_set_graph_replay(int on) {
+    if (g_replay_on < 0) { const char * e = getenv("GGML_GFX950_GRAPH_REPLAY"); g_replay_on = !(e && atoi(e) == 0); }
+    const int before = g_replay_on;
+    g_replay_on = on != 0;
+    return before;
+}
 
 // ---- weight placement (declared and explained in ggml-gfx950.h) ------------------------------------------------------
 extern "C" int ggml_backend_gfx950_weight_on_device(const char * tensor_name) {

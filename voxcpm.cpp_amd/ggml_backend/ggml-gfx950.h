@@ -37,6 +37,8 @@ GGML_BACKEND_API bool ggml_backend_gfx950_alloc_weights(struct ggml_context * ct
 
 /* diagnostics and switches */
 GGML_BACKEND_API int ggml_backend_gfx950_last_launches(void);
+GGML_BACKEND_API int ggml_backend_gfx950_set_graph_replay(int on);  /* recognise recurring graphs and replay them; returns the previous setting */
+GGML_BACKEND_API int ggml_backend_gfx950_replays(void);   /* graph_compute calls served by replaying recorded launches */
 GGML_BACKEND_API int ggml_backend_gfx950_set_mul_mat_act(int mode);
 
 #ifdef __cplusplus
