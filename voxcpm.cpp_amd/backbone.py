@@ -266,6 +266,7 @@ class MiniCPMBackbone:
                     check(rc, fn.__name__)
 
         run._keep = keep
+        run.calls = calls           # (function, arguments) in launch order, for tools that time parts of a step
         run.n_calls = len(calls)
         return run, out
 
