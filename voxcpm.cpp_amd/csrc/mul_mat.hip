@@ -69,6 +69,12 @@ struct mm_args {
     // (x is then the un-normalised tensor): x[t][k] / rms(x[t]) * norm_w[k], rounded after each product
     const float * norm_w;
     float norm_eps;
+    // GEMV prologue helpers, filled in by launch_gemv: everything a wave needs before it can request its weights is
+    // kept free of integer divisions (a dependent chain of some thirty instructions each, ahead of the first load)
+    int   nbatch;     // ne12 * ne13 of the activations; 1: no batch index arithmetic at all
+    float inv_upr;    // 1 / (K / 8): (unit + 0.5) * inv_upr truncates to unit / (K / 8) exactly for every unit of a chunk
+    int   half_shift; // log2(head_dim / 2) when that is a power of two, else -1
+    int   exact;      // every wave's blocks fill its load rounds exactly: no clamping of block indices
 };
 
 // a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
@@ -309,7 +315,7 @@ constexpr int GV_UNROLL = 8;
 template <int WT, bool ACT_Q8, int NW, bool AL4, bool SEG, int UNR = GV_UNROLL>
 __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
-    const int64_t nkb = a.K / 32;
+    const int nkb = (int) (a.K / 32);
     _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][K]
     const int NL = (int) (a.N < 16 ? a.N : 16);                              // tokens a work-group stages
     float *    xd  = (float *) (gv_smem + (size_t) NL * a.K * 2);            // [NL][K/32] (ACT_Q8)
@@ -320,14 +326,24 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
     const int j = lane >> 4, c = lane & 15;
     const int     batch = blockIdx.z;
-    const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
     // more than 16 tokens: blockIdx.y picks a chunk of 16; the chunks' work-groups stream the same weight
     // rows, which the first one pulls into L2
     const int     tok0 = 16 * (int) blockIdx.y;
-    const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) tok0 * a.nb11;
-    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
-    char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
-    int64_t       M = a.M;
+    // batch offsets: all zero for the common single-sequence call, which then skips the divisions and the 64-bit products
+    int           i12 = 0, i13 = 0;
+    uint64_t      w_off = 0, x_off = 0, d_off = 0, r_off = 0;
+    if (a.nbatch > 1) { // uniform
+        i12 = batch % a.ne12; i13 = batch / a.ne12;
+        w_off = (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+        x_off = (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
+        d_off = (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+        r_off = (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3;
+    }
+    if (tok0) { x_off += (uint64_t) tok0 * a.nb11; r_off += (uint64_t) tok0 * a.rnb1; } // uniform
+    const char *  xb  = a.x + x_off;
+    const char *  wb  = a.w + w_off;
+    char *        db  = a.dst + d_off;
+    int           M = (int) a.M;
     uint64_t      nb01 = a.nb01, nb1 = a.nb1;
     int           wl = blockIdx.x; // work-group index within its matrix
     bool          rope = false;
@@ -336,35 +352,38 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         if (a.nseg > 1 && wl >= a.seg[1].wg0) sg = 1;
         if (a.nseg > 2 && wl >= a.seg[2].wg0) sg = 2;
         const gv_seg & S = a.seg[sg];
-        wb = S.w; db = S.dst + (uint64_t) i12 * S.nb2 + (uint64_t) i13 * S.nb3;
-        M = S.M; nb01 = S.nb01; nb1 = S.nb1;
+        wb = S.w; db = S.dst;
+        if (a.nbatch > 1) db += (uint64_t) i12 * S.nb2 + (uint64_t) i13 * S.nb3;
+        M = (int) S.M; nb01 = S.nb01; nb1 = S.nb1;
         wl -= S.wg0;
         rope = S.rope != 0;
     }
-    // R = a.rows_wg of the 16 MFMA columns carry weight rows; fewer rows per work-group put a short
+    // R = a.rows_wg (16, 8 or 4) of the 16 MFMA columns carry weight rows; fewer rows per work-group put a short
     // matrix on more CUs (a CU sustains only so many outstanding lines, so 64 work-groups cannot
     // pull what 256 can).  Lanes c >= R load nothing; their columns are never stored.
     // With a second matrix (SwiGLU: dst = silu(W x) * (W2 x)) the MFMA columns are split: the first half of
     // them carries rows of W, the second half the same rows of W2, and the epilogue pairs them up.
     const bool    dual = a.w2 != nullptr;                 // uniform
-    const int     R  = a.rows_wg, Rr = dual ? R / 2 : R;   // MFMA columns in use, output rows per work-group
+    const int     R  = a.rows_wg, Rr = dual ? R / 2 : R;   // MFMA columns in use, output rows per work-group (powers of two)
     // the weight row of MFMA column cc.  Plain: consecutive rows.  With the rotation the R columns hold R/2
     // pairs (d, d + head_dim/2) of one head, first elements in columns 0 .. R/2-1, partners in the rest.
+    // Rows are counted in 32 bits (the host checks M < 2^31).
     const int     h2 = R >> 1, half_dim = a.head_dim >> 1;
-    auto column = [&](int cc, int64_t & row_, int & pair_, bool & ok_, const char *& wrow_) {
-        const int cr = dual ? cc % Rr : cc;
-        row_  = (int64_t) wl * Rr + cr;
+    auto column = [&](int cc, int & row_, int & pair_, bool & ok_, const char *& wrow_) {
+        const int cr = dual ? (cc & (Rr - 1)) : cc;
+        row_  = wl * Rr + cr;
         pair_ = 0; // index of the pair within its head: the rotation's frequency index
         if (SEG && rope) {
-            const int64_t f = (int64_t) wl * h2 + (cc & (h2 - 1));
-            pair_ = (int) (f % half_dim);
-            row_  = (f / half_dim) * a.head_dim + pair_ + (cc >= h2 ? half_dim : 0);
+            const unsigned f = (unsigned) (wl * h2 + (cc & (h2 - 1)));
+            const unsigned head = a.half_shift >= 0 ? f >> a.half_shift : f / (unsigned) half_dim;
+            pair_ = (int) (f - head * (unsigned) half_dim);
+            row_  = (int) head * a.head_dim + pair_ + (cc >= h2 ? half_dim : 0);
         }
         ok_ = cc < R && row_ < M;
-        const char * wsel = (dual && cc >= Rr) ? a.w2 + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03 : wb;
-        wrow_ = wsel + (uint64_t) min(row_, M - 1) * nb01;
+        const char * wsel = (dual && cc >= Rr) ? a.w2 + w_off : wb;
+        wrow_ = wsel + (uint64_t) (unsigned) min(row_, M - 1) * nb01;
     };
-    int64_t       row;
+    int           row;
     int           pair;
     bool          row_ok;
     const char *  wrow;
@@ -375,7 +394,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // per 16 lanes) and the dwords are handed to their MFMA lanes by a cross-lane permute once they have arrived;
     // the block scale rides in the first dword of chunk 0, so it needs no load of its own.
     constexpr bool PERM = WT == WT_Q8 && AL4;
-    int64_t       row_ld;
+    int           row_ld;
     int           pair_ld;
     bool          ld_ok = row_ok;
     const char *  wrow_ld = wrow;
@@ -383,20 +402,38 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     const int     j_ld = PERM ? (lane & 3) : j;
     const int     perm_src = (4 * c + j) * 4, perm_src0 = (4 * c) * 4; // byte addresses of the source lanes
     const int     N = min(16, (int) a.N - tok0); // tokens of this chunk
-    db += (uint64_t) tok0 * nb1;
+    if (tok0) db += (uint64_t) tok0 * nb1;
 
     // ---- this wave's weight blocks: kb = wid + NW * i
     constexpr bool al4 = AL4;
     q8_raw   wq[UNR];
     half8_t  wh[UNR];
     _Float16 wdv[UNR];
-    auto load_blocks = [&](int64_t i0) {
+    // Exact rounds (the usual shapes): block wid + NW * (i0 + u) of the lane's row sits at a compile-time distance from the
+    // round's first block, and an even wave count keeps the parity of a wave's blocks fixed -- one base address per lane and
+    // round, the loads take immediate offsets.  Otherwise block indices are clamped (a valid address, the result unused).
+    auto load_blocks = [&](int i0) {
+        if (!ld_ok) {
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) { wq[u] = q8_raw{0, 0, 0}; wdv[u] = (_Float16) 0.0f; wh[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+            return;
+        }
+        if constexpr (WT == WT_Q8 && PERM && NW % 2 == 0) {
+            if (a.exact) { // uniform
+                const char * p0 = wrow_ld + (wid + NW * i0) * VX_Q8_BLOCK + 8 * j_ld - ((wid & 1) ? 2 : 0);
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    uint32_t v[3];
+                    __builtin_memcpy(v, (const char *) __builtin_assume_aligned(p0 + u * NW * VX_Q8_BLOCK, 4), 12);
+                    wq[u] = q8_raw{v[0], v[1], v[2]};
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-            const int64_t kb = min((int64_t) wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, result unused
-            if (!ld_ok) {
-                wq[u] = q8_raw{0, 0, 0}; wdv[u] = (_Float16) 0.0f; wh[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            } else if constexpr (WT == WT_Q8) {
+            const int kb = min(wid + NW * (i0 + u), nkb - 1);
+            if constexpr (WT == WT_Q8) {
                 if constexpr (!PERM) wdv[u] = *(const _Float16 *) (wrow_ld + (uint64_t) kb * VX_Q8_BLOCK);
                 wq[u] = q8_load(wrow_ld, kb, j_ld, al4);
             } else {
@@ -408,8 +445,9 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // one) is requested before the weights: loads return in order, so its conversion then waits for
     // an L2 hit only, not for the weight stream behind it.
     const int upr = (int) (a.K / 8), units = N * upr;
+    auto unit_token = [&](int unit) { return (int) (((float) unit + 0.5f) * a.inv_upr); }; // = unit / upr
     auto fetch = [&](int unit, float4_t & v0, float4_t & v1) {
-        const int t = unit / upr, u = unit % upr;
+        const int t = unit_token(unit), u = unit - t * upr;
         const float * xp = (const float *) (xb + (uint64_t) t * a.nb11) + 8 * u;
         if (a.x_aligned) {
             v0 = ((const float4_t *) xp)[0]; v1 = ((const float4_t *) xp)[1];
@@ -419,7 +457,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
         }
     };
     auto stage = [&](int unit, const float4_t & v0, const float4_t & v1, const float4_t & g0, const float4_t & g1) {
-        const int t = unit / upr, u = unit % upr;
+        const int t = unit_token(unit), u = unit - t * upr;
         float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
@@ -452,7 +490,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0}, g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
     if (tid < units) fetch(tid, f0, f1);
     auto fetch_gain = [&](int unit, float4_t & a0, float4_t & a1) { // the norm weights of a unit's 8 columns (16-byte aligned)
-        const float4_t * gp = (const float4_t *) (a.norm_w + 8 * (unit % upr));
+        const float4_t * gp = (const float4_t *) (a.norm_w + 8 * (unit - unit_token(unit) * upr));
         a0 = gp[0]; a1 = gp[1];
     };
     if (a.norm_w && tid < units) fetch_gain(tid, g0, g1);
@@ -464,7 +502,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     // the residual values the storing wave will need, requested ahead of the weight stream as well
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.res && wid == 0 && row_ok && c < Rr) {
-        const char * rb = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) tok0 * a.rnb1 + (uint64_t) row * 4;
+        const char * rb = a.res + r_off + (uint64_t) row * 4;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
@@ -515,14 +553,13 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             for (int r = 0; r < 4; ++r) { const float2 v = rcs[r * 64 + lane]; rc[r] = v.x; rs[r] = v.y; }
         }
     }
-
     float4_t acc = {0, 0, 0, 0};
-    const int64_t per = (nkb + NW - 1) / NW; // blocks per wave
-    for (int64_t i0 = 0; i0 < per; i0 += UNR) {
+    const int per = (nkb + NW - 1) / NW; // blocks per wave
+    for (int i0 = 0; i0 < per; i0 += UNR) {
         if (i0) load_blocks(i0);
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-            const int64_t kb = (int64_t) wid + NW * (i0 + u);
+            const int kb = wid + NW * (i0 + u);
             if (kb >= nkb) break; // wave-uniform
             half8_t aop = {0, 0, 0, 0, 0, 0, 0, 0};
             if (c < N) aop = *(const half8_t *) (xs + (size_t) c * a.K + kb * 32 + 8 * j);
@@ -552,7 +589,6 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
             }
         }
     }
-
     if constexpr (NW > 1) {
         if (wid > 0) red[(wid - 1) * 64 + lane] = acc;
         __syncthreads();
@@ -647,7 +683,15 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
         if (a.nseg > 0) { rows = 0; for (int i = 0; i < a.nseg; ++i) rows += a.seg[i].M; }
         if (!gemv_shape_ok(a.N, rows, a.K)) return false;
     }
+    if (a.M >= ((int64_t) 1 << 31) || a.K >= ((int64_t) 1 << 31)) return false;
     a.rows_wg = 16;
+    a.nbatch  = nbatch;
+    a.inv_upr = 1.0f / (float) (a.K / 8);
+    {
+        const int half = a.head_dim / 2;
+        a.half_shift = -1;
+        if (half > 0 && (half & (half - 1)) == 0) { a.half_shift = 0; while ((1 << a.half_shift) < half) ++a.half_shift; }
+    }
     const int split = a.w2 ? 2 : 1; // with two matrices a work-group's MFMA columns hold half as many output rows
     auto groups = [&](int rows_wg) { // work-groups per batch entry
         if (a.nseg == 0) return (a.M * split + rows_wg - 1) / rows_wg;
@@ -695,6 +739,7 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     } while (0)
     // a wave with at most four blocks requests four: the loads past a wave's last block are clamped re-reads of it
     const bool few = (a.K / 32 + nw - 1) / nw <= 4;
+    a.exact = (a.K / 32) % ((int64_t) nw * (few ? 4 : GV_UNROLL)) == 0;
     switch (nw) {
         case 1:  VX_GEMV(1); break;
         case 2:  VX_GEMV(2); break;
