@@ -75,6 +75,11 @@ struct mm_args {
     float inv_upr;    // 1 / (K / 8): (unit + 0.5) * inv_upr truncates to unit / (K / 8) exactly for every unit of a chunk
     int   half_shift; // log2(head_dim / 2) when that is a power of two, else -1
     int   exact;      // every wave's blocks fill its load rounds exactly: no clamping of block indices
+    // gemv_dma_kernel: the weight rows of a work-group as an image in LDS
+    int   w_lds_off;  // byte offset of the image in the work-group's dynamic LDS (a multiple of 16)
+    int   w_slot;     // bytes between the images of consecutive MFMA columns: the row's bytes plus padding
+    int   w_ipr;      // direct-load instructions per row: 64 lanes x 16 bytes each
+    int   w_magic;    // (task * w_magic) >> 16 == task / w_ipr for every task of a work-group
 };
 
 // a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
@@ -627,6 +632,284 @@ __global__ __launch_bounds__(64 * NW) void gemv_kernel(const mm_args a) {
     }
 }
 
+// ---- GEMV shape, weights through LDS --------------------------------------------------------------------
+// The same product as gemv_kernel -- same work-groups, same k blocks per wave, same order of every sum -- for the common
+// case (Q8_0 rows and F32 activation rows on 16-byte boundaries, one batch entry, eight or sixteen waves), organised around
+// two facts measured on this chip: a wave issues one instruction every four cycles or so, whatever the instruction, and a
+// wave's loads return in order.  So
+//   * the weight rows do not pass through registers: the first half of the waves copies them into LDS with direct loads
+//     (64 lanes x 16 consecutive bytes of one row per instruction -- whole cache lines instead of 12-byte pieces of sixteen
+//     rows), starts doing so a few dozen instructions after the kernel begins, and then only waits for them;
+//   * the other half does everything on the activations' side (fetch, the fused norm, staging as f16 or Q8, the rotation's
+//     angles): with no weight loads of their own in flight, they see their data after an L2 hit;
+//   * after the barrier every wave takes its k blocks' bytes from the LDS image (each column's image padded so that the
+//     sixteen columns fall into different banks), all reads of a round issued before the first is used.
+// What is fused is a template parameter here, so that a wave executes no instruction of a path it does not take.
+__device__ __forceinline__ void gv_dma16(const char * g, uint32_t lds_base) {
+    // 16 bytes per lane from global memory straight into LDS: lane l's land at lds_base + 16 l (lds_base uniform).  M0 carries
+    // the LDS address; the compiler keeps nothing in M0 across statements (it sets it right before each instruction that reads it).
+    const uint32_t base = (uint32_t) __builtin_amdgcn_readfirstlane((int) lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory");
+}
+
+enum gv_epilogue : int { GV_PLAIN = 0, GV_RES = 1, GV_SWIGLU = 2 };
+
+template <bool ACT_Q8, int NW, bool SEG, bool NORM, int EPI>
+__global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
+    static_assert(NW == 8 || NW == 16, "eight or sixteen waves");
+    constexpr int  NWD = NW / 2, NA = NW - NWD; // waves 0 .. NWD-1 fetch the weights, the rest handle the activations
+    constexpr bool dual = EPI == GV_SWIGLU;
+    extern __shared__ __attribute__((aligned(16))) char gv_smem[];
+    const int K = (int) a.K, nkb = K >> 5;
+    const int KP = K + 8; // halfs between staged tokens; the padding spreads the tokens over the banks
+    const int tok0 = 16 * (int) blockIdx.y;
+    const int N  = min(16, (int) a.N - tok0); // tokens of this chunk
+    const int NL = (int) (a.N < 16 ? a.N : 16);
+    _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][KP]
+    float *    xd  = (float *) (gv_smem + (size_t) NL * KP * 2);             // [NL][K/32] (ACT_Q8)
+    float4_t * red = (float4_t *) (gv_smem + (size_t) NL * KP * 2 + (ACT_Q8 ? (size_t) NL * nkb * 4 : 0));
+    float *    nsc = (float *) (red + (NW - 1) * 64);                        // [16] per-token 1 / rms (fused RMS_NORM)
+    float2 *   rcs = (float2 *) (nsc + 16);                                  // [4][64] cos / sin of four token slots (SEG)
+    const char * w_lds = gv_smem + a.w_lds_off;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane >> 4, c = lane & 15;
+
+    // ---- which matrix, which rows
+    int          wl = blockIdx.x; // work-group index within its matrix
+    int          M = (int) a.M;
+    const char * wb = a.w;
+    char *       db = a.dst;
+    uint64_t     nb01 = a.nb01, nb1 = a.nb1;
+    bool         rope = false;
+    if constexpr (SEG) {
+        int sg = 0;
+        if (a.nseg > 1 && wl >= a.seg[1].wg0) sg = 1;
+        if (a.nseg > 2 && wl >= a.seg[2].wg0) sg = 2;
+        const gv_seg & S = a.seg[sg];
+        wb = S.w; db = S.dst; M = (int) S.M; nb01 = S.nb01; nb1 = S.nb1;
+        wl -= S.wg0;
+        rope = S.rope != 0;
+    }
+    const int R = a.rows_wg, Rr = dual ? R / 2 : R; // MFMA columns in use, output rows per work-group (powers of two)
+    const int h2 = R >> 1, half_dim = a.head_dim >> 1;
+    // the weight row of MFMA column cc, as gemv_kernel has it
+    auto column = [&](int cc, int & row_, int & pair_, bool & ok_, const char *& wrow_) {
+        const int cr = dual ? (cc & (Rr - 1)) : cc;
+        row_  = wl * Rr + cr;
+        pair_ = 0;
+        if (SEG && rope) {
+            const unsigned f = (unsigned) (wl * h2 + (cc & (h2 - 1)));
+            const unsigned head = a.half_shift >= 0 ? f >> a.half_shift : f / (unsigned) half_dim;
+            pair_ = (int) (f - head * (unsigned) half_dim);
+            row_  = (int) head * a.head_dim + pair_ + (cc >= h2 ? half_dim : 0);
+        }
+        ok_ = cc < R && row_ < M;
+        const char * wsel = (dual && cc >= Rr) ? a.w2 : wb;
+        wrow_ = wsel + (uint64_t) (unsigned) min(row_, M - 1) * nb01;
+    };
+
+    const int upr = K >> 3, units = N * upr; // a unit: 8 consecutive k of one token
+    auto unit_token = [&](int unit) { return (int) (((float) unit + 0.5f) * a.inv_upr); }; // = unit / upr
+    const char * xb = a.x + (uint64_t) tok0 * a.nb11;
+    float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    if (wid < NWD) {
+        // ---- weight rows -> LDS; task = (column, 1 KiB piece of its row), all of it uniform
+        const uint32_t lds0 = (uint32_t) (uintptr_t) (__attribute__((address_space(3))) char *) gv_smem + (uint32_t) a.w_lds_off;
+        const int units_row = (nkb * VX_Q8_BLOCK) >> 4;
+        for (int task = wid; task < R * a.w_ipr; task += NWD) {
+            const int cc = (task * a.w_magic) >> 16, piece = task - cc * a.w_ipr;
+            int          row_t, pair_t;
+            bool         ok_t;
+            const char * wrow_t;
+            column(cc, row_t, pair_t, ok_t, wrow_t);
+            const int u = piece * 64 + lane;
+            if (ok_t && u < units_row) gv_dma16(wrow_t + (size_t) u * 16, lds0 + (uint32_t) (cc * a.w_slot + piece * 1024));
+        }
+        if constexpr (EPI == GV_RES) { // the residual values the storing wave will need: in flight with the weights
+            int          row_c, pair_c;
+            bool         ok_c;
+            const char * wrow_c;
+            column(c, row_c, pair_c, ok_c, wrow_c);
+            if (wid == 0 && ok_c) {
+                const char * rb = a.res + (uint64_t) tok0 * a.rnb1 + (uint64_t) row_c * 4;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
+            }
+        }
+        if constexpr (NORM) __syncthreads(); // the activation waves' barrier after the norm scales (the direct loads are not
+                                             // known to the compiler: no wait for them here)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's direct loads have landed
+    } else {
+        // ---- activations -> LDS as f16 (or quantised), [token][k]
+        const int awid = wid - NWD, atid = tid - 64 * NWD;
+        auto fetch = [&](int unit, float4_t & v0, float4_t & v1, float4_t & g0, float4_t & g1) {
+            const int t = unit_token(unit), u = unit - t * upr;
+            const float4_t * xp = (const float4_t *) ((const float *) (xb + (uint64_t) t * a.nb11) + 8 * u);
+            v0 = xp[0]; v1 = xp[1];
+            if constexpr (NORM) { const float4_t * gp = (const float4_t *) (a.norm_w + 8 * u); g0 = gp[0]; g1 = gp[1]; }
+        };
+        auto stage = [&](int unit, const float4_t & v0, const float4_t & v1, const float4_t & g0, const float4_t & g1) {
+            const int t = unit_token(unit), u = unit - t * upr;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
+            if constexpr (NORM) { // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
+                const float sc = nsc[t];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    v[i]     *= sc; v[i]     *= g0[i];
+                    v[4 + i] *= sc; v[4 + i] *= g1[i];
+                }
+            }
+            half8_t h;
+            if constexpr (ACT_Q8) { // 4 consecutive units = one 32-wide block
+                float amax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                const float d  = amax / 127.f;
+                const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
+                if ((u & 3) == 0) xd[t * nkb + (u >> 2)] = (float) (_Float16) d;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
+            }
+            *(half8_t *) (xs + (size_t) t * KP + 8 * u) = h;
+        };
+        float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0}, g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
+        if (atid < units) fetch(atid, f0, f1, g0, g1);
+        vx_rms_row nrow, nrow2; // the tokens this wave normalises first, requested up front
+        if constexpr (NORM) {
+            if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
+            if (awid + NA < N) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (awid + NA) * a.nb11), a.K, lane);
+        }
+        if constexpr (SEG) { // the rotation's cos / sin: wave r of the first four takes token slot r of every lane
+            if (rope && awid < 4) {
+                int  row_c, pair_c;
+                bool ok_c;
+                const char * wrow_c;
+                column(c, row_c, pair_c, ok_c, wrow_c);
+                float cv = 1.0f, sv = 0.0f;
+                if (ok_c && 4 * j + awid < N) {
+                    const int n = tok0 + 4 * j + awid;
+                    rope_cos_sin(a.rp, (float) a.pos[n % a.rope_T], pair_c, a.ff ? a.ff[pair_c] : 1.0f, cv, sv);
+                }
+                rcs[awid * 64 + lane] = float2{cv, sv};
+            }
+        }
+        if constexpr (NORM) { // one wave per token, as the RMS_NORM kernel has it; a wave with several tokens takes two at a time
+            for (int t = awid; t < N; t += 2 * NA) {
+                if (t != awid) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
+                if (t + NA < N) {
+                    if (t != awid) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (t + NA) * a.nb11), a.K, lane);
+                    float s1, s2;
+                    vx_rms_row_scale2(nrow, nrow2, a.K, lane, a.norm_eps, s1, s2);
+                    if (lane == 0) { nsc[t] = s1; nsc[t + NA] = s2; }
+                } else {
+                    const float sc = vx_rms_row_scale(nrow, a.K, lane, a.norm_eps);
+                    if (lane == 0) nsc[t] = sc;
+                }
+            }
+            __syncthreads();
+        }
+        if (atid < units) stage(atid, f0, f1, g0, g1);
+        for (int unit = atid + 64 * NA; unit < units; unit += 64 * NA) {
+            fetch(unit, f0, f1, g0, g1);
+            stage(unit, f0, f1, g0, g1);
+        }
+    }
+    __syncthreads();
+
+    // ---- this wave's k blocks: kb = wid + NW * i, the LDS reads of four blocks issued together
+    float4_t acc = {0, 0, 0, 0};
+    {
+        const char *     wcol = w_lds + min(c, R - 1) * a.w_slot; // lanes past the last column read a valid image; never stored
+        const _Float16 * xrow = xs + (size_t) min(c, N - 1) * KP + 8 * j; // rows past the last token likewise
+        const int per = (nkb + NW - 1) / NW;
+        constexpr int PB = 4;
+        for (int i0 = 0; i0 < per; i0 += PB) {
+            q8_raw   raw[PB];
+            _Float16 dwh[PB];
+            half8_t  aop[PB];
+#pragma unroll
+            for (int u = 0; u < PB; ++u) {
+                const int kb = min(wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, the result unused
+                const char *     blk_p = wcol + kb * VX_Q8_BLOCK;
+                const uint32_t * q     = (const uint32_t *) (blk_p + 8 * j - ((kb & 1) ? 2 : 0)); // dword-aligned, as q8_load has it
+                raw[u] = q8_raw{ q[0], q[1], q[2] };
+                dwh[u] = *(const _Float16 *) blk_p;
+                aop[u] = *(const half8_t *) (xrow + kb * 32);
+            }
+#pragma unroll
+            for (int u = 0; u < PB; ++u) {
+                const int kb = wid + NW * (i0 + u);
+                if (kb >= nkb) break; // wave-uniform
+                const float    dw  = (float) dwh[u];
+                const half8_t  bop = q8_unpack(raw[u], kb, true);
+                const float4_t blk = mfma16(aop[u], bop, float4_t{0, 0, 0, 0});
+                if constexpr (ACT_Q8) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[r] += blk[r] * (dw * (4 * j + r < N ? xd[(4 * j + r) * nkb + kb] : 0.0f));
+                } else {
+                    acc += blk * dw;
+                }
+            }
+        }
+    }
+
+    // ---- the waves' partial sums, added in wave order by wave 0, which also finishes and stores
+    int          row, pair;
+    bool         row_ok;
+    const char * wrow;
+    column(c, row, pair, row_ok, wrow);
+    if (wid > 0) red[(wid - 1) * 64 + lane] = acc;
+    __syncthreads();
+    if (wid > 0) return;
+#pragma unroll
+    for (int ww = 0; ww < NW - 1; ++ww) acc += red[ww * 64 + lane];
+    // lane (j,c), register r: token 4j + r, row of column c
+    if constexpr (dual) { // lane c < Rr holds W's row, lane c + Rr the same row of W2: dst = silu(gate) * up
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float up = __shfl(acc[r], lane + Rr, 64);
+            acc[r] = (acc[r] / (1.0f + expf(-acc[r]))) * up;
+        }
+    }
+    if constexpr (EPI == GV_RES) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = scaled_residual(acc[r], a.res_scale, resv[r]);
+    }
+    if constexpr (SEG) {
+        if (rope) { // column c < R/2 holds x0 of its pair, column c + R/2 the partner x1
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float2 cs = rcs[r * 64 + lane];
+                const float other = __shfl_xor(acc[r], h2, 64);
+                const bool  first = c < h2;
+                float y0, y1;
+                rope_rotate(first ? acc[r] : other, first ? other : acc[r], cs.x, cs.y, y0, y1);
+                acc[r] = first ? y0 : y1;
+            }
+        }
+    }
+    if (row_ok && c < Rr) {
+        char * out = db + (uint64_t) tok0 * nb1 + (uint64_t) row * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int tok = 4 * j + r;
+            if (tok < N) *(float *) (out + (uint64_t) tok * nb1) = acc[r];
+        }
+    }
+}
+
+
 constexpr size_t GV_MAX_LDS  = 160 * 1024;    // what a gfx950 CU has
 constexpr size_t GV_ROPE_LDS = 4 * 64 * 8;     // cos / sin of four token slots per lane, exchanged between waves
 
@@ -641,10 +924,77 @@ bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
     return nl * K * 2 + nl * (K / 32) * 4 + 15 * 64 * 16 + 16 * sizeof(float) + GV_ROPE_LDS <= GV_MAX_LDS;
 }
 
-size_t gemv_smem(const mm_args & a, bool act_q8, int nw) {
+size_t gemv_smem(const mm_args & a, bool act_q8, int nw, bool dma = false) {
     const size_t nl = (size_t) (a.N < 16 ? a.N : 16);
-    return nl * a.K * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
+    return nl * (a.K + (dma ? 8 : 0)) * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
            (a.nseg > 0 ? GV_ROPE_LDS : 0);
+}
+
+// gemv_dma_kernel's weight image: bytes between consecutive columns.  The padding is chosen so that the dword reads of the
+// sixteen columns (lane (j, c): dword c * slot / 4 + 2 j + const) spread over the 64 banks as evenly as they can.
+int gemv_dma_slot(int64_t K) {
+    const int row_bytes = (int) (K / 32) * VX_Q8_BLOCK;
+    int best_pad = 16, best = 1 << 30;
+    for (int pad = 16; pad <= 256; pad += 16) {
+        const int sd = (row_bytes + pad) / 4;
+        int worst = 0;
+        for (int half = 0; half < 2; ++half) { // 32 lanes at a time
+            int count[64] = {0};
+            for (int l = 32 * half; l < 32 * half + 32; ++l) {
+                const int n = ++count[((l & 15) * sd + 2 * (l >> 4)) & 63];
+                worst = n > worst ? n : worst;
+            }
+        }
+        if (worst < best) { best = worst; best_pad = pad; }
+    }
+    return row_bytes + best_pad;
+}
+
+// Launches gemv_dma_kernel if the call is one it takes (a: as launch_gemv has prepared it, rows_wg and the prologue
+// helpers included; nw: the wave count every kernel uses for this shape).
+template <bool ACT_Q8>
+bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st) {
+    static const bool on = [] { const char * e = getenv("VX_GEMV_DMA"); return !e || atoi(e) != 0; }();
+    if (!on || nbatch != 1 || (nw != 8 && nw != 16) || !a.x_aligned || !a.w_aligned || a.K % 256) return false;
+    if (a.norm_w && a.K > 2048) return false;
+    if (a.w2 && a.res) return false;
+    if (a.nseg > 0 && (a.w2 || a.res)) return false;
+    auto al16 = [](const void * p_, uint64_t stride) { return (uintptr_t) p_ % 16 == 0 && stride % 16 == 0; };
+    if (a.nseg == 0 && (!al16(a.w, a.nb01) || (a.w2 && !al16(a.w2, 0)))) return false;
+    for (int i = 0; i < a.nseg; ++i) if (!al16(a.seg[i].w, a.seg[i].nb01)) return false;
+    a.w_slot    = gemv_dma_slot(a.K);
+    a.w_lds_off = (int) ((gemv_smem(a, ACT_Q8, nw, true) + 15) / 16 * 16);
+    a.w_ipr     = (int) ((a.K / 32 * VX_Q8_BLOCK / 16 + 63) / 64);
+    a.w_magic   = (65536 + a.w_ipr - 1) / a.w_ipr;
+    for (int t = 0; t < 16 * a.w_ipr; ++t) if (((t * a.w_magic) >> 16) != t / a.w_ipr) return false;
+    const size_t smem = (size_t) a.w_lds_off + (size_t) a.rows_wg * a.w_slot;
+    if (smem > GV_MAX_LDS) return false;
+    const dim3 block((unsigned) (64 * nw));
+#define VX_DMA_GO(NW_, SEG_, NORM_, EPI_)                                                                              \
+    do {                                                                                                               \
+        auto kern = gemv_dma_kernel<ACT_Q8, NW_, SEG_, NORM_, EPI_>;                                                   \
+        if (smem > 64 * 1024) { /* above 64 KiB of LDS a kernel has to be told once that it may be given that much */  \
+            static bool raised = false;                                                                                \
+            if (!raised) {                                                                                             \
+                if (hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize,               \
+                                        (int) GV_MAX_LDS) != hipSuccess) { (void) hipGetLastError(); return false; }   \
+                raised = true;                                                                                         \
+            }                                                                                                          \
+        }                                                                                                              \
+        kern<<<grid, block, smem, st>>>(a);                                                                            \
+        return true;                                                                                                   \
+    } while (0)
+#define VX_DMA_NW(SEG_, NORM_, EPI_)                                                                                   \
+    do { if (nw == 8) VX_DMA_GO(8, SEG_, NORM_, EPI_); else VX_DMA_GO(16, SEG_, NORM_, EPI_); } while (0)
+    const bool norm = a.norm_w != nullptr;
+    if (a.nseg > 0) { if (norm) VX_DMA_NW(true, true, GV_PLAIN); else VX_DMA_NW(true, false, GV_PLAIN); }
+    if (a.w2)       { if (norm) VX_DMA_NW(false, true, GV_SWIGLU); else VX_DMA_NW(false, false, GV_SWIGLU); }
+    if (a.res)      { if (norm) return false; VX_DMA_NW(false, false, GV_RES); }
+    if (norm) VX_DMA_NW(false, true, GV_PLAIN);
+    VX_DMA_NW(false, false, GV_PLAIN);
+#undef VX_DMA_NW
+#undef VX_DMA_GO
+    return false;
 }
 
 // waves per work-group for a matrix of M rows: about 4 blocks per wave for one chunk of tokens (K = 1024: 8 waves; measured
@@ -712,6 +1062,7 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     }
     const dim3 grid((unsigned) nwg, (unsigned) nchunk, (unsigned) nbatch);
     const dim3 block((unsigned) (64 * nw));
+    if constexpr (WT == WT_Q8) { if (launch_gemv_dma<ACT_Q8>(a, nbatch, nw, grid, st)) return true; }
     // above 64 KiB of LDS a kernel has to be told once that it may be given that much
 #define VX_GEMV_GO(...)                                                                                                \
     do {                                                                                                               \
