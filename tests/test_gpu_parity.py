@@ -426,6 +426,29 @@ def test_mul_mat_q8_0(gpu, M, K, N):
     assert nmse(f64, got_fl) <= 1e-5
 
 
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 1), (1024, 1024, 2), (1000, 1024, 14), (1536, 1024, 16), (1024, 4096, 2), (1024, 4096, 14),
+                                   (8192, 1024, 2), (200, 2048, 3), (64, 512, 2), (1024, 768, 5), (24, 1024, 2), (1024, 1024, 17),
+                                   (1024, 1024, 40), (4096, 4096, 16)])
+def test_gemv_weights_through_lds_equals_the_register_path(gpu, M, K, N, monkeypatch):
+    """Products of up to 16 tokens per chunk take the kernel that brings the weight rows into LDS by direct loads when rows
+    and activations sit on 16-byte boundaries (K a multiple of 256); VX_GEMV_DMA=0 keeps them on the kernel that loads
+    the weights into registers.  Both walk the same k blocks per wave and add in the same order: bit-equal, in both
+    activation modes; shapes: ragged rows, 4 / 8 / 16 rows per work-group, four, eight and sixteen waves, K with and
+    without whole four-block rounds, several chunks of tokens."""
+    say(f"gemv through LDS vs registers M={M} K={K} N={N}")
+    w, x = mm_inputs(("dma", M, K, N), M, K, N)
+    wq, xd = dev(reflib.quantize_q8_0(w)), dev(x)
+    for mode in (gpu.ACT_FLOAT, gpu.ACT_Q8):
+        monkeypatch.delenv("VX_GEMV_DMA", raising=False)
+        a = sync_np(gpu.mul_mat(wq, xd, mode, w_ne0=K))
+        monkeypatch.setenv("VX_GEMV_DMA", "0")
+        b = sync_np(gpu.mul_mat(wq, xd, mode, w_ne0=K))
+        assert np.array_equal(a, b), (mode, np.abs(a - b).max())
+    monkeypatch.delenv("VX_GEMV_DMA", raising=False)
+    cpu = reflib.oracle_mul_mat(reflib.quantize_q8_0(w), x, K, act_mode=0)
+    assert np.abs(sync_np(gpu.mul_mat(wq, xd, gpu.ACT_Q8, w_ne0=K)) - cpu).max() / np.abs(cpu).max() <= 1e-5
+
+
 @pytest.mark.parametrize("wtype", [np.float16, np.float32])
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 2), (1024, 64, 14), (333, 256, 40), (64, 1024, 300), (2048, 256, 1600),
                                    (1000, 256, 3000), (200, 192, 700)])

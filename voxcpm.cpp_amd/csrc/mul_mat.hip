@@ -78,8 +78,6 @@ struct mm_args {
     // gemv_dma_kernel: the weight rows of a work-group as an image in LDS
     int   w_lds_off;  // byte offset of the image in the work-group's dynamic LDS (a multiple of 16)
     int   w_slot;     // bytes between the images of consecutive MFMA columns: the row's bytes plus padding
-    int   w_ipr;      // direct-load instructions per row: 64 lanes x 16 bytes each
-    int   w_magic;    // (task * w_magic) >> 16 == task / w_ipr for every task of a work-group
 };
 
 // a + x * s with the product rounded before the sum, as a SCALE node followed by an ADD node rounds
@@ -654,9 +652,49 @@ __device__ __forceinline__ void gv_dma16(const char * g, uint32_t lds_base) {
 
 enum gv_epilogue : int { GV_PLAIN = 0, GV_RES = 1, GV_SWIGLU = 2 };
 
+// Four k blocks of one wave from the LDS images: blocks kb, kb + NW, kb + 2 NW, kb + 3 NW sit at compile-time distances, and
+// with an even wave count they share their parity, so a round is straight-line code over three addresses: all reads first,
+// then the four products, then the four scaled additions (in block order, as everywhere).
+//   sp: this lane's column image at block kb (where the block's scale sits); xp: this lane's token at k = 32 kb + 8 j;
+//   xdp (ACT_Q8): the activations' block scales of block kb, [block][16 tokens], at token 4 j
+template <bool ACT_Q8, int NW, bool ODD>
+__device__ __forceinline__ void gv_round4(const char * sp, int j, const _Float16 * xp, const float * xdp, float4_t & acc) {
+    q8_raw   raw[4];
+    _Float16 dwh[4];
+    half8_t  aop[4];
+    float4_t xdv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const char * bp = sp + u * NW * VX_Q8_BLOCK;
+        if constexpr (ODD) { // the block starts 2 bytes past a dword: its quants are dword-aligned
+            const uint32_t * q = (const uint32_t *) (bp + 2 + 8 * j);
+            raw[u] = q8_raw{ 0, q[0], q[1] };
+        } else {             // the block starts on a dword: the quants sit 2 bytes in
+            const uint32_t * q = (const uint32_t *) (bp + 8 * j);
+            raw[u] = q8_raw{ q[0], q[1], q[2] };
+        }
+        dwh[u] = *(const _Float16 *) bp;
+        aop[u] = *(const half8_t *) (xp + u * NW * 32);
+        if constexpr (ACT_Q8) xdv[u] = *(const float4_t *) (xdp + u * NW * 16);
+    }
+    float4_t blk[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) blk[u] = mfma16(aop[u], q8_unpack(raw[u], ODD ? 1 : 0, true), float4_t{0, 0, 0, 0});
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const float dw = (float) dwh[u];
+        if constexpr (ACT_Q8) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] += blk[u][r] * (dw * xdv[u][r]);
+        } else {
+            acc += blk[u] * dw;
+        }
+    }
+}
+
 template <bool ACT_Q8, int NW, bool SEG, bool NORM, int EPI>
 __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
-    static_assert(NW == 8 || NW == 16, "eight or sixteen waves");
+    static_assert(NW == 4 || NW == 8 || NW == 16, "four, eight or sixteen waves");
     constexpr int  NWD = NW / 2, NA = NW - NWD; // waves 0 .. NWD-1 fetch the weights, the rest handle the activations
     constexpr bool dual = EPI == GV_SWIGLU;
     extern __shared__ __attribute__((aligned(16))) char gv_smem[];
@@ -666,8 +704,8 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     const int N  = min(16, (int) a.N - tok0); // tokens of this chunk
     const int NL = (int) (a.N < 16 ? a.N : 16);
     _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][KP]
-    float *    xd  = (float *) (gv_smem + (size_t) NL * KP * 2);             // [NL][K/32] (ACT_Q8)
-    float4_t * red = (float4_t *) (gv_smem + (size_t) NL * KP * 2 + (ACT_Q8 ? (size_t) NL * nkb * 4 : 0));
+    float *    xd  = (float *) (gv_smem + (size_t) NL * KP * 2);             // [K/32][16 tokens] (ACT_Q8): the activations' block scales
+    float4_t * red = (float4_t *) (gv_smem + (size_t) NL * KP * 2 + (ACT_Q8 ? (size_t) 16 * nkb * 4 : 0));
     float *    nsc = (float *) (red + (NW - 1) * 64);                        // [16] per-token 1 / rms (fused RMS_NORM)
     float2 *   rcs = (float2 *) (nsc + 16);                                  // [4][64] cos / sin of four token slots (SEG)
     const char * w_lds = gv_smem + a.w_lds_off;
@@ -716,18 +754,21 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 
     if (wid < NWD) {
-        // ---- weight rows -> LDS; task = (column, 1 KiB piece of its row), all of it uniform
+        // ---- weight rows -> LDS.  These waves share their SIMDs with the activation waves: until the requests are out they go first
+        __builtin_amdgcn_s_setprio(3);
         const uint32_t lds0 = (uint32_t) (uintptr_t) (__attribute__((address_space(3))) char *) gv_smem + (uint32_t) a.w_lds_off;
         const int units_row = (nkb * VX_Q8_BLOCK) >> 4;
-        for (int task = wid; task < R * a.w_ipr; task += NWD) {
-            const int cc = (task * a.w_magic) >> 16, piece = task - cc * a.w_ipr;
+        for (int cc = wid; cc < R; cc += NWD) { // a wave takes whole columns: one row address, then 1 KiB pieces of it
             int          row_t, pair_t;
             bool         ok_t;
             const char * wrow_t;
             column(cc, row_t, pair_t, ok_t, wrow_t);
-            const int u = piece * 64 + lane;
-            if (ok_t && u < units_row) gv_dma16(wrow_t + (size_t) u * 16, lds0 + (uint32_t) (cc * a.w_slot + piece * 1024));
+            if (!ok_t) continue;
+            const char * g   = wrow_t + (size_t) lane * 16;
+            uint32_t     dst = lds0 + (uint32_t) (cc * a.w_slot);
+            for (int u = lane; u < units_row; u += 64, g += 1024, dst += 1024) gv_dma16(g, dst);
         }
+        __builtin_amdgcn_s_setprio(0);
         if constexpr (EPI == GV_RES) { // the residual values the storing wave will need: in flight with the weights
             int          row_c, pair_c;
             bool         ok_c;
@@ -776,7 +817,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
                 const float id = amax != 0.0f ? 127.f / amax : 0.0f;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
-                if ((u & 3) == 0) xd[t * nkb + (u >> 2)] = (float) (_Float16) d;
+                if ((u & 3) == 0) xd[(u >> 2) * 16 + t] = (float) (_Float16) d;
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
@@ -790,18 +831,18 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
             if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
             if (awid + NA < N) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (awid + NA) * a.nb11), a.K, lane);
         }
-        if constexpr (SEG) { // the rotation's cos / sin: wave r of the first four takes token slot r of every lane
+        if constexpr (SEG) { // the rotation's cos / sin: the waves share the four token slots of every lane
             if (rope && awid < 4) {
                 int  row_c, pair_c;
                 bool ok_c;
                 const char * wrow_c;
                 column(c, row_c, pair_c, ok_c, wrow_c);
-                float cv = 1.0f, sv = 0.0f;
-                if (ok_c && 4 * j + awid < N) {
-                    const int n = tok0 + 4 * j + awid;
-                    rope_cos_sin(a.rp, (float) a.pos[n % a.rope_T], pair_c, a.ff ? a.ff[pair_c] : 1.0f, cv, sv);
+                const float ffv = a.ff ? a.ff[pair_c] : 1.0f;
+                for (int slot = awid; slot < 4; slot += NA) {
+                    float cv = 1.0f, sv = 0.0f;
+                    if (ok_c && 4 * j + slot < N) rope_cos_sin(a.rp, (float) a.pos[(tok0 + 4 * j + slot) % a.rope_T], pair_c, ffv, cv, sv);
+                    rcs[slot * 64 + lane] = float2{cv, sv};
                 }
-                rcs[awid * 64 + lane] = float2{cv, sv};
             }
         }
         if constexpr (NORM) { // one wave per token, as the RMS_NORM kernel has it; a wave with several tokens takes two at a time
@@ -833,32 +874,45 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
         const char *     wcol = w_lds + min(c, R - 1) * a.w_slot; // lanes past the last column read a valid image; never stored
         const _Float16 * xrow = xs + (size_t) min(c, N - 1) * KP + 8 * j; // rows past the last token likewise
         const int per = (nkb + NW - 1) / NW;
-        constexpr int PB = 4;
-        for (int i0 = 0; i0 < per; i0 += PB) {
-            q8_raw   raw[PB];
-            _Float16 dwh[PB];
-            half8_t  aop[PB];
-#pragma unroll
-            for (int u = 0; u < PB; ++u) {
-                const int kb = min(wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, the result unused
-                const char *     blk_p = wcol + kb * VX_Q8_BLOCK;
-                const uint32_t * q     = (const uint32_t *) (blk_p + 8 * j - ((kb & 1) ? 2 : 0)); // dword-aligned, as q8_load has it
-                raw[u] = q8_raw{ q[0], q[1], q[2] };
-                dwh[u] = *(const _Float16 *) blk_p;
-                aop[u] = *(const half8_t *) (xrow + kb * 32);
+        if (a.exact) { // uniform: every wave has a whole number of four-block rounds
+            const char *     sp  = wcol + wid * VX_Q8_BLOCK;
+            const _Float16 * xp  = xrow + wid * 32;
+            const float *    xdp = xd + wid * 16 + 4 * j;
+            if (wid & 1) {
+                for (int i0 = 0; i0 < per; i0 += 4, sp += 4 * NW * VX_Q8_BLOCK, xp += 4 * NW * 32, xdp += 4 * NW * 16)
+                    gv_round4<ACT_Q8, NW, true>(sp, j, xp, xdp, acc);
+            } else {
+                for (int i0 = 0; i0 < per; i0 += 4, sp += 4 * NW * VX_Q8_BLOCK, xp += 4 * NW * 32, xdp += 4 * NW * 16)
+                    gv_round4<ACT_Q8, NW, false>(sp, j, xp, xdp, acc);
             }
+        } else {
+            constexpr int PB = 4;
+            for (int i0 = 0; i0 < per; i0 += PB) {
+                q8_raw   raw[PB];
+                _Float16 dwh[PB];
+                half8_t  aop[PB];
 #pragma unroll
-            for (int u = 0; u < PB; ++u) {
-                const int kb = wid + NW * (i0 + u);
-                if (kb >= nkb) break; // wave-uniform
-                const float    dw  = (float) dwh[u];
-                const half8_t  bop = q8_unpack(raw[u], kb, true);
-                const float4_t blk = mfma16(aop[u], bop, float4_t{0, 0, 0, 0});
-                if constexpr (ACT_Q8) {
+                for (int u = 0; u < PB; ++u) {
+                    const int kb = min(wid + NW * (i0 + u), nkb - 1); // clamped: a valid address, the result unused
+                    const char *     blk_p = wcol + kb * VX_Q8_BLOCK;
+                    const uint32_t * q     = (const uint32_t *) (blk_p + 8 * j - ((kb & 1) ? 2 : 0)); // dword-aligned, as q8_load has it
+                    raw[u] = q8_raw{ q[0], q[1], q[2] };
+                    dwh[u] = *(const _Float16 *) blk_p;
+                    aop[u] = *(const half8_t *) (xrow + kb * 32);
+                }
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[r] += blk[r] * (dw * (4 * j + r < N ? xd[(4 * j + r) * nkb + kb] : 0.0f));
-                } else {
-                    acc += blk * dw;
+                for (int u = 0; u < PB; ++u) {
+                    const int kb = wid + NW * (i0 + u);
+                    if (kb >= nkb) break; // wave-uniform
+                    const float    dw  = (float) dwh[u];
+                    const half8_t  bop = q8_unpack(raw[u], kb, true);
+                    const float4_t blk = mfma16(aop[u], bop, float4_t{0, 0, 0, 0});
+                    if constexpr (ACT_Q8) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[r] += blk[r] * (dw * (4 * j + r < N ? xd[kb * 16 + 4 * j + r] : 0.0f));
+                    } else {
+                        acc += blk * dw;
+                    }
                 }
             }
         }
@@ -926,7 +980,7 @@ bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
 
 size_t gemv_smem(const mm_args & a, bool act_q8, int nw, bool dma = false) {
     const size_t nl = (size_t) (a.N < 16 ? a.N : 16);
-    return nl * (a.K + (dma ? 8 : 0)) * 2 + (act_q8 ? nl * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
+    return nl * (a.K + (dma ? 8 : 0)) * 2 + (act_q8 ? (dma ? 16 : nl) * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
            (a.nseg > 0 ? GV_ROPE_LDS : 0);
 }
 
@@ -954,8 +1008,8 @@ int gemv_dma_slot(int64_t K) {
 // helpers included; nw: the wave count every kernel uses for this shape).
 template <bool ACT_Q8>
 bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st) {
-    static const bool on = [] { const char * e = getenv("VX_GEMV_DMA"); return !e || atoi(e) != 0; }();
-    if (!on || nbatch != 1 || (nw != 8 && nw != 16) || !a.x_aligned || !a.w_aligned || a.K % 256) return false;
+    const char * env = getenv("VX_GEMV_DMA"); // read on every call; 0 keeps the weights on the register path of gemv_kernel
+    if ((env && atoi(env) == 0) || nbatch != 1 || (nw != 4 && nw != 8 && nw != 16) || !a.x_aligned || !a.w_aligned || a.K % 256) return false;
     if (a.norm_w && a.K > 2048) return false;
     if (a.w2 && a.res) return false;
     if (a.nseg > 0 && (a.w2 || a.res)) return false;
@@ -964,11 +1018,9 @@ bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st)
     for (int i = 0; i < a.nseg; ++i) if (!al16(a.seg[i].w, a.seg[i].nb01)) return false;
     a.w_slot    = gemv_dma_slot(a.K);
     a.w_lds_off = (int) ((gemv_smem(a, ACT_Q8, nw, true) + 15) / 16 * 16);
-    a.w_ipr     = (int) ((a.K / 32 * VX_Q8_BLOCK / 16 + 63) / 64);
-    a.w_magic   = (65536 + a.w_ipr - 1) / a.w_ipr;
-    for (int t = 0; t < 16 * a.w_ipr; ++t) if (((t * a.w_magic) >> 16) != t / a.w_ipr) return false;
     const size_t smem = (size_t) a.w_lds_off + (size_t) a.rows_wg * a.w_slot;
     if (smem > GV_MAX_LDS) return false;
+    a.exact = (a.K / 32) % (4 * nw) == 0; // whole four-block rounds for every wave
     const dim3 block((unsigned) (64 * nw));
 #define VX_DMA_GO(NW_, SEG_, NORM_, EPI_)                                                                              \
     do {                                                                                                               \
@@ -985,7 +1037,7 @@ bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st)
         return true;                                                                                                   \
     } while (0)
 #define VX_DMA_NW(SEG_, NORM_, EPI_)                                                                                   \
-    do { if (nw == 8) VX_DMA_GO(8, SEG_, NORM_, EPI_); else VX_DMA_GO(16, SEG_, NORM_, EPI_); } while (0)
+    do { if (nw == 4) VX_DMA_GO(4, SEG_, NORM_, EPI_); else if (nw == 8) VX_DMA_GO(8, SEG_, NORM_, EPI_); else VX_DMA_GO(16, SEG_, NORM_, EPI_); } while (0)
     const bool norm = a.norm_w != nullptr;
     if (a.nseg > 0) { if (norm) VX_DMA_NW(true, true, GV_PLAIN); else VX_DMA_NW(true, false, GV_PLAIN); }
     if (a.w2)       { if (norm) VX_DMA_NW(false, true, GV_SWIGLU); else VX_DMA_NW(false, false, GV_SWIGLU); }
