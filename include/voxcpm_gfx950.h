@@ -368,10 +368,15 @@ enum { VX_NODE_ADD = 0, VX_NODE_SUB = 1, VX_NODE_MUL = 2, VX_NODE_DIV = 3,  /* v
        VX_NODE_REPEAT = 9,                                                  /* vx_repeat                        */
        VX_NODE_SUM = 10,                                                    /* vx_sum                           */
        VX_NODE_ARANGE = 11 };                                               /* vx_arange: p0 = start, p1 = step */
+/* flags: VX_SMALL_DST_PRIVATE -- the caller knows that nothing but later nodes of the same run reads dst (the plugin: every
+ * reader of the graph node is a member of the run and the node is no graph output).  Such a destination is then carried in
+ * LDS only, when there is room for it, and its memory is left untouched; without room it is written like any other. */
+#define VX_SMALL_DST_PRIVATE 1
 typedef struct vx_small_node {
     int32_t op, aux;
     float   p0, p1;
     const vx_tensor * src0, * src1, * dst;   /* src1 NULL where the operator has one operand, src0 NULL for ARANGE */
+    int32_t flags, reserved;
 } vx_small_node;
 VX_API vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx_stream stream);
 VX_API int vx_supports_small_node(const vx_small_node * node);

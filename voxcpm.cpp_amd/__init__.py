@@ -41,8 +41,12 @@ class VxSmallNode(C.Structure):
         ("src0", C.POINTER(VxTensor)),
         ("src1", C.POINTER(VxTensor)),
         ("dst", C.POINTER(VxTensor)),
+        ("flags", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
+
+SMALL_DST_PRIVATE = 1
 
 EXPORTS = [
     "vx_device_count", "vx_init", "vx_last_error", "vx_device_info", "vx_malloc", "vx_free",
@@ -372,10 +376,12 @@ def get_rows(table, rows, ne0=None, out=None):
     return out
 
 
-def small_node(op, dst, src0=None, src1=None, aux=0, p0=0.0, p1=0.0):
-    """One node of a small graph: tensors as descriptors (VxTensor) or torch tensors."""
+def small_node(op, dst, src0=None, src1=None, aux=0, p0=0.0, p1=0.0, private=False):
+    """One node of a small graph: tensors as descriptors (VxTensor) or torch tensors.  private: only later nodes of the
+    same run read dst (it may then live in LDS only and its memory stay untouched)."""
     nd = VxSmallNode()
     nd.op, nd.aux, nd.p0, nd.p1 = op, aux, p0, p1
+    nd.flags = SMALL_DST_PRIVATE if private else 0
     keep = []
     for name, t in (("src0", src0), ("src1", src1), ("dst", dst)):
         if t is None:

@@ -76,30 +76,31 @@ class LocDiTCfmSolver:
         for step in range(1, n_steps + 1):
             xn = xs[step % 2]
             if zero_star and step <= zero_init_steps:
-                graph([small_node(NODE_SCALE, tmp["dphi"], x, p0=0.0), small_node(NODE_SCALE, tmp["step"], tmp["dphi"], p0=float(dt)),
+                graph([small_node(NODE_SCALE, tmp["dphi"], x, p0=0.0, private=True), small_node(NODE_SCALE, tmp["step"], tmp["dphi"], p0=float(dt), private=True),
                        small_node(NODE_SUB, xn, x, tmp["step"])])
             else:
                 project(self.in_proj, x, x_proj)
                 row = table[step - 1:step]                       # the step's combined time embedding, (1, hidden)
-                graph([small_node(NODE_ADD, comb_c, row, mu.view(1, H)),
-                       small_node(NODE_CONCAT, a5, comb_c, cond_p, aux=1), small_node(NODE_CONCAT, a7, a5, x_proj, aux=1),
-                       small_node(NODE_CONCAT, b5, row, cond_p, aux=1), small_node(NODE_CONCAT, b7, b5, x_proj, aux=1),
+                # (everything but the last node of a run is read inside the run only, as the plugin finds from the graph)
+                graph([small_node(NODE_ADD, comb_c, row, mu.view(1, H), private=True),
+                       small_node(NODE_CONCAT, a5, comb_c, cond_p, aux=1, private=True), small_node(NODE_CONCAT, a7, a5, x_proj, aux=1, private=True),
+                       small_node(NODE_CONCAT, b5, row, cond_p, aux=1, private=True), small_node(NODE_CONCAT, b7, b5, x_proj, aux=1, private=True),
                        small_node(NODE_CONCAT, pair, a7, b7, aux=1)])
                 calls.append((dec_run, None))
                 n_dec += 1
                 project(self.out_proj, hc, vc)
                 project(self.out_proj, hu, vu)
                 if zero_star:
-                    nodes = [small_node(NODE_MUL, tmp["pc"], vc, vu), small_node(NODE_SUM, sc["dot"], tmp["pc"]),
-                             small_node(NODE_MUL, tmp["uu"], vu, vu), small_node(NODE_SUM, sc["nrm"], tmp["uu"]),
-                             small_node(NODE_ARANGE, sc["eps"], p0=1.0e-8, p1=1.0), small_node(NODE_ADD, sc["den"], sc["nrm"], sc["eps"]),
-                             small_node(NODE_DIV, sc["st"], sc["dot"], sc["den"]), small_node(NODE_REPEAT, tmp["rep"], sc["st"]),
-                             small_node(NODE_MUL, tmp["us"], vu, tmp["rep"]), small_node(NODE_SUB, tmp["diff"], vc, tmp["us"]),
-                             small_node(NODE_SCALE, tmp["cs"], tmp["diff"], p0=cfg_value), small_node(NODE_ADD, tmp["dphi"], tmp["us"], tmp["cs"])]
+                    nodes = [small_node(NODE_MUL, tmp["pc"], vc, vu, private=True), small_node(NODE_SUM, sc["dot"], tmp["pc"], private=True),
+                             small_node(NODE_MUL, tmp["uu"], vu, vu, private=True), small_node(NODE_SUM, sc["nrm"], tmp["uu"], private=True),
+                             small_node(NODE_ARANGE, sc["eps"], p0=1.0e-8, p1=1.0, private=True), small_node(NODE_ADD, sc["den"], sc["nrm"], sc["eps"], private=True),
+                             small_node(NODE_DIV, sc["st"], sc["dot"], sc["den"], private=True), small_node(NODE_REPEAT, tmp["rep"], sc["st"], private=True),
+                             small_node(NODE_MUL, tmp["us"], vu, tmp["rep"], private=True), small_node(NODE_SUB, tmp["diff"], vc, tmp["us"], private=True),
+                             small_node(NODE_SCALE, tmp["cs"], tmp["diff"], p0=cfg_value, private=True), small_node(NODE_ADD, tmp["dphi"], tmp["us"], tmp["cs"], private=True)]
                 else:
-                    nodes = [small_node(NODE_SUB, tmp["diff"], vc, vu), small_node(NODE_SCALE, tmp["cs"], tmp["diff"], p0=cfg_value),
-                             small_node(NODE_ADD, tmp["dphi"], vu, tmp["cs"])]
-                nodes += [small_node(NODE_SCALE, tmp["step"], tmp["dphi"], p0=float(dt)), small_node(NODE_SUB, xn, x, tmp["step"])]
+                    nodes = [small_node(NODE_SUB, tmp["diff"], vc, vu, private=True), small_node(NODE_SCALE, tmp["cs"], tmp["diff"], p0=cfg_value, private=True),
+                             small_node(NODE_ADD, tmp["dphi"], vu, tmp["cs"], private=True)]
+                nodes += [small_node(NODE_SCALE, tmp["step"], tmp["dphi"], p0=float(dt), private=True), small_node(NODE_SUB, xn, x, tmp["step"])]
                 graph(nodes)
             x = xn
             t = f(t - dt)

@@ -11,6 +11,7 @@
 #include "vx_common.hpp"
 #include "kvs_common.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <type_traits>
 
@@ -420,10 +421,14 @@ __global__ __launch_bounds__(SUM_BLOCKS) void sum_partials_kernel(const double *
 // merely overlaps something written earlier in the run (a view of it) is read from memory after a full barrier.
 constexpr int SG_MAX_NODES = 16;
 constexpr int SG_MAX_ELEMS = 16384;
-constexpr int SG_LDS_ELEMS = 12288; // 48 KiB of 4-byte slots (an F16 value sits in the low half of its slot)
+constexpr int SG_LDS_ELEMS = 38912; // 152 KiB of 4-byte slots at most (an F16 value sits in the low half of its slot); a run is given what it uses
 
 enum sg_kind : int { SG_EW2 = 0, SG_ADD1, SG_SCALE, SG_UNARY, SG_CPY, SG_CONCAT, SG_REPEAT, SG_SUM, SG_ARANGE };
 
+struct sg_shape {
+    int32_t ne[4];
+    int64_t nb[4];
+};
 struct sg_tensor {
     char *  p;
     int32_t ne[4];
@@ -438,10 +443,17 @@ struct sg_node {
     int32_t flat;        // 1: element e of the destination takes element e (or the only element) of every operand, all of
                          // them dense or imaged in LDS -- no index arithmetic; 2: a CONCAT of such tensors along their outermost dim
     int32_t one0, one1;  // with flat: operand 0 / 1 is a single element
-    sg_tensor s0, s1, d;
+    // all a flat node needs of its tensors, together at the front (the kernel reads these 22 dwords of a node first and
+    // the full descriptors only for the indexed forms): base, type and LDS slot of operand 0, operand 1, destination;
+    // element counts of the destination and of operand 0
+    char *   fp[3];
+    int32_t  ftype[3], flds[3];
+    uint32_t fn, fn0;
+    sg_shape sh[3];      // shapes and strides of operand 0, operand 1, destination (the indexed forms)
 };
+constexpr int SG_HEAD_DWORDS = (int) (offsetof(sg_node, sh) / 4);
 struct sg_args {
-    int32_t n, pad;
+    int32_t n, pad[3];
     sg_node node[SG_MAX_NODES];
 };
 
@@ -464,9 +476,11 @@ __device__ __forceinline__ uint32_t sg_get(const sg_tensor & t, const uint32_t (
 }
 // element e (row-major) = index i of the destination: to memory, and to the LDS image when it has one
 __device__ __forceinline__ void sg_put(const sg_tensor & t, uint32_t e, const uint32_t (&i)[4], uint32_t bits, uint32_t * lds) {
-    char * p = t.p + i[0] * t.nb[0] + i[1] * t.nb[1] + i[2] * t.nb[2] + i[3] * t.nb[3];
-    if (t.type == VX_TYPE_F16) *(uint16_t *) p = (uint16_t) bits;
-    else                       *(uint32_t *) p = bits;
+    if (t.p) { // (no memory behind a private destination that has its image)
+        char * p = t.p + i[0] * t.nb[0] + i[1] * t.nb[1] + i[2] * t.nb[2] + i[3] * t.nb[3];
+        if (t.type == VX_TYPE_F16) *(uint16_t *) p = (uint16_t) bits;
+        else                       *(uint32_t *) p = bits;
+    }
     if (t.lds >= 0) lds[(uint32_t) t.lds + e] = bits;
 }
 // the same for the flat case: element e in row-major order of a dense tensor (or its LDS image)
@@ -503,16 +517,49 @@ __device__ __forceinline__ double sum_lane_lds(const uint32_t * img, uint32_t fi
 
 __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
     __shared__ double   part[16];
-    __shared__ uint32_t lds[SG_LDS_ELEMS];
-    // The node table is fetched ONCE, by all threads together, into LDS: kernel arguments live in host-visible memory, and
-    // reading a node's fields where they are first needed costs a trip there per cache line and node.
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[]; // the images: as many slots as the host counted
+    // The node table is fetched ONCE, by all threads together, into LDS: read from the argument block where a field is
+    // first needed, every cache line of every node is a trip to memory of its own.  A node's fields then become scalars,
+    // once per node -- the head for every node, the full tensor descriptors only for the indexed forms.
     __shared__ __attribute__((aligned(16))) uint32_t table[(sizeof(sg_args) + 3) / 4];
-    static_assert(sizeof(sg_args) <= 4 * 1024, "one dword per thread");
-    if (threadIdx.x < (sizeof(sg_args) + 3) / 4) table[threadIdx.x] = ((const uint32_t *) &a0)[threadIdx.x];
+    {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        static_assert(sizeof(sg_args) % 16 == 0 && sizeof(sg_args) <= 256 * 16, "16 bytes per thread of the smallest work-group");
+        const uint32_t quads = (uint32_t) (offsetof(sg_args, node) + (size_t) a0.n * sizeof(sg_node) + 15) / 16;
+        if (threadIdx.x < quads) ((u32x4 *) table)[threadIdx.x] = ((const u32x4 *) &a0)[threadIdx.x]; // one trip to memory for the whole table
+    }
     __syncthreads();
-    const sg_args & a = *(const sg_args *) table;
-    for (int k = 0; k < a.n; ++k) { // uniform: every thread walks every node and meets every barrier
-        const sg_node & nd = a.node[k];
+    const uint32_t nt = blockDim.x; // the host sizes the work-group to the run: a run of 128-element nodes is two waves' work
+    const int n_nodes = a0.n;
+    // a node's head is read from the table one node ahead, so that its LDS latency passes under the node before it
+    uint32_t head[SG_HEAD_DWORDS];
+    auto read_head = [&](int k) {
+        const uint32_t * src = table + (offsetof(sg_args, node) + (size_t) k * sizeof(sg_node)) / 4;
+#pragma unroll
+        for (int i = 0; i < SG_HEAD_DWORDS; ++i) head[i] = src[i];
+    };
+    read_head(0);
+    for (int k = 0; k < n_nodes; ++k) { // uniform: every thread walks every node and meets every barrier
+        sg_node nd;
+        const uint32_t * nsrc = table + (offsetof(sg_args, node) + (size_t) k * sizeof(sg_node)) / 4;
+        {
+            uint32_t * dst = (uint32_t *) &nd;
+#pragma unroll
+            for (int i = 0; i < SG_HEAD_DWORDS; ++i) dst[i] = (uint32_t) __builtin_amdgcn_readfirstlane((int) head[i]);
+        }
+        if (k + 1 < n_nodes) read_head(k + 1);
+        if (nd.flat == 0) {
+            uint32_t * dst = (uint32_t *) &nd;
+#pragma unroll
+            for (int i = SG_HEAD_DWORDS; i < (int) (sizeof(sg_node) / 4); ++i) dst[i] = (uint32_t) __builtin_amdgcn_readfirstlane((int) nsrc[i]);
+        }
+        auto tensor_of = [&](int o) {
+            sg_tensor t;
+            t.p = nd.fp[o]; t.type = nd.ftype[o]; t.lds = nd.flds[o];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { t.ne[q] = nd.sh[o].ne[q]; t.nb[q] = nd.sh[o].nb[q]; }
+            return t;
+        };
         if (k > 0) {
             if (nd.wait_memory) {
                 __syncthreads(); // earlier nodes' stores to memory are complete and visible to the work-group
@@ -522,52 +569,76 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
             }
         }
-        const uint32_t n = sg_count(nd.d);
-        if (nd.flat == 1) { // dense operands of the destination's shape (or single elements): no index arithmetic
-            for (uint32_t e = threadIdx.x; e < n; e += 1024) {
-                uint32_t r;
-                if (nd.kind == SG_ARANGE) {
-                    r = sg_b(arange_value(nd.p0, nd.p1, (int64_t) e));
-                } else {
-                    const uint32_t xb = sg_get_flat(nd.s0, nd.one0 ? 0 : e, lds);
-                    const float x = sg_f(xb);
-                    switch (nd.kind) {
-                        case SG_EW2: {
-                            const float y = sg_f(sg_get_flat(nd.s1, nd.one1 ? 0 : e, lds));
-                            switch (nd.aux) {
-                                case VX_BIN_ADD: r = sg_b(ew_apply<EW_ADD>(0, 0, 0, x, y)); break;
-                                case VX_BIN_SUB: r = sg_b(ew_apply<EW_SUB>(0, 0, 0, x, y)); break;
-                                case VX_BIN_MUL: r = sg_b(ew_apply<EW_MUL>(0, 0, 0, x, y)); break;
-                                default:         r = sg_b(ew_apply<EW_DIV>(0, 0, 0, x, y)); break;
-                            }
-                        } break;
-                        case SG_ADD1:  r = sg_b(ew_apply<EW_ADD1>(0, 0, 0, x, sg_f(sg_get_flat(nd.s1, 0, lds)))); break;
-                        case SG_SCALE: r = sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, x, 0.0f)); break;
-                        case SG_UNARY: r = sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, x, 0.0f)); break;
-                        default: // SG_CPY between dense tensors (element e to element e), SG_REPEAT of one value
-                            if (nd.s0.type == VX_TYPE_I32)      r = nd.d.type == VX_TYPE_I32 ? xb : sg_convert<int32_t, float>(xb);
-                            else if (nd.d.type == VX_TYPE_I32)  r = sg_convert<float, int32_t>(xb);
-                            else if (nd.s0.type == VX_TYPE_F32) r = nd.d.type == VX_TYPE_F32 ? xb : sg_convert<float, _Float16>(xb);
-                            else                                r = nd.d.type == VX_TYPE_F32 ? sg_convert<_Float16, float>(xb) : xb;
-                            break;
-                    }
-                }
-                sg_put_flat(nd.d, e, r, lds);
+        const uint32_t n = nd.fn;
+        // where each tensor's elements are, decided once: its LDS image, or memory as F32 / I32 or F16
+        const uint32_t * img0 = nd.flds[0] >= 0 ? lds + nd.flds[0] : nullptr, * img1 = nd.flds[1] >= 0 ? lds + nd.flds[1] : nullptr;
+        uint32_t *       imgd = nd.flds[2] >= 0 ? lds + nd.flds[2] : nullptr;
+        auto get0 = [&](uint32_t e) -> uint32_t {
+            if (img0) return img0[e];
+            return nd.ftype[0] == VX_TYPE_F16 ? (uint32_t) ((const uint16_t *) nd.fp[0])[e] : ((const uint32_t *) nd.fp[0])[e];
+        };
+        auto get1 = [&](uint32_t e) -> uint32_t {
+            if (img1) return img1[e];
+            return nd.ftype[1] == VX_TYPE_F16 ? (uint32_t) ((const uint16_t *) nd.fp[1])[e] : ((const uint32_t *) nd.fp[1])[e];
+        };
+        auto put = [&](uint32_t e, uint32_t bits) { // (no memory behind a private destination that has its image)
+            if (nd.fp[2]) {
+                if (nd.ftype[2] == VX_TYPE_F16) ((uint16_t *) nd.fp[2])[e] = (uint16_t) bits;
+                else                            ((uint32_t *) nd.fp[2])[e] = bits;
             }
+            if (imgd) imgd[e] = bits;
+        };
+        if (nd.flat == 1) { // dense operands of the destination's shape (or single elements): no index arithmetic
+#define SG_FLAT_LOOP(expr) for (uint32_t e = threadIdx.x; e < n; e += nt) put(e, (expr))
+#define SG_X (sg_f(get0(nd.one0 ? 0 : e)))
+#define SG_Y (sg_f(get1(nd.one1 ? 0 : e)))
+            switch (nd.kind) {
+                case SG_ARANGE: SG_FLAT_LOOP(sg_b(arange_value(nd.p0, nd.p1, (int64_t) e))); break;
+                case SG_EW2:
+                    switch (nd.aux) {
+                        case VX_BIN_ADD: SG_FLAT_LOOP(sg_b(ew_apply<EW_ADD>(0, 0, 0, SG_X, SG_Y))); break;
+                        case VX_BIN_SUB: SG_FLAT_LOOP(sg_b(ew_apply<EW_SUB>(0, 0, 0, SG_X, SG_Y))); break;
+                        case VX_BIN_MUL: SG_FLAT_LOOP(sg_b(ew_apply<EW_MUL>(0, 0, 0, SG_X, SG_Y))); break;
+                        default:         SG_FLAT_LOOP(sg_b(ew_apply<EW_DIV>(0, 0, 0, SG_X, SG_Y))); break;
+                    }
+                    break;
+                case SG_ADD1: {
+                    const float y = sg_f(get1(0));
+                    SG_FLAT_LOOP(sg_b(ew_apply<EW_ADD1>(0, 0, 0, SG_X, y)));
+                } break;
+                case SG_SCALE: SG_FLAT_LOOP(sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, SG_X, 0.0f))); break;
+                case SG_UNARY: SG_FLAT_LOOP(sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, SG_X, 0.0f))); break;
+                default: // SG_CPY between dense tensors (element e to element e), SG_REPEAT of one value
+#define SG_BITS (get0(nd.one0 ? 0 : e))
+                    if (nd.ftype[0] == VX_TYPE_I32) {
+                        if (nd.ftype[2] == VX_TYPE_I32) SG_FLAT_LOOP(SG_BITS); else SG_FLAT_LOOP((sg_convert<int32_t, float>(SG_BITS)));
+                    } else if (nd.ftype[2] == VX_TYPE_I32) {
+                        SG_FLAT_LOOP((sg_convert<float, int32_t>(SG_BITS)));
+                    } else if (nd.ftype[0] == VX_TYPE_F32) {
+                        if (nd.ftype[2] == VX_TYPE_F32) SG_FLAT_LOOP(SG_BITS); else SG_FLAT_LOOP((sg_convert<float, _Float16>(SG_BITS)));
+                    } else {
+                        if (nd.ftype[2] == VX_TYPE_F32) SG_FLAT_LOOP((sg_convert<_Float16, float>(SG_BITS))); else SG_FLAT_LOOP(SG_BITS);
+                    }
+#undef SG_BITS
+                    break;
+            }
+#undef SG_X
+#undef SG_Y
+#undef SG_FLAT_LOOP
             continue;
         }
         if (nd.flat == 2) { // CONCAT along the outermost dim: the first operand's elements, then the second's
-            const uint32_t n0 = sg_count(nd.s0);
-            for (uint32_t e = threadIdx.x; e < n; e += 1024)
-                sg_put_flat(nd.d, e, e < n0 ? sg_get_flat(nd.s0, e, lds) : sg_get_flat(nd.s1, e - n0, lds), lds);
+            const uint32_t n0 = nd.fn0;
+            for (uint32_t e = threadIdx.x; e < n; e += nt) put(e, e < n0 ? get0(e) : get1(e - n0));
             continue;
         }
+        const sg_tensor S0 = tensor_of(0), S1 = tensor_of(1), D = tensor_of(2); // only the indexed forms get here
         switch (nd.kind) {
             case SG_EW2:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    const float x = sg_f(sg_get<false>(nd.s0, i, lds)), y = sg_f(sg_get<true>(nd.s1, i, lds));
+                    sg_index(D, e, i);
+                    const float x = sg_f(sg_get<false>(S0, i, lds)), y = sg_f(sg_get<true>(S1, i, lds));
                     float r;
                     switch (nd.aux) {
                         case VX_BIN_ADD: r = ew_apply<EW_ADD>(0, 0, 0, x, y); break;
@@ -575,92 +646,92 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
                         case VX_BIN_MUL: r = ew_apply<EW_MUL>(0, 0, 0, x, y); break;
                         default:         r = ew_apply<EW_DIV>(0, 0, 0, x, y); break;
                     }
-                    sg_put(nd.d, e, i, sg_b(r), lds);
+                    sg_put(D, e, i, sg_b(r), lds);
                 }
                 break;
             case SG_ADD1: {
                 const uint32_t zero[4] = { 0, 0, 0, 0 };
-                const float y = sg_f(sg_get<false>(nd.s1, zero, lds));
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                const float y = sg_f(sg_get<false>(S1, zero, lds));
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_ADD1>(0, 0, 0, sg_f(sg_get<false>(nd.s0, i, lds)), y)), lds);
+                    sg_index(D, e, i);
+                    sg_put(D, e, i, sg_b(ew_apply<EW_ADD1>(0, 0, 0, sg_f(sg_get<false>(S0, i, lds)), y)), lds);
                 }
             } break;
             case SG_SCALE:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, sg_f(sg_get<false>(nd.s0, i, lds)), 0.0f)), lds);
+                    sg_index(D, e, i);
+                    sg_put(D, e, i, sg_b(ew_apply<EW_SCALE>(nd.p0, nd.p1, 0, sg_f(sg_get<false>(S0, i, lds)), 0.0f)), lds);
                 }
                 break;
             case SG_UNARY:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    sg_put(nd.d, e, i, sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, sg_f(sg_get<false>(nd.s0, i, lds)), 0.0f)), lds);
+                    sg_index(D, e, i);
+                    sg_put(D, e, i, sg_b(ew_apply<EW_UNARY>(0, 0, nd.aux, sg_f(sg_get<false>(S0, i, lds)), 0.0f)), lds);
                 }
                 break;
             case SG_CPY: // element e of the source shape -> element e of the destination shape
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t is[4], id[4];
-                    sg_index(nd.s0, e, is);
-                    sg_index(nd.d, e, id);
-                    const uint32_t x = sg_get<false>(nd.s0, is, lds);
+                    sg_index(S0, e, is);
+                    sg_index(D, e, id);
+                    const uint32_t x = sg_get<false>(S0, is, lds);
                     uint32_t y;
-                    if (nd.s0.type == VX_TYPE_I32)      y = nd.d.type == VX_TYPE_I32 ? x : sg_convert<int32_t, float>(x);
-                    else if (nd.d.type == VX_TYPE_I32)  y = sg_convert<float, int32_t>(x);
-                    else if (nd.s0.type == VX_TYPE_F32) y = nd.d.type == VX_TYPE_F32 ? x : sg_convert<float, _Float16>(x);
-                    else                                y = nd.d.type == VX_TYPE_F32 ? sg_convert<_Float16, float>(x) : x;
-                    sg_put(nd.d, e, id, y, lds);
+                    if (S0.type == VX_TYPE_I32)      y = D.type == VX_TYPE_I32 ? x : sg_convert<int32_t, float>(x);
+                    else if (D.type == VX_TYPE_I32)  y = sg_convert<float, int32_t>(x);
+                    else if (S0.type == VX_TYPE_F32) y = D.type == VX_TYPE_F32 ? x : sg_convert<float, _Float16>(x);
+                    else                                y = D.type == VX_TYPE_F32 ? sg_convert<_Float16, float>(x) : x;
+                    sg_put(D, e, id, y, lds);
                 }
                 break;
             case SG_CONCAT:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4], j[4];
-                    sg_index(nd.d, e, i);
+                    sg_index(D, e, i);
 #pragma unroll
                     for (int q = 0; q < 4; ++q) j[q] = i[q];
                     uint32_t off = 0;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) if (q == nd.aux) off = (uint32_t) nd.s0.ne[q];
+                    for (int q = 0; q < 4; ++q) if (q == nd.aux) off = (uint32_t) S0.ne[q];
                     bool second = false;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) if (q == nd.aux && i[q] >= off) { j[q] = i[q] - off; second = true; }
-                    sg_put(nd.d, e, i, second ? sg_get<false>(nd.s1, j, lds) : sg_get<false>(nd.s0, j, lds), lds);
+                    sg_put(D, e, i, second ? sg_get<false>(S1, j, lds) : sg_get<false>(S0, j, lds), lds);
                 }
                 break;
             case SG_REPEAT:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    sg_put(nd.d, e, i, sg_get<true>(nd.s0, i, lds), lds);
+                    sg_index(D, e, i);
+                    sg_put(D, e, i, sg_get<true>(S0, i, lds), lds);
                 }
                 break;
             case SG_SUM: { // vx_sum's two single-block orders: one wave up to VX_SUM_ONE_WAVE_UNITS units, the block beyond
                 vx_dims s;
-                for (int q = 0; q < 4; ++q) { s.ne[q] = nd.s0.ne[q]; s.nb[q] = (uint64_t) nd.s0.nb[q]; }
-                const uint32_t units = sg_count(nd.s0) / (nd.aux ? 4 : 1);
+                for (int q = 0; q < 4; ++q) { s.ne[q] = S0.ne[q]; s.nb[q] = (uint64_t) S0.nb[q]; }
+                const uint32_t units = sg_count(S0) / (nd.aux ? 4 : 1);
                 const bool one_wave = units <= VX_SUM_ONE_WAVE_UNITS;
-                const uint32_t step = one_wave ? 64 : 1024;
+                const uint32_t step = one_wave ? 64 : 1024; // (a sum over the whole block: the host launches 1024 threads for such a run)
                 double acc = 0.0;
                 if (!one_wave || threadIdx.x < 64) {
-                    if (nd.s0.lds >= 0) acc = nd.aux ? sum_lane_lds<true>(lds + nd.s0.lds, threadIdx.x, step, units) : sum_lane_lds<false>(lds + nd.s0.lds, threadIdx.x, step, units);
-                    else                acc = nd.aux ? sum_lane<true>(nd.s0.p, s, threadIdx.x, step, units) : sum_lane<false>(nd.s0.p, s, threadIdx.x, step, units);
+                    if (S0.lds >= 0) acc = nd.aux ? sum_lane_lds<true>(lds + S0.lds, threadIdx.x, step, units) : sum_lane_lds<false>(lds + S0.lds, threadIdx.x, step, units);
+                    else                acc = nd.aux ? sum_lane<true>(S0.p, s, threadIdx.x, step, units) : sum_lane<false>(S0.p, s, threadIdx.x, step, units);
                 }
                 double t;
                 if (one_wave) t = threadIdx.x < 64 ? vx_wave_sum(acc) : 0.0;
                 else          t = block_total(acc, part);
                 if (threadIdx.x == 0) {
                     const uint32_t zero[4] = { 0, 0, 0, 0 };
-                    sg_put(nd.d, 0, zero, sg_b((float) t), lds);
+                    sg_put(D, 0, zero, sg_b((float) t), lds);
                 }
             } break;
             case SG_ARANGE:
-                for (uint32_t e = threadIdx.x; e < n; e += 1024) {
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
                     uint32_t i[4];
-                    sg_index(nd.d, e, i);
-                    sg_put(nd.d, e, i, sg_b(arange_value(nd.p0, nd.p1, (int64_t) e)), lds);
+                    sg_index(D, e, i);
+                    sg_put(D, e, i, sg_b(arange_value(nd.p0, nd.p1, (int64_t) e)), lds);
                 }
                 break;
             default: break;
@@ -1082,7 +1153,8 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         if (!vx_supports_small_node(&nd)) return vx_fail(VX_ERR_UNSUPPORTED, "small graph: node %d (op %d) is not a small elementwise / copy / sum node", k, nd.op);
         if (!nd.dst->data || (nd.src0 && !nd.src0->data) || (nd.src1 && !nd.src1->data)) return vx_fail(VX_ERR_INVALID, "small graph: null data in node %d", k);
         sg_node & g = a.node[k];
-        g.s0 = sg_desc(nd.op == VX_NODE_ARANGE ? nullptr : nd.src0); g.s1 = sg_desc(nd.src1); g.d = sg_desc(nd.dst);
+        struct { sg_tensor s0, s1, d; } gt; // the three descriptors while the node is put together
+        gt.s0 = sg_desc(nd.op == VX_NODE_ARANGE ? nullptr : nd.src0); gt.s1 = sg_desc(nd.src1); gt.d = sg_desc(nd.dst);
         g.p0 = nd.p0; g.p1 = nd.p1; g.aux = nd.aux;
         switch (nd.op) {
             case VX_NODE_ADD: case VX_NODE_SUB: case VX_NODE_MUL: case VX_NODE_DIV: g.kind = SG_EW2; g.aux = nd.op - VX_NODE_ADD; break;
@@ -1097,7 +1169,7 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         }
         // operands: the LDS image of exactly this tensor, else memory -- after a full barrier if the run wrote there
         const vx_tensor * ops[2] = { nd.op == VX_NODE_ARANGE ? nullptr : nd.src0, nd.src1 };
-        sg_tensor * gops[2] = { &g.s0, &g.s1 };
+        sg_tensor * gops[2] = { &gt.s0, &gt.s1 };
         for (int o = 0; o < 2; ++o) {
             if (!ops[o]) continue;
             for (int m = 0; m < n_images; ++m)
@@ -1120,14 +1192,24 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             if (dsp.lo < written[m].hi && written[m].lo < dsp.hi && !sg_same(&written_t[m], nd.dst)) g.wait_memory = 1;
         const int32_t cnt = (int32_t) vx_nelements(nd.dst);
         if (mine >= 0) {
-            g.d.lds = images[mine].off;
+            gt.d.lds = images[mine].off;
         } else if (lds_used + cnt <= SG_LDS_ELEMS) {
             images[n_images] = { *nd.dst, lds_used, true };
-            g.d.lds = lds_used;
+            gt.d.lds = lds_used;
             lds_used += cnt;
             ++n_images;
         }
-        written[n_written] = dsp; written_t[n_written] = *nd.dst; ++n_written;
+        // a private destination with an image is not stored at all (and so leaves no bytes for later nodes to wait for)
+        const bool in_lds_only = (nd.flags & VX_SMALL_DST_PRIVATE) && gt.d.lds >= 0;
+        if (in_lds_only) gt.d.p = nullptr;
+        else { written[n_written] = dsp; written_t[n_written] = *nd.dst; ++n_written; }
+        const sg_tensor * gts[3] = { &gt.s0, &gt.s1, &gt.d };
+        for (int o = 0; o < 3; ++o)
+            for (int q = 0; q < 4; ++q) { g.sh[o].ne[q] = gts[o]->ne[q]; g.sh[o].nb[q] = gts[o]->nb[q]; }
+        g.fp[0] = gt.s0.p; g.fp[1] = gt.s1.p; g.fp[2] = gt.d.p;
+        g.ftype[0] = gt.s0.type; g.ftype[1] = gt.s1.type; g.ftype[2] = gt.d.type;
+        g.flds[0] = gt.s0.lds; g.flds[1] = gt.s1.lds; g.flds[2] = gt.d.lds;
+        g.fn = (uint32_t) vx_nelements(nd.dst); g.fn0 = ops[0] ? (uint32_t) vx_nelements(ops[0]) : 0;
         // the flat forms: dense row-major tensors (or LDS images) indexed by the destination's element number
         if (vx_is_contiguous(nd.dst)) {
             auto flat_operand = [&](const vx_tensor * t, const sg_tensor & gt, int32_t * one) {
@@ -1135,24 +1217,43 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
                 if (vx_nelements(t) == 1) { *one = 1; return true; }
                 return vx_same_shape(t, nd.dst) && (gt.lds >= 0 || vx_is_contiguous(t));
             };
-            const bool f0 = ops[0] ? flat_operand(ops[0], g.s0, &g.one0) : true;
-            const bool f1 = ops[1] ? flat_operand(ops[1], g.s1, &g.one1) : true;
+            const bool f0 = ops[0] ? flat_operand(ops[0], gt.s0, &g.one0) : true;
+            const bool f1 = ops[1] ? flat_operand(ops[1], gt.s1, &g.one1) : true;
             switch (g.kind) {
                 case SG_EW2: case SG_SCALE: case SG_UNARY: if (f0 && f1) g.flat = 1; break;
                 case SG_ADD1:   if (f0) g.flat = 1; break;
                 case SG_REPEAT: if (g.one0) g.flat = 1; break; // one value over the whole destination
                 case SG_ARANGE: g.flat = 1; break;
-                case SG_CPY:    if (g.s0.lds >= 0 || vx_is_contiguous(ops[0])) g.flat = 1; break; // element e -> element e whatever the shapes
+                case SG_CPY:    if (gt.s0.lds >= 0 || vx_is_contiguous(ops[0])) g.flat = 1; break; // element e -> element e whatever the shapes
                 case SG_CONCAT: {
                     bool outer = true;
                     for (int q = nd.aux + 1; q < 4; ++q) outer = outer && nd.dst->ne[q] == 1;
-                    if (outer && (g.s0.lds >= 0 || vx_is_contiguous(ops[0])) && (g.s1.lds >= 0 || vx_is_contiguous(ops[1]))) g.flat = 2;
+                    if (outer && (gt.s0.lds >= 0 || vx_is_contiguous(ops[0])) && (gt.s1.lds >= 0 || vx_is_contiguous(ops[1]))) g.flat = 2;
                 } break;
                 default: break;
             }
         }
     }
-    small_graph_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
+    // the work-group: a thread per element of the largest node, in whole waves; a sum that takes the whole block's order
+    // (more than one wave's units) needs all 1024
+    int64_t most = 64;
+    bool    block_sum = false;
+    for (int k = 0; k < n_nodes; ++k) {
+        most = std::max(most, vx_nelements(nodes[k].dst));
+        if (a.node[k].kind == SG_SUM && vx_nelements(nodes[k].src0) / (a.node[k].aux ? 4 : 1) > VX_SUM_ONE_WAVE_UNITS) block_sum = true;
+    }
+    const unsigned threads = block_sum ? 1024u : (unsigned) std::min<int64_t>(1024, std::max<int64_t>(256, (most + 63) / 64 * 64));
+    static_assert(sizeof(sg_args) <= 4096, "the node table rides in the kernel's argument block");
+    const size_t smem = (size_t) lds_used * 4;
+    if (smem > 48 * 1024) { // a kernel has to be told once that it may be given more dynamic LDS than the default limit
+        static bool raised = false;
+        if (!raised) {
+            if (hipFuncSetAttribute((const void *) small_graph_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SG_LDS_ELEMS * 4) != hipSuccess)
+                return vx_fail(VX_ERR_HIP, "small graph: %s", hipGetErrorString(hipGetLastError()));
+            raised = true;
+        }
+    }
+    small_graph_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -692,7 +692,7 @@ __device__ __forceinline__ void gv_round4(const char * sp, int j, const _Float16
     }
 }
 
-template <bool ACT_Q8, int NW, bool SEG, bool NORM, int EPI>
+template <bool ACT_Q8, int NW, bool SEG, bool NORM, int EPI, bool MANY>
 __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     static_assert(NW == 4 || NW == 8 || NW == 16, "four, eight or sixteen waves");
     constexpr int  NWD = NW / 2, NA = NW - NWD; // waves 0 .. NWD-1 fetch the weights, the rest handle the activations
@@ -787,11 +787,14 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     } else {
         // ---- activations -> LDS as f16 (or quantised), [token][k]
         const int awid = wid - NWD, atid = tid - 64 * NWD;
-        auto fetch = [&](int unit, float4_t & v0, float4_t & v1, float4_t & g0, float4_t & g1) {
+        auto fetch = [&](int unit, float4_t & v0, float4_t & v1) {
             const int t = unit_token(unit), u = unit - t * upr;
             const float4_t * xp = (const float4_t *) ((const float *) (xb + (uint64_t) t * a.nb11) + 8 * u);
             v0 = xp[0]; v1 = xp[1];
-            if constexpr (NORM) { const float4_t * gp = (const float4_t *) (a.norm_w + 8 * u); g0 = gp[0]; g1 = gp[1]; }
+        };
+        auto fetch_gain = [&](int unit, float4_t & g0, float4_t & g1) { // the norm weights of a unit's 8 columns
+            const float4_t * gp = (const float4_t *) (a.norm_w + 8 * (unit - unit_token(unit) * upr));
+            g0 = gp[0]; g1 = gp[1];
         };
         auto stage = [&](int unit, const float4_t & v0, const float4_t & v1, const float4_t & g0, const float4_t & g1) {
             const int t = unit_token(unit), u = unit - t * upr;
@@ -824,8 +827,24 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
             }
             *(half8_t *) (xs + (size_t) t * KP + 8 * u) = h;
         };
-        float4_t f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0}, g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
-        if (atid < units) fetch(atid, f0, f1, g0, g1);
+        // A thread's units are requested together, up to UB of them, before the first is staged: a round trip per unit
+        // would be paid a dozen times with sixteen tokens.  When the threads' stride is a multiple of a row's units (the usual
+        // shapes) all units of a thread sit in the same columns and share their norm weights.
+        // (MANY: more than one unit per thread; the one-unit kernel keeps few enough registers for two work-groups per CU)
+        constexpr int UB = MANY ? (NW == 16 ? 4 : 8) : 1;
+        const bool same_cols = (64 * NA) % upr == 0; // uniform
+        float4_t f0[UB], f1[UB], g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
+        // with a fused norm and many units the requests wait until the norm's rows have left the registers (two
+        // work-groups per CU need the kernel under 128 of them); the rows have pulled the same lines into the cache
+        constexpr bool LATE = NORM && MANY;
+        if (same_cols && !LATE) {
+#pragma unroll
+            for (int i = 0; i < UB; ++i) {
+                const int unit = atid + i * 64 * NA;
+                if (unit < units) fetch(unit, f0[i], f1[i]);
+            }
+            if constexpr (NORM) { if (atid < units) fetch_gain(atid, g0, g1); }
+        }
         vx_rms_row nrow, nrow2; // the tokens this wave normalises first, requested up front
         if constexpr (NORM) {
             if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
@@ -860,10 +879,25 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
             }
             __syncthreads();
         }
-        if (atid < units) stage(atid, f0, f1, g0, g1);
-        for (int unit = atid + 64 * NA; unit < units; unit += 64 * NA) {
-            fetch(unit, f0, f1, g0, g1);
-            stage(unit, f0, f1, g0, g1);
+        if (same_cols) {
+            if constexpr (LATE) {
+#pragma unroll
+                for (int i = 0; i < UB; ++i) {
+                    const int unit = atid + i * 64 * NA;
+                    if (unit < units) fetch(unit, f0[i], f1[i]);
+                }
+                if (atid < units) fetch_gain(atid, g0, g1);
+            }
+#pragma unroll
+            for (int i = 0; i < UB; ++i) {
+                const int unit = atid + i * 64 * NA;
+                if (unit < units) stage(unit, f0[i], f1[i], g0, g1);
+            }
+        }
+        for (int unit = atid + (same_cols ? UB : 0) * 64 * NA; unit < units; unit += 64 * NA) {
+            fetch(unit, f0[0], f1[0]);
+            if constexpr (NORM) { if (!same_cols) fetch_gain(unit, g0, g1); }
+            stage(unit, f0[0], f1[0], g0, g1);
         }
     }
     __syncthreads();
@@ -1004,18 +1038,28 @@ int gemv_dma_slot(int64_t K) {
     return row_bytes + best_pad;
 }
 
-// Launches gemv_dma_kernel if the call is one it takes (a: as launch_gemv has prepared it, rows_wg and the prologue
-// helpers included; nw: the wave count every kernel uses for this shape).
-template <bool ACT_Q8>
-bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st) {
+// Everything gemv_dma_kernel asks of a call except room in LDS
+bool gemv_dma_takes(const mm_args & a, int nbatch, int nw) {
     const char * env = getenv("VX_GEMV_DMA"); // read on every call; 0 keeps the weights on the register path of gemv_kernel
     if ((env && atoi(env) == 0) || nbatch != 1 || (nw != 4 && nw != 8 && nw != 16) || !a.x_aligned || !a.w_aligned || a.K % 256) return false;
     if (a.norm_w && a.K > 2048) return false;
     if (a.w2 && a.res) return false;
     if (a.nseg > 0 && (a.w2 || a.res)) return false;
+    if (a.res && a.norm_w) return false;
     auto al16 = [](const void * p_, uint64_t stride) { return (uintptr_t) p_ % 16 == 0 && stride % 16 == 0; };
     if (a.nseg == 0 && (!al16(a.w, a.nb01) || (a.w2 && !al16(a.w2, 0)))) return false;
     for (int i = 0; i < a.nseg; ++i) if (!al16(a.seg[i].w, a.seg[i].nb01)) return false;
+    return true;
+}
+size_t gemv_dma_lds(const mm_args & a, bool act_q8, int nw, int rows_wg) {
+    return (gemv_smem(a, act_q8, nw, true) + 15) / 16 * 16 + (size_t) rows_wg * gemv_dma_slot(a.K);
+}
+
+// Launches gemv_dma_kernel if the call is one it takes (a: as launch_gemv has prepared it, rows_wg and the prologue
+// helpers included; nw: the wave count every kernel uses for this shape).
+template <bool ACT_Q8>
+bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st) {
+    if (!gemv_dma_takes(a, nbatch, nw)) return false;
     a.w_slot    = gemv_dma_slot(a.K);
     a.w_lds_off = (int) ((gemv_smem(a, ACT_Q8, nw, true) + 15) / 16 * 16);
     const size_t smem = (size_t) a.w_lds_off + (size_t) a.rows_wg * a.w_slot;
@@ -1024,13 +1068,14 @@ bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st)
     const dim3 block((unsigned) (64 * nw));
 #define VX_DMA_GO(NW_, SEG_, NORM_, EPI_)                                                                              \
     do {                                                                                                               \
-        auto kern = gemv_dma_kernel<ACT_Q8, NW_, SEG_, NORM_, EPI_>;                                                   \
+        auto kern = many ? gemv_dma_kernel<ACT_Q8, NW_, SEG_, NORM_, EPI_, true>                                       \
+                         : gemv_dma_kernel<ACT_Q8, NW_, SEG_, NORM_, EPI_, false>;                                     \
         if (smem > 64 * 1024) { /* above 64 KiB of LDS a kernel has to be told once that it may be given that much */  \
-            static bool raised = false;                                                                                \
-            if (!raised) {                                                                                             \
+            static bool raised[2] = { false, false };                                                                  \
+            if (!raised[many]) {                                                                                       \
                 if (hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize,               \
                                         (int) GV_MAX_LDS) != hipSuccess) { (void) hipGetLastError(); return false; }   \
-                raised = true;                                                                                         \
+                raised[many] = true;                                                                                   \
             }                                                                                                          \
         }                                                                                                              \
         kern<<<grid, block, smem, st>>>(a);                                                                            \
@@ -1039,6 +1084,7 @@ bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st)
 #define VX_DMA_NW(SEG_, NORM_, EPI_)                                                                                   \
     do { if (nw == 4) VX_DMA_GO(4, SEG_, NORM_, EPI_); else if (nw == 8) VX_DMA_GO(8, SEG_, NORM_, EPI_); else VX_DMA_GO(16, SEG_, NORM_, EPI_); } while (0)
     const bool norm = a.norm_w != nullptr;
+    const bool many = (a.N < 16 ? a.N : 16) * (a.K / 8) > 64 * (nw - nw / 2); // an activation thread stages more than one unit
     if (a.nseg > 0) { if (norm) VX_DMA_NW(true, true, GV_PLAIN); else VX_DMA_NW(true, false, GV_PLAIN); }
     if (a.w2)       { if (norm) VX_DMA_NW(false, true, GV_SWIGLU); else VX_DMA_NW(false, false, GV_SWIGLU); }
     if (a.res)      { if (norm) return false; VX_DMA_NW(false, false, GV_RES); }
@@ -1107,6 +1153,10 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     if (nw < 0) return false;
     const size_t smem = gemv_smem(a, ACT_Q8, nw);
     if (smem > GV_MAX_LDS) return false;
+    if constexpr (WT == WT_Q8) { // the kernel that keeps a work-group's rows in LDS: fewer rows each when they would not fit
+        if (gemv_dma_takes(a, nbatch, nw))
+            while (a.rows_wg > 4 && gemv_dma_lds(a, ACT_Q8, nw, a.rows_wg) > GV_MAX_LDS) a.rows_wg /= 2;
+    }
     int64_t nwg = groups(a.rows_wg);
     if (a.nseg > 0) {
         int wg0 = 0;

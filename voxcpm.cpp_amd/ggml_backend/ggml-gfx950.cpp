@@ -754,7 +754,8 @@ bool small_node_of(const ggml_tensor * n, vx_small_node * out, vx_tensor (&t)[3]
 
 // The run of tiny nodes that starts at node i (at most 16, view nodes in between skipped) as ONE launch: the bias adds,
 // sequence-assembling CONCATs, guidance arithmetic and Euler update around the LocDiT estimator (src/locdit.cpp:401-464,
-// src/unified_cfm.cpp:30-149).  Every node still writes its own tensor, in graph order, so no reader analysis is needed.
+// src/unified_cfm.cpp:30-149).  A node all of whose readers are members of the run (and which is no graph output) is
+// marked private: the kernel may keep it in LDS only.  Every other node writes its own tensor, in graph order.
 // The run stops in front of anything another group claims.  Returns the index of the run's last node, or -1 when fewer
 // than two nodes qualify.
 int compute_small_run(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers,
@@ -777,6 +778,28 @@ int compute_small_run(backend_ctx * ctx, const ggml_cgraph * g, int i, const rea
         last = j;
     }
     if (count < 2) return -1;
+    // readers inside the run, per member (a view of a member is a reader outside it: views are not members)
+    const ggml_tensor * member[MAX_RUN];
+    int inside[MAX_RUN] = {0};
+    {
+        int m = 0;
+        for (int j = i; j <= last; ++j) {
+            const ggml_tensor * n = g->nodes[j];
+            if (ggml_op_is_empty(n->op) || ggml_is_empty(n)) continue;
+            member[m++] = n;
+        }
+        for (int k = 0; k < count; ++k)
+            for (int sidx = 0; sidx < GGML_MAX_SRC; ++sidx) {
+                const ggml_tensor * src = member[k]->src[sidx];
+                if (!src) continue;
+                for (int q = 0; q < k; ++q) if (member[q] == src) ++inside[q];
+            }
+    }
+    for (int k = 0; k + 1 < count; ++k) { // (the last member has no reader in the run)
+        const auto it = readers.find(member[k]);
+        const bool out = (member[k]->flags & GGML_TENSOR_FLAG_OUTPUT) != 0;
+        if (!out && it != readers.end() && it->second == inside[k] && inside[k] > 0) nodes[k].flags |= VX_SMALL_DST_PRIVATE;
+    }
     *rc = vx_small_graph(nodes, count, ctx->stream);
     return last;
 }
