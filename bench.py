@@ -324,14 +324,21 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         # through the product boundary: ggml hands the reference-structured graph to the plugin's graph_compute
         assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) == 0
         assert ref.rh_use_device(b"GFX950_0", 1, 0) == 0
+        plug = C.CDLL(pkg.PLUGIN_PATH)
         reflib.ref_backbone_create(params, max_len, batch, use_mup=True, kv_f16=kv_f16)
+        plug.ggml_backend_gfx950_set_graph_replay(0)   # a decode step's graph changes with the KV length: launched node group by node group
         _, _, n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps)
         st = stats(reflib.ref_last_times())
+        launches = plug.ggml_backend_gfx950_last_launches()
+        plug.ggml_backend_gfx950_set_graph_replay(1)   # the same graph again and again (what a fixed-length step would be): recorded, then replayed
+        reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps)
+        st_r = stats(reflib.ref_last_times()[3:])
         ref.rh_bb_free()
-        launches = C.CDLL(pkg.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
         res["plugin_graph_compute"] = {"decode_steps_per_s": 1.0 / st["mean"], "ms_per_step": {n: st[n] * 1e3 for n in ("mean", "median", "p90", "best")},
                                        "graph_nodes": n_nodes, "launches": launches, "kv_length": mid,
-                                       "how": "ggml_backend_graph_compute on libggml-gfx950.so, eager, synchronised per call"}
+                                       "how": "ggml_backend_graph_compute on libggml-gfx950.so, eager, synchronised per call",
+                                       "same_graph_replayed": {"decode_steps_per_s": 1.0 / st_r["mean"], "ms_per_step": {n: st_r[n] * 1e3 for n in ("mean", "median", "p90", "best")},
+                                                               "how": "the identical graph computed repeatedly: the plugin records it at its third run and replays one HIP graph"}}
         assert ref.rh_use_device(b"CPU", threads, 0) == 0
     if ref is not None and with_cpu:
         assert ref.rh_use_device(b"CPU", threads, 0) == 0
@@ -451,6 +458,53 @@ def cfm_solve_bench(pkg, timer, side, threads, with_cpu, layers=4, patch=2, pref
     return res
 
 
+def cfm_requests_bench(pkg, threads, with_cpu, requests=8, layers=4, patch=2, prefix=4, timesteps=10, reps=12):
+    """BASELINE config 3 at its batch: whole UnifiedCFM solves of `requests` concurrent requests (CFG pair each) as ONE
+    ggml graph with the requests in ggml's batch dimension, through the plugin's graph_compute (recorded at its third
+    run, replayed after) and on ggml-cpu."""
+    import reflib
+    ref = reflib.load_ref()
+    if ref is None:
+        return None
+    params = reflib.backbone_params("bench-locdit", 1)
+    lw = params["layers"][0]
+    params["dims"]["n_layer"] = layers
+    params["layers"] = [lw] * layers
+    cp = reflib.cfm_params("bench-cfm")
+    T = 2 * (1 + prefix + patch)
+    rs = np.random.default_rng(12)
+    z, mu = rs.standard_normal((requests, patch, 64)).astype(np.float32), rs.standard_normal((requests, 1024)).astype(np.float32)
+    cond, table = rs.standard_normal((requests, prefix, 64)).astype(np.float32), rs.standard_normal((timesteps, 1024)).astype(np.float32)
+
+    def run(device, n_threads, n):
+        assert ref.rh_use_device(device, n_threads, 0) == 0
+        try:
+            reflib.ref_backbone_create(params, T, requests, use_mup=False, kv_f16=False, fused_weights=True)
+            reflib.ref_cfm_create(cp)
+            _, _, n_nodes = reflib.ref_cfm_solve(z, mu, cond, table, n_steps=timesteps, reps=n)
+            return reflib.ref_last_times(), n_nodes
+        finally:
+            ref.rh_cfm_free()
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", threads, 0) == 0
+
+    assert ref.rh_load_plugin(pkg.PLUGIN_PATH.encode()) == 0
+    times, n_nodes = run(b"GFX950_0", 1, reps)
+    plug = C.CDLL(pkg.PLUGIN_PATH)
+    st = stats(times[3:])   # the first runs are launched group by group while the graph is being recognised
+    res = {"requests": requests, "ms_per_batch_of_solves": {n: st[n] * 1e3 for n in ("mean", "median", "p90", "best")},
+           "us_per_request_solve": st["mean"] / requests * 1e6, "solves_per_s": requests / st["mean"],
+           "first_runs_ms": [t * 1e3 for t in times[:3]], "graph_nodes": n_nodes, "launches": plug.ggml_backend_gfx950_last_launches(),
+           "how": "ONE ggml graph for all requests (batch dimension), ggml_backend_graph_compute on libggml-gfx950.so, synchronised per call; "
+                  "replayed as a recorded HIP graph from the third run"}
+    if with_cpu:
+        ctimes, _ = run(b"CPU", threads, 3)
+        cs = stats(ctimes)
+        res["ggml_cpu"] = {"ms_per_batch_of_solves": cs["mean"] * 1e3, "threads": threads, "sample": "3 repeats of the same graph"}
+        res["speedup_vs_ggml_cpu"] = cs["mean"] / st["mean"]
+    return res
+
+
 def load_peaks():
     lib = C.CDLL(os.path.join(ROOT, "voxcpm.cpp_amd", "lib", "libvx_peaks.so"))
     lib.vxp_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
@@ -498,7 +552,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
-    ap.add_argument("--profile", choices=["decode5", "decode2", "prefill", "prefill1", "backbone", "backbone16", "cfm", "gemm", "peaks"], default=None,
+    ap.add_argument("--profile", choices=["decode5", "decode2", "prefill", "prefill1", "backbone", "backbone16", "cfm", "cfm8", "gemm", "peaks"], default=None,
                     help="run only this workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -546,6 +600,9 @@ def main():
         return
     if args.profile == "cfm":       # config 3: whole CFM solves of one request, replayed from a HIP graph
         print(json.dumps({"profile": "cfg3_cfm_solve_one_request", **cfm_solve_bench(pkg, timer, torch.cuda.Stream(), 1, False)}))
+        return
+    if args.profile == "cfm8":      # config 3 at its batch: 8 requests' solves as one graph through the plugin
+        print(json.dumps({"profile": "cfg3_cfm_solve_8_requests_through_plugin", **cfm_requests_bench(pkg, 1, False)}))
         return
     if args.profile == "backbone":  # config 4 decode steps (f16 cache)
         print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16, kv_f16=True, plugin_reps=5)}))
@@ -631,6 +688,7 @@ def main():
         others["cfg4_backbone_24layers_b2_f16kv"] = backbone_bench(pkg, timer, side, threads, False, kv_f16=True)
         others["cfg3_locdit_stack_8req_x14"] = locdit_stack_bench(pkg, timer, side, threads, cpu_on)
         others["cfg3_cfm_solve_one_request"] = cfm_solve_bench(pkg, timer, side, threads, cpu_on)
+        others["cfg3_cfm_solve_8_requests_through_plugin"] = cfm_requests_bench(pkg, threads, cpu_on)
         # BASELINE config 5 as a whole stack: 8 streams x CFG pair (batch 16), prefill 4096 tokens, decode from 4096 to 8192
         others["cfg5_backbone_24layers_b16_f16kv"] = backbone_bench(pkg, timer, side, threads, cpu_on, batch=16, prefill=4096, steps=4096,
                                                                     kv_f16=True, cpu_reps=3, cpu_prefill=False, plugin_reps=10)

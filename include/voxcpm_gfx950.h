@@ -217,6 +217,10 @@ VX_API vx_status vx_cpy(const vx_tensor * src, const vx_tensor * dst, vx_stream 
 VX_API vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * dst, int dim, vx_stream stream);
 /* GGML_OP_SUM: every element summed in double, rounded once (ops.cpp:1275-1300) */
 VX_API vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+/* GGML_OP_SUM_ROWS: dst[0, i1, i2, i3] = the row's elements summed in double, rounded once
+ * (ggml_compute_forward_sum_rows_f32, ops.cpp:1451-1482, ggml_vec_sum_f32, vec.h:1510-1520) */
+VX_API vx_status vx_sum_rows(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+VX_API int vx_supports_sum_rows(const vx_tensor * src, const vx_tensor * dst);
 /* GGML_OP_ARANGE: dst[i] = start + step * i over a contiguous F32 tensor, the product rounded before the sum
  * (ggml_compute_forward_arange_f32, ops.cpp:7881-7902); the element count is dst's (ggml fixes it at graph build) */
 VX_API vx_status vx_arange(const vx_tensor * dst, float start, float step, vx_stream stream);

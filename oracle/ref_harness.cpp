@@ -614,7 +614,7 @@ void rh_cfm_free(void) {
 // hidden / hidden / feat
 int rh_cfm_create(int feat, const void * in_w, const float * in_b, const void * cond_w, const float * cond_b,
                   const void * out_w, const float * out_b) {
-    if (!g_bb || !g_backend || g_bb->batch != 1) return 100;
+    if (!g_bb || !g_backend) return 100;
     rh_cfm_free();
     cfm_extra * e = new cfm_extra;
     e->feat = feat;
@@ -653,24 +653,30 @@ int rh_cfm_set_time_mlp(int which, const void * w, const float * b) {
     return 0;
 }
 
-// z [feat, patch], mu [hidden], cond [feat, prefix], time_table [hidden, n_steps] (the combined time embedding of every
-// step, as LocDiTModel::precompute_cfg_time_table hands it over), t_span n_steps + 1 values, pair_pos / pair_mask the
-// CFG-pair constants for a branch of 1 + prefix + patch tokens.  out [feat, patch].  seconds: mean, best, node count.
-int rh_cfm_solve(const float * z, const float * mu, const float * cond, const float * time_table, const float * t_span,
-                 int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
-                 int zero_star, float * out, int reps, double * seconds) {
-    if (!g_bb || !g_cfm || !g_backend || n_steps < 1 || prefix < 1) return 100;
+// z [feat, patch, n_req], mu [hidden, n_req], cond [feat, prefix, n_req] (request-major), time_table [hidden, n_steps] (the
+// combined time embedding of every step, as LocDiTModel::precompute_cfg_time_table hands it over; all requests step
+// together), t_span n_steps + 1 values, pair_pos / pair_mask the CFG-pair constants for a branch of 1 + prefix + patch
+// tokens.  out [feat, patch, n_req].  seconds: mean, best, node count.
+// n_req > 1 (the decoder stack must have been made with that batch): the requests ride in dim 2 / as further sequences of
+// the decoder's token dimension -- products, assembly and update are the same nodes over one more dimension, the
+// zero-star sums become SUM_ROWS over each request's values (the reference runs one graph per request,
+// src/voxcpm.cpp:1067-1093; this is how its graph reads with ggml's own batching).
+static int cfm_solve_n(const float * z, const float * mu, const float * cond, const float * time_table, const float * t_span,
+                       int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
+                       int zero_star, int n_req, float * out, int reps, double * seconds) {
+    if (!g_bb || !g_cfm || !g_backend || n_steps < 1 || prefix < 1 || n_req < 1) return 100;
     if (!time_table && !g_cfm->has_time_mlp) return 103;
     const backbone & m = *g_bb;
     const cfm_extra & e = *g_cfm;
-    const int H = m.hidden, F = e.feat, L = 1 + prefix + patch, T = 2 * L;
-    if (T > m.max_len) return 104;
-    const size_t n_nodes = (size_t) n_steps * ((size_t) m.n_layer * 64 + 160) + 128;
+    const int H = m.hidden, F = e.feat, L = 1 + prefix + patch, T = 2 * L, R = n_req;
+    if (T > m.max_len || R != m.batch) return 104;
+    const size_t n_nodes = (size_t) n_steps * ((size_t) m.n_layer * 64 + 192) + 128;
     ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
     ggml_context * c = ggml_init(ip);
-    ggml_tensor * zin  = ggml_new_tensor_2d(c, GGML_TYPE_F32, F, patch);
-    ggml_tensor * muin = ggml_new_tensor_1d(c, GGML_TYPE_F32, H);
-    ggml_tensor * cin  = ggml_new_tensor_2d(c, GGML_TYPE_F32, F, prefix);
+    // (one request: exactly the reference's tensors and nodes)
+    ggml_tensor * zin  = R == 1 ? ggml_new_tensor_2d(c, GGML_TYPE_F32, F, patch) : ggml_new_tensor_3d(c, GGML_TYPE_F32, F, patch, R);
+    ggml_tensor * muin = R == 1 ? ggml_new_tensor_1d(c, GGML_TYPE_F32, H) : ggml_new_tensor_3d(c, GGML_TYPE_F32, H, 1, R);
+    ggml_tensor * cin  = R == 1 ? ggml_new_tensor_2d(c, GGML_TYPE_F32, F, prefix) : ggml_new_tensor_3d(c, GGML_TYPE_F32, F, prefix, R);
     ggml_tensor * tab  = ggml_new_tensor_1d(c, GGML_TYPE_F32, (int64_t) H * n_steps);
     ggml_tensor * pos  = ggml_new_tensor_1d(c, GGML_TYPE_I32, T);
     ggml_tensor * msk  = ggml_new_tensor_2d(c, GGML_TYPE_F16, T, T);
@@ -678,7 +684,7 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
 
     std::vector<ggml_tensor *> roots;
     ggml_tensor * x = zin;
-    ggml_tensor * cond_proj = ggml_add(c, ggml_mul_mat(c, e.w[1], cin), e.b[1]);
+    ggml_tensor * cond_proj = ggml_add(c, ggml_mul_mat(c, e.w[1], cin), e.b[1]); // [H, prefix, R]
     // LocDiTModel::sinusoidal_embedding + timestep_mlp (src/locdit.cpp:186-232)
     auto time_embedding = [&](ggml_tensor * scalar, int mlp) {
         const int   half = H / 2;
@@ -697,25 +703,42 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
         if (zero_star && step <= zero_init_steps) {
             dphi = ggml_scale(c, x, 0.0f);
         } else {
-            ggml_tensor * x_proj   = ggml_add(c, ggml_mul_mat(c, e.w[0], x), e.b[0]);
+            ggml_tensor * x_proj   = ggml_add(c, ggml_mul_mat(c, e.w[0], x), e.b[0]); // [H, patch, R]
             ggml_tensor * combined = time_table ? ggml_view_1d(c, tab, H, (size_t) (step - 1) * H * sizeof(float))
                                                 : ggml_add(c, time_embedding(ggml_arange(c, t, t + 1.0f, 1.0f), 0), delta_zero);
-            ggml_tensor * comb_c   = ggml_reshape_2d(c, ggml_add(c, ggml_reshape_1d(c, combined, H), muin), H, 1);
-            ggml_tensor * comb_u   = ggml_reshape_2d(c, combined, H, 1);
+            ggml_tensor * comb_c, * comb_u;
+            if (R == 1) { // the reference's nodes (src/locdit.cpp:401-452)
+                comb_c = ggml_reshape_2d(c, ggml_add(c, ggml_reshape_1d(c, combined, H), muin), H, 1);
+                comb_u = ggml_reshape_2d(c, combined, H, 1);
+            } else {
+                ggml_tensor * comb1 = ggml_reshape_3d(c, combined, H, 1, 1);
+                comb_c = ggml_add(c, muin, comb1);      // mu of every request + the step's embedding
+                comb_u = ggml_repeat(c, comb1, muin);   // the embedding alone, once per request
+            }
             ggml_tensor * seq_c    = ggml_concat(c, ggml_concat(c, comb_c, cond_proj, 1), x_proj, 1);
             ggml_tensor * seq_u    = ggml_concat(c, ggml_concat(c, comb_u, cond_proj, 1), x_proj, 1);
             ggml_tensor * h        = ggml_concat(c, seq_c, seq_u, 1);
+            if (R > 1) h = ggml_reshape_2d(c, h, H, (int64_t) T * R); // request after request in the decoder's token dimension
             for (const auto & Lr : m.layers) h = bb_layer_forward(c, m, Lr, h, pos, msk, T, 0, false, roots);
             h = bb_norm(c, m, h, m.final_norm);
-            ggml_tensor * hc = ggml_view_2d(c, h, H, patch, h->nb[1], (size_t) (prefix + 1) * h->nb[1]);
-            ggml_tensor * hu = ggml_view_2d(c, h, H, patch, h->nb[1], (size_t) (L + prefix + 1) * h->nb[1]);
-            ggml_tensor * vc = ggml_add(c, ggml_mul_mat(c, e.w[2], hc), e.b[2]);
+            const size_t tok = h->nb[1];
+            ggml_tensor * hc = R == 1 ? ggml_view_2d(c, h, H, patch, tok, (size_t) (prefix + 1) * tok)
+                                      : ggml_view_3d(c, h, H, patch, R, tok, (size_t) T * tok, (size_t) (prefix + 1) * tok);
+            ggml_tensor * hu = R == 1 ? ggml_view_2d(c, h, H, patch, tok, (size_t) (L + prefix + 1) * tok)
+                                      : ggml_view_3d(c, h, H, patch, R, tok, (size_t) T * tok, (size_t) (L + prefix + 1) * tok);
+            ggml_tensor * vc = ggml_add(c, ggml_mul_mat(c, e.w[2], hc), e.b[2]); // [F, patch, R]
             ggml_tensor * vu = ggml_add(c, ggml_mul_mat(c, e.w[2], hu), e.b[2]);
             if (zero_star) {
-                ggml_tensor * dot = ggml_sum(c, ggml_mul(c, vc, vu));
-                ggml_tensor * nrm = ggml_sum(c, ggml_mul(c, vu, vu));
+                ggml_tensor * dot, * nrm;
+                if (R == 1) {
+                    dot = ggml_sum(c, ggml_mul(c, vc, vu));
+                    nrm = ggml_sum(c, ggml_mul(c, vu, vu));
+                } else { // one sum per request
+                    dot = ggml_sum_rows(c, ggml_reshape_2d(c, ggml_mul(c, vc, vu), (int64_t) F * patch, R)); // [1, R]
+                    nrm = ggml_sum_rows(c, ggml_reshape_2d(c, ggml_mul(c, vu, vu), (int64_t) F * patch, R));
+                }
                 ggml_tensor * st  = ggml_div(c, dot, ggml_add(c, nrm, ggml_arange(c, 1.0e-8f, 1.0e-8f + 1.0f, 1.0f)));
-                ggml_tensor * us  = ggml_mul(c, vu, ggml_repeat(c, st, vu));
+                ggml_tensor * us  = ggml_mul(c, vu, ggml_repeat(c, R == 1 ? st : ggml_reshape_3d(c, st, 1, 1, R), vu));
                 dphi = ggml_add(c, us, ggml_scale(c, ggml_sub(c, vc, us), cfg_value));
             } else {
                 dphi = ggml_add(c, vu, ggml_scale(c, ggml_sub(c, vc, vu), cfg_value));
@@ -766,6 +789,17 @@ int rh_cfm_solve(const float * z, const float * mu, const float * cond, const fl
     ggml_gallocr_free(ga);
     ggml_free(c);
     return rc;
+}
+
+int rh_cfm_solve(const float * z, const float * mu, const float * cond, const float * time_table, const float * t_span,
+                 int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
+                 int zero_star, float * out, int reps, double * seconds) {
+    return cfm_solve_n(z, mu, cond, time_table, t_span, n_steps, patch, prefix, pair_pos, pair_mask, cfg_value, zero_star, 1, out, reps, seconds);
+}
+int rh_cfm_solve_requests(const float * z, const float * mu, const float * cond, const float * time_table, const float * t_span,
+                          int n_steps, int patch, int prefix, const int32_t * pair_pos, const uint16_t * pair_mask, float cfg_value,
+                          int zero_star, int n_req, float * out, int reps, double * seconds) {
+    return cfm_solve_n(z, mu, cond, time_table, t_span, n_steps, patch, prefix, pair_pos, pair_mask, cfg_value, zero_star, n_req, out, reps, seconds);
 }
 
 

@@ -187,6 +187,8 @@ def load_ref():
     lib.rh_cfm_create.argtypes = [C.c_int, C.c_void_p, f32p_, C.c_void_p, f32p_, C.c_void_p, f32p_]
     lib.rh_cfm_solve.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int,
                                  f32p_, C.c_int, C.POINTER(C.c_double)]
+    lib.rh_cfm_solve_requests.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int, C.c_int,
+                                          f32p_, C.c_int, C.POINTER(C.c_double)]
     lib.rh_cfm_set_time_mlp.argtypes = [C.c_int, C.c_void_p, f32p_]
     lib.rh_cfm_free.argtypes = []
     lib.rh_cfm_free.restype = None
@@ -434,11 +436,14 @@ def ref_cfm_create(p):
 
 def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_star=True, reps=0):
     """One UnifiedCFM solve as a single graph on the harness's device.  z (patch, feat), mu (hidden,), cond (prefix, feat),
-    table (n_steps, hidden).  Returns (x (patch, feat), seconds[mean, best], n_nodes)."""
+    table (n_steps, hidden).  Returns (x (patch, feat), seconds[mean, best], n_nodes).
+    With a leading request dimension -- z (R, patch, feat), mu (R, hidden), cond (R, prefix, feat) -- the R requests are
+    solved by ONE graph (the decoder stack must have been created with batch R)."""
     lib, orc = load_ref(), load_oracle()
     z, mu, cond = (np.ascontiguousarray(a, dtype=np.float32) for a in (z, mu, cond))
     table = None if table is None else np.ascontiguousarray(table, dtype=np.float32)   # None: the time embeddings are built in the graph
-    patch, prefix = z.shape[0], cond.shape[0]
+    n_req = z.shape[0] if z.ndim == 3 else 1
+    patch, prefix = z.shape[-2], cond.shape[-2]
     L = 1 + prefix + patch
     t_span = np.zeros(n_steps + 1, np.float32)
     orc.orc_t_span(n_steps, sway, ptr(t_span, C.c_float))
@@ -447,9 +452,14 @@ def ref_cfm_solve(z, mu, cond, table, n_steps=10, sway=1.0, cfg_value=2.0, zero_
     orc.orc_cfg_pair_constants(L, ptr(pos, C.c_int32), ptr(mk, C.c_uint16))
     out = np.empty_like(z)
     sec = np.zeros(3, np.float64)
-    rc = lib.rh_cfm_solve(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), None if table is None else ptr(table, C.c_float), ptr(t_span, C.c_float),
-                          n_steps, patch, prefix, ptr(pos, C.c_int32), ptr(mk, C.c_uint16), cfg_value, int(zero_star),
-                          ptr(out, C.c_float), reps, ptr(sec, C.c_double))
+    if z.ndim == 3:
+        rc = lib.rh_cfm_solve_requests(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), None if table is None else ptr(table, C.c_float),
+                                       ptr(t_span, C.c_float), n_steps, patch, prefix, ptr(pos, C.c_int32), ptr(mk, C.c_uint16), cfg_value,
+                                       int(zero_star), n_req, ptr(out, C.c_float), reps, ptr(sec, C.c_double))
+    else:
+        rc = lib.rh_cfm_solve(ptr(z, C.c_float), ptr(mu, C.c_float), ptr(cond, C.c_float), None if table is None else ptr(table, C.c_float), ptr(t_span, C.c_float),
+                              n_steps, patch, prefix, ptr(pos, C.c_int32), ptr(mk, C.c_uint16), cfg_value, int(zero_star),
+                              ptr(out, C.c_float), reps, ptr(sec, C.c_double))
     assert rc == 0, rc
     return out, sec[:2].copy(), int(sec[2])
 

@@ -281,6 +281,51 @@ def test_plugin_runs_the_whole_forward_graph_without_a_scheduler(gpu, ref, T0):
         assert np.array_equal(b, c), i
 
 
+def test_plugin_runs_a_cfm_solve_of_eight_requests(gpu, ref):
+    """BASELINE config 3 at its batch: the CFG pair of 8 concurrent requests, whole UnifiedCFM solves (ten Euler steps,
+    projections, sequence assembly, 4 decoder layers, zero-star guidance, update of x) as ONE graph with the requests in
+    ggml's own batch dimension -- the decoder sees 8 x 14 tokens, the guidance sums are SUM_ROWS over each request.
+    Checked three ways: the plugin against ggml-cpu on the same graph; ggml-cpu's batched graph against eight solves of
+    the reference's single-request graph (the batching changes no request's arithmetic: bit-equal on the CPU); and the
+    plugin's batched result against its own single-request results (each request within the product kernels' own
+    difference between 14 and 112 tokens)."""
+    R = 8
+    params = reflib.backbone_params("locdit", 4)
+    cp = reflib.cfm_params("cfm")
+    z = rng("cfm8", "z").standard_normal((R, 2, 64)).astype(np.float32)
+    mu = rng("cfm8", "mu").standard_normal((R, 1024)).astype(np.float32)
+    cond = rng("cfm8", "cond").standard_normal((R, 4, 64)).astype(np.float32)
+    table = rng("cfm8", "table").standard_normal((10, 1024)).astype(np.float32)
+
+    def run(device, batch, reps=0):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        try:
+            reflib.ref_backbone_create(params, 32, batch, use_mup=True, kv_f16=False, fused_weights=True)
+            reflib.ref_cfm_create(cp)
+            if batch == R:
+                return reflib.ref_cfm_solve(z, mu, cond, table, reps=reps)
+            return np.stack([reflib.ref_cfm_solve(z[r], mu[r], cond[r], table)[0] for r in range(R)]), None, None
+        finally:
+            ref.rh_cfm_free()
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+
+    cpu8, cpu_s, n_nodes = run(b"CPU", R, reps=2)
+    cpu1 = run(b"CPU", 1)[0]
+    assert np.isfinite(cpu8).all() and np.abs(cpu8 - z).max() > 1e-2
+    assert np.array_equal(cpu8, cpu1), np.abs(cpu8 - cpu1).max()        # batching leaves every request's arithmetic alone
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug8, plug_s, _ = run(b"GFX950_0", R, reps=6)
+    import ctypes
+    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    plug1 = run(b"GFX950_0", 1)[0]
+    e8, e1, e81 = nmse(cpu8, plug8), nmse(cpu1, plug1), nmse(plug1, plug8)
+    print(f"CFM solve of {R} requests, 10 steps: {n_nodes} graph nodes, {launches} launches on the plugin; nmse vs ggml-cpu {e8:.3e} "
+          f"(single-request graphs {e1:.3e}), batched vs single on the plugin {e81:.3e}; ggml-cpu (8 threads) {cpu_s[1] * 1e3:.2f} ms, "
+          f"plugin {plug_s[1] * 1e3:.3f} ms per {R} solves", flush=True)
+    assert e8 <= 1e-3 and e1 <= 1e-3 and e81 <= 1e-3
+
+
 @pytest.mark.parametrize("time_table", [True, False])
 def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref, time_table):
     """BASELINE config 3 as the reference builds it (src/unified_cfm.cpp:88-184 around src/locdit.cpp:401-464): ten

@@ -56,7 +56,7 @@ EXPORTS = [
     "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_flash_attn_ext_static", "vx_mul_mat",
     "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
     "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
-    "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum",
+    "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum", "vx_sum_rows", "vx_supports_sum_rows",
     "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
     "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
@@ -127,6 +127,8 @@ def lib():
     l.vx_cpy.argtypes = [TP, TP, vp]
     l.vx_concat.argtypes = [TP, TP, TP, C.c_int, vp]
     l.vx_sum.argtypes = [TP, TP, vp]
+    l.vx_sum_rows.argtypes = [TP, TP, vp]
+    l.vx_supports_sum_rows.argtypes = [TP, TP]
     l.vx_supports_binary.argtypes = [C.c_int, TP, TP, TP]
     l.vx_supports_add1.argtypes = [TP, TP, TP]
     l.vx_supports_unary_like.argtypes = [TP, TP]

@@ -1288,6 +1288,35 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
     return VX_OK;
 }
 
+// ---- GGML_OP_SUM_ROWS: one wave per row ---------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(64) void sum_rows_kernel(const char * src, vx_dims s, char * dst, vx_dims d) {
+    const uint32_t row = blockIdx.x;
+    const uint32_t i1 = row % (uint32_t) s.ne[1], r2 = row / (uint32_t) s.ne[1], i2 = r2 % (uint32_t) s.ne[2], i3 = r2 / (uint32_t) s.ne[2];
+    const float * x = (const float *) (src + i1 * s.nb[1] + i2 * s.nb[2] + i3 * s.nb[3]);
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < s.ne[0]; i += 64) acc += (double) x[i];
+    acc = vx_wave_sum(acc);
+    if (threadIdx.x == 0) *(float *) (dst + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]) = (float) acc;
+}
+} // namespace
+
+extern "C" int vx_supports_sum_rows(const vx_tensor * src, const vx_tensor * dst) {
+    if (!f32(src) || !f32(dst) || !vx_positive(src)) return 0;
+    if (dst->ne[0] != 1 || dst->ne[1] != src->ne[1] || dst->ne[2] != src->ne[2] || dst->ne[3] != src->ne[3]) return 0;
+    if (src->nb[0] != 4 || !nb_multiple(src, 4) || !nb_multiple(dst, 4)) return 0;
+    return src->ne[1] * src->ne[2] * src->ne[3] <= 0x7fffffff;
+}
+
+extern "C" vx_status vx_sum_rows(const vx_tensor * src, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_sum_rows(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "sum_rows: F32 rows (nb0 == 4) to an F32 tensor of one element per row");
+    if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "sum_rows: null data");
+    const int64_t rows = src->ne[1] * src->ne[2] * src->ne[3];
+    sum_rows_kernel<<<dim3((unsigned) rows), dim3(64), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (char *) dst->data, vx_dims_of(dst));
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
 extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                          const vx_tensor * x, const vx_tensor * dst) {
     if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;

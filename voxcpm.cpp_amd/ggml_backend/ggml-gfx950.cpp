@@ -320,6 +320,10 @@ bool supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
             return vx_supports_sum(&a, &d) != 0;
         }
+        case GGML_OP_SUM_ROWS: {
+            const vx_tensor a = to_vx(op->src[0]), d = to_vx(op);
+            return vx_supports_sum_rows(&a, &d) != 0;
+        }
         case GGML_OP_SQR:
         case GGML_OP_SQRT:
         case GGML_OP_LOG:
@@ -390,6 +394,10 @@ vx_status compute_node(backend_ctx * ctx, ggml_tensor * node) {
         case GGML_OP_SUM: {
             const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
             return vx_sum(&a, &d, ctx->stream);
+        }
+        case GGML_OP_SUM_ROWS: {
+            const vx_tensor a = to_vx(node->src[0]), d = to_vx(node);
+            return vx_sum_rows(&a, &d, ctx->stream);
         }
         case GGML_OP_SQR:
         case GGML_OP_SQRT:
