@@ -222,6 +222,27 @@ def test_kv_store_sync_limits(pkg, gpu):
     assert L.vx_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x), 0.0, 0.0, None) != 0
 
 
+@pytest.mark.parametrize("shape", [(8, 128), (1, 1), (3, 5, 7, 1000), (2, 4100), (16, 2, 64)])
+def test_sum_rows_matches_ggml_cpu_arithmetic(gpu, shape):
+    """GGML_OP_SUM_ROWS (ggml_compute_forward_sum_rows_f32, ops.cpp:1451-1482): a row's elements added in double and
+    rounded once.  Checked against numpy's float64 row sums rounded to float32 (bit-equal whenever the double sum is
+    exact, which it is for these magnitudes up to the order of the additions: at most one float32 ulp otherwise), on
+    dense tensors and on a strided view."""
+    say(f"sum_rows {shape}")
+    x = rng("sumrows", shape).standard_normal(shape).astype(np.float32)
+    import torch
+    sync_np = lambda t: (torch.cuda.synchronize(), t.cpu().numpy())[1]
+    got = sync_np(gpu.sum_rows(dev(x)))
+    want = x.astype(np.float64).sum(axis=-1, keepdims=True).astype(np.float32)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= np.spacing(np.abs(want).max())
+    if len(shape) >= 2 and shape[-2] > 1:   # rows of a view: every second row
+        xv = dev(x)[..., ::2, :]
+        got = sync_np(gpu.sum_rows(xv))
+        want = x[..., ::2, :].astype(np.float64).sum(axis=-1, keepdims=True).astype(np.float32)
+        assert np.abs(got - want).max() <= np.spacing(np.abs(want).max())
+
+
 @pytest.mark.parametrize("shape", [(2, 512, 2, 64), (3, 70000), (1, 20000)])
 def test_sum_large_matches_fp64(pkg, gpu, shape):
     import torch

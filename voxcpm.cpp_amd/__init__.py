@@ -401,6 +401,14 @@ def small_graph(nodes):
     check(lib().vx_small_graph(arr, len(nodes), _stream()), "vx_small_graph")
 
 
+def sum_rows(a, out=None):
+    """GGML_OP_SUM_ROWS: every row (the innermost dimension) of an F32 tensor summed; shape (..., 1)."""
+    import torch
+    out = torch.empty(tuple(a.shape[:-1]) + (1,), dtype=torch.float32, device=a.device) if out is None else out
+    check(lib().vx_sum_rows(desc(a), desc(out), _stream()), "vx_sum_rows")
+    return out
+
+
 def sum_all(a, out=None):
     import torch
     out = torch.empty((1,), dtype=torch.float32, device=a.device) if out is None else out
