@@ -331,7 +331,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         st = stats(reflib.ref_last_times())
         launches = plug.ggml_backend_gfx950_last_launches()
         plug.ggml_backend_gfx950_set_graph_replay(1)   # the same graph again and again (what a fixed-length step would be): recorded, then replayed
-        reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps)
+        reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps + 3)   # three runs until the replay is in place
         st_r = stats(reflib.ref_last_times()[3:])
         ref.rh_bb_free()
         res["plugin_graph_compute"] = {"decode_steps_per_s": 1.0 / st["mean"], "ms_per_step": {n: st[n] * 1e3 for n in ("mean", "median", "p90", "best")},

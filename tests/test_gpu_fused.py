@@ -123,7 +123,7 @@ def test_mul_mat_swiglu(pkg, gpu, M, K, N, nb, act):
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 4096, 40, 2)])
+@pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 2048, 40, 2)])
 @pytest.mark.parametrize("act", ["float", "q8"])
 def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     import torch
@@ -155,6 +155,11 @@ def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     rl = torch.zeros((1, 1, nbig, M), dtype=torch.float32, device="cuda")
     assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl)) == 0
     assert L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl), 1.0, mode, None) != 0
+    # so are several chunks of tokens over a long K (they belong to the tiled kernel)
+    if K > 2048:
+        x17 = dev(np.zeros((1, 1, 17, K), dtype=np.float32))
+        r17 = torch.zeros((1, 1, 17, M), dtype=torch.float32, device="cuda")
+        assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(x17), d(r17), d(r17)) == 0
 
 
 @pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2)])

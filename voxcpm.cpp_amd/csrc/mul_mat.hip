@@ -1010,6 +1010,9 @@ bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
     static const int64_t max_tokens = [] { const char * e = getenv("VX_GEMV_MAX_TOKENS"); const int n = e ? atoi(e) : 0; return n >= 16 ? (int64_t) n : (int64_t) 1 << 30; }();
     if (K % 32 || K < 32 || N < 1) return false;
     if (N > 16 && (N > max_tokens || N * rows > 256 * 1024)) return false;
+    // chunks of 16 tokens each stage 16 x K activations: with a long K a work-group fills a CU's LDS alone and the chunks
+    // queue up behind each other (1024 rows x K = 4096 at 112 tokens: 63 us against 26 us on the tiled kernel with its K cut)
+    if (N > 16 && K > 2048) return false;
     const size_t nl = (size_t) (N < 16 ? N : 16);
     return nl * K * 2 + nl * (K / 32) * 4 + 15 * 64 * 16 + 16 * sizeof(float) + GV_ROPE_LDS <= GV_MAX_LDS;
 }
@@ -1111,7 +1114,7 @@ int gemv_waves_for(int64_t K, int64_t tokens, int64_t M) {
     const int bpw = tokens <= 16 ? 4 : GV_UNROLL; // blocks per wave aimed at
     while (nw < 16 && nkb > (int64_t) nw * bpw) nw *= 2;
     static const int many = [] { const char * e = getenv("VX_GEMV_MANY_TOKENS"); return e ? atoi(e) : 5; }();
-    if (tokens >= many && tokens <= 16 && nkb >= 16 && M <= 2048) nw = 16; // one chunk of tokens; several chunks multiply the waves instead
+    if (tokens >= many && nkb >= 16 && M <= 2048) nw = 16; // (also with several chunks of tokens: every chunk has its 16 tokens of norm, staging and angles)
     return nw;
 }
 
