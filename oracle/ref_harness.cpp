@@ -578,6 +578,99 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     return rc;
 }
 
+// ---- two dependent stages, with and without a trip through the host -----------------------------------------
+// The reference's decode step runs the base LM's step graph, fetches its hidden state to the host, adds the step's
+// embedding there and uploads the sum as the input of the residual LM's step graph (src/voxcpm.cpp:1067-1093): two
+// synchronous copies and a host loop between two graphs.  resident = 0 does exactly that with two forward graphs of the
+// stack made by rh_bb_create (T tokens, no cache): out = forward(forward(x) + x).  resident = 1 keeps everything on
+// the backend's device: the input and the first stage's result live in tensors of a persistent backend buffer (like
+// the KV cache does), the first graph ends in a CPY into that state, the second graph begins with the ADD -- no
+// tensor_get / tensor_set between the stages, one synchronisation at the end.  Same nodes, same arithmetic: the two
+// variants must agree bit for bit.  seconds: mean and best wall time of one two-stage step (uploads of x included in
+// both variants), repeats >= 1.
+int rh_bb_two_stage(const float * x, const uint16_t * mask, int n_tokens, int resident, float * out, int reps, double * seconds) {
+    if (!g_bb || !g_backend || reps < 1) return 100;
+    const backbone & m = *g_bb;
+    const int T = n_tokens, B = m.batch;
+    if (T > m.max_len) return 104;
+    const int64_t n_tok = (int64_t) T * B;
+    const size_t n_nodes = (size_t) m.n_layer * 64 + 64;
+    // persistent state on the device: the step's input and the first stage's hidden state
+    ggml_init_params sp = { ggml_tensor_overhead() * 8, nullptr, true };
+    ggml_context * sc = ggml_init(sp);
+    ggml_tensor * x_dev = ggml_new_tensor_2d(sc, GGML_TYPE_F32, m.hidden, n_tok);
+    ggml_tensor * h_dev = ggml_new_tensor_2d(sc, GGML_TYPE_F32, m.hidden, n_tok);
+    ggml_tensor * pos_d = ggml_new_tensor_1d(sc, GGML_TYPE_I32, T);
+    ggml_tensor * msk_d = mask ? ggml_new_tensor_2d(sc, GGML_TYPE_F16, T, T) : nullptr;
+    ggml_backend_buffer_t sbuf = ggml_backend_alloc_ctx_tensors(sc, g_backend);
+    if (!sbuf) { ggml_free(sc); return 101; }
+    std::vector<int32_t> p((size_t) T);
+    for (int i = 0; i < T; ++i) p[(size_t) i] = i;
+    ggml_backend_tensor_set(pos_d, p.data(), 0, ggml_nbytes(pos_d));
+    if (msk_d) ggml_backend_tensor_set(msk_d, mask, 0, ggml_nbytes(msk_d));
+
+    struct stage { ggml_context * c = nullptr; ggml_cgraph * g = nullptr; ggml_gallocr_t ga = nullptr; ggml_tensor * in = nullptr, * out = nullptr; };
+    auto build = [&](int which) {
+        stage st;
+        ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
+        st.c = ggml_init(ip);
+        ggml_tensor * h;
+        if (resident) {
+            h = which == 0 ? x_dev : ggml_add(st.c, h_dev, x_dev);
+        } else {
+            st.in = ggml_new_tensor_2d(st.c, GGML_TYPE_F32, m.hidden, n_tok);
+            ggml_set_input(st.in);
+            h = st.in;
+        }
+        std::vector<ggml_tensor *> roots;
+        for (const auto & L : m.layers) h = bb_layer_forward(st.c, m, L, h, pos_d, msk_d, T, 0, false, roots);
+        h = bb_norm(st.c, m, h, m.final_norm);
+        if (resident && which == 0) h = ggml_cpy(st.c, h, h_dev); // the state the next stage reads
+        ggml_set_output(h);
+        st.out = h;
+        st.g = ggml_new_graph_custom(st.c, n_nodes, false);
+        ggml_build_forward_expand(st.g, h);
+        st.ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend));
+        return st;
+    };
+    stage s0 = build(0), s1 = build(1);
+    int rc = 0;
+    if (!ggml_gallocr_alloc_graph(s0.ga, s0.g) || !ggml_gallocr_alloc_graph(s1.ga, s1.g)) rc = 101;
+    const size_t nbytes = (size_t) n_tok * m.hidden * sizeof(float);
+    std::vector<float> h1((size_t) n_tok * m.hidden), r((size_t) n_tok * m.hidden);
+    double best = 1e30, total = 0;
+    for (int it = 0; it < reps + 1 && !rc; ++it) { // the first pass is a warm-up
+        auto t0 = std::chrono::steady_clock::now();
+        if (resident) {
+            ggml_backend_tensor_set(x_dev, x, 0, nbytes);
+            if (ggml_backend_graph_compute_async(g_backend, s0.g) != GGML_STATUS_SUCCESS) rc = 102;
+            if (!rc && ggml_backend_graph_compute_async(g_backend, s1.g) != GGML_STATUS_SUCCESS) rc = 102;
+            if (!rc) ggml_backend_tensor_get(s1.out, out, 0, nbytes); // synchronises
+        } else {
+            ggml_backend_tensor_set(s0.in, x, 0, nbytes);
+            if (ggml_backend_graph_compute(g_backend, s0.g) != GGML_STATUS_SUCCESS) rc = 102;
+            if (!rc) {
+                ggml_backend_tensor_get(s0.out, h1.data(), 0, nbytes);
+                for (size_t i = 0; i < r.size(); ++i) r[i] = h1[i] + x[i];
+                ggml_backend_tensor_set(s1.in, r.data(), 0, nbytes);
+                if (ggml_backend_graph_compute(g_backend, s1.g) != GGML_STATUS_SUCCESS) rc = 102;
+            }
+            if (!rc) ggml_backend_tensor_get(s1.out, out, 0, nbytes);
+        }
+        auto t1 = std::chrono::steady_clock::now();
+        if (it > 0) {
+            const double d = std::chrono::duration<double>(t1 - t0).count();
+            total += d;
+            if (d < best) best = d;
+        }
+    }
+    if (seconds) { seconds[0] = total / reps; seconds[1] = best; }
+    for (stage * st : { &s0, &s1 }) { ggml_gallocr_free(st->ga); ggml_free(st->c); }
+    ggml_backend_buffer_free(sbuf);
+    ggml_free(sc);
+    return rc;
+}
+
 // ---- a whole CFM solve as one graph ---------------------------------------------------------------------------
 // The graph UnifiedCFM::forward builds (src/unified_cfm.cpp:88-184) around the LocDiT estimator's CFG-pair pass
 // (src/locdit.cpp:248-258, 401-464): per Euler step the noisy patches are projected to the hidden size, the

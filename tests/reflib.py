@@ -187,6 +187,7 @@ def load_ref():
     lib.rh_cfm_create.argtypes = [C.c_int, C.c_void_p, f32p_, C.c_void_p, f32p_, C.c_void_p, f32p_]
     lib.rh_cfm_solve.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int,
                                  f32p_, C.c_int, C.POINTER(C.c_double)]
+    lib.rh_bb_two_stage.argtypes = [f32p_, u16p_, C.c_int, C.c_int, f32p_, C.c_int, C.POINTER(C.c_double)]
     lib.rh_cfm_solve_requests.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int, C.c_int,
                                           f32p_, C.c_int, C.POINTER(C.c_double)]
     lib.rh_cfm_set_time_mlp.argtypes = [C.c_int, C.c_void_p, f32p_]
@@ -419,6 +420,22 @@ def cfm_params(tag, feat=64, hidden=1024):
             # time_mlp linear1 / linear2, delta_time_mlp linear1 / linear2 (src/locdit.cpp:213-246)
             "time_w": [(g("time_w", i).standard_normal((hidden, hidden)) / np.sqrt(hidden)).astype(np.float32) for i in range(4)],
             "time_b": [(0.1 * g("time_b", i).standard_normal(hidden)).astype(np.float32) for i in range(4)]}
+
+
+def ref_backbone_two_stage(x, mask, resident, reps=1):
+    """out = forward(forward(x) + x) on the stack made by ref_backbone_create, as two graphs: with the first stage's
+    result fetched, added on the host and uploaded again (resident=False, the reference's decode step,
+    src/voxcpm.cpp:1067-1093) or kept in a persistent device tensor (resident=True).  x (batch, T, hidden).
+    Returns (out, seconds[mean, best])."""
+    lib = load_ref()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    sec = np.zeros(2, np.float64)
+    m = None if mask is None else np.ascontiguousarray(mask).view(np.uint16)
+    rc = lib.rh_bb_two_stage(ptr(x, C.c_float), None if m is None else ptr(m, C.c_uint16), x.shape[1], int(resident),
+                             ptr(out, C.c_float), reps, ptr(sec, C.c_double))
+    assert rc == 0, rc
+    return out, sec
 
 
 def ref_cfm_create(p):

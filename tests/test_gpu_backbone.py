@@ -282,6 +282,39 @@ def test_plugin_runs_the_whole_forward_graph_without_a_scheduler(gpu, ref, T0):
         assert np.array_equal(b, c), i
 
 
+@pytest.mark.parametrize("T", [1, 9])
+def test_plugin_keeps_state_on_the_device_between_two_graphs(gpu, ref, T):
+    """Two dependent stages as the reference's decode step has them (base LM step, then the residual LM step on its
+    hidden state plus the step's embedding, src/voxcpm.cpp:1067-1093): with the state fetched, added on the host and
+    uploaded again between the graphs, and with the state in a persistent tensor of the backend's buffer (the second
+    graph begins with the ADD, nothing crosses the bus between the stages).  Same nodes, same arithmetic: bit-equal on
+    ggml-cpu and on the plugin; the plugin against ggml-cpu within the stack's bar."""
+    params = reflib.backbone_params("bb", N_LAYER)
+    x = rng("two-stage", T).standard_normal((BATCH, T, 1024)).astype(np.float32)
+    mask = reflib.causal_mask(T, T)
+
+    def run(device):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        try:
+            reflib.ref_backbone_create(params, T + 4, BATCH, use_mup=True, kv_f16=False)
+            host, host_s = reflib.ref_backbone_two_stage(x, mask, False, reps=5)
+            dev_, dev_s = reflib.ref_backbone_two_stage(x, mask, True, reps=5)
+        finally:
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return host, dev_, host_s, dev_s
+
+    c_host, c_dev, _, _ = run(b"CPU")
+    assert np.isfinite(c_host).all() and np.array_equal(c_host, c_dev)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    g_host, g_dev, hs, ds = run(b"GFX950_0")
+    assert np.array_equal(g_host, g_dev)
+    e = nmse(c_host, g_dev)
+    print(f"two stages of {N_LAYER} layers, T={T}: host round trip {hs[1] * 1e6:.0f} us, state on the device {ds[1] * 1e6:.0f} us per step "
+          f"(best of 5); nmse vs ggml-cpu {e:.3e}", flush=True)
+    assert e <= 1e-4
+
+
 def test_plugin_runs_a_cfm_solve_of_eight_requests(gpu, ref):
     """BASELINE config 3 at its batch: the CFG pair of 8 concurrent requests, whole UnifiedCFM solves (ten Euler steps,
     projections, sequence assembly, 4 decoder layers, zero-star guidance, update of x) as ONE graph with the requests in
