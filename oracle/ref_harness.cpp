@@ -645,7 +645,10 @@ int rh_bb_two_stage(const float * x, const uint16_t * mask, int n_tokens, int re
             ggml_backend_tensor_set(x_dev, x, 0, nbytes);
             if (ggml_backend_graph_compute_async(g_backend, s0.g) != GGML_STATUS_SUCCESS) rc = 102;
             if (!rc && ggml_backend_graph_compute_async(g_backend, s1.g) != GGML_STATUS_SUCCESS) rc = 102;
-            if (!rc) ggml_backend_tensor_get(s1.out, out, 0, nbytes); // synchronises
+            if (!rc) { // buffer transfers are not ordered behind a backend's asynchronous work: wait for it first
+                ggml_backend_synchronize(g_backend);
+                ggml_backend_tensor_get(s1.out, out, 0, nbytes);
+            }
         } else {
             ggml_backend_tensor_set(s0.in, x, 0, nbytes);
             if (ggml_backend_graph_compute(g_backend, s0.g) != GGML_STATUS_SUCCESS) rc = 102;

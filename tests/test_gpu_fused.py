@@ -737,6 +737,64 @@ def test_small_graph_sequence_assembly_copies_and_sums(gpu):
     assert np.array_equal(got["tile"].cpu().numpy(), np.tile(t["seed"], (3, 1, 4, 1)))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [64, 1001, 2700])
+@pytest.mark.parametrize("private", [False, True])
+def test_small_graph_dense_runs_barriers_and_wide_moves(gpu, n, private):
+    """Runs of dense F32 nodes take the kernel that the host has resolved every operand for: operands the run only reads
+    are in LDS before the first node, a node whose inputs were written by the reading thread itself meets no barrier,
+    plain moves go 16 bytes per thread.  The cases that tests: rows longer than the work-group (several elements per
+    thread), a value broadcast from a sum of the same run, an image rewritten in place after other threads read it,
+    concatenations with and without 16-byte alignment, intermediates with and without memory behind them."""
+    import torch
+    say(f"small graph: dense run n={n} private={private}")
+    N = gpu
+    t = {"a": rng("sgd", "a", n).standard_normal((3, n)).astype(np.float32), "b": rng("sgd", "b", n).standard_normal((3, n)).astype(np.float32),
+         "row": rng("sgd", "r", n).standard_normal((1, n)).astype(np.float32)}
+    for name in ("p", "q", "r", "u", "out"):
+        t[name] = np.zeros((3, n), np.float32)
+    for name in ("s", "s2"):
+        t[name] = np.zeros((1,), np.float32)
+    t["cat"] = np.zeros((6, n), np.float32); t["cat1"] = np.zeros((4, n), np.float32)
+    t["flat"] = np.zeros((3 * n,), np.float32); t["shift"] = np.zeros((3 * n + 3,), np.float32)
+    t["three"] = np.array([1.0, 2.0, 3.0], np.float32)
+    prog = [(N.NODE_MUL, "p", "a", "b", 0, 0, 0), (N.NODE_UNARY, "q", "p", None, N.UNARY_SILU, 0, 0),       # q from p: own elements
+            (N.NODE_SUM, "s", "q", None, 0, 0, 0),                                                        # reads across threads
+            (N.NODE_ADD1, "r", "q", "s", 0, 0, 0),                                                        # broadcast of the run's own scalar
+            (N.NODE_SCALE, "q", "r", None, 0, 0.5, -1.0),                                                 # q rewritten after the sum read it
+            (N.NODE_SUM, "s2", "q", None, 0, 0, 0), (N.NODE_DIV, "s2", "s2", "s", 0, 0, 0),               # scalars stay with thread 0
+            (N.NODE_REPEAT, "u", "s2", None, 0, 0, 0), (N.NODE_SUB, "u", "u", "q", 0, 0, 0),
+            (N.NODE_CONCAT, "cat", "u", "a", 1, 0, 0),                                                    # whole quads when n % 4 == 0
+            (N.NODE_CONCAT, "cat1", "row", "r", 1, 0, 0),
+            (N.NODE_CPY, "flat", "u", None, 0, 0, 0), (N.NODE_CONCAT, "shift", "three", "flat", 0, 0, 0),   # 3 elements first: no quads
+            (N.NODE_CPY, "out", "u", None, 0, 0, 0), (N.NODE_ADD, "out", "out", "r", 0, 0, 0)]
+    keep = {"out", "cat", "cat1", "s2", "shift"} if private else None
+    sets = []
+    for mode in ("separate", "one launch"):
+        T = {k: dev(v) for k, v in t.items()}
+        if mode == "separate":
+            for op, dst, s0, s1, aux, p0, p1 in prog:
+                d, a, b = T[dst], (None if s0 is None else T[s0]), (None if s1 is None else T[s1])
+                if op <= N.NODE_DIV: N.binary(op, a, b, out=d)
+                elif op == N.NODE_ADD1: N.add1(a, b, out=d)
+                elif op == N.NODE_SCALE: N.scale(a, p0, p1, out=d)
+                elif op == N.NODE_UNARY: N.unary(aux, a, out=d)
+                elif op == N.NODE_CPY: N.cpy(a, d)
+                elif op == N.NODE_CONCAT: N.concat(a, b, aux, out=d)
+                elif op == N.NODE_REPEAT: N.repeat(a, None, out=d)
+                else: N.sum_all(a, out=d)
+        else:
+            last = {dst: i for i, (_, dst, *_r) in enumerate(prog)}
+            nodes = [N.small_node(op, T[dst], None if s0 is None else T[s0], None if s1 is None else T[s1], aux, p0, p1,
+                                  private=bool(private and not (dst in keep and last[dst] == i)))
+                     for i, (op, dst, s0, s1, aux, p0, p1) in enumerate(prog)]
+            N.small_graph(nodes)
+        torch.cuda.synchronize()
+        sets.append(T if keep is None else {k: T[k] for k in keep})
+    _assert_same(sets, f"dense n={n} private={private}")
+    assert float(sets[1]["out"].abs().sum()) > 0
+
+
 def test_small_graph_limits(gpu, pkg):
     """What a run may hold: at most 16 nodes, tensors of at most 16384 elements, only the tiny operators."""
     import torch

@@ -452,10 +452,39 @@ struct sg_node {
     sg_shape sh[3];      // shapes and strides of operand 0, operand 1, destination (the indexed forms)
 };
 constexpr int SG_HEAD_DWORDS = (int) (offsetof(sg_node, sh) / 4);
+// Operands that the run only reads (dense 4-byte tensors that no node of the run writes) are brought into LDS images
+// before the first node, all loads in flight together: read where they are used, each would cost the run a trip to
+// memory of its own, one behind the other.
+constexpr int SG_MAX_PRELOADS = 8;
+struct sg_preload {
+    const uint32_t * p;
+    uint32_t         n;   // elements
+    int32_t          lds; // first slot of the image
+};
+struct sg_head {
+    int32_t    n, n_pre;
+    uint32_t   pre_most, pad; // the largest preloaded tensor's elements
+    sg_preload pre[SG_MAX_PRELOADS];
+};
 struct sg_args {
-    int32_t n, pad[3];
+    sg_head h;
     sg_node node[SG_MAX_NODES];
 };
+
+// every thread of the work-group; the caller's next barrier publishes the images
+__device__ __forceinline__ void sg_preload_images(const sg_head & h, uint32_t * lds) {
+    const uint32_t nt = blockDim.x;
+    for (uint32_t base = 0; base < h.pre_most; base += nt) {
+        const uint32_t e = base + threadIdx.x;
+        uint32_t v[SG_MAX_PRELOADS];
+#pragma unroll
+        for (int i = 0; i < SG_MAX_PRELOADS; ++i)
+            if (i < h.n_pre && e < h.pre[i].n) v[i] = h.pre[i].p[e];
+#pragma unroll
+        for (int i = 0; i < SG_MAX_PRELOADS; ++i)
+            if (i < h.n_pre && e < h.pre[i].n) lds[h.pre[i].lds + e] = v[i];
+    }
+}
 
 __device__ __forceinline__ void sg_index(const sg_tensor & t, uint32_t e, uint32_t (&i)[4]) {
     i[0] = e % (uint32_t) t.ne[0]; e /= (uint32_t) t.ne[0];
@@ -525,12 +554,13 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
     {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         static_assert(sizeof(sg_args) % 16 == 0 && sizeof(sg_args) <= 256 * 16, "16 bytes per thread of the smallest work-group");
-        const uint32_t quads = (uint32_t) (offsetof(sg_args, node) + (size_t) a0.n * sizeof(sg_node) + 15) / 16;
+        const uint32_t quads = (uint32_t) (offsetof(sg_args, node) + (size_t) a0.h.n * sizeof(sg_node) + 15) / 16;
         if (threadIdx.x < quads) ((u32x4 *) table)[threadIdx.x] = ((const u32x4 *) &a0)[threadIdx.x]; // one trip to memory for the whole table
     }
+    sg_preload_images(a0.h, lds);
     __syncthreads();
     const uint32_t nt = blockDim.x; // the host sizes the work-group to the run: a run of 128-element nodes is two waves' work
-    const int n_nodes = a0.n;
+    const int n_nodes = a0.h.n;
     // a node's head is read from the table one node ahead, so that its LDS latency passes under the node before it
     uint32_t head[SG_HEAD_DWORDS];
     auto read_head = [&](int k) {
@@ -736,6 +766,120 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
                 break;
             default: break;
         }
+    }
+}
+
+// ---- the same run when every node is dense F32 -----------------------------------------------------------
+// The interpreter above pays for its generality in instructions: ≈ 360 per node and wave for a chain of 128-element
+// nodes, at the 4 cycles a wave needs per instruction.  When every node of a run is a dense F32 operator (element e of the
+// destination from element e, or the only element, of each operand; a CONCAT along the outermost dimension; a sum in the
+// one-wave order) the host resolves everything else beforehand into 16 dwords per node -- operator code, counts, where
+// each operand lies (its LDS image or a global address) -- and the kernel only scalarises them (read one node ahead),
+// meets the barrier and runs a loop of a handful of instructions.  Same device functions, same orders, same bits.
+enum sgd_code : uint32_t { SGD_ADD = 0, SGD_SUB, SGD_MUL, SGD_DIV, SGD_ADD1, SGD_SCALE, SGD_UNARY, SGD_COPY, SGD_CONCAT, SGD_SUM4, SGD_SUM1, SGD_ARANGE,
+                           SGD_COPY4, SGD_CONCAT4 }; // the last two: 16 bytes per thread, counts in quads
+// SGD_NO_BARRIER: every value this node reads from an image written since the last barrier was written by the reading
+// thread itself (element e of a dense node is always thread e mod work-group size), and its destination is a fresh image
+constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8;
+struct sgd_op {
+    uint32_t code, n, n0, flags; // n: destination elements (SUM: units of the source); n0: CONCAT's first operand
+    float    p0, p1;
+    int32_t  s0_lds, s1_lds, d_lds, aux; // first LDS slot of the operand's image, or -1 (then the global address below)
+    const float * s0, * s1;
+    float *       d;              // null: a private destination that lives in its image only
+};
+static_assert(sizeof(sgd_op) == 64, "16 dwords per node");
+struct sgd_args {
+    sg_head h;
+    sgd_op  op[SG_MAX_NODES];
+};
+
+__global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args a0) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[]; // the images
+    __shared__ u32x4 table[sizeof(sgd_args) / 16];
+    static_assert(sizeof(sgd_args) % 16 == 0 && sizeof(sgd_args) / 16 <= 256, "16 bytes per thread of the smallest work-group");
+    const int n_nodes = a0.h.n;
+    constexpr int OPS_AT = (int) (offsetof(sgd_args, op) / 16);
+    static_assert(offsetof(sgd_args, op) % 16 == 0, "nodes on 16-byte boundaries");
+    if (threadIdx.x < OPS_AT + 4 * (uint32_t) n_nodes) table[threadIdx.x] = ((const u32x4 *) &a0)[threadIdx.x]; // one trip for the whole table
+    sg_preload_images(a0.h, lds);
+    __syncthreads();
+    const uint32_t nt = blockDim.x;
+    const float *  ldsf = (const float *) lds;
+    u32x4 nx[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) nx[q] = table[OPS_AT + q];
+    for (int k = 0; k < n_nodes; ++k) { // uniform: every thread walks every node and meets every barrier
+        sgd_op op;
+        {
+            uint32_t * w = (uint32_t *) &op;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w[4 * q + i] = (uint32_t) __builtin_amdgcn_readfirstlane((int) nx[q][i]);
+        }
+        if (k + 1 < n_nodes) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) nx[q] = table[OPS_AT + 4 * (k + 1) + q];
+        }
+        if (k > 0 && !(op.flags & SGD_NO_BARRIER)) {
+            if (op.flags & SGD_WAIT_MEMORY) {
+                __syncthreads(); // earlier nodes' stores to memory are complete and visible to the work-group
+            } else {             // only the LDS images carry values between the nodes: no wait for stores in flight
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            }
+        }
+        const uint32_t n = op.n;
+        const bool l0 = op.s0_lds >= 0, l1 = op.s1_lds >= 0, ld = op.d_lds >= 0, one0 = op.flags & SGD_ONE0, one1 = op.flags & SGD_ONE1;
+        auto x_at = [&](uint32_t e) { return l0 ? ldsf[op.s0_lds + e] : op.s0[e]; };
+        auto y_at = [&](uint32_t e) { return l1 ? ldsf[op.s1_lds + e] : op.s1[e]; };
+        auto put = [&](uint32_t e, float r) {
+            if (ld) lds[op.d_lds + e] = __builtin_bit_cast(uint32_t, r);
+            if (op.d) op.d[e] = r;
+        };
+#define SGD_LOOP(expr) for (uint32_t e = threadIdx.x; e < n; e += nt) put(e, (expr))
+#define SGD_X x_at(one0 ? 0 : e)
+#define SGD_Y y_at(one1 ? 0 : e)
+        switch (op.code) {
+            case SGD_ADD:    SGD_LOOP(ew_apply<EW_ADD>(0, 0, 0, SGD_X, SGD_Y)); break;
+            case SGD_SUB:    SGD_LOOP(ew_apply<EW_SUB>(0, 0, 0, SGD_X, SGD_Y)); break;
+            case SGD_MUL:    SGD_LOOP(ew_apply<EW_MUL>(0, 0, 0, SGD_X, SGD_Y)); break;
+            case SGD_DIV:    SGD_LOOP(ew_apply<EW_DIV>(0, 0, 0, SGD_X, SGD_Y)); break;
+            case SGD_ADD1: { const float y = y_at(0); SGD_LOOP(ew_apply<EW_ADD1>(0, 0, 0, SGD_X, y)); } break;
+            case SGD_SCALE:  SGD_LOOP(ew_apply<EW_SCALE>(op.p0, op.p1, 0, SGD_X, 0.0f)); break;
+            case SGD_UNARY:  SGD_LOOP(ew_apply<EW_UNARY>(0, 0, op.aux, SGD_X, 0.0f)); break;
+            case SGD_COPY:   SGD_LOOP(SGD_X); break;
+            case SGD_CONCAT: SGD_LOOP(e < op.n0 ? x_at(e) : y_at(e - op.n0)); break;
+            case SGD_ARANGE: SGD_LOOP(arange_value(op.p0, op.p1, (int64_t) e)); break;
+            case SGD_COPY4: case SGD_CONCAT4: { // (a COPY4 has n0 == n)
+                const u32x4 * g0 = (const u32x4 *) op.s0, * g1 = (const u32x4 *) op.s1;
+                const u32x4 * i0 = (const u32x4 *) (lds + (l0 ? op.s0_lds : 0)), * i1 = (const u32x4 *) (lds + (l1 ? op.s1_lds : 0));
+                u32x4 * gd = (u32x4 *) op.d, * id = (u32x4 *) (lds + (ld ? op.d_lds : 0));
+                for (uint32_t e = threadIdx.x; e < n; e += nt) {
+                    u32x4 v;
+                    if (e < op.n0) v = l0 ? i0[e] : g0[e];
+                    else           v = l1 ? i1[e - op.n0] : g1[e - op.n0];
+                    if (ld) id[e] = v;
+                    if (gd) gd[e] = v;
+                }
+            } break;
+            default: { // SGD_SUM4 / SGD_SUM1: vx_sum's one-wave order -- lane-strided units in fp64, one butterfly
+                if (threadIdx.x < 64) {
+                    const int W = op.code == SGD_SUM4 ? 4 : 1;
+                    double acc = 0.0;
+                    for (uint32_t u = threadIdx.x; u < n; u += 64)
+                        for (int q = 0; q < W; ++q) acc += (double) x_at(u * W + q);
+                    const double t = vx_wave_sum(acc);
+                    if (threadIdx.x == 0) put(0, (float) t);
+                }
+            } break;
+        }
+#undef SGD_LOOP
+#undef SGD_X
+#undef SGD_Y
     }
 }
 
@@ -1142,8 +1286,8 @@ struct sg_image { vx_tensor t; int32_t off; bool valid; };
 extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx_stream stream) {
     if (!nodes || n_nodes < 1 || n_nodes > SG_MAX_NODES) return vx_fail(VX_ERR_UNSUPPORTED, "small graph: 1 to %d nodes", SG_MAX_NODES);
     sg_args a = {};
-    a.n = n_nodes;
-    sg_image images[SG_MAX_NODES];
+    a.h.n = n_nodes;
+    sg_image images[SG_MAX_NODES + SG_MAX_PRELOADS];
     sg_span  written[SG_MAX_NODES];
     vx_tensor written_t[SG_MAX_NODES];
     int n_images = 0, n_written = 0;
@@ -1152,6 +1296,33 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         const vx_small_node & nd = nodes[k];
         if (!vx_supports_small_node(&nd)) return vx_fail(VX_ERR_UNSUPPORTED, "small graph: node %d (op %d) is not a small elementwise / copy / sum node", k, nd.op);
         if (!nd.dst->data || (nd.src0 && !nd.src0->data) || (nd.src1 && !nd.src1->data)) return vx_fail(VX_ERR_INVALID, "small graph: null data in node %d", k);
+    }
+    // operands that the run only reads get their images first (at most half of the slots, so that the nodes' own
+    // destinations keep theirs): dense F32 / I32 tensors that overlap no destination of the run
+    static const bool preload_allowed = [] { const char * e = getenv("VX_SMALL_GRAPH_PRELOAD"); return !(e && e[0] == '0'); }();
+    for (int k = 0; k < n_nodes && preload_allowed; ++k) {
+        const vx_tensor * ops[2] = { nodes[k].op == VX_NODE_ARANGE ? nullptr : nodes[k].src0, nodes[k].src1 };
+        for (int o = 0; o < 2; ++o) {
+            const vx_tensor * t = ops[o];
+            if (!t || a.h.n_pre == SG_MAX_PRELOADS || vx_type_size(t->type) != 4 || !vx_is_contiguous(t)) continue;
+            const int32_t cnt = (int32_t) vx_nelements(t);
+            if (lds_used + cnt > SG_LDS_ELEMS / 2) continue;
+            const sg_span sp = sg_span_of(t);
+            bool keep = true;
+            for (int m = 0; m < n_nodes && keep; ++m) {
+                const sg_span d = sg_span_of(nodes[m].dst);
+                keep = !(sp.lo < d.hi && d.lo < sp.hi);
+            }
+            for (int m = 0; m < n_images && keep; ++m) keep = !sg_same(&images[m].t, t);
+            if (!keep) continue;
+            a.h.pre[a.h.n_pre++] = { (const uint32_t *) t->data, (uint32_t) cnt, lds_used };
+            a.h.pre_most = std::max(a.h.pre_most, (uint32_t) cnt);
+            images[n_images++] = { *t, lds_used, true };
+            lds_used += (cnt + 3) & ~3; // images start on 16-byte boundaries
+        }
+    }
+    for (int k = 0; k < n_nodes; ++k) {
+        const vx_small_node & nd = nodes[k];
         sg_node & g = a.node[k];
         struct { sg_tensor s0, s1, d; } gt; // the three descriptors while the node is put together
         gt.s0 = sg_desc(nd.op == VX_NODE_ARANGE ? nullptr : nd.src0); gt.s1 = sg_desc(nd.src1); gt.d = sg_desc(nd.dst);
@@ -1196,7 +1367,7 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         } else if (lds_used + cnt <= SG_LDS_ELEMS) {
             images[n_images] = { *nd.dst, lds_used, true };
             gt.d.lds = lds_used;
-            lds_used += cnt;
+            lds_used += (cnt + 3) & ~3;
             ++n_images;
         }
         // a private destination with an image is not stored at all (and so leaves no bytes for later nodes to wait for)
@@ -1245,15 +1416,89 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
     const unsigned threads = block_sum ? 1024u : (unsigned) std::min<int64_t>(1024, std::max<int64_t>(256, (most + 63) / 64 * 64));
     static_assert(sizeof(sg_args) <= 4096, "the node table rides in the kernel's argument block");
     const size_t smem = (size_t) lds_used * 4;
+    // a run of dense F32 nodes (and one-wave sums) goes to the kernel that has nothing left to decode
+    static const bool dense_allowed = [] { const char * e = getenv("VX_SMALL_GRAPH_DENSE"); return !(e && e[0] == '0'); }();
+    sgd_args da = {};
+    da.h = a.h;
+    bool dense = dense_allowed && !block_sum;
+    struct { int32_t off; int writer; bool quads; } wrote[SG_MAX_NODES]; // images written by the run: by which node, in which thread order
+    int n_wrote = 0, last_barrier = 0;
+    for (int k = 0; k < n_nodes && dense; ++k) {
+        const sg_node & g = a.node[k];
+        const vx_small_node & nd = nodes[k];
+        sgd_op & op = da.op[k];
+        const bool has0 = nd.op != VX_NODE_ARANGE && nd.src0, has1 = nd.src1 != nullptr;
+        if ((has0 && g.ftype[0] != VX_TYPE_F32) || (has1 && g.ftype[1] != VX_TYPE_F32) || g.ftype[2] != VX_TYPE_F32) { dense = false; break; }
+        op.n = g.fn; op.n0 = g.fn0; op.p0 = g.p0; op.p1 = g.p1; op.aux = g.aux;
+        op.flags = (g.one0 ? SGD_ONE0 : 0) | (g.one1 ? SGD_ONE1 : 0) | (g.wait_memory ? SGD_WAIT_MEMORY : 0);
+        op.s0_lds = has0 ? g.flds[0] : -1; op.s1_lds = has1 ? g.flds[1] : -1; op.d_lds = g.flds[2];
+        op.s0 = has0 ? (const float *) g.fp[0] : nullptr; op.s1 = has1 ? (const float *) g.fp[1] : nullptr; op.d = (float *) g.fp[2];
+        if (g.kind == SG_SUM) {
+            if (g.flds[0] < 0 && !vx_is_contiguous(nd.src0)) { dense = false; break; }
+            op.code = g.aux ? SGD_SUM4 : SGD_SUM1;
+            op.n = (uint32_t) (vx_nelements(nd.src0) / (g.aux ? 4 : 1));
+        } else if (g.flat == 2) {
+            op.code = SGD_CONCAT;
+        } else if (g.flat == 1) {
+            switch (g.kind) {
+                case SG_EW2:    op.code = SGD_ADD + (uint32_t) g.aux; break;
+                case SG_ADD1:   op.code = SGD_ADD1; break;
+                case SG_SCALE:  op.code = SGD_SCALE; break;
+                case SG_UNARY:  op.code = SGD_UNARY; break;
+                case SG_ARANGE: op.code = SGD_ARANGE; break;
+                default:        op.code = SGD_COPY; break; // CPY of dense F32, REPEAT of one value
+            }
+        } else {
+            dense = false;
+        }
+        if (!dense) break;
+        // 16 bytes per thread for the plain moves
+        auto al = [&](const void * ptr, int32_t off) { return off >= 0 ? off % 4 == 0 : (uintptr_t) ptr % 16 == 0; };
+        if ((op.code == SGD_CONCAT || (op.code == SGD_COPY && !g.one0)) && op.n % 4 == 0 && al(op.s0, op.s0_lds) && (op.d_lds < 0 || op.d_lds % 4 == 0) &&
+            (uintptr_t) op.d % 16 == 0 && (op.code == SGD_COPY || (op.n0 % 4 == 0 && al(op.s1, op.s1_lds)))) {
+            op.n0 = op.code == SGD_COPY ? op.n / 4 : op.n0 / 4;
+            op.n /= 4;
+            op.code = op.code == SGD_COPY ? SGD_COPY4 : SGD_CONCAT4;
+        }
+        // which barriers the run can do without
+        const bool quads = op.code == SGD_COPY4 || op.code == SGD_CONCAT4;
+        const bool own_elements = !quads && op.code != SGD_CONCAT && op.code != SGD_SUM4 && op.code != SGD_SUM1; // thread e mod size reads element e
+        bool need = g.wait_memory != 0;
+        const int32_t src_lds[2] = { op.s0_lds, op.s1_lds };
+        const bool    single[2]  = { g.one0 != 0, g.one1 != 0 || op.code == SGD_ADD1 }; // every thread reads element 0
+        for (int o = 0; o < 2 && !need; ++o) {
+            if (src_lds[o] < 0) continue;
+            for (int m = 0; m < n_wrote; ++m) {
+                if (wrote[m].off != src_lds[o] || wrote[m].writer < last_barrier) continue; // (preloaded, or published by a later barrier)
+                // element 0 is thread 0's: a node of one element reads what thread 0 wrote
+                const bool same_thread = own_elements && !wrote[m].quads && (!single[o] || op.n == 1);
+                if (!same_thread) need = true;
+            }
+        }
+        int mine = -1;
+        for (int m = 0; m < n_wrote; ++m) if (wrote[m].off == op.d_lds) mine = m;
+        if (mine >= 0) need = true; // a rewritten image may still have readers
+        if (op.d_lds >= 0) {
+            if (mine < 0) mine = n_wrote++;
+            wrote[mine] = { op.d_lds, k, quads };
+        }
+        if (k > 0 && !need) op.flags |= SGD_NO_BARRIER;
+        else                last_barrier = k;
+    }
     if (smem > 48 * 1024) { // a kernel has to be told once that it may be given more dynamic LDS than the default limit
-        static bool raised = false;
-        if (!raised) {
-            if (hipFuncSetAttribute((const void *) small_graph_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SG_LDS_ELEMS * 4) != hipSuccess)
+        static bool raised[2] = { false, false };
+        if (!raised[dense]) {
+            const void * fn = dense ? (const void *) small_graph_dense_kernel : (const void *) small_graph_kernel;
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, SG_LDS_ELEMS * 4) != hipSuccess)
                 return vx_fail(VX_ERR_HIP, "small graph: %s", hipGetErrorString(hipGetLastError()));
-            raised = true;
+            raised[dense] = true;
         }
     }
-    small_graph_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(a);
+    if (dense) {
+        small_graph_dense_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(da);
+    } else {
+        small_graph_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(a);
+    }
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
