@@ -32,6 +32,7 @@
 // Algorithmic HBM bytes: each K and V element is read once per 16-column tile; in decode
 // (one tile per KV head) that is n_kv * D * 2 * sizeof(kv) per (b, g), the figure the
 // benchmark divides by.
+#include <type_traits>
 #include "vx_common.hpp"
 #include "kvs_common.hpp"
 
@@ -62,9 +63,15 @@ struct fa_args {
     int seg2_f32; // the second segment holds F32 values while the first is an F16 cache (rounded to f16 as they are loaded)
     int n_q, n_kv, Hq, Hkv, gqa, ne3, rk3, nem2, nem3;
     int n_col_tiles, n_splits, chunk;
+    float inv_gqa, inv_hkv; // reciprocals for fa_div
     float scale, softcap, max_bias, m0, m1;
     uint32_t n_head_log2;
 };
+
+// x / d for 0 <= x < 2^22 with inv = 1 / d: half a step away from every multiple of d the rounding of the product cannot
+// reach the next integer.  (An integer division costs a wave some thirty instructions; the index arithmetic at the top of
+// these kernels stands between the launch and the first load.)
+__device__ __forceinline__ int fa_div(int x, float inv) { return (int) (((float) x + 0.5f) * inv); }
 
 __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -103,16 +110,18 @@ template <> struct kv_load<true> {
 // the K and V rows one wave consumes per iteration: 32 keys, as MFMA operands
 template <int NP, bool KV_F32> struct kv_tile {
     half8_t khi[2][NP], klo[2][NP], vhi[2][NP], vlo[2][NP];
+    __half  mk[2][4]; // the mask's entries for this lane's 8 keys, requested with the tile
 };
 
 // sinks (ops.cpp:8306-8322), normalisation and the permuted store of ggml's result for 4
 // consecutive d of one column
-__device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float M, float L, int b, int g, int col,
-                                          int D, int d0, bool has_addend, float addend) {
+// (the sink and the addend are read by the caller, once and before its first store: a load behind a store waits for the
+// store's completion as well, the memory counter being one for both)
+__device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float M, float L, int b, int iq1, int head,
+                                          int D, int d0, bool has_sink, float sink, bool has_addend, float addend) {
 #pragma clang fp contract(off) // the normalised value is rounded before the addend joins it, as two nodes would
-    const int iq1 = col / a.gqa, head = g * a.gqa + col % a.gqa;
-    if (a.sinks) {
-        const float sk = a.sinks[head] * 1.44269504088896341f; // M is in the log2 domain
+    if (has_sink) {
+        const float sk = sink * 1.44269504088896341f; // M is in the log2 domain
         float ms = 1.0f, vs = 1.0f;
         if (sk > M) { ms = __builtin_amdgcn_exp2f(M - sk); } else { vs = __builtin_amdgcn_exp2f(sk - M); }
         acc *= ms;
@@ -129,7 +138,8 @@ __device__ __forceinline__ void fa_finish(const fa_args & a, float4_t acc, float
 // 2 = the first pair is an F16 cache and the second pair F32 (the step's own keys and values, as the projections
 // left them): they are rounded to f16, to nearest even, while they are loaded -- exactly what a CPY node to an F16
 // tensor in front of a CONCAT would have stored.
-template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP, int TWO_SEG>
+// HALF: the whole key range is at most 16 keys (chosen by the host: one range, one pair of tensors).
+template <int D, bool KV_F32, bool HAS_MASK, bool SOFTCAP, int TWO_SEG, bool HALF = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fattn_cols16_kernel(const fa_args a) {
     constexpr int NP  = D / 32;          // MFMAs along the head dimension
     constexpr int SEG = D / 4;           // elements of a row owned by lane-group j
@@ -138,28 +148,35 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     const int lane = threadIdx.x;
     const int j = lane >> 4, c = lane & 15;
 
-    int w = blockIdx.x;
-    const int ct = w % a.n_col_tiles; w /= a.n_col_tiles;
-    const int sp = w % a.n_splits;    w /= a.n_splits;
-    const int g  = w % a.Hkv;
-    const int b  = w / a.Hkv;
-    const int tile = (b * a.Hkv + g) * a.n_col_tiles + ct;
+    // the grid is (column tile, key range, batch entry x KV head): dispatched in the same order as one flat index
+    const int ct = blockIdx.x, sp = blockIdx.y, bg = blockIdx.z;
+    const int b  = fa_div(bg, a.inv_hkv);
+    const int g  = bg - b * a.Hkv;
+    const int tile = bg * a.n_col_tiles + ct;
 
     const int  ncols  = a.n_q * a.gqa;
     const int  col    = ct * 16 + c;
     const bool col_ok = col < ncols;
-    const int  iq1    = col_ok ? col / a.gqa : 0;
-    const int  head   = g * a.gqa + (col_ok ? col % a.gqa : 0);
+    const int  iq1    = col_ok ? fa_div(col, a.inv_gqa) : 0;
+    const int  head   = g * a.gqa + (col_ok ? col - iq1 * a.gqa : 0);
+    const int  bk     = a.rk3 == 1 ? b : b / a.rk3; // K / V broadcast over the batch dimension: rare
 
-    const char * kbase = a.k + (uint64_t) g * a.nbk2 + (uint64_t) (b / a.rk3) * a.nbk3 + (uint64_t) (SEG * j) * ES;
-    const char * vbase = a.v + (uint64_t) g * a.nbv2 + (uint64_t) (b / a.rk3) * a.nbv3 + (uint64_t) (SEG * j) * ES;
+    const char * kbase = a.k + (uint64_t) g * a.nbk2 + (uint64_t) bk * a.nbk3 + (uint64_t) (SEG * j) * ES;
+    const char * vbase = a.v + (uint64_t) g * a.nbv2 + (uint64_t) bk * a.nbv3 + (uint64_t) (SEG * j) * ES;
 
     const char * kbase2 = kbase;
     const char * vbase2 = vbase;
     if constexpr (TWO_SEG != 0) {
         constexpr int ES2 = TWO_SEG == 2 ? 4 : ES;
-        kbase2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) (b / a.rk3) * a.nbk3b + (uint64_t) (SEG * j) * ES2;
-        vbase2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) (b / a.rk3) * a.nbv3b + (uint64_t) (SEG * j) * ES2;
+        kbase2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) bk * a.nbk3b + (uint64_t) (SEG * j) * ES2;
+        vbase2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) bk * a.nbv3b + (uint64_t) (SEG * j) * ES2;
+    }
+
+    float slope = 1.0f;
+    const __half * mrow = nullptr;
+    if constexpr (HAS_MASK) {
+        slope = vx_alibi_slope(a.max_bias, (uint32_t) head, a.n_head_log2, a.m0, a.m1) * 1.44269504088896341f;
+        if (a.mask) mrow = (const __half *) (a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (a.nem2 == 1 ? 0 : head % a.nem2) * a.nbm2 + (uint64_t) (a.nem3 == 1 ? 0 : b % a.nem3) * a.nbm3);
     }
 
     const int kv0 = sp * a.chunk;
@@ -170,6 +187,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     const int pure   = TWO_SEG == 2 ? a.n_kv1 / 32 * 32 : 0;
     const int kv1p   = TWO_SEG == 2 ? min(kv1, pure) : kv1;  // end of the pipelined tiles
     const int kclamp = TWO_SEG == 2 ? a.n_kv1 - 1 : a.n_kv - 1;
+
+    // the mask's entries of a tile's keys kb + 16h + 4j + r, requested behind the tile itself (clamped like the rows)
+    auto load_mask = [&](int kb, kv_tile<NP, KV_F32> & t, int halves) {
+        if constexpr (HAS_MASK) {
+            if (SOFTCAP ? mrow != nullptr : true) { // (without a soft cap this kernel is only launched with a mask)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (h < halves) t.mk[h][r] = mrow[min(kb + 16 * h + 4 * j + r, a.n_kv - 1)];
+            }
+        }
+    };
 
     // rows this lane loads (MFMA row c of each 16-key half); clamped, masked out later
     auto load_tile = [&](int kb, kv_tile<NP, KV_F32> & t) {
@@ -192,10 +222,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
             kv_load<KV_F32>::run(v0p + p * 8 * ES, t.vhi[0][p], t.vlo[0][p]);
             kv_load<KV_F32>::run(v1p + p * 8 * ES, t.vhi[1][p], t.vlo[1][p]);
         }
+        load_mask(kb, t, 2);
+    };
+
+    // the first 16 keys of a tile only: all a range of at most 16 keys needs
+    auto load_half0 = [&](int kb, kv_tile<NP, KV_F32> & t) {
+        const int key0 = min(kb + c, kclamp);
+        const char * k0p = kbase + (uint64_t) key0 * a.nbk1;
+        const char * v0p = vbase + (uint64_t) key0 * a.nbv1;
+        if constexpr (TWO_SEG == 1) {
+            if (key0 >= a.n_kv1) { k0p = kbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbk1b; v0p = vbase2 + (uint64_t) (key0 - a.n_kv1) * a.nbv1b; }
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) kv_load<KV_F32>::run(k0p + p * 8 * ES, t.khi[0][p], t.klo[0][p]);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) kv_load<KV_F32>::run(v0p + p * 8 * ES, t.vhi[0][p], t.vlo[0][p]);
+        load_mask(kb, t, 1);
     };
 
     // a tile at or behind the type boundary: each lane reads its two keys from the tensor that holds them
     auto load_mixed = [&](int kb, kv_tile<NP, KV_F32> & t) {
+        load_mask(kb, t, 2);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int key = min(kb + 16 * h + c, a.n_kv - 1);
@@ -224,12 +271,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         }
     };
 
+    // Q's values are requested first: the tile loads below sit in branches, F32 tiles are converted where they are
+    // loaded, and whatever is requested behind a branch waits for that conversion's data.
+    float4_t qraw[NP][2];
+    {
+        const float * qp = (const float *) (a.q + (uint64_t) iq1 * a.nbq1 + (uint64_t) head * a.nbq2 + (uint64_t) b * a.nbq3) + SEG * j;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) { qraw[p][0] = ((const float4_t *) (qp + 8 * p))[0]; qraw[p][1] = ((const float4_t *) (qp + 8 * p))[1]; }
+    }
+
     // two tiles alternate in registers: while one is consumed the other is in flight
     kv_tile<NP, KV_F32> t0, t1, t2;
     const int kmix = max(kv0, pure); // first tile of the lane-by-lane part (TWO_SEG == 2)
+    // A range of at most 16 keys (LocDiT's 14-token sequence) is half a tile: the second half's loads, conversions and
+    // products would all be of keys that are switched off.  (A kernel of its own, not a branch: tile loads in a branch
+    // would hold back every request behind it until their conversions have their data.)
+    static_assert(!HALF || TWO_SEG == 0, "the half-tile kernel reads one pair of tensors");
     if constexpr (TWO_SEG == 2) {
         if (kmix < kv1) load_mixed(kmix, t2);  // requested first, consumed last
         if (kv0 < kv1p) load_tile(kv0, t0);
+    } else if constexpr (HALF) {
+        load_half0(kv0, t0);
     } else {
         load_tile(kv0, t0);
     }
@@ -237,10 +299,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     // ---- Q^T operand: column c, elements d = SEG*j + 8p + i, split into hi + lo
     half8_t qhi[NP], qlo[NP];
     {
-        const float * qp = (const float *) (a.q + (uint64_t) iq1 * a.nbq1 + (uint64_t) head * a.nbq2 + (uint64_t) b * a.nbq3) + SEG * j;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            float4_t x0 = ((const float4_t *) (qp + 8 * p))[0], x1 = ((const float4_t *) (qp + 8 * p))[1];
+            float4_t x0 = qraw[p][0], x1 = qraw[p][1];
             if (!col_ok) { x0 = float4_t{0, 0, 0, 0}; x1 = float4_t{0, 0, 0, 0}; }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -260,12 +321,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 #pragma unroll
         for (int i = 0; i < 8; ++i) sel[u][i] = (j == 2 * u + (c >> 3) && i == (c & 7)) ? (_Float16) 1.0f : (_Float16) 0.0f;
 
-    float slope = 1.0f;
-    const __half * mrow = nullptr;
-    if constexpr (HAS_MASK) {
-        slope = vx_alibi_slope(a.max_bias, (uint32_t) head, a.n_head_log2, a.m0, a.m1) * 1.44269504088896341f;
-        if (a.mask) mrow = (const __half *) (a.mask + (uint64_t) iq1 * a.nbm1 + (uint64_t) (head % a.nem2) * a.nbm2 + (uint64_t) (b % a.nem3) * a.nbm3);
-    }
 
     float4_t o[NP][2];
 #pragma unroll
@@ -273,19 +328,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     float m = -INFINITY; // running max of column c (identical in the 4 lanes of a column)
     float l = 0.0f;      // this lane's share of the running sum
 
-    auto consume = [&](const kv_tile<NP, KV_F32> & t, int kb) {
+    auto consume = [&](const kv_tile<NP, KV_F32> & t, int kb, auto first_half_only) {
+        constexpr int NH = decltype(first_half_only)::value ? 1 : 2; // 16-key halves that take part
         // additive mask of this lane's 8 keys (kb + 16h + 4j + r); loads are clamped, keys
         // past the end of the range (only in a wave's last tile) are switched off
         const bool tail = kb + 32 > kv1; // wave-uniform
         float mv[2][4];
         if (HAS_MASK || tail) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < NH; ++h)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int key = kb + 16 * h + 4 * j + r;
                     float x = 0.0f;
-                    if constexpr (HAS_MASK) { if (mrow) x = slope * __half2float(mrow[min(key, a.n_kv - 1)]); } // slope carries log2(e)
+                    if constexpr (HAS_MASK) { if (SOFTCAP ? mrow != nullptr : true) x = slope * __half2float(t.mk[h][r]); } // slope carries log2(e)
                     mv[h][r] = key < kv1 ? x : -INFINITY;
                 }
         }
@@ -293,7 +349,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         // ---- S^T for the two 16-key halves
         float4_t s[2];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < NH; ++h) {
             float4_t acc = {0, 0, 0, 0};
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
@@ -307,7 +363,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         // ---- scale, soft cap, mask
         float cmax = -INFINITY;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < NH; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 // a.scale carries log2(e) (the soft cap path applies it after tanh)
@@ -327,9 +383,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
         const float alpha  = __builtin_amdgcn_exp2f(m - shift); // m = -inf -> 0
         float psum = 0.0f;
         half8_t phi, plo;
-        float pvv[8];
+        float pvv[8] = { 0, 0, 0, 0, 0, 0, 0, 0 }; // (the weights of a half that takes no part: exactly what its switched-off keys would get)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < NH; ++h)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 pvv[4 * h + r] = __builtin_amdgcn_exp2f(s[h][r] - shift);
@@ -352,8 +408,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 float4_t t0 = mfma16(t.vhi[0][p], sel[u], float4_t{0, 0, 0, 0});
-                float4_t t1 = mfma16(t.vhi[1][p], sel[u], float4_t{0, 0, 0, 0});
-                if constexpr (KV_F32) { t0 = mfma16(t.vlo[0][p], sel[u], t0); t1 = mfma16(t.vlo[1][p], sel[u], t1); }
+                float4_t t1 = float4_t{0, 0, 0, 0};
+                if constexpr (NH == 2) t1 = mfma16(t.vhi[1][p], sel[u], t1);
+                if constexpr (KV_F32) {
+                    t0 = mfma16(t.vlo[0][p], sel[u], t0);
+                    if constexpr (NH == 2) t1 = mfma16(t.vlo[1][p], sel[u], t1);
+                }
                 half8_t vt;
 #pragma unroll
                 for (int r = 0; r < 4; r += 2) { pk2(vt, r, t0[r], t0[r + 1]); pk2(vt, 4 + r, t1[r], t1[r + 1]); }
@@ -376,17 +436,21 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     // conditional prefetch forces the compiler to wait for everything and exposes the whole
     // memory latency in every iteration.
     const int klast = kv0 + ((kv1p - kv0 - 1) / 32) * 32;
-    for (int kb = kv0; kb < kv1p; kb += 64) {
-        load_tile(min(kb + 32, klast), t1);
-        consume(t0, kb);
-        if (kb + 32 >= kv1p) break;
-        load_tile(min(kb + 64, klast), t0);
-        consume(t1, kb + 32);
+    if constexpr (HALF) {
+        consume(t0, kv0, std::true_type{});
+    } else {
+        for (int kb = kv0; kb < kv1p; kb += 64) {
+            load_tile(min(kb + 32, klast), t1);
+            consume(t0, kb, std::false_type{});
+            if (kb + 32 >= kv1p) break;
+            load_tile(min(kb + 64, klast), t0);
+            consume(t1, kb + 32, std::false_type{});
+        }
     }
     if constexpr (TWO_SEG == 2) {
         for (int kb = kmix; kb < kv1; kb += 32) {
             if (kb != kmix) load_mixed(kb, t2);
-            consume(t2, kb);
+            consume(t2, kb, std::false_type{});
         }
     }
 
@@ -396,11 +460,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 
     // lane (j,c), tile (p,u), register r holds d = SEG*(2u + j/2) + 8p + 4*(j%2) + r of column c
     if (a.n_splits == 1) {
+        const bool  has_sink = a.sinks != nullptr, has_addend = a.add1 != nullptr;
+        const float sink = has_sink ? a.sinks[head] : 0.0f, addend = has_addend ? *a.add1 : 0.0f;
 #pragma unroll
         for (int p = 0; p < NP; ++p)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
-                fa_finish(a, o[p][u], m, l, b, g, col, D, SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1), a.add1 != nullptr, a.add1 ? *a.add1 : 0.0f);
+                fa_finish(a, o[p][u], m, l, b, iq1, head, D, SEG * (2 * u + (j >> 1)) + 8 * p + 4 * (j & 1), has_sink, sink, has_addend, addend);
     } else {
         const uint64_t pbase = ((uint64_t) tile * a.n_splits + sp) * 16 + c;
 #pragma unroll
@@ -505,7 +571,11 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
         addend     = kvs_addend;
         has_addend = true;
     }
-    if (q == 0) fa_finish(a, acc, M, L, b, g, col, D, d0, has_addend, addend);
+    if (q == 0) {
+        const int  iq1 = fa_div(col, a.inv_gqa), head = g * a.gqa + (col - iq1 * a.gqa);
+        const bool has_sink = a.sinks != nullptr;
+        fa_finish(a, acc, M, L, b, iq1, head, D, d0, has_sink, has_sink ? a.sinks[head] : 0.0f, has_addend, addend);
+    }
 }
 
 int g_num_cus = 0;
@@ -557,8 +627,8 @@ int64_t fa_tiles(const vx_tensor * q, const vx_tensor * k) {
 }
 
 template <int D, bool KV_F32>
-void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
-    const dim3 grid((unsigned) nblocks), block(64);
+void launch_cols16(const fa_args & a, hipStream_t st) {
+    const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv)), block(64);
     if constexpr (D == 64 && !KV_F32) {
         if (a.k2 && a.seg2_f32) { // an F16 cache and the step's F32 keys
             if (a.softcap != 0.0f) fattn_cols16_kernel<D, false, true, true, 2><<<grid, block, 0, st>>>(a);
@@ -575,6 +645,9 @@ void launch_cols16(const fa_args & a, int nblocks, hipStream_t st) {
     }
     if (a.softcap != 0.0f) { // rare: always take the masked variant
         fattn_cols16_kernel<D, KV_F32, true, true, 0><<<grid, block, 0, st>>>(a);
+    } else if (a.n_kv <= 16 && a.n_splits == 1) {
+        if (a.mask) fattn_cols16_kernel<D, KV_F32, true, false, 0, true><<<grid, block, 0, st>>>(a);
+        else        fattn_cols16_kernel<D, KV_F32, false, false, 0, true><<<grid, block, 0, st>>>(a);
     } else if (a.mask) {
         fattn_cols16_kernel<D, KV_F32, true, false, 0><<<grid, block, 0, st>>>(a);
     } else {
@@ -595,6 +668,7 @@ extern "C" int vx_supports_flash_attn_ext(const vx_tensor * q, const vx_tensor *
     if (k->ne[0] != D || v->ne[0] != D) return 0;
     if (k->ne[1] != v->ne[1] || k->ne[2] != v->ne[2] || k->ne[3] != v->ne[3]) return 0;
     if (q->ne[2] % k->ne[2] || q->ne[3] % k->ne[3]) return 0;
+    if (q->ne[3] * k->ne[2] > 65535) return 0; // (batch entry x KV head is one dimension of the grid)
     if (q->nb[0] != 4 || k->nb[0] != vx_type_size(k->type) || v->nb[0] != vx_type_size(v->type)) return 0;
     // strides must keep 16-byte vector loads aligned; the data pointers are checked at launch
     for (int i = 1; i < 4; ++i)
@@ -818,6 +892,8 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
 
     const int ncols = a.n_q * a.gqa;
     a.n_col_tiles   = (ncols + 15) / 16;
+    a.inv_gqa = 1.0f / (float) a.gqa; a.inv_hkv = 1.0f / (float) a.Hkv;
+    if (ncols >= (1 << 22) || (int64_t) a.ne3 * a.Hkv > 65535) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext: launch too large");
     const int64_t tiles = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
 
     fa_split_plan(tiles, a.n_kv, &a.n_splits, &a.chunk);
@@ -850,8 +926,8 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     }
 
     const bool f32 = k->type == VX_TYPE_F32;
-    if (D == 64) { if (f32) launch_cols16<64, true>(a, (int) nblocks, st); else launch_cols16<64, false>(a, (int) nblocks, st); }
-    else         { if (f32) launch_cols16<128, true>(a, (int) nblocks, st); else launch_cols16<128, false>(a, (int) nblocks, st); }
+    if (D == 64) { if (f32) launch_cols16<64, true>(a, st); else launch_cols16<64, false>(a, st); }
+    else         { if (f32) launch_cols16<128, true>(a, st); else launch_cols16<128, false>(a, st); }
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
         const dim3 grid((unsigned) (tiles * 16));

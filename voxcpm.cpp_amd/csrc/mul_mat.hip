@@ -781,9 +781,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
                     if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
             }
         }
-        if constexpr (NORM) __syncthreads(); // the activation waves' barrier after the norm scales (the direct loads are not
-                                             // known to the compiler: no wait for them here)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's direct loads have landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's direct loads have landed (they are not known to the compiler)
     } else {
         // ---- activations -> LDS as f16 (or quantised), [token][k]
         const int awid = wid - NWD, atid = tid - 64 * NWD;
@@ -834,17 +832,16 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
         constexpr int UB = MANY ? (NW == 16 ? 4 : 8) : 1;
         const bool same_cols = (64 * NA) % upr == 0; // uniform
         float4_t f0[UB], f1[UB], g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
-        // with a fused norm and many units the requests wait until the norm's rows have left the registers (two
-        // work-groups per CU need the kernel under 128 of them); the rows have pulled the same lines into the cache
-        constexpr bool LATE = NORM && MANY;
-        if (same_cols && !LATE) {
+        if (!NORM && same_cols) {
 #pragma unroll
             for (int i = 0; i < UB; ++i) {
                 const int unit = atid + i * 64 * NA;
                 if (unit < units) fetch(unit, f0[i], f1[i]);
             }
-            if constexpr (NORM) { if (atid < units) fetch_gain(atid, g0, g1); }
         }
+        // With a fused norm a token's row belongs to ONE wave, as in the RMS_NORM kernel: the wave reads the row once, sums
+        // its squares, and stages the normalised row from the registers it already holds -- no second trip for the values,
+        // no exchange of scales between the waves.  Lane l holds columns 4 (l + 64 c) .. + 3 of the row.
         vx_rms_row nrow, nrow2; // the tokens this wave normalises first, requested up front
         if constexpr (NORM) {
             if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
@@ -866,40 +863,76 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
                 }
             }
         }
-        if constexpr (NORM) { // one wave per token, as the RMS_NORM kernel has it; a wave with several tokens takes two at a time
+        if constexpr (NORM) { // a wave with several tokens takes two at a time
+            const int nv = (int) (a.K >> 8); // 16-byte pieces of a row per lane (K is a multiple of 256 here)
+            auto stage_row = [&](int t, const vx_rms_row & r, float sc) {
+#pragma unroll
+                for (int cc = 0; cc < 8; ++cc) {
+                    if (cc >= nv) break;
+                    const int    iv = lane + 64 * cc;
+                    const float4 g  = ((const float4 *) a.norm_w)[iv];
+                    // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
+                    float v[4] = { r.v[cc].x, r.v[cc].y, r.v[cc].z, r.v[cc].w };
+                    const float gg[4] = { g.x, g.y, g.z, g.w };
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { v[i] *= sc; v[i] *= gg[i]; }
+                    half4_t h;
+                    if constexpr (ACT_Q8) { // 8 consecutive lanes = one 32-wide block
+                        float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+                        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+                        const float d  = amax / 127.f;
+                        const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) h[i] = (_Float16) rintf(v[i] * id);
+                        if ((lane & 7) == 0) xd[(iv >> 3) * 16 + t] = (float) (_Float16) d;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) h[i] = (_Float16) v[i];
+                    }
+                    *(half4_t *) (xs + (size_t) t * KP + 4 * iv) = h;
+                }
+            };
             for (int t = awid; t < N; t += 2 * NA) {
                 if (t != awid) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
                 if (t + NA < N) {
                     if (t != awid) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (t + NA) * a.nb11), a.K, lane);
                     float s1, s2;
                     vx_rms_row_scale2(nrow, nrow2, a.K, lane, a.norm_eps, s1, s2);
-                    if (lane == 0) { nsc[t] = s1; nsc[t + NA] = s2; }
+                    stage_row(t, nrow, s1);
+                    stage_row(t + NA, nrow2, s2);
                 } else {
-                    const float sc = vx_rms_row_scale(nrow, a.K, lane, a.norm_eps);
-                    if (lane == 0) nsc[t] = sc;
+                    stage_row(t, nrow, vx_rms_row_scale(nrow, a.K, lane, a.norm_eps));
                 }
             }
-            __syncthreads();
-        }
-        if (same_cols) {
-            if constexpr (LATE) {
-#pragma unroll
-                for (int i = 0; i < UB; ++i) {
-                    const int unit = atid + i * 64 * NA;
-                    if (unit < units) fetch(unit, f0[i], f1[i]);
-                }
-                if (atid < units) fetch_gain(atid, g0, g1);
-            }
+        } else if (same_cols) {
 #pragma unroll
             for (int i = 0; i < UB; ++i) {
                 const int unit = atid + i * 64 * NA;
                 if (unit < units) stage(unit, f0[i], f1[i], g0, g1);
             }
         }
-        for (int unit = atid + (same_cols ? UB : 0) * 64 * NA; unit < units; unit += 64 * NA) {
-            fetch(unit, f0[0], f1[0]);
-            if constexpr (NORM) { if (!same_cols) fetch_gain(unit, g0, g1); }
-            stage(unit, f0[0], f1[0], g0, g1);
+        if (NORM) { // (every row is staged)
+        } else if (same_cols) { // what is left after the first UB units of a thread: again UB requests together, then their staging
+            for (int base = atid + UB * 64 * NA; base < units; base += UB * 64 * NA) {
+#pragma unroll
+                for (int i = 0; i < UB; ++i) {
+                    const int unit = base + i * 64 * NA;
+                    if (unit < units) fetch(unit, f0[i], f1[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < UB; ++i) {
+                    const int unit = base + i * 64 * NA;
+                    if (unit < units) stage(unit, f0[i], f1[i], g0, g1);
+                }
+            }
+        } else {
+            for (int unit = atid; unit < units; unit += 64 * NA) {
+                fetch(unit, f0[0], f1[0]);
+                if constexpr (NORM) fetch_gain(unit, g0, g1);
+                stage(unit, f0[0], f1[0], g0, g1);
+            }
         }
     }
     __syncthreads();
