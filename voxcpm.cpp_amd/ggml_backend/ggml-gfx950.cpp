@@ -1203,26 +1203,39 @@ uint64_t graph_cheap_signature(const ggml_cgraph * g) {
     }
     return h | 1;
 }
-void fingerprint_tensor(uint64_t & h, const ggml_tensor * t) {
-    h = mix64(h, (uint64_t) (uintptr_t) t->data);
-    h = mix64(h, ((uint64_t) t->type << 32) ^ (uint64_t) t->op ^ ((uint64_t) t->flags << 48));
-    for (int d = 0; d < GGML_MAX_DIMS; ++d) h = mix64(h, (uint64_t) t->ne[d] ^ ((uint64_t) t->nb[d] << 24));
+// full: everything a launch is derived from.  A thousand nodes are some 25 000 words, hashed on every graph_compute of a
+// caller that waits for each step: four independent multiply-xor chains take the words in turn (a single chain is bound
+// by the multiplier's latency: 40 us for a decode step's graph, a twentieth of the step itself).
+struct fingerprint_state {
+    uint64_t h[4] = { 0x243F6A8885A308D3ull, 0x13198A2E03707344ull, 0xA4093822299F31D0ull, 0x082EFA98EC4E6C89ull };
+    unsigned n = 0;
+    void add(uint64_t v) {
+        uint64_t & x = h[n++ & 3];
+        x = (x ^ v) * 0x9E3779B97F4A7C15ull;
+        x ^= x >> 29;
+    }
+    uint64_t finish() const { return mix64(mix64(mix64(mix64((uint64_t) n, h[0]), h[1]), h[2]), h[3]); }
+};
+void fingerprint_tensor(fingerprint_state & f, const ggml_tensor * t) {
+    f.add((uint64_t) (uintptr_t) t->data);
+    f.add(((uint64_t) t->type << 32) ^ (uint64_t) t->op ^ ((uint64_t) t->flags << 48));
+    for (int d = 0; d < GGML_MAX_DIMS; ++d) f.add((uint64_t) t->ne[d] ^ ((uint64_t) t->nb[d] << 24));
 }
-// full: everything a launch is derived from
 uint64_t graph_fingerprint(const ggml_cgraph * g) {
-    uint64_t h = 0x243F6A8885A308D3ull ^ (uint64_t) g->n_nodes;
+    fingerprint_state f;
+    f.add((uint64_t) g->n_nodes);
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
-        fingerprint_tensor(h, n);
+        fingerprint_tensor(f, n);
         const uint64_t * op = (const uint64_t *) n->op_params;
-        for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(uint64_t); ++k) h = mix64(h, op[k]);
-        for (int k = 0; k < GGML_MAX_SRC; ++k) {
-            if (!n->src[k]) { h = mix64(h, 0x55); continue; }
-            fingerprint_tensor(h, n->src[k]);
-        }
-        h = mix64(h, (uint64_t) (uintptr_t) (n->view_src ? n->view_src->data : nullptr) ^ (uint64_t) n->view_offs);
+        for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(uint64_t); ++k) f.add(op[k]);
+        uint64_t present = 0; // which operand slots are in use, then the operands themselves
+        for (int k = 0; k < GGML_MAX_SRC; ++k) if (n->src[k]) present |= (uint64_t) 1 << k;
+        f.add(present);
+        for (int k = 0; k < GGML_MAX_SRC; ++k) if (n->src[k]) fingerprint_tensor(f, n->src[k]);
+        f.add((uint64_t) (uintptr_t) (n->view_src ? n->view_src->data : nullptr) ^ ((uint64_t) n->view_offs << 1));
     }
-    return h | 1;
+    return f.finish() | 1;
 }
 
 ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out);
