@@ -108,16 +108,32 @@ typedef float    float4_t __attribute__((ext_vector_type(4)));
 typedef float    float16_t __attribute__((ext_vector_type(16)));
 typedef int      int4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float vx_wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+// The value of lane (i + N) mod 16 of the same row of 16 lanes, by a DPP move (a register read; a lane exchange through
+// LDS hardware costs a round trip of a hundred cycles).  In a butterfly sum whose steps run 32, 16, 8, 4, 2, 1 the steps
+// 8 .. 1 may take it in place of the xor partner: when step s is reached the values repeat every 2 s lanes, and i + s and
+// i ^ s differ by 0 or 2 s -- the same bits are added in the same order.
+template <int N>
+__device__ __forceinline__ float vx_row_ror(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
+}
+template <int N>
+__device__ __forceinline__ double vx_row_ror(double v) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), 0x120 + N, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), 0x120 + N, 0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+template <typename T>
+__device__ __forceinline__ T vx_wave_sum_t(T v) {
+    v += __shfl_xor(v, 32, 64);
+    v += __shfl_xor(v, 16, 64);
+    v += vx_row_ror<8>(v);
+    v += vx_row_ror<4>(v);
+    v += vx_row_ror<2>(v);
+    v += vx_row_ror<1>(v);
     return v;
 }
-__device__ __forceinline__ double vx_wave_sum(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
+__device__ __forceinline__ float  vx_wave_sum(float v)  { return vx_wave_sum_t(v); }
+__device__ __forceinline__ double vx_wave_sum(double v) { return vx_wave_sum_t(v); }
 // 1 / rms of one dense, 16-byte aligned row of ne00 <= 2048 floats, by one wave, exactly as the RMS_NORM
 // kernel's wave-per-row path forms it: fp32 squares, fp64 lane sums in float4 order, xor butterfly, one
 // rounding of the mean to fp32.  The same value in every lane.
@@ -159,11 +175,15 @@ __device__ __forceinline__ void vx_rms_row_scale2(const vx_rms_row & r1, const v
                                                   float & s1, float & s2) {
     double a = vx_rms_row_lane_sum(r1, ne00, lane), b = vx_rms_row_lane_sum(r2, ne00, lane);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
+    for (int off = 32; off > 8; off >>= 1) {
         const double ta = __shfl_xor(a, off, 64), tb = __shfl_xor(b, off, 64);
         a += ta;
         b += tb;
     }
+    { const double ta = vx_row_ror<8>(a), tb = vx_row_ror<8>(b); a += ta; b += tb; }
+    { const double ta = vx_row_ror<4>(a), tb = vx_row_ror<4>(b); a += ta; b += tb; }
+    { const double ta = vx_row_ror<2>(a), tb = vx_row_ror<2>(b); a += ta; b += tb; }
+    { const double ta = vx_row_ror<1>(a), tb = vx_row_ror<1>(b); a += ta; b += tb; }
     s1 = vx_rms_finish(a, ne00, eps);
     s2 = vx_rms_finish(b, ne00, eps);
 }
@@ -174,7 +194,11 @@ __device__ __forceinline__ float vx_rms_scale_wave(const float * x, int64_t ne00
 }
 __device__ __forceinline__ float vx_wave_max(float v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    for (int off = 32; off > 8; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    v = fmaxf(v, vx_row_ror<8>(v));
+    v = fmaxf(v, vx_row_ror<4>(v));
+    v = fmaxf(v, vx_row_ror<2>(v));
+    v = fmaxf(v, vx_row_ror<1>(v));
     return v;
 }
 
