@@ -753,6 +753,104 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     const char * xb = a.x + (uint64_t) tok0 * a.nb11;
     float resv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 
+    // ---- activations without a norm: units of 8 values, a thread's units UB at a time (requested together, then staged: a
+    // round trip per unit would be paid a dozen times with sixteen tokens).  With many units the waves that fetch the weights
+    // take a share once their requests are out -- until the rows land they have nothing else to do.
+    auto fetch = [&](int unit, float4_t & v0, float4_t & v1) {
+        const int t = unit_token(unit), u = unit - t * upr;
+        const float4_t * xp = (const float4_t *) ((const float *) (xb + (uint64_t) t * a.nb11) + 8 * u);
+        v0 = xp[0]; v1 = xp[1];
+    };
+    auto stage = [&](int unit, const float4_t & v0, const float4_t & v1) {
+        const int t = unit_token(unit), u = unit - t * upr;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
+        half8_t h;
+        if constexpr (ACT_Q8) { // 4 consecutive units = one 32-wide block
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+            amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+            const float d  = amax / 127.f;
+            const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
+            if ((u & 3) == 0) xd[(u >> 2) * 16 + t] = (float) (_Float16) d;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
+        }
+        *(half8_t *) (xs + (size_t) t * KP + 8 * u) = h;
+    };
+    constexpr int  UB = MANY ? (NW == 16 ? 4 : 8) : 1;
+    constexpr bool SHARE = MANY && !NORM;                 // the weight-fetching waves stage units too
+    constexpr int  USTRIDE = 64 * (SHARE ? NW : NA);      // the staging threads' stride in units
+    auto stage_rest = [&](int first) { // units first, first + USTRIDE, ... : UB requests together, then their staging
+        float4_t f0[UB], f1[UB];
+        for (int base = first; base < units; base += UB * USTRIDE) {
+#pragma unroll
+            for (int i = 0; i < UB; ++i) {
+                const int unit = base + i * USTRIDE;
+                if (unit < units) fetch(unit, f0[i], f1[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < UB; ++i) {
+                const int unit = base + i * USTRIDE;
+                if (unit < units) stage(unit, f0[i], f1[i]);
+            }
+        }
+    };
+
+    // ---- fused RMS_NORM: a token's row belongs to ONE wave, as in the RMS_NORM kernel: the wave reads the row once, sums its
+    // squares, and stages the normalised row from the registers it already holds.  Lane l holds columns 4 (l + 64 c) .. + 3.
+    // Tokens are dealt in pairs: the first 2 NA to the activation waves (t, t + NA), the next 2 NWD to the waves that fetch
+    // the weights (they have nothing to do while their requests are under way), anything beyond to the activation waves again.
+        const int nv = (int) (a.K >> 8); // 16-byte pieces of a row per lane (K is a multiple of 256 here)
+        auto stage_row = [&](int t, const vx_rms_row & r, float sc) {
+#pragma unroll
+            for (int cc = 0; cc < 8; ++cc) {
+                if (cc >= nv) break;
+                const int    iv = lane + 64 * cc;
+                const float4 g  = ((const float4 *) a.norm_w)[iv];
+                // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
+                float v[4] = { r.v[cc].x, r.v[cc].y, r.v[cc].z, r.v[cc].w };
+                const float gg[4] = { g.x, g.y, g.z, g.w };
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { v[i] *= sc; v[i] *= gg[i]; }
+                half4_t h;
+                if constexpr (ACT_Q8) { // 8 consecutive lanes = one 32-wide block
+                    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+                    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+                    const float d  = amax / 127.f;
+                    const float id = amax != 0.0f ? 127.f / amax : 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) h[i] = (_Float16) rintf(v[i] * id);
+                    if ((lane & 7) == 0) xd[(iv >> 3) * 16 + t] = (float) (_Float16) d;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) h[i] = (_Float16) v[i];
+                }
+                *(half4_t *) (xs + (size_t) t * KP + 4 * iv) = h;
+            }
+        };
+    auto norm_pair = [&](int t, int stride) { // tokens t and t + stride (if there is one) by this wave
+        vx_rms_row r1, r2;
+        vx_rms_row_load(r1, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
+        if (t + stride < N) {
+            vx_rms_row_load(r2, (const float *) (xb + (uint64_t) (t + stride) * a.nb11), a.K, lane);
+            float s1, s2;
+            vx_rms_row_scale2(r1, r2, a.K, lane, a.norm_eps, s1, s2);
+            stage_row(t, r1, s1);
+            stage_row(t + stride, r2, s2);
+        } else {
+            stage_row(t, r1, vx_rms_row_scale(r1, a.K, lane, a.norm_eps));
+        }
+    };
+
     if (wid < NWD) {
         // ---- weight rows -> LDS.  These waves share their SIMDs with the activation waves: until the requests are out they go first
         __builtin_amdgcn_s_setprio(3);
@@ -781,61 +879,19 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
                     if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
             }
         }
+        if constexpr (NORM) { // (requested behind the weights, these rows arrive behind them)
+            if (2 * NA + wid < N) norm_pair(2 * NA + wid, NWD);
+        }
+        if constexpr (SHARE) stage_rest(64 * NA + tid);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's direct loads have landed (they are not known to the compiler)
     } else {
         // ---- activations -> LDS as f16 (or quantised), [token][k]
         const int awid = wid - NWD, atid = tid - 64 * NWD;
-        auto fetch = [&](int unit, float4_t & v0, float4_t & v1) {
-            const int t = unit_token(unit), u = unit - t * upr;
-            const float4_t * xp = (const float4_t *) ((const float *) (xb + (uint64_t) t * a.nb11) + 8 * u);
-            v0 = xp[0]; v1 = xp[1];
-        };
-        auto fetch_gain = [&](int unit, float4_t & g0, float4_t & g1) { // the norm weights of a unit's 8 columns
-            const float4_t * gp = (const float4_t *) (a.norm_w + 8 * (unit - unit_token(unit) * upr));
-            g0 = gp[0]; g1 = gp[1];
-        };
-        auto stage = [&](int unit, const float4_t & v0, const float4_t & v1, const float4_t & g0, const float4_t & g1) {
-            const int t = unit_token(unit), u = unit - t * upr;
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { v[i] = v0[i]; v[4 + i] = v1[i]; }
-            if constexpr (NORM) { // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
-                const float sc = nsc[t];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    v[i]     *= sc; v[i]     *= g0[i];
-                    v[4 + i] *= sc; v[4 + i] *= g1[i];
-                }
-            }
-            half8_t h;
-            if constexpr (ACT_Q8) { // 4 consecutive units = one 32-wide block
-                float amax = 0.0f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-                const float d  = amax / 127.f;
-                const float id = amax != 0.0f ? 127.f / amax : 0.0f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) h[i] = (_Float16) rintf(v[i] * id);
-                if ((u & 3) == 0) xd[(u >> 2) * 16 + t] = (float) (_Float16) d;
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) h[i] = (_Float16) v[i];
-            }
-            *(half8_t *) (xs + (size_t) t * KP + 8 * u) = h;
-        };
-        // A thread's units are requested together, up to UB of them, before the first is staged: a round trip per unit
-        // would be paid a dozen times with sixteen tokens.  When the threads' stride is a multiple of a row's units (the usual
-        // shapes) all units of a thread sit in the same columns and share their norm weights.
-        // (MANY: more than one unit per thread; the one-unit kernel keeps few enough registers for two work-groups per CU)
-        constexpr int UB = MANY ? (NW == 16 ? 4 : 8) : 1;
-        const bool same_cols = (64 * NA) % upr == 0; // uniform
-        float4_t f0[UB], f1[UB], g0 = {1, 1, 1, 1}, g1 = {1, 1, 1, 1};
-        if (!NORM && same_cols) {
+        float4_t f0[UB], f1[UB]; // this thread's first UB units, requested before the other work of the wave
+        if constexpr (!NORM) {
 #pragma unroll
             for (int i = 0; i < UB; ++i) {
-                const int unit = atid + i * 64 * NA;
+                const int unit = atid + i * USTRIDE;
                 if (unit < units) fetch(unit, f0[i], f1[i]);
             }
         }
@@ -864,75 +920,24 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
             }
         }
         if constexpr (NORM) { // a wave with several tokens takes two at a time
-            const int nv = (int) (a.K >> 8); // 16-byte pieces of a row per lane (K is a multiple of 256 here)
-            auto stage_row = [&](int t, const vx_rms_row & r, float sc) {
-#pragma unroll
-                for (int cc = 0; cc < 8; ++cc) {
-                    if (cc >= nv) break;
-                    const int    iv = lane + 64 * cc;
-                    const float4 g  = ((const float4 *) a.norm_w)[iv];
-                    // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
-                    float v[4] = { r.v[cc].x, r.v[cc].y, r.v[cc].z, r.v[cc].w };
-                    const float gg[4] = { g.x, g.y, g.z, g.w };
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { v[i] *= sc; v[i] *= gg[i]; }
-                    half4_t h;
-                    if constexpr (ACT_Q8) { // 8 consecutive lanes = one 32-wide block
-                        float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-                        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-                        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-                        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-                        const float d  = amax / 127.f;
-                        const float id = amax != 0.0f ? 127.f / amax : 0.0f;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) h[i] = (_Float16) rintf(v[i] * id);
-                        if ((lane & 7) == 0) xd[(iv >> 3) * 16 + t] = (float) (_Float16) d;
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) h[i] = (_Float16) v[i];
-                    }
-                    *(half4_t *) (xs + (size_t) t * KP + 4 * iv) = h;
-                }
-            };
-            for (int t = awid; t < N; t += 2 * NA) {
-                if (t != awid) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
-                if (t + NA < N) {
-                    if (t != awid) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (t + NA) * a.nb11), a.K, lane);
+            if (awid < N) { // the first pair: its rows were requested up front
+                if (awid + NA < N) {
                     float s1, s2;
                     vx_rms_row_scale2(nrow, nrow2, a.K, lane, a.norm_eps, s1, s2);
-                    stage_row(t, nrow, s1);
-                    stage_row(t + NA, nrow2, s2);
+                    stage_row(awid, nrow, s1);
+                    stage_row(awid + NA, nrow2, s2);
                 } else {
-                    stage_row(t, nrow, vx_rms_row_scale(nrow, a.K, lane, a.norm_eps));
+                    stage_row(awid, nrow, vx_rms_row_scale(nrow, a.K, lane, a.norm_eps));
                 }
             }
-        } else if (same_cols) {
+            for (int t = 2 * NW + awid; t < N; t += 2 * NA) norm_pair(t, NA); // (more than 2 NW tokens: four-wave work-groups only)
+        } else {
 #pragma unroll
             for (int i = 0; i < UB; ++i) {
-                const int unit = atid + i * 64 * NA;
-                if (unit < units) stage(unit, f0[i], f1[i], g0, g1);
+                const int unit = atid + i * USTRIDE;
+                if (unit < units) stage(unit, f0[i], f1[i]);
             }
-        }
-        if (NORM) { // (every row is staged)
-        } else if (same_cols) { // what is left after the first UB units of a thread: again UB requests together, then their staging
-            for (int base = atid + UB * 64 * NA; base < units; base += UB * 64 * NA) {
-#pragma unroll
-                for (int i = 0; i < UB; ++i) {
-                    const int unit = base + i * 64 * NA;
-                    if (unit < units) fetch(unit, f0[i], f1[i]);
-                }
-#pragma unroll
-                for (int i = 0; i < UB; ++i) {
-                    const int unit = base + i * 64 * NA;
-                    if (unit < units) stage(unit, f0[i], f1[i], g0, g1);
-                }
-            }
-        } else {
-            for (int unit = atid; unit < units; unit += 64 * NA) {
-                fetch(unit, f0[0], f1[0]);
-                if constexpr (NORM) fetch_gain(unit, g0, g1);
-                stage(unit, f0[0], f1[0], g0, g1);
-            }
+            stage_rest(atid + UB * USTRIDE);
         }
     }
     __syncthreads();
