@@ -879,6 +879,21 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
                     if (4 * j + r < N) resv[r] = *(const float *) (rb + (uint64_t) (4 * j + r) * a.rnb1);
             }
         }
+        if constexpr (SEG) { // the rotation's cos / sin, four token slots per lane: arithmetic that waits for nothing, done
+                             // by these waves while their requests are under way (the other waves have the tokens' rows)
+            if (rope && wid < 4) {
+                int  row_c, pair_c;
+                bool ok_c;
+                const char * wrow_c;
+                column(c, row_c, pair_c, ok_c, wrow_c);
+                const float ffv = a.ff ? a.ff[pair_c] : 1.0f;
+                for (int slot = wid; slot < 4; slot += NWD) {
+                    float cv = 1.0f, sv = 0.0f;
+                    if (ok_c && 4 * j + slot < N) rope_cos_sin(a.rp, (float) a.pos[(tok0 + 4 * j + slot) % a.rope_T], pair_c, ffv, cv, sv);
+                    rcs[slot * 64 + lane] = float2{cv, sv};
+                }
+            }
+        }
         if constexpr (NORM) { // (requested behind the weights, these rows arrive behind them)
             if (2 * NA + wid < N) norm_pair(2 * NA + wid, NWD);
         }
@@ -902,22 +917,6 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
         if constexpr (NORM) {
             if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
             if (awid + NA < N) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (awid + NA) * a.nb11), a.K, lane);
-        }
-        if constexpr (SEG) { // the rotation's cos / sin: the waves share the four token slots of every lane
-            if (rope && (NA >= 4 ? awid >= NA - 4 : true)) {
-                int  row_c, pair_c;
-                bool ok_c;
-                const char * wrow_c;
-                column(c, row_c, pair_c, ok_c, wrow_c);
-                const float ffv = a.ff ? a.ff[pair_c] : 1.0f;
-                // token slots are dealt from the last wave down: the first waves are the ones that normalise tokens, and with
-                // few tokens the slots that hold any (the low ones) then go to waves that have nothing else to do
-                for (int slot = (NA - 1 - awid) & 3; slot < 4; slot += NA) {
-                    float cv = 1.0f, sv = 0.0f;
-                    if (ok_c && 4 * j + slot < N) rope_cos_sin(a.rp, (float) a.pos[(tok0 + 4 * j + slot) % a.rope_T], pair_c, ffv, cv, sv);
-                    rcs[slot * 64 + lane] = float2{cv, sv};
-                }
-            }
         }
         if constexpr (NORM) { // a wave with several tokens takes two at a time
             if (awid < N) { // the first pair: its rows were requested up front
