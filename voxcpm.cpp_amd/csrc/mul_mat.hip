@@ -808,12 +808,18 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     // Tokens are dealt in pairs: the first 2 NA to the activation waves (t, t + NA), the next 2 NWD to the waves that fetch
     // the weights (they have nothing to do while their requests are under way), anything beyond to the activation waves again.
         const int nv = (int) (a.K >> 8); // 16-byte pieces of a row per lane (K is a multiple of 256 here)
-        auto stage_row = [&](int t, const vx_rms_row & r, float sc) {
+        // the norm weights of this lane's columns: requested with the rows, in registers when the scale is known
+        auto load_gains = [&](vx_rms_row & gn) {
+#pragma unroll
+            for (int cc = 0; cc < 8; ++cc)
+                if (cc < nv) gn.v[cc] = ((const float4 *) a.norm_w)[lane + 64 * cc];
+        };
+        auto stage_row = [&](int t, const vx_rms_row & r, float sc, const vx_rms_row & gn) {
 #pragma unroll
             for (int cc = 0; cc < 8; ++cc) {
                 if (cc >= nv) break;
                 const int    iv = lane + 64 * cc;
-                const float4 g  = ((const float4 *) a.norm_w)[iv];
+                const float4 g  = gn.v[cc];
                 // RMS_NORM's product, then the MUL node's, each rounded as the separate kernels round them
                 float v[4] = { r.v[cc].x, r.v[cc].y, r.v[cc].z, r.v[cc].w };
                 const float gg[4] = { g.x, g.y, g.z, g.w };
@@ -838,16 +844,18 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
             }
         };
     auto norm_pair = [&](int t, int stride) { // tokens t and t + stride (if there is one) by this wave
-        vx_rms_row r1, r2;
+        vx_rms_row r1, r2, gn;
         vx_rms_row_load(r1, (const float *) (xb + (uint64_t) t * a.nb11), a.K, lane);
         if (t + stride < N) {
             vx_rms_row_load(r2, (const float *) (xb + (uint64_t) (t + stride) * a.nb11), a.K, lane);
+            load_gains(gn);
             float s1, s2;
             vx_rms_row_scale2(r1, r2, a.K, lane, a.norm_eps, s1, s2);
-            stage_row(t, r1, s1);
-            stage_row(t + stride, r2, s2);
+            stage_row(t, r1, s1, gn);
+            stage_row(t + stride, r2, s2, gn);
         } else {
-            stage_row(t, r1, vx_rms_row_scale(r1, a.K, lane, a.norm_eps));
+            load_gains(gn);
+            stage_row(t, r1, vx_rms_row_scale(r1, a.K, lane, a.norm_eps), gn);
         }
     };
 
@@ -913,20 +921,21 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
         // With a fused norm a token's row belongs to ONE wave, as in the RMS_NORM kernel: the wave reads the row once, sums
         // its squares, and stages the normalised row from the registers it already holds -- no second trip for the values,
         // no exchange of scales between the waves.  Lane l holds columns 4 (l + 64 c) .. + 3 of the row.
-        vx_rms_row nrow, nrow2; // the tokens this wave normalises first, requested up front
+        vx_rms_row nrow, nrow2, ngain; // the tokens this wave normalises first (and the norm weights), requested up front
         if constexpr (NORM) {
             if (awid < N) vx_rms_row_load(nrow, (const float *) (xb + (uint64_t) awid * a.nb11), a.K, lane);
             if (awid + NA < N) vx_rms_row_load(nrow2, (const float *) (xb + (uint64_t) (awid + NA) * a.nb11), a.K, lane);
+            if (awid < N) load_gains(ngain);
         }
         if constexpr (NORM) { // a wave with several tokens takes two at a time
             if (awid < N) { // the first pair: its rows were requested up front
                 if (awid + NA < N) {
                     float s1, s2;
                     vx_rms_row_scale2(nrow, nrow2, a.K, lane, a.norm_eps, s1, s2);
-                    stage_row(awid, nrow, s1);
-                    stage_row(awid + NA, nrow2, s2);
+                    stage_row(awid, nrow, s1, ngain);
+                    stage_row(awid + NA, nrow2, s2, ngain);
                 } else {
-                    stage_row(awid, nrow, vx_rms_row_scale(nrow, a.K, lane, a.norm_eps));
+                    stage_row(awid, nrow, vx_rms_row_scale(nrow, a.K, lane, a.norm_eps), ngain);
                 }
             }
             for (int t = 2 * NW + awid; t < N; t += 2 * NA) norm_pair(t, NA); // (more than 2 NW tokens: four-wave work-groups only)
