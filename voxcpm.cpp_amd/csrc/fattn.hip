@@ -491,10 +491,10 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
     constexpr int DU = D / 4;       // lanes per row
     constexpr int PH = 64 / DU;     // split phases
     constexpr int NB = 16;          // rows a lane has in flight
-    const int tile = blockIdx.x >> 4, c = blockIdx.x & 15;
-    const int ct = tile % a.n_col_tiles;
-    const int bg = tile / a.n_col_tiles;
-    const int g = bg % a.Hkv, b = bg / a.Hkv;
+    // the grid is (16 columns x column tile, batch entry x KV head): no division of a flat index
+    const int c = blockIdx.x & 15, ct = blockIdx.x >> 4, bg = blockIdx.y;
+    const int tile = bg * a.n_col_tiles + ct;
+    const int b = fa_div(bg, a.inv_hkv), g = bg - b * a.Hkv;
     const int col = ct * 16 + c;
     if (col >= a.n_q * a.gqa) return; // whole block
     // With the cache write folded in the block has a second wave: it stores the slots (block 0), forms the two sums
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
     __shared__ float kvs_addend;
     if (threadIdx.x >= 64) {
         const int  lane1 = threadIdx.x - 64;
-        const bool store = blockIdx.x == 0;
+        const bool store = blockIdx.x == 0 && blockIdx.y == 0;
         double tk, tv;
         if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
         else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
@@ -930,7 +930,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     else         { if (f32) launch_cols16<128, true>(a, st); else launch_cols16<128, false>(a, st); }
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
-        const dim3 grid((unsigned) (tiles * 16));
+        const dim3 grid((unsigned) (a.n_col_tiles * 16), (unsigned) (a.ne3 * a.Hkv));
         const dim3 mblock(a.has_kvs ? 128 : 64); // the second wave carries the folded cache write
         if (D == 64) fattn_merge_kernel<64><<<grid, mblock, 0, st>>>(a);
         else         fattn_merge_kernel<128><<<grid, mblock, 0, st>>>(a);
