@@ -337,3 +337,39 @@ def test_weight_placement_policy(pkg):
     for fn in ("ggml_backend_gfx950_weight_on_device", "ggml_backend_gfx950_alloc_weights", "ggml_backend_gfx950_last_launches"):
         assert ggml.ggml_backend_reg_get_proc_address(reg(), fn.encode())
     assert not ggml.ggml_backend_reg_get_proc_address(reg(), b"no_such_function")
+
+
+def test_index_division_by_reciprocal_is_exact():
+    """The attention kernels divide small indices (column / heads per group, grid z / KV heads) as
+    (int) ((x + 0.5f) * (1.0f / d)) in single precision; the matrix kernels divide a unit number by the units per row
+    the same way.  Exact for every 0 <= x < 2^22 (the kernels refuse larger launches): checked here over the whole range
+    for the divisors the path meets and for awkward ones, in the same float32 arithmetic."""
+    x = np.arange(1 << 22, dtype=np.int64)
+    xf = x.astype(np.float32) + np.float32(0.5)
+    for d in (1, 2, 3, 5, 6, 7, 8, 12, 16, 24, 40, 64, 96, 127, 128, 512, 1000, 4099):
+        inv = np.float32(1.0) / np.float32(d)
+        got = (xf * inv).astype(np.int64)   # float32 product, truncated like the kernel's conversion
+        assert np.array_equal(got, x // d), d
+
+
+def test_row_rotations_reproduce_the_xor_butterfly():
+    """A wave sum's steps 32, 16, 8, 4, 2, 1: the kernels take the last four as rotations within rows of 16 lanes
+    (lane i reads lane (i + s) mod 16 of its row) instead of the xor partner i ^ s.  The same bits: when step s is reached
+    the values repeat every 2 s lanes.  Simulated here in float64 and float32 on random and on badly conditioned values."""
+    rng = np.random.default_rng(7)
+    lanes = np.arange(64)
+    for dtype in (np.float64, np.float32):
+        for trial in range(50):
+            v = rng.standard_normal(64).astype(dtype)
+            if trial % 5 == 0:
+                v = (v * dtype(10.0) ** rng.integers(-6, 7, 64).astype(dtype)).astype(dtype)
+            a = v.copy()
+            for s in (32, 16, 8, 4, 2, 1):
+                a = (a + a[lanes ^ s]).astype(dtype)
+            b = v.copy()
+            for s in (32, 16):
+                b = (b + b[lanes ^ s]).astype(dtype)
+            for s in (8, 4, 2, 1):
+                b = (b + b[(lanes & ~15) | ((lanes + s) & 15)]).astype(dtype)
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), (dtype, trial)
+            assert len(set(a.tolist())) == 1   # every lane holds the same total
