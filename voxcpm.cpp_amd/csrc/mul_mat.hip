@@ -705,8 +705,11 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     const int NL = (int) (a.N < 16 ? a.N : 16);
     _Float16 * xs  = (_Float16 *) gv_smem;                                   // [N][KP]
     float *    xd  = (float *) (gv_smem + (size_t) NL * KP * 2);             // [K/32][16 tokens] (ACT_Q8): the activations' block scales
-    float4_t * red = (float4_t *) (gv_smem + (size_t) NL * KP * 2 + (ACT_Q8 ? (size_t) 16 * nkb * 4 : 0));
-    float *    nsc = (float *) (red + (NW - 1) * 64);                        // [16] per-token 1 / rms (fused RMS_NORM)
+    // the waves' partial sums take the activations' place once every wave has walked its blocks (sixteen tokens of K = 4096
+    // and the partials of sixteen waves do not fit a CU's LDS side by side); the region holds whichever is larger
+    float4_t * red = (float4_t *) gv_smem;
+    const size_t act_bytes = (size_t) NL * KP * 2 + (ACT_Q8 ? (size_t) 16 * nkb * 4 : 0), red_bytes = (size_t) (NW - 1) * 64 * 16;
+    float *    nsc = (float *) (gv_smem + (act_bytes > red_bytes ? act_bytes : red_bytes)); // [16] (unused: kept for the layout)
     float2 *   rcs = (float2 *) (nsc + 16);                                  // [4][64] cos / sin of four token slots (SEG)
     const char * w_lds = gv_smem + a.w_lds_off;
 
@@ -1005,6 +1008,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_dma_kernel(const mm_args a) {
     bool         row_ok;
     const char * wrow;
     column(c, row, pair, row_ok, wrow);
+    __syncthreads(); // every wave is done with the staged activations: their place takes the partial sums
     if (wid > 0) red[(wid - 1) * 64 + lane] = acc;
     __syncthreads();
     if (wid > 0) return;
@@ -1055,7 +1059,8 @@ constexpr size_t GV_ROPE_LDS = 4 * 64 * 8;     // cos / sin of four token slots 
 bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
     static const int64_t max_tokens = [] { const char * e = getenv("VX_GEMV_MAX_TOKENS"); const int n = e ? atoi(e) : 0; return n >= 16 ? (int64_t) n : (int64_t) 1 << 30; }();
     if (K % 32 || K < 32 || N < 1) return false;
-    if (N > 16 && (N > max_tokens || N * rows > 256 * 1024)) return false;
+    static const int64_t max_work = [] { const char * e = getenv("VX_GEMV_MAX_WORK"); const long n = e ? atol(e) : 0; return n > 0 ? (int64_t) n : (int64_t) 256 * 1024; }();
+    if (N > 16 && (N > max_tokens || N * rows > max_work)) return false;
     // chunks of 16 tokens each stage 16 x K activations: with a long K a work-group fills a CU's LDS alone and the chunks
     // queue up behind each other (1024 rows x K = 4096 at 112 tokens: 63 us against 26 us on the tiled kernel with its K cut)
     if (N > 16 && K > 2048) return false;
@@ -1065,8 +1070,9 @@ bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
 
 size_t gemv_smem(const mm_args & a, bool act_q8, int nw, bool dma = false) {
     const size_t nl = (size_t) (a.N < 16 ? a.N : 16);
-    return nl * (a.K + (dma ? 8 : 0)) * 2 + (act_q8 ? (dma ? 16 : nl) * (a.K / 32) * 4 : 0) + (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16 + 16 * sizeof(float) +
-           (a.nseg > 0 ? GV_ROPE_LDS : 0);
+    const size_t act = nl * (a.K + (dma ? 8 : 0)) * 2 + (act_q8 ? (dma ? 16 : nl) * (a.K / 32) * 4 : 0), red = (size_t) (nw > 1 ? nw - 1 : 0) * 64 * 16;
+    // (gemv_dma_kernel puts the partial sums where the activations were)
+    return (dma ? (act > red ? act : red) : act + red) + 16 * sizeof(float) + (a.nseg > 0 ? GV_ROPE_LDS : 0);
 }
 
 // gemv_dma_kernel's weight image: bytes between consecutive columns.  The padding is chosen so that the dword reads of the
