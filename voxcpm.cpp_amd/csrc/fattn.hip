@@ -52,11 +52,12 @@ struct fa_args {
     uint64_t nbq1, nbq2, nbq3, nbk1, nbk2, nbk3, nbv1, nbv2, nbv3, nbm1, nbm2, nbm3;
     // keys n_kv1 .. n_kv-1 may lie in a second pair of tensors (the current step's K and V, which the
     // reference appends to the cached ones with GGML_OP_CONCAT before attention); null = one segment
-    // the reference's cache write with its ordering scalar folded into the merge kernel (has_kvs):
+    // the reference's cache write with its ordering scalar folded in (has_kvs): an extra block of the first kernel does it,
     // block 0 stores both slots, every block forms the two sums and adds the scalar to its column
     kvs_side kvs_k, kvs_v;
     float kvs_scale, kvs_bias;
     int has_kvs;
+    float * kvs_out; // the scalar, written by the first kernel's extra block and read by every merge block
     const char * k2; const char * v2;
     uint64_t nbk1b, nbk2b, nbk3b, nbv1b, nbv2b, nbv3b;
     int n_kv1;
@@ -148,8 +149,25 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     const int lane = threadIdx.x;
     const int j = lane >> 4, c = lane & 15;
 
+    // With the cache write folded in, the grid has one more slice in front: its first wave stores the slots, forms the
+    // two sums and leaves the scalar for the merge kernel; the slice's other waves have nothing to do.  (One wave reads
+    // the step's keys and values: when every merge block formed the sums itself, sixteen streams' 512 blocks asked the
+    // same few cache lines at once and the merge took 9 us instead of 4.)
+    if constexpr (TWO_SEG != 0) {
+        if (a.has_kvs && blockIdx.z == 0) {
+            if (blockIdx.x == 0 && blockIdx.y == 0) {
+                double tk, tv;
+                if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
+                else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
+                else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
+                else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
+                if (lane == 0) *a.kvs_out = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
+            }
+            return;
+        }
+    }
     // the grid is (column tile, key range, batch entry x KV head): dispatched in the same order as one flat index
-    const int ct = blockIdx.x, sp = blockIdx.y, bg = blockIdx.z;
+    const int ct = blockIdx.x, sp = blockIdx.y, bg = (int) blockIdx.z - ((TWO_SEG != 0 && a.has_kvs) ? 1 : 0);
     const int b  = fa_div(bg, a.inv_hkv);
     const int g  = bg - b * a.Hkv;
     const int tile = bg * a.n_col_tiles + ct;
@@ -487,7 +505,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
 // between the phases and a store.
 constexpr int FA_MERGE_MAX_SPLITS = 256;
 template <int D>
-__global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
+__global__ __launch_bounds__(64) void fattn_merge_kernel(const fa_args a) {
     constexpr int DU = D / 4;       // lanes per row
     constexpr int PH = 64 / DU;     // split phases
     constexpr int NB = 16;          // rows a lane has in flight
@@ -497,24 +515,13 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
     const int b = fa_div(bg, a.inv_hkv), g = bg - b * a.Hkv;
     const int col = ct * 16 + c;
     if (col >= a.n_q * a.gqa) return; // whole block
-    // With the cache write folded in the block has a second wave: it stores the slots (block 0), forms the two sums
-    // (a chain of fp64 cross-lane steps) and hands over the scalar, while the first wave merges.
-    __shared__ float kvs_addend;
-    if (threadIdx.x >= 64) {
-        const int  lane1 = threadIdx.x - 64;
-        const bool store = blockIdx.x == 0 && blockIdx.y == 0;
-        double tk, tv;
-        if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
-        else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
-        else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
-        else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane1, store, tk, tv);
-        if (lane1 == 0) kvs_addend = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
-        __syncthreads();
-        return;
-    }
     const int lane = threadIdx.x, q = lane / DU, d0 = 4 * (lane % DU);
-    bool  has_addend = a.add1 != nullptr;
-    float addend     = has_addend ? *a.add1 : 0.0f;
+    // (with the cache write folded in, the addend is the scalar that the first kernel's extra block left: when every
+    // merge block formed the sums itself in a second wave, sixteen streams' 512 blocks asked the same few cache lines at
+    // once and the merge took 9 us instead of 4)
+    const float * addend_p   = a.has_kvs ? a.kvs_out : a.add1;
+    const bool    has_addend = addend_p != nullptr;
+    const float   addend     = has_addend ? *addend_p : 0.0f;
     const uint64_t tbase = (uint64_t) tile * a.n_splits * 16 + c; // + split * 16
     // A lane works on the splits of its phase only: q, q + PH, q + 2 PH, ...  It reads their (max, sum) pairs and rows itself
     // and forms their weights itself, so the only cross-lane traffic is between the PH phases (log2 PH steps for the maximum,
@@ -565,11 +572,6 @@ __global__ __launch_bounds__(128) void fattn_merge_kernel(const fa_args a) {
         L += __shfl_xor(L, off, 64);
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], off, 64);
-    }
-    if (a.has_kvs) { // uniform: the block was launched with its second wave
-        __syncthreads();
-        addend     = kvs_addend;
-        has_addend = true;
     }
     if (q == 0) {
         const int  iq1 = fa_div(col, a.inv_gqa), head = g * a.gqa + (col - iq1 * a.gqa);
@@ -628,7 +630,7 @@ int64_t fa_tiles(const vx_tensor * q, const vx_tensor * k) {
 
 template <int D, bool KV_F32>
 void launch_cols16(const fa_args & a, hipStream_t st) {
-    const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv)), block(64);
+    const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv + (a.has_kvs ? 1 : 0))), block(64);
     if constexpr (D == 64 && !KV_F32) {
         if (a.k2 && a.seg2_f32) { // an F16 cache and the step's F32 keys
             if (a.softcap != 0.0f) fattn_cols16_kernel<D, false, true, true, 2><<<grid, block, 0, st>>>(a);
@@ -668,7 +670,7 @@ extern "C" int vx_supports_flash_attn_ext(const vx_tensor * q, const vx_tensor *
     if (k->ne[0] != D || v->ne[0] != D) return 0;
     if (k->ne[1] != v->ne[1] || k->ne[2] != v->ne[2] || k->ne[3] != v->ne[3]) return 0;
     if (q->ne[2] % k->ne[2] || q->ne[3] % k->ne[3]) return 0;
-    if (q->ne[3] * k->ne[2] > 65535) return 0; // (batch entry x KV head is one dimension of the grid)
+    if (q->ne[3] * k->ne[2] > 65534) return 0; // (batch entry x KV head is one dimension of the grid, plus one slice for a folded cache write)
     if (q->nb[0] != 4 || k->nb[0] != vx_type_size(k->type) || v->nb[0] != vx_type_size(v->type)) return 0;
     // strides must keep 16-byte vector loads aligned; the data pointers are checked at launch
     for (int i = 1; i < 4; ++i)
@@ -862,7 +864,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
                         const vx_tensor * vs_slot, float kvs_scale, float kvs_bias, void * fixed_ws, size_t fixed_ws_bytes) {
     (void) vall;
     fa_args a;
-    a.has_kvs = 0;
+    a.has_kvs = 0; a.kvs_out = nullptr;
     a.k2 = k2 ? (const char *) k2->data : nullptr; a.v2 = v2 ? (const char *) v2->data : nullptr;
     a.nbk1b = k2 ? k2->nb[1] : 0; a.nbk2b = k2 ? k2->nb[2] : 0; a.nbk3b = k2 ? k2->nb[3] : 0;
     a.nbv1b = v2 ? v2->nb[1] : 0; a.nbv2b = v2 ? v2->nb[2] : 0; a.nbv3b = v2 ? v2->nb[3] : 0;
@@ -893,7 +895,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     const int ncols = a.n_q * a.gqa;
     a.n_col_tiles   = (ncols + 15) / 16;
     a.inv_gqa = 1.0f / (float) a.gqa; a.inv_hkv = 1.0f / (float) a.Hkv;
-    if (ncols >= (1 << 22) || (int64_t) a.ne3 * a.Hkv > 65535) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext: launch too large");
+    if (ncols >= (1 << 22) || (int64_t) a.ne3 * a.Hkv > 65534) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext: launch too large");
     const int64_t tiles = (int64_t) a.ne3 * a.Hkv * a.n_col_tiles;
 
     fa_split_plan(tiles, a.n_kv, &a.n_splits, &a.chunk);
@@ -911,7 +913,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
 
     if (a.n_splits > 1) {
         const size_t o_bytes  = (size_t) nblocks * 16 * D * sizeof(float);
-        const size_t ml_bytes = (size_t) nblocks * 16 * 2 * sizeof(float);
+        const size_t ml_bytes = (size_t) nblocks * 16 * 2 * sizeof(float) + (a.has_kvs ? 16 : 0); // (+ the folded cache write's scalar)
         void * ws = fixed_ws;
         if (fixed_ws) { // the caller's fixed block: nothing is allocated, larger shapes are refused
             if (o_bytes + ml_bytes > fixed_ws_bytes)
@@ -923,6 +925,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
         }
         a.part_o  = (float *) ws;
         a.part_ml = (float *) ((char *) ws + o_bytes);
+        a.kvs_out = a.has_kvs ? (float *) ((char *) ws + o_bytes + ml_bytes - 16) : nullptr;
     }
 
     const bool f32 = k->type == VX_TYPE_F32;
@@ -931,7 +934,7 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
         const dim3 grid((unsigned) (a.n_col_tiles * 16), (unsigned) (a.ne3 * a.Hkv));
-        const dim3 mblock(a.has_kvs ? 128 : 64); // the second wave carries the folded cache write
+        const dim3 mblock(64);
         if (D == 64) fattn_merge_kernel<64><<<grid, mblock, 0, st>>>(a);
         else         fattn_merge_kernel<128><<<grid, mblock, 0, st>>>(a);
         VX_LAUNCH_CHECK();
