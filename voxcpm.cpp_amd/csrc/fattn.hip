@@ -149,19 +149,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void fa
     const int lane = threadIdx.x;
     const int j = lane >> 4, c = lane & 15;
 
-    // With the cache write folded in, the grid has one more slice in front: its first wave stores the slots, forms the
-    // two sums and leaves the scalar for the merge kernel; the slice's other waves have nothing to do.  (One wave reads
+    // With the cache write folded in, the grid has one more slice in front: its first wave forms the two sums and leaves
+    // the scalar for the merge kernel, its other waves store the slots.  (One wave reads
     // the step's keys and values: when every merge block formed the sums itself, sixteen streams' 512 blocks asked the
     // same few cache lines at once and the merge took 9 us instead of 4.)
     if constexpr (TWO_SEG != 0) {
         if (a.has_kvs && blockIdx.z == 0) {
-            if (blockIdx.x == 0 && blockIdx.y == 0) {
+            if (blockIdx.x != 0) return;
+            if (blockIdx.y == 0) { // the sums, in GGML_OP_SUM's order, by one wave (no stores: their index arithmetic is the others' work)
                 double tk, tv;
-                if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
-                else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
-                else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
-                else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane, true, tk, tv);
+                if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+                else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+                else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+                else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
                 if (lane == 0) *a.kvs_out = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
+            } else { // the stores, dealt over the slice's other waves (there are n_splits - 1 >= 1 of them)
+                const uint32_t first = (blockIdx.y - 1) * 64 + lane, step = (gridDim.y - 1) * 64;
+                double unused = 0.0;
+                const uint32_t nk = kvs_units(a.kvs_k, a.kvs_k.vec != 0), nv = kvs_units(a.kvs_v, a.kvs_v.vec != 0);
+                if (a.kvs_k.vec) { for (uint32_t e = first; e < nk; e += step) kvs_unit<true>(a.kvs_k, e, true, unused); }
+                else             { for (uint32_t e = first; e < nk; e += step) kvs_unit<false>(a.kvs_k, e, true, unused); }
+                if (a.kvs_v.vec) { for (uint32_t e = first; e < nv; e += step) kvs_unit<true>(a.kvs_v, e, true, unused); }
+                else             { for (uint32_t e = first; e < nv; e += step) kvs_unit<false>(a.kvs_v, e, true, unused); }
             }
             return;
         }
