@@ -1292,12 +1292,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // token tiles are partitioned over the XCDs (tile ty goes to XCD ty % 8) and inside an XCD the row
     // tiles of one token tile run side by side: its activations are fetched into that L2 once, and the
     // weights stream through it once per couple of token tiles instead of once per work-group.
+    // (with fewer than 8 token tiles the row tiles are dealt over the XCDs instead: no XCD without work)
     const int64_t gx = (a.M + 127) / 128, gy = (a.N + 127) / 128;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int64_t ty = (slot / gx) * 8 + xcd;
-    if (ty >= gy) return; // padding of the last group of 8 token tiles (whole work-group)
+    int64_t ty, tx;
+    if (gy >= 8) { ty = (slot / gx) * 8 + xcd; tx = slot % gx; }
+    else         { ty = slot % gy; tx = (slot / gy) * 8 + xcd; }
+    if (ty >= gy || tx >= gx) return; // padding of the last group of 8 tiles (whole work-group)
     const int64_t tok0 = ty * 128;
-    const int64_t row0 = (slot % gx) * 128 + wr * 64;
+    const int64_t row0 = tx * 128 + wr * 64;
     // addresses are (uniform base + uniform round offset) + a 32-bit lane offset that never changes, so the
     // loads take a scalar base and no per-load vector address arithmetic (the launcher checks the ranges)
     uint32_t woff[4];
@@ -1466,7 +1469,7 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
     if (WT == WT_F32 || a.K % 32 || a.K < 32 || a.N < 128) return false;
     const int64_t gx = (a.M + 127) / 128, gy = (a.N + 127) / 128;
     if (gx * gy * nbatch < 192) return false; // small problems spread wider on the 64 x 64 tiles
-    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
+    const int64_t blocks = gy >= 8 ? gx * ((gy + 7) / 8) * 8 : ((gx + 7) / 8) * 8 * gy; // (the kernel's two ways of dealing tiles to XCDs)
     if (blocks > 0x7fffffff) return false;
     // 32-bit lane offsets inside the kernel: rows of the weight matrix and the 128 tokens of a tile
     if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 128 * a.nb11 + 256 >= (1ull << 32)) return false;
@@ -1516,13 +1519,18 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
 
-    // token tiles partitioned over the XCDs, row tiles of one token tile side by side (see gemm128_kernel)
+    // token tiles partitioned over the XCDs, row tiles of one token tile side by side (see gemm128_kernel).  With fewer
+    // than 8 token tiles that would leave XCDs without work (112 tokens are 2 tiles: a quarter of the chip, and three empty
+    // blocks dispatched for every working one): then the ROW tiles are dealt over the XCDs and a row tile's few token tiles
+    // sit side by side on one, where they share the weight rows in its L2.
     const int64_t gx = (a.M + ROWS - 1) / ROWS, gy = (a.N + TOKS - 1) / TOKS;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int64_t ty = (slot / gx) * 8 + xcd;
-    if (ty >= gy) return;
+    int64_t ty, tx;
+    if (gy >= 8) { ty = (slot / gx) * 8 + xcd; tx = slot % gx; }
+    else         { ty = slot % gy; tx = (slot / gy) * 8 + xcd; }
+    if (ty >= gy || tx >= gx) return;
     const int64_t tok0 = ty * TOKS;
-    const int64_t rowg = (slot % gx) * ROWS;
+    const int64_t rowg = tx * ROWS;
     const int64_t nround = a.K / (32 * GL_KC); // the launcher takes whole rounds only
 
     // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
@@ -1719,7 +1727,7 @@ template <int WT, bool FOLD, int RT, int CT, int WR, int WC>
 bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
     constexpr size_t lds = gl_lds(RT * WR, CT * WC);
     const int64_t gx = (a.M + 16 * RT * WR - 1) / (16 * RT * WR), gy = (a.N + 16 * CT * WC - 1) / (16 * CT * WC);
-    const int64_t blocks = gx * ((gy + 7) / 8) * 8;
+    const int64_t blocks = gy >= 8 ? gx * ((gy + 7) / 8) * 8 : ((gx + 7) / 8) * 8 * gy; // (the kernel's two ways of dealing tiles to XCDs)
     if (blocks > 0x7fffffff) return false;
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
