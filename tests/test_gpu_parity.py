@@ -408,7 +408,10 @@ def mm_inputs(tag, M, K, N, batch=()):
                                    # operands through LDS: ragged rows and tokens on 128 x 128 and 64 x 64 tiles, few rows
                                    (2000, 1024, 1700), (1000, 1024, 333), (64, 1024, 4100), (130, 2048, 9000),
                                    # a long K on a small grid: K cut across work-groups, partials added by a second kernel
-                                   (1024, 4096, 600), (1000, 2176, 300)])
+                                   (1024, 4096, 600), (1000, 2176, 300),
+                                   # the same on the LDS-operand kernel when its 64 x 64 tiles are few (the down-projection of
+                                   # 8 requests' 112 tokens): 8, 8 and 4 splits, ragged rows and tokens
+                                   (1024, 4096, 112), (1000, 4096, 70), (512, 2048, 64)])
 def test_mul_mat_q8_0(gpu, M, K, N):
     say(f"mul_mat Q8_0 M={M} K={K} N={N}")
     w, x = mm_inputs(("q8", M, K, N), M, K, N)

@@ -1513,11 +1513,19 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     const int j = lane >> 4, c = lane & 15;
     const int wr = wid / WC, wt = wid % WC;
 
-    const int     batch = blockIdx.z;
+    // a long K on a grid of few tiles is cut across nsplit work-groups (blockIdx.z = batch x split): each leaves its share
+    // in its slab of the partial buffer, dense [token][row], for mm_splitk_reduce_kernel to add in split order
+    const int     nsplit = a.ksplit > 1 ? a.ksplit : 1; // uniform
+    const int     batch = (int) blockIdx.z / nsplit, split = (int) blockIdx.z % nsplit;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
     const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    uint64_t      dnb1 = a.nb1;
+    if (nsplit > 1) {
+        db   = (char *) (a.partial + ((uint64_t) batch * nsplit + split) * (uint64_t) a.N * a.M);
+        dnb1 = (uint64_t) a.M * 4;
+    }
 
     // token tiles partitioned over the XCDs, row tiles of one token tile side by side (see gemm128_kernel).  With fewer
     // than 8 token tiles that would leave XCDs without work (112 tokens are 2 tiles: a quarter of the chip, and three empty
@@ -1531,7 +1539,9 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     if (ty >= gy || tx >= gx) return;
     const int64_t tok0 = ty * TOKS;
     const int64_t rowg = tx * ROWS;
-    const int64_t nround = a.K / (32 * GL_KC); // the launcher takes whole rounds only
+    // the launcher takes whole rounds only, and an even number of them per split (a round's register set and LDS buffer
+    // are its parity)
+    const int64_t rounds_all = a.K / (32 * GL_KC), rbeg = rounds_all / nsplit * split, nround = rbeg + rounds_all / nsplit;
 
     // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
     // products are computed and dropped), so no load carries a predicate.  They are buffer loads: a uniform
@@ -1668,9 +1678,9 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // round's MFMAs to arrive before it is converted.
     using set0 = std::integral_constant<int, 0>;
     using set1 = std::integral_constant<int, 1>;
-    load_weights(0, set0{});
-    load_acts(0, set0{});
-    if (nround > 1) { load_weights(1, set1{}); load_acts(1, set1{}); }
+    load_weights(rbeg, set0{});
+    load_acts(rbeg, set0{});
+    if (rbeg + 1 < nround) { load_weights(rbeg + 1, set1{}); load_acts(rbeg + 1, set1{}); }
     store_weights(0, set0{});
     store_acts(0, set0{});
     __syncthreads();
@@ -1689,7 +1699,7 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
         if (round + 1 < nround) { store_weights(buf ^ 1, other{}); store_acts(buf ^ 1, other{}); }
         __syncthreads();
     };
-    for (int64_t round = 0; round < nround; round += 2) {
+    for (int64_t round = rbeg; round < nround; round += 2) {
         one_round(round, set0{});
         if (round + 1 < nround) one_round(round + 1, set1{});
     }
@@ -1697,13 +1707,13 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // lane (j,c), tile (rt, tt), register r: token tok0 + 16 (CT wt + tt) + 4j + r, row rowg + 16 (RT wr + rt) + c
     if (tok0 + TOKS <= a.N && rowg + ROWS <= a.M) { // uniform: a tile inside the matrix stores without tests,
         // at a uniform base plus one 32-bit lane offset (the launcher checks the range)
-        char * tb = db + (uint64_t) tok0 * a.nb1 + (uint64_t) rowg * 4;
-        const uint32_t loff = (uint32_t) ((uint64_t) (16 * CT * wt + 4 * j) * a.nb1 + (uint64_t) (16 * RT * wr + c) * 4);
+        char * tb = db + (uint64_t) tok0 * dnb1 + (uint64_t) rowg * 4;
+        const uint32_t loff = (uint32_t) ((uint64_t) (16 * CT * wt + 4 * j) * dnb1 + (uint64_t) (16 * RT * wr + c) * 4);
 #pragma unroll
         for (int tt = 0; tt < CT; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                char * tr = tb + (uint64_t) (16 * tt + r) * a.nb1; // uniform
+                char * tr = tb + (uint64_t) (16 * tt + r) * dnb1; // uniform
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) *(float *) (tr + 64 * rt + loff) = acc[rt][tt][r];
             }
@@ -1718,7 +1728,7 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t tok = tok0 + 16 * (CT * wt + tt) + 4 * j + r;
-                if (tok < a.N) *(float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4) = acc[rt][tt][r];
+                if (tok < a.N) *(float *) (db + (uint64_t) tok * dnb1 + (uint64_t) row * 4) = acc[rt][tt][r];
             }
     }
 }
@@ -1737,7 +1747,8 @@ bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
         }
         raised = true;
     }
-    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC><<<dim3((unsigned) blocks, 1, (unsigned) nbatch), dim3(64 * WR * WC), lds, st>>>(a);
+    const int nsplit = a.ksplit > 1 ? a.ksplit : 1;
+    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC><<<dim3((unsigned) blocks, 1, (unsigned) (nbatch * nsplit)), dim3(64 * WR * WC), lds, st>>>(a);
     return true;
 }
 
@@ -1758,7 +1769,24 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     const bool fold = WT == WT_Q8 && mode == 2;
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
-    if (!big && ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch < 64) return false;
+    const int64_t tiles64 = ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch;
+    if (!big && tiles64 < 64) {
+        // Few tiles and a long K (the down-projection of a hundred tokens: 32 tiles, 64 rounds): the K range is cut so
+        // that some 256 work-groups walk 8 or more rounds each, and a second kernel adds their partials in split order.
+        const int64_t rounds = a.K / (32 * GL_KC);
+        int ks = 1;
+        while (ks < 16 && tiles64 * ks < 192 && rounds % (4 * ks) == 0 && rounds / (2 * ks) >= 4) ks *= 2;
+        if (ks < 2 || a.M % 4 || (uintptr_t) a.dst % 16 || a.nb1 % 16 || a.nb2 % 16 || a.nb3 % 16 || (int64_t) nbatch * ks > 65535) return false;
+        void * ws = nullptr;
+        if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) != VX_OK) { (void) hipGetLastError(); return false; }
+        mm_args b = a;
+        b.ksplit = ks; b.partial = (float *) ws;
+        const bool ok = WT == WT_Q8 && mode == 2 ? launch_gemm_lds_tile<WT, WT == WT_Q8, 2, 2, 2, 2>(b, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(b, nbatch, st);
+        if (!ok) return false;
+        const int64_t units = a.N * (a.M / 4);
+        mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+        return true;
+    }
     // 128 x 128: 8 waves of 64 rows x 32 tokens (4 waves per SIMD with two work-groups per CU measured 5-10 % above
     // 4 waves of 64 x 64); 64 x 64: 4 waves of 32 x 32
     if constexpr (WT == WT_Q8) {
