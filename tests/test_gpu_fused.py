@@ -123,7 +123,9 @@ def test_mul_mat_swiglu(pkg, gpu, M, K, N, nb, act):
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 2048, 40, 2)])
+@pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 2048, 40, 2),
+                                      # a long K over few tiles: the tiled kernels with K cut, the update in the kernel that adds the partials
+                                      (1024, 4096, 112, 1), (1000, 4096, 70, 1)])
 @pytest.mark.parametrize("act", ["float", "q8"])
 def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     import torch

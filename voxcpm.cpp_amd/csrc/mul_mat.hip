@@ -300,6 +300,11 @@ __global__ __launch_bounds__(256) void mm_splitk_reduce_kernel(const mm_args a) 
     const float * p = a.partial + (uint64_t) batch * a.ksplit * (uint64_t) a.N * a.M + (uint64_t) tok * a.M + r4;
     float4_t acc = *(const float4_t *) p;
     for (int s = 1; s < a.ksplit; ++s) acc += *(const float4_t *) (p + (uint64_t) s * a.N * a.M);
+    if (a.res) { // the fused residual update: dst = res + scale * (W x), rounded as the SCALE and the ADD node would
+        const float * rp = (const float *) (a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) tok * a.rnb1 + (uint64_t) r4 * 4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = scaled_residual(acc[r], a.res_scale, rp[r]);
+    }
     *(float4_t *) (a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3 + (uint64_t) tok * a.nb1 + (uint64_t) r4 * 4) = acc;
 }
 
@@ -1767,6 +1772,7 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 256 * a.nb11 + 256 >= (1ull << 32) ||
         (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32) || a.K >= (1ll << 28)) return false;
     const bool fold = WT == WT_Q8 && mode == 2;
+    // (a residual update is fused into the kernel that adds a cut K's partials, nowhere else here)
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     const int64_t tiles64 = ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch;
@@ -1787,12 +1793,34 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
         mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
         return true;
     }
+    if (a.res) return false;
     // 128 x 128: 8 waves of 64 rows x 32 tokens (4 waves per SIMD with two work-groups per CU measured 5-10 % above
     // 4 waves of 64 x 64); 64 x 64: 4 waves of 32 x 32
     if constexpr (WT == WT_Q8) {
         if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2>(a, nbatch, st);
     }
     return big ? launch_gemm_lds_tile<WT, false, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(a, nbatch, st);
+}
+
+// A long K on a grid that leaves most CUs with one work-group is a chain of ~3 us rounds: cut K so that every split walks
+// about 1024 of it, and add the partials in a second launch (which also applies a fused residual update).
+template <int WT, bool ACT_Q8>
+bool launch_mm_cut(const mm_args & a, int nbatch, hipStream_t st) {
+    if (a.N <= 32) return false;
+    const int64_t gx = (a.M + 63) / 64, gy = (a.N + 63) / 64;
+    if (!(a.K >= 2048 && a.K % 128 == 0 && a.M % 4 == 0 && gx * gy * nbatch <= 512 && (uintptr_t) a.dst % 16 == 0 && a.nb1 % 16 == 0 &&
+          a.nb2 % 16 == 0 && a.nb3 % 16 == 0)) return false;
+    int ks = (int) (a.K / 1024);
+    if (ks > 8) ks = 8;
+    if (ks < 2 || (int64_t) nbatch * ks > 65535) return false;
+    void * ws = nullptr;
+    if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) != VX_OK) { (void) hipGetLastError(); return false; }
+    mm_args b = a;
+    b.ksplit = ks; b.partial = (float *) ws;
+    mm_kernel<WT, 4, ACT_Q8, false><<<dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st>>>(b);
+    const int64_t units = a.N * (a.M / 4);
+    mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+    return true;
 }
 
 template <int WT, bool ACT_Q8>
@@ -1807,27 +1835,8 @@ void launch(const mm_args & a, int nbatch, hipStream_t st) {
         const dim3 grid((unsigned) ((a.M + 63) / 64), 1, (unsigned) nbatch);
         mm_kernel<WT, 2, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
     } else {
-        // A long K on a grid that leaves most CUs with one work-group is a chain of ~3 us rounds: cut K so that every
-        // split walks about 1024 of it, and add the partials in a second launch.
+        if (launch_mm_cut<WT, ACT_Q8>(a, nbatch, st)) return;
         const int64_t gx = (a.M + 63) / 64, gy = (a.N + 63) / 64;
-        int ks = 1;
-        if (a.K >= 2048 && a.K % 128 == 0 && a.M % 4 == 0 && gx * gy * nbatch <= 512 && (uintptr_t) a.dst % 16 == 0 && a.nb1 % 16 == 0 &&
-            a.nb2 % 16 == 0 && a.nb3 % 16 == 0) {
-            ks = (int) (a.K / 1024);
-            if (ks > 8) ks = 8;
-        }
-        if (ks > 1 && (int64_t) nbatch * ks <= 65535) {
-            void * ws = nullptr;
-            if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) == VX_OK) {
-                mm_args b = a;
-                b.ksplit = ks; b.partial = (float *) ws;
-                mm_kernel<WT, 4, ACT_Q8, false><<<dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st>>>(b);
-                const int64_t units = a.N * (a.M / 4);
-                mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
-                return;
-            }
-            (void) hipGetLastError();
-        }
         const dim3 grid((unsigned) gx, (unsigned) gy, (unsigned) nbatch);
         mm_kernel<WT, 4, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
     }
@@ -1981,7 +1990,12 @@ extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_te
     // dst's shape, or one row / one matrix repeated over it (a bias: ggml_add repeats src1)
     for (int i = 1; i < 4; ++i) if (residual->ne[i] != dst->ne[i] && residual->ne[i] != 1) return 0;
     if (residual->nb[1] % 4 || residual->nb[2] % 4 || residual->nb[3] % 4) return 0;
-    return gemv_shape_ok(src1->ne[1], src0->ne[1], src0->ne[0]);
+    if (gemv_shape_ok(src1->ne[1], src0->ne[1], src0->ne[0])) return 1;
+    // a long K over few tiles (the down-projection of a hundred tokens): the product's K range is cut across work-groups
+    // and the kernel that adds the partials applies the update
+    const int64_t M = src0->ne[1], K = src0->ne[0], N = src1->ne[1], nbatch = src1->ne[2] * src1->ne[3];
+    return N >= 64 && K >= 2048 && K % 128 == 0 && M % 4 == 0 && ((M + 63) / 64) * ((N + 63) / 64) * nbatch < 64 && nbatch * 16 <= 65535 &&
+           (uintptr_t) dst->data % 16 == 0 && dst->nb[1] % 16 == 0 && dst->nb[2] % 16 == 0 && dst->nb[3] % 16 == 0;
 }
 
 extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst,
@@ -2015,7 +2029,15 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     bool ok;
     if (src0->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
     else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
-    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: shape outside the streaming kernel");
+    if (!ok) { // not the streaming kernel's shape: the tiled kernels with K cut (see vx_supports_mul_mat_scale_add)
+        if (src0->type == VX_TYPE_Q8_0) {
+            if (act_mode == VX_ACT_Q8) ok = launch_mm_cut<WT_Q8, true>(a, nbatch, st);
+            else                       ok = launch_gemm_lds<WT_Q8>(a, nbatch, st) || launch_mm_cut<WT_Q8, false>(a, nbatch, st);
+        } else {
+            ok = launch_gemm_lds<WT_F16>(a, nbatch, st) || launch_mm_cut<WT_F16, false>(a, nbatch, st);
+        }
+    }
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: shape outside the streaming kernel and the K-cut tiled kernels");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
