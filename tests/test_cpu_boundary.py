@@ -195,9 +195,9 @@ def test_supports_truth_table_node_groups(pkg):
     assert order(K, 14, 8192) == order(K, 14, 4096)                                # gate_up_proj and its halves
     assert order(K, 14, 1024) != order(K, 14, 4096)                                # few rows spread the token work over more waves
     assert order(K, 14, 1024) != order(K, 2, 1024)
-    # one chunk of tokens aims at 4 blocks per wave, several chunks (which multiply the work-groups) at 8; few rows keep
-    # their 16 waves over several chunks (every chunk has its own 16 tokens of norm, staging and angles)
-    assert order(K, 2, 1024) == order(K, 16, 4096) == 8 and order(K, 17, 4096) == 4 and order(K, 112, 1024) == 16
+    # one chunk of tokens aims at 4 blocks per wave, several chunks (which multiply the work-groups) at 8; the 16 waves of
+    # few-row products are for one chunk only
+    assert order(K, 2, 1024) == order(K, 16, 4096) == 8 and order(K, 17, 4096) == 4 and order(K, 112, 1024) == 4 and order(K, 14, 1024) == 16
     assert order(4096, 2, 1024) == order(4096, 112, 1024) == 16
     assert order(K, 0, 1024) == 0 and order(33, 2, 1024) == 0
     # gate / up / SwiGLU: both matrices count as rows
