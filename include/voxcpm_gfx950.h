@@ -322,8 +322,10 @@ VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up,
                                    int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst);
 /* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for few tokens (as above),
- * the residual updates of MiniCPMModel::layer_forward (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32
- * of dst's shape */
+ * and for 64 or more tokens over a long K (>= 2048, a multiple of 128) when the product is fewer than 64 tiles of
+ * 64 x 64 (the down-projection of a hundred tokens): there the K range is cut across work-groups and the kernel that
+ * adds the partials applies the update.  The residual updates of MiniCPMModel::layer_forward
+ * (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32 of dst's shape */
 VX_API vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,
                                       const vx_tensor * dst, float scale, int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,
