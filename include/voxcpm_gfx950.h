@@ -373,7 +373,8 @@ enum { VX_NODE_ADD = 0, VX_NODE_SUB = 1, VX_NODE_MUL = 2, VX_NODE_DIV = 3,  /* v
        VX_NODE_CONCAT = 8,                                                  /* vx_concat: aux = dim             */
        VX_NODE_REPEAT = 9,                                                  /* vx_repeat                        */
        VX_NODE_SUM = 10,                                                    /* vx_sum                           */
-       VX_NODE_ARANGE = 11 };                                               /* vx_arange: p0 = start, p1 = step */
+       VX_NODE_ARANGE = 11,                                                 /* vx_arange: p0 = start, p1 = step */
+       VX_NODE_SUM_ROWS = 12 };                                             /* vx_sum_rows                      */
 /* flags: VX_SMALL_DST_PRIVATE -- the caller knows that nothing but later nodes of the same run reads dst (the plugin: every
  * reader of the graph node is a member of the run and the node is no graph output).  Such a destination is then carried in
  * LDS only, when there is room for it, and its memory is left untouched; without room it is written like any other. */

@@ -740,6 +740,59 @@ def test_small_graph_sequence_assembly_copies_and_sums(gpu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("R,n", [(8, 128), (3, 100), (1, 64), (5, 1001)])
+@pytest.mark.parametrize("private", [0, 1])
+def test_small_graph_row_sums_and_repeats_per_request(gpu, R, n, private):
+    """The guidance arithmetic of several requests at once (src/unified_cfm.cpp:100-140 with a request per row): row sums,
+    a value per request repeated over the request's elements, a row repeated for every request, and a reshaped view of a
+    tensor the run wrote read from where the run keeps it.  One launch against a launch per node, bit for bit."""
+    import torch
+    say(f"small graph: row sums R={R} n={n} private={private}")
+    N = gpu
+    t = {"vc": rng("sgr", "c", R, n).standard_normal((R, n)).astype(np.float32), "vu": rng("sgr", "u", R, n).standard_normal((R, n)).astype(np.float32),
+         "row": rng("sgr", "r", n).standard_normal((1, n)).astype(np.float32)}
+    for name in ("diff", "dot", "sq", "st", "fill", "tile", "out"):
+        t[name] = np.zeros((R, n), np.float32)
+    for name in ("sdot", "ssq", "eps", "den", "star"):
+        t[name] = np.zeros((R, 1), np.float32)
+    t["flat_sum"] = np.zeros((R,), np.float32)
+    views = {"star_flat": ("star", (R,)), "ssq_flat": ("ssq", (R,))}
+    prog = [(N.NODE_SUB, "diff", "vc", "vu", 0, 0, 0), (N.NODE_MUL, "dot", "vc", "vu", 0, 0, 0), (N.NODE_MUL, "sq", "vu", "vu", 0, 0, 0),
+            (N.NODE_SUM_ROWS, "sdot", "dot", None, 0, 0, 0), (N.NODE_SUM_ROWS, "ssq", "sq", None, 0, 0, 0),
+            (N.NODE_SCALE, "den", "ssq", None, 0, 1.0, 1e-8), (N.NODE_DIV, "star", "sdot", "den", 0, 0, 0),
+            (N.NODE_REPEAT, "fill", "star", None, 0, 0, 0),                                                # a value per request
+            (N.NODE_MUL, "st", "vu", "fill", 0, 0, 0),
+            (N.NODE_REPEAT, "tile", "row", None, 0, 0, 0),                                                # the same row for every request
+            (N.NODE_ADD, "flat_sum", "star_flat", "ssq_flat", 0, 0, 0),                                   # reshaped views of the run's own tensors
+            (N.NODE_ADD, "out", "st", "tile", 0, 0, 0), (N.NODE_ADD, "out", "out", "diff", 0, 0, 0)]
+    keep = {"out", "flat_sum", "star"} if private else None
+    sets = []
+    for mode in ("separate", "one launch"):
+        T = {k: dev(v) for k, v in t.items()}
+        for k, (base, shape) in views.items():
+            T[k] = T[base].view(*shape)
+        if mode == "separate":
+            for op, dst, s0, s1, aux, p0, p1 in prog:
+                d, a, b = T[dst], (None if s0 is None else T[s0]), (None if s1 is None else T[s1])
+                if op <= N.NODE_DIV: N.binary(op, a, b, out=d)
+                elif op == N.NODE_SCALE: N.scale(a, p0, p1, out=d)
+                elif op == N.NODE_REPEAT: N.repeat(a, None, out=d)
+                else: N.sum_rows(a, out=d)
+        else:
+            last = {dst: i for i, (_, dst, *_r) in enumerate(prog)}
+            nodes = [N.small_node(op, T[dst], None if s0 is None else T[s0], None if s1 is None else T[s1], aux, p0, p1,
+                                  private=bool(private and not (dst in keep and last[dst] == i)))
+                     for i, (op, dst, s0, s1, aux, p0, p1) in enumerate(prog)]
+            for nd in nodes:
+                assert N.lib().vx_supports_small_node(nd) == 1
+            N.small_graph(nodes)
+        torch.cuda.synchronize()
+        sets.append({k: v for k, v in T.items() if k not in views} if keep is None else {k: T[k] for k in keep})
+    _assert_same(sets, f"row sums R={R} n={n} private={private}")
+    assert float(sets[1]["out"].abs().sum()) > 0
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("n", [64, 1001, 2700])
 @pytest.mark.parametrize("private", [False, True])
 def test_small_graph_dense_runs_barriers_and_wide_moves(gpu, n, private):

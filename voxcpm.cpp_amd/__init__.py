@@ -70,7 +70,7 @@ UNARY_FLOOR, UNARY_CEIL, UNARY_ROUND, UNARY_TRUNC = 18, 19, 20, 21
 UNARY_SQR, UNARY_SQRT, UNARY_LOG, UNARY_SIN, UNARY_COS = 100, 101, 102, 103, 104   # ggml's stand-alone ops
 GLU_REGLU, GLU_SWIGLU = 0, 2
 (NODE_ADD, NODE_SUB, NODE_MUL, NODE_DIV, NODE_ADD1, NODE_SCALE, NODE_UNARY, NODE_CPY, NODE_CONCAT, NODE_REPEAT, NODE_SUM,
- NODE_ARANGE) = range(12)
+ NODE_ARANGE, NODE_SUM_ROWS) = range(13)
 
 _lib = None
 

@@ -423,7 +423,7 @@ constexpr int SG_MAX_NODES = 16;
 constexpr int SG_MAX_ELEMS = 16384;
 constexpr int SG_LDS_ELEMS = 38912; // 152 KiB of 4-byte slots at most (an F16 value sits in the low half of its slot); a run is given what it uses
 
-enum sg_kind : int { SG_EW2 = 0, SG_ADD1, SG_SCALE, SG_UNARY, SG_CPY, SG_CONCAT, SG_REPEAT, SG_SUM, SG_ARANGE };
+enum sg_kind : int { SG_EW2 = 0, SG_ADD1, SG_SCALE, SG_UNARY, SG_CPY, SG_CONCAT, SG_REPEAT, SG_SUM, SG_ARANGE, SG_SUM_ROWS };
 
 struct sg_shape {
     int32_t ne[4];
@@ -764,6 +764,19 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
                     sg_put(D, e, i, sg_b(arange_value(nd.p0, nd.p1, (int64_t) e)), lds);
                 }
                 break;
+            case SG_SUM_ROWS: { // vx_sum_rows' order: a wave per row, lane-strided in fp64, one butterfly
+                const uint32_t ne0 = (uint32_t) S0.ne[0], rows = sg_count(S0) / ne0, lane = threadIdx.x & 63;
+                for (uint32_t r = threadIdx.x >> 6; r < rows; r += nt >> 6) {
+                    uint32_t i[4] = { 0, r % (uint32_t) S0.ne[1], 0, 0 };
+                    const uint32_t r2 = r / (uint32_t) S0.ne[1];
+                    i[2] = r2 % (uint32_t) S0.ne[2]; i[3] = r2 / (uint32_t) S0.ne[2];
+                    double acc = 0.0;
+                    for (uint32_t c0 = lane; c0 < ne0; c0 += 64) { i[0] = c0; acc += (double) sg_f(sg_get<false>(S0, i, lds)); }
+                    acc = vx_wave_sum(acc);
+                    i[0] = 0;
+                    if (lane == 0) sg_put(D, r, i, sg_b((float) acc), lds);
+                }
+            } break;
             default: break;
         }
     }
@@ -777,10 +790,13 @@ __global__ __launch_bounds__(1024) void small_graph_kernel(const sg_args a0) {
 // each operand lies (its LDS image or a global address) -- and the kernel only scalarises them (read one node ahead),
 // meets the barrier and runs a loop of a handful of instructions.  Same device functions, same orders, same bits.
 enum sgd_code : uint32_t { SGD_ADD = 0, SGD_SUB, SGD_MUL, SGD_DIV, SGD_ADD1, SGD_SCALE, SGD_UNARY, SGD_COPY, SGD_CONCAT, SGD_SUM4, SGD_SUM1, SGD_ARANGE,
-                           SGD_COPY4, SGD_CONCAT4 }; // the last two: 16 bytes per thread, counts in quads
+                           SGD_COPY4, SGD_CONCAT4,   // these two: 16 bytes per thread, counts in quads
+                           SGD_SUM_ROWS };           // n rows of n0 values each, a wave per row
 // SGD_NO_BARRIER: every value this node reads from an image written since the last barrier was written by the reading
 // thread itself (element e of a dense node is always thread e mod work-group size), and its destination is a fresh image
-constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8;
+// SGD_BLK0 / SGD_MOD0 (a REPEAT as SGD_COPY): destination element e takes source element e / block (p0 = 1 / block: a value
+// per request repeated over the request's elements) or e mod n0 (p0 = 1 / n0: a row repeated for every request)
+constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8, SGD_BLK0 = 16, SGD_MOD0 = 32;
 struct sgd_op {
     uint32_t code, n, n0, flags; // n: destination elements (SUM: units of the source); n0: CONCAT's first operand
     float    p0, p1;
@@ -851,7 +867,17 @@ __global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args 
             case SGD_ADD1: { const float y = y_at(0); SGD_LOOP(ew_apply<EW_ADD1>(0, 0, 0, SGD_X, y)); } break;
             case SGD_SCALE:  SGD_LOOP(ew_apply<EW_SCALE>(op.p0, op.p1, 0, SGD_X, 0.0f)); break;
             case SGD_UNARY:  SGD_LOOP(ew_apply<EW_UNARY>(0, 0, op.aux, SGD_X, 0.0f)); break;
-            case SGD_COPY:   SGD_LOOP(SGD_X); break;
+            case SGD_COPY:
+                if (op.flags & (SGD_BLK0 | SGD_MOD0)) { // exact below 2^22 elements (a node holds at most 16384)
+                    const bool blk = op.flags & SGD_BLK0;
+                    for (uint32_t e = threadIdx.x; e < n; e += nt) {
+                        const uint32_t q = (uint32_t) (((float) e + 0.5f) * op.p0);
+                        put(e, x_at(blk ? q : e - q * op.n0));
+                    }
+                } else {
+                    SGD_LOOP(SGD_X);
+                }
+                break;
             case SGD_CONCAT: SGD_LOOP(e < op.n0 ? x_at(e) : y_at(e - op.n0)); break;
             case SGD_ARANGE: SGD_LOOP(arange_value(op.p0, op.p1, (int64_t) e)); break;
             case SGD_COPY4: case SGD_CONCAT4: { // (a COPY4 has n0 == n)
@@ -864,6 +890,15 @@ __global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args 
                     else           v = l1 ? i1[e - op.n0] : g1[e - op.n0];
                     if (ld) id[e] = v;
                     if (gd) gd[e] = v;
+                }
+            } break;
+            case SGD_SUM_ROWS: { // vx_sum_rows' order: a wave per row, lane-strided in fp64, one butterfly
+                const uint32_t lane = threadIdx.x & 63;
+                for (uint32_t r = threadIdx.x >> 6; r < n; r += nt >> 6) {
+                    double acc = 0.0;
+                    for (uint32_t c0 = lane; c0 < op.n0; c0 += 64) acc += (double) x_at(r * op.n0 + c0);
+                    acc = vx_wave_sum(acc);
+                    if (lane == 0) put(r, (float) acc);
                 }
             } break;
             default: { // SGD_SUM4 / SGD_SUM1: vx_sum's one-wave order -- lane-strided units in fp64, one butterfly
@@ -1254,6 +1289,7 @@ extern "C" int vx_supports_small_node(const vx_small_node * nd) {
         case VX_NODE_REPEAT: return sg_fits(a) && vx_supports_repeat(a, d);
         case VX_NODE_SUM:    return sg_fits(a) && vx_supports_sum(a, d);
         case VX_NODE_ARANGE: return vx_supports_arange(d);
+        case VX_NODE_SUM_ROWS: return sg_fits(a) && vx_supports_sum_rows(a, d);
         default:             return 0;
     }
 }
@@ -1281,6 +1317,12 @@ bool sg_same(const vx_tensor * a, const vx_tensor * b) {
     return true;
 }
 struct sg_image { vx_tensor t; int32_t off; bool valid; };
+// an operand reads a tensor's image when it IS that tensor, or a reshape of it (both dense: the same elements in the same
+// row-major order -- ggml's RESHAPE / VIEW of a whole contiguous tensor, e.g. the [F * patch, requests] view that SUM_ROWS sums)
+bool sg_reads_image(const vx_tensor * img, const vx_tensor * op) {
+    if (sg_same(img, op)) return true;
+    return img->data == op->data && img->type == op->type && vx_nelements(img) == vx_nelements(op) && vx_is_contiguous(img) && vx_is_contiguous(op);
+}
 } // namespace
 
 extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx_stream stream) {
@@ -1336,6 +1378,7 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             case VX_NODE_CONCAT: g.kind = SG_CONCAT; break;
             case VX_NODE_REPEAT: g.kind = SG_REPEAT; break;
             case VX_NODE_SUM:    g.kind = SG_SUM; g.aux = nd.src0->ne[0] % 4 == 0 && al16(nd.src0->data, nd.src0->nb); break; // vx_sum's unit rule
+            case VX_NODE_SUM_ROWS: g.kind = SG_SUM_ROWS; break;
             default:             g.kind = SG_ARANGE; break;
         }
         // operands: the LDS image of exactly this tensor, else memory -- after a full barrier if the run wrote there
@@ -1344,7 +1387,7 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         for (int o = 0; o < 2; ++o) {
             if (!ops[o]) continue;
             for (int m = 0; m < n_images; ++m)
-                if (images[m].valid && sg_same(&images[m].t, ops[o])) gops[o]->lds = images[m].off;
+                if (images[m].valid && sg_reads_image(&images[m].t, ops[o])) gops[o]->lds = images[m].off;
             if (gops[o]->lds >= 0) continue;
             const sg_span sp = sg_span_of(ops[o]);
             for (int m = 0; m < n_written; ++m) if (sp.lo < written[m].hi && written[m].lo < sp.hi) g.wait_memory = 1;
@@ -1437,6 +1480,26 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             if (g.flds[0] < 0 && !vx_is_contiguous(nd.src0)) { dense = false; break; }
             op.code = g.aux ? SGD_SUM4 : SGD_SUM1;
             op.n = (uint32_t) (vx_nelements(nd.src0) / (g.aux ? 4 : 1));
+        } else if (g.kind == SG_SUM_ROWS) {
+            if ((g.flds[0] < 0 && !vx_is_contiguous(nd.src0)) || !vx_is_contiguous(nd.dst)) { dense = false; break; }
+            op.code = SGD_SUM_ROWS;
+            op.n0 = (uint32_t) nd.src0->ne[0];
+            op.n  = (uint32_t) (vx_nelements(nd.src0) / nd.src0->ne[0]);
+        } else if (g.kind == SG_REPEAT && g.flat == 0) {
+            // a dense source repeated block-wise (its leading dims are 1) or tile-wise (its trailing dims are 1)
+            const vx_tensor * sr = nd.src0, * ds = nd.dst;
+            if ((g.flds[0] < 0 && !vx_is_contiguous(sr)) || !vx_is_contiguous(ds)) { dense = false; break; }
+            int64_t lead = 1, ns = vx_nelements(sr);
+            int d0 = 0;
+            while (d0 < 4 && sr->ne[d0] == 1) { lead *= ds->ne[d0]; ++d0; }
+            bool blk = true, mod = true;
+            for (int q = d0; q < 4; ++q) blk = blk && sr->ne[q] == ds->ne[q];
+            int d1 = 4;
+            while (d1 > 0 && sr->ne[d1 - 1] == 1) --d1;
+            for (int q = 0; q < d1; ++q) mod = mod && sr->ne[q] == ds->ne[q];
+            if (blk)      { op.code = SGD_COPY; op.flags |= SGD_BLK0; op.p0 = 1.0f / (float) lead; }
+            else if (mod) { op.code = SGD_COPY; op.flags |= SGD_MOD0; op.p0 = 1.0f / (float) ns; op.n0 = (uint32_t) ns; }
+            else          { dense = false; break; }
         } else if (g.flat == 2) {
             op.code = SGD_CONCAT;
         } else if (g.flat == 1) {
@@ -1454,15 +1517,17 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         if (!dense) break;
         // 16 bytes per thread for the plain moves
         auto al = [&](const void * ptr, int32_t off) { return off >= 0 ? off % 4 == 0 : (uintptr_t) ptr % 16 == 0; };
-        if ((op.code == SGD_CONCAT || (op.code == SGD_COPY && !g.one0)) && op.n % 4 == 0 && al(op.s0, op.s0_lds) && (op.d_lds < 0 || op.d_lds % 4 == 0) &&
+        if ((op.code == SGD_CONCAT || (op.code == SGD_COPY && !g.one0 && !(op.flags & (SGD_BLK0 | SGD_MOD0)))) && op.n % 4 == 0 && al(op.s0, op.s0_lds) && (op.d_lds < 0 || op.d_lds % 4 == 0) &&
             (uintptr_t) op.d % 16 == 0 && (op.code == SGD_COPY || (op.n0 % 4 == 0 && al(op.s1, op.s1_lds)))) {
             op.n0 = op.code == SGD_COPY ? op.n / 4 : op.n0 / 4;
             op.n /= 4;
             op.code = op.code == SGD_COPY ? SGD_COPY4 : SGD_CONCAT4;
         }
         // which barriers the run can do without
-        const bool quads = op.code == SGD_COPY4 || op.code == SGD_CONCAT4;
-        const bool own_elements = !quads && op.code != SGD_CONCAT && op.code != SGD_SUM4 && op.code != SGD_SUM1; // thread e mod size reads element e
+        // (quads: the destination's elements are not written by thread e mod size -- readers of such an image meet a barrier)
+        const bool quads = op.code == SGD_COPY4 || op.code == SGD_CONCAT4 || op.code == SGD_SUM_ROWS;
+        const bool own_elements = !quads && op.code != SGD_CONCAT && op.code != SGD_SUM4 && op.code != SGD_SUM1 &&
+                                  !(op.flags & (SGD_BLK0 | SGD_MOD0)); // thread e mod size reads element e
         bool need = g.wait_memory != 0;
         const int32_t src_lds[2] = { op.s0_lds, op.s1_lds };
         const bool    single[2]  = { g.one0 != 0, g.one1 != 0 || op.code == SGD_ADD1 }; // every thread reads element 0

@@ -719,7 +719,7 @@ int compute_kv_store_group(backend_ctx * ctx, const ggml_cgraph * g, int i, cons
     return idx;
 }
 
-// A graph node as a node of vx_small_graph (tiny elementwise / copy / concat / repeat / sum / arange work); t holds the
+// A graph node as a node of vx_small_graph (tiny elementwise / copy / concat / repeat / sum / row-sum / arange work); t holds the
 // descriptors the node points to.  False for every other operator and for tensors above the small-graph size.
 bool small_node_of(const ggml_tensor * n, vx_small_node * out, vx_tensor (&t)[3]) {
     *out = vx_small_node{};
@@ -743,6 +743,7 @@ bool small_node_of(const ggml_tensor * n, vx_small_node * out, vx_tensor (&t)[3]
         case GGML_OP_CONCAT: out->op = VX_NODE_CONCAT; out->aux = ((const int32_t *) n->op_params)[0]; two = true; break;
         case GGML_OP_REPEAT: out->op = VX_NODE_REPEAT; break;
         case GGML_OP_SUM:    out->op = VX_NODE_SUM; break;
+        case GGML_OP_SUM_ROWS: out->op = VX_NODE_SUM_ROWS; break;
         case GGML_OP_ARANGE:
             out->op = VX_NODE_ARANGE;
             memcpy(&out->p0, (const float *) n->op_params + 0, sizeof(float));
