@@ -764,7 +764,8 @@ def test_small_graph_row_sums_and_repeats_per_request(gpu, R, n, private):
             (N.NODE_MUL, "st", "vu", "fill", 0, 0, 0),
             (N.NODE_REPEAT, "tile", "row", None, 0, 0, 0),                                                # the same row for every request
             (N.NODE_ADD, "flat_sum", "star_flat", "ssq_flat", 0, 0, 0),                                   # reshaped views of the run's own tensors
-            (N.NODE_ADD, "out", "st", "tile", 0, 0, 0), (N.NODE_ADD, "out", "out", "diff", 0, 0, 0)]
+            (N.NODE_ADD, "out", "st", "tile", 0, 0, 0), (N.NODE_ADD, "out", "out", "diff", 0, 0, 0),
+            (N.NODE_MUL, "out", "out", "row", 0, 0, 0)]                                                   # a row under every request, no REPEAT
     keep = {"out", "flat_sum", "star"} if private else None
     sets = []
     for mode in ("separate", "one launch"):

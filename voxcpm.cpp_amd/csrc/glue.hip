@@ -796,7 +796,8 @@ enum sgd_code : uint32_t { SGD_ADD = 0, SGD_SUB, SGD_MUL, SGD_DIV, SGD_ADD1, SGD
 // thread itself (element e of a dense node is always thread e mod work-group size), and its destination is a fresh image
 // SGD_BLK0 / SGD_MOD0 (a REPEAT as SGD_COPY): destination element e takes source element e / block (p0 = 1 / block: a value
 // per request repeated over the request's elements) or e mod n0 (p0 = 1 / n0: a row repeated for every request)
-constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8, SGD_BLK0 = 16, SGD_MOD0 = 32;
+constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8, SGD_BLK0 = 16, SGD_MOD0 = 32,
+                   SGD_MOD1 = 64; // a binary node whose second operand repeats every aux elements (p1 = 1 / aux: a row added to every request)
 struct sgd_op {
     uint32_t code, n, n0, flags; // n: destination elements (SUM: units of the source); n0: CONCAT's first operand
     float    p0, p1;
@@ -860,10 +861,12 @@ __global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args 
 #define SGD_X x_at(one0 ? 0 : e)
 #define SGD_Y y_at(one1 ? 0 : e)
         switch (op.code) {
-            case SGD_ADD:    SGD_LOOP(ew_apply<EW_ADD>(0, 0, 0, SGD_X, SGD_Y)); break;
-            case SGD_SUB:    SGD_LOOP(ew_apply<EW_SUB>(0, 0, 0, SGD_X, SGD_Y)); break;
-            case SGD_MUL:    SGD_LOOP(ew_apply<EW_MUL>(0, 0, 0, SGD_X, SGD_Y)); break;
-            case SGD_DIV:    SGD_LOOP(ew_apply<EW_DIV>(0, 0, 0, SGD_X, SGD_Y)); break;
+#define SGD_Y_TILED y_at(e - (uint32_t) (((float) e + 0.5f) * op.p1) * (uint32_t) op.aux)
+#define SGD_BINARY(OP) if (op.flags & SGD_MOD1) SGD_LOOP(ew_apply<OP>(0, 0, 0, SGD_X, SGD_Y_TILED)); else SGD_LOOP(ew_apply<OP>(0, 0, 0, SGD_X, SGD_Y))
+            case SGD_ADD:    SGD_BINARY(EW_ADD); break;
+            case SGD_SUB:    SGD_BINARY(EW_SUB); break;
+            case SGD_MUL:    SGD_BINARY(EW_MUL); break;
+            case SGD_DIV:    SGD_BINARY(EW_DIV); break;
             case SGD_ADD1: { const float y = y_at(0); SGD_LOOP(ew_apply<EW_ADD1>(0, 0, 0, SGD_X, y)); } break;
             case SGD_SCALE:  SGD_LOOP(ew_apply<EW_SCALE>(op.p0, op.p1, 0, SGD_X, 0.0f)); break;
             case SGD_UNARY:  SGD_LOOP(ew_apply<EW_UNARY>(0, 0, op.aux, SGD_X, 0.0f)); break;
@@ -915,6 +918,8 @@ __global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args 
 #undef SGD_LOOP
 #undef SGD_X
 #undef SGD_Y
+#undef SGD_Y_TILED
+#undef SGD_BINARY
     }
 }
 
@@ -1500,6 +1505,20 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             if (blk)      { op.code = SGD_COPY; op.flags |= SGD_BLK0; op.p0 = 1.0f / (float) lead; }
             else if (mod) { op.code = SGD_COPY; op.flags |= SGD_MOD0; op.p0 = 1.0f / (float) ns; op.n0 = (uint32_t) ns; }
             else          { dense = false; break; }
+        } else if (g.kind == SG_EW2 && g.flat == 0) {
+            // a dense second operand whose trailing dims are 1, under a first operand of the destination's shape
+            const vx_tensor * x = nd.src0, * y = nd.src1, * ds = nd.dst;
+            const bool x_ok = g.one0 || (vx_same_shape(x, ds) && (g.flds[0] >= 0 || vx_is_contiguous(x)));
+            if (!x_ok || !vx_is_contiguous(ds) || (g.flds[1] < 0 && !vx_is_contiguous(y))) { dense = false; break; }
+            int d1 = 4;
+            while (d1 > 0 && y->ne[d1 - 1] == 1) --d1;
+            bool tiled = true;
+            for (int q = 0; q < d1; ++q) tiled = tiled && y->ne[q] == ds->ne[q];
+            if (!tiled) { dense = false; break; }
+            op.code = SGD_ADD + (uint32_t) g.aux;
+            op.flags |= SGD_MOD1;
+            op.aux = (int32_t) vx_nelements(y);
+            op.p1 = 1.0f / (float) op.aux;
         } else if (g.flat == 2) {
             op.code = SGD_CONCAT;
         } else if (g.flat == 1) {
@@ -1527,7 +1546,7 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         // (quads: the destination's elements are not written by thread e mod size -- readers of such an image meet a barrier)
         const bool quads = op.code == SGD_COPY4 || op.code == SGD_CONCAT4 || op.code == SGD_SUM_ROWS;
         const bool own_elements = !quads && op.code != SGD_CONCAT && op.code != SGD_SUM4 && op.code != SGD_SUM1 &&
-                                  !(op.flags & (SGD_BLK0 | SGD_MOD0)); // thread e mod size reads element e
+                                  !(op.flags & (SGD_BLK0 | SGD_MOD0 | SGD_MOD1)); // thread e mod size reads element e
         bool need = g.wait_memory != 0;
         const int32_t src_lds[2] = { op.s0_lds, op.s1_lds };
         const bool    single[2]  = { g.one0 != 0, g.one1 != 0 || op.code == SGD_ADD1 }; // every thread reads element 0
@@ -1549,6 +1568,23 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         }
         if (k > 0 && !need) op.flags |= SGD_NO_BARRIER;
         else                last_barrier = k;
+    }
+    // VX_SMALL_GRAPH_EXPLAIN=1: say on stderr which node kept a run from the resolved kernel
+    static const bool explain = [] { const char * e = getenv("VX_SMALL_GRAPH_EXPLAIN"); return e && e[0] == '1'; }();
+    if (explain && !dense) {
+        int k = 0;
+        while (k + 1 < n_nodes && da.op[k + 1].n != 0) ++k; // the nodes behind the one that failed were not looked at
+        fprintf(stderr, "small graph of %d nodes: general kernel%s\n", n_nodes, block_sum ? " (a sum in the whole block's order)" : "");
+        for (int q = 0; q < n_nodes; ++q) {
+            const vx_small_node & nd = nodes[q];
+            const vx_tensor * ts[3] = { nd.dst, nd.op == VX_NODE_ARANGE ? nullptr : nd.src0, nd.src1 };
+            fprintf(stderr, "  node %d op %d aux %d flat %d%s:", q, nd.op, nd.aux, a.node[q].flat, q == k ? "  <- first unresolved" : "");
+            for (const vx_tensor * t : ts)
+                if (t) fprintf(stderr, " [%lld %lld %lld %lld | %llu %llu %llu %llu t%d]", (long long) t->ne[0], (long long) t->ne[1], (long long) t->ne[2],
+                               (long long) t->ne[3], (unsigned long long) t->nb[0], (unsigned long long) t->nb[1], (unsigned long long) t->nb[2],
+                               (unsigned long long) t->nb[3], t->type);
+            fprintf(stderr, "\n");
+        }
     }
     if (smem > 48 * 1024) { // a kernel has to be told once that it may be given more dynamic LDS than the default limit
         static bool raised[2] = { false, false };
