@@ -228,6 +228,15 @@ VX_API vx_status vx_arange(const vx_tensor * dst, float start, float step, vx_st
  * (ggml_compute_forward_repeat, ops.cpp:1689-1810).  The reference builds its attention masks from ARANGE +
  * REPEAT (src/minicpm.cpp:602-620, src/locdit.cpp:283-305). */
 VX_API vx_status vx_repeat(const vx_tensor * src, const vx_tensor * dst, vx_stream stream);
+
+/* A tree of GGML_OP_CONCAT nodes along one dimension as one launch: dst is its 2 .. 8 leaves side by side along `dim`, leaf k
+ * filling extents[k] indices.  A leaf smaller than its slot (in any dimension) is repeated as GGML_OP_REPEAT would have
+ * repeated it in front of the CONCAT.  LocDiT's sequence assembly for several requests is such a tree: (mu + t | cond | x)
+ * and (t repeated | cond | x) joined once more (src/locdit.cpp:401-452; with one request per graph the same nodes are a few
+ * KB and ride in vx_small_graph).  The bytes written are those of the node-by-node sequence.  F32 / I32. */
+VX_API vx_status vx_concat_many(const vx_tensor * const * srcs, const int64_t * extents, int n_src, int dim, const vx_tensor * dst,
+                                vx_stream stream);
+VX_API int vx_supports_concat_many(const vx_tensor * const * srcs, const int64_t * extents, int n_src, int dim, const vx_tensor * dst);
 /* GGML_OP_GET_ROWS: dst[:, i, j, k] = row rows[i, j, k] of table matrix (j, k), as F32; table F32 / F16 / Q8_0
  * (dequantised exactly as dequantize_row_q8_0, ggml/src/ggml-quants.c:401-415) or I32 (dst I32); rows I32
  * (ggml_compute_forward_get_rows, ops.cpp:4653-4870; the token embedding, src/components.cpp:223).  An index

@@ -121,6 +121,18 @@ def test_supports_truth_table_glue(pkg):
     assert lib.vx_supports_concat(past, cur, both, 1) == 1
     assert lib.vx_supports_concat(past, cur, both, 0) == 0
     assert lib.vx_supports_concat(past, f16(pkg, [64, 1, 2, 2]), both, 1) == 0
+    # a tree of CONCATs from its leaves: 2 to 8 sources whose shapes divide their slots, the slots filling the dimension
+    import ctypes as C
+    def many(srcs, extents, dim, dst):
+        arr = (C.POINTER(pkg.VxTensor) * len(srcs))(*[C.pointer(t) for t in srcs])
+        return lib.vx_supports_concat_many(arr, (C.c_int64 * len(srcs))(*extents), len(srcs), dim, dst)
+    tok, four, two, seq = f32(pkg, [1024, 1, 8, 1]), f32(pkg, [1024, 4, 8, 1]), f32(pkg, [1024, 2, 8, 1]), f32(pkg, [1024, 14, 8, 1])
+    row = f32(pkg, [1024, 1, 1, 1])
+    assert many([tok, four, two, row, four, two], [1, 4, 2, 1, 4, 2], 1, seq) == 1           # (t + mu | cond | x | t, once per request | cond | x)
+    assert many([tok, four, two, row, four, two], [1, 4, 2, 1, 4, 3], 1, seq) == 0           # slots must fill the dimension
+    assert many([tok, four], [1, 13], 1, seq) == 0                                           # 13 is no multiple of 4
+    assert many([seq], [14], 1, seq) == 0 and many([tok] * 9, [1] * 9, 1, f32(pkg, [1024, 9, 8, 1])) == 0
+    assert many([tok, f16(pkg, [1024, 13, 8, 1])], [1, 13], 1, seq) == 0
     # SUM: dense F32 rows to a scalar
     assert lib.vx_supports_sum(a, one) == 1 and lib.vx_supports_sum(a, f32(pkg, [2, 1, 1, 1])) == 0
     permuted = D(pkg, pkg.F32, [5, 1024, 1, 1], [4096, 4, 20480, 20480])

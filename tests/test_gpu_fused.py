@@ -740,6 +740,37 @@ def test_small_graph_sequence_assembly_copies_and_sums(gpu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,R,prefix,patch", [(1024, 8, 4, 2), (1024, 3, 4, 2), (30, 5, 3, 1), (8, 2, 1, 1)])
+def test_concat_tree_from_its_leaves(gpu, H, R, prefix, patch):
+    """LocDiT's sequence assembly for R requests (src/locdit.cpp:401-452 with a request dimension): two sequences
+    (t + mu | cond | x) and (t for every request | cond | x) joined along the token dimension, as one launch from the six
+    leaves against the five CONCATs and the REPEAT node by node.  Rows of 16-byte multiples and not; dim 0 as well."""
+    import torch
+    say(f"concat tree: H={H} R={R} prefix={prefix} patch={patch}")
+    g = lambda tag, *shape: dev(rng("cattree", tag, H, R).standard_normal(shape).astype(np.float32))
+    comb_c, cond, x, t_row = g("c", R, 1, H), g("k", R, prefix, H), g("x", R, patch, H), g("t", 1, 1, H)
+    # node by node
+    comb_u = gpu.repeat(t_row, (R, 1, H))
+    seq_c = gpu.concat(gpu.concat(comb_c, cond, 1), x, 1)
+    seq_u = gpu.concat(gpu.concat(comb_u, cond, 1), x, 1)
+    want = gpu.concat(seq_c, seq_u, 1)
+    L = 1 + prefix + patch
+    got = torch.full((R, 2 * L, H), float("nan"), dtype=torch.float32, device="cuda")
+    gpu.concat_many([comb_c, cond, x, t_row, cond, x], [1, prefix, patch, 1, prefix, patch], 1, got)
+    torch.cuda.synchronize()
+    assert torch.equal(want.view(torch.int32), got.view(torch.int32))
+    # along dim 0 (no 16-byte units), a strided source and a source repeated along the dimension itself
+    a, b = g("a", R, 3, 5), g("b", R, 3, 7)
+    wide = g("w", R, 3, 12)[:, :, 2:6]                       # a view: rows 48 bytes apart, 4 of them used
+    pair = g("p", R, 3, 2)
+    want0 = gpu.concat(gpu.concat(gpu.concat(a, b, 0), wide.contiguous(), 0), gpu.repeat(pair, (R, 3, 6)), 0)
+    got0 = torch.full((R, 3, 22), float("nan"), dtype=torch.float32, device="cuda")
+    gpu.concat_many([a, b, wide, pair], [5, 7, 4, 6], 0, got0)
+    torch.cuda.synchronize()
+    assert torch.equal(want0.view(torch.int32), got0.view(torch.int32))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("R,n", [(8, 128), (3, 100), (1, 64), (5, 1001)])
 @pytest.mark.parametrize("private", [0, 1])
 def test_small_graph_row_sums_and_repeats_per_request(gpu, R, n, private):

@@ -56,7 +56,7 @@ EXPORTS = [
     "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_flash_attn_ext_static", "vx_mul_mat",
     "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
     "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
-    "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_sum", "vx_sum_rows", "vx_supports_sum_rows",
+    "vx_binary", "vx_add1", "vx_scale", "vx_unary", "vx_glu", "vx_cpy", "vx_concat", "vx_concat_many", "vx_supports_concat_many", "vx_sum", "vx_sum_rows", "vx_supports_sum_rows",
     "vx_supports_binary", "vx_supports_add1", "vx_supports_unary_like", "vx_supports_unary", "vx_supports_glu",
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
     "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
@@ -126,6 +126,8 @@ def lib():
     l.vx_glu.argtypes = [C.c_int, TP, TP, TP, C.c_int, vp]
     l.vx_cpy.argtypes = [TP, TP, vp]
     l.vx_concat.argtypes = [TP, TP, TP, C.c_int, vp]
+    l.vx_concat_many.argtypes = [C.POINTER(TP), C.POINTER(C.c_int64), C.c_int, C.c_int, TP, vp]
+    l.vx_supports_concat_many.argtypes = [C.POINTER(TP), C.POINTER(C.c_int64), C.c_int, C.c_int, TP]
     l.vx_sum.argtypes = [TP, TP, vp]
     l.vx_sum_rows.argtypes = [TP, TP, vp]
     l.vx_supports_sum_rows.argtypes = [TP, TP]
@@ -343,6 +345,16 @@ def concat(a, b, ggml_dim, out=None):
         shape[a.dim() - 1 - ggml_dim] += b.shape[b.dim() - 1 - ggml_dim]
         out = torch.empty(shape, dtype=a.dtype, device=a.device)
     check(lib().vx_concat(desc(a), desc(b), desc(out), ggml_dim, _stream()), "vx_concat")
+    return out
+
+
+def concat_many(srcs, extents, ggml_dim, out):
+    """A tree of concatenations along one ggml dimension written from its leaves: source k fills extents[k] indices of
+    `out` along that dimension and is repeated where it is smaller than its slot."""
+    ds = [desc(t) for t in srcs]
+    arr = (C.POINTER(VxTensor) * len(ds))(*[C.pointer(d) for d in ds])
+    ext = (C.c_int64 * len(ds))(*extents)
+    check(lib().vx_concat_many(arr, ext, len(ds), ggml_dim, desc(out), _stream()), "vx_concat_many")
     return out
 
 

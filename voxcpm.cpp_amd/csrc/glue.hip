@@ -265,6 +265,48 @@ __global__ __launch_bounds__(256) void concat_kernel(const cat_args a) {
     else                          *(int16_t *) pd = *(const int16_t *) ps;
 }
 
+// A tree of CONCATs along one dimension written from its leaves: up to CATM_MAX sources side by side along `dim`, a
+// source smaller than its slot is repeated (GGML_OP_REPEAT's index rule: the slot's index modulo the source's shape).
+constexpr int CATM_MAX = 8;
+struct catm_src { const char * p; uint32_t ne[4]; uint32_t end; uint32_t pad; uint64_t nb[4]; }; // end: one past its last index along dim
+struct catm_args {
+    catm_src s[CATM_MAX];
+    char *   d;
+    uint32_t ne[4];
+    uint64_t nbd[4];
+    int      dim, n_src;
+    uint32_t n; // dst units
+};
+template <bool VEC>
+__global__ __launch_bounds__(256) void concat_many_kernel(const catm_args a) {
+    const uint32_t u = blockIdx.x * 256u + threadIdx.x;
+    if (u >= a.n) return;
+    const uint32_t units0 = VEC ? a.ne[0] / 4 : a.ne[0];
+    uint32_t i[4], r = u;
+    i[0] = (r % units0) * (VEC ? 4 : 1); r /= units0;
+    i[1] = r % a.ne[1]; r /= a.ne[1];
+    i[2] = r % a.ne[2]; i[3] = r / a.ne[2];
+    char * pd = a.d + i[0] * a.nbd[0] + i[1] * a.nbd[1] + i[2] * a.nbd[2] + i[3] * a.nbd[3];
+    const uint32_t at = i[a.dim];
+    uint32_t begin = 0;
+#pragma unroll
+    for (int k = 0; k < CATM_MAX; ++k) { // (k is uniform: the sources stay in scalar registers)
+        if (k < a.n_src) {
+            const catm_src & sr = a.s[k];
+            if (at >= begin && at < sr.end) {
+                uint32_t j[4] = { i[0], i[1], i[2], i[3] };
+                j[a.dim] = at - begin;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) if (j[q] >= sr.ne[q]) j[q] %= sr.ne[q];
+                const char * ps = sr.p + j[0] * sr.nb[0] + j[1] * sr.nb[1] + j[2] * sr.nb[2] + j[3] * sr.nb[3];
+                if constexpr (VEC) *(int4_t *) pd = *(const int4_t *) ps;
+                else               *(int32_t *) pd = *(const int32_t *) ps;
+            }
+            begin = sr.end;
+        }
+    }
+}
+
 // ---- ARANGE / REPEAT / GET_ROWS -----------------------------------------------------------------
 // The ops the reference's graphs use around the decoder stacks: the causal and CFG-pair masks are
 // built from ARANGE + REPEAT (src/minicpm.cpp:602-620, src/locdit.cpp:283-305), token embeddings are
@@ -1186,6 +1228,52 @@ extern "C" vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, c
     if (vec)          { if (es == 4) concat_kernel<16, 4><<<grid, block, 0, st>>>(a); else concat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
     else if (es == 4) concat_kernel<4, 4><<<grid, block, 0, st>>>(a);
     else              concat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+extern "C" int vx_supports_concat_many(const vx_tensor * const * srcs, const int64_t * extents, int n_src, int dim, const vx_tensor * dst) {
+    if (!srcs || !extents || !dst || n_src < 2 || n_src > CATM_MAX || dim < 0 || dim > 3) return 0;
+    if (dst->type != VX_TYPE_F32 && dst->type != VX_TYPE_I32) return 0;
+    if (!vx_positive(dst) || vx_nelements(dst) >= ((int64_t) 1 << 31) || !nb_multiple(dst, 4) || dst->nb[0] != 4) return 0;
+    int64_t total = 0;
+    for (int k = 0; k < n_src; ++k) {
+        const vx_tensor * t = srcs[k];
+        if (!t || t->type != dst->type || !vx_positive(t) || t->nb[0] != 4 || !nb_multiple(t, 4)) return 0;
+        for (int q = 0; q < 4; ++q) {
+            const int64_t slot = q == dim ? extents[k] : dst->ne[q];
+            if (slot <= 0 || slot % t->ne[q]) return 0;
+        }
+        total += extents[k];
+    }
+    return total == dst->ne[dim];
+}
+
+extern "C" vx_status vx_concat_many(const vx_tensor * const * srcs, const int64_t * extents, int n_src, int dim, const vx_tensor * dst, vx_stream stream) {
+    if (!vx_supports_concat_many(srcs, extents, n_src, dim, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "concat_many: 2 to %d F32 / I32 sources whose shapes divide their slots along dim %d", CATM_MAX, dim);
+    if (!dst->data) return vx_fail(VX_ERR_INVALID, "concat_many: null data");
+    catm_args a = {};
+    auto dense16 = [](const vx_tensor * t) {
+        return (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+    };
+    bool vec = dim != 0 && dst->ne[0] % 4 == 0 && dense16(dst);
+    int64_t end = 0;
+    for (int k = 0; k < n_src; ++k) {
+        const vx_tensor * t = srcs[k];
+        if (!t->data) return vx_fail(VX_ERR_INVALID, "concat_many: null data");
+        a.s[k].p = (const char *) t->data;
+        end += extents[k];
+        a.s[k].end = (uint32_t) end;
+        for (int q = 0; q < 4; ++q) { a.s[k].ne[q] = (uint32_t) t->ne[q]; a.s[k].nb[q] = t->nb[q]; }
+        vec = vec && t->ne[0] == dst->ne[0] && dense16(t); // 16 bytes per thread: whole rows side by side
+    }
+    a.d = (char *) dst->data; a.dim = dim; a.n_src = n_src;
+    for (int q = 0; q < 4; ++q) { a.ne[q] = (uint32_t) dst->ne[q]; a.nbd[q] = dst->nb[q]; }
+    a.n = (uint32_t) (vec ? vx_nelements(dst) / 4 : vx_nelements(dst));
+    const dim3 grid((a.n + 255) / 256), block(256);
+    if (vec) concat_many_kernel<true><<<grid, block, 0, (hipStream_t) stream>>>(a);
+    else     concat_many_kernel<false><<<grid, block, 0, (hipStream_t) stream>>>(a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

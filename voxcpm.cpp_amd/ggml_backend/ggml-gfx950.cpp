@@ -26,6 +26,7 @@
 #include "ggml-gfx950.h"
 #include "voxcpm_gfx950.h"
 
+#include <algorithm>
 #include <cstddef>
 #include <cstdint>
 #include <cstdlib>
@@ -908,6 +909,79 @@ void find_kv2_groups(const ggml_cgraph * g, const reader_map & readers, std::uno
     }
 }
 
+// LocDiT's sequence assembly for several requests at once (src/locdit.cpp:401-452 with a request dimension): CONCATs of
+// CONCATs along one dimension, some leaves REPEATed to their slot first, every inner node read by its parent only.  Each
+// inner node would copy its rows once more (a row reaches the pair through up to three copies); the tree's root is written
+// from the leaves in one launch instead and the inner nodes are never run.  Only trees too large for a small-graph run
+// (the one-request graph's assembly is a few KB and rides there).  The leaves are then read at the root's position, not at
+// the inner nodes': no node run in between (nor the root itself) may have been given a leaf's memory.
+struct concat_tree {
+    std::vector<const ggml_tensor *> leaves;
+    std::vector<int64_t>             extents;
+    int                              dim;
+};
+
+void find_concat_trees(const ggml_cgraph * g, const reader_map & readers, std::unordered_map<const ggml_tensor *, concat_tree> & by_root,
+                       std::unordered_map<const ggml_tensor *, const ggml_tensor *> & absorbed) {
+    constexpr int64_t SMALL_GRAPH_ELEMENTS = 16384; // below this a CONCAT is a member of a small-graph run
+    constexpr size_t  MAX_LEAVES = 8;
+    std::unordered_map<const ggml_tensor *, int> pos;
+    for (int i = 0; i < g->n_nodes; ++i) pos[g->nodes[i]] = i;
+    const auto inner_ok = [&](const ggml_tensor * t) {
+        return pos.count(t) && t->type == GGML_TYPE_F32 && !t->view_src && (t->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 &&
+               private_to_group(readers, t) && absorbed.find(t) == absorbed.end();
+    };
+    for (int i = g->n_nodes - 1; i >= 0; --i) { // parents before children: a root is never a node some other root absorbs
+        const ggml_tensor * root = g->nodes[i];
+        if (root->op != GGML_OP_CONCAT || root->type != GGML_TYPE_F32 || (root->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+        if (absorbed.find(root) != absorbed.end() || ggml_nelements(root) <= SMALL_GRAPH_ELEMENTS) continue;
+        const int dim = ((const int32_t *) root->op_params)[0];
+        concat_tree tree;
+        tree.dim = dim;
+        std::vector<const ggml_tensor *> inner;
+        bool ok = true;
+        // leaves in order: depth first, first operand first
+        std::vector<const ggml_tensor *> stack = { root->src[1], root->src[0] };
+        while (!stack.empty() && ok) {
+            const ggml_tensor * t = stack.back();
+            stack.pop_back();
+            if (!t) { ok = false; break; }
+            if (t->op == GGML_OP_CONCAT && ((const int32_t *) t->op_params)[0] == dim && inner_ok(t)) {
+                inner.push_back(t);
+                stack.push_back(t->src[1]);
+                stack.push_back(t->src[0]);
+            } else if (t->op == GGML_OP_REPEAT && inner_ok(t) && t->src[0] && t->src[0]->type == GGML_TYPE_F32) {
+                inner.push_back(t);
+                tree.leaves.push_back(t->src[0]);
+                tree.extents.push_back(t->ne[dim]);
+            } else {
+                tree.leaves.push_back(t);
+                tree.extents.push_back(t->ne[dim]);
+            }
+            ok = tree.leaves.size() <= MAX_LEAVES;
+        }
+        if (!ok || inner.empty()) continue;
+        std::vector<vx_tensor> ts(tree.leaves.size());
+        std::vector<const vx_tensor *> tp(tree.leaves.size());
+        for (size_t k = 0; k < ts.size(); ++k) { ts[k] = to_vx(tree.leaves[k]); tp[k] = &ts[k]; }
+        const vx_tensor d = to_vx(root);
+        if (!vx_supports_concat_many(tp.data(), tree.extents.data(), (int) tp.size(), dim, &d)) continue;
+        int first = i;
+        for (const ggml_tensor * t : inner) first = std::min(first, pos[t]);
+        for (const ggml_tensor * leaf : tree.leaves) ok = ok && apart(root, leaf);
+        for (int k = first + 1; k < i && ok; ++k) {
+            const ggml_tensor * n = g->nodes[k];
+            if (ggml_op_is_empty(n->op) || ggml_is_empty(n) || (n->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) continue;
+            if (std::find(inner.begin(), inner.end(), n) != inner.end()) continue;
+            for (const ggml_tensor * leaf : tree.leaves)
+                if (n != leaf && n != leaf->view_src) ok = ok && apart(n, leaf);
+        }
+        if (!ok) continue;
+        for (const ggml_tensor * t : inner) absorbed[t] = root;
+        by_root[root] = std::move(tree);
+    }
+}
+
 // FLASH_ATTN_EXT over absorbed CONCATs directly followed by the cache-write group on its result (the decode
 // step of attention_forward): one call, the write rides on the kernel that merges the key-range partials.
 // Returns the index of the group's last node, or -1.
@@ -1368,6 +1442,9 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
     std::unordered_map<const ggml_tensor *, const ggml_tensor *> kv2_absorbed;
     std::unordered_set<const ggml_tensor *> done;
     if (fusion && cgraph->n_nodes > 2) find_kv2_groups(cgraph, readers, kv2_by_fa, kv2_absorbed);
+    std::unordered_map<const ggml_tensor *, concat_tree> cat_by_root;
+    static const bool concat_trees = getenv("GGML_GFX950_NO_CONCAT_TREES") == nullptr;
+    if (fusion && concat_trees && cgraph->n_nodes > 2) find_concat_trees(cgraph, readers, cat_by_root, kv2_absorbed); // (inner nodes are skipped like absorbed CONCATs)
     for (int i = 0; i < cgraph->n_nodes; ++i) {
         ggml_tensor * node = cgraph->nodes[i];
         // the same two skips ggml-cpu applies (ggml/src/ggml-cpu/ggml-cpu.c:2956-2966)
@@ -1413,6 +1490,23 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                 ++launches;
                 if (rc != VX_OK) {
                     GGML_LOG_ERROR("ggml-gfx950: node %d (%s, rms_norm + projections) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    return GGML_STATUS_FAILED;
+                }
+                continue;
+            }
+        }
+        if (node->op == GGML_OP_CONCAT) {
+            const auto it = cat_by_root.find(node);
+            if (it != cat_by_root.end()) {
+                const concat_tree & tree = it->second;
+                vx_tensor ts[8];
+                const vx_tensor * tp[8];
+                for (size_t k = 0; k < tree.leaves.size(); ++k) { ts[k] = to_vx(tree.leaves[k]); tp[k] = &ts[k]; }
+                const vx_tensor d = to_vx(node);
+                rc = vx_concat_many(tp, tree.extents.data(), (int) tree.leaves.size(), tree.dim, &d, ctx->stream);
+                ++launches;
+                if (rc != VX_OK) {
+                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, a tree of CONCATs) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
                     return GGML_STATUS_FAILED;
                 }
                 continue;
