@@ -891,7 +891,7 @@ def test_small_graph_limits(gpu, pkg):
     nd = gpu.small_node(gpu.NODE_ADD, small, small, small)
     assert L.vx_supports_small_node(nd) == 1
     assert L.vx_supports_small_node(gpu.small_node(gpu.NODE_ADD, big, big, big)) == 0
-    assert L.vx_supports_small_node(gpu.small_node(12, small, small, small)) == 0
+    assert L.vx_supports_small_node(gpu.small_node(13, small, small, small)) == 0                    # no such operator
     assert L.vx_supports_small_node(gpu.small_node(gpu.NODE_UNARY, small, small, aux=8)) == 0       # GELU
     arr = (pkg.VxSmallNode * 17)(*([nd] * 17))
     assert L.vx_small_graph(arr, 17, None) == 2   # VX_ERR_UNSUPPORTED
