@@ -1523,7 +1523,9 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
 
     // a long K on a grid of few tiles is cut across nsplit work-groups (blockIdx.z = batch x split): each leaves its share
     // in its slab of the partial buffer, dense [token][row], for mm_splitk_reduce_kernel to add in split order
-    const int     nsplit = a.ksplit > 1 ? a.ksplit : 1; // uniform
+    // (only the 64 x 64 tile is launched with a cut K: the larger tile keeps its registers for the accumulators)
+    constexpr bool CUT = RT * CT <= 4;
+    const int     nsplit = CUT && a.ksplit > 1 ? a.ksplit : 1; // uniform
     const int     batch = (int) blockIdx.z / nsplit, split = (int) blockIdx.z % nsplit;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
     const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
@@ -1539,14 +1541,15 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // than 8 token tiles that would leave XCDs without work (112 tokens are 2 tiles: a quarter of the chip, and three empty
     // blocks dispatched for every working one): then the ROW tiles are dealt over the XCDs and a row tile's few token tiles
     // sit side by side on one, where they share the weight rows in its L2.
-    const int64_t gx = (a.M + ROWS - 1) / ROWS, gy = (a.N + TOKS - 1) / TOKS;
-    const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    int64_t ty, tx;
-    if (gy >= 8) { ty = (slot / gx) * 8 + xcd; tx = slot % gx; }
-    else         { ty = slot % gy; tx = (slot / gy) * 8 + xcd; }
+    // (32-bit and uniform: the larger tile has no register to spare)
+    const uint32_t gx = (uint32_t) ((a.M + ROWS - 1) / ROWS), gy = (uint32_t) ((a.N + TOKS - 1) / TOKS);
+    const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const bool     by_tokens = gy >= 8;
+    const uint32_t inner = by_tokens ? gx : gy, q = slot / inner, rem = slot - q * inner;
+    const uint32_t ty = by_tokens ? q * 8 + xcd : rem, tx = by_tokens ? rem : q * 8 + xcd;
     if (ty >= gy || tx >= gx) return;
-    const int64_t tok0 = ty * TOKS;
-    const int64_t rowg = tx * ROWS;
+    const int64_t tok0 = (int64_t) ty * TOKS;
+    const int64_t rowg = (int64_t) tx * ROWS;
     // the launcher takes whole rounds only, and an even number of them per split (a round's register set and LDS buffer
     // are its parity)
     const int64_t rounds_all = a.K / (32 * GL_KC), rbeg = rounds_all / nsplit * split, nround = rbeg + rounds_all / nsplit;
