@@ -333,8 +333,11 @@ VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * 
 /* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for few tokens (as above),
  * and for 64 or more tokens over a long K (>= 2048, a multiple of 128) when the product is fewer than 64 tiles of
  * 64 x 64 (the down-projection of a hundred tokens): there the K range is cut across work-groups and the kernel that
- * adds the partials applies the update.  The residual updates of MiniCPMModel::layer_forward
- * (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32 of dst's shape */
+ * adds the partials applies the update.  At prefill sizes (more than 16 tokens, rows a multiple of 4, dst dense and 16-byte
+ * aligned) the LDS-tiled kernels apply the update as they store their tile, which saves the pass over dst that the ADD node
+ * is; where no such kernel takes the shape or the activation mode, the plain product is followed by that pass (through the
+ * per-stream workspace when the residual is dst itself).  The residual updates of MiniCPMModel::layer_forward
+ * (src/minicpm.cpp:762-777); w Q8_0 or F16, residual F32 of dst's shape (or a bias row).  Bit-equal to the three nodes. */
 VX_API vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,
                                       const vx_tensor * dst, float scale, int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual,

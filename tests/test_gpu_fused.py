@@ -125,7 +125,10 @@ def test_mul_mat_swiglu(pkg, gpu, M, K, N, nb, act):
 
 @pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 2048, 40, 2),
                                       # a long K over few tiles: the tiled kernels with K cut, the update in the kernel that adds the partials
-                                      (1024, 4096, 112, 1), (1000, 4096, 70, 1)])
+                                      (1024, 4096, 112, 1), (1000, 4096, 70, 1),
+                                      # prefill sizes: the update in the tiled kernels' epilogue (whole and ragged tiles of 64 and of 128),
+                                      # or the plain product and a pass of its own (17 tokens; every shape under VX_ACT_Q8)
+                                      (1024, 1024, 512, 1), (1024, 4096, 300, 1), (1000, 1024, 200, 2), (4096, 1024, 1024, 1), (1024, 4096, 17, 1)])
 @pytest.mark.parametrize("act", ["float", "q8"])
 def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     import torch
@@ -151,17 +154,14 @@ def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     ok(pkg, L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(x), d(r2), d(r2), 1.0, mode, None), "mul_mat_scale_add in place")
     torch.cuda.synchronize()
     assert torch.equal(a, r2)
-    # token counts beyond the streaming kernel are refused, not computed some other way
+    # beyond the streaming kernel's token counts the destination has to be dense (the update may need a pass of its own)
     nbig = 256 * 1024 // M + 17   # beyond tokens x rows <= 256 Ki
     xl = dev(np.zeros((1, 1, nbig, K), dtype=np.float32))
     rl = torch.zeros((1, 1, nbig, M), dtype=torch.float32, device="cuda")
-    assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl)) == 0
-    assert L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl), 1.0, mode, None) != 0
-    # so are several chunks of tokens over a long K (they belong to the tiled kernel)
-    if K > 2048:
-        x17 = dev(np.zeros((1, 1, 17, K), dtype=np.float32))
-        r17 = torch.zeros((1, 1, 17, M), dtype=torch.float32, device="cuda")
-        assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(x17), d(r17), d(r17)) == 0
+    dl = torch.zeros((1, 1, nbig, M + 8), dtype=torch.float32, device="cuda")[..., :M]
+    assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(rl)) == (1 if M % 4 == 0 else 0)
+    assert L.vx_supports_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(dl)) == 0
+    assert L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(dl), 1.0, mode, None) != 0
 
 
 @pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2)])

@@ -1716,10 +1716,27 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     }
 
     // lane (j,c), tile (rt, tt), register r: token tok0 + 16 (CT wt + tt) + 4j + r, row rowg + 16 (RT wr + rt) + c
+    // A fused residual update (dst = res + scale * (W x), rounded as the SCALE and the ADD node would) is applied here
+    // unless K is cut: then the kernel that adds the partials applies it.  The residual may be dst itself: an element is
+    // read by the lane that writes it.
+    const bool    residual = a.res != nullptr && nsplit == 1; // uniform
+    const char *  rbase    = residual ? a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 : nullptr;
     if (tok0 + TOKS <= a.N && rowg + ROWS <= a.M) { // uniform: a tile inside the matrix stores without tests,
         // at a uniform base plus one 32-bit lane offset (the launcher checks the range)
         char * tb = db + (uint64_t) tok0 * dnb1 + (uint64_t) rowg * 4;
         const uint32_t loff = (uint32_t) ((uint64_t) (16 * CT * wt + 4 * j) * dnb1 + (uint64_t) (16 * RT * wr + c) * 4);
+        if (residual) {
+            const char *   rb    = rbase + (uint64_t) tok0 * a.rnb1 + (uint64_t) rowg * 4;
+            const uint32_t rloff = (uint32_t) ((uint64_t) (16 * CT * wt + 4 * j) * a.rnb1 + (uint64_t) (16 * RT * wr + c) * 4);
+#pragma unroll
+            for (int tt = 0; tt < CT; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const char * rr = rb + (uint64_t) (16 * tt + r) * a.rnb1; // uniform
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) acc[rt][tt][r] = scaled_residual(acc[rt][tt][r], a.res_scale, *(const float *) (rr + 64 * rt + rloff));
+                }
+        }
 #pragma unroll
         for (int tt = 0; tt < CT; ++tt)
 #pragma unroll
@@ -1739,7 +1756,10 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t tok = tok0 + 16 * (CT * wt + tt) + 4 * j + r;
-                if (tok < a.N) *(float *) (db + (uint64_t) tok * dnb1 + (uint64_t) row * 4) = acc[rt][tt][r];
+                if (tok >= a.N) continue;
+                float v = acc[rt][tt][r];
+                if (residual) v = scaled_residual(v, a.res_scale, *(const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) row * 4));
+                *(float *) (db + (uint64_t) tok * dnb1 + (uint64_t) row * 4) = v;
             }
     }
 }
@@ -1799,7 +1819,7 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
         mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
         return true;
     }
-    if (a.res) return false;
+    if (a.res && (uint64_t) 256 * a.rnb1 + 1024 >= (1ull << 32)) return false; // (the residual's 32-bit lane offsets)
     // 128 x 128: 8 waves of 64 rows x 32 tokens (4 waves per SIMD with two work-groups per CU measured 5-10 % above
     // 4 waves of 64 x 64); 64 x 64: 4 waves of 32 x 32
     if constexpr (WT == WT_Q8) {
@@ -2000,8 +2020,12 @@ extern "C" int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_te
     // a long K over few tiles (the down-projection of a hundred tokens): the product's K range is cut across work-groups
     // and the kernel that adds the partials applies the update
     const int64_t M = src0->ne[1], K = src0->ne[0], N = src1->ne[1], nbatch = src1->ne[2] * src1->ne[3];
-    return N >= 64 && K >= 2048 && K % 128 == 0 && M % 4 == 0 && ((M + 63) / 64) * ((N + 63) / 64) * nbatch < 64 && nbatch * 16 <= 65535 &&
-           (uintptr_t) dst->data % 16 == 0 && dst->nb[1] % 16 == 0 && dst->nb[2] % 16 == 0 && dst->nb[3] % 16 == 0;
+    if (N >= 64 && K >= 2048 && K % 128 == 0 && M % 4 == 0 && ((M + 63) / 64) * ((N + 63) / 64) * nbatch < 64 && nbatch * 16 <= 65535 &&
+        (uintptr_t) dst->data % 16 == 0 && dst->nb[1] % 16 == 0 && dst->nb[2] % 16 == 0 && dst->nb[3] % 16 == 0) return 1;
+    // prefill sizes: the LDS-tiled kernels apply the update as they store; a shape or activation mode that they do not
+    // take gets the plain product and a second pass over dst, which must then be dense
+    return N > 16 && M % 4 == 0 && (uintptr_t) dst->data % 16 == 0 && dst->nb[1] == (uint64_t) M * 4 &&
+           (dst->ne[2] == 1 || dst->nb[2] == dst->nb[1] * (uint64_t) N) && (dst->ne[3] == 1 || dst->nb[3] == dst->nb[1] * (uint64_t) N * (uint64_t) dst->ne[2]);
 }
 
 extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor * src1, const vx_tensor * residual, const vx_tensor * dst,
@@ -2043,7 +2067,27 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
             ok = launch_gemm_lds<WT_F16>(a, nbatch, st) || launch_mm_cut<WT_F16, false>(a, nbatch, st);
         }
     }
-    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: shape outside the streaming kernel and the K-cut tiled kernels");
+    if (!ok) { // the plain product, then the update in a pass of its own (dense dst: checked by vx_supports_mul_mat_scale_add)
+        const size_t bytes = (size_t) nbatch * a.N * a.M * sizeof(float);
+        const char * r0 = (const char *) residual->data, * d0 = (const char *) dst->data;
+        const size_t rbytes = (size_t) ((residual->ne[1] - 1) * residual->nb[1] + (residual->ne[2] - 1) * residual->nb[2] + (residual->ne[3] - 1) * residual->nb[3]) +
+                              (size_t) residual->ne[0] * 4;
+        void * product = dst->data;
+        if (r0 < d0 + bytes && d0 < r0 + rbytes) { // the residual is (in) dst: the product needs a place of its own
+            const vx_status rc = vx_workspace(st, bytes, &product);
+            if (rc != VX_OK) return rc;
+        }
+        mm_args p = a;
+        p.res = nullptr; p.dst = (char *) product;
+        p.nb1 = (uint64_t) a.M * 4; p.nb2 = p.nb1 * (uint64_t) a.N; p.nb3 = p.nb2 * (uint64_t) a.ne12;
+        if (src0->type == VX_TYPE_Q8_0) { if (act_mode == VX_ACT_Q8) launch<WT_Q8, true>(p, nbatch, st); else launch<WT_Q8, false>(p, nbatch, st); }
+        else                            launch<WT_F16, false>(p, nbatch, st);
+        mm_args b = a;
+        b.ksplit = 1; b.partial = (float *) product;
+        const int64_t units = a.N * (a.M / 4);
+        if ((units + 255) / 256 > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: launch too large");
+        mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+    }
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
