@@ -191,9 +191,15 @@ def test_supports_truth_table_node_groups(pkg):
     def acts(n, k=K):
         return f32(pkg, [k, n, 1, 1])
 
-    # projection + scale + residual: the streaming kernel's token counts (16, or tokens x rows <= 256 Ki)
-    for n, want in ((1, 1), (16, 1), (17, 1), (256, 1), (257, 0)):
+    # projection + scale + residual: every token count; beyond the streaming kernel's (16, or tokens x rows <= 256 Ki) and
+    # the K-cut shapes only into a dense destination with rows in whole 16-byte groups
+    for n, want in ((1, 1), (16, 1), (17, 1), (256, 1), (257, 1), (65536, 1)):
         assert lib.vx_supports_mul_mat_scale_add(wo, acts(n), acts(n), acts(n)) == want, n
+    strided = D(pkg, pkg.F32, [K, 257, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 257, 4 * (K + 8) * 257])
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(257), acts(257), strided) == 0
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(14), D(pkg, pkg.F32, [K, 14, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 14, 4 * (K + 8) * 14])) == 1
+    odd = q8(pkg, [K, 1002, 1, 1])
+    assert lib.vx_supports_mul_mat_scale_add(odd, acts(300), f32(pkg, [1002, 300, 1, 1]), f32(pkg, [1002, 300, 1, 1])) == 0
     assert lib.vx_supports_mul_mat_scale_add(wdown, acts(14, 4096), acts(14), acts(14)) == 1      # 16 x 4096 halves of LDS
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), acts(3), acts(2)) == 0                  # residual of another shape
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(1), acts(14)) == 1                # a bias row, repeated over the tokens
