@@ -330,6 +330,12 @@ VX_API int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor 
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
                                    int act_mode, vx_stream stream);
 VX_API int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst);
+/* The same group at prefill sizes (64 tokens or more, f16 activations): both products on the LDS-tiled kernel, whose
+ * work-groups hold a tile of gate rows and the same rows of up and apply the GLU as they store -- the two F32 products
+ * (tokens x 2 x rows x 4 bytes written and read again) never reach memory.  vx_mul_mat_swiglu takes these shapes too;
+ * this predicate needs the activation mode because under VX_ACT_Q8 the tiled products run on kernels without that epilogue. */
+VX_API int vx_supports_mul_mat_swiglu_tiled(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,
+                                            int act_mode);
 /* MUL_MAT(w, x) -> SCALE(., scale) -> ADD(residual, .): dst = residual + scale * (w x) for few tokens (as above),
  * and for 64 or more tokens over a long K (>= 2048, a multiple of 128) when the product is fewer than 64 tiles of
  * 64 x 64 (the down-projection of a hundred tokens): there the K range is cut across work-groups and the kernel that

@@ -123,6 +123,38 @@ def test_mul_mat_swiglu(pkg, gpu, M, K, N, nb, act):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("M,K,N,nb", [(4096, 1024, 1024, 1), (4096, 1024, 112, 1), (1000, 1024, 300, 1), (520, 512, 600, 2), (2048, 4096, 128, 1)])
+@pytest.mark.parametrize("wtype", ["q8", "f16"])
+def test_mul_mat_swiglu_tiled(pkg, gpu, M, K, N, nb, wtype):
+    """gate, up and the GLU at prefill sizes: the tiled kernel's work-groups hold a tile of gate rows and the same rows of up
+    (mlp_forward, src/minicpm.cpp:724-731).  Whole and ragged tiles of both sizes, rows that are no multiple of 16, a batch;
+    bit-equal to the two products and the GLU node.  Under VX_ACT_Q8 the shape is not announced and the call refuses it."""
+    import torch
+    say(f"tiled gate/up/swiglu M={M} K={K} N={N} batch={nb} weights={wtype}")
+    L, d = pkg.lib(), pkg.desc
+    g = rng("f-swiglu-t", M, K, N)
+    wgf, wuf = (0.05 * g.standard_normal((M, K))).astype(np.float32), (0.05 * g.standard_normal((M, K))).astype(np.float32)
+    if wtype == "q8":
+        wg, _ = q8_dev(wgf); wu, _ = q8_dev(wuf)
+        dg, du = pkg.desc_q8(wg, K), pkg.desc_q8(wu, K)
+    else:
+        wg, wu = dev(wgf.astype(np.float16)), dev(wuf.astype(np.float16))
+        dg, du = d(wg), d(wu)
+    x = dev(g.standard_normal((nb, 1, N, K)).astype(np.float32))
+    gate = torch.empty((nb, 1, N, M), dtype=torch.float32, device="cuda")
+    up, a, b = torch.empty_like(gate), torch.empty_like(gate), torch.full_like(gate, float("nan"))
+    assert L.vx_supports_mul_mat_swiglu_tiled(dg, du, d(x), d(b), pkg.ACT_FLOAT) == 1
+    assert L.vx_supports_mul_mat_swiglu_tiled(dg, du, d(x), d(b), pkg.ACT_Q8) == 0
+    ok(pkg, L.vx_mul_mat(dg, d(x), d(gate), pkg.ACT_FLOAT, None), "gate")
+    ok(pkg, L.vx_mul_mat(du, d(x), d(up), pkg.ACT_FLOAT, None), "up")
+    ok(pkg, L.vx_glu(pkg.GLU_SWIGLU, d(gate), d(up), d(a), 0, None), "glu")
+    ok(pkg, L.vx_mul_mat_swiglu(dg, du, d(x), d(b), pkg.ACT_FLOAT, None), "mul_mat_swiglu")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    if not L.vx_supports_mul_mat_swiglu(dg, du, d(x), d(b)):
+        assert L.vx_mul_mat_swiglu(dg, du, d(x), d(b), pkg.ACT_Q8, None) != 0
+
+
 @pytest.mark.parametrize("M,K,N,nb", [(1024, 1024, 1, 2), (1024, 4096, 2, 1), (1000, 512, 16, 1), (20, 1024, 5, 3), (1024, 4096, 14, 1), (1024, 1024, 112, 1), (1024, 2048, 40, 2),
                                       # a long K over few tiles: the tiled kernels with K cut, the update in the kernel that adds the partials
                                       (1024, 4096, 112, 1), (1000, 4096, 70, 1),

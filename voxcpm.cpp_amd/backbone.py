@@ -244,7 +244,8 @@ class MiniCPMBackbone:
             if fuse and L.vx_supports_norm_mul_mat_swiglu(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], desc(act)):
                 # rms_norm, gate, up and SwiGLU as one launch
                 call(L.vx_norm_mul_mat_swiglu, desc(h_mid), desc(nw_post), self.eps, wd["gate_proj"], wd["up_proj"], desc(act), self.act_mode)
-            elif fuse and N <= 16:     # gate, up and SwiGLU as one launch
+            elif fuse and (N <= 16 or L.vx_supports_mul_mat_swiglu_tiled(wd["gate_proj"], wd["up_proj"], desc(normed), desc(act), self.act_mode)):
+                # gate, up and SwiGLU as one launch (few tokens: the streaming kernel; prefill sizes: the tiled kernel's epilogue)
                 norm(h_mid, nw_post, normed)
                 call(L.vx_mul_mat_swiglu, wd["gate_proj"], wd["up_proj"], desc(normed), desc(act), self.act_mode)
             else:

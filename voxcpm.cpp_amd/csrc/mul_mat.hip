@@ -1502,8 +1502,13 @@ constexpr size_t gl_lds(int TR, int TC) { return 2 * GL_KC * (TR + TC) * 64 * si
 // error 2^-12 on average -- the size of the activations' own rounding) and the MFMAs accumulate across blocks;
 // otherwise the weights stay the exact integers and each 32-wide partial product is scaled in fp32.
 // A wave owns RT x CT MFMA tiles (16 rows x 16 tokens each), the work-group WR x WC waves.
-template <int WT, bool FOLD, int RT, int CT, int WR, int WC>
+// DUAL: two matrices of one layout (mlp_forward's gate and up, src/minicpm.cpp:724-731) and dst = silu(W x) * (W2 x), the
+// GLU node's arithmetic.  The work-group's 16-row tiles alternate between the matrices -- tile 2p holds rows
+// 16p .. 16p + 15 of W, tile 2p + 1 the same rows of W2 -- so that a wave (an even number of row tiles) holds both halves
+// of every value it stores, and a wave's weight units (its index picks the tile's parity) come from one matrix only.
+template <int WT, bool FOLD, int RT, int CT, int WR, int WC, bool DUAL = false>
 __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT * CT >= 16 ? 2 : 4))) void gemm_lds_kernel(const mm_args a) {
+    static_assert(!DUAL || (RT % 2 == 0 && (WR * WC) % 2 == 0), "pairs of row tiles inside a wave, a matrix per wave parity");
     static_assert(GL_KC == 2, "the parity of a block inside a round is its index in the round");
     constexpr int  TR = WR * RT, TC = WC * CT; // 16-wide tiles per work-group: rows, tokens
     constexpr int  NT = 64 * WR * WC;          // threads
@@ -1524,11 +1529,13 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // a long K on a grid of few tiles is cut across nsplit work-groups (blockIdx.z = batch x split): each leaves its share
     // in its slab of the partial buffer, dense [token][row], for mm_splitk_reduce_kernel to add in split order
     // (only the 64 x 64 tile is launched with a cut K: the larger tile keeps its registers for the accumulators)
-    constexpr bool CUT = RT * CT <= 4;
+    constexpr bool CUT = RT * CT <= 4 && !DUAL;
     const int     nsplit = CUT && a.ksplit > 1 ? a.ksplit : 1; // uniform
     const int     batch = (int) blockIdx.z / nsplit, split = (int) blockIdx.z % nsplit;
     const int     i12 = batch % a.ne12, i13 = batch / a.ne12;
-    const char *  wb  = a.w + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
+    // (DUAL: odd waves fetch the second matrix -- unit idx of a thread lies in row tile idx / 64 = wave + waves * (it / 2))
+    const char *  wsel = DUAL && (wid & 1) ? a.w2 : a.w; // uniform per wave
+    const char *  wb  = wsel + (uint64_t) (i12 / a.r2) * a.nb02 + (uint64_t) (i13 / a.r3) * a.nb03;
     const char *  xb  = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13;
     char *        db  = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
     uint64_t      dnb1 = a.nb1;
@@ -1542,7 +1549,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // blocks dispatched for every working one): then the ROW tiles are dealt over the XCDs and a row tile's few token tiles
     // sit side by side on one, where they share the weight rows in its L2.
     // (32-bit and uniform: the larger tile has no register to spare)
-    const uint32_t gx = (uint32_t) ((a.M + ROWS - 1) / ROWS), gy = (uint32_t) ((a.N + TOKS - 1) / TOKS);
+    const int64_t  MV = DUAL ? 2 * a.M : a.M; // rows of the tiled (virtual) matrix
+    const uint32_t gx = (uint32_t) ((MV + ROWS - 1) / ROWS), gy = (uint32_t) ((a.N + TOKS - 1) / TOKS);
     const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const bool     by_tokens = gy >= 8;
     const uint32_t inner = by_tokens ? gx : gy, q = slot / inner, rem = slot - q * inner;
@@ -1569,7 +1577,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     for (int it = 0; it < WU; ++it) {
         const int idx = tid + NT * (it >> 1), kbl = it & 1;
         const int row = idx >> 2, uj = idx & 3;
-        const uint64_t rowoff = (uint64_t) min(rowg + row, a.M - 1) * a.nb01;
+        const uint32_t wrow   = DUAL ? (uint32_t) (rowg >> 1) + 16 * (row >> 5) + (row & 15) : (uint32_t) rowg + row; // the row of its own matrix
+        const uint64_t rowoff = (uint64_t) min(wrow, (uint32_t) a.M - 1) * a.nb01;
         if (kbl == 0) woff[it >> 1] = (uint32_t) (rowoff + (WT == WT_Q8 ? 8 : 16) * uj);
         wslot[it] = (uint32_t) lds_slot(kbl, row >> 4, TR, uj, row & 15);
     }
@@ -1719,6 +1728,23 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     // A fused residual update (dst = res + scale * (W x), rounded as the SCALE and the ADD node would) is applied here
     // unless K is cut: then the kernel that adds the partials applies it.  The residual may be dst itself: an element is
     // read by the lane that writes it.
+    if constexpr (DUAL) {
+        // lane (j,c), tile pair (2p, 2p + 1), register r: dst row rowg / 2 + 16 (RT wr / 2 + p) + c of token ... + 4j + r
+#pragma unroll
+        for (int p2 = 0; p2 < RT / 2; ++p2) {
+            const int64_t row = (rowg >> 1) + 16 * ((RT * wr) / 2 + p2) + c;
+            if (row >= a.M) continue;
+#pragma unroll
+            for (int tt = 0; tt < CT; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t tok = tok0 + 16 * (CT * wt + tt) + 4 * j + r;
+                    const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
+                    if (tok < a.N) *(float *) (db + (uint64_t) tok * dnb1 + (uint64_t) row * 4) = (g / (1.0f + expf(-g))) * u;
+                }
+        }
+        return;
+    }
     const bool    residual = a.res != nullptr && nsplit == 1; // uniform
     const char *  rbase    = residual ? a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 : nullptr;
     if (tok0 + TOKS <= a.N && rowg + ROWS <= a.M) { // uniform: a tile inside the matrix stores without tests,
@@ -1764,22 +1790,22 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     }
 }
 
-template <int WT, bool FOLD, int RT, int CT, int WR, int WC>
+template <int WT, bool FOLD, int RT, int CT, int WR, int WC, bool DUAL = false>
 bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
     constexpr size_t lds = gl_lds(RT * WR, CT * WC);
-    const int64_t gx = (a.M + 16 * RT * WR - 1) / (16 * RT * WR), gy = (a.N + 16 * CT * WC - 1) / (16 * CT * WC);
+    const int64_t gx = ((DUAL ? 2 : 1) * a.M + 16 * RT * WR - 1) / (16 * RT * WR), gy = (a.N + 16 * CT * WC - 1) / (16 * CT * WC);
     const int64_t blocks = gy >= 8 ? gx * ((gy + 7) / 8) * 8 : ((gx + 7) / 8) * 8 * gy; // (the kernel's two ways of dealing tiles to XCDs)
     if (blocks > 0x7fffffff) return false;
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
-        if (hipFuncSetAttribute((const void *) gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
+        if (hipFuncSetAttribute((const void *) gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
             (void) hipGetLastError();
             return false;
         }
         raised = true;
     }
     const int nsplit = a.ksplit > 1 ? a.ksplit : 1;
-    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC><<<dim3((unsigned) blocks, 1, (unsigned) (nbatch * nsplit)), dim3(64 * WR * WC), lds, st>>>(a);
+    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC, DUAL><<<dim3((unsigned) blocks, 1, (unsigned) (nbatch * nsplit)), dim3(64 * WR * WC), lds, st>>>(a);
     return true;
 }
 
@@ -1826,6 +1852,18 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
         if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2>(a, nbatch, st);
     }
     return big ? launch_gemm_lds_tile<WT, false, 4, 2, 2, 4>(a, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(a, nbatch, st);
+}
+
+// gate and up of mlp_forward with the GLU node's arithmetic in the tile's epilogue (gemm_lds_kernel's DUAL form); the
+// shapes are those of gemm_lds_swiglu_ok
+template <int WT>
+bool launch_gemm_lds_swiglu(const mm_args & a, int nbatch, hipStream_t st) {
+    const bool fold = WT == WT_Q8 && gemm_lds_mode() == 2;
+    const bool big  = ((2 * a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
+    if constexpr (WT == WT_Q8) {
+        if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4, true>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2, true>(a, nbatch, st);
+    }
+    return big ? launch_gemm_lds_tile<WT, false, 4, 2, 2, 4, true>(a, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2, true>(a, nbatch, st);
 }
 
 // A long K on a grid that leaves most CUs with one work-group is a chain of ~3 us rounds: cut K so that every split walks
@@ -1940,6 +1978,29 @@ extern "C" int vx_supports_mul_mat_swiglu(const vx_tensor * gate, const vx_tenso
     return gemv_shape_ok(src1->ne[1], 2 * gate->ne[1], gate->ne[0]);
 }
 
+// Prefill sizes: both products on the LDS-tiled kernel, the GLU in its epilogue (f16 activations only: under VX_ACT_Q8
+// the tiled products run on other kernels, and the node-by-node sequence stays).
+static bool gemm_lds_swiglu_ok(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst, int act_mode) {
+    if (act_mode != VX_ACT_FLOAT || gemm_lds_mode() == 0) return false;
+    const int64_t K = gate->ne[0], M = gate->ne[1], N = src1->ne[1], nbatch = src1->ne[2] * src1->ne[3];
+    if (K % (32 * GL_KC) || N < 64 || K >= (1ll << 28)) return false;
+    auto al = [](const vx_tensor * t, uint64_t m) { return (uintptr_t) t->data % m == 0 && t->nb[1] % m == 0 && t->nb[2] % m == 0 && t->nb[3] % m == 0; };
+    if (!al(src1, 16)) return false;
+    const uint64_t wm = gate->type == VX_TYPE_Q8_0 ? 4 : 16;
+    if (!al(gate, wm) || !al(up, wm)) return false;
+    if ((uint64_t) M * gate->nb[1] >= (1ull << 32) || (uint64_t) 256 * src1->nb[1] + 256 >= (1ull << 32) || (uint64_t) 256 * dst->nb[1] + 1024 >= (1ull << 32)) return false;
+    // (each product on its own must be one that the tiled kernel walks with its K whole: a cut K is summed in another order)
+    return ((M + 63) / 64) * ((N + 63) / 64) * nbatch >= 64;
+}
+
+extern "C" int vx_supports_mul_mat_swiglu_tiled(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst, int act_mode) {
+    if (!vx_supports_mul_mat(gate, src1, dst) || !up) return 0;
+    if (gate->type != VX_TYPE_Q8_0 && gate->type != VX_TYPE_F16) return 0;
+    if (up->type != gate->type) return 0;
+    for (int i = 0; i < 4; ++i) if (up->ne[i] != gate->ne[i] || up->nb[i] != gate->nb[i]) return 0;
+    return !gemv_shape_ok(src1->ne[1], 2 * gate->ne[1], gate->ne[0]) && gemm_lds_swiglu_ok(gate, up, src1, dst, act_mode);
+}
+
 // whether the activations of a streaming-kernel launch can be normalised on the fly: rows of at most 1024
 // floats (the RMS_NORM kernel's wave-per-row regime), everything 16-byte aligned, one F32 weight row
 static bool norm_prologue_ok(const vx_tensor * x, const vx_tensor * norm_w) {
@@ -1977,9 +2038,11 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
                             const vx_tensor * dst, int act_mode, vx_stream stream) {
     if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
         return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
-    if (!vx_supports_mul_mat_swiglu(gate, up, src1, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, a token count the streaming kernel takes");
     if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
+    const bool tiled = !norm_w && vx_supports_mul_mat_swiglu_tiled(gate, up, src1, dst, act_mode);
+    if (!tiled && !vx_supports_mul_mat_swiglu(gate, up, src1, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, a token count the streaming kernel takes "
+                       "(or, with f16 activations, 64 tokens or more for the tiled kernel: vx_supports_mul_mat_swiglu_tiled)");
     if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
         return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
     mm_args a = {};
@@ -1999,9 +2062,10 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
     bool ok;
-    if (gate->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
-    else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
-    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: shape outside the streaming kernel");
+    if (tiled)                           ok = gate->type == VX_TYPE_Q8_0 ? launch_gemm_lds_swiglu<WT_Q8>(a, nbatch, st) : launch_gemm_lds_swiglu<WT_F16>(a, nbatch, st);
+    else if (gate->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
+    else                                 ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: shape outside the streaming and the tiled kernel");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -1252,7 +1252,7 @@ bool compute_fused_gate_up_group(backend_ctx * ctx, const ggml_cgraph * g, int i
         *rc = vx_norm_mul_mat_swiglu(&xx, &nw, eps, &gw, &uw, &d, mul_mat_act_mode(), ctx->stream);
         done.insert(scale); done.insert(mm);
     } else {
-        if (!vx_supports_mul_mat_swiglu(&gw, &uw, &xx, &d)) return false;
+        if (!vx_supports_mul_mat_swiglu(&gw, &uw, &xx, &d) && !vx_supports_mul_mat_swiglu_tiled(&gw, &uw, &xx, &d, mul_mat_act_mode())) return false;
         *rc = vx_mul_mat_swiglu(&gw, &uw, &xx, &d, mul_mat_act_mode(), ctx->stream);
     }
     done.insert(glu);
@@ -1558,7 +1558,8 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                     ggml_get_glu_op(glu) == GGML_GLU_OP_SWIGLU && ((const int32_t *) glu->op_params)[1] == 0 &&
                     next->src[1] == node->src[1] && (next->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && readers[next] == 1) {
                     const vx_tensor g = to_vx(node->src[0]), u = to_vx(next->src[0]), x = to_vx(node->src[1]), d = to_vx(glu);
-                    if (vx_supports_mul_mat_swiglu(&g, &u, &x, &d) && apart(glu, node->src[1])) {
+                    if ((vx_supports_mul_mat_swiglu(&g, &u, &x, &d) || vx_supports_mul_mat_swiglu_tiled(&g, &u, &x, &d, mul_mat_act_mode())) &&
+                        apart(glu, node->src[1])) {
                         rc = vx_mul_mat_swiglu(&g, &u, &x, &d, mul_mat_act_mode(), ctx->stream);
                         fused = true;
                         ++i; // one more node than a pair
