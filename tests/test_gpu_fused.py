@@ -914,6 +914,83 @@ def test_small_graph_dense_runs_barriers_and_wide_moves(gpu, n, private):
     assert float(sets[1]["out"].abs().sum()) > 0
 
 
+@pytest.mark.parametrize("seed", list(range(160)))
+def test_small_graph_random_programs(gpu, seed):
+    """Random runs of up to 16 nodes over a small pool of tensors -- results rewritten in place, values read again after
+    their source changed, scalars and per-request columns produced inside the run and broadcast later, reshaped views of the
+    run's own tensors, temporaries that are private to the run -- one launch against a launch per node, bit for bit.  What
+    it is after: the host-side decisions of the dense kernel (which barriers a run can do without, which operands are
+    brought into LDS beforehand, which image a view reads) and the general kernel's fallbacks for strided operands."""
+    import torch
+    N = gpu
+    r = rng("sg-random", seed)
+    R, n = int(r.choice([1, 2, 3, 5])), int(r.choice([64, 100, 257, 1024]))
+    say(f"small graph: random program seed={seed} R={R} n={n}")
+    init = {}
+    for name in ("A0", "A1", "A2", "T0", "T1", "T2"):
+        init[name] = r.standard_normal((R, n)).astype(np.float32)
+    init["W"] = r.standard_normal((R, n + 8)).astype(np.float32)          # its first n columns: a strided operand
+    init["row"] = r.standard_normal((1, n)).astype(np.float32)
+    for name in ("c0", "ct"):
+        init[name] = r.standard_normal((R, 1)).astype(np.float32)
+    for name in ("s0", "st"):
+        init[name] = r.standard_normal((1,)).astype(np.float32)
+    init["cat"] = np.zeros((2 * R, n), np.float32)
+    init["wide"] = np.zeros((R, 2 * n), np.float32)
+    temps = {"T0", "T1", "T2", "ct", "st"}
+    full, cols, scalars = ["A0", "A1", "A2", "T0", "T1", "T2"], ["c0", "ct"], ["s0", "st"]
+    pick = lambda names: names[int(r.integers(len(names)))]
+    prog = []
+    for _ in range(int(r.integers(6, 17))):
+        kind = pick(["ew", "ew", "ew", "bcast", "add1", "scale", "unary", "cpy", "repeat", "sum", "sum_rows", "concat", "colop", "strided", "flat"])
+        if kind == "ew":        prog.append((pick([N.NODE_ADD, N.NODE_SUB, N.NODE_MUL]), pick(full), pick(full), pick(full), 0, 0.0, 0.0))
+        elif kind == "bcast":   prog.append((pick([N.NODE_ADD, N.NODE_MUL]), pick(full), pick(full), pick(["row", "c0", "ct", "s0", "st"]), 0, 0.0, 0.0))
+        elif kind == "add1":    prog.append((N.NODE_ADD1, pick(full), pick(full), pick(scalars), 0, 0.0, 0.0))
+        elif kind == "scale":   prog.append((N.NODE_SCALE, pick(full + cols + scalars), None, None, 0, float(r.uniform(-1.5, 1.5)), float(r.uniform(-1, 1))))
+        elif kind == "unary":   prog.append((N.NODE_UNARY, pick(full), pick(full), None, pick([N.UNARY_SILU, N.UNARY_NEG, N.UNARY_TANH]), 0.0, 0.0))
+        elif kind == "cpy":     prog.append((N.NODE_CPY, pick(full), pick(full), None, 0, 0.0, 0.0))
+        elif kind == "repeat":  prog.append((N.NODE_REPEAT, pick(full), pick(["row", "c0", "ct", "s0", "st"]), None, 0, 0.0, 0.0))
+        elif kind == "sum":     prog.append((N.NODE_SUM, pick(scalars), pick(full), None, 0, 0.0, 0.0))
+        elif kind == "sum_rows": prog.append((N.NODE_SUM_ROWS, pick(cols), pick(full), None, 0, 0.0, 0.0))
+        elif kind == "concat":
+            if r.integers(2): prog.append((N.NODE_CONCAT, "cat", pick(full), pick(full), 1, 0.0, 0.0))
+            else:             prog.append((N.NODE_CONCAT, "wide", pick(full), pick(full), 0, 0.0, 0.0))
+        elif kind == "colop":   prog.append((pick([N.NODE_ADD, N.NODE_MUL, N.NODE_DIV]), pick(cols), pick(cols), pick(cols + scalars), 0, 0.0, 0.0))
+        elif kind == "strided": prog.append((pick([N.NODE_ADD, N.NODE_MUL]), pick(full), "Wv", pick(full), 0, 0.0, 0.0))
+        else:                   prog.append((N.NODE_ADD, "A0f", pick(["A1f", "T0f"]), "A2f", 0, 0.0, 0.0))   # flat views of the run's tensors
+    for i, p in enumerate(prog):                      # SCALE in place
+        if p[0] == N.NODE_SCALE: prog[i] = (p[0], p[1], p[1], None, 0, p[5], p[6])
+    base = lambda name: name[:-1] if name.endswith("f") else name
+    sets = []
+    for mode in ("separate", "one launch"):
+        T = {k: dev(v) for k, v in init.items()}
+        T["Wv"] = T["W"][:, :n]
+        for k in ("A0", "A1", "A2", "T0"):
+            T[k + "f"] = T[k].view(R * n)
+        nodes = []
+        for op, dst, s0, s1, aux, p0, p1 in prog:
+            d, a, b = T[dst], (None if s0 is None else T[s0]), (None if s1 is None else T[s1])
+            if mode == "separate":
+                if op <= N.NODE_DIV: N.binary(op, a, b, out=d)
+                elif op == N.NODE_ADD1: N.add1(a, b, out=d)
+                elif op == N.NODE_SCALE: N.scale(a, p0, p1, out=d)
+                elif op == N.NODE_UNARY: N.unary(aux, a, out=d)
+                elif op == N.NODE_CPY: N.cpy(a, d)
+                elif op == N.NODE_CONCAT: N.concat(a, b, aux, out=d)
+                elif op == N.NODE_REPEAT: N.repeat(a, None, out=d)
+                elif op == N.NODE_SUM: N.sum_all(a, out=d)
+                else: N.sum_rows(a, out=d)
+            else:
+                nd = N.small_node(op, d, a, b, aux, p0, p1, private=base(dst) in temps)
+                assert N.lib().vx_supports_small_node(nd) == 1, (op, dst, s0, s1)
+                nodes.append(nd)
+        if mode == "one launch":
+            N.small_graph(nodes)
+        torch.cuda.synchronize()
+        sets.append({k: v for k, v in T.items() if base(k) not in temps and k in init})
+    _assert_same(sets, f"random program seed={seed}: {prog}")
+
+
 def test_small_graph_limits(gpu, pkg):
     """What a run may hold: at most 16 nodes, tensors of at most 16384 elements, only the tiny operators."""
     import torch

@@ -1558,6 +1558,8 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
     da.h = a.h;
     bool dense = dense_allowed && !block_sum;
     struct { int32_t off; int writer; bool quads; } wrote[SG_MAX_NODES]; // images written by the run: by which node, in which thread order
+    sg_span touched[3 * SG_MAX_NODES]; // memory that the nodes since the last barrier read or stored
+    int     n_touched = 0;
     int n_wrote = 0, last_barrier = 0;
     for (int k = 0; k < n_nodes && dense; ++k) {
         const sg_node & g = a.node[k];
@@ -1654,8 +1656,18 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             if (mine < 0) mine = n_wrote++;
             wrote[mine] = { op.d_lds, k, quads };
         }
+        // ... and through memory: a destination that is stored must not overlap anything that a node since the last barrier
+        // read from memory (another thread may still be reading it: a sum walks its operand with one wave while the other
+        // waves go on) or stored there (two stores of different threads to one address land in either order)
+        if (op.d) {
+            const sg_span dsp = sg_span_of(nd.dst);
+            for (int m = 0; m < n_touched && !need; ++m) if (dsp.lo < touched[m].hi && touched[m].lo < dsp.hi) need = true;
+        }
         if (k > 0 && !need) op.flags |= SGD_NO_BARRIER;
-        else                last_barrier = k;
+        else              { last_barrier = k; n_touched = 0; }
+        if (has0 && op.s0_lds < 0) touched[n_touched++] = sg_span_of(nd.src0);
+        if (has1 && op.s1_lds < 0) touched[n_touched++] = sg_span_of(nd.src1);
+        if (op.d)                  touched[n_touched++] = sg_span_of(nd.dst);
     }
     // VX_SMALL_GRAPH_EXPLAIN=1: say on stderr which node kept a run from the resolved kernel
     static const bool explain = [] { const char * e = getenv("VX_SMALL_GRAPH_EXPLAIN"); return e && e[0] == '1'; }();
