@@ -445,6 +445,74 @@ def test_f16_cache_write_with_ordering_scalar(pkg, gpu, T, n_past, B, poison):
         assert torch.equal(kc2[:, :, n_past:n_past + T], k.transpose(1, 2).to(torch.float16))
 
 
+@pytest.mark.parametrize("seed", list(range(40)))
+def test_decode_attention_groups_random_shapes(pkg, gpu, seed):
+    """attention_forward's decode step (src/minicpm.cpp:682-713) at random shapes: cached keys + the step's keys read in
+    place against CONCAT, CONCAT, FLASH_ATTN_EXT, and the cache write with its ordering scalar against its nodes, for F32
+    and F16 caches, head sizes 64 and 128, past lengths on both sides of every tile and range boundary.  Bit for bit."""
+    import torch
+    L, d = pkg.lib(), pkg.desc
+    r = rng("f-decode-random", seed)
+    B, Hkv, gqa = int(r.choice([1, 2, 3, 16])), int(r.choice([1, 2, 4])), int(r.choice([1, 4, 8]))
+    D, T = int(r.choice([64, 64, 128])), int(r.choice([1, 1, 1, 2, 3]))
+    n_past = int(r.choice([1, 15, 16, 31, 32, 33, 63, 64, 65, 255, 256, 257, 300, 511, 640, 767, 1023, 1025, 2049, 4100]))
+    f16 = bool(r.integers(2))
+    H = Hkv * gqa
+    say(f"decode groups random seed={seed}: B={B} heads={H}/{Hkv} D={D} T={T} n_past={n_past} cache={'f16' if f16 else 'f32'}")
+    cdt = np.float16 if f16 else np.float32
+    q = dev(r.standard_normal((B, H, T, D)).astype(np.float32))
+    kc1, vc1 = (dev(r.standard_normal((B, Hkv, n_past + T + 3, D)).astype(cdt)) for _ in range(2))
+    kc2, vc2 = kc1.clone(), vc1.clone()
+    k = dev(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    v = dev(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    kcur, vcur = k.transpose(1, 2), v.transpose(1, 2)
+    mask = dev(reflib.causal_mask(T, n_past + T, n_past)) if T > 1 else None
+    scale = float(1.0 / np.sqrt(D))
+    slot = lambda c: c[:, :, n_past:n_past + T].transpose(1, 2)
+    # node by node: (cast,) CONCAT, CONCAT, attention; then the write and its scalar
+    if f16:
+        k16, v16 = torch.empty((B, Hkv, T, D), dtype=torch.float16, device="cuda"), torch.empty((B, Hkv, T, D), dtype=torch.float16, device="cuda")
+        ok(pkg, L.vx_cpy(d(kcur), d(k16), None), "cast k"); ok(pkg, L.vx_cpy(d(vcur), d(v16), None), "cast v")
+        kseg, vseg = k16, v16
+    else:
+        kseg, vseg = kcur, vcur
+    kall = torch.empty((B, Hkv, n_past + T, D), dtype=kc1.dtype, device="cuda"); vall = torch.empty_like(kall)
+    ok(pkg, L.vx_concat(d(kc1[:, :, :n_past]), d(kseg), d(kall), 1, None), "concat k")
+    ok(pkg, L.vx_concat(d(vc1[:, :, :n_past]), d(vseg), d(vall), 1, None), "concat v")
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    ok(pkg, L.vx_flash_attn_ext(d(q), d(kall), d(vall), d(mask), None, d(a), scale, 0.0, 0.0, None), "attention")
+    cont = torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda")
+    sk, sv, sync = (torch.empty(1, dtype=torch.float32, device="cuda") for _ in range(3))
+    for src, c, s_ in ((k, kc1, sk), (v, vc1, sv)):
+        ok(pkg, L.vx_cpy(d(src), d(slot(c)), None), "cpy")
+        ok(pkg, L.vx_cpy(d(slot(c)), d(cont), None), "cont")
+        ok(pkg, L.vx_sum(d(cont), d(s_), None), "sum")
+    ok(pkg, L.vx_binary(pkg.BIN_ADD, d(sk), d(sv), d(sync), None), "add")
+    ok(pkg, L.vx_scale(d(sync), d(sync), 0.25, 0.125, None), "scale")
+    a1 = torch.empty_like(a)
+    ok(pkg, L.vx_add1(d(a), d(sync), d(a1), None), "add1")
+    # the groups
+    args = (d(q), d(kc2[:, :, :n_past]), d(kcur), d(vc2[:, :, :n_past]), d(vcur), d(mask))
+    if L.vx_supports_flash_attn_ext_kv2(*args, d(a)):
+        b = torch.full_like(a, float("nan"))
+        ok(pkg, L.vx_flash_attn_ext_kv2(*args, None, d(b), scale, 0.0, 0.0, None), "kv2")
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), "two segments against CONCAT + attention"
+    else:
+        say("   (two-segment attention declines the shape)")
+    if L.vx_supports_flash_attn_ext_kv2_store(*args, d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(a)):
+        c_ = torch.full_like(a, float("nan"))
+        ok(pkg, L.vx_flash_attn_ext_kv2_store(*args, None, d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(c_), scale, 0.0, 0.0, 0.25, 0.125, None), "kv2_store")
+        torch.cuda.synchronize()
+        assert torch.equal(a1, c_), "attention with the cache write against its nodes"
+        assert same_bits(kc1, kc2) and same_bits(vc1, vc2)
+    elif L.vx_supports_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(a), d(a)):
+        c_ = torch.full_like(a, float("nan"))
+        ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(a), d(c_), 0.25, 0.125, None), "kv_store_sync")
+        torch.cuda.synchronize()
+        assert torch.equal(a1, c_) and same_bits(kc1, kc2) and same_bits(vc1, vc2)
+
+
 @pytest.mark.parametrize("T,B,H,Hkv,D,K", [(1, 2, 16, 2, 64, 1024), (1, 1, 16, 2, 64, 1024), (3, 2, 8, 8, 128, 512), (16, 1, 4, 1, 32, 256), (14, 8, 16, 2, 64, 1024), (21, 1, 16, 2, 64, 1024)])
 @pytest.mark.parametrize("act", ["float", "q8"])
 @pytest.mark.parametrize("yarn", [False, True])

@@ -278,6 +278,35 @@ def test_fa_sinks_softcap_alibi(gpu):
     fa_case(gpu, q, k, v, None, sinks=sinks, name="sinks + split")
 
 
+@pytest.mark.parametrize("seed", list(range(64)))
+def test_fa_random_shapes(gpu, seed):
+    """Random shapes around every boundary the kernels have (16-column tiles, 32-key tiles, the cut into key ranges, the
+    half tile of at most 16 keys, the LDS-tiled prefill kernel's 64-key tiles): batch, GQA ratio, query rows, key count,
+    head size, K/V type, mask with switched-off keys and whole switched-off rows per head or shared, ALiBi, soft cap, sinks --
+    against the scalar oracle, with the tolerance of every other attention test."""
+    r = rng("fa-random", seed)
+    B, Hkv, gqa = int(r.choice([1, 2, 3])), int(r.choice([1, 2, 4])), int(r.choice([1, 2, 4, 8]))
+    n_q = int(r.choice([1, 1, 2, 5, 16, 17, 40, 70]))
+    n_kv = int(r.choice([1, 7, 16, 17, 31, 32, 33, 64, 100, 255, 256, 257, 300, 513, 777, 1024, 1300]))
+    D = int(r.choice([64, 64, 128]))
+    kv_dtype = np.float16 if r.integers(3) else np.float32
+    q, k, v = qkv(("far", seed), B, Hkv * gqa, Hkv, n_q, n_kv, D=D, kv_dtype=kv_dtype)
+    mask = None
+    if r.integers(3):
+        per = int(r.choice([1, Hkv * gqa])) if r.integers(2) else 1          # one mask for all heads, or one per head
+        mm = r.standard_normal((int(r.choice([1, B])), per, n_q, n_kv)).astype(np.float32)
+        mm[r.random(mm.shape) < 0.3] = -np.inf
+        if n_q > 1 and r.integers(2): mm[:, :, int(r.integers(n_q))] = -np.inf   # a row that sees no key
+        mask = mm.astype(np.float16)
+    extra = int(r.integers(4))
+    max_bias = 8.0 if extra == 1 and mask is not None else 0.0
+    softcap = 10.0 if extra == 2 else 0.0
+    sinks = r.standard_normal(Hkv * gqa).astype(np.float32) if extra == 3 else None
+    say(f"flash_attn random seed={seed}: B={B} heads={Hkv * gqa}/{Hkv} n_q={n_q} n_kv={n_kv} D={D} kv={kv_dtype.__name__} "
+        f"mask={None if mask is None else mask.shape} max_bias={max_bias} softcap={softcap} sinks={sinks is not None}")
+    fa_case(gpu, q, k, v, mask, scale=1.0 / np.sqrt(D), max_bias=max_bias, softcap=softcap, sinks=sinks, name=f"random {seed}")
+
+
 def test_fa_cfg5_shape_properties(gpu):
     """BASELINE config 5 decode shape (batch 16, L = 8192): too big for the scalar oracle in
     seconds, so check a sample of (batch, head) slices against it plus convexity everywhere."""
