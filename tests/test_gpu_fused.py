@@ -196,6 +196,53 @@ def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     assert L.vx_mul_mat_scale_add(pkg.desc_q8(w, K), d(xl), d(rl), d(dl), 1.0, mode, None) != 0
 
 
+@pytest.mark.parametrize("seed", list(range(120)))
+def test_projection_groups_random_shapes(pkg, gpu, seed):  # (seed 29: one product alone is a streaming shape, the pair is not)
+    """MUL_MAT + SCALE + ADD and MUL_MAT, MUL_MAT, GLU as one call each against their nodes at random row, column and token
+    counts on both sides of every kernel choice (streaming, K cut, 64 x 64 and 128 x 128 tiles, the second pass), both
+    activation modes.  Whatever the predicates announce must come out bit-equal; what they do not announce must be refused."""
+    import torch
+    L, d = pkg.lib(), pkg.desc
+    r = rng("f-proj-random", seed)
+    M = int(r.choice([16, 20, 64, 128, 200, 512, 1000, 1024, 2048]))
+    K = 32 * int(r.choice([2, 8, 16, 32, 33, 64, 128]))
+    N = int(r.choice([1, 2, 5, 14, 16, 17, 40, 63, 64, 65, 112, 128, 200, 300, 700]))
+    nb = int(r.choice([1, 1, 2]))
+    mode = pkg.ACT_Q8 if r.integers(2) else pkg.ACT_FLOAT
+    say(f"projection groups random seed={seed}: M={M} K={K} N={N} batch={nb} act={'q8' if mode == pkg.ACT_Q8 else 'float'}")
+    w, _ = q8_dev((0.05 * r.standard_normal((M, K))).astype(np.float32))
+    w2, _ = q8_dev((0.05 * r.standard_normal((M, K))).astype(np.float32))
+    x = dev(r.standard_normal((nb, 1, N, K)).astype(np.float32))
+    res = dev(r.standard_normal((nb, 1, N, M)).astype(np.float32))
+    prod = torch.empty((nb, 1, N, M), dtype=torch.float32, device="cuda")
+    up, a, b = torch.empty_like(prod), torch.empty_like(prod), torch.full_like(prod, float("nan"))
+    dw, dw2 = pkg.desc_q8(w, K), pkg.desc_q8(w2, K)
+    # projection + scale + residual
+    ok(pkg, L.vx_mul_mat(dw, d(x), d(prod), mode, None), "mul_mat")
+    ok(pkg, L.vx_scale(d(prod), d(up), 0.2857738, 0.0, None), "scale")
+    ok(pkg, L.vx_binary(pkg.BIN_ADD, d(res), d(up), d(a), None), "add")
+    if L.vx_supports_mul_mat_scale_add(dw, d(x), d(res), d(b)):
+        ok(pkg, L.vx_mul_mat_scale_add(dw, d(x), d(res), d(b), 0.2857738, mode, None), "mul_mat_scale_add")
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), "projection + scale + residual"
+        r2 = res.clone()
+        ok(pkg, L.vx_mul_mat_scale_add(dw, d(x), d(r2), d(r2), 0.2857738, mode, None), "mul_mat_scale_add in place")
+        torch.cuda.synchronize()
+        assert torch.equal(a, r2), "in place on the residual"
+    else:
+        assert L.vx_mul_mat_scale_add(dw, d(x), d(res), d(b), 0.2857738, mode, None) != 0
+    # gate, up, GLU
+    ok(pkg, L.vx_mul_mat(dw2, d(x), d(up), mode, None), "up")
+    ok(pkg, L.vx_glu(pkg.GLU_SWIGLU, d(prod), d(up), d(a), 0, None), "glu")
+    b.fill_(float("nan"))
+    if L.vx_supports_mul_mat_swiglu(dw, dw2, d(x), d(b)) or L.vx_supports_mul_mat_swiglu_tiled(dw, dw2, d(x), d(b), mode):
+        ok(pkg, L.vx_mul_mat_swiglu(dw, dw2, d(x), d(b), mode, None), "mul_mat_swiglu")
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), "gate, up, GLU"
+    else:
+        assert L.vx_mul_mat_swiglu(dw, dw2, d(x), d(b), mode, None) != 0
+
+
 @pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2)])
 @pytest.mark.parametrize("poison", [None, "nan", "inf"])
 def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):

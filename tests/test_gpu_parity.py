@@ -458,6 +458,28 @@ def test_mul_mat_q8_0(gpu, M, K, N):
     assert nmse(f64, got_fl) <= 1e-5
 
 
+@pytest.mark.parametrize("seed", list(range(48)))
+def test_mul_mat_q8_0_random_shapes(gpu, seed):
+    """Random row, column and token counts around every threshold the launcher has (streaming kernel up to 16 tokens and a
+    work bound beyond, 64 x 64 and 128 x 128 tiles, the K cut of few tiles, K in whole rounds of 64 or not, rows that are
+    no multiple of 4 or 16): both activation modes against the oracle with test_mul_mat_q8_0's bars."""
+    r = rng("mm-random", seed)
+    M = int(r.choice([1, 3, 16, 24, 64, 65, 130, 200, 512, 1000, 1024, 1030, 2048]))
+    K = 32 * int(r.choice([1, 2, 3, 8, 16, 17, 32, 33, 64, 128]))
+    N = int(r.choice([1, 2, 3, 5, 14, 16, 17, 31, 33, 63, 64, 65, 100, 112, 127, 128, 129, 200, 300, 520]))
+    say(f"mul_mat Q8_0 random seed={seed}: M={M} K={K} N={N}")
+    w, x = mm_inputs(("q8r", seed), M, K, N)
+    wq = reflib.quantize_q8_0(w)
+    cpu = reflib.oracle_mul_mat(wq, x, K, act_mode=0)
+    f64 = reflib.oracle_mul_mat(wq, x, K, f64=True)
+    got_q8 = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_Q8, w_ne0=K))
+    got_fl = sync_np(gpu.mul_mat(dev(wq), dev(x), gpu.ACT_FLOAT, w_ne0=K))
+    scale = np.abs(cpu).max()
+    assert np.abs(got_q8 - cpu).max() / scale <= 1e-5
+    assert nmse(cpu, got_fl) <= 5e-4
+    assert nmse(f64, got_fl) <= 1e-5
+
+
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 1), (1024, 1024, 2), (1000, 1024, 14), (1536, 1024, 16), (1024, 4096, 2), (1024, 4096, 14),
                                    (8192, 1024, 2), (200, 2048, 3), (64, 512, 2), (1024, 768, 5), (24, 1024, 2), (1024, 1024, 17),
                                    (1024, 1024, 40), (4096, 4096, 16)])

@@ -1998,7 +1998,9 @@ extern "C" int vx_supports_mul_mat_swiglu_tiled(const vx_tensor * gate, const vx
     if (gate->type != VX_TYPE_Q8_0 && gate->type != VX_TYPE_F16) return 0;
     if (up->type != gate->type) return 0;
     for (int i = 0; i < 4; ++i) if (up->ne[i] != gate->ne[i] || up->nb[i] != gate->nb[i]) return 0;
-    return !gemv_shape_ok(src1->ne[1], 2 * gate->ne[1], gate->ne[0]) && gemm_lds_swiglu_ok(gate, up, src1, dst, act_mode);
+    // (neither the pair nor one product on its own may be a shape of the streaming kernel: it sums the K blocks in another order)
+    return !gemv_shape_ok(src1->ne[1], 2 * gate->ne[1], gate->ne[0]) && !gemv_shape_ok(src1->ne[1], gate->ne[1], gate->ne[0]) &&
+           gemm_lds_swiglu_ok(gate, up, src1, dst, act_mode);
 }
 
 // whether the activations of a streaming-kernel launch can be normalised on the fly: rows of at most 1024
