@@ -595,10 +595,11 @@ def test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn):
     assert torch.equal(v1, v2)
     assert torch.equal(k1, k2)
     assert torch.equal(q1, q2)
-    if True:   # the same with every sequence's tokens flattened into one token dimension, as a 2-D activation tensor
-        q3, k3, v3 = outs()
-        xf, vf = x.view(B * T, K), v3.view(B * T, Hkv * D)
-        assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(xf), d(q3), d(k3), d(vf), D, 2) == 1
+    # the same with every sequence's tokens flattened into one token dimension, as a 2-D activation tensor (all the
+    # sequences' tokens are then one call's tokens: beyond the streaming kernel's work bound the flattened form is declined)
+    q3, k3, v3 = outs()
+    xf, vf = x.view(B * T, K), v3.view(B * T, Hkv * D)
+    if L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(xf), d(q3), d(k3), d(vf), D, 2):
         ok(pkg, L.vx_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(xf), pos.data_ptr(), ff.data_ptr(),
                                    d(q3), d(k3), d(vf), *rope_args, mode, None), "qkv_proj_rope flattened")
         torch.cuda.synchronize()
@@ -606,6 +607,41 @@ def test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn):
     # NORMAL-mode rotation and partial rotation are left to the separate operators
     assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D, 0) == 0
     assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D // 2, 2) == 0
+
+
+@pytest.mark.parametrize("seed", list(range(40)))
+def test_qkv_and_mlp_groups_random_shapes(pkg, gpu, seed):
+    """The q/k/v + rope group, with and without the norm in front, and the norm + gate/up + SwiGLU group at random token
+    counts, batches, head counts, head sizes and K (several chunks of 16 tokens, K with and without whole rounds, one to
+    eight KV heads): whatever the predicates announce is run through the parametrised tests' own bodies, bit for bit."""
+    import torch
+    L, d = pkg.lib(), pkg.desc
+    r = rng("f-qkv-random", seed)
+    T, B = int(r.choice([1, 2, 3, 5, 14, 16, 17, 21, 40])), int(r.choice([1, 2, 8]))
+    Hkv, gqa, D = int(r.choice([1, 2, 4, 8])), int(r.choice([1, 4, 8])), int(r.choice([32, 64, 128]))
+    K = int(r.choice([256, 512, 768, 1024, 2048]))
+    act, yarn = ("q8" if r.integers(2) else "float"), bool(r.integers(2))
+    H = Hkv * gqa
+    z = lambda rows: pkg.desc_q8(torch.zeros((rows, K // 32 * 34), dtype=torch.uint8, device="cuda"), K)
+    x = torch.empty((B, 1, T, K), dtype=torch.float32, device="cuda")
+    q, k, v = (torch.empty((B, T, H, D), dtype=torch.float32, device="cuda"), torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda"),
+               torch.empty((B, 1, T, Hkv * D), dtype=torch.float32, device="cuda"))
+    ran = []
+    if L.vx_supports_qkv_proj_rope(z(H * D), z(Hkv * D), z(Hkv * D), d(x), d(q), d(k), d(v), D, 2):
+        test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn)
+        ran.append("qkv")
+        nw = torch.empty((K,), dtype=torch.float32, device="cuda")
+        xf, vf = x.view(B * T, K), v.view(B * T, Hkv * D)   # (that test hands over the flattened form)
+        if L.vx_supports_norm_qkv_proj_rope(d(xf), d(nw), z(H * D), z(Hkv * D), z(Hkv * D), d(q), d(k), d(vf), D, 2):
+            test_norm_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act)
+            ran.append("norm + qkv")
+    M = int(r.choice([64, 1000, 2048, 4096]))
+    nw = torch.empty((K,), dtype=torch.float32, device="cuda")
+    act_out = torch.empty((B, 1, T, M), dtype=torch.float32, device="cuda")
+    if L.vx_supports_norm_mul_mat_swiglu(d(x), d(nw), z(M), z(M), d(act_out)):
+        test_norm_mul_mat_swiglu(pkg, gpu, T, B, K, M, act)
+        ran.append("norm + gate/up")
+    say(f"qkv / mlp groups random seed={seed}: T={T} B={B} heads={H}/{Hkv} D={D} K={K} M={M} act={act} yarn={yarn}: ran {ran}")
 
 
 @pytest.mark.parametrize("T,B,K,M", [(1, 2, 1024, 4096), (2, 1, 1024, 4096), (16, 1, 512, 1000), (3, 2, 256, 64), (14, 1, 1024, 4096), (40, 1, 1024, 2048)])
