@@ -35,7 +35,7 @@ GGML_BACKEND_API bool ggml_backend_gfx950_alloc_weights(struct ggml_context * ct
                                                         ggml_backend_buffer_t * device_buffer,
                                                         ggml_backend_buffer_t * host_buffer);
 
-/* diagnostics and switches (see INTEGRATION.md) */
+/* diagnostics and switches */
 GGML_BACKEND_API int ggml_backend_gfx950_last_launches(void);
 GGML_BACKEND_API int ggml_backend_gfx950_set_graph_replay(int on);  /* recognise recurring graphs and replay them; returns the previous setting */
 GGML_BACKEND_API int ggml_backend_gfx950_replays(void);   /* graph_compute calls served by replaying recorded launches */
