@@ -753,6 +753,54 @@ def test_glue_arange_repeat_and_the_mask_chains(gpu):
     assert np.array_equal(sync_np(m16), want)
 
 
+@pytest.mark.parametrize("seed", list(range(48)))
+def test_glue_random_shapes(gpu, seed):
+    """Binary operators with ggml's broadcast rule, REPEAT, CONCAT along every dimension, a tree of CONCATs and copies
+    between shapes, at random 4-d shapes with strided (sliced, permuted) operands: the results are fixed by IEEE arithmetic
+    and by indexing alone, so numpy is the reference and the comparison is exact."""
+    import torch
+    r = rng("glue-random", seed)
+    ne = [int(r.choice([1, 2, 3, 5])), int(r.choice([1, 2, 4, 7])), int(r.choice([1, 3, 14, 17])), int(r.choice([1, 4, 30, 64, 100, 257]))]   # torch order
+    say(f"glue random seed={seed}: shape {ne}")
+    a = r.standard_normal(ne).astype(np.float32)
+    # src1 broadcast: every dim is 1 or the full extent
+    nb_ = [n if r.integers(2) else 1 for n in ne]
+    b = (r.standard_normal(nb_) + 3.0).astype(np.float32)
+    A, Bt = dev(a), dev(b)
+    for op, f in ((gpu.BIN_ADD, np.add), (gpu.BIN_SUB, np.subtract), (gpu.BIN_MUL, np.multiply), (gpu.BIN_DIV, np.divide)):
+        got = sync_np(gpu.binary(op, A, Bt))
+        assert np.array_equal(got, f(a, b).astype(np.float32)), ("binary", op)
+    # a strided first operand: a slice of a wider tensor, and a permuted view
+    wide = r.standard_normal(ne[:3] + [ne[3] + 5]).astype(np.float32)
+    Wd = dev(wide)
+    got = sync_np(gpu.binary(gpu.BIN_ADD, Wd[..., 2:2 + ne[3]], Bt))
+    assert np.array_equal(got, wide[..., 2:2 + ne[3]] + b)
+    perm = dev(np.ascontiguousarray(a.transpose(0, 2, 1, 3)))        # stored [n0, n2, n1, n3], viewed back as [n0, n1, n2, n3]
+    out = torch.empty(ne, dtype=torch.float32, device="cuda")
+    gpu.cpy(perm.permute(0, 2, 1, 3), out)
+    assert np.array_equal(sync_np(out), a), "cpy of a permuted view"
+    # REPEAT of the broadcast operand to the full shape
+    assert np.array_equal(sync_np(gpu.repeat(Bt, tuple(ne))), np.broadcast_to(b, ne)), "repeat"
+    # CONCAT along every ggml dimension (ggml dim d = torch dim 3 - d)
+    for gd in range(4):
+        td = 3 - gd
+        other = list(ne); other[td] = int(r.choice([1, 2, 5]))
+        c = r.standard_normal(other).astype(np.float32)
+        assert np.array_equal(sync_np(gpu.concat(A, dev(c), gd)), np.concatenate([a, c], axis=td)), ("concat", gd)
+    # a tree of CONCATs from its leaves, one leaf repeated, along ggml dim 1 and dim 0
+    for gd in (1, 0):
+        td = 3 - gd
+        l1, l2 = list(ne), list(ne)
+        l1[td], l2[td] = 3, 2
+        small = [1 if i != 3 else ne[3] for i in range(4)] if gd == 1 else [1, 1, ne[2], 1]
+        x1, x2, x3 = r.standard_normal(l1).astype(np.float32), r.standard_normal(l2).astype(np.float32), r.standard_normal(small).astype(np.float32)
+        rep_shape = list(ne); rep_shape[td] = 4 if gd == 1 else 4 * small[3]
+        want = np.concatenate([x1, np.broadcast_to(x3, rep_shape) if gd == 1 else np.tile(x3, [ne[0], ne[1], 1, 4]), x2], axis=td)
+        out = torch.full(want.shape, float("nan"), dtype=torch.float32, device="cuda")
+        gpu.concat_many([dev(x1), dev(x3), dev(x2)], [l1[td], rep_shape[td], l2[td]], gd, out)
+        assert np.array_equal(sync_np(out), want), ("concat_many", gd)
+
+
 def test_glue_get_rows(gpu):
     """GET_ROWS gathers exactly: F32 / I32 rows as bits, F16 widened, Q8_0 as quant * scale (one rounding,
     the oracle's dequantisation); batched tables and a strided index view as ggml's tests use them."""
