@@ -899,4 +899,84 @@ int rh_cfm_solve_requests(const float * z, const float * mu, const float * cond,
 }
 
 
+// ---- a random graph of the small operators around the stacks ------------------------------------------------
+// What the plugin decides per graph (runs of tiny nodes as one launch, values that live in LDS only, trees of CONCATs
+// written from their leaves, pairs of nodes) depends on reader counts and on the memory ggml-alloc hands out -- and
+// ggml-alloc reuses a dead tensor's block at once.  A seeded random DAG of the exact operators (ADD, SUB, MUL with ggml's
+// broadcast, SCALE, SQR, NEG, CONT, REPEAT, CONCAT + a view back, SUM_ROWS, SUM, DIV on the small results) over a handful
+// of inputs, allocated by ggml_gallocr and computed on the selected backend: the same seed gives the same graph on every
+// backend, so ggml-cpu is the reference.  out receives the final [n, R] tensor; *n_nodes the graph's node count.
+int rh_random_graph(uint64_t seed, int n_ops, float * out, int64_t out_cap, int64_t * out_n, int * n_nodes) {
+    if (!g_backend) return 100;
+    uint64_t st = seed * 6364136223846793005ull + 1442695040888963407ull;
+    auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (uint32_t) (st >> 33); };
+    auto pick = [&](int n) { return (int) (rnd() % (uint32_t) n); };
+    auto unif = [&]() { return (float) (rnd() % 20001) / 10000.0f - 1.0f; };
+    const int64_t ns[] = { 64, 100, 257, 1024 }, rs[] = { 1, 2, 3, 8 };
+    const int64_t n = ns[pick(4)], R = rs[pick(4)];
+    ggml_init_params ip = { ggml_tensor_overhead() * (size_t) (32 + 8 * n_ops) + ggml_graph_overhead_custom(1024, false), nullptr, true };
+    ggml_context * ic = ggml_init(ip);   // inputs: their own buffer
+    ggml_context * c  = ggml_init(ip);   // the graph: ggml_gallocr's memory
+    std::vector<ggml_tensor *> full, cols, scal;
+    std::vector<ggml_tensor *> inputs;
+    for (int k = 0; k < 4; ++k) { ggml_tensor * t = ggml_new_tensor_2d(ic, GGML_TYPE_F32, n, R); inputs.push_back(t); full.push_back(t); }
+    ggml_tensor * row = ggml_new_tensor_2d(ic, GGML_TYPE_F32, n, 1); inputs.push_back(row);
+    { ggml_tensor * t = ggml_new_tensor_2d(ic, GGML_TYPE_F32, 1, R); inputs.push_back(t); cols.push_back(t); }
+    { ggml_tensor * t = ggml_new_tensor_1d(ic, GGML_TYPE_F32, 1); inputs.push_back(t); scal.push_back(t); }
+    ggml_backend_buffer_t ibuf = ggml_backend_alloc_ctx_tensors(ic, g_backend);
+    if (!ibuf) { ggml_free(ic); ggml_free(c); return 101; }
+    for (ggml_tensor * t : inputs) {
+        std::vector<float> v((size_t) ggml_nelements(t));
+        for (float & x : v) x = unif();
+        if (ggml_nelements(t) <= R) for (float & x : v) x += 2.5f; // (divisors and scalars away from zero)
+        ggml_backend_tensor_set(t, v.data(), 0, ggml_nbytes(t));
+    }
+    std::vector<int> uses(full.size(), 0);
+    auto take = [&]() { const int k = pick((int) full.size()); ++uses[k]; return full[k]; };
+    auto put  = [&](ggml_tensor * t) { full.push_back(t); uses.push_back(0); };
+    for (int k = 0; k < n_ops; ++k) {
+        switch (pick(14)) {
+            case 0: put(ggml_add(c, take(), take())); break;
+            case 1: put(ggml_sub(c, take(), take())); break;
+            case 2: put(ggml_mul(c, take(), take())); break;
+            case 3: put(ggml_add(c, take(), pick(2) ? row : (pick(2) ? cols[pick((int) cols.size())] : scal[pick((int) scal.size())]))); break;
+            case 4: put(ggml_mul(c, take(), pick(2) ? row : (pick(2) ? cols[pick((int) cols.size())] : scal[pick((int) scal.size())]))); break;
+            case 5: put(ggml_scale(c, take(), 0.25f + 0.5f * (float) pick(4))); break;
+            case 6: put(pick(2) ? ggml_sqr(c, take()) : ggml_neg(c, take())); break;
+            case 7: put(ggml_cont(c, take())); break;
+            case 8: put(ggml_repeat(c, pick(2) ? row : (pick(2) ? cols[pick((int) cols.size())] : scal[pick((int) scal.size())]), full[0])); break;
+            case 9: { // CONCAT of two along the row dimension (or of a CONCAT and a third), then one half back as a view
+                ggml_tensor * cat = ggml_concat(c, take(), take(), 1);
+                if (pick(2)) cat = ggml_concat(c, cat, take(), 1);
+                const int64_t first = pick((int) (cat->ne[1] / R)) * R;
+                put(ggml_cont(c, ggml_view_2d(c, cat, n, R, cat->nb[1], (size_t) first * cat->nb[1])));
+            } break;
+            case 10: cols.push_back(ggml_sum_rows(c, take())); break;
+            case 11: scal.push_back(ggml_sum(c, take())); break;
+            case 12: cols.push_back(ggml_div(c, cols[pick((int) cols.size())], cols[pick((int) cols.size())])); break;
+            default: scal.push_back(ggml_scale(c, scal[pick((int) scal.size())], 0.5f)); break;
+        }
+    }
+    // everything nobody read yet flows into the result, so that (nearly) every node is an ancestor of it
+    ggml_tensor * res = full.back();
+    for (size_t k = 4; k + 1 < full.size(); ++k) if (uses[k] == 0) res = ggml_add(c, res, full[k]);
+    res = ggml_add(c, res, ggml_repeat(c, cols.back(), res));
+    res = ggml_add(c, res, scal.back());
+    ggml_set_output(res);
+    ggml_cgraph * gf = ggml_new_graph_custom(c, 1024, false);
+    ggml_build_forward_expand(gf, res);
+    ggml_gallocr_t ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend));
+    int rc = 0;
+    if (!ggml_gallocr_alloc_graph(ga, gf)) rc = 101;
+    for (int rep = 0; rep < 2 && !rc; ++rep) // twice: the second computation finds whatever the first left in reused blocks
+        if (ggml_backend_graph_compute(g_backend, gf) != GGML_STATUS_SUCCESS) rc = 102;
+    if (!rc && ggml_nelements(res) > out_cap) rc = 103;
+    if (!rc) { ggml_backend_tensor_get(res, out, 0, ggml_nbytes(res)); *out_n = ggml_nelements(res); *n_nodes = ggml_graph_n_nodes(gf); }
+    ggml_gallocr_free(ga);
+    ggml_backend_buffer_free(ibuf);
+    ggml_free(c);
+    ggml_free(ic);
+    return rc;
+}
+
 } // extern "C"

@@ -188,6 +188,7 @@ def load_ref():
     lib.rh_cfm_solve.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int,
                                  f32p_, C.c_int, C.POINTER(C.c_double)]
     lib.rh_bb_two_stage.argtypes = [f32p_, u16p_, C.c_int, C.c_int, f32p_, C.c_int, C.POINTER(C.c_double)]
+    lib.rh_random_graph.argtypes = [C.c_uint64, C.c_int, C.POINTER(C.c_float), C.c_int64, C.POINTER(C.c_int64), C.POINTER(C.c_int)]
     lib.rh_cfm_solve_requests.argtypes = [f32p_, f32p_, f32p_, f32p_, f32p_, C.c_int, C.c_int, C.c_int, i32p_, u16p_, C.c_float, C.c_int, C.c_int,
                                           f32p_, C.c_int, C.POINTER(C.c_double)]
     lib.rh_cfm_set_time_mlp.argtypes = [C.c_int, C.c_void_p, f32p_]

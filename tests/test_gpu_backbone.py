@@ -498,3 +498,40 @@ def test_plugin_replays_a_recurring_graph(gpu, ref):
     cpu = solve_all(b"CPU", False, 0)
     for i, (a, b) in enumerate(zip(cpu, replayed)):
         assert nmse(a, b) <= 1e-3, i
+
+
+@pytest.mark.gpu
+def test_plugin_on_random_graphs_of_small_operators(gpu, ref):
+    """Seeded random DAGs of the exact small operators (binary operators with broadcast, SCALE, SQR, NEG, CONT, REPEAT,
+    CONCAT and a view back, SUM_ROWS, SUM, DIV), allocated by ggml_gallocr -- which hands a dead tensor's memory to the next
+    node at once -- and computed twice: the plugin's per-graph decisions (runs of tiny nodes in one launch, values kept in LDS
+    only, CONCAT trees written from their leaves, node pairs) against ggml-cpu on the same graph.  The operators are exact,
+    so the results agree bit for bit except through the order of a sum's fp64 additions."""
+    import ctypes as C
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plug = C.CDLL(gpu.PLUGIN_PATH)
+    cap = 1024 * 8
+    worst, fused, exact = 0.0, 0, 0
+    seeds = list(range(400))
+    for seed in seeds:
+        outs = []
+        for device in (b"CPU", b"GFX950_0"):
+            assert ref.rh_use_device(device, 8, 0) == 0
+            buf = np.zeros(cap, np.float32)
+            n, nodes = C.c_int64(0), C.c_int(0)
+            rc = ref.rh_random_graph(seed, 8 + seed % 40, buf.ctypes.data_as(C.POINTER(C.c_float)), cap, C.byref(n), C.byref(nodes))
+            assert rc == 0, (seed, device, rc)
+            outs.append(buf[:n.value].copy())
+            if device != b"CPU":
+                launches = plug.ggml_backend_gfx950_last_launches()
+                fused += launches < nodes.value
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        cpu, dev_ = outs
+        assert np.isfinite(cpu).all(), seed
+        err = float(np.abs(cpu - dev_).max() / max(1.0, float(np.abs(cpu).max())))
+        exact += bool(np.array_equal(cpu, dev_))
+        worst = max(worst, err)
+        assert err <= 1e-5, (seed, err, nodes.value)
+    print(f"random graphs: {len(seeds)} seeds, {exact} bit-equal, worst relative difference {worst:.2e}, {fused} with fewer launches than nodes", flush=True)
+    assert fused >= len(seeds) // 2 and exact >= len(seeds) // 2
+
