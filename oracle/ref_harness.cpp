@@ -912,8 +912,8 @@ int rh_random_graph(uint64_t seed, int n_ops, float * out, int64_t out_cap, int6
     auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (uint32_t) (st >> 33); };
     auto pick = [&](int n) { return (int) (rnd() % (uint32_t) n); };
     auto unif = [&]() { return (float) (rnd() % 20001) / 10000.0f - 1.0f; };
-    const int64_t ns[] = { 64, 100, 257, 1024 }, rs[] = { 1, 2, 3, 8 };
-    const int64_t n = ns[pick(4)], R = rs[pick(4)];
+    const int64_t ns[] = { 64, 100, 257, 1024, 4096 }, rs[] = { 1, 2, 3, 8 }; // (4096 x 8: beyond a small-graph run, every node its own launch or pair)
+    const int64_t n = ns[pick(5)], R = rs[pick(4)];
     ggml_init_params ip = { ggml_tensor_overhead() * (size_t) (32 + 8 * n_ops) + ggml_graph_overhead_custom(1024, false), nullptr, true };
     ggml_context * ic = ggml_init(ip);   // inputs: their own buffer
     ggml_context * c  = ggml_init(ip);   // the graph: ggml_gallocr's memory

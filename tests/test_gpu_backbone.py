@@ -510,9 +510,9 @@ def test_plugin_on_random_graphs_of_small_operators(gpu, ref):
     import ctypes as C
     assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
     plug = C.CDLL(gpu.PLUGIN_PATH)
-    cap = 1024 * 8
-    worst, fused, exact = 0.0, 0, 0
-    seeds = list(range(400))
+    cap = 4096 * 8
+    worst, fused, exact, overflowed = 0.0, 0, 0, 0
+    seeds = list(range(600))
     for seed in seeds:
         outs = []
         for device in (b"CPU", b"GFX950_0"):
@@ -527,11 +527,14 @@ def test_plugin_on_random_graphs_of_small_operators(gpu, ref):
                 fused += launches < nodes.value
         assert ref.rh_use_device(b"CPU", 8, 0) == 0
         cpu, dev_ = outs
-        assert np.isfinite(cpu).all(), seed
+        if not np.isfinite(cpu).all():   # a chain of squares ran out of range: the same non-finite values have to come back
+            assert np.array_equal(np.isnan(cpu), np.isnan(dev_)), seed
+            overflowed += 1
+            continue
         err = float(np.abs(cpu - dev_).max() / max(1.0, float(np.abs(cpu).max())))
         exact += bool(np.array_equal(cpu, dev_))
         worst = max(worst, err)
         assert err <= 1e-5, (seed, err, nodes.value)
-    print(f"random graphs: {len(seeds)} seeds, {exact} bit-equal, worst relative difference {worst:.2e}, {fused} with fewer launches than nodes", flush=True)
-    assert fused >= len(seeds) // 2 and exact >= len(seeds) // 2
+    print(f"random graphs: {len(seeds)} seeds ({overflowed} out of range), {exact} bit-equal, worst relative difference {worst:.2e}, {fused} with fewer launches than nodes", flush=True)
+    assert fused >= len(seeds) // 2 and exact >= len(seeds) * 9 // 10 and overflowed <= len(seeds) // 50
 
