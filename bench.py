@@ -732,6 +732,10 @@ def main():
             "backbone_decode_steps_per_s_cfg4_through_plugin": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_ggml_cpu": pick("cfg4_backbone_24layers_b2", "ggml_cpu", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg5_f16kv": pick("cfg5_backbone_24layers_b16_f16kv", "decode_steps_per_s"),
+            "backbone_prefill_tokens_per_s_cfg4": pick("cfg4_backbone_24layers_b2", "prefill_tokens_per_s"),
+            "backbone_prefill_tokens_per_s_cfg5_f16kv": pick("cfg5_backbone_24layers_b16_f16kv", "prefill_tokens_per_s"),
+            "cfm_solve_us_cfg3_one_request": pick("cfg3_cfm_solve_one_request", "us_per_cfm_solve"),
+            "cfm_solves_per_s_cfg3_8_requests_through_plugin": pick("cfg3_cfm_solve_8_requests_through_plugin", "solves_per_s"),
         },
         "others": others,
     }
