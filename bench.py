@@ -730,6 +730,7 @@ def main():
             "backbone_decode_steps_per_s_cfg4": pick("cfg4_backbone_24layers_b2", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_f16kv": pick("cfg4_backbone_24layers_b2_f16kv", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_through_plugin": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_through_plugin_same_graph_replayed": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "same_graph_replayed", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_ggml_cpu": pick("cfg4_backbone_24layers_b2", "ggml_cpu", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg5_f16kv": pick("cfg5_backbone_24layers_b16_f16kv", "decode_steps_per_s"),
             "backbone_prefill_tokens_per_s_cfg4": pick("cfg4_backbone_24layers_b2", "prefill_tokens_per_s"),
