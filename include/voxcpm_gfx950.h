@@ -351,8 +351,10 @@ VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor
 /* The reference's KV append with its write-ordering scalar (attention_forward, src/minicpm.cpp:682-713), nine graph
  * nodes as one launch:  CPY(k, k_slot) CONT SUM , CPY(v, v_slot) CONT SUM , ADD , SCALE(scale, bias) , ADD1(x, .)
  *   k_slot <- k ; v_slot <- v ; dst = x + ((sum(k_slot) + sum(v_slot)) * scale + bias)
- * k, v, x F32; a cache write of at most 16384 elements (decode-sized), x of at most 65536; k_slot / v_slot with
- * dense rows, F32 or F16.  With F16 slots the node sequence is CPY(k, k_slot) CPY(k_slot -> F32) SUM ...: the values are
+ * k, v, x F32; a cache write of at most 16384 elements (decode-sized) with x of at most 65536, or a prefill's write --
+ * both of more than 16 Ki sum units (4 elements of a 16-byte aligned row, else one), i.e. sums that vx_sum spreads over
+ * its 128 blocks -- as two launches (stores and block totals; totals, scalar and ADD1) in place of eleven; k_slot /
+ * v_slot with dense rows, F32 or F16.  With F16 slots the node sequence is CPY(k, k_slot) CPY(k_slot -> F32) SUM ...: the values are
  * rounded to nearest even on the way in and the sums see the rounded values.  The sums are formed in vx_sum's order,
  * so dst equals what the separate nodes give. */
 VX_API vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,

@@ -298,14 +298,62 @@ def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):
 
 def test_kv_store_sync_limits(pkg, gpu):
     import torch
-    say("fused cache write: sizes beyond one block are refused")
+    say("fused cache write: sizes between one block's sum and the 128-block sum are refused")
     L, d = pkg.lib(), pkg.desc
-    k = torch.zeros((2, 512, 2, 64), dtype=torch.float32, device="cuda")
+    k = torch.zeros((2, 100, 2, 64), dtype=torch.float32, device="cuda")      # 25600 elements: 6400 units, one block's sum
     c = torch.zeros((2, 2, 600, 64), dtype=torch.float32, device="cuda")
-    x = torch.zeros((2, 512, 16, 64), dtype=torch.float32, device="cuda")
-    s = c[:, :, :512].transpose(1, 2)
+    x = torch.zeros((2, 100, 16, 64), dtype=torch.float32, device="cuda")
+    s = c[:, :, :100].transpose(1, 2)
     assert L.vx_supports_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x)) == 0
     assert L.vx_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x), 0.0, 0.0, None) != 0
+
+
+@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 512, 2, 64, 16), (16, 300, 2, 64, 16), (1, 1100, 1, 64, 4), (3, 600, 2, 30, 2)])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("poison", [None, "nan"])
+def test_kv_store_sync_prefill_sized(pkg, gpu, B, T, Hkv, D, H, f16, poison):
+    """The cache write of a prefill (src/minicpm.cpp:682-690 with hundreds of tokens): CPY into the slot, CONT (the cast
+    back from an F16 cache), SUM -- then the 128-block form of the sum kernel and the kernel that adds its partials --,
+    twice, ADD, SCALE, ADD1 over the attention output: eleven launches against the two of vx_kv_store_sync, bit for bit,
+    cache contents included.  Rows of 64 and of 30 values (with and without 16-byte units)."""
+    import torch
+    say(f"prefill-sized cache write B={B} T={T} Hkv={Hkv} D={D} H={H} f16={f16} poison={poison}")
+    if f16 and D % 4:
+        pytest.skip("an F16 slot needs rows in whole 8-byte groups")
+    L, d = pkg.lib(), pkg.desc
+    g = rng("f-kvs-large", B, T, Hkv, D)
+    n_past = 7
+    k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    if poison:
+        v[B - 1, T // 2, 0, 3] = float("nan")
+    attn = dev(g.standard_normal((B, T, H, D)).astype(np.float32))
+    cdt = torch.float16 if f16 else torch.float32
+    kc1, vc1, kc2, vc2 = (torch.zeros((B, Hkv, n_past + T + 5, D), dtype=cdt, device="cuda") for _ in range(4))
+    slot = lambda c: c[:, :, n_past:n_past + T].transpose(1, 2)
+    cont = torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda")
+    sk, sv, sync = (torch.empty(1, dtype=torch.float32, device="cuda") for _ in range(3))
+    a = torch.empty_like(attn)
+    for src, c, s_ in ((k, kc1, sk), (v, vc1, sv)):
+        ok(pkg, L.vx_cpy(d(src), d(slot(c)), None), "cpy")
+        ok(pkg, L.vx_cpy(d(slot(c)), d(cont), None), "cont")
+        ok(pkg, L.vx_sum(d(cont), d(s_), None), "sum")
+    ok(pkg, L.vx_binary(pkg.BIN_ADD, d(sk), d(sv), d(sync), None), "add")
+    ok(pkg, L.vx_scale(d(sync), d(sync), 0.25, 0.5, None), "scale")
+    ok(pkg, L.vx_add1(d(attn), d(sync), d(a), None), "add1")
+    b = torch.full_like(attn, 7.0)
+    assert L.vx_supports_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(attn), d(b)) == 1
+    ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(attn), d(b), 0.25, 0.5, None), "kv_store_sync")
+    torch.cuda.synchronize()
+    assert torch.equal(kc1.view(torch.uint8), kc2.view(torch.uint8)) and torch.equal(vc1.view(torch.uint8), vc2.view(torch.uint8))
+    assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
+    if poison:
+        assert not bool(torch.isfinite(b).any())
+    # in place on the attention output
+    x2 = attn.clone()
+    ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(x2), d(x2), 0.25, 0.5, None), "in place")
+    torch.cuda.synchronize()
+    assert torch.equal(a.nan_to_num(123.0), x2.nan_to_num(123.0))
 
 
 @pytest.mark.parametrize("shape", [(8, 128), (1, 1), (3, 5, 7, 1000), (2, 4100), (16, 2, 64)])

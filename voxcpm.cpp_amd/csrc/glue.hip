@@ -1033,6 +1033,49 @@ __global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
     }
 }
 
+// A prefill's cache write (tens of thousands of keys at once): the same nodes, of which the two SUMs are then the
+// 128-block form of GGML_OP_SUM's kernel -- thread t of block b walks units b * 1024 + t, + 128 * 1024, ...; the
+// blocks' fp64 totals are added in block order by a second kernel.  Here the first kernel also stores the slots (one
+// grid half per cache), and the second, which adds the totals, forms the scalar and applies the ADD1 to x.
+template <bool VK, bool VV>
+__global__ __launch_bounds__(1024) void kv_store_large_kernel(const kvs_args a, double * partials) {
+    __shared__ double part[16];
+    const bool     second = blockIdx.x >= SUM_BLOCKS; // uniform
+    const uint32_t b = blockIdx.x - (second ? SUM_BLOCKS : 0);
+    double acc = 0.0;
+    if (!second) { const uint32_t n = kvs_units(a.k, VK); for (uint32_t e = b * 1024 + threadIdx.x; e < n; e += SUM_BLOCKS * 1024) kvs_unit<VK>(a.k, e, true, acc); }
+    else         { const uint32_t n = kvs_units(a.v, VV); for (uint32_t e = b * 1024 + threadIdx.x; e < n; e += SUM_BLOCKS * 1024) kvs_unit<VV>(a.v, e, true, acc); }
+    const double t = block_total(acc, part);
+    if (threadIdx.x == 0) partials[blockIdx.x] = t;
+}
+
+__global__ __launch_bounds__(256) void kv_sync_add1_kernel(const kvs_args a, const double * partials) {
+    __shared__ double part[2 * SUM_BLOCKS];
+    __shared__ float  y_s;
+    static_assert(2 * SUM_BLOCKS == 256, "a partial per thread");
+    part[threadIdx.x] = partials[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tk = 0.0, tv = 0.0;
+        for (int i = 0; i < SUM_BLOCKS; ++i) tk += part[i];               // (sum_partials_kernel's order)
+        for (int i = 0; i < SUM_BLOCKS; ++i) tv += part[SUM_BLOCKS + i];
+        y_s = kvs_scalar((float) tk, (float) tv, a.scale, a.bias);
+    }
+    __syncthreads();
+    const float y = y_s;
+    const uint32_t n0 = (uint32_t) a.ne[0], n1 = (uint32_t) a.ne[1], n2 = (uint32_t) a.ne[2];
+    const uint64_t nx = (uint64_t) n0 * n1 * (uint64_t) (n2 * a.ne[3]);
+    for (uint64_t e = (uint64_t) blockIdx.x * 256 + threadIdx.x; e < nx; e += (uint64_t) gridDim.x * 256) {
+        uint64_t r = e;
+        const uint32_t i0 = (uint32_t) (r % n0); r /= n0;
+        const uint32_t i1 = (uint32_t) (r % n1); r /= n1;
+        const uint32_t i2 = (uint32_t) (r % n2), i3 = (uint32_t) (r / n2);
+        const uint64_t ox = i0 * a.nbx[0] + i1 * a.nbx[1] + i2 * a.nbx[2] + i3 * a.nbx[3];
+        const uint64_t od = i0 * a.nbd[0] + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
+        *(float *) (a.d + od) = *(const float *) (a.x + ox) + y;  // the ADD1 node
+    }
+}
+
 } // namespace
 
 // ================================================================================== C ABI
@@ -1763,18 +1806,28 @@ extern "C" vx_status vx_sum_rows(const vx_tensor * src, const vx_tensor * dst, v
     return VX_OK;
 }
 
+// a prefill-sized write: both sums are ones that GGML_OP_SUM's kernel spreads over its 128 blocks (more than 16 Ki units)
+static bool kvs_large(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot) {
+    if (!kvs_side_ok(k, k_slot, (int64_t) 1 << 24) || !kvs_side_ok(v, v_slot, (int64_t) 1 << 24)) return false;
+    kvs_side sk, sv;
+    kvs_side_fill(sk, k, k_slot);
+    kvs_side_fill(sv, v, v_slot);
+    return vx_nelements(k) / (sk.vec ? 4 : 1) > 16 * 1024 && vx_nelements(v) / (sv.vec ? 4 : 1) > 16 * 1024;
+}
+
 extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                          const vx_tensor * x, const vx_tensor * dst) {
     if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;
-    if (!kvs_side_ok(k, k_slot) || !kvs_side_ok(v, v_slot)) return 0;
-    if (!f32(x) || !f32(dst) || !vx_positive(x) || !vx_same_shape(x, dst) || vx_nelements(x) > 65536) return 0;
-    return nb_multiple(x, 4) && nb_multiple(dst, 4);
+    if (!f32(x) || !f32(dst) || !vx_positive(x) || !vx_same_shape(x, dst) || !nb_multiple(x, 4) || !nb_multiple(dst, 4)) return 0;
+    if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) return vx_nelements(x) <= 65536;
+    return kvs_large(k, k_slot, v, v_slot) && vx_nelements(x) < ((int64_t) 1 << 31);
 }
 
 extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                       const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream) {
     if (!vx_supports_kv_store_sync(k, k_slot, v, v_slot, x, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors, at most 16384 elements per cache write and 65536 in x");
+        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors; at most 16384 elements per cache write and 65536 in x, or both writes of more than "
+                       "65536 elements (a prefill's)");
     if (!k->data || !k_slot->data || !v->data || !v_slot->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "kv_store_sync: null data");
     kvs_args a;
     kvs_side_fill(a.k, k, k_slot);
@@ -1782,7 +1835,22 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
     a.x = (const char *) x->data; a.d = (char *) dst->data;
     for (int i = 0; i < 4; ++i) { a.ne[i] = x->ne[i]; a.nbx[i] = x->nb[i]; a.nbd[i] = dst->nb[i]; }
     a.scale = scale; a.bias = bias;
-    kv_store_sync_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
+    if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) {
+        kv_store_sync_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
+    } else { // a prefill's write: stores and block totals, then totals, scalar and ADD1
+        void * ws = nullptr;
+        const vx_status rc = vx_workspace((hipStream_t) stream, 2 * SUM_BLOCKS * sizeof(double), &ws);
+        if (rc != VX_OK) return rc;
+        const dim3 grid(2 * SUM_BLOCKS), block(1024);
+        hipStream_t st = (hipStream_t) stream;
+        if (a.k.vec && a.v.vec) kv_store_large_kernel<true, true><<<grid, block, 0, st>>>(a, (double *) ws);
+        else if (a.k.vec)       kv_store_large_kernel<true, false><<<grid, block, 0, st>>>(a, (double *) ws);
+        else if (a.v.vec)       kv_store_large_kernel<false, true><<<grid, block, 0, st>>>(a, (double *) ws);
+        else                    kv_store_large_kernel<false, false><<<grid, block, 0, st>>>(a, (double *) ws);
+        const int64_t nx = vx_nelements(x);
+        const unsigned blocks = (unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096);
+        kv_sync_add1_kernel<<<dim3(blocks), dim3(256), 0, st>>>(a, (const double *) ws);
+    }
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -17,9 +17,9 @@ struct kvs_side {
 };
 
 // host side: what one cache write may look like, and its kernel argument
-static inline bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot) {
+static inline bool kvs_side_ok(const vx_tensor * src, const vx_tensor * slot, int64_t max_elements = 16384) {
     if (!src || !slot || src->type != VX_TYPE_F32 || (slot->type != VX_TYPE_F32 && slot->type != VX_TYPE_F16) || !vx_positive(src)) return false;
-    if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > 16384) return false;
+    if (vx_nelements(src) != vx_nelements(slot) || vx_nelements(src) > max_elements) return false;
     for (int i = 0; i < 4; ++i) if (src->nb[i] % 4) return false;
     if (slot->type == VX_TYPE_F16) {
         // the sum is taken over a dense F32 copy of the slot (vx_sum's 4-element units need ne0 % 4 == 0 only); the
