@@ -260,8 +260,10 @@ def test_supports_truth_table_node_groups(pkg):
     assert lib.vx_supports_kv_store_sync(k_src, D(pkg, pkg.F16, [Dh, Hkv, 1, 2], [2, 2 * Dh * 768, 2 * Dh, 2 * Dh * 768 * Hkv], 0x1002),
                                          k_src, slot, attn, attn) == 0                                            # slot not 8-byte aligned
     assert lib.vx_supports_kv_store_sync(f16(pkg, [Dh, Hkv, 1, 2]), slot16, k_src, slot, attn, attn) == 0       # F16 source
-    big = f32(pkg, [Dh, Hkv, 512, 2])
-    assert lib.vx_supports_kv_store_sync(big, big, big, big, attn, attn) == 0                                     # prefill-sized
+    big, mid = f32(pkg, [Dh, Hkv, 512, 2]), f32(pkg, [Dh, Hkv, 100, 2])
+    assert lib.vx_supports_kv_store_sync(big, big, big, big, attn, attn) == 1                                     # a prefill's write: sums over 128 blocks
+    assert lib.vx_supports_kv_store_sync(mid, mid, mid, mid, attn, attn) == 0                                     # in between: one block's sum
+    assert lib.vx_supports_kv_store_sync(big, big, mid, mid, attn, attn) == 0
     # attention over cached + current keys
     q = f32(pkg, [Dh, 1, H, 2])
     past = D(pkg, pkg.F32, [Dh, 640, Hkv, 2], [4, 4 * Dh, 4 * Dh * 768, 4 * Dh * 768 * Hkv])
