@@ -1814,6 +1814,25 @@ bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
 // 10-22 % faster).  Read on every call: a product of this size takes tens of microseconds.
 int gemm_lds_mode() { const char * e = getenv("VX_GEMM_LDS"); return e ? atoi(e) : 1; }
 
+// The cut of K for a product of 64 x 64 tiles, from its shape alone (the groups that promise a single product's bits ask it
+// too).  Fewer than 64 tiles (the down-projection of a hundred tokens: 32 tiles, 64 rounds): cut so that some 256
+// work-groups walk 8 or more rounds each.  Up to 256 tiles -- one work-group or less to a compute unit, whose rounds then
+// follow each other with nothing to hide a load behind -- and 32 or more rounds (the down-projection of a thousand tokens:
+// 256 tiles, 64 rounds, 51 us): halves or quarters, so that several work-groups share a compute unit.
+int gemm_lds_cut(int64_t M, int64_t N, int64_t K, int64_t nbatch) {
+    if (((M + 127) / 128) * ((N + 127) / 128) * nbatch >= 192) return 1;
+    const int64_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64) * nbatch, rounds = K / (32 * GL_KC);
+    int ks = 1;
+    if (tiles64 < 64) {
+        while (ks < 16 && tiles64 * ks < 192 && rounds % (4 * ks) == 0 && rounds / (2 * ks) >= 4) ks *= 2;
+    } else if (tiles64 <= 256 && rounds >= 32) {
+        // (measured on 24 layers at 2 x 512 tokens, K = 4096: whole 4.98 ms, halves 4.67, quarters 4.62; the same cut for the
+        // 16 rounds of K = 1024 costs more in partials than it hides: 4.68)
+        ks = rounds >= 64 && rounds % 4 == 0 ? 4 : (rounds % 2 == 0 ? 2 : 1);
+    }
+    return ks;
+}
+
 template <int WT>
 bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     const int mode = gemm_lds_mode();
@@ -1828,13 +1847,11 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     const int64_t tiles64 = ((a.M + 63) / 64) * ((a.N + 63) / 64) * nbatch;
-    if (!big && tiles64 < 64) {
-        // Few tiles and a long K (the down-projection of a hundred tokens: 32 tiles, 64 rounds): the K range is cut so
-        // that some 256 work-groups walk 8 or more rounds each, and a second kernel adds their partials in split order.
-        const int64_t rounds = a.K / (32 * GL_KC);
-        int ks = 1;
-        while (ks < 16 && tiles64 * ks < 192 && rounds % (4 * ks) == 0 && rounds / (2 * ks) >= 4) ks *= 2;
-        if (ks < 2 || a.M % 4 || (uintptr_t) a.dst % 16 || a.nb1 % 16 || a.nb2 % 16 || a.nb3 % 16 || (int64_t) nbatch * ks > 65535) return false;
+    const int  ks = gemm_lds_cut(a.M, a.N, a.K, nbatch);
+    const bool cut_fits = !(a.M % 4 || (uintptr_t) a.dst % 16 || a.nb1 % 16 || a.nb2 % 16 || a.nb3 % 16 || (int64_t) nbatch * ks > 65535);
+    if (!big && tiles64 < 64 && !(ks >= 2 && cut_fits)) return false; // (few tiles with K whole: the other kernels' shape)
+    if (ks >= 2 && cut_fits) {
+        // the K range is cut across ks work-groups per tile; a second kernel adds their partials in split order
         void * ws = nullptr;
         if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) != VX_OK) { (void) hipGetLastError(); return false; }
         mm_args b = a;
@@ -1990,7 +2007,7 @@ static bool gemm_lds_swiglu_ok(const vx_tensor * gate, const vx_tensor * up, con
     if (!al(gate, wm) || !al(up, wm)) return false;
     if ((uint64_t) M * gate->nb[1] >= (1ull << 32) || (uint64_t) 256 * src1->nb[1] + 256 >= (1ull << 32) || (uint64_t) 256 * dst->nb[1] + 1024 >= (1ull << 32)) return false;
     // (each product on its own must be one that the tiled kernel walks with its K whole: a cut K is summed in another order)
-    return ((M + 63) / 64) * ((N + 63) / 64) * nbatch >= 64;
+    return ((M + 63) / 64) * ((N + 63) / 64) * nbatch >= 64 && gemm_lds_cut(M, N, K, nbatch) == 1;
 }
 
 extern "C" int vx_supports_mul_mat_swiglu_tiled(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst, int act_mode) {
