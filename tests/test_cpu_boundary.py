@@ -212,6 +212,12 @@ def test_supports_truth_table_node_groups(pkg):
     small = q8(pkg, [K, 1024, 1, 1])
     assert tiled(small, small, acts(128), acts(128), pkg.ACT_FLOAT) == 0                       # 32 tiles: its K would be cut
     assert tiled(wgate, q8(pkg, [K, 2048, 1, 1]), acts(1024), ffn(1024), pkg.ACT_FLOAT) == 0   # matrices of different shapes
+    # 64..256 tiles with K of 2048 or more: one product on its own is cut in two or four, the pair is not
+    long_k = q8(pkg, [4096, 2048, 1, 1])
+    pair_out = lambda n: f32(pkg, [2048, n, 1, 1])
+    assert tiled(long_k, long_k, acts(128, 4096), pair_out(128), pkg.ACT_FLOAT) == 0           # 64 tiles
+    assert tiled(long_k, long_k, acts(512, 4096), pair_out(512), pkg.ACT_FLOAT) == 0           # 256 tiles
+    assert tiled(long_k, long_k, acts(576, 4096), pair_out(576), pkg.ACT_FLOAT) == 1           # 288 tiles: K whole
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), acts(3), acts(2)) == 0                  # residual of another shape
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(1), acts(14)) == 1                # a bias row, repeated over the tokens
     assert lib.vx_supports_mul_mat_scale_add(q8(pkg, [64, K, 1, 1]), acts(2, 64), acts(1), acts(2)) == 1   # LocDiT's in_proj + bias
