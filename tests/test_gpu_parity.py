@@ -347,8 +347,11 @@ def test_fa_full_size_invariants(gpu):
     o12 = gpu.flash_attn_ext(qd, kd.float(), vsum, None, 0.125)
     e_lin = float((o12 - (base + 2.0 * o2)).abs().max())
     say(f"   key permutation: max-abs {e_perm:.3e};  linearity in V: max-abs {e_lin:.3e}")
-    assert e_perm <= 2e-5
-    assert e_lin <= 2e-5
+    # the streaming kernel of an f16 cache rounds Q and the probabilities to f16 (the prefill kernel's arithmetic): the
+    # order of the keys moves which probabilities share a reference, and the F32 comparison run keeps hi + lo parts of
+    # everything; both stay two orders of magnitude inside the 2e-3 bar
+    assert e_perm <= 2e-4
+    assert e_lin <= 2e-4
 
     T = 4096
     q, k, v = qkv("cfg5pre", 1, 16, 2, T, T)

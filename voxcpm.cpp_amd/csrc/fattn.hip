@@ -637,6 +637,304 @@ int64_t fa_tiles(const vx_tensor * q, const vx_tensor * k) {
     return q->ne[3] * k->ne[2] * ((q->ne[1] * gqa + 15) / 16);
 }
 
+// ---- the streaming kernel for an f16 cache at decode (head size 64, one pair of tensors, no mask, no soft cap) -------
+// The same work split as above (a wave = 16 columns x one key range), built for the one thing that bounds a long
+// cache: bytes in flight per instruction issued.  A 32-key tile of K and of V is 8 direct loads into LDS
+// (global_load_lds_dwordx4: 1 KB each, no registers, no address arithmetic: a scalar base per 8 rows and one lane
+// offset; non-temporal, which alone is worth a microsecond and a half on a 64 MiB call), three tiles deep; K rows are
+// read back as the A operand of S^T = K Q^T (16-byte chunks xor-swizzled by the row, 8-row blocks 128 bytes apart:
+// conflict-free), V^T comes from the row-major V tile through the transposing LDS read (ds_read_b64_tr_b16), so no
+// matrix instruction and no conversion is spent on the transpose.  Q (pre-scaled by scale * log2 e) and P are single
+// f16 operands, as in the prefill kernel: 8 matrix instructions a tile where the general kernel issues 24, and 8 exp2.
+// Scores are taken relative to a lazily moved reference that enters as the accumulator's initial value, so the common
+// tile has no cross-lane step at all.
+//
+// Merging the key ranges inside this kernel (four ranges to a work-group meeting in LDS, a ticket per work-group from a
+// per-tile counter, the last work-group adding up what the others left, partials stored and loaded past L2 with
+// device-scope accesses and no fence) was built and gives the same results, and is slower than the second launch:
+// 20.0 us against 17.3 for the 64 MiB call, 11.6 against 7.4 us for a 4 MiB one -- a device-scope store, the ticket
+// and the loads are three dependent trips across the dies at two microseconds each.
+constexpr int DEC_STAGES = 3;
+constexpr int DEC_KBLK   = 1152;           // 8 rows of K and 128 bytes
+constexpr int DEC_KTILE  = 4 * DEC_KBLK;   // 32 keys
+constexpr int DEC_VTILE  = 32 * 128;
+constexpr float DEC_SUM_LIMIT = 2048.0f;   // a lane's 8 probabilities of a tile may add up to this before the reference moves
+
+typedef __attribute__((address_space(3))) char fa_lds_char;
+
+__device__ __forceinline__ void dec_dma16(const char * base, uint32_t off, uint32_t lds) {
+    // 16 bytes per lane from global memory (uniform base + per-lane offset) straight into LDS at lds + 16 lane
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(off), "s"(base), "s"(lds) : "memory");
+}
+
+__device__ __forceinline__ half8_t dec_tr8(const fa_lds_char * p) { // keys 4j .. 4j+3 and 16 + 4j .. of one d
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3))) *) p);
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3))) *) (p + 16 * 128));
+    return __builtin_bit_cast(half8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+__global__ __launch_bounds__(64) void fattn_dec64_kernel(const fa_args a) {
+    constexpr int D = 64;
+    __shared__ __attribute__((aligned(1024))) char k_lds[DEC_STAGES + 1][DEC_KTILE]; // (the last one: a tile with keys of the second pair)
+    __shared__ __attribute__((aligned(1024))) char v_lds[DEC_STAGES + 1][DEC_VTILE];
+    const int lane = threadIdx.x;
+    const int j = lane >> 4, c = lane & 15;
+    if (a.has_kvs && blockIdx.z == 0) { // the folded cache write: see fattn_cols16_kernel
+        if (blockIdx.x != 0) return;
+        if (blockIdx.y == 0) {
+            double tk, tv;
+            if (a.kvs_k.vec && a.kvs_v.vec) kvs_wave_totals<true, true>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+            else if (a.kvs_k.vec)           kvs_wave_totals<true, false>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+            else if (a.kvs_v.vec)           kvs_wave_totals<false, true>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+            else                            kvs_wave_totals<false, false>(a.kvs_k, a.kvs_v, lane, false, tk, tv);
+            if (lane == 0) *a.kvs_out = kvs_scalar((float) tk, (float) tv, a.kvs_scale, a.kvs_bias);
+        } else {
+            const uint32_t first = (blockIdx.y - 1) * 64 + lane, step = (gridDim.y - 1) * 64;
+            double unused = 0.0;
+            const uint32_t nk = kvs_units(a.kvs_k, a.kvs_k.vec != 0), nv = kvs_units(a.kvs_v, a.kvs_v.vec != 0);
+            if (a.kvs_k.vec) { for (uint32_t e = first; e < nk; e += step) kvs_unit<true>(a.kvs_k, e, true, unused); }
+            else             { for (uint32_t e = first; e < nk; e += step) kvs_unit<false>(a.kvs_k, e, true, unused); }
+            if (a.kvs_v.vec) { for (uint32_t e = first; e < nv; e += step) kvs_unit<true>(a.kvs_v, e, true, unused); }
+            else             { for (uint32_t e = first; e < nv; e += step) kvs_unit<false>(a.kvs_v, e, true, unused); }
+        }
+        return;
+    }
+    const int ct = blockIdx.x, sp = blockIdx.y, bg = (int) blockIdx.z - (a.has_kvs ? 1 : 0);
+    const int b  = fa_div(bg, a.inv_hkv);
+    const int g  = bg - b * a.Hkv;
+    const int tile = bg * a.n_col_tiles + ct;
+    const int  ncols  = a.n_q * a.gqa;
+    const int  col    = ct * 16 + c;
+    const bool col_ok = col < ncols;
+    const int  iq1    = col_ok ? fa_div(col, a.inv_gqa) : 0;
+    const int  head   = g * a.gqa + (col_ok ? col - iq1 * a.gqa : 0);
+    const int  bk     = a.rk3 == 1 ? b : b / a.rk3;
+
+    float4_t qraw[2][2];
+    {
+        const float * qp = (const float *) (a.q + (uint64_t) iq1 * a.nbq1 + (uint64_t) head * a.nbq2 + (uint64_t) b * a.nbq3) + 16 * j;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) { qraw[p][0] = ((const float4_t *) (qp + 8 * p))[0]; qraw[p][1] = ((const float4_t *) (qp + 8 * p))[1]; }
+    }
+
+    const int kv0 = sp * a.chunk, kv1 = min(a.n_kv, kv0 + a.chunk);
+    const int ntile = (kv1 - kv0 + 31) / 32;
+    // With a second pair of tensors (the step's own keys behind the cached ones) the tiles that lie wholly in the cache
+    // stream as described; a tile with later keys is put together lane by lane -- each row from the tensor that holds
+    // it, F32 rows rounded to f16 as a CAST node would round them -- into a buffer of its own, in the layout the direct
+    // loads leave.  The first such tile is fetched before the walk begins and consumed in its turn (after the cached
+    // tiles, as the one-tensor call consumes it: the results are the same bits); further ones are fetched as they come.
+    const int ndma = a.k2 ? min(ntile, max(0, (a.n_kv1 - kv0) / 32)) : ntile;
+
+    // ---- direct loads: an instruction copies 8 rows; lane = (row lane / 8, chunk position lane % 8), the chunk it
+    //      fetches is the position un-swizzled
+    const char * kg = a.k + (uint64_t) g * a.nbk2 + (uint64_t) bk * a.nbk3;
+    const char * vg = a.v + (uint64_t) g * a.nbv2 + (uint64_t) bk * a.nbv3;
+    const uint32_t k_base = (uint32_t) (uintptr_t) (fa_lds_char *) &k_lds[0][0];
+    const uint32_t v_base = (uint32_t) (uintptr_t) (fa_lds_char *) &v_lds[0][0];
+    const int dr = lane >> 3, dp = lane & 7;
+    const uint32_t kch = (uint32_t) ((dp ^ dr) << 4), vch = (uint32_t) ((dp ^ (2 * (dr & 3))) << 4);
+    const uint32_t kof = (uint32_t) dr * (uint32_t) a.nbk1 + kch, vof = (uint32_t) dr * (uint32_t) a.nbv1 + vch;
+    // tiles are sent in order: the next tile's row pointers are kept and moved on by 8 rows per instruction
+    const uint64_t k8 = 8 * a.nbk1, v8 = 8 * a.nbv1;
+    const char * knext = kg + (uint64_t) kv0 * a.nbk1;
+    const char * vnext = vg + (uint64_t) kv0 * a.nbv1;
+    int kb_next = kv0;
+    auto issue = [&](int stage) { // the next tile of this wave's range into `stage`: always 8 loads
+        const uint32_t kl = k_base + stage * DEC_KTILE, vl = v_base + stage * DEC_VTILE;
+        if (kb_next + 32 <= a.n_kv) { // wave-uniform
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                dec_dma16(knext, kof, kl + u * DEC_KBLK);
+                dec_dma16(vnext, vof, vl + u * 1024);
+                knext += k8;
+                vnext += v8;
+            }
+        } else { // the cache's last rows: clamped (their scores are switched off)
+            const int last = a.n_kv - 1 - kb_next;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int r = min(8 * u + dr, last);
+                dec_dma16(knext, (uint32_t) r * (uint32_t) a.nbk1 + kch, kl + u * DEC_KBLK);
+                dec_dma16(vnext, (uint32_t) r * (uint32_t) a.nbv1 + vch, vl + u * 1024);
+            }
+        }
+        kb_next += 32;
+    };
+#pragma unroll
+    for (int t = 0; t < DEC_STAGES; ++t)
+        if (t < ndma) issue(t);
+    const char * kg2 = nullptr, * vg2 = nullptr;
+    if (a.k2) {
+        kg2 = a.k2 + (uint64_t) g * a.nbk2b + (uint64_t) bk * a.nbk3b;
+        vg2 = a.v2 + (uint64_t) g * a.nbv2b + (uint64_t) bk * a.nbv3b;
+    }
+    auto fill_mixed = [&](int kb) { // the 32 keys from kb on into the last buffer
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int key = min(kb + 8 * u + dr, a.n_kv - 1);
+            const int ck = dp ^ dr, cv = dp ^ (2 * (dr & 3)); // the chunks this lane's positions hold
+            half8_t kh, vh;
+            if (key < a.n_kv1) {
+                kh = *(const half8_t *) (kg + (uint64_t) key * a.nbk1 + ck * 16);
+                vh = *(const half8_t *) (vg + (uint64_t) key * a.nbv1 + cv * 16);
+            } else if (a.seg2_f32) {
+                const float4_t * kp = (const float4_t *) (kg2 + (uint64_t) (key - a.n_kv1) * a.nbk1b + ck * 32);
+                const float4_t * vp = (const float4_t *) (vg2 + (uint64_t) (key - a.n_kv1) * a.nbv1b + cv * 32);
+                const float4_t k0 = kp[0], k1 = kp[1], v0 = vp[0], v1 = vp[1];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    kh[i] = (_Float16) k0[i]; kh[4 + i] = (_Float16) k1[i];
+                    vh[i] = (_Float16) v0[i]; vh[4 + i] = (_Float16) v1[i];
+                }
+            } else {
+                kh = *(const half8_t *) (kg2 + (uint64_t) (key - a.n_kv1) * a.nbk1b + ck * 16);
+                vh = *(const half8_t *) (vg2 + (uint64_t) (key - a.n_kv1) * a.nbv1b + cv * 16);
+            }
+            *(half8_t *) &k_lds[DEC_STAGES][u * DEC_KBLK + lane * 16] = kh;
+            *(half8_t *) &v_lds[DEC_STAGES][u * 1024 + lane * 16] = vh;
+        }
+    };
+    if (ndma < ntile) fill_mixed(kv0 + 32 * ndma);
+
+    // ---- Q^T operand: column c, d = 16 j + 8 p + i, pre-scaled (a.scale carries log2 e)
+    half8_t qh[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        float4_t x0 = qraw[p][0] * a.scale, x1 = qraw[p][1] * a.scale;
+        if (!col_ok) { x0 = float4_t{0, 0, 0, 0}; x1 = float4_t{0, 0, 0, 0}; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { qh[p][i] = (_Float16) x0[i]; qh[p][4 + i] = (_Float16) x1[i]; }
+    }
+
+    // ---- operand addresses inside a stage
+    uint32_t kad[2], vad[4];
+    {
+        const int r8 = c & 7;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) kad[p] = (uint32_t) ((c >> 3) * DEC_KBLK + r8 * 128 + (((2 * j + p) ^ r8) << 4)); // + 2 DEC_KBLK for keys 16 ..
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+            vad[dt] = (uint32_t) ((4 * j + (c >> 2)) * 128 + (((2 * dt + ((c & 3) >> 1)) ^ (2 * (c >> 2))) << 4) + 8 * (c & 1));
+    }
+    const fa_lds_char * const k_lds0 = (const fa_lds_char *) &k_lds[0][0];
+    const fa_lds_char * const v_lds0 = (const fa_lds_char *) &v_lds[0][0];
+
+    float4_t o[4], negm = float4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] = float4_t{0, 0, 0, 0};
+    float l = 0.0f;
+    bool  seen = false, all_seen = false;
+
+    typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
+    auto probs = [&](const float4_t (&s)[2], int4_t & pb, float & lt) {
+        half2_t acc = half2_t{(_Float16) 0.0f, (_Float16) 0.0f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; r += 2) {
+                const fp16x2 pr = __builtin_amdgcn_cvt_pkrtz(__builtin_amdgcn_exp2f(s[h][r]), __builtin_amdgcn_exp2f(s[h][r + 1]));
+                pb[2 * h + (r >> 1)] = __builtin_bit_cast(int, pr);
+                acc += __builtin_bit_cast(half2_t, pr);
+            }
+        lt = (float) acc[0] + (float) acc[1];
+    };
+
+    for (int t = 0; t < ntile; ++t) {
+        const bool streamed = t < ndma; // wave-uniform
+        const int stage = streamed ? t % DEC_STAGES : DEC_STAGES;
+        const int kb = kv0 + 32 * t;
+        if (streamed) {
+            // this tile has landed once at most the younger tiles' loads are outstanding (8 each)
+            const int younger = min(DEC_STAGES - 1, ndma - 1 - t);
+            if (younger >= 2)      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            else if (younger == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            else                   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else if (t > ndma) {
+            fill_mixed(kb); // (the buffer's previous tile is in registers: the wait below)
+        }
+        half8_t kk[2][2], vv[4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int p = 0; p < 2; ++p) kk[h][p] = *(const __attribute__((address_space(3))) half8_t *) (k_lds0 + stage * DEC_KTILE + kad[p] + h * 2 * DEC_KBLK);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) vv[dt] = dec_tr8(v_lds0 + stage * DEC_VTILE + vad[dt]);
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the stage is in registers, the tile three ahead may overwrite it
+        if (t + DEC_STAGES < ndma) issue(stage);
+
+        float4_t s[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            s[h] = mfma16(kk[h][0], qh[0], negm);
+            s[h] = mfma16(kk[h][1], qh[1], s[h]);
+        }
+        int4_t pb;
+        float  lt;
+        probs(s, pb, lt);
+        const bool tail = kb + 32 > kv1; // wave-uniform
+        if (tail || !all_seen || __builtin_amdgcn_ballot_w64(!(lt <= DEC_SUM_LIMIT)) != 0) {
+            if (tail) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) s[h][r] = kb + 16 * h + 4 * j + r < kv1 ? s[h][r] : -INFINITY;
+            }
+            float cm = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])), fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+            cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+            cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+            // move the reference: up to the new maximum, or (first visible key of the column) onto it wherever it lies
+            const bool  vis   = cm != -INFINITY;
+            const float delta = !vis ? 0.0f : (seen ? fmaxf(cm, 0.0f) : cm);
+            seen = seen || vis;
+            const float f = __builtin_amdgcn_exp2f(-delta);
+            s[0] -= delta;
+            s[1] -= delta;
+            negm -= delta;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) o[dt] *= f;
+            l *= f;
+            probs(s, pb, lt);
+            all_seen = __builtin_amdgcn_ballot_w64(!seen) == 0;
+        }
+        l += lt;
+        const half8_t p8 = __builtin_bit_cast(half8_t, pb);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) o[dt] = mfma16(vv[dt], p8, o[dt]);
+    }
+
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const float m = seen ? -negm[0] : -INFINITY;
+
+    // lane (j, c), tile dt, register r holds d = 16 dt + 4 j + r of column c
+    if (!col_ok) return;
+    if (a.n_splits == 1) {
+        const bool  has_sink = a.sinks != nullptr, has_addend = a.add1 != nullptr;
+        const float sink = has_sink ? a.sinks[head] : 0.0f, addend = has_addend ? *a.add1 : 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) fa_finish(a, o[dt], m, l, b, iq1, head, D, 16 * dt + 4 * j, has_sink, sink, has_addend, addend);
+    } else {
+        const uint64_t pbase = ((uint64_t) tile * a.n_splits + sp) * 16 + c;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) *(float4_t *) (a.part_o + pbase * D + 16 * dt + 4 * j) = o[dt];
+        if (j == 0) { a.part_ml[pbase * 2] = m; a.part_ml[pbase * 2 + 1] = l; }
+    }
+}
+
+// whether the streaming kernel takes this launch (decided from the arguments alone); VX_FA_DEC=0 keeps every launch on
+// the general kernel
+bool fa_dec64_takes(const fa_args & a, int D, bool kv_f32) {
+    static const bool off = [] { const char * e = getenv("VX_FA_DEC"); return e && atoi(e) == 0; }();
+    if (off) return false;
+    return D == 64 && !kv_f32 && !a.mask && a.softcap == 0.0f && a.n_kv > 64 && a.nbk1 < (1u << 28) && a.nbv1 < (1u << 28);
+}
+void launch_dec64(const fa_args & a, hipStream_t st) {
+    const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv + (a.has_kvs ? 1 : 0)));
+    fattn_dec64_kernel<<<grid, dim3(64), 0, st>>>(a);
+}
+
 template <int D, bool KV_F32>
 void launch_cols16(const fa_args & a, hipStream_t st) {
     const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv + (a.has_kvs ? 1 : 0))), block(64);
@@ -919,6 +1217,9 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     const int64_t nblocks = tiles * a.n_splits;
     if (nblocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext: launch too large");
     const int D = (int) q->ne[0];
+    const bool f32 = k->type == VX_TYPE_F32;
+
+    const bool dec = fa_dec64_takes(a, D, f32);
 
     if (a.n_splits > 1) {
         const size_t o_bytes  = (size_t) nblocks * 16 * D * sizeof(float);
@@ -937,8 +1238,8 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
         a.kvs_out = a.has_kvs ? (float *) ((char *) ws + o_bytes + ml_bytes - 16) : nullptr;
     }
 
-    const bool f32 = k->type == VX_TYPE_F32;
-    if (D == 64) { if (f32) launch_cols16<64, true>(a, st); else launch_cols16<64, false>(a, st); }
+    if (dec) launch_dec64(a, st);
+    else if (D == 64) { if (f32) launch_cols16<64, true>(a, st); else launch_cols16<64, false>(a, st); }
     else         { if (f32) launch_cols16<128, true>(a, st); else launch_cols16<128, false>(a, st); }
     VX_LAUNCH_CHECK();
     if (a.n_splits > 1) {
