@@ -229,7 +229,9 @@ def cpu_baseline(batch, length, core_share):
         runs[threads] = {"GB/s": nbytes / st["mean"] / 1e9, "us": {n: st[n] * 1e6 for n in ("mean", "median", "p90", "best")}, "repeats": st["repeats"]}
     assert ref.rh_use_device(b"CPU", min(8, core_share), 0) == 0
     top = runs[core_share]
+    eight = runs[min(8, core_share)]
     return {"value": top["GB/s"], "unit": "GB/s", "cores": core_share, "kind": "reference", "cpu": cpu_model(),
+            "value_8_threads": eight["GB/s"], "us_8_threads": eight["us"]["mean"], "us": top["us"]["mean"],
             "host_logical_cpus": os.cpu_count(),
             "sample": f"{top['repeats']} repeats of one layer's ggml_flash_attn_ext on ggml-cpu (batch {batch}, KV {length}, f16 K/V, "
                       f"{nbytes >> 20} MiB of K/V): mean {top['us']['mean']:.0f} us, median {top['us']['median']:.0f}, p90 {top['us']['p90']:.0f}; "
@@ -333,9 +335,23 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         plug.ggml_backend_gfx950_set_graph_replay(1)   # the same graph again and again (what a fixed-length step would be): recorded, then replayed
         reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=plugin_reps + 3)   # three runs until the replay is in place
         st_r = stats(reflib.ref_last_times()[3:])
+        # what "decode steps/s" means for a drop-in: consecutive steps, a graph built per position as the reference builds it
+        # (src/voxcpm.cpp:485-513), laid out, its inputs uploaded, computed, the hidden state fetched -- wall clock of the loop
+        plug.ggml_backend_gfx950_set_graph_replay(1)
+        n_loop = min(256, steps)
+        _, lp = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop)
+        _, lpo = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop, overlap=True)
         ref.rh_bb_free()
+        consecutive = {"decode_steps_per_s": 1.0 / lp["wall"], "ms_per_step": lp["wall"] * 1e3, "graph_compute_ms": lp["graph_compute"] * 1e3,
+                       "graph_build_and_layout_ms": lp["build"] * 1e3, "steps": n_loop, "from_kv_length": prefill,
+                       "nodes_at_another_address_than_the_step_before": lp["moved"],
+                       "how": "the drop-in figure: every step's graph rebuilt for its position, ggml_backend_graph_compute (synchronous), "
+                              "wall clock over the loop including graph construction, layout, uploads and the fetch of the hidden state",
+                       "next_graph_built_under_the_running_one": {"decode_steps_per_s": 1.0 / lpo["wall"], "ms_per_step": lpo["wall"] * 1e3,
+                           "how": "the same loop with graph_compute_async: the host builds the next position's graph while the device computes"}}
         res["plugin_graph_compute"] = {"decode_steps_per_s": 1.0 / st["mean"], "ms_per_step": {n: st[n] * 1e3 for n in ("mean", "median", "p90", "best")},
                                        "graph_nodes": n_nodes, "launches": launches, "kv_length": mid,
+                                       "consecutive_steps": consecutive,
                                        "how": "ggml_backend_graph_compute on libggml-gfx950.so, eager, synchronised per call",
                                        "same_graph_replayed": {"decode_steps_per_s": 1.0 / st_r["mean"], "ms_per_step": {n: st_r[n] * 1e3 for n in ("mean", "median", "p90", "best")},
                                                                "how": "the identical graph computed repeatedly: the plugin records it at its third run and replays one HIP graph"}}
@@ -349,12 +365,19 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
             tp0 = time.perf_counter()
             reflib.ref_backbone_forward(xph, 0, reflib.causal_mask(prefill, prefill))
             cpu_pf = time.perf_counter() - tp0
+        if not cpu_prefill:   # no prefill (it would take minutes): the cache gets seeded values instead, one array for every layer
+            kvt = np.float16 if kv_f16 else np.float32
+            fill = np.random.default_rng(5).standard_normal(batch * HKV * max_len * D, dtype=np.float32).astype(kvt)
+            for li in range(layers):
+                for which in (0, 1):
+                    assert ref.rh_bb_cache_set(li, which, fill.ctypes.data, fill.nbytes) == 0
+            del fill
         _, (mean, best), n_nodes = reflib.ref_backbone_forward(x1.cpu().numpy(), mid, None, reps=cpu_reps)
         st = stats(reflib.ref_last_times())
         ref.rh_bb_free()
         res["ggml_cpu"] = {"decode_steps_per_s": 1.0 / mean, "ms_per_step": mean * 1e3, "median_ms": st["median"] * 1e3, "p90_ms": st["p90"] * 1e3,
                            "best_ms": best * 1e3, "threads": threads, "graph_nodes": n_nodes, "prefill_ms": cpu_pf * 1e3 if cpu_pf else None,
-                           "sample": f"{cpu_reps} repeats of the decode step at KV length {mid}" + (", one prefill" if cpu_prefill else ", cache contents as left by allocation, no prefill (it would take minutes)")}
+                           "sample": f"{cpu_reps} repeats of the decode step at KV length {mid}" + (", one prefill" if cpu_prefill else ", the cache filled with seeded N(0,1) values, no prefill (it would take minutes)")}
         res["speedup_vs_ggml_cpu"] = mean / t_step
     return res
 
@@ -636,7 +659,7 @@ def main():
     achieved = kv_bytes(B, L) / launch_sec / 1e9
     traffic, traffic_commit = measured_traffic(B, L)
     peaks = peaks_bench(timer)
-    roofline = {"bound": "hbm", "kernel": "fattn_cols16_kernel<64, f16 K/V> + fattn_merge_kernel<64>", "achieved": achieved,
+    roofline = {"bound": "hbm", "kernel": "fattn_dec64_kernel + fattn_merge_kernel<64>", "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "traffic_source": (f"profiles/decode_attn_B{B}_L{L}_hbm_counters.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain copy, taken at commit {traffic_commit})"
                                    if traffic else None),
@@ -674,9 +697,16 @@ def main():
                               ("q8_0_proj_1024x1024_n1024", 1024, 1024, 1024), ("q8_0_ffn_up_4096x1024_n1024", 4096, 1024, 1024),
                               ("q8_0_proj_1024x1024_n16384", 1024, 1024, 16384), ("q8_0_ffn_up_4096x1024_n16384", 4096, 1024, 16384)):
             call, keep = q8_proj_setup(pkg, M, K, N)
-            s = timer.run(call, iters=200 if N <= 1024 else 20, warmup=5)
+            if N <= 16:   # a few microseconds a call: 64 calls replayed from one HIP graph, so that the kernel is timed and not Python
+                def many(call=call):
+                    for _ in range(64):
+                        call()
+                s = timer.run(graphed(many, side), iters=50, warmup=5) / 64
+            else:
+                s = timer.run(call, iters=200 if N <= 1024 else 20, warmup=5)
             wbytes = M * K // 32 * 34
-            others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12}
+            others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12,
+                            "launch": "64 calls per HIP graph replay (the same weights: they stay in cache)" if N <= 16 else "eager"}
             del keep, call
         torch.cuda.empty_cache()
 
@@ -731,6 +761,8 @@ def main():
             "backbone_decode_steps_per_s_cfg4_f16kv": pick("cfg4_backbone_24layers_b2_f16kv", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_through_plugin": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_through_plugin_same_graph_replayed": pick("cfg4_backbone_24layers_b2", "plugin_graph_compute", "same_graph_replayed", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg4_f16kv_through_plugin_consecutive_steps": pick("cfg4_backbone_24layers_b2_f16kv", "plugin_graph_compute", "consecutive_steps", "decode_steps_per_s"),
+            "backbone_decode_steps_per_s_cfg5_f16kv_through_plugin_consecutive_steps": pick("cfg5_backbone_24layers_b16_f16kv", "plugin_graph_compute", "consecutive_steps", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg4_ggml_cpu": pick("cfg4_backbone_24layers_b2", "ggml_cpu", "decode_steps_per_s"),
             "backbone_decode_steps_per_s_cfg5_f16kv": pick("cfg5_backbone_24layers_b16_f16kv", "decode_steps_per_s"),
             "backbone_prefill_tokens_per_s_cfg4": pick("cfg4_backbone_24layers_b2", "prefill_tokens_per_s"),

@@ -578,6 +578,93 @@ int rh_bb_forward(const float * x, const uint16_t * mask, int n_tokens, int n_pa
     return rc;
 }
 
+// A run of consecutive decode steps as the reference drives them (src/voxcpm.cpp:485-513, 1027-1128): every step gets
+// a fresh context and a graph built for its own position (n_past is baked into the views of the cache), the graph
+// is laid out by the one graph allocator the run keeps, the step's input and position are uploaded, the graph is
+// computed and the hidden state fetched.  x: [hidden, 1, batch], the same input every step.  seconds[0] = wall
+// time per step over the whole loop, [1] = the graph_compute calls' share per step (with overlap: compute and the
+// next graph's construction together), [2] = nodes of the last graph, [3] = graph construction + layout per step,
+// [4] = the share of nodes whose address differs from the previous step's.  The cache is written: steps n_past0 ..
+// n_past0 + steps - 1.
+int rh_bb_decode_loop(const float * x, int n_past0, int steps, int overlap, float * out, double * seconds) {
+    if (!g_bb || !g_backend || steps < 1) return 100;
+    const backbone & m = *g_bb;
+    const int B = m.batch;
+    if (n_past0 + steps > m.max_len) return 104;
+    const size_t n_nodes = (size_t) m.n_layer * 64 + 64;
+    // overlap = 1: the next step's graph is built and laid out while the device works on the current one (its shape
+    // depends on the position only, not on the step's result): two contexts and two graph allocators take turns, the
+    // graph is enqueued with ggml_backend_graph_compute_async and the host synchronises when it needs the hidden state
+    ggml_gallocr_t ga[2] = { ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend)),
+                             overlap ? ggml_gallocr_new(ggml_backend_get_default_buffer_type(g_backend)) : nullptr };
+    int rc = 0, last_nodes = 0;
+    long long moved = 0, compared = 0;
+    double t_compute = 0.0, t_build = 0.0;
+    std::vector<float> hidden((size_t) m.hidden * B);
+    std::vector<const void *> prev_addr;
+    struct built { ggml_context * c = nullptr; ggml_cgraph * gf = nullptr; ggml_tensor * inp = nullptr, * pos = nullptr, * h = nullptr; };
+    auto build = [&](int n_past, ggml_gallocr_t alloc) {
+        const auto tb0 = std::chrono::steady_clock::now();
+        built b;
+        ggml_init_params ip = { ggml_tensor_overhead() * n_nodes + ggml_graph_overhead_custom(n_nodes, false), nullptr, true };
+        b.c = ggml_init(ip);
+        b.inp = ggml_new_tensor_2d(b.c, GGML_TYPE_F32, m.hidden, (int64_t) B);
+        b.pos = ggml_new_tensor_1d(b.c, GGML_TYPE_I32, 1);
+        ggml_set_input(b.inp); ggml_set_input(b.pos);
+        ggml_tensor * h = b.inp;
+        std::vector<ggml_tensor *> roots;
+        for (const auto & L : m.layers) h = bb_layer_forward(b.c, m, L, h, b.pos, nullptr, 1, n_past, true, roots);
+        h = bb_norm(b.c, m, h, m.final_norm);
+        ggml_set_output(h);
+        b.h = h;
+        b.gf = ggml_new_graph_custom(b.c, n_nodes, false);
+        ggml_build_forward_expand(b.gf, h);
+        for (ggml_tensor * r : roots) ggml_build_forward_expand(b.gf, r);
+        if (!ggml_gallocr_alloc_graph(alloc, b.gf)) rc = 101;
+        t_build += std::chrono::duration<double>(std::chrono::steady_clock::now() - tb0).count();
+        return b;
+    };
+    const auto t_loop = std::chrono::steady_clock::now();
+    built cur = build(n_past0, ga[0]);
+    for (int s = 0; s < steps && !rc; ++s) {
+        const int n_past = n_past0 + s;
+        ggml_backend_tensor_set(cur.inp, x, 0, ggml_nbytes(cur.inp));
+        const int32_t p = n_past;
+        ggml_backend_tensor_set(cur.pos, &p, 0, sizeof p);
+        last_nodes = ggml_graph_n_nodes(cur.gf);
+        if (!overlap) { // how many nodes lie at another address than in the step before (the graph is otherwise the same)
+            if ((int) prev_addr.size() == last_nodes)
+                for (int i = 0; i < last_nodes; ++i) { ++compared; if (prev_addr[(size_t) i] != ggml_graph_node(cur.gf, i)->data) ++moved; }
+            prev_addr.resize((size_t) last_nodes);
+            for (int i = 0; i < last_nodes; ++i) prev_addr[(size_t) i] = ggml_graph_node(cur.gf, i)->data;
+        }
+        const auto t0 = std::chrono::steady_clock::now();
+        built next;
+        if (overlap) {
+            if (ggml_backend_graph_compute_async(g_backend, cur.gf) != GGML_STATUS_SUCCESS) rc = 102;
+            if (!rc && s + 1 < steps) next = build(n_past + 1, ga[(s + 1) & 1]);
+            ggml_backend_synchronize(g_backend);
+        } else {
+            if (ggml_backend_graph_compute(g_backend, cur.gf) != GGML_STATUS_SUCCESS) rc = 102;
+        }
+        t_compute += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (!rc) ggml_backend_tensor_get(cur.h, hidden.data(), 0, ggml_nbytes(cur.h));
+        ggml_free(cur.c);
+        cur = built{};
+        if (!rc && s + 1 < steps) cur = overlap ? next : build(n_past + 1, ga[0]);
+    }
+    if (cur.c) ggml_free(cur.c);
+    const double t_all = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_loop).count();
+    if (seconds) {
+        seconds[0] = t_all / steps; seconds[1] = t_compute / steps; seconds[2] = (double) last_nodes; seconds[3] = t_build / steps;
+        seconds[4] = compared ? (double) moved / (double) compared : 0.0;
+    }
+    if (!rc && out) memcpy(out, hidden.data(), hidden.size() * sizeof(float));
+    ggml_gallocr_free(ga[0]);
+    if (ga[1]) ggml_gallocr_free(ga[1]);
+    return rc;
+}
+
 // ---- two dependent stages, with and without a trip through the host -----------------------------------------
 // The reference's decode step runs the base LM's step graph, fetches its hidden state to the host, adds the step's
 // embedding there and uploads the sum as the input of the residual LM's step graph (src/voxcpm.cpp:1067-1093): two

@@ -196,6 +196,7 @@ def load_ref():
     lib.rh_cfm_free.restype = None
     lib.rh_bb_fuse_weights.argtypes = []
     lib.rh_bb_forward.argtypes = [f32p, u16p, C.c_int, C.c_int, C.c_int, f32p, C.c_int, f64p]
+    lib.rh_bb_decode_loop.argtypes = [f32p, C.c_int, C.c_int, C.c_int, f32p, f64p]
     assert lib.rh_use_device(b"CPU", min(8, os.cpu_count() or 1), 0) == 0
     _ref = lib
     return lib
@@ -405,6 +406,21 @@ def ref_backbone_forward(x, n_past, mask=None, write_kv=True, reps=0):
                            ptr(out, C.c_float), reps, ptr(sec, C.c_double))
     assert rc == 0, rc
     return out, sec[:2].copy(), int(sec[2])
+
+
+def ref_backbone_decode_loop(x, n_past0, steps, overlap=False):
+    """`steps` consecutive decode steps from cache length n_past0, each with a graph built for its own position as the
+    reference builds them (src/voxcpm.cpp:485-513).  x: (batch, 1, hidden) f32, the same input every step.  Returns the
+    last step's hidden state and a dict of per-step seconds (wall over the loop, graph_compute's share, graph
+    construction + layout), the node count and the share of nodes that moved between steps.  overlap: the next step's
+    graph is built while the device computes the current one."""
+    lib = load_ref()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    sec = np.zeros(5, np.float64)
+    rc = lib.rh_bb_decode_loop(ptr(x, C.c_float), n_past0, steps, int(overlap), ptr(out, C.c_float), ptr(sec, C.c_double))
+    assert rc == 0, rc
+    return out, {"wall": float(sec[0]), "graph_compute": float(sec[1]), "build": float(sec[3]), "n_nodes": int(sec[2]), "moved": float(sec[4])}
 
 
 def cfm_params(tag, feat=64, hidden=1024):

@@ -453,6 +453,71 @@ def test_plugin_runs_a_whole_cfm_solve_graph(gpu, ref, time_table):
     assert x.cpu().numpy().tobytes() == plug.tobytes()
 
 
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
+    """A run of decode steps as the reference drives them (src/voxcpm.cpp:485-513, 1027-1128): a graph built for every
+    position, laid out by one graph allocator, computed, the hidden state fetched.  72 consecutive steps behind a
+    prefill of 300 tokens (so the key ranges are cut and merged, and the cut changes along the way) through the plugin:
+    against ggml-cpu on the same loop, against the same steps computed one by one through rh_bb_forward (the same
+    launches: bit for bit, the caches included), and with the next step's graph built while the device computes the
+    current one (the same launches again)."""
+    import ctypes
+    T0, N = 300, 72
+    max_len = T0 + N + 8
+    params = reflib.backbone_params("bb", N_LAYER)
+    xp = rng("bbl", "x", 0).standard_normal((BATCH, T0, 1024)).astype(np.float32)
+    x1 = rng("bbl", "x", 1).standard_normal((BATCH, 1, 1024)).astype(np.float32)
+    cache_bytes = 64 * max_len * 2 * BATCH * (2 if kv_f16 else 4)
+
+    def caches():
+        out = []
+        for layer in range(N_LAYER):
+            for which in (0, 1):
+                buf = np.empty(cache_bytes, np.uint8)
+                assert ref.rh_bb_cache_get(layer, which, buf.ctypes.data, buf.nbytes) == 0
+                out.append(buf)
+        return out
+
+    def run(device, how):
+        assert ref.rh_use_device(device, 8, 0) == 0
+        reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=kv_f16)
+        try:
+            reflib.ref_backbone_forward(xp, 0, reflib.causal_mask(T0, T0))
+            if how == "one by one":
+                for s in range(N):
+                    out = reflib.ref_backbone_forward(x1, T0 + s, None)[0]
+                info = None
+            else:
+                out, info = reflib.ref_backbone_decode_loop(x1, T0, N, overlap=(how == "overlapped"))
+            return out, caches(), info
+        finally:
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    cpu, cpu_cache, _ = run(b"CPU", "loop")
+    loop, loop_cache, info = run(b"GFX950_0", "loop")
+    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    print(f"consecutive decode steps, kv_f16={kv_f16}: {N} steps, {info['n_nodes']} nodes and {launches} launches a step, "
+          f"{info['moved'] * 100:.0f} % of the nodes at another address than the step before", flush=True)
+    assert launches == 5 * N_LAYER + 1
+    e = nmse(cpu, loop)
+    print(f"   last hidden state, plugin vs ggml-cpu: nmse {e:.3e}", flush=True)
+    assert e <= 1e-4
+    for a, b in zip(cpu_cache, loop_cache):  # what the steps appended (f16 or F32 values of O(1))
+        w = np.float16 if kv_f16 else np.float32
+        af, bf = a.view(w).astype(np.float32), b.view(w).astype(np.float32)
+        assert nmse(af, bf) <= 2e-4 and np.abs(af - bf).max() <= 5e-2
+    single, single_cache, _ = run(b"GFX950_0", "one by one")
+    assert np.array_equal(loop, single), "the loop's last step differs from the step computed on its own"
+    for a, b in zip(loop_cache, single_cache):
+        assert np.array_equal(a, b), "cache contents differ"
+    over, over_cache, _ = run(b"GFX950_0", "overlapped")
+    assert np.array_equal(loop, over), "building the next graph under the running one changed a result"
+    for a, b in zip(loop_cache, over_cache):
+        assert np.array_equal(a, b), "cache contents differ (overlapped)"
+
+
 def test_plugin_replays_a_recurring_graph(gpu, ref):
     """A graph the plugin has run twice is recorded on its third run and replayed from then on (a CFM solve has the same
     shapes and addresses on every call; the reference rebuilds and relaunches it each time, src/voxcpm.cpp:485-495).
@@ -498,6 +563,47 @@ def test_plugin_replays_a_recurring_graph(gpu, ref):
     cpu = solve_all(b"CPU", False, 0)
     for i, (a, b) in enumerate(zip(cpu, replayed)):
         assert nmse(a, b) <= 1e-3, i
+
+
+def test_plugin_replay_keys_on_the_activation_mode(gpu, ref):
+    """A recording holds the launches of the activation mode it was made under (ggml_backend_gfx950_set_mul_mat_act): the
+    same graph at the same addresses after a switch of the mode is another graph.  Four solves with float activations
+    (recorded at the third, replayed at the fourth), the switch to Q8 activations, four more: they must give what Q8
+    launches give without any replay, and not what the float recording holds."""
+    import ctypes
+    params = reflib.backbone_params("locdit", 4)
+    cp = reflib.cfm_params("cfm")
+    mu = rng("cfmr", "mu").standard_normal(1024).astype(np.float32)
+    cond = rng("cfmr", "cond").standard_normal((4, 64)).astype(np.float32)
+    table = rng("cfmr", "table").standard_normal((10, 1024)).astype(np.float32)
+    z = rng("cfmr", "z", 0).standard_normal((2, 64)).astype(np.float32)
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    assert ref.rh_use_device(b"GFX950_0", 8, 0) == 0
+    replay_before = plugin.ggml_backend_gfx950_set_graph_replay(1)
+    act_before = plugin.ggml_backend_gfx950_set_mul_mat_act(0)
+    ref.rh_out_after_reps(1)
+    try:
+        reflib.ref_backbone_create(params, 32, 1, use_mup=True, kv_f16=False, fused_weights=True)
+        reflib.ref_cfm_create(cp)
+        n0 = plugin.ggml_backend_gfx950_replays()
+        out_float = reflib.ref_cfm_solve(z, mu, cond, table, reps=4)[0]
+        n1 = plugin.ggml_backend_gfx950_replays()
+        assert n1 > n0, "the float-mode graph was never replayed: the test would prove nothing"
+        plugin.ggml_backend_gfx950_set_mul_mat_act(1)
+        out_q8 = reflib.ref_cfm_solve(z, mu, cond, table, reps=4)[0]
+        plugin.ggml_backend_gfx950_set_graph_replay(0)
+        out_q8_plain = reflib.ref_cfm_solve(z, mu, cond, table, reps=1)[0]
+    finally:
+        ref.rh_out_after_reps(0)
+        plugin.ggml_backend_gfx950_set_mul_mat_act(act_before)
+        plugin.ggml_backend_gfx950_set_graph_replay(replay_before)
+        ref.rh_cfm_free()
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+    print(f"activation mode and replay: float vs q8 max-abs {np.abs(out_float - out_q8).max():.3e}", flush=True)
+    assert np.array_equal(out_q8, out_q8_plain), "a recording made under another activation mode was replayed"
+    assert not np.array_equal(out_float, out_q8)
 
 
 @pytest.mark.gpu

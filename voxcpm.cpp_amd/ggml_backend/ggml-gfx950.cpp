@@ -30,6 +30,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdlib>
+#include <chrono>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -114,9 +115,6 @@ struct backend_ctx {
     vx_stream stream;
     std::vector<seen_graph> seen;   // a handful of entries, least recently used one replaced
     uint64_t  clock = 0;
-    // what graph_optimize worked out for a graph object, for the graph_compute that follows on the same object
-    const ggml_cgraph * opt_graph = nullptr;
-    uint64_t  opt_cheap = 0, opt_fingerprint = 0;
     int       replays = 0;          // diagnostic: graph_compute calls served by a replay
 };
 
@@ -1271,7 +1269,9 @@ inline uint64_t mix64(uint64_t h, uint64_t v) {
 // cheap: node count, and per node the operator, the output address and the two outer extents (what changes from one
 // decode step to the next: the key count) -- a few hundred nanoseconds per thousand nodes
 uint64_t graph_cheap_signature(const ggml_cgraph * g) {
-    uint64_t h = (uint64_t) g->n_nodes;
+    // (the activation mode of the Q8_0 products is part of what a recording holds: a graph recorded under one mode is
+    // another graph under the other)
+    uint64_t h = (uint64_t) g->n_nodes ^ ((uint64_t) mul_mat_act_mode() << 40);
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
         h = mix64(h, (uint64_t) (uintptr_t) n->data ^ ((uint64_t) n->op << 56) ^ ((uint64_t) n->ne[1] << 20) ^ ((uint64_t) n->ne[2] << 40));
@@ -1298,7 +1298,7 @@ void fingerprint_tensor(fingerprint_state & f, const ggml_tensor * t) {
 }
 uint64_t graph_fingerprint(const ggml_cgraph * g) {
     fingerprint_state f;
-    f.add((uint64_t) g->n_nodes);
+    f.add((uint64_t) g->n_nodes ^ ((uint64_t) mul_mat_act_mode() << 40));
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
         fingerprint_tensor(f, n);
@@ -1314,17 +1314,14 @@ uint64_t graph_fingerprint(const ggml_cgraph * g) {
 }
 
 ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out);
+long long g_host_ns[2] = { 0, 0 }; // the most recent node-by-node graph_compute: host time of the analysis, and of issuing the launches
 
 // graph_optimize (ggml/src/ggml-backend-impl.h:118-119): ggml_backend_sched calls it once per split when it lays a graph
-// out.  Nothing is reordered; the graph's signatures are worked out here, once, so that the graph_compute calls on the
-// same graph object need not hash it again.
+// out, before the tensors have addresses.  Nothing is reordered here, and nothing is remembered: a signature taken now
+// could be matched to a graph object that was edited, or rebuilt at the same address, before it is computed.
 void backend_graph_optimize(ggml_backend_t backend, ggml_cgraph * cgraph) {
-    backend_ctx * ctx = (backend_ctx *) backend->context;
-    ctx->opt_graph = nullptr;
-    if (!cgraph || cgraph->n_nodes < 8) return;
-    ctx->opt_cheap       = graph_cheap_signature(cgraph);
-    ctx->opt_fingerprint = graph_fingerprint(cgraph);
-    ctx->opt_graph       = cgraph;
+    (void) backend;
+    (void) cgraph;
 }
 
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
@@ -1342,7 +1339,6 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         return st;
     }
     const uint64_t cheap = graph_cheap_signature(cgraph);
-    const bool from_opt = ctx->opt_graph == cgraph && ctx->opt_cheap == cheap;
     seen_graph * entry = nullptr;
     for (seen_graph & g : ctx->seen) if (g.cheap == cheap) { entry = &g; break; }
     ++ctx->clock;
@@ -1364,7 +1360,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         return st;
     }
     entry->last_use = ctx->clock;
-    const uint64_t fp = from_opt ? ctx->opt_fingerprint : graph_fingerprint(cgraph);
+    const uint64_t fp = graph_fingerprint(cgraph);
     if (entry->fingerprint != fp) { // second sight (or a different graph with the same quick signature): start counting
         if (entry->recorded) vx_graph_destroy(entry->recorded);
         entry->recorded = nullptr;
@@ -1407,6 +1403,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
 
 ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out) {
     int launches = 0;
+    const auto t_begin = std::chrono::steady_clock::now();
     // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
     // nodes is only run as one launch when nothing else looks at the value between them
     static const bool fusion = getenv("GGML_GFX950_NO_FUSION") == nullptr;
@@ -1445,6 +1442,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
     std::unordered_map<const ggml_tensor *, concat_tree> cat_by_root;
     static const bool concat_trees = getenv("GGML_GFX950_NO_CONCAT_TREES") == nullptr;
     if (fusion && concat_trees && cgraph->n_nodes > 2) find_concat_trees(cgraph, readers, cat_by_root, kv2_absorbed); // (inner nodes are skipped like absorbed CONCATs)
+    const auto t_analysed = std::chrono::steady_clock::now();
     for (int i = 0; i < cgraph->n_nodes; ++i) {
         ggml_tensor * node = cgraph->nodes[i];
         // the same two skips ggml-cpu applies (ggml/src/ggml-cpu/ggml-cpu.c:2956-2966)
@@ -1578,6 +1576,9 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
         }
     }
     *launches_out = launches;
+    const auto t_end = std::chrono::steady_clock::now();
+    g_host_ns[0] = std::chrono::duration_cast<std::chrono::nanoseconds>(t_analysed - t_begin).count();
+    g_host_ns[1] = std::chrono::duration_cast<std::chrono::nanoseconds>(t_end - t_analysed).count();
     return GGML_STATUS_SUCCESS;
 }
 
@@ -1746,6 +1747,8 @@ GGML_BACKEND_API int                ggml_backend_score(void) { return vx_device_
 // Diagnostic: how many operator calls the most recent graph_compute of this process issued (an attention
 // call counts once although it may launch a split and a merge kernel).
 extern "C" int ggml_backend_gfx950_last_launches(void) { return g_last_launches; }
+// Diagnostic: host nanoseconds the most recent node-by-node graph_compute spent (0) analysing the graph, (1) issuing launches
+extern "C" long long ggml_backend_gfx950_host_ns(int which) { return which == 0 || which == 1 ? g_host_ns[which] : 0; }
 // how many graph_compute calls of this process were served by replaying a recorded graph
 extern "C" int ggml_backend_gfx950_replays(void) { return g_replays; }
 // switches the recognition of recurring graphs on (1) or off (0); returns the previous setting
