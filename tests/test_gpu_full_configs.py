@@ -206,3 +206,51 @@ def test_fa_cfg5_prefill_b16_t4096(gpu):
         worst = max(worst, err)
         assert err <= 2e-3, (b, r, err)
     say(f"   {len(pairs)} sampled rows against the oracle: worst max-abs {worst:.3e}")
+
+
+def test_backbone_cfg5_prefill_b16_t4096(gpu, ref):
+    """Config 5's prefill at its full size through the plugin: 16 sequences x 4096 tokens (65536 tokens a product, the
+    causal attention of test_fa_cfg5_prefill_b16_t4096 inside), f16 KV cache, two layers of the stack and the final norm.
+    Against ggml-cpu on the whole output and on the cache that the call wrote, and grouped launches against every node
+    as its own launch."""
+    N_LAYER, BATCH, T = 2, 16, 4096
+    say(f"cfg 5 prefill through the plugin: {N_LAYER} layers, {BATCH} x {T} tokens, f16 KV cache")
+    params = reflib.backbone_params("bb5p", N_LAYER)
+    x = rng("bb5p", "x").standard_normal((BATCH, T, 1024)).astype(np.float32)
+    mask = reflib.causal_mask(T, T)
+
+    def run(device, threads):
+        assert ref.rh_use_device(device, threads, 0) == 0
+        reflib.ref_backbone_create(params, T, BATCH, use_mup=True, kv_f16=True)
+        try:
+            out = reflib.ref_backbone_forward(x, 0, mask)[0]
+            cache = np.empty((BATCH, 2, T, 64), np.float16)
+            assert ref.rh_bb_cache_get(N_LAYER - 1, 1, cache.ctypes.data, cache.nbytes) == 0
+        finally:
+            ref.rh_bb_free()
+            assert ref.rh_use_device(b"CPU", 8, 0) == 0
+        return out, cache
+
+    say("   ggml-cpu ...")
+    cpu, cpu_cache = run(b"CPU", 16)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+    say("   plugin ...")
+    plug, plug_cache = run(b"GFX950_0", 8)
+    launches = plugin.ggml_backend_gfx950_last_launches()
+    e, ec = nmse(cpu, plug), nmse(cpu_cache.astype(np.float32), plug_cache.astype(np.float32))
+    say(f"   plugin ({launches} launches) vs ggml-cpu: hidden states nmse {e:.3e}, last layer's V cache nmse {ec:.3e}")
+    assert np.isfinite(plug).all() and e <= 1e-4 and ec <= 1e-4
+    rows = np.abs(cpu - plug).reshape(BATCH * T, -1).max(axis=1) / np.abs(cpu).max()
+    say(f"   worst token: {rows.max():.3e} of the largest value (token {int(rows.argmax()) % T} of sequence {int(rows.argmax()) // T})")
+    assert rows.max() <= 5e-2
+    before = plugin.ggml_backend_gfx950_set_fusion(0)
+    try:
+        plain, plain_cache = run(b"GFX950_0", 8)
+    finally:
+        plugin.ggml_backend_gfx950_set_fusion(before)
+    plain_launches = plugin.ggml_backend_gfx950_last_launches()
+    same = np.array_equal(plain, plug) and np.array_equal(plain_cache, plug_cache)
+    say(f"   every node its own launch ({plain_launches} launches): bit-equal to the grouped run: {same}; nmse {nmse(plain, plug):.3e}")
+    assert plain_launches > launches
+    assert same, "grouped launches changed a result"

@@ -441,6 +441,9 @@ def mm_inputs(tag, M, K, N, batch=()):
                                    (2000, 1024, 1700), (1000, 1024, 333), (64, 1024, 4100), (130, 2048, 9000),
                                    # a long K on a small grid: K cut across work-groups, partials added by a second kernel
                                    (1024, 4096, 600), (1000, 2176, 300),
+                                   # 64 to 256 tiles of 64 x 64 with 68 and 34 rounds of K: quarters and halves of 17 rounds, an odd
+                                   # number for the two-round loop of the LDS-operand kernel
+                                   (1024, 4352, 1000), (1000, 2176, 600),
                                    # the same on the LDS-operand kernel when its 64 x 64 tiles are few (the down-projection of
                                    # 8 requests' 112 tokens): 8, 8 and 4 splits, ragged rows and tokens
                                    (1024, 4096, 112), (1000, 4096, 70), (512, 2048, 64)])
@@ -459,6 +462,36 @@ def test_mul_mat_q8_0(gpu, M, K, N):
     assert e_q8 <= 1e-5
     assert nmse(cpu, got_fl) <= 5e-4
     assert nmse(f64, got_fl) <= 1e-5
+
+
+def test_mul_mat_q8_0_full_size_prefill(gpu):
+    """The gate/up product of a full-size prefill: 4096 rows, K = 1024, 16 sequences x 1024 tokens (the shape the Q8_0 GEMM
+    is measured on).  Every token's row of the result depends on that token alone, so the oracle is run on a sample of 96
+    tokens (the first and last tiles, and random ones) with test_mul_mat_q8_0's bars; the whole result is compared with
+    ggml-cpu where its build is there."""
+    M, K, N = 4096, 1024, 16384
+    say(f"mul_mat Q8_0 M={M} K={K} N={N}")
+    w, x = mm_inputs(("q8-full", M, K, N), M, K, N)
+    wq = reflib.quantize_q8_0(w)
+    wd, xd = dev(wq), dev(x)
+    got_q8 = sync_np(gpu.mul_mat(wd, xd, gpu.ACT_Q8, w_ne0=K))
+    got_fl = sync_np(gpu.mul_mat(wd, xd, gpu.ACT_FLOAT, w_ne0=K))
+    pick = np.unique(np.concatenate([np.arange(32), np.arange(N - 32, N), rng("q8-full", "pick").integers(0, N, 32)]))
+    xs = np.ascontiguousarray(x[pick])
+    cpu = reflib.oracle_mul_mat(wq, xs, K, act_mode=0)
+    f64 = reflib.oracle_mul_mat(wq, xs, K, f64=True)
+    e_q8 = np.abs(got_q8[pick] - cpu).max() / np.abs(cpu).max()
+    say(f"   {len(pick)} sampled tokens: ACT_Q8 vs ggml-cpu arithmetic rel max {e_q8:.3e};  ACT_FLOAT nmse vs cpu "
+        f"{nmse(cpu, got_fl[pick]):.3e}, vs fp64 dequant {nmse(f64, got_fl[pick]):.3e}")
+    assert e_q8 <= 1e-5
+    assert nmse(cpu, got_fl[pick]) <= 5e-4
+    assert nmse(f64, got_fl[pick]) <= 1e-5
+    if reflib.load_ref() is not None:
+        r = reflib.ref_mul_mat(wq, x, K)
+        e = np.abs(got_q8 - r).max() / np.abs(r).max()
+        say(f"   all {N} tokens vs ggml-cpu (reference build): ACT_Q8 rel max {e:.3e}, ACT_FLOAT nmse {nmse(r, got_fl):.3e}")
+        assert e <= 1e-5
+        assert nmse(r, got_fl) <= 5e-4
 
 
 @pytest.mark.parametrize("seed", list(range(48)))

@@ -31,7 +31,6 @@ def make(B, Hq, Hkv, D, L, n_q, tag, kv_dtype=np.float16):
 
 def test_static_scratch_matches_the_allocating_call(gpu, oracle):
     import torch
-    free0 = torch.cuda.mem_get_info()[0]
     cases = [  # (B, Hq, Hkv, D, L, n_q): the second call is smaller than the first in every respect
         (16, 16, 2, 64, 8192, 1),
         (2, 16, 2, 64, 700, 1),
@@ -58,7 +57,6 @@ def test_static_scratch_matches_the_allocating_call(gpu, oracle):
                                    reflib.desc(want), 0.125, 0.0, 0.0, 1, 1)
     assert rc == 0
     assert np.abs(got - want).max() <= 2e-3
-    del free0
 
 
 def test_static_scratch_with_mask_and_f32_cache(gpu):
@@ -80,12 +78,29 @@ def test_static_scratch_with_mask_and_f32_cache(gpu):
 
 
 def test_static_scratch_refuses_what_does_not_fit(gpu):
-    """A shape whose partials exceed the fixed array is refused before anything is launched."""
+    """A shape whose partials exceed the fixed array is refused before anything is launched.
+
+    The largest partials come from the largest number of sixteen-column tiles that is still cut into key ranges: one
+    less than the library's four waves per compute unit, cut in two.  The shape is therefore derived from the device's
+    compute-unit count (1023 tiles on 256 units: 2046 partial blocks of 8 KiB and their maxima and sums, more than the
+    16 MiB array).  The VX_FA_* variables move those thresholds and are read once per process: with any of them set the
+    test has no shape to offer."""
+    import ctypes as C
+    import os
     import torch
-    say("no-alloc attention: oversized request")
+    moved = [n for n in ("VX_FA_WAVES_PER_CU", "VX_FA_MAX_SPLITS", "VX_FA_MIN_CHUNK") if os.environ.get(n)]
+    if moved:
+        pytest.skip(f"{moved} change how many key ranges a call is cut into")
     lib = gpu.lib()
-    # 1023 sixteen-column tiles of head_dim 128 with a cache that is cut in two: 2046 partial blocks of 8 KiB
-    B, Hkv, D, L = 341, 3, 128, 512
+    cus = C.c_int(0)
+    assert lib.vx_device_info(0, None, 0, None, None, C.byref(cus)) == 0
+    D, L = 128, 512
+    tiles = 4 * cus.value - 1
+    need = 2 * tiles * 16 * (D + 2) * 4
+    say(f"no-alloc attention: oversized request ({tiles} tiles in two key ranges on {cus.value} compute units: {need} bytes)")
+    if need <= 16 * 1024 * 1024:
+        pytest.skip(f"no decode shape of head size {D} exceeds the fixed array on a device with {cus.value} compute units")
+    B, Hkv = tiles, 1
     q = torch.zeros((B, Hkv, 1, D), device="cuda")
     k = torch.zeros((B, Hkv, L, D), dtype=torch.float16, device="cuda")
     out = torch.full((B, 1, Hkv, D), 7.0, device="cuda")

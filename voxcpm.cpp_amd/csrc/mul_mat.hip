@@ -65,6 +65,7 @@ struct mm_args {
     // [batch][split][token][row] for a second kernel to add in split order (ksplit <= 1: off)
     int ksplit;
     float * partial;
+    size_t ws_offset; // bytes at the start of the stream's workspace that the caller keeps for itself: partials go behind them
     // GEMV with RMS_NORM and the norm-weight MUL applied to the activations as they are staged
     // (x is then the un-normalised tensor): x[t][k] / rms(x[t]) * norm_w[k], rounded after each product
     const float * norm_w;
@@ -1558,8 +1559,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(RT
     if (ty >= gy || tx >= gx) return;
     const int64_t tok0 = (int64_t) ty * TOKS;
     const int64_t rowg = (int64_t) tx * ROWS;
-    // the launcher takes whole rounds only, and an even number of them per split (a round's register set and LDS buffer
-    // are its parity)
+    // the launcher takes whole rounds only; a split may hold an odd number of them (a round's register set and LDS buffer
+    // are the parity of its index within the split, and the loop below guards the second round of each pair)
     const int64_t rounds_all = a.K / (32 * GL_KC), rbeg = rounds_all / nsplit * split, nround = rbeg + rounds_all / nsplit;
 
     // Loads never leave the operands: rows past M and tokens past N are clamped to the last one (their
@@ -1833,6 +1834,13 @@ int gemm_lds_cut(int64_t M, int64_t N, int64_t K, int64_t nbatch) {
     return ks;
 }
 
+// A cut product whose workspace request fails (a growing request on a stream under capture, or no memory) must not
+// quietly become another kernel's product with another summation order: the launcher records the status here, every
+// launcher after it stands back, and the entry point returns the status (thread-local: launches come from any thread).
+thread_local vx_status t_ws_status = VX_OK;
+bool ws_failed() { return t_ws_status != VX_OK; }
+vx_status take_ws_status() { const vx_status rc = t_ws_status; t_ws_status = VX_OK; return rc; }
+
 template <int WT>
 bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     const int mode = gemm_lds_mode();
@@ -1853,9 +1861,9 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     if (ks >= 2 && cut_fits) {
         // the K range is cut across ks work-groups per tile; a second kernel adds their partials in split order
         void * ws = nullptr;
-        if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) != VX_OK) { (void) hipGetLastError(); return false; }
+        if ((t_ws_status = vx_workspace(st, a.ws_offset + (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
         mm_args b = a;
-        b.ksplit = ks; b.partial = (float *) ws;
+        b.ksplit = ks; b.partial = (float *) ((char *) ws + a.ws_offset);
         const bool ok = WT == WT_Q8 && mode == 2 ? launch_gemm_lds_tile<WT, WT == WT_Q8, 2, 2, 2, 2>(b, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(b, nbatch, st);
         if (!ok) return false;
         const int64_t units = a.N * (a.M / 4);
@@ -1895,9 +1903,9 @@ bool launch_mm_cut(const mm_args & a, int nbatch, hipStream_t st) {
     if (ks > 8) ks = 8;
     if (ks < 2 || (int64_t) nbatch * ks > 65535) return false;
     void * ws = nullptr;
-    if (vx_workspace(st, (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws) != VX_OK) { (void) hipGetLastError(); return false; }
+    if ((t_ws_status = vx_workspace(st, a.ws_offset + (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
     mm_args b = a;
-    b.ksplit = ks; b.partial = (float *) ws;
+    b.ksplit = ks; b.partial = (float *) ((char *) ws + a.ws_offset);
     mm_kernel<WT, 4, ACT_Q8, false><<<dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st>>>(b);
     const int64_t units = a.N * (a.M / 4);
     mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
@@ -1907,7 +1915,7 @@ bool launch_mm_cut(const mm_args & a, int nbatch, hipStream_t st) {
 template <int WT, bool ACT_Q8>
 void launch(const mm_args & a, int nbatch, hipStream_t st) {
     if constexpr (WT != WT_F32) { if (launch_gemv<WT, ACT_Q8>(a, nbatch, st)) return; }
-    if constexpr (WT != WT_F32 && !ACT_Q8) { if (launch_gemm_lds<WT>(a, nbatch, st)) return; }
+    if constexpr (WT != WT_F32 && !ACT_Q8) { if (launch_gemm_lds<WT>(a, nbatch, st) || ws_failed()) return; }
     if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
@@ -1916,7 +1924,7 @@ void launch(const mm_args & a, int nbatch, hipStream_t st) {
         const dim3 grid((unsigned) ((a.M + 63) / 64), 1, (unsigned) nbatch);
         mm_kernel<WT, 2, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
     } else {
-        if (launch_mm_cut<WT, ACT_Q8>(a, nbatch, st)) return;
+        if (launch_mm_cut<WT, ACT_Q8>(a, nbatch, st) || ws_failed()) return;
         const int64_t gx = (a.M + 63) / 64, gy = (a.N + 63) / 64;
         const dim3 grid((unsigned) gx, (unsigned) gy, (unsigned) nbatch);
         mm_kernel<WT, 4, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
@@ -1980,6 +1988,7 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
         case VX_TYPE_F16: launch<WT_F16, false>(a, nbatch, st); break;
         default:          launch<WT_F32, false>(a, nbatch, st); break;
     }
+    if (ws_failed()) return take_ws_status();
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -2145,10 +2154,11 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     if (!ok) { // not the streaming kernel's shape: the tiled kernels with K cut (see vx_supports_mul_mat_scale_add)
         if (src0->type == VX_TYPE_Q8_0) {
             if (act_mode == VX_ACT_Q8) ok = launch_mm_cut<WT_Q8, true>(a, nbatch, st);
-            else                       ok = launch_gemm_lds<WT_Q8>(a, nbatch, st) || launch_mm_cut<WT_Q8, false>(a, nbatch, st);
+            else                       ok = launch_gemm_lds<WT_Q8>(a, nbatch, st) || (!ws_failed() && launch_mm_cut<WT_Q8, false>(a, nbatch, st));
         } else {
-            ok = launch_gemm_lds<WT_F16>(a, nbatch, st) || launch_mm_cut<WT_F16, false>(a, nbatch, st);
+            ok = launch_gemm_lds<WT_F16>(a, nbatch, st) || (!ws_failed() && launch_mm_cut<WT_F16, false>(a, nbatch, st));
         }
+        if (ws_failed()) return take_ws_status();
     }
     if (!ok) { // the plain product, then the update in a pass of its own (dense dst: checked by vx_supports_mul_mat_scale_add)
         const size_t bytes = (size_t) nbatch * a.N * a.M * sizeof(float);
@@ -2162,9 +2172,13 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
         }
         mm_args p = a;
         p.res = nullptr; p.dst = (char *) product;
+        // (a cut of this product puts its partials behind the product when that lies in the workspace; if the request
+        // grows the workspace, the block with the product stays valid: retired blocks live as long as the stream)
+        if (product != dst->data) p.ws_offset = (bytes + 255) & ~(size_t) 255;
         p.nb1 = (uint64_t) a.M * 4; p.nb2 = p.nb1 * (uint64_t) a.N; p.nb3 = p.nb2 * (uint64_t) a.ne12;
         if (src0->type == VX_TYPE_Q8_0) { if (act_mode == VX_ACT_Q8) launch<WT_Q8, true>(p, nbatch, st); else launch<WT_Q8, false>(p, nbatch, st); }
         else                            launch<WT_F16, false>(p, nbatch, st);
+        if (ws_failed()) return take_ws_status();
         mm_args b = a;
         b.ksplit = 1; b.partial = (float *) product;
         const int64_t units = a.N * (a.M / 4);

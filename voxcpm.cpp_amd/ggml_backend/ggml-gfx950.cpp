@@ -1259,6 +1259,11 @@ bool compute_fused_gate_up_group(backend_ctx * ctx, const ggml_cgraph * g, int i
 
 int g_last_launches = 0; // operator launches of the most recent graph_compute (diagnostic)
 int g_replays = 0;       // graph_compute calls of this process that were served by replaying recorded launches
+int g_fusion_on = -1;    // run groups of nodes as one launch (GGML_GFX950_NO_FUSION switches it off, ggml_backend_gfx950_set_fusion either way)
+bool fusion_on() {
+    if (g_fusion_on < 0) g_fusion_on = getenv("GGML_GFX950_NO_FUSION") == nullptr;
+    return g_fusion_on != 0;
+}
 int g_replay_on = -1;    // recognise recurring graphs and replay them (GGML_GFX950_GRAPH_REPLAY, ggml_backend_gfx950_set_graph_replay)
 
 // ---- recognising a graph ---------------------------------------------------------------------------------------------
@@ -1271,7 +1276,7 @@ inline uint64_t mix64(uint64_t h, uint64_t v) {
 uint64_t graph_cheap_signature(const ggml_cgraph * g) {
     // (the activation mode of the Q8_0 products is part of what a recording holds: a graph recorded under one mode is
     // another graph under the other)
-    uint64_t h = (uint64_t) g->n_nodes ^ ((uint64_t) mul_mat_act_mode() << 40);
+    uint64_t h = (uint64_t) g->n_nodes ^ (((uint64_t) mul_mat_act_mode() << 40) ^ ((uint64_t) fusion_on() << 42));
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
         h = mix64(h, (uint64_t) (uintptr_t) n->data ^ ((uint64_t) n->op << 56) ^ ((uint64_t) n->ne[1] << 20) ^ ((uint64_t) n->ne[2] << 40));
@@ -1298,7 +1303,7 @@ void fingerprint_tensor(fingerprint_state & f, const ggml_tensor * t) {
 }
 uint64_t graph_fingerprint(const ggml_cgraph * g) {
     fingerprint_state f;
-    f.add((uint64_t) g->n_nodes ^ ((uint64_t) mul_mat_act_mode() << 40));
+    f.add((uint64_t) g->n_nodes ^ (((uint64_t) mul_mat_act_mode() << 40) ^ ((uint64_t) fusion_on() << 42)));
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
         fingerprint_tensor(f, n);
@@ -1406,7 +1411,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
     const auto t_begin = std::chrono::steady_clock::now();
     // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
     // nodes is only run as one launch when nothing else looks at the value between them
-    static const bool fusion = getenv("GGML_GFX950_NO_FUSION") == nullptr;
+    const bool fusion = fusion_on();
     reader_map readers;
     if (fusion && cgraph->n_nodes > 1) {
         readers.reserve((size_t) cgraph->n_nodes * 2);
@@ -1722,6 +1727,7 @@ void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
     if (strcmp(name, "ggml_backend_gfx950_replays") == 0) return (void *) ggml_backend_gfx950_replays;
     if (strcmp(name, "ggml_backend_gfx950_set_graph_replay") == 0) return (void *) ggml_backend_gfx950_set_graph_replay;
     if (strcmp(name, "ggml_backend_gfx950_set_mul_mat_act") == 0) return (void *) ggml_backend_gfx950_set_mul_mat_act;
+    if (strcmp(name, "ggml_backend_gfx950_set_fusion") == 0) return (void *) ggml_backend_gfx950_set_fusion;
     return nullptr;
 }
 
@@ -1756,6 +1762,14 @@ extern "C" int ggml_backend_gfx950_set_graph_replay(int on) {
     if (g_replay_on < 0) { const char * e = getenv("GGML_GFX950_GRAPH_REPLAY"); g_replay_on = !(e && atoi(e) == 0); }
     const int before = g_replay_on;
     g_replay_on = on != 0;
+    return before;
+}
+
+// switches the grouping of nodes into single launches on (1) or off (0: every node its own launch) for later graph_compute
+// calls; returns the previous setting.  Results do not depend on it.
+extern "C" int ggml_backend_gfx950_set_fusion(int on) {
+    const int before = fusion_on();
+    g_fusion_on = on != 0;
     return before;
 }
 

@@ -40,6 +40,8 @@ GGML_BACKEND_API int ggml_backend_gfx950_last_launches(void);
 GGML_BACKEND_API int ggml_backend_gfx950_set_graph_replay(int on);  /* recognise recurring graphs and replay them; returns the previous setting */
 GGML_BACKEND_API int ggml_backend_gfx950_replays(void);   /* graph_compute calls served by replaying recorded launches */
 GGML_BACKEND_API int ggml_backend_gfx950_set_mul_mat_act(int mode);
+GGML_BACKEND_API int ggml_backend_gfx950_set_fusion(int on);        /* groups of nodes as one launch (default) or every node its own; returns the previous setting */
+GGML_BACKEND_API long long ggml_backend_gfx950_host_ns(int which);  /* the last node-by-node graph_compute: host ns spent (0) analysing the graph, (1) issuing launches */
 
 #ifdef __cplusplus
 }
