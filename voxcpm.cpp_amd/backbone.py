@@ -23,6 +23,8 @@ to the unfused sequence.
 """
 import math
 
+import numpy as np
+
 from . import (ACT_FLOAT, BIN_ADD, BIN_MUL, F16, F32, GLU_SWIGLU, _p, _stream, check, desc, desc_q8, lib)
 
 WEIGHT_NAMES = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
@@ -37,7 +39,9 @@ class MiniCPMBackbone:
         self.n_layer, self.hidden, self.n_heads, self.n_kv, self.D = n_layer, hidden, n_heads, n_kv_heads, head_dim
         self.ffn, self.max_length, self.batch, self.eps = ffn, max_length, batch, eps
         self.use_mup = use_mup
-        self.residual_scale = scale_depth / math.sqrt(max(1, n_layer)) if use_mup else 1.0
+        # in single precision, as MiniCPMModel computes it (src/minicpm.cpp:276): the double-precision quotient rounds to
+        # the neighbouring float for some layer counts (6, 24), and every residual update would differ in its last bit
+        self.residual_scale = float(np.float32(scale_depth) / np.sqrt(np.float32(max(1, n_layer)))) if use_mup else 1.0
         self.act_mode = act_mode
         self.fuse_pairs = fuse_pairs
         self.rope_base, self.rope_original_max = rope_base, rope_original_max
