@@ -38,9 +38,9 @@ HQ, HKV, D, LAYERS = 16, 2, 64, 24
 
 def measured_traffic(batch, length):
     """HBM bytes per vx_flash_attn_ext call from the counter profile on file for this shape (rocprofv3 FETCH_SIZE /
-    WRITE_SIZE scaled by a plain copy; profiles/decode_attn_*_hbm_counters.txt carries a line
+    WRITE_SIZE scaled by a plain copy; profiles/decode_attn_*_kernel_trace_and_counters.txt carries a line
     `traffic_bytes_per_call: N` and the commit it was taken at), or None."""
-    path = os.path.join(ROOT, "profiles", f"decode_attn_B{batch}_L{length}_hbm_counters.txt")
+    path = os.path.join(ROOT, "profiles", f"decode_attn_B{batch}_L{length}_kernel_trace_and_counters.txt")
     try:
         text = open(path).read()
     except OSError:
@@ -534,6 +534,7 @@ def load_peaks():
     lib.vxp_mfma_f16.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.vxp_mfma_f16_flop.argtypes = [C.c_int, C.c_int]
     lib.vxp_mfma_f16_flop.restype = C.c_double
+    lib.vxp_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     return lib
 
 
@@ -558,10 +559,150 @@ def peaks_bench(timer):
     fsink = torch.zeros(4096 * 256, dtype=torch.float32, device="cuda")
     blocks, iters = 2048, 4096
     s_mfma = timer.run(lambda: lib.vxp_mfma_f16(blocks, iters, fsink.data_ptr(), st()), iters=5, warmup=2)
-    return {"hbm_stream_read_1GiB_GB/s": big.numel() / s_big / 1e9,
+    # a barrier across a resident grid: 1000 rounds a launch, the counter cleared by a fill kernel before each
+    flags = torch.zeros(2, dtype=torch.int32, device="cuda")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    barrier = {}
+    for per_cu in (1, 2):
+        for ordered in (0, 1):
+            rounds = 1000
+
+            def one():
+                flags.zero_()
+                rc = lib.vxp_grid_barrier(per_cu * cus, rounds, ordered, flags.data_ptr(), flags.data_ptr() + 4, st())
+                assert rc == 0, rc
+
+            empty = timer.run(lambda: flags.zero_(), iters=10, warmup=2)
+            s_bar = timer.run(one, iters=5, warmup=2)
+            assert int(flags[1].item()) == 0, "a work-group gave up waiting at the grid barrier"
+            barrier[f"{per_cu * cus}_work_groups_{'release_acquire' if ordered else 'relaxed'}_us"] = (s_bar - empty) / rounds * 1e6
+    return {"grid_barrier": barrier,
+            "hbm_stream_read_1GiB_GB/s": big.numel() / s_big / 1e9,
             "hbm_stream_read_64MiB_per_launch_GB/s": chunk / s_chunk / 1e9, "hbm_stream_read_64MiB_us": s_chunk * 1e6,
             "mfma_f16_TFLOP/s": lib.vxp_mfma_f16_flop(blocks, iters) / s_mfma / 1e12,
             "how": "libvx_peaks.so: 16-byte nontemporal loads, 8 in flight per lane, 8 blocks per CU; 8 independent v_mfma_f32_32x32x16_f16 per wave in a loop"}
+
+
+# ---- profiles/: the rocprofv3 runs behind the committed summaries, and the summariser --------------------------------
+SQ_SET_1 = "SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_WAVES"
+SQ_SET_2 = "SQ_INSTS_SALU SQ_INSTS_LDS SQ_WAIT_ANY SQ_ACTIVE_INST_ANY SQ_INST_CYCLES_VMEM SQ_ACTIVE_INST_VALU SQ_LDS_BANK_CONFLICT GRBM_GUI_ACTIVE"
+TCC_SET = "TCC_HIT_sum TCC_MISS_sum TCC_EA0_RDREQ_sum TCC_REQ_sum"
+TCP_SET = "TCP_PENDING_STALL_CYCLES_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_sum TCP_TCP_TA_DATA_STALL_CYCLES_sum"
+# file stem, bench.py --profile name, title, counter passes (tag, counters), kernels whose counters are listed
+PROFILE_RUNS = [
+    ("decode_attn_B16_L8192", "decode5", "Decode attention, batch 16, 8192 keys, 2 KV heads x 8 query heads, head_dim 64, f16 K/V",
+     [("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE"), ("sq1", SQ_SET_1), ("sq2", SQ_SET_2), ("tcc", TCC_SET), ("tcp", TCP_SET)], "fattn"),
+    ("decode_attn_B2_L4096", "decode2", "Decode attention, batch 2, 4096 keys, 2 KV heads x 8 query heads, head_dim 64, f16 K/V",
+     [("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")], "fattn"),
+    ("prefill_attn_cfg5_T4096_B16", "prefill", "Prefill attention, 16 sequences x 4096 tokens, 16 query / 2 KV heads, head_dim 64 (BASELINE config 5)",
+     [("sq1", SQ_SET_1), ("sq2", SQ_SET_2)], "pf_"),
+    ("prefill_attn_cfg5_T4096_B1", "prefill1", "Prefill attention, one sequence of 4096 tokens, 16 query / 2 KV heads, head_dim 64",
+     [("sq1", SQ_SET_1), ("sq2", SQ_SET_2)], "pf_"),
+    ("mul_mat_q8_0_4096x1024x16384", "gemm", "Q8_0 MUL_MAT, 4096 rows x K 1024 x 16384 tokens (the gate/up projection of 16 x 1024 prefill tokens)",
+     [("sq1", SQ_SET_1), ("sq2", SQ_SET_2), ("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")], "gemm|mm_"),
+    ("backbone_decode_cfg4", "backbone", "Backbone decode step, 24 layers, batch 2, Q8_0 weights, f16 KV cache at ~520 keys (BASELINE config 4)", [], ""),
+    ("backbone_decode_cfg5", "backbone16", "Backbone stack at BASELINE config 5 (batch 16, f16 KV 4096 -> 8192, prefill 16 x 4096)", [], ""),
+    ("cfm_solve_cfg3", "cfm", "One UnifiedCFM solve of one request (10 Euler steps, CFG pair as one 14-token sequence, 4 LocDiT layers; BASELINE config 3)", [], ""),
+    ("cfm_solve_cfg3_8_requests", "cfm8", "UnifiedCFM solves of 8 concurrent requests as one ggml graph through the plugin (BASELINE config 3 at its batch)", [], ""),
+]
+
+
+def profile_commands(raw):
+    """The rocprofv3 runs of PROFILE_RUNS, one per line as 'name<TAB>command' (each is its own process; run them from
+    /tmp with TMPDIR=/tmp, every line under a time limit of its own).  Outputs go under `raw`."""
+    here = os.path.abspath(__file__)
+    out = []
+    for stem, prof, _, passes, _ in PROFILE_RUNS:
+        out.append((f"kt_{prof}", f"rocprofv3 --kernel-trace --stats --output-format csv -d {raw}/kt_{prof} -o kt -- python3 {here} --profile {prof}"))
+        for tag, counters in passes:
+            out.append((f"pmc_{prof}_{tag}", f"rocprofv3 --pmc {counters} --output-format csv -d {raw}/pmc_{prof}_{tag} -o pm -- python3 {here} --profile {prof}"))
+    for tag, counter in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
+        out.append((f"cal_{tag}", f"rocprofv3 --pmc {counter} --output-format csv -d {raw}/cal_{tag} -o pm -- python3 {here} --calibrate-copy"))
+    return out
+
+
+def summarize_profiles(raw, out, commit):
+    """Writes profiles/*.txt from the raw rocprofv3 output of profile_commands(): per kernel the calls and average
+    duration, per counter pass the mean / min / max over dispatches, and for FETCH_SIZE / WRITE_SIZE the traffic scaled
+    by what the same counter reads on a copy of known size."""
+    import collections
+    import csv
+    import glob
+
+    def kstats(d):
+        rows = []
+        for f in glob.glob(d + "/**/*kernel_stats.csv", recursive=True):
+            for r in csv.DictReader(open(f)):
+                rows.append((r["Name"], int(r["Calls"]), float(r["AverageNs"]), float(r["TotalDurationNs"]), float(r["Percentage"])))
+        return sorted(rows, key=lambda r: -r[3])
+
+    def counters(d):
+        acc = collections.defaultdict(list)
+        for f in glob.glob(d + "/**/*counter_collection.csv", recursive=True):
+            for r in csv.DictReader(open(f)):
+                acc[(r["Kernel_Name"], r["Counter_Name"])].append(float(r["Counter_Value"]))
+        return acc
+
+    def short(n, w=100):
+        return n.replace("(anonymous namespace)::", "").replace("void ", "")[:w]
+
+    def ours(n):
+        return "at::native" not in n and "rocclr" not in n and "elementwise_kernel" not in n
+
+    def bench_line(name):
+        try:
+            lines = [ln for ln in open(f"{raw}/{name}.log").read().split("\n") if ln.startswith("{")]
+            return lines[-1][:2500]
+        except OSError as e:
+            return f"(no log: {e})"
+
+    cal = {}
+    for tag in ("fetch", "write"):
+        vals = max((v for (k, c), v in counters(f"{raw}/cal_{tag}").items() if "elementwise" in k), key=len, default=None)
+        if vals and len(vals) > 1:
+            mean = sum(vals[1:]) / len(vals[1:])
+            cal[tag] = (mean, 262144.0 / mean)
+    os.makedirs(out, exist_ok=True)
+    import re
+    for stem, prof, title, passes, kernels in PROFILE_RUNS:
+        ks = kstats(f"{raw}/kt_{prof}")
+        if not ks:
+            print(f"summarize: no kernel trace for {prof}, {stem} left alone", file=sys.stderr)
+            continue
+        cmds = dict(profile_commands("<out>"))
+        here = os.path.abspath(__file__)
+        with open(f"{out}/{stem}_kernel_trace{'_and_counters' if passes else ''}.txt", "w") as f:
+            f.write(f"{title}\ncommit: {commit}\nOne MI355X (gfx950), rocprofv3 run from /tmp with TMPDIR=/tmp; every run is its own process.\nCommands:\n")
+            for name in [f"kt_{prof}"] + [f"pmc_{prof}_{t}" for t, _ in passes] + (["cal_fetch", "cal_write"] if any(t in ("fetch", "write") for t, _ in passes) else []):
+                f.write("  " + cmds[name].replace(here, "bench.py") + "\n")
+            f.write(f"\nbench.py's own line of the kernel-trace run:\n  {bench_line('kt_' + prof)}\n\n")
+            f.write(f"  {'kernel':100s} {'calls':>7s} {'avg us':>9s} {'total ms':>9s} {'%':>6s}\n")
+            for n, c, a, t, p in [r for r in ks if ours(r[0])][:16]:
+                f.write(f"  {short(n):100s} {c:7d} {a / 1e3:9.2f} {t / 1e6:9.3f} {p:6.2f}\n")
+            scaled = {}
+            for tag, _ in passes:
+                acc = counters(f"{raw}/pmc_{prof}_{tag}")
+                note = " (SQ cycle counters count in units of four cycles)" if tag.startswith("sq") else " (KiB)" if tag in cal else ""
+                f.write(f"\nCounters per dispatch, pass '{tag}'{note}:\n")
+                for (k, c), v in sorted(acc.items()):
+                    if ours(k) and re.search(kernels, k):
+                        f.write(f"  {short(k, 72):72s} {c:34s} n={len(v):5d} mean {sum(v) / len(v):15.1f} min {min(v):15.1f} max {max(v):15.1f}\n")
+                        if tag in cal:
+                            scaled[(tag, short(k, 72))] = sum(v) / len(v) * cal[tag][1]
+            if scaled:
+                f.write("\nCalibration (torch elementwise copy kernel, 262144 KiB read and 262144 KiB written per launch, first launch excluded):\n")
+                for tag in ("fetch", "write"):
+                    if tag in cal:
+                        f.write(f"  {tag.upper()}_SIZE mean {cal[tag][0]:.1f} KiB -> factor {cal[tag][1]:.3f}\n")
+                f.write("Scaled HBM traffic per dispatch (KiB):\n")
+                for (tag, k), v in sorted(scaled.items()):
+                    f.write(f"  {tag:6s} {k:72s} {v:12.0f}\n")
+                f.write(f"traffic_bytes_per_call: {int(sum(scaled.values()) * 1024)}   (every kernel above, reads plus writes)\n")
+    peaks_log = f"{raw}/peaks.log"
+    if os.path.exists(peaks_log):
+        with open(f"{out}/peaks_measured.txt", "w") as f:
+            f.write(f"What the box delivers on the simplest kernels (libvx_peaks.so)\ncommit: {commit}\nCommand:\n  python3 bench.py --profile peaks\n\n")
+            f.write(open(peaks_log).read().strip().split("\n")[-1] + "\n")
 
 
 def main():
@@ -575,9 +716,18 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 256 MiB -> 256 MiB elementwise copy kernel a few times (the known-size "
                          "launch that hardware byte counters are scaled by) and exit")
+    ap.add_argument("--profile-commands", metavar="RAW", default=None, help="print the rocprofv3 runs behind profiles/ (name, tab, command), outputs under RAW")
+    ap.add_argument("--summarize", nargs=3, metavar=("RAW", "OUT", "COMMIT"), default=None, help="write profiles/*.txt from the raw output of those runs")
     ap.add_argument("--profile", choices=["decode5", "decode2", "prefill", "prefill1", "backbone", "backbone16", "cfm", "cfm8", "gemm", "peaks"], default=None,
                     help="run only this workload a few times (for rocprofv3) and print its figures")
     args = ap.parse_args()
+    if args.profile_commands:
+        for name, cmd in profile_commands(args.profile_commands):
+            print(f"{name}\t{cmd}")
+        return
+    if args.summarize:
+        summarize_profiles(*args.summarize)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no cross-GPU step); run with --gpus 1")
 
@@ -661,7 +811,7 @@ def main():
     peaks = peaks_bench(timer)
     roofline = {"bound": "hbm", "kernel": "fattn_dec64_kernel + fattn_merge_kernel<64>", "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                "traffic_source": (f"profiles/decode_attn_B{B}_L{L}_hbm_counters.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain copy, taken at commit {traffic_commit})"
+                "traffic_source": (f"profiles/decode_attn_B{B}_L{L}_kernel_trace_and_counters.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain copy, taken at commit {traffic_commit})"
                                    if traffic else None),
                 "achievable_peak": peaks["hbm_stream_read_64MiB_per_launch_GB/s"],
                 "frac_of_achievable": achieved / peaks["hbm_stream_read_64MiB_per_launch_GB/s"],

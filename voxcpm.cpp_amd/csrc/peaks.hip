@@ -1,7 +1,8 @@
-// peaks.hip -- what this GPU actually delivers, measured with the two simplest kernels there are: a streaming
-// read of a large buffer (HBM) and a loop of independent matrix-core instructions (MFMA).  The benchmark
-// reports its rooflines against the published peaks AND against these; nothing in the product path uses
-// this file.  Built as its own small library (libvx_peaks.so).
+// peaks.hip -- what this GPU actually delivers, measured with the simplest kernels there are: a streaming
+// read of a large buffer (HBM), a loop of independent matrix-core instructions (MFMA), and a barrier across
+// all work-groups of a resident grid (what a kernel that stays on the chip for a whole layer would pay where
+// launches now follow each other).  The benchmark reports its rooflines against the published peaks AND
+// against these; nothing in the product path uses this file.  Built as its own small library (libvx_peaks.so).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -56,6 +57,34 @@ __global__ __launch_bounds__(256) void mfma_f16_kernel(int iters, float * __rest
     if (s == 123.456f) sink[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
+// `rounds` barriers over the whole grid, nothing else: lane 0 of every work-group adds 1 to a counter in device memory
+// and polls it (sleeping between polls) until all work-groups of the round have arrived; the other lanes wait at the
+// work-group barrier.  ORDERED = false: relaxed device-scope accesses, the bare cost of the round trip through L2.
+// ORDERED = true: the arrival is a release and the last poll an acquire, as a barrier must be when the work-groups
+// exchange data through memory (L2 write-back of what the work-group wrote, invalidation of what it cached).
+// A work-group gives up after spin_limit polls in all, raises *failed and leaves, so the grid drains whatever happens;
+// the launcher only accepts grids that are resident all at once.
+template <bool ORDERED>
+__global__ __launch_bounds__(256) void grid_barrier_kernel(unsigned * __restrict__ counter, int rounds, unsigned spin_limit, int * __restrict__ failed) {
+    __shared__ int gave_up;
+    if (threadIdx.x == 0) gave_up = 0;
+    unsigned spins = 0; // polls of the whole kernel, not of a round: a grid that cannot meet is gone after spin_limit polls in all
+    for (int r = 0; r < rounds; ++r) {
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const unsigned target = (unsigned) (r + 1) * gridDim.x;
+            __hip_atomic_fetch_add(counter, 1u, ORDERED ? __ATOMIC_RELEASE : __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+                __builtin_amdgcn_s_sleep(1);
+                if (++spins > spin_limit) { *failed = 1; gave_up = 1; break; }
+            }
+            if (ORDERED) __atomic_thread_fence(__ATOMIC_ACQUIRE); // (device scope for global memory)
+        }
+        __syncthreads();
+        if (gave_up) return;
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -81,6 +110,20 @@ __attribute__((visibility("default"))) int vxp_mfma_f16(int blocks, int iters, f
 }
 __attribute__((visibility("default"))) double vxp_mfma_f16_flop(int blocks, int iters) {
     return (double) blocks * 4.0 * (double) iters * 8.0 * 32768.0;
+}
+
+
+// `rounds` grid-wide barriers of `blocks` work-groups of 256 lanes (at most 4 per compute unit, so that all are resident);
+// *counter must be 0 at the start, *failed is raised if a work-group ever gave up waiting (2^22 polls)
+__attribute__((visibility("default"))) int vxp_grid_barrier(int blocks, int rounds, int ordered, unsigned * counter, int * failed, void * stream) {
+    if (!counter || !failed || blocks <= 0 || rounds <= 0) return 1;
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 2;
+    if (blocks > 4 * p.multiProcessorCount) return 1;
+    if (ordered) grid_barrier_kernel<true><<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>(counter, rounds, 1u << 22, failed);
+    else         grid_barrier_kernel<false><<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>(counter, rounds, 1u << 22, failed);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
 } // extern "C"
