@@ -494,6 +494,56 @@ def test_mul_mat_q8_0_full_size_prefill(gpu):
         assert nmse(r, got_fl) <= 5e-4
 
 
+@pytest.mark.parametrize("M,K,N,batch", [(4096, 1024, 4096, 1), (1024, 4096, 2048, 1), (2000, 1056, 1700, 1), (1030, 1024, 1100, 1),
+                                         (1024, 1024, 1024, 3), (1024, 2176, 1500, 2)])
+def test_mul_mat_q8_0_pretiled_equals_the_lds_kernel(gpu, M, K, N, batch, monkeypatch):
+    """Products of 1024 rows and tokens or more take the kernel whose operands two passes lay out beforehand (weights as
+    exact f16 integers with their scales apart, activations rounded to f16); VX_GEMM_Q8T=0 keeps them on the kernel that
+    converts inside every tile.  Both form a block's partial product with the same matrix instruction and scale and add
+    it in fp32 in the same order: the plain product, the fused residual update and the fused gate/up SwiGLU must be the
+    same bits -- full and ragged tiles in both dimensions, K with an odd number of blocks, a batch of sequences."""
+    import torch
+    L, d = gpu.lib(), gpu.desc
+    say(f"pre-tiled Q8_0 product vs the LDS kernel M={M} K={K} N={N} batch={batch}")
+    w = (rng("q8t", "w", M, K).standard_normal((M, K)) * 0.02).astype(np.float32)
+    w2 = (rng("q8t", "w2", M, K).standard_normal((M, K)) * 0.02).astype(np.float32)
+    x = rng("q8t", "x", N, K).standard_normal((batch, N, K) if batch > 1 else (N, K)).astype(np.float32)
+    wq, wq2, xd = dev(reflib.quantize_q8_0(w)), dev(reflib.quantize_q8_0(w2)), dev(x)
+
+    def both(fn):
+        monkeypatch.delenv("VX_GEMM_Q8T", raising=False)
+        a = fn()
+        monkeypatch.setenv("VX_GEMM_Q8T", "0")
+        b = fn()
+        monkeypatch.delenv("VX_GEMM_Q8T", raising=False)
+        torch.cuda.synchronize()
+        return a, b
+
+    a, b = both(lambda: gpu.mul_mat(wq, xd, gpu.ACT_FLOAT, w_ne0=K))
+    assert torch.equal(a, b), float((a - b).abs().max())
+    cpu = reflib.oracle_mul_mat(reflib.quantize_q8_0(w), x[..., :64, :] if batch == 1 else x[0, :64], K, f64=True)
+    got = a[:64] if batch == 1 else a[0, :64]
+    assert nmse(cpu, got.cpu().numpy()) <= 1e-5
+    res = dev(rng("q8t", "res", M, N).standard_normal(tuple(a.shape)).astype(np.float32))
+
+    def scale_add():
+        out = torch.empty_like(a)
+        gpu.check(L.vx_mul_mat_scale_add(gpu.desc_q8(wq, K), d(xd), d(res), d(out), 0.2857738, gpu.ACT_FLOAT, None), "mul_mat_scale_add")
+        return out
+
+    def swiglu():
+        out = torch.empty_like(a)
+        gpu.check(L.vx_mul_mat_swiglu(gpu.desc_q8(wq, K), gpu.desc_q8(wq2, K), d(xd), d(out), gpu.ACT_FLOAT, None), "mul_mat_swiglu")
+        return out
+
+    if L.vx_supports_mul_mat_scale_add(gpu.desc_q8(wq, K), d(xd), d(res), d(a)):
+        a2, b2 = both(scale_add)
+        assert torch.equal(a2, b2), float((a2 - b2).abs().max())
+    if L.vx_supports_mul_mat_swiglu_tiled(gpu.desc_q8(wq, K), gpu.desc_q8(wq2, K), d(xd), d(a), gpu.ACT_FLOAT):
+        a3, b3 = both(swiglu)
+        assert torch.equal(a3, b3), float((a3 - b3).abs().max())
+
+
 @pytest.mark.parametrize("seed", list(range(48)))
 def test_mul_mat_q8_0_random_shapes(gpu, seed):
     """Random row, column and token counts around every threshold the launcher has (streaming kernel up to 16 tokens and a

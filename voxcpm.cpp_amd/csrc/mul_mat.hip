@@ -1841,6 +1841,296 @@ thread_local vx_status t_ws_status = VX_OK;
 bool ws_failed() { return t_ws_status != VX_OK; }
 vx_status take_ws_status() { const vx_status rc = t_ws_status; t_ws_status = VX_OK; return rc; }
 
+// ---- Q8_0 weights x many tokens, both operands laid out for the matrix cores beforehand -----------------------------
+// At prefill sizes every weight is used by hundreds of token tiles and every activation by dozens of row tiles; the
+// kernel above converts each of them (int8 -> f16, f32 -> f16) once per tile that uses it, and that conversion work, not
+// the matrix cores, bounds it.  Here two small passes convert once: the weights into exact f16 integers with their block
+// scales apart, the activations into f16 (to nearest even, as the kernel above rounds them), both written as the 1 KB
+// operand tiles of v_mfma_f32_16x16x32_f16 -- [k block][16-row tile][lane (j, c): row c, k 8j .. 8j + 7] -- so that the
+// product kernel brings a tile into LDS with one direct load (global_load_lds_dwordx4, no register, no address
+// arithmetic) and reads an operand with one conflict-free 16-byte LDS load.  The arithmetic is the kernel above's: a 32-wide
+// partial product per block from one MFMA, scaled by the block's d in fp32 and added -- the same bits.
+//
+// Work-group: 8 waves, 256 rows x 128 tokens (a wave: 64 x 64 = 4 x 4 MFMA tiles), three stages of one k block
+// (16 KB of weights, 8 KB of activations, 1 KB of scales), one barrier a block, two work-groups to a compute unit (75 KB
+// of LDS and 128 registers each): everything a wave does besides its MFMAs -- issuing the direct loads (a hundred
+// cycles apiece), the barrier, the operand reads, the 64 scaled additions of a block, the stores at the end -- was
+// measured to add up unhidden with one work-group's waves in step; the second work-group's waves fill those gaps.
+// The weights are the MFMA's row operand, so a lane ends up with four consecutive rows of one token: 16-byte stores.
+// Work-groups are dealt to the XCDs in groups of 4 row tiles x 8 token tiles that run side by side on one XCD's 32
+// compute units and share its L2.
+// Measured on 4096 rows x K 1024 x 16384 tokens: 215 us with both passes (12 and 22 us) against 300 us for the kernel
+// above; without the stores 189 us, without the direct loads 195 us -- what bounds it is no single unit: a block's MFMAs
+// (512 cycles per SIMD), its scaled additions (608), its LDS reads (516 at the LDS's full rate) and its direct loads
+// are each about as long, and they overlap only as far as four waves per SIMD interleave.
+constexpr int QT_ROWS = 256, QT_TOKS = 128, QT_STAGES = 3;
+constexpr int QT_STAGE_BYTES = (QT_ROWS + QT_TOKS) / 16 * 1024 + QT_ROWS * 4;
+constexpr size_t QT_LDS = (size_t) QT_STAGES * QT_STAGE_BYTES;
+
+struct qt_args {
+    const char * w; const char * w2; // Q8_0 rows (w2: the second matrix of a gate/up pair, else null)
+    const char * x; char * dst; const char * res;
+    int64_t  K, M, N;                // M: rows of one matrix
+    uint64_t nb01, nb11, nb12, nb13, nb1, nb2, nb3, rnb1, rnb2, rnb3;
+    int      ne12;
+    float    res_scale;
+    half8_t * wt; float * wdt; half8_t * xt; // the operand tiles in the workspace
+    int      n_rt, n_tt, n_kb;       // 16-row tiles (of the virtual matrix: gate and up tiles alternate), token tiles, k blocks
+    int      w_al4;
+};
+
+// one thread = 8 quants of a block: (virtual row, block, j)
+__global__ __launch_bounds__(256) void qt_weights_kernel(const qt_args a) {
+    const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    const int     slot = (int) (idx & 63), c = slot & 15, j = slot >> 4;
+    const int64_t t = idx >> 6;
+    const int64_t kb = t % a.n_kb; // (neighbouring waves: neighbouring blocks of the same 16 rows, which share cache lines)
+    const int64_t rt = t / a.n_kb;
+    if (rt >= a.n_rt) return;
+    const bool    dual = a.w2 != nullptr;
+    const int64_t row  = dual ? 16 * (int64_t) (rt >> 1) + c : 16 * (int64_t) rt + c; // of its own matrix
+    const char *  wsel = dual && (rt & 1) ? a.w2 : a.w;
+    half8_t h = {0, 0, 0, 0, 0, 0, 0, 0};
+    float   d = 0.0f;
+    if (row < a.M) {
+        const char * wrow = wsel + (uint64_t) row * a.nb01;
+        h = q8_unpack(q8_load(wrow, kb, j, a.w_al4 != 0), kb, a.w_al4 != 0);
+        d = (float) *(const _Float16 *) (wrow + kb * VX_Q8_BLOCK);
+    }
+    a.wt[(kb * a.n_rt + rt) * 64 + slot] = h;
+    if (j == 0) a.wdt[kb * ((int64_t) a.n_rt * 16) + 16 * rt + c] = d;
+}
+
+// one thread = 8 consecutive k of a token: (token, block, j); blockIdx.y = batch entry
+__global__ __launch_bounds__(256) void qt_acts_kernel(const qt_args a) {
+    const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    const int     slot = (int) (idx & 63), c = slot & 15, j = slot >> 4;
+    const int64_t t = idx >> 6;
+    const int     kb = (int) (t % a.n_kb); // (a wave's neighbours in k: the four j of a token read one 128-byte line)
+    const int64_t tt = t / a.n_kb;
+    if (tt >= a.n_tt) return;
+    const int     batch = blockIdx.y, i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const int64_t tok = 16 * tt + c;
+    half8_t h = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (tok < a.N) {
+        const float4_t * p = (const float4_t *) (a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) tok * a.nb11 + (uint64_t) (32 * kb + 8 * j) * 4);
+        const float4_t lo = p[0], hi = p[1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { h[i] = (_Float16) lo[i]; h[4 + i] = (_Float16) hi[i]; }
+    }
+    a.xt[(((int64_t) batch * a.n_kb + kb) * a.n_tt + tt) * 64 + slot] = h;
+}
+
+__device__ __forceinline__ void qt_dma16(const void * base, uint32_t off, uint32_t lds) {
+    // 16 bytes per lane from global memory (uniform base + lane offset) into LDS at lds + 16 lane
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "memory");
+}
+
+template <bool DUAL>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_q8t_kernel(const qt_args a) {
+    extern __shared__ __align__(1024) char qt_smem[]; // per stage: 8 token tiles, 16 row tiles, 256 scales
+    typedef __attribute__((address_space(3))) char lds_char;
+    const int lane = threadIdx.x & 63, wid = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+    const int j = lane >> 4, c = lane & 15;
+    const int wr = wid >> 1, wc = wid & 1;
+
+    // which tile: groups of 4 row tiles x 8 token tiles, a group's 32 work-groups on one XCD
+    const int gx = (a.n_rt + 15) / 16, gy = (a.n_tt + 7) / 8; // tiles of 256 rows / 128 tokens
+    const int Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int group = (seq >> 5) * 8 + xcd, within = seq & 31;
+    if (group >= Gx * Gy) return;
+    const int tx = (group % Gx) * 4 + (within & 3), ty = (group / Gx) * 8 + (within >> 2);
+    if (tx >= gx || ty >= gy) return;
+    const int batch = blockIdx.y, i12 = batch % a.ne12, i13 = batch / a.ne12;
+
+    // ---- direct loads of a stage: wave w brings row tiles 2w and 2w + 1 and token tile w; wave 0 the scales as well.
+    // A tile past the operand's last one is not loaded (its products are dropped at the store).
+    const int rt0 = 16 * tx, tt0 = 8 * ty;
+    const uint32_t smem0 = (uint32_t) (uintptr_t) (lds_char *) qt_smem;
+    const bool     have_w0 = rt0 + 2 * wid < a.n_rt, have_w1 = rt0 + 2 * wid + 1 < a.n_rt, have_x = tt0 + wid < a.n_tt;
+    const half8_t * wsrc = a.wt + ((int64_t) rt0 + 2 * wid) * 64;
+    const half8_t * xsrc = a.xt + ((int64_t) batch * a.n_kb * a.n_tt + tt0 + wid) * 64;
+    const float *   dsrc = a.wdt + (int64_t) rt0 * 16;
+    const uint32_t  loff = (uint32_t) lane * 16;
+    const int       n_dsc = min(256, (a.n_rt - rt0) * 16) / 4; // 16-byte pieces of the scale row that exist
+    auto issue = [&](int kb) {
+        const uint32_t st = smem0 + (uint32_t) (kb % QT_STAGES) * QT_STAGE_BYTES;
+        if (have_x)  qt_dma16(xsrc + (int64_t) kb * a.n_tt * 64, loff, st + wid * 1024);
+        if (have_w0) qt_dma16(wsrc + (int64_t) kb * a.n_rt * 64, loff, st + 8192 + 2 * wid * 1024);
+        if (have_w1) qt_dma16(wsrc + (int64_t) kb * a.n_rt * 64 + 64, loff, st + 8192 + (2 * wid + 1) * 1024);
+        if (wid == 0) qt_dma16(dsrc + (int64_t) kb * a.n_rt * 16, lane < n_dsc ? loff : 0u, st + 8192 + 16384);
+    };
+    // (a wave waits for its own loads, so it counts what it issued per stage)
+    const int mine = (have_x ? 1 : 0) + (have_w0 ? 1 : 0) + (have_w1 ? 1 : 0) + (wid == 0 ? 1 : 0);
+
+    float4_t acc[4][4]; // [row tile][token tile]
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) acc[rt][tt] = float4_t{0, 0, 0, 0};
+
+    const int nkb = a.n_kb;
+    auto wait_stage = [&](int kb) { // stage kb has landed once only the younger stages' loads of this wave are outstanding
+        const int younger = min(QT_STAGES - 2, nkb - 1 - kb) * mine;
+        if (younger >= 8)      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else if (younger == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        else if (younger == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if (younger == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+        else if (younger == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else                   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    // 16 MFMAs and their 64 scaled additions: the additions of a product follow the MFMA two further on, so that matrix
+    // instructions are in flight while the vector unit scales an earlier one
+    auto multiply = [&](int kb) {
+        const lds_char * st = (const lds_char *) qt_smem + (kb % QT_STAGES) * QT_STAGE_BYTES;
+        half8_t  bop[4];
+        float4_t dw[4]; // the scales of the four rows a lane holds of a row tile
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            bop[rt] = *(const __attribute__((address_space(3))) half8_t *) (st + 8192 + (4 * wr + rt) * 1024 + lane * 16);
+            dw[rt]  = *(const __attribute__((address_space(3))) float4_t *) (st + 8192 + 16384 + (64 * wr + 16 * rt + 4 * j) * 4);
+        }
+        half8_t aop[2];
+        aop[0] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc) * 1024 + lane * 16);
+        float4_t blk[3];
+#pragma unroll
+        for (int i = 0; i < 18; ++i) {
+            const int tt = i >> 2, rt = i & 3;
+            if (i < 16) {
+                if (rt == 0 && tt < 3) aop[(tt + 1) & 1] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc + tt + 1) * 1024 + lane * 16);
+                blk[i % 3] = mfma16(bop[rt], aop[tt & 1], float4_t{0, 0, 0, 0}); // (weights as the row operand: a lane gets 4 consecutive rows of one token)
+            }
+            if (i >= 2) {
+                const int p = i - 2;
+                acc[p & 3][p >> 2] += blk[p % 3] * dw[p & 3];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < QT_STAGES - 1; ++s)
+        if (s < nkb) issue(s);
+    for (int kb = 0; kb < nkb; ++kb) {
+        wait_stage(kb);
+        __syncthreads(); // every wave's part of stage kb is in LDS, and every wave is done with stage kb - 1
+        if (kb + QT_STAGES - 1 < nkb) issue(kb + QT_STAGES - 1);
+        multiply(kb);
+    }
+
+    // lane (j, c), tile (rt, tt), register r: token tok0 + 16 tt + c, virtual row 16 (rt0 + 4 wr + rt) + 4 j + r:
+    // four consecutive elements of a row of dst
+    const int64_t tok0 = (int64_t) ty * QT_TOKS + 64 * wc;
+    char * db = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    const bool vec = a.M % 4 == 0 && ((uintptr_t) db | a.nb1) % 16 == 0; // uniform
+    if constexpr (DUAL) {
+        // tile pair (2p, 2p + 1) holds gate and up of rows 16 (rt0 / 2 + 2 wr + p) + 4 j + r
+#pragma unroll
+        for (int p2 = 0; p2 < 2; ++p2) {
+            const int64_t row = 16 * ((int64_t) (rt0 >> 1) + 2 * wr + p2) + 4 * j;
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                const int64_t tok = tok0 + 16 * tt + c;
+                if (tok >= a.N) continue;
+                float4_t v;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
+                    v[r] = (g / (1.0f + expf(-g))) * u;
+                }
+                float * pd = (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4);
+                if (vec && row + 3 < a.M) __builtin_nontemporal_store(v, (float4_t *) pd);
+                else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) if (row + r < a.M) pd[r] = v[r];
+                }
+            }
+        }
+        return;
+    }
+    const bool   residual = a.res != nullptr; // uniform
+    const char * rbase    = residual ? a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 : nullptr;
+    const bool   rvec     = residual && ((uintptr_t) rbase | a.rnb1) % 16 == 0;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const int64_t row = 16 * ((int64_t) rt0 + 4 * wr + rt) + 4 * j;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            const int64_t tok = tok0 + 16 * tt + c;
+            if (tok >= a.N) continue;
+            float4_t v = acc[rt][tt];
+            float * pd = (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4);
+            if (vec && row + 3 < a.M) {
+                if (residual) {
+                    const float * pr = (const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) row * 4);
+                    float4_t rv;
+                    if (rvec) rv = *(const float4_t *) pr; else rv = float4_t{pr[0], pr[1], pr[2], pr[3]};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = scaled_residual(v[r], a.res_scale, rv[r]);
+                }
+                __builtin_nontemporal_store(v, (float4_t *) pd);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (row + r < a.M) {
+                        float x = v[r];
+                        if (residual) x = scaled_residual(x, a.res_scale, *(const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) (row + r) * 4));
+                        pd[r] = x;
+                    }
+            }
+        }
+    }
+}
+
+// VX_GEMM_Q8T=0 keeps these products on gemm_lds_kernel (read on every call: a product of this size takes a hundred
+// microseconds, and a test compares the two in one process)
+bool gemm_q8t_on() { const char * e = getenv("VX_GEMM_Q8T"); return !(e && atoi(e) == 0); }
+
+// the shapes the pre-tiled kernel takes: one weight matrix for every batch entry, at least 1024 (virtual) rows and
+// 1024 tokens -- below that the two passes in front cost more than they save
+bool gemm_q8t_takes(const mm_args & a, int nbatch, bool dual) {
+    const int64_t MV = dual ? 2 * a.M : a.M;
+    return gemm_q8t_on() && a.K % 32 == 0 && (!dual || a.M % 16 == 0) && MV >= 1024 && a.N >= 1024 && a.x_aligned && (nbatch == 1 || (a.r2 == a.ne12 && a.r3 * a.ne12 == nbatch)) &&
+           a.K < (1ll << 24) && nbatch <= 65535;
+}
+
+template <bool DUAL>
+bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st) {
+    qt_args q = {};
+    q.w = a.w; q.w2 = DUAL ? a.w2 : nullptr; q.x = a.x; q.dst = a.dst; q.res = DUAL ? nullptr : a.res;
+    q.K = a.K; q.M = a.M; q.N = a.N;
+    q.nb01 = a.nb01; q.nb11 = a.nb11; q.nb12 = a.nb12; q.nb13 = a.nb13; q.nb1 = a.nb1; q.nb2 = a.nb2; q.nb3 = a.nb3;
+    q.rnb1 = a.rnb1; q.rnb2 = a.rnb2; q.rnb3 = a.rnb3;
+    q.ne12 = a.ne12; q.res_scale = a.res_scale;
+    q.w_al4 = a.w_aligned;
+    const int64_t MV = DUAL ? 2 * a.M : a.M;
+    q.n_rt = (int) ((MV + 15) / 16); q.n_tt = (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
+    const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * q.n_rt * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
+    const size_t xt_bytes = (size_t) nbatch * q.n_kb * q.n_tt * 1024;
+    void * ws = nullptr;
+    if ((t_ws_status = vx_workspace(st, a.ws_offset + wt_bytes + wd_bytes + xt_bytes, &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
+    char * base = (char *) ws + a.ws_offset;
+    q.wt = (half8_t *) base; q.wdt = (float *) (base + wt_bytes); q.xt = (half8_t *) (base + wt_bytes + wd_bytes);
+    static bool raised = false;
+    if (!raised) {
+        if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess) {
+            (void) hipGetLastError();
+            return false;
+        }
+        raised = true;
+    }
+    const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) q.n_kb * q.n_tt * 64;
+    if ((wunits + 255) / 256 > 0x7fffffff || (xunits + 255) / 256 > 0x7fffffff) return false;
+    qt_weights_kernel<<<dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st>>>(q);
+    qt_acts_kernel<<<dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st>>>(q);
+    const int gx = (q.n_rt + 15) / 16, gy = (q.n_tt + 7) / 8, Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
+    const int64_t blocks = ((int64_t) Gx * Gy + 7) / 8 * 8 * 32;
+    if (blocks > 0x7fffffff) return false;
+    gemm_q8t_kernel<DUAL><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
+    return true;
+}
+
 template <int WT>
 bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     const int mode = gemm_lds_mode();
@@ -1851,6 +2141,9 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 256 * a.nb11 + 256 >= (1ull << 32) ||
         (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32) || a.K >= (1ll << 28)) return false;
     const bool fold = WT == WT_Q8 && mode == 2;
+    if constexpr (WT == WT_Q8) {
+        if (mode == 1 && gemm_q8t_takes(a, nbatch, false) && !(a.res && (uint64_t) 256 * a.rnb1 + 1024 >= (1ull << 32))) return launch_gemm_q8t<false>(a, nbatch, st);
+    }
     // (a residual update is fused into the kernel that adds a cut K's partials, nowhere else here)
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
     const bool big = ((a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
@@ -1884,6 +2177,9 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
 template <int WT>
 bool launch_gemm_lds_swiglu(const mm_args & a, int nbatch, hipStream_t st) {
     const bool fold = WT == WT_Q8 && gemm_lds_mode() == 2;
+    if constexpr (WT == WT_Q8) {
+        if (!fold && gemm_q8t_takes(a, nbatch, true)) return launch_gemm_q8t<true>(a, nbatch, st);
+    }
     const bool big  = ((2 * a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     if constexpr (WT == WT_Q8) {
         if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4, true>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2, true>(a, nbatch, st);
