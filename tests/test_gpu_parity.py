@@ -496,15 +496,21 @@ def test_mul_mat_q8_0_full_size_prefill(gpu):
 
 @pytest.mark.parametrize("M,K,N,batch", [(4096, 1024, 4096, 1), (1024, 4096, 2048, 1), (2000, 1056, 1700, 1), (1030, 1024, 1100, 1),
                                          (1024, 1024, 1024, 3), (1024, 2176, 1500, 2)])
-def test_mul_mat_q8_0_pretiled_equals_the_lds_kernel(gpu, M, K, N, batch, monkeypatch):
+@pytest.mark.parametrize("folded", [False, True])
+def test_mul_mat_q8_0_pretiled_equals_the_lds_kernel(gpu, M, K, N, batch, folded, monkeypatch):
     """Products of 1024 rows and tokens or more take the kernel whose operands two passes lay out beforehand (weights as
     exact f16 integers with their scales apart, activations rounded to f16); VX_GEMM_Q8T=0 keeps them on the kernel that
     converts inside every tile.  Both form a block's partial product with the same matrix instruction and scale and add
     it in fp32 in the same order: the plain product, the fused residual update and the fused gate/up SwiGLU must be the
-    same bits -- full and ragged tiles in both dimensions, K with an odd number of blocks, a batch of sequences."""
+    same bits -- full and ragged tiles in both dimensions, K with an odd number of blocks, a batch of sequences.  folded:
+    the opt-in form of both kernels (VX_GEMM_LDS=2) in which the block scale is multiplied into the f16 weights."""
     import torch
     L, d = gpu.lib(), gpu.desc
-    say(f"pre-tiled Q8_0 product vs the LDS kernel M={M} K={K} N={N} batch={batch}")
+    say(f"pre-tiled Q8_0 product vs the LDS kernel M={M} K={K} N={N} batch={batch} folded={folded}")
+    if folded:
+        monkeypatch.setenv("VX_GEMM_LDS", "2")
+    else:
+        monkeypatch.delenv("VX_GEMM_LDS", raising=False)
     w = (rng("q8t", "w", M, K).standard_normal((M, K)) * 0.02).astype(np.float32)
     w2 = (rng("q8t", "w2", M, K).standard_normal((M, K)) * 0.02).astype(np.float32)
     x = rng("q8t", "x", N, K).standard_normal((batch, N, K) if batch > 1 else (N, K)).astype(np.float32)

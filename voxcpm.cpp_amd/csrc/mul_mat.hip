@@ -1877,6 +1877,7 @@ struct qt_args {
     half8_t * wt; float * wdt; half8_t * xt; // the operand tiles in the workspace
     int      n_rt, n_tt, n_kb;       // 16-row tiles (of the virtual matrix: gate and up tiles alternate), token tiles, k blocks
     int      w_al4;
+    int      fold;                   // the block scale multiplied into the f16 weights by the weight pass (VX_GEMM_LDS=2)
 };
 
 // one thread = 8 quants of a block: (virtual row, block, j)
@@ -1895,30 +1896,52 @@ __global__ __launch_bounds__(256) void qt_weights_kernel(const qt_args a) {
     if (row < a.M) {
         const char * wrow = wsel + (uint64_t) row * a.nb01;
         h = q8_unpack(q8_load(wrow, kb, j, a.w_al4 != 0), kb, a.w_al4 != 0);
-        d = (float) *(const _Float16 *) (wrow + kb * VX_Q8_BLOCK);
+        const _Float16 dh = *(const _Float16 *) (wrow + kb * VX_Q8_BLOCK);
+        d = (float) dh;
+        if (a.fold) { // q * d rounded once to f16, as gemm_lds_kernel's FOLD form parks it
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] *= dh;
+        }
     }
     a.wt[(kb * a.n_rt + rt) * 64 + slot] = h;
     if (j == 0) a.wdt[kb * ((int64_t) a.n_rt * 16) + 16 * rt + c] = d;
 }
 
-// one thread = 8 consecutive k of a token: (token, block, j); blockIdx.y = batch entry
+// one thread = 8 consecutive k of a token in each of QT_ACT_UNROLL k blocks: (token, group of blocks, j); blockIdx.y =
+// batch entry.  A wave reads 16 tokens x 128 bytes per block, all blocks' loads in flight together, and writes one 1 KB
+// tile per block.
+constexpr int QT_ACT_UNROLL = 4;
 __global__ __launch_bounds__(256) void qt_acts_kernel(const qt_args a) {
     const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
     const int     slot = (int) (idx & 63), c = slot & 15, j = slot >> 4;
     const int64_t t = idx >> 6;
-    const int     kb = (int) (t % a.n_kb); // (a wave's neighbours in k: the four j of a token read one 128-byte line)
-    const int64_t tt = t / a.n_kb;
+    const int     n_kg = (a.n_kb + QT_ACT_UNROLL - 1) / QT_ACT_UNROLL;
+    const int     kb0 = (int) (t % n_kg) * QT_ACT_UNROLL;
+    const int64_t tt = t / n_kg;
     if (tt >= a.n_tt) return;
     const int     batch = blockIdx.y, i12 = batch % a.ne12, i13 = batch / a.ne12;
     const int64_t tok = 16 * tt + c;
-    half8_t h = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (tok < a.N) {
-        const float4_t * p = (const float4_t *) (a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) tok * a.nb11 + (uint64_t) (32 * kb + 8 * j) * 4);
-        const float4_t lo = p[0], hi = p[1];
+    float4_t lo[QT_ACT_UNROLL], hi[QT_ACT_UNROLL];
+    const bool live = tok < a.N;
+    const char * row = a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) (live ? tok : 0) * a.nb11;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { h[i] = (_Float16) lo[i]; h[4 + i] = (_Float16) hi[i]; }
+    for (int u = 0; u < QT_ACT_UNROLL; ++u) {
+        const int kb = min(kb0 + u, a.n_kb - 1);
+        const float4_t * p = (const float4_t *) (row + (uint64_t) (32 * kb + 8 * j) * 4);
+        lo[u] = __builtin_nontemporal_load(p);
+        hi[u] = __builtin_nontemporal_load(p + 1);
     }
-    a.xt[(((int64_t) batch * a.n_kb + kb) * a.n_tt + tt) * 64 + slot] = h;
+#pragma unroll
+    for (int u = 0; u < QT_ACT_UNROLL; ++u) {
+        const int kb = kb0 + u;
+        if (kb >= a.n_kb) break;
+        half8_t h = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { h[i] = (_Float16) lo[u][i]; h[4 + i] = (_Float16) hi[u][i]; }
+        }
+        a.xt[(((int64_t) batch * a.n_kb + kb) * a.n_tt + tt) * 64 + slot] = h;
+    }
 }
 
 __device__ __forceinline__ void qt_dma16(const void * base, uint32_t off, uint32_t lds) {
@@ -1926,7 +1949,7 @@ __device__ __forceinline__ void qt_dma16(const void * base, uint32_t off, uint32
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "memory");
 }
 
-template <bool DUAL>
+template <bool DUAL, bool FOLD>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_q8t_kernel(const qt_args a) {
     extern __shared__ __align__(1024) char qt_smem[]; // per stage: 8 token tiles, 16 row tiles, 256 scales
     typedef __attribute__((address_space(3))) char lds_char;
@@ -1993,6 +2016,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
         half8_t aop[2];
         aop[0] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc) * 1024 + lane * 16);
+        if constexpr (FOLD) { // the scale is in the weights: the MFMAs accumulate across blocks
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                if (tt < 3) aop[(tt + 1) & 1] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc + tt + 1) * 1024 + lane * 16);
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) acc[rt][tt] = mfma16(bop[rt], aop[tt & 1], acc[rt][tt]);
+            }
+            return;
+        }
         float4_t blk[3];
 #pragma unroll
         for (int i = 0; i < 18; ++i) {
@@ -2000,6 +2032,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             if (i < 16) {
                 if (rt == 0 && tt < 3) aop[(tt + 1) & 1] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc + tt + 1) * 1024 + lane * 16);
                 blk[i % 3] = mfma16(bop[rt], aop[tt & 1], float4_t{0, 0, 0, 0}); // (weights as the row operand: a lane gets 4 consecutive rows of one token)
+                __builtin_amdgcn_sched_barrier(0); // (the MFMA first: the additions below belong to the one two before it)
             }
             if (i >= 2) {
                 const int p = i - 2;
@@ -2095,7 +2128,7 @@ bool gemm_q8t_takes(const mm_args & a, int nbatch, bool dual) {
 }
 
 template <bool DUAL>
-bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st) {
+bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     qt_args q = {};
     q.w = a.w; q.w2 = DUAL ? a.w2 : nullptr; q.x = a.x; q.dst = a.dst; q.res = DUAL ? nullptr : a.res;
     q.K = a.K; q.M = a.M; q.N = a.N;
@@ -2103,6 +2136,7 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st) {
     q.rnb1 = a.rnb1; q.rnb2 = a.rnb2; q.rnb3 = a.rnb3;
     q.ne12 = a.ne12; q.res_scale = a.res_scale;
     q.w_al4 = a.w_aligned;
+    q.fold  = fold;
     const int64_t MV = DUAL ? 2 * a.M : a.M;
     q.n_rt = (int) ((MV + 15) / 16); q.n_tt = (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
     const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * q.n_rt * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
@@ -2113,21 +2147,24 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st) {
     q.wt = (half8_t *) base; q.wdt = (float *) (base + wt_bytes); q.xt = (half8_t *) (base + wt_bytes + wd_bytes);
     static bool raised = false;
     if (!raised) {
-        if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
-            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess) {
+        if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess) {
             (void) hipGetLastError();
             return false;
         }
         raised = true;
     }
-    const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) q.n_kb * q.n_tt * 64;
+    const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) ((q.n_kb + QT_ACT_UNROLL - 1) / QT_ACT_UNROLL) * q.n_tt * 64;
     if ((wunits + 255) / 256 > 0x7fffffff || (xunits + 255) / 256 > 0x7fffffff) return false;
     qt_weights_kernel<<<dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st>>>(q);
     qt_acts_kernel<<<dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st>>>(q);
     const int gx = (q.n_rt + 15) / 16, gy = (q.n_tt + 7) / 8, Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
     const int64_t blocks = ((int64_t) Gx * Gy + 7) / 8 * 8 * 32;
     if (blocks > 0x7fffffff) return false;
-    gemm_q8t_kernel<DUAL><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
+    if (fold) gemm_q8t_kernel<DUAL, true><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
+    else      gemm_q8t_kernel<DUAL, false><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
     return true;
 }
 
@@ -2142,7 +2179,7 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
         (uint64_t) 256 * a.nb1 + 1024 >= (1ull << 32) || a.K >= (1ll << 28)) return false;
     const bool fold = WT == WT_Q8 && mode == 2;
     if constexpr (WT == WT_Q8) {
-        if (mode == 1 && gemm_q8t_takes(a, nbatch, false) && !(a.res && (uint64_t) 256 * a.rnb1 + 1024 >= (1ull << 32))) return launch_gemm_q8t<false>(a, nbatch, st);
+        if (gemm_q8t_takes(a, nbatch, false)) return launch_gemm_q8t<false>(a, nbatch, st, fold);
     }
     // (a residual update is fused into the kernel that adds a cut K's partials, nowhere else here)
     // 128 x 128 tiles once they fill most of the chip, else 64 x 64
@@ -2178,7 +2215,7 @@ template <int WT>
 bool launch_gemm_lds_swiglu(const mm_args & a, int nbatch, hipStream_t st) {
     const bool fold = WT == WT_Q8 && gemm_lds_mode() == 2;
     if constexpr (WT == WT_Q8) {
-        if (!fold && gemm_q8t_takes(a, nbatch, true)) return launch_gemm_q8t<true>(a, nbatch, st);
+        if (gemm_q8t_takes(a, nbatch, true)) return launch_gemm_q8t<true>(a, nbatch, st, fold);
     }
     const bool big  = ((2 * a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     if constexpr (WT == WT_Q8) {
@@ -2276,6 +2313,7 @@ extern "C" vx_status vx_mul_mat(const vx_tensor * src0, const vx_tensor * src1, 
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
 
+    (void) take_ws_status();
     switch (src0->type) {
         case VX_TYPE_Q8_0:
             if (act_mode == VX_ACT_Q8) launch<WT_Q8, true>(a, nbatch, st);
@@ -2386,9 +2424,11 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
     bool ok;
+    (void) take_ws_status();
     if (tiled)                           ok = gate->type == VX_TYPE_Q8_0 ? launch_gemm_lds_swiglu<WT_Q8>(a, nbatch, st) : launch_gemm_lds_swiglu<WT_F16>(a, nbatch, st);
     else if (gate->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
     else                                 ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (ws_failed()) return take_ws_status(); // (the pre-tiled kernel's workspace: never answered by another kernel)
     if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: shape outside the streaming and the tiled kernel");
     VX_LAUNCH_CHECK();
     return VX_OK;
@@ -2445,6 +2485,7 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
     bool ok;
+    (void) take_ws_status();
     if (src0->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
     else                            ok = launch_gemv<WT_F16, false>(a, nbatch, st);
     if (!ok) { // not the streaming kernel's shape: the tiled kernels with K cut (see vx_supports_mul_mat_scale_add)
