@@ -980,6 +980,7 @@ struct kvs_args {
     int64_t  ne[4];
     uint64_t nbx[4], nbd[4];
     float scale, bias;
+    int dense4; // x and d are contiguous, 16-byte aligned, a multiple of 4 elements: the ADD1 walks them 16 bytes at a time
 };
 
 // stores the slot and returns the sum of what was stored, the same value in every thread of the block
@@ -1065,6 +1066,13 @@ __global__ __launch_bounds__(256) void kv_sync_add1_kernel(const kvs_args a, con
     const float y = y_s;
     const uint32_t n0 = (uint32_t) a.ne[0], n1 = (uint32_t) a.ne[1], n2 = (uint32_t) a.ne[2];
     const uint64_t nx = (uint64_t) n0 * n1 * (uint64_t) (n2 * a.ne[3]);
+    if (a.dense4) { // (a prefill's attention output: 256 MiB at 16 x 4096 tokens; element by element with its index
+        // arithmetic this pass took 228 us)
+        const float4_t * px = (const float4_t *) a.x;
+        float4_t *       pd = (float4_t *) a.d;
+        for (uint64_t e = (uint64_t) blockIdx.x * 256 + threadIdx.x; e < nx / 4; e += (uint64_t) gridDim.x * 256) pd[e] = px[e] + y;
+        return;
+    }
     for (uint64_t e = (uint64_t) blockIdx.x * 256 + threadIdx.x; e < nx; e += (uint64_t) gridDim.x * 256) {
         uint64_t r = e;
         const uint32_t i0 = (uint32_t) (r % n0); r /= n0;
@@ -1835,6 +1843,7 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
     a.x = (const char *) x->data; a.d = (char *) dst->data;
     for (int i = 0; i < 4; ++i) { a.ne[i] = x->ne[i]; a.nbx[i] = x->nb[i]; a.nbd[i] = dst->nb[i]; }
     a.scale = scale; a.bias = bias;
+    a.dense4 = vx_is_contiguous(x) && vx_is_contiguous(dst) && vx_nelements(x) % 4 == 0 && ((uintptr_t) x->data | (uintptr_t) dst->data) % 16 == 0;
     if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) {
         kv_store_sync_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
     } else { // a prefill's write: stores and block totals, then totals, scalar and ADD1
