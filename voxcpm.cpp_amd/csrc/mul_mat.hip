@@ -1856,13 +1856,15 @@ vx_status take_ws_status() { const vx_status rc = t_ws_status; t_ws_status = VX_
 // of LDS and 128 registers each): everything a wave does besides its MFMAs -- issuing the direct loads (a hundred
 // cycles apiece), the barrier, the operand reads, the 64 scaled additions of a block, the stores at the end -- was
 // measured to add up unhidden with one work-group's waves in step; the second work-group's waves fill those gaps.
-// The weights are the MFMA's row operand, so a lane ends up with four consecutive rows of one token: 16-byte stores.
+// The weights are the MFMA's column operand: lane c holds row c of every row tile and needs one scale per tile, which the
+// weight pass lays out so that a lane's four come with one 16-byte LDS load.
 // Work-groups are dealt to the XCDs in groups of 4 row tiles x 8 token tiles that run side by side on one XCD's 32
 // compute units and share its L2.
-// Measured on 4096 rows x K 1024 x 16384 tokens: 215 us with both passes (12 and 22 us) against 300 us for the kernel
-// above; without the stores 189 us, without the direct loads 195 us -- what bounds it is no single unit: a block's MFMAs
-// (512 cycles per SIMD), its scaled additions (608), its LDS reads (516 at the LDS's full rate) and its direct loads
-// are each about as long, and they overlap only as far as four waves per SIMD interleave.
+// Measured on 4096 rows x K 1024 x 16384 tokens: 210 us with both passes (11 and 21 us) against 300 us for the kernel
+// above.  What bounds it: 16-byte LDS reads deliver about 64 bytes a cycle per compute unit, counted at their full 64
+// lanes x 16 bytes whatever they broadcast (9 KB per wave and block: 148 us for this product), and a SIMD's vector unit
+// and matrix core do not run side by side (16 + 4 x 4.75 cycles per MFMA with its four scaled additions: 143 us); the
+// kernel runs at 175 us.
 constexpr int QT_ROWS = 256, QT_TOKS = 128, QT_STAGES = 3;
 constexpr int QT_STAGE_BYTES = (QT_ROWS + QT_TOKS) / 16 * 1024 + QT_ROWS * 4;
 constexpr size_t QT_LDS = (size_t) QT_STAGES * QT_STAGE_BYTES;
@@ -1904,7 +1906,9 @@ __global__ __launch_bounds__(256) void qt_weights_kernel(const qt_args a) {
         }
     }
     a.wt[(kb * a.n_rt + rt) * 64 + slot] = h;
-    if (j == 0) a.wdt[kb * ((int64_t) a.n_rt * 16) + 16 * rt + c] = d;
+    // (scales: within every 64 rows, row 16 t + c sits at 4 c + t, so that a lane of the product kernel reads the scales of
+    // its row c in the wave's four row tiles with one 16-byte load)
+    if (j == 0) a.wdt[kb * ((int64_t) ((a.n_rt + 3) & ~3) * 16) + 64 * (rt >> 2) + 4 * c + (rt & 3)] = d; // (a row of whole groups of 64)
 }
 
 // one thread = 8 consecutive k of a token in each of QT_ACT_UNROLL k blocks: (token, group of blocks, j); blockIdx.y =
@@ -1976,13 +1980,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const half8_t * xsrc = a.xt + ((int64_t) batch * a.n_kb * a.n_tt + tt0 + wid) * 64;
     const float *   dsrc = a.wdt + (int64_t) rt0 * 16;
     const uint32_t  loff = (uint32_t) lane * 16;
-    const int       n_dsc = min(256, (a.n_rt - rt0) * 16) / 4; // 16-byte pieces of the scale row that exist
+    const int       n_rt4 = (a.n_rt + 3) & ~3;                  // the scale rows hold whole groups of 64 rows
+    const int       n_dsc = min(256, (n_rt4 - rt0) * 16) / 4;  // 16-byte pieces of the scale row that exist
     auto issue = [&](int kb) {
         const uint32_t st = smem0 + (uint32_t) (kb % QT_STAGES) * QT_STAGE_BYTES;
         if (have_x)  qt_dma16(xsrc + (int64_t) kb * a.n_tt * 64, loff, st + wid * 1024);
         if (have_w0) qt_dma16(wsrc + (int64_t) kb * a.n_rt * 64, loff, st + 8192 + 2 * wid * 1024);
         if (have_w1) qt_dma16(wsrc + (int64_t) kb * a.n_rt * 64 + 64, loff, st + 8192 + (2 * wid + 1) * 1024);
-        if (wid == 0) qt_dma16(dsrc + (int64_t) kb * a.n_rt * 16, lane < n_dsc ? loff : 0u, st + 8192 + 16384);
+        if (wid == 0) qt_dma16(dsrc + (int64_t) kb * n_rt4 * 16, lane < n_dsc ? loff : 0u, st + 8192 + 16384);
     };
     // (a wave waits for its own loads, so it counts what it issued per stage)
     const int mine = (have_x ? 1 : 0) + (have_w0 ? 1 : 0) + (have_w1 ? 1 : 0) + (wid == 0 ? 1 : 0);
@@ -2007,13 +2012,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // instructions are in flight while the vector unit scales an earlier one
     auto multiply = [&](int kb) {
         const lds_char * st = (const lds_char *) qt_smem + (kb % QT_STAGES) * QT_STAGE_BYTES;
-        half8_t  bop[4];
-        float4_t dw[4]; // the scales of the four rows a lane holds of a row tile
+        half8_t bop[4];
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) {
-            bop[rt] = *(const __attribute__((address_space(3))) half8_t *) (st + 8192 + (4 * wr + rt) * 1024 + lane * 16);
-            dw[rt]  = *(const __attribute__((address_space(3))) float4_t *) (st + 8192 + 16384 + (64 * wr + 16 * rt + 4 * j) * 4);
-        }
+        for (int rt = 0; rt < 4; ++rt) bop[rt] = *(const __attribute__((address_space(3))) half8_t *) (st + 8192 + (4 * wr + rt) * 1024 + lane * 16);
+        // the scales of row c in the wave's four row tiles: one load (LDS reads, counted at their full 64 lanes x 16 bytes
+        // whatever they broadcast, are what bounds this loop: four loads here were a quarter of its time)
+        const float4_t dw = *(const __attribute__((address_space(3))) float4_t *) (st + 8192 + 16384 + (64 * wr + 4 * c) * 4);
         half8_t aop[2];
         aop[0] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc) * 1024 + lane * 16);
         if constexpr (FOLD) { // the scale is in the weights: the MFMAs accumulate across blocks
@@ -2021,7 +2025,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             for (int tt = 0; tt < 4; ++tt) {
                 if (tt < 3) aop[(tt + 1) & 1] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc + tt + 1) * 1024 + lane * 16);
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt) acc[rt][tt] = mfma16(bop[rt], aop[tt & 1], acc[rt][tt]);
+                for (int rt = 0; rt < 4; ++rt) acc[rt][tt] = mfma16(aop[tt & 1], bop[rt], acc[rt][tt]);
             }
             return;
         }
@@ -2031,12 +2035,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int tt = i >> 2, rt = i & 3;
             if (i < 16) {
                 if (rt == 0 && tt < 3) aop[(tt + 1) & 1] = *(const __attribute__((address_space(3))) half8_t *) (st + (4 * wc + tt + 1) * 1024 + lane * 16);
-                blk[i % 3] = mfma16(bop[rt], aop[tt & 1], float4_t{0, 0, 0, 0}); // (weights as the row operand: a lane gets 4 consecutive rows of one token)
+                blk[i % 3] = mfma16(aop[tt & 1], bop[rt], float4_t{0, 0, 0, 0});
                 __builtin_amdgcn_sched_barrier(0); // (the MFMA first: the additions below belong to the one two before it)
             }
             if (i >= 2) {
                 const int p = i - 2;
-                acc[p & 3][p >> 2] += blk[p % 3] * dw[p & 3];
+                acc[p & 3][p >> 2] += blk[p % 3] * dw[p & 3]; // (one scale per lane: the weights are the MFMA's column operand, lane c = row c)
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -2051,67 +2055,87 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         multiply(kb);
     }
 
-    // lane (j, c), tile (rt, tt), register r: token tok0 + 16 tt + c, virtual row 16 (rt0 + 4 wr + rt) + 4 j + r:
-    // four consecutive elements of a row of dst
+    // lane (j, c), tile (rt, tt), register r: token tok0 + 16 tt + 4 j + r, virtual row 16 (rt0 + 4 wr + rt) + c
     const int64_t tok0 = (int64_t) ty * QT_TOKS + 64 * wc;
     char * db = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
-    const bool vec = a.M % 4 == 0 && ((uintptr_t) db | a.nb1) % 16 == 0; // uniform
-    if constexpr (DUAL) {
-        // tile pair (2p, 2p + 1) holds gate and up of rows 16 (rt0 / 2 + 2 wr + p) + 4 j + r
+    // A tile inside the matrix stores without tests, at a uniform base plus one 32-bit lane offset (the launcher checks the
+    // range): computed per element in 64-bit arithmetic, the addresses of a tile's 64 stores per lane were a fifth of the
+    // kernel's vector instructions.
+    const bool inside = (int64_t) (ty + 1) * QT_TOKS <= a.N && (int64_t) (tx + 1) * QT_ROWS <= (DUAL ? 2 * a.M : a.M); // uniform
+    if (inside) {
+        const int64_t  row0 = DUAL ? 16 * ((int64_t) (rt0 >> 1) + 2 * wr) : 16 * ((int64_t) rt0 + 4 * wr);
+        char *         tb   = db + (uint64_t) tok0 * a.nb1 + (uint64_t) row0 * 4;
+        const uint32_t lo   = (uint32_t) ((uint64_t) (4 * j) * a.nb1 + (uint64_t) c * 4);
+        if constexpr (DUAL) {
 #pragma unroll
-        for (int p2 = 0; p2 < 2; ++p2) {
-            const int64_t row = 16 * ((int64_t) (rt0 >> 1) + 2 * wr + p2) + 4 * j;
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
-                const int64_t tok = tok0 + 16 * tt + c;
-                if (tok >= a.N) continue;
-                float4_t v;
+            for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
-                    v[r] = (g / (1.0f + expf(-g))) * u;
-                }
-                float * pd = (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4);
-                if (vec && row + 3 < a.M) __builtin_nontemporal_store(v, (float4_t *) pd);
-                else {
+                    char * tr = tb + (uint64_t) (16 * tt + r) * a.nb1; // uniform
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) if (row + r < a.M) pd[r] = v[r];
+                    for (int p2 = 0; p2 < 2; ++p2) {
+                        const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
+                        __builtin_nontemporal_store((g / (1.0f + expf(-g))) * u, (float *) (tr + 64 * p2 + lo));
+                    }
                 }
+            return;
+        } else {
+            if (a.res) {
+                const char *   rb  = a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 + (uint64_t) tok0 * a.rnb1 + (uint64_t) row0 * 4;
+                const uint32_t rlo = (uint32_t) ((uint64_t) (4 * j) * a.rnb1 + (uint64_t) c * 4);
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const char * rr = rb + (uint64_t) (16 * tt + r) * a.rnb1; // uniform
+#pragma unroll
+                        for (int rt = 0; rt < 4; ++rt) acc[rt][tt][r] = scaled_residual(acc[rt][tt][r], a.res_scale, *(const float *) (rr + 64 * rt + rlo));
+                    }
             }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    char * tr = tb + (uint64_t) (16 * tt + r) * a.nb1; // uniform
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt) __builtin_nontemporal_store(acc[rt][tt][r], (float *) (tr + 64 * rt + lo));
+                }
+            return;
+        }
+    }
+    if constexpr (DUAL) {
+        // tile pair (2p, 2p + 1) holds gate and up of row 16 (rt0 / 2 + 2 wr + p) + c
+#pragma unroll
+        for (int p2 = 0; p2 < 2; ++p2) {
+            const int64_t row = 16 * ((int64_t) (rt0 >> 1) + 2 * wr + p2) + c;
+            if (row >= a.M) continue;
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t tok = tok0 + 16 * tt + 4 * j + r;
+                    const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
+                    if (tok < a.N) __builtin_nontemporal_store((g / (1.0f + expf(-g))) * u, (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4));
+                }
         }
         return;
     }
     const bool   residual = a.res != nullptr; // uniform
     const char * rbase    = residual ? a.res + (uint64_t) i12 * a.rnb2 + (uint64_t) i13 * a.rnb3 : nullptr;
-    const bool   rvec     = residual && ((uintptr_t) rbase | a.rnb1) % 16 == 0;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
-        const int64_t row = 16 * ((int64_t) rt0 + 4 * wr + rt) + 4 * j;
+        const int64_t row = 16 * ((int64_t) rt0 + 4 * wr + rt) + c;
+        if (row >= a.M) continue;
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            const int64_t tok = tok0 + 16 * tt + c;
-            if (tok >= a.N) continue;
-            float4_t v = acc[rt][tt];
-            float * pd = (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4);
-            if (vec && row + 3 < a.M) {
-                if (residual) {
-                    const float * pr = (const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) row * 4);
-                    float4_t rv;
-                    if (rvec) rv = *(const float4_t *) pr; else rv = float4_t{pr[0], pr[1], pr[2], pr[3]};
+        for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) v[r] = scaled_residual(v[r], a.res_scale, rv[r]);
-                }
-                __builtin_nontemporal_store(v, (float4_t *) pd);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (row + r < a.M) {
-                        float x = v[r];
-                        if (residual) x = scaled_residual(x, a.res_scale, *(const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) (row + r) * 4));
-                        pd[r] = x;
-                    }
+            for (int r = 0; r < 4; ++r) {
+                const int64_t tok = tok0 + 16 * tt + 4 * j + r;
+                if (tok >= a.N) continue;
+                float v = acc[rt][tt][r];
+                if (residual) v = scaled_residual(v, a.res_scale, *(const float *) (rbase + (uint64_t) tok * a.rnb1 + (uint64_t) row * 4));
+                __builtin_nontemporal_store(v, (float *) (db + (uint64_t) tok * a.nb1 + (uint64_t) row * 4));
             }
-        }
     }
 }
 
@@ -2123,6 +2147,8 @@ bool gemm_q8t_on() { const char * e = getenv("VX_GEMM_Q8T"); return !(e && atoi(
 // 1024 tokens -- below that the two passes in front cost more than they save
 bool gemm_q8t_takes(const mm_args & a, int nbatch, bool dual) {
     const int64_t MV = dual ? 2 * a.M : a.M;
+    // (32-bit lane offsets inside a tile: the 128 tokens of dst and of a residual)
+    if ((uint64_t) 128 * a.nb1 + 1024 >= (1ull << 32) || (a.res && (uint64_t) 128 * a.rnb1 + 1024 >= (1ull << 32))) return false;
     return gemm_q8t_on() && a.K % 32 == 0 && (!dual || a.M % 16 == 0) && MV >= 1024 && a.N >= 1024 && a.x_aligned && (nbatch == 1 || (a.r2 == a.ne12 && a.r3 * a.ne12 == nbatch)) &&
            a.K < (1ll << 24) && nbatch <= 65535;
 }
@@ -2139,7 +2165,7 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     q.fold  = fold;
     const int64_t MV = DUAL ? 2 * a.M : a.M;
     q.n_rt = (int) ((MV + 15) / 16); q.n_tt = (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
-    const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * q.n_rt * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
+    const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * ((q.n_rt + 3) & ~3) * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
     const size_t xt_bytes = (size_t) nbatch * q.n_kb * q.n_tt * 1024;
     void * ws = nullptr;
     if ((t_ws_status = vx_workspace(st, a.ws_offset + wt_bytes + wd_bytes + xt_bytes, &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
