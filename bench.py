@@ -599,7 +599,7 @@ PROFILE_RUNS = [
     ("prefill_attn_cfg5_T4096_B1", "prefill1", "Prefill attention, one sequence of 4096 tokens, 16 query / 2 KV heads, head_dim 64",
      [("sq1", SQ_SET_1), ("sq2", SQ_SET_2)], "pf_"),
     ("mul_mat_q8_0_4096x1024x16384", "gemm", "Q8_0 MUL_MAT, 4096 rows x K 1024 x 16384 tokens (the gate/up projection of 16 x 1024 prefill tokens)",
-     [("sq1", SQ_SET_1), ("sq2", SQ_SET_2), ("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")], "gemm|mm_"),
+     [("sq1", SQ_SET_1), ("sq2", SQ_SET_2), ("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")], "gemm|mm_|qt_"),
     ("backbone_decode_cfg4", "backbone", "Backbone decode step, 24 layers, batch 2, Q8_0 weights, f16 KV cache at ~520 keys (BASELINE config 4)", [], ""),
     ("backbone_decode_cfg5", "backbone16", "Backbone stack at BASELINE config 5 (batch 16, f16 KV 4096 -> 8192, prefill 16 x 4096)", [], ""),
     ("cfm_solve_cfg3", "cfm", "One UnifiedCFM solve of one request (10 Euler steps, CFG pair as one 14-token sequence, 4 LocDiT layers; BASELINE config 3)", [], ""),

@@ -2139,17 +2139,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
 }
 
-// VX_GEMM_Q8T=0 keeps these products on gemm_lds_kernel (read on every call: a product of this size takes a hundred
-// microseconds, and a test compares the two in one process)
-bool gemm_q8t_on() { const char * e = getenv("VX_GEMM_Q8T"); return !(e && atoi(e) == 0); }
+// VX_GEMM_Q8T=0 keeps these products on gemm_lds_kernel, 2 sends every shape the kernel can take to it, however few its
+// tiles (read on every call: a product of this size takes a hundred microseconds, and a test compares the two kernels in
+// one process)
+int gemm_q8t_mode() { const char * e = getenv("VX_GEMM_Q8T"); return e ? atoi(e) : 1; }
 
 // the shapes the pre-tiled kernel takes: one weight matrix for every batch entry, at least 1024 (virtual) rows and
-// 1024 tokens -- below that the two passes in front cost more than they save
+// 1024 tokens -- below that the two passes in front cost more than they save -- and two tiles of 256 x 128 or more per
+// compute unit (the 2 x 512-token prefill of a 24-layer stack is 32 to 256 such tiles a product: 4.6 ms on the smaller
+// tiles of gemm_lds_kernel and its K cut, 7.2 ms here)
 bool gemm_q8t_takes(const mm_args & a, int nbatch, bool dual) {
     const int64_t MV = dual ? 2 * a.M : a.M;
+    const int mode = gemm_q8t_mode();
+    if (mode == 0 || (mode != 2 && ((MV + QT_ROWS - 1) / QT_ROWS) * ((a.N + QT_TOKS - 1) / QT_TOKS) * nbatch < 512)) return false;
     // (32-bit lane offsets inside a tile: the 128 tokens of dst and of a residual)
     if ((uint64_t) 128 * a.nb1 + 1024 >= (1ull << 32) || (a.res && (uint64_t) 128 * a.rnb1 + 1024 >= (1ull << 32))) return false;
-    return gemm_q8t_on() && a.K % 32 == 0 && (!dual || a.M % 16 == 0) && MV >= 1024 && a.N >= 1024 && a.x_aligned && (nbatch == 1 || (a.r2 == a.ne12 && a.r3 * a.ne12 == nbatch)) &&
+    return a.K % 32 == 0 && (!dual || a.M % 16 == 0) && MV >= 1024 && a.N >= 1024 && a.x_aligned && (nbatch == 1 || (a.r2 == a.ne12 && a.r3 * a.ne12 == nbatch)) &&
            a.K < (1ll << 24) && nbatch <= 65535;
 }
 
