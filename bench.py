@@ -535,6 +535,9 @@ def load_peaks():
     lib.vxp_mfma_f16_flop.argtypes = [C.c_int, C.c_int]
     lib.vxp_mfma_f16_flop.restype = C.c_double
     lib.vxp_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.vxp_coexec.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.vxp_lds_read.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.vxp_fill_rate.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p]
     return lib
 
 
@@ -576,7 +579,28 @@ def peaks_bench(timer):
             s_bar = timer.run(one, iters=5, warmup=2)
             assert int(flags[1].item()) == 0, "a work-group gave up waiting at the grid barrier"
             barrier[f"{per_cu * cus}_work_groups_{'release_acquire' if ordered else 'relaxed'}_us"] = (s_bar - empty) / rounds * 1e6
-    return {"grid_barrier": barrier,
+    # two instruction streams on one SIMD (waves 0-3 and 4-7 of an 8-wave work-group): alone and in pairs
+    names = {1: "mfma", 2: "fma", 3: "exp"}
+    coexec = {}
+    it_ = 20000
+    for ra, rb in ((1, 0), (2, 0), (3, 0), (1, 1), (2, 2), (3, 3), (1, 2), (1, 3), (2, 3)):
+        s_co = timer.run(lambda: lib.vxp_coexec(cus, ra, rb, it_, fsink.data_ptr(), st()), iters=3, warmup=1)
+        coexec[names[ra] + ("_alone" if rb == 0 else "_with_" + names[rb])] = s_co / it_ * 1e9
+    coexec["unit"] = ("ns per iteration of a wave: mfma = 4 independent v_mfma_f32_32x32x16_f16 (128 cycles), fma = 32 v_fma_f32 in 8 chains, "
+                      "exp = 16 v_exp_f32 + 16 v_sub_f32; a pair that ran side by side would take the longer of its two times alone")
+    # LDS read rate per compute unit (16-byte reads, 8 per iteration and wave) and a compute unit's fill rate with all pulling
+    lds = {}
+    lit = 4000
+    for waves in (4, 8, 16):
+        for same in (0, 1):
+            s_l = timer.run(lambda: lib.vxp_lds_read(cus, waves, lit, same, fsink.data_ptr(), st()), iters=3, warmup=1)
+            lds[f"{waves}_waves_{'one_address_per_16_lanes' if same else 'lane_contiguous'}_bytes_per_ns_per_cu"] = lit * 8 * waves * 1024 / (s_l * 1e9)
+    fill = {}
+    per_wg = 8 << 20
+    for region in (2 << 20, 16 << 20, 64 << 20):
+        s_f = timer.run(lambda: lib.vxp_fill_rate(big.data_ptr(), region, per_wg, cus, sink.data_ptr(), st()), iters=3, warmup=1)
+        fill[f"region_{region >> 20}MiB_GB/s_per_cu"] = per_wg / s_f / 1e9
+    return {"grid_barrier": barrier, "two_streams_on_one_simd": coexec, "lds_read_16_bytes_per_lane": lds, "fill_rate_all_compute_units_pulling": fill,
             "hbm_stream_read_1GiB_GB/s": big.numel() / s_big / 1e9,
             "hbm_stream_read_64MiB_per_launch_GB/s": chunk / s_chunk / 1e9, "hbm_stream_read_64MiB_us": s_chunk * 1e6,
             "mfma_f16_TFLOP/s": lib.vxp_mfma_f16_flop(blocks, iters) / s_mfma / 1e12,

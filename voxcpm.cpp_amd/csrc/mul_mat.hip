@@ -1851,21 +1851,21 @@ vx_status take_ws_status() { const vx_status rc = t_ws_status; t_ws_status = VX_
 // arithmetic) and reads an operand with one conflict-free 16-byte LDS load.  The arithmetic is the kernel above's: a 32-wide
 // partial product per block from one MFMA, scaled by the block's d in fp32 and added -- the same bits.
 //
-// Work-group: 8 waves, 256 rows x 128 tokens (a wave: 64 x 64 = 4 x 4 MFMA tiles), three stages of one k block
-// (16 KB of weights, 8 KB of activations, 1 KB of scales), one barrier a block, two work-groups to a compute unit (75 KB
-// of LDS and 128 registers each): everything a wave does besides its MFMAs -- issuing the direct loads (a hundred
+// Work-group: 8 waves, 256 rows x 128 tokens (a wave: 64 x 64 = 4 x 4 MFMA tiles), two stages of one k block
+// (16 KB of weights, 8 KB of activations, 1 KB of scales; a third stage measured 5 % slower), one barrier a block, two
+// work-groups to a compute unit (50 KB of LDS and 128 registers each): everything a wave does besides its MFMAs -- issuing the direct loads (a hundred
 // cycles apiece), the barrier, the operand reads, the 64 scaled additions of a block, the stores at the end -- was
 // measured to add up unhidden with one work-group's waves in step; the second work-group's waves fill those gaps.
 // The weights are the MFMA's column operand: lane c holds row c of every row tile and needs one scale per tile, which the
 // weight pass lays out so that a lane's four come with one 16-byte LDS load.
 // Work-groups are dealt to the XCDs in groups of 4 row tiles x 8 token tiles that run side by side on one XCD's 32
 // compute units and share its L2.
-// Measured on 4096 rows x K 1024 x 16384 tokens: 210 us with both passes (11 and 21 us) against 300 us for the kernel
-// above.  What bounds it: 16-byte LDS reads deliver about 64 bytes a cycle per compute unit, counted at their full 64
-// lanes x 16 bytes whatever they broadcast (9 KB per wave and block: 148 us for this product), and a SIMD's vector unit
-// and matrix core do not run side by side (16 + 4 x 4.75 cycles per MFMA with its four scaled additions: 143 us); the
-// kernel runs at 175 us.
-constexpr int QT_ROWS = 256, QT_TOKS = 128, QT_STAGES = 3;
+// Measured on 4096 rows x K 1024 x 16384 tokens: 205 us with both passes (11 and 21 us) against 300 us for the kernel
+// above; the kernel alone 167 us.  Per compute unit and block (two work-groups, 16 waves) that is 2600 cycles against
+// 1024 of MFMAs and 1216 of scaled additions per SIMD (which do run side by side), 600 of LDS reads and some 1100 to
+// bring 50 KB in from L2: no single unit bounds it; what is left is the waves of a work-group meeting at a barrier every
+// block and the issue of the direct loads (a fifth of the time when they are taken out).
+constexpr int QT_ROWS = 256, QT_TOKS = 128, QT_STAGES = 2;
 constexpr int QT_STAGE_BYTES = (QT_ROWS + QT_TOKS) / 16 * 1024 + QT_ROWS * 4;
 constexpr size_t QT_LDS = (size_t) QT_STAGES * QT_STAGE_BYTES;
 

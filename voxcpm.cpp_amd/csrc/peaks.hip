@@ -1,7 +1,8 @@
 // peaks.hip -- what this GPU actually delivers, measured with the simplest kernels there are: a streaming
-// read of a large buffer (HBM), a loop of independent matrix-core instructions (MFMA), and a barrier across
+// read of a large buffer (HBM), a loop of independent matrix-core instructions (MFMA), a barrier across
 // all work-groups of a resident grid (what a kernel that stays on the chip for a whole layer would pay where
-// launches now follow each other).  The benchmark reports its rooflines against the published peaks AND
+// launches now follow each other), and pairs of instruction streams on one SIMD (whether matrix and vector
+// work run side by side).  The benchmark reports its rooflines against the published peaks AND
 // against these; nothing in the product path uses this file.  Built as its own small library (libvx_peaks.so).
 #include <hip/hip_runtime.h>
 
@@ -85,6 +86,106 @@ __global__ __launch_bounds__(256) void grid_barrier_kernel(unsigned * __restrict
     }
 }
 
+// Do a SIMD's matrix core and its vector unit run side by side?  A work-group of 8 waves puts two waves on every SIMD;
+// waves 0-3 run role_a, waves 4-7 role_b: 0 idle, 1 four independent v_mfma_f32_32x32x16_f16 per iteration (128 cycles of
+// matrix work), 2 thirty-two v_fma_f32 in eight independent chains, 3 sixteen v_exp_f32 (each followed by a v_sub_f32 that
+// keeps the argument in range).  Times of the pairs against the times of the roles alone answer the question.
+__device__ __forceinline__ void coexec_mfma(int iters, float * sink) {
+    f16x8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { a[i] = (_Float16) (0.001f * (float) ((threadIdx.x + i) & 7)); b[i] = (_Float16) (0.002f * (float) ((threadIdx.x + 3 * i) & 7)); }
+    f32x16 acc[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[k][i] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[k], 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s += acc[k][i];
+    if (s == 123.456f) sink[threadIdx.x] = s;
+}
+__device__ __forceinline__ void coexec_fma(int iters, float * sink) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.5f + (float) threadIdx.x * 1e-3f + (float) i;
+    const float m = 0.999f, c = 1e-3f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[i]) : "v"(m), "v"(c));
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += v[i];
+    if (s == 123.456f) sink[threadIdx.x] = s;
+}
+__device__ __forceinline__ void coexec_exp(int iters, float * sink) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = -0.5f - (float) threadIdx.x * 1e-3f - (float) i;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) asm volatile("v_exp_f32 %0, %0\n\tv_sub_f32 %0, 0, %0" : "+v"(v[i]));
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += v[i];
+    if (s == 123.456f) sink[threadIdx.x] = s;
+}
+__global__ __launch_bounds__(512) void coexec_kernel(int role_a, int role_b, int iters, float * __restrict__ sink) {
+    const int role = (threadIdx.x >> 8) ? role_b : role_a; // uniform per wave
+    if (role == 1) coexec_mfma(iters, sink);
+    else if (role == 2) coexec_fma(iters, sink);
+    else if (role == 3) coexec_exp(iters, sink);
+}
+
+// LDS read rate of a compute unit: every wave of a work-group issues 16-byte reads at lane-contiguous addresses (or, with
+// `same`, one address per 16 lanes) from a 64 KB array, eight per iteration; the address moves behind an opaque
+// constraint so that the reads stay in the loop.
+__global__ __launch_bounds__(1024) void lds_read_kernel(int iters, int same, float * __restrict__ sink) {
+    __shared__ __attribute__((aligned(16))) char lds[65536];
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) ((float *) lds)[i] = (float) i;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int base = (wave * 4096 + (same ? (lane >> 4) * 16 : lane * 16)) & 65535;
+    f32x4 acc = {0, 0, 0, 0};
+    for (int it = 0; it < iters; ++it) {
+        asm volatile("" : "+v"(base));
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += *(const f32x4 *) (lds + ((base + u * 1024) & 65535));
+    }
+    if (acc[0] + acc[1] + acc[2] + acc[3] == 123.456f) sink[threadIdx.x] = acc[0];
+}
+
+// Fill rate of a compute unit with every compute unit pulling: work-groups of 8 waves re-read a region of `region`
+// bytes (2 MiB: an XCD's L2 holds it; 16 MiB: the memory-side cache does), each wave 1 KB per load, 8 loads in flight,
+// the work-groups starting at scattered places.
+__global__ __launch_bounds__(512) void fill_rate_kernel(const char * __restrict__ src, size_t region, size_t per_wg, int * __restrict__ sink) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const size_t per_wave = per_wg / 8;
+    size_t pos = ((size_t) blockIdx.x * 7919 * 1024 + (size_t) wid * per_wave) % region;
+    const int n_kb = (int) (per_wave / 1024);
+    i32x4 acc = {0, 0, 0, 0};
+    for (int i = 0; i < n_kb; i += 8) {
+        i32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = *(const i32x4 *) (src + (pos + (size_t) u * 1024) % region + lane * 16);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u];
+        pos = (pos + 8 * 1024) % region;
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a5a5a5a) sink[blockIdx.x] = acc[0];
+}
+
 } // namespace
 
 extern "C" {
@@ -123,6 +224,30 @@ __attribute__((visibility("default"))) int vxp_grid_barrier(int blocks, int roun
     if (blocks > 4 * p.multiProcessorCount) return 1;
     if (ordered) grid_barrier_kernel<true><<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>(counter, rounds, 1u << 22, failed);
     else         grid_barrier_kernel<false><<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>(counter, rounds, 1u << 22, failed);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+
+// one work-group of 8 waves per compute unit slot (`blocks` of them), `iters` iterations of the two roles (see coexec_kernel);
+// sink: 512 floats
+__attribute__((visibility("default"))) int vxp_coexec(int blocks, int role_a, int role_b, int iters, float * sink, void * stream) {
+    if (!sink || blocks <= 0 || iters <= 0 || role_a < 0 || role_a > 3 || role_b < 0 || role_b > 3) return 1;
+    coexec_kernel<<<dim3((unsigned) blocks), dim3(512), 0, (hipStream_t) stream>>>(role_a, role_b, iters, sink);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+
+// `blocks` work-groups of `waves` waves (1 .. 16), `iters` iterations of eight 16-byte LDS reads per wave; sink: 1024 floats
+__attribute__((visibility("default"))) int vxp_lds_read(int blocks, int waves, int iters, int same, float * sink, void * stream) {
+    if (!sink || blocks <= 0 || waves < 1 || waves > 16 || iters <= 0) return 1;
+    lds_read_kernel<<<dim3((unsigned) blocks), dim3(64 * waves), 0, (hipStream_t) stream>>>(iters, same, sink);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+// `blocks` work-groups of 8 waves each read `per_wg` bytes (a multiple of 64 KiB) of the first `region` bytes of src
+// (region a multiple of 8 KiB, at most the buffer's size); sink: `blocks` ints
+__attribute__((visibility("default"))) int vxp_fill_rate(const void * src, size_t region, size_t per_wg, int blocks, int * sink, void * stream) {
+    if (!src || !sink || blocks <= 0 || region == 0 || region % 8192 || per_wg == 0 || per_wg % 65536) return 1;
+    fill_rate_kernel<<<dim3((unsigned) blocks), dim3(512), 0, (hipStream_t) stream>>>((const char *) src, region, per_wg, sink);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
