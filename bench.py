@@ -339,10 +339,29 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
         # (src/voxcpm.cpp:485-513), laid out, its inputs uploaded, computed, the hidden state fetched -- wall clock of the loop
         plug.ggml_backend_gfx950_set_graph_replay(1)
         n_loop = min(256, steps)
+        patch_before = plug.ggml_backend_gfx950_set_graph_patch(0)   # the default: every step launched node group by node group
         _, lp = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop)
+        plug.ggml_backend_gfx950_host_ns.restype = C.c_longlong
+        host0 = [plug.ggml_backend_gfx950_host_ns(i) / 1e3 for i in (0, 1)]
         _, lpo = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop, overlap=True)
+        plug.ggml_backend_gfx950_set_graph_patch(1)   # a step as an earlier step's recording with the changed arguments set on its nodes
+        n_p0 = plug.ggml_backend_gfx950_patched_replays()
+        _, lp1 = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop)
+        n_p1 = plug.ggml_backend_gfx950_patched_replays()
+        host1 = [plug.ggml_backend_gfx950_host_ns(i) / 1e3 for i in (0, 1)]
+        changed = plug.ggml_backend_gfx950_last_patched()
+        _, lpo1 = reflib.ref_backbone_decode_loop(x1.cpu().numpy(), prefill, n_loop, overlap=True)
+        plug.ggml_backend_gfx950_set_graph_patch(patch_before)
         ref.rh_bb_free()
         consecutive = {"decode_steps_per_s": 1.0 / lp["wall"], "ms_per_step": lp["wall"] * 1e3, "graph_compute_ms": lp["graph_compute"] * 1e3,
+                       "host_us_last_step_analysis_and_issue": host0,
+                       "steps_as_patched_recordings_GGML_GFX950_GRAPH_PATCH=1": {
+                           "decode_steps_per_s": 1.0 / lp1["wall"], "ms_per_step": lp1["wall"] * 1e3, "graph_compute_ms": lp1["graph_compute"] * 1e3,
+                           "next_graph_built_under_the_running_one_decode_steps_per_s": 1.0 / lpo1["wall"],
+                           "host_us_last_step_analysis_and_comparison": host1, "steps_run_this_way": n_p1 - n_p0,
+                           "kernels_whose_arguments_changed_in_the_last_step": changed,
+                           "how": "each step's node-by-node pass is made against a recording of an earlier step (nothing launched, differing arguments "
+                                  "set with hipGraphExecKernelNodeSetParams), then one hipGraphLaunch: the host pass runs before the GPU starts"},
                        "graph_build_and_layout_ms": lp["build"] * 1e3, "steps": n_loop, "from_kv_length": prefill,
                        "nodes_at_another_address_than_the_step_before": lp["moved"],
                        "how": "the drop-in figure: every step's graph rebuilt for its position, ggml_backend_graph_compute (synchronous), "
@@ -802,7 +821,7 @@ def main():
         print(json.dumps({"profile": "cfg3_cfm_solve_8_requests_through_plugin", **cfm_requests_bench(pkg, 1, False)}))
         return
     if args.profile == "backbone":  # config 4 decode steps (f16 cache)
-        print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=16, kv_f16=True, plugin_reps=5)}))
+        print(json.dumps({"profile": "cfg4_backbone_24layers_b2", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, steps=128, kv_f16=True, plugin_reps=5)}))
         return
     if args.profile == "backbone16":  # config 5 decode steps (f16 cache)
         print(json.dumps({"profile": "cfg5_backbone_24layers_b16", **backbone_bench(pkg, timer, torch.cuda.Stream(), 1, False, batch=16, prefill=4096,

@@ -94,6 +94,21 @@ VX_API vx_status    vx_graph_begin(vx_stream stream);
 VX_API vx_status    vx_graph_end(vx_stream stream, vx_graph * graph);   /* *graph = NULL when nothing usable was recorded */
 VX_API vx_status    vx_graph_launch(vx_graph graph, vx_stream stream);
 VX_API vx_status    vx_graph_destroy(vx_graph graph);
+/* Running a recording again with other arguments.  A decode step's graph differs from the previous step's only in what
+ * follows from the position (the key count of the attention launches, the cache slot that is written: the reference's
+ * src/minicpm.cpp:393-470 builds them from n_past), so its launches are the recorded ones with a few arguments changed.
+ * Between patch_begin and patch_end every vx_* operator call of the calling thread launches nothing: each launch it
+ * would have made is compared, in order, with the recording's, and where the grid, the block, the LDS size or the
+ * argument bytes differ they are set on the recorded graph's node.  patch_end returns VX_OK when the calls made the same
+ * kernels in the same order and number as the recording (*patched = how many nodes were changed): vx_graph_launch then
+ * runs the graph with the new arguments.  VX_ERR_UNSUPPORTED means they did not: the graph's arguments are then a
+ * mixture, destroy it and run the calls again normally.  patch_begin waits for the graph's previous launch to finish
+ * (its arguments must not change under it): a caller that wants the host to run ahead of the GPU alternates between two
+ * recordings.  vx_graph_patchable says whether a recording can be used this way (all of its launches are kernels of this
+ * library).  No counterpart in ggml-cpu. */
+VX_API int          vx_graph_patchable(vx_graph graph);
+VX_API vx_status    vx_graph_patch_begin(vx_graph graph);
+VX_API vx_status    vx_graph_patch_end(vx_graph graph, int * patched);
 
 /* ---- GGML_OP_RMS_NORM -------------------------------------------------------------------
  * replaces ggml_compute_forward_rms_norm (ggml/src/ggml-cpu/ops.cpp:3710-3777).

@@ -460,7 +460,9 @@ def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
     prefill of 300 tokens (so the key ranges are cut and merged, and the cut changes along the way) through the plugin:
     against ggml-cpu on the same loop, against the same steps computed one by one through rh_bb_forward (the same
     launches: bit for bit, the caches included), and with the next step's graph built while the device computes the
-    current one (the same launches again)."""
+    current one (the same launches again).  All of that with every step launched node by node; then the same loops with
+    the steps run as patched recordings (from the fourth step on a step is the recorded HIP graph of an earlier one with
+    the arguments that follow from the position set on its nodes): the same bits again, the caches included."""
     import ctypes
     T0, N = 300, 72
     max_len = T0 + N + 8
@@ -478,8 +480,11 @@ def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
                 out.append(buf)
         return out
 
-    def run(device, how):
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+
+    def run(device, how, patch=False):
         assert ref.rh_use_device(device, 8, 0) == 0
+        patch_before = plugin.ggml_backend_gfx950_set_graph_patch(int(patch))
         reflib.ref_backbone_create(params, max_len, BATCH, use_mup=True, kv_f16=kv_f16)
         try:
             reflib.ref_backbone_forward(xp, 0, reflib.causal_mask(T0, T0))
@@ -492,12 +497,13 @@ def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
             return out, caches(), info
         finally:
             ref.rh_bb_free()
+            plugin.ggml_backend_gfx950_set_graph_patch(patch_before)
             assert ref.rh_use_device(b"CPU", 8, 0) == 0
 
     assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
     cpu, cpu_cache, _ = run(b"CPU", "loop")
     loop, loop_cache, info = run(b"GFX950_0", "loop")
-    launches = ctypes.CDLL(gpu.PLUGIN_PATH).ggml_backend_gfx950_last_launches()
+    launches = plugin.ggml_backend_gfx950_last_launches()
     print(f"consecutive decode steps, kv_f16={kv_f16}: {N} steps, {info['n_nodes']} nodes and {launches} launches a step, "
           f"{info['moved'] * 100:.0f} % of the nodes at another address than the step before", flush=True)
     assert launches == 5 * N_LAYER + 1
@@ -516,6 +522,17 @@ def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
     assert np.array_equal(loop, over), "building the next graph under the running one changed a result"
     for a, b in zip(loop_cache, over_cache):
         assert np.array_equal(a, b), "cache contents differ (overlapped)"
+    for how in ("loop", "overlapped", "one by one"):
+        n0 = plugin.ggml_backend_gfx950_patched_replays()
+        out, cache, _ = run(b"GFX950_0", how, patch=True)
+        n1 = plugin.ggml_backend_gfx950_patched_replays()
+        print(f"   steps as patched recordings ({how}): {n1 - n0} of {N} steps, {plugin.ggml_backend_gfx950_last_patched()} kernels' "
+              f"arguments changed in the last one", flush=True)
+        assert n1 - n0 >= N - 12, "the steps were not run as patched recordings"
+        assert plugin.ggml_backend_gfx950_last_launches() == launches
+        assert np.array_equal(loop, out), f"a patched recording gave another result than node-by-node launches ({how})"
+        for a, b in zip(loop_cache, cache):
+            assert np.array_equal(a, b), f"cache contents differ (patched recordings, {how})"
 
 
 def test_plugin_replays_a_recurring_graph(gpu, ref):

@@ -92,3 +92,70 @@ def test_workspace_growth_during_capture_is_refused(gpu):
         graph2.replay()
         side.synchronize()
         assert float(out.abs().max()) == 0.0
+
+
+def test_a_recording_runs_again_with_other_arguments(gpu):
+    """vx_graph_patch_begin/_end: the calls of a decode step made against a recording launch nothing, the recorded graph
+    then runs with their arguments.  A step with a growing key count, another query and alternating outputs, each run
+    checked against the same calls made directly, with direct work between the runs; then a call sequence with another
+    kernel in it, which the comparison must refuse."""
+    import ctypes as C
+    import torch
+    lib = gpu.lib()
+    side = torch.cuda.Stream()
+    B, Hq, Hkv, D, cap = 2, 16, 2, 64, 1400
+    g = lambda *tag: rng("patch", *tag)
+    kc = torch.from_numpy(g("k").standard_normal((B, Hkv, cap, D)).astype(np.float16)).cuda()
+    vc = torch.from_numpy(g("v").standard_normal((B, Hkv, cap, D)).astype(np.float16)).cuda()
+    w = torch.from_numpy(g("w").standard_normal(Hq * D).astype(np.float32)).cuda()
+    qs = [torch.from_numpy(g("q", i).standard_normal((B, Hq, 1, D)).astype(np.float32)).cuda() for i in range(3)]
+    outs = [torch.zeros((B, 1, Hq, D), device="cuda") for _ in range(2)]
+    normed = [torch.zeros((B, 1, Hq * D), device="cuda") for _ in range(2)]
+    torch.cuda.synchronize()
+
+    def step(L, i):   # attention over the first L keys, then a norm of its output
+        gpu.flash_attn_ext(qs[i % 3], kc[:, :, :L], vc[:, :, :L], None, 0.125, out=outs[i % 2])
+        gpu.rms_norm(outs[i % 2].view(B, 1, Hq * D), 1e-5, out=normed[i % 2])
+
+    with torch.cuda.stream(side):
+        gpu.check(lib.vx_workspace_reserve(side.cuda_stream, 8 << 20), "reserve")
+        step(900, 0)
+        side.synchronize()
+        gpu.check(lib.vx_graph_begin(side.cuda_stream), "begin")
+        step(900, 0)
+        rec = C.c_void_p()
+        gpu.check(lib.vx_graph_end(side.cuda_stream, C.byref(rec)), "end")
+        assert rec.value and lib.vx_graph_patchable(rec) == 1
+        changed = C.c_int()
+        for i, L in enumerate([900, 901, 902, 1023, 1024, 1025, 1399, 64, 1]):
+            say(f"recording run again for {L} keys")
+            step(L, i)   # directly
+            side.synchronize()
+            want = (outs[i % 2].clone(), normed[i % 2].clone())
+            outs[i % 2].zero_(); normed[i % 2].zero_()
+            gpu.check(lib.vx_graph_patch_begin(rec), "patch_begin")
+            step(L, i)   # compared with the recording: nothing runs
+            side.synchronize()
+            assert float(outs[i % 2].abs().max()) == 0.0, "a call made during the comparison ran"
+            rc = lib.vx_graph_patch_end(rec, C.byref(changed))
+            if rc == 2:  # another kernel for this key count than the recorded one: the recording is of no use for it
+                say(f"   {L} keys take other kernels than the recording's")
+                assert L in (64, 1)
+                gpu.check(lib.vx_graph_destroy(rec), "destroy")
+                gpu.check(lib.vx_graph_begin(side.cuda_stream), "begin")
+                step(L, i)
+                gpu.check(lib.vx_graph_end(side.cuda_stream, C.byref(rec)), "end")
+                assert rec.value and lib.vx_graph_patchable(rec) == 1
+            else:
+                assert rc == 0 and (changed.value >= 1 or i == 0)
+            gpu.check(lib.vx_graph_launch(rec, side.cuda_stream), "launch")
+            side.synchronize()
+            assert torch.equal(outs[i % 2], want[0]) and torch.equal(normed[i % 2], want[1]), L
+        # a different sequence of calls: refused, and the thread launches normally again afterwards
+        gpu.check(lib.vx_graph_patch_begin(rec), "patch_begin")
+        gpu.rms_norm(outs[0].view(B, 1, Hq * D), 1e-5, out=normed[0])
+        assert lib.vx_graph_patch_end(rec, C.byref(changed)) == 2
+        gpu.check(lib.vx_graph_destroy(rec), "destroy")
+        step(900, 0)
+        side.synchronize()
+        assert float(outs[0].abs().max()) > 0.0

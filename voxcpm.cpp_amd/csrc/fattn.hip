@@ -932,7 +932,7 @@ bool fa_dec64_takes(const fa_args & a, int D, bool kv_f32) {
 }
 void launch_dec64(const fa_args & a, hipStream_t st) {
     const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv + (a.has_kvs ? 1 : 0)));
-    fattn_dec64_kernel<<<grid, dim3(64), 0, st>>>(a);
+    vx_launch(fattn_dec64_kernel, grid, dim3(64), 0, st, a);
 }
 
 template <int D, bool KV_F32>
@@ -940,27 +940,27 @@ void launch_cols16(const fa_args & a, hipStream_t st) {
     const dim3 grid((unsigned) a.n_col_tiles, (unsigned) a.n_splits, (unsigned) (a.ne3 * a.Hkv + (a.has_kvs ? 1 : 0))), block(64);
     if constexpr (D == 64 && !KV_F32) {
         if (a.k2 && a.seg2_f32) { // an F16 cache and the step's F32 keys
-            if (a.softcap != 0.0f) fattn_cols16_kernel<D, false, true, true, 2><<<grid, block, 0, st>>>(a);
-            else if (a.mask)       fattn_cols16_kernel<D, false, true, false, 2><<<grid, block, 0, st>>>(a);
-            else                   fattn_cols16_kernel<D, false, false, false, 2><<<grid, block, 0, st>>>(a);
+            if (a.softcap != 0.0f) vx_launch(fattn_cols16_kernel<D, false, true, true, 2>, grid, block, 0, st, a);
+            else if (a.mask)       vx_launch(fattn_cols16_kernel<D, false, true, false, 2>, grid, block, 0, st, a);
+            else                   vx_launch(fattn_cols16_kernel<D, false, false, false, 2>, grid, block, 0, st, a);
             return;
         }
     }
     if (a.k2) {
-        if (a.softcap != 0.0f) fattn_cols16_kernel<D, KV_F32, true, true, 1><<<grid, block, 0, st>>>(a);
-        else if (a.mask)       fattn_cols16_kernel<D, KV_F32, true, false, 1><<<grid, block, 0, st>>>(a);
-        else                   fattn_cols16_kernel<D, KV_F32, false, false, 1><<<grid, block, 0, st>>>(a);
+        if (a.softcap != 0.0f) vx_launch(fattn_cols16_kernel<D, KV_F32, true, true, 1>, grid, block, 0, st, a);
+        else if (a.mask)       vx_launch(fattn_cols16_kernel<D, KV_F32, true, false, 1>, grid, block, 0, st, a);
+        else                   vx_launch(fattn_cols16_kernel<D, KV_F32, false, false, 1>, grid, block, 0, st, a);
         return;
     }
     if (a.softcap != 0.0f) { // rare: always take the masked variant
-        fattn_cols16_kernel<D, KV_F32, true, true, 0><<<grid, block, 0, st>>>(a);
+        vx_launch(fattn_cols16_kernel<D, KV_F32, true, true, 0>, grid, block, 0, st, a);
     } else if (a.n_kv <= 16 && a.n_splits == 1) {
-        if (a.mask) fattn_cols16_kernel<D, KV_F32, true, false, 0, true><<<grid, block, 0, st>>>(a);
-        else        fattn_cols16_kernel<D, KV_F32, false, false, 0, true><<<grid, block, 0, st>>>(a);
+        if (a.mask) vx_launch(fattn_cols16_kernel<D, KV_F32, true, false, 0, true>, grid, block, 0, st, a);
+        else        vx_launch(fattn_cols16_kernel<D, KV_F32, false, false, 0, true>, grid, block, 0, st, a);
     } else if (a.mask) {
-        fattn_cols16_kernel<D, KV_F32, true, false, 0><<<grid, block, 0, st>>>(a);
+        vx_launch(fattn_cols16_kernel<D, KV_F32, true, false, 0>, grid, block, 0, st, a);
     } else {
-        fattn_cols16_kernel<D, KV_F32, false, false, 0><<<grid, block, 0, st>>>(a);
+        vx_launch(fattn_cols16_kernel<D, KV_F32, false, false, 0>, grid, block, 0, st, a);
     }
 }
 
@@ -1245,8 +1245,8 @@ static vx_status fa_run(const vx_tensor * q, const vx_tensor * k, const vx_tenso
     if (a.n_splits > 1) {
         const dim3 grid((unsigned) (a.n_col_tiles * 16), (unsigned) (a.ne3 * a.Hkv));
         const dim3 mblock(64);
-        if (D == 64) fattn_merge_kernel<64><<<grid, mblock, 0, st>>>(a);
-        else         fattn_merge_kernel<128><<<grid, mblock, 0, st>>>(a);
+        if (D == 64) vx_launch(fattn_merge_kernel<64>, grid, mblock, 0, st, a);
+        else         vx_launch(fattn_merge_kernel<128>, grid, mblock, 0, st, a);
         VX_LAUNCH_CHECK();
     }
     return VX_OK;

@@ -712,7 +712,7 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
         ws = (char *) p;
     }
     if (mask) {
-        pf_mask_flags_kernel<<<dim3((unsigned) n_tiles, (unsigned) n_rb, (unsigned) (a.nem2 * a.nem3)), dim3(64), 0, st>>>(
+        vx_launch(pf_mask_flags_kernel, dim3((unsigned) n_tiles, (unsigned) n_rb, (unsigned) (a.nem2 * a.nem3)), dim3(64), 0, st,
             a.mask, a.nbm1, a.nbm2, a.nbm3, a.nem2, n_q, n_kv, RB, n_rb, n_tiles,
             (int) ((uintptr_t) a.mask % 16 == 0 && a.nbm1 % 16 == 0 && a.nbm2 % 16 == 0 && a.nbm3 % 16 == 0), (uint8_t *) ws + bits_bytes,
             (uint8_t *) ws);
@@ -722,7 +722,7 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     }
     if (a.kv_f32) {
         _Float16 * k16 = (_Float16 *) (ws + flag_bytes), * vhi = (_Float16 *) (ws + flag_bytes + plane), * vlo = (_Float16 *) (ws + flag_bytes + 2 * plane);
-        pf_convert_kernel<<<dim3((unsigned) ((n_kv * 8 + 255) / 256), (unsigned) Hkv, (unsigned) k->ne[3]), dim3(256), 0, st>>>(
+        vx_launch(pf_convert_kernel, dim3((unsigned) ((n_kv * 8 + 255) / 256), (unsigned) Hkv, (unsigned) k->ne[3]), dim3(256), 0, st,
             a.k, a.v, a.nbk1, a.nbk2, a.nbk3, a.nbv1, a.nbv2, a.nbv3, n_kv, Hkv, k16, vhi, vlo);
         VX_LAUNCH_CHECK();
         a.k = (const char *) k16; a.v = (const char *) vhi; a.vl = (const char *) vlo;
@@ -730,10 +730,10 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     }
     const dim3 grid((unsigned) (n_rb * n_groups)), block(64 * PF_WAVES);
     if (half_cols) {
-        if (a.kv_f32) pf_kernel<true, 1><<<grid, block, 0, st>>>(a);
-        else          pf_kernel<false, 1><<<grid, block, 0, st>>>(a);
+        if (a.kv_f32) vx_launch(pf_kernel<true, 1>, grid, block, 0, st, a);
+        else          vx_launch(pf_kernel<false, 1>, grid, block, 0, st, a);
     } else {
-        pf_kernel<false, 2><<<grid, block, 0, st>>>(a);
+        vx_launch(pf_kernel<false, 2>, grid, block, 0, st, a);
     }
     VX_LAUNCH_CHECK();
     return VX_OK;

@@ -150,8 +150,8 @@ vx_status ew_launch(ew_args & a, hipStream_t st) {
     a.nchunk    = (a.ne[0] + 256 * V - 1) / (256 * V);
     const int64_t blocks = rows * a.nchunk;
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "elementwise op: launch too large");
-    if (vec) ew_kernel<OP, 4><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
-    else     ew_kernel<OP, 1><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    if (vec) vx_launch(ew_kernel<OP, 4>, dim3((unsigned) blocks), dim3(256), 0, st, a);
+    else     vx_launch(ew_kernel<OP, 1>, dim3((unsigned) blocks), dim3(256), 0, st, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -225,8 +225,8 @@ vx_status cpy_launch(const cpy_args & a, bool vec, hipStream_t st) {
     const int V = vec ? 4 : 1;
     const int64_t blocks = (a.n / V + 255) / 256;
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "cpy: launch too large");
-    if (vec) cpy_kernel<TS, TD, 4><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
-    else     cpy_kernel<TS, TD, 1><<<dim3((unsigned) blocks), dim3(256), 0, st>>>(a);
+    if (vec) vx_launch(cpy_kernel<TS, TD, 4>, dim3((unsigned) blocks), dim3(256), 0, st, a);
+    else     vx_launch(cpy_kernel<TS, TD, 1>, dim3((unsigned) blocks), dim3(256), 0, st, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1276,9 +1276,9 @@ extern "C" vx_status vx_concat(const vx_tensor * src0, const vx_tensor * src1, c
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "concat: launch too large");
     const dim3 grid((unsigned) blocks), block(256);
     hipStream_t st = (hipStream_t) stream;
-    if (vec)          { if (es == 4) concat_kernel<16, 4><<<grid, block, 0, st>>>(a); else concat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
-    else if (es == 4) concat_kernel<4, 4><<<grid, block, 0, st>>>(a);
-    else              concat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    if (vec)          { if (es == 4) vx_launch(concat_kernel<16, 4>, grid, block, 0, st, a); else vx_launch(concat_kernel<16, 2>, grid, block, 0, st, a); }
+    else if (es == 4) vx_launch(concat_kernel<4, 4>, grid, block, 0, st, a);
+    else              vx_launch(concat_kernel<2, 2>, grid, block, 0, st, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1323,8 +1323,8 @@ extern "C" vx_status vx_concat_many(const vx_tensor * const * srcs, const int64_
     for (int q = 0; q < 4; ++q) { a.ne[q] = (uint32_t) dst->ne[q]; a.nbd[q] = dst->nb[q]; }
     a.n = (uint32_t) (vec ? vx_nelements(dst) / 4 : vx_nelements(dst));
     const dim3 grid((a.n + 255) / 256), block(256);
-    if (vec) concat_many_kernel<true><<<grid, block, 0, (hipStream_t) stream>>>(a);
-    else     concat_many_kernel<false><<<grid, block, 0, (hipStream_t) stream>>>(a);
+    if (vec) vx_launch(concat_many_kernel<true>, grid, block, 0, (hipStream_t) stream, a);
+    else     vx_launch(concat_many_kernel<false>, grid, block, 0, (hipStream_t) stream, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1338,7 +1338,7 @@ extern "C" vx_status vx_arange(const vx_tensor * dst, float start, float step, v
     if (!dst->data) return vx_fail(VX_ERR_INVALID, "arange: null data");
     const int64_t n = vx_nelements(dst), blocks = (n + 255) / 256;
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "arange: launch too large");
-    arange_kernel<<<dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream>>>((float *) dst->data, n, start, step);
+    vx_launch(arange_kernel, dim3((unsigned) blocks), dim3(256), 0, (hipStream_t) stream, (float *) dst->data, n, start, step);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1368,9 +1368,9 @@ extern "C" vx_status vx_repeat(const vx_tensor * src, const vx_tensor * dst, vx_
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "repeat: launch too large");
     const dim3 grid((unsigned) blocks), block(256);
     hipStream_t st = (hipStream_t) stream;
-    if (vec)          { if (es == 4) repeat_kernel<16, 4><<<grid, block, 0, st>>>(a); else repeat_kernel<16, 2><<<grid, block, 0, st>>>(a); }
-    else if (es == 4) repeat_kernel<4, 4><<<grid, block, 0, st>>>(a);
-    else              repeat_kernel<2, 2><<<grid, block, 0, st>>>(a);
+    if (vec)          { if (es == 4) vx_launch(repeat_kernel<16, 4>, grid, block, 0, st, a); else vx_launch(repeat_kernel<16, 2>, grid, block, 0, st, a); }
+    else if (es == 4) vx_launch(repeat_kernel<4, 4>, grid, block, 0, st, a);
+    else              vx_launch(repeat_kernel<2, 2>, grid, block, 0, st, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1405,9 +1405,9 @@ extern "C" vx_status vx_get_rows(const vx_tensor * table, const vx_tensor * rows
     if (blocks > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "get_rows: launch too large");
     const dim3 grid((unsigned) blocks), block(256);
     hipStream_t st = (hipStream_t) stream;
-    if (table->type == VX_TYPE_F16)       get_rows_kernel<1><<<grid, block, 0, st>>>(a);
-    else if (table->type == VX_TYPE_Q8_0) get_rows_kernel<2><<<grid, block, 0, st>>>(a);
-    else                                  get_rows_kernel<0><<<grid, block, 0, st>>>(a);
+    if (table->type == VX_TYPE_F16)       vx_launch(get_rows_kernel<1>, grid, block, 0, st, a);
+    else if (table->type == VX_TYPE_Q8_0) vx_launch(get_rows_kernel<2>, grid, block, 0, st, a);
+    else                                  vx_launch(get_rows_kernel<0>, grid, block, 0, st, a);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1747,9 +1747,9 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         }
     }
     if (dense) {
-        small_graph_dense_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(da);
+        vx_launch(small_graph_dense_kernel, dim3(1), dim3(threads), smem, (hipStream_t) stream, da);
     } else {
-        small_graph_kernel<<<dim3(1), dim3(threads), smem, (hipStream_t) stream>>>(a);
+        vx_launch(small_graph_kernel, dim3(1), dim3(threads), smem, (hipStream_t) stream, a);
     }
     VX_LAUNCH_CHECK();
     return VX_OK;
@@ -1778,9 +1778,9 @@ extern "C" vx_status vx_sum(const vx_tensor * src, const vx_tensor * dst, vx_str
         partials = (double *) ws; blocks = SUM_BLOCKS;
     }
     const dim3 block(units <= VX_SUM_ONE_WAVE_UNITS ? 64 : 1024); // small sums are one wave's work
-    if (vec) sum_kernel<true><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
-    else     sum_kernel<false><<<dim3(blocks), block, 0, st>>>((const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
-    if (partials) sum_partials_kernel<<<dim3(1), dim3(SUM_BLOCKS), 0, st>>>(partials, blocks, (float *) dst->data);
+    if (vec) vx_launch(sum_kernel<true>, dim3(blocks), block, 0, st, (const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    else     vx_launch(sum_kernel<false>, dim3(blocks), block, 0, st, (const char *) src->data, vx_dims_of(src), (float *) dst->data, partials);
+    if (partials) vx_launch(sum_partials_kernel, dim3(1), dim3(SUM_BLOCKS), 0, st, partials, blocks, (float *) dst->data);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1809,7 +1809,7 @@ extern "C" vx_status vx_sum_rows(const vx_tensor * src, const vx_tensor * dst, v
     if (!vx_supports_sum_rows(src, dst)) return vx_fail(VX_ERR_UNSUPPORTED, "sum_rows: F32 rows (nb0 == 4) to an F32 tensor of one element per row");
     if (!src->data || !dst->data) return vx_fail(VX_ERR_INVALID, "sum_rows: null data");
     const int64_t rows = src->ne[1] * src->ne[2] * src->ne[3];
-    sum_rows_kernel<<<dim3((unsigned) rows), dim3(64), 0, (hipStream_t) stream>>>((const char *) src->data, vx_dims_of(src), (char *) dst->data, vx_dims_of(dst));
+    vx_launch(sum_rows_kernel, dim3((unsigned) rows), dim3(64), 0, (hipStream_t) stream, (const char *) src->data, vx_dims_of(src), (char *) dst->data, vx_dims_of(dst));
     VX_LAUNCH_CHECK();
     return VX_OK;
 }
@@ -1845,20 +1845,20 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
     a.scale = scale; a.bias = bias;
     a.dense4 = vx_is_contiguous(x) && vx_is_contiguous(dst) && vx_nelements(x) % 4 == 0 && ((uintptr_t) x->data | (uintptr_t) dst->data) % 16 == 0;
     if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) {
-        kv_store_sync_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t) stream>>>(a);
+        vx_launch(kv_store_sync_kernel, dim3(1), dim3(1024), 0, (hipStream_t) stream, a);
     } else { // a prefill's write: stores and block totals, then totals, scalar and ADD1
         void * ws = nullptr;
         const vx_status rc = vx_workspace((hipStream_t) stream, 2 * SUM_BLOCKS * sizeof(double), &ws);
         if (rc != VX_OK) return rc;
         const dim3 grid(2 * SUM_BLOCKS), block(1024);
         hipStream_t st = (hipStream_t) stream;
-        if (a.k.vec && a.v.vec) kv_store_large_kernel<true, true><<<grid, block, 0, st>>>(a, (double *) ws);
-        else if (a.k.vec)       kv_store_large_kernel<true, false><<<grid, block, 0, st>>>(a, (double *) ws);
-        else if (a.v.vec)       kv_store_large_kernel<false, true><<<grid, block, 0, st>>>(a, (double *) ws);
-        else                    kv_store_large_kernel<false, false><<<grid, block, 0, st>>>(a, (double *) ws);
+        if (a.k.vec && a.v.vec) vx_launch(kv_store_large_kernel<true, true>, grid, block, 0, st, a, (double *) ws);
+        else if (a.k.vec)       vx_launch(kv_store_large_kernel<true, false>, grid, block, 0, st, a, (double *) ws);
+        else if (a.v.vec)       vx_launch(kv_store_large_kernel<false, true>, grid, block, 0, st, a, (double *) ws);
+        else                    vx_launch(kv_store_large_kernel<false, false>, grid, block, 0, st, a, (double *) ws);
         const int64_t nx = vx_nelements(x);
         const unsigned blocks = (unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096);
-        kv_sync_add1_kernel<<<dim3(blocks), dim3(256), 0, st>>>(a, (const double *) ws);
+        vx_launch(kv_sync_add1_kernel, dim3(blocks), dim3(256), 0, st, a, (const double *) ws);
     }
     VX_LAUNCH_CHECK();
     return VX_OK;

@@ -69,9 +69,9 @@ extern "C" vx_status vx_kv_store(const vx_tensor * src, const vx_tensor * view, 
     if (n < 0 || (n + 255) / 256 > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "kv_store: too many elements");
     const dim3 grid((unsigned) ((n + 255) / 256)), block(256);
     if (view->type == VX_TYPE_F16)
-        kv_store_kernel<_Float16><<<grid, block, 0, (hipStream_t) stream>>>((const char *) src->data, (char *) view->data, vx_dims_of(src), vx_dims_of(view));
+        vx_launch(kv_store_kernel<_Float16>, grid, block, 0, (hipStream_t) stream, (const char *) src->data, (char *) view->data, vx_dims_of(src), vx_dims_of(view));
     else
-        kv_store_kernel<float><<<grid, block, 0, (hipStream_t) stream>>>((const char *) src->data, (char *) view->data, vx_dims_of(src), vx_dims_of(view));
+        vx_launch(kv_store_kernel<float>, grid, block, 0, (hipStream_t) stream, (const char *) src->data, (char *) view->data, vx_dims_of(src), vx_dims_of(view));
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

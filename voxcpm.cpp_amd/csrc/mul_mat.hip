@@ -1141,7 +1141,7 @@ bool launch_gemv_dma(mm_args & a, int nbatch, int nw, dim3 grid, hipStream_t st)
                 raised[many] = true;                                                                                   \
             }                                                                                                          \
         }                                                                                                              \
-        kern<<<grid, block, smem, st>>>(a);                                                                            \
+        vx_launch(kern, grid, block, smem, st, a);                                                                            \
         return true;                                                                                                   \
     } while (0)
 #define VX_DMA_NW(SEG_, NORM_, EPI_)                                                                                   \
@@ -1242,7 +1242,7 @@ bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
                 raised = true;                                                                                         \
             }                                                                                                          \
         }                                                                                                              \
-        __VA_ARGS__<<<grid, block, smem, st>>>(a);                                                                     \
+        vx_launch(__VA_ARGS__, grid, block, smem, st, a);                                                                     \
     } while (0)
 #define VX_GEMV(NW_)                                                                                                   \
     do {                                                                                                               \
@@ -1483,8 +1483,8 @@ bool launch_gemm128(const mm_args & a, int nbatch, hipStream_t st) {
     // 32-bit lane offsets inside the kernel: rows of the weight matrix and the 128 tokens of a tile
     if ((uint64_t) a.M * a.nb01 >= (1ull << 32) || (uint64_t) 128 * a.nb11 + 256 >= (1ull << 32)) return false;
     const dim3 grid((unsigned) blocks, 1, (unsigned) nbatch);
-    if (WT == WT_Q8 && a.w_aligned) gemm128_kernel<WT, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
-    else                            gemm128_kernel<WT, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+    if (WT == WT_Q8 && a.w_aligned) vx_launch(gemm128_kernel<WT, ACT_Q8, true>, grid, dim3(256), 0, st, a);
+    else                            vx_launch(gemm128_kernel<WT, ACT_Q8, false>, grid, dim3(256), 0, st, a);
     return true;
 }
 
@@ -1806,7 +1806,7 @@ bool launch_gemm_lds_tile(const mm_args & a, int nbatch, hipStream_t st) {
         raised = true;
     }
     const int nsplit = a.ksplit > 1 ? a.ksplit : 1;
-    gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC, DUAL><<<dim3((unsigned) blocks, 1, (unsigned) (nbatch * nsplit)), dim3(64 * WR * WC), lds, st>>>(a);
+    vx_launch(gemm_lds_kernel<WT, FOLD, RT, CT, WR, WC, DUAL>, dim3((unsigned) blocks, 1, (unsigned) (nbatch * nsplit)), dim3(64 * WR * WC), lds, st, a);
     return true;
 }
 
@@ -2192,13 +2192,13 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     }
     const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) ((q.n_kb + QT_ACT_UNROLL - 1) / QT_ACT_UNROLL) * q.n_tt * 64;
     if ((wunits + 255) / 256 > 0x7fffffff || (xunits + 255) / 256 > 0x7fffffff) return false;
-    qt_weights_kernel<<<dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st>>>(q);
-    qt_acts_kernel<<<dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st>>>(q);
+    vx_launch(qt_weights_kernel, dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st, q);
+    vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
     const int gx = (q.n_rt + 15) / 16, gy = (q.n_tt + 7) / 8, Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
     const int64_t blocks = ((int64_t) Gx * Gy + 7) / 8 * 8 * 32;
     if (blocks > 0x7fffffff) return false;
-    if (fold) gemm_q8t_kernel<DUAL, true><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
-    else      gemm_q8t_kernel<DUAL, false><<<dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st>>>(q);
+    if (fold) vx_launch(gemm_q8t_kernel<DUAL, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
+    else      vx_launch(gemm_q8t_kernel<DUAL, false>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     return true;
 }
 
@@ -2231,7 +2231,7 @@ bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
         const bool ok = WT == WT_Q8 && mode == 2 ? launch_gemm_lds_tile<WT, WT == WT_Q8, 2, 2, 2, 2>(b, nbatch, st) : launch_gemm_lds_tile<WT, false, 2, 2, 2, 2>(b, nbatch, st);
         if (!ok) return false;
         const int64_t units = a.N * (a.M / 4);
-        mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+        vx_launch(mm_splitk_reduce_kernel, dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st, b);
         return true;
     }
     if (a.res && (uint64_t) 256 * a.rnb1 + 1024 >= (1ull << 32)) return false; // (the residual's 32-bit lane offsets)
@@ -2273,9 +2273,9 @@ bool launch_mm_cut(const mm_args & a, int nbatch, hipStream_t st) {
     if ((t_ws_status = vx_workspace(st, a.ws_offset + (size_t) nbatch * ks * a.N * a.M * sizeof(float), &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
     mm_args b = a;
     b.ksplit = ks; b.partial = (float *) ((char *) ws + a.ws_offset);
-    mm_kernel<WT, 4, ACT_Q8, false><<<dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st>>>(b);
+    vx_launch(mm_kernel<WT, 4, ACT_Q8, false>, dim3((unsigned) gx, (unsigned) gy, (unsigned) (nbatch * ks)), dim3(256), 0, st, b);
     const int64_t units = a.N * (a.M / 4);
-    mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+    vx_launch(mm_splitk_reduce_kernel, dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st, b);
     return true;
 }
 
@@ -2286,15 +2286,15 @@ void launch(const mm_args & a, int nbatch, hipStream_t st) {
     if constexpr (WT != WT_F32) { if (launch_gemm128<WT, ACT_Q8>(a, nbatch, st)) return; }
     if (a.N <= 16) {
         const dim3 grid((unsigned) ((a.M + 15) / 16), 1, (unsigned) nbatch);
-        mm_kernel<WT, 1, ACT_Q8, true><<<grid, dim3(256), 0, st>>>(a);
+        vx_launch(mm_kernel<WT, 1, ACT_Q8, true>, grid, dim3(256), 0, st, a);
     } else if (a.N <= 32) {
         const dim3 grid((unsigned) ((a.M + 63) / 64), 1, (unsigned) nbatch);
-        mm_kernel<WT, 2, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+        vx_launch(mm_kernel<WT, 2, ACT_Q8, false>, grid, dim3(256), 0, st, a);
     } else {
         if (launch_mm_cut<WT, ACT_Q8>(a, nbatch, st) || ws_failed()) return;
         const int64_t gx = (a.M + 63) / 64, gy = (a.N + 63) / 64;
         const dim3 grid((unsigned) gx, (unsigned) gy, (unsigned) nbatch);
-        mm_kernel<WT, 4, ACT_Q8, false><<<grid, dim3(256), 0, st>>>(a);
+        vx_launch(mm_kernel<WT, 4, ACT_Q8, false>, grid, dim3(256), 0, st, a);
     }
 }
 
@@ -2554,7 +2554,7 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
         b.ksplit = 1; b.partial = (float *) product;
         const int64_t units = a.N * (a.M / 4);
         if ((units + 255) / 256 > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: launch too large");
-        mm_splitk_reduce_kernel<<<dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st>>>(b);
+        vx_launch(mm_splitk_reduce_kernel, dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st, b);
     }
     VX_LAUNCH_CHECK();
     return VX_OK;

@@ -124,10 +124,10 @@ static vx_status rms_norm_launch(const vx_tensor * src, const vx_tensor * dst, f
     hipStream_t   st = (hipStream_t) stream;
     if (src->ne[0] <= 1024) {
         const int rpb = 4; // one wave per row
-        rms_norm_kernel<256><<<dim3((unsigned) ((nrows + rpb - 1) / rpb)), dim3(256), 0, st>>>(
+        vx_launch(rms_norm_kernel<256>, dim3((unsigned) ((nrows + rpb - 1) / rpb)), dim3(256), 0, st, 
             (const char *) src->data, (char *) dst->data, s, d, eps, rpb, w);
     } else {
-        rms_norm_kernel<256><<<dim3((unsigned) nrows), dim3(256), 0, st>>>(
+        vx_launch(rms_norm_kernel<256>, dim3((unsigned) nrows), dim3(256), 0, st, 
             (const char *) src->data, (char *) dst->data, s, d, eps, 1, w);
     }
     VX_LAUNCH_CHECK();

@@ -77,7 +77,7 @@ extern "C" vx_status vx_rope(const vx_tensor * src, const int32_t * pos, const f
     const rope_params p = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
     const int64_t total = vx_nrows(src) * (src->ne[0] / 2);
     const unsigned grid = (unsigned) ((total + 255) / 256);
-    rope_kernel<<<dim3(grid), dim3(256), 0, (hipStream_t) stream>>>((const char *) src->data, (char *) dst->data,
+    vx_launch(rope_kernel, dim3(grid), dim3(256), 0, (hipStream_t) stream, (const char *) src->data, (char *) dst->data,
                                                                     vx_dims_of(src), vx_dims_of(dst), pos,
                                                                     freq_factors, p);
     VX_LAUNCH_CHECK();

@@ -122,7 +122,7 @@ extern "C" vx_status vx_soft_max(const vx_tensor * src, const vx_tensor * mask, 
     p.m1          = powf(2.0f, -(max_bias / 2.0f) / p.n_head_log2);
     p.mask_f16    = mask && mask->type == VX_TYPE_F16;
     vx_dims md    = mask ? vx_dims_of(mask) : vx_dims_of(src);
-    soft_max_kernel<<<dim3((unsigned) vx_nrows(src)), dim3(SM_BLOCK), 0, (hipStream_t) stream>>>(
+    vx_launch(soft_max_kernel, dim3((unsigned) vx_nrows(src)), dim3(SM_BLOCK), 0, (hipStream_t) stream, 
         (const char *) src->data, mask ? (const char *) mask->data : nullptr, sinks, (char *) dst->data,
         vx_dims_of(src), md, vx_dims_of(dst), p);
     VX_LAUNCH_CHECK();

@@ -7,6 +7,8 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <tuple>
+#include <utility>
 
 #include "../../include/voxcpm_gfx950.h"
 
@@ -33,6 +35,32 @@ vx_status  vx_fail(vx_status st, const char * fmt, ...) __attribute__((format(pr
             return vx_fail(VX_ERR_HIP, "kernel launch failed: %s (%s:%d)",                   \
                            hipGetErrorString(e_), __FILE__, __LINE__);                       \
     } while (0)
+
+// ---- launching --------------------------------------------------------------------------------------------------------
+// Every kernel of the operators goes to the GPU through vx_launch, so that a recording made between vx_graph_begin and
+// vx_graph_end knows its launches one by one (function, grid, block, LDS bytes, argument bytes), and so that a later run
+// of the same operators can be compared with it without launching anything (vx_graph_patch_begin): the launches whose
+// arguments differ are then set on the recorded graph, and one hipGraphLaunch issues them all.
+//   0  launch;   1  launch (into the capture) and note;   2  compare with the recording, launch nothing
+extern thread_local int vx_tl_launch_mode;
+void vx_launch_note(const void * func, dim3 grid, dim3 block, size_t lds_bytes, void * const * params, const size_t * sizes, int n_params);
+
+template <typename... P, size_t... I>
+inline void vx_launch_note_tuple(const void * func, dim3 grid, dim3 block, size_t lds_bytes, std::tuple<P...> & vals, std::index_sequence<I...>) {
+    void * const        ptrs[]  = { (void *) &std::get<I>(vals)... };
+    static const size_t sizes[] = { sizeof(P)... };
+    vx_launch_note(func, grid, block, lds_bytes, ptrs, sizes, (int) sizeof...(P));
+}
+template <typename... P, typename... A>
+inline void vx_launch(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, const A &... args) {
+    static_assert(sizeof...(P) == sizeof...(A) && sizeof...(P) > 0, "one argument per kernel parameter");
+    if (__builtin_expect(vx_tl_launch_mode != 0, 0)) {
+        std::tuple<P...> vals(args...); // converted to the kernel's own parameter types, as the launch would
+        vx_launch_note_tuple((const void *) kernel, grid, block, lds_bytes, vals, std::index_sequence_for<P...>{});
+        if (vx_tl_launch_mode == 2) return;
+    }
+    kernel<<<grid, block, lds_bytes, stream>>>(args...);
+}
 
 // per-stream scratch memory, grown on demand.  A block stays allocated at its address until the stream is
 // destroyed, also after a larger one has replaced it (ws_policy.hpp), so launches already queued and graphs

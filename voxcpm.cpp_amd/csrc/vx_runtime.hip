@@ -5,6 +5,7 @@
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 namespace {
 
@@ -17,7 +18,94 @@ unsigned long long ws_key(int dev, hipStream_t stream) {
     return ((unsigned long long) dev << 56) ^ (unsigned long long) (uintptr_t) stream;
 }
 
+// ---- recorded graphs ----------------------------------------------------------------------------------------------
+// What a vx_graph handle points to: the instantiated HIP graph, and -- when every launch of the recording went through
+// vx_launch and the captured graph's kernel nodes agree with them one for one -- the launches themselves, so that a
+// later run of the same operators can be compared with the recording and the differences set on the graph's nodes.
+struct launch_rec {
+    const void * func;
+    dim3         grid, block;
+    unsigned     lds_bytes;
+    unsigned     first_param, n_params; // into recorded_graph::params
+};
+struct param_rec { unsigned offset, size; }; // into recorded_graph::bytes
+struct recorded_graph {
+    hipGraphExec_t              exec = nullptr;
+    hipGraph_t                  graph = nullptr; // kept while `nodes` are in use: they belong to it
+    hipEvent_t                  done = nullptr;  // recorded after each launch of a patchable graph
+    bool                        in_flight = false;
+    std::vector<hipGraphNode_t> nodes;           // one per launch, in launch order; empty = replay only
+    std::vector<launch_rec>     launches;
+    std::vector<param_rec>      params;
+    std::vector<char>           bytes;
+};
+thread_local recorded_graph * t_rec     = nullptr; // the recording being made (mode 1) or compared with (mode 2)
+thread_local size_t           t_next    = 0;       // mode 2: the launch the next note is compared with
+thread_local bool             t_differs = false;   // mode 2: another function, another count, or a node that would not take its arguments
+thread_local int              t_patched = 0;
+
+void destroy_recorded(recorded_graph * r) {
+    if (!r) return;
+    if (r->exec) (void) hipGraphExecDestroy(r->exec);
+    if (r->graph) (void) hipGraphDestroy(r->graph);
+    if (r->done) (void) hipEventDestroy(r->done);
+    delete r;
+}
+
 } // namespace
+
+thread_local int vx_tl_launch_mode = 0;
+
+void vx_launch_note(const void * func, dim3 grid, dim3 block, size_t lds_bytes, void * const * params, const size_t * sizes, int n_params) {
+    recorded_graph * r = t_rec;
+    if (!r) return;
+    if (vx_tl_launch_mode == 1) { // recording: keep the launch
+        launch_rec l = { func, grid, block, (unsigned) lds_bytes, (unsigned) r->params.size(), (unsigned) n_params };
+        for (int i = 0; i < n_params; ++i) {
+            const size_t at = (r->bytes.size() + 15) & ~(size_t) 15;
+            r->bytes.resize(at + sizes[i]);
+            memcpy(r->bytes.data() + at, params[i], sizes[i]);
+            r->params.push_back({ (unsigned) at, (unsigned) sizes[i] });
+        }
+        r->launches.push_back(l);
+        return;
+    }
+    if (t_differs) return;
+    if (t_next >= r->launches.size()) { t_differs = true; return; }
+    launch_rec & l = r->launches[t_next];
+    if (l.func != func || (int) l.n_params != n_params) { t_differs = true; return; }
+    bool same = l.grid.x == grid.x && l.grid.y == grid.y && l.grid.z == grid.z && l.block.x == block.x && l.block.y == block.y &&
+                l.block.z == block.z && l.lds_bytes == (unsigned) lds_bytes;
+    for (int i = 0; i < n_params; ++i) {
+        const param_rec & pr = r->params[l.first_param + i];
+        if (pr.size != sizes[i]) { t_differs = true; return; }
+        if (memcmp(r->bytes.data() + pr.offset, params[i], sizes[i]) != 0) {
+            memcpy(r->bytes.data() + pr.offset, params[i], sizes[i]);
+            same = false;
+        }
+    }
+    if (!same) {
+        constexpr int MAX_PARAMS = 16;
+        void * ptrs[MAX_PARAMS];
+        if (n_params > MAX_PARAMS) { t_differs = true; return; }
+        for (int i = 0; i < n_params; ++i) ptrs[i] = r->bytes.data() + r->params[l.first_param + i].offset;
+        l.grid = grid; l.block = block; l.lds_bytes = (unsigned) lds_bytes;
+        hipKernelNodeParams kp = {};
+        kp.func = const_cast<void *>(func);
+        kp.gridDim = grid;
+        kp.blockDim = block;
+        kp.sharedMemBytes = (unsigned) lds_bytes;
+        kp.kernelParams = ptrs;
+        kp.extra = nullptr;
+        if (hipGraphExecKernelNodeSetParams(r->exec, r->nodes[t_next], &kp) != hipSuccess) {
+            (void) hipGetLastError();
+            t_differs = true;
+            return;
+        }
+        ++t_patched;
+    }
+    ++t_next;
+}
 
 void vx_set_error(const char * fmt, ...) {
     va_list ap;
@@ -188,36 +276,105 @@ vx_status vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int *
     return VX_OK;
 }
 vx_status vx_graph_begin(vx_stream stream) {
+    if (vx_tl_launch_mode != 0) return vx_fail(VX_ERR_INVALID, "vx_graph_begin: this thread is already recording or comparing");
     VX_HIP(hipStreamBeginCapture((hipStream_t) stream, hipStreamCaptureModeThreadLocal));
+    t_rec = new recorded_graph;
+    vx_tl_launch_mode = 1;
     return VX_OK;
 }
 vx_status vx_graph_end(vx_stream stream, vx_graph * graph) {
-    if (!graph) return vx_fail(VX_ERR_INVALID, "vx_graph_end: null out pointer");
+    recorded_graph * r = t_rec;
+    t_rec = nullptr;
+    if (vx_tl_launch_mode == 1) vx_tl_launch_mode = 0;
+    if (!graph) { destroy_recorded(r); return vx_fail(VX_ERR_INVALID, "vx_graph_end: null out pointer"); }
     *graph = nullptr;
     hipGraph_t g = nullptr;
     const hipError_t e = hipStreamEndCapture((hipStream_t) stream, &g);
     if (e != hipSuccess || !g) { // an invalidated recording: the stream is usable again, nothing to replay
         (void) hipGetLastError();
         if (g) (void) hipGraphDestroy(g);
+        destroy_recorded(r);
         return VX_OK;
     }
-    hipGraphExec_t exec = nullptr;
-    const hipError_t e2 = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
-    (void) hipGraphDestroy(g);
-    if (e2 != hipSuccess || !exec) {
+    if (!r) r = new recorded_graph;
+    r->graph = g;
+    const hipError_t e2 = hipGraphInstantiate(&r->exec, g, nullptr, nullptr, 0);
+    if (e2 != hipSuccess || !r->exec) {
         (void) hipGetLastError();
+        r->exec = nullptr;
+        destroy_recorded(r);
         return VX_OK;
     }
-    *graph = (vx_graph) exec;
+    // the graph's nodes against the noted launches: the same count, kernels all, the same functions and grids in the same
+    // order (a capture of one stream is a chain, and hipGraphGetNodes lists it in the order of capture; anything else --
+    // launches that did not go through vx_launch, another order -- leaves a graph that can be replayed but not patched)
+    size_t n = 0;
+    bool patchable = !r->launches.empty() && hipGraphGetNodes(g, nullptr, &n) == hipSuccess && n == r->launches.size();
+    if (patchable) {
+        r->nodes.resize(n);
+        patchable = hipGraphGetNodes(g, r->nodes.data(), &n) == hipSuccess && n == r->launches.size();
+    }
+    for (size_t i = 0; patchable && i < n; ++i) {
+        hipGraphNodeType type;
+        hipKernelNodeParams kp;
+        patchable = hipGraphNodeGetType(r->nodes[i], &type) == hipSuccess && type == hipGraphNodeTypeKernel &&
+                    hipGraphKernelNodeGetParams(r->nodes[i], &kp) == hipSuccess && kp.func == r->launches[i].func &&
+                    kp.gridDim.x == r->launches[i].grid.x && kp.gridDim.y == r->launches[i].grid.y && kp.gridDim.z == r->launches[i].grid.z;
+    }
+    if (patchable) patchable = hipEventCreateWithFlags(&r->done, hipEventDisableTiming) == hipSuccess;
+    if (!patchable) {
+        (void) hipGetLastError();
+        r->nodes.clear(); r->launches.clear(); r->params.clear(); r->bytes.clear();
+        (void) hipGraphDestroy(r->graph);
+        r->graph = nullptr;
+    }
+    *graph = (vx_graph) r;
     return VX_OK;
 }
 vx_status vx_graph_launch(vx_graph graph, vx_stream stream) {
-    if (!graph) return vx_fail(VX_ERR_INVALID, "vx_graph_launch: null graph");
-    VX_HIP(hipGraphLaunch((hipGraphExec_t) graph, (hipStream_t) stream));
+    recorded_graph * r = (recorded_graph *) graph;
+    if (!r || !r->exec) return vx_fail(VX_ERR_INVALID, "vx_graph_launch: null graph");
+    VX_HIP(hipGraphLaunch(r->exec, (hipStream_t) stream));
+    if (r->done) {
+        VX_HIP(hipEventRecord(r->done, (hipStream_t) stream));
+        r->in_flight = true;
+    }
     return VX_OK;
 }
 vx_status vx_graph_destroy(vx_graph graph) {
-    if (graph) VX_HIP(hipGraphExecDestroy((hipGraphExec_t) graph));
+    recorded_graph * r = (recorded_graph *) graph;
+    if (r && r == t_rec) { t_rec = nullptr; vx_tl_launch_mode = 0; }
+    if (r && r->in_flight && r->done) (void) hipEventSynchronize(r->done);
+    destroy_recorded(r);
+    return VX_OK;
+}
+int vx_graph_patchable(vx_graph graph) {
+    const recorded_graph * r = (const recorded_graph *) graph;
+    return r && !r->nodes.empty();
+}
+vx_status vx_graph_patch_begin(vx_graph graph) {
+    recorded_graph * r = (recorded_graph *) graph;
+    if (!r || r->nodes.empty()) return vx_fail(VX_ERR_UNSUPPORTED, "vx_graph_patch_begin: this recording cannot be compared with");
+    if (vx_tl_launch_mode != 0) return vx_fail(VX_ERR_INVALID, "vx_graph_patch_begin: this thread is already recording or comparing");
+    if (r->in_flight) { // its last launch may still be reading the arguments that are about to change
+        VX_HIP(hipEventSynchronize(r->done));
+        r->in_flight = false;
+    }
+    t_rec = r;
+    t_next = 0;
+    t_differs = false;
+    t_patched = 0;
+    vx_tl_launch_mode = 2;
+    return VX_OK;
+}
+vx_status vx_graph_patch_end(vx_graph graph, int * patched) {
+    recorded_graph * r = (recorded_graph *) graph;
+    if (vx_tl_launch_mode != 2 || r != t_rec) return vx_fail(VX_ERR_INVALID, "vx_graph_patch_end: no comparison with this graph is open");
+    vx_tl_launch_mode = 0;
+    t_rec = nullptr;
+    if (patched) *patched = t_patched;
+    if (t_differs || t_next != r->launches.size())
+        return vx_fail(VX_ERR_UNSUPPORTED, "vx_graph_patch_end: the launches differ from the recording's (%zu of %zu matched)", t_next, r->launches.size());
     return VX_OK;
 }
 vx_status vx_stream_synchronize(vx_stream stream) {

@@ -110,10 +110,26 @@ struct seen_graph {
     uint64_t last_use = 0;
 };
 
+// Graphs that agree in their nodes' operators and types but not in addresses, extents or parameters: the steps of a
+// decode loop, each with one key more than the one before.  Such a graph never comes back, but its launches are the
+// previous step's with a few arguments changed: the node-by-node pass is then made against a recording (nothing is
+// launched, the arguments that differ are set on the recorded HIP graph) and the graph is launched as one unit.  Two
+// recordings are used in turn, so that one can be prepared while the other still runs.
+struct step_family {
+    uint64_t shape = 0;       // node count, operators and types
+    int      sightings = 0;
+    int      failures = 0;    // recordings that could not be made, or passes that made other launches than recorded
+    vx_graph recorded[2] = { nullptr, nullptr };
+    int      turn = 0;
+    int      launches = 0;
+    uint64_t last_use = 0;
+};
+
 struct backend_ctx {
     int       device;
     vx_stream stream;
     std::vector<seen_graph> seen;   // a handful of entries, least recently used one replaced
+    std::vector<step_family> families;
     uint64_t  clock = 0;
     int       replays = 0;          // diagnostic: graph_compute calls served by a replay
 };
@@ -475,6 +491,7 @@ void backend_free(ggml_backend_t backend) {
     vx_init(ctx->device);
     vx_stream_synchronize(ctx->stream);
     for (seen_graph & g : ctx->seen) if (g.recorded) vx_graph_destroy(g.recorded);
+    for (step_family & f : ctx->families) for (vx_graph & r : f.recorded) if (r) vx_graph_destroy(r);
     vx_stream_destroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -1273,14 +1290,19 @@ inline uint64_t mix64(uint64_t h, uint64_t v) {
 }
 // cheap: node count, and per node the operator, the output address and the two outer extents (what changes from one
 // decode step to the next: the key count) -- a few hundred nanoseconds per thousand nodes
-uint64_t graph_cheap_signature(const ggml_cgraph * g) {
+// `shape`, taken in the same pass: node count, operators and types only -- what the steps of a decode loop share
+uint64_t graph_cheap_signature(const ggml_cgraph * g, uint64_t * shape) {
     // (the activation mode of the Q8_0 products is part of what a recording holds: a graph recorded under one mode is
     // another graph under the other)
     uint64_t h = (uint64_t) g->n_nodes ^ (((uint64_t) mul_mat_act_mode() << 40) ^ ((uint64_t) fusion_on() << 42));
+    uint64_t s = h;
     for (int i = 0; i < g->n_nodes; ++i) {
         const ggml_tensor * n = g->nodes[i];
         h = mix64(h, (uint64_t) (uintptr_t) n->data ^ ((uint64_t) n->op << 56) ^ ((uint64_t) n->ne[1] << 20) ^ ((uint64_t) n->ne[2] << 40));
+        s = (s ^ (((uint64_t) n->op << 8) ^ (uint64_t) n->type)) * 0x9E3779B97F4A7C15ull;
+        s ^= s >> 31;
     }
+    *shape = s | 1;
     return h | 1;
 }
 // full: everything a launch is derived from.  A thousand nodes are some 25 000 words, hashed on every graph_compute of a
@@ -1319,6 +1341,58 @@ uint64_t graph_fingerprint(const ggml_cgraph * g) {
 }
 
 ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out);
+int g_patch_on = -1;     // run a decode loop's steps as patched recordings (GGML_GFX950_GRAPH_PATCH, ggml_backend_gfx950_set_graph_patch)
+int g_patched_replays = 0; // graph_compute calls served by a recording whose arguments were brought up to date first
+int g_last_patched = 0;    // nodes whose arguments the most recent such call changed
+bool patch_on() {
+    // off unless asked for: the comparison pass takes the host a quarter of a millisecond for a 24-layer step before the
+    // GPU gets anything to do, where node-by-node launches keep the GPU busy from the first launch on
+    if (g_patch_on < 0) { const char * e = getenv("GGML_GFX950_GRAPH_PATCH"); g_patch_on = e && atoi(e) != 0; }
+    return g_patch_on != 0;
+}
+
+// One more member of a family: true when the graph has been computed here (by a patched recording, or by a new one).
+bool family_compute(backend_ctx * ctx, step_family & fam, ggml_cgraph * cgraph) {
+    constexpr int MAX_FAILURES = 3;
+    if (fam.failures >= MAX_FAILURES) return false;
+    vx_graph & rec = fam.recorded[fam.turn];
+    int launches = 0;
+    if (rec) {
+        if (vx_graph_patch_begin(rec) == VX_OK) {
+            const ggml_status st = graph_compute_eager(ctx, cgraph, &launches); // compares, launches nothing
+            int patched = 0;
+            const bool same = vx_graph_patch_end(rec, &patched) == VX_OK;
+            if (st == GGML_STATUS_SUCCESS && same && vx_graph_launch(rec, ctx->stream) == VX_OK) {
+                fam.turn ^= 1;
+                ++g_replays;
+                ++g_patched_replays;
+                g_last_patched = patched;
+                g_last_launches = fam.launches;
+                return true;
+            }
+        }
+        vx_graph_destroy(rec); // other launches than recorded (another kernel for this key count, say): its arguments are a mixture now
+        rec = nullptr;
+        ++fam.failures;
+        return false;
+    }
+    if (vx_graph_begin(ctx->stream) != VX_OK) { ++fam.failures; return false; }
+    const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+    vx_graph made = nullptr;
+    vx_graph_end(ctx->stream, &made);
+    if (st == GGML_STATUS_SUCCESS && made && vx_graph_patchable(made) && vx_graph_launch(made, ctx->stream) == VX_OK) {
+        rec = made;
+        fam.launches = launches;
+        fam.turn ^= 1;
+        fam.failures = 0;
+        ++g_replays;
+        g_last_launches = launches;
+        return true;
+    }
+    if (made) vx_graph_destroy(made);
+    ++fam.failures; // e.g. a launch that must allocate
+    return false;
+}
 long long g_host_ns[2] = { 0, 0 }; // the most recent node-by-node graph_compute: host time of the analysis, and of issuing the launches
 
 // graph_optimize (ggml/src/ggml-backend-impl.h:118-119): ggml_backend_sched calls it once per split when it lays a graph
@@ -1343,10 +1417,28 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         g_last_launches = launches;
         return st;
     }
-    const uint64_t cheap = graph_cheap_signature(cgraph);
+    uint64_t shape = 0;
+    const uint64_t cheap = graph_cheap_signature(cgraph, &shape);
     seen_graph * entry = nullptr;
     for (seen_graph & g : ctx->seen) if (g.cheap == cheap) { entry = &g; break; }
     ++ctx->clock;
+    if (!entry && patch_on()) { // never seen as it is: a further step of a loop that has been seen?
+        step_family * fam = nullptr;
+        for (step_family & f : ctx->families) if (f.shape == shape) { fam = &f; break; }
+        if (!fam) {
+            constexpr size_t MAX_FAMILIES = 4;
+            if (ctx->families.size() < MAX_FAMILIES) { ctx->families.emplace_back(); fam = &ctx->families.back(); }
+            else {
+                fam = &ctx->families[0];
+                for (step_family & f : ctx->families) if (f.last_use < fam->last_use) fam = &f;
+                for (vx_graph & r : fam->recorded) if (r) vx_graph_destroy(r);
+                *fam = step_family{};
+            }
+            fam->shape = shape;
+        }
+        fam->last_use = ctx->clock;
+        if (++fam->sightings >= 2 && family_compute(ctx, *fam, cgraph)) return GGML_STATUS_SUCCESS;
+    }
     if (!entry) { // first sight: remember the cheap signature only (a decode step's graph never comes back)
         constexpr size_t MAX_SEEN = 8;
         if (ctx->seen.size() < MAX_SEEN) { ctx->seen.emplace_back(); entry = &ctx->seen.back(); }
@@ -1725,6 +1817,8 @@ void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
     if (strcmp(name, "ggml_backend_gfx950_alloc_weights") == 0) return (void *) ggml_backend_gfx950_alloc_weights;
     if (strcmp(name, "ggml_backend_gfx950_last_launches") == 0) return (void *) ggml_backend_gfx950_last_launches;
     if (strcmp(name, "ggml_backend_gfx950_replays") == 0) return (void *) ggml_backend_gfx950_replays;
+    if (strcmp(name, "ggml_backend_gfx950_patched_replays") == 0) return (void *) ggml_backend_gfx950_patched_replays;
+    if (strcmp(name, "ggml_backend_gfx950_set_graph_patch") == 0) return (void *) ggml_backend_gfx950_set_graph_patch;
     if (strcmp(name, "ggml_backend_gfx950_set_graph_replay") == 0) return (void *) ggml_backend_gfx950_set_graph_replay;
     if (strcmp(name, "ggml_backend_gfx950_set_mul_mat_act") == 0) return (void *) ggml_backend_gfx950_set_mul_mat_act;
     if (strcmp(name, "ggml_backend_gfx950_set_fusion") == 0) return (void *) ggml_backend_gfx950_set_fusion;
@@ -1757,6 +1851,15 @@ extern "C" int ggml_backend_gfx950_last_launches(void) { return g_last_launches;
 extern "C" long long ggml_backend_gfx950_host_ns(int which) { return which == 0 || which == 1 ? g_host_ns[which] : 0; }
 // how many graph_compute calls of this process were served by replaying a recorded graph
 extern "C" int ggml_backend_gfx950_replays(void) { return g_replays; }
+// how many of them brought a recording's arguments up to date first (the steps of a decode loop)
+extern "C" int ggml_backend_gfx950_patched_replays(void) { return g_patched_replays; }
+// nodes whose arguments the most recent such call changed
+extern "C" int ggml_backend_gfx950_last_patched(void) { return g_last_patched; }
+extern "C" int ggml_backend_gfx950_set_graph_patch(int on) {
+    const int before = patch_on();
+    g_patch_on = on != 0;
+    return before;
+}
 // switches the recognition of recurring graphs on (1) or off (0); returns the previous setting
 extern "C" int ggml_backend_gfx950_set_graph_replay(int on) {
     if (g_replay_on < 0) { const char * e = getenv("GGML_GFX950_GRAPH_REPLAY"); g_replay_on = !(e && atoi(e) == 0); }

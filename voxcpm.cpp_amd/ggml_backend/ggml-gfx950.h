@@ -39,6 +39,14 @@ GGML_BACKEND_API bool ggml_backend_gfx950_alloc_weights(struct ggml_context * ct
 GGML_BACKEND_API int ggml_backend_gfx950_last_launches(void);
 GGML_BACKEND_API int ggml_backend_gfx950_set_graph_replay(int on);  /* recognise recurring graphs and replay them; returns the previous setting */
 GGML_BACKEND_API int ggml_backend_gfx950_replays(void);   /* graph_compute calls served by replaying recorded launches */
+/* Graphs that share their nodes' operators and types with one seen before but differ in addresses, extents or
+ * parameters (the steps of a decode loop) are run as that graph's recording with the differing launch arguments set
+ * first.  Off by default (the comparison pass runs on the host before the GPU gets its first launch, which costs a
+ * caller that waits for every step more than the launches it saves); GGML_GFX950_GRAPH_PATCH=1 or set_graph_patch(1)
+ * switches it on; the setter returns the previous setting. */
+GGML_BACKEND_API int ggml_backend_gfx950_set_graph_patch(int on);
+GGML_BACKEND_API int ggml_backend_gfx950_patched_replays(void);   /* how many of the replays were of that kind */
+GGML_BACKEND_API int ggml_backend_gfx950_last_patched(void);      /* launches whose arguments the latest one changed */
 GGML_BACKEND_API int ggml_backend_gfx950_set_mul_mat_act(int mode);
 GGML_BACKEND_API int ggml_backend_gfx950_set_fusion(int on);        /* groups of nodes as one launch (default) or every node its own; returns the previous setting */
 GGML_BACKEND_API long long ggml_backend_gfx950_host_ns(int which);  /* the last node-by-node graph_compute: host ns spent (0) analysing the graph, (1) issuing launches */
