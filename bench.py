@@ -186,6 +186,18 @@ def q8_proj_setup(pkg, M, K, N):
     return call, (wq, x, out)
 
 
+def pinned_in_turns(pkg, timer, call, wq, rounds, iters):
+    """The same product timed in turns with its weights' tiles made on every call and made once and kept (vx_weights_pin),
+    so that both see the same clocks (a run of large products slows the clocks down, and they recover over seconds)."""
+    turns = {"tiles_made_per_call": [], "weights_pinned": []}
+    for _ in range(rounds):
+        turns["tiles_made_per_call"].append(timer.run(call, iters=iters, warmup=2))
+        pkg.check(pkg.lib().vx_weights_pin(wq.data_ptr(), wq.numel()), "vx_weights_pin")
+        turns["weights_pinned"].append(timer.run(call, iters=iters, warmup=2))
+        pkg.check(pkg.lib().vx_weights_unpin(wq.data_ptr()), "vx_weights_unpin")
+    return turns
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -282,7 +294,15 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     mask = torch.from_numpy(reflib.causal_mask(prefill, prefill)).cuda()
     run_p, _ = m.plan(xp, prefill, 0, mask)
     big = batch * prefill > 4096
-    t_prefill = timer.run(run_p, iters=1 if big else 3, warmup=1)
+    # in turns (a run of large products slows the clocks down): the weights as they are / declared constant, as the plugin declares
+    # a buffer that ggml marks as weights -- the products of 1024 tokens and more then keep their weights' tiles between calls
+    t_un, t_pin = [], []
+    for _ in range(2):
+        m.unpin_weights()
+        t_un.append(timer.run(run_p, iters=1 if big else 3, warmup=1))
+        m.pin_weights()
+        t_pin.append(timer.run(run_p, iters=1 if big else 3, warmup=1))
+    t_prefill_unpinned, t_prefill = min(t_un), min(t_pin)
     t_prefill_f16 = None
     if f32_prefill_switch:
         # the same prefill with its F32 keys and values on the hi/lo wave kernel instead of the LDS-tiled one (read per call)
@@ -313,6 +333,7 @@ def backbone_bench(pkg, timer, side, threads, with_cpu, layers=LAYERS, batch=2, 
     res = {"decode_steps_per_s": 1.0 / t_step, "ms_per_step": t_step * 1e3, "launches_per_step": n_calls,
            "weight_GB/s": weight_bytes / t_step / 1e9, "hbm_frac_weights_plus_kv": (weight_bytes + kvb) / t_step / 1e9 / HBM_PEAK_GBS,
            "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": batch * prefill / t_prefill,
+           "prefill_ms_weights_not_pinned": t_prefill_unpinned * 1e3,
            "prefill_ms_VX_FA_F32_PREFILL=0": t_prefill_f16 * 1e3 if t_prefill_f16 else None,
            "kv_cache": "f16" if kv_f16 else "f32 (the reference's cache type)",
            "launch": f"captured HIP graph per step, KV lengths {points} ({per} replays each)"}
@@ -810,9 +831,15 @@ def main():
     if args.profile == "gemm":      # the prefill-sized Q8_0 projection, 4096 rows x 1024 x 16384 tokens
         M, K, N = 4096, 1024, 16384
         call, keep = q8_proj_setup(pkg, M, K, N)
-        s = timer.run(call, iters=5, warmup=2)
-        print(json.dumps({"profile": "q8_0_mul_mat_4096x1024x16384", "us": s * 1e6, "TFLOP/s": 2.0 * M * K * N / s / 1e12,
-                          "mfma_frac": 2.0 * M * K * N / s / 1e12 / MFMA_F16_PEAK_TFLOPS, "VX_GEMM_LDS": os.environ.get("VX_GEMM_LDS", "1")}))
+        s = timer.run(call, iters=5, warmup=2)   # the first calls of a process: the clocks have not settled under the load yet
+        # then in turns, so that both see the same clocks: the weights' tiles made on every call / made once and kept
+        # (vx_weights_pin), 4 rounds of 25 calls each
+        turns = pinned_in_turns(pkg, timer, call, keep[0], 4, 25)
+        flops = 2.0 * M * K * N
+        fig = lambda v: {"us": v * 1e6, "TFLOP/s": flops / v / 1e12, "mfma_frac": flops / v / 1e12 / MFMA_F16_PEAK_TFLOPS}
+        print(json.dumps({"profile": "q8_0_mul_mat_4096x1024x16384", **fig(s), "how": "the first 5 calls of the process after 2 warm-up calls",
+                          "sustained": {k: {**fig(float(np.median(v))), "rounds_us": [x * 1e6 for x in v]} for k, v in turns.items()},
+                          "VX_GEMM_LDS": os.environ.get("VX_GEMM_LDS", "1")}))
         return
     if args.profile == "cfm":       # config 3: whole CFM solves of one request, replayed from a HIP graph
         print(json.dumps({"profile": "cfg3_cfm_solve_one_request", **cfm_solve_bench(pkg, timer, torch.cuda.Stream(), 1, False)}))
@@ -900,6 +927,10 @@ def main():
             wbytes = M * K // 32 * 34
             others[name] = {"us": s * 1e6, "weight_GB/s": wbytes / s / 1e9, "TFLOP/s": 2.0 * M * K * N / s / 1e12,
                             "launch": "64 calls per HIP graph replay (the same weights: they stay in cache)" if N <= 16 else "eager"}
+            if N >= 16384 and M >= 4096:   # the same call in turns with the weights declared constant (vx_weights_pin: their tiles are made once)
+                turns = pinned_in_turns(pkg, timer, call, keep[0], 3, 20)
+                others[name]["in_turns"] = {k: {"us": float(np.median(v)) * 1e6, "TFLOP/s": 2.0 * M * K * N / float(np.median(v)) / 1e12,
+                                                "rounds_us": [x * 1e6 for x in v]} for k, v in turns.items()}
             del keep, call
         torch.cuda.empty_cache()
 

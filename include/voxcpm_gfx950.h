@@ -83,6 +83,19 @@ VX_API vx_status    vx_workspace_reserve(vx_stream stream, size_t bytes);
 /* current block, its size and the number of superseded blocks still held for this stream (any out pointer may be NULL) */
 VX_API vx_status    vx_workspace_info(vx_stream stream, void ** ptr, size_t * bytes, int * retired_blocks);
 
+/* Constant weights.  ggml marks the buffers that hold a model's weights (ggml_backend_buffer_set_usage(...,
+ * GGML_BACKEND_BUFFER_USAGE_WEIGHTS), the reference's src/weight-store.cpp:86 and src/minicpm.cpp:472); this is the same
+ * statement for the C ABI.  For a tensor that lies wholly inside a pinned range an operator may keep a re-laid-out copy
+ * between calls instead of producing it on every call (today: the tiles of the Q8_0 weights of products with 1024 tokens
+ * or more, 2.1 bytes per weight, at most VX_DERIVED_WEIGHTS_MB megabytes per process, default 8192).  Results do not
+ * depend on it.  The owner of the memory calls vx_weights_changed for every range it writes to afterwards (copies derived
+ * from those bytes are dropped), and vx_weights_unpin(base) before it frees or reuses the memory.  Ranges are per device
+ * (the current one); the calls are thread-safe.  vx_weights_info reports the ranges pinned and the copies held. */
+VX_API vx_status    vx_weights_pin(const void * base, size_t bytes);
+VX_API vx_status    vx_weights_changed(const void * base, size_t bytes);
+VX_API vx_status    vx_weights_unpin(const void * base);
+VX_API vx_status    vx_weights_info(size_t * pinned_ranges, size_t * derived_copies, size_t * derived_bytes);
+
 /* Recording the launches of a stream and replaying them as one unit (a HIP graph).  The reference builds and launches
  * its step graph anew on every call (src/voxcpm.cpp:485-495); a backend that recognises a graph it has already run can
  * replay the recorded launches instead of issuing them one by one.  Between begin and end every vx_* call on `stream`

@@ -252,6 +252,8 @@ struct backbone {
     bool  use_mup, fused_glu;
     ggml_context *        wctx = nullptr;
     ggml_backend_buffer_t wbuf = nullptr;
+    ggml_context *        cctx = nullptr; // the KV cache: a buffer of its own, as MiniCPMKVCache allocates it (src/minicpm.cpp:178-187)
+    ggml_backend_buffer_t cbuf = nullptr;
     ggml_context *        fctx = nullptr;
     ggml_backend_buffer_t fbuf = nullptr;
     std::vector<bb_layer> layers;
@@ -357,6 +359,8 @@ void rh_bb_free(void) {
     if (!g_bb) return;
     if (g_bb->fbuf) ggml_backend_buffer_free(g_bb->fbuf);
     if (g_bb->fctx) ggml_free(g_bb->fctx);
+    if (g_bb->cbuf) ggml_backend_buffer_free(g_bb->cbuf);
+    if (g_bb->cctx) ggml_free(g_bb->cctx);
     if (g_bb->wbuf) ggml_backend_buffer_free(g_bb->wbuf);
     if (g_bb->wctx) ggml_free(g_bb->wctx);
     delete g_bb;
@@ -374,20 +378,24 @@ int rh_bb_create(int n_layer, int hidden, int n_heads, int n_kv, int head_dim, i
     m->residual_scale = use_mup ? scale_depth / sqrtf((float) (n_layer > 0 ? n_layer : 1)) : 1.0f;
     ggml_init_params ip = { ggml_tensor_overhead() * ((size_t) n_layer * 11 + 4), nullptr, true };
     m->wctx = ggml_init(ip);
+    m->cctx = ggml_init(ip);
     const int64_t qd = (int64_t) n_heads * head_dim, kd = (int64_t) n_kv * head_dim;
     const int64_t shapes[7][2] = { { hidden, qd }, { hidden, kd }, { hidden, kd }, { qd, hidden }, { hidden, ffn }, { hidden, ffn }, { ffn, hidden } };
     m->layers.resize((size_t) n_layer);
     for (auto & L : m->layers) {
         for (int i = 0; i < 7; ++i) L.w[i] = ggml_new_tensor_2d(m->wctx, GGML_TYPE_Q8_0, shapes[i][0], shapes[i][1]);
         for (int i = 0; i < 2; ++i) L.ln[i] = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, hidden);
-        L.kc = ggml_new_tensor_4d(m->wctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
-        L.vc = ggml_new_tensor_4d(m->wctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
+        L.kc = ggml_new_tensor_4d(m->cctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
+        L.vc = ggml_new_tensor_4d(m->cctx, (ggml_type) kv_type, head_dim, max_len, n_kv, batch);
     }
     m->final_norm   = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, hidden);
     m->rope_factors = ggml_new_tensor_1d(m->wctx, GGML_TYPE_F32, head_dim / 2);
     m->wbuf = ggml_backend_alloc_ctx_tensors(m->wctx, g_backend);
-    if (!m->wbuf) { g_bb = m; rh_bb_free(); return 101; }
+    m->cbuf = ggml_backend_alloc_ctx_tensors(m->cctx, g_backend);
+    if (!m->wbuf || !m->cbuf) { g_bb = m; rh_bb_free(); return 101; }
+    ggml_backend_buffer_set_usage(m->wbuf, GGML_BACKEND_BUFFER_USAGE_WEIGHTS); // src/weight-store.cpp:86
     ggml_backend_buffer_clear(m->wbuf, 0);
+    ggml_backend_buffer_clear(m->cbuf, 0);
     // mlp_forward fuses SwiGLU when the weights are not in host memory (src/minicpm.cpp:729-745)
     m->fused_glu = !ggml_backend_buffer_is_host(m->wbuf);
     g_bb = m;
@@ -418,6 +426,7 @@ int rh_bb_fuse_weights(void) {
     }
     m.fbuf = ggml_backend_alloc_ctx_tensors(m.fctx, g_backend);
     if (!m.fbuf) return 101;
+    ggml_backend_buffer_set_usage(m.fbuf, GGML_BACKEND_BUFFER_USAGE_WEIGHTS); // src/minicpm.cpp:472
     std::vector<uint8_t> scratch;
     auto copy_rows = [&](ggml_tensor * src, ggml_tensor * dst, int64_t row0) {
         scratch.resize(ggml_nbytes(src));

@@ -385,14 +385,20 @@ def ref_backbone_create(params, max_len, batch, use_mup=False, kv_f16=False, eps
     rc = lib.rh_bb_create(d["n_layer"], d["hidden"], d["n_heads"], d["n_kv"], d["head_dim"], d["ffn"], max_len, batch,
                           eps, int(use_mup), 1.4, 1 if kv_f16 else 0)
     assert rc == 0, rc
+    ref_backbone_upload(params)
+    if fused_weights:
+        assert lib.rh_bb_fuse_weights() == 0
+
+
+def ref_backbone_upload(params):
+    """(Re-)uploads params into the decoder stack that exists: the same tensors at the same addresses."""
+    lib = load_ref()
     for li, lw in enumerate(params["layers"]):
         for wi, n in enumerate(BB_WEIGHTS + ("input_layernorm", "post_layernorm")):
             a = np.ascontiguousarray(lw[n])
             assert lib.rh_bb_set(li, wi, a.ctypes.data, a.nbytes) == 0, (li, n)
     assert lib.rh_bb_set(-1, 0, params["final_norm"].ctypes.data, params["final_norm"].nbytes) == 0
     assert lib.rh_bb_set(-1, 1, params["rope_factors"].ctypes.data, params["rope_factors"].nbytes) == 0
-    if fused_weights:
-        assert lib.rh_bb_fuse_weights() == 0
 
 
 def ref_backbone_forward(x, n_past, mask=None, write_kv=True, reps=0):

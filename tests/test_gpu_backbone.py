@@ -535,6 +535,59 @@ def test_plugin_runs_consecutive_decode_steps(gpu, ref, kv_f16):
             assert np.array_equal(a, b), f"cache contents differ (patched recordings, {how})"
 
 
+def test_plugin_follows_weights_rewritten_in_place(gpu, ref, monkeypatch):
+    """The plugin tells the library that a buffer marked GGML_BACKEND_BUFFER_USAGE_WEIGHTS is constant, and the large
+    products then keep their weights' tiles between graphs; a ggml_backend_tensor_set into such a buffer must drop what
+    was derived from the bytes it writes.  A 1024-token prefill, the same again (served from the kept tiles), new weights
+    uploaded into the same tensors, the prefill again: against ggml-cpu on the new weights, and bit for bit against a
+    stack created with the new weights from the start."""
+    import ctypes as C
+    T0, layers = 1024, 2
+    monkeypatch.setenv("VX_GEMM_Q8T", "2")   # (the prefill's products are smaller than what takes the pre-tiled kernel by itself)
+    pa, pb = reflib.backbone_params("pin-a", layers), reflib.backbone_params("pin-b", layers)
+    x = rng("pin", "x").standard_normal((1, T0, 1024)).astype(np.float32)
+    mask = reflib.causal_mask(T0, T0)
+    lib = gpu.lib()
+
+    def held():
+        v = [C.c_size_t() for _ in range(3)]
+        gpu.check(lib.vx_weights_info(*[C.byref(a) for a in v]), "info")
+        return tuple(a.value for a in v)
+
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    base = held()
+    assert ref.rh_use_device(b"GFX950_0", 8, 0) == 0
+    try:
+        reflib.ref_backbone_create(pa, T0 + 8, 1, use_mup=True, kv_f16=True)
+        a1 = reflib.ref_backbone_forward(x, 0, mask)[0]
+        h1 = held()
+        print(f"weights buffer pinned: {h1[0] - base[0]} range, {h1[1] - base[1]} copies, {(h1[2] - base[2]) >> 20} MiB", flush=True)
+        assert h1[0] == base[0] + 1 and h1[1] > base[1]
+        a2 = reflib.ref_backbone_forward(x, 0, mask)[0]
+        assert held() == h1 and np.array_equal(a1, a2)
+        reflib.ref_backbone_upload(pb)
+        assert held()[1] == base[1], "copies of rewritten weights were kept"
+        b1 = reflib.ref_backbone_forward(x, 0, mask)[0]
+        b2 = reflib.ref_backbone_forward(x, 0, mask)[0]
+        assert np.array_equal(b1, b2) and not np.array_equal(a1, b1)
+        ref.rh_bb_free()
+        assert held() == base, "freeing the buffer left a pinned range or copies behind"
+        reflib.ref_backbone_create(pb, T0 + 8, 1, use_mup=True, kv_f16=True)
+        fresh = reflib.ref_backbone_forward(x, 0, mask)[0]
+        assert np.array_equal(b1, fresh), "results after an in-place upload differ from a stack created with those weights"
+    finally:
+        ref.rh_bb_free()
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
+    reflib.ref_backbone_create(pb, T0 + 8, 1, use_mup=True, kv_f16=True)
+    try:
+        cpu = reflib.ref_backbone_forward(x, 0, mask)[0]
+    finally:
+        ref.rh_bb_free()
+    e = nmse(cpu, b1)
+    print(f"   prefill after the upload vs ggml-cpu: nmse {e:.3e}", flush=True)
+    assert e <= 1e-4
+
+
 def test_plugin_replays_a_recurring_graph(gpu, ref):
     """A graph the plugin has run twice is recorded on its third run and replayed from then on (a CFM solve has the same
     shapes and addresses on every call; the reference rebuilds and relaunches it each time, src/voxcpm.cpp:485-495).

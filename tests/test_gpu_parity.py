@@ -550,6 +550,90 @@ def test_mul_mat_q8_0_pretiled_equals_the_lds_kernel(gpu, M, K, N, batch, folded
         assert torch.equal(a3, b3), float((a3 - b3).abs().max())
 
 
+@pytest.mark.parametrize("folded", [False, True])
+def test_mul_mat_q8_0_pinned_weights_keep_their_tiles(gpu, folded, monkeypatch):
+    """vx_weights_pin: the tiles of pinned Q8_0 weights are made once and kept; the product, the residual update and the
+    gate/up SwiGLU give the same bits as with the tiles made on every call, on the stream that made the copy and on
+    another one; vx_weights_changed drops the copies made from the bytes it names (the next call sees the new weights),
+    vx_weights_unpin drops the rest; nothing is kept for weights outside a pinned range."""
+    import ctypes as C
+    import torch
+    L, d = gpu.lib(), gpu.desc
+    M, K, N = 2048, 1024, 1100
+    monkeypatch.setenv("VX_GEMM_Q8T", "2")
+    if folded:
+        monkeypatch.setenv("VX_GEMM_LDS", "2")
+    else:
+        monkeypatch.delenv("VX_GEMM_LDS", raising=False)
+    mk = lambda *tag: dev(reflib.quantize_q8_0((rng("pin", *tag).standard_normal((M, K)) * 0.02).astype(np.float32)))
+    # one allocation for the two matrices of the pair and a third matrix outside the pinned part
+    pool = torch.empty((3,) + tuple(mk("shape").shape), dtype=torch.uint8, device="cuda")
+    pool[0], pool[1], pool[2] = mk("w"), mk("w2"), mk("w3")
+    wq, wq2, wq3 = pool[0], pool[1], pool[2]
+    xd = dev(rng("pin", "x").standard_normal((N, K)).astype(np.float32))
+    res = dev(rng("pin", "res").standard_normal((N, M)).astype(np.float32))
+
+    def info():
+        v = [C.c_size_t() for _ in range(3)]
+        gpu.check(L.vx_weights_info(*[C.byref(x) for x in v]), "info")
+        return tuple(x.value for x in v)
+
+    def three(w=wq):
+        a = gpu.mul_mat(w, xd, gpu.ACT_FLOAT, w_ne0=K)
+        b, c = torch.empty_like(a), torch.empty_like(a)
+        gpu.check(L.vx_mul_mat_scale_add(gpu.desc_q8(w, K), d(xd), d(res), d(b), 0.2857738, gpu.ACT_FLOAT, gpu._stream()), "scale_add")
+        gpu.check(L.vx_mul_mat_swiglu(gpu.desc_q8(w, K), gpu.desc_q8(wq2, K), d(xd), d(c), gpu.ACT_FLOAT, gpu._stream()), "swiglu")
+        torch.cuda.synchronize()
+        return a, b, c
+
+    base = info()
+    plain = three()
+    assert info() == base, "a copy was kept for weights nobody pinned"
+    say(f"pinned Q8_0 weights, folded={folded}")
+    one = wq.numel()
+    gpu.check(L.vx_weights_pin(pool.data_ptr(), 2 * one), "pin")
+    try:
+        first = three()                      # makes the copies (single matrix, pair)
+        held = info()
+        assert held[0] == base[0] + 1 and held[1] == base[1] + 2 and held[2] - base[2] >= 3 * 2 * M * K
+        again = three()
+        assert info() == held
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            other = three()                  # the copies were filled on another stream
+        for want, a, b, c in zip(plain, first, again, other):
+            assert torch.equal(want, a) and torch.equal(want, b) and torch.equal(want, c)
+        p3 = three(wq3)                      # outside the pinned bytes: the pair (wq3, wq2) is not kept either
+        assert info() == held
+        # new weights at the same address
+        wq.copy_(mk("w, rewritten"))
+        gpu.check(L.vx_weights_changed(wq.data_ptr(), one), "changed")
+        assert info()[1] == base[1]          # both copies held bytes of the first matrix
+        monkeypatch.setenv("VX_GEMM_Q8T", "0")
+        want = three()
+        monkeypatch.setenv("VX_GEMM_Q8T", "2")
+        got, got2 = three(), three()
+        for w_, a, b in zip(want, got, got2):
+            assert torch.equal(w_, a) and torch.equal(w_, b)
+        assert not torch.equal(got[0], plain[0])
+        assert info() == held
+        # under a recording nothing is taken from the copies (a recording must not hold their addresses)
+        g = torch.cuda.CUDAGraph()
+        out = torch.empty_like(got[0])
+        gpu.check(L.vx_workspace_reserve(side.cuda_stream, 64 << 20), "reserve")
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                gpu.mul_mat(wq, xd, gpu.ACT_FLOAT, w_ne0=K, out=out)
+        gpu.check(L.vx_weights_unpin(pool.data_ptr()), "unpin")
+        assert info() == base
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, got[0])
+    finally:
+        L.vx_weights_unpin(pool.data_ptr())
+    assert L.vx_weights_unpin(pool.data_ptr()) == 3   # VX_ERR_INVALID: nothing is pinned there any more
+
+
 @pytest.mark.parametrize("seed", list(range(48)))
 def test_mul_mat_q8_0_random_shapes(gpu, seed):
     """Random row, column and token counts around every threshold the launcher has (streaming kernel up to 16 tokens and a

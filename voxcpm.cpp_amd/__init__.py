@@ -54,6 +54,7 @@ EXPORTS = [
     "vx_stream_create", "vx_stream_destroy", "vx_stream_synchronize", "vx_workspace_reserve", "vx_workspace_info",
     "vx_graph_begin", "vx_graph_end", "vx_graph_launch", "vx_graph_destroy",
     "vx_graph_patchable", "vx_graph_patch_begin", "vx_graph_patch_end",
+    "vx_weights_pin", "vx_weights_changed", "vx_weights_unpin", "vx_weights_info",
     "vx_rms_norm", "vx_rope", "vx_soft_max", "vx_flash_attn_ext", "vx_flash_attn_ext_static", "vx_mul_mat",
     "vx_supports_rms_norm", "vx_supports_rope", "vx_supports_soft_max", "vx_supports_flash_attn_ext",
     "vx_supports_mul_mat", "vx_kv_read_view", "vx_kv_write_view", "vx_kv_store",
@@ -107,6 +108,10 @@ def lib():
     l.vx_graph_patchable.argtypes = [vp]
     l.vx_graph_patch_begin.argtypes = [vp]
     l.vx_graph_patch_end.argtypes = [vp, C.POINTER(C.c_int)]
+    l.vx_weights_pin.argtypes = [vp, C.c_size_t]
+    l.vx_weights_changed.argtypes = [vp, C.c_size_t]
+    l.vx_weights_unpin.argtypes = [vp]
+    l.vx_weights_info.argtypes = [C.POINTER(C.c_size_t)] * 3
     l.vx_workspace_reserve.argtypes = [vp, C.c_size_t]
     l.vx_workspace_info.argtypes = [vp, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
     l.vx_rms_norm.argtypes = [TP, TP, C.c_float, vp]

@@ -51,6 +51,7 @@ class MiniCPMBackbone:
         self.k_cache = [torch.zeros((batch, n_kv_heads, max_length, head_dim), dtype=self.kv_dtype, device=dev) for _ in range(n_layer)]
         self.v_cache = [torch.zeros((batch, n_kv_heads, max_length, head_dim), dtype=self.kv_dtype, device=dev) for _ in range(n_layer)]
         self.weights = [dict() for _ in range(n_layer)]   # name -> (uint8 Q8_0 rows, K)
+        self._pinned = {}                                 # base address -> tensor, for the ranges given to vx_weights_pin
         self.norms = [dict() for _ in range(n_layer)]     # "input_layernorm" / "post_layernorm" -> f32 [hidden]
         self.final_norm = None
         self.rope_factors = None                          # f32 [head_dim / 2] or None
@@ -58,7 +59,30 @@ class MiniCPMBackbone:
     # ---- loading --------------------------------------------------------------------------
     def set_weight(self, layer, name, q8_rows, K):
         """q8_rows: uint8 tensor (rows, K/32*34) of Q8_0 blocks, on the device."""
+        self.unpin_weights()
         self.weights[layer][name] = (q8_rows, K)
+
+    def pin_weights(self):
+        """Declare the loaded weights constant (vx_weights_pin), as the reference marks its weight buffers
+        (src/weight-store.cpp:86): the large products then keep their weights' tiles between calls.  The tensors must
+        not be written to or released while pinned; set_weight and the destructor unpin."""
+        for layer in self.weights:
+            for q8_rows, _ in layer.values():
+                base, size = q8_rows.data_ptr(), q8_rows.numel() * q8_rows.element_size()
+                if base not in self._pinned:
+                    check(lib().vx_weights_pin(base, size), "vx_weights_pin")
+                    self._pinned[base] = q8_rows   # (kept alive while pinned)
+
+    def unpin_weights(self):
+        for base in list(self._pinned):
+            lib().vx_weights_unpin(base)
+            del self._pinned[base]
+
+    def __del__(self):
+        try:
+            self.unpin_weights()
+        except Exception:
+            pass
 
     def set_norm(self, layer, name, w):
         if layer < 0:

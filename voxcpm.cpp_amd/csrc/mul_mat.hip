@@ -2175,10 +2175,6 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     q.n_rt = (int) ((MV + 15) / 16); q.n_tt = (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
     const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * ((q.n_rt + 3) & ~3) * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
     const size_t xt_bytes = (size_t) nbatch * q.n_kb * q.n_tt * 1024;
-    void * ws = nullptr;
-    if ((t_ws_status = vx_workspace(st, a.ws_offset + wt_bytes + wd_bytes + xt_bytes, &ws)) != VX_OK) { (void) hipGetLastError(); return false; }
-    char * base = (char *) ws + a.ws_offset;
-    q.wt = (half8_t *) base; q.wdt = (float *) (base + wt_bytes); q.xt = (half8_t *) (base + wt_bytes + wd_bytes);
     static bool raised = false;
     if (!raised) {
         if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
@@ -2192,11 +2188,27 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     }
     const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) ((q.n_kb + QT_ACT_UNROLL - 1) / QT_ACT_UNROLL) * q.n_tt * 64;
     if ((wunits + 255) / 256 > 0x7fffffff || (xunits + 255) / 256 > 0x7fffffff) return false;
-    vx_launch(qt_weights_kernel, dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st, q);
-    vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
     const int gx = (q.n_rt + 15) / 16, gy = (q.n_tt + 7) / 8, Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
     const int64_t blocks = ((int64_t) Gx * Gy + 7) / 8 * 8 * 32;
     if (blocks > 0x7fffffff) return false;
+    // the weights' tiles: kept from call to call when the caller has pinned the weights, else made in the workspace
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void) hipGetLastError(); return false; }
+    const vx_derived_key key = { dev, fold ? 2 : 1, a.w, DUAL ? a.w2 : nullptr, a.K, a.M, a.nb01 };
+    bool fresh = false;
+    char * kept = (char *) vx_derived_get(key, wt_bytes + wd_bytes, st, &fresh);
+    void * ws = nullptr;
+    if ((t_ws_status = vx_workspace(st, a.ws_offset + (kept ? 0 : wt_bytes + wd_bytes) + xt_bytes, &ws)) != VX_OK) {
+        (void) hipGetLastError();
+        if (fresh) vx_derived_abandon(key, st);
+        return false;
+    }
+    char * base = (char *) ws + a.ws_offset;
+    if (kept) { q.wt = (half8_t *) kept; q.wdt = (float *) (kept + wt_bytes); q.xt = (half8_t *) base; }
+    else      { q.wt = (half8_t *) base; q.wdt = (float *) (base + wt_bytes); q.xt = (half8_t *) (base + wt_bytes + wd_bytes); }
+    if (!kept || fresh) vx_launch(qt_weights_kernel, dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st, q);
+    if (fresh) vx_derived_filled(key, st);
+    vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
     if (fold) vx_launch(gemm_q8t_kernel<DUAL, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     else      vx_launch(gemm_q8t_kernel<DUAL, false>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     return true;

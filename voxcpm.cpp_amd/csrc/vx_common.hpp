@@ -67,6 +67,22 @@ inline void vx_launch(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds_by
 // already captured keep valid arguments; growth during a stream capture is refused.
 vx_status vx_workspace(hipStream_t stream, size_t bytes, void ** ptr);
 
+// Copies derived from pinned weights (vx_weights_pin), kept from call to call.  vx_derived_get returns the copy for `key`
+// (the calling stream is made to wait for the kernel that filled it, if that ran on another stream), or a new block of
+// `bytes` with *fresh set -- the caller then fills it on `stream` and calls vx_derived_filled -- or null: the weights are
+// not pinned, launches are being recorded or compared, the stream is under capture, or the budget is spent.
+struct vx_derived_key {
+    int          dev;
+    int          kind;     // which layout (and variant of it)
+    const void * w;
+    const void * w2;       // second matrix of a pair, or null
+    int64_t      K, M;
+    uint64_t     nb01;
+};
+void * vx_derived_get(const vx_derived_key & key, size_t bytes, hipStream_t stream, bool * fresh);
+void   vx_derived_filled(const vx_derived_key & key, hipStream_t stream);
+void   vx_derived_abandon(const vx_derived_key & key, hipStream_t stream); // a fresh block that will not be filled after all
+
 // vx_flash_attn_ext_static's fixed scratch array (fattn.hip): the per-device address lookup that vx_init performs
 // so that the first call of the entry point does no set-up work
 vx_status vx_fattn_static_setup(void);

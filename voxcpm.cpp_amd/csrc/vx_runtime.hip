@@ -2,6 +2,7 @@
 #include "vx_common.hpp"
 #include "ws_policy.hpp"
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -52,9 +53,113 @@ void destroy_recorded(recorded_graph * r) {
     delete r;
 }
 
+// ---- pinned weights and what is derived from them -----------------------------------------------------------------
+// A caller may declare ranges of device memory constant (vx_weights_pin).  For tensors inside such a range an operator
+// may keep a re-laid-out copy from one call to the next (the pre-tiled Q8_0 weights of the large products) instead of
+// producing it on every call; vx_weights_changed / vx_weights_unpin drop whatever was derived from the bytes they name.
+struct pinned_range { int dev; uintptr_t lo, hi; };
+struct derived_entry {
+    vx_derived_key key;
+    uintptr_t      src[2][2]; // the byte ranges it was derived from (second one empty for a single matrix)
+    void *         ptr;
+    size_t         bytes;
+    hipEvent_t     ready;     // recorded behind the kernel that fills it
+    hipStream_t    filled_on;
+    bool           filled;
+};
+std::mutex                 g_pin_mutex;
+std::vector<pinned_range>  g_pinned;
+std::vector<derived_entry> g_derived;
+size_t                     g_derived_bytes = 0;
+
+bool same_key(const vx_derived_key & a, const vx_derived_key & b) {
+    return a.dev == b.dev && a.kind == b.kind && a.w == b.w && a.w2 == b.w2 && a.K == b.K && a.M == b.M && a.nb01 == b.nb01;
+}
+bool inside_pinned(int dev, uintptr_t lo, uintptr_t hi) { // (g_pin_mutex held)
+    for (const pinned_range & r : g_pinned) if (r.dev == dev && lo >= r.lo && hi <= r.hi) return true;
+    return false;
+}
+void drop_derived_from(int dev, uintptr_t lo, uintptr_t hi) { // (g_pin_mutex held) hipFree waits for the kernels still reading
+    for (size_t i = 0; i < g_derived.size();) {
+        derived_entry & e = g_derived[i];
+        bool hit = false;
+        for (int k = 0; k < 2; ++k) hit = hit || (e.src[k][0] < e.src[k][1] && e.src[k][0] < hi && lo < e.src[k][1]);
+        if (e.key.dev == dev && hit) {
+            (void) hipFree(e.ptr);
+            if (e.ready) (void) hipEventDestroy(e.ready);
+            g_derived_bytes -= e.bytes;
+            g_derived[i] = g_derived.back();
+            g_derived.pop_back();
+        } else ++i;
+    }
+}
+size_t derived_cap() { // bytes this process may hold in derived copies (VX_DERIVED_WEIGHTS_MB, default 8192; 0 keeps none)
+    static const size_t cap = [] { const char * e = getenv("VX_DERIVED_WEIGHTS_MB"); return (size_t) (e ? atoll(e) : 8192) << 20; }();
+    return cap;
+}
+
 } // namespace
 
 thread_local int vx_tl_launch_mode = 0;
+
+void * vx_derived_get(const vx_derived_key & key, size_t bytes, hipStream_t stream, bool * fresh) {
+    *fresh = false;
+    // Not while launches are recorded, compared or captured: a fill would be recorded (or not run at all), a capture may
+    // not allocate, and a recording must not hold the address of a copy that a later vx_weights_changed frees.
+    if (vx_tl_launch_mode != 0) return nullptr;
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    if (g_pinned.empty()) return nullptr;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
+    if (cs != hipStreamCaptureStatusNone) return nullptr;
+    for (derived_entry & e : g_derived)
+        if (same_key(e.key, key) && e.bytes == bytes) {
+            if (!e.filled) return nullptr; // (a fill that was never confirmed: not used)
+            if (e.filled_on != stream && hipStreamWaitEvent(stream, e.ready, 0) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
+            return e.ptr;
+        }
+    const uintptr_t w = (uintptr_t) key.w, w2 = (uintptr_t) key.w2, span = (uintptr_t) key.M * key.nb01;
+    if (!inside_pinned(key.dev, w, w + span) || (w2 && !inside_pinned(key.dev, w2, w2 + span))) return nullptr;
+    if (g_derived_bytes + bytes > derived_cap()) return nullptr;
+    derived_entry e = {};
+    e.key = key;
+    e.src[0][0] = w; e.src[0][1] = w + span;
+    e.src[1][0] = w2; e.src[1][1] = w2 ? w2 + span : 0;
+    e.bytes = bytes;
+    if (hipMalloc(&e.ptr, bytes) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
+    if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess) { (void) hipGetLastError(); (void) hipFree(e.ptr); return nullptr; }
+    e.filled_on = stream;
+    e.filled = false;
+    g_derived.push_back(e);
+    g_derived_bytes += bytes;
+    *fresh = true;
+    return e.ptr;
+}
+
+void vx_derived_abandon(const vx_derived_key & key, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    for (size_t i = 0; i < g_derived.size(); ++i) {
+        derived_entry & e = g_derived[i];
+        if (same_key(e.key, key) && !e.filled && e.filled_on == stream) {
+            (void) hipFree(e.ptr);
+            (void) hipEventDestroy(e.ready);
+            g_derived_bytes -= e.bytes;
+            g_derived[i] = g_derived.back();
+            g_derived.pop_back();
+            return;
+        }
+    }
+}
+
+void vx_derived_filled(const vx_derived_key & key, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    for (derived_entry & e : g_derived)
+        if (same_key(e.key, key) && !e.filled && e.filled_on == stream) {
+            if (hipEventRecord(e.ready, stream) == hipSuccess) e.filled = true;
+            else (void) hipGetLastError();
+            return;
+        }
+}
 
 void vx_launch_note(const void * func, dim3 grid, dim3 block, size_t lds_bytes, void * const * params, const size_t * sizes, int n_params) {
     recorded_graph * r = t_rec;
@@ -375,6 +480,46 @@ vx_status vx_graph_patch_end(vx_graph graph, int * patched) {
     if (patched) *patched = t_patched;
     if (t_differs || t_next != r->launches.size())
         return vx_fail(VX_ERR_UNSUPPORTED, "vx_graph_patch_end: the launches differ from the recording's (%zu of %zu matched)", t_next, r->launches.size());
+    return VX_OK;
+}
+vx_status vx_weights_pin(const void * base, size_t bytes) {
+    if (!base || !bytes) return vx_fail(VX_ERR_INVALID, "vx_weights_pin: empty range");
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    for (const pinned_range & r : g_pinned)
+        if (r.dev == dev && r.lo == (uintptr_t) base) {
+            if (r.hi == (uintptr_t) base + bytes) return VX_OK;
+            return vx_fail(VX_ERR_INVALID, "vx_weights_pin: a range of another size is pinned at this address");
+        }
+    g_pinned.push_back({ dev, (uintptr_t) base, (uintptr_t) base + bytes });
+    return VX_OK;
+}
+vx_status vx_weights_changed(const void * base, size_t bytes) {
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    if (!g_derived.empty()) drop_derived_from(dev, (uintptr_t) base, (uintptr_t) base + bytes);
+    return VX_OK;
+}
+vx_status vx_weights_unpin(const void * base) {
+    int dev = 0;
+    VX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    for (size_t i = 0; i < g_pinned.size(); ++i)
+        if (g_pinned[i].dev == dev && g_pinned[i].lo == (uintptr_t) base) {
+            drop_derived_from(dev, g_pinned[i].lo, g_pinned[i].hi);
+            g_pinned[i] = g_pinned.back();
+            g_pinned.pop_back();
+            return VX_OK;
+        }
+    return vx_fail(VX_ERR_INVALID, "vx_weights_unpin: no range is pinned at this address");
+}
+vx_status vx_weights_info(size_t * pinned_ranges, size_t * derived_copies, size_t * derived_bytes) {
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    if (pinned_ranges) *pinned_ranges = g_pinned.size();
+    if (derived_copies) *derived_copies = g_derived.size();
+    if (derived_bytes) *derived_bytes = g_derived_bytes;
     return VX_OK;
 }
 vx_status vx_stream_synchronize(vx_stream stream) {

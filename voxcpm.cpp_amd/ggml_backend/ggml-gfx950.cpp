@@ -137,6 +137,7 @@ struct backend_ctx {
 struct buffer_ctx {
     int    device;
     void * base;
+    bool   pinned = false; // declared constant to the library (vx_weights_pin): writes into it are reported
 };
 
 ggml_backend_buffer_type_t device_buffer_type(ggml_backend_dev_t dev);
@@ -145,8 +146,24 @@ ggml_backend_buffer_type_t device_buffer_type(ggml_backend_dev_t dev);
 void buffer_free(ggml_backend_buffer_t buffer) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     vx_init(ctx->device);
+    if (ctx->pinned) vx_weights_unpin(ctx->base);
     vx_free(ctx->base);
     delete ctx;
+}
+
+// The caller's statement that a buffer holds weights (ggml_backend_buffer_set_usage(..., GGML_BACKEND_BUFFER_USAGE_WEIGHTS):
+// the reference's src/weight-store.cpp:86, src/minicpm.cpp:472) is passed on to the library when a product first reads a
+// weight from the buffer: the library may then keep re-laid-out copies of those weights between calls.  Every write into
+// such a buffer -- through the buffer interface, the backend's asynchronous upload or a graph node -- is reported, which
+// drops the copies made from the bytes written.
+void pin_if_weights(ggml_backend_buffer_t buffer) {
+    if (!buffer || buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS || buffer->iface.free_buffer != buffer_free) return;
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    if (!ctx->pinned && vx_weights_pin(ctx->base, buffer->size) == VX_OK) ctx->pinned = true;
+}
+void written_to(ggml_backend_buffer_t buffer, const void * p, size_t bytes) {
+    if (!buffer || buffer->iface.free_buffer != buffer_free) return;
+    if (((buffer_ctx *) buffer->context)->pinned) vx_weights_changed(p, bytes);
 }
 
 void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) buffer->context)->base; }
@@ -154,6 +171,7 @@ void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) bu
 void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     vx_init(ctx->device);
+    written_to(buffer, (char *) tensor->data + offset, size);
     if (vx_memset((char *) tensor->data + offset, value, size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
         GGML_ABORT("ggml-gfx950: memset_tensor failed: %s", vx_last_error());
 }
@@ -161,6 +179,7 @@ void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, ui
 void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     vx_init(ctx->device);
+    written_to(buffer, (char *) tensor->data + offset, size);
     if (vx_memcpy_h2d((char *) tensor->data + offset, data, size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
         GGML_ABORT("ggml-gfx950: set_tensor failed: %s", vx_last_error());
 }
@@ -176,6 +195,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
     vx_init(ctx->device);
+    written_to(buffer, dst->data, ggml_nbytes(dst));
     vx_status rc;
     if (ggml_backend_buffer_is_host(src->buffer)) {
         rc = vx_memcpy_h2d(dst->data, src->data, ggml_nbytes(src), nullptr);
@@ -192,6 +212,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
 void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     vx_init(ctx->device);
+    written_to(buffer, ctx->base, buffer->size);
     if (vx_memset(ctx->base, value, buffer->size, nullptr) != VX_OK || vx_stream_synchronize(nullptr) != VX_OK)
         GGML_ABORT("ggml-gfx950: clear failed: %s", vx_last_error());
 }
@@ -506,6 +527,7 @@ void backend_synchronize(ggml_backend_t backend) {
 void backend_set_tensor_async(ggml_backend_t backend, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     vx_init(ctx->device);
+    written_to(tensor->buffer, (char *) tensor->data + offset, size);
     if (vx_memcpy_h2d((char *) tensor->data + offset, data, size, ctx->stream) != VX_OK)
         GGML_ABORT("ggml-gfx950: set_tensor_async failed: %s", vx_last_error());
 }
@@ -1341,6 +1363,10 @@ uint64_t graph_fingerprint(const ggml_cgraph * g) {
 }
 
 ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * launches_out);
+// A node that fails while a recording is being made (a launch that would have to grow the workspace under the capture)
+// is no error and is not logged: the recording is dropped and the graph is launched node by node.
+bool g_trial_pass = false;
+#define NODE_FAILED(...) do { if (!g_trial_pass) GGML_LOG_ERROR(__VA_ARGS__); } while (0)
 int g_patch_on = -1;     // run a decode loop's steps as patched recordings (GGML_GFX950_GRAPH_PATCH, ggml_backend_gfx950_set_graph_patch)
 int g_patched_replays = 0; // graph_compute calls served by a recording whose arguments were brought up to date first
 int g_last_patched = 0;    // nodes whose arguments the most recent such call changed
@@ -1359,7 +1385,9 @@ bool family_compute(backend_ctx * ctx, step_family & fam, ggml_cgraph * cgraph) 
     int launches = 0;
     if (rec) {
         if (vx_graph_patch_begin(rec) == VX_OK) {
+            g_trial_pass = true;
             const ggml_status st = graph_compute_eager(ctx, cgraph, &launches); // compares, launches nothing
+            g_trial_pass = false;
             int patched = 0;
             const bool same = vx_graph_patch_end(rec, &patched) == VX_OK;
             if (st == GGML_STATUS_SUCCESS && same && vx_graph_launch(rec, ctx->stream) == VX_OK) {
@@ -1377,7 +1405,9 @@ bool family_compute(backend_ctx * ctx, step_family & fam, ggml_cgraph * cgraph) 
         return false;
     }
     if (vx_graph_begin(ctx->stream) != VX_OK) { ++fam.failures; return false; }
+    g_trial_pass = true;
     const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+    g_trial_pass = false;
     vx_graph made = nullptr;
     vx_graph_end(ctx->stream, &made);
     if (st == GGML_STATUS_SUCCESS && made && vx_graph_patchable(made) && vx_graph_launch(made, ctx->stream) == VX_OK) {
@@ -1478,7 +1508,9 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     }
     if (entry->runs >= 3 && !entry->no_replay) { // the same graph for the third time: record its launches, then replay them
         if (vx_graph_begin(ctx->stream) == VX_OK) {
+            g_trial_pass = true;
             const ggml_status st = graph_compute_eager(ctx, cgraph, &launches);
+            g_trial_pass = false;
             vx_graph rec = nullptr;
             vx_graph_end(ctx->stream, &rec);
             if (st == GGML_STATUS_SUCCESS && rec && vx_graph_launch(rec, ctx->stream) == VX_OK) {
@@ -1504,6 +1536,11 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
     // readers of every tensor in this graph (as an operand or as the source of a view): a pair of
     // nodes is only run as one launch when nothing else looks at the value between them
     const bool fusion = fusion_on();
+    for (int i = 0; i < cgraph->n_nodes; ++i) { // weights buffers: pinned at their first product, writes into them reported
+        const ggml_tensor * n = cgraph->nodes[i];
+        if (n->op == GGML_OP_MUL_MAT && n->src[0]) pin_if_weights(n->src[0]->buffer);
+        if (n->buffer && n->buffer->usage == GGML_BACKEND_BUFFER_USAGE_WEIGHTS && !ggml_op_is_empty(n->op)) written_to(n->buffer, n->data, ggml_nbytes(n));
+    }
     reader_map readers;
     if (fusion && cgraph->n_nodes > 1) {
         readers.reserve((size_t) cgraph->n_nodes * 2);
@@ -1584,7 +1621,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
             if (grouped) {
                 ++launches;
                 if (rc != VX_OK) {
-                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, rms_norm + projections) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    NODE_FAILED("ggml-gfx950: node %d (%s, rms_norm + projections) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
                     return GGML_STATUS_FAILED;
                 }
                 continue;
@@ -1601,7 +1638,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                 rc = vx_concat_many(tp, tree.extents.data(), (int) tree.leaves.size(), tree.dim, &d, ctx->stream);
                 ++launches;
                 if (rc != VX_OK) {
-                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, a tree of CONCATs) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    NODE_FAILED("ggml-gfx950: node %d (%s, a tree of CONCATs) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
                     return GGML_STATUS_FAILED;
                 }
                 continue;
@@ -1613,7 +1650,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
              compute_fused_gate_up_group(ctx, cgraph, i, readers, done, &rc))) {
             ++launches;
             if (rc != VX_OK) {
-                GGML_LOG_ERROR("ggml-gfx950: node %d (%s, q/k/v projections + rope) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                NODE_FAILED("ggml-gfx950: node %d (%s, q/k/v projections + rope) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
                 return GGML_STATUS_FAILED;
             }
             continue;
@@ -1626,7 +1663,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                 else rc = compute_kv2_attention(ctx, node, it->second);
                 ++launches;
                 if (rc != VX_OK) {
-                    GGML_LOG_ERROR("ggml-gfx950: node %d (%s, two-segment attention) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                    NODE_FAILED("ggml-gfx950: node %d (%s, two-segment attention) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
                     return GGML_STATUS_FAILED;
                 }
                 continue;
@@ -1667,7 +1704,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
         else rc = compute_node(ctx, node);
         ++launches;
         if (rc != VX_OK) {
-            GGML_LOG_ERROR("ggml-gfx950: node %d (%s, op %s) failed with status %d: %s\n", i, node->name,
+            NODE_FAILED("ggml-gfx950: node %d (%s, op %s) failed with status %d: %s\n", i, node->name,
                            ggml_op_name(node->op), (int) rc, rc == VX_ERR_UNSUPPORTED && !*vx_last_error() ? "operator not claimed by this backend" : vx_last_error());
             return GGML_STATUS_FAILED;
         }
