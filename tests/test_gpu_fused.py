@@ -166,8 +166,10 @@ def test_mul_mat_swiglu_tiled(pkg, gpu, M, K, N, nb, wtype):
                                       # a long K over few tiles: the tiled kernels with K cut, the update in the kernel that adds the partials
                                       (1024, 4096, 112, 1), (1000, 4096, 70, 1),
                                       # prefill sizes: the update in the tiled kernels' epilogue (whole and ragged tiles of 64 and of 128),
-                                      # or the plain product and a pass of its own (17 tokens; every shape under VX_ACT_Q8)
-                                      (1024, 1024, 512, 1), (1024, 4096, 300, 1), (1000, 1024, 200, 2), (4096, 1024, 1024, 1), (1024, 4096, 17, 1)])
+                                      # or the plain product and a pass of its own (every shape under VX_ACT_Q8)
+                                      (1024, 1024, 512, 1), (1024, 4096, 300, 1), (1000, 1024, 200, 2), (4096, 1024, 1024, 1),
+                                      # 17 to 63 tokens behind a K the streaming kernel declines: one ragged token tile, K cut
+                                      (1024, 4096, 17, 1), (1024, 4096, 40, 1), (1000, 2304, 63, 2)])
 @pytest.mark.parametrize("act", ["float", "q8"])
 def test_mul_mat_scale_add(pkg, gpu, M, K, N, nb, act):
     import torch

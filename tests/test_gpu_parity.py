@@ -446,7 +446,10 @@ def mm_inputs(tag, M, K, N, batch=()):
                                    (1024, 4352, 1000), (1000, 2176, 600),
                                    # the same on the LDS-operand kernel when its 64 x 64 tiles are few (the down-projection of
                                    # 8 requests' 112 tokens): 8, 8 and 4 splits, ragged rows and tokens
-                                   (1024, 4096, 112), (1000, 4096, 70), (512, 2048, 64)])
+                                   (1024, 4096, 112), (1000, 4096, 70), (512, 2048, 64),
+                                   # 17 to 63 tokens behind a K beyond the streaming kernel's 2048: one ragged token tile of the
+                                   # LDS-operand kernel with its K cut (a short prompt's down-projection)
+                                   (1024, 4096, 17), (1024, 4096, 40), (1000, 2304, 63), (2048, 4096, 33)])
 def test_mul_mat_q8_0(gpu, M, K, N):
     say(f"mul_mat Q8_0 M={M} K={K} N={N}")
     w, x = mm_inputs(("q8", M, K, N), M, K, N)

@@ -2217,7 +2217,10 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
 template <int WT>
 bool launch_gemm_lds(const mm_args & a, int nbatch, hipStream_t st) {
     const int mode = gemm_lds_mode();
-    if (mode == 0 || WT == WT_F32 || a.K % (32 * GL_KC) || a.N < 64 || !a.x_aligned) return false;
+    // (from 17 tokens on: what reaches this point with fewer than 64 is a product the streaming kernel has declined -- K beyond
+    // 2048, or too many rows for its token chunks -- and the one ragged token tile with its K cut is 12 us where the older
+    // kernels took 21 to 54)
+    if (mode == 0 || WT == WT_F32 || a.K % (32 * GL_KC) || a.N <= 16 || !a.x_aligned) return false;
     if (WT == WT_Q8 && !a.w_aligned) return false;
     if (WT == WT_F16 && (((uintptr_t) a.w | a.nb01 | a.nb02 | a.nb03) % 16 != 0)) return false;
     // 32-bit lane offsets: rows of the weight matrix, the (up to 256) tokens of a tile
