@@ -252,14 +252,16 @@ def test_projection_groups_random_shapes(pkg, gpu, seed):  # (seed 29: one produ
         assert L.vx_mul_mat_swiglu(dw, dw2, d(x), d(b), mode, None) != 0
 
 
-@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2)])
+@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2),
+                                        # a short prompt's write: the sums in one work-group, the ADD1 over x a launch of its own
+                                        (1, 48, 2, 64, 16), (1, 64, 2, 64, 16), (2, 20, 2, 64, 16)])
 @pytest.mark.parametrize("poison", [None, "nan", "inf"])
 def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):
     import torch
     say(f"fused cache write + ordering scalar B={B} T={T} Hkv={Hkv} D={D} poison={poison}")
     L, d = pkg.lib(), pkg.desc
     g = rng("f-kvs", B, T, Hkv, D)
-    max_len, n_past = 40, 17
+    max_len, n_past = 40 + T, 17
     k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
     v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
     if poison == "nan":

@@ -981,6 +981,8 @@ struct kvs_args {
     uint64_t nbx[4], nbd[4];
     float scale, bias;
     int dense4; // x and d are contiguous, 16-byte aligned, a multiple of 4 elements: the ADD1 walks them 16 bytes at a time
+    double * defer; // kv_store_sync_kernel leaves the two sums here (in the layout of kv_store_large_kernel's block totals) and the
+                    // ADD1 to kv_sync_add1_kernel: one work-group adding a scalar to a prompt's 64 x 1024 values took 40 us
 };
 
 // stores the slot and returns the sum of what was stored, the same value in every thread of the block
@@ -1014,6 +1016,12 @@ __global__ __launch_bounds__(1024) void kv_store_sync_kernel(const kvs_args a) {
         ox = i0 * a.nbx[0] + i1 * a.nbx[1] + i2 * a.nbx[2] + i3 * a.nbx[3];
         od = i0 * a.nbd[0] + i1 * a.nbd[1] + i2 * a.nbd[2] + i3 * a.nbd[3];
     };
+    if (a.defer) { // (uniform) the sums only: as floats, as the scalar takes them, in the first slot of each half
+        const float sk = a.k.vec ? store_and_sum<true>(a.k, part) : store_and_sum<false>(a.k, part);
+        const float sv = a.v.vec ? store_and_sum<true>(a.v, part) : store_and_sum<false>(a.v, part);
+        if (threadIdx.x < 2 * SUM_BLOCKS) a.defer[threadIdx.x] = threadIdx.x == 0 ? (double) sk : threadIdx.x == SUM_BLOCKS ? (double) sv : 0.0;
+        return;
+    }
     float    xv[KVS_PRE];
     uint64_t xo[KVS_PRE];
 #pragma unroll
@@ -1844,8 +1852,19 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
     for (int i = 0; i < 4; ++i) { a.ne[i] = x->ne[i]; a.nbx[i] = x->nb[i]; a.nbd[i] = dst->nb[i]; }
     a.scale = scale; a.bias = bias;
     a.dense4 = vx_is_contiguous(x) && vx_is_contiguous(dst) && vx_nelements(x) % 4 == 0 && ((uintptr_t) x->data | (uintptr_t) dst->data) % 16 == 0;
+    a.defer = nullptr;
     if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) {
+        // beyond a few thousand values of x the ADD1 is a launch of its own over many work-groups (the sums stay with the one
+        // work-group whose order they are defined by); a workspace that cannot be had (a capture without a reservation)
+        // leaves everything in the one launch
+        void * ws = nullptr;
+        if (vx_nelements(x) > 16384 && vx_workspace((hipStream_t) stream, 2 * SUM_BLOCKS * sizeof(double), &ws) == VX_OK) a.defer = (double *) ws;
+        else (void) hipGetLastError();
         vx_launch(kv_store_sync_kernel, dim3(1), dim3(1024), 0, (hipStream_t) stream, a);
+        if (a.defer) {
+            const int64_t nx = vx_nelements(x);
+            vx_launch(kv_sync_add1_kernel, dim3((unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096)), dim3(256), 0, (hipStream_t) stream, a, (const double *) a.defer);
+        }
     } else { // a prefill's write: stores and block totals, then totals, scalar and ADD1
         void * ws = nullptr;
         const vx_status rc = vx_workspace((hipStream_t) stream, 2 * SUM_BLOCKS * sizeof(double), &ws);
