@@ -254,7 +254,7 @@ def test_projection_groups_random_shapes(pkg, gpu, seed):  # (seed 29: one produ
 
 @pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 1, 2, 64, 16), (1, 3, 2, 64, 16), (2, 4, 4, 128, 8), (3, 1, 1, 30, 2),
                                         # a short prompt's write: the sums in one work-group, the ADD1 over x a launch of its own
-                                        (1, 48, 2, 64, 16), (1, 64, 2, 64, 16), (2, 20, 2, 64, 16)])
+                                        (1, 48, 2, 64, 16), (1, 64, 2, 64, 16), (2, 20, 2, 64, 16), (1, 128, 2, 64, 16)])
 @pytest.mark.parametrize("poison", [None, "nan", "inf"])
 def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):
     import torch

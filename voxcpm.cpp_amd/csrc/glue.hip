@@ -1835,15 +1835,14 @@ extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * 
                                          const vx_tensor * x, const vx_tensor * dst) {
     if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;
     if (!f32(x) || !f32(dst) || !vx_positive(x) || !vx_same_shape(x, dst) || !nb_multiple(x, 4) || !nb_multiple(dst, 4)) return 0;
-    if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) return vx_nelements(x) <= 65536;
-    return kvs_large(k, k_slot, v, v_slot) && vx_nelements(x) < ((int64_t) 1 << 31);
+    // (x of any size: beyond 16384 values the ADD1 is a launch of its own)
+    return (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) || kvs_large(k, k_slot, v, v_slot) ? vx_nelements(x) < ((int64_t) 1 << 31) : 0;
 }
 
 extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                       const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream) {
     if (!vx_supports_kv_store_sync(k, k_slot, v, v_slot, x, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors; at most 16384 elements per cache write and 65536 in x, or both writes of more than "
-                       "65536 elements (a prefill's)");
+        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors; at most 16384 elements per cache write, or both writes of more than 65536 elements (a prefill's)");
     if (!k->data || !k_slot->data || !v->data || !v_slot->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "kv_store_sync: null data");
     kvs_args a;
     kvs_side_fill(a.k, k, k_slot);
