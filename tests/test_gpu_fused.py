@@ -1215,3 +1215,50 @@ def test_small_graph_limits(gpu, pkg):
     arr = (pkg.VxSmallNode * 17)(*([nd] * 17))
     assert L.vx_small_graph(arr, 17, None) == 2   # VX_ERR_UNSUPPORTED
     assert L.vx_small_graph(arr, 0, None) == 2   # VX_ERR_UNSUPPORTED
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,n", [(2, 512), (8, 64), (3, 30), (5, 101)])
+@pytest.mark.parametrize("private", [0, 1])
+def test_small_graph_sequence_assembly_per_request(gpu, R, n, private):
+    """The CFG-pair sequence of several requests at once (src/locdit.cpp's CONCATs with the requests in the next dimension): a
+    token row, the prefix rows and the patch rows joined along dim 1 for every request, a row repeated for every request and
+    added -- CONCATs below the outermost dimension, whole 16-byte quads (n % 4 == 0) and single values.  One launch against a
+    launch per node, bit for bit."""
+    import torch
+    say(f"small graph: per-request sequence assembly R={R} n={n} private={private}")
+    N = gpu
+    g = lambda tag, *shape: rng("sgq", tag, R, n).standard_normal(shape).astype(np.float32)
+    t = {"tok": g("tok", R, 1, n), "cond": g("cond", R, 4, n), "xp": g("xp", R, 2, n), "row": g("row", 1, 1, n),
+         "rep": np.zeros((R, 1, n), np.float32), "tokb": np.zeros((R, 1, n), np.float32),
+         "a5": np.zeros((R, 5, n), np.float32), "a7": np.zeros((R, 7, n), np.float32), "b7": np.zeros((R, 7, n), np.float32),
+         "pair": np.zeros((R, 14, n), np.float32), "out": np.zeros((R, 14, n), np.float32)}
+    prog = [(N.NODE_REPEAT, "rep", "row", None, 0, 0, 0), (N.NODE_ADD, "tokb", "tok", "rep", 0, 0, 0),
+            (N.NODE_CONCAT, "a5", "tokb", "cond", 1, 0, 0), (N.NODE_CONCAT, "a7", "a5", "xp", 1, 0, 0),
+            (N.NODE_CONCAT, "b7", "a5", "xp", 1, 0, 0), (N.NODE_CONCAT, "pair", "a7", "b7", 1, 0, 0),
+            (N.NODE_SCALE, "out", "pair", None, 0, 0.5, 0.25)]
+    keep = {"out", "a7"} if private else None
+    sets = []
+    for mode in ("separate", "one launch"):
+        T = {k: dev(v) for k, v in t.items()}
+        if mode == "separate":
+            for op, dst, s0, s1, aux, p0, p1 in prog:
+                d, a, b = T[dst], T[s0], (None if s1 is None else T[s1])
+                if op == N.NODE_ADD: N.binary(op, a, b, out=d)
+                elif op == N.NODE_SCALE: N.scale(a, p0, p1, out=d)
+                elif op == N.NODE_REPEAT: N.repeat(a, None, out=d)
+                else: N.concat(a, b, aux, out=d)
+        else:
+            last = {dst: i for i, (_, dst, *_r) in enumerate(prog)}
+            nodes = [N.small_node(op, T[dst], T[s0], None if s1 is None else T[s1], aux, p0, p1,
+                                  private=bool(private and not (dst in keep and last[dst] == i)))
+                     for i, (op, dst, s0, s1, aux, p0, p1) in enumerate(prog)]
+            for nd in nodes:
+                assert N.lib().vx_supports_small_node(nd) == 1
+            N.small_graph(nodes)
+        torch.cuda.synchronize()
+        sets.append(dict(T) if keep is None else {k: T[k] for k in keep})
+    _assert_same(sets, f"per-request assembly R={R} n={n} private={private}")
+    want = np.concatenate([t["tok"] + t["row"], t["cond"], t["xp"]], axis=1)
+    want = np.concatenate([want, want], axis=1) * 0.5 + 0.25
+    assert np.array_equal(sets[1]["out"].cpu().numpy(), want.astype(np.float32))

@@ -839,7 +839,9 @@ enum sgd_code : uint32_t { SGD_ADD = 0, SGD_SUB, SGD_MUL, SGD_DIV, SGD_ADD1, SGD
 // SGD_BLK0 / SGD_MOD0 (a REPEAT as SGD_COPY): destination element e takes source element e / block (p0 = 1 / block: a value
 // per request repeated over the request's elements) or e mod n0 (p0 = 1 / n0: a row repeated for every request)
 constexpr uint32_t SGD_ONE0 = 1, SGD_ONE1 = 2, SGD_WAIT_MEMORY = 4, SGD_NO_BARRIER = 8, SGD_BLK0 = 16, SGD_MOD0 = 32,
-                   SGD_MOD1 = 64; // a binary node whose second operand repeats every aux elements (p1 = 1 / aux: a row added to every request)
+                   SGD_MOD1 = 64, // a binary node whose second operand repeats every aux elements (p1 = 1 / aux: a row added to every request)
+                   SGD_BLOCKS = 128; // a CONCAT below the outermost dimension (a sequence assembled per request): the destination is
+                                     // blocks of aux elements (p0 = 1 / aux), each n0 of the first operand's followed by aux - n0 of the second's
 struct sgd_op {
     uint32_t code, n, n0, flags; // n: destination elements (SUM: units of the source); n0: CONCAT's first operand
     float    p0, p1;
@@ -923,16 +925,29 @@ __global__ __launch_bounds__(1024) void small_graph_dense_kernel(const sgd_args 
                     SGD_LOOP(SGD_X);
                 }
                 break;
-            case SGD_CONCAT: SGD_LOOP(e < op.n0 ? x_at(e) : y_at(e - op.n0)); break;
+            case SGD_CONCAT:
+                if (op.flags & SGD_BLOCKS) { // (the quotient is exact below 2^22 elements)
+                    const uint32_t inner = (uint32_t) op.aux, n1 = inner - op.n0;
+                    for (uint32_t e = threadIdx.x; e < n; e += nt) {
+                        const uint32_t b = (uint32_t) (((float) e + 0.5f) * op.p0), r = e - b * inner;
+                        put(e, r < op.n0 ? x_at(b * op.n0 + r) : y_at(b * n1 + r - op.n0));
+                    }
+                } else {
+                    SGD_LOOP(e < op.n0 ? x_at(e) : y_at(e - op.n0));
+                }
+                break;
             case SGD_ARANGE: SGD_LOOP(arange_value(op.p0, op.p1, (int64_t) e)); break;
             case SGD_COPY4: case SGD_CONCAT4: { // (a COPY4 has n0 == n)
                 const u32x4 * g0 = (const u32x4 *) op.s0, * g1 = (const u32x4 *) op.s1;
                 const u32x4 * i0 = (const u32x4 *) (lds + (l0 ? op.s0_lds : 0)), * i1 = (const u32x4 *) (lds + (l1 ? op.s1_lds : 0));
                 u32x4 * gd = (u32x4 *) op.d, * id = (u32x4 *) (lds + (ld ? op.d_lds : 0));
+                const bool     blocks = op.code == SGD_CONCAT4 && (op.flags & SGD_BLOCKS);
+                const uint32_t inner = blocks ? (uint32_t) op.aux : n, n1 = inner - op.n0;
                 for (uint32_t e = threadIdx.x; e < n; e += nt) {
+                    const uint32_t b = blocks ? (uint32_t) (((float) e + 0.5f) * op.p0) : 0u, r = e - b * inner;
                     u32x4 v;
-                    if (e < op.n0) v = l0 ? i0[e] : g0[e];
-                    else           v = l1 ? i1[e - op.n0] : g1[e - op.n0];
+                    if (r < op.n0) v = l0 ? i0[b * op.n0 + r] : g0[b * op.n0 + r];
+                    else           v = l1 ? i1[b * n1 + r - op.n0] : g1[b * n1 + r - op.n0];
                     if (ld) id[e] = v;
                     if (gd) gd[e] = v;
                 }
@@ -1670,6 +1685,19 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
             op.p1 = 1.0f / (float) op.aux;
         } else if (g.flat == 2) {
             op.code = SGD_CONCAT;
+        } else if (g.kind == SG_CONCAT && g.flat == 0) {
+            // dense operands joined below the outermost dimension: blocks of the destination, each the first operand's part
+            // followed by the second's
+            const vx_tensor * x = nd.src0, * y = nd.src1, * ds = nd.dst;
+            if (!vx_is_contiguous(ds) || (g.flds[0] < 0 && !vx_is_contiguous(x)) || (g.flds[1] < 0 && !vx_is_contiguous(y))) { dense = false; break; }
+            int64_t inner = 1, in0 = 1;
+            for (int q = 0; q <= nd.aux; ++q) { inner *= ds->ne[q]; in0 *= x->ne[q]; }
+            if (inner <= in0 || inner >= (1 << 22)) { dense = false; break; }
+            op.code = SGD_CONCAT;
+            op.flags |= SGD_BLOCKS;
+            op.n0 = (uint32_t) in0;
+            op.aux = (int32_t) inner;
+            op.p0 = 1.0f / (float) inner;
         } else if (g.flat == 1) {
             switch (g.kind) {
                 case SG_EW2:    op.code = SGD_ADD + (uint32_t) g.aux; break;
@@ -1686,9 +1714,10 @@ extern "C" vx_status vx_small_graph(const vx_small_node * nodes, int n_nodes, vx
         // 16 bytes per thread for the plain moves
         auto al = [&](const void * ptr, int32_t off) { return off >= 0 ? off % 4 == 0 : (uintptr_t) ptr % 16 == 0; };
         if ((op.code == SGD_CONCAT || (op.code == SGD_COPY && !g.one0 && !(op.flags & (SGD_BLK0 | SGD_MOD0)))) && op.n % 4 == 0 && al(op.s0, op.s0_lds) && (op.d_lds < 0 || op.d_lds % 4 == 0) &&
-            (uintptr_t) op.d % 16 == 0 && (op.code == SGD_COPY || (op.n0 % 4 == 0 && al(op.s1, op.s1_lds)))) {
+            (uintptr_t) op.d % 16 == 0 && (op.code == SGD_COPY || (op.n0 % 4 == 0 && al(op.s1, op.s1_lds))) && (!(op.flags & SGD_BLOCKS) || op.aux % 4 == 0)) {
             op.n0 = op.code == SGD_COPY ? op.n / 4 : op.n0 / 4;
             op.n /= 4;
+            if (op.flags & SGD_BLOCKS) { op.aux /= 4; op.p0 = 1.0f / (float) op.aux; }
             op.code = op.code == SGD_COPY ? SGD_COPY4 : SGD_CONCAT4;
         }
         // which barriers the run can do without
