@@ -391,10 +391,15 @@ vx_status vx_graph_end(vx_stream stream, vx_graph * graph) {
     recorded_graph * r = t_rec;
     t_rec = nullptr;
     if (vx_tl_launch_mode == 1) vx_tl_launch_mode = 0;
-    if (!graph) { destroy_recorded(r); return vx_fail(VX_ERR_INVALID, "vx_graph_end: null out pointer"); }
-    *graph = nullptr;
     hipGraph_t g = nullptr;
-    const hipError_t e = hipStreamEndCapture((hipStream_t) stream, &g);
+    const hipError_t e = hipStreamEndCapture((hipStream_t) stream, &g); // (whatever follows: the stream must not stay in its capture)
+    if (!graph) {
+        (void) hipGetLastError();
+        if (g) (void) hipGraphDestroy(g);
+        destroy_recorded(r);
+        return vx_fail(VX_ERR_INVALID, "vx_graph_end: null out pointer");
+    }
+    *graph = nullptr;
     if (e != hipSuccess || !g) { // an invalidated recording: the stream is usable again, nothing to replay
         (void) hipGetLastError();
         if (g) (void) hipGraphDestroy(g);
