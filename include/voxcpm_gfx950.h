@@ -353,6 +353,21 @@ VX_API vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * n
                                         const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream);
 VX_API int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate,
                                            const vx_tensor * up, const vx_tensor * dst);
+/* the same call at prefill sizes (vx_supports_mul_mat_swiglu_tiled's shapes on the pre-tiled Q8_0 kernel, 1024 tokens or
+ * more): the norm and its weight are applied by the pass that lays the activations out in tiles, x is read once and the
+ * normalised tensor is never stored.  Same bits as RMS_NORM, MUL, then vx_mul_mat_swiglu. */
+VX_API int vx_supports_norm_mul_mat_swiglu_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate,
+                                                 const vx_tensor * up, const vx_tensor * dst, int act_mode);
+/* mlp_forward and the residual update behind it at prefill sizes (src/minicpm.cpp:718-747, 775-786):
+ *   dst = residual + scale * (down . (silu(gate . n) * (up . n))),  n = RMS_NORM(x) * norm_w
+ * for the node chain RMS_NORM, MUL, MUL_MAT, MUL_MAT, GLU(SWIGLU), MUL_MAT, SCALE, ADD.  The pair's results go to the down
+ * projection as f16 tiles; the [tokens x ffn] tensor between them is not stored.  Same bits as the separate calls
+ * (vx_norm_mul_mat_swiglu, vx_mul_mat_scale_add).  Q8_0 weights, VX_ACT_FLOAT, shapes that the pre-tiled kernel takes. */
+VX_API int vx_supports_mlp_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up,
+                                 const vx_tensor * down, const vx_tensor * residual, const vx_tensor * dst, int act_mode);
+VX_API vx_status vx_mlp_tiled(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate,
+                              const vx_tensor * up, const vx_tensor * down, const vx_tensor * residual, float scale,
+                              const vx_tensor * dst, int act_mode, vx_stream stream);
 /* MUL_MAT(gate, x), MUL_MAT(up, x) -> GLU(SWIGLU split): dst = silu(gate x) * (up x) for few tokens (16, or more while tokens x rows <= 256 Ki)
  * (MiniCPMModel::mlp_forward, src/minicpm.cpp:718-747); gate and up Q8_0 or F16 of one shape and layout */
 VX_API vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * dst,

@@ -726,6 +726,79 @@ def test_norm_mul_mat_swiglu(pkg, gpu, T, B, K, M, act):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("T,B,K,M", [(2048, 1, 1024, 4096), (1100, 2, 1024, 2048), (1024, 1, 768, 1024), (1030, 1, 256, 1040)])
+def test_norm_mul_mat_swiglu_at_prefill_sizes(pkg, gpu, T, B, K, M, monkeypatch):
+    """RMS_NORM, MUL, gate, up, SwiGLU at prefill sizes: the norm and its weight applied by the pass that lays the
+    activations out in tiles for the pre-tiled Q8_0 kernel (one trip over x, the normalised tensor never stored), against
+    RMS_NORM+MUL followed by the tiled pair: the same bits -- whole and ragged token tiles, rows shorter than 1024, a batch."""
+    import torch
+    say(f"fused rms_norm+mul in front of the pre-tiled gate/up/swiglu T={T} B={B} K={K} M={M}")
+    L, d = pkg.lib(), pkg.desc
+    monkeypatch.setenv("VX_GEMM_Q8T", "2")   # (also where the launcher would find too few tiles for the pre-tiled kernel)
+    g = rng("f-nswiglu-t", T, B, K, M)
+    wg, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    wu, _ = q8_dev((0.05 * g.standard_normal((M, K))).astype(np.float32))
+    x = dev((3.0 * g.standard_normal((B, T, K) if B > 1 else (T, K))).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    normed = torch.empty_like(x)
+    a = torch.empty(tuple(x.shape[:-1]) + (M,), dtype=torch.float32, device="cuda")
+    b = torch.full_like(a, float("nan"))
+    dg, du = pkg.desc_q8(wg, K), pkg.desc_q8(wu, K)
+    assert L.vx_supports_norm_mul_mat_swiglu(d(x), d(nw), dg, du, d(b)) == 0
+    assert L.vx_supports_norm_mul_mat_swiglu_tiled(d(x), d(nw), dg, du, d(b), pkg.ACT_FLOAT) == 1
+    assert L.vx_supports_norm_mul_mat_swiglu_tiled(d(x), d(nw), dg, du, d(b), pkg.ACT_Q8) == 0
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    ok(pkg, L.vx_mul_mat_swiglu(dg, du, d(normed), d(a), pkg.ACT_FLOAT, None), "mul_mat_swiglu")
+    ok(pkg, L.vx_norm_mul_mat_swiglu(d(x), d(nw), 1e-5, dg, du, d(b), pkg.ACT_FLOAT, None), "norm_mul_mat_swiglu")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b), float((a - b).abs().max())
+    monkeypatch.setenv("VX_GEMM_Q8T", "0")   # without the pre-tiled kernel there is no fused form: said so, not answered otherwise
+    assert L.vx_supports_norm_mul_mat_swiglu_tiled(d(x), d(nw), dg, du, d(b), pkg.ACT_FLOAT) == 0
+    assert L.vx_norm_mul_mat_swiglu(d(x), d(nw), 1e-5, dg, du, d(b), pkg.ACT_FLOAT, None) != 0
+
+
+@pytest.mark.parametrize("T,B,K,F", [(2048, 1, 1024, 4096), (1100, 2, 1024, 2048), (1024, 1, 1024, 1280), (1030, 3, 1024, 1088)])
+@pytest.mark.parametrize("folded", [False, True])
+def test_mlp_tiled(pkg, gpu, T, B, K, F, folded, monkeypatch):
+    """mlp_forward and its residual update at prefill sizes as one call (RMS_NORM, MUL, gate, up, SwiGLU, down, SCALE, ADD):
+    the pair's results reach the down projection as f16 tiles, the tokens x ffn tensor between them is never stored.  Against
+    the three separate calls: the same bits -- whole and ragged token tiles, a batch, an ffn that is not a multiple of the
+    row tile, the residual in place, the scale folded into the weights or not."""
+    import torch
+    say(f"fused mlp at prefill sizes T={T} B={B} K={K} ffn={F} folded={folded}")
+    L, d = pkg.lib(), pkg.desc
+    monkeypatch.setenv("VX_GEMM_Q8T", "2")
+    if folded:
+        monkeypatch.setenv("VX_GEMM_LDS", "2")
+    else:
+        monkeypatch.delenv("VX_GEMM_LDS", raising=False)
+    g = rng("f-mlp-t", T, B, K, F)
+    wg, _ = q8_dev((0.05 * g.standard_normal((F, K))).astype(np.float32))
+    wu, _ = q8_dev((0.05 * g.standard_normal((F, K))).astype(np.float32))
+    wd, _ = q8_dev((0.05 * g.standard_normal((K, F))).astype(np.float32))
+    x = dev((3.0 * g.standard_normal((B, T, K) if B > 1 else (T, K))).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    normed, act = torch.empty_like(x), torch.empty(tuple(x.shape[:-1]) + (F,), dtype=torch.float32, device="cuda")
+    a, b = torch.empty_like(x), torch.full_like(x, float("nan"))
+    dg, du, dd = pkg.desc_q8(wg, K), pkg.desc_q8(wu, K), pkg.desc_q8(wd, F)
+    scale = 0.2857738
+    assert L.vx_supports_mlp_tiled(d(x), d(nw), dg, du, dd, d(x), d(b), pkg.ACT_FLOAT) == 1
+    assert L.vx_supports_mlp_tiled(d(x), d(nw), dg, du, dd, d(x), d(b), pkg.ACT_Q8) == 0
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    ok(pkg, L.vx_mul_mat_swiglu(dg, du, d(normed), d(act), pkg.ACT_FLOAT, None), "mul_mat_swiglu")
+    ok(pkg, L.vx_mul_mat_scale_add(dd, d(act), d(x), d(a), scale, pkg.ACT_FLOAT, None), "mul_mat_scale_add")
+    ok(pkg, L.vx_mlp_tiled(d(x), d(nw), 1e-5, dg, du, dd, d(x), scale, d(b), pkg.ACT_FLOAT, None), "mlp_tiled")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b), float((a - b).abs().max())
+    x2 = x.clone()   # the update in place, as the graph's residual stream has it
+    ok(pkg, L.vx_mlp_tiled(d(x2), d(nw), 1e-5, dg, du, dd, d(x2), scale, d(x2), pkg.ACT_FLOAT, None), "mlp_tiled in place")
+    torch.cuda.synchronize()
+    assert torch.equal(a, x2)
+    monkeypatch.setenv("VX_GEMM_Q8T", "0")
+    assert L.vx_supports_mlp_tiled(d(x), d(nw), dg, du, dd, d(x), d(b), pkg.ACT_FLOAT) == 0
+    assert L.vx_mlp_tiled(d(x), d(nw), 1e-5, dg, du, dd, d(x), scale, d(b), pkg.ACT_FLOAT, None) != 0
+
+
 def test_norm_prologue_limits(pkg, gpu):
     import torch
     say("norm prologue: rows beyond 1024 floats stay with the separate RMS_NORM")

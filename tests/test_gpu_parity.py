@@ -71,10 +71,14 @@ def test_rms_norm_strided_and_inplace(gpu):
 
 # ---------------------------------------------------------------------------------- ROPE
 @pytest.mark.parametrize("mode", [0, 2])
-@pytest.mark.parametrize("case", ["decode", "prefill", "long", "partial", "yarn"])
+@pytest.mark.parametrize("case", ["decode", "prefill", "long", "partial", "yarn", "prefill batch partial", "prefill yarn"])
 def test_rope(gpu, mode, case):
     say(f"rope mode={mode} case={case}")
-    if case == "decode":
+    if case == "prefill batch partial":   # many tokens: the kernel that walks a token's heads; 6 heads (a ragged group of four), a tail that is copied
+        shape, pos = (3, 300, 6, 80), np.arange(300, dtype=np.int32) * 3 + 7
+    elif case == "prefill yarn":
+        shape, pos = (1, 512, 5, 128), np.arange(512, dtype=np.int32) * 17
+    elif case == "decode":
         shape, pos = (2, 1, 16, 64), np.array([4095], np.int32)
     elif case == "prefill":
         shape, pos = (1, 256, 16, 64), np.arange(256, dtype=np.int32)
@@ -85,11 +89,11 @@ def test_rope(gpu, mode, case):
     else:
         shape, pos = (1, 33, 4, 128), np.arange(33, dtype=np.int32) * 301
     x = rng("rope", case, mode).standard_normal(shape).astype(np.float32)
-    n_dims = 64 if case in ("decode", "prefill", "long", "partial") else 128
-    ff = (1.0 + rng("rope", "ff").random(n_dims // 2)).astype(np.float32) if case != "partial" else None
+    n_dims = 64 if case in ("decode", "prefill", "long", "partial", "prefill batch partial") else 128
+    ff = (1.0 + rng("rope", "ff").random(n_dims // 2)).astype(np.float32) if "partial" not in case else None
     kw = dict(n_ctx_orig=32768, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
               beta_fast=32.0, beta_slow=1.0)
-    if case == "yarn":
+    if "yarn" in case:
         kw.update(freq_scale=0.25, ext_factor=1.0, attn_factor=1.3, n_ctx_orig=4096)
     want = reflib.oracle_rope(x, pos, ff, n_dims, mode, **kw)
     got = sync_np(gpu.rope_ext(dev(x), dev(pos), None if ff is None else dev(ff), n_dims, mode, kw["n_ctx_orig"],

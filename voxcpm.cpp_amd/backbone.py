@@ -269,7 +269,16 @@ class MiniCPMBackbone:
             project_residual(wd["o_proj"], attn.view(N, H * D), attn_o, cur_x, h_mid)
             # -- mlp_forward
             nw_post = nrm["post_layernorm"]
-            if fuse and L.vx_supports_norm_mul_mat_swiglu(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], desc(act)):
+            nxt = hs[li % 2]
+            sc_res = self.residual_scale if self.use_mup else 1.0
+            if fuse and L.vx_supports_mlp_tiled(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], wd["down_proj"], desc(h_mid), desc(nxt), self.act_mode):
+                # prefill sizes: the whole of mlp_forward with its residual update as one call (the tokens x ffn tensor is never stored)
+                call(L.vx_mlp_tiled, desc(h_mid), desc(nw_post), self.eps, wd["gate_proj"], wd["up_proj"], wd["down_proj"], desc(h_mid), sc_res,
+                     desc(nxt), self.act_mode)
+                cur_x = nxt
+                continue
+            if fuse and (L.vx_supports_norm_mul_mat_swiglu(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], desc(act)) or
+                         L.vx_supports_norm_mul_mat_swiglu_tiled(desc(h_mid), desc(nw_post), wd["gate_proj"], wd["up_proj"], desc(act), self.act_mode)):
                 # rms_norm, gate, up and SwiGLU as one launch
                 call(L.vx_norm_mul_mat_swiglu, desc(h_mid), desc(nw_post), self.eps, wd["gate_proj"], wd["up_proj"], desc(act), self.act_mode)
             elif fuse and (N <= 16 or L.vx_supports_mul_mat_swiglu_tiled(wd["gate_proj"], wd["up_proj"], desc(normed), desc(act), self.act_mode)):

@@ -66,6 +66,10 @@ struct mm_args {
     int ksplit;
     float * partial;
     size_t ws_offset; // bytes at the start of the stream's workspace that the caller keeps for itself: partials go behind them
+    // pre-tiled kernel, mlp_forward as one call: the pair's epilogue writes silu(g) * u as the f16 activation tiles of the
+    // product that follows (tile_out) instead of storing dst, and that product takes them as they are (tile_in) instead of
+    // laying x out itself; tile_tt: 16-token tiles per k block in that buffer (whole 128-token tiles of the pair)
+    void * tile_out; const void * tile_in; int tile_tt;
     // GEMV with RMS_NORM and the norm-weight MUL applied to the activations as they are staged
     // (x is then the un-normalised tensor): x[t][k] / rms(x[t]) * norm_w[k], rounded after each product
     const float * norm_w;
@@ -1880,6 +1884,8 @@ struct qt_args {
     int      n_rt, n_tt, n_kb;       // 16-row tiles (of the virtual matrix: gate and up tiles alternate), token tiles, k blocks
     int      w_al4;
     int      fold;                   // the block scale multiplied into the f16 weights by the weight pass (VX_GEMM_LDS=2)
+    const float * norm_w; float norm_eps; // the activation pass applies RMS_NORM and the norm-weight MUL (x is the un-normalised tensor)
+    _Float16 * tile_out; int out_tt;      // DUAL: the results leave as the next product's activation tiles (out_tt tiles per k block)
 };
 
 // one thread = 8 quants of a block: (virtual row, block, j)
@@ -1946,6 +1952,46 @@ __global__ __launch_bounds__(256) void qt_acts_kernel(const qt_args a) {
         }
         a.xt[(((int64_t) batch * a.n_kb + kb) * a.n_tt + tt) * 64 + slot] = h;
     }
+}
+
+// The same tiles from an un-normalised x: RMS_NORM and the norm-weight MUL on the way, rounded as the two separate kernels
+// round them.  A work-group = one tile of 16 tokens, a wave = one token in the RMS_NORM kernel's wave-per-row order (rows
+// of at most 1024 values: lane l holds columns 4 (l + 64 c) .. + 3); the sixteen rows meet in LDS as f16 and leave as the
+// tile's k blocks, 1 KB each.  Against the norm kernel followed by the pass above that is one trip over x instead of two
+// and the normalised tensor neither written nor read back.
+__global__ __launch_bounds__(1024) void qt_acts_norm_kernel(const qt_args a) {
+    constexpr int ROW = 1024 + 8; // halfs between the staged rows: the padding spreads the sixteen tokens over the banks
+    __shared__ __attribute__((aligned(16))) _Float16 rows[16 * ROW];
+    const int     lane = threadIdx.x & 63, wid = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+    const int64_t tt = blockIdx.x;
+    const int     batch = blockIdx.y, i12 = batch % a.ne12, i13 = batch / a.ne12;
+    const int64_t tok = 16 * tt + wid;
+    const int     nv = (int) ((a.K + 255) >> 8); // 16-byte pieces of a row per lane
+    const int64_t nvec = a.K / 4;
+    if (tok < a.N) { // (uniform per wave)
+        vx_rms_row r, gn;
+        vx_rms_row_load(r, (const float *) (a.x + (uint64_t) i12 * a.nb12 + (uint64_t) i13 * a.nb13 + (uint64_t) tok * a.nb11), a.K, lane);
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc)
+            if (cc < nv && lane + 64 * cc < nvec) gn.v[cc] = ((const float4 *) a.norm_w)[lane + 64 * cc];
+        const float sc = vx_rms_row_scale(r, a.K, lane, a.norm_eps);
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            if (cc >= nv || lane + 64 * cc >= nvec) break;
+            float       v[4]  = { r.v[cc].x, r.v[cc].y, r.v[cc].z, r.v[cc].w };
+            const float gg[4] = { gn.v[cc].x, gn.v[cc].y, gn.v[cc].z, gn.v[cc].w };
+            half4_t h;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[i] *= sc; v[i] *= gg[i]; h[i] = (_Float16) v[i]; } // RMS_NORM's product, then the MUL node's
+            *(half4_t *) &rows[wid * ROW + 4 * (lane + 64 * cc)] = h;
+        }
+    } else {
+        for (int64_t e = lane; e < nvec; e += 64) *(half4_t *) &rows[wid * ROW + 4 * e] = half4_t{0, 0, 0, 0};
+    }
+    __syncthreads();
+    const int j = lane >> 4, c = lane & 15;
+    for (int kb = wid; kb < a.n_kb; kb += 16)
+        a.xt[(((int64_t) batch * a.n_kb + kb) * a.n_tt + tt) * 64 + lane] = *(const half8_t *) &rows[c * ROW + 32 * kb + 8 * j];
 }
 
 __device__ __forceinline__ void qt_dma16(const void * base, uint32_t off, uint32_t lds) {
@@ -2061,6 +2107,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // A tile inside the matrix stores without tests, at a uniform base plus one 32-bit lane offset (the launcher checks the
     // range): computed per element in 64-bit arithmetic, the addresses of a tile's 64 stores per lane were a fifth of the
     // kernel's vector instructions.
+    if constexpr (DUAL) {
+        if (a.tile_out) { // (uniform) silu(g) * u rounded to f16, as the next product's activation pass would round it, straight
+            // into that product's tiles: row = its k index.  Tile (k block, 16 tokens), slot (k / 8 mod 4, token mod 16), 8 halfs.
+            const uint32_t n_kb2 = (uint32_t) (a.M >> 5);
+#pragma unroll
+            for (int p2 = 0; p2 < 2; ++p2) {
+                const uint32_t row = 16u * ((uint32_t) (rt0 >> 1) + 2u * wr + p2) + c;
+                if (row >= (uint32_t) a.M) continue;
+                const uint32_t kb2 = row >> 5, slot_j = (row >> 3) & 3, e = row & 7;
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t tok = (uint32_t) tok0 + 16u * tt + 4u * j + r;
+                        const float g = acc[2 * p2][tt][r], u = acc[2 * p2 + 1][tt][r];
+                        const uint64_t tile = ((uint64_t) batch * n_kb2 + kb2) * (uint32_t) a.out_tt + (tok >> 4);
+                        float h = (g / (1.0f + expf(-g))) * u; // the fp32 value the GLU node holds ...
+                        asm volatile("" : "+v"(h));             // ... formed as such, then rounded as the activation pass rounds it
+                        a.tile_out[(tile * 64 + slot_j * 16 + (tok & 15)) * 8 + e] = (_Float16) h;
+                    }
+            }
+            return;
+        }
+    }
     const bool inside = (int64_t) (ty + 1) * QT_TOKS <= a.N && (int64_t) (tx + 1) * QT_ROWS <= (DUAL ? 2 * a.M : a.M); // uniform
     if (inside) {
         const int64_t  row0 = DUAL ? 16 * ((int64_t) (rt0 >> 1) + 2 * wr) : 16 * ((int64_t) rt0 + 4 * wr);
@@ -2150,6 +2220,7 @@ int gemm_q8t_mode() { const char * e = getenv("VX_GEMM_Q8T"); return e ? atoi(e)
 // tiles of gemm_lds_kernel and its K cut, 7.2 ms here)
 bool gemm_q8t_takes(const mm_args & a, int nbatch, bool dual) {
     const int64_t MV = dual ? 2 * a.M : a.M;
+    if (a.norm_w && (a.K > 1024 || a.K % 8 || (uintptr_t) a.norm_w % 16)) return false; // (the norm's wave-per-row regime)
     const int mode = gemm_q8t_mode();
     const int64_t tiles = ((MV + QT_ROWS - 1) / QT_ROWS) * ((a.N + QT_TOKS - 1) / QT_TOKS) * nbatch;
     // (and a thousand tiles' worth of K = 1024: 1024 x 1024 x 16384 is 86 us here against 74, 4096 x 1024 x 4096 a tie, every
@@ -2172,9 +2243,10 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     q.w_al4 = a.w_aligned;
     q.fold  = fold;
     const int64_t MV = DUAL ? 2 * a.M : a.M;
-    q.n_rt = (int) ((MV + 15) / 16); q.n_tt = (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
+    q.n_rt = (int) ((MV + 15) / 16); q.n_tt = a.tile_in ? a.tile_tt : (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
+    q.tile_out = DUAL ? (_Float16 *) a.tile_out : nullptr; q.out_tt = a.tile_tt;
     const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * ((q.n_rt + 3) & ~3) * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
-    const size_t xt_bytes = (size_t) nbatch * q.n_kb * q.n_tt * 1024;
+    const size_t xt_bytes = a.tile_in ? 0 : (size_t) nbatch * q.n_kb * q.n_tt * 1024;
     static bool raised = false;
     if (!raised) {
         if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
@@ -2206,9 +2278,13 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     char * base = (char *) ws + a.ws_offset;
     if (kept) { q.wt = (half8_t *) kept; q.wdt = (float *) (kept + wt_bytes); q.xt = (half8_t *) base; }
     else      { q.wt = (half8_t *) base; q.wdt = (float *) (base + wt_bytes); q.xt = (half8_t *) (base + wt_bytes + wd_bytes); }
+    if (a.tile_in) q.xt = (half8_t *) const_cast<void *>(a.tile_in);
     if (!kept || fresh) vx_launch(qt_weights_kernel, dim3((unsigned) ((wunits + 255) / 256)), dim3(256), 0, st, q);
     if (fresh) vx_derived_filled(key, st);
-    vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
+    q.norm_w = a.norm_w; q.norm_eps = a.norm_eps;
+    if (a.tile_in) {} // (the activations are the tiles the product before left)
+    else if (a.norm_w) vx_launch(qt_acts_norm_kernel, dim3((unsigned) q.n_tt, (unsigned) nbatch), dim3(1024), 0, st, q);
+    else          vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
     if (fold) vx_launch(gemm_q8t_kernel<DUAL, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     else      vx_launch(gemm_q8t_kernel<DUAL, false>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     return true;
@@ -2266,6 +2342,7 @@ bool launch_gemm_lds_swiglu(const mm_args & a, int nbatch, hipStream_t st) {
     if constexpr (WT == WT_Q8) {
         if (gemm_q8t_takes(a, nbatch, true)) return launch_gemm_q8t<true>(a, nbatch, st, fold);
     }
+    if (a.norm_w) return false; // (a fused norm exists in the pre-tiled kernel's activation pass only)
     const bool big  = ((2 * a.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
     if constexpr (WT == WT_Q8) {
         if (fold) return big ? launch_gemm_lds_tile<WT, true, 4, 2, 2, 4, true>(a, nbatch, st) : launch_gemm_lds_tile<WT, true, 2, 2, 2, 2, true>(a, nbatch, st);
@@ -2431,32 +2508,8 @@ extern "C" vx_status vx_mul_mat_swiglu(const vx_tensor * gate, const vx_tensor *
 
 // RMS_NORM , MUL(norm weight) , MUL_MAT(gate) , MUL_MAT(up) , GLU(SWIGLU): mlp_forward behind its rms_norm
 // (src/minicpm.cpp:572-580, 718-747) as one launch; x is the un-normalised hidden state.
-extern "C" int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up,
-                                               const vx_tensor * dst) {
-    return vx_supports_mul_mat_swiglu(gate, up, x, dst) && norm_prologue_ok(x, norm_w);
-}
-
-extern "C" vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate,
-                                            const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream) {
-    if (!x || !norm_w || !gate || !up || !dst || !norm_w->data) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: null tensor");
-    if (!vx_supports_norm_mul_mat_swiglu(x, norm_w, gate, up, dst) || (uintptr_t) x->data % 16 || (uintptr_t) norm_w->data % 16)
-        return vx_fail(VX_ERR_UNSUPPORTED, "norm_mul_mat_swiglu: as mul_mat_swiglu, with 16-byte aligned rows of at most 1024 floats and one F32 norm weight row");
-    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: eps must be >= 0");
-    return swiglu_run(gate, up, x, norm_w, eps, dst, act_mode, stream);
-}
-
-static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * norm_w, float eps,
-                            const vx_tensor * dst, int act_mode, vx_stream stream) {
-    if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
-        return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
-    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
-    const bool tiled = !norm_w && vx_supports_mul_mat_swiglu_tiled(gate, up, src1, dst, act_mode);
-    if (!tiled && !vx_supports_mul_mat_swiglu(gate, up, src1, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, a token count the streaming kernel takes "
-                       "(or, with f16 activations, 64 tokens or more for the tiled kernel: vx_supports_mul_mat_swiglu_tiled)");
-    if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
-        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
-    mm_args a = {};
+static void swiglu_fill(mm_args & a, const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * norm_w, float eps,
+                        const vx_tensor * dst) {
     a.w = (const char *) gate->data; a.x = (const char *) src1->data; a.dst = (char *) dst->data;
     a.K = gate->ne[0]; a.M = gate->ne[1]; a.N = src1->ne[1];
     a.nb01 = gate->nb[1]; a.nb02 = gate->nb[2]; a.nb03 = gate->nb[3];
@@ -2470,6 +2523,52 @@ static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const 
     a.norm_eps  = eps;
     a.w_aligned = (((uintptr_t) gate->data | (uintptr_t) up->data) % 4 == 0) && gate->nb[1] % 4 == 0 && gate->nb[2] % 4 == 0 && gate->nb[3] % 4 == 0;
     a.x_aligned = ((uintptr_t) src1->data % 16 == 0) && src1->nb[1] % 16 == 0 && src1->nb[2] % 16 == 0 && src1->nb[3] % 16 == 0;
+}
+
+// The same at prefill sizes: the pair on the pre-tiled kernel (vx_supports_mul_mat_swiglu_tiled, Q8_0 weights, a shape that
+// kernel takes), the norm in its activation pass.
+static bool norm_swiglu_tiled_ok(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up, const vx_tensor * dst,
+                                 int act_mode) {
+    if (!gate || gate->type != VX_TYPE_Q8_0 || !norm_prologue_ok(x, norm_w) || !norm_w->data || (uintptr_t) norm_w->data % 16 || !x->data ||
+        (uintptr_t) x->data % 16) return false;
+    if (!vx_supports_mul_mat_swiglu_tiled(gate, up, x, dst, act_mode)) return false;
+    mm_args a = {};
+    swiglu_fill(a, gate, up, x, norm_w, 0.0f, dst);
+    return gemm_q8t_takes(a, (int) (x->ne[2] * x->ne[3]), true);
+}
+extern "C" int vx_supports_norm_mul_mat_swiglu_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up,
+                                                     const vx_tensor * dst, int act_mode) {
+    return x && norm_w && up && dst && norm_swiglu_tiled_ok(x, norm_w, gate, up, dst, act_mode);
+}
+
+extern "C" int vx_supports_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up,
+                                               const vx_tensor * dst) {
+    return vx_supports_mul_mat_swiglu(gate, up, x, dst) && norm_prologue_ok(x, norm_w);
+}
+
+extern "C" vx_status vx_norm_mul_mat_swiglu(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate,
+                                            const vx_tensor * up, const vx_tensor * dst, int act_mode, vx_stream stream) {
+    if (!x || !norm_w || !gate || !up || !dst || !norm_w->data) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: null tensor");
+    if ((!vx_supports_norm_mul_mat_swiglu(x, norm_w, gate, up, dst) && !norm_swiglu_tiled_ok(x, norm_w, gate, up, dst, act_mode)) ||
+        (uintptr_t) x->data % 16 || (uintptr_t) norm_w->data % 16)
+        return vx_fail(VX_ERR_UNSUPPORTED, "norm_mul_mat_swiglu: as mul_mat_swiglu, with 16-byte aligned rows of at most 1024 floats and one F32 norm weight row");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "norm_mul_mat_swiglu: eps must be >= 0");
+    return swiglu_run(gate, up, x, norm_w, eps, dst, act_mode, stream);
+}
+
+static vx_status swiglu_run(const vx_tensor * gate, const vx_tensor * up, const vx_tensor * src1, const vx_tensor * norm_w, float eps,
+                            const vx_tensor * dst, int act_mode, vx_stream stream) {
+    if (!gate || !up || !src1 || !dst || !gate->data || !up->data || !src1->data || !dst->data)
+        return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: null tensor");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "mul_mat_swiglu: bad act_mode");
+    const bool tiled = norm_w ? norm_swiglu_tiled_ok(src1, norm_w, gate, up, dst, act_mode) : vx_supports_mul_mat_swiglu_tiled(gate, up, src1, dst, act_mode) != 0;
+    if (!tiled && !vx_supports_mul_mat_swiglu(gate, up, src1, dst))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: two Q8_0/F16 matrices of one layout, a token count the streaming kernel takes "
+                       "(or, with f16 activations, 64 tokens or more for the tiled kernel: vx_supports_mul_mat_swiglu_tiled)");
+    if ((uintptr_t) src1->data % 4 || (uintptr_t) dst->data % 4 || (gate->type == VX_TYPE_F16 && (((uintptr_t) gate->data | (uintptr_t) up->data) % 2)))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_swiglu: misaligned tensor data");
+    mm_args a = {};
+    swiglu_fill(a, gate, up, src1, norm_w, eps, dst);
     const int nbatch = (int) (src1->ne[2] * src1->ne[3]);
     hipStream_t st = (hipStream_t) stream;
     bool ok;
@@ -2571,6 +2670,78 @@ extern "C" vx_status vx_mul_mat_scale_add(const vx_tensor * src0, const vx_tenso
         if ((units + 255) / 256 > 0x7fffffff) return vx_fail(VX_ERR_UNSUPPORTED, "mul_mat_scale_add: launch too large");
         vx_launch(mm_splitk_reduce_kernel, dim3((unsigned) ((units + 255) / 256), 1, (unsigned) nbatch), dim3(256), 0, st, b);
     }
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// mlp_forward and the residual update behind it at prefill sizes (src/minicpm.cpp:718-747, 775-786): RMS_NORM, MUL, gate, up,
+// SwiGLU, down, SCALE, ADD.  Three launches on the pre-tiled kernel: the activation pass with the norm, the gate/up pair
+// whose epilogue writes silu(g) * u as f16 tiles, and the down projection that takes those tiles as they are, with the
+// update in its epilogue.  The intermediate [tokens x ffn] tensor is neither stored in fp32 nor read back and re-laid-out
+// (at 65536 tokens x 4096: a gigabyte each way).  Every value is rounded where the separate calls round it: same bits.
+static bool mlp_fill(mm_args & a, mm_args & b, const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate, const vx_tensor * up,
+                     const vx_tensor * down, const vx_tensor * residual, float scale, const vx_tensor * dst, int act_mode) {
+    if (!x || !norm_w || !gate || !up || !down || !residual || !dst) return false;
+    if (down->type != VX_TYPE_Q8_0 || down->ne[2] != 1 || down->ne[3] != 1 || gate->ne[2] != 1 || gate->ne[3] != 1) return false;
+    if (down->ne[0] != gate->ne[1] || gate->ne[1] % 32 || dst->ne[0] != down->ne[1] || dst->ne[1] != x->ne[1] || dst->ne[2] != x->ne[2] || dst->ne[3] != x->ne[3]) return false;
+    if (dst->type != VX_TYPE_F32 || dst->nb[0] != 4 || residual->type != VX_TYPE_F32 || residual->nb[0] != 4 || !vx_same_shape(residual, dst)) return false;
+    // the intermediate as the separate calls would see it: dense [ffn, tokens, batch]
+    vx_tensor act = *dst;
+    act.ne[0] = gate->ne[1];
+    act.nb[1] = (uint64_t) act.ne[0] * 4; act.nb[2] = act.nb[1] * (uint64_t) act.ne[1]; act.nb[3] = act.nb[2] * (uint64_t) act.ne[2];
+    act.data = x->data; // (only its alignment is looked at)
+    if (!norm_swiglu_tiled_ok(x, norm_w, gate, up, &act, act_mode)) return false;
+    if (!vx_supports_mul_mat_scale_add(down, &act, residual, dst)) return false;
+    swiglu_fill(a, gate, up, x, norm_w, eps, &act);
+    b = mm_args{};
+    b.w = (const char *) down->data; b.x = (const char *) x->data; b.dst = (char *) dst->data;
+    b.K = down->ne[0]; b.M = down->ne[1]; b.N = x->ne[1];
+    b.nb01 = down->nb[1]; b.nb02 = down->nb[2]; b.nb03 = down->nb[3];
+    b.nb11 = act.nb[1]; b.nb12 = act.nb[2]; b.nb13 = act.nb[3];
+    b.nb1 = dst->nb[1]; b.nb2 = dst->nb[2]; b.nb3 = dst->nb[3];
+    b.ne12 = (int) x->ne[2];
+    b.r2 = (int) x->ne[2]; b.r3 = (int) x->ne[3];
+    b.rows_wg = 16;
+    b.res = (const char *) residual->data;
+    b.rnb1 = residual->nb[1]; b.rnb2 = residual->nb[2]; b.rnb3 = residual->nb[3];
+    b.res_scale = scale;
+    b.w_aligned = ((uintptr_t) down->data % 4 == 0) && down->nb[1] % 4 == 0;
+    b.x_aligned = 1;
+    const int nbatch = (int) (x->ne[2] * x->ne[3]);
+    // both products on the pre-tiled kernel, as the separate calls would run them
+    return gemm_lds_mode() != 0 && b.w_aligned && (uintptr_t) dst->data % 4 == 0 && (uintptr_t) residual->data % 4 == 0 &&
+           gemm_q8t_takes(a, nbatch, true) && gemm_q8t_takes(b, nbatch, false) && (uint64_t) 256 * b.rnb1 + 1024 < (1ull << 32);
+}
+
+extern "C" int vx_supports_mlp_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * gate, const vx_tensor * up, const vx_tensor * down,
+                                     const vx_tensor * residual, const vx_tensor * dst, int act_mode) {
+    mm_args a = {}, b = {};
+    return mlp_fill(a, b, x, norm_w, 0.0f, gate, up, down, residual, 0.0f, dst, act_mode);
+}
+
+extern "C" vx_status vx_mlp_tiled(const vx_tensor * x, const vx_tensor * norm_w, float eps, const vx_tensor * gate, const vx_tensor * up,
+                                  const vx_tensor * down, const vx_tensor * residual, float scale, const vx_tensor * dst, int act_mode, vx_stream stream) {
+    mm_args a = {}, b = {};
+    if (!mlp_fill(a, b, x, norm_w, eps, gate, up, down, residual, scale, dst, act_mode))
+        return vx_fail(VX_ERR_UNSUPPORTED, "mlp_tiled: the shapes of vx_supports_norm_mul_mat_swiglu_tiled, a Q8_0 down projection that the pre-tiled kernel takes, "
+                       "an F32 residual of dst's shape");
+    if (!x->data || !norm_w->data || !gate->data || !up->data || !down->data || !residual->data || !dst->data) return vx_fail(VX_ERR_INVALID, "mlp_tiled: null data");
+    if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "mlp_tiled: eps must be >= 0");
+    const int nbatch = (int) (x->ne[2] * x->ne[3]);
+    hipStream_t st = (hipStream_t) stream;
+    // the tiles between the two products: whole 128-token tiles of the pair (it writes every token of its tiles), at the front of
+    // the workspace; both products put what they need behind them (a block that a later, larger request replaces stays valid)
+    const int    tile_tt = (int) ((a.N + QT_TOKS - 1) / QT_TOKS) * (QT_TOKS / 16);
+    const size_t tiles   = ((size_t) nbatch * (size_t) (a.M / 32) * (size_t) tile_tt * 1024 + 255) & ~(size_t) 255;
+    void * ws = nullptr;
+    (void) take_ws_status();
+    const vx_status rc = vx_workspace(st, tiles, &ws);
+    if (rc != VX_OK) return rc;
+    a.ws_offset = tiles; a.tile_out = ws; a.tile_tt = tile_tt;
+    b.ws_offset = tiles; b.tile_in = ws;  b.tile_tt = tile_tt;
+    const bool fold = gemm_lds_mode() == 2;
+    if (!launch_gemm_q8t<true>(a, nbatch, st, fold)) return ws_failed() ? take_ws_status() : vx_fail(VX_ERR_UNSUPPORTED, "mlp_tiled: the gate/up product could not be launched");
+    if (!launch_gemm_q8t<false>(b, nbatch, st, fold)) return ws_failed() ? take_ws_status() : vx_fail(VX_ERR_UNSUPPORTED, "mlp_tiled: the down projection could not be launched");
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

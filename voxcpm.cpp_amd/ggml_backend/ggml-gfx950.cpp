@@ -1610,7 +1610,47 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                     const vx_tensor x = to_vx(node->src[0]), nw = to_vx(mul->src[1]), gw = to_vx(gate->src[0]), uw = to_vx(up->src[0]), d = to_vx(glu);
                     float eps;
                     memcpy(&eps, node->op_params, sizeof(float));
-                    if (vx_supports_norm_mul_mat_swiglu(&x, &nw, &gw, &uw, &d) && (uintptr_t) x.data % 16 == 0 && (uintptr_t) nw.data % 16 == 0 &&
+                    // Prefill sizes, and the GLU's value read by the down projection alone (MUL_MAT [SCALE] ADD behind it): the
+                    // whole of mlp_forward with its residual update as one call, the tokens x ffn tensor never stored
+                    if (i + 6 < cgraph->n_nodes && private_to_group(readers, glu) && (glu->flags & GGML_TENSOR_FLAG_OUTPUT) == 0) {
+                        ggml_tensor * down = cgraph->nodes[i + 5];
+                        ggml_tensor * val = down;
+                        float sc = 1.0f;
+                        int ia = i + 6;
+                        bool chain = down->op == GGML_OP_MUL_MAT && down->src[1] == glu && private_to_group(readers, down) &&
+                                     (down->flags & GGML_TENSOR_FLAG_OUTPUT) == 0;
+                        if (chain && cgraph->nodes[ia]->op == GGML_OP_SCALE) {
+                            ggml_tensor * scn = cgraph->nodes[ia];
+                            float bias;
+                            memcpy(&sc, (const float *) scn->op_params + 0, sizeof(float));
+                            memcpy(&bias, (const float *) scn->op_params + 1, sizeof(float));
+                            chain = scn->src[0] == down && bias == 0.0f && private_to_group(readers, scn) && (scn->flags & GGML_TENSOR_FLAG_OUTPUT) == 0;
+                            val = scn;
+                            if (++ia >= cgraph->n_nodes) chain = false;
+                        }
+                        if (chain) {
+                            ggml_tensor * add = cgraph->nodes[ia];
+                            chain = add->op == GGML_OP_ADD && (add->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 && (add->src[0] == val) != (add->src[1] == val);
+                            if (chain) {
+                                ggml_tensor * residual = add->src[0] == val ? add->src[1] : add->src[0];
+                                const vx_tensor dw = to_vx(down->src[0]), r = to_vx(residual), out = to_vx(add);
+                                if (residual != down && residual != glu && apart(add, down->src[0]) && apart(add, gate->src[0]) && apart(add, up->src[0]) &&
+                                    apart(add, mul->src[1]) && apart_or_same(add, residual) && apart_or_same(add, node->src[0]) &&
+                                    (uintptr_t) x.data % 16 == 0 && (uintptr_t) nw.data % 16 == 0 &&
+                                    vx_supports_mlp_tiled(&x, &nw, &gw, &uw, &dw, &r, &out, mul_mat_act_mode())) {
+                                    rc = vx_mlp_tiled(&x, &nw, eps, &gw, &uw, &dw, &r, sc, &out, mul_mat_act_mode(), ctx->stream);
+                                    done.insert(mul); done.insert(gate); done.insert(up); done.insert(glu); done.insert(down);
+                                    if (val != down) done.insert(val);
+                                    done.insert(add);
+                                    grouped = true;
+                                }
+                            }
+                        }
+                    }
+                    if (grouped) {} else
+                    // (decode sizes on the streaming kernel, prefill sizes in the pre-tiled kernel's activation pass)
+                    if ((vx_supports_norm_mul_mat_swiglu(&x, &nw, &gw, &uw, &d) || vx_supports_norm_mul_mat_swiglu_tiled(&x, &nw, &gw, &uw, &d, mul_mat_act_mode())) &&
+                        (uintptr_t) x.data % 16 == 0 && (uintptr_t) nw.data % 16 == 0 &&
                         apart(glu, node->src[0])) {
                         rc = vx_norm_mul_mat_swiglu(&x, &nw, eps, &gw, &uw, &d, mul_mat_act_mode(), ctx->stream);
                         done.insert(mul); done.insert(gate); done.insert(up); done.insert(glu);
