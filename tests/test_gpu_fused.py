@@ -845,6 +845,51 @@ def test_norm_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act):
     assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
 
 
+@pytest.mark.parametrize("T,B,H,Hkv,D,K,batched", [(2304, 1, 16, 2, 64, 1024, False), (1100, 2, 16, 2, 64, 1024, False), (2100, 2, 16, 2, 64, 1024, True),
+                                                    (1030, 1, 8, 4, 128, 768, False)])
+def test_norm_qkv_proj_rope_at_prefill_sizes(pkg, gpu, T, B, H, Hkv, D, K, batched, monkeypatch):
+    """RMS_NORM, MUL, the q, k and v projections and both rotations at prefill sizes as one call: the norm in the pre-tiled
+    kernel's activation pass, the three matrices as one product over those tiles, the rotations in place behind it.  Against
+    the separate calls (RMS_NORM+MUL, three MUL_MATs, two ROPEs): the same bits -- the sequences flattened into one token
+    dimension or as a batch, ragged token tiles, 64- and 128-wide heads."""
+    import torch
+    say(f"fused rms_norm+mul, q/k/v as one pre-tiled product, rope: T={T} B={B} H={H}/{Hkv} D={D} K={K} batched={batched}")
+    L, d = pkg.lib(), pkg.desc
+    monkeypatch.setenv("VX_GEMM_Q8T", "2")
+    g = rng("f-nqkv-t", T, B, H, D, K)
+    ws = [q8_dev((0.05 * g.standard_normal((n * D, K))).astype(np.float32))[0] for n in (H, Hkv, Hkv)]
+    wd = [pkg.desc_q8(w, K) for w in ws]
+    x = dev((2.0 * g.standard_normal((B, 1, T, K) if batched else (B * T, K))).astype(np.float32))
+    nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
+    pos = torch.arange(300, 300 + T, dtype=torch.int32, device="cuda")
+    ff = dev((1.0 + g.random(D // 2)).astype(np.float32))
+    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+
+    def outs():
+        return (torch.full((B, T, H, D), float("nan"), dtype=torch.float32, device="cuda"),
+                torch.full((B, T, Hkv, D), float("nan"), dtype=torch.float32, device="cuda"),
+                torch.full((B, 1, T, Hkv * D) if batched else (B * T, Hkv * D), float("nan"), dtype=torch.float32, device="cuda"))
+
+    q1, k1, v1 = outs()
+    normed = torch.empty_like(x)
+    flat = (lambda t, rows: t.view(B, 1, T, rows)) if batched else (lambda t, rows: t.view(B * T, rows))
+    ok(pkg, L.vx_rms_norm_mul(d(x), d(nw), d(normed), 1e-5, None), "rms_norm_mul")
+    ok(pkg, L.vx_mul_mat(wd[0], d(normed), d(flat(q1, H * D)), pkg.ACT_FLOAT, None), "q")
+    ok(pkg, L.vx_mul_mat(wd[1], d(normed), d(flat(k1, Hkv * D)), pkg.ACT_FLOAT, None), "k")
+    ok(pkg, L.vx_mul_mat(wd[2], d(normed), d(v1), pkg.ACT_FLOAT, None), "v")
+    for t in (q1, k1):
+        ok(pkg, L.vx_rope(d(t), pos.data_ptr(), ff.data_ptr(), d(t), *rope_args, None), "rope")
+    q2, k2, v2 = outs()
+    assert L.vx_supports_norm_qkv_proj_rope(d(x), d(nw), *wd, d(q2), d(k2), d(v2), D, 2) == 0
+    assert L.vx_supports_norm_qkv_proj_rope_tiled(d(x), d(nw), *wd, d(q2), d(k2), d(v2), D, 2, pkg.ACT_FLOAT) == 1
+    assert L.vx_supports_norm_qkv_proj_rope_tiled(d(x), d(nw), *wd, d(q2), d(k2), d(v2), D, 2, pkg.ACT_Q8) == 0
+    ok(pkg, L.vx_norm_qkv_proj_rope(d(x), d(nw), 1e-5, *wd, pos.data_ptr(), ff.data_ptr(), d(q2), d(k2), d(v2), *rope_args, pkg.ACT_FLOAT, None),
+       "norm_qkv_proj_rope")
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert bool(torch.isfinite(q2).all()) and bool(torch.isfinite(v2).all())
+
+
 @pytest.mark.parametrize("T,n_past,B,Hkv,D", [(1, 639, 2, 2, 64), (1, 300, 1, 2, 64), (2, 1000, 2, 4, 128), (3, 4000, 2, 2, 64)])
 @pytest.mark.parametrize("poison", [None, "nan"])
 def test_flash_attn_two_segments_with_cache_write(pkg, gpu, T, n_past, B, Hkv, D, poison):

@@ -184,8 +184,10 @@ class MiniCPMBackbone:
             plain_order = n_past == 0 or not f16_cache or write_kv
             wqkv = (wd["q_proj"], wd["k_proj"], wd["v_proj"])
             nw_in = nrm["input_layernorm"]
-            if fuse and plain_order and L.vx_supports_norm_qkv_proj_rope(desc(cur_x), desc(nw_in), *wqkv, desc(q4), desc(k4), desc(v), D, 2):
-                # rms_norm, the three projections and both rotations as one launch (decode-sized token counts)
+            if fuse and plain_order and (L.vx_supports_norm_qkv_proj_rope(desc(cur_x), desc(nw_in), *wqkv, desc(q4), desc(k4), desc(v), D, 2) or
+                                         L.vx_supports_norm_qkv_proj_rope_tiled(desc(cur_x), desc(nw_in), *wqkv, desc(q4), desc(k4), desc(v), D, 2, self.act_mode)):
+                # rms_norm, the three projections and both rotations as one call (one launch at decode sizes; at prefill sizes the
+                # norm in the activation pass, one product for the three matrices, the rotations behind it)
                 call(L.vx_norm_qkv_proj_rope, desc(cur_x), desc(nw_in), self.eps, *wqkv, _p(pos), ff, desc(q4), desc(k4), desc(v),
                      *rope_args, self.act_mode)
             elif fuse and plain_order and L.vx_supports_qkv_proj_rope(*wqkv, desc(normed), desc(q4), desc(k4), desc(v), D, 2):

@@ -1886,6 +1886,12 @@ struct qt_args {
     int      fold;                   // the block scale multiplied into the f16 weights by the weight pass (VX_GEMM_LDS=2)
     const float * norm_w; float norm_eps; // the activation pass applies RMS_NORM and the norm-weight MUL (x is the un-normalised tensor)
     _Float16 * tile_out; int out_tt;      // DUAL: the results leave as the next product's activation tiles (out_tt tiles per k block)
+    // several matrices over the same activations as one virtual matrix (q, k and v): rows [seg_row[s], seg_row[s + 1]) are
+    // matrix s (whole 64-row groups each), stored to its own destination
+    int          nseg;
+    int          seg_row[4];
+    const char * seg_w[3]; uint64_t seg_nb01[3];
+    char *       seg_dst[3]; uint64_t seg_nb1[3], seg_nb3[3];
 };
 
 // one thread = 8 quants of a block: (virtual row, block, j)
@@ -1897,12 +1903,19 @@ __global__ __launch_bounds__(256) void qt_weights_kernel(const qt_args a) {
     const int64_t rt = t / a.n_kb;
     if (rt >= a.n_rt) return;
     const bool    dual = a.w2 != nullptr;
-    const int64_t row  = dual ? 16 * (int64_t) (rt >> 1) + c : 16 * (int64_t) rt + c; // of its own matrix
+    int64_t       row  = dual ? 16 * (int64_t) (rt >> 1) + c : 16 * (int64_t) rt + c; // of its own matrix
     const char *  wsel = dual && (rt & 1) ? a.w2 : a.w;
+    uint64_t      nb01 = a.nb01;
+    int64_t       rows = a.M;
+    if (a.nseg) { // (a 16-row tile lies in one matrix: they are whole 64-row groups)
+        const int sg = row >= a.seg_row[2] ? 2 : row >= a.seg_row[1] ? 1 : 0;
+        wsel = a.seg_w[sg]; nb01 = a.seg_nb01[sg]; rows = a.seg_row[sg + 1] - a.seg_row[sg];
+        row -= a.seg_row[sg];
+    }
     half8_t h = {0, 0, 0, 0, 0, 0, 0, 0};
     float   d = 0.0f;
-    if (row < a.M) {
-        const char * wrow = wsel + (uint64_t) row * a.nb01;
+    if (row < rows) {
+        const char * wrow = wsel + (uint64_t) row * nb01;
         h = q8_unpack(q8_load(wrow, kb, j, a.w_al4 != 0), kb, a.w_al4 != 0);
         const _Float16 dh = *(const _Float16 *) (wrow + kb * VX_Q8_BLOCK);
         d = (float) dh;
@@ -1999,7 +2012,7 @@ __device__ __forceinline__ void qt_dma16(const void * base, uint32_t off, uint32
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "memory");
 }
 
-template <bool DUAL, bool FOLD>
+template <bool DUAL, bool FOLD, bool SEGS = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_q8t_kernel(const qt_args a) {
     extern __shared__ __align__(1024) char qt_smem[]; // per stage: 8 token tiles, 16 row tiles, 256 scales
     typedef __attribute__((address_space(3))) char lds_char;
@@ -2009,11 +2022,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
     // which tile: groups of 4 row tiles x 8 token tiles, a group's 32 work-groups on one XCD
     const int gx = (a.n_rt + 15) / 16, gy = (a.n_tt + 7) / 8; // tiles of 256 rows / 128 tokens
-    const int Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
     const int group = (seq >> 5) * 8 + xcd, within = seq & 31;
-    if (group >= Gx * Gy) return;
-    const int tx = (group % Gx) * 4 + (within & 3), ty = (group / Gx) * 8 + (within >> 2);
+    int tx, ty;
+    if constexpr (SEGS) {
+        // several matrices of few rows in all (q, k and v: 1280 rows, five row tiles): a group is ALL the row tiles of
+        // 32 / gx token tiles, so that every token tile's activations are fetched into one XCD's L2 once and the small
+        // matrices' tiles run beside the large one's (as a group of four row tiles plus a leftover group the last tile's
+        // work-groups ran alone at the end, every one of them fetching its tokens from memory: 309 us against 200 for q alone)
+        const int per = 32 / gx; // (the launcher takes this form for gx <= 8 only)
+        if (within >= gx * per) return;
+        const int wy = within / gx;
+        tx = __builtin_amdgcn_readfirstlane(within - wy * gx);
+        ty = __builtin_amdgcn_readfirstlane(group * per + wy);
+    } else {
+        const int Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
+        if (group >= Gx * Gy) return;
+        tx = (group % Gx) * 4 + (within & 3);
+        ty = (group / Gx) * 8 + (within >> 2);
+    }
     if (tx >= gx || ty >= gy) return;
     const int batch = blockIdx.y, i12 = batch % a.ne12, i13 = batch / a.ne12;
 
@@ -2104,6 +2131,41 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // lane (j, c), tile (rt, tt), register r: token tok0 + 16 tt + 4 j + r, virtual row 16 (rt0 + 4 wr + rt) + c
     const int64_t tok0 = (int64_t) ty * QT_TOKS + 64 * wc;
     char * db = a.dst + (uint64_t) i12 * a.nb2 + (uint64_t) i13 * a.nb3;
+    if constexpr (SEGS) { // (a form of its own: in the common kernel the extra addresses cost the registers it has none to spare of)
+        { // (uniform per wave) the wave's 64 rows belong to one matrix: its destination, its row numbers
+            const int vrow = 16 * (rt0 + 4 * wr);
+            if (vrow >= a.seg_row[3]) return;
+            const int sg = vrow >= a.seg_row[2] ? 2 : vrow >= a.seg_row[1] ? 1 : 0;
+            char *         sb  = a.seg_dst[sg] + (uint64_t) i13 * a.seg_nb3[sg];
+            const uint64_t nb1 = a.seg_nb1[sg];
+            const int      r0  = vrow - a.seg_row[sg];
+            if ((int64_t) (ty + 1) * QT_TOKS <= a.N) { // (uniform) a whole token tile: a uniform base and one 32-bit lane offset, no tests
+                char *         tb = sb + (uint64_t) tok0 * nb1 + (uint64_t) r0 * 4;
+                const uint32_t lo = (uint32_t) ((uint64_t) (4 * j) * nb1 + (uint64_t) c * 4);
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        char * tr = tb + (uint64_t) (16 * tt + r) * nb1; // uniform
+#pragma unroll
+                        for (int rt = 0; rt < 4; ++rt) __builtin_nontemporal_store(acc[rt][tt][r], (float *) (tr + 64 * rt + lo));
+                    }
+                return;
+            }
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                const int row = r0 + 16 * rt + c; // (inside the matrix: whole 64-row groups)
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int64_t tok = tok0 + 16 * tt + 4 * j + r;
+                        if (tok < a.N) __builtin_nontemporal_store(acc[rt][tt][r], (float *) (sb + (uint64_t) tok * nb1 + (uint64_t) row * 4));
+                    }
+            }
+            return;
+        }
+    }
     // A tile inside the matrix stores without tests, at a uniform base plus one 32-bit lane offset (the launcher checks the
     // range): computed per element in 64-bit arithmetic, the addresses of a tile's 64 stores per lane were a fifth of the
     // kernel's vector instructions.
@@ -2245,6 +2307,24 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     const int64_t MV = DUAL ? 2 * a.M : a.M;
     q.n_rt = (int) ((MV + 15) / 16); q.n_tt = a.tile_in ? a.tile_tt : (int) ((a.N + 15) / 16); q.n_kb = (int) (a.K / 32);
     q.tile_out = DUAL ? (_Float16 *) a.tile_out : nullptr; q.out_tt = a.tile_tt;
+    const bool segs = !DUAL && a.nseg > 0; // (the streaming kernel's segments: rotation is the caller's business here)
+    if (segs) {
+        if (a.nseg > 3 || a.res) return false;
+        int at = 0;
+        for (int i = 0; i < 3; ++i) {
+            q.seg_row[i] = at;
+            if (i < a.nseg) {
+                if (a.seg[i].M % 64 || (uint64_t) 128 * a.seg[i].nb1 + 1024 >= (1ull << 32)) return false; // (whole 64-row groups; 32-bit lane offsets in a tile)
+                q.seg_w[i] = a.seg[i].w; q.seg_nb01[i] = a.seg[i].nb01; q.seg_dst[i] = a.seg[i].dst; q.seg_nb1[i] = a.seg[i].nb1; q.seg_nb3[i] = a.seg[i].nb3;
+                at += (int) a.seg[i].M;
+            } else {
+                q.seg_w[i] = nullptr; q.seg_nb01[i] = 0; q.seg_dst[i] = nullptr; q.seg_nb1[i] = 0; q.seg_nb3[i] = 0;
+            }
+        }
+        q.seg_row[3] = at;
+        q.nseg = a.nseg;
+        if (at != a.M) return false;
+    }
     const size_t wt_bytes = (size_t) q.n_kb * q.n_rt * 1024, wd_bytes = ((size_t) q.n_kb * ((q.n_rt + 3) & ~3) * 16 * 4 + 1023) / 1024 * 1024 + 1024; // (+ a scale row's worth: the last stage's 1 KB load of a ragged row tile count stays inside)
     const size_t xt_bytes = a.tile_in ? 0 : (size_t) nbatch * q.n_kb * q.n_tt * 1024;
     static bool raised = false;
@@ -2252,7 +2332,9 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
         if (hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *) gemm_q8t_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
-            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess) {
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void *) gemm_q8t_kernel<false, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) QT_LDS) != hipSuccess) {
             (void) hipGetLastError();
             return false;
         }
@@ -2261,14 +2343,17 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     const int64_t wunits = (int64_t) q.n_kb * q.n_rt * 64, xunits = (int64_t) ((q.n_kb + QT_ACT_UNROLL - 1) / QT_ACT_UNROLL) * q.n_tt * 64;
     if ((wunits + 255) / 256 > 0x7fffffff || (xunits + 255) / 256 > 0x7fffffff) return false;
     const int gx = (q.n_rt + 15) / 16, gy = (q.n_tt + 7) / 8, Gx = (gx + 3) / 4, Gy = (gy + 7) / 8;
-    const int64_t blocks = ((int64_t) Gx * Gy + 7) / 8 * 8 * 32;
+    if (segs && gx > 8) return false; // (the segment form's groups hold all the row tiles)
+    // groups of 32 work-groups, dealt to the XCDs in turn: 4 row tiles x 8 token tiles, or (segments) all gx row tiles x 32 / gx token tiles
+    const int64_t groups = segs ? ((int64_t) gy + 32 / gx - 1) / (32 / gx) : (int64_t) Gx * Gy;
+    const int64_t blocks = (groups + 7) / 8 * 8 * 32;
     if (blocks > 0x7fffffff) return false;
     // the weights' tiles: kept from call to call when the caller has pinned the weights, else made in the workspace
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void) hipGetLastError(); return false; }
     const vx_derived_key key = { dev, fold ? 2 : 1, a.w, DUAL ? a.w2 : nullptr, a.K, a.M, a.nb01 };
     bool fresh = false;
-    char * kept = (char *) vx_derived_get(key, wt_bytes + wd_bytes, st, &fresh);
+    char * kept = segs ? nullptr : (char *) vx_derived_get(key, wt_bytes + wd_bytes, st, &fresh); // (three matrices: tiles made per call)
     void * ws = nullptr;
     if ((t_ws_status = vx_workspace(st, a.ws_offset + (kept ? 0 : wt_bytes + wd_bytes) + xt_bytes, &ws)) != VX_OK) {
         (void) hipGetLastError();
@@ -2285,6 +2370,13 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     if (a.tile_in) {} // (the activations are the tiles the product before left)
     else if (a.norm_w) vx_launch(qt_acts_norm_kernel, dim3((unsigned) q.n_tt, (unsigned) nbatch), dim3(1024), 0, st, q);
     else          vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
+    if constexpr (!DUAL) {
+        if (segs) {
+            if (fold) vx_launch(gemm_q8t_kernel<false, true, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
+            else      vx_launch(gemm_q8t_kernel<false, false, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
+            return true;
+        }
+    }
     if (fold) vx_launch(gemm_q8t_kernel<DUAL, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     else      vx_launch(gemm_q8t_kernel<DUAL, false>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
     return true;
@@ -2802,6 +2894,59 @@ static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * 
                          float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, int act_mode,
                          vx_stream stream);
 
+// The same group at prefill sizes: RMS_NORM and the norm weight in the activation pass of the pre-tiled kernel, q, k and v
+// as one virtual matrix over those tiles (one product launch instead of three, x laid out once), each stored to its own
+// destination; the two rotations follow as launches of their own, in place.  Taken when every piece is what the separate
+// nodes would run -- each product on a tiled kernel with its K whole (the pre-tiled kernel and the LDS-operand kernel form
+// and add a block's products identically) -- so the bits are those of RMS_NORM, MUL, three MUL_MATs and two ROPEs.
+static bool qkv_tiled_fill(mm_args & a, const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,
+                           const vx_tensor * x, const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode, int act_mode) {
+    if (!wq || !wk || !wv || !x || !norm_w || !q_dst || !k_dst || !v_dst || act_mode != VX_ACT_FLOAT || gemm_lds_mode() == 0) return false;
+    const vx_tensor * ws[3] = { wq, wk, wv };
+    const vx_tensor * ds[3] = { q_dst, k_dst, v_dst };
+    if (!norm_prologue_ok(x, norm_w) || x->type != VX_TYPE_F32 || x->ne[2] != 1 || x->nb[0] != 4 || x->ne[3] > 65535) return false;
+    if (mode != 2 || n_dims <= 0 || !qkv_rope_dst_ok(wq, x, q_dst, n_dims) || !qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return false;
+    if (v_dst->type != VX_TYPE_F32 || v_dst->nb[0] != 4 || v_dst->nb[1] % 4 || v_dst->nb[3] % 4 || v_dst->nb[1] < (uint64_t) v_dst->ne[0] * 4 ||
+        (v_dst->ne[3] > 1 && v_dst->nb[3] < v_dst->nb[1] * (uint64_t) v_dst->ne[1])) return false;
+    if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return false;
+    a = mm_args{};
+    a.x = (const char *) x->data;
+    a.K = wq->ne[0]; a.N = x->ne[1]; a.M = 0;
+    a.nb11 = x->nb[1]; a.nb12 = x->nb[2]; a.nb13 = x->nb[3];
+    a.ne12 = 1; a.r2 = 1; a.r3 = (int) x->ne[3];
+    a.w_aligned = 1;
+    a.nseg = 3;
+    const int nbatch = (int) x->ne[3];
+    for (int i = 0; i < 3; ++i) {
+        const vx_tensor * w = ws[i];
+        if (w->type != VX_TYPE_Q8_0 || w->ne[0] != wq->ne[0] || w->ne[2] != 1 || w->ne[3] != 1 || !vx_positive(w) || w->ne[1] % 64) return false;
+        if (w->nb[0] != VX_Q8_BLOCK || w->nb[1] < vx_row_size(w->type, w->ne[0])) return false;
+        gv_seg & sg = a.seg[i];
+        sg.w = (const char *) w->data; sg.dst = (char *) ds[i]->data;
+        sg.M = w->ne[1]; sg.nb01 = w->nb[1];
+        sg.nb1 = (uint64_t) sg.M * 4; sg.nb2 = 0; sg.nb3 = (uint64_t) sg.M * 4 * x->ne[1];
+        if (i == 2) { sg.nb1 = v_dst->nb[1]; sg.nb3 = v_dst->nb[3]; }
+        a.w_aligned = a.w_aligned && ((uintptr_t) w->data % 4 == 0) && w->nb[1] % 4 == 0;
+        a.M += sg.M;
+        // the product on its own: a tiled kernel with its K whole (not the streaming kernel, no cut K, not the older kernels)
+        const int64_t t64 = ((sg.M + 63) / 64) * ((a.N + 63) / 64) * nbatch;
+        const bool    big = ((sg.M + 127) / 128) * ((a.N + 127) / 128) * nbatch >= 192;
+        if (gemv_shape_ok(a.N, sg.M, a.K) || a.K % (32 * GL_KC) || gemm_lds_cut(sg.M, a.N, a.K, nbatch) != 1 || (!big && t64 < 64)) return false;
+    }
+    a.w = a.seg[0].w; a.dst = a.seg[0].dst; a.nb01 = a.seg[0].nb01; a.nb1 = a.seg[0].nb1; a.nb3 = a.seg[0].nb3;
+    a.x_aligned = ((uintptr_t) x->data % 16 == 0) && x->nb[1] % 16 == 0 && x->nb[3] % 16 == 0;
+    a.norm_w = (const float *) norm_w->data; a.norm_eps = eps;
+    return a.w_aligned && a.x_aligned && norm_w->data && (uintptr_t) norm_w->data % 16 == 0 && gemm_q8t_takes(a, nbatch, false);
+}
+
+extern "C" int vx_supports_norm_qkv_proj_rope_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * wq, const vx_tensor * wk,
+                                                    const vx_tensor * wv, const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst,
+                                                    int n_dims, int mode, int act_mode) {
+    mm_args a;
+    return qkv_tiled_fill(a, norm_w, 0.0f, wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode, act_mode) &&
+           vx_supports_rope(q_dst, q_dst, n_dims, mode) && vx_supports_rope(k_dst, k_dst, n_dims, mode);
+}
+
 extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x,
                                       const int32_t * pos, const float * freq_factors, const vx_tensor * q_dst, const vx_tensor * k_dst,
                                       const vx_tensor * v_dst, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
@@ -2825,6 +2970,22 @@ extern "C" vx_status vx_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor 
                                            int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
                                            float beta_fast, float beta_slow, int act_mode, vx_stream stream) {
     if (!x || !norm_w || !norm_w->data) return vx_fail(VX_ERR_INVALID, "norm_qkv_proj_rope: null tensor");
+    if (!vx_supports_norm_qkv_proj_rope(x, norm_w, wq, wk, wv, q_dst, k_dst, v_dst, n_dims, mode) &&
+        vx_supports_norm_qkv_proj_rope_tiled(x, norm_w, wq, wk, wv, q_dst, k_dst, v_dst, n_dims, mode, act_mode)) {
+        // prefill sizes: the norm in the activation pass, one product launch for the three matrices, the rotations in place
+        if (!pos || !x->data || !q_dst->data || !k_dst->data || !v_dst->data || !wq->data || !wk->data || !wv->data)
+            return vx_fail(VX_ERR_INVALID, "norm_qkv_proj_rope: null data");
+        if (!(eps >= 0.0f)) return vx_fail(VX_ERR_INVALID, "norm_qkv_proj_rope: eps must be >= 0");
+        mm_args a;
+        if (!qkv_tiled_fill(a, norm_w, eps, wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode, act_mode))
+            return vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: shape outside the pre-tiled kernel");
+        (void) take_ws_status();
+        if (!launch_gemm_q8t<false>(a, (int) x->ne[3], (hipStream_t) stream, gemm_lds_mode() == 2))
+            return ws_failed() ? take_ws_status() : vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: the product could not be launched");
+        vx_status rc = vx_rope(q_dst, pos, freq_factors, q_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, stream);
+        if (rc == VX_OK) rc = vx_rope(k_dst, pos, freq_factors, k_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, stream);
+        return rc;
+    }
     if (!vx_supports_norm_qkv_proj_rope(x, norm_w, wq, wk, wv, q_dst, k_dst, v_dst, n_dims, mode) || (uintptr_t) x->data % 16 ||
         (uintptr_t) norm_w->data % 16)
         return vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: as qkv_proj_rope, with 16-byte aligned rows of at most 1024 floats and one F32 norm weight row");

@@ -1138,7 +1138,11 @@ bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const re
         const vx_tensor nw = to_vx(scale->src[1]);
         float eps;
         memcpy(&eps, norm->op_params, sizeof(float));
-        if (!vx_supports_norm_qkv_proj_rope(&xx, &nw, &wq, &wk, &wv, &dq, &dk, &dv, n_dims, mode) || (uintptr_t) xx.data % 16 || (uintptr_t) nw.data % 16) return false;
+        // (decode sizes: one launch of the streaming kernel; prefill sizes: the norm in the pre-tiled kernel's activation pass,
+        // the three matrices as one product, the rotations behind it)
+        if ((!vx_supports_norm_qkv_proj_rope(&xx, &nw, &wq, &wk, &wv, &dq, &dk, &dv, n_dims, mode) &&
+             !vx_supports_norm_qkv_proj_rope_tiled(&xx, &nw, &wq, &wk, &wv, &dq, &dk, &dv, n_dims, mode, mul_mat_act_mode())) ||
+            (uintptr_t) xx.data % 16 || (uintptr_t) nw.data % 16) return false;
         *rc = vx_norm_qkv_proj_rope(&xx, &nw, eps, &wq, &wk, &wv, posd, ffd, &dq, &dk, &dv, n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3],
                                     fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
         done.insert(scale); done.insert(mq);
