@@ -320,6 +320,20 @@ VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_te
                                                 const vx_tensor * v_past, const vx_tensor * v_cur, const vx_tensor * mask,
                                                 const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
                                                 const vx_tensor * v_slot, const vx_tensor * dst);
+/* The prefill attention block of attention_forward (src/minicpm.cpp:682-713) as one call: vx_flash_attn_ext over the
+ * projections' own k / v, followed by vx_kv_store_sync on its result.  The cache write and the ordering scalar are
+ * launched first and the scalar is added in the attention kernel's epilogue (as vx_flash_attn_ext_add1 adds one), so
+ * the tokens x hidden result is stored once instead of stored, read and stored again.  For query counts the LDS-tiled
+ * kernel takes (logit_softcap 0) and the prefill-sized cache writes vx_kv_store_sync takes (more than 65536 elements
+ * each); the slots must not overlap anything the attention reads.  Result and cache contents equal the two separate calls'. */
+VX_API vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                         const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                         const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst,
+                                         float scale, float max_bias, float logit_softcap, float sync_scale,
+                                         float sync_bias, vx_stream stream);
+VX_API int vx_supports_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                            const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                            const vx_tensor * v_slot, const vx_tensor * dst, float logit_softcap);
 /* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
  * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for few tokens
  * (as above).  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE

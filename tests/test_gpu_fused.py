@@ -367,6 +367,70 @@ def test_kv_store_sync_prefill_sized(pkg, gpu, B, T, Hkv, D, H, f16, poison):
     assert torch.equal(a.nan_to_num(123.0), x2.nan_to_num(123.0))
 
 
+@pytest.mark.parametrize("B,T,Hkv,H", [(2, 512, 2, 16), (3, 600, 2, 16), (2, 1100, 1, 4), (16, 300, 2, 16)])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("poison", [None, "nan"])
+def test_flash_attn_ext_store(pkg, gpu, B, T, Hkv, H, f16, poison):
+    """The prefill attention block of attention_forward (src/minicpm.cpp:682-713) as one call: the cache write and its
+    ordering scalar are launched first and the scalar joins the attention's epilogue.  Against vx_flash_attn_ext followed
+    by vx_kv_store_sync, bit for bit, cache contents included; a NaN in the written values poisons the whole result,
+    as it does through the reference's ADD1."""
+    import torch
+    say(f"prefill attention + cache write as one call B={B} T={T} Hkv={Hkv} H={H} f16 cache={f16} poison={poison}")
+    L, d = pkg.lib(), pkg.desc
+    D = 64
+    g = rng("f-attn-store", B, T, Hkv, H)
+    n_past = 5
+    q = dev(g.standard_normal((B, T, H, D)).astype(np.float32))
+    k = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    v = dev(g.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    if poison:
+        k[B - 1, T // 3, 0, 7] = float("nan")
+    mask = torch.full((T, T), float("-inf"), dtype=torch.float16, device="cuda").triu(1).contiguous()
+    qd, kd, vd = d(q.transpose(1, 2)), d(k.transpose(1, 2)), d(v.transpose(1, 2))
+    cdt = torch.float16 if f16 else torch.float32
+    kc1, vc1, kc2, vc2 = (torch.zeros((B, Hkv, n_past + T + 3, D), dtype=cdt, device="cuda") for _ in range(4))
+    slot = lambda c: c[:, :, n_past:n_past + T].transpose(1, 2)
+    scale = 1.0 / 8.0
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    ok(pkg, L.vx_flash_attn_ext(qd, kd, vd, d(mask), None, d(a), scale, 0.0, 0.0, None), "flash_attn_ext")
+    ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc1)), d(v), d(slot(vc1)), d(a), d(a), 0.25, 0.5, None), "kv_store_sync")
+    b = torch.full_like(a, 7.0)
+    assert L.vx_supports_flash_attn_ext_store(qd, kd, vd, d(mask), d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b), 0.0) == 1
+    ok(pkg, L.vx_flash_attn_ext_store(qd, kd, vd, d(mask), None, d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b), scale, 0.0, 0.0,
+                                      0.25, 0.5, None), "flash_attn_ext_store")
+    torch.cuda.synchronize()
+    assert torch.equal(kc1.view(torch.uint8), kc2.view(torch.uint8)) and torch.equal(vc1.view(torch.uint8), vc2.view(torch.uint8))
+    assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
+    if poison:
+        assert not bool(torch.isfinite(b).any())
+    else:
+        assert bool(torch.isfinite(b).all())
+    # a second call on the same stream with another scalar: the workspace's front is written anew
+    ok(pkg, L.vx_flash_attn_ext_store(qd, kd, vd, d(mask), None, d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(b), scale, 0.0, 0.0,
+                                      0.0, 0.0, None), "flash_attn_ext_store again")
+    ok(pkg, L.vx_flash_attn_ext(qd, kd, vd, d(mask), None, d(a), scale, 0.0, 0.0, None), "flash_attn_ext")
+    ok(pkg, L.vx_kv_store_sync(d(k), d(slot(kc1)), d(v), d(slot(vc1)), d(a), d(a), 0.0, 0.0, None), "kv_store_sync")
+    torch.cuda.synchronize()
+    assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
+
+
+def test_flash_attn_ext_store_limits(pkg, gpu):
+    import torch
+    say("prefill attention + cache write: decode-sized and softcapped calls are refused")
+    L, d = pkg.lib(), pkg.desc
+    z = lambda *s: torch.zeros(s, dtype=torch.float32, device="cuda")
+    q, k, c, o = z(2, 1, 16, 64), z(2, 1, 2, 64), z(2, 2, 64, 64), z(2, 1, 16, 64)
+    s = c[:, :, :1].transpose(1, 2)
+    assert L.vx_supports_flash_attn_ext_store(d(q.transpose(1, 2)), d(k.transpose(1, 2)), d(k.transpose(1, 2)), None, d(k), d(s), d(k), d(s), d(o), 0.0) == 0
+    q, k, c, o = z(2, 512, 16, 64), z(2, 512, 2, 64), z(2, 2, 600, 64), z(2, 512, 16, 64)
+    s = c[:, :, :512].transpose(1, 2)
+    args = (d(q.transpose(1, 2)), d(k.transpose(1, 2)), d(k.transpose(1, 2)), None, d(k), d(s), d(k), d(s), d(o))
+    assert L.vx_supports_flash_attn_ext_store(*args, 0.0) == 1
+    assert L.vx_supports_flash_attn_ext_store(*args, 30.0) == 0
+    assert L.vx_flash_attn_ext_store(args[0], args[1], args[2], None, None, *args[4:], 0.125, 0.0, 30.0, 0.0, 0.0, None) != 0
+
+
 @pytest.mark.parametrize("shape", [(8, 128), (1, 1), (3, 5, 7, 1000), (2, 4100), (16, 2, 64)])
 def test_sum_rows_matches_ggml_cpu_arithmetic(gpu, shape):
     """GGML_OP_SUM_ROWS (ggml_compute_forward_sum_rows_f32, ops.cpp:1451-1482): a row's elements added in double and

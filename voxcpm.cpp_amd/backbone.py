@@ -239,8 +239,18 @@ class MiniCPMBackbone:
                     call(L.vx_concat, desc(vp), desc(v_all), desc(vall), 1)
                     k_all, v_all = kall, vall
             if k_all is not None:
-                call(L.vx_flash_attn_ext, desc(q4.transpose(1, 2)), desc(k_all), desc(v_all), desc(mask), None, desc(attn),
-                     scale, 0.0, 0.0)
+                qd = desc(q4.transpose(1, 2))
+                kw = kc[:, :, n_past:n_past + T].transpose(1, 2)
+                vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
+                if write_kv and chain and fuse and L.vx_supports_flash_attn_ext_store(qd, desc(k_all), desc(v_all), desc(mask), desc(k4), desc(kw),
+                                                                                      desc(v4), desc(vw), desc(attn), 0.0):
+                    # a prefill: the cache write and its scalar first, the scalar added in the attention's epilogue
+                    keep += [kw, vw]
+                    call(L.vx_flash_attn_ext_store, qd, desc(k_all), desc(v_all), desc(mask), None, desc(k4), desc(kw), desc(v4), desc(vw),
+                         desc(attn), scale, 0.0, 0.0, 0.0, 0.0)
+                    stored = True
+                else:
+                    call(L.vx_flash_attn_ext, qd, desc(k_all), desc(v_all), desc(mask), None, desc(attn), scale, 0.0, 0.0)
             grouped = stored
             if write_kv and not stored:
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)   # ggml [D, Hkv, T, B], src/minicpm.cpp:222-236

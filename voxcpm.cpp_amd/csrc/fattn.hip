@@ -1113,6 +1113,45 @@ extern "C" vx_status vx_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_t
                   k_src, k_slot, v_src, v_slot, sync_scale, sync_bias);
 }
 
+// attention_forward at prefill size (src/minicpm.cpp:682-713): FLASH_ATTN_EXT over the projections' own K/V, then the
+// cache write, its two sums, the ordering scalar and the ADD1 on the attention's result.  The write and the scalar are
+// launched first and the scalar joins the attention's epilogue, so the result is stored once.
+struct pf_store_ctx {
+    const vx_tensor * k_src, * k_slot, * v_src, * v_slot;
+    float scale, bias;
+};
+constexpr size_t PF_STORE_FRONT = 4096, PF_STORE_ADDEND_AT = 2048; // 256 block totals, then the scalar
+
+static vx_status pf_store_launch(void * front, void * ctx, hipStream_t st) {
+    const pf_store_ctx * c = (const pf_store_ctx *) ctx;
+    return vx_kv_store_scalar(c->k_src, c->k_slot, c->v_src, c->v_slot, c->scale, c->bias, front, (float *) ((char *) front + PF_STORE_ADDEND_AT), st);
+}
+
+extern "C" int vx_supports_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                                const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                                const vx_tensor * v_slot, const vx_tensor * dst, float logit_softcap) {
+    static const bool off = getenv("VX_FA_NO_PREFILL") != nullptr;
+    if (off || !vx_supports_flash_attn_ext(q, k, v, mask, dst)) return 0;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (uintptr_t) dst->data % 16) return 0;
+    if (!vx_fattn_prefill_accepts(q, k, logit_softcap)) return 0;
+    return vx_kv_store_scalar_ok(k_src, k_slot, v_src, v_slot) ? 1 : 0;
+}
+
+extern "C" vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                             const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                             const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst, float scale,
+                                             float max_bias, float logit_softcap, float sync_scale, float sync_bias, vx_stream stream) {
+    if (!q || !k || !v || !k_src || !k_slot || !v_src || !v_slot || !dst || !q->data || !k->data || !v->data || !k_src->data ||
+        !k_slot->data || !v_src->data || !v_slot->data || !dst->data || (mask && !mask->data))
+        return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: null tensor");
+    if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, dst, logit_softcap))
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store: a query count the LDS-tiled kernel takes, and prefill-sized cache writes (more than 65536 elements each)");
+    if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: max_bias > 0 requires a mask");
+    pf_store_ctx c{ k_src, k_slot, v_src, v_slot, sync_scale, sync_bias };
+    const vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_launch, &c };
+    return vx_fattn_prefill(q, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream, &front);
+}
+
 // ---- the entry point that allocates nothing ------------------------------------------------------------
 // The key-range partials of vx_flash_attn_ext_static live in a fixed array in device memory that is part of the
 // loaded code object: every GPU the library runs on holds its own copy, at its own address, until the process

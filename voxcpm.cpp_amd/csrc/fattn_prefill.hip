@@ -662,7 +662,7 @@ bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float lo
 
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                            const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
-                           float logit_softcap, hipStream_t st) {
+                           float logit_softcap, hipStream_t st, const vx_pf_front * front) {
     if (!vx_fattn_prefill_accepts(q, k, logit_softcap)) return VX_ERR_UNSUPPORTED;
     const int Hq = (int) q->ne[2], Hkv = (int) k->ne[2], gqa = Hq / Hkv;
     const int n_q = (int) q->ne[1], n_kv = (int) k->ne[1];
@@ -705,11 +705,18 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     const size_t flag_bytes = mask ? ((bits_bytes + (size_t) a.nem2 * a.nem3 * n_rb * n_tiles + 255) & ~(size_t) 255) : 0;
     const size_t plane = a.kv_f32 ? (size_t) k->ne[3] * Hkv * n_kv * 64 * sizeof(_Float16) : 0;
     char * ws = nullptr;
-    if (flag_bytes + 3 * plane) {
+    const size_t front_bytes = front ? front->bytes : 0;
+    if (front_bytes + flag_bytes + 3 * plane) {
         void * p = nullptr;
-        vx_status rc = vx_workspace(st, flag_bytes + 3 * plane, &p);
+        vx_status rc = vx_workspace(st, front_bytes + flag_bytes + 3 * plane, &p);
         if (rc != VX_OK) return rc;
         ws = (char *) p;
+    }
+    if (front) { // the caller's launches first: they own the front of the block, and leave the addend there
+        const vx_status rc = front->launch(ws, front->ctx, st);
+        if (rc != VX_OK) return rc;
+        a.add1 = (const float *) (ws + front->addend_at);
+        ws += front_bytes;
     }
     if (mask) {
         vx_launch(pf_mask_flags_kernel, dim3((unsigned) n_tiles, (unsigned) n_rb, (unsigned) (a.nem2 * a.nem3)), dim3(64), 0, st,

@@ -1073,7 +1073,8 @@ __global__ __launch_bounds__(1024) void kv_store_large_kernel(const kvs_args a, 
     if (threadIdx.x == 0) partials[blockIdx.x] = t;
 }
 
-__global__ __launch_bounds__(256) void kv_sync_add1_kernel(const kvs_args a, const double * partials) {
+// the block totals of the two sums, added in block order, as the scalar of the SCALE node (256 threads)
+__device__ __forceinline__ float kvs_scalar_of_totals(const kvs_args & a, const double * partials) {
     __shared__ double part[2 * SUM_BLOCKS];
     __shared__ float  y_s;
     static_assert(2 * SUM_BLOCKS == 256, "a partial per thread");
@@ -1086,7 +1087,17 @@ __global__ __launch_bounds__(256) void kv_sync_add1_kernel(const kvs_args a, con
         y_s = kvs_scalar((float) tk, (float) tv, a.scale, a.bias);
     }
     __syncthreads();
-    const float y = y_s;
+    return y_s;
+}
+
+// the scalar alone, for a consumer that adds it itself (the prefill attention's epilogue)
+__global__ __launch_bounds__(256) void kv_sync_scalar_kernel(const kvs_args a, const double * partials, float * y_out) {
+    const float y = kvs_scalar_of_totals(a, partials);
+    if (threadIdx.x == 0) *y_out = y;
+}
+
+__global__ __launch_bounds__(256) void kv_sync_add1_kernel(const kvs_args a, const double * partials) {
+    const float y = kvs_scalar_of_totals(a, partials);
     const uint32_t n0 = (uint32_t) a.ne[0], n1 = (uint32_t) a.ne[1], n2 = (uint32_t) a.ne[2];
     const uint64_t nx = (uint64_t) n0 * n1 * (uint64_t) (n2 * a.ne[3]);
     if (a.dense4) { // (a prefill's attention output: 256 MiB at 16 x 4096 tokens; element by element with its index
@@ -1907,6 +1918,34 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
         const unsigned blocks = (unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096);
         vx_launch(kv_sync_add1_kernel, dim3(blocks), dim3(256), 0, st, a, (const double *) ws);
     }
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
+// The cache write and the ordering scalar of vx_kv_store_sync without its ADD1: the scalar goes to y_out for a kernel
+// launched behind this call on the same stream to add.  partials: 2 * SUM_BLOCKS doubles of device memory.
+bool vx_kv_store_scalar_ok(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot) {
+    // (a prefill's write only: attention shapes with a smaller one do not reach the kernel that adds the scalar)
+    return k && k_slot && v && v_slot && kvs_large(k, k_slot, v, v_slot);
+}
+
+vx_status vx_kv_store_scalar(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                             float scale, float bias, void * partials, float * y_out, hipStream_t st) {
+    if (!vx_kv_store_scalar_ok(k, k_slot, v, v_slot)) return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_scalar: shapes vx_kv_store_sync does not take");
+    kvs_args a;
+    kvs_side_fill(a.k, k, k_slot);
+    kvs_side_fill(a.v, v, v_slot);
+    a.x = nullptr; a.d = nullptr;
+    for (int i = 0; i < 4; ++i) { a.ne[i] = 0; a.nbx[i] = 0; a.nbd[i] = 0; }
+    a.scale = scale; a.bias = bias;
+    a.dense4 = 0;
+    a.defer = nullptr;
+    const dim3 grid(2 * SUM_BLOCKS), block(1024);
+    if (a.k.vec && a.v.vec) vx_launch(kv_store_large_kernel<true, true>, grid, block, 0, st, a, (double *) partials);
+    else if (a.k.vec)       vx_launch(kv_store_large_kernel<true, false>, grid, block, 0, st, a, (double *) partials);
+    else if (a.v.vec)       vx_launch(kv_store_large_kernel<false, true>, grid, block, 0, st, a, (double *) partials);
+    else                    vx_launch(kv_store_large_kernel<false, false>, grid, block, 0, st, a, (double *) partials);
+    vx_launch(kv_sync_scalar_kernel, dim3(1), dim3(256), 0, st, a, (const double *) partials, y_out);
     VX_LAUNCH_CHECK();
     return VX_OK;
 }

@@ -87,10 +87,25 @@ void   vx_derived_abandon(const vx_derived_key & key, hipStream_t stream); // a 
 // so that the first call of the entry point does no set-up work
 vx_status vx_fattn_static_setup(void);
 
+// Work that a caller of vx_fattn_prefill wants launched in front of the attention's own kernels, with a piece of the
+// call's workspace block to itself: `bytes` (a multiple of 256) at the front of the block, handed to `launch` once the
+// block is known; the float at `addend_at` bytes into it is then the attention's addend.
+struct vx_pf_front {
+    size_t bytes, addend_at;
+    vx_status (*launch)(void * front, void * ctx, hipStream_t stream);
+    void * ctx;
+};
+
 // LDS-tiled prefill kernel (fattn_prefill.hip); VX_ERR_UNSUPPORTED means "use the general kernel"
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                            const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
-                           float logit_softcap, hipStream_t stream);
+                           float logit_softcap, hipStream_t stream, const vx_pf_front * front = nullptr);
+
+// vx_kv_store_sync's cache write and ordering scalar without the ADD1 (glue.hip): the scalar is left in *y_out
+// (device memory), partials are 2 KiB of device memory
+bool      vx_kv_store_scalar_ok(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot);
+vx_status vx_kv_store_scalar(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
+                             float scale, float bias, void * partials, float * y_out, hipStream_t stream);
 
 // whether vx_fattn_prefill would take this shape (k describes all keys)
 bool vx_fattn_prefill_accepts(const vx_tensor * q, const vx_tensor * k, float logit_softcap);

@@ -1050,6 +1050,39 @@ int compute_kv2_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i,
     return last;
 }
 
+// FLASH_ATTN_EXT at prefill size directly followed by the cache-write group on its result: one call that launches the
+// write and the ordering scalar first and lets the attention add the scalar as it stores.  The write moves in front of
+// the attention, so its slots must lie apart from everything the attention reads.  Returns the index of the group's
+// last node, or -1.
+int compute_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, vx_status * rc) {
+    const ggml_tensor * f = g->nodes[i];
+    const int j = next_real(g, i);
+    if (j >= g->n_nodes || g->nodes[j]->op != GGML_OP_CPY || !private_to_group(readers, f)) return -1;
+    if (f->src[4] && (f->src[4]->type != GGML_TYPE_F32 || f->src[4]->ne[0] != f->src[0]->ne[2])) return -1;
+    ggml_tensor * n[9];
+    const int last = match_kv_store_group(g, j, readers, n);
+    if (last < 0 || n[8]->src[0] != f) return -1;
+    const ggml_tensor * dst = n[8];
+    for (int k = 0; k < 5; ++k) {
+        const ggml_tensor * r = f->src[k];
+        if (r && (!apart(dst, r) || !apart(n[0], r) || !apart(n[3], r))) return -1;
+    }
+    float scale, max_bias, softcap, sc, bias;
+    memcpy(&scale, (const float *) f->op_params + 0, sizeof(float));
+    memcpy(&max_bias, (const float *) f->op_params + 1, sizeof(float));
+    memcpy(&softcap, (const float *) f->op_params + 2, sizeof(float));
+    memcpy(&sc, (const float *) n[7]->op_params + 0, sizeof(float));
+    memcpy(&bias, (const float *) n[7]->op_params + 1, sizeof(float));
+    const vx_tensor q = to_vx(f->src[0]), k = to_vx(f->src[1]), v = to_vx(f->src[2]), ksrc = to_vx(n[0]->src[0]), ks = to_vx(n[0]),
+                    vsrc = to_vx(n[3]->src[0]), vs = to_vx(n[3]), d = to_vx(dst);
+    vx_tensor m;
+    if (f->src[3]) m = to_vx(f->src[3]);
+    if (!vx_supports_flash_attn_ext_store(&q, &k, &v, f->src[3] ? &m : nullptr, &ksrc, &ks, &vsrc, &vs, &d, softcap)) return -1;
+    *rc = vx_flash_attn_ext_store(&q, &k, &v, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
+                                  &ksrc, &ks, &vsrc, &vs, &d, scale, max_bias, softcap, sc, bias, ctx->stream);
+    return last;
+}
+
 vx_status compute_kv2_attention(backend_ctx * ctx, const ggml_tensor * f, const kv2_group & grp) {
     float scale, max_bias, softcap;
     memcpy(&scale, (const float *) f->op_params + 0, sizeof(float));
@@ -1711,6 +1744,18 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
                     return GGML_STATUS_FAILED;
                 }
                 continue;
+            }
+            if (fusion) {
+                const int last = compute_attention_store(ctx, cgraph, i, readers, &rc);
+                if (last >= 0) {
+                    ++launches;
+                    if (rc != VX_OK) {
+                        NODE_FAILED("ggml-gfx950: node %d (%s, attention + cache write) failed with status %d: %s\n", i, node->name, (int) rc, vx_last_error());
+                        return GGML_STATUS_FAILED;
+                    }
+                    i = last;
+                    continue;
+                }
             }
         }
         if (fusion && i + 1 < cgraph->n_nodes) {
