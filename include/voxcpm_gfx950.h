@@ -365,7 +365,9 @@ VX_API int vx_supports_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor *
                                           const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode);
 /* the same call at prefill sizes (Q8_0 weights, VX_ACT_FLOAT, every product one that a tiled kernel runs with its K
  * whole): the norm in the pre-tiled kernel's activation pass, q, k and v as one product launch over those tiles, the two
- * rotations as launches of their own in place.  Same bits as RMS_NORM, MUL, three MUL_MATs, two ROPEs. */
+ * rotations in that product's epilogue (heads of 64 rows: the angles come from a table filled in front of the product by
+ * vx_rope's own arithmetic; VX_QKV_ROPE_EPILOGUE=0 or other head sizes: launches of their own, in place).  Same bits as
+ * RMS_NORM, MUL, three MUL_MATs, two ROPEs. */
 VX_API int vx_supports_norm_qkv_proj_rope_tiled(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * wq,
                                                 const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * q_dst,
                                                 const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode, int act_mode);

@@ -911,13 +911,15 @@ def test_norm_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act):
 
 @pytest.mark.parametrize("T,B,H,Hkv,D,K,batched", [(2304, 1, 16, 2, 64, 1024, False), (1100, 2, 16, 2, 64, 1024, False), (2100, 2, 16, 2, 64, 1024, True),
                                                     (1030, 1, 8, 4, 128, 768, False)])
-def test_norm_qkv_proj_rope_at_prefill_sizes(pkg, gpu, T, B, H, Hkv, D, K, batched, monkeypatch):
+@pytest.mark.parametrize("yarn", [False, True])
+def test_norm_qkv_proj_rope_at_prefill_sizes(pkg, gpu, T, B, H, Hkv, D, K, batched, yarn, monkeypatch):
     """RMS_NORM, MUL, the q, k and v projections and both rotations at prefill sizes as one call: the norm in the pre-tiled
-    kernel's activation pass, the three matrices as one product over those tiles, the rotations in place behind it.  Against
-    the separate calls (RMS_NORM+MUL, three MUL_MATs, two ROPEs): the same bits -- the sequences flattened into one token
-    dimension or as a batch, ragged token tiles, 64- and 128-wide heads."""
+    kernel's activation pass, the three matrices as one product over those tiles, the rotations in that product's epilogue
+    from a table of angles (heads of 64 rows) or in place behind it (128).  Against the separate calls (RMS_NORM+MUL, three
+    MUL_MATs, two ROPEs): the same bits -- the sequences flattened into one token dimension or as a batch, ragged token
+    tiles, 64- and 128-wide heads, plain and YaRN-mixed angles with frequency factors."""
     import torch
-    say(f"fused rms_norm+mul, q/k/v as one pre-tiled product, rope: T={T} B={B} H={H}/{Hkv} D={D} K={K} batched={batched}")
+    say(f"fused rms_norm+mul, q/k/v as one pre-tiled product, rope: T={T} B={B} H={H}/{Hkv} D={D} K={K} batched={batched} yarn={yarn}")
     L, d = pkg.lib(), pkg.desc
     monkeypatch.setenv("VX_GEMM_Q8T", "2")
     g = rng("f-nqkv-t", T, B, H, D, K)
@@ -927,7 +929,7 @@ def test_norm_qkv_proj_rope_at_prefill_sizes(pkg, gpu, T, B, H, Hkv, D, K, batch
     nw = dev((1 + 0.1 * g.standard_normal(K)).astype(np.float32))
     pos = torch.arange(300, 300 + T, dtype=torch.int32, device="cuda")
     ff = dev((1.0 + g.random(D // 2)).astype(np.float32))
-    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+    rope_args = (D, 2, 4096, 10000.0, 0.5, 1.0, 1.1, 32.0, 1.0) if yarn else (D, 2, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
 
     def outs():
         return (torch.full((B, T, H, D), float("nan"), dtype=torch.float32, device="cuda"),

@@ -1892,7 +1892,23 @@ struct qt_args {
     int          seg_row[4];
     const char * seg_w[3]; uint64_t seg_nb01[3];
     char *       seg_dst[3]; uint64_t seg_nb1[3], seg_nb3[3];
+    // the NEOX rotation of GGML_OP_ROPE on the first rope_segs matrices (heads of 64 rows, rotated whole), applied to the
+    // accumulators before the store: (cos, sin) of (token of a batch entry, pair) from a table that a kernel in front of
+    // the product fills with the ROPE kernel's own arithmetic
+    const float2 * rope_tab; int rope_segs;
 };
+
+// (cos, sin) of every (position index, pair): what rope_heads_kernel forms per (token, pair), once per call
+// (one wave a work-group: a thread's work is a chain of up to 31 multiplications and a sine and cosine of a large angle,
+// so the kernel's time is one thread's latency and the waves are spread over every SIMD)
+__global__ __launch_bounds__(64) void qt_rope_table_kernel(const int32_t * __restrict__ pos, const float * __restrict__ ff, rope_params p,
+                                                           int N, int T, float2 * __restrict__ tab) {
+    const uint32_t gid = blockIdx.x * 64u + threadIdx.x, tok = gid >> 5, ip = gid & 31;
+    if (tok >= (uint32_t) N) return;
+    float c, sn;
+    rope_cos_sin(p, (float) pos[tok % (uint32_t) T], (int) ip, ff ? ff[ip] : 1.0f, c, sn);
+    tab[gid] = make_float2(c, sn);
+}
 
 // one thread = 8 quants of a block: (virtual row, block, j)
 __global__ __launch_bounds__(256) void qt_weights_kernel(const qt_args a) {
@@ -2139,6 +2155,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             char *         sb  = a.seg_dst[sg] + (uint64_t) i13 * a.seg_nb3[sg];
             const uint64_t nb1 = a.seg_nb1[sg];
             const int      r0  = vrow - a.seg_row[sg];
+            if (a.rope_tab && sg < a.rope_segs) { // (uniform) the wave's 64 rows are one head: pair (d, d + 32) is tiles (rt, rt + 2) of a lane
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int r2 = 0; r2 < 4; r2 += 2) {
+                        float2 cs[2][2];
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            uint32_t tok = min((uint32_t) tok0 + (uint32_t) (16 * tt + 4 * j + r2 + r), (uint32_t) a.N - 1u); // (a ragged tile's spare tokens: stores dropped below)
+                            const uint32_t off = tok * 256u + (uint32_t) c * 8u; // (uniform base + 32-bit lane offset; the launcher checks the range)
+                            cs[r][0] = *(const float2 *) ((const char *) a.rope_tab + off);
+                            cs[r][1] = *(const float2 *) ((const char *) a.rope_tab + off + 128u);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 2; ++r)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                float y0, y1;
+                                rope_rotate(acc[h][tt][r2 + r], acc[h + 2][tt][r2 + r], cs[r][h].x, cs[r][h].y, y0, y1);
+                                acc[h][tt][r2 + r] = y0; acc[h + 2][tt][r2 + r] = y1;
+                            }
+                        __builtin_amdgcn_sched_barrier(0); // (eight table values at a time: the accumulators leave few registers)
+                    }
+            }
             if ((int64_t) (ty + 1) * QT_TOKS <= a.N) { // (uniform) a whole token tile: a uniform base and one 32-bit lane offset, no tests
                 char *         tb = sb + (uint64_t) tok0 * nb1 + (uint64_t) r0 * 4;
                 const uint32_t lo = (uint32_t) ((uint64_t) (4 * j) * nb1 + (uint64_t) c * 4);
@@ -2355,7 +2395,12 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     bool fresh = false;
     char * kept = segs ? nullptr : (char *) vx_derived_get(key, wt_bytes + wd_bytes, st, &fresh); // (three matrices: tiles made per call)
     void * ws = nullptr;
-    if ((t_ws_status = vx_workspace(st, a.ws_offset + (kept ? 0 : wt_bytes + wd_bytes) + xt_bytes, &ws)) != VX_OK) {
+    // (segments with a rotation: the angle table behind the tiles)
+    const bool   rotate = segs && a.pos != nullptr;
+    // (token n of a batch entry sits at position index n % rope_T: sequences may be flattened into the token dimension)
+    const size_t tab_bytes = rotate ? (size_t) a.N * 32 * sizeof(float2) : 0;
+    if (rotate && (a.head_dim != 64 || a.rp.n_dims != 64 || a.rp.mode != 2 || a.rope_T <= 0 || a.N * 256 >= ((int64_t) 1 << 32))) return false;
+    if ((t_ws_status = vx_workspace(st, a.ws_offset + (kept ? 0 : wt_bytes + wd_bytes) + xt_bytes + tab_bytes, &ws)) != VX_OK) {
         (void) hipGetLastError();
         if (fresh) vx_derived_abandon(key, st);
         return false;
@@ -2372,6 +2417,12 @@ bool launch_gemm_q8t(const mm_args & a, int nbatch, hipStream_t st, bool fold) {
     else          vx_launch(qt_acts_kernel, dim3((unsigned) ((xunits + 255) / 256), (unsigned) nbatch), dim3(256), 0, st, q);
     if constexpr (!DUAL) {
         if (segs) {
+            if (rotate) {
+                q.rope_tab = (const float2 *) (base + (kept ? 0 : wt_bytes + wd_bytes) + xt_bytes);
+                q.rope_segs = 2;
+                vx_launch(qt_rope_table_kernel, dim3((unsigned) ((a.N * 32 + 63) / 64)), dim3(64), 0, st, a.pos, a.ff, a.rp, (int) a.N, a.rope_T,
+                          const_cast<float2 *>(q.rope_tab));
+            }
             if (fold) vx_launch(gemm_q8t_kernel<false, true, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
             else      vx_launch(gemm_q8t_kernel<false, false, true>, dim3((unsigned) blocks, (unsigned) nbatch), dim3(512), QT_LDS, st, q);
             return true;
@@ -2896,7 +2947,7 @@ static vx_status qkv_run(const vx_tensor * norm_w, float eps, const vx_tensor * 
 
 // The same group at prefill sizes: RMS_NORM and the norm weight in the activation pass of the pre-tiled kernel, q, k and v
 // as one virtual matrix over those tiles (one product launch instead of three, x laid out once), each stored to its own
-// destination; the two rotations follow as launches of their own, in place.  Taken when every piece is what the separate
+// destination; the two rotations in the product's epilogue (heads of 64 rows) or as launches of their own, in place.  Taken when every piece is what the separate
 // nodes would run -- each product on a tiled kernel with its K whole (the pre-tiled kernel and the LDS-operand kernel form
 // and add a block's products identically) -- so the bits are those of RMS_NORM, MUL, three MUL_MATs and two ROPEs.
 static bool qkv_tiled_fill(mm_args & a, const vx_tensor * norm_w, float eps, const vx_tensor * wq, const vx_tensor * wk, const vx_tensor * wv,
@@ -2980,8 +3031,18 @@ extern "C" vx_status vx_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor 
         if (!qkv_tiled_fill(a, norm_w, eps, wq, wk, wv, x, q_dst, k_dst, v_dst, n_dims, mode, act_mode))
             return vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: shape outside the pre-tiled kernel");
         (void) take_ws_status();
+        // heads of 64 rows: the rotations in the product's epilogue, from an angle table (VX_QKV_ROPE_EPILOGUE=0: as launches of their own)
+        static const bool rope_apart = [] { const char * e = getenv("VX_QKV_ROPE_EPILOGUE"); return e && atoi(e) == 0; }();
+        const bool in_epilogue = !rope_apart && n_dims == 64 && q_dst->ne[0] == 64 && k_dst->ne[0] == 64 && q_dst->ne[2] == k_dst->ne[2];
+        if (in_epilogue) {
+            a.pos = pos; a.ff = freq_factors;
+            a.rp = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+            a.head_dim = 64;
+            a.rope_T   = (int) q_dst->ne[2];
+        }
         if (!launch_gemm_q8t<false>(a, (int) x->ne[3], (hipStream_t) stream, gemm_lds_mode() == 2))
             return ws_failed() ? take_ws_status() : vx_fail(VX_ERR_UNSUPPORTED, "norm_qkv_proj_rope: the product could not be launched");
+        if (in_epilogue) return VX_OK;
         vx_status rc = vx_rope(q_dst, pos, freq_factors, q_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, stream);
         if (rc == VX_OK) rc = vx_rope(k_dst, pos, freq_factors, k_dst, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow, stream);
         return rc;
