@@ -324,8 +324,8 @@ VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_te
  * projections' own k / v, followed by vx_kv_store_sync on its result.  The cache write and the ordering scalar are
  * launched first and the scalar is added in the attention kernel's epilogue (as vx_flash_attn_ext_add1 adds one), so
  * the tokens x hidden result is stored once instead of stored, read and stored again.  For query counts the LDS-tiled
- * kernel takes (logit_softcap 0) and the prefill-sized cache writes vx_kv_store_sync takes (more than 65536 elements
- * each); the slots must not overlap anything the attention reads.  Result and cache contents equal the two separate calls'. */
+ * kernel takes (logit_softcap 0) and the two-launch cache writes vx_kv_store_sync takes (a prompt's or a prefill's); the
+ * slots must not overlap anything the attention reads.  Result and cache contents equal the two separate calls'. */
 VX_API vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                                          const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
                                          const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst,
@@ -416,10 +416,12 @@ VX_API int vx_supports_mul_mat_scale_add(const vx_tensor * src0, const vx_tensor
 /* The reference's KV append with its write-ordering scalar (attention_forward, src/minicpm.cpp:682-713), nine graph
  * nodes as one launch:  CPY(k, k_slot) CONT SUM , CPY(v, v_slot) CONT SUM , ADD , SCALE(scale, bias) , ADD1(x, .)
  *   k_slot <- k ; v_slot <- v ; dst = x + ((sum(k_slot) + sum(v_slot)) * scale + bias)
- * k, v, x F32; a cache write of at most 16384 elements (decode-sized) with x of at most 65536, or a prefill's write --
- * both of more than 16 Ki sum units (4 elements of a 16-byte aligned row, else one), i.e. sums that vx_sum spreads over
- * its 128 blocks -- as two launches (stores and block totals; totals, scalar and ADD1) in place of eleven; k_slot /
- * v_slot with dense rows, F32 or F16.  With F16 slots the node sequence is CPY(k, k_slot) CPY(k_slot -> F32) SUM ...: the values are
+ * k, v, x F32; a cache write of at most 16384 elements (decode-sized: one launch, two when x has more than 16384
+ * elements), a prompt's -- both sums within vx_sum's one block of 1024 threads (16 Ki sum units: 4 elements of a
+ * 16-byte aligned row, else one), every wave of that block a work-group of its own here -- or a prefill's -- both of
+ * more than 16 Ki units, i.e. sums that vx_sum spreads over its 128 blocks --, the latter two as two launches (stores
+ * and wave or block totals; totals, scalar and ADD1) in place of eight to eleven; k_slot / v_slot with dense rows, F32
+ * or F16.  With F16 slots the node sequence is CPY(k, k_slot) CPY(k_slot -> F32) SUM ...: the values are
  * rounded to nearest even on the way in and the sums see the rounded values.  The sums are formed in vx_sum's order,
  * so dst equals what the separate nodes give. */
 VX_API vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,

@@ -268,7 +268,8 @@ def test_supports_truth_table_node_groups(pkg):
     assert lib.vx_supports_kv_store_sync(f16(pkg, [Dh, Hkv, 1, 2]), slot16, k_src, slot, attn, attn) == 0       # F16 source
     big, mid = f32(pkg, [Dh, Hkv, 512, 2]), f32(pkg, [Dh, Hkv, 100, 2])
     assert lib.vx_supports_kv_store_sync(big, big, big, big, attn, attn) == 1                                     # a prefill's write: sums over 128 blocks
-    assert lib.vx_supports_kv_store_sync(mid, mid, mid, mid, attn, attn) == 0                                     # in between: one block's sum
+    assert lib.vx_supports_kv_store_sync(mid, mid, mid, mid, attn, attn) == 1                                     # a prompt's: one block's sum each
+    assert lib.vx_supports_kv_store_sync(mid, mid, big, big, attn, attn) == 0                                     # one of each
     assert lib.vx_supports_kv_store_sync(big, big, mid, mid, attn, attn) == 0
     # attention over cached + current keys
     q = f32(pkg, [Dh, 1, H, 2])
@@ -429,7 +430,7 @@ def test_hot_kernels_do_not_spill():
         assert len(names) == len(sizes), f
         scratch.update({n: int(s) for n, s in zip(names, sizes)})
     assert len(scratch) > 250
-    hot = [r"gemm_q8t_kernel", r"qt_weights_kernel", r"qt_acts_kernel", r"qt_acts_norm_kernel", r"qt_rope_table_kernel", r"rope_heads_kernel", r"kv_sync_add1_kernel", r"kv_sync_scalar_kernel", "kv_sync_scalar_kernel", r"fattn_dec64_kernel", r"gemm_lds_kernel", r"gemv_dma_kernel", r"gemv_kernel", r"mm_kernel", r"mm_splitk_reduce_kernel", r"fattn_merge_kernel",
+    hot = [r"gemm_q8t_kernel", r"qt_weights_kernel", r"qt_acts_kernel", r"qt_acts_norm_kernel", r"qt_rope_table_kernel", r"rope_heads_kernel", r"kv_sync_add1_kernel", r"kv_sync_scalar_kernel", r"kv_store_mid_kernel", "kv_sync_scalar_kernel", r"fattn_dec64_kernel", r"gemm_lds_kernel", r"gemv_dma_kernel", r"gemv_kernel", r"mm_kernel", r"mm_splitk_reduce_kernel", r"fattn_merge_kernel",
            r"fattn_cols16_kernelILi64ELb0", r"pf_kernel", r"small_graph_dense_kernel", r"small_graph_kernel", r"rms_norm_kernel",
            r"rope_kernel", r"concat_many_kernel"]
     known = [r"fattn_cols16_kernelILi(64|128)ELb1", r"fattn_cols16_kernelILi128ELb0ELb1ELb[01]ELi1", r"kv_store_sync_kernel",

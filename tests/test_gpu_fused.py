@@ -309,24 +309,29 @@ def test_kv_store_sync(pkg, gpu, B, T, Hkv, D, H, poison):
 
 def test_kv_store_sync_limits(pkg, gpu):
     import torch
-    say("fused cache write: sizes between one block's sum and the 128-block sum are refused")
+    say("fused cache write: one write whose sum is one block's beside one whose sum is spread over 128 blocks is refused")
     L, d = pkg.lib(), pkg.desc
     k = torch.zeros((2, 100, 2, 64), dtype=torch.float32, device="cuda")      # 25600 elements: 6400 units, one block's sum
-    c = torch.zeros((2, 2, 600, 64), dtype=torch.float32, device="cuda")
+    v = torch.zeros((2, 600, 2, 64), dtype=torch.float32, device="cuda")      # 153600 elements: 38400 units, 128 blocks
+    c = torch.zeros((2, 2, 700, 64), dtype=torch.float32, device="cuda")
     x = torch.zeros((2, 100, 16, 64), dtype=torch.float32, device="cuda")
-    s = c[:, :, :100].transpose(1, 2)
-    assert L.vx_supports_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x)) == 0
-    assert L.vx_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x), 0.0, 0.0, None) != 0
+    s, s2 = c[:, :, :100].transpose(1, 2), c[:, :, :600].transpose(1, 2)
+    assert L.vx_supports_kv_store_sync(d(k), d(s), d(k), d(s), d(x), d(x)) == 1
+    assert L.vx_supports_kv_store_sync(d(k), d(s), d(v), d(s2), d(x), d(x)) == 0
+    assert L.vx_kv_store_sync(d(k), d(s), d(v), d(s2), d(x), d(x), 0.0, 0.0, None) != 0
 
 
-@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 512, 2, 64, 16), (16, 300, 2, 64, 16), (1, 1100, 1, 64, 4), (3, 600, 2, 30, 2)])
+@pytest.mark.parametrize("B,T,Hkv,D,H", [(2, 512, 2, 64, 16), (16, 300, 2, 64, 16), (1, 1100, 1, 64, 4), (3, 600, 2, 30, 2),
+                                        # a prompt's write: each sum one block's, its waves spread over work-groups
+                                        (1, 129, 2, 64, 16), (1, 256, 2, 64, 16), (1, 512, 2, 64, 16), (2, 100, 2, 64, 16), (1, 300, 1, 64, 4)])
 @pytest.mark.parametrize("f16", [False, True])
 @pytest.mark.parametrize("poison", [None, "nan"])
 def test_kv_store_sync_prefill_sized(pkg, gpu, B, T, Hkv, D, H, f16, poison):
-    """The cache write of a prefill (src/minicpm.cpp:682-690 with hundreds of tokens): CPY into the slot, CONT (the cast
-    back from an F16 cache), SUM -- then the 128-block form of the sum kernel and the kernel that adds its partials --,
-    twice, ADD, SCALE, ADD1 over the attention output: eleven launches against the two of vx_kv_store_sync, bit for bit,
-    cache contents included.  Rows of 64 and of 30 values (with and without 16-byte units)."""
+    """The cache write of a prompt or a prefill (src/minicpm.cpp:682-690 with hundreds or thousands of tokens): CPY into
+    the slot, CONT (the cast back from an F16 cache), SUM -- one block of 1024 threads up to 16 Ki units, beyond that the
+    128-block form of the sum kernel and the kernel that adds its partials --, twice, ADD, SCALE, ADD1 over the attention
+    output: eight to eleven launches against the two of vx_kv_store_sync, bit for bit, cache contents included.  Rows of
+    64 and of 30 values (with and without 16-byte units)."""
     import torch
     say(f"prefill-sized cache write B={B} T={T} Hkv={Hkv} D={D} H={H} f16={f16} poison={poison}")
     if f16 and D % 4:
@@ -367,7 +372,7 @@ def test_kv_store_sync_prefill_sized(pkg, gpu, B, T, Hkv, D, H, f16, poison):
     assert torch.equal(a.nan_to_num(123.0), x2.nan_to_num(123.0))
 
 
-@pytest.mark.parametrize("B,T,Hkv,H", [(2, 512, 2, 16), (3, 600, 2, 16), (2, 1100, 1, 4), (16, 300, 2, 16)])
+@pytest.mark.parametrize("B,T,Hkv,H", [(2, 512, 2, 16), (3, 600, 2, 16), (2, 1100, 1, 4), (16, 300, 2, 16), (1, 512, 2, 16), (2, 256, 2, 16)])
 @pytest.mark.parametrize("f16", [False, True])
 @pytest.mark.parametrize("poison", [None, "nan"])
 def test_flash_attn_ext_store(pkg, gpu, B, T, Hkv, H, f16, poison):

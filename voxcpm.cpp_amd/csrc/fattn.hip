@@ -1145,7 +1145,7 @@ extern "C" vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tenso
         !k_slot->data || !v_src->data || !v_slot->data || !dst->data || (mask && !mask->data))
         return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: null tensor");
     if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, dst, logit_softcap))
-        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store: a query count the LDS-tiled kernel takes, and prefill-sized cache writes (more than 65536 elements each)");
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store: a query count the LDS-tiled kernel takes, and cache writes of a prompt's or a prefill's size");
     if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: max_bias > 0 requires a mask");
     pf_store_ctx c{ k_src, k_slot, v_src, v_slot, sync_scale, sync_bias };
     const vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_launch, &c };

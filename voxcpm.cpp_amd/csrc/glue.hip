@@ -1073,6 +1073,35 @@ __global__ __launch_bounds__(1024) void kv_store_large_kernel(const kvs_args a, 
     if (threadIdx.x == 0) partials[blockIdx.x] = t;
 }
 
+// A write between the two (a prompt of a few hundred tokens): each SUM is still GGML_OP_SUM's one block of 1024 threads
+// -- thread t walks units t, t + 1024, ..., a wave adds its lanes by butterfly, the 16 wave totals are added in order --
+// but one work-group storing and adding 2 x 64 Ki values is 17 us.  Here every wave of that block is a work-group of its
+// own (16 per cache) and leaves its total where the kernel behind adds the block totals in order: the same additions in
+// the same order, the zeros of the 112 further slots change nothing.
+template <bool VEC>
+__device__ __forceinline__ double kvs_mid_wave(const kvs_side & s, uint32_t w, uint32_t lane) {
+    const uint32_t n = kvs_units(s, VEC);
+    double acc = 0.0;
+    if (n <= VX_SUM_ONE_WAVE_UNITS) { // (uniform) a sum of one wave's size: its order, by the first wave
+        if (w) return 0.0;
+        for (uint32_t e = lane; e < n; e += 64) kvs_unit<VEC>(s, e, true, acc);
+        return vx_wave_sum(acc);
+    }
+    if (w * 64 >= n) return 0.0;
+    for (uint32_t e = w * 64 + lane; e < n; e += 1024) kvs_unit<VEC>(s, e, true, acc);
+    return vx_wave_sum(acc);
+}
+
+template <bool VK, bool VV>
+__global__ __launch_bounds__(64) void kv_store_mid_kernel(const kvs_args a, double * partials) {
+    const bool     second = blockIdx.x >= 16; // uniform
+    const uint32_t w = blockIdx.x - (second ? 16 : 0);
+    const double   t = second ? kvs_mid_wave<VV>(a.v, w, threadIdx.x) : kvs_mid_wave<VK>(a.k, w, threadIdx.x);
+    double * half = partials + (second ? SUM_BLOCKS : 0);
+    if (threadIdx.x == 0) half[w] = t;
+    if (w == 0) for (int i = 16 + (int) threadIdx.x; i < SUM_BLOCKS; i += 64) half[i] = 0.0;
+}
+
 // the block totals of the two sums, added in block order, as the scalar of the SCALE node (256 threads)
 __device__ __forceinline__ float kvs_scalar_of_totals(const kvs_args & a, const double * partials) {
     __shared__ double part[2 * SUM_BLOCKS];
@@ -1871,18 +1900,47 @@ static bool kvs_large(const vx_tensor * k, const vx_tensor * k_slot, const vx_te
     return vx_nelements(k) / (sk.vec ? 4 : 1) > 16 * 1024 && vx_nelements(v) / (sv.vec ? 4 : 1) > 16 * 1024;
 }
 
+// both sums are ones that GGML_OP_SUM's kernel forms in one block (at most 16 Ki units each), and at least one write is
+// beyond what the one-launch form takes
+static bool kvs_mid(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot) {
+    if (!kvs_side_ok(k, k_slot, (int64_t) 1 << 24) || !kvs_side_ok(v, v_slot, (int64_t) 1 << 24)) return false;
+    if (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) return false;
+    kvs_side sk, sv;
+    kvs_side_fill(sk, k, k_slot);
+    kvs_side_fill(sv, v, v_slot);
+    return vx_nelements(k) / (sk.vec ? 4 : 1) <= 16 * 1024 && vx_nelements(v) / (sv.vec ? 4 : 1) <= 16 * 1024;
+}
+
 extern "C" int vx_supports_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                          const vx_tensor * x, const vx_tensor * dst) {
     if (!k || !k_slot || !v || !v_slot || !x || !dst) return 0;
     if (!f32(x) || !f32(dst) || !vx_positive(x) || !vx_same_shape(x, dst) || !nb_multiple(x, 4) || !nb_multiple(dst, 4)) return 0;
     // (x of any size: beyond 16384 values the ADD1 is a launch of its own)
-    return (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) || kvs_large(k, k_slot, v, v_slot) ? vx_nelements(x) < ((int64_t) 1 << 31) : 0;
+    return (kvs_side_ok(k, k_slot) && kvs_side_ok(v, v_slot)) || kvs_mid(k, k_slot, v, v_slot) || kvs_large(k, k_slot, v, v_slot)
+               ? vx_nelements(x) < ((int64_t) 1 << 31) : 0;
+}
+
+// the launches of a mid-sized or prefill-sized write: stores and (wave or block) totals to partials
+static void kvs_launch_store(const kvs_args & a, bool mid, double * partials, hipStream_t st) {
+    if (mid) {
+        const dim3 grid(32), block(64);
+        if (a.k.vec && a.v.vec) vx_launch(kv_store_mid_kernel<true, true>, grid, block, 0, st, a, partials);
+        else if (a.k.vec)       vx_launch(kv_store_mid_kernel<true, false>, grid, block, 0, st, a, partials);
+        else if (a.v.vec)       vx_launch(kv_store_mid_kernel<false, true>, grid, block, 0, st, a, partials);
+        else                    vx_launch(kv_store_mid_kernel<false, false>, grid, block, 0, st, a, partials);
+        return;
+    }
+    const dim3 grid(2 * SUM_BLOCKS), block(1024);
+    if (a.k.vec && a.v.vec) vx_launch(kv_store_large_kernel<true, true>, grid, block, 0, st, a, partials);
+    else if (a.k.vec)       vx_launch(kv_store_large_kernel<true, false>, grid, block, 0, st, a, partials);
+    else if (a.v.vec)       vx_launch(kv_store_large_kernel<false, true>, grid, block, 0, st, a, partials);
+    else                    vx_launch(kv_store_large_kernel<false, false>, grid, block, 0, st, a, partials);
 }
 
 extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
                                       const vx_tensor * x, const vx_tensor * dst, float scale, float bias, vx_stream stream) {
     if (!vx_supports_kv_store_sync(k, k_slot, v, v_slot, x, dst))
-        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors; at most 16384 elements per cache write, or both writes of more than 65536 elements (a prefill's)");
+        return vx_fail(VX_ERR_UNSUPPORTED, "kv_store_sync: F32 tensors; both cache writes of at most 16 Ki units (of four elements where rows are 16-byte aligned), or both of more");
     if (!k->data || !k_slot->data || !v->data || !v_slot->data || !x->data || !dst->data) return vx_fail(VX_ERR_INVALID, "kv_store_sync: null data");
     kvs_args a;
     kvs_side_fill(a.k, k, k_slot);
@@ -1904,16 +1962,12 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
             const int64_t nx = vx_nelements(x);
             vx_launch(kv_sync_add1_kernel, dim3((unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096)), dim3(256), 0, (hipStream_t) stream, a, (const double *) a.defer);
         }
-    } else { // a prefill's write: stores and block totals, then totals, scalar and ADD1
+    } else { // a prompt's or a prefill's write: stores and wave or block totals, then totals, scalar and ADD1
         void * ws = nullptr;
         const vx_status rc = vx_workspace((hipStream_t) stream, 2 * SUM_BLOCKS * sizeof(double), &ws);
         if (rc != VX_OK) return rc;
-        const dim3 grid(2 * SUM_BLOCKS), block(1024);
         hipStream_t st = (hipStream_t) stream;
-        if (a.k.vec && a.v.vec) vx_launch(kv_store_large_kernel<true, true>, grid, block, 0, st, a, (double *) ws);
-        else if (a.k.vec)       vx_launch(kv_store_large_kernel<true, false>, grid, block, 0, st, a, (double *) ws);
-        else if (a.v.vec)       vx_launch(kv_store_large_kernel<false, true>, grid, block, 0, st, a, (double *) ws);
-        else                    vx_launch(kv_store_large_kernel<false, false>, grid, block, 0, st, a, (double *) ws);
+        kvs_launch_store(a, kvs_mid(k, k_slot, v, v_slot), (double *) ws, st);
         const int64_t nx = vx_nelements(x);
         const unsigned blocks = (unsigned) std::min<int64_t>((nx + 1023) / 1024, 4096);
         vx_launch(kv_sync_add1_kernel, dim3(blocks), dim3(256), 0, st, a, (const double *) ws);
@@ -1925,8 +1979,8 @@ extern "C" vx_status vx_kv_store_sync(const vx_tensor * k, const vx_tensor * k_s
 // The cache write and the ordering scalar of vx_kv_store_sync without its ADD1: the scalar goes to y_out for a kernel
 // launched behind this call on the same stream to add.  partials: 2 * SUM_BLOCKS doubles of device memory.
 bool vx_kv_store_scalar_ok(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot) {
-    // (a prefill's write only: attention shapes with a smaller one do not reach the kernel that adds the scalar)
-    return k && k_slot && v && v_slot && kvs_large(k, k_slot, v, v_slot);
+    // (a prompt's or a prefill's write: attention shapes with a smaller one do not reach the kernel that adds the scalar)
+    return k && k_slot && v && v_slot && (kvs_mid(k, k_slot, v, v_slot) || kvs_large(k, k_slot, v, v_slot));
 }
 
 vx_status vx_kv_store_scalar(const vx_tensor * k, const vx_tensor * k_slot, const vx_tensor * v, const vx_tensor * v_slot,
@@ -1940,11 +1994,7 @@ vx_status vx_kv_store_scalar(const vx_tensor * k, const vx_tensor * k_slot, cons
     a.scale = scale; a.bias = bias;
     a.dense4 = 0;
     a.defer = nullptr;
-    const dim3 grid(2 * SUM_BLOCKS), block(1024);
-    if (a.k.vec && a.v.vec) vx_launch(kv_store_large_kernel<true, true>, grid, block, 0, st, a, (double *) partials);
-    else if (a.k.vec)       vx_launch(kv_store_large_kernel<true, false>, grid, block, 0, st, a, (double *) partials);
-    else if (a.v.vec)       vx_launch(kv_store_large_kernel<false, true>, grid, block, 0, st, a, (double *) partials);
-    else                    vx_launch(kv_store_large_kernel<false, false>, grid, block, 0, st, a, (double *) partials);
+    kvs_launch_store(a, kvs_mid(k, k_slot, v, v_slot), (double *) partials, st);
     vx_launch(kv_sync_scalar_kernel, dim3(1), dim3(256), 0, st, a, (const double *) partials, y_out);
     VX_LAUNCH_CHECK();
     return VX_OK;
