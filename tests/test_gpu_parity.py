@@ -75,9 +75,9 @@ def test_rms_norm_strided_and_inplace(gpu):
 def test_rope(gpu, mode, case):
     say(f"rope mode={mode} case={case}")
     if case == "prefill batch partial":   # many tokens: the kernel that walks a token's heads; 6 heads (a ragged group of four), a tail that is copied
-        shape, pos = (3, 300, 6, 80), np.arange(300, dtype=np.int32) * 3 + 7
+        shape, pos = (4, 300, 6, 80), np.arange(300, dtype=np.int32) * 3 + 7
     elif case == "prefill yarn":
-        shape, pos = (1, 512, 5, 128), np.arange(512, dtype=np.int32) * 17
+        shape, pos = (1, 1100, 5, 128), np.arange(1100, dtype=np.int32) * 7
     elif case == "decode":
         shape, pos = (2, 1, 16, 64), np.array([4095], np.int32)
     elif case == "prefill":
