@@ -334,6 +334,26 @@ VX_API vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * 
 VX_API int vx_supports_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                                             const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
                                             const vx_tensor * v_slot, const vx_tensor * dst, float logit_softcap);
+/* The same block with the output projection and the residual update behind it (attention_forward's o_proj product,
+ * src/minicpm.cpp:714-715, and layer_forward's update, :762-768): vx_flash_attn_ext_store followed by
+ * vx_mul_mat_scale_add(w_o, attn, residual) -> dst.  The attention kernel's epilogue rounds its result to f16 straight
+ * into the activation tiles of the pre-tiled Q8_0 product, so the tokens x hidden attention output is neither stored in
+ * fp32 nor read back and laid out again.  attn describes that output as the projection reads it ([hidden, tokens] with
+ * the sequences one after the other, or [hidden, tokens, batch]; dense, the attention result's own memory order): its
+ * memory is NOT written -- for callers whose only reader of it is the projection.  Where vx_flash_attn_ext_store applies
+ * and the projection alone would run on the pre-tiled kernel (Q8_0, VX_ACT_FLOAT).  dst and the cache contents equal the
+ * separate calls'. */
+VX_API vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                              const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                              const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * attn,
+                                              const vx_tensor * w_o, const vx_tensor * residual, const vx_tensor * dst,
+                                              float scale, float max_bias, float logit_softcap, float sync_scale,
+                                              float sync_bias, float res_scale, int act_mode, vx_stream stream);
+VX_API int vx_supports_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                                 const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                                 const vx_tensor * v_slot, const vx_tensor * attn, const vx_tensor * w_o,
+                                                 const vx_tensor * residual, const vx_tensor * dst, float logit_softcap,
+                                                 int act_mode);
 /* MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x): the three projections of
  * attention_forward with apply_rope on Q and K (src/minicpm.cpp:669-680, 582-600) as one launch for few tokens
  * (as above).  x [K, tokens, 1, batch] or [K, tokens * batch] (sequence after sequence); q_dst / k_dst are the ROPE

@@ -420,6 +420,55 @@ def test_flash_attn_ext_store(pkg, gpu, B, T, Hkv, H, f16, poison):
     assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
 
 
+@pytest.mark.parametrize("B,T,flat", [(16, 2048, True), (8, 4100, True), (16, 2048, False), (5, 7000, True)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_flash_attn_ext_store_proj(pkg, gpu, B, T, flat, f16):
+    """Prefill attention, cache write, o projection and residual update as one call: the attention's epilogue writes the
+    projection's f16 activation tiles (the attention output is never stored).  Against vx_flash_attn_ext_store followed by
+    vx_mul_mat_scale_add, bit for bit, cache contents included; the sequences flattened into one token dimension (ragged
+    token tiles too) and as a batch."""
+    import torch
+    say(f"prefill attention + cache write + o projection as one call B={B} T={T} flat={flat} f16 cache={f16}")
+    L, d = pkg.lib(), pkg.desc
+    H, Hkv, D, hidden = 16, 2, 64, 1024
+    g = rng("f-attn-store-proj", B, T)
+    q = torch.randn((B, T, H, D), device="cuda", generator=torch.Generator(device="cuda").manual_seed(B * T))
+    k = torch.randn((B, T, Hkv, D), device="cuda", generator=torch.Generator(device="cuda").manual_seed(B * T + 1))
+    v = torch.randn((B, T, Hkv, D), device="cuda", generator=torch.Generator(device="cuda").manual_seed(B * T + 2))
+    res = torch.randn((B, T, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(B * T + 3))
+    w = q8_dev((0.05 * g.standard_normal((hidden, hidden))).astype(np.float32))[0]
+    wd = pkg.desc_q8(w, hidden)
+    mask = torch.full((T, T), float("-inf"), dtype=torch.float16, device="cuda").triu(1).contiguous()
+    qd, kd, vd = d(q.transpose(1, 2)), d(k.transpose(1, 2)), d(v.transpose(1, 2))
+    cdt = torch.float16 if f16 else torch.float32
+    kc1, vc1, kc2, vc2 = (torch.zeros((B, Hkv, T + 3, D), dtype=cdt, device="cuda") for _ in range(4))
+    slot = lambda c: c[:, :, 2:2 + T].transpose(1, 2)
+    shape = (lambda t, rows: t.view(B * T, rows)) if flat else (lambda t, rows: t.view(B, T, rows))
+    scale = 1.0 / 8.0
+    a = torch.empty((B, T, H, D), dtype=torch.float32, device="cuda")
+    o1 = torch.empty((B, T, hidden), dtype=torch.float32, device="cuda")
+    ok(pkg, L.vx_flash_attn_ext_store(qd, kd, vd, d(mask), None, d(k), d(slot(kc1)), d(v), d(slot(vc1)), d(a), scale, 0.0, 0.0, 0.25, 0.5, None),
+       "flash_attn_ext_store")
+    ok(pkg, L.vx_mul_mat_scale_add(wd, d(shape(a, hidden)), d(shape(res, hidden)), d(shape(o1, hidden)), 0.7, pkg.ACT_FLOAT, None), "mul_mat_scale_add")
+    b = torch.full_like(a, 7.0)
+    o2 = torch.full_like(o1, float("nan"))
+    args = (qd, kd, vd, d(mask))
+    tail = (d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(shape(b, hidden)), wd, d(shape(res, hidden)), d(shape(o2, hidden)))
+    assert L.vx_supports_flash_attn_ext_store_proj(*args, *tail, 0.0, pkg.ACT_FLOAT) == 1
+    assert L.vx_supports_flash_attn_ext_store_proj(*args, *tail, 0.0, pkg.ACT_Q8) == 0
+    ok(pkg, L.vx_flash_attn_ext_store_proj(*args, None, *tail, scale, 0.0, 0.0, 0.25, 0.5, 0.7, pkg.ACT_FLOAT, None), "flash_attn_ext_store_proj")
+    torch.cuda.synchronize()
+    assert torch.equal(kc1.view(torch.uint8), kc2.view(torch.uint8)) and torch.equal(vc1.view(torch.uint8), vc2.view(torch.uint8))
+    assert bool(torch.isfinite(o2).all()) and torch.equal(o1, o2)
+    assert bool((b == 7.0).all()), "the attention output is not stored"
+    # in place on the residual, as layer_forward's update is laid out
+    r2 = res.clone()
+    ok(pkg, L.vx_flash_attn_ext_store_proj(*args, None, *tail[:6], d(shape(r2, hidden)), d(shape(r2, hidden)), scale, 0.0, 0.0, 0.25, 0.5, 0.7,
+                                           pkg.ACT_FLOAT, None), "in place")
+    torch.cuda.synchronize()
+    assert torch.equal(o1, r2)
+
+
 def test_flash_attn_ext_store_limits(pkg, gpu):
     import torch
     say("prefill attention + cache write: decode-sized and softcapped calls are refused")

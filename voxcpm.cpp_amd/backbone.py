@@ -204,6 +204,7 @@ class MiniCPMBackbone:
             # then the cache append with its ordering chain, then add1 (only adjacent nodes are run as one launch)
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)
             stored = False
+            projected = False
             if n_past > 0:
                 kp, vp = kc[:, :, :n_past], vc[:, :, :n_past]
                 qd = desc(q4.transpose(1, 2))
@@ -242,7 +243,19 @@ class MiniCPMBackbone:
                 qd = desc(q4.transpose(1, 2))
                 kw = kc[:, :, n_past:n_past + T].transpose(1, 2)
                 vw = vc[:, :, n_past:n_past + T].transpose(1, 2)
-                if write_kv and chain and fuse and L.vx_supports_flash_attn_ext_store(qd, desc(k_all), desc(v_all), desc(mask), desc(k4), desc(kw),
+                sc_o = self.residual_scale if self.use_mup else 1.0
+                attn2 = attn.view(N, H * D)
+                if write_kv and chain and fuse and L.vx_supports_flash_attn_ext_store_proj(
+                        qd, desc(k_all), desc(v_all), desc(mask), desc(k4), desc(kw), desc(v4), desc(vw), desc(attn2), wd["o_proj"], desc(cur_x),
+                        desc(h_mid), 0.0, self.act_mode):
+                    # a large prefill: as below, and the attention's result goes to the o projection as that product's f16
+                    # tiles (it is never stored); the projection applies the residual update
+                    keep += [kw, vw, attn2]
+                    call(L.vx_flash_attn_ext_store_proj, qd, desc(k_all), desc(v_all), desc(mask), None, desc(k4), desc(kw), desc(v4), desc(vw),
+                         desc(attn2), wd["o_proj"], desc(cur_x), desc(h_mid), scale, 0.0, 0.0, 0.0, 0.0, sc_o, self.act_mode)
+                    stored = True
+                    projected = True
+                elif write_kv and chain and fuse and L.vx_supports_flash_attn_ext_store(qd, desc(k_all), desc(v_all), desc(mask), desc(k4), desc(kw),
                                                                                       desc(v4), desc(vw), desc(attn), 0.0):
                     # a prefill: the cache write and its scalar first, the scalar added in the attention's epilogue
                     keep += [kw, vw]
@@ -278,7 +291,8 @@ class MiniCPMBackbone:
                 call(L.vx_scale, desc(sync), desc(sync), 0.0, 0.0)
             if chain and not grouped:
                 call(L.vx_add1, desc(attn), desc(sync), desc(attn))
-            project_residual(wd["o_proj"], attn.view(N, H * D), attn_o, cur_x, h_mid)
+            if not projected:
+                project_residual(wd["o_proj"], attn.view(N, H * D), attn_o, cur_x, h_mid)
             # -- mlp_forward
             nw_post = nrm["post_layernorm"]
             nxt = hs[li % 2]

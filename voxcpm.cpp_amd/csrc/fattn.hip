@@ -1152,6 +1152,81 @@ extern "C" vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tenso
     return vx_fattn_prefill(q, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream, &front);
 }
 
+// The same block with the o projection and its residual update behind it (src/minicpm.cpp:708-715, 762-768): the
+// attention's epilogue rounds its result to f16 straight into the projection's activation tiles, so the tokens x hidden
+// attention output is neither stored in fp32 nor read back and laid out again.
+struct pf_store_proj_ctx {
+    pf_store_ctx store;
+    void *       front;
+};
+
+static vx_status pf_store_proj_launch(void * front, void * ctx, hipStream_t st) {
+    pf_store_proj_ctx * c = (pf_store_proj_ctx *) ctx;
+    c->front = front;
+    return pf_store_launch(front, &c->store, st);
+}
+
+// attn: the attention's result as the projection reads it, [hidden, tokens (, batch)], dense; the same memory order as the
+// attention's own [head_dim, heads, tokens, batch]
+static bool pf_proj_geometry(const vx_tensor * q, const vx_tensor * attn, const vx_tensor * w_o, const vx_tensor * residual, const vx_tensor * dst,
+                             int act_mode, vx_pf_front * front) {
+    if (!attn || !w_o || !residual || !dst || attn->type != VX_TYPE_F32 || !vx_is_contiguous(attn)) return false;
+    const int64_t hidden = q->ne[0] * q->ne[2], T = q->ne[1], B = q->ne[3];
+    if (attn->ne[0] != hidden || vx_nelements(attn) != hidden * T * B) return false;
+    const bool flat = attn->ne[1] == T * B && attn->ne[2] == 1 && attn->ne[3] == 1;
+    const bool by_batch = attn->ne[1] == T && attn->ne[2] * attn->ne[3] == B;
+    if (!flat && !by_batch) return false;
+    uint32_t tile_tt = 0, n_kb = 0;
+    size_t   tile_bytes = 0;
+    if (!vx_proj_tiles_ok(w_o, attn, residual, dst, act_mode, &tile_tt, &n_kb, &tile_bytes)) return false;
+    front->tiles = true; front->tiles_at = PF_STORE_FRONT;
+    front->tile_tt = tile_tt;
+    front->tile_bs = by_batch && !flat ? n_kb * tile_tt : 0;
+    front->tile_ts = by_batch && !flat ? 0 : (uint32_t) T;
+    front->bytes = PF_STORE_FRONT + tile_bytes;
+    return (int64_t) B * T < ((int64_t) 1 << 31);
+}
+
+extern "C" int vx_supports_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                                     const vx_tensor * k_src, const vx_tensor * k_slot, const vx_tensor * v_src,
+                                                     const vx_tensor * v_slot, const vx_tensor * attn, const vx_tensor * w_o,
+                                                     const vx_tensor * residual, const vx_tensor * dst, float logit_softcap, int act_mode) {
+    if (!attn || !q) return 0;
+    // (the attention's own destination: the tensor attn describes, in the attention's shape)
+    vx_tensor ad = *attn;
+    ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
+    ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+    if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, &ad, logit_softcap)) return 0;
+    vx_pf_front front{};
+    return pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front) ? 1 : 0;
+}
+
+extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
+                                                  const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
+                                                  const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * attn,
+                                                  const vx_tensor * w_o, const vx_tensor * residual, const vx_tensor * dst, float scale,
+                                                  float max_bias, float logit_softcap, float sync_scale, float sync_bias, float res_scale,
+                                                  int act_mode, vx_stream stream) {
+    if (!q || !k || !v || !k_src || !k_slot || !v_src || !v_slot || !attn || !w_o || !residual || !dst || !q->data || !k->data || !v->data ||
+        !k_src->data || !k_slot->data || !v_src->data || !v_slot->data || !attn->data || !w_o->data || !residual->data || !dst->data ||
+        (mask && !mask->data))
+        return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store_proj: null tensor");
+    if (!vx_supports_flash_attn_ext_store_proj(q, k, v, mask, k_src, k_slot, v_src, v_slot, attn, w_o, residual, dst, logit_softcap, act_mode))
+        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: the shapes of flash_attn_ext_store, and a Q8_0 projection with an F32 residual that the pre-tiled kernel takes");
+    if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store_proj: max_bias > 0 requires a mask");
+    pf_store_proj_ctx c{ { k_src, k_slot, v_src, v_slot, sync_scale, sync_bias }, nullptr };
+    vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_proj_launch, &c };
+    if (!pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front)) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: tile geometry");
+    vx_tensor ad = *attn; // (never written: the result leaves as tiles)
+    ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
+    ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+    hipStream_t st = (hipStream_t) stream;
+    vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, nullptr, &ad, scale, max_bias, logit_softcap, st, &front);
+    if (rc != VX_OK) return rc == VX_ERR_UNSUPPORTED ? vx_fail(rc, "flash_attn_ext_store_proj: the LDS-tiled kernel declined") : rc;
+    // the projection: its own needs go behind the front (a block that a larger request replaces stays valid)
+    return vx_proj_tiles_run(w_o, attn, residual, dst, res_scale, act_mode, (const char *) c.front + PF_STORE_FRONT, front.bytes, st);
+}
+
 // ---- the entry point that allocates nothing ------------------------------------------------------------
 // The key-range partials of vx_flash_attn_ext_static live in a fixed array in device memory that is part of the
 // loaded code object: every GPU the library runs on holds its own copy, at its own address, until the process

@@ -29,6 +29,8 @@ struct pf_args {
     const char * q; const char * k; const char * v; const char * vl; const char * mask;
     const float * sinks;
     const float * add1; // optional scalar added to every output element (a fused GGML_OP_ADD1)
+    _Float16 * tile_out; // optional: the result as f16 activation tiles of the product that follows, instead of dst
+    uint32_t tile_tt, tile_bs, tile_ts;
     float * dst;
     const uint8_t * flags; // [nem3][nem2][n_rb][n_tiles]: 0 skip, 1 no mask, 2 apply mask values, 3 apply visibility bits
     const uint8_t * bits;  // [nem3][nem2][n_q][n_tiles] 8 bytes each: one bit per key of the tile (flag 3)
@@ -617,7 +619,20 @@ __global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2
             L = L * ms + vs;
         }
         const float inv = L == 0.0f ? 0.0f : ms / L;
-        if (ok) {
+        if (ok && a.tile_out) { // (uniform choice) rounded to f16 as the product's activation pass would round the stored value
+            // k = hd * 64 + d: tile (k block 2 hd + dt, 16 tokens), slot (q4, token mod 16), halves 4 hl .. 4 hl + 3
+            const uint32_t tokf = (uint32_t) b * a.tile_ts + (uint32_t) row;
+            _Float16 * tb = a.tile_out + ((((uint64_t) b * a.tile_bs + (uint64_t) (2 * hd) * a.tile_tt + (tokf >> 4)) * 64 + (tokf & 15)) * 8 + 4 * hl_e);
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    float4_t r = float4_t{o[cb][dt][4 * q4], o[cb][dt][4 * q4 + 1], o[cb][dt][4 * q4 + 2], o[cb][dt][4 * q4 + 3]} * inv;
+                    if (a.add1) r += *a.add1;
+                    asm volatile("" : "+v"(r)); // the fp32 value the node holds, formed as such, then rounded
+                    *(half4_t *) (tb + ((uint64_t) dt * a.tile_tt * 64 + 16 * q4) * 8) = half4_t{(_Float16) r[0], (_Float16) r[1], (_Float16) r[2], (_Float16) r[3]};
+                }
+        } else if (ok) {
             float * out = a.dst + (((uint64_t) b * a.n_q + row) * a.Hq + hd) * D;
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
@@ -678,6 +693,7 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
     a.mask = mask ? (const char *) mask->data : nullptr;
     a.sinks = sinks;
     a.add1 = addend;
+    a.tile_out = nullptr; a.tile_tt = a.tile_bs = a.tile_ts = 0;
     a.dst = (float *) dst->data;
     a.flags = nullptr;
     a.bits = nullptr;
@@ -716,6 +732,10 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
         const vx_status rc = front->launch(ws, front->ctx, st);
         if (rc != VX_OK) return rc;
         a.add1 = (const float *) (ws + front->addend_at);
+        if (front->tiles) {
+            a.tile_out = (_Float16 *) (ws + front->tiles_at);
+            a.tile_tt = front->tile_tt; a.tile_bs = front->tile_bs; a.tile_ts = front->tile_ts;
+        }
         ws += front_bytes;
     }
     if (mask) {

@@ -2889,6 +2889,60 @@ extern "C" vx_status vx_mlp_tiled(const vx_tensor * x, const vx_tensor * norm_w,
     return VX_OK;
 }
 
+// A projection with its residual update whose activations a kernel in front of it (the prefill attention's epilogue) has
+// left as this kernel's f16 tiles: vx_mul_mat_scale_add without its activation pass.  Taken where the separate call runs
+// on the pre-tiled kernel, so the bits are the same.
+static bool proj_tiles_fill(mm_args & b, const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, float scale, int act_mode) {
+    if (!w || !x || !residual || !dst || act_mode != VX_ACT_FLOAT || gemm_lds_mode() == 0) return false;
+    if (w->type != VX_TYPE_Q8_0 || w->ne[2] != 1 || w->ne[3] != 1 || x->type != VX_TYPE_F32 || !vx_is_contiguous(x)) return false;
+    if (!vx_supports_mul_mat_scale_add(w, x, residual, dst) || !vx_same_shape(residual, dst) || residual->nb[0] != 4 || dst->nb[0] != 4) return false;
+    b = mm_args{};
+    b.w = (const char *) w->data; b.x = (const char *) x->data; b.dst = (char *) dst->data;
+    b.K = w->ne[0]; b.M = w->ne[1]; b.N = x->ne[1];
+    b.nb01 = w->nb[1]; b.nb02 = w->nb[2]; b.nb03 = w->nb[3];
+    b.nb11 = x->nb[1]; b.nb12 = x->nb[2]; b.nb13 = x->nb[3];
+    b.nb1 = dst->nb[1]; b.nb2 = dst->nb[2]; b.nb3 = dst->nb[3];
+    b.ne12 = (int) x->ne[2];
+    b.r2 = (int) x->ne[2]; b.r3 = (int) x->ne[3];
+    b.rows_wg = 16;
+    b.res = (const char *) residual->data;
+    b.rnb1 = residual->nb[1]; b.rnb2 = residual->nb[2]; b.rnb3 = residual->nb[3];
+    b.res_scale = scale;
+    b.w_aligned = ((uintptr_t) w->data % 4 == 0) && w->nb[1] % 4 == 0;
+    b.x_aligned = ((uintptr_t) x->data % 16 == 0) && x->nb[1] % 16 == 0 && x->nb[2] % 16 == 0 && x->nb[3] % 16 == 0;
+    const int64_t nbatch = x->ne[2] * x->ne[3];
+    // (what launch_gemm_lds asks for before it hands a product to the pre-tiled kernel)
+    if ((uint64_t) b.M * b.nb01 >= (1ull << 32) || (uint64_t) 256 * b.nb11 + 256 >= (1ull << 32) || (uint64_t) 256 * b.nb1 + 1024 >= (1ull << 32) ||
+        b.K >= (1ll << 28) || b.N <= 16) return false;
+    return b.w_aligned && b.x_aligned && nbatch <= 65535 && (uintptr_t) dst->data % 4 == 0 && (uintptr_t) residual->data % 4 == 0 &&
+           !gemv_shape_ok(b.N, b.M, b.K) && b.K % (32 * GL_KC) == 0 && gemm_q8t_takes(b, (int) nbatch, false) &&
+           (uint64_t) 256 * b.rnb1 + 1024 < (1ull << 32);
+}
+
+bool vx_proj_tiles_ok(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, int act_mode,
+                      uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes) {
+    mm_args b;
+    if (!proj_tiles_fill(b, w, x, residual, dst, 0.0f, act_mode)) return false;
+    const int64_t tt = (b.N + QT_TOKS - 1) / QT_TOKS * (QT_TOKS / 16), nbatch = x->ne[2] * x->ne[3];
+    if (tt * (b.K / 32) * nbatch >= ((int64_t) 1 << 31)) return false;
+    *tile_tt = (uint32_t) tt; *n_kb = (uint32_t) (b.K / 32);
+    *tile_bytes = ((size_t) nbatch * (size_t) (b.K / 32) * (size_t) tt * 1024 + 255) & ~(size_t) 255;
+    return true;
+}
+
+vx_status vx_proj_tiles_run(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, float scale,
+                            int act_mode, const void * tiles, size_t ws_offset, hipStream_t st) {
+    mm_args b;
+    if (!proj_tiles_fill(b, w, x, residual, dst, scale, act_mode)) return vx_fail(VX_ERR_UNSUPPORTED, "projection over tiles: a shape outside the pre-tiled kernel");
+    if (!w->data || !residual->data || !dst->data || !tiles) return vx_fail(VX_ERR_INVALID, "projection over tiles: null data");
+    b.ws_offset = ws_offset; b.tile_in = tiles; b.tile_tt = (int) ((b.N + QT_TOKS - 1) / QT_TOKS * (QT_TOKS / 16));
+    (void) take_ws_status();
+    if (!launch_gemm_q8t<false>(b, (int) (x->ne[2] * x->ne[3]), st, gemm_lds_mode() == 2))
+        return ws_failed() ? take_ws_status() : vx_fail(VX_ERR_UNSUPPORTED, "projection over tiles: the product could not be launched");
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
 // The Q, K and V projections of one attention block with the NEOX rotation of Q and K, one launch:
 //   MUL_MAT(wq, x) RESHAPE ROPE , MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x)
 // (MiniCPMModel::attention_forward, src/minicpm.cpp:640-680).  q_dst and k_dst are the ROPE nodes'

@@ -94,12 +94,27 @@ struct vx_pf_front {
     size_t bytes, addend_at;
     vx_status (*launch)(void * front, void * ctx, hipStream_t stream);
     void * ctx;
+    // optionally the result leaves as the pre-tiled product kernel's f16 activation tiles (k = head * 64 + d) at
+    // tiles_at bytes into the front instead of being stored to dst: tile_tt 16-token tiles per k block; tile_bs tiles
+    // per batch entry (0: the sequences are flattened into one token dimension, tile_ts tokens apart)
+    bool     tiles;
+    size_t   tiles_at;
+    uint32_t tile_tt, tile_bs, tile_ts;
 };
 
 // LDS-tiled prefill kernel (fattn_prefill.hip); VX_ERR_UNSUPPORTED means "use the general kernel"
 vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                            const float * sinks, const float * addend, const vx_tensor * dst, float scale, float max_bias,
                            float logit_softcap, hipStream_t stream, const vx_pf_front * front = nullptr);
+
+// A Q8_0 projection with its residual update (vx_mul_mat_scale_add) over activations that a kernel in front of it left
+// as the pre-tiled kernel's f16 tiles in the stream's workspace (mul_mat.hip).  x describes the F32 activations the
+// separate call would read (only shape and strides are looked at).  _ok: the separate call would run on the pre-tiled
+// kernel; it reports the tile geometry.  _run: tiles at `tiles`, the first ws_offset bytes of the workspace are the caller's.
+bool      vx_proj_tiles_ok(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, int act_mode,
+                           uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes);
+vx_status vx_proj_tiles_run(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, float scale,
+                            int act_mode, const void * tiles, size_t ws_offset, hipStream_t stream);
 
 // vx_kv_store_sync's cache write and ordering scalar without the ADD1 (glue.hip): the scalar is left in *y_out
 // (device memory), partials are 2 KiB of device memory

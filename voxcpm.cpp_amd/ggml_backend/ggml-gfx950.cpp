@@ -1078,6 +1078,52 @@ int compute_attention_store(backend_ctx * ctx, const ggml_cgraph * g, int i, con
     vx_tensor m;
     if (f->src[3]) m = to_vx(f->src[3]);
     if (!vx_supports_flash_attn_ext_store(&q, &k, &v, f->src[3] ? &m : nullptr, &ksrc, &ks, &vsrc, &vs, &d, softcap)) return -1;
+    {   // the o projection and its residual update behind the ADD1 (attention_forward's last two lines, layer_forward's update):
+        //   RESHAPE(attn) MUL_MAT(o_proj, .) [SCALE] ADD(residual, .)
+        // with the reshape the ADD1's only reader and the product its only one, the attention's result goes to the product
+        // as its f16 activation tiles and is never stored
+        int im = last + 1;
+        const ggml_tensor * view = nullptr;
+        while (im < g->n_nodes && (ggml_op_is_empty(g->nodes[im]->op) || ggml_is_empty(g->nodes[im]))) {
+            if (g->nodes[im]->view_src == dst && g->nodes[im]->src[0] == dst && !view) view = g->nodes[im];
+            ++im;
+        }
+        const auto rd = readers.find(dst);
+        const ggml_tensor * mm = im < g->n_nodes ? g->nodes[im] : nullptr;
+        if (view && mm && mm->op == GGML_OP_MUL_MAT && mm->src[1] == view && (dst->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 &&
+            (view->flags & GGML_TENSOR_FLAG_OUTPUT) == 0 && rd != readers.end() && rd->second == 2 && private_to_group(readers, view) &&
+            view->view_offs == 0 && ggml_is_contiguous(view) && private_to_group(readers, mm) && im + 1 < g->n_nodes) {
+            const ggml_tensor * val = mm;
+            float rs = 1.0f;
+            int ia = im + 1;
+            bool ok = true;
+            if (g->nodes[ia]->op == GGML_OP_SCALE) {
+                const ggml_tensor * scn = g->nodes[ia];
+                float sb;
+                memcpy(&rs, (const float *) scn->op_params + 0, sizeof(float));
+                memcpy(&sb, (const float *) scn->op_params + 1, sizeof(float));
+                ok = scn->src[0] == mm && sb == 0.0f && private_to_group(readers, scn) && ia + 1 < g->n_nodes;
+                val = scn;
+                ++ia;
+            }
+            const ggml_tensor * add = ok ? g->nodes[ia] : nullptr;
+            if (add && add->op == GGML_OP_ADD && (add->flags & GGML_TENSOR_FLAG_COMPUTE) != 0 && (add->src[0] == val) != (add->src[1] == val)) {
+                const ggml_tensor * residual = add->src[0] == val ? add->src[1] : add->src[0];
+                // (the update is the call's last kernel: what the cache write and the attention read is done with by then, and the
+                // update may well have been given the memory of q; the weights and the residual are what its kernel reads)
+                ok = residual != mm && residual != dst && residual != view && apart(add, mm->src[0]) && apart_or_same(add, residual) &&
+                     apart(n[0], residual) && apart(n[3], residual);
+                const vx_tensor av = to_vx(view), wo = to_vx(mm->src[0]), r = to_vx(residual), od = to_vx(add);
+                if (ok && vx_supports_flash_attn_ext_store_proj(&q, &k, &v, f->src[3] ? &m : nullptr, &ksrc, &ks, &vsrc, &vs, &av, &wo, &r, &od, softcap,
+                                                                mul_mat_act_mode())) {
+                    *rc = vx_flash_attn_ext_store_proj(&q, &k, &v, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
+                                                       &ksrc, &ks, &vsrc, &vs, &av, &wo, &r, &od, scale, max_bias, softcap, sc, bias, rs,
+                                                       mul_mat_act_mode(), ctx->stream);
+                    return ia;
+                }
+            }
+        }
+    }
     *rc = vx_flash_attn_ext_store(&q, &k, &v, f->src[3] ? &m : nullptr, f->src[4] ? (const float *) f->src[4]->data : nullptr,
                                   &ksrc, &ks, &vsrc, &vs, &d, scale, max_bias, softcap, sc, bias, ctx->stream);
     return last;
