@@ -325,7 +325,8 @@ VX_API int vx_supports_flash_attn_ext_kv2_store(const vx_tensor * q, const vx_te
  * launched first and the scalar is added in the attention kernel's epilogue (as vx_flash_attn_ext_add1 adds one), so
  * the tokens x hidden result is stored once instead of stored, read and stored again.  For query counts the LDS-tiled
  * kernel takes (logit_softcap 0) and the two-launch cache writes vx_kv_store_sync takes (a prompt's or a prefill's); the
- * slots must not overlap anything the attention reads.  Result and cache contents equal the two separate calls'. */
+ * slots must not overlap anything the attention reads.  Result and cache contents equal the two separate calls'.
+ * (vx_supports_flash_attn_ext_store says whether the call takes this form; shapes outside it run as the two calls.) */
 VX_API vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                                          const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
                                          const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * dst,
@@ -341,8 +342,8 @@ VX_API int vx_supports_flash_attn_ext_store(const vx_tensor * q, const vx_tensor
  * fp32 nor read back and laid out again.  attn describes that output as the projection reads it ([hidden, tokens] with
  * the sequences one after the other, or [hidden, tokens, batch]; dense, the attention result's own memory order): its
  * memory is NOT written -- for callers whose only reader of it is the projection.  Where vx_flash_attn_ext_store applies
- * and the projection alone would run on the pre-tiled kernel (Q8_0, VX_ACT_FLOAT).  dst and the cache contents equal the
- * separate calls'. */
+ * and the projection alone would run on the pre-tiled kernel (Q8_0, VX_ACT_FLOAT) -- what the supports function reports;
+ * other shapes run as the separate calls, through attn's memory.  dst and the cache contents equal the separate calls'. */
 VX_API vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
                                               const float * sinks, const vx_tensor * k_src, const vx_tensor * k_slot,
                                               const vx_tensor * v_src, const vx_tensor * v_slot, const vx_tensor * attn,

@@ -1144,9 +1144,14 @@ extern "C" vx_status vx_flash_attn_ext_store(const vx_tensor * q, const vx_tenso
     if (!q || !k || !v || !k_src || !k_slot || !v_src || !v_slot || !dst || !q->data || !k->data || !v->data || !k_src->data ||
         !k_slot->data || !v_src->data || !v_slot->data || !dst->data || (mask && !mask->data))
         return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: null tensor");
-    if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, dst, logit_softcap))
-        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store: a query count the LDS-tiled kernel takes, and cache writes of a prompt's or a prefill's size");
     if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store: max_bias > 0 requires a mask");
+    if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, dst, logit_softcap)) {
+        // not this form's shapes (or the LDS-tiled kernel switched off since the caller asked): the two calls it stands for
+        if (!vx_supports_flash_attn_ext(q, k, v, mask, dst) || !vx_supports_kv_store_sync(k_src, k_slot, v_src, v_slot, dst, dst))
+            return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store: shapes that neither the one call nor flash_attn_ext followed by kv_store_sync takes");
+        const vx_status rc = vx_flash_attn_ext(q, k, v, mask, sinks, dst, scale, max_bias, logit_softcap, stream);
+        return rc != VX_OK ? rc : vx_kv_store_sync(k_src, k_slot, v_src, v_slot, dst, dst, sync_scale, sync_bias, stream);
+    }
     pf_store_ctx c{ k_src, k_slot, v_src, v_slot, sync_scale, sync_bias };
     const vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_launch, &c };
     return vx_fattn_prefill(q, k, v, mask, sinks, nullptr, dst, scale, max_bias, logit_softcap, (hipStream_t) stream, &front);
@@ -1211,9 +1216,18 @@ extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_
         !k_src->data || !k_slot->data || !v_src->data || !v_slot->data || !attn->data || !w_o->data || !residual->data || !dst->data ||
         (mask && !mask->data))
         return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store_proj: null tensor");
-    if (!vx_supports_flash_attn_ext_store_proj(q, k, v, mask, k_src, k_slot, v_src, v_slot, attn, w_o, residual, dst, logit_softcap, act_mode))
-        return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: the shapes of flash_attn_ext_store, and a Q8_0 projection with an F32 residual that the pre-tiled kernel takes");
     if (max_bias > 0.0f && !mask) return vx_fail(VX_ERR_INVALID, "flash_attn_ext_store_proj: max_bias > 0 requires a mask");
+    if (!vx_supports_flash_attn_ext_store_proj(q, k, v, mask, k_src, k_slot, v_src, v_slot, attn, w_o, residual, dst, logit_softcap, act_mode)) {
+        // not this form's shapes (or a kernel it needs switched off since the caller asked): the calls it stands for, through attn's memory
+        if (attn->type != VX_TYPE_F32 || !vx_is_contiguous(attn) || vx_nelements(attn) != vx_nelements(q))
+            return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: attn must be the attention's dense F32 result");
+        vx_tensor ad = *attn;
+        ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
+        ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+        const vx_status rc = vx_flash_attn_ext_store(q, k, v, mask, sinks, k_src, k_slot, v_src, v_slot, &ad, scale, max_bias, logit_softcap, sync_scale,
+                                                     sync_bias, stream);
+        return rc != VX_OK ? rc : vx_mul_mat_scale_add(w_o, attn, residual, dst, res_scale, act_mode, stream);
+    }
     pf_store_proj_ctx c{ { k_src, k_slot, v_src, v_slot, sync_scale, sync_bias }, nullptr };
     vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_proj_launch, &c };
     if (!pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front)) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: tile geometry");
