@@ -249,3 +249,48 @@ def test_backbone_cfg5_prefill_b16_t4096(gpu, ref):
     say(f"   every node its own launch ({plain_launches} launches): bit-equal to the grouped run: {same}; nmse {nmse(plain, plug):.3e}")
     assert plain_launches > launches
     assert same, "grouped launches changed a result"
+
+
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_backbone_prompt_lengths_grouped_equals_node_by_node(gpu, ref, kv_f16):
+    """A two-layer stack through the plugin at prompt lengths on both sides of every dispatch boundary a prompt crosses --
+    the streaming kernel's token limits (16, 64, 204), the three regimes of the cache write (128 / 129 and 512 / 513
+    tokens at batch 1), the LDS-tiled attention's minimum, the ROPE kernels' switch at 1024 tokens, the pre-tiled product's
+    thresholds --, batch 1 to 3: with node groups on, hidden states and the written cache are bit-equal to every node run
+    as its own launch, and finite."""
+    say(f"plugin prefill, grouped against node by node, over prompt lengths; f16 cache {kv_f16}")
+    layers = 2
+    params = reflib.backbone_params("bb-lengths", layers)
+    assert ref.rh_load_plugin(gpu.PLUGIN_PATH.encode()) == 0
+    plugin = ctypes.CDLL(gpu.PLUGIN_PATH)
+    assert ref.rh_use_device(b"GFX950_0", 1, 0) == 0
+    replay = plugin.ggml_backend_gfx950_set_graph_replay(0)
+    lengths = {1: (17, 63, 64, 65, 128, 129, 204, 205, 256, 511, 512, 513, 1023, 1024, 1100, 2048, 4096),
+               2: (64, 65, 128, 200, 256, 257, 512, 700, 1024, 2100),
+               3: (63, 100, 171, 342, 1000, 1536)}
+    try:
+        for B, Ts in lengths.items():
+            for T in Ts:
+                reflib.ref_backbone_create(params, T + 8, B, use_mup=True, kv_f16=kv_f16)
+                try:
+                    x = rng("bb-lengths", B, T).standard_normal((B, T, 1024)).astype(np.float32)
+                    mask = reflib.causal_mask(T, T)
+                    runs = []
+                    for fusion in (1, 0):
+                        before = plugin.ggml_backend_gfx950_set_fusion(fusion)
+                        try:
+                            out = reflib.ref_backbone_forward(x, 0, mask)[0].copy()
+                            cache = np.empty((B, 2, T + 8, 64), np.float16 if kv_f16 else np.float32)
+                            assert ref.rh_bb_cache_get(layers - 1, 0, cache.ctypes.data, cache.nbytes) == 0
+                        finally:
+                            plugin.ggml_backend_gfx950_set_fusion(before)
+                        runs.append((out, cache[:, :, :T].copy(), plugin.ggml_backend_gfx950_last_launches()))
+                finally:
+                    ref.rh_bb_free()
+                (o1, c1, l1), (o0, c0, l0) = runs
+                assert np.isfinite(o1).all(), (B, T)
+                assert l1 < l0, (B, T, l1, l0)
+                assert np.array_equal(o1, o0) and np.array_equal(c1, c0), f"batch {B}, {T} tokens: {l1} grouped launches differ from {l0} separate ones"
+    finally:
+        plugin.ggml_backend_gfx950_set_graph_replay(replay)
+        assert ref.rh_use_device(b"CPU", 8, 0) == 0
