@@ -289,6 +289,19 @@ def test_backbone_prompt_lengths_grouped_equals_node_by_node(gpu, ref, kv_f16):
                     ref.rh_bb_free()
                 (o1, c1, l1), (o0, c0, l0) = runs
                 assert np.isfinite(o1).all(), (B, T)
+                if (B, T) in ((1, 129), (1, 256), (1, 513), (2, 257), (3, 342)):   # and against ggml-cpu where that is quick
+                    assert ref.rh_use_device(b"CPU", 16, 0) == 0
+                    reflib.ref_backbone_create(params, T + 8, B, use_mup=True, kv_f16=kv_f16)
+                    try:
+                        cpu = reflib.ref_backbone_forward(x, 0, mask)[0].copy()
+                        ccache = np.empty((B, 2, T + 8, 64), np.float16 if kv_f16 else np.float32)
+                        assert ref.rh_bb_cache_get(layers - 1, 0, ccache.ctypes.data, ccache.nbytes) == 0
+                    finally:
+                        ref.rh_bb_free()
+                        assert ref.rh_use_device(b"GFX950_0", 1, 0) == 0
+                    e, ec = nmse(cpu, o1), nmse(ccache[:, :, :T].astype(np.float32), c1.astype(np.float32))
+                    say(f"   batch {B}, {T} tokens ({l1} launches): nmse vs ggml-cpu {e:.3e}, last layer's K cache {ec:.3e}")
+                    assert e <= 1e-4 and ec <= 1e-4, (B, T, e, ec)
                 assert l1 < l0, (B, T, l1, l0)
                 assert np.array_equal(o1, o0) and np.array_equal(c1, c0), f"batch {B}, {T} tokens: {l1} grouped launches differ from {l0} separate ones"
     finally:
