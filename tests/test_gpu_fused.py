@@ -789,6 +789,43 @@ def test_qkv_proj_rope(pkg, gpu, T, B, H, Hkv, D, K, act, yarn):
     assert L.vx_supports_qkv_proj_rope(pkg.desc_q8(wq, K), pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(q2), d(k2), d(v2), D // 2, 2) == 0
 
 
+@pytest.mark.parametrize("T,B,Hkv,D,K,flat", [(205, 1, 2, 64, 1024, False), (256, 1, 2, 64, 1024, True), (512, 2, 2, 64, 1024, True), (1024, 1, 2, 64, 1024, False),
+                                              (700, 1, 2, 64, 1024, True), (300, 3, 2, 64, 1024, False), (333, 1, 1, 128, 512, True), (40, 2, 4, 64, 2048, False)])
+@pytest.mark.parametrize("act", ["float", "q8"])
+@pytest.mark.parametrize("yarn", [False, True])
+def test_kv_proj_rope(pkg, gpu, T, B, Hkv, D, K, flat, act, yarn):
+    """The k and v projections with k's rotation as one launch of the streaming kernel, at token counts beyond the
+    three-matrix launch's (q's product is on a tiled kernel there): against two MUL_MATs and a ROPE, bit for bit, the
+    sequences as a batch or flattened into one token dimension."""
+    import torch
+    say(f"k/v projections + rope as one launch T={T} B={B} Hkv={Hkv} D={D} K={K} flat={flat} act={act} yarn={yarn}")
+    L, d = pkg.lib(), pkg.desc
+    mode = pkg.ACT_Q8 if act == "q8" else pkg.ACT_FLOAT
+    g = rng("f-kv", T, B, Hkv, D, K)
+    wk, _ = q8_dev((0.05 * g.standard_normal((Hkv * D, K))).astype(np.float32))
+    wv, _ = q8_dev((0.05 * g.standard_normal((Hkv * D, K))).astype(np.float32))
+    x = dev(g.standard_normal((B * T, K) if flat else (B, 1, T, K)).astype(np.float32))
+    pos = torch.arange(90, 90 + T, dtype=torch.int32, device="cuda")
+    ff = dev((1.0 + g.random(D // 2)).astype(np.float32))
+    rope_args = (D, 2, 4096, 10000.0, 1.0, 0.0, 1.1, 32.0, 1.0) if not yarn else (D, 2, 512, 10000.0, 0.5, 1.0, 1.0, 32.0, 1.0)
+    shape = (lambda t: t.view(B * T, Hkv * D)) if flat else (lambda t: t.view(B, 1, T, Hkv * D))
+    k1 = torch.empty((B, T, Hkv, D), dtype=torch.float32, device="cuda")
+    v1 = torch.empty((B, T, Hkv * D), dtype=torch.float32, device="cuda")
+    ok(pkg, L.vx_mul_mat(pkg.desc_q8(wk, K), d(x), d(shape(k1)), mode, None), "k")
+    ok(pkg, L.vx_mul_mat(pkg.desc_q8(wv, K), d(x), d(shape(v1)), mode, None), "v")
+    ok(pkg, L.vx_rope(d(k1), pos.data_ptr(), ff.data_ptr(), d(k1), *rope_args, None), "rope")
+    k2, v2 = torch.full_like(k1, float("nan")), torch.full_like(v1, float("nan"))
+    if not L.vx_supports_kv_proj_rope(pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(k2), d(shape(v2)), D, 2):
+        assert flat and B * T * 2 * Hkv * D > 256 * 1024   # (beyond the streaming kernel's work bound)
+        assert L.vx_kv_proj_rope(pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), pos.data_ptr(), ff.data_ptr(), d(k2), d(shape(v2)), *rope_args, mode, None) != 0
+        return
+    ok(pkg, L.vx_kv_proj_rope(pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), pos.data_ptr(), ff.data_ptr(), d(k2), d(shape(v2)), *rope_args, mode, None),
+       "kv_proj_rope")
+    torch.cuda.synchronize()
+    assert torch.equal(v1, v2) and torch.equal(k1, k2)
+    assert L.vx_supports_kv_proj_rope(pkg.desc_q8(wk, K), pkg.desc_q8(wv, K), d(x), d(k2), d(shape(v2)), D, 0) == 0
+
+
 @pytest.mark.parametrize("seed", list(range(40)))
 def test_qkv_and_mlp_groups_random_shapes(pkg, gpu, seed):
     """The q/k/v + rope group, with and without the norm in front, and the norm + gate/up + SwiGLU group at random token

@@ -63,7 +63,7 @@ EXPORTS = [
     "vx_supports_cpy", "vx_supports_concat", "vx_supports_sum",
     "vx_arange", "vx_repeat", "vx_get_rows", "vx_supports_arange", "vx_supports_repeat", "vx_supports_get_rows",
     "vx_small_graph", "vx_supports_small_node", "vx_mul_mat_sum_order",
-    "vx_rms_norm_mul", "vx_scale_add", "vx_add_scale", "vx_flash_attn_ext_add1", "vx_mul_mat_swiglu", "vx_supports_mul_mat_swiglu", "vx_supports_mul_mat_swiglu_tiled", "vx_mul_mat_scale_add", "vx_supports_mul_mat_scale_add", "vx_kv_store_sync", "vx_supports_kv_store_sync", "vx_flash_attn_ext_kv2", "vx_supports_flash_attn_ext_kv2", "vx_flash_attn_ext_kv2_store", "vx_supports_flash_attn_ext_kv2_store", "vx_flash_attn_ext_store", "vx_supports_flash_attn_ext_store", "vx_flash_attn_ext_store_proj", "vx_supports_flash_attn_ext_store_proj", "vx_qkv_proj_rope", "vx_supports_qkv_proj_rope", "vx_norm_qkv_proj_rope", "vx_supports_norm_qkv_proj_rope", "vx_norm_mul_mat_swiglu", "vx_supports_norm_qkv_proj_rope_tiled", "vx_supports_mlp_tiled", "vx_mlp_tiled", "vx_supports_norm_mul_mat_swiglu_tiled", "vx_supports_norm_mul_mat_swiglu", "vx_supports_rms_norm_mul", "vx_supports_fused_pair",
+    "vx_rms_norm_mul", "vx_scale_add", "vx_add_scale", "vx_flash_attn_ext_add1", "vx_mul_mat_swiglu", "vx_supports_mul_mat_swiglu", "vx_supports_mul_mat_swiglu_tiled", "vx_mul_mat_scale_add", "vx_supports_mul_mat_scale_add", "vx_kv_store_sync", "vx_supports_kv_store_sync", "vx_flash_attn_ext_kv2", "vx_supports_flash_attn_ext_kv2", "vx_flash_attn_ext_kv2_store", "vx_supports_flash_attn_ext_kv2_store", "vx_flash_attn_ext_store", "vx_supports_flash_attn_ext_store", "vx_flash_attn_ext_store_proj", "vx_supports_flash_attn_ext_store_proj", "vx_qkv_proj_rope", "vx_supports_qkv_proj_rope", "vx_kv_proj_rope", "vx_supports_kv_proj_rope", "vx_norm_qkv_proj_rope", "vx_supports_norm_qkv_proj_rope", "vx_norm_mul_mat_swiglu", "vx_supports_norm_qkv_proj_rope_tiled", "vx_supports_mlp_tiled", "vx_mlp_tiled", "vx_supports_norm_mul_mat_swiglu_tiled", "vx_supports_norm_mul_mat_swiglu", "vx_supports_rms_norm_mul", "vx_supports_fused_pair",
 ]
 
 BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV = 0, 1, 2, 3
@@ -178,6 +178,8 @@ def lib():
     l.vx_supports_flash_attn_ext_store_proj.argtypes = [TP] * 12 + [C.c_float, C.c_int]
     l.vx_qkv_proj_rope.argtypes = [TP, TP, TP, TP, i32p, f32p, TP, TP, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [C.c_int, vp]
     l.vx_supports_qkv_proj_rope.argtypes = [TP, TP, TP, TP, TP, TP, TP, C.c_int, C.c_int]
+    l.vx_kv_proj_rope.argtypes = [TP, TP, TP, i32p, f32p, TP, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [C.c_int, vp]
+    l.vx_supports_kv_proj_rope.argtypes = [TP, TP, TP, TP, TP, C.c_int, C.c_int]
     l.vx_norm_qkv_proj_rope.argtypes = [TP, TP, C.c_float, TP, TP, TP, i32p, f32p, TP, TP, TP, C.c_int, C.c_int, C.c_int] + [C.c_float] * 6 + [C.c_int, vp]
     l.vx_supports_norm_qkv_proj_rope.argtypes = [TP, TP, TP, TP, TP, TP, TP, TP, C.c_int, C.c_int]
     l.vx_supports_norm_qkv_proj_rope_tiled.argtypes = [TP, TP, TP, TP, TP, TP, TP, TP, C.c_int, C.c_int, C.c_int]

@@ -196,10 +196,14 @@ class MiniCPMBackbone:
             else:
                 norm(cur_x, nw_in, normed)
                 call(L.vx_mul_mat, wd["q_proj"], desc(normed), desc(q), self.act_mode)
-                call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
-                call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
-                for t4 in (q4, k4):
-                    call(L.vx_rope, desc(t4), _p(pos), ff, desc(t4), *rope_args)
+                call(L.vx_rope, desc(q4), _p(pos), ff, desc(q4), *rope_args)
+                if fuse and plain_order and L.vx_supports_kv_proj_rope(wd["k_proj"], wd["v_proj"], desc(normed), desc(k4), desc(v), D, 2):
+                    # a prompt of a few hundred tokens: k, v and k's rotation still fit one launch of the streaming kernel
+                    call(L.vx_kv_proj_rope, wd["k_proj"], wd["v_proj"], desc(normed), _p(pos), ff, desc(k4), desc(v), *rope_args, self.act_mode)
+                else:
+                    call(L.vx_mul_mat, wd["k_proj"], desc(normed), desc(k), self.act_mode)
+                    call(L.vx_rope, desc(k4), _p(pos), ff, desc(k4), *rope_args)
+                    call(L.vx_mul_mat, wd["v_proj"], desc(normed), desc(v), self.act_mode)
             # from here on in the order ggml_build_forward_expand gives the reference's graph: concat, attention,
             # then the cache append with its ordering chain, then add1 (only adjacent nodes are run as one launch)
             k_all, v_all = k4.transpose(1, 2), v4.transpose(1, 2)   # ggml_permute(0, 2, 1, 3)

@@ -3061,6 +3061,80 @@ extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk
                    ext_factor, attn_factor, beta_fast, beta_slow, act_mode, stream);
 }
 
+// K and V alone: MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x).  From 205 tokens on the three-matrix launch above no longer
+// applies (q's product leaves the streaming kernel there, and with it the order of its sums), but the two 128-row
+// products stay on it up to 1024 tokens: one launch for the two of them and k's rotation instead of three.
+extern "C" int vx_supports_kv_proj_rope(const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x, const vx_tensor * k_dst,
+                                        const vx_tensor * v_dst, int n_dims, int mode) {
+    if (!wk || !wv || !x || !k_dst || !v_dst) return 0;
+    if (wk->type != VX_TYPE_Q8_0 && wk->type != VX_TYPE_F16) return 0;
+    const vx_tensor * ws[2] = { wk, wv };
+    for (const vx_tensor * w : ws) {
+        if (w->type != wk->type || w->ne[0] != wk->ne[0] || w->ne[2] != 1 || w->ne[3] != 1 || !vx_positive(w)) return 0;
+        if (w->nb[0] != vx_type_size(w->type) || w->nb[1] < vx_row_size(w->type, w->ne[0])) return 0;
+        if (w->type == VX_TYPE_F16 && w->nb[1] % 2) return 0;
+    }
+    if (x->type != VX_TYPE_F32 || !vx_positive(x) || x->ne[0] != wk->ne[0] || x->ne[2] != 1 || x->nb[0] != 4) return 0;
+    if (x->nb[1] % 4 || x->nb[3] % 4 || x->ne[3] > 65535) return 0;
+    if (wk->ne[0] % 32 || wk->ne[0] < 32) return 0;
+    if (mode != 2 || n_dims <= 0 || n_dims % 16) return 0;
+    if (!qkv_rope_dst_ok(wk, x, k_dst, n_dims)) return 0;
+    if (v_dst->type != VX_TYPE_F32 || v_dst->nb[0] != 4 || v_dst->nb[1] % 4 || v_dst->nb[3] % 4) return 0;
+    if (v_dst->nb[1] < (uint64_t) v_dst->ne[0] * 4 || (v_dst->ne[3] > 1 && v_dst->nb[3] < v_dst->nb[1] * (uint64_t) v_dst->ne[1])) return 0;
+    if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
+    const int64_t tokens = x->ne[1] * x->ne[2] * x->ne[3];
+    if (gemv_waves_for(wk->ne[0], tokens, wk->ne[1]) != gemv_waves_for(wk->ne[0], tokens, wv->ne[1])) return 0;
+    return gemv_shape_ok(x->ne[1], wk->ne[1] + wv->ne[1], wk->ne[0]);
+}
+
+extern "C" vx_status vx_kv_proj_rope(const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x, const int32_t * pos,
+                                     const float * freq_factors, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims, int mode,
+                                     int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                                     float beta_fast, float beta_slow, int act_mode, vx_stream stream) {
+    if (!vx_supports_kv_proj_rope(wk, wv, x, k_dst, v_dst, n_dims, mode))
+        return vx_fail(VX_ERR_UNSUPPORTED, "kv_proj_rope: two Q8_0/F16 matrices over one activation tensor, a token count the streaming kernel takes, NEOX rotation over the whole head, contiguous k output");
+    if (!pos || !wk->data || !wv->data || !x->data || !k_dst->data || !v_dst->data) return vx_fail(VX_ERR_INVALID, "kv_proj_rope: null data");
+    if (act_mode != VX_ACT_FLOAT && act_mode != VX_ACT_Q8) return vx_fail(VX_ERR_INVALID, "kv_proj_rope: bad act_mode");
+    const vx_tensor * ws[2] = { wk, wv };
+    const vx_tensor * ds[2] = { k_dst, v_dst };
+    if ((uintptr_t) x->data % 4) return vx_fail(VX_ERR_UNSUPPORTED, "kv_proj_rope: misaligned activations");
+    mm_args a = {};
+    a.x = (const char *) x->data;
+    a.K = wk->ne[0]; a.N = x->ne[1];
+    a.M = 0;
+    a.nb11 = x->nb[1]; a.nb12 = x->nb[2]; a.nb13 = x->nb[3];
+    a.ne12 = 1; a.r2 = 1; a.r3 = 1;
+    a.rows_wg = 16;
+    a.w_aligned = 1;
+    a.nseg = 2;
+    for (int i = 0; i < 2; ++i) {
+        if ((uintptr_t) ds[i]->data % 4 || (ws[i]->type == VX_TYPE_F16 && (uintptr_t) ws[i]->data % 2))
+            return vx_fail(VX_ERR_UNSUPPORTED, "kv_proj_rope: misaligned tensor data");
+        gv_seg & sg = a.seg[i];
+        sg.w = (const char *) ws[i]->data; sg.dst = (char *) ds[i]->data;
+        sg.M = ws[i]->ne[1]; sg.nb01 = ws[i]->nb[1];
+        sg.nb1 = (uint64_t) sg.M * 4; sg.nb2 = 0; sg.nb3 = (uint64_t) sg.M * 4 * x->ne[1];
+        if (i == 1) { sg.nb1 = v_dst->nb[1]; sg.nb3 = v_dst->nb[3]; }
+        sg.rope = i == 0;
+        a.w_aligned = a.w_aligned && ((uintptr_t) ws[i]->data % 4 == 0) && ws[i]->nb[1] % 4 == 0;
+        a.M += sg.M;
+    }
+    a.w = a.seg[0].w; a.dst = a.seg[0].dst;
+    a.x_aligned = ((uintptr_t) x->data % 16 == 0) && x->nb[1] % 16 == 0 && x->nb[3] % 16 == 0;
+    a.pos = pos; a.ff = freq_factors;
+    a.rp = rope_make_params(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    a.head_dim = n_dims;
+    a.rope_T   = (int) k_dst->ne[2];
+    const int nbatch = (int) x->ne[3];
+    hipStream_t st = (hipStream_t) stream;
+    bool ok;
+    if (wk->type == VX_TYPE_Q8_0) ok = act_mode == VX_ACT_Q8 ? launch_gemv<WT_Q8, true>(a, nbatch, st) : launch_gemv<WT_Q8, false>(a, nbatch, st);
+    else                          ok = launch_gemv<WT_F16, false>(a, nbatch, st);
+    if (!ok) return vx_fail(VX_ERR_UNSUPPORTED, "kv_proj_rope: shape outside the streaming kernel");
+    VX_LAUNCH_CHECK();
+    return VX_OK;
+}
+
 // RMS_NORM , MUL(norm weight) in front of the three projections: layer_forward's input rms_norm
 // (src/minicpm.cpp:572-580, 761) joins the launch; x is the un-normalised hidden state.
 extern "C" int vx_supports_norm_qkv_proj_rope(const vx_tensor * x, const vx_tensor * norm_w, const vx_tensor * wq, const vx_tensor * wk,

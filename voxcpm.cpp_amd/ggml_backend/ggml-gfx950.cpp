@@ -1234,6 +1234,36 @@ bool compute_qkv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const re
     return true;
 }
 
+// The same for K and V alone, where q's product has left the streaming kernel (a prompt of 205 to 1024 tokens):
+//   MUL_MAT(wk, x) RESHAPE ROPE  [views, absorbed CONCAT]  MUL_MAT(wv, x)      -> one launch at the first node
+bool compute_kv_group(backend_ctx * ctx, const ggml_cgraph * g, int i, const reader_map & readers, const absorbed_map & absorbed,
+                      std::unordered_set<const ggml_tensor *> & done, vx_status * rc) {
+    const ggml_tensor * mk = g->nodes[i];
+    if (mk->op != GGML_OP_MUL_MAT) return false;
+    int idx = i;
+    const ggml_tensor * rk = rope_of_projection(g, idx, mk, readers, absorbed);
+    if (!rk) return false;
+    ++idx;
+    while (idx < g->n_nodes && (ggml_op_is_empty(g->nodes[idx]->op) || ggml_is_empty(g->nodes[idx]) || absorbed.count(g->nodes[idx]))) ++idx;
+    if (idx >= g->n_nodes) return false;
+    const ggml_tensor * mv = g->nodes[idx];
+    if (mv->op != GGML_OP_MUL_MAT || mv->src[1] != mk->src[1] || (mv->flags & GGML_TENSOR_FLAG_COMPUTE) == 0) return false;
+    if (!rk->src[1] || rk->src[1]->type != GGML_TYPE_I32 || rk->src[1]->ne[0] != rk->ne[2]) return false;
+    if (rk->src[2] && (rk->src[2]->type != GGML_TYPE_F32 || rk->src[2]->ne[0] < rk->ne[0] / 2)) return false;
+    const int32_t * ip = (const int32_t *) rk->op_params;
+    const int n_dims = ip[1], mode = ip[2], n_ctx_orig = ip[4];
+    float fp[6];
+    memcpy(fp, ip + 5, sizeof(fp));
+    const ggml_tensor * x = mk->src[1];
+    if (!apart(rk, x) || !apart(mv, x) || !apart(rk, mv)) return false;
+    const vx_tensor wk = to_vx(mk->src[0]), wv = to_vx(mv->src[0]), xx = to_vx(x), dk = to_vx(rk), dv = to_vx(mv);
+    if (!vx_supports_kv_proj_rope(&wk, &wv, &xx, &dk, &dv, n_dims, mode)) return false;
+    *rc = vx_kv_proj_rope(&wk, &wv, &xx, (const int32_t *) rk->src[1]->data, rk->src[2] ? (const float *) rk->src[2]->data : nullptr, &dk, &dv,
+                          n_dims, mode, n_ctx_orig, fp[0], fp[1], fp[2], fp[3], fp[4], fp[5], mul_mat_act_mode(), ctx->stream);
+    done.insert(rk); done.insert(mv);
+    return true;
+}
+
 // The reference's row-fused weights (MiniCPMModel::load_from_store makes them for the LocDiT decoder on a GPU backend,
 // src/minicpm.cpp:427-492): one MUL_MAT over qkv_proj, strided views of it as q, k, v, ROPE on the q and k views
 // (src/minicpm.cpp:644-680)
@@ -1769,6 +1799,7 @@ ggml_status graph_compute_eager(backend_ctx * ctx, ggml_cgraph * cgraph, int * l
         }
         if (fusion && node->op == GGML_OP_MUL_MAT &&
             (compute_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc) ||
+             compute_kv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc) ||
              compute_fused_qkv_group(ctx, cgraph, i, readers, kv2_absorbed, done, &rc) ||
              compute_fused_gate_up_group(ctx, cgraph, i, readers, done, &rc))) {
             ++launches;
