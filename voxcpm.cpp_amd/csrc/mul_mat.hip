@@ -1065,12 +1065,15 @@ constexpr size_t GV_ROPE_LDS = 4 * 64 * 8;     // cos / sin of four token slots 
 
 // Shapes the streaming kernel takes: up to 16 tokens always; more (in chunks of 16, the chunks re-reading
 // the weight rows from L2) while tokens x rows stays small -- measured against the tiled kernels: 1024 rows win up
-// to 256 tokens, 4096 rows up to 64.  VX_GEMV_MAX_TOKENS=16 restores the 16-token limit.
+// to 448 tokens, 4096 rows up to 64.  VX_GEMV_MAX_TOKENS=16 restores the 16-token limit.
 bool gemv_shape_ok(int64_t N, int64_t rows, int64_t K) {
     static const int64_t max_tokens = [] { const char * e = getenv("VX_GEMV_MAX_TOKENS"); const int n = e ? atoi(e) : 0; return n >= 16 ? (int64_t) n : (int64_t) 1 << 30; }();
     if (K % 32 || K < 32 || N < 1) return false;
     static const int64_t max_work = [] { const char * e = getenv("VX_GEMV_MAX_WORK"); const long n = e ? atol(e) : 0; return n > 0 ? (int64_t) n : (int64_t) 256 * 1024; }();
-    if (N > 16 && (N > max_tokens || N * rows > max_work)) return false;
+    // (up to 1024 rows the tiled kernels' 64-token tiles are under a work-group per compute unit until some 500 tokens, 14 to
+    // 15 us whatever the count: the chunks win up to 448 tokens -- 9.2 us at 256, 11.2 at 384)
+    static const bool wide = getenv("VX_GEMV_MAX_WORK") == nullptr;
+    if (N > 16 && (N > max_tokens || (N * rows > max_work && !(wide && rows <= 1024 && N <= 448)))) return false;
     // chunks of 16 tokens each stage 16 x K activations: with a long K a work-group fills a CU's LDS alone and the chunks
     // queue up behind each other (1024 rows x K = 4096 at 112 tokens: 63 us against 26 us on the tiled kernel with its K cut)
     if (N > 16 && K > 2048) return false;
