@@ -191,15 +191,17 @@ def test_supports_truth_table_node_groups(pkg):
     def acts(n, k=K):
         return f32(pkg, [k, n, 1, 1])
 
-    # projection + scale + residual: every token count; beyond the streaming kernel's (16, or tokens x rows <= 256 Ki) and
-    # the K-cut shapes only into a dense destination with rows in whole 16-byte groups
-    for n, want in ((1, 1), (16, 1), (17, 1), (256, 1), (257, 1), (65536, 1)):
+    # projection + scale + residual: every token count; beyond the streaming kernel's (16, tokens x rows <= 256 Ki, or 448
+    # tokens of at most 1024 rows) and the K-cut shapes only into a dense destination with rows in whole 16-byte groups
+    for n, want in ((1, 1), (16, 1), (17, 1), (256, 1), (257, 1), (449, 1), (65536, 1)):
         assert lib.vx_supports_mul_mat_scale_add(wo, acts(n), acts(n), acts(n)) == want, n
-    strided = D(pkg, pkg.F32, [K, 257, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 257, 4 * (K + 8) * 257])
-    assert lib.vx_supports_mul_mat_scale_add(wo, acts(257), acts(257), strided) == 0
+    strided = D(pkg, pkg.F32, [K, 449, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 449, 4 * (K + 8) * 449])
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(449), acts(449), strided) == 0
+    strided = D(pkg, pkg.F32, [K, 448, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 448, 4 * (K + 8) * 448])
+    assert lib.vx_supports_mul_mat_scale_add(wo, acts(448), acts(448), strided) == 1
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(14), acts(14), D(pkg, pkg.F32, [K, 14, 1, 1], [4, 4 * (K + 8), 4 * (K + 8) * 14, 4 * (K + 8) * 14])) == 1
     odd = q8(pkg, [K, 1002, 1, 1])
-    assert lib.vx_supports_mul_mat_scale_add(odd, acts(300), f32(pkg, [1002, 300, 1, 1]), f32(pkg, [1002, 300, 1, 1])) == 0
+    assert lib.vx_supports_mul_mat_scale_add(odd, acts(500), f32(pkg, [1002, 500, 1, 1]), f32(pkg, [1002, 500, 1, 1])) == 0
     assert lib.vx_supports_mul_mat_scale_add(wdown, acts(14, 4096), acts(14), acts(14)) == 1      # 16 x 4096 halves of LDS
     # gate + up + GLU on the tiled kernel: f16 activations, 64 tokens or more, shapes the streaming kernel does not take, and
     # products that the tiled kernel walks with K whole (at least 64 tiles of 64 x 64 each)
