@@ -371,8 +371,8 @@ VX_API int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk,
                                      const vx_tensor * q_dst, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims,
                                      int mode);
 /* K and V alone -- MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x) (src/minicpm.cpp:671-680) -- as one launch of the same
- * kernel: for token counts where q's product is no longer one the streaming kernel runs (from 205 tokens at 1024 rows)
- * but those of k and v still are (up to 1024 tokens at 2 x 128 rows).  Arguments and bits as in vx_qkv_proj_rope. */
+ * kernel: for token counts where q's product is no longer one the streaming kernel runs (from 449 tokens at 1024 rows)
+ * but those of k and v still are (up to 2048 tokens at 128 rows each).  Arguments and bits as in vx_qkv_proj_rope. */
 VX_API vx_status vx_kv_proj_rope(const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x, const int32_t * pos,
                                  const float * freq_factors, const vx_tensor * k_dst, const vx_tensor * v_dst, int n_dims,
                                  int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,

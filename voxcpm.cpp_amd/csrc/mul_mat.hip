@@ -1200,9 +1200,10 @@ template <int WT, bool ACT_Q8>
 bool launch_gemv(const mm_args & a0, int nbatch, hipStream_t st) {
     mm_args a = a0;
     {
-        int64_t rows = a.w2 ? 2 * a.M : a.M;
-        if (a.nseg > 0) { rows = 0; for (int i = 0; i < a.nseg; ++i) rows += a.seg[i].M; }
-        if (!gemv_shape_ok(a.N, rows, a.K)) return false;
+        // (several matrices in one launch: wherever each of them alone is this kernel's shape -- the launch then sums every
+        // product as its own call would)
+        if (a.nseg > 0) { for (int i = 0; i < a.nseg; ++i) if (!gemv_shape_ok(a.N, a.seg[i].M, a.K)) return false; }
+        else if (!gemv_shape_ok(a.N, a.w2 ? 2 * a.M : a.M, a.K)) return false;
     }
     if (a.M >= ((int64_t) 1 << 31) || a.K >= ((int64_t) 1 << 31)) return false;
     a.rows_wg = 16;
@@ -2984,7 +2985,7 @@ extern "C" int vx_supports_qkv_proj_rope(const vx_tensor * wq, const vx_tensor *
         const int nw = gemv_waves_for(wq->ne[0], tokens, wq->ne[1]);
         if (gemv_waves_for(wq->ne[0], tokens, wk->ne[1]) != nw || gemv_waves_for(wq->ne[0], tokens, wv->ne[1]) != nw) return 0;
     }
-    return gemv_shape_ok(x->ne[1], wq->ne[1] + wk->ne[1] + wv->ne[1], wq->ne[0]);
+    return gemv_shape_ok(x->ne[1], wq->ne[1], wq->ne[0]) && gemv_shape_ok(x->ne[1], wk->ne[1], wq->ne[0]) && gemv_shape_ok(x->ne[1], wv->ne[1], wq->ne[0]);
 }
 
 // The order in which vx_mul_mat (and every group built on it) sums the K blocks of a product, as an opaque number: two
@@ -3064,9 +3065,9 @@ extern "C" vx_status vx_qkv_proj_rope(const vx_tensor * wq, const vx_tensor * wk
                    ext_factor, attn_factor, beta_fast, beta_slow, act_mode, stream);
 }
 
-// K and V alone: MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x).  From 205 tokens on the three-matrix launch above no longer
+// K and V alone: MUL_MAT(wk, x) RESHAPE ROPE , MUL_MAT(wv, x).  From 449 tokens on the three-matrix launch above no longer
 // applies (q's product leaves the streaming kernel there, and with it the order of its sums), but the two 128-row
-// products stay on it up to 1024 tokens: one launch for the two of them and k's rotation instead of three.
+// products stay on it up to 2048 tokens: one launch for the two of them and k's rotation instead of three.
 extern "C" int vx_supports_kv_proj_rope(const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x, const vx_tensor * k_dst,
                                         const vx_tensor * v_dst, int n_dims, int mode) {
     if (!wk || !wv || !x || !k_dst || !v_dst) return 0;
@@ -3087,7 +3088,7 @@ extern "C" int vx_supports_kv_proj_rope(const vx_tensor * wk, const vx_tensor * 
     if (v_dst->ne[0] != wv->ne[1] || v_dst->ne[1] != x->ne[1] || v_dst->ne[2] != 1 || v_dst->ne[3] != x->ne[3]) return 0;
     const int64_t tokens = x->ne[1] * x->ne[2] * x->ne[3];
     if (gemv_waves_for(wk->ne[0], tokens, wk->ne[1]) != gemv_waves_for(wk->ne[0], tokens, wv->ne[1])) return 0;
-    return gemv_shape_ok(x->ne[1], wk->ne[1] + wv->ne[1], wk->ne[0]);
+    return gemv_shape_ok(x->ne[1], wk->ne[1], wk->ne[0]) && gemv_shape_ok(x->ne[1], wv->ne[1], wk->ne[0]);
 }
 
 extern "C" vx_status vx_kv_proj_rope(const vx_tensor * wk, const vx_tensor * wv, const vx_tensor * x, const int32_t * pos,
