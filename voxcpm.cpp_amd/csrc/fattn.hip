@@ -1174,7 +1174,7 @@ static vx_status pf_store_proj_launch(void * front, void * ctx, hipStream_t st) 
 // attn: the attention's result as the projection reads it, [hidden, tokens (, batch)], dense; the same memory order as the
 // attention's own [head_dim, heads, tokens, batch]
 static bool pf_proj_geometry(const vx_tensor * q, const vx_tensor * attn, const vx_tensor * w_o, const vx_tensor * residual, const vx_tensor * dst,
-                             int act_mode, vx_pf_front * front) {
+                             int act_mode, vx_pf_front * front, size_t * proj_bytes) {
     if (!attn || !w_o || !residual || !dst || attn->type != VX_TYPE_F32 || !vx_is_contiguous(attn)) return false;
     const int64_t hidden = q->ne[0] * q->ne[2], T = q->ne[1], B = q->ne[3];
     if (attn->ne[0] != hidden || vx_nelements(attn) != hidden * T * B) return false;
@@ -1183,7 +1183,7 @@ static bool pf_proj_geometry(const vx_tensor * q, const vx_tensor * attn, const 
     if (!flat && !by_batch) return false;
     uint32_t tile_tt = 0, n_kb = 0;
     size_t   tile_bytes = 0;
-    if (!vx_proj_tiles_ok(w_o, attn, residual, dst, act_mode, &tile_tt, &n_kb, &tile_bytes)) return false;
+    if (!vx_proj_tiles_ok(w_o, attn, residual, dst, act_mode, &tile_tt, &n_kb, &tile_bytes, proj_bytes)) return false;
     front->tiles = true; front->tiles_at = PF_STORE_FRONT;
     front->tile_tt = tile_tt;
     front->tile_bs = by_batch && !flat ? n_kb * tile_tt : 0;
@@ -1203,7 +1203,8 @@ extern "C" int vx_supports_flash_attn_ext_store_proj(const vx_tensor * q, const 
     ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
     if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, &ad, logit_softcap)) return 0;
     vx_pf_front front{};
-    return pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front) ? 1 : 0;
+    size_t proj_bytes = 0;
+    return pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front, &proj_bytes) ? 1 : 0;
 }
 
 extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_tensor * k, const vx_tensor * v, const vx_tensor * mask,
@@ -1230,11 +1231,18 @@ extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_
     }
     pf_store_proj_ctx c{ { k_src, k_slot, v_src, v_slot, sync_scale, sync_bias }, nullptr };
     vx_pf_front front{ PF_STORE_FRONT, PF_STORE_ADDEND_AT, pf_store_proj_launch, &c };
-    if (!pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front)) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: tile geometry");
+    size_t proj_bytes = 0;
+    if (!pf_proj_geometry(q, attn, w_o, residual, dst, act_mode, &front, &proj_bytes)) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: tile geometry");
+    hipStream_t st = (hipStream_t) stream;
+    {   // one block for both phases: the projection's request must not find the block too small once the attention has run
+        // (a request that grows the block moves it, and under a capture growth is refused)
+        void * p = nullptr;
+        const vx_status rc = vx_workspace(st, front.bytes + proj_bytes, &p);
+        if (rc != VX_OK) return rc;
+    }
     vx_tensor ad = *attn; // (never written: the result leaves as tiles)
     ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
     ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
-    hipStream_t st = (hipStream_t) stream;
     vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, nullptr, &ad, scale, max_bias, logit_softcap, st, &front);
     if (rc != VX_OK) return rc == VX_ERR_UNSUPPORTED ? vx_fail(rc, "flash_attn_ext_store_proj: the LDS-tiled kernel declined") : rc;
     // the projection: its own needs go behind the front (a block that a larger request replaces stays valid)

@@ -2924,9 +2924,13 @@ static bool proj_tiles_fill(mm_args & b, const vx_tensor * w, const vx_tensor * 
 }
 
 bool vx_proj_tiles_ok(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, int act_mode,
-                      uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes) {
+                      uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes, size_t * own_bytes) {
     mm_args b;
     if (!proj_tiles_fill(b, w, x, residual, dst, 0.0f, act_mode)) return false;
+    {   // what the product itself puts behind the tiles when the weights' tiles are not kept: as launch_gemm_q8t sizes them
+        const size_t kb = (size_t) (b.K / 32), rt = (size_t) ((b.M + 15) / 16);
+        *own_bytes = kb * rt * 1024 + (kb * ((rt + 3) & ~(size_t) 3) * 16 * 4 + 1023) / 1024 * 1024 + 1024;
+    }
     const int64_t tt = (b.N + QT_TOKS - 1) / QT_TOKS * (QT_TOKS / 16), nbatch = x->ne[2] * x->ne[3];
     if (tt * (b.K / 32) * nbatch >= ((int64_t) 1 << 31)) return false;
     *tile_tt = (uint32_t) tt; *n_kb = (uint32_t) (b.K / 32);

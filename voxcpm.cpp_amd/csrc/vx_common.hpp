@@ -112,7 +112,7 @@ vx_status vx_fattn_prefill(const vx_tensor * q, const vx_tensor * k, const vx_te
 // separate call would read (only shape and strides are looked at).  _ok: the separate call would run on the pre-tiled
 // kernel; it reports the tile geometry.  _run: tiles at `tiles`, the first ws_offset bytes of the workspace are the caller's.
 bool      vx_proj_tiles_ok(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, int act_mode,
-                           uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes);
+                           uint32_t * tile_tt, uint32_t * n_kb, size_t * tile_bytes, size_t * own_bytes);
 vx_status vx_proj_tiles_run(const vx_tensor * w, const vx_tensor * x, const vx_tensor * residual, const vx_tensor * dst, float scale,
                             int act_mode, const void * tiles, size_t ws_offset, hipStream_t stream);
 
