@@ -307,3 +307,54 @@ def test_backbone_prompt_lengths_grouped_equals_node_by_node(gpu, ref, kv_f16):
     finally:
         plugin.ggml_backend_gfx950_set_graph_replay(replay)
         assert ref.rh_use_device(b"CPU", 8, 0) == 0
+
+
+def test_mirror_prefill_one_pass_calls_grouped_unfused_and_captured(gpu):
+    """A two-layer stack at 16 x 2048 tokens through the C ABI -- the size from which a layer is three one-pass calls
+    (vx_norm_qkv_proj_rope with the rotations in the product's epilogue, vx_flash_attn_ext_store_proj, vx_mlp_tiled) --:
+    the same bits as every node as its own call, cache included; and captured into a HIP graph, every replay (with other
+    work on the stream between them) gives the eager run's bits again."""
+    import torch
+    from voxcpm_cpp_amd import backbone as bb
+    layers, B, T = 2, 16, 2048
+    say(f"C ABI mirror, {layers} layers, {B} x {T} tokens: one-pass calls against separate ones, eager and replayed")
+    params = reflib.backbone_params("bb-onepass", layers)
+    x = torch.from_numpy(rng("bb-onepass", "x").standard_normal((B, T, 1024)).astype(np.float32)).cuda()
+    mask = torch.from_numpy(reflib.causal_mask(T, T)).cuda()
+    outs, caches, calls = [], [], []
+    for fuse in (True, False):
+        m = bb.MiniCPMBackbone(n_layer=layers, max_length=T + 8, batch=B, use_mup=True, kv_f16=True, act_mode=gpu.ACT_FLOAT, fuse_pairs=fuse)
+        for li, lw in enumerate(params["layers"]):
+            for n in reflib.BB_WEIGHTS:
+                m.set_weight(li, n, torch.from_numpy(lw[n]).cuda(), params["shapes"][n][1])
+            for n in ("input_layernorm", "post_layernorm"):
+                m.set_norm(li, n, torch.from_numpy(lw[n]).cuda())
+        m.set_norm(-1, "norm", torch.from_numpy(params["final_norm"]).cuda())
+        m.rope_factors = torch.from_numpy(params["rope_factors"]).cuda()
+        run, got = m.plan(x, T, 0, mask)
+        run()
+        torch.cuda.synchronize()
+        outs.append(got.clone()); caches.append(m.k_cache[layers - 1].clone()); calls.append(run.n_calls)
+        if fuse:
+            fused_model, fused_run, fused_out = m, run, got
+    say(f"   {calls[0]} calls against {calls[1]}")
+    assert calls[0] == 3 * layers + 1
+    assert bool(torch.isfinite(outs[0]).all())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(caches[0].view(torch.uint8), caches[1].view(torch.uint8))
+    # captured and replayed (two eager runs on the capture stream first: its workspace block must exist before the capture)
+    cap = torch.cuda.Stream()
+    with torch.cuda.stream(cap):
+        for _ in range(2):
+            fused_run()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=cap):
+        fused_run()
+    for rep in range(3):
+        fused_out.zero_()
+        fused_model.k_cache[layers - 1].zero_()
+        (torch.randn(1 << 20, device="cuda") * 2).sum().item()   # other work between the replays
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(fused_out, outs[0]), f"replay {rep}"
+        assert torch.equal(fused_model.k_cache[layers - 1].view(torch.uint8), caches[0].view(torch.uint8)), f"replay {rep}: cache"
