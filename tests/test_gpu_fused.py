@@ -420,7 +420,7 @@ def test_flash_attn_ext_store(pkg, gpu, B, T, Hkv, H, f16, poison):
     assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(a.nan_to_num(123.0), b.nan_to_num(123.0))
 
 
-@pytest.mark.parametrize("B,T,flat", [(16, 2048, True), (8, 4100, True), (16, 2048, False), (5, 7000, True)])
+@pytest.mark.parametrize("B,T,flat", [(16, 2048, True), (8, 4100, True), (16, 2048, False), (5, 7000, True), (16, 1024, True), (2, 300, False)])
 @pytest.mark.parametrize("f16", [False, True])
 def test_flash_attn_ext_store_proj(pkg, gpu, B, T, flat, f16):
     """Prefill attention, cache write, o projection and residual update as one call: the attention's epilogue writes the
@@ -454,13 +454,19 @@ def test_flash_attn_ext_store_proj(pkg, gpu, B, T, flat, f16):
     o2 = torch.full_like(o1, float("nan"))
     args = (qd, kd, vd, d(mask))
     tail = (d(k), d(slot(kc2)), d(v), d(slot(vc2)), d(shape(b, hidden)), wd, d(shape(res, hidden)), d(shape(o2, hidden)))
-    assert L.vx_supports_flash_attn_ext_store_proj(*args, *tail, 0.0, pkg.ACT_FLOAT) == 1
+    one_pass = B * T >= 32768   # (from there on the projection alone is a product the pre-tiled kernel takes)
+    assert L.vx_supports_flash_attn_ext_store_proj(*args, *tail, 0.0, pkg.ACT_FLOAT) == (1 if one_pass else 0)
     assert L.vx_supports_flash_attn_ext_store_proj(*args, *tail, 0.0, pkg.ACT_Q8) == 0
     ok(pkg, L.vx_flash_attn_ext_store_proj(*args, None, *tail, scale, 0.0, 0.0, 0.25, 0.5, 0.7, pkg.ACT_FLOAT, None), "flash_attn_ext_store_proj")
     torch.cuda.synchronize()
     assert torch.equal(kc1.view(torch.uint8), kc2.view(torch.uint8)) and torch.equal(vc1.view(torch.uint8), vc2.view(torch.uint8))
     assert bool(torch.isfinite(o2).all()) and torch.equal(o1, o2)
-    assert bool((b == 7.0).all()), "the attention output is not stored"
+    if one_pass:
+        assert bool((b == 7.0).all()), "the attention output is not stored"
+    else:   # smaller shapes run as the calls the entry point stands for, through attn's memory
+        assert torch.equal(a, b)
+        assert L.vx_flash_attn_ext_store_proj(*args, None, *tail[:4], d(shape(o2, hidden)), *tail[5:], scale, 0.0, 0.0, 0.25, 0.5, 0.7, pkg.ACT_FLOAT, None) != 0, \
+            "dst over attn's memory must be refused on this route"
     # in place on the residual, as layer_forward's update is laid out
     r2 = res.clone()
     ok(pkg, L.vx_flash_attn_ext_store_proj(*args, None, *tail[:6], d(shape(r2, hidden)), d(shape(r2, hidden)), scale, 0.0, 0.0, 0.25, 0.5, 0.7,

@@ -1171,6 +1171,14 @@ static vx_status pf_store_proj_launch(void * front, void * ctx, hipStream_t st) 
     return pf_store_launch(front, &c->store, st);
 }
 
+// the tensor attn describes, in the attention's own shape [head_dim, heads, tokens, batch] (the same dense memory order)
+static vx_tensor pf_attn_shape(const vx_tensor * q, const vx_tensor * attn) {
+    vx_tensor ad = *attn;
+    ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
+    ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+    return ad;
+}
+
 // attn: the attention's result as the projection reads it, [hidden, tokens (, batch)], dense; the same memory order as the
 // attention's own [head_dim, heads, tokens, batch]
 static bool pf_proj_geometry(const vx_tensor * q, const vx_tensor * attn, const vx_tensor * w_o, const vx_tensor * residual, const vx_tensor * dst,
@@ -1197,10 +1205,7 @@ extern "C" int vx_supports_flash_attn_ext_store_proj(const vx_tensor * q, const 
                                                      const vx_tensor * v_slot, const vx_tensor * attn, const vx_tensor * w_o,
                                                      const vx_tensor * residual, const vx_tensor * dst, float logit_softcap, int act_mode) {
     if (!attn || !q) return 0;
-    // (the attention's own destination: the tensor attn describes, in the attention's shape)
-    vx_tensor ad = *attn;
-    ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
-    ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+    const vx_tensor ad = pf_attn_shape(q, attn);
     if (!vx_supports_flash_attn_ext_store(q, k, v, mask, k_src, k_slot, v_src, v_slot, &ad, logit_softcap)) return 0;
     vx_pf_front front{};
     size_t proj_bytes = 0;
@@ -1222,9 +1227,12 @@ extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_
         // not this form's shapes (or a kernel it needs switched off since the caller asked): the calls it stands for, through attn's memory
         if (attn->type != VX_TYPE_F32 || !vx_is_contiguous(attn) || vx_nelements(attn) != vx_nelements(q))
             return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: attn must be the attention's dense F32 result");
-        vx_tensor ad = *attn;
-        ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
-        ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+        {   // (this route stores the attention's result in attn's memory and the projection reads it there: dst must lie apart)
+            const char * a0 = (const char *) attn->data, * d0 = (const char *) dst->data;
+            const size_t ab = (size_t) vx_nelements(attn) * 4, db = (size_t) ((dst->ne[1] - 1) * dst->nb[1] + (dst->ne[2] - 1) * dst->nb[2] + (dst->ne[3] - 1) * dst->nb[3]) + (size_t) dst->ne[0] * 4;
+            if (a0 < d0 + db && d0 < a0 + ab) return vx_fail(VX_ERR_UNSUPPORTED, "flash_attn_ext_store_proj: dst overlaps attn and the shapes need attn's memory");
+        }
+        const vx_tensor ad = pf_attn_shape(q, attn);
         const vx_status rc = vx_flash_attn_ext_store(q, k, v, mask, sinks, k_src, k_slot, v_src, v_slot, &ad, scale, max_bias, logit_softcap, sync_scale,
                                                      sync_bias, stream);
         return rc != VX_OK ? rc : vx_mul_mat_scale_add(w_o, attn, residual, dst, res_scale, act_mode, stream);
@@ -1240,9 +1248,7 @@ extern "C" vx_status vx_flash_attn_ext_store_proj(const vx_tensor * q, const vx_
         const vx_status rc = vx_workspace(st, front.bytes + proj_bytes, &p);
         if (rc != VX_OK) return rc;
     }
-    vx_tensor ad = *attn; // (never written: the result leaves as tiles)
-    ad.ne[0] = q->ne[0]; ad.ne[1] = q->ne[2]; ad.ne[2] = q->ne[1]; ad.ne[3] = q->ne[3];
-    ad.nb[0] = 4; ad.nb[1] = (uint64_t) ad.ne[0] * 4; ad.nb[2] = ad.nb[1] * (uint64_t) ad.ne[1]; ad.nb[3] = ad.nb[2] * (uint64_t) ad.ne[2];
+    const vx_tensor ad = pf_attn_shape(q, attn); // (never written: the result leaves as tiles)
     vx_status rc = vx_fattn_prefill(q, k, v, mask, sinks, nullptr, &ad, scale, max_bias, logit_softcap, st, &front);
     if (rc != VX_OK) return rc == VX_ERR_UNSUPPORTED ? vx_fail(rc, "flash_attn_ext_store_proj: the LDS-tiled kernel declined") : rc;
     // the projection: its own needs go behind the front (a block that a larger request replaces stays valid)
