@@ -284,7 +284,30 @@ def test_supports_truth_table_node_groups(pkg):
     short = D(pkg, pkg.F32, [Dh, 100, Hkv, 2], [4, 4 * Dh, 4 * Dh * 768, 4 * Dh * 768 * Hkv])
     assert lib.vx_supports_flash_attn_ext_kv2(q, short, cur, short, cur, None, attn) == 1
     assert lib.vx_supports_flash_attn_ext_kv2_store(q, short, cur, short, cur, None, k_src, slot, k_src, slot, attn) == 0  # no merge kernel to ride on
+    # a prefill's attention block: the cache write in front of the attention, the o projection behind it
+    T = 4096
+    qp, kp = f32(pkg, [Dh, T, H, 16]), f32(pkg, [Dh, T, Hkv, 16])
+    ks_, slotp = f32(pkg, [Dh, Hkv, T, 16]), D(pkg, pkg.F16, [Dh, Hkv, T, 16], [2, 2 * Dh * (T + 8), 2 * Dh, 2 * Dh * (T + 8) * Hkv])
+    outp = f32(pkg, [Dh, H, T, 16])
+    assert lib.vx_supports_flash_attn_ext_store(qp, kp, kp, None, ks_, slotp, ks_, slotp, outp, 0.0) == 1
+    assert lib.vx_supports_flash_attn_ext_store(qp, kp, kp, None, ks_, slotp, ks_, slotp, outp, 30.0) == 0          # soft cap: the general kernel
+    assert lib.vx_supports_flash_attn_ext_store(q, f32(pkg, [Dh, 1, Hkv, 2]), f32(pkg, [Dh, 1, Hkv, 2]), None, k_src, slot, k_src, slot, attn, 0.0) == 0  # decode-sized
+    flat, hid = f32(pkg, [K, 16 * T, 1, 1]), f32(pkg, [K, 16 * T, 1, 1])
+    assert lib.vx_supports_flash_attn_ext_store_proj(qp, kp, kp, None, ks_, slotp, ks_, slotp, flat, wo, hid, hid, 0.0, pkg.ACT_FLOAT) == 1
+    assert lib.vx_supports_flash_attn_ext_store_proj(qp, kp, kp, None, ks_, slotp, ks_, slotp, flat, wo, hid, hid, 0.0, pkg.ACT_Q8) == 0
+    assert lib.vx_supports_flash_attn_ext_store_proj(qp, kp, kp, None, ks_, slotp, ks_, slotp, f32(pkg, [K, T, 16, 1]), wo,
+                                                     f32(pkg, [K, T, 16, 1]), f32(pkg, [K, T, 16, 1]), 0.0, pkg.ACT_FLOAT) == 1   # as a batch
+    assert lib.vx_supports_flash_attn_ext_store_proj(qp, kp, kp, None, ks_, slotp, ks_, slotp, f32(pkg, [K, 8 * T, 2, 1]), wo,
+                                                     f32(pkg, [K, 8 * T, 2, 1]), f32(pkg, [K, 8 * T, 2, 1]), 0.0, pkg.ACT_FLOAT) == 0  # neither layout
+    # k and v alone with k's rotation: while both are the streaming kernel's shapes
+    for n, want in ((300, 1), (2048, 1), (2049, 0)):
+        xn = f32(pkg, [K, n, 1, 1])
+        assert lib.vx_supports_kv_proj_rope(wk, wk, xn, f32(pkg, [Dh, Hkv, n, 1]), f32(pkg, [Hkv * Dh, n, 1, 1]), Dh, 2) == want, n
+    assert lib.vx_supports_kv_proj_rope(wk, wk, f32(pkg, [K, 300, 1, 1]), f32(pkg, [Dh, Hkv, 300, 1]), f32(pkg, [Hkv * Dh, 300, 1, 1]), Dh, 0) == 0
     # null operands are refused, not dereferenced
+    assert lib.vx_supports_flash_attn_ext_store(qp, kp, kp, None, None, slotp, ks_, slotp, outp, 0.0) == 0
+    assert lib.vx_supports_flash_attn_ext_store_proj(qp, kp, kp, None, ks_, slotp, ks_, slotp, flat, None, hid, hid, 0.0, pkg.ACT_FLOAT) == 0
+    assert lib.vx_supports_kv_proj_rope(wk, None, xb, k_dst, vb, Dh, 2) == 0
     assert lib.vx_supports_flash_attn_ext_kv2(q, past, None, past, cur, None, attn) == 0
     assert lib.vx_supports_mul_mat_scale_add(wo, acts(2), None, acts(2)) == 0
     assert lib.vx_supports_kv_store_sync(k_src, slot, None, slot, attn, attn) == 0
