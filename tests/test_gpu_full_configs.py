@@ -257,7 +257,7 @@ def test_backbone_prompt_lengths_grouped_equals_node_by_node(gpu, ref, kv_f16):
     the streaming kernel's token limits (16, 64, 204), the three regimes of the cache write (128 / 129 and 512 / 513
     tokens at batch 1), the LDS-tiled attention's minimum, the ROPE kernels' switch at 1024 tokens, the pre-tiled product's
     thresholds --, batch 1 to 3: with node groups on, hidden states and the written cache are bit-equal to every node run
-    as its own launch, and finite."""
+    as its own launch, and finite.  The same for a second chunk of tokens behind cached keys."""
     say(f"plugin prefill, grouped against node by node, over prompt lengths; f16 cache {kv_f16}")
     layers = 2
     params = reflib.backbone_params("bb-lengths", layers)
@@ -304,6 +304,26 @@ def test_backbone_prompt_lengths_grouped_equals_node_by_node(gpu, ref, kv_f16):
                     assert e <= 1e-4 and ec <= 1e-4, (B, T, e, ec)
                 assert l1 < l0, (B, T, l1, l0)
                 assert np.array_equal(o1, o0) and np.array_equal(c1, c0), f"batch {B}, {T} tokens: {l1} grouped launches differ from {l0} separate ones"
+        # and a second chunk behind cached keys (the CONCAT / cast nodes of a step with a past, at prompt sizes)
+        for B, T0, T in ((1, 512, 600), (2, 100, 1000), (1, 1024, 64), (1, 2048, 256), (2, 300, 300)):
+            runs = []
+            for fusion in (1, 0):
+                reflib.ref_backbone_create(params, T0 + T + 8, B, use_mup=True, kv_f16=kv_f16)
+                before = plugin.ggml_backend_gfx950_set_fusion(fusion)
+                try:
+                    x0 = rng("bb-lengths", B, T0, "first").standard_normal((B, T0, 1024)).astype(np.float32)
+                    reflib.ref_backbone_forward(x0, 0, reflib.causal_mask(T0, T0))
+                    x = rng("bb-lengths", B, T, "second").standard_normal((B, T, 1024)).astype(np.float32)
+                    out = reflib.ref_backbone_forward(x, T0, reflib.causal_mask(T, T0 + T, T0))[0].copy()
+                    cache = np.empty((B, 2, T0 + T + 8, 64), np.float16 if kv_f16 else np.float32)
+                    assert ref.rh_bb_cache_get(layers - 1, 0, cache.ctypes.data, cache.nbytes) == 0
+                finally:
+                    plugin.ggml_backend_gfx950_set_fusion(before)
+                    ref.rh_bb_free()
+                runs.append((out, cache[:, :, :T0 + T].copy(), plugin.ggml_backend_gfx950_last_launches()))
+            (o1, c1, l1), (o0, c0, l0) = runs
+            assert np.isfinite(o1).all() and l1 < l0, (B, T0, T, l1, l0)
+            assert np.array_equal(o1, o0) and np.array_equal(c1, c0), f"batch {B}, {T} tokens behind {T0}: {l1} grouped launches differ from {l0} separate ones"
     finally:
         plugin.ggml_backend_gfx950_set_graph_replay(replay)
         assert ref.rh_use_device(b"CPU", 8, 0) == 0
